@@ -1,0 +1,396 @@
+// causal_conv1d prefill (depthwise causal convolution, width 2..4, optional bias,
+// optional SiLU, optional initial state, final-state write-back).
+//
+// Bandwidth-bound: each element of x is read once (plus a W-1 row halo per
+// token tile) and each element of y written once.  One thread owns 8 adjacent
+// channels (one 16-byte access) and walks TOK_PER_THREAD consecutive tokens with
+// the last W-1 inputs held in registers, so a wave reads and writes 1 KiB
+// contiguous per token row.  Semantics: causal_conv1d/README.md:15-31 and
+// op_kernel/causal_conv1d.h:424-498 (tap loop), :753-776 (state write-back).
+#include "common.h"
+#include "device_utils.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 128;
+constexpr int kTok = 32;  // tokens per thread
+constexpr int kMaxW = 4;
+
+struct ConvParams {
+    const void *x;
+    const void *weight;
+    const void *bias;
+    void *conv_states;
+    void *out;
+    const int32_t *qsl;    // [N+1] device, varlen only
+    const int32_t *cache;  // [N] device or null
+    const int32_t *init;   // [N] device or null
+    int64_t x_sb, x_ss;            // batch / token strides of x (elements)
+    int64_t o_sb, o_sh, o_ss;      // out strides: batch, head, token
+    int64_t w_sr;                  // weight row stride
+    int64_t cs_sn, cs_sp;          // conv_states strides: slot, position
+    int B, S, D, W, N;
+    int head_dim;                  // D / head_num, or D when no head split
+    int tiles_per_seq;             // dense only
+    int activation;
+    int pad_slot;
+    int varlen;
+};
+
+template <typename T> __device__ __forceinline__ void load8(const T *p, float (&f)[8]) {
+    typename Vec8<T>::type v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec8<T>::type *>(p));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+}
+template <typename T> __device__ __forceinline__ void load8_cached(const T *p, float (&f)[8]) {
+    typename Vec8<T>::type v = *reinterpret_cast<const typename Vec8<T>::type *>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+}
+template <typename T> __device__ __forceinline__ void store8(T *p, const float (&f)[8]) {
+    typename Vec8<T>::type v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (T)f[i];
+    __builtin_nontemporal_store(v, reinterpret_cast<typename Vec8<T>::type *>(p));
+}
+
+__device__ __forceinline__ int find_seq(const int32_t *qsl, int N, int t) {
+    // largest n with qsl[n] <= t, skipping empty sequences implicitly
+    int lo = 0, hi = N - 1;
+    while (lo < hi) {
+        int mid = (lo + hi + 1) >> 1;
+        if (qsl[mid] <= t) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+}
+
+template <typename T, int W>
+__global__ void __launch_bounds__(kThreads) conv1d_fwd_kernel(const ConvParams p) {
+    const int d0 = (blockIdx.y * kThreads + threadIdx.x) * 8;
+    if (d0 >= p.D) return;
+    const T *x = static_cast<const T *>(p.x);
+    T *out = static_cast<T *>(p.out);
+
+    float w[W][8], bias[8];
+#pragma unroll
+    for (int r = 0; r < W; ++r) load8_cached(static_cast<const T *>(p.weight) + r * p.w_sr + d0, w[r]);
+    if (p.bias) {
+        load8_cached(static_cast<const T *>(p.bias) + d0, bias);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bias[i] = 0.f;
+    }
+
+    // token range of this tile and the sequence it starts in
+    int b, t0, t_end, n, bos, eos;
+    if (p.varlen) {
+        b = 0;
+        t0 = blockIdx.x * kTok;
+        t_end = min(t0 + kTok, p.S);
+        n = find_seq(p.qsl, p.N, t0);
+        bos = p.qsl[n];
+        eos = p.qsl[n + 1];
+    } else {
+        b = blockIdx.x / p.tiles_per_seq;
+        t0 = (blockIdx.x % p.tiles_per_seq) * kTok;
+        t_end = min(t0 + kTok, p.S);
+        n = b;
+        bos = 0;
+        eos = p.S;
+    }
+    const T *xb = x + b * p.x_sb + d0;
+    const int hd = d0 / p.head_dim, dd = d0 % p.head_dim;
+    T *ob = out + b * p.o_sb + hd * p.o_sh + dd;
+    const T *cs = static_cast<const T *>(p.conv_states);
+
+    float win[W - 1][8];  // win[r] = input row (t - (W-1) + r)
+    auto seed_window = [&](int t, int seq, int seq_bos) {
+        const int slot = p.cache ? p.cache[seq] : seq;
+        const bool use_init = cs != nullptr && p.init != nullptr && p.init[seq] == 1 && slot != p.pad_slot;
+#pragma unroll
+        for (int r = 0; r < W - 1; ++r) {
+            const int tt = t - (W - 1) + r;
+            if (tt >= seq_bos) {
+                load8_cached(xb + (int64_t)tt * p.x_ss, win[r]);
+            } else if (use_init) {
+                // row (W-1) + (tt - seq_bos) of the saved state (negative offset from its end)
+                load8_cached(cs + slot * p.cs_sn + (int64_t)(W - 1 + tt - seq_bos) * p.cs_sp + d0, win[r]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) win[r][i] = 0.f;
+            }
+        }
+    };
+    seed_window(t0, n, bos);
+    bool skip = p.varlen && p.cache && p.cache[n] == p.pad_slot;
+
+    for (int tb = t0; tb < t_end; tb += 8) {
+        float cur[8][8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (tb + j < t_end) load8(xb + (int64_t)(tb + j) * p.x_ss, cur[j]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int t = tb + j;
+            if (t >= t_end) break;
+            if (p.varlen && t >= eos) {  // entered the next non-empty sequence
+                do {
+                    ++n;
+                    bos = p.qsl[n];
+                    eos = p.qsl[n + 1];
+                } while (t >= eos);
+                seed_window(t, n, bos);
+                skip = p.cache && p.cache[n] == p.pad_slot;
+            }
+            float acc[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float a = bias[i];
+#pragma unroll
+                for (int r = 0; r < W - 1; ++r) a = fmaf(w[r][i], win[r][i], a);
+                a = fmaf(w[W - 1][i], cur[j][i], a);
+                if (p.activation == 1) a = a / (1.f + __expf(-a));
+                acc[i] = a;
+            }
+#pragma unroll
+            for (int r = 0; r + 1 < W - 1; ++r)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) win[r][i] = win[r + 1][i];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[W - 2][i] = cur[j][i];
+            if (!skip) store8(ob + (int64_t)t * p.o_ss, acc);
+        }
+    }
+}
+
+// Final-state write-back, one thread per (sequence, 8 channels): conv_states[slot, pos]
+// = row (len + pos) of [head rows | x rows], pos = 0..W-2.  Runs after the main
+// kernel on the same stream, so initial states have already been consumed.
+template <typename T>
+__global__ void conv1d_state_kernel(const ConvParams p) {
+    const int d0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const int n = blockIdx.y;
+    if (d0 >= p.D) return;
+    const int W = p.W;
+    const int slot = p.cache ? p.cache[n] : n;
+    if (slot == p.pad_slot) return;
+    int b = 0, bos = 0, len = p.S;
+    if (p.varlen) {
+        bos = p.qsl[n];
+        len = p.qsl[n + 1] - bos;
+    } else {
+        b = n;
+    }
+    T *cs = static_cast<T *>(p.conv_states) + slot * p.cs_sn + d0;
+    const T *xb = static_cast<const T *>(p.x) + b * p.x_sb + d0;
+    const bool use_init = p.init != nullptr && p.init[n] == 1;
+    float rows[kMaxW - 1][8];
+    for (int pos = 0; pos < W - 1; ++pos) {
+        const int j = len + pos - (W - 1);  // index into x rows of this sequence
+        if (j >= 0) {
+            load8_cached(xb + (int64_t)(bos + j) * p.x_ss, rows[pos]);
+        } else if (use_init) {
+            load8_cached(cs + (int64_t)(len + pos) * p.cs_sp, rows[pos]);
+        } else {
+            for (int i = 0; i < 8; ++i) rows[pos][i] = 0.f;
+        }
+    }
+    for (int pos = 0; pos < W - 1; ++pos) {
+        typename Vec8<T>::type v;
+        for (int i = 0; i < 8; ++i) v[i] = (T)rows[pos][i];
+        *reinterpret_cast<typename Vec8<T>::type *>(cs + (int64_t)pos * p.cs_sp) = v;
+    }
+}
+
+int copy_int_array(std::vector<int32_t> &dst, const fla_int_array *a) {
+    dst.clear();
+    if (a == nullptr || a->data == nullptr) return 0;
+    dst.resize(a->size);
+    for (uint64_t i = 0; i < a->size; ++i) dst[i] = (int32_t)a->data[i];
+    return (int)a->size;
+}
+
+int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias, const fla_tensor *conv_states,
+              const fla_int_array *query_start_loc, const fla_int_array *cache_indices,
+              const fla_int_array *initial_state_mode, const fla_int_array *num_accepted_tokens,
+              int64_t activation_mode, int64_t pad_slot_id, int64_t run_mode, int64_t head_num, const fla_tensor *out,
+              void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "causal_conv1d";
+    const int half_mask = dt_bit(FLA_BF16) | dt_bit(FLA_F16);
+    int rc;
+    if ((rc = check_tensor(x, op, "x", -1, half_mask))) return rc;
+    if ((rc = check_tensor(weight, op, "weight", 2, dt_bit(x->dtype)))) return rc;
+    if ((rc = check_tensor(out, op, "out", -1, dt_bit(x->dtype)))) return rc;
+    FLA_REQUIRE(run_mode == 0, FLA_ERR_UNSUPPORTED, "%s: only run_mode=0 (prefill) is implemented, got %lld.", op,
+                (long long)run_mode);
+    FLA_REQUIRE(num_accepted_tokens == nullptr || num_accepted_tokens->data == nullptr, FLA_ERR_UNSUPPORTED,
+                "%s: num_accepted_tokens is only meaningful for run_mode=1.", op);
+    FLA_REQUIRE(activation_mode == 0 || activation_mode == 1, FLA_ERR_SHAPE, "%s: activation_mode must be 0 or 1.", op);
+    FLA_REQUIRE(x->ndim == 2 || x->ndim == 3, FLA_ERR_SHAPE, "%s: x must be [B,S,D] or [T,D].", op);
+    const bool packed = x->ndim == 2;
+    const int64_t D = x->shape[x->ndim - 1];
+    const int64_t S = x->shape[x->ndim - 2];
+    const int64_t B = packed ? 1 : x->shape[0];
+    const int64_t W = weight->shape[0];
+    FLA_REQUIRE(W >= 2 && W <= kMaxW, FLA_ERR_SHAPE, "%s: width must be 2, 3 or 4, got %lld.", op, (long long)W);
+    FLA_REQUIRE(weight->shape[1] == D, FLA_ERR_SHAPE, "%s: weight must be [W,D].", op);
+    FLA_REQUIRE(D % 16 == 0, FLA_ERR_SHAPE, "%s: D must be a multiple of 16, got %lld.", op, (long long)D);
+    FLA_REQUIRE(inner_unit(x) && inner_unit(weight) && inner_unit(out), FLA_ERR_SHAPE,
+                "%s: innermost stride of x, weight and out must be 1.", op);
+    FLA_REQUIRE(B * S < ((int64_t)1 << 31) && D < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents exceed int32.", op);
+    if (bias && bias->data) {
+        if ((rc = check_tensor(bias, op, "bias", 1, dt_bit(x->dtype)))) return rc;
+        FLA_REQUIRE(bias->shape[0] == D && inner_unit(bias), FLA_ERR_SHAPE, "%s: bias must be a contiguous [D].", op);
+    }
+    FLA_REQUIRE(head_num >= 0, FLA_ERR_SHAPE, "%s: head_num must be >= 0.", op);
+    int64_t head_dim = D;
+    if (head_num > 0) {
+        FLA_REQUIRE(D % head_num == 0 && (D / head_num) % 8 == 0, FLA_ERR_SHAPE,
+                    "%s: D/head_num must be a multiple of 8.", op);
+        head_dim = D / head_num;
+    }
+
+    std::vector<int32_t> qsl, cache, init;
+    int N = (int)B;
+    if (packed) {
+        FLA_REQUIRE(query_start_loc && query_start_loc->data && query_start_loc->size >= 2, FLA_ERR_METADATA,
+                    "%s: a packed [T,D] input needs query_start_loc.", op);
+        copy_int_array(qsl, query_start_loc);
+        N = (int)qsl.size() - 1;
+        FLA_REQUIRE(qsl[0] == 0 && qsl[N] == S, FLA_ERR_METADATA, "%s: query_start_loc must span [0, T].", op);
+        for (int i = 0; i < N; ++i)
+            FLA_REQUIRE(qsl[i] <= qsl[i + 1], FLA_ERR_METADATA, "%s: query_start_loc must be non-decreasing.", op);
+    } else {
+        FLA_REQUIRE(query_start_loc == nullptr || query_start_loc->data == nullptr, FLA_ERR_METADATA,
+                    "%s: query_start_loc requires a packed [T,D] input.", op);
+    }
+    if (copy_int_array(cache, cache_indices))
+        FLA_REQUIRE((int)cache.size() == N, FLA_ERR_METADATA, "%s: cache_indices must have one entry per sequence.", op);
+    if (copy_int_array(init, initial_state_mode))
+        FLA_REQUIRE((int)init.size() == N, FLA_ERR_METADATA, "%s: initial_state_mode must have one entry per sequence.",
+                    op);
+    const bool has_states = conv_states && conv_states->data;
+    if (has_states) {
+        if ((rc = check_tensor(conv_states, op, "conv_states", 3, dt_bit(x->dtype)))) return rc;
+        FLA_REQUIRE(conv_states->shape[1] >= W - 1 && conv_states->shape[2] == D && inner_unit(conv_states),
+                    FLA_ERR_SHAPE, "%s: conv_states must be [N, >=W-1, D] with unit channel stride.", op);
+        for (int i = 0; i < N; ++i) {
+            const int64_t slot = cache.empty() ? i : cache[i];
+            FLA_REQUIRE(slot == pad_slot_id || (slot >= 0 && slot < conv_states->shape[0]), FLA_ERR_METADATA,
+                        "%s: cache index %lld out of range.", op, (long long)slot);
+        }
+    }
+    // output shape
+    if (head_num > 0) {
+        const int nd = packed ? 3 : 4;
+        FLA_REQUIRE(out->ndim == nd, FLA_ERR_SHAPE, "%s: head-split out must be rank %d.", op, nd);
+        const int o = packed ? 0 : 1;
+        FLA_REQUIRE(out->shape[o] == head_num && out->shape[o + 1] == S && out->shape[o + 2] == head_dim &&
+                        (packed || out->shape[0] == B),
+                    FLA_ERR_SHAPE, "%s: out must be [B,head_num,S,D/head_num].", op);
+    } else {
+        FLA_REQUIRE(same_shape(out, x), FLA_ERR_SHAPE, "%s: out must have the shape of x.", op);
+    }
+
+    const size_t meta_ints = qsl.size() + cache.size() + init.size();
+    const uint64_t need = ((meta_ints * 4 + 255) / 256) * 256;
+    if (query) {
+        *query = need;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(need == 0 || (workspace != nullptr && workspace_size >= need), FLA_ERR_WORKSPACE,
+                "%s: workspace of %llu bytes required.", op, (unsigned long long)need);
+    if (B * S == 0) return FLA_OK;
+
+    ConvParams p{};
+    p.x = x->data;
+    p.weight = weight->data;
+    p.bias = (bias && bias->data) ? bias->data : nullptr;
+    p.conv_states = has_states ? conv_states->data : nullptr;
+    p.out = out->data;
+    if (meta_ints) {
+        std::vector<int32_t> meta;
+        meta.insert(meta.end(), qsl.begin(), qsl.end());
+        meta.insert(meta.end(), cache.begin(), cache.end());
+        meta.insert(meta.end(), init.begin(), init.end());
+        if ((rc = stage_to_device(workspace, meta.data(), meta.size() * 4, stream))) return rc;
+        const int32_t *base = static_cast<const int32_t *>(workspace);
+        p.qsl = qsl.empty() ? nullptr : base;
+        p.cache = cache.empty() ? nullptr : base + qsl.size();
+        p.init = init.empty() ? nullptr : base + qsl.size() + cache.size();
+    }
+    p.x_sb = packed ? 0 : x->stride[0];
+    p.x_ss = x->stride[x->ndim - 2];
+    if (head_num > 0) {
+        const int o = packed ? 0 : 1;
+        p.o_sb = packed ? 0 : out->stride[0];
+        p.o_sh = out->stride[o];
+        p.o_ss = out->stride[o + 1];
+    } else {
+        p.o_sb = packed ? 0 : out->stride[0];
+        p.o_sh = 0;
+        p.o_ss = out->stride[out->ndim - 2];
+    }
+    p.w_sr = weight->stride[0];
+    if (has_states) {
+        p.cs_sn = conv_states->stride[0];
+        p.cs_sp = conv_states->stride[1];
+    }
+    p.B = (int)B;
+    p.S = (int)S;
+    p.D = (int)D;
+    p.W = (int)W;
+    p.N = N;
+    p.head_dim = (int)head_dim;
+    p.tiles_per_seq = (int)((S + kTok - 1) / kTok);
+    p.activation = (int)activation_mode;
+    p.pad_slot = (int)pad_slot_id;
+    p.varlen = packed ? 1 : 0;
+
+    const dim3 block(kThreads);
+    const dim3 grid((unsigned)(p.tiles_per_seq * (packed ? 1 : B)), (unsigned)((D / 8 + kThreads - 1) / kThreads));
+    const bool is_bf16 = x->dtype == FLA_BF16;
+#define FLA_LAUNCH_CONV(WW)                                                                  \
+    if (is_bf16) hipLaunchKernelGGL((conv1d_fwd_kernel<bf16, WW>), grid, block, 0, stream, p); \
+    else hipLaunchKernelGGL((conv1d_fwd_kernel<f16, WW>), grid, block, 0, stream, p)
+    switch (W) {
+        case 2: FLA_LAUNCH_CONV(2); break;
+        case 3: FLA_LAUNCH_CONV(3); break;
+        default: FLA_LAUNCH_CONV(4); break;
+    }
+#undef FLA_LAUNCH_CONV
+    FLA_HIP_CHECK(hipGetLastError());
+    if (has_states && N > 0) {
+        const dim3 sgrid((unsigned)((D / 8 + 63) / 64), (unsigned)N);
+        if (is_bf16) hipLaunchKernelGGL(conv1d_state_kernel<bf16>, sgrid, dim3(64), 0, stream, p);
+        else hipLaunchKernelGGL(conv1d_state_kernel<f16>, sgrid, dim3(64), 0, stream, p);
+        FLA_HIP_CHECK(hipGetLastError());
+    }
+    return FLA_OK;
+}
+
+}  // namespace
+}  // namespace fla
+
+extern "C" int fla_causal_conv1d_get_workspace_size(
+    const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias, const fla_tensor *conv_states,
+    const fla_int_array *query_start_loc, const fla_int_array *cache_indices, const fla_int_array *initial_state_mode,
+    const fla_int_array *num_accepted_tokens, int64_t activation_mode, int64_t pad_slot_id, int64_t run_mode,
+    int64_t head_num, const fla_tensor *out, uint64_t *workspace_size) {
+    if (workspace_size == nullptr) return fla::fail(FLA_ERR_NULL, "causal_conv1d: workspace_size must not be null.");
+    return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
+                          num_accepted_tokens, activation_mode, pad_slot_id, run_mode, head_num, out, nullptr, 0,
+                          nullptr, workspace_size);
+}
+
+extern "C" int fla_causal_conv1d(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias,
+                                 const fla_tensor *conv_states, const fla_int_array *query_start_loc,
+                                 const fla_int_array *cache_indices, const fla_int_array *initial_state_mode,
+                                 const fla_int_array *num_accepted_tokens, int64_t activation_mode,
+                                 int64_t pad_slot_id, int64_t run_mode, int64_t head_num, const fla_tensor *out,
+                                 void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
+                          num_accepted_tokens, activation_mode, pad_slot_id, run_mode, head_num, out, workspace,
+                          workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}

@@ -1,0 +1,125 @@
+"""Public operator namespace: the names of ``fla_npu.ops.ascendc`` backed by HIP kernels.
+
+Every operator is exported twice, as ``npu_<op>`` and ``<op>``
+(torch_custom/fla_npu/fla_npu/ops/ascendc/__init__.py:28-50,426-431).  Operators
+that write into an argument declare it in ``MUTATED_ARGUMENTS``; their wrapper
+rejects tensors that require grad and bumps the autograd version counter after
+the launch (:61-71,146-185).  Names of reference operators that this library
+does not implement raise ``NotImplementedError`` when called.
+"""
+from __future__ import annotations
+
+import functools
+import inspect
+from typing import Callable
+
+from ._hip_ctypes import HIP_CTYPES_OPS, gdn_chunk_fwd
+
+_REFERENCE_OPS = (
+    "npu_fast_gelu_custom",
+    "npu_fast_gelu_custom_backward",
+    "npu_causal_conv1d",
+    "npu_causal_conv1d_bwd",
+    "npu_prepare_wy_repr_bwd_full",
+    "npu_prepare_wy_repr_bwd",
+    "npu_chunk_gated_delta_rule_bwd_dhu",
+    "npu_chunk_bwd_dv_local",
+    "npu_prepare_wy_repr_bwd_da",
+    "npu_chunk_bwd_dqkwg",
+    "npu_chunk_fwd_o",
+    "npu_chunk_gated_delta_rule_fwd_h",
+    "npu_recompute_w_u_fwd",
+    "npu_recurrent_gated_delta_rule",
+    "npu_chunk_local_cumsum",
+    "npu_chunk_scaled_dot_kkt",
+    "npu_solve_tri",
+    "npu_chunk_kda_fwd",
+    "npu_chunk_kda_bwd_intra",
+    "npu_kda_gate_cumsum",
+    "npu_recurrent_kda",
+)
+
+MUTATED_ARGUMENTS = {
+    "causal_conv1d": ("conv_states",),
+    "npu_causal_conv1d": ("conv_states",),
+    "recurrent_gated_delta_rule": ("state",),
+    "npu_recurrent_gated_delta_rule": ("state",),
+}
+
+
+def _strip_npu_prefix(name: str) -> str:
+    return name[4:] if name.startswith("npu_") else name
+
+
+def _wrap_mutable_op(name: str, op: Callable) -> Callable:
+    mutated_names = MUTATED_ARGUMENTS.get(name, ())
+    if not mutated_names:
+        return op
+    signature = inspect.signature(op)
+
+    @functools.wraps(op)
+    def wrapper(*args, **kwargs):
+        import torch
+
+        bound = signature.bind(*args, **kwargs)
+        bound.apply_defaults()
+        mutated = [bound.arguments[n] for n in mutated_names]
+        requiring_grad = [n for n in mutated_names if getattr(bound.arguments[n], "requires_grad", False)]
+        if requiring_grad:
+            names = ", ".join(requiring_grad)
+            raise RuntimeError(
+                f"{name} mutates {names} in place through ctypes. Mutable state tensors "
+                "must not require gradients; use a functional state API for training."
+            )
+        result = op(*args, **kwargs)
+        mutated = [t for t in mutated if isinstance(t, torch.Tensor)]
+        if mutated:
+            torch.autograd.graph.increment_version(mutated)
+        return result
+
+    return wrapper
+
+
+def _missing_op(name: str) -> Callable:
+    def op(*args, **kwargs):
+        raise NotImplementedError(
+            f"fla_hip.ops.{name} is not implemented by this library (outside the accelerated path)."
+        )
+
+    op.__name__ = name
+    op.__qualname__ = name
+    return op
+
+
+for _name in _REFERENCE_OPS:
+    _op = HIP_CTYPES_OPS.get(_name)
+    _op = _missing_op(_name) if _op is None else _wrap_mutable_op(_name, _op)
+    globals()[_name] = _op
+    globals()[_strip_npu_prefix(_name)] = _op
+
+
+def causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=None, cache_indices=None,
+                  initial_state_mode=None, num_accepted_tokens=None, activation_mode=0, pad_slot_id=-1,
+                  run_mode=0, head_num=0):
+    """Causal conv1d prefill (ops/ascendc/__init__.py:299-392).  ``conv_states`` is
+    mutable state and must not require gradients.  The backward operator is outside
+    this library, so inputs that require grad are rejected instead of silently
+    detached."""
+    import torch
+
+    for t in (x, weight, bias):
+        if isinstance(t, torch.Tensor) and t.requires_grad and torch.is_grad_enabled():
+            raise NotImplementedError("fla_hip.ops.causal_conv1d: backward is not implemented; pass detached inputs.")
+    return globals()["npu_causal_conv1d"](
+        x=x, weight=weight, bias=bias, conv_states=conv_states, query_start_loc=query_start_loc,
+        cache_indices=cache_indices, initial_state_mode=initial_state_mode,
+        num_accepted_tokens=num_accepted_tokens, activation_mode=activation_mode, pad_slot_id=pad_slot_id,
+        run_mode=run_mode, head_num=head_num)
+
+
+__all__ = [
+    "MUTATED_ARGUMENTS",
+    "gdn_chunk_fwd",
+    *sorted(set(_REFERENCE_OPS)),
+    *sorted({_strip_npu_prefix(n) for n in _REFERENCE_OPS}),
+]

@@ -1,0 +1,397 @@
+"""Per-operator ctypes wrappers over ``libfla_hip.so``.
+
+Each function keeps the name, positional / keyword structure, defaults, output
+allocation and error text of its counterpart in
+torch_custom/fla_npu/fla_npu/ops/ascendc/_aclnn_ctypes.py (line numbers in the
+docstrings); only the device type (ROCm ``cuda`` tensors) and the C symbol
+differ.  Argument order of every C call equals the aclnn prototype's.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+from . import _runtime
+from ._runtime import INT_ARRAY_P, TENSOR_P
+
+_call_op = _runtime.call_op
+_empty = _runtime.empty
+_empty_like = _runtime.empty_like
+_shape = _runtime.shape
+
+_T, _IA = TENSOR_P, INT_ARRAY_P
+
+# C operand types of each operator, in prototype order (workspace / stream tail excluded).
+OP_ARGTYPES = {
+    "chunk_local_cumsum": [_T, _IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_double, ctypes.c_bool,
+                           ctypes.c_char_p, _T],
+    "chunk_scaled_dot_kkt": [_T, _T, _T, _IA, _IA, ctypes.c_int64, _T],
+    "solve_tri": [_T, _IA, _IA, ctypes.c_char_p, _T],
+    "recompute_w_u_fwd": [_T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_int64, _T, _T],
+    "chunk_gated_delta_rule_fwd_h": [_T, _T, _T, _T, _T, _T, ctypes.c_bool, ctypes.c_int64, _IA, _IA,
+                                     ctypes.c_bool, _T, _T, _T],
+    "chunk_fwd_o": [_T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
+    "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, _T, _T, _T],
+    "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
+    "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                      ctypes.c_int64, _T],
+}
+
+
+def _optional_int(value, default: int) -> int:
+    return default if value is None else int(value)
+
+
+def _optional_bool(value, default: bool) -> bool:
+    return default if value is None else bool(value)
+
+
+def _optional_float(value, default: float) -> float:
+    return default if value is None else float(value)
+
+
+def _as_int_tuple(values) -> Optional[tuple]:
+    if values is None:
+        return None
+    import torch
+
+    if isinstance(values, torch.Tensor):
+        values = values.detach().cpu().flatten().tolist()
+    return tuple(int(v) for v in values)
+
+
+def _build_chunk_indices(cu: tuple, chunk_size: int) -> tuple:
+    """Canonical sequence-major (seq, chunk) list; empty sequences own no chunk."""
+    out = []
+    for n, (s, e) in enumerate(zip(cu, cu[1:])):
+        for c in range((e - s + chunk_size - 1) // chunk_size):
+            out.extend((n, c))
+    return tuple(out)
+
+
+def _total_chunks(B: int, T: int, chunk_size: int, cu: Optional[tuple]) -> int:
+    if cu is None:
+        return (T + chunk_size - 1) // chunk_size
+    return sum((e - s + chunk_size - 1) // chunk_size for s, e in zip(cu, cu[1:]))
+
+
+# ---------------------------------------------------------------------------------------------
+def npu_chunk_fwd_o(q, k, v, h, scale, *, g=None, g_gamma=None, cu_seqlens=None, chunk_indices=None,
+                    chunk_size=None, transpose_state_layout=False):
+    """_aclnn_ctypes.py:517-549.  ``g_gamma`` and ``transpose_state_layout`` are ignored there too."""
+    del g_gamma, transpose_state_layout
+    chunk_size = _optional_int(chunk_size, 64)
+    out = _empty_like(v)
+    return _call_op(
+        "chunk_fwd_o", OP_ARGTYPES["chunk_fwd_o"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(h, "h"), ctx.tensor(g, "g"),
+            ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices),
+            ctypes.c_double(float(scale)), ctypes.c_int64(chunk_size), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def npu_chunk_gated_delta_rule_fwd_h(k, w, u, g=None, *, gk=None, initial_state=None, output_final_state=False,
+                                     chunk_size=None, cu_seqlens=None, chunk_indices=None, state_v_first=False):
+    """_aclnn_ctypes.py:552-615."""
+    import torch
+
+    if g is None and gk is None:
+        raise RuntimeError("npu_chunk_gated_delta_rule_fwd_h: either g or gk must be provided.")
+    output_final_state = _optional_bool(output_final_state, False)
+    state_v_first = _optional_bool(state_v_first, False)
+    chunk_size = _optional_int(chunk_size, 64)
+    B, _, T, K = _shape(k)
+    _, HV, _, V = _shape(u)
+    cu = _as_int_tuple(cu_seqlens)
+    indices = _as_int_tuple(chunk_indices)
+    if indices is None and cu is not None:
+        indices = _build_chunk_indices(cu, chunk_size)
+    NT = _total_chunks(B, T, chunk_size, cu)
+    N = len(cu) - 1 if cu is not None else B
+    state_tail = (V, K) if state_v_first else (K, V)
+    if initial_state is not None and _shape(initial_state) != (N, HV, *state_tail):
+        raise RuntimeError("npu_chunk_gated_delta_rule_fwd_h: initial_state shape does not match state_v_first.")
+    h_out = _empty((B, HV, NT, *state_tail), k)
+    v_new_out = _empty_like(u)
+    if output_final_state:
+        if initial_state is not None:
+            final_state_out = _empty((N, HV, *state_tail), initial_state)
+        else:
+            final_state_out = _empty((N, HV, *state_tail), k, dtype=torch.float32)
+    else:
+        final_state_out = None
+    outputs = (h_out, v_new_out, final_state_out if output_final_state else None)
+    return _call_op(
+        "chunk_gated_delta_rule_fwd_h", OP_ARGTYPES["chunk_gated_delta_rule_fwd_h"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(w, "w"), ctx.tensor(u, "u"), ctx.tensor(g, "g"), ctx.tensor(gk, "gk"),
+            ctx.tensor(initial_state, "initial_state"),
+            ctypes.c_bool(output_final_state), ctypes.c_int64(chunk_size),
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_bool(state_v_first),
+            ctx.tensor(h_out, "h"), ctx.tensor(v_new_out, "v_new"), ctx.tensor(final_state_out, "final_state"),
+        ],
+        outputs,
+    )
+
+
+def npu_recompute_w_u_fwd(k, v, beta, A, chunk_size, *, g=None, gk=None, cu_seqlens=None, chunk_indices=None):
+    """_aclnn_ctypes.py:618-651."""
+    w_shape = list(_shape(v))
+    w_shape[3] = int(k.shape[3])
+    w_out = _empty(w_shape, v, dtype=k.dtype)
+    u_out = _empty_like(v)
+    outputs = (w_out, u_out)
+    return _call_op(
+        "recompute_w_u_fwd", OP_ARGTYPES["recompute_w_u_fwd"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"),
+            ctx.tensor(g, "g"), ctx.tensor(gk, "gk"),
+            ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(w_out, "w"), ctx.tensor(u_out, "u"),
+        ],
+        outputs,
+    )
+
+
+def npu_recurrent_gated_delta_rule(query, key, value, state, *, beta, scale=1.0, actual_seq_lengths,
+                                   ssm_state_indices, num_accepted_tokens=None, g=None, gk=None):
+    """Run recurrent GDN and update ``state`` in place (_aclnn_ctypes.py:654-846).
+
+    ``g`` and ``gk`` are independent optional gates; one of them must be given.
+    """
+    op_name = "npu_recurrent_gated_delta_rule"
+    if g is None and gk is None:
+        raise RuntimeError(f"{op_name}: either g or gk must be provided.")
+
+    import torch
+
+    tensors = {
+        "query": query, "key": key, "value": value, "state": state, "beta": beta,
+        "actual_seq_lengths": actual_seq_lengths, "ssm_state_indices": ssm_state_indices,
+    }
+    optional_tensors = {"g": g, "gk": gk, "num_accepted_tokens": num_accepted_tokens}
+    for name, tensor in (*tensors.items(), *optional_tensors.items()):
+        if tensor is None:
+            if name in tensors:
+                raise TypeError(f"{op_name}: {name} must be a torch.Tensor, got None.")
+            continue
+        if not isinstance(tensor, torch.Tensor):
+            raise TypeError(f"{op_name}: {name} must be a torch.Tensor, got {type(tensor)!r}.")
+        if tensor.device.type != "cuda":
+            raise TypeError(f"{op_name}: {name} must be a torch GPU tensor, got device {tensor.device}.")
+
+    dtype_requirements = {
+        "query": (torch.bfloat16,), "key": (torch.bfloat16,), "value": (torch.bfloat16,),
+        "beta": (torch.bfloat16,), "state": (torch.bfloat16, torch.float32),
+        "actual_seq_lengths": (torch.int32,), "ssm_state_indices": (torch.int32,),
+        "g": (torch.float32,), "gk": (torch.float32,), "num_accepted_tokens": (torch.int32,),
+    }
+    for name, supported in dtype_requirements.items():
+        tensor = tensors.get(name, optional_tensors.get(name))
+        if tensor is not None and tensor.dtype not in supported:
+            names = ", ".join(str(d) for d in supported)
+            raise TypeError(f"{op_name}: {name} dtype must be one of ({names}), got {tensor.dtype}.")
+
+    shapes = {n: _shape(t) for n, t in (*tensors.items(), *optional_tensors.items()) if t is not None}
+    expected_ranks = {"query": 3, "key": 3, "value": 3, "beta": 2, "state": 4, "actual_seq_lengths": 1,
+                      "ssm_state_indices": 1, "g": 2, "gk": 3, "num_accepted_tokens": 1}
+    for name, rank in expected_ranks.items():
+        shp = shapes.get(name)
+        if shp is not None and len(shp) != rank:
+            raise RuntimeError(f"{op_name}: {name} must be rank {rank}, got shape {shp}.")
+
+    if shapes["query"] != shapes["key"]:
+        raise RuntimeError(
+            f"{op_name}: key shape must equal query shape, got query={shapes['query']}, key={shapes['key']}.")
+    total_tokens, key_heads, key_dim = shapes["query"]
+    value_tokens, value_heads, value_dim = shapes["value"]
+    state_blocks = shapes["state"][0]
+    for name, size in {"T": total_tokens, "Nk": key_heads, "Nv": value_heads, "Dk": key_dim, "Dv": value_dim,
+                       "state blocks": state_blocks}.items():
+        if size <= 0:
+            raise RuntimeError(f"{op_name}: {name} must be positive, got {size}.")
+    if value_tokens != total_tokens:
+        raise RuntimeError(f"{op_name}: value T dimension must be {total_tokens}, got {value_tokens}.")
+    if shapes["beta"] != (total_tokens, value_heads):
+        raise RuntimeError(f"{op_name}: beta shape must be {(total_tokens, value_heads)}, got {shapes['beta']}.")
+    expected_state = (state_blocks, value_heads, value_dim, key_dim)
+    if shapes["state"] != expected_state:
+        raise RuntimeError(f"{op_name}: state shape must be {expected_state}, got {shapes['state']}.")
+    if shapes["actual_seq_lengths"][0] < 2:
+        raise RuntimeError(
+            f"{op_name}: actual_seq_lengths must contain the prefix entry and at least one sequence length.")
+    if shapes["ssm_state_indices"] != (total_tokens,):
+        raise RuntimeError(
+            f"{op_name}: ssm_state_indices shape must be ({total_tokens},), got {shapes['ssm_state_indices']}.")
+    batch_size = shapes["actual_seq_lengths"][0] - 1
+    for name, expected in {"g": (total_tokens, value_heads), "gk": (total_tokens, value_heads, key_dim),
+                           "num_accepted_tokens": (batch_size,)}.items():
+        shp = shapes.get(name)
+        if shp is not None and shp != expected:
+            raise RuntimeError(f"{op_name}: {name} shape must be {expected}, got {shp}.")
+    if key_heads > 256 or value_heads > 256 or key_dim > 512 or value_dim > 512:
+        raise RuntimeError(
+            f"{op_name}: Nk and Nv must be <= 256 and Dk and Dv must be <= 512, "
+            f"got Nk={key_heads}, Nv={value_heads}, Dk={key_dim}, Dv={value_dim}.")
+    if value_heads % key_heads != 0:
+        raise RuntimeError(
+            f"{op_name}: Nv must be an integer multiple of Nk, got Nv={value_heads}, Nk={key_heads}.")
+    scale = _optional_float(scale, 1.0)
+    if not math.isfinite(scale):
+        raise ValueError(f"{op_name}: scale must be finite, got {scale}.")
+
+    out = _empty_like(value)
+    return _call_op(
+        "recurrent_gated_delta_rule", OP_ARGTYPES["recurrent_gated_delta_rule"],
+        lambda ctx: [
+            ctx.tensor(query, "query"), ctx.tensor(key, "key"), ctx.tensor(value, "value"),
+            ctx.tensor(beta, "beta"), ctx.tensor(state, "state"),
+            ctx.tensor(actual_seq_lengths, "actual_seq_lengths"),
+            ctx.tensor(ssm_state_indices, "ssm_state_indices"),
+            ctx.tensor(g, "g"), ctx.tensor(gk, "gk"), ctx.tensor(num_accepted_tokens, "num_accepted_tokens"),
+            ctypes.c_float(scale), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def _chunk_local_cumsum_output_dtype(g, output_dtype):
+    """_aclnn_ctypes.py:849-872."""
+    import torch
+
+    if output_dtype is None:
+        return "float32", torch.float32
+    if isinstance(output_dtype, torch.dtype):
+        if output_dtype in (torch.float, torch.float32):
+            return "float32", torch.float32
+        if output_dtype in (torch.float16, torch.half):
+            return "float16", torch.float16
+        if output_dtype == torch.bfloat16:
+            return "bfloat16", torch.bfloat16
+        raise TypeError(f"Unsupported chunk_local_cumsum output_dtype: {output_dtype}.")
+    normalized = str(output_dtype).removeprefix("torch.").lower()
+    if normalized in {"float", "float32"}:
+        return "float32", torch.float32
+    if normalized in {"half", "float16"}:
+        return "float16", torch.float16
+    if normalized in {"bf16", "bfloat16"}:
+        return "bfloat16", torch.bfloat16
+    if normalized in {"same", "input", "none"}:
+        return normalized, g.dtype
+    raise TypeError(f"Unsupported chunk_local_cumsum output_dtype: {output_dtype}.")
+
+
+def npu_chunk_local_cumsum(g, chunk_size, *, cu_seqlens=None, chunk_indices_out=None, reverse=False, scale=1.0,
+                           head_first=True, output_dtype="float32"):
+    """_aclnn_ctypes.py:875-904."""
+    output_dtype_name, out_dtype = _chunk_local_cumsum_output_dtype(g, output_dtype)
+    g_contig = g.contiguous()
+    out = _empty(_shape(g_contig), g_contig, dtype=out_dtype)
+    name_buf = ctypes.create_string_buffer(output_dtype_name.encode("utf-8"))
+    return _call_op(
+        "chunk_local_cumsum", OP_ARGTYPES["chunk_local_cumsum"],
+        lambda ctx: [
+            ctx.tensor(g_contig, "g"), ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices_out),
+            ctypes.c_int64(int(chunk_size)), ctypes.c_bool(bool(reverse)), ctypes.c_double(float(scale)),
+            ctypes.c_bool(bool(head_first)), ctypes.cast(name_buf, ctypes.c_char_p), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def npu_chunk_scaled_dot_kkt(k, g, beta, *, cu_seqlens=None, chunk_indices=None, chunk_size=64):
+    """_aclnn_ctypes.py:907-936."""
+    import torch
+
+    k_contig, g_contig, beta_contig = k.contiguous(), g.contiguous(), beta.contiguous()
+    B, _, T, _ = _shape(k_contig)
+    _, Hv, _ = _shape(g_contig)
+    out = _empty((B, Hv, T, int(chunk_size)), k_contig, dtype=torch.float32)
+    return _call_op(
+        "chunk_scaled_dot_kkt", OP_ARGTYPES["chunk_scaled_dot_kkt"],
+        lambda ctx: [
+            ctx.tensor(k_contig, "k"), ctx.tensor(g_contig, "g"), ctx.tensor(beta_contig, "beta"),
+            ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def _infer_causal_conv1d_y(x, head_num: int, run_mode: int):
+    """_aclnn_ctypes.py:939-948."""
+    if run_mode == 0 and head_num > 0:
+        if x.dim() == 3:
+            b, s, d_model = _shape(x)
+            return _empty((b, head_num, s, d_model // head_num), x)
+        if x.dim() == 2:
+            s, d_model = _shape(x)
+            return _empty((head_num, s, d_model // head_num), x)
+    return _empty_like(x)
+
+
+def npu_causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=None, cache_indices=None,
+                      initial_state_mode=None, num_accepted_tokens=None, activation_mode=0, pad_slot_id=-1,
+                      run_mode=0, head_num=0):
+    """_aclnn_ctypes.py:951-985."""
+    out = _infer_causal_conv1d_y(x, int(head_num), int(run_mode))
+    return _call_op(
+        "causal_conv1d", OP_ARGTYPES["causal_conv1d"],
+        lambda ctx: [
+            ctx.tensor(x, "x"), ctx.tensor(weight, "weight"), ctx.tensor(bias, "bias"),
+            ctx.tensor(conv_states, "conv_states"),
+            ctx.int_array(query_start_loc), ctx.int_array(cache_indices), ctx.int_array(initial_state_mode),
+            ctx.int_array(num_accepted_tokens),
+            ctypes.c_int64(int(activation_mode)), ctypes.c_int64(int(pad_slot_id)), ctypes.c_int64(int(run_mode)),
+            ctypes.c_int64(int(head_num)), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def npu_solve_tri(x, *, cu_seqlens=None, chunk_indices=None, layout="bsnd"):
+    """_aclnn_ctypes.py:1786-1800."""
+    x_contig = x.contiguous()
+    out = _empty_like(x_contig)
+    layout_arg = ctypes.c_char_p(str(layout).encode("utf-8"))
+    return _call_op(
+        "solve_tri", OP_ARGTYPES["solve_tri"],
+        lambda ctx: [
+            ctx.tensor(x_contig, "x"), ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices), layout_arg,
+            ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size):
+    """Whole chunk forward in one library call (replaces the composition at
+    examples/flash_gated_delta_rule.py:796-881).  q,k,v [B,H,T,D]; g,beta [B,T,H] f32.
+    Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], final_state or None)."""
+    import torch
+
+    B, _, T, K = _shape(k)
+    _, HV, _, V = _shape(v)
+    cu = _as_int_tuple(cu_seqlens)
+    N = len(cu) - 1 if cu is not None else B
+    o = _empty((B, T, HV, V), v)
+    g_out = _empty((B, T, HV), v, dtype=torch.float32)
+    final = _empty((N, HV, K, V), v, dtype=torch.float32) if output_final_state else None
+    _call_op(
+        "gdn_chunk_fwd", OP_ARGTYPES["gdn_chunk_fwd"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"),
+            ctx.tensor(beta, "beta"), ctypes.c_double(float(scale)), ctx.tensor(initial_state, "initial_state"),
+            ctypes.c_bool(bool(output_final_state)), ctx.int_array(cu), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(o, "o"), ctx.tensor(g_out, "g_cumsum"), ctx.tensor(final, "final_state"),
+        ],
+        (o, g_out, final),
+    )
+    return g_out, o, final
+
+
+HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

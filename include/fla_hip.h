@@ -1,0 +1,242 @@
+/*
+ * fla_hip.h - C ABI of libfla_hip.so, the gfx950 (MI355X) linear-attention
+ * operator library.
+ *
+ * Every operator of the reference's custom-op library is exposed there as a
+ * two-phase pair
+ *     aclnn<Op>GetWorkspaceSize(<inputs>, <attrs>, <outputs>, uint64_t *ws, aclOpExecutor **)
+ *     aclnn<Op>(void *ws, uint64_t ws_size, aclOpExecutor *, aclrtStream)
+ * bound from Python with ctypes
+ * (torch_custom/fla_npu/fla_npu/ops/ascendc/_runtime.py:388-429).  This library
+ * keeps the argument order of each aclnn prototype but is stateless: there is
+ * no executor object, so phase two takes the operands again.
+ *
+ *     int fla_<op>_get_workspace_size(<operands>, uint64_t *workspace_size);
+ *     int fla_<op>(<operands>, void *workspace, uint64_t workspace_size, void *stream);
+ *
+ * Contract (mirrors _runtime.py:191-207,413-428,463-482):
+ *   - the caller owns every buffer: inputs, outputs and the workspace; the
+ *     library never allocates or frees device memory and keeps no pointer
+ *     after a call returns;
+ *   - an absent optional tensor / int array is a NULL pointer;
+ *   - host int arrays (cu_seqlens, chunk_indices, ...) are consumed before the
+ *     call returns;
+ *   - `stream` is a hipStream_t; kernels are enqueued on it and the call
+ *     returns without synchronising;
+ *   - return value 0 is success; any other value is an fla_status and
+ *     fla_last_error() describes it (thread-local string);
+ *   - all tensors of one call live on the current HIP device.
+ */
+#ifndef FLA_HIP_H_
+#define FLA_HIP_H_
+
+#include <stdbool.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLA_MAX_DIMS 8
+
+typedef enum fla_dtype {
+    FLA_F32 = 0,
+    FLA_F16 = 1,
+    FLA_BF16 = 2,
+    FLA_I32 = 3,
+    FLA_I64 = 4
+} fla_dtype;
+
+typedef enum fla_status {
+    FLA_OK = 0,
+    FLA_ERR_NULL = 1,        /* a required pointer is NULL                      */
+    FLA_ERR_DTYPE = 2,       /* unsupported dtype or dtype combination          */
+    FLA_ERR_SHAPE = 3,       /* rank / extent / stride violates the op contract */
+    FLA_ERR_UNSUPPORTED = 4, /* valid request this build has no kernel for      */
+    FLA_ERR_WORKSPACE = 5,   /* workspace missing or smaller than required      */
+    FLA_ERR_LAUNCH = 6,      /* the HIP runtime refused the launch              */
+    FLA_ERR_METADATA = 7     /* cu_seqlens / chunk_indices are inconsistent     */
+} fla_status;
+
+/* Replaces the opaque aclTensor built by aclCreateTensor(shape, ndim, dtype,
+ * strides, offset, format, storage_shape, n, storage_ptr) (_runtime.py:239-249).
+ * `data` already includes the storage offset; strides are in elements. */
+typedef struct fla_tensor {
+    void *data;
+    int32_t dtype; /* fla_dtype */
+    int32_t ndim;
+    int64_t shape[FLA_MAX_DIMS];
+    int64_t stride[FLA_MAX_DIMS];
+} fla_tensor;
+
+/* Replaces aclIntArray (aclCreateIntArray, _runtime.py:259-273): host int64 values. */
+typedef struct fla_int_array {
+    const int64_t *data;
+    uint64_t size;
+} fla_int_array;
+
+const char *fla_last_error(void);
+/* ABI version of this header; bumped on any signature change. */
+int fla_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * chunk_local_cumsum - replaces aclnnChunkLocalCumsum
+ * (_aclnn_ctypes.py:875-904; chunk_local_cumsum/README.md:7-24).
+ * g, out: [B,H,T] or [B,H,T,K] contiguous, head_first must be true.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_local_cumsum_get_workspace_size(
+    const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices_out,
+    int64_t chunk_size, bool reverse, double scale, bool head_first, const char *output_dtype,
+    const fla_tensor *out, uint64_t *workspace_size);
+int fla_chunk_local_cumsum(
+    const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices_out,
+    int64_t chunk_size, bool reverse, double scale, bool head_first, const char *output_dtype,
+    const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * chunk_scaled_dot_kkt - replaces aclnnChunkScaledDotKkt (_aclnn_ctypes.py:907-936).
+ * k [B,Hk,T,K] bf16; g, beta [B,Hv,T] f32; out A [B,Hv,T,C] f32.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_scaled_dot_kkt_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size,
+    const fla_tensor *out, uint64_t *workspace_size);
+int fla_chunk_scaled_dot_kkt(
+    const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size,
+    const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * solve_tri - replaces aclnnSolveTri (_aclnn_ctypes.py:1786-1800):
+ * out = (I + x)^-1 per C x C chunk block, x strictly lower triangular.
+ * layout "bnsd": x [B,H,T,C]; "bsnd": x [B,T,H,C]; bf16 in and out.
+ * ------------------------------------------------------------------------ */
+int fla_solve_tri_get_workspace_size(
+    const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    const char *layout, const fla_tensor *out, uint64_t *workspace_size);
+int fla_solve_tri(
+    const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    const char *layout, const fla_tensor *out, void *workspace, uint64_t workspace_size,
+    void *stream);
+
+/* ------------------------------------------------------------------------
+ * recompute_w_u_fwd - replaces aclnnRecomputeWUFwd (_aclnn_ctypes.py:618-651).
+ * k [B,Hk,T,K], v [B,Hv,T,V] bf16; beta, g [B,Hv,T] f32; A [B,Hv,T,C] bf16;
+ * gk must be NULL.  Outputs w [B,Hv,T,K], u [B,Hv,T,V] bf16.
+ * ------------------------------------------------------------------------ */
+int fla_recompute_w_u_fwd_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+    const fla_tensor *g, const fla_tensor *gk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *w,
+    const fla_tensor *u, uint64_t *workspace_size);
+int fla_recompute_w_u_fwd(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+    const fla_tensor *g, const fla_tensor *gk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *w,
+    const fla_tensor *u, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * chunk_gated_delta_rule_fwd_h - replaces aclnnChunkGatedDeltaRuleFwdH
+ * (_aclnn_ctypes.py:552-615).  k [B,Hk,T,K], w [B,Hv,T,K], u [B,Hv,T,V] bf16;
+ * g [B,Hv,T] f32 (chunk-cumsummed); gk must be NULL; initial_state
+ * [N,Hv,K,V] f32 or NULL.  Outputs h [B,Hv,NT,K,V] bf16 (state at chunk
+ * start), v_new [B,Hv,T,V] bf16, final_state [N,Hv,K,V] f32 (NULL unless
+ * output_final_state).
+ * ------------------------------------------------------------------------ */
+int fla_chunk_gated_delta_rule_fwd_h_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g,
+    const fla_tensor *gk, const fla_tensor *initial_state, bool output_final_state,
+    int64_t chunk_size, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *final_state, uint64_t *workspace_size);
+int fla_chunk_gated_delta_rule_fwd_h(
+    const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g,
+    const fla_tensor *gk, const fla_tensor *initial_state, bool output_final_state,
+    int64_t chunk_size, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * chunk_fwd_o - replaces aclnnChunkFwdO (_aclnn_ctypes.py:517-549).
+ * q,k [B,Hk,T,K], v (= v_new) [B,Hv,T,V], h [B,Hv,NT,K,V] bf16; g [B,Hv,T] f32.
+ * Output o [B,Hv,T,V] bf16.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_fwd_o_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
+    const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    double scale, int64_t chunk_size, const fla_tensor *out, uint64_t *workspace_size);
+int fla_chunk_fwd_o(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
+    const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    double scale, int64_t chunk_size, const fla_tensor *out, void *workspace,
+    uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * gdn_chunk_fwd - the whole chunk forward in one call.  Replaces the Python
+ * composition flash_chunk_gated_delta_rule_fwd
+ * (examples/flash_gated_delta_rule.py:796-881), which issues the six ops
+ * above plus transposes.  q,k [B,Hk,T,K], v [B,Hv,T,V] bf16 (any strides with
+ * unit innermost stride); g (raw per-token log gate), beta [B,T,Hv] f32 as the
+ * pipeline passes them; initial_state [N,Hv,K,V] f32 or NULL.
+ * Outputs: o [B,T,Hv,V] bf16, g_cumsum [B,T,Hv] f32 (may be NULL),
+ * final_state [N,Hv,K,V] f32 (NULL unless output_final_state).
+ * ------------------------------------------------------------------------ */
+int fla_gdn_chunk_fwd_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, double scale, const fla_tensor *initial_state,
+    bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
+    const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
+    uint64_t *workspace_size);
+int fla_gdn_chunk_fwd(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, double scale, const fla_tensor *initial_state,
+    bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
+    const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
+    void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * recurrent_gated_delta_rule - replaces aclnnRecurrentGatedDeltaRule
+ * (recurrent_gated_delta_rule/README.md:46-70; _aclnn_ctypes.py:654-846).
+ * query,key [T,Nk,Dk], value [T,Nv,Dv], beta [T,Nv] bf16; state
+ * [Block,Nv,Dv,Dk] f32 or bf16, updated in place, may be strided over the
+ * first two dims; actual_seq_lengths [B+1] i32 and ssm_state_indices [T] i32
+ * are DEVICE tensors; g [T,Nv] f32, gk [T,Nv,Dk] f32, num_accepted_tokens
+ * [B] i32 optional.  out [T,Nv,Dv] bf16.
+ * ------------------------------------------------------------------------ */
+int fla_recurrent_gated_delta_rule_get_workspace_size(
+    const fla_tensor *query, const fla_tensor *key, const fla_tensor *value,
+    const fla_tensor *beta, const fla_tensor *state, const fla_tensor *actual_seq_lengths,
+    const fla_tensor *ssm_state_indices, const fla_tensor *g, const fla_tensor *gk,
+    const fla_tensor *num_accepted_tokens, float scale, const fla_tensor *out,
+    uint64_t *workspace_size);
+int fla_recurrent_gated_delta_rule(
+    const fla_tensor *query, const fla_tensor *key, const fla_tensor *value,
+    const fla_tensor *beta, const fla_tensor *state, const fla_tensor *actual_seq_lengths,
+    const fla_tensor *ssm_state_indices, const fla_tensor *g, const fla_tensor *gk,
+    const fla_tensor *num_accepted_tokens, float scale, const fla_tensor *out,
+    void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * causal_conv1d - replaces aclnnCausalConv1d (docs/aclnnCausalConv1d.md:31-48;
+ * _aclnn_ctypes.py:951-985).  x [B,S,D] or [T,D] bf16/f16; weight [W,D];
+ * bias [D] optional; conv_states [N,>=W-1,D] optional, updated in place.
+ * run_mode 0 (prefill) only.  out like x, or [B,head_num,S,D/head_num].
+ * ------------------------------------------------------------------------ */
+int fla_causal_conv1d_get_workspace_size(
+    const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias,
+    const fla_tensor *conv_states, const fla_int_array *query_start_loc,
+    const fla_int_array *cache_indices, const fla_int_array *initial_state_mode,
+    const fla_int_array *num_accepted_tokens, int64_t activation_mode, int64_t pad_slot_id,
+    int64_t run_mode, int64_t head_num, const fla_tensor *out, uint64_t *workspace_size);
+int fla_causal_conv1d(
+    const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias,
+    const fla_tensor *conv_states, const fla_int_array *query_start_loc,
+    const fla_int_array *cache_indices, const fla_int_array *initial_state_mode,
+    const fla_int_array *num_accepted_tokens, int64_t activation_mode, int64_t pad_slot_id,
+    int64_t run_mode, int64_t head_num, const fla_tensor *out, void *workspace,
+    uint64_t workspace_size, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLA_HIP_H_ */

@@ -1,0 +1,136 @@
+"""Parity of the HIP recurrent_gated_delta_rule (through the C ABI) against the CPU oracle.
+
+Shapes follow fla/ops/ascendc/gdn/recurrent_gdn/recurrent_gated_delta_rule/tests/pta
+(T=2..., K=V=128) plus the decode benchmark layout; tolerance: bf16 out 2e-2, fp32 state 1e-3."""
+import pytest
+import torch
+
+from oracle import decode as od
+from util import assert_close, TOL_BF16, TOL_STATE
+
+pytestmark = pytest.mark.gpu
+F = torch.nn.functional
+
+
+def make_inputs(lens, Nk, Nv, Dk, Dv, *, seed=0, skip=0, blocks=None, state_dtype=torch.float32, gk=False, g=True):
+    gen = torch.Generator().manual_seed(seed)
+    T = skip + sum(lens)
+    q = F.normalize(torch.randn(T, Nk, Dk, generator=gen), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(T, Nk, Dk, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(T, Nv, Dv, generator=gen).bfloat16()
+    beta = torch.sigmoid(torch.randn(T, Nv, generator=gen)).bfloat16()
+    gate = F.logsigmoid(torch.randn(T, Nv, generator=gen)) if g else None
+    gkk = F.logsigmoid(torch.randn(T, Nv, Dk, generator=gen)) * 0.1 if gk else None
+    blocks = blocks or T
+    state = (torch.randn(blocks, Nv, Dv, Dk, generator=gen) * 0.01).to(state_dtype)
+    seq = torch.tensor([skip] + list(lens), dtype=torch.int32)
+    idx = torch.randperm(blocks, generator=gen)[:T].to(torch.int32)
+    return dict(q=q, k=k, v=v, beta=beta, g=gate, gk=gkk, state=state, lens=seq, idx=idx, scale=Dk ** -0.5)
+
+
+def run(dev, d, accepted=None, idx=None):
+    from fla_hip import ops
+    idx = d["idx"] if idx is None else idx
+    o_ref, s_ref = od.recurrent_gated_delta_rule(
+        d["q"], d["k"], d["v"], d["state"], beta=d["beta"], scale=d["scale"], actual_seq_lengths=d["lens"],
+        ssm_state_indices=idx, num_accepted_tokens=accepted, g=d["g"], gk=d["gk"])
+    st = d["state"].to(dev)
+    to = lambda t: None if t is None else t.to(dev)
+    o = ops.recurrent_gated_delta_rule(
+        to(d["q"]), to(d["k"]), to(d["v"]), st, beta=to(d["beta"]), scale=d["scale"],
+        actual_seq_lengths=to(d["lens"]), ssm_state_indices=to(idx), num_accepted_tokens=to(accepted),
+        g=to(d["g"]), gk=to(d["gk"]))
+    return o, o_ref, st, s_ref
+
+
+@pytest.mark.parametrize("dims", [(128, 128), (64, 64), (128, 256), (64, 128)])
+def test_single_token_decode(dev, dims):
+    Dk, Dv = dims
+    d = make_inputs([1] * 6, 2, 4, Dk, Dv, seed=1)   # GVA: Nv = 2 * Nk; K != V cases check the V-first layout
+    o, o_ref, st, s_ref = run(dev, d)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref, TOL_STATE, "state")
+
+
+def test_multi_token_and_skip_prefix(dev):
+    d = make_inputs([3, 8, 1, 0, 5], 2, 2, 128, 128, seed=2, skip=2, blocks=40)
+    o, o_ref, st, s_ref = run(dev, d)
+    # skipped leading tokens are not produced by the op: compare from the prefix on
+    assert_close(o[2:], o_ref[2:], TOL_BF16, "out")
+    assert_close(st, s_ref, TOL_STATE, "state")
+
+
+def test_accepted_tokens_select_source_slot(dev):
+    d = make_inputs([4, 4], 1, 2, 128, 128, seed=3, blocks=16)
+    acc = torch.tensor([2, 4], dtype=torch.int32)
+    o, o_ref, st, s_ref = run(dev, d, accepted=acc)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref, TOL_STATE, "state")
+
+
+def test_gk_only_and_both_gates(dev):
+    for g, gk in ((False, True), (True, True)):
+        d = make_inputs([2, 3], 2, 2, 128, 128, seed=4, g=g, gk=gk)
+        o, o_ref, st, s_ref = run(dev, d)
+        assert_close(o, o_ref, TOL_BF16, "out")
+        assert_close(st, s_ref, TOL_STATE, "state")
+
+
+def test_bf16_state(dev):
+    d = make_inputs([1, 2, 1], 2, 2, 128, 128, seed=5, state_dtype=torch.bfloat16)
+    o, o_ref, st, s_ref = run(dev, d)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref.bfloat16(), TOL_BF16, "state")
+
+
+def test_long_sequence_same_slot(dev):
+    """Prefill through the recurrent kernel: 300 tokens, every token mapped to one slot
+    (beyond the reference op's 8-token limit; oracle = the same recurrence)."""
+    d = make_inputs([300, 70], 1, 2, 128, 128, seed=6, blocks=4)
+    idx = torch.cat([torch.full((300,), 2), torch.full((70,), 0)]).to(torch.int32)
+    o, o_ref, st, s_ref = run(dev, d, idx=idx)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref, TOL_STATE, "state")
+
+
+def test_strided_state_pool(dev):
+    from fla_hip import ops
+    d = make_inputs([1, 1, 1], 2, 2, 128, 128, seed=7, blocks=3)
+    pool = torch.zeros(3, 4, 128, 128)
+    pool[:, ::2] = d["state"]
+    o_ref, s_ref = od.recurrent_gated_delta_rule(
+        d["q"], d["k"], d["v"], d["state"], beta=d["beta"], scale=d["scale"], actual_seq_lengths=d["lens"],
+        ssm_state_indices=d["idx"], g=d["g"])
+    pool_d = pool.to(dev)
+    o = ops.recurrent_gated_delta_rule(
+        d["q"].to(dev), d["k"].to(dev), d["v"].to(dev), pool_d[:, ::2], beta=d["beta"].to(dev), scale=d["scale"],
+        actual_seq_lengths=d["lens"].to(dev), ssm_state_indices=d["idx"].to(dev), g=d["g"].to(dev))
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(pool_d[:, ::2], s_ref, TOL_STATE, "state")
+    assert float(pool_d[:, 1::2].abs().max()) == 0.0
+
+
+def test_decode_benchmark_shape_properties(dev):
+    """256 sequences x 1 token, 32 heads, K=V=128: oracle on a subset of sequences."""
+    from fla_hip import ops
+    d = make_inputs([1] * 256, 32, 32, 128, 128, seed=0, blocks=256)
+    d["idx"] = torch.arange(256, dtype=torch.int32)
+    st = d["state"].to(dev)
+    to = lambda t: t.to(dev)
+    o = ops.recurrent_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), st, beta=to(d["beta"]), scale=d["scale"],
+                                       actual_seq_lengths=to(d["lens"]), ssm_state_indices=to(d["idx"]), g=to(d["g"]))
+    sub = [0, 17, 255]
+    for t in sub:
+        o_ref, s_ref = od.recurrent_gated_delta_rule(
+            d["q"][t:t + 1], d["k"][t:t + 1], d["v"][t:t + 1], d["state"][t:t + 1], beta=d["beta"][t:t + 1],
+            scale=d["scale"], actual_seq_lengths=torch.tensor([0, 1], dtype=torch.int32),
+            ssm_state_indices=torch.zeros(1, dtype=torch.int32), g=d["g"][t:t + 1])
+        assert_close(o[t:t + 1], o_ref, TOL_BF16, "out")
+        assert_close(st[t:t + 1], s_ref, TOL_STATE, "state")
+
+
+def test_wrapper_errors(dev):
+    from fla_hip import ops
+    with pytest.raises(RuntimeError, match=r"^npu_recurrent_gated_delta_rule: either g or gk must be provided\.$"):
+        ops.npu_recurrent_gated_delta_rule(None, None, None, None, beta=None, actual_seq_lengths=None,
+                                           ssm_state_indices=None)
