@@ -1,0 +1,556 @@
+// Chunk-parallel stages of the gated-delta-rule forward, one workgroup per
+// (chunk, value head, batch row), bf16 MFMA with fp32 accumulation:
+//   chunk_scaled_dot_kkt   A0 = strict_lower(beta_i e^{clip(G_i-G_j)} <k_i,k_j>)
+//   solve_tri              (I + A0)^-1 by fp32 forward substitution
+//   recompute_w_u_fwd      w = Ainv (k beta e^G), u = Ainv (v beta)
+//   chunk_fwd_o            o = scale (e^G (q h) + tril(q k^T e^{min(G_i-G_j,0)}) v_new)
+// Stage math and rounding points: chunk_scaled_dot_kkt/README.md:11-29,
+// solve_tri/README.md:7-19, recompute_w_u_fwd/README.md:12-32,
+// chunk_fwd_o/README.md:6-15 (+ qkmask epilogue, op_kernel/.../block_epilogue_gdn_fwdo_qkmask.hpp:210-262).
+#include "gdn_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+// =============================================================================
+// chunk_scaled_dot_kkt
+// =============================================================================
+struct KktParams {
+    ChunkGeom geom;
+    View4 k;
+    View3 g, beta;
+    float *out;
+    int64_t o_sb, o_sh, o_st;
+};
+
+__global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int K = p.geom.K, pitch = K + 8;
+    bf16 *kS = reinterpret_cast<bf16 *>(smem);
+    float *gS = reinterpret_cast<float *>(kS + kChunk * pitch);
+    float *bS = gS + kChunk;
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    load_tile<kThreads>(kS, pitch, kg, p.k.st, kChunk, K, len);
+    if (threadIdx.x < kChunk) {
+        const int t = threadIdx.x;
+        gS[t] = t < len ? load_scalar(p.g, b, hv, start + t) : 0.f;
+        bS[t] = t < len ? load_scalar(p.beta, b, hv, start + t) : 0.f;
+    }
+    __syncthreads();
+
+    const int I = wave_id();  // t block owned by this wave
+    const int t = I * 16 + acc_col();
+    float *orow = p.out + b * p.o_sb + hv * p.o_sh + (int64_t)(start + t) * p.o_st;
+    const float gt = gS[t], bt = bS[t];
+    for (int J = 0; J < 4; ++J) {  // s block
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (J <= I) {
+            for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pitch, J * 16, kk), frag_kc(kS, pitch, I * 16, kk), acc);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int s = J * 16 + acc_row(e);
+                const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
+                acc[e] = (s < t && t < len) ? bt * __expf(d) * acc[e] : 0.f;
+            }
+        }
+        if (t < len) *reinterpret_cast<f32x4 *>(orow + J * 16 + 4 * (lane_id() >> 4)) = acc;
+    }
+}
+
+// =============================================================================
+// solve_tri: one wave per 64x64 block, lane j owns column j of the inverse.
+// =============================================================================
+struct SolveParams {
+    ChunkGeom geom;  // Hv = heads of x
+    const bf16 *x;
+    bf16 *out;
+    int64_t sb, sh, st;  // strides of (batch, head, token) in x and out
+};
+
+__global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
+    __shared__ __align__(16) float A[kChunk][kChunk];
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
+    const int lane = threadIdx.x;
+    for (int idx = lane; idx < kChunk * 8; idx += 64) {
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        bf16x8 v;
+        if (r < len) v = *reinterpret_cast<const bf16x8 *>(p.x + base + (int64_t)r * p.st + c8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) A[r][c8 + e] = (r < len && c8 + e < r) ? (float)v[e] : 0.f;
+    }
+    __syncthreads();
+
+    float x[kChunk];
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) x[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) {
+        float acc = (i == lane) ? 1.f : 0.f;
+#pragma unroll
+        for (int s4 = 0; s4 < (i + 3) / 4; ++s4) {
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(&A[i][4 * s4]);  // same address in every lane
+            acc -= a[0] * x[4 * s4] + a[1] * x[4 * s4 + 1] + a[2] * x[4 * s4 + 2] + a[3] * x[4 * s4 + 3];
+        }
+        x[i] = acc;
+    }
+    __syncthreads();
+    bf16 *O = reinterpret_cast<bf16 *>(&A[0][0]);  // [64][72] bf16 staging, fits in the fp32 tile
+#pragma unroll
+    for (int i = 0; i < kChunk; ++i) O[i * 72 + lane] = (bf16)x[i];
+    __syncthreads();
+    for (int idx = lane; idx < len * 8; idx += 64) {
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(O + r * 72 + c8);
+    }
+}
+
+// =============================================================================
+// recompute_w_u_fwd
+// =============================================================================
+struct WuParams {
+    ChunkGeom geom;
+    View4 k, v, A, w, u;
+    View3 g, beta;
+};
+
+__global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int K = p.geom.K, V = p.geom.V;
+    const int pa = kChunk + 8, pk = K + 16, pv = V + 16;
+    bf16 *aS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = aS + kChunk * pa;
+    bf16 *vS = kS + kChunk * pk;
+    float *gS = reinterpret_cast<float *>(vS + kChunk * pv);
+    float *bS = gS + kChunk;
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    if (threadIdx.x < kChunk) {
+        const int t = threadIdx.x;
+        gS[t] = t < len ? __expf(load_scalar(p.g, b, hv, start + t)) : 0.f;
+        bS[t] = t < len ? load_scalar(p.beta, b, hv, start + t) : 0.f;
+    }
+    const bf16 *ag = static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
+    for (int idx = threadIdx.x; idx < kChunk * 8; idx += kThreads) {
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        bf16x8 a;
+        if (r < len) a = *reinterpret_cast<const bf16x8 *>(ag + (int64_t)r * p.A.st + c8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (!(r < len && c8 + e < len)) a[e] = (bf16)0.f;  // columns past the tail are not part of the block
+        *reinterpret_cast<bf16x8 *>(aS + r * pa + c8) = a;
+    }
+    __syncthreads();  // gS, bS visible
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    for (int idx = threadIdx.x; idx < kChunk * (K >> 3); idx += kThreads) {
+        const int r = idx / (K >> 3), c8 = (idx % (K >> 3)) << 3;
+        bf16x8 o;
+        if (r < len) {
+            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(kg + (int64_t)r * p.k.st + c8);
+            const float s = bS[r] * gS[r];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)a[e] * s);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
+        }
+        *reinterpret_cast<bf16x8 *>(kS + r * pk + c8) = o;
+    }
+    for (int idx = threadIdx.x; idx < kChunk * (V >> 3); idx += kThreads) {
+        const int r = idx / (V >> 3), c8 = (idx % (V >> 3)) << 3;
+        bf16x8 o;
+        if (r < len) {
+            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(vg + (int64_t)r * p.v.st + c8);
+            const float s = bS[r];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)a[e] * s);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
+        }
+        *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = o;
+    }
+    __syncthreads();
+
+    // Each wave owns a quarter of the output columns of w and of u and overwrites
+    // exactly those columns of the staged operand once its products are done.
+    const int w = wave_id();
+    auto product = [&](bf16 *tile, int pitch, int ncols) {
+        const int per_wave = ncols / 64;  // 16-column tiles per wave
+        for (int m = 0; m < per_wave; ++m) {
+            const int c0 = (w * per_wave + m) * 16;
+            f32x4 acc[4];
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16x8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);
+            }
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(tile, pitch, rt * 16, c0, acc[rt]);
+        }
+    };
+    product(kS, pk, K);
+    product(vS, pv, V);
+    __syncthreads();
+    bf16 *wg = static_cast<bf16 *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
+    bf16 *ug = static_cast<bf16 *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
+    store_tile<kThreads>(wg, p.w.st, kS, pk, K, len);
+    store_tile<kThreads>(ug, p.u.st, vS, pv, V, len);
+}
+
+// =============================================================================
+// chunk_fwd_o
+// =============================================================================
+struct FwdOParams {
+    ChunkGeom geom;
+    View4 q, k, v, o;
+    const bf16 *h;
+    int64_t h_sb, h_sh, h_sc;  // h [B,Hv,NT,K,V]: batch, head, chunk strides (K,V contiguous)
+    View3 g;
+    float scale;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pq = K + 8, pv = V + 16, pp = kChunk + 8;
+    constexpr int CT = V / 64;  // 16-column tiles per wave
+    bf16 *qS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = qS + kChunk * pq;
+    bf16 *vS = kS + kChunk * pq;
+    bf16 *hS = vS + kChunk * pv;
+    bf16 *pS = hS + K * pv;
+    float *gS = reinterpret_cast<float *>(pS + kChunk * pp);
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
+    load_tile<kThreads>(qS, pq, qg, p.q.st, kChunk, K, len);
+    load_tile<kThreads>(kS, pq, kg, p.k.st, kChunk, K, len);
+    load_tile<kThreads>(vS, pv, vg, p.v.st, kChunk, V, len);
+    load_tile<kThreads>(hS, pv, hg, V, K, V, K);
+    if (threadIdx.x < kChunk) gS[threadIdx.x] = threadIdx.x < len ? load_scalar(p.g, b, hv, start + threadIdx.x) : 0.f;
+    __syncthreads();
+
+    const int w = wave_id();
+    // masked, decayed scores P[t][s] (computed as the transposed tile so that a lane
+    // holds four consecutive s of one row t)
+    for (int m = 0; m < 4; ++m) {
+        const int id = w + 4 * m, I = id >> 2, J = id & 3;  // t block, s block
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const int t = I * 16 + acc_col();
+        if (J <= I) {
+#pragma unroll
+            for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pq, J * 16, kk), frag_kc(qS, pq, I * 16, kk), acc);
+            const float gt = gS[t];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int s = J * 16 + acc_row(e);
+                acc[e] = (s <= t) ? acc[e] * __expf(fminf(gt - gS[s], 0.f)) : 0.f;
+            }
+        }
+        *reinterpret_cast<bf16x4 *>(pS + t * pp + J * 16 + 4 * (lane_id() >> 4)) = cvt4(acc);
+    }
+
+    // inter-chunk term e^{G_t} (q h) for this wave's V columns
+    f32x4 acc[4][CT];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < K / 32; ++j) {
+        bf16x8 bfrag[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(hS, pv, (w * CT + ct) * 16, 32 * j);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const bf16x8 afrag = frag_kc(qS, pq, rt * 16, 32 * j);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float eg = __expf(gS[rt * 16 + acc_row(e)]);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[rt][ct][e] *= eg;
+        }
+    __syncthreads();  // P complete
+
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        bf16x8 bfrag[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(vS, pv, (w * CT + ct) * 16, 32 * j);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const bf16x8 afrag = frag_kc(pS, pp, rt * 16, 32 * j);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+        }
+    }
+    // this wave's columns of the v tile are no longer needed: stage o there
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc_to_tile(vS, pv, rt * 16, (w * CT + ct) * 16, acc[rt][ct] * p.scale);
+    __syncthreads();
+    bf16 *og = static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)start * p.o.st;
+    store_tile<kThreads>(og, p.o.st, vS, pv, V, len);
+}
+
+// ---- host side ------------------------------------------------------------------
+int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query) {
+    int rc = build_varlen(vl, op, cu, ci, kChunk, geom.T);
+    if (rc) return rc;
+    FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
+    if (vl.enabled) {
+        geom.NT = vl.NT;
+        geom.N = vl.N;
+    }
+    if (query) {
+        *query = vl.bytes();
+        return FLA_OK;
+    }
+    FLA_REQUIRE(vl.bytes() == 0 || (workspace && workspace_size >= vl.bytes()), FLA_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes required.", op, vl.bytes());
+    if ((rc = upload_varlen(vl, workspace, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    return FLA_OK;
+}
+
+int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, const fla_int_array *cu,
+             const fla_int_array *ci, int64_t chunk_size, const fla_tensor *out, void *ws, uint64_t ws_size,
+             hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_scaled_dot_kkt";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_tensor(out, op, "out", 4, dt_bit(FLA_F32)))) return rc;
+    FLA_REQUIRE(out->shape[0] == geom.B && out->shape[1] == geom.Hv && out->shape[2] == geom.T && out->shape[3] == kChunk &&
+                    inner_unit(out) && out->stride[2] % 4 == 0 && out->stride[1] % 4 == 0 && out->stride[0] % 4 == 0,
+                FLA_ERR_SHAPE, "%s: out must be a 16-byte aligned [B,Hv,T,%d].", op, kChunk);
+    FLA_REQUIRE(geom.K % 32 == 0 && geom.K >= 32 && geom.K <= 256, FLA_ERR_UNSUPPORTED,
+                "%s: K must be a multiple of 32 in [32,256], got %d.", op, geom.K);
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    KktParams p{geom, view4(k), view3(g), view3(beta), static_cast<float *>(out->data), out->stride[0], out->stride[1],
+                out->stride[2]};
+    const size_t smem = (size_t)kChunk * (geom.K + 8) * 2 + 2 * kChunk * 4;
+    hipLaunchKernelGGL(kkt_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array *ci, const char *layout,
+               const fla_tensor *out, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "solve_tri";
+    int rc;
+    if ((rc = check_tensor(x, op, "x", -1, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_tensor(out, op, "out", -1, dt_bit(FLA_BF16)))) return rc;
+    FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
+    FLA_REQUIRE(same_shape(x, out), FLA_ERR_SHAPE, "%s: out must have the shape of x.", op);
+    FLA_REQUIRE(is_contiguous(x) && is_contiguous(out), FLA_ERR_SHAPE, "%s: x and out must be contiguous.", op);
+    int ib, ih, it;  // dims of batch, head, token (-1: absent)
+    char lay[8] = {0};
+    for (int i = 0; i < 7 && layout[i]; ++i) lay[i] = (char)tolower(layout[i]);
+    if (!strcmp(lay, "bnsd")) { ib = 0; ih = 1; it = 2; }
+    else if (!strcmp(lay, "bsnd")) { ib = 0; it = 1; ih = 2; }
+    else if (!strcmp(lay, "tnd")) { ib = -1; it = 0; ih = 1; }
+    else if (!strcmp(lay, "ntd")) { ib = -1; ih = 0; it = 1; }
+    else return fail(FLA_ERR_UNSUPPORTED, "%s: unknown layout '%s' (bsnd, bnsd, tnd, ntd).", op, layout);
+    FLA_REQUIRE(x->ndim == (ib < 0 ? 3 : 4), FLA_ERR_SHAPE, "%s: rank does not match layout '%s'.", op, layout);
+    FLA_REQUIRE(x->shape[x->ndim - 1] == kChunk, FLA_ERR_UNSUPPORTED, "%s: block size must be %d, got %lld.", op, kChunk,
+                (long long)x->shape[x->ndim - 1]);
+    ChunkGeom geom{};
+    geom.B = ib < 0 ? 1 : (int)x->shape[ib];
+    geom.Hv = geom.Hk = (int)x->shape[ih];
+    geom.T = (int)x->shape[it];
+    FLA_REQUIRE(x->shape[it] < ((int64_t)1 << 31) && x->shape[ih] < 65536 && geom.B < 65536, FLA_ERR_SHAPE,
+                "%s: extents too large.", op);
+    geom.NT = (geom.T + kChunk - 1) / kChunk;
+    geom.N = geom.B;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0 || geom.Hv == 0) return FLA_OK;
+    SolveParams p{geom, static_cast<const bf16 *>(x->data), static_cast<bf16 *>(out->data), ib < 0 ? 0 : x->stride[ib],
+                  x->stride[ih], x->stride[it]};
+    hipLaunchKernelGGL(solve_tri_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(64), 0, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *g,
+            const fla_tensor *gk, const fla_int_array *cu, const fla_int_array *ci, int64_t chunk_size,
+            const fla_tensor *w, const fla_tensor *u, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "recompute_w_u_fwd";
+    FLA_REQUIRE(gk == nullptr || gk->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: gk must be None.", op);
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    FLA_REQUIRE(geom.K % 64 == 0 && geom.V % 64 == 0 && geom.K <= 256 && geom.V <= 256, FLA_ERR_UNSUPPORTED,
+                "%s: K and V must be multiples of 64 up to 256, got K=%d V=%d.", op, geom.K, geom.V);
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    WuParams p{geom, view4(k), view4(v), view4(A), view4(w), view4(u), view3(g), view3(beta)};
+    const size_t smem = (size_t)kChunk * ((kChunk + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(wu_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)smem));
+    hipLaunchKernelGGL(wu_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+template <int K, int V>
+int launch_fwd_o(const FwdOParams &p, hipStream_t stream) {
+    const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + kChunk * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL((fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h, const fla_tensor *g,
+               const fla_int_array *cu, const fla_int_array *ci, double scale, int64_t chunk_size, const fla_tensor *out,
+               void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_fwd_o";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "out", out, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
+    if ((rc = check_tensor(h, op, "h", 5, bf))) return rc;
+    FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
+                    h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 8 == 0 &&
+                    h->stride[1] % 8 == 0 && h->stride[0] % 8 == 0,
+                FLA_ERR_SHAPE, "%s: h must be [B,Hv,NT=%d,K,V] with contiguous K x V blocks.", op, geom.NT);
+    if (query) return FLA_OK;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    FwdOParams p{geom, view4(q), view4(k), view4(v), view4(out), static_cast<const bf16 *>(h->data),
+                 h->stride[0], h->stride[1], h->stride[2], view3(g), (float)scale};
+    if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128>(p, stream);
+    if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256>(p, stream);
+    if (geom.K == 64 && geom.V == 64) return launch_fwd_o<64, 64>(p, stream);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(128,256),(64,64).", op, geom.K,
+                geom.V);
+}
+
+}  // namespace
+}  // namespace fla
+
+#define FLA_NULL_WS(op) \
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, op ": workspace_size must not be null.")
+
+extern "C" int fla_chunk_scaled_dot_kkt_get_workspace_size(const fla_tensor *k, const fla_tensor *g,
+                                                           const fla_tensor *beta, const fla_int_array *cu_seqlens,
+                                                           const fla_int_array *chunk_indices, int64_t chunk_size,
+                                                           const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_NULL_WS("chunk_scaled_dot_kkt");
+    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size);
+}
+extern "C" int fla_chunk_scaled_dot_kkt(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+                                        const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                                        int64_t chunk_size, const fla_tensor *out, void *workspace,
+                                        uint64_t workspace_size, void *stream) {
+    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_solve_tri_get_workspace_size(const fla_tensor *x, const fla_int_array *cu_seqlens,
+                                                const fla_int_array *chunk_indices, const char *layout,
+                                                const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_NULL_WS("solve_tri");
+    return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, nullptr, 0, nullptr, workspace_size);
+}
+extern "C" int fla_solve_tri(const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                             const char *layout, const fla_tensor *out, void *workspace, uint64_t workspace_size,
+                             void *stream) {
+    return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_recompute_w_u_fwd_get_workspace_size(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
+                                                        const fla_tensor *A, const fla_tensor *g, const fla_tensor *gk,
+                                                        const fla_int_array *cu_seqlens,
+                                                        const fla_int_array *chunk_indices, int64_t chunk_size,
+                                                        const fla_tensor *w, const fla_tensor *u,
+                                                        uint64_t *workspace_size) {
+    FLA_NULL_WS("recompute_w_u_fwd");
+    return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, nullptr, 0, nullptr,
+                        workspace_size);
+}
+extern "C" int fla_recompute_w_u_fwd(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
+                                     const fla_tensor *A, const fla_tensor *g, const fla_tensor *gk,
+                                     const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                                     int64_t chunk_size, const fla_tensor *w, const fla_tensor *u, void *workspace,
+                                     uint64_t workspace_size, void *stream) {
+    return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size,
+                        static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_chunk_fwd_o_get_workspace_size(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
+                                                  const fla_tensor *h, const fla_tensor *g,
+                                                  const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                                                  double scale, int64_t chunk_size, const fla_tensor *out,
+                                                  uint64_t *workspace_size) {
+    FLA_NULL_WS("chunk_fwd_o");
+    return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0, nullptr,
+                           workspace_size);
+}
+extern "C" int fla_chunk_fwd_o(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
+                               const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                               double scale, int64_t chunk_size, const fla_tensor *out, void *workspace,
+                               uint64_t workspace_size, void *stream) {
+    return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr);
+}

@@ -1,0 +1,66 @@
+// Geometry shared by the chunked gated-delta-rule kernels: how a launch maps to
+// (batch row, sequence, chunk) for dense and packed variable-length inputs.
+#pragma once
+
+#include "common.h"
+#include "device_utils.h"
+
+namespace fla {
+
+constexpr int kChunk = 64;  // tokens per chunk of every MFMA kernel
+
+struct ChunkGeom {
+    int B, T;            // batch rows, tokens per row (packed total when varlen)
+    int Hk, Hv;          // key / value heads (Hv % Hk == 0)
+    int K, V;
+    int NT;              // chunks per batch row (varlen: over all sequences)
+    int N;               // sequences
+    const int32_t *cu;   // [N+1] or null (dense)
+    const int32_t *choff;  // [N+1] first chunk of each sequence
+    const int32_t *tab;  // [NT][2] (sequence, chunk within sequence)
+};
+
+// Head-first activations [B, H, T, D] with arbitrary outer strides and unit inner stride.
+struct View4 {
+    const void *p;
+    int64_t sb, sh, st;
+};
+// Per-token scalars [B, H, T] (or [B, T, H]) through strides; f32 or bf16.
+struct View3 {
+    const void *p;
+    int64_t sb, sh, st;
+    int is_bf16;
+};
+
+__device__ __forceinline__ float load_scalar(const View3 &v, int b, int h, int t) {
+    const int64_t off = b * v.sb + h * v.sh + (int64_t)t * v.st;
+    return v.is_bf16 ? (float)static_cast<const bf16 *>(v.p)[off] : static_cast<const float *>(v.p)[off];
+}
+
+// Chunk `c` of batch row `b` -> first token and length.
+__device__ __forceinline__ void chunk_span(const ChunkGeom &g, int b, int c, int &seq, int &start, int &len) {
+    if (g.cu == nullptr) {
+        seq = b;
+        start = c * kChunk;
+        len = min(kChunk, g.T - start);
+    } else {
+        seq = g.tab[2 * c];
+        start = g.cu[seq] + g.tab[2 * c + 1] * kChunk;
+        len = min(kChunk, g.cu[seq + 1] - start);
+    }
+}
+
+inline View4 view4(const fla_tensor *t) { return View4{t->data, t->stride[0], t->stride[1], t->stride[2]}; }
+inline View3 view3(const fla_tensor *t) {
+    return View3{t->data, t->stride[0], t->stride[1], t->stride[2], t->dtype == FLA_BF16 ? 1 : 0};
+}
+
+// Common validation of the [B,H,T,D] / [B,H,T] operand family; fills geometry
+// (without varlen pointers).  `v` may be null when the op has no V-sized operand.
+int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, const fla_tensor *g_like,
+                 int64_t chunk_size, ChunkGeom &geom);
+int check_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, int64_t D,
+               int dtype_mask);
+int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T);
+
+}  // namespace fla

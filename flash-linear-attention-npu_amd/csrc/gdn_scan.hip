@@ -1,0 +1,304 @@
+// chunk_gated_delta_rule_fwd_h: the sequential inter-chunk state scan.
+//
+// One 256-thread workgroup per (sequence, value head, 64*CT-column slab of V)
+// walks the chunks of its sequence.  Wave w owns 16*CT columns of V for ALL K
+// rows of the state, so the fp32 state lives in accumulator registers for the
+// whole sequence and never touches LDS or HBM between chunks:
+//     wh     = w_i . h          (A = w tile in LDS, B = state registers as bf16)
+//     v_new  = u_i - wh
+//     h     <- e^{g_last} h + k_i^T . (v_new * e^{g_last - g})
+//              (A = k tile read with transposing LDS loads, B = v_new registers)
+// Per chunk the workgroup stages w, k and its u slab once; h (state at chunk
+// start) and v_new are emitted as bf16, the final state as fp32.
+// Stage math: chunk_gated_delta_rule_fwd_h/README.md:16-30,52-61; kernel
+// op_kernel/gemm/kernel/gdn_fwd_h_kernel.hpp:441-753.
+#include "gdn_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct ScanParams {
+    ChunkGeom geom;
+    View4 k, w, u, v_new;
+    View3 g;
+    const float *h0;     // [N,Hv,K,V] or [N,Hv,V,K] fp32, or null
+    float *hT;           // final state, same layout, or null
+    bf16 *h;             // [B,Hv,NT,K,V] (or V,K) bf16, or null
+    int64_t h_sb, h_sh, h_sc;
+    int64_t s_sn, s_sh;  // strides of h0 / hT over (sequence, head)
+    int v_first;         // state blocks are [V][K] instead of [K][V]
+};
+
+template <int K, int CT>
+__global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int VS = 64 * CT;           // V columns of this workgroup
+    constexpr int pw = K + 8, pk = K + 16, pu = VS + 16;
+    constexpr int KT = K / 16, KS = K / 32;
+    bf16 *wS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = wS + kChunk * pw;
+    bf16 *uS = kS + kChunk * pk;
+    float *gS = reinterpret_cast<float *>(uS + kChunk * pu);
+
+    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+        chunk0 = p.geom.choff[n];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int wv = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int vcol0 = slab * VS + wv * 16 * CT;  // first V column of this wave
+
+    // state element (kk = 16*kt + 4*lg + e, v = vcol0 + 16*ct + li)
+    f32x4 hacc[KT][CT];
+    auto state_off = [&](int kk, int v) -> int64_t { return p.v_first ? (int64_t)v * K + kk : (int64_t)kk * V + v; };
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            if (p.h0) {
+                const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] = s[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)];
+            }
+            hacc[kt][ct] = a;
+        }
+
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const bf16 *ug = static_cast<const bf16 *>(p.u.p) + b * p.u.sb + hv * p.u.sh + slab * VS;
+    bf16 *vng = static_cast<bf16 *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + slab * VS;
+
+    for (int c = 0; c < nchunks; ++c) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        __syncthreads();  // previous chunk's tiles fully consumed
+        load_tile<kThreads>(wS, pw, wg + (int64_t)start * p.w.st, p.w.st, kChunk, K, len);
+        load_tile<kThreads>(kS, pk, kg + (int64_t)start * p.k.st, p.k.st, kChunk, K, len);
+        load_tile<kThreads>(uS, pu, ug + (int64_t)start * p.u.st, p.u.st, kChunk, VS, len);
+        if (threadIdx.x < kChunk) gS[threadIdx.x] = threadIdx.x < len ? load_scalar(p.g, b, hv, start + threadIdx.x) : 0.f;
+        __syncthreads();
+
+        // state at chunk start as a bf16 operand (and as the emitted h)
+        bf16x8 hB[KS][CT];
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
+        if (p.h) {
+            bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        hg[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)] = hB[kt >> 1][ct][(kt & 1) * 4 + e];
+        }
+
+        // v_new = u - w h   (rows = tokens, columns = this wave's V columns)
+        f32x4 vn[4][CT];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) vn[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                const bf16x8 afrag = frag_kc(wS, pw, rt * 16, 32 * j);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) vn[rt][ct] = mfma16x32(afrag, hB[j][ct], vn[rt][ct]);
+            }
+        const float g_last = gS[len - 1];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const bf16x4 uu = frag_tr4(uS, pu, (wv * CT + ct) * 16, rt * 16);  // u[16rt+4g+e][col]
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vn[rt][ct][e] = (float)uu[e] - vn[rt][ct][e];
+            }
+        // emit v_new through this wave's own columns of the u tile
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc_to_tile(uS, pu, rt * 16, (wv * CT + ct) * 16, vn[rt][ct]);
+
+        // h <- e^{g_last} h + k^T (v_new e^{g_last - g}); padded rows carry zeros
+        const float dec_all = __expf(g_last);
+        bf16x8 vB[2][CT];
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                f32x4 lo = vn[2 * j][ct], hi = vn[2 * j + 1][ct];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int t0 = 32 * j + 4 * lg + e, t1 = t0 + 16;
+                    lo[e] = t0 < len ? (float)(bf16)lo[e] * __expf(g_last - gS[t0]) : 0.f;
+                    hi[e] = t1 < len ? (float)(bf16)hi[e] * __expf(g_last - gS[t1]) : 0.f;
+                }
+                vB[j][ct] = frag_from_acc(lo, hi);
+            }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= dec_all;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const bf16x8 afrag = frag_tr(kS, pk, kt * 16, 32 * j);  // k^T: rows kk, contraction over tokens
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] = mfma16x32(afrag, vB[j][ct], hacc[kt][ct]);
+            }
+        __syncthreads();  // v_new tile complete
+        store_tile<kThreads>(vng + (int64_t)start * p.v_new.st, p.v_new.st, uS, pu, VS, len);
+    }
+
+    if (p.hT) {
+        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)] = hacc[kt][ct][e];
+    }
+}
+
+template <int K, int CT>
+int launch_fwd_h(const ScanParams &p, int slabs, hipStream_t stream) {
+    constexpr int VS = 64 * CT;
+    const size_t smem = ((size_t)kChunk * (K + 8) + (size_t)kChunk * (K + 16) + (size_t)kChunk * (VS + 16)) * 2 + kChunk * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_h_kernel<K, CT>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL((fwd_h_kernel<K, CT>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g, const fla_tensor *gk,
+               const fla_tensor *initial_state, bool output_final_state, int64_t chunk_size, const fla_int_array *cu,
+               const fla_int_array *ci, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
+               const fla_tensor *final_state, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_gated_delta_rule_fwd_h";
+    FLA_REQUIRE(gk == nullptr || gk->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: gk is not supported; pass g.", op);
+    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: either g or gk must be provided.", op);
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    Varlen vl;
+    if ((rc = build_varlen(vl, op, cu, ci, kChunk, geom.T))) return rc;
+    FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
+    if (vl.enabled) {
+        geom.NT = vl.NT;
+        geom.N = vl.N;
+    }
+    const int64_t d2 = state_v_first ? geom.V : geom.K, d3 = state_v_first ? geom.K : geom.V;
+    auto check_state = [&](const fla_tensor *s, const char *name) -> int {
+        int r = check_tensor(s, op, name, 4, dt_bit(FLA_F32));
+        if (r) return r;
+        FLA_REQUIRE(s->shape[0] == geom.N && s->shape[1] == geom.Hv && s->shape[2] == d2 && s->shape[3] == d3 &&
+                        s->stride[3] == 1 && s->stride[2] == d3,
+                    FLA_ERR_SHAPE, "%s: %s must be [N=%d,Hv,%lld,%lld] with contiguous blocks.", op, name, geom.N,
+                    (long long)d2, (long long)d3);
+        return FLA_OK;
+    };
+    const bool has_h0 = initial_state && initial_state->data;
+    if (has_h0 && (rc = check_state(initial_state, "initial_state"))) return rc;
+    if (output_final_state && (rc = check_state(final_state, "final_state"))) return rc;
+    if (has_h0 && output_final_state)
+        FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1],
+                    FLA_ERR_SHAPE, "%s: initial_state and final_state must share strides.", op);
+    const bool has_h = h && h->data;
+    if (has_h) {
+        if ((rc = check_tensor(h, op, "h", 5, bf))) return rc;
+        FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == d2 &&
+                        h->shape[4] == d3 && h->stride[4] == 1 && h->stride[3] == d3,
+                    FLA_ERR_SHAPE, "%s: h must be [B,Hv,NT=%d,%lld,%lld] with contiguous blocks.", op, geom.NT,
+                    (long long)d2, (long long)d3);
+    }
+    FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
+    FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
+    if (query) {
+        *query = vl.bytes();
+        return FLA_OK;
+    }
+    FLA_REQUIRE(vl.bytes() == 0 || (ws && ws_size >= vl.bytes()), FLA_ERR_WORKSPACE, "%s: workspace of %zu bytes required.",
+                op, vl.bytes());
+    if ((rc = upload_varlen(vl, ws, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    if (geom.N == 0 || geom.Hv == 0) return FLA_OK;
+
+    ScanParams p{};
+    p.geom = geom;
+    p.k = view4(k);
+    p.w = view4(w);
+    p.u = view4(u);
+    p.v_new = view4(v_new);
+    p.g = view3(g);
+    p.h0 = has_h0 ? static_cast<const float *>(initial_state->data) : nullptr;
+    p.hT = output_final_state ? static_cast<float *>(final_state->data) : nullptr;
+    const fla_tensor *sref = has_h0 ? initial_state : (output_final_state ? final_state : nullptr);
+    if (sref) {
+        p.s_sn = sref->stride[0];
+        p.s_sh = sref->stride[1];
+    }
+    p.h = has_h ? static_cast<bf16 *>(h->data) : nullptr;
+    if (has_h) {
+        p.h_sb = h->stride[0];
+        p.h_sh = h->stride[1];
+        p.h_sc = h->stride[2];
+    }
+    p.v_first = state_v_first ? 1 : 0;
+
+    // Two 16-column tiles per wave (128-column slabs) halve the LDS operand traffic per
+    // FLOP; fall back to 64-column slabs when that leaves compute units idle.
+    const int64_t chains = (int64_t)geom.N * geom.Hv;
+    const bool wide = geom.V % 128 == 0 && chains * (geom.V / 128) >= 2 * (int64_t)num_cus();
+    if (geom.K == 128) return wide ? launch_fwd_h<128, 2>(p, geom.V / 128, stream) : launch_fwd_h<128, 1>(p, geom.V / 64, stream);
+    return wide ? launch_fwd_h<64, 2>(p, geom.V / 128, stream) : launch_fwd_h<64, 1>(p, geom.V / 64, stream);
+}
+
+}  // namespace
+}  // namespace fla
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_h_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g, const fla_tensor *gk,
+    const fla_tensor *initial_state, bool output_final_state, int64_t chunk_size, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *final_state, uint64_t *workspace_size) {
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_fwd_h: workspace_size must not be null.");
+    return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
+                           state_v_first, h, v_new, final_state, nullptr, 0, nullptr, workspace_size);
+}
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_h(
+    const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g, const fla_tensor *gk,
+    const fla_tensor *initial_state, bool output_final_state, int64_t chunk_size, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
+                           state_v_first, h, v_new, final_state, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr);
+}

@@ -1,0 +1,100 @@
+// LDS-tile <-> MFMA-operand plumbing for the chunk kernels (gfx950).
+//
+// All matrix products use v_mfma_f32_16x16x32_bf16 with ONE fixed assignment of
+// the 32 contraction indices of a step to the 8 operand slots of a lane
+// ("split" mapping):
+//     lane l = 16*g + i,  slot e:   c(g,e) = 4*g + e          for e < 4
+//                                   c(g,e) = 16 + 4*g + e - 4  for e >= 4
+// Any permutation works as long as both operands use the same one; this one is
+// chosen because
+//   * a pair of 16x16 accumulator tiles (lane holds rows 4g..4g+3 of column i)
+//     rounded to bf16 IS an operand in this mapping (rows = contraction), so
+//     products can be chained through registers;
+//   * an LDS tile whose contraction index is the contiguous dimension is read
+//     with two 8-byte loads (frag_kc);
+//   * an LDS tile whose contraction index is the ROW dimension is read with two
+//     ds_read_b64_tr_b16 transposing loads (frag_tr), so no tile is ever
+//     transposed explicitly.
+#pragma once
+
+#include "device_utils.h"
+
+namespace fla {
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane s supplies the address
+// of 4 consecutive 16-bit elements; lane i receives element (i % 4) of lanes
+// i/4, i/4 + 4, i/4 + 8, i/4 + 12.
+__device__ __forceinline__ bf16x4 lds_tr4(const bf16 *p) {
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)p);
+    return __builtin_bit_cast(bf16x4, r);
+}
+
+// Operand with rows r0..r0+15 and contraction c0..c0+31 along the contiguous
+// dimension of `tile` (pitch in elements).
+__device__ __forceinline__ bf16x8 frag_kc(const bf16 *tile, int pitch, int r0, int c0) {
+    const int l = lane_id(), i = l & 15, g = l >> 4;
+    const bf16 *p = tile + (r0 + i) * pitch + c0 + 4 * g;
+    return cat8(*reinterpret_cast<const bf16x4 *>(p), *reinterpret_cast<const bf16x4 *>(p + 16));
+}
+// 16-wide contraction variant for v_mfma_f32_16x16x16_bf16.
+__device__ __forceinline__ bf16x4 frag_kc4(const bf16 *tile, int pitch, int r0, int c0) {
+    const int l = lane_id(), i = l & 15, g = l >> 4;
+    return *reinterpret_cast<const bf16x4 *>(tile + (r0 + i) * pitch + c0 + 4 * g);
+}
+
+// Operand with index r0..r0+15 along the contiguous dimension and contraction
+// c0..c0+31 along the rows of `tile`:  slot (g,e) = tile[c0 + c(g,e)][r0 + i].
+__device__ __forceinline__ bf16x8 frag_tr(const bf16 *tile, int pitch, int r0, int c0) {
+    const int l = lane_id(), i = l & 15, g = l >> 4;
+    const bf16 *p = tile + (c0 + 4 * g + (i >> 2)) * pitch + r0 + 4 * (i & 3);
+    return cat8(lds_tr4(p), lds_tr4(p + 16 * pitch));
+}
+__device__ __forceinline__ bf16x4 frag_tr4(const bf16 *tile, int pitch, int r0, int c0) {
+    const int l = lane_id(), i = l & 15, g = l >> 4;
+    return lds_tr4(tile + (c0 + 4 * g + (i >> 2)) * pitch + r0 + 4 * (i & 3));
+}
+
+// Two accumulator tiles (rows 0..15 and 16..31 of a 32-row block) as an operand
+// whose contraction runs over those rows.
+__device__ __forceinline__ bf16x8 frag_from_acc(f32x4 lo, f32x4 hi) { return cat8(cvt4(lo), cvt4(hi)); }
+
+// Accumulator tile element e of lane l sits at row 4*(l/16)+e, column l%16.
+__device__ __forceinline__ int acc_row(int e) { return 4 * (lane_id() >> 4) + e; }
+__device__ __forceinline__ int acc_col() { return lane_id() & 15; }
+
+// ---- cooperative global <-> LDS tile copies (all threads of the block) -----------
+// Copies rows [0, valid) x cols [0, ncols) of a row-major global matrix (row stride
+// `gstride` elements, 16-byte aligned rows) into `tile`; rows [valid, nrows) are zeroed.
+template <int THREADS>
+__device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsrc, int64_t gstride, int nrows,
+                                          int ncols, int valid) {
+    const int cpr = ncols >> 3;  // 16-byte chunks per row
+    for (int idx = threadIdx.x; idx < nrows * cpr; idx += THREADS) {
+        const int r = idx / cpr, c = (idx % cpr) << 3;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (r < valid) v = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)r * gstride + c);
+        *reinterpret_cast<u32x4 *>(tile + r * pitch + c) = v;
+    }
+}
+template <int THREADS>
+__device__ __forceinline__ void store_tile(bf16 *gdst, int64_t gstride, const bf16 *tile, int pitch, int ncols,
+                                           int valid) {
+    const int cpr = ncols >> 3;
+    for (int idx = threadIdx.x; idx < valid * cpr; idx += THREADS) {
+        const int r = idx / cpr, c = (idx % cpr) << 3;
+        *reinterpret_cast<u32x4 *>(gdst + (int64_t)r * gstride + c) = *reinterpret_cast<const u32x4 *>(tile + r * pitch + c);
+    }
+}
+
+// Writes one accumulator tile, rounded to bf16, into a row-major LDS tile at (r0, c0).
+__device__ __forceinline__ void acc_to_tile(bf16 *tile, int pitch, int r0, int c0, f32x4 acc) {
+    const int col = c0 + acc_col();
+#pragma unroll
+    for (int e = 0; e < 4; ++e) tile[(r0 + acc_row(e)) * pitch + col] = (bf16)acc[e];
+}
+
+}  // namespace fla

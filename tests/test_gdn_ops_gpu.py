@@ -1,0 +1,170 @@
+"""Per-operator parity of the GDN chunk-forward kernels (through the C ABI) against the CPU
+oracle, on the cases the reference sweeps: dense, GVA (Hv = 2 Hk), ragged tails
+(lengths 1, 15, 16, 17, 63, 64, 65), packed variable-length batches with an empty sequence."""
+import pytest
+import torch
+
+from oracle import gdn
+from util import assert_close, err_stats, TOL_BF16, TOL_STATE
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def inputs(B, T, H, K, V, Hk=None, seed=0, init=False):
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=BF, seed=seed, Hk=Hk, init_std=0.01 if init else None,
+                            head_first_gates=True)
+    return d
+
+
+CASES = [
+    # B, T, H, Hk, K, V, cu_seqlens
+    (2, 128, 2, 2, 128, 128, None),
+    (1, 200, 4, 2, 128, 128, None),                     # GVA + ragged tail (200 = 3*64 + 8)
+    (1, 1, 1, 1, 128, 128, None),
+    (1, 65, 2, 2, 128, 128, None),
+    (1, 261, 2, 1, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261]),   # lengths 1,15,17,0,63,64,101
+]
+
+
+def dev_kw(d, dev):
+    return {k: (None if v is None else v.to(dev)) for k, v in d.items()}
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_stagewise_against_oracle(dev, case):
+    from fla_hip import ops
+    B, T, H, Hk, K, V, cu = case
+    d = inputs(B, T, H, K, V, Hk=Hk, seed=T)
+    N = B if cu is None else len(cu) - 1
+    gen = torch.Generator().manual_seed(5)
+    h0 = torch.randn(N, H, K, V, generator=gen) * 0.01
+    x = dev_kw(d, dev)
+
+    # a1 cumsum
+    G = ops.chunk_local_cumsum(x["g"], 64, cu_seqlens=cu)
+    G_ref = gdn.chunk_local_cumsum(d["g"], 64, cu_seqlens=cu)
+    assert_close(G, G_ref, 1e-5, "cumsum")
+
+    # a2 kkt (fp32 out; inputs are bf16 k so the only difference is accumulation order)
+    A0 = ops.chunk_scaled_dot_kkt(x["k"], G, x["beta"], cu_seqlens=cu, chunk_size=64)
+    A0_ref = gdn.chunk_scaled_dot_kkt(d["k"], G_ref, d["beta"], 64, cu_seqlens=cu)
+    assert_close(A0, A0_ref, 1e-4, "kkt")
+    # structural zeros: on/above the diagonal and tail columns are exactly zero
+    a0 = A0.cpu()
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        blk = a0[b, :, s:e]
+        assert float(torch.triu(blk[:, :, : e - s], 0).abs().max()) == 0.0
+        assert float(blk[:, :, e - s:].abs().max() if e - s < 64 else 0.0) == 0.0
+
+    # a3 solve_tri on the bf16-rounded A0 (as the pipeline does); residual test of the reference
+    A0b = A0.to(BF)
+    Ainv = ops.solve_tri(A0b, cu_seqlens=cu, layout="bnsd")
+    Ainv_ref = gdn.solve_tri(A0b.cpu().float(), cu_seqlens=cu, output_dtype=torch.float32)
+    assert_close(Ainv, Ainv_ref, TOL_BF16, "solve_tri")
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        L = e - s
+        M = torch.eye(L) + A0b.cpu().float()[b, :, s:e, :L]
+        res = torch.matmul(M, Ainv.cpu().float()[b, :, s:e, :L]) - torch.eye(L)
+        assert float(res.abs().max()) < 2e-2      # test_npu_solve_tri_ascend910b.py:39-41
+
+    # a4 w, u
+    w, u = ops.recompute_w_u_fwd(x["k"], x["v"], x["beta"], Ainv, 64, g=G, cu_seqlens=cu)
+    w_ref, u_ref = gdn.recompute_w_u_fwd(d["k"], d["v"], d["beta"], Ainv.cpu(), 64, g=G_ref, cu_seqlens=cu,
+                                         output_dtype=torch.float32)
+    assert_close(w, w_ref, TOL_BF16, "w")
+    assert_close(u, u_ref, TOL_BF16, "u")
+
+    # a5 state scan
+    h, v_new, final = ops.chunk_gated_delta_rule_fwd_h(x["k"], w, u, g=G, initial_state=h0.to(dev),
+                                                       output_final_state=True, chunk_size=64, cu_seqlens=cu)
+    h_ref, vn_ref, final_ref = gdn.chunk_gated_delta_rule_fwd_h(
+        d["k"], w.cpu(), u.cpu(), G_ref, initial_state=h0, output_final_state=True, chunk=64, cu_seqlens=cu,
+        output_dtype=torch.float32)
+    assert_close(v_new, vn_ref, TOL_BF16, "v_new")
+    assert_close(h, h_ref, TOL_BF16, "h")
+    assert_close(final, final_ref, TOL_STATE, "final_state")
+    assert final.dtype == torch.float32 and h.dtype == BF
+
+    # a6 output
+    scale = K ** -0.5
+    o = ops.chunk_fwd_o(x["q"], x["k"], v_new, h, scale, g=G, cu_seqlens=cu, chunk_size=64)
+    o_ref = gdn.chunk_fwd_o(d["q"], d["k"], v_new.cpu(), h.cpu(), scale, g=G_ref, chunk=64, cu_seqlens=cu,
+                            output_dtype=torch.float32)
+    assert_close(o, o_ref, TOL_BF16, "o")
+
+    # composition against the naive recurrence (the acceptance oracle)
+    o_nv, final_nv = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], scale,
+                                                          initial_state=h0, output_final_state=True, cu_seqlens=cu)
+    st = assert_close(o, o_nv, TOL_BF16, "o vs naive")
+    assert st["rel_max"] < 5e-2, st
+    assert_close(final, final_nv, TOL_STATE * 4, "final vs naive")   # unfused path rounds A, w, u to bf16
+
+
+def test_cumsum_variants(dev):
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(3)
+    g = torch.randn(2, 3, 300, generator=gen)
+    for chunk in (16, 64, 128):
+        for rev in (False, True):
+            out = ops.chunk_local_cumsum(g.to(dev), chunk, reverse=rev, scale=0.5)
+            ref = gdn.chunk_local_cumsum(g, chunk, reverse=rev, scale=0.5)
+            assert_close(out, ref, 1e-5, f"cumsum c={chunk} rev={rev}")
+    g4 = torch.randn(1, 2, 130, 96, generator=gen)
+    out = ops.chunk_local_cumsum(g4.to(dev), 64, cu_seqlens=[0, 70, 130])
+    assert_close(out, gdn.chunk_local_cumsum(g4, 64, cu_seqlens=[0, 70, 130]), 1e-5, "cumsum 4d")
+    out = ops.chunk_local_cumsum(g.bfloat16().to(dev), 64, output_dtype=torch.bfloat16)
+    assert out.dtype == BF
+    assert_close(out, gdn.chunk_local_cumsum(g.bfloat16(), 64), 2e-2, "cumsum bf16")
+
+
+def test_solve_tri_layouts_and_inverse(dev):
+    """Against numpy.linalg.inv and across the bsnd / bnsd / tnd / ntd layouts."""
+    import numpy as np
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(9)
+    B, H, T = 2, 3, 128
+    A = torch.tril(torch.randn(B, H, T // 64, 64, 64, generator=gen) * 0.2, -1).reshape(B, H, T, 64).to(BF)
+    ref = torch.from_numpy(np.linalg.inv(np.eye(64) + A.float().reshape(B, H, 2, 64, 64).numpy())).reshape(B, H, T, 64)
+    out = ops.solve_tri(A.to(dev), layout="bnsd")
+    assert_close(out, ref, TOL_BF16, "bnsd")
+    out = ops.solve_tri(A.transpose(1, 2).contiguous().to(dev), layout="bsnd")
+    assert_close(out.transpose(1, 2), ref, TOL_BF16, "bsnd")
+    out = ops.solve_tri(A[0].contiguous().to(dev), layout="ntd")
+    assert_close(out, ref[0], TOL_BF16, "ntd")
+    out = ops.solve_tri(A[0].transpose(0, 1).contiguous().to(dev), layout="tnd")
+    assert_close(out.transpose(0, 1), ref[0], TOL_BF16, "tnd")
+
+
+def test_state_v_first_and_no_final(dev):
+    from fla_hip import ops
+    d = inputs(1, 130, 2, 128, 128, seed=4)
+    x = dev_kw(d, dev)
+    G = ops.chunk_local_cumsum(x["g"], 64)
+    gen = torch.Generator().manual_seed(1)
+    w = (torch.randn(1, 2, 130, 128, generator=gen) * 0.1).to(BF)
+    u = torch.randn(1, 2, 130, 128, generator=gen).to(BF)
+    h0 = torch.randn(1, 2, 128, 128, generator=gen) * 0.01
+    h_a, vn_a, f_a = ops.chunk_gated_delta_rule_fwd_h(x["k"], w.to(dev), u.to(dev), g=G, initial_state=h0.to(dev),
+                                                      output_final_state=True)
+    h_b, vn_b, f_b = ops.chunk_gated_delta_rule_fwd_h(
+        x["k"], w.to(dev), u.to(dev), g=G, initial_state=h0.transpose(-1, -2).contiguous().to(dev),
+        output_final_state=True, state_v_first=True)
+    assert torch.equal(vn_a, vn_b)
+    assert torch.equal(h_a, h_b.transpose(-1, -2))
+    assert torch.equal(f_a, f_b.transpose(-1, -2))
+    h_c, vn_c, f_c = ops.chunk_gated_delta_rule_fwd_h(x["k"], w.to(dev), u.to(dev), g=G, initial_state=h0.to(dev))
+    assert f_c is None and torch.equal(vn_a, vn_c)
+
+
+def test_rejects_bad_metadata(dev):
+    from fla_hip import ops
+    d = inputs(1, 128, 1, 128, 128)
+    x = dev_kw(d, dev)
+    G = ops.chunk_local_cumsum(x["g"], 64)
+    with pytest.raises(RuntimeError, match="canonical"):
+        ops.chunk_scaled_dot_kkt(x["k"], G, x["beta"], cu_seqlens=[0, 64, 128], chunk_indices=[0, 0, 0, 1])
+    with pytest.raises(RuntimeError, match="chunk_size must be 64"):
+        ops.chunk_scaled_dot_kkt(x["k"], G, x["beta"], chunk_size=32)
+    with pytest.raises(RuntimeError, match="either g or gk"):
+        ops.chunk_gated_delta_rule_fwd_h(x["k"], x["k"], x["v"])
