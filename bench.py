@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the accelerated path on one MI355X.
+
+Default workload (the configuration the headline metric is quoted on): GDN chunk forward,
+bf16 in / fp32 accumulation and state, B=4, T=8192, H=32, K=V=128, chunk 64, fp32 initial
+state, final state on.  One "step" is one pass of the whole chunk forward over that batch
+with inputs resident in HBM.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode|conv1d]
+
+`roofline` describes the dominant kernel of the step: algorithmic FLOPs (or bytes) per launch
+divided by its average duration, measured with HIP events recorded on the launch stream by the
+library's own per-launch timing hooks in a second pass of K steps directly after the timed region.
+`cpu_baseline` times the CPU oracle (a port of the reference's PyTorch CPU path) on the host cores
+on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for _p in (str(ROOT), str(ROOT / "flash-linear-attention-npu_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# Dense-tile FLOP count per token-head of the chunk forward (C=64, K=V=128):
+#   kkt, w, q.k^T = 3*C*K ; u, P.v_new = 2*C*V ; w.h, k^T.v_new, q.h = 3*K*V ; unit-lower inverse C^2/3
+def gdn_flops_per_token_head(C=64, K=128, V=128):
+    return 2 * (3 * C * K + 2 * C * V + 3 * K * V + C * C // 3)
+
+# share of those FLOPs executed by each kernel of the step
+def gdn_kernel_flops_per_token_head(C=64, K=128, V=128):
+    prep = 2 * (2 * C * K + C * V + C * C // 3)          # kkt, inverse, w, u
+    scan = 2 * (C * K + C * V + 3 * K * V)               # q.k^T, P.v_new, w.h, k^T.v_new, q.h
+    return {"prep": prep, "scan": scan, "total": prep + scan}
+
+
+def profile_report(lib):
+    buf = ctypes.create_string_buffer(1 << 16)
+    lib.fla_profile_report.argtypes = [ctypes.c_char_p, ctypes.c_uint64]
+    lib.fla_profile_report.restype = ctypes.c_int
+    lib.fla_profile_report(buf, len(buf))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, n, ms = line.split()
+        out[name] = (int(n), float(ms))
+    return out
+
+
+def bench_gdn(args, torch, dev):
+    import fla_hip
+    from fla_hip import pipeline
+    from oracle import gdn as ogdn
+
+    lib = fla_hip.load_library()
+    B, T, H, K, V, C = 4, 8192, 32, 128, 128, 64
+    F = torch.nn.functional
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = F.normalize(torch.randn(B, H, T, K, device=dev, generator=g), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(B, H, T, K, device=dev, generator=g), dim=-1).bfloat16()
+    v = torch.randn(B, H, T, V, device=dev, generator=g).bfloat16()
+    beta = torch.sigmoid(torch.randn(B, T, H, device=dev, generator=g))
+    gate = F.logsigmoid(torch.randn(B, T, H, device=dev, generator=g))
+    h0 = torch.randn(B, H, K, V, device=dev, generator=g) * 0.01
+    fused = args.route == "fused"
+
+    def step():
+        return pipeline.flash_gated_delta_rule(q, k, v, gate, beta, None, h0, True, chunk_size=C, fused=fused)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        o, final = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+    tokens_per_s = B * T * args.steps / dt
+
+    # per-kernel durations: second pass with the library's event hooks on the launch stream
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    prof = profile_report(lib)
+    kern = {name: ms / n for name, (n, ms) in prof.items()}
+    dominant = max(kern, key=kern.get) if kern else None
+    th = B * T * H
+    fl = gdn_kernel_flops_per_token_head(C, K, V)
+    flops_of = {  # algorithmic FLOPs of one launch of each kernel
+        "gdn_fused": fl["total"] * th, "gdn_prep": fl["prep"] * th, "gdn_scan": fl["scan"] * th,
+        "kkt": 2 * C * K * th, "solve_tri": 2 * (C * C // 3) * th, "wu": 2 * (C * K + C * V) * th,
+        "fwd_h": 2 * (2 * K * V) * th, "fwd_o": 2 * (C * K + C * V + K * V) * th,
+    }
+    roofline = None
+    if dominant in flops_of:
+        ach = flops_of[dominant] / (kern[dominant] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                    "avg_kernel_ms": round(kern[dominant], 4),
+                    "all_kernels_ms": {n: round(t, 4) for n, t in kern.items()}}
+    step_tflops = gdn_flops_per_token_head(C, K, V) * th / (ms_per_step * 1e-3) / 1e12
+
+    # CPU baseline: the oracle's chunked fp32 path on the host cores, bounded sample
+    cpu = None
+    if not args.no_cpu:
+        import torch as _t
+        cores = os.cpu_count() or 1
+        _t.set_num_threads(cores)
+        Ts = args.cpu_tokens
+        d = ogdn.make_gdn_inputs(1, Ts, H, K, V, dtype=_t.bfloat16, seed=0, init_std=0.01, head_first_gates=True)
+        ogdn.chunk_gated_delta_rule_fwd(d["q"][:, :, :128], d["k"][:, :, :128], d["v"][:, :, :128],
+                                        d["g"][:, :, :128], d["beta"][:, :, :128], initial_state=d["initial_state"])
+        t1 = time.perf_counter()
+        reps = 0
+        while reps == 0 or time.perf_counter() - t1 < args.cpu_seconds:
+            ogdn.chunk_gated_delta_rule_fwd(d["q"], d["k"], d["v"], d["g"], d["beta"],
+                                            initial_state=d["initial_state"], output_final_state=True)
+            reps += 1
+        cdt = time.perf_counter() - t1
+        cpu = {"value": round(Ts * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x (B=1 T={Ts} H={H} K=V={K}) chunked fp32 torch oracle, {cdt:.1f} s"}
+    # sanity of the timed result (not a parity test): finite outputs
+    assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(final).all())
+    return {
+        "metric": "gdn_chunk_fwd_tokens_per_s", "value": round(tokens_per_s, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "GDN chunk forward B=4 T=8192 H=32 K=V=128 chunk=64, fp32 initial+final state",
+                   "route": args.route},
+        "step_tflops": round(step_tflops, 2), "step_frac_of_bf16_peak": round(step_tflops / PEAK_BF16_TFLOPS, 4),
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+
+
+def bench_decode(args, torch, dev):
+    import fla_hip
+    from fla_hip import ops
+    from oracle import decode as odec
+
+    lib = fla_hip.load_library()
+    N, H, D = 256, 32, 128
+    F = torch.nn.functional
+    g = torch.Generator(device=dev).manual_seed(0)
+    q = F.normalize(torch.randn(N, H, D, device=dev, generator=g), dim=-1).bfloat16()
+    k = F.normalize(torch.randn(N, H, D, device=dev, generator=g), dim=-1).bfloat16()
+    v = torch.randn(N, H, D, device=dev, generator=g).bfloat16()
+    beta = torch.sigmoid(torch.randn(N, H, device=dev, generator=g)).bfloat16()
+    gate = F.logsigmoid(torch.randn(N, H, device=dev, generator=g))
+    state = torch.randn(N, H, D, D, device=dev, generator=g) * 0.01
+    lens = torch.tensor([0] + [1] * N, dtype=torch.int32, device=dev)
+    idx = torch.arange(N, dtype=torch.int32, device=dev)
+
+    def step():
+        return ops.recurrent_gated_delta_rule(q, k, v, state, beta=beta, scale=D ** -0.5, actual_seq_lengths=lens,
+                                              ssm_state_indices=idx, g=gate)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    prof = profile_report(lib)
+    n, ms = prof["recurrent_gdn"]
+    bytes_per_launch = 2 * N * H * D * D * 4 + 4 * N * H * D * 2 + N * H * (2 + 4)
+    ach = bytes_per_launch / (ms / n * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        ns = N
+        c = lambda t: t[:ns].cpu()
+        cq, ck, cv, cs, cb, cg = c(q), c(k), c(v), c(state), c(beta), c(gate)
+        t1 = time.perf_counter()
+        reps = 0
+        while reps == 0 or time.perf_counter() - t1 < args.cpu_seconds:
+            odec.recurrent_gated_delta_rule(cq, ck, cv, cs, beta=cb, scale=D ** -0.5,
+                                            actual_seq_lengths=torch.tensor([0] + [1] * ns, dtype=torch.int32),
+                                            ssm_state_indices=torch.arange(ns, dtype=torch.int32), g=cg)
+            reps += 1
+        cdt = time.perf_counter() - t1
+        cpu = {"value": round(ns * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x ({ns} sequences x 1 token, H=32 K=V=128) fp32 torch oracle, {cdt:.1f} s"}
+    return {
+        "metric": "gdn_decode_tokens_per_s", "value": round(N * args.steps / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "GDN recurrent decode 256 sequences x 1 token, H=32 K=V=128, fp32 state in place"},
+        "roofline": {"bound": "hbm", "kernel": "recurrent_gdn", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "avg_kernel_ms": round(ms / n, 4)},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_conv1d(args, torch, dev):
+    import fla_hip
+    from fla_hip import ops
+    from oracle import conv1d as oconv
+
+    lib = fla_hip.load_library()
+    B, T, D, W = 4, 4096, 4096, 4
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(B, T, D, device=dev, generator=g).bfloat16()
+    w = (torch.randn(W, D, device=dev, generator=g) * 0.1).bfloat16()
+    b = (torch.randn(D, device=dev, generator=g) * 0.01).bfloat16()
+
+    def step():
+        return ops.causal_conv1d(x, w, b, activation_mode=1)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    n, ms = profile_report(lib)["conv1d_fwd"]
+    bytes_per_launch = 2 * B * T * D * 2 + (W + 1) * D * 2
+    ach = bytes_per_launch / (ms / n * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)
+        xs, ws, bs = x.cpu(), w.cpu(), b.cpu()
+        t1 = time.perf_counter()
+        reps = 0
+        while reps == 0 or time.perf_counter() - t1 < args.cpu_seconds:
+            oconv.causal_conv1d(xs, ws, bs, activation_mode=1)
+            reps += 1
+        cdt = time.perf_counter() - t1
+        cpu = {"value": round(B * T * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x (B=4 T=4096 D=4096 W=4) fp32 torch oracle, {cdt:.1f} s"}
+    return {
+        "metric": "causal_conv1d_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "causal_conv1d fwd + SiLU B=4 T=4096 D=4096 width=4 + bias, zero left pad"},
+        "roofline": {"bound": "hbm", "kernel": "conv1d_fwd", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "avg_kernel_ms": round(ms / n, 4)},
+        "cpu_baseline": cpu,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d"])
+    ap.add_argument("--route", default="ops", choices=["fused", "ops"],
+                    help="gdn_chunk: one fused library call, or the six per-stage operators")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-tokens", type=int, default=8192, help="tokens per pass of the CPU baseline sample")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="minimum CPU time spent on the baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU; every kernel works on one GPU's share and there are no "
+              "collectives to time. Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible.", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d}[args.workload]
+    print(json.dumps(fn(args, torch, dev)))
+
+
+if __name__ == "__main__":
+    main()

@@ -13,8 +13,10 @@
 namespace fla {
 namespace {
 
-constexpr int kThreads = 128;
-constexpr int kTok = 32;  // tokens per thread
+#ifndef FLA_CONV_THREADS
+#define FLA_CONV_THREADS 128
+#endif
+constexpr int kThreads = FLA_CONV_THREADS;
 constexpr int kMaxW = 4;
 
 struct ConvParams {
@@ -33,13 +35,18 @@ struct ConvParams {
     int B, S, D, W, N;
     int head_dim;                  // D / head_num, or D when no head split
     int tiles_per_seq;             // dense only
+    int tok;                       // tokens per thread (tile height)
     int activation;
     int pad_slot;
     int varlen;
 };
 
 template <typename T> __device__ __forceinline__ void load8(const T *p, float (&f)[8]) {
+#ifdef FLA_CONV_NT_LOAD
     typename Vec8<T>::type v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec8<T>::type *>(p));
+#else
+    typename Vec8<T>::type v = *reinterpret_cast<const typename Vec8<T>::type *>(p);
+#endif
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
 }
@@ -52,7 +59,11 @@ template <typename T> __device__ __forceinline__ void store8(T *p, const float (
     typename Vec8<T>::type v;
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (T)f[i];
+#ifdef FLA_CONV_NT_STORE
     __builtin_nontemporal_store(v, reinterpret_cast<typename Vec8<T>::type *>(p));
+#else
+    *reinterpret_cast<typename Vec8<T>::type *>(p) = v;
+#endif
 }
 
 __device__ __forceinline__ int find_seq(const int32_t *qsl, int N, int t) {
@@ -65,7 +76,7 @@ __device__ __forceinline__ int find_seq(const int32_t *qsl, int N, int t) {
     return lo;
 }
 
-template <typename T, int W>
+template <typename T, int W, int kTok>
 __global__ void __launch_bounds__(kThreads) conv1d_fwd_kernel(const ConvParams p) {
     const int d0 = (blockIdx.y * kThreads + threadIdx.x) * 8;
     if (d0 >= p.D) return;
@@ -150,7 +161,7 @@ __global__ void __launch_bounds__(kThreads) conv1d_fwd_kernel(const ConvParams p
 #pragma unroll
                 for (int r = 0; r < W - 1; ++r) a = fmaf(w[r][i], win[r][i], a);
                 a = fmaf(w[W - 1][i], cur[j][i], a);
-                if (p.activation == 1) a = a / (1.f + __expf(-a));
+                if (p.activation == 1) a = a * __frcp_rn(1.f + __expf(-a));  // SiLU; 1-ulp reciprocal is ample for a 16-bit result
                 acc[i] = a;
             }
 #pragma unroll
@@ -160,6 +171,71 @@ __global__ void __launch_bounds__(kThreads) conv1d_fwd_kernel(const ConvParams p
 #pragma unroll
             for (int i = 0; i < 8; ++i) win[W - 2][i] = cur[j][i];
             if (!skip) store8(ob + (int64_t)t * p.o_ss, acc);
+        }
+    }
+}
+
+// Dense fast path: no packed sequences, no cache indirection, no initial states.  The tile
+// loop is fully unrolled so the W-1 row window rotates through register renaming and the only
+// per-row scalar work is one pointer increment; rows past the end of a sequence are loaded
+// from a clamped address and never stored.
+template <typename T, int W, int TOK, bool ACT>
+__global__ void __launch_bounds__(kThreads) conv1d_dense_kernel(const ConvParams p) {
+    typedef typename Vec8<T>::type V8;
+    const int d0 = (blockIdx.y * kThreads + threadIdx.x) * 8;
+    if (d0 >= p.D) return;
+    const int b = blockIdx.x / p.tiles_per_seq;
+    const int t0 = (blockIdx.x % p.tiles_per_seq) * TOK;
+    const int nvalid = min(TOK, p.S - t0);
+    const T *xp = static_cast<const T *>(p.x) + b * p.x_sb + (int64_t)t0 * p.x_ss + d0;
+    const int hd = d0 / p.head_dim, dd = d0 % p.head_dim;
+    T *op = static_cast<T *>(p.out) + b * p.o_sb + hd * p.o_sh + (int64_t)t0 * p.o_ss + dd;
+
+    float w[W][8], bias[8];
+#pragma unroll
+    for (int r = 0; r < W; ++r) load8_cached(static_cast<const T *>(p.weight) + r * p.w_sr + d0, w[r]);
+    if (p.bias) {
+        load8_cached(static_cast<const T *>(p.bias) + d0, bias);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bias[i] = 0.f;
+    }
+    float win[W - 1][8];
+#pragma unroll
+    for (int r = 0; r < W - 1; ++r) {
+        if (t0 - (W - 1) + r >= 0) {
+            load8_cached(xp - (int64_t)(W - 1 - r) * p.x_ss, win[r]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[r][i] = 0.f;
+        }
+    }
+#pragma unroll
+    for (int j0 = 0; j0 < TOK; j0 += 8) {
+        V8 raw[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) raw[j] = *reinterpret_cast<const V8 *>(xp + (int64_t)min(j0 + j, nvalid - 1) * p.x_ss);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            float cur[8];
+            V8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                cur[i] = (float)raw[j][i];
+                float a = bias[i];
+#pragma unroll
+                for (int r = 0; r < W - 1; ++r) a = fmaf(w[r][i], win[r][i], a);
+                a = fmaf(w[W - 1][i], cur[i], a);
+                if (ACT) a = a * __frcp_rn(1.f + __expf(-a));  // SiLU; a 1-ulp reciprocal is ample for a 16-bit result
+                o[i] = (T)a;
+            }
+#pragma unroll
+            for (int r = 0; r + 1 < W - 1; ++r)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) win[r][i] = win[r + 1][i];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) win[W - 2][i] = cur[i];
+            if (j0 + j < nvalid) __builtin_nontemporal_store(o, reinterpret_cast<V8 *>(op + (int64_t)(j0 + j) * p.o_ss));
         }
     }
 }
@@ -343,28 +419,74 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
     p.W = (int)W;
     p.N = N;
     p.head_dim = (int)head_dim;
-    p.tiles_per_seq = (int)((S + kTok - 1) / kTok);
+    // Tile height: tall tiles amortise the W-1 row halo, short tiles give the scheduler enough
+    // workgroups to keep every CU busy through the tail of the launch.
+    int tok = 32;
+    {
+        const int64_t col_blocks = (D / 8 + kThreads - 1) / kThreads;
+        while (tok > 8 && ((B * S + tok - 1) / tok) * col_blocks < (int64_t)24 * num_cus()) tok >>= 1;
+        if (const char *env = getenv("FLA_HIP_CONV_TOK")) {
+            const int v = atoi(env);
+            if (v == 8 || v == 16 || v == 32 || v == 64) tok = v;
+        }
+    }
+    p.tok = tok;
+    p.tiles_per_seq = (int)((S + tok - 1) / tok);
     p.activation = (int)activation_mode;
     p.pad_slot = (int)pad_slot_id;
     p.varlen = packed ? 1 : 0;
 
+    const bool is_bf16 = x->dtype == FLA_BF16;
     const dim3 block(kThreads);
     const dim3 grid((unsigned)(p.tiles_per_seq * (packed ? 1 : B)), (unsigned)((D / 8 + kThreads - 1) / kThreads));
-    const bool is_bf16 = x->dtype == FLA_BF16;
-#define FLA_LAUNCH_CONV(WW)                                                                  \
-    if (is_bf16) hipLaunchKernelGGL((conv1d_fwd_kernel<bf16, WW>), grid, block, 0, stream, p); \
-    else hipLaunchKernelGGL((conv1d_fwd_kernel<f16, WW>), grid, block, 0, stream, p)
+    const bool dense_fast = !packed && cache.empty() && init.empty();
+    if (dense_fast) {
+        // 16-row tiles keep ~4k workgroups in flight for the benchmark shape; the 3-row halo is an L2 hit
+        const int ft = (B * ((S + 31) / 32) * (int64_t)grid.y >= (int64_t)16 * num_cus()) ? 32 : 16;
+        p.tok = ft;
+        p.tiles_per_seq = (int)((S + ft - 1) / ft);
+        const dim3 fgrid((unsigned)(p.tiles_per_seq * B), grid.y);
+        const bool act = activation_mode == 1;
+#define FLA_LAUNCH_DENSE(TT, WW, TK)                                                                              \
+    if (act) FLA_LAUNCH("conv1d_fwd", stream, (conv1d_dense_kernel<TT, WW, TK, true>), fgrid, block, 0, stream, p); \
+    else FLA_LAUNCH("conv1d_fwd", stream, (conv1d_dense_kernel<TT, WW, TK, false>), fgrid, block, 0, stream, p)
+#define FLA_LAUNCH_DENSE_W(TT, TK)               \
+    switch (W) {                                 \
+        case 2: FLA_LAUNCH_DENSE(TT, 2, TK); break; \
+        case 3: FLA_LAUNCH_DENSE(TT, 3, TK); break; \
+        default: FLA_LAUNCH_DENSE(TT, 4, TK); break; \
+    }
+        if (is_bf16) {
+            if (ft == 32) { FLA_LAUNCH_DENSE_W(bf16, 32) } else { FLA_LAUNCH_DENSE_W(bf16, 16) }
+        } else {
+            if (ft == 32) { FLA_LAUNCH_DENSE_W(f16, 32) } else { FLA_LAUNCH_DENSE_W(f16, 16) }
+        }
+#undef FLA_LAUNCH_DENSE_W
+#undef FLA_LAUNCH_DENSE
+    } else {
+#define FLA_LAUNCH_CONV_T(WW, TT)                                                                      \
+    if (is_bf16) FLA_LAUNCH("conv1d_fwd", stream, (conv1d_fwd_kernel<bf16, WW, TT>), grid, block, 0, stream, p); \
+    else FLA_LAUNCH("conv1d_fwd", stream, (conv1d_fwd_kernel<f16, WW, TT>), grid, block, 0, stream, p)
+#define FLA_LAUNCH_CONV(WW)                                      \
+    switch (tok) {                                               \
+        case 8: FLA_LAUNCH_CONV_T(WW, 8); break;                 \
+        case 16: FLA_LAUNCH_CONV_T(WW, 16); break;               \
+        case 64: FLA_LAUNCH_CONV_T(WW, 64); break;               \
+        default: FLA_LAUNCH_CONV_T(WW, 32); break;               \
+    }
     switch (W) {
         case 2: FLA_LAUNCH_CONV(2); break;
         case 3: FLA_LAUNCH_CONV(3); break;
         default: FLA_LAUNCH_CONV(4); break;
     }
 #undef FLA_LAUNCH_CONV
+#undef FLA_LAUNCH_CONV_T
+    }
     FLA_HIP_CHECK(hipGetLastError());
     if (has_states && N > 0) {
         const dim3 sgrid((unsigned)((D / 8 + 63) / 64), (unsigned)N);
-        if (is_bf16) hipLaunchKernelGGL(conv1d_state_kernel<bf16>, sgrid, dim3(64), 0, stream, p);
-        else hipLaunchKernelGGL(conv1d_state_kernel<f16>, sgrid, dim3(64), 0, stream, p);
+        if (is_bf16) FLA_LAUNCH("conv1d_state", stream, conv1d_state_kernel<bf16>, sgrid, dim3(64), 0, stream, p);
+        else FLA_LAUNCH("conv1d_state", stream, conv1d_state_kernel<f16>, sgrid, dim3(64), 0, stream, p);
         FLA_HIP_CHECK(hipGetLastError());
     }
     return FLA_OK;

@@ -163,7 +163,64 @@ int num_cus() {
     return cached[dev];
 }
 
+// ---- per-kernel timing -------------------------------------------------------
+namespace {
+struct ProfRec {
+    const char *name;
+    hipEvent_t start, stop;
+};
+std::mutex g_prof_mu;
+std::vector<ProfRec> g_prof;
+bool g_prof_on = false;
+}  // namespace
+
+bool profile_enabled() { return g_prof_on; }
+
+void profile_begin(const char *name, hipStream_t stream) {
+    ProfRec r{name, nullptr, nullptr};
+    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
+    (void)hipEventRecord(r.start, stream);
+    std::lock_guard<std::mutex> lock(g_prof_mu);
+    g_prof.push_back(r);
+}
+
+void profile_end(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_prof_mu);
+    if (!g_prof.empty()) (void)hipEventRecord(g_prof.back().stop, stream);
+}
+
 }  // namespace fla
+
+extern "C" void fla_profile_enable(int on) { fla::g_prof_on = on != 0; }
+
+// Waits for every recorded launch, writes one "name count total_ms" line per kernel
+// name into buf (NUL-terminated, truncated to cap) and clears the records.
+extern "C" int fla_profile_report(char *buf, uint64_t cap) {
+    std::lock_guard<std::mutex> lock(fla::g_prof_mu);
+    struct Agg { const char *name; int n; double ms; };
+    std::vector<Agg> agg;
+    for (auto &r : fla::g_prof) {
+        float ms = 0.f;
+        if (hipEventSynchronize(r.stop) == hipSuccess && hipEventElapsedTime(&ms, r.start, r.stop) == hipSuccess) {
+            bool found = false;
+            for (auto &a : agg)
+                if (!strcmp(a.name, r.name)) { a.n++; a.ms += ms; found = true; break; }
+            if (!found) agg.push_back(Agg{r.name, 1, ms});
+        }
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    fla::g_prof.clear();
+    size_t off = 0;
+    if (buf && cap) buf[0] = 0;
+    for (auto &a : agg) {
+        if (!buf || off >= cap) break;
+        int w = snprintf(buf + off, cap - off, "%s %d %.6f\n", a.name, a.n, a.ms);
+        if (w < 0) break;
+        off += (size_t)w;
+    }
+    return (int)agg.size();
+}
 
 extern "C" const char *fla_last_error(void) { return fla::last_error_buffer(); }
 extern "C" int fla_abi_version(void) { return 1; }

@@ -93,7 +93,31 @@ int stage_to_device(void *dst, const void *src, size_t bytes, hipStream_t stream
 
 int num_cus();
 
+// ---- optional per-kernel timing (off by default) ---------------------------
+// When enabled through fla_profile_enable(1), every kernel launch site brackets
+// its launch with two HIP events on the launch stream; fla_profile_report()
+// synchronises them and returns "name count total_ms" lines.
+bool profile_enabled();
+void profile_begin(const char *name, hipStream_t stream);
+void profile_end(hipStream_t stream);
+struct ProfileScope {
+    hipStream_t s;
+    bool on;
+    ProfileScope(const char *name, hipStream_t stream) : s(stream), on(profile_enabled()) {
+        if (on) profile_begin(name, s);
+    }
+    ~ProfileScope() {
+        if (on) profile_end(s);
+    }
+};
+
 }  // namespace fla
+
+#define FLA_LAUNCH(name, stream_, ...)                     \
+    do {                                                   \
+        ::fla::ProfileScope prof__(name, stream_);         \
+        hipLaunchKernelGGL(__VA_ARGS__);                   \
+    } while (0)
 
 // Workspace-query / launch pair generator: each operator is written once as
 //   static int impl(<operands>, void* ws, uint64_t ws_size, hipStream_t s, uint64_t* query)

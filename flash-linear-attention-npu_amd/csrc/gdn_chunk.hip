@@ -369,7 +369,7 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
     KktParams p{geom, view4(k), view3(g), view3(beta), static_cast<float *>(out->data), out->stride[0], out->stride[1],
                 out->stride[2]};
     const size_t smem = (size_t)kChunk * (geom.K + 8) * 2 + 2 * kChunk * 4;
-    hipLaunchKernelGGL(kkt_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("kkt", stream, kkt_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -407,7 +407,7 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
     if (geom.NT == 0 || geom.B == 0 || geom.Hv == 0) return FLA_OK;
     SolveParams p{geom, static_cast<const bf16 *>(x->data), static_cast<bf16 *>(out->data), ib < 0 ? 0 : x->stride[ib],
                   x->stride[ih], x->stride[it]};
-    hipLaunchKernelGGL(solve_tri_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(64), 0, stream, p);
+    FLA_LAUNCH("solve_tri", stream, solve_tri_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(64), 0, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -438,7 +438,7 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     const size_t smem = (size_t)kChunk * ((kChunk + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(wu_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       (int)smem));
-    hipLaunchKernelGGL(wu_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("wu", stream, wu_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -448,7 +448,7 @@ int launch_fwd_o(const FwdOParams &p, hipStream_t stream) {
     const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + kChunk * 4;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL((fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }

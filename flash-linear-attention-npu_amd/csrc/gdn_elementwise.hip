@@ -132,10 +132,10 @@ template <typename TI, typename TO>
 void launch_cumsum(const CumsumParams &p, hipStream_t stream) {
     const dim3 grid(p.geom.NT, p.geom.Hv, p.geom.B);
     if (p.feat == 1) {
-        hipLaunchKernelGGL((cumsum_tokens_kernel<TI, TO>), grid, dim3(64), 0, stream, p);
+        FLA_LAUNCH("cumsum_tokens", stream, (cumsum_tokens_kernel<TI, TO>), grid, dim3(64), 0, stream, p);
     } else {
         const int threads = p.feat >= 256 ? 256 : ((p.feat + 63) / 64) * 64;
-        hipLaunchKernelGGL((cumsum_features_kernel<TI, TO>), grid, dim3(threads), 0, stream, p);
+        FLA_LAUNCH("cumsum_features", stream, (cumsum_features_kernel<TI, TO>), grid, dim3(threads), 0, stream, p);
     }
 }
 

@@ -184,7 +184,7 @@ int launch_fwd_h(const ScanParams &p, int slabs, hipStream_t stream) {
     const size_t smem = ((size_t)kChunk * (K + 8) + (size_t)kChunk * (K + 16) + (size_t)kChunk * (VS + 16)) * 2 + kChunk * 4;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_h_kernel<K, CT>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL((fwd_h_kernel<K, CT>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("fwd_h", stream, (fwd_h_kernel<K, CT>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }

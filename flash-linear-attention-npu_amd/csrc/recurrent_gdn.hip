@@ -36,8 +36,13 @@ struct RecParams {
 
 template <typename ST> struct StateIO;
 template <> struct StateIO<float> {
-    static __device__ __forceinline__ f32x4 load(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
-    static __device__ __forceinline__ void store(float *p, f32x4 v) { *reinterpret_cast<f32x4 *>(p) = v; }
+    // the state is streamed exactly once in and once out: keep it out of the caches
+    static __device__ __forceinline__ f32x4 load(const float *p) {
+        return __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p));
+    }
+    static __device__ __forceinline__ void store(float *p, f32x4 v) {
+        __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p));
+    }
 };
 template <> struct StateIO<bf16> {
     static __device__ __forceinline__ f32x4 load(const bf16 *p) {
@@ -253,8 +258,8 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
     const dim3 grid((unsigned)(B * Nv)), block(kThreads);
     const bool f32s = state->dtype == FLA_F32;
 #define FLA_LAUNCH_REC(DK, DV)                                                                       \
-    if (f32s) hipLaunchKernelGGL((recurrent_gdn_kernel<float, DK, DV>), grid, block, 0, stream, p);   \
-    else hipLaunchKernelGGL((recurrent_gdn_kernel<bf16, DK, DV>), grid, block, 0, stream, p)
+    if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<float, DK, DV>), grid, block, 0, stream, p);   \
+    else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<bf16, DK, DV>), grid, block, 0, stream, p)
     if (Dk == 128 && Dv == 128) { FLA_LAUNCH_REC(128, 128); }
     else if (Dk == 64 && Dv == 64) { FLA_LAUNCH_REC(64, 64); }
     else if (Dk == 128 && Dv == 256) { FLA_LAUNCH_REC(128, 256); }
