@@ -277,7 +277,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d"])
-    ap.add_argument("--route", default="ops", choices=["fused", "ops"],
+    ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=8192, help="tokens per pass of the CPU baseline sample")

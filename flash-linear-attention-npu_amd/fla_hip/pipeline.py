@@ -74,11 +74,14 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
         raise ValueError("g and beta must be rank-3 tensors with shape [B, T, H].")
     if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
         raise ValueError("q, k and v must be rank-4 tensors with shape [B, H, T, D].")
-    if q.shape[:3] != k.shape[:3] or q.shape[:3] != v.shape[:3]:
+    # the reference requires equal head counts here; grouped value heads (Hv a multiple of Hk) are
+    # supported by every kernel of this library, so only batch and length must agree
+    if q.shape[:3] != k.shape[:3] or (q.shape[0], q.shape[2]) != (v.shape[0], v.shape[2]) \
+            or v.shape[1] % q.shape[1] != 0:
         raise ValueError(f"q/k/v shape prefixes must match, got {q.shape}, {k.shape}, {v.shape}.")
     if g.shape != beta.shape:
         raise ValueError(f"g and beta shapes must match, got {g.shape} and {beta.shape}.")
-    if g.shape[0] != q.shape[0] or g.shape[1] != q.shape[2] or g.shape[2] != q.shape[1]:
+    if g.shape[0] != q.shape[0] or g.shape[1] != q.shape[2] or g.shape[2] != v.shape[1]:
         raise ValueError(
             "Expected q/k/v in [B, H, T, D] and g/beta in [B, T, H]; "
             f"got q={tuple(q.shape)}, g={tuple(g.shape)}.")

@@ -1,0 +1,126 @@
+"""End-to-end parity of the GDN chunk forward (fused library call and the six-operator route)
+against the fp32 naive recurrence, with the pipeline-level layouts of
+examples/flash_gated_delta_rule.py:1126-1228: q,k,v [B,H,T,D]; g,beta [B,T,H]; o [B,T,H,V];
+final_state [N,H,K,V].  Tolerances: bf16 output 2e-2, fp32 state 1e-3 (fused route)."""
+import pytest
+import torch
+
+from oracle import gdn
+from util import assert_close, err_stats, TOL_BF16, TOL_STATE
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def run_both(dev, d, cu=None, scale=None, h0=None, fused=True):
+    from fla_hip import pipeline
+    to = lambda t: None if t is None else t.to(dev)
+    o, final = pipeline.flash_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), to(d["g"]), to(d["beta"]),
+                                               scale, to(h0), True, cu_seqlens=cu, fused=fused)
+    o_ref, f_ref = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], scale, h0, True,
+                                              cu_seqlens=cu, naive=True)
+    return o, final, o_ref, f_ref
+
+
+CASES = [
+    # B, T, H, Hk, K, V, cu
+    (2, 256, 2, 2, 128, 128, None),
+    (1, 200, 4, 2, 128, 128, None),                   # GVA, ragged tail
+    (1, 1, 1, 1, 128, 128, None),
+    (1, 63, 2, 2, 128, 128, None),
+    (1, 65, 2, 2, 128, 128, None),
+    (1, 130, 2, 2, 128, 256, None),                   # V = 256
+    (1, 130, 2, 2, 64, 64, None),                     # K = V = 64
+    (1, 192, 8, 8, 128, 128, None),
+    (1, 261, 2, 1, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261]),   # lengths 1,15,17,0,63,64,101
+]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("case", CASES)
+def test_against_naive_recurrence(dev, case, fused):
+    B, T, H, Hk, K, V, cu = case
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=BF, seed=T + H, Hk=Hk)
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, H, K, V, generator=torch.Generator().manual_seed(2)) * 0.01
+    o, final, o_ref, f_ref = run_both(dev, d, cu=cu, h0=h0, fused=fused)
+    assert o.shape == (B, T, H, V) and o.dtype == BF and final.shape == (N, H, K, V) and final.dtype == torch.float32
+    st = assert_close(o, o_ref, TOL_BF16, "o")
+    assert st["rel_max"] < 3e-2, st
+    assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
+
+
+def test_no_initial_state_and_default_scale(dev):
+    from fla_hip import pipeline
+    d = gdn.make_gdn_inputs(2, 128, 2, 128, 128, dtype=BF, seed=3)
+    to = lambda t: t.to(dev)
+    o, final = pipeline.flash_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), to(d["g"]), to(d["beta"]))
+    assert final is None
+    o_ref, _ = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"])
+    assert_close(o, o_ref, TOL_BF16, "o")
+
+
+def test_special_cases_fix_the_formula(dev):
+    """beta = 0: the state only decays, o_t = scale * q_t . (prod decay) S0.  g = 0, beta = 1: plain delta rule."""
+    from fla_hip import pipeline
+    d = gdn.make_gdn_inputs(1, 128, 2, 128, 128, dtype=BF, seed=5)
+    h0 = torch.randn(1, 2, 128, 128, generator=torch.Generator().manual_seed(1))
+    to = lambda t: t.to(dev)
+    beta0 = torch.zeros_like(d["beta"])
+    o, final = pipeline.flash_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), to(d["g"]), to(beta0), 0.5, to(h0), True)
+    G = torch.cumsum(d["g"], 1)                                   # [B,T,H]
+    expect = 0.5 * torch.einsum("bhtk,bhkv->bthv", d["q"].float(), h0) * torch.exp(G)[..., None]
+    assert_close(o, expect, TOL_BF16, "o beta=0")
+    assert_close(final, h0 * torch.exp(G[:, -1])[..., None, None], TOL_STATE, "state beta=0")
+    g0, beta1 = torch.zeros_like(d["g"]), torch.ones_like(d["beta"])
+    o, final = pipeline.flash_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), to(g0), to(beta1), None, None, True)
+    # delta rule with beta = 1 stores v_t exactly under key k_t: S_t^T k_t = v_t  =>  o_t(q = k_t) = scale v_t
+    o2, _ = pipeline.flash_gated_delta_rule(to(d["k"]), to(d["k"]), to(d["v"]), to(g0), to(beta1), 1.0, None, False)
+    assert_close(o2.transpose(1, 2), d["v"].float(), 3e-2, "delta-rule write/read identity")
+
+
+def test_wrapper_errors(dev):
+    from fla_hip import pipeline
+    d = gdn.make_gdn_inputs(1, 64, 2, 128, 128, dtype=BF)
+    to = lambda t: t.to(dev)
+    with pytest.raises(ValueError, match="does not support float32"):
+        pipeline.flash_gated_delta_rule(to(d["q"]).float(), to(d["k"]).float(), to(d["v"]).float(), to(d["g"]), to(d["beta"]))
+    with pytest.raises(ValueError, match="g and beta must be rank-3"):
+        pipeline.flash_gated_delta_rule(to(d["q"]), to(d["k"]), to(d["v"]), to(d["g"])[0], to(d["beta"])[0])
+    with pytest.raises(ValueError, match="batch size is expected to be 1"):
+        q2 = torch.cat([to(d["q"])] * 2)
+        pipeline.flash_gated_delta_rule(q2, q2, q2, torch.cat([to(d["g"])] * 2), torch.cat([to(d["beta"])] * 2),
+                                        cu_seqlens=[0, 32, 64])
+
+
+def test_benchmark_shape(dev):
+    """B=4, T=8192, H=32, K=V=128: oracle on two batch rows; hand-off, route agreement and determinism on all."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 4, 8192, 32, 128, 128
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=BF, seed=0, init_std=0.01)
+    x = {k: v.to(dev) for k, v in d.items()}
+    o, final = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, x["initial_state"], True)
+    # (1) fp32 chunked oracle == naive recurrence to 1e-5 is a CPU test; here the chunked fp32 oracle on rows 0, 3
+    for b in (0, 3):
+        sl = slice(b, b + 1)
+        o_ref, f_ref = gdn.flash_gated_delta_rule(d["q"][sl], d["k"][sl], d["v"][sl], d["g"][sl], d["beta"][sl], None,
+                                                  d["initial_state"][sl], True, naive=False)
+        st = assert_close(o[sl], o_ref, TOL_BF16, f"o row {b}")
+        assert st["rel_max"] < 3e-2, st
+        assert_close(final[sl], f_ref, TOL_STATE, f"final_state row {b}")
+    # (2) state hand-off at a chunk boundary reproduces the single call bit for bit
+    half = T // 2
+    o1, f1 = pipeline.flash_gated_delta_rule(x["q"][:, :, :half], x["k"][:, :, :half], x["v"][:, :, :half],
+                                             x["g"][:, :half], x["beta"][:, :half], None, x["initial_state"], True)
+    o2, f2 = pipeline.flash_gated_delta_rule(x["q"][:, :, half:], x["k"][:, :, half:], x["v"][:, :, half:],
+                                             x["g"][:, half:], x["beta"][:, half:], None, f1, True)
+    assert torch.equal(torch.cat([o1, o2], 1), o)
+    assert torch.equal(f2, final)
+    # (3) the six-operator route agrees within tolerance; (4) reruns are bit-identical
+    o_ops, f_ops = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, x["initial_state"],
+                                                   True, fused=False)
+    assert_close(o_ops, o.float(), TOL_BF16, "ops vs fused o")
+    assert_close(f_ops, final, 4 * TOL_STATE, "ops vs fused state")
+    o_again, f_again = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None,
+                                                       x["initial_state"], True)
+    assert torch.equal(o_again, o) and torch.equal(f_again, final)
