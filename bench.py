@@ -271,12 +271,35 @@ def bench_conv1d(args, torch, dev):
     }
 
 
+def bench_copy(args, torch, dev):
+    """Calibration only (not a product kernel): a plain device-to-device copy of known size, used to
+    scale the FETCH_SIZE / WRITE_SIZE counters and as the practical bandwidth ceiling of the box."""
+    n = 512 * 1024 * 1024  # bytes each way
+    x = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+    y = torch.empty_like(x)
+    for _ in range(args.warmup):
+        y.copy_(x)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        y.copy_(x)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    gbs = 2 * n * args.steps / dt / 1e9
+    return {"metric": "device_copy_GBps", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "torch device copy 512 MiB -> 512 MiB (calibration, not a product kernel)"},
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}, "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d", "copy"])
     ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -293,7 +316,7 @@ def main():
         print("bench.py: no GPU visible.", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d}[args.workload]
+    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d, "copy": bench_copy}[args.workload]
     print(json.dumps(fn(args, torch, dev)))
 
 

@@ -46,15 +46,23 @@ template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
-// Inclusive prefix sum over the 64 lanes of a wave.
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves: four
+// shifts inside each row of 16 lanes (sources outside the row read 0), then lane 15 of rows 0 / 2
+// broadcast into rows 1 / 3 and lane 31 into rows 2 and 3.
+#define FLA_DPP_ADD(v, ctrl, row_mask) \
+    ((v) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), (row_mask), 0xf, true)))
 __device__ __forceinline__ float wave_inclusive_scan(float v) {
-    const int lane = threadIdx.x & 63;
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        float n = __shfl_up(v, off, kWave);
-        if (lane >= off) v += n;
-    }
+    v = FLA_DPP_ADD(v, 0x111, 0xf);  // row_shr:1
+    v = FLA_DPP_ADD(v, 0x112, 0xf);  // row_shr:2
+    v = FLA_DPP_ADD(v, 0x114, 0xf);  // row_shr:4
+    v = FLA_DPP_ADD(v, 0x118, 0xf);  // row_shr:8
+    v = FLA_DPP_ADD(v, 0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    v = FLA_DPP_ADD(v, 0x143, 0xc);  // row_bcast:31 into rows 2 and 3
     return v;
+}
+#undef FLA_DPP_ADD
+__device__ __forceinline__ float read_lane(float v, int lane) {  // lane must be wave-uniform
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
 // ---- MFMA wrappers ---------------------------------------------------------
@@ -73,13 +81,14 @@ __device__ __forceinline__ f32x4 mfma16x16(bf16x4 a, bf16x4 b, f32x4 c) {
                                                      0, 0, 0);
 }
 
+// fp32 -> bf16 (round to nearest even), two values per v_cvt_pk_bf16_f32
+__device__ __forceinline__ bf16x2 cvt2(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_convertvector(v, bf16x2);
+}
 __device__ __forceinline__ bf16x4 cvt4(f32x4 v) {
-    bf16x4 r;
-    r[0] = (bf16)v[0];
-    r[1] = (bf16)v[1];
-    r[2] = (bf16)v[2];
-    r[3] = (bf16)v[3];
-    return r;
+    const bf16x2 lo = cvt2(v[0], v[1]), hi = cvt2(v[2], v[3]);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
 }
 __device__ __forceinline__ bf16x8 cat8(bf16x4 lo, bf16x4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);

@@ -7,21 +7,22 @@
 //
 // One 256-thread workgroup per (sequence, value head, 64*CT-column slab of V) walks the chunks
 // of its sequence.  Wave w owns 16*CT columns of V for all K rows of the state, which stays in
-// fp32 MFMA accumulators for the whole sequence.  Per chunk (C = 64 tokens):
-//   A  scores      wave 0 : the four 16x16 diagonal blocks of beta_i e^{G_i-G_j} <k_i,k_j>, then
-//                           their unit-lower inverses by fp32 forward substitution (lane = column)
-//                  waves 1-3 : the six off-diagonal blocks (stored negated, bf16) and the masked,
-//                           decayed q k^T tile P
+// fp32 MFMA accumulators for the whole sequence.  Per chunk (C = 64 tokens, 16-token blocks):
+//   A  scores      wave w: row block w of  A0 = beta_i e^{G_i-G_j} <k_i,k_j>  (off-diagonal blocks
+//                  stored negated as bf16; the diagonal block inverted in registers with the
+//                  nilpotent product (I-A)(I+A^2)(I+A^4)(I+A^8), eight 16x16x16 MFMAs) and row
+//                  block 3-w of the masked, decayed q k^T tile P  (5 tiles per wave)
 //   B  WY solve    block forward substitution X_i = D_i^-1 (B_i - sum_{j<i} A_ij X_j) on the
 //                  right-hand sides [k beta e^G | v beta]; X_j feeds the next block product
 //                  straight from accumulator registers.  Wave w solves its own u columns (kept
-//                  in registers, residuals as hi+lo bf16 pairs) and two 16-column tiles of w
-//                  (rounded to bf16 into LDS, since w is an MFMA operand next)
+//                  in fp32 registers, residuals fed as hi+lo bf16 pairs) and K/64 16-column
+//                  tiles of w (rounded to bf16 into LDS, since w is an MFMA operand next)
 //   C  scan        v_new = u - w h ; o = scale (e^G (q h) + P v_new) ;
-//                  h <- e^{g_last} h + k^T (v_new e^{g_last - g})   (v_new e^.. as hi+lo bf16)
-//   D  epilogue    o tile stored; the next chunk's q/k/v, prefetched into registers during A-C,
-//                  are written to LDS
-// Math and rounding points: SURVEY of the reference stages in chunk_scaled_dot_kkt/README.md:11-29,
+//                  h <- e^{g_last} h + k^T (v_new e^{g_last - g})   (right operand as hi+lo bf16)
+// The next chunk's q/k/v rows are prefetched into registers at the top of a chunk and written to
+// the second LDS buffer between B and C, so HBM latency hides behind A and B.  LDS operand reads
+// are software-pipelined by hand one k-step ahead of the MFMAs that consume them.
+// Math and rounding points of the stages: chunk_scaled_dot_kkt/README.md:11-29,
 // recompute_w_u_fwd/README.md:12-32, chunk_gated_delta_rule_fwd_h/README.md:16-30,
 // chunk_fwd_o/README.md:6-15; acceptance oracle examples/flash_gated_delta_rule.py:1545-1571.
 #include "gdn_common.h"
@@ -31,6 +32,23 @@ namespace fla {
 namespace {
 
 constexpr int kThreads = 256;
+
+#ifdef FLA_NO_FENCE
+#define FLA_SCHED_FENCE()
+#else
+#define FLA_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#endif
+
+#ifdef FLA_FUSED_TIMING
+#define FLA_TICK(i)                      \
+    {                                    \
+        long long now_ = clock64();      \
+        tacc[i] += now_ - tlast;         \
+        tlast = now_;                    \
+    }
+#else
+#define FLA_TICK(i)
+#endif
 
 struct FusedParams {
     ChunkGeom geom;
@@ -48,77 +66,177 @@ struct FusedParams {
 
 template <int K, int CT> struct FusedSmem {
     static constexpr int VS = 64 * CT;
-    static constexpr int pq = K + 8, pk = K + 16, pv = VS + 16, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
-                         po = VS + 8, pd = 24, a32_blk = 16 * 16 + 16;
-    static constexpr size_t q_off = 0;
-    static constexpr size_t k_off = q_off + (size_t)kChunk * pq * 2;
-    static constexpr size_t v_off = k_off + (size_t)kChunk * pk * 2;
-    static constexpr size_t a_off = v_off + (size_t)kChunk * pv * 2;
+    static constexpr bool DB = CT == 1;   // q/k/v tiles double-buffered in LDS
+    static constexpr int NB = DB ? 2 : 1;
+    static constexpr int pq = K + 8, pk = KTile<K>::pitch, pv = VS + 16, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
+                         po = VS + 8, pd = 24;
+    static constexpr size_t q_bytes = (size_t)kChunk * pq * 2, k_bytes = (size_t)kChunk * pk * 2,
+                            v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (6 * kChunk + 16) * 4;
+    static constexpr size_t buf_bytes = q_bytes + k_bytes + v_bytes + tab_bytes;
+    static constexpr size_t a_off = NB * buf_bytes;
     static constexpr size_t w_off = a_off + (size_t)kChunk * pa * 2;
     static constexpr size_t p_off = w_off + (size_t)kChunk * pw * 2;
     static constexpr size_t o_off = p_off + (size_t)kChunk * pp * 2;
     static constexpr size_t d_off = o_off + (size_t)kChunk * po * 2;
-    static constexpr size_t a32_off = d_off + (size_t)4 * 16 * pd * 2;
-    static constexpr size_t tab_off = a32_off + (size_t)4 * a32_blk * 4;
-    static constexpr size_t bytes = tab_off + 4 * kChunk * 4;
+    static constexpr size_t bytes = d_off + (size_t)kChunk * pd * 2;
 };
 
-// D^-1 R for one 16x16 diagonal block; HILO feeds R as hi + lo bf16 pairs.
-template <bool HILO>
-__device__ __forceinline__ f32x4 diag_mul(const bf16 *dblk, int pd, f32x4 r) {
-    const bf16x4 a = frag_kc4(dblk, pd, 0, 0);
+struct Tiles {      // one LDS buffer of chunk inputs
+    bf16 *q, *k, *v;
+    // per token: cumulated gate G, scale e^G, beta, beta e^G, and the factors of
+    //   e^{G_t - G_s} = ROWF[t] * BLKF[blk(t)][blk(s)] * COLF[s]   for blk(s) < blk(t)
+    // with ROWF[t] = e^{G_t - G(first token of blk(t))}, COLF[s] = e^{G(last token of blk(s)) - G_s};
+    // every factor is <= 1 for non-positive gates, so nothing overflows.
+    float *G, *EGS, *B, *BEG, *ROWF, *COLF, *BLKF;
+};
+template <int K, int CT>
+__device__ __forceinline__ Tiles tiles_at(unsigned char *smem, int buf) {
+    typedef FusedSmem<K, CT> L;
+    unsigned char *b = smem + buf * L::buf_bytes;
+    Tiles t;
+    t.q = reinterpret_cast<bf16 *>(b);
+    t.k = reinterpret_cast<bf16 *>(b + L::q_bytes);
+    t.v = reinterpret_cast<bf16 *>(b + L::q_bytes + L::k_bytes);
+    t.G = reinterpret_cast<float *>(b + L::q_bytes + L::k_bytes + L::v_bytes);
+    t.EGS = t.G + kChunk;
+    t.B = t.EGS + kChunk;
+    t.BEG = t.B + kChunk;
+    t.ROWF = t.BEG + kChunk;
+    t.COLF = t.ROWF + kChunk;
+    t.BLKF = t.COLF + kChunk;
+    return t;
+}
+
+__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+__device__ __forceinline__ f32x4 lds4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+
+// ---------------------------------------------------------------------------------------------
+// Phase A for wave W: row block I1 = W of the score matrix, row block I2 = 3 - W of P.
+// ---------------------------------------------------------------------------------------------
+template <int K, int W>
+__device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16 *dS, float scale) {
+    constexpr int I1 = W, I2 = 3 - W, JM = I1 > I2 ? I1 : I2, KS = K / 32;
+    constexpr int pq = K + 8, pa = kChunk + 8, pp = kChunk + 8, pd = 24;
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+
+    f32x4 kacc[I1 + 1], pacc[I2 + 1];
+#pragma unroll
+    for (int J = 0; J <= I1; ++J) kacc[J] = zero4();
+#pragma unroll
+    for (int J = 0; J <= I2; ++J) pacc[J] = zero4();
+    bf16x8 kf[2][JM + 1], qf[2];
+#pragma unroll
+    for (int J = 0; J <= JM; ++J) kf[0][J] = KTile<K>::kc(t.k, 16 * J, 0);
+    qf[0] = frag_kc(t.q, pq, 16 * I2, 0);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int cb = s & 1, nb = cb ^ 1;
+        if (s + 1 < KS) {
+#pragma unroll
+            for (int J = 0; J <= JM; ++J) kf[nb][J] = KTile<K>::kc(t.k, 16 * J, 32 * (s + 1));
+            qf[nb] = frag_kc(t.q, pq, 16 * I2, 32 * (s + 1));
+        }
+        FLA_SCHED_FENCE();
+        // rows of the tile = tokens s of block J (A operand), columns = tokens t of block I (B operand)
+#pragma unroll
+        for (int J = 0; J <= I1; ++J) kacc[J] = mfma16x32(kf[cb][J], kf[cb][I1], kacc[J]);
+#pragma unroll
+        for (int J = 0; J <= I2; ++J) pacc[J] = mfma16x32(kf[cb][J], qf[cb], pacc[J]);
+        FLA_SCHED_FENCE();
+    }
+
+    // lane holds (row s = 16J + 4lg + e, column t = 16I + li) of each tile
+    const int t1 = 16 * I1 + li, t2 = 16 * I2 + li;
+    const float gt1 = t.G[t1], bt1 = t.B[t1], gt2 = t.G[t2];
+    const float rf1 = -bt1 * t.ROWF[t1], rf2 = scale * t.ROWF[t2];
+#pragma unroll
+    for (int J = 0; J < I1; ++J) {  // off-diagonal score blocks, negated: -beta_t e^{G_t-G_s} <k_s,k_t>
+        const f32x4 cf = lds4(t.COLF + 16 * J + 4 * lg);
+        const float coef = rf1 * t.BLKF[4 * I1 + J];
+        f32x4 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = coef * cf[e] * kacc[J][e];
+        *reinterpret_cast<bf16x4 *>(aS + t1 * pa + 16 * J + 4 * lg) = cvt4(a);
+    }
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {  // scale * P[t][s] = scale q_t.k_s e^{min(G_t-G_s,0)} for s <= t
+        f32x4 a = zero4();
+        if (J < I2) {
+            const f32x4 cf = lds4(t.COLF + 16 * J + 4 * lg);
+            const float coef = rf2 * t.BLKF[4 * I2 + J];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = coef * cf[e] * pacc[J < I2 ? J : 0][e];
+        } else if (J == I2) {
+            const f32x4 gs = lds4(t.G + 16 * J + 4 * lg);
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                a[e] = 4 * lg + e <= li ? scale * __expf(fminf(gt2 - gs[e], 0.f)) * pacc[I2][e] : 0.f;
+        }
+        *reinterpret_cast<bf16x4 *>(pS + t2 * pp + 16 * J + 4 * lg) = cvt4(a);
+    }
+
+    // diagonal block A (16x16, strictly lower): both operand views from the symmetric raw tile
+    const f32x4 gs = lds4(t.G + 16 * I1 + 4 * lg), bs = lds4(t.B + 16 * I1 + 4 * lg);
+    f32x4 a1, a2, Y;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int r = 4 * lg + e;
+        const float raw = kacc[I1][e];
+        a1[e] = r < li ? bt1 * __expf(fmaxf(gt1 - gs[e], -50.f)) * raw : 0.f;    // A[li][r]
+        a2[e] = li < r ? bs[e] * __expf(fmaxf(gs[e] - gt1, -50.f)) * raw : 0.f;  // A[r][li]
+        Y[e] = (r == li ? 1.f : 0.f) - a1[e];                                     // (I - A^T)[r][li]
+    }
+    // An accumulator tile of M is the right operand of M and the left operand of M^T, so the
+    // chains S_k = A^(2^k) and T_k = S_k^T are advanced together and
+    //   Y <- Y + T_k Y   accumulates   Y = ((I-A)(I+A^2)(I+A^4)(I+A^8))^T = ((I+A)^-1)^T.
+    const bf16x4 A1 = cvt4(a1), A2 = cvt4(a2);
+    const f32x4 S1 = mfma16x16(A1, A2, zero4());
+    const f32x4 T1 = mfma16x16(A2, A1, zero4());
+    const bf16x4 S1b = cvt4(S1), T1b = cvt4(T1);
+    Y = mfma16x16(S1b, cvt4(Y), Y);
+    const f32x4 S2 = mfma16x16(T1b, S1b, zero4());
+    const f32x4 T2 = mfma16x16(S1b, T1b, zero4());
+    const bf16x4 S2b = cvt4(S2);
+    Y = mfma16x16(S2b, cvt4(Y), Y);
+    const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());
+    Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
+    // lane holds Dinv^T[4lg+e][li] = Dinv[li][4lg+e]: the left-operand layout, 8 contiguous bytes
+    *reinterpret_cast<bf16x4 *>(dS + (16 * I1 + li) * pd + 4 * lg) = cvt4(Y);
+}
+
+// D^-1 R for one diagonal block; hilo feeds R as hi + lo bf16 pairs.
+__device__ __forceinline__ f32x4 diag_mul(bf16x4 d, f32x4 r, bool hilo) {
     const bf16x4 hi = cvt4(r);
-    f32x4 acc = mfma16x16(a, hi, f32x4{0.f, 0.f, 0.f, 0.f});
-    if (HILO) {
+    f32x4 acc = mfma16x16(d, hi, zero4());
+    if (hilo) {
         f32x4 rest;
 #pragma unroll
         for (int e = 0; e < 4; ++e) rest[e] = r[e] - (float)hi[e];
-        acc = mfma16x16(a, cvt4(rest), acc);
+        acc = mfma16x16(d, cvt4(rest), acc);
     }
     return acc;
-}
-
-// Block forward substitution for one 16-column tile.  In: r[i] = rows 16i..16i+15 of the
-// right-hand side (accumulator layout).  Out: r[i] = the same rows of (I + A0)^-1 RHS.
-// aS holds -A0 (bf16), dS the four inverted diagonal blocks.
-template <bool HILO>
-__device__ __forceinline__ void wy_solve_tile(const bf16 *aS, int pa, const bf16 *dS, int pd, f32x4 (&r)[4]) {
-    r[0] = diag_mul<HILO>(dS, pd, r[0]);
-    r[1] = mfma16x16(frag_kc4(aS, pa, 16, 0), cvt4(r[0]), r[1]);
-    r[1] = diag_mul<HILO>(dS + 16 * pd, pd, r[1]);
-    const bf16x8 x01 = frag_from_acc(r[0], r[1]);
-    r[2] = mfma16x32(frag_kc(aS, pa, 32, 0), x01, r[2]);
-    r[2] = diag_mul<HILO>(dS + 32 * pd, pd, r[2]);
-    r[3] = mfma16x32(frag_kc(aS, pa, 48, 0), x01, r[3]);
-    r[3] = mfma16x16(frag_kc4(aS, pa, 48, 32), cvt4(r[2]), r[3]);
-    r[3] = diag_mul<HILO>(dS + 48 * pd, pd, r[3]);
 }
 
 template <int K, int CT>
 __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p) {
     typedef FusedSmem<K, CT> L;
-    constexpr int VS = L::VS, pq = L::pq, pk = L::pk, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, po = L::po,
+    constexpr int VS = L::VS, pq = L::pq, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, po = L::po,
                   pd = L::pd;
+    constexpr bool DB = L::DB;
     constexpr int KT = K / 16, KS = K / 32;
-    constexpr int QCH = kChunk * (K / 8) / kThreads;    // 16-byte chunks of a q/k tile per thread
+    constexpr int QCH = kChunk * (K / 8) / kThreads;    // 16-byte pieces of a q/k tile per thread
     constexpr int VCH = kChunk * (VS / 8) / kThreads;   // ... of the v slab tile
+    constexpr int QROWS = kThreads / (K / 8), VROWS = kThreads / (VS / 8);
+    constexpr int NTW = K / 64, NT = NTW + CT;          // w tiles per wave, all solved tiles per wave
     extern __shared__ __align__(16) unsigned char smem[];
-    bf16 *qS = reinterpret_cast<bf16 *>(smem + L::q_off);
-    bf16 *kS = reinterpret_cast<bf16 *>(smem + L::k_off);
-    bf16 *vS = reinterpret_cast<bf16 *>(smem + L::v_off);
     bf16 *aS = reinterpret_cast<bf16 *>(smem + L::a_off);
     bf16 *wS = reinterpret_cast<bf16 *>(smem + L::w_off);
     bf16 *pS = reinterpret_cast<bf16 *>(smem + L::p_off);
     bf16 *oS = reinterpret_cast<bf16 *>(smem + L::o_off);
     bf16 *dS = reinterpret_cast<bf16 *>(smem + L::d_off);
-    float *a32 = reinterpret_cast<float *>(smem + L::a32_off);
-    float *GS = reinterpret_cast<float *>(smem + L::tab_off);  // cumulated gate G_t
-    float *EG = GS + kChunk;                                    // e^{G_t}
-    float *BS = EG + kChunk;                                    // beta_t
-    float *BEG = BS + kChunk;                                   // beta_t e^{G_t}
 
     // ---- which (sequence, head, slab) ---------------------------------------------------
-    int lin = blockIdx.x;
+    const int lin = blockIdx.x;
     int slab, hv, n;
     if (p.remap) {  // blocks L and L+8 run on the same XCD: make them the two slabs of one head
         const int pair = (lin >> 4) * 8 + (lin & 7);
@@ -151,7 +269,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            f32x4 a = zero4();
             if (p.h0) {
                 const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
 #pragma unroll
@@ -160,188 +278,191 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
             hacc[kt][ct] = a;
         }
 
-    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
-    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + slab * VS;
-    bf16 *og = static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + slab * VS;
+    // ---- prefetch addressing: one uniform base per tensor and chunk, 32-bit per-lane byte offsets
+    // (row r of the chunk, 8 columns from cq / cv) computed once ------------------------------------
+    const int rq = tid / (K / 8), cq = (tid % (K / 8)) * 8;
+    const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
+    const char *qbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
+    const char *kbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
+    const char *vbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
+    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + slab * VS);
+    unsigned qoff[QCH], koff[QCH], voff[VCH], ooff[VCH];
+#pragma unroll
+    for (int m = 0; m < QCH; ++m) {
+        qoff[m] = (unsigned)(((rq + m * QROWS) * p.q.st + cq) * 2);
+        koff[m] = (unsigned)(((rq + m * QROWS) * p.k.st + cq) * 2);
+    }
+#pragma unroll
+    for (int m = 0; m < VCH; ++m) {
+        voff[m] = (unsigned)(((rv + m * VROWS) * p.v.st + cv) * 2);
+        ooff[m] = (unsigned)(((rv + m * VROWS) * p.o.st + cv) * 2);
+    }
 
-    // ---- register prefetch of one chunk's q, k, v rows and gates ------------------------------
+    const float *gptr = static_cast<const float *>(p.g.p) + b * p.g.sb + hv * p.g.sh;
+    const float *bptr = static_cast<const float *>(p.beta.p) + b * p.beta.sb + hv * p.beta.sh;
     u32x4 pre_q[QCH], pre_k[QCH], pre_v[VCH];
     float pre_g = 0.f, pre_b = 0.f;
-    auto prefetch = [&](int c) {
+    auto prefetch = [&](int c) {  // global -> registers
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
+        const char *qb = qbase + (int64_t)c * kChunk * p.q.st * 2, *kb = kbase + (int64_t)c * kChunk * p.k.st * 2,
+                   *vb = vbase + (int64_t)c * kChunk * p.v.st * 2;
+        if (len == kChunk) {
 #pragma unroll
-        for (int m = 0; m < QCH; ++m) {
-            const int idx = tid + m * kThreads, r = idx / (K / 8), cc = (idx % (K / 8)) * 8;
-            u32x4 zq = {0u, 0u, 0u, 0u}, zk = zq;
-            if (r < len) {
-                zq = *reinterpret_cast<const u32x4 *>(qg + (int64_t)(start + r) * p.q.st + cc);
-                zk = *reinterpret_cast<const u32x4 *>(kg + (int64_t)(start + r) * p.k.st + cc);
+            for (int m = 0; m < QCH; ++m) {
+                pre_q[m] = *reinterpret_cast<const u32x4 *>(qb + qoff[m]);
+                pre_k[m] = *reinterpret_cast<const u32x4 *>(kb + koff[m]);
             }
-            pre_q[m] = zq;
-            pre_k[m] = zk;
-        }
 #pragma unroll
-        for (int m = 0; m < VCH; ++m) {
-            const int idx = tid + m * kThreads, r = idx / (VS / 8), cc = (idx % (VS / 8)) * 8;
-            u32x4 z = {0u, 0u, 0u, 0u};
-            if (r < len) z = *reinterpret_cast<const u32x4 *>(vg + (int64_t)(start + r) * p.v.st + cc);
-            pre_v[m] = z;
+            for (int m = 0; m < VCH; ++m) pre_v[m] = *reinterpret_cast<const u32x4 *>(vb + voff[m]);
+        } else {
+            const u32x4 z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int m = 0; m < QCH; ++m) {
+                const bool in = rq + m * QROWS < len;
+                pre_q[m] = in ? *reinterpret_cast<const u32x4 *>(qb + qoff[m]) : z;
+                pre_k[m] = in ? *reinterpret_cast<const u32x4 *>(kb + koff[m]) : z;
+            }
+#pragma unroll
+            for (int m = 0; m < VCH; ++m)
+                pre_v[m] = rv + m * VROWS < len ? *reinterpret_cast<const u32x4 *>(vb + voff[m]) : z;
         }
-        if (tid < kChunk) {
-            pre_g = tid < len ? load_scalar(p.g, b, hv, start + tid) : 0.f;
-            pre_b = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
+        if (tid < len) {  // fp32 gates: plain loads, no dtype branch whose join would wait for them
+            pre_g = gptr[(int64_t)(start + tid) * p.g.st];
+            pre_b = bptr[(int64_t)(start + tid) * p.beta.st];
+        } else {
+            pre_g = 0.f;
+            pre_b = 0.f;
         }
     };
-    auto commit = [&](int c) {  // prefetched registers -> LDS tiles and gate tables of chunk c
+    auto commit = [&](int c, const Tiles &t) {  // registers -> LDS tiles and gate tables of chunk c
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
 #pragma unroll
         for (int m = 0; m < QCH; ++m) {
-            const int idx = tid + m * kThreads, r = idx / (K / 8), cc = (idx % (K / 8)) * 8;
-            *reinterpret_cast<u32x4 *>(qS + r * pq + cc) = pre_q[m];
-            *reinterpret_cast<u32x4 *>(kS + r * pk + cc) = pre_k[m];
+            *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = pre_q[m];
+            *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = pre_k[m];
         }
 #pragma unroll
-        for (int m = 0; m < VCH; ++m) {
-            const int idx = tid + m * kThreads, r = idx / (VS / 8), cc = (idx % (VS / 8)) * 8;
-            *reinterpret_cast<u32x4 *>(vS + r * pv + cc) = pre_v[m];
-        }
+        for (int m = 0; m < VCH; ++m) *reinterpret_cast<u32x4 *>(t.v + (rv + m * VROWS) * pv + cv) = pre_v[m];
         if (wv == 0) {  // wave 0 holds token t = lane: chunk-local cumulative gate
             float G = wave_inclusive_scan(pre_g);
-            const float g_end = __shfl(G, len - 1, kWave);
+            const float g_end = read_lane(G, len - 1);
             if (l >= len) G = g_end;  // padded rows: finite, harmless (their q, k, v, beta are zero)
+            // gate at the first / last token of each 16-token block
+            const float s0 = read_lane(G, 0), s1 = read_lane(G, 16), s2 = read_lane(G, 32), s3 = read_lane(G, 48);
+            const float e0 = read_lane(G, 15), e1 = read_lane(G, 31), e2 = read_lane(G, 47), e3 = read_lane(G, 63);
+            const int blk = l >> 4;
+            const float Gs = blk == 0 ? s0 : (blk == 1 ? s1 : (blk == 2 ? s2 : s3));
+            const float Ge = blk == 0 ? e0 : (blk == 1 ? e1 : (blk == 2 ? e2 : e3));
+            const int bi = (l >> 2) & 3, bj = l & 3;
+            const float gsI = bi == 0 ? s0 : (bi == 1 ? s1 : (bi == 2 ? s2 : s3));
+            const float geJ = bj == 0 ? e0 : (bj == 1 ? e1 : (bj == 2 ? e2 : e3));
             const float eg = __expf(G);
-            GS[l] = G;
-            EG[l] = eg;
-            BS[l] = pre_b;
-            BEG[l] = pre_b * eg;
+            t.G[l] = G;
+            t.EGS[l] = eg * p.scale;
+            t.B[l] = pre_b;
+            t.BEG[l] = pre_b * eg;
+            t.ROWF[l] = __expf(G - Gs);
+            t.COLF[l] = __expf(Ge - G);
+            if (l < 16) t.BLKF[l] = bj < bi ? __expf(gsI - geJ) : 0.f;
             if (p.g_out != nullptr && slab == 0 && l < len)
                 p.g_out[b * p.go_sb + hv * p.go_sh + (int64_t)(start + l) * p.go_st] = G;
         }
     };
+    auto store_o = [&](int c) {  // staged o tile of chunk c -> HBM, 16 bytes per lane
+        const int len = min(kChunk, eos - (bos + c * kChunk));
+        char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
+#pragma unroll
+        for (int m = 0; m < VCH; ++m)
+            if (rv + m * VROWS < len)
+                *reinterpret_cast<u32x4 *>(ob + ooff[m]) = *reinterpret_cast<const u32x4 *>(oS + (rv + m * VROWS) * po + cv);
+    };
 
     if (nchunks > 0) {
         prefetch(0);
-        commit(0);
+        commit(0, tiles_at<K, CT>(smem, 0));
     }
     __syncthreads();
+#ifdef FLA_FUSED_TIMING
+    long long tacc[16] = {0};
+#endif
 
     for (int c = 0; c < nchunks; ++c) {
-        const int start = bos + c * kChunk;
-        const int len = min(kChunk, eos - start);
+        const int len = min(kChunk, eos - (bos + c * kChunk));
+        const Tiles t = tiles_at<K, CT>(smem, DB ? (c & 1) : 0);
+#ifdef FLA_FUSED_TIMING
+        long long tlast = clock64();
+#endif
+        if (DB && c > 0) store_o(c - 1);
         if (c + 1 < nchunks) prefetch(c + 1);
+        FLA_TICK(0)
 
         // =========================== A: scores ===========================================
-        if (wv == 0) {
-            // diagonal blocks: fp32 into a32 (strictly lower part, rest zero)
-#pragma unroll
-            for (int I = 0; I < 4; ++I) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int kk = 0; kk < K; kk += 32)
-                    acc = mfma16x32(frag_kc(kS, pk, I * 16, kk), frag_kc(kS, pk, I * 16, kk), acc);
-                // lane holds <k_s, k_t> for s = 16I + 4lg + e (row), t = 16I + li (column)
-                const int t = I * 16 + li;
-                const float gt = GS[t], bt = BS[t];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int s = I * 16 + 4 * lg + e;
-                    acc[e] = s < t ? bt * __expf(fmaxf(gt - GS[s], -50.f)) * acc[e] : 0.f;
-                }
-                *reinterpret_cast<f32x4 *>(a32 + I * L::a32_blk + li * 16 + 4 * lg) = acc;
-            }
-            __builtin_amdgcn_wave_barrier();
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            // inverse of (I + A_II): lane = (block, column j); x[i] = row i of that column
-            const int blk = lg, j = li;
-            const float *ab = a32 + blk * L::a32_blk;
-            float x[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) x[i] = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float acc = (i == j) ? 1.f : 0.f;
-#pragma unroll
-                for (int s4 = 0; s4 < (i + 3) / 4; ++s4) {
-                    const f32x4 a = *reinterpret_cast<const f32x4 *>(ab + i * 16 + 4 * s4);
-                    acc -= a[0] * x[4 * s4] + a[1] * x[4 * s4 + 1] + a[2] * x[4 * s4 + 2] + a[3] * x[4 * s4 + 3];
-                }
-                x[i] = acc;
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) dS[(blk * 16 + i) * pd + j] = (bf16)x[i];
-        } else {
-            // 6 off-diagonal score blocks + 16 tiles of P (10 computed, 6 zero) over waves 1..3
-            for (int id = wv - 1; id < 22; id += 3) {
-                if (id < 6) {
-                    // (I, J): (1,0) (2,0) (2,1) (3,0) (3,1) (3,2)
-                    const int I = id < 1 ? 1 : (id < 3 ? 2 : 3);
-                    const int J = id < 1 ? 0 : (id < 3 ? id - 1 : id - 3);
-                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int kk = 0; kk < K; kk += 32)
-                        acc = mfma16x32(frag_kc(kS, pk, J * 16, kk), frag_kc(kS, pk, I * 16, kk), acc);
-                    const int t = I * 16 + li;
-                    const float gt = GS[t], bt = BS[t];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int s = J * 16 + 4 * lg + e;
-                        acc[e] = -bt * __expf(fmaxf(gt - GS[s], -50.f)) * acc[e];
-                    }
-                    *reinterpret_cast<bf16x4 *>(aS + t * pa + J * 16 + 4 * lg) = cvt4(acc);
-                } else {
-                    const int pid = id - 6, I = pid >> 2, J = pid & 3;  // t block, s block
-                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-                    const int t = I * 16 + li;
-                    if (J <= I) {
-#pragma unroll
-                        for (int kk = 0; kk < K; kk += 32)
-                            acc = mfma16x32(frag_kc(kS, pk, J * 16, kk), frag_kc(qS, pq, I * 16, kk), acc);
-                        const float gt = GS[t];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int s = J * 16 + 4 * lg + e;
-                            acc[e] = s <= t ? acc[e] * __expf(fminf(gt - GS[s], 0.f)) : 0.f;
-                        }
-                    }
-                    *reinterpret_cast<bf16x4 *>(pS + t * pp + J * 16 + 4 * lg) = cvt4(acc);
-                }
-            }
+        switch (wv) {
+            case 0: phase_a<K, 0>(t, aS, pS, dS, p.scale); break;
+            case 1: phase_a<K, 1>(t, aS, pS, dS, p.scale); break;
+            case 2: phase_a<K, 2>(t, aS, pS, dS, p.scale); break;
+            default: phase_a<K, 3>(t, aS, pS, dS, p.scale); break;
         }
+        FLA_TICK(1)
         __syncthreads();  // #1: aS, dS, pS complete
+        FLA_TICK(2)
 
         // =========================== B: WY solve =========================================
-        f32x4 U[4][CT];
+        // tiles 0..CT-1: this wave's u columns; tiles CT..NT-1: its w columns
+        f32x4 r[NT][4];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            f32x4 r[4];
+        for (int i = 0; i < 4; ++i) {
+            const f32x4 b4 = lds4(t.B + 16 * i + 4 * lg), be4 = lds4(t.BEG + 16 * i + 4 * lg);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bf16x4 vv = frag_tr4(vS, pv, (vtile0 + ct) * 16, 16 * i);
+            for (int ct = 0; ct < CT; ++ct) {
+                const bf16x4 vv = frag_tr4(t.v, pv, (vtile0 + ct) * 16, 16 * i);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) r[i][e] = (float)vv[e] * BS[16 * i + 4 * lg + e];
+                for (int e = 0; e < 4; ++e) r[ct][i][e] = (float)vv[e] * b4[e];
             }
-            wy_solve_tile<true>(aS, pa, dS, pd, r);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) U[i][ct] = r[i];
+            for (int m = 0; m < NTW; ++m) {
+                const bf16x4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[CT + m][i][e] = (float)kv[e] * be4[e];
+            }
+        }
+        {
+            const bf16x4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
+                         d3 = frag_kc4(dS, pd, 48, 0);
+            const bf16x4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
+            const bf16x8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
+            FLA_SCHED_FENCE();
+            bf16x8 x01[NT];
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][0] = diag_mul(d0, r[q][0], q < CT);
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][1] = mfma16x16(a10, cvt4(r[q][0]), r[q][1]);
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][1] = diag_mul(d1, r[q][1], q < CT);
+#pragma unroll
+            for (int q = 0; q < NT; ++q) {
+                x01[q] = frag_from_acc(r[q][0], r[q][1]);
+                r[q][2] = mfma16x32(a2x, x01[q], r[q][2]);
+                r[q][3] = mfma16x32(a3x, x01[q], r[q][3]);
+            }
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][2] = diag_mul(d2, r[q][2], q < CT);
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][3] = mfma16x16(a32, cvt4(r[q][2]), r[q][3]);
+#pragma unroll
+            for (int q = 0; q < NT; ++q) r[q][3] = diag_mul(d3, r[q][3], q < CT);
         }
 #pragma unroll
-        for (int m = 0; m < K / 64; ++m) {
-            const int ctile = wv * (K / 64) + m;
-            f32x4 r[4];
+        for (int m = 0; m < NTW; ++m)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bf16x4 kv = frag_tr4(kS, pk, ctile * 16, 16 * i);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) r[i][e] = (float)kv[e] * BEG[16 * i + 4 * lg + e];
-            }
-            wy_solve_tile<false>(aS, pa, dS, pd, r);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc_to_tile(wS, pw, 16 * i, ctile * 16, r[i]);
-        }
-        __syncthreads();  // #2: wS complete
+            for (int i = 0; i < 4; ++i) acc_to_tile(wS, pw, 16 * i, (wv * NTW + m) * 16, -r[CT + m][i]);
+        FLA_TICK(6)
+        if (DB && c + 1 < nchunks) commit(c + 1, tiles_at<K, CT>(smem, (c + 1) & 1));
+        FLA_TICK(7)
+        __syncthreads();  // #2: wS complete (and, double-buffered, the next chunk's tiles)
+        FLA_TICK(3)
 
         // =========================== C: scan + output ====================================
         bf16x8 hB[KS][CT];
@@ -350,102 +471,144 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
 
-        f32x4 oacc[4][CT];
+        // wS holds -w:  U = u + (-w) h = v_new ;  oacc = q h
+        f32x4 U[4][CT], oacc[4][CT];
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-        // U <- v_new = u - w h (accumulated as -(w h - u)) ; oacc <- q h
-#pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) U[rt][ct] *= -1.f;
-#pragma unroll
-        for (int j = 0; j < KS; ++j)
+            for (int ct = 0; ct < CT; ++ct) {
+                U[rt][ct] = r[ct][rt];
+                oacc[rt][ct] = zero4();
+            }
+        {
+            bf16x8 wf[2][4], qf[2][4];
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
-                const bf16x8 wf = frag_kc(wS, pw, rt * 16, 32 * j);
-                const bf16x8 qf = frag_kc(qS, pq, rt * 16, 32 * j);
+                wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
+                qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
+            }
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    oacc[rt][ct] = mfma16x32(qf, hB[j][ct], oacc[rt][ct]);
-                    U[rt][ct] = mfma16x32(wf, hB[j][ct], U[rt][ct]);
+            for (int j = 0; j < KS; ++j) {
+                const int cb = j & 1, nb = cb ^ 1;
+                if (j + 1 < KS) {
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt) {
+                        wf[nb][rt] = frag_kc(wS, pw, rt * 16, 32 * (j + 1));
+                        qf[nb][rt] = frag_kc(t.q, pq, rt * 16, 32 * (j + 1));
+                    }
                 }
+                FLA_SCHED_FENCE();
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        U[rt][ct] = mfma16x32(wf[cb][rt], hB[j][ct], U[rt][ct]);
+                        oacc[rt][ct] = mfma16x32(qf[cb][rt], hB[j][ct], oacc[rt][ct]);
+                    }
+                FLA_SCHED_FENCE();
             }
+        }
+        FLA_TICK(8)
+        // operands of the next two products, issued before the element-wise work below
+        bf16x8 pf[2][4], kfa[KT];
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) U[rt][ct] *= -1.f;
+            for (int rt = 0; rt < 4; ++rt) pf[j][rt] = frag_kc(pS, pp, rt * 16, 32 * j);
+        f32x4 eg4[4], dk4[4];
+        const float g_last = t.G[len - 1];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            eg4[rt] = lds4(t.EGS + 16 * rt + 4 * lg);
+            dk4[rt] = lds4(t.G + 16 * rt + 4 * lg);
+        }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) kfa[kt] = KTile<K>::tr(t.k, kt * 16, 0);
+        FLA_SCHED_FENCE();
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dk4[rt][e] = __expf(g_last - dk4[rt][e]);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] *= eg4[rt];  // scale e^{G_t} (q h)
+        }
+        FLA_TICK(9)
         // o = scale (e^{G_t} q h + P v_new)
-#pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float eg = EG[rt * 16 + 4 * lg + e];
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) oacc[rt][ct][e] *= eg;
-            }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             bf16x8 vb[CT];
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) vb[ct] = frag_from_acc(U[2 * j][ct], U[2 * j + 1][ct]);
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) {
-                const bf16x8 pf = frag_kc(pS, pp, rt * 16, 32 * j);
+            for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] = mfma16x32(pf, vb[ct], oacc[rt][ct]);
-            }
+                for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] = mfma16x32(pf[j][rt], vb[ct], oacc[rt][ct]);
         }
-#pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc_to_tile(oS, po, rt * 16, (vtile0 + ct) * 16, oacc[rt][ct] * p.scale);
-
+        FLA_TICK(10)
         // h <- e^{g_last} h + k^T (v_new e^{g_last - g}), the right operand as hi + lo bf16
-        const float g_last = GS[len - 1];
         const float dec_all = __expf(g_last);
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= dec_all;
+        bf16x8 vhi[2][CT], vlo[2][CT];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            bf16x8 vhi[CT], vlo[CT];
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                f32x4 a0 = U[2 * j][ct], a1 = U[2 * j + 1][ct], r0, r1;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    a0[e] *= __expf(g_last - GS[32 * j + 4 * lg + e]);
-                    a1[e] *= __expf(g_last - GS[32 * j + 16 + 4 * lg + e]);
-                }
+                const f32x4 a0 = U[2 * j][ct] * dk4[2 * j], a1 = U[2 * j + 1][ct] * dk4[2 * j + 1];
                 const bf16x4 h0 = cvt4(a0), h1 = cvt4(a1);
+                f32x4 r0, r1;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     r0[e] = a0[e] - (float)h0[e];
                     r1[e] = a1[e] - (float)h1[e];
                 }
-                vhi[ct] = cat8(h0, h1);
-                vlo[ct] = frag_from_acc(r0, r1);
+                vhi[j][ct] = cat8(h0, h1);
+                vlo[j][ct] = frag_from_acc(r0, r1);
             }
+        {
+            bf16x8 kfb[KT];
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-                const bf16x8 kf = frag_tr(kS, pk, kt * 16, 32 * j);
+            for (int kt = 0; kt < KT; ++kt) kfb[kt] = KTile<K>::tr(t.k, kt * 16, 32);
+            FLA_SCHED_FENCE();
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
-                    hacc[kt][ct] = mfma16x32(kf, vhi[ct], hacc[kt][ct]);
-                    hacc[kt][ct] = mfma16x32(kf, vlo[ct], hacc[kt][ct]);
+                    hacc[kt][ct] = mfma16x32(kfa[kt], vhi[0][ct], hacc[kt][ct]);
+                    hacc[kt][ct] = mfma16x32(kfa[kt], vlo[0][ct], hacc[kt][ct]);
                 }
-            }
+            FLA_SCHED_FENCE();
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    hacc[kt][ct] = mfma16x32(kfb[kt], vhi[1][ct], hacc[kt][ct]);
+                    hacc[kt][ct] = mfma16x32(kfb[kt], vlo[1][ct], hacc[kt][ct]);
+                }
         }
+        FLA_TICK(11)
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc_to_tile(oS, po, rt * 16, (vtile0 + ct) * 16, oacc[rt][ct]);
+        FLA_TICK(12)
         __syncthreads();  // #3: every read of this chunk's tiles is done, oS complete
+        FLA_TICK(4)
 
-        // =========================== D: epilogue ==========================================
-        store_tile<kThreads>(og + (int64_t)start * p.o.st, p.o.st, oS, po, VS, len);
-        if (c + 1 < nchunks) commit(c + 1);
-        __syncthreads();  // #4
+        if (!DB) {
+            store_o(c);
+            if (c + 1 < nchunks) commit(c + 1, tiles_at<K, CT>(smem, 0));
+            __syncthreads();  // #4
+        }
+        FLA_TICK(5)
     }
+    if (DB && nchunks > 0) store_o(nchunks - 1);
+#ifdef FLA_FUSED_TIMING
+    if (blockIdx.x == 0 && l == 0 && p.g_out)
+        for (int i = 0; i < 16; ++i) p.g_out[wv * 16 + i] = (float)tacc[i] / (float)nchunks;
+#endif
 
     if (p.hT) {
         float *s = p.hT + n * p.s_sn + hv * p.s_sh;
@@ -491,7 +654,7 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                     "%s: %s must be [B,T,Hv] = [%d,%d,%d].", op, name, geom.B, geom.T, geom.Hv);
         return FLA_OK;
     };
-    const int gmask = dt_bit(FLA_F32) | dt_bit(FLA_BF16);
+    const int gmask = dt_bit(FLA_F32);  // the Python front end casts gates to fp32
     if ((rc = check_bth(g, "g", gmask))) return rc;
     if ((rc = check_bth(beta, "beta", gmask))) return rc;
     if ((rc = check_tensor(o, op, "o", 4, bf))) return rc;
@@ -562,7 +725,11 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     // score / w work once per head; 64-column slabs double the number of workgroups.  Use the
     // wide form once it alone fills the GPU.
     const int64_t chains = (int64_t)geom.N * geom.Hv;
-    const bool wide = geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
+    bool wide = geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
+    if (const char *env = getenv("FLA_HIP_GDN_SLAB")) {  // tuning override: 64 or 128 columns per workgroup
+        if (atoi(env) == 128 && geom.V % 128 == 0) wide = true;
+        if (atoi(env) == 64) wide = false;
+    }
     p.slabs = wide ? geom.V / 128 : geom.V / 64;
     if (geom.K == 128) return wide ? launch_fused<128, 2>(p, stream) : launch_fused<128, 1>(p, stream);
     return wide ? launch_fused<64, 2>(p, stream) : launch_fused<64, 1>(p, stream);

@@ -91,10 +91,52 @@ __device__ __forceinline__ void store_tile(bf16 *gdst, int64_t gstride, const bf
 }
 
 // Writes one accumulator tile, rounded to bf16, into a row-major LDS tile at (r0, c0).
+// Neighbouring lanes hold neighbouring columns; they swap half of their values so that every
+// lane writes two whole dwords (even lanes rows e = 0,1; odd lanes rows e = 2,3 of the column
+// pair) instead of four 16-bit pieces, which also keeps the write free of bank conflicts.
 __device__ __forceinline__ void acc_to_tile(bf16 *tile, int pitch, int r0, int c0, f32x4 acc) {
-    const int col = c0 + acc_col();
-#pragma unroll
-    for (int e = 0; e < 4; ++e) tile[(r0 + acc_row(e)) * pitch + col] = (bf16)acc[e];
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
+    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
+    const bool odd = li & 1;
+    const unsigned send = odd ? p01 : p23;
+    const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+    const unsigned left = odd ? recv : p01;    // column li & ~1
+    const unsigned right = odd ? p23 : recv;   // column li | 1
+    bf16 *dst = tile + (r0 + 4 * lg + (odd ? 2 : 0)) * pitch + c0 + (li & ~1);
+    *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);          // low halves
+    *reinterpret_cast<unsigned *>(dst + pitch) = __builtin_amdgcn_perm(right, left, 0x07060302u);  // high halves
 }
+
+// ---- the k tile -------------------------------------------------------------------------------
+// The k tile is read both ways (contraction along columns for k k^T and q k^T, along rows for
+// k^T v and the right-hand sides).  No padding keeps both patterns conflict free, an XOR swizzle
+// of the 16-byte column chunks does: chunk c of row r is stored at chunk c ^ f(r),
+// f(r) = 2*(r % 8) + (r / 8) % 2.  Sixteen consecutive rows get sixteen different f (column-wise
+// reads of one chunk hit 16 different bank groups); eight consecutive rows get eight different
+// f >> 1 (row-wise reads of a chunk pair hit 8 different bank-group pairs).  K = 64 rows are too
+// short for the swizzle and use a padded pitch instead.
+template <int K> struct KTile {
+    static constexpr int pitch = K == 128 ? 128 : K + 16;
+    static __device__ __forceinline__ int f(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
+    static __device__ __forceinline__ int off(int r, int col) {  // element offset of (row r, column col)
+        if (K == 128) return r * 128 + ((((col >> 3) ^ f(r)) << 3) | (col & 7));
+        return r * pitch + col;
+    }
+    static __device__ __forceinline__ bf16x8 kc(const bf16 *t, int r0, int c0) {
+        const int l = lane_id(), i = l & 15, g = l >> 4;
+        return cat8(*reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 4 * g)),
+                    *reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 16 + 4 * g)));
+    }
+    static __device__ __forceinline__ bf16x4 tr4(const bf16 *t, int r0, int c0) {
+        const int l = lane_id(), i = l & 15, g = l >> 4;
+        return lds_tr4(t + off(c0 + 4 * g + (i >> 2), r0 + 4 * (i & 3)));
+    }
+    static __device__ __forceinline__ bf16x8 tr(const bf16 *t, int r0, int c0) {
+        const int l = lane_id(), i = l & 15, g = l >> 4;
+        return cat8(lds_tr4(t + off(c0 + 4 * g + (i >> 2), r0 + 4 * (i & 3))),
+                    lds_tr4(t + off(c0 + 16 + 4 * g + (i >> 2), r0 + 4 * (i & 3))));
+    }
+};
 
 }  // namespace fla
