@@ -1,0 +1,207 @@
+"""Boundary tests that need no GPU: the shared library loads and exports every symbol that
+include/fla_hip.h declares; the ctypes wrappers build exactly one value per C operand, in the
+prototype's order and with the prototype's C types; host-side validation rejects bad calls
+before any launch.  Modelled on torch_custom/fla_npu/test/test_aclnn_ctypes_abi.py and
+test_ascendc_mutation_contract.py."""
+import ctypes
+import re
+from pathlib import Path
+from unittest import mock
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "fla_hip.h"
+
+
+def declared_symbols():
+    text = HEADER.read_text()
+    return sorted(set(re.findall(r"\b(fla_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    import fla_hip
+
+    return fla_hip.load_library()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = declared_symbols()
+    assert len(names) >= 20
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared in fla_hip.h but not exported: {missing}"
+    assert lib.fla_abi_version() == 1
+
+
+def test_every_operator_has_a_query_and_a_launch_symbol():
+    names = declared_symbols()
+    ops = [n[:-len("_get_workspace_size")] for n in names if n.endswith("_get_workspace_size")]
+    assert ops and all(op in names for op in ops)
+
+
+class FakeTensor:
+    def __init__(self, shape, dtype=torch.bfloat16):
+        self.shape = tuple(shape)
+        self.dtype = dtype
+
+    def dim(self):
+        return len(self.shape)
+
+    def contiguous(self):
+        return self
+
+
+class FakeCallContext:
+    def __init__(self):
+        self.names = []
+
+    def tensor(self, tensor, name="tensor"):
+        self.names.append(name)
+        from fla_hip.ops._runtime import TENSOR_P
+        return TENSOR_P()
+
+    def int_array(self, values):
+        self.names.append("int_array")
+        from fla_hip.ops._runtime import INT_ARRAY_P
+        return INT_ARRAY_P()
+
+
+def capture_call(fn, *args, **kwargs):
+    from fla_hip.ops import _hip_ctypes as H
+
+    captured = {}
+
+    def fake_empty(shape, like, **kw):
+        return FakeTensor(shape, kw.get("dtype") or like.dtype)
+
+    def fake_empty_like(t, **kw):
+        return FakeTensor(t.shape, kw.get("dtype") or t.dtype)
+
+    def fake_call(name, argtypes, build_args, outputs):
+        ctx = FakeCallContext()
+        captured.update(name=name, argtypes=list(argtypes), args=build_args(ctx), names=ctx.names)
+        return outputs
+
+    with mock.patch.object(H, "_empty", side_effect=fake_empty), \
+            mock.patch.object(H, "_empty_like", side_effect=fake_empty_like), \
+            mock.patch.object(H, "_call_op", side_effect=fake_call), \
+            mock.patch.object(H, "_shape", side_effect=lambda t: tuple(t.shape)):
+        out = fn(*args, **kwargs)
+    return captured, out
+
+
+def assert_args_match_argtypes(captured):
+    assert len(captured["args"]) == len(captured["argtypes"])
+    for value, ctype in zip(captured["args"], captured["argtypes"]):
+        assert isinstance(value, ctype), (captured["name"], value, ctype)
+
+
+def test_fwd_h_wrapper_operand_order_and_outputs():
+    from fla_hip.ops import _hip_ctypes as H
+    k = FakeTensor((1, 2, 130, 128))
+    u = FakeTensor((1, 4, 130, 128))
+    g = FakeTensor((1, 4, 130), torch.float32)
+    cap, out = capture_call(H.npu_chunk_gated_delta_rule_fwd_h, k, u, u, g, output_final_state=True, chunk_size=None)
+    assert cap["name"] == "chunk_gated_delta_rule_fwd_h"
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["k", "w", "u", "g", "gk", "initial_state", "h", "v_new", "final_state"]
+    assert cap["args"][7].value == 64                           # chunk_size=None -> 64 (_aclnn_ctypes.py:572)
+    h, v_new, final = out
+    assert h.shape == (1, 4, 3, 128, 128) and final.shape == (1, 4, 128, 128) and final.dtype == torch.float32
+
+
+def test_fwd_h_varlen_shapes_and_state_layout_check():
+    from fla_hip.ops import _hip_ctypes as H
+    k = FakeTensor((1, 2, 130, 128))
+    u = FakeTensor((1, 2, 130, 64))
+    g = FakeTensor((1, 2, 130), torch.float32)
+    cap, out = capture_call(H.npu_chunk_gated_delta_rule_fwd_h, k, u, u, g, cu_seqlens=[0, 1, 66, 130], state_v_first=True)
+    assert out[0].shape == (1, 2, 4, 64, 128) and out[2] is None
+    with pytest.raises(RuntimeError, match="initial_state shape does not match state_v_first"):
+        capture_call(H.npu_chunk_gated_delta_rule_fwd_h, k, u, u, g, initial_state=FakeTensor((1, 2, 128, 64), torch.float32),
+                     state_v_first=True)
+    with pytest.raises(RuntimeError, match=r"^npu_chunk_gated_delta_rule_fwd_h: either g or gk must be provided\.$"):
+        H.npu_chunk_gated_delta_rule_fwd_h(k, u, u)
+
+
+@pytest.mark.parametrize("name,args,kwargs", [
+    ("npu_chunk_fwd_o", (FakeTensor((1, 2, 64, 128)),) * 3 + (FakeTensor((1, 2, 1, 128, 128)), 0.1), {"g": FakeTensor((1, 2, 64), torch.float32)}),
+    ("npu_recompute_w_u_fwd", (FakeTensor((1, 2, 64, 128)), FakeTensor((1, 2, 64, 128)), FakeTensor((1, 2, 64), torch.float32), FakeTensor((1, 2, 64, 64)), 64), {"g": FakeTensor((1, 2, 64), torch.float32)}),
+    ("npu_chunk_scaled_dot_kkt", (FakeTensor((1, 2, 64, 128)), FakeTensor((1, 2, 64), torch.float32), FakeTensor((1, 2, 64), torch.float32)), {}),
+    ("npu_solve_tri", (FakeTensor((1, 64, 2, 64)),), {}),
+    ("npu_chunk_local_cumsum", (FakeTensor((1, 2, 64), torch.float32), 64), {}),
+    ("npu_causal_conv1d", (FakeTensor((2, 8, 32)), FakeTensor((4, 32))), {"head_num": 2}),
+])
+def test_wrappers_build_one_value_per_c_operand(name, args, kwargs):
+    from fla_hip.ops import _hip_ctypes as H
+    cap, _ = capture_call(getattr(H, name), *args, **kwargs)
+    assert_args_match_argtypes(cap)
+    assert cap["argtypes"] == H.OP_ARGTYPES[cap["name"]]
+
+
+def test_defaults_follow_the_reference():
+    import inspect
+    from fla_hip.ops import _hip_ctypes as H
+    sig = inspect.signature(H.npu_chunk_local_cumsum)
+    assert sig.parameters["output_dtype"].default == "float32" and sig.parameters["head_first"].default is True
+    assert inspect.signature(H.npu_chunk_scaled_dot_kkt).parameters["chunk_size"].default == 64
+    assert inspect.signature(H.npu_solve_tri).parameters["layout"].default == "bsnd"
+    assert inspect.signature(H.npu_recurrent_gated_delta_rule).parameters["scale"].default == 1.0
+    cap, out = capture_call(H.npu_causal_conv1d, FakeTensor((2, 8, 32)), FakeTensor((4, 32)), head_num=2)
+    assert out.shape == (2, 2, 8, 16)                           # [B, head_num, S, D/head_num]
+
+
+def test_public_namespace_and_mutation_contract():
+    from fla_hip import ops
+    for name in ("npu_causal_conv1d", "causal_conv1d", "npu_recurrent_gated_delta_rule", "recurrent_gated_delta_rule",
+                 "npu_chunk_fwd_o", "chunk_fwd_o", "npu_solve_tri", "chunk_local_cumsum", "chunk_scaled_dot_kkt",
+                 "recompute_w_u_fwd", "chunk_gated_delta_rule_fwd_h"):
+        assert callable(getattr(ops, name))
+    assert ops.MUTATED_ARGUMENTS["recurrent_gated_delta_rule"] == ("state",)
+    assert ops.MUTATED_ARGUMENTS["causal_conv1d"] == ("conv_states",)
+    with pytest.raises(NotImplementedError):
+        ops.npu_fast_gelu_custom(torch.zeros(1))
+    state = torch.zeros(1, 1, 4, 4, requires_grad=True)
+    with pytest.raises(RuntimeError, match="mutates state in place"):
+        ops.recurrent_gated_delta_rule(None, None, None, state, beta=None, actual_seq_lengths=None,
+                                       ssm_state_indices=None, g=torch.zeros(1))
+
+
+def test_recurrent_wrapper_requires_a_gate_before_any_launch():
+    from fla_hip.ops import _hip_ctypes as H
+    with mock.patch.object(H, "_call_op") as call:
+        with pytest.raises(RuntimeError, match=r"^npu_recurrent_gated_delta_rule: either g or gk must be provided\.$"):
+            H.npu_recurrent_gated_delta_rule(None, None, None, None, beta=None, actual_seq_lengths=None,
+                                             ssm_state_indices=None)
+    call.assert_not_called()
+
+
+def test_library_rejects_null_and_bad_descriptors_without_a_gpu(lib):
+    """Status codes and fla_last_error() for calls that fail validation (no launch happens)."""
+    from fla_hip.ops._runtime import FlaTensor, TENSOR_P, INT_ARRAY_P
+    lib.fla_last_error.restype = ctypes.c_char_p
+    ws = ctypes.c_uint64(0)
+    fn = lib.fla_chunk_scaled_dot_kkt_get_workspace_size
+    fn.restype = ctypes.c_int
+    fn.argtypes = [TENSOR_P, TENSOR_P, TENSOR_P, INT_ARRAY_P, INT_ARRAY_P, ctypes.c_int64, TENSOR_P,
+                   ctypes.POINTER(ctypes.c_uint64)]
+    assert fn(TENSOR_P(), TENSOR_P(), TENSOR_P(), INT_ARRAY_P(), INT_ARRAY_P(), 64, TENSOR_P(), ctypes.byref(ws)) == 1
+    assert b"k must not be null" in lib.fla_last_error()
+    t = FlaTensor()
+    t.data = 16
+    t.dtype = 0          # fp32 where bf16 is required
+    t.ndim = 4
+    for i, d in enumerate((1, 1, 64, 128)):
+        t.shape[i] = d
+    assert fn(ctypes.pointer(t), TENSOR_P(), TENSOR_P(), INT_ARRAY_P(), INT_ARRAY_P(), 64, TENSOR_P(), ctypes.byref(ws)) == 2
+    assert fn(ctypes.pointer(t), TENSOR_P(), TENSOR_P(), INT_ARRAY_P(), INT_ARRAY_P(), 32, TENSOR_P(), ctypes.byref(ws)) == 4
+    assert b"chunk_size must be 64" in lib.fla_last_error()
+
+
+def test_cpu_tensors_are_rejected():
+    from fla_hip import ops
+    x = torch.zeros(1, 4, 16, dtype=torch.bfloat16)
+    with pytest.raises(TypeError, match="ROCm GPU tensor"):
+        ops.causal_conv1d(x, torch.zeros(4, 16, dtype=torch.bfloat16))

@@ -1,0 +1,276 @@
+"""CPU pins of the oracle (no GPU, no product code): every oracle function is checked against
+something that does not share its formula - a different algorithm, a library routine, a closed
+form, autograd, or the reference's own deterministic inputs."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import conv1d as oc, decode as od, gdn, kda
+
+F = torch.nn.functional
+
+
+# --------------------------------------------------------------------------- GDN
+def test_cfg1_chunked_equals_naive_fp32():
+    """BASELINE config 1: fp32, B=1 T=256 H=2 K=V=64, chunk 64, zero initial state, seed 0."""
+    d = gdn.make_gdn_inputs(1, 256, 2, 64, 64, seed=0)
+    o_n, f_n = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True, naive=True)
+    o_c, f_c = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True, naive=False)
+    assert o_n.shape == (1, 256, 2, 64) and f_n.shape == (1, 2, 64, 64)
+    assert float((o_n - o_c).abs().max()) <= 1e-5
+    assert float((f_n - f_c).abs().max()) <= 1e-5
+
+
+def test_naive_recurrence_against_float64_bruteforce_numpy():
+    d = gdn.make_gdn_inputs(1, 20, 1, 8, 5, seed=3, head_first_gates=True)
+    o, f = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], 0.7, output_final_state=True)
+    q, k, v = (d[n][0, 0].double().numpy() for n in "qkv")
+    g, b = d["g"][0, 0].double().numpy(), d["beta"][0, 0].double().numpy()
+    S = np.zeros((8, 5))
+    for t in range(20):
+        S = math.exp(g[t]) * S
+        S = S + np.outer(k[t], b[t] * (v[t] - S.T @ k[t]))     # (I - b k k^T) S + b k v^T
+        np.testing.assert_allclose(o[0, 0, t].numpy(), 0.7 * (S.T @ q[t]), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(f[0, 0].numpy(), S, rtol=1e-4, atol=1e-5)
+
+
+def test_closed_forms():
+    d = gdn.make_gdn_inputs(1, 40, 2, 16, 16, seed=1, head_first_gates=True)
+    h0 = torch.randn(1, 2, 16, 16, generator=torch.Generator().manual_seed(0))
+    # beta = 0: the state only decays
+    o, f = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], torch.zeros_like(d["beta"]), 1.0,
+                                                initial_state=h0, output_final_state=True)
+    G = torch.cumsum(d["g"], -1)
+    assert torch.allclose(o, torch.einsum("bhtk,bhkv->bhtv", d["q"], h0) * torch.exp(G)[..., None], atol=1e-5)
+    assert torch.allclose(f, h0 * torch.exp(G[:, :, -1])[..., None, None], atol=1e-5)
+    # g = 0, beta = 1, unit keys: the state stores v_t under k_t exactly
+    o, _ = gdn.naive_recurrent_gated_delta_rule(d["k"], d["k"], d["v"], torch.zeros_like(d["g"]),
+                                                torch.ones_like(d["beta"]), 1.0)
+    assert torch.allclose(o, d["v"], atol=1e-4)
+
+
+@pytest.mark.parametrize("chunk", [16, 32, 64, 128])
+def test_chunk_size_invariance_and_varlen(chunk):
+    d = gdn.make_gdn_inputs(1, 200, 2, 32, 48, seed=2, head_first_gates=True, Hk=1)
+    ref, fref = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True)
+    o, f = gdn.chunk_gated_delta_rule_fwd(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True, chunk=chunk)
+    assert float((o - ref).abs().max()) < 1e-5 and float((f - fref).abs().max()) < 1e-5
+    cu = [0, 7, 7, 90, 200]
+    o_v, f_v = gdn.chunk_gated_delta_rule_fwd(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True,
+                                              chunk=chunk, cu_seqlens=cu)
+    for n, (s, e) in enumerate(zip(cu, cu[1:])):
+        if e == s:
+            continue
+        o_s, f_s = gdn.naive_recurrent_gated_delta_rule(d["q"][:, :, s:e], d["k"][:, :, s:e], d["v"][:, :, s:e],
+                                                        d["g"][:, :, s:e], d["beta"][:, :, s:e], output_final_state=True)
+        assert float((o_v[:, :, s:e] - o_s).abs().max()) < 1e-5
+        assert float((f_v[n] - f_s[0]).abs().max()) < 1e-5
+
+
+def test_stage_oracles_against_library_routines():
+    gen = torch.Generator().manual_seed(4)
+    g = torch.randn(2, 3, 130, generator=gen)
+    ref = torch.cat([torch.cumsum(c, -1) for c in g.split(64, dim=-1)], -1)
+    assert torch.allclose(gdn.chunk_local_cumsum(g, 64), ref, atol=1e-6)
+    rev = torch.cat([torch.flip(torch.cumsum(torch.flip(c, [-1]), -1), [-1]) for c in g.split(64, dim=-1)], -1)
+    assert torch.allclose(gdn.chunk_local_cumsum(g, 64, reverse=True, scale=2.0), 2.0 * rev, atol=1e-5)
+    # kkt: structural zeros + library matmul
+    k = torch.randn(1, 1, 70, 16, generator=gen)
+    G = gdn.chunk_local_cumsum(-torch.rand(1, 1, 70, generator=gen), 64)
+    beta = torch.rand(1, 1, 70, generator=gen)
+    A = gdn.chunk_scaled_dot_kkt(k, G, beta, 64)
+    blk = A[0, 0, :64]
+    assert float(torch.triu(blk).abs().max()) == 0.0 and float(A[0, 0, 64:, 6:].abs().max()) == 0.0
+    i, j = 37, 5
+    expect = beta[0, 0, i] * math.exp(float(G[0, 0, i] - G[0, 0, j])) * float(k[0, 0, i] @ k[0, 0, j])
+    assert abs(float(blk[i, j]) - expect) < 1e-5
+    # solve_tri against numpy.linalg.inv, incl. a tail block
+    X = gdn.solve_tri(A)
+    inv = np.linalg.inv(np.eye(64) + blk.double().numpy())
+    np.testing.assert_allclose(X[0, 0, :64].numpy(), inv, rtol=1e-5, atol=1e-5)
+    inv_t = np.linalg.inv(np.eye(6) + A[0, 0, 64:, :6].double().numpy())
+    np.testing.assert_allclose(X[0, 0, 64:, :6].numpy(), inv_t, rtol=1e-5, atol=1e-5)
+
+
+# --------------------------------------------------------------------------- conv1d
+def test_conv1d_against_F_conv1d_and_reference_kat_inputs():
+    def make_tensor(shape, start):  # test_npu_causal_conv1d.py:154-161
+        n = int(np.prod(shape))
+        return (torch.arange(start, start + n, dtype=torch.float32).reshape(shape) / 128.0).to(torch.float16)
+
+    x, w, b = make_tensor((2, 4, 16), 1.0), make_tensor((4, 16), 101.0), make_tensor((16,), 201.0)
+    cs = make_tensor((2, 3, 16), 301.0)
+    for act in (0, 1):
+        y, new_cs = oc.causal_conv1d(x, w, b, cs, activation_mode=act)
+        ref = F.conv1d(x.float().permute(0, 2, 1), w.float().t().unsqueeze(1), b.float(), padding=3, groups=16)[..., :4]
+        ref = F.silu(ref) if act else ref
+        assert torch.allclose(y.float(), ref.permute(0, 2, 1).to(torch.float16).float(), atol=2e-3, rtol=2e-3)
+        assert torch.equal(new_cs[:, 2], x[:, 3]) and torch.equal(new_cs[:, 0], x[:, 1])
+    # with initial state: equals a convolution over [state | x]
+    y, new_cs = oc.causal_conv1d(x, w, None, cs, initial_state_mode=[1, 1])
+    xc = torch.cat([cs, x], 1).float().permute(0, 2, 1)
+    ref = F.conv1d(xc, w.float().t().unsqueeze(1), None, padding=0, groups=16)
+    assert torch.allclose(y.float(), ref.permute(0, 2, 1).to(torch.float16).float(), atol=2e-3, rtol=2e-3)
+
+
+def test_conv1d_short_sequences_shift_the_state():
+    x = torch.randn(1, 2, 16).half()
+    cs = torch.randn(1, 3, 16).half()
+    w = torch.randn(4, 16).half()
+    _, new_cs = oc.causal_conv1d(x, w, None, cs, initial_state_mode=[1])
+    assert torch.equal(new_cs[0, 0], cs[0, 2]) and torch.equal(new_cs[0, 1:], x[0])
+    _, new_cs = oc.causal_conv1d(x, w, None, cs)           # no initial state: zero history
+    assert float(new_cs[0, 0].abs().max()) == 0.0
+
+
+# --------------------------------------------------------------------------- decode
+def test_decode_equals_naive_recurrence_with_transposed_state():
+    gen = torch.Generator().manual_seed(6)
+    T, H, K, V = 6, 2, 8, 12
+    q, k = torch.randn(T, H, K, generator=gen), torch.randn(T, H, K, generator=gen)
+    v, beta = torch.randn(T, H, V, generator=gen), torch.rand(T, H, generator=gen)
+    g = -torch.rand(T, H, generator=gen)
+    S0 = torch.randn(2, H, V, K, generator=gen)
+    lens = torch.tensor([0, 4, 2], dtype=torch.int32)
+    idx = torch.tensor([0, 0, 0, 0, 1, 1], dtype=torch.int32)
+    o, S = od.recurrent_gated_delta_rule(q, k, v, S0, beta=beta, scale=0.5, actual_seq_lengths=lens,
+                                         ssm_state_indices=idx, g=g)
+    for n, (s, e) in enumerate([(0, 4), (4, 6)]):
+        tr = lambda x: x[s:e].transpose(0, 1).unsqueeze(0)      # [1,H,L,D]
+        o_n, f_n = gdn.naive_recurrent_gated_delta_rule(tr(q), tr(k), tr(v), g[s:e].t().unsqueeze(0),
+                                                        beta[s:e].t().unsqueeze(0), 0.5,
+                                                        initial_state=S0[n:n + 1].transpose(-1, -2),
+                                                        output_final_state=True)
+        assert torch.allclose(o[s:e], o_n[0].transpose(0, 1), atol=1e-5)
+        assert torch.allclose(S[n], f_n[0].transpose(-1, -2), atol=1e-5)
+
+
+def test_decode_accepted_tokens_and_no_gate():
+    gen = torch.Generator().manual_seed(7)
+    T, H, D = 3, 1, 4
+    q, k, v = (torch.randn(T, H, D, generator=gen) for _ in range(3))
+    beta = torch.rand(T, H, generator=gen)
+    S0 = torch.randn(3, H, D, D, generator=gen)
+    lens = torch.tensor([0, 3], dtype=torch.int32)
+    idx = torch.tensor([0, 1, 2], dtype=torch.int32)
+    acc = torch.tensor([2], dtype=torch.int32)
+    o, S = od.recurrent_gated_delta_rule(q, k, v, S0, beta=beta, actual_seq_lengths=lens, ssm_state_indices=idx,
+                                         num_accepted_tokens=acc, gk=torch.zeros(T, H, D))
+    St = S0[1].clone()                                           # slot of token seq0 + accepted - 1
+    for t in range(T):
+        delta = beta[t, 0] * (v[t, 0] - St[0] @ k[t, 0])
+        St[0] = St[0] + torch.outer(delta, k[t, 0])
+        assert torch.allclose(o[t, 0], St[0] @ q[t, 0], atol=1e-5)
+        assert torch.allclose(S[t], St, atol=1e-5)
+
+
+# --------------------------------------------------------------------------- KDA
+def kda_inputs(B, T, H, K, V, seed=0, gate_scale=1.0):
+    gen = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, H, T, K, generator=gen), dim=-1)
+    k = F.normalize(torch.randn(B, H, T, K, generator=gen), dim=-1)
+    v = torch.randn(B, H, T, V, generator=gen)
+    gate = F.logsigmoid(torch.randn(B, H, T, K, generator=gen)) * gate_scale
+    beta = torch.sigmoid(torch.randn(B, H, T, generator=gen))
+    return q, k, v, gate, beta
+
+
+@pytest.mark.parametrize("cu", [None, [0, 5, 70, 150]])
+def test_kda_chunked_equals_naive(cu):
+    q, k, v, gate, beta = kda_inputs(1, 150, 2, 16, 24, seed=1, gate_scale=0.3)
+    h0 = torch.randn(1 if cu is None else 3, 2, 16, 24, generator=torch.Generator().manual_seed(9))
+    o_n, f_n = kda.naive_recurrent_kda(q, k, v, gate, beta, 0.3, initial_state=h0, output_final_state=True,
+                                       cu_seqlens=cu, compute_dtype=torch.float64)
+    gk = kda.kda_gate_cumsum(gate, 64, cu_seqlens=cu)
+    out = kda.chunk_kda_fwd(q, k, v, gk, beta, 0.3, 64, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                            compute_dtype=torch.float64)
+    assert float((out["o"] - o_n).abs().max()) < 1e-5
+    assert float((out["final_state"] - f_n.float()).abs().max()) < 1e-5
+
+
+def test_kda_reduces_to_gdn_for_channel_constant_gate():
+    d = gdn.make_gdn_inputs(1, 100, 2, 16, 16, seed=5, head_first_gates=True)
+    gate = d["g"][..., None].expand(-1, -1, -1, 16).contiguous()
+    o_k, f_k = kda.naive_recurrent_kda(d["q"], d["k"], d["v"], gate, d["beta"], output_final_state=True)
+    o_g, f_g = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True)
+    assert torch.allclose(o_k, o_g, atol=1e-6) and torch.allclose(f_k, f_g, atol=1e-6)
+
+
+def test_kda_gate_activations():
+    gen = torch.Generator().manual_seed(2)
+    g = torch.randn(1, 2, 70, 8, generator=gen)
+    A_log, dt = torch.randn(2, generator=gen) * 0.3, torch.randn(16, generator=gen) * 0.1
+    gk = kda.kda_gate_cumsum(g, 64, A_log=A_log, dt_bias=dt, use_gate_in_kernel=True)
+    act = -torch.exp(A_log).view(1, 2, 1, 1) * F.softplus(g + dt.view(1, 2, 1, 8))
+    ref = torch.cat([torch.cumsum(c, 2) for c in act.split(64, dim=2)], 2) / math.log(2.0)
+    assert torch.allclose(gk, ref, atol=1e-5)
+    gk = kda.kda_gate_cumsum(g, 64, A_log=A_log, dt_bias=dt, use_gate_in_kernel=True, safe_gate=True, lower_bound=-3.0)
+    act = -3.0 * torch.sigmoid(torch.exp(A_log).view(1, 2, 1, 1) * (g + dt.view(1, 2, 1, 8)))
+    ref = torch.cat([torch.cumsum(c, 2) for c in act.split(64, dim=2)], 2) / math.log(2.0)
+    assert torch.allclose(gk, ref, atol=1e-5)
+
+
+@pytest.mark.parametrize("mode", ["g", "gK"])
+def test_bwd_dhu_against_autograd(mode):
+    """dh0 and dv2 of the reverse scan equal autograd through the forward state recurrence."""
+    gen = torch.Generator().manual_seed(8)
+    B, H, T, K, V, C = 1, 2, 150, 8, 6, 64
+    dd = torch.float64
+    q, k, w = (torch.randn(B, H, T, K, generator=gen, dtype=dd) * 0.3 for _ in range(3))
+    u = torch.randn(B, H, T, V, generator=gen, dtype=dd).requires_grad_(True)
+    do, dv = torch.randn(B, H, T, V, generator=gen, dtype=dd), torch.randn(B, H, T, V, generator=gen, dtype=dd)
+    dht = torch.randn(B, H, K, V, generator=gen, dtype=dd)
+    h0 = torch.randn(B, H, K, V, generator=gen, dtype=dd).requires_grad_(True)
+    if mode == "g":
+        g = torch.cat([torch.cumsum(c, -1) for c in (-torch.rand(B, H, T, generator=gen, dtype=dd) * 0.1).split(C, -1)], -1)
+    else:
+        gK = torch.cat([torch.cumsum(c, 2) for c in (-torch.rand(B, H, T, K, generator=gen, dtype=dd) * 0.1).split(C, 2)], 2)
+    S, loss = h0, 0.0
+    for s in range(0, T, C):
+        e = min(s + C, T)
+        vn = u[:, :, s:e] - w[:, :, s:e] @ S
+        loss = loss + (vn * dv[:, :, s:e]).sum()
+        if mode == "g":
+            gc = g[:, :, s:e]
+            loss = loss + 0.7 * (((q[:, :, s:e] * torch.exp(gc)[..., None]) @ S) * do[:, :, s:e]).sum()
+            S = S * torch.exp(gc[:, :, -1])[..., None, None] + k[:, :, s:e].transpose(-1, -2) @ (vn * torch.exp(gc[:, :, -1:] - gc)[..., None])
+        else:
+            loss = loss + 0.7 * ((q[:, :, s:e] @ S) * do[:, :, s:e]).sum()
+            S = S * torch.exp2(gK[:, :, e - 1])[..., None] + k[:, :, s:e].transpose(-1, -2) @ vn
+    loss = loss + (S * dht).sum()
+    loss.backward()
+    kw = dict(g=g) if mode == "g" else dict(gK=gK)
+    dh, dh0, dv2 = kda.chunk_gated_delta_rule_bwd_dhu(q, k, w, do, dv, 0.7, C, dht=dht, compute_dtype=dd, **kw)
+    assert torch.allclose(dh0, h0.grad, atol=1e-9)
+    assert torch.allclose(dv2, u.grad, atol=1e-9)
+    assert torch.allclose(dh[:, :, -1], dht, atol=0)            # state gradient seen by the last chunk
+
+
+def test_bwd_intra_against_autograd_and_anchored_evaluation():
+    """The four accumulations equal autograd through Aqk / Akk as functions of (q, k, gk, beta)."""
+    gen = torch.Generator().manual_seed(10)
+    B, H, T, K = 1, 2, 70, 8
+    dd = torch.float64
+    q = torch.randn(B, H, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    k = torch.randn(B, H, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    beta = torch.rand(B, H, T, generator=gen, dtype=dd).requires_grad_(True)
+    inc = -torch.rand(B, H, T, K, generator=gen, dtype=dd) * 0.2
+    gk = torch.cat([torch.cumsum(c, 2) for c in inc.split(64, 2)], 2).requires_grad_(True)
+    dAqk = torch.randn(B, H, T, 64, generator=gen, dtype=dd)
+    dAkk = torch.tril(torch.randn(B, H, T, 64, generator=gen, dtype=dd))
+    loss = 0.0
+    for s in range(0, T, 64):
+        e = min(s + 64, T)
+        L = e - s
+        dec = torch.exp2(gk[:, :, s:e, None, :] - gk[:, :, None, s:e, :])
+        aqk = torch.tril(torch.einsum("bhik,bhijk,bhjk->bhij", q[:, :, s:e], dec, k[:, :, s:e]))
+        akk = torch.tril(torch.einsum("bhik,bhijk,bhjk->bhij", k[:, :, s:e], dec, k[:, :, s:e])) * beta[:, :, s:e, None]
+        loss = loss + (aqk * dAqk[:, :, s:e, :L]).sum() + (akk * torch.tril(dAkk[:, :, s:e, :L])).sum()
+    loss.backward()
+    z4, z3 = torch.zeros(B, H, T, K, dtype=dd), torch.zeros(B, H, T, dtype=dd)
+    dq, dk, db, dg = kda.chunk_kda_bwd_intra(q.detach(), k.detach(), gk.detach(), beta.detach(), dAqk, dAkk, z4, z4, z3, z4)
+    assert torch.allclose(dq, q.grad, atol=1e-9) and torch.allclose(dk, k.grad, atol=1e-9)
+    assert torch.allclose(db, beta.grad, atol=1e-9)
+    assert torch.allclose(dg, gk.grad / math.log(2.0), atol=1e-9)   # dg is the gradient w.r.t. ln2 * gk
