@@ -280,6 +280,338 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     return wide ? launch_fwd_h<64, 2>(p, geom.V / 128, stream) : launch_fwd_h<64, 1>(p, geom.V / 64, stream);
 }
 
+
+// =============================================================================================
+// chunk_gated_delta_rule_bwd_dhu: reverse scan of the state gradient.
+//   dh[c]   = gradient of the state entering from later chunks (emitted before the update)
+//   dv2     = dv + (k . dh) * e^{g_last - g}                         (g variant; gK: no factor)
+//   dh     <- decay * dh + scale * (q e^{g})^T . do - w^T . dv2      (gK: decay = 2^{gK_last} per K row,
+//                                                                     q and k already carry their gates)
+// Same ownership as the forward scan: wave w keeps 16*CT columns of V for all K rows of dh in
+// fp32 accumulators.  q and w are read with transposing LDS loads (contraction over tokens).
+// Math: chunk_gated_delta_rule_bwd_dhu/README.md:6-13, design note
+// chunk_gated_delta_rule_bwd_dhu_design.md:81-182, golden torch_custom/fla_npu/test/test_bwd_dhu.py:61-290.
+// Unlike the reference kernel the terminal gradient dht is consumed, and dh0 may be the fp32
+// [N,Hv,K,V] tensor of the design note as well as the reference's [B,Hv,NT,K,V] form.
+// =============================================================================================
+struct DhuParams {
+    ChunkGeom geom;
+    View4 q, k, w, d_o, dv, dv2;
+    View3 g;             // scalar gate [B,Hv,T] (natural log) or null
+    const float *gK;     // per-channel gate [B,Hv,T,K] fp32 (log2) or null
+    int64_t gk_sb, gk_sh, gk_st;
+    const float *dht;    // [N,Hv,K,V] fp32 or null
+    int64_t t_sn, t_sh;
+    bf16 *dh;            // [B,Hv,NT,K,V]
+    int64_t h_sb, h_sh, h_sc;
+    float *dh0_f32;      // [N,Hv,K,V] fp32 or null
+    int64_t z_sn, z_sh;
+    bf16 *dh0_ref;       // [B,Hv,NT,K,V] bf16 (value stored at each sequence's first chunk) or null
+    float scale;
+};
+
+template <int K, int CT, bool GK>
+__global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int VS = 64 * CT;
+    constexpr int pk = K + 8, pt = K + 16, pv = VS + 16;
+    constexpr int KT = K / 16, KS = K / 32;
+    bf16 *kS = reinterpret_cast<bf16 *>(smem);
+    bf16 *qS = kS + kChunk * pk;
+    bf16 *wS = qS + kChunk * pt;
+    bf16 *oS = wS + kChunk * pt;     // d_o slab
+    bf16 *vS = oS + kChunk * pv;     // dv slab in, dv2 slab out
+    float *gS = reinterpret_cast<float *>(vS + kChunk * pv);   // [64] gate / [K] last-row channel gate
+    float *fS = gS + (GK ? K : kChunk);                        // [64] factor scale * e^{g_t}
+
+    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+        chunk0 = p.geom.choff[n];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int wv = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int vcol0 = slab * VS + wv * 16 * CT;
+
+    f32x4 dacc[KT][CT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f};
+            if (p.dht) {
+                const float *s = p.dht + n * p.t_sn + hv * p.t_sh;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li];
+            }
+            dacc[kt][ct] = a;
+        }
+
+    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const bf16 *og = static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
+    const bf16 *vg = static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
+    bf16 *v2g = static_cast<bf16 *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + slab * VS;
+
+    for (int c = nchunks - 1; c >= 0; --c) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        __syncthreads();
+        load_tile<kThreads>(kS, pk, kg + (int64_t)start * p.k.st, p.k.st, kChunk, K, len);
+        load_tile<kThreads>(qS, pt, qg + (int64_t)start * p.q.st, p.q.st, kChunk, K, len);
+        load_tile<kThreads>(wS, pt, wg + (int64_t)start * p.w.st, p.w.st, kChunk, K, len);
+        load_tile<kThreads>(oS, pv, og + (int64_t)start * p.d_o.st, p.d_o.st, kChunk, VS, len);
+        load_tile<kThreads>(vS, pv, vg + (int64_t)start * p.dv.st, p.dv.st, kChunk, VS, len);
+        if (GK) {
+            if (threadIdx.x < K)
+                gS[threadIdx.x] = exp2f(p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + threadIdx.x]);
+            if (threadIdx.x < kChunk) fS[threadIdx.x] = p.scale;
+        } else if (threadIdx.x < kChunk) {
+            const int t = threadIdx.x;
+            const float gt = t < len ? load_scalar(p.g, b, hv, start + t) : 0.f;
+            gS[t] = gt;
+            fS[t] = t < len ? p.scale * __expf(gt) : 0.f;
+        }
+        __syncthreads();
+
+        bf16x8 hB[KS][CT];
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
+        {   // dh of this chunk = the incoming gradient
+            bf16 *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        hg[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li] = hB[kt >> 1][ct][(kt & 1) * 4 + e];
+        }
+
+        // dv2 = dv + (k . dh) * e^{g_last - g}
+        f32x4 dv2[4][CT];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                const bf16x8 afrag = frag_kc(kS, pk, rt * 16, 32 * j);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = mfma16x32(afrag, hB[j][ct], dv2[rt][ct]);
+            }
+        const float g_last = GK ? 0.f : gS[len - 1];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const bf16x4 old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int t = rt * 16 + 4 * lg + e;
+                    const float f = GK ? 1.f : __expf(g_last - gS[t]);
+                    dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + (float)old[e] : 0.f;
+                }
+            }
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc_to_tile(vS, pv, rt * 16, (wv * CT + ct) * 16, dv2[rt][ct]);
+
+        // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            f32x4 dec;
+            if (GK) {
+                dec = *reinterpret_cast<const f32x4 *>(gS + 16 * kt + 4 * lg);
+            } else {
+                const float d = __expf(g_last);
+                dec = f32x4{d, d, d, d};
+            }
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) dacc[kt][ct] *= dec;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            bf16x8 ob[CT], nb[CT];
+            const f32x4 f0 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 4 * lg),
+                        f1 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 16 + 4 * lg);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const bf16x8 raw = frag_tr(oS, pv, (wv * CT + ct) * 16, 32 * j);   // do[t][col], t = 32j + c(g,e)
+                f32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = (float)raw[e] * f0[e];
+                    hi[e] = (float)raw[4 + e] * f1[e];
+                }
+                ob[ct] = frag_from_acc(lo, hi);
+                nb[ct] = frag_from_acc(-dv2[2 * j][ct], -dv2[2 * j + 1][ct]);
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const bf16x8 qf = frag_tr(qS, pt, kt * 16, 32 * j);
+                const bf16x8 wf = frag_tr(wS, pt, kt * 16, 32 * j);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    dacc[kt][ct] = mfma16x32(qf, ob[ct], dacc[kt][ct]);
+                    dacc[kt][ct] = mfma16x32(wf, nb[ct], dacc[kt][ct]);
+                }
+            }
+        }
+        __syncthreads();
+        store_tile<kThreads>(v2g + (int64_t)start * p.dv2.st, p.dv2.st, vS, pv, VS, len);
+    }
+
+    // gradient of the initial state
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t off = (int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li;
+                if (p.dh0_f32) p.dh0_f32[n * p.z_sn + hv * p.z_sh + off] = dacc[kt][ct][e];
+                if (p.dh0_ref && nchunks > 0)
+                    p.dh0_ref[b * p.h_sb + hv * p.h_sh + (int64_t)chunk0 * p.h_sc + off] = (bf16)dacc[kt][ct][e];
+            }
+}
+
+template <int K, int CT, bool GK>
+int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
+    constexpr int VS = 64 * CT;
+    const size_t smem = ((size_t)kChunk * (K + 8) + 2 * (size_t)kChunk * (K + 16) + 2 * (size_t)kChunk * (VS + 16)) * 2 +
+                        ((GK ? K : kChunk) + kChunk) * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, CT, GK>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, CT, GK>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
+                 const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
+                 const fla_int_array *cu, const fla_int_array *ci, double scale, int64_t chunk_size, bool use_exp2,
+                 const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, void *ws, uint64_t ws_size,
+                 hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_gated_delta_rule_bwd_dhu";
+    (void)h0;  // only its presence matters to the caller (it decides whether dh0 is allocated)
+    const bool has_g = g && g->data, has_gk = gK && gK->data;
+    FLA_REQUIRE(has_g != has_gk, FLA_ERR_NULL, "%s: exactly one of g and gK must be provided.", op);
+    FLA_REQUIRE(!has_gk || use_exp2, FLA_ERR_UNSUPPORTED, "%s: use_exp2 must be true when gK is provided.", op);
+    FLA_REQUIRE(!has_g || !use_exp2, FLA_ERR_UNSUPPORTED, "%s: the scalar gate g is a natural-log gate (use_exp2=false).", op);
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv2", dv2, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if (has_gk) {
+        if ((rc = check_tensor(gK, op, "gK", 4, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE(gK->shape[0] == geom.B && gK->shape[1] == geom.Hv && gK->shape[2] == geom.T && gK->shape[3] == geom.K &&
+                        inner_unit(gK),
+                    FLA_ERR_SHAPE, "%s: gK must be fp32 [B,Hv,T,K].", op);
+    }
+    Varlen vl;
+    if ((rc = build_varlen(vl, op, cu, ci, kChunk, geom.T))) return rc;
+    FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
+    if (vl.enabled) {
+        geom.NT = vl.NT;
+        geom.N = vl.N;
+    }
+    if ((rc = check_tensor(dh, op, "dh", 5, bf))) return rc;
+    FLA_REQUIRE(dh->shape[0] == geom.B && dh->shape[1] == geom.Hv && dh->shape[2] == geom.NT && dh->shape[3] == geom.K &&
+                    dh->shape[4] == geom.V && dh->stride[4] == 1 && dh->stride[3] == geom.V,
+                FLA_ERR_SHAPE, "%s: dh must be [B,Hv,NT=%d,K,V] with contiguous blocks.", op, geom.NT);
+    const bool has_dh0 = dh0 && dh0->data;
+    bool dh0_is_ref = false;
+    if (has_dh0) {
+        if (dh0->ndim == 5) {
+            dh0_is_ref = true;
+            if ((rc = check_tensor(dh0, op, "dh0", 5, bf))) return rc;
+            FLA_REQUIRE(same_shape(dh0, dh) && dh0->stride[0] == dh->stride[0] && dh0->stride[1] == dh->stride[1] &&
+                            dh0->stride[2] == dh->stride[2] && dh0->stride[3] == geom.V && dh0->stride[4] == 1,
+                        FLA_ERR_SHAPE, "%s: a 5-D dh0 must have the shape and strides of dh.", op);
+        } else {
+            if ((rc = check_tensor(dh0, op, "dh0", 4, dt_bit(FLA_F32)))) return rc;
+            FLA_REQUIRE(dh0->shape[0] == geom.N && dh0->shape[1] == geom.Hv && dh0->shape[2] == geom.K &&
+                            dh0->shape[3] == geom.V && dh0->stride[3] == 1 && dh0->stride[2] == geom.V,
+                        FLA_ERR_SHAPE, "%s: a 4-D dh0 must be fp32 [N=%d,Hv,K,V].", op, geom.N);
+        }
+    }
+    const bool has_dht = dht && dht->data;
+    if (has_dht) {
+        if ((rc = check_tensor(dht, op, "dht", 4, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE(dht->shape[0] == geom.N && dht->shape[1] == geom.Hv && dht->shape[2] == geom.K && dht->shape[3] == geom.V &&
+                        dht->stride[3] == 1 && dht->stride[2] == geom.V,
+                    FLA_ERR_SHAPE, "%s: dht must be fp32 [N=%d,Hv,K,V].", op, geom.N);
+    }
+    FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
+    FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
+    if (query) {
+        *query = vl.bytes();
+        return FLA_OK;
+    }
+    FLA_REQUIRE(vl.bytes() == 0 || (ws && ws_size >= vl.bytes()), FLA_ERR_WORKSPACE, "%s: workspace of %zu bytes required.",
+                op, vl.bytes());
+    if ((rc = upload_varlen(vl, ws, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    if (geom.N == 0 || geom.Hv == 0) return FLA_OK;
+
+    DhuParams p{};
+    p.geom = geom;
+    p.q = view4(q);
+    p.k = view4(k);
+    p.w = view4(w);
+    p.d_o = view4(d_o);
+    p.dv = view4(dv);
+    p.dv2 = view4(dv2);
+    if (has_g) p.g = view3(g);
+    if (has_gk) {
+        p.gK = static_cast<const float *>(gK->data);
+        p.gk_sb = gK->stride[0];
+        p.gk_sh = gK->stride[1];
+        p.gk_st = gK->stride[2];
+    }
+    if (has_dht) {
+        p.dht = static_cast<const float *>(dht->data);
+        p.t_sn = dht->stride[0];
+        p.t_sh = dht->stride[1];
+    }
+    p.dh = static_cast<bf16 *>(dh->data);
+    p.h_sb = dh->stride[0];
+    p.h_sh = dh->stride[1];
+    p.h_sc = dh->stride[2];
+    if (has_dh0 && dh0_is_ref) p.dh0_ref = static_cast<bf16 *>(dh0->data);
+    if (has_dh0 && !dh0_is_ref) {
+        p.dh0_f32 = static_cast<float *>(dh0->data);
+        p.z_sn = dh0->stride[0];
+        p.z_sh = dh0->stride[1];
+    }
+    p.scale = (float)scale;
+    const int slabs = geom.V / 64;
+    if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, 1, true>(p, slabs, stream) : launch_bwd_dhu<128, 1, false>(p, slabs, stream);
+    return has_gk ? launch_bwd_dhu<64, 1, true>(p, slabs, stream) : launch_bwd_dhu<64, 1, false>(p, slabs, stream);
+}
+
 }  // namespace
 }  // namespace fla
 
@@ -301,4 +633,24 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_h(
     return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
                            state_v_first, h, v_new, final_state, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
+    const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale, int64_t chunk_size, bool use_exp2,
+    const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, uint64_t *workspace_size) {
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_bwd_dhu: workspace_size must not be null.");
+    return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
+                             dv2, nullptr, 0, nullptr, workspace_size);
+}
+
+extern "C" int fla_chunk_gated_delta_rule_bwd_dhu(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
+    const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale, int64_t chunk_size, bool use_exp2,
+    const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, void *workspace, uint64_t workspace_size,
+    void *stream) {
+    return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
+                             dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }

@@ -36,6 +36,9 @@ OP_ARGTYPES = {
     "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
+    "kda_gate_cumsum": [_T, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool, ctypes.c_double, _T],
+    "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
+                                       ctypes.c_bool, _T, _T, _T],
 }
 
 
@@ -392,6 +395,79 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
         (o, g_out, final),
     )
     return g_out, o, final
+
+
+def npu_kda_gate_cumsum(g, chunk_size, *, A_log=None, dt_bias=None, cu_seqlens=None, use_gate_in_kernel=False,
+                        safe_gate=False, lower_bound=None):
+    """_aclnn_ctypes.py:1268-1296.  ``g [B,Hv,T,K]`` -> ``gk`` fp32, chunk-local cumsum in log2 units."""
+    import torch
+
+    out = _empty(_shape(g), g, dtype=torch.float32)
+    return _call_op(
+        "kda_gate_cumsum", OP_ARGTYPES["kda_gate_cumsum"],
+        lambda ctx: [
+            ctx.tensor(g, "g"), ctx.tensor(A_log, "A_log"), ctx.tensor(dt_bias, "dt_bias"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctypes.c_int64(int(chunk_size)),
+            ctypes.c_bool(_optional_bool(use_gate_in_kernel, False)), ctypes.c_bool(_optional_bool(safe_gate, False)),
+            ctypes.c_double(_optional_float(lower_bound, -5.0)), ctx.tensor(out, "gk"),
+        ],
+        out,
+    )
+
+
+def npu_chunk_gated_delta_rule_bwd_dhu(q, k, w, d_o, dv, scale, chunk_size, *, g=None, gK=None, h0=None, dht=None,
+                                       cu_seqlens=None, chunk_indices=None, use_exp2=False,
+                                       transpose_state_layout=False, dh0_per_sequence=False):
+    """_aclnn_ctypes.py:324-394.  Returns ``(dh, dh0, dv2)``; ``dh0`` is allocated only when ``h0`` is given.
+
+    ``dh0_per_sequence=True`` (an extension) returns ``dh0`` as fp32 ``[N,Hv,K,V]`` instead of the
+    reference's bf16 ``[B,Hv,NT,K,V]`` buffer whose first chunk of each sequence holds the value.
+    ``dht`` (fp32 ``[N,Hv,K,V]``) seeds the scan; the reference accepts and ignores it.
+    """
+    import torch
+
+    B, _, T, K = _shape(q)
+    Hv, V = _shape(dv)[1], _shape(dv)[3]
+    if (g is None) == (gK is None):
+        raise ValueError("Exactly one of g and gK must be provided.")
+    if gK is not None and not _optional_bool(use_exp2, True):
+        raise ValueError("use_exp2 must be true when gK is provided.")
+    if any(t.dtype != q.dtype for t in (k, w, d_o, dv)):
+        raise ValueError("q, k, w, d_o and dv must have the same dtype.")
+    gate = g if g is not None else gK
+    if gate.dtype not in (q.dtype, torch.float32):
+        raise ValueError("g or gK must be float32 or have the same dtype as q and k.")
+    if g is not None and _shape(g) != (B, Hv, T):
+        raise ValueError(f"g must have shape {(B, Hv, T)}, got {_shape(g)}.")
+    if gK is not None and _shape(gK) != (B, Hv, T, K):
+        raise ValueError(f"gK must have shape {(B, Hv, T, K)}, got {_shape(gK)}.")
+    chunk_size = int(chunk_size)
+    cu = _as_int_tuple(cu_seqlens)
+    indices = _as_int_tuple(chunk_indices)
+    if indices is None and cu is not None:
+        indices = _build_chunk_indices(cu, chunk_size)
+    NT = _total_chunks(B, T, chunk_size, cu) if indices is None else len(indices) // 2
+    N = len(cu) - 1 if cu is not None else B
+    dh = _empty((B, Hv, NT, K, V), q)
+    if h0 is None:
+        dh0 = None
+    elif dh0_per_sequence:
+        dh0 = _empty((N, Hv, K, V), q, dtype=torch.float32)
+    else:
+        dh0 = _empty((B, Hv, NT, K, V), q)
+    dv2 = _empty_like(dv)
+    outputs = (dh, dh0, dv2)
+    return _call_op(
+        "chunk_gated_delta_rule_bwd_dhu", OP_ARGTYPES["chunk_gated_delta_rule_bwd_dhu"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(w, "w"), ctx.tensor(d_o, "d_o"), ctx.tensor(dv, "dv"),
+            ctx.tensor(g, "g"), ctx.tensor(gK, "gK"), ctx.tensor(h0, "h0"), ctx.tensor(dht, "dht"),
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_double(float(scale)), ctypes.c_int64(chunk_size),
+            ctypes.c_bool(_optional_bool(use_exp2, gK is not None)),
+            ctx.tensor(dh, "dh"), ctx.tensor(dh0, "dh0"), ctx.tensor(dv2, "dv2"),
+        ],
+        outputs,
+    )
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

@@ -236,6 +236,48 @@ int fla_causal_conv1d(
     int64_t run_mode, int64_t head_num, const fla_tensor *out, void *workspace,
     uint64_t workspace_size, void *stream);
 
+/* ------------------------------------------------------------------------
+ * kda_gate_cumsum - replaces aclnnKdaGateCumsum (_aclnn_ctypes.py:1268-1296;
+ * kda_gate_cumsum/op_kernel/kda_gate_cumsum_kernel.h:374-419,516-534).
+ * g [B,Hv,T,K] f32/bf16 raw gate; A_log [Hv] f32 and dt_bias [Hv*K] f32 are
+ * used when use_gate_in_kernel (softplus gate, or lower_bound * sigmoid when
+ * safe_gate).  Output gk [B,Hv,T,K] f32 = chunk-local cumsum / ln 2.
+ * ------------------------------------------------------------------------ */
+int fla_kda_gate_cumsum_get_workspace_size(
+    const fla_tensor *g, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const fla_int_array *cu_seqlens, int64_t chunk_size, bool use_gate_in_kernel,
+    bool safe_gate, double lower_bound, const fla_tensor *gk, uint64_t *workspace_size);
+int fla_kda_gate_cumsum(
+    const fla_tensor *g, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const fla_int_array *cu_seqlens, int64_t chunk_size, bool use_gate_in_kernel,
+    bool safe_gate, double lower_bound, const fla_tensor *gk, void *workspace,
+    uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
+ * chunk_gated_delta_rule_bwd_dhu - replaces aclnnChunkGatedDeltaRuleBwdDhu
+ * (_aclnn_ctypes.py:324-394; chunk_gated_delta_rule_bwd_dhu/README.md:6-13).
+ * q,k [B,Hk,T,K], w [B,Hv,T,K], d_o,dv [B,Hv,T,V] bf16.  Exactly one gate:
+ * g [B,Hv,T] f32/bf16 (natural log, use_exp2 false) or gK [B,Hv,T,K] f32
+ * (log2, use_exp2 true; q and k then already carry their gates).
+ * h0 is only a presence flag for the caller; dht [N,Hv,K,V] f32 optional.
+ * Outputs dh [B,Hv,NT,K,V] bf16, dv2 like dv, dh0 optional: either the
+ * reference form (bf16, shape of dh, written at each sequence's first chunk)
+ * or f32 [N,Hv,K,V].
+ * ------------------------------------------------------------------------ */
+int fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o,
+    const fla_tensor *dv, const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0,
+    const fla_tensor *dht, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    double scale, int64_t chunk_size, bool use_exp2, const fla_tensor *dh,
+    const fla_tensor *dh0, const fla_tensor *dv2, uint64_t *workspace_size);
+int fla_chunk_gated_delta_rule_bwd_dhu(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o,
+    const fla_tensor *dv, const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0,
+    const fla_tensor *dht, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    double scale, int64_t chunk_size, bool use_exp2, const fla_tensor *dh,
+    const fla_tensor *dh0, const fla_tensor *dv2, void *workspace, uint64_t workspace_size,
+    void *stream);
+
 #ifdef __cplusplus
 }
 #endif

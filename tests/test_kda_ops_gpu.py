@@ -1,0 +1,161 @@
+"""Parity of the KDA-side operators (through the C ABI) against the CPU oracle:
+kda_gate_cumsum and chunk_gated_delta_rule_bwd_dhu (scalar-gate and per-channel-gate variants),
+on dense, GVA, ragged-tail and packed variable-length cases."""
+import math
+
+import pytest
+import torch
+
+from oracle import gdn, kda
+from util import assert_close, TOL_BF16, TOL_STATE
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+# ---------------------------------------------------------------------------------------------
+# kda_gate_cumsum
+# ---------------------------------------------------------------------------------------------
+GATE_CASES = [
+    # B, Hv, T, K, chunk, cu, dtype, use_gate, safe, bias
+    (2, 3, 200, 128, 64, None, torch.float32, False, False, False),
+    (1, 2, 261, 128, 64, [0, 1, 16, 33, 33, 96, 160, 261], torch.float32, True, False, True),
+    (1, 2, 300, 64, 128, None, BF, True, True, True),
+    (2, 2, 65, 32, 64, None, BF, True, False, False),
+    (1, 1, 1, 256, 64, None, torch.float32, True, True, False),
+]
+
+
+@pytest.mark.parametrize("case", GATE_CASES)
+def test_kda_gate_cumsum(dev, case):
+    from fla_hip import ops
+    B, Hv, T, K, chunk, cu, dt, use_gate, safe, bias = case
+    gen = torch.Generator().manual_seed(T + K)
+    g = (torch.randn(B, Hv, T, K, generator=gen) * (1.5 if use_gate else 0.1) - (0.0 if use_gate else 0.05)).to(dt)
+    A_log = torch.randn(Hv, generator=gen) * 0.5
+    dt_bias = torch.randn(Hv * K, generator=gen) * 0.5 if bias else None
+    out = ops.kda_gate_cumsum(g.to(dev), chunk, A_log=A_log.to(dev) if use_gate else None,
+                              dt_bias=None if dt_bias is None else dt_bias.to(dev), cu_seqlens=cu,
+                              use_gate_in_kernel=use_gate, safe_gate=safe, lower_bound=-3.0 if safe else None)
+    ref = kda.kda_gate_cumsum(g, chunk, A_log=A_log, dt_bias=dt_bias, cu_seqlens=cu, use_gate_in_kernel=use_gate,
+                              safe_gate=safe, lower_bound=-3.0)
+    assert out.dtype == torch.float32 and out.shape == g.shape
+    assert_close(out, ref, 1e-5, "gk")
+
+
+def test_kda_gate_cumsum_errors(dev):
+    from fla_hip import ops
+    g = torch.zeros(1, 2, 64, 128, device=dev)
+    with pytest.raises(RuntimeError, match="A_log"):
+        ops.kda_gate_cumsum(g, 64, use_gate_in_kernel=True)
+    with pytest.raises(RuntimeError, match="chunk_size"):
+        ops.kda_gate_cumsum(g, 32)
+    with pytest.raises(RuntimeError, match="lower_bound"):
+        ops.kda_gate_cumsum(g, 64, A_log=torch.zeros(2, device=dev), use_gate_in_kernel=True, safe_gate=True,
+                            lower_bound=-7.0)
+
+
+# ---------------------------------------------------------------------------------------------
+# chunk_gated_delta_rule_bwd_dhu
+# ---------------------------------------------------------------------------------------------
+def dhu_inputs(B, T, Hk, Hv, K, V, seed, per_channel):
+    gen = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=gen)
+    q = (rn(B, Hk, T, K) * K ** -0.5).to(BF)
+    k = torch.nn.functional.normalize(rn(B, Hk, T, K), dim=-1).to(BF)
+    w = (rn(B, Hv, T, K) * 0.1).to(BF)
+    d_o = (rn(B, Hv, T, V) * 0.5).to(BF)
+    dv = (rn(B, Hv, T, V) * 0.5).to(BF)
+    if per_channel:
+        gate = -torch.rand(B, Hv, T, K, generator=gen) * 0.1
+    else:
+        gate = -torch.rand(B, Hv, T, generator=gen) * 0.1
+    return q, k, w, d_o, dv, gate
+
+
+DHU_CASES = [
+    # B, T, Hk, Hv, K, V, cu, per_channel, dht
+    (2, 256, 2, 2, 128, 128, None, False, False),
+    (1, 200, 2, 4, 128, 128, None, False, True),                      # GVA + ragged tail + terminal gradient
+    (1, 261, 1, 2, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261], False, True),
+    (2, 192, 2, 2, 128, 128, None, True, False),
+    (1, 261, 2, 2, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261], True, True),
+    (1, 130, 2, 2, 64, 64, None, False, False),
+    (1, 130, 1, 2, 64, 128, None, True, True),
+    (1, 96, 1, 1, 128, 256, None, False, False),
+]
+
+
+@pytest.mark.parametrize("case", DHU_CASES)
+def test_bwd_dhu(dev, case):
+    from fla_hip import ops
+    B, T, Hk, Hv, K, V, cu, per_channel, with_dht = case
+    q, k, w, d_o, dv, gate = dhu_inputs(B, T, Hk, Hv, K, V, seed=T + V, per_channel=per_channel)
+    scale = K ** -0.5
+    # chunk-local cumulated gates, as the callers provide them
+    if per_channel:
+        gcum = kda.kda_gate_cumsum(gate, 64, cu_seqlens=cu)        # log2 units
+        # q and k carry their gates in this variant (they stay O(1): 2^{gk} <= 1, 2^{gk_last - gk} <= 1)
+        qg = (q.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(gcum)).to(BF)
+        last = torch.zeros_like(gcum)
+        for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+            last[b, :, s:e] = gcum[b, :, e - 1:e]
+        kg = (k.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(last - gcum)).to(BF)
+        q_in, k_in = qg, kg
+    else:
+        gcum = gdn.chunk_local_cumsum(gate, 64, cu_seqlens=cu)
+        q_in, k_in = q, k
+    N = B if cu is None else len(cu) - 1
+    gen = torch.Generator().manual_seed(3)
+    dht = torch.randn(N, Hv, K, V, generator=gen) * 0.1 if with_dht else None
+    h0 = torch.zeros(N, Hv, K, V)
+
+    kw = dict(gK=gcum.to(dev), use_exp2=True) if per_channel else dict(g=gcum.to(dev))
+    args = [t.to(dev) for t in (q_in, k_in, w, d_o, dv)]
+    dh, dh0, dv2 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, h0=h0.to(dev),
+                                                      dht=None if dht is None else dht.to(dev), cu_seqlens=cu,
+                                                      dh0_per_sequence=True, **kw)
+    okw = dict(gK=gcum) if per_channel else dict(g=gcum)
+    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(q_in, k_in, w, d_o, dv, scale, 64, dht=dht,
+                                                                  cu_seqlens=cu, **okw)
+    assert dh.dtype == BF and dv2.dtype == BF and dh0.dtype == torch.float32
+    assert_close(dv2, dv2_ref, TOL_BF16, "dv2")
+    assert_close(dh, dh_ref, TOL_BF16, "dh")
+    assert_close(dh0, dh0_ref, TOL_BF16, "dh0")
+
+    # reference-form dh0: bf16 buffer of dh's shape, written at the first chunk of each sequence
+    dh_b, dh0_b, dv2_b = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, h0=h0.to(dev),
+                                                            dht=None if dht is None else dht.to(dev), cu_seqlens=cu,
+                                                            **kw)
+    assert torch.equal(dh_b, dh) and torch.equal(dv2_b, dv2)
+    assert dh0_b.shape == dh.shape and dh0_b.dtype == BF
+    first = {}
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        first.setdefault(n, (b, ci))
+    for n, (b, ci) in first.items():
+        assert torch.equal(dh0_b[b, :, ci].float(), dh0[n].to(BF).float())
+    # without h0 no dh0 is produced
+    out3 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, cu_seqlens=cu, **kw)
+    assert out3[1] is None
+
+
+def test_bwd_dhu_first_chunk_is_terminal_gradient(dev):
+    """dh of the last chunk is the terminal gradient itself (zero without dht)."""
+    from fla_hip import ops
+    q, k, w, d_o, dv, gate = dhu_inputs(1, 128, 1, 1, 128, 128, seed=1, per_channel=False)
+    g = gdn.chunk_local_cumsum(gate, 64)
+    dh, _, dv2 = ops.chunk_gated_delta_rule_bwd_dhu(*[t.to(dev) for t in (q, k, w, d_o, dv)], 0.1, 64, g=g.to(dev))
+    assert float(dh[:, :, -1].abs().max()) == 0.0
+    assert torch.equal(dv2[:, :, 64:].cpu(), dv[:, :, 64:])          # k . 0 adds nothing
+
+
+def test_bwd_dhu_errors(dev):
+    from fla_hip import ops
+    q, k, w, d_o, dv, gate = dhu_inputs(1, 64, 1, 1, 128, 128, seed=1, per_channel=False)
+    a = [t.to(dev) for t in (q, k, w, d_o, dv)]
+    with pytest.raises(ValueError, match="Exactly one"):
+        ops.chunk_gated_delta_rule_bwd_dhu(*a, 0.1, 64)
+    with pytest.raises(ValueError, match="g must have shape"):
+        ops.chunk_gated_delta_rule_bwd_dhu(*a, 0.1, 64, g=torch.zeros(1, 2, 64, device=dev))
+    with pytest.raises(RuntimeError, match="chunk_size"):
+        ops.chunk_gated_delta_rule_bwd_dhu(*a, 0.1, 32, g=gate.to(dev))
