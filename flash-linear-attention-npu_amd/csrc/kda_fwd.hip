@@ -1,0 +1,784 @@
+// chunk_kda_fwd: chunked forward of the per-channel gated delta rule (KDA).
+//
+// Two kernels:
+//   kda_intra_kernel  one workgroup per (chunk, value head): gate activation + chunk-local prefix
+//                     sum (log2 units), the decayed scores Aqk = scale * tril(q k^T . 2^{g_i-g_j})
+//                     and A0 = beta * stril(k k^T . 2^{g_i-g_j}), the explicit inverse
+//                     Akk = (I + A0)^-1, and the WY factors  w = Akk (k beta 2^g),  u = Akk (v beta),
+//                     plus the gated operands qg = q 2^g and kg = k 2^{g_last - g}.
+//   kda_scan_kernel   one workgroup per (sequence, value head, 64-column slab of V) walks the chunks
+//                     with the fp32 state in accumulator registers:
+//                         v_new = u - w S ;  o = scale qg S + Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new
+//
+// The pairwise decay 2^{g_i - g_j} is never formed from a quotient of two exponentials of the
+// absolute gates (those under/overflow); every 16-row tile r is evaluated against the gate of its
+// last row:  (x_i 2^{g_i - s_r}) . (k_j 2^{s_r - g_j}),  both factors rounded to bf16 before the MFMA.
+// Math and tiling: tests/atk/chunk_kda_fwd/executor_chunk_kda_fwd.py:316-530,
+// fla/ops/ascendc/kda/chunk_kda_fwd/docs/api.md:60-180; operand order of the launch:
+// torch_custom/fla_npu/fla_npu/ops/ascendc/_aclnn_ctypes.py:1066-1265.
+#include <cctype>
+
+#include "gdn_common.h"
+#include "kda_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ f32x4 lds4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+struct KdaIntraParams {
+    ChunkGeom geom;
+    View4 q, k, v;       // bf16, strides of (batch, head, token) in the caller's layout
+    const void *g;       // raw gate, f32 or bf16, same layout family
+    int g_bf16;
+    int64_t g_sb, g_sh, g_st;
+    View3 beta;
+    const float *a_log, *dt_bias;
+    int use_gate, safe_gate;
+    float lower_bound;
+    float scale;
+    float *gk;                // [B,Hv,T,K] or null
+    bf16 *aqk, *akk;          // [B,Hv,T,64]
+    bf16 *w, *u, *qg, *kg;    // [B,Hv,T,K] / [B,Hv,T,V]
+    float *dec;               // [B,NT,Hv,K]: 2^{g_last} of every chunk
+};
+
+// A operand of a 16x16x16 product from four fp32 values, split into a bf16 head and remainder.
+struct HiLo {
+    bf16x4 hi, lo;
+};
+__device__ __forceinline__ HiLo split(f32x4 x) {
+    HiLo r;
+    r.hi = cvt4(x);
+    f32x4 rem;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) rem[e] = x[e] - (float)r.hi[e];
+    r.lo = cvt4(rem);
+    return r;
+}
+// acc += a * b with both operands carried as head + remainder (the lo*lo term is dropped).
+__device__ __forceinline__ f32x4 mm3(f32x4 a, f32x4 b, f32x4 acc) {
+    const HiLo A = split(a), B = split(b);
+    acc = mfma16x16(A.hi, B.hi, acc);
+    acc = mfma16x16(A.lo, B.hi, acc);
+    acc = mfma16x16(A.hi, B.lo, acc);
+    return acc;
+}
+
+// rows row0..row0+15 of `tile` times 2^{+-(g_row - g_anchor)} as an MFMA operand (contraction
+// slots 32j .. 32j+31 along the channels)
+template <bool LEFT>
+__device__ __forceinline__ bf16x8 scaled_frag(const bf16 *tile, int pitch, const float *gS, int pg, int row0, int arow,
+                                              int j) {
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const bf16x8 raw = frag_kc(tile, pitch, row0, 32 * j);
+    const float *gr = gS + (row0 + li) * pg + 32 * j + 4 * lg;
+    const float *ga = gS + arow * pg + 32 * j + 4 * lg;
+    const f32x4 g0 = lds4(gr), g1 = lds4(gr + 16), s0 = lds4(ga), s1 = lds4(ga + 16);
+    f32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        lo[e] = (float)raw[e] * ex2(LEFT ? g0[e] - s0[e] : s0[e] - g0[e]);
+        hi[e] = (float)raw[4 + e] * ex2(LEFT ? g1[e] - s1[e] : s1[e] - g1[e]);
+    }
+    return frag_from_acc(lo, hi);
+}
+
+template <int K, int V> struct IntraSmem {
+    static constexpr int pq = K + 16, pk = K + 8, pg = K + 4, pv = V + 16, pa = 68, pb = 72;
+    static constexpr int SEG = 256 / K;  // token segments of the gate scan
+    static constexpr size_t bytes =
+        (size_t)kChunk * (pq + pk + pv + 2 * pb) * 2 + (size_t)kChunk * (pg + pa + 1) * 4 + (size_t)SEG * K * 4;
+};
+
+// Everything a wave does after the gate scan.  W = wave index (static so tile loops unroll).
+template <int K, int V, int W>
+__device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf16 *kS, bf16 *vS, bf16 *akS, bf16 *aqS,
+                                           float *gS, float *aS, const float *bS, int len, int64_t row_base,
+                                           int64_t dec_base) {
+    using S = IntraSmem<K, V>;
+    constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb;
+    constexpr int KS = K / 32, R1 = W, R2 = 3 - W;
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+
+    // ---- scores: k k^T row tile R1 (and its transposed diagonal tile), q k^T row tile R2 ------------
+    f32x4 kacc[R1 + 1], kaccT = zero4(), qacc[R2 + 1];
+#pragma unroll
+    for (int c = 0; c <= R1; ++c) kacc[c] = zero4();
+#pragma unroll
+    for (int c = 0; c <= R2; ++c) qacc[c] = zero4();
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+        const bf16x8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
+#pragma unroll
+        for (int c = 0; c <= R1; ++c) {
+            const bf16x8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+            kacc[c] = mfma16x32(lk, rk, kacc[c]);
+            if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+        }
+        const bf16x8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+#pragma unroll
+        for (int c = 0; c <= R2; ++c) {
+            const bf16x8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+            qacc[c] = mfma16x32(lq, rk, qacc[c]);
+        }
+    }
+    // lane holds (row 16R + 4lg + e, column 16c + li) of each tile
+    const f32x4 brow = lds4(bS + 16 * R1 + 4 * lg);
+    const float bcol = bS[16 * R1 + li];
+#pragma unroll
+    for (int c = 0; c < R1; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) aS[(16 * R1 + 4 * lg + e) * pa + 16 * c + li] = brow[e] * kacc[c][e];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        f32x4 a = zero4();
+        if (c <= R2) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = (c < R2 || li <= 4 * lg + e) ? p.scale * qacc[c <= R2 ? c : 0][e] : 0.f;
+        }
+        acc_to_tile(aqS, pb, 16 * R2, 16 * c, a);
+    }
+
+    // ---- inverse of the diagonal block: (I + A)^-1 = (I - A)(I + A^2)(I + A^4)(I + A^8) ------------
+    // a2 = A[4lg+e][li] (right operand of A, left operand of A^T); a1 = A[li][4lg+e] (the converse).
+    f32x4 a1, a2, Y;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int r = 4 * lg + e;
+        a2[e] = li < r ? brow[e] * kacc[R1][e] : 0.f;
+        a1[e] = r < li ? bcol * kaccT[e] : 0.f;
+        Y[e] = (r == li ? 1.f : 0.f) - a1[e];   // (I - A^T)[r][li]
+    }
+    {
+        const bf16x4 A1 = cvt4(a1), A2 = cvt4(a2);
+        const f32x4 S1 = mfma16x16(A1, A2, zero4());   // A^2
+        const f32x4 T1 = mfma16x16(A2, A1, zero4());   // (A^2)^T
+        const bf16x4 S1b = cvt4(S1), T1b = cvt4(T1);
+        Y = mfma16x16(S1b, cvt4(Y), Y);
+        const f32x4 S2 = mfma16x16(T1b, S1b, zero4());  // A^4
+        const f32x4 T2 = mfma16x16(S1b, T1b, zero4());  // (A^4)^T
+        const bf16x4 S2b = cvt4(S2);
+        Y = mfma16x16(S2b, cvt4(Y), Y);
+        const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());  // A^8
+        Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
+    }
+    // lane holds Dinv[li][4lg+e]
+    *reinterpret_cast<f32x4 *>(aS + (16 * R1 + li) * pa + 16 * R1 + 4 * lg) = Y;
+    *reinterpret_cast<bf16x4 *>(akS + (16 * R1 + li) * pb + 16 * R1 + 4 * lg) = cvt4(Y);
+#pragma unroll
+    for (int c = R1 + 1; c < 4; ++c)
+        *reinterpret_cast<bf16x4 *>(akS + (16 * R1 + li) * pb + 16 * c + 4 * lg) = bf16x4{(bf16)0.f, (bf16)0.f, (bf16)0.f, (bf16)0.f};
+    __syncthreads();
+
+    // ---- off-diagonal blocks of the inverse, column block W: X_rc = -Dinv_r sum_m A_rm X_mc --------
+    if constexpr (W < 3) {
+        constexpr int C = W;
+        f32x4 X[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) X[C][e] = aS[(16 * C + 4 * lg + e) * pa + 16 * C + li];
+#pragma unroll
+        for (int r = C + 1; r < 4; ++r) {
+            f32x4 sum = zero4();
+#pragma unroll
+            for (int m = C; m < r; ++m) sum = mm3(lds4(aS + (16 * r + li) * pa + 16 * m + 4 * lg), X[m], sum);
+            const f32x4 dinv = lds4(aS + (16 * r + li) * pa + 16 * r + 4 * lg);
+            X[r] = mm3(-dinv, sum, zero4());
+            acc_to_tile(akS, pb, 16 * r, 16 * C, X[r]);
+        }
+    }
+    // ---- gated operands: qg, kg to memory; k beta 2^g over the q tile ----------------------------------
+    for (int idx = threadIdx.x; idx < kChunk * (K / 8); idx += kThreads) {
+        const int r = idx / (K / 8), c8 = (idx % (K / 8)) * 8;
+        const bf16x8 q8 = *reinterpret_cast<const bf16x8 *>(qS + r * pq + c8);
+        const bf16x8 k8 = *reinterpret_cast<const bf16x8 *>(kS + r * pk + c8);
+        const float br = bS[r];
+        bf16x8 qg8, kg8, kb8;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + 63 * pg + c8 + 4 * h);
+            f32x4 a, b, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float eg = ex2(gg[e]), kk = (float)k8[4 * h + e];
+                a[e] = (float)q8[4 * h + e] * eg;
+                b[e] = kk * ex2(gl[e] - gg[e]);
+                c[e] = kk * br * eg;
+            }
+            const bf16x4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                qg8[4 * h + e] = a4[e];
+                kg8[4 * h + e] = b4[e];
+                kb8[4 * h + e] = c4[e];
+            }
+        }
+        if (r < len) {
+            *reinterpret_cast<bf16x8 *>(p.qg + (row_base + r) * K + c8) = qg8;
+            *reinterpret_cast<bf16x8 *>(p.kg + (row_base + r) * K + c8) = kg8;
+        }
+        *reinterpret_cast<bf16x8 *>(qS + r * pq + c8) = kb8;
+    }
+    if (threadIdx.x < K) p.dec[dec_base + threadIdx.x] = ex2(gS[63 * pg + threadIdx.x]);
+    __syncthreads();
+
+    // ---- w = Akk (k beta 2^g), u = Akk (v beta): row tile W ------------------------------------------------
+    f32x4 wacc[K / 16], uacc[V / 16];
+#pragma unroll
+    for (int ct = 0; ct < K / 16; ++ct) wacc[ct] = zero4();
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) uacc[ct] = zero4();
+#pragma unroll
+    for (int j = 0; j < (W < 2 ? 1 : 2); ++j) {   // Akk is lower triangular
+        const bf16x8 a = frag_kc(akS, pb, 16 * W, 32 * j);
+#pragma unroll
+        for (int ct = 0; ct < K / 16; ++ct) wacc[ct] = mfma16x32(a, frag_tr(qS, pq, 16 * ct, 32 * j), wacc[ct]);
+#pragma unroll
+        for (int ct = 0; ct < V / 16; ++ct) uacc[ct] = mfma16x32(a, frag_tr(vS, pv, 16 * ct, 32 * j), uacc[ct]);
+    }
+    __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
+#pragma unroll
+    for (int ct = 0; ct < K / 16; ++ct) acc_to_tile(qS, pq, 16 * W, 16 * ct, wacc[ct]);
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) acc_to_tile(vS, pv, 16 * W, 16 * ct, uacc[ct]);
+    __syncthreads();
+}
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    using S = IntraSmem<K, V>;
+    constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb, SEG = S::SEG;
+    bf16 *qS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = qS + kChunk * pq;
+    bf16 *vS = kS + kChunk * pk;
+    bf16 *akS = vS + kChunk * pv;
+    bf16 *aqS = akS + kChunk * pb;
+    float *gS = reinterpret_cast<float *>(aqS + kChunk * pb);
+    float *aS = gS + kChunk * pg;
+    float *bS = aS + kChunk * pa;
+    float *tS = bS + kChunk;
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x;
+
+    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    load_tile<kThreads>(qS, pq, qg, p.q.st, kChunk, K, len);
+    load_tile<kThreads>(kS, pk, kg, p.k.st, kChunk, K, len);
+    for (int idx = tid; idx < kChunk * (V / 8); idx += kThreads) {   // v * beta
+        const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
+        bf16x8 out;
+        if (r < len) {
+            const bf16x8 v8 = *reinterpret_cast<const bf16x8 *>(vg + (int64_t)r * p.v.st + c8);
+            const float br = load_scalar(p.beta, b, hv, start + r);
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)v8[e] * br;
+                hi[e] = (float)v8[4 + e] * br;
+            }
+            out = frag_from_acc(lo, hi);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[e] = (bf16)0.f;
+        }
+        *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = out;
+    }
+    if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
+
+    // gate activation and prefix sum: thread = (token segment, channel)
+    const int64_t row_base = ((int64_t)b * p.geom.Hv + hv) * p.geom.T + start;   // head-major row of token 0
+    {
+        constexpr int TS = kChunk / SEG;
+        const int ch = tid % K, sg = tid / K;
+        const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
+        float eig = 0.f, bias = 0.f;
+        if (p.use_gate) {
+            eig = __expf(p.a_log[hv]);
+            if (p.dt_bias) bias = p.dt_bias[(int64_t)hv * K + ch];
+        }
+        float acc = 0.f;
+        for (int t0 = 0; t0 < TS; t0 += 8) {
+            float raw[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = sg * TS + t0 + j;
+                raw[j] = 0.f;
+                if (t < len) {
+                    const int64_t off = gbase + (int64_t)t * p.g_st;
+                    raw[j] = p.g_bf16 ? (float)static_cast<const bf16 *>(p.g)[off] : static_cast<const float *>(p.g)[off];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = sg * TS + t0 + j;
+                if (t < len) {
+                    const float a = p.use_gate ? kda_activate(raw[j], bias, eig, p.safe_gate, p.lower_bound) : raw[j];
+                    acc += a * kRcpLn2;
+                }
+                gS[t * pg + ch] = acc;
+            }
+        }
+        tS[sg * K + ch] = acc;
+        __syncthreads();
+        float off = 0.f;
+        for (int s = 0; s < sg; ++s) off += tS[s * K + ch];
+        for (int j = 0; j < TS; ++j) {
+            const int t = sg * TS + j;
+            const float v = gS[t * pg + ch] + off;
+            gS[t * pg + ch] = v;
+            if (p.gk && t < len) p.gk[(row_base + t) * K + ch] = v;
+        }
+    }
+    __syncthreads();
+
+    const int64_t dec_base = (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
+    switch (wave_id()) {
+        case 0: intra_wave<K, V, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 1: intra_wave<K, V, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 2: intra_wave<K, V, 2>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        default: intra_wave<K, V, 3>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+    }
+
+    store_tile<kThreads>(p.w + row_base * K, K, qS, pq, K, len);
+    store_tile<kThreads>(p.u + row_base * V, V, vS, pv, V, len);
+    store_tile<kThreads>(p.aqk + row_base * kChunk, kChunk, aqS, pb, kChunk, len);
+    store_tile<kThreads>(p.akk + row_base * kChunk, kChunk, akS, pb, kChunk, len);
+}
+
+// =============================================================================================
+// inter-chunk scan
+// =============================================================================================
+struct KdaScanParams {
+    ChunkGeom geom;
+    const bf16 *w, *u, *qg, *kg, *aqk;   // head-major [B,Hv,T,*]
+    const float *dec;                    // [B,NT,Hv,K]
+    View4 o;                             // attention output in the caller's layout
+    bf16 *v_new;                         // [B,Hv,T,V] or null
+    const float *h0;
+    float *hT;
+    bf16 *h;
+    int64_t h_sb, h_sc, h_sh;            // strides of h over (batch, chunk, head)
+    int64_t s_sn, s_sh;                  // strides of h0 / hT over (sequence, head)
+    int v_first;
+    float scale;
+};
+
+template <int K>
+__global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int VS = 64;
+    constexpr int pw = K + 8, pt = K + 16, pu = VS + 16, pb = 72, po = VS + 8;
+    constexpr int KT = K / 16, KS = K / 32;
+    bf16 *wS = reinterpret_cast<bf16 *>(smem);   // w, later the o staging
+    bf16 *qS = wS + kChunk * pw;                 // qg
+    bf16 *kS = qS + kChunk * pw;                 // kg (read transposed)
+    bf16 *uS = kS + kChunk * pt;                 // u slab, later v_new
+    bf16 *aS = uS + kChunk * pu;                 // Aqk
+    float *dS = reinterpret_cast<float *>(aS + kChunk * pb);   // [K] decay of the chunk
+
+    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+        chunk0 = p.geom.choff[n];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int wv = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int vcol0 = slab * VS + wv * 16;
+
+    f32x4 hacc[KT];
+    auto state_off = [&](int kk, int v) -> int64_t { return p.v_first ? (int64_t)v * K + kk : (int64_t)kk * V + v; };
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        f32x4 a = zero4();
+        if (p.h0) {
+            const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = s[state_off(16 * kt + 4 * lg + e, vcol0 + li)];
+        }
+        hacc[kt] = a;
+    }
+
+    const int64_t head_row = ((int64_t)b * p.geom.Hv + hv) * p.geom.T;
+    bf16 *og = static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + slab * VS;
+
+    for (int c = 0; c < nchunks; ++c) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        const int64_t row = head_row + start;
+        __syncthreads();
+        load_tile<kThreads>(wS, pw, p.w + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(qS, pw, p.qg + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(kS, pt, p.kg + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(uS, pu, p.u + row * V + slab * VS, V, kChunk, VS, len);
+        load_tile<kThreads>(aS, pb, p.aqk + row * kChunk, kChunk, kChunk, kChunk, len);
+        if (threadIdx.x < K) dS[threadIdx.x] = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c) * p.geom.Hv + hv) * K + threadIdx.x];
+        __syncthreads();
+
+        bf16x8 hB[KS];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+        if (p.h) {
+            bf16 *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c) * p.h_sc + hv * p.h_sh;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hg[state_off(16 * kt + 4 * lg + e, vcol0 + li)] = hB[kt >> 1][(kt & 1) * 4 + e];
+        }
+
+        // v_new = u - w S ;  o = scale qg S
+        f32x4 vn[4], oacc[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) vn[rt] = oacc[rt] = zero4();
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                vn[rt] = mfma16x32(frag_kc(wS, pw, rt * 16, 32 * j), hB[j], vn[rt]);
+                oacc[rt] = mfma16x32(frag_kc(qS, pw, rt * 16, 32 * j), hB[j], oacc[rt]);
+            }
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const bf16x4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vn[rt][e] = (float)uu[e] - vn[rt][e];
+                oacc[rt][e] *= p.scale;
+            }
+        }
+        if (p.v_new) {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
+        }
+        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same bf16 v_new operand serves both)
+        bf16x8 vB[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(aS, pb, rt * 16, 32 * j), vB[j], oacc[rt]);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) hacc[kt] *= lds4(dS + 16 * kt + 4 * lg);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 32 * j), vB[j], hacc[kt]);
+        __syncthreads();   // w tile consumed by every wave, v_new tile complete
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) acc_to_tile(wS, po, rt * 16, wv * 16, oacc[rt]);
+        if (p.v_new) store_tile<kThreads>(p.v_new + row * V + slab * VS, V, uS, pu, VS, len);
+        __syncthreads();
+        store_tile<kThreads>(og + (int64_t)start * p.o.st, p.o.st, wS, po, VS, len);
+    }
+
+    if (p.hT) {
+        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[state_off(16 * kt + 4 * lg + e, vcol0 + li)] = hacc[kt][e];
+    }
+}
+
+// =============================================================================================
+// host side
+// =============================================================================================
+struct Layout {
+    int ib, ih, it;   // dims of batch / head / token; ib < 0 when rank 3
+    bool rank3() const { return ib < 0; }
+};
+
+int parse_layout(const char *op, const char *layout, Layout &L) {
+    FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
+    if (!strcmp(layout, "BSND")) L = Layout{0, 2, 1};
+    else if (!strcmp(layout, "BNSD")) L = Layout{0, 1, 2};
+    else if (!strcmp(layout, "TND")) L = Layout{-1, 1, 0};
+    else if (!strcmp(layout, "NTD")) L = Layout{-1, 0, 1};
+    else return fail(FLA_ERR_UNSUPPORTED, "%s: layout must be uppercase and one of BSND, BNSD, TND, NTD.", op);
+    return FLA_OK;
+}
+
+// [.., D] activation in layout L: checks rank, extents, alignment and returns the strided view
+int layout_view(const char *op, const char *name, const fla_tensor *t, const Layout &L, int64_t B, int64_t H, int64_t T,
+                int64_t D, int dtype_mask, int64_t &sb, int64_t &sh, int64_t &st) {
+    int rc = check_tensor(t, op, name, L.rank3() ? 3 : 4, dtype_mask);
+    if (rc) return rc;
+    const int last = t->ndim - 1;
+    FLA_REQUIRE((L.rank3() || t->shape[L.ib] == B) && t->shape[L.ih] == H && t->shape[L.it] == T && t->shape[last] == D,
+                FLA_ERR_SHAPE, "%s: shape of %s does not match the selected layout.", op, name);
+    FLA_REQUIRE(inner_unit(t), FLA_ERR_SHAPE, "%s: innermost stride of %s must be 1.", op, name);
+    sb = L.rank3() ? 0 : t->stride[L.ib];
+    sh = t->stride[L.ih];
+    st = t->stride[L.it];
+    const int64_t al = 16 / (int64_t)dtype_size(t->dtype);
+    FLA_REQUIRE(sb % al == 0 && sh % al == 0 && st % al == 0 && reinterpret_cast<uintptr_t>(t->data) % 16 == 0, FLA_ERR_SHAPE,
+                "%s: rows of %s must be 16-byte aligned.", op, name);
+    return FLA_OK;
+}
+
+// head-major output [B,Hv,T,D] (or [Hv,T,D]); contiguous
+int head_major(const char *op, const char *name, const fla_tensor *t, bool rank3, int64_t B, int64_t H, int64_t T, int64_t D,
+               int dtype) {
+    int rc = check_tensor(t, op, name, rank3 ? 3 : 4, dt_bit(dtype));
+    if (rc) return rc;
+    const int o = rank3 ? 0 : 1;
+    FLA_REQUIRE((rank3 || t->shape[0] == B) && t->shape[o] == H && t->shape[o + 1] == T && t->shape[o + 2] == D &&
+                    is_contiguous(t) && reinterpret_cast<uintptr_t>(t->data) % 16 == 0,
+                FLA_ERR_SHAPE, "%s: %s must be a contiguous head-major tensor [..,%lld,%lld,%lld].", op, name, (long long)H,
+                (long long)T, (long long)D);
+    return FLA_OK;
+}
+
+inline bool present(const fla_tensor *t) { return t != nullptr && t->data != nullptr; }
+inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+template <int K, int V>
+int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
+    const size_t smem = IntraSmem<K, V>::bytes;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem,
+               stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+template <int K>
+int launch_scan(const KdaScanParams &p, hipStream_t stream) {
+    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (K + 16) + 80 + 72)) * 2 + K * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(kThreads), smem,
+               stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
+                 const fla_tensor *a_log, const fla_tensor *dt_bias, const fla_tensor *initial_state,
+                 const fla_int_array *cu, const fla_int_array *ci, const char *layout, double scale, int64_t chunk_size,
+                 bool safe_gate, double lower_bound, bool use_gate, bool state_v_first, const fla_tensor *attn_out,
+                 const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *aqk, const fla_tensor *akk,
+                 const fla_tensor *w, const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg,
+                 const fla_tensor *v_new, const fla_tensor *h, void *ws, uint64_t ws_size, hipStream_t stream,
+                 uint64_t *query) {
+    const char *op = "chunk_kda_fwd";
+    Layout L;
+    int rc;
+    if ((rc = parse_layout(op, layout, L))) return rc;
+    FLA_REQUIRE(chunk_size == 64 || chunk_size == 128, FLA_ERR_SHAPE, "%s: chunk_size must be 64 or 128.", op);
+    FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: only chunk_size 64 is implemented.", op);
+    if ((rc = check_tensor(q, op, "q", L.rank3() ? 3 : 4, dt_bit(FLA_BF16) | dt_bit(FLA_F16)))) return rc;
+    FLA_REQUIRE(q->dtype == FLA_BF16, FLA_ERR_UNSUPPORTED, "%s: only bfloat16 q/k/v are implemented.", op);
+    if ((rc = check_tensor(v, op, "v", L.rank3() ? 3 : 4, dt_bit(FLA_BF16)))) return rc;
+    const int last = q->ndim - 1;
+    ChunkGeom geom{};
+    geom.B = L.rank3() ? 1 : (int)q->shape[L.ib];
+    geom.T = (int)q->shape[L.it];
+    geom.Hk = (int)q->shape[L.ih];
+    geom.K = (int)q->shape[last];
+    geom.Hv = (int)v->shape[L.ih];
+    geom.V = (int)v->shape[last];
+    FLA_REQUIRE(q->shape[L.it] < ((int64_t)1 << 31) && geom.B < 65536, FLA_ERR_SHAPE, "%s: extents too large.", op);
+    FLA_REQUIRE(geom.Hk > 0 && geom.Hv >= geom.Hk && geom.Hv % geom.Hk == 0 && geom.Hv <= 128, FLA_ERR_SHAPE,
+                "%s: H/HV must satisfy 0 < H <= HV <= 128 and HV %% H == 0.", op);
+    FLA_REQUIRE((geom.K == 64 || geom.K == 128) && (geom.V == 64 || geom.V == 128 || geom.V == 256) && geom.V >= geom.K,
+                FLA_ERR_UNSUPPORTED, "%s: implemented head sizes are K in {64,128} with V in {K, 2K}, got K=%d V=%d.", op,
+                geom.K, geom.V);
+    const int64_t B = geom.B, T = geom.T, Hk = geom.Hk, Hv = geom.Hv, K = geom.K, V = geom.V;
+    const int bf = dt_bit(FLA_BF16), f32 = dt_bit(FLA_F32);
+    KdaIntraParams ip{};
+    if ((rc = layout_view(op, "q", q, L, B, Hk, T, K, bf, ip.q.sb, ip.q.sh, ip.q.st))) return rc;
+    if ((rc = layout_view(op, "k", k, L, B, Hk, T, K, bf, ip.k.sb, ip.k.sh, ip.k.st))) return rc;
+    if ((rc = layout_view(op, "v", v, L, B, Hv, T, V, bf, ip.v.sb, ip.v.sh, ip.v.st))) return rc;
+    ip.q.p = q->data;
+    ip.k.p = k->data;
+    ip.v.p = v->data;
+    {   // g: scalar loads, no alignment requirement beyond the element
+        if ((rc = check_tensor(g, op, "g", L.rank3() ? 3 : 4, bf | f32))) return rc;
+        FLA_REQUIRE((L.rank3() || g->shape[L.ib] == B) && g->shape[L.ih] == Hv && g->shape[L.it] == T &&
+                        g->shape[g->ndim - 1] == K && inner_unit(g),
+                    FLA_ERR_SHAPE, "%s: v/g/beta shapes do not match the selected layout.", op);
+        ip.g = g->data;
+        ip.g_bf16 = g->dtype == FLA_BF16;
+        ip.g_sb = L.rank3() ? 0 : g->stride[L.ib];
+        ip.g_sh = g->stride[L.ih];
+        ip.g_st = g->stride[L.it];
+    }
+    {
+        if ((rc = check_tensor(beta, op, "beta", L.rank3() ? 2 : 3, bf | f32))) return rc;
+        FLA_REQUIRE((L.rank3() || beta->shape[L.ib] == B) && beta->shape[L.ih] == Hv && beta->shape[L.it] == T, FLA_ERR_SHAPE,
+                    "%s: v/g/beta shapes do not match the selected layout.", op);
+        ip.beta = View3{beta->data, L.rank3() ? 0 : beta->stride[L.ib], beta->stride[L.ih], beta->stride[L.it],
+                        beta->dtype == FLA_BF16 ? 1 : 0};
+    }
+    if (use_gate) {
+        FLA_REQUIRE(present(a_log) && a_log->ndim == 1 && a_log->shape[0] == Hv && a_log->dtype == FLA_F32 &&
+                        a_log->stride[0] == 1,
+                    FLA_ERR_SHAPE, "%s: A_log must be float32 [HV] when use_gate_in_kernel=True.", op);
+        if (present(dt_bias))
+            FLA_REQUIRE(dt_bias->ndim == 1 && dt_bias->shape[0] == Hv * K && dt_bias->dtype == FLA_F32 && dt_bias->stride[0] == 1,
+                        FLA_ERR_SHAPE, "%s: dt_bias must be float32 [HV*K].", op);
+        FLA_REQUIRE(!safe_gate || (lower_bound >= -5.0 && lower_bound < 0.0), FLA_ERR_SHAPE,
+                    "%s: lower_bound must be in [-5, 0) for safe gate.", op);
+    }
+    Varlen vl;
+    if ((rc = build_varlen(vl, op, cu, ci, kChunk, T))) return rc;
+    FLA_REQUIRE(!vl.enabled || B == 1, FLA_ERR_SHAPE, "%s: rank4 varlen input requires B=1.", op);
+    FLA_REQUIRE(!vl.enabled || vl.N <= 1024, FLA_ERR_SHAPE, "%s: varlen input supports at most 1024 sequences.", op);
+    geom.NT = vl.enabled ? vl.NT : (int)((T + kChunk - 1) / kChunk);
+    geom.N = vl.enabled ? vl.N : (int)B;
+    const int64_t NT = geom.NT, N = geom.N;
+
+    // outputs
+    KdaScanParams sp{};
+    if ((rc = layout_view(op, "attn_out", attn_out, L, B, Hv, T, V, bf, sp.o.sb, sp.o.sh, sp.o.st))) return rc;
+    sp.o.p = attn_out->data;
+    if ((rc = head_major(op, "Aqk", aqk, L.rank3(), B, Hv, T, kChunk, FLA_BF16))) return rc;
+    if ((rc = head_major(op, "Akk", akk, L.rank3(), B, Hv, T, kChunk, FLA_BF16))) return rc;
+    if (present(gk) && (rc = head_major(op, "gk", gk, L.rank3(), B, Hv, T, K, FLA_F32))) return rc;
+    if (present(w) && (rc = head_major(op, "w", w, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
+    if (present(u) && (rc = head_major(op, "u", u, L.rank3(), B, Hv, T, V, FLA_BF16))) return rc;
+    if (present(qg) && (rc = head_major(op, "qg", qg, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
+    if (present(kg) && (rc = head_major(op, "kg", kg, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
+    if (present(v_new) && (rc = head_major(op, "v_new", v_new, L.rank3(), B, Hv, T, V, FLA_BF16))) return rc;
+    const int64_t d2 = state_v_first ? V : K, d3 = state_v_first ? K : V;
+    auto check_state = [&](const fla_tensor *s, const char *name) -> int {
+        int r = check_tensor(s, op, name, 4, f32);
+        if (r) return r;
+        FLA_REQUIRE(s->shape[0] == N && s->shape[1] == Hv && s->shape[2] == d2 && s->shape[3] == d3 && s->stride[3] == 1 &&
+                        s->stride[2] == d3,
+                    FLA_ERR_SHAPE, "%s: %s shape/dtype does not match state_v_first.", op, name);
+        return FLA_OK;
+    };
+    if (present(initial_state) && (rc = check_state(initial_state, "initial_state"))) return rc;
+    if (present(final_state) && (rc = check_state(final_state, "final_state"))) return rc;
+    if (present(h)) {
+        if ((rc = check_tensor(h, op, "h", L.rank3() ? 4 : 5, bf))) return rc;
+        const int o = L.rank3() ? 0 : 1;
+        FLA_REQUIRE((L.rank3() || h->shape[0] == B) && h->shape[o] == NT && h->shape[o + 1] == Hv && h->shape[o + 2] == d2 &&
+                        h->shape[o + 3] == d3 && h->stride[o + 3] == 1 && h->stride[o + 2] == d3,
+                    FLA_ERR_SHAPE, "%s: h must be [..,NT=%lld,HV,%lld,%lld].", op, (long long)NT, (long long)d2, (long long)d3);
+        sp.h = static_cast<bf16 *>(h->data);
+        sp.h_sb = L.rank3() ? 0 : h->stride[0];
+        sp.h_sc = h->stride[o];
+        sp.h_sh = h->stride[o + 1];
+    }
+
+    // workspace: varlen table | decay rows | the intermediates the caller did not ask for
+    const size_t rows = (size_t)B * Hv * T;
+    size_t off = vl.bytes();
+    const size_t dec_off = off;
+    off += align256((size_t)B * NT * Hv * K * 4);
+    size_t w_off = 0, u_off = 0, qg_off = 0, kg_off = 0;
+    if (!present(w)) { w_off = off; off += align256(rows * K * 2); }
+    if (!present(u)) { u_off = off; off += align256(rows * V * 2); }
+    if (!present(qg)) { qg_off = off; off += align256(rows * K * 2); }
+    if (!present(kg)) { kg_off = off; off += align256(rows * K * 2); }
+    if (query) {
+        *query = off;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(off == 0 || (ws && ws_size >= off), FLA_ERR_WORKSPACE, "%s: workspace of %zu bytes required.", op, off);
+    FLA_REQUIRE(reinterpret_cast<uintptr_t>(ws) % 256 == 0, FLA_ERR_WORKSPACE, "%s: workspace must be 256-byte aligned.", op);
+    if ((rc = upload_varlen(vl, ws, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    if (B == 0 || T == 0 || NT == 0) return FLA_OK;
+    unsigned char *wsb = static_cast<unsigned char *>(ws);
+
+    ip.geom = geom;
+    ip.a_log = use_gate ? static_cast<const float *>(a_log->data) : nullptr;
+    ip.dt_bias = use_gate && present(dt_bias) ? static_cast<const float *>(dt_bias->data) : nullptr;
+    ip.use_gate = use_gate;
+    ip.safe_gate = safe_gate;
+    ip.lower_bound = (float)lower_bound;
+    ip.scale = (float)scale;
+    ip.gk = present(gk) ? static_cast<float *>(gk->data) : nullptr;
+    ip.aqk = static_cast<bf16 *>(aqk->data);
+    ip.akk = static_cast<bf16 *>(akk->data);
+    ip.w = present(w) ? static_cast<bf16 *>(w->data) : reinterpret_cast<bf16 *>(wsb + w_off);
+    ip.u = present(u) ? static_cast<bf16 *>(u->data) : reinterpret_cast<bf16 *>(wsb + u_off);
+    ip.qg = present(qg) ? static_cast<bf16 *>(qg->data) : reinterpret_cast<bf16 *>(wsb + qg_off);
+    ip.kg = present(kg) ? static_cast<bf16 *>(kg->data) : reinterpret_cast<bf16 *>(wsb + kg_off);
+    ip.dec = reinterpret_cast<float *>(wsb + dec_off);
+    if (K == 128 && V == 128) rc = launch_intra<128, 128>(ip, stream);
+    else if (K == 128 && V == 256) rc = launch_intra<128, 256>(ip, stream);
+    else if (K == 64 && V == 64) rc = launch_intra<64, 64>(ip, stream);
+    else rc = launch_intra<64, 128>(ip, stream);
+    if (rc) return rc;
+
+    sp.geom = geom;
+    sp.w = ip.w;
+    sp.u = ip.u;
+    sp.qg = ip.qg;
+    sp.kg = ip.kg;
+    sp.aqk = ip.aqk;
+    sp.dec = ip.dec;
+    sp.v_new = present(v_new) ? static_cast<bf16 *>(v_new->data) : nullptr;
+    if (present(initial_state)) {
+        sp.h0 = static_cast<const float *>(initial_state->data);
+        sp.s_sn = initial_state->stride[0];
+        sp.s_sh = initial_state->stride[1];
+    }
+    if (present(final_state)) {
+        sp.hT = static_cast<float *>(final_state->data);
+        FLA_REQUIRE(!sp.h0 || (final_state->stride[0] == sp.s_sn && final_state->stride[1] == sp.s_sh), FLA_ERR_SHAPE,
+                    "%s: initial_state and final_state must share strides.", op);
+        sp.s_sn = final_state->stride[0];
+        sp.s_sh = final_state->stride[1];
+    }
+    sp.v_first = state_v_first;
+    sp.scale = (float)scale;
+    if (N == 0) return FLA_OK;
+    return K == 128 ? launch_scan<128>(sp, stream) : launch_scan<64>(sp, stream);
+}
+
+}  // namespace
+}  // namespace fla
+
+extern "C" int fla_chunk_kda_fwd_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
+    const fla_tensor *A_log, const fla_tensor *dt_bias, const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size, bool safe_gate,
+    double lower_bound, bool use_gate_in_kernel, bool state_v_first, const fla_tensor *attn_out,
+    const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w,
+    const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
+    uint64_t *workspace_size) {
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_fwd: workspace_size must not be null.");
+    return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
+                             chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
+                             Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, workspace_size);
+}
+
+extern "C" int fla_chunk_kda_fwd(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
+    const fla_tensor *A_log, const fla_tensor *dt_bias, const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size, bool safe_gate,
+    double lower_bound, bool use_gate_in_kernel, bool state_v_first, const fla_tensor *attn_out,
+    const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w,
+    const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
+    void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
+                             chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
+                             Aqk, Akk, w, u, qg, kg, v_new, h, workspace, workspace_size, static_cast<hipStream_t>(stream),
+                             nullptr);
+}

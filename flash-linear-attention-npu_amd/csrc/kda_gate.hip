@@ -7,11 +7,10 @@
 // channels of one chunk and walks its tokens; eight token rows are in flight per thread so the
 // serial dependence of the prefix sum does not serialise the loads.
 #include "gdn_common.h"
+#include "kda_common.h"
 
 namespace fla {
 namespace {
-
-constexpr float kRcpLn2 = 1.4426950408889634f;
 
 struct GateParams {
     const void *g;
@@ -33,13 +32,6 @@ template <> __device__ __forceinline__ f32x4 load4<float>(const void *p, int64_t
 template <> __device__ __forceinline__ f32x4 load4<bf16>(const void *p, int64_t i) {
     const bf16x4 v = *reinterpret_cast<const bf16x4 *>(static_cast<const bf16 *>(p) + i);
     return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
-}
-
-__device__ __forceinline__ float activate(float x, float bias, float eig, int safe, float lb) {
-    const float raw = x + bias;
-    if (safe) return lb / (1.f + __expf(-eig * raw));
-    const float sp = fmaxf(raw, 0.f) + __logf(1.f + __expf(-fabsf(raw)));
-    return -eig * sp;
 }
 
 template <typename TI, int TPC>  // TPC = threads per chunk = K / 4
@@ -80,7 +72,7 @@ __global__ void __launch_bounds__(256) kda_gate_cumsum_kernel(const GateParams p
                 f32x4 v = rows[j];
                 if (p.use_gate) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = activate(v[e], bias[e], eig, p.safe_gate, p.lower_bound);
+                    for (int e = 0; e < 4; ++e) v[e] = kda_activate(v[e], bias[e], eig, p.safe_gate, p.lower_bound);
                 }
                 acc += v * kRcpLn2;
                 __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(p.out + base + (int64_t)(t0 + j) * K));

@@ -37,6 +37,8 @@ OP_ARGTYPES = {
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
     "kda_gate_cumsum": [_T, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool, ctypes.c_double, _T],
+    "chunk_kda_fwd": [_T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_char_p, ctypes.c_double, ctypes.c_int64,
+                      ctypes.c_bool, ctypes.c_double, ctypes.c_bool, ctypes.c_bool] + [_T] * 11,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
 }
@@ -468,6 +470,126 @@ def npu_chunk_gated_delta_rule_bwd_dhu(q, k, w, d_o, dv, scale, chunk_size, *, g
         ],
         outputs,
     )
+
+
+def kda_fwd_optional_output_mask(*, output_final_state, use_gate_in_kernel, disable_recompute,
+                                 return_intermediate_states):
+    """Which of the 12 values of ``npu_chunk_kda_fwd`` are materialised
+    (ops/ascendc/_kda_policy.py:16-39): o, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, initial_state."""
+    keep = bool(disable_recompute)
+    return (True, bool(output_final_state), (not use_gate_in_kernel) or keep, True, True, keep, keep, keep, keep, keep,
+            keep or bool(return_intermediate_states), True)
+
+
+def npu_chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", initial_state=None,
+                      output_final_state=False, cu_seqlens=None, chunk_indices=None, safe_gate=False, lower_bound=None,
+                      use_gate_in_kernel=False, A_log=None, dt_bias=None, disable_recompute=False,
+                      return_intermediate_states=False, state_v_first=False):
+    """KDA chunk forward (_aclnn_ctypes.py:1066-1265).  Returns the 12-tuple
+    ``(o, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, initial_state)``; entries the output policy
+    hides are ``None``."""
+    import torch
+
+    op = "npu_chunk_kda_fwd"
+    layout = str(layout)
+    if layout not in {"BSND", "BNSD", "TND", "NTD"}:
+        raise RuntimeError(f"{op}: layout must be uppercase and one of BSND, BNSD, TND, NTD.")
+    chunk_size = int(chunk_size)
+    if chunk_size not in {64, 128}:
+        raise RuntimeError(f"{op}: chunk_size must be 64 or 128.")
+    rank3 = layout in {"TND", "NTD"}
+    shapes = [_shape(t) for t in (q, k, v, g, beta)]
+    qs, ks, vs, gs, bs = shapes
+    rank = 3 if rank3 else 4
+    if any(len(s) != rank for s in (qs, ks, vs, gs)):
+        raise RuntimeError(f"{op}: q/k/v/g rank does not match layout.")
+    if len(bs) != rank - 1 or qs != ks:
+        raise RuntimeError(f"{op}: beta rank must match layout and q/k shapes must be identical.")
+    t_dim, h_dim = {"BSND": (1, 2), "BNSD": (2, 1), "TND": (0, 1), "NTD": (1, 0)}[layout]
+    B = 1 if rank3 else qs[0]
+    T, H, K = qs[t_dim], qs[h_dim], qs[-1]
+    HV, V = vs[h_dim], vs[-1]
+
+    def in_layout(heads, *tail):
+        dims = [None] * (rank - 1)
+        dims[t_dim], dims[h_dim] = T, heads
+        if not rank3:
+            dims[0] = B
+        return (*dims, *tail)
+
+    if vs != in_layout(HV, V) or gs != in_layout(HV, K) or bs != in_layout(HV):
+        raise RuntimeError(f"{op}: v/g/beta shapes do not match the selected layout.")
+    if H <= 0 or HV < H or HV % H != 0 or H > 128 or HV > 128:
+        raise RuntimeError(f"{op}: H/HV must satisfy 0 < H <= HV <= 128 and HV % H == 0.")
+    if q.dtype not in {torch.float16, torch.bfloat16} or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError(f"{op}: q/k/v must use the same float16 or bfloat16 dtype.")
+    if g.dtype not in {torch.float32, torch.bfloat16} or beta.dtype not in {torch.float32, torch.bfloat16}:
+        raise RuntimeError(f"{op}: g and beta must be float32 or bfloat16.")
+    if K < 16 or K > 256 or K % 16 or V < 16 or V > 256 or V % 16:
+        raise RuntimeError(f"{op}: K/V must be multiples of 16 with K,V <= 256.")
+    use_gate_in_kernel = _optional_bool(use_gate_in_kernel, False)
+    safe_gate = _optional_bool(safe_gate, False)
+    disable_recompute = _optional_bool(disable_recompute, False)
+    return_intermediate_states = _optional_bool(return_intermediate_states, False)
+    output_final_state = _optional_bool(output_final_state, False)
+    state_v_first = _optional_bool(state_v_first, False)
+    if use_gate_in_kernel:
+        if A_log is None or _shape(A_log) != (HV,) or A_log.dtype != torch.float32:
+            raise RuntimeError(f"{op}: A_log must be float32 [HV] when use_gate_in_kernel=True.")
+        if dt_bias is not None and (_shape(dt_bias) != (HV * K,) or dt_bias.dtype != torch.float32):
+            raise RuntimeError(f"{op}: dt_bias must be float32 [HV*K].")
+    lower_bound = _optional_float(lower_bound, -5.0)
+    if use_gate_in_kernel and safe_gate and not (-5.0 <= lower_bound < 0.0):
+        raise RuntimeError(f"{op}: lower_bound must be in [-5, 0) for safe gate.")
+    cu = _as_int_tuple(cu_seqlens)
+    if cu is not None:
+        if len(cu) < 2 or cu[0] != 0 or cu[-1] != T or any(a > b for a, b in zip(cu, cu[1:])):
+            raise RuntimeError(f"{op}: cu_seqlens must be nondecreasing, start at 0 and end at T.")
+        if len(cu) - 1 > 1024:
+            raise RuntimeError(f"{op}: varlen input supports at most 1024 sequences.")
+        if not rank3 and B != 1:
+            raise RuntimeError(f"{op}: rank4 varlen input requires B=1.")
+    N = len(cu) - 1 if cu is not None else B
+    canonical = None if cu is None else _build_chunk_indices(cu, chunk_size)
+    indices = canonical if chunk_indices is None else _as_int_tuple(chunk_indices)
+    if indices is not None and indices != canonical:
+        raise RuntimeError(f"{op}: chunk_indices must use canonical sequence-major order.")
+    NT = _total_chunks(B, T, chunk_size, cu)
+    state_shape = (N, HV, V, K) if state_v_first else (N, HV, K, V)
+    if initial_state is not None and (_shape(initial_state) != state_shape or initial_state.dtype != torch.float32):
+        raise RuntimeError(f"{op}: initial_state shape/dtype does not match state_v_first.")
+
+    lead = () if rank3 else (B,)
+    block = (V, K) if state_v_first else (K, V)
+    mask = kda_fwd_optional_output_mask(output_final_state=output_final_state, use_gate_in_kernel=use_gate_in_kernel,
+                                        disable_recompute=disable_recompute,
+                                        return_intermediate_states=return_intermediate_states)
+    attn_out = _empty(in_layout(HV, V), q)
+    final_state = _empty(state_shape, q, dtype=torch.float32) if mask[1] else None
+    gk = _empty((*lead, HV, T, K), q, dtype=torch.float32) if mask[2] else None
+    aqk = _empty((*lead, HV, T, chunk_size), q)
+    akk = _empty((*lead, HV, T, chunk_size), q)
+    w = _empty((*lead, HV, T, K), q) if mask[5] else None
+    u = _empty((*lead, HV, T, V), q) if mask[6] else None
+    qg = _empty((*lead, HV, T, K), q) if mask[7] else None
+    kg = _empty((*lead, HV, T, K), q) if mask[8] else None
+    v_new = _empty((*lead, HV, T, V), q) if mask[9] else None
+    h = _empty((*lead, NT, HV, *block), q) if mask[10] else None
+    outputs = (attn_out, final_state, gk, aqk, akk, w, u, qg, kg, v_new, h)
+    names = ("attn_out", "final_state", "gk", "Aqk", "Akk", "w", "u", "qg", "kg", "v_new", "h")
+    _call_op(
+        "chunk_kda_fwd", OP_ARGTYPES["chunk_kda_fwd"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"), ctx.tensor(beta, "beta"),
+            ctx.tensor(A_log, "A_log"), ctx.tensor(dt_bias, "dt_bias"), ctx.tensor(initial_state, "initial_state"),
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_char_p(layout.encode("utf-8")),
+            ctypes.c_double(float(scale)), ctypes.c_int64(chunk_size), ctypes.c_bool(safe_gate),
+            ctypes.c_double(lower_bound), ctypes.c_bool(use_gate_in_kernel), ctypes.c_bool(state_v_first),
+            *[ctx.tensor(t, n) for t, n in zip(outputs, names)],
+        ],
+        outputs,
+    )
+    return (*outputs, initial_state)
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

@@ -278,6 +278,40 @@ int fla_chunk_gated_delta_rule_bwd_dhu(
     const fla_tensor *dh0, const fla_tensor *dv2, void *workspace, uint64_t workspace_size,
     void *stream);
 
+/* ------------------------------------------------------------------------
+ * chunk_kda_fwd - replaces aclnnChunkKdaFwd (_aclnn_ctypes.py:1066-1265;
+ * fla/ops/ascendc/kda/chunk_kda_fwd/docs/api.md).  layout is "BSND", "BNSD",
+ * "TND" or "NTD" and applies to q,k [..H,K], v [..HV,V], g [..HV,K] (raw gate,
+ * f32/bf16), beta [..HV] (f32/bf16) and attn_out (like v).  A_log [HV] and
+ * dt_bias [HV*K] f32 are used when use_gate_in_kernel.  States are f32
+ * [N,HV,K,V] ([N,HV,V,K] when state_v_first).  The remaining outputs are
+ * head-major: gk f32 [..HV,T,K] (chunk-local cumulated gate, log2 units),
+ * Aqk, Akk [..HV,T,chunk], w, qg, kg [..HV,T,K], u, v_new [..HV,T,V], and
+ * h [B,NT,HV,K,V] (rank-3 layouts: [NT,HV,K,V]).  final_state, gk, w, u, qg,
+ * kg, v_new and h may be null.  Implemented: bf16 q/k/v, chunk_size 64,
+ * K in {64,128}, V in {K, 2K}.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_kda_fwd_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size,
+    bool safe_gate, double lower_bound, bool use_gate_in_kernel, bool state_v_first,
+    const fla_tensor *attn_out, const fla_tensor *final_state, const fla_tensor *gk,
+    const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w, const fla_tensor *u,
+    const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
+    uint64_t *workspace_size);
+int fla_chunk_kda_fwd(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size,
+    bool safe_gate, double lower_bound, bool use_gate_in_kernel, bool state_v_first,
+    const fla_tensor *attn_out, const fla_tensor *final_state, const fla_tensor *gk,
+    const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w, const fla_tensor *u,
+    const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
+    void *workspace, uint64_t workspace_size, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,169 @@
+"""Parity of chunk_kda_fwd (through the C ABI) against the CPU oracle.
+
+Acceptance: attention output within 2e-2 and final state within 1e-3 (relative to the state's
+scale) of the fp32 per-token recurrence; every intermediate of the 12-tuple within 2e-2 of the
+chunked fp32 restatement.  Cases follow the reference sweep: the four layouts, GVA, ragged tails,
+packed variable-length batches with an empty sequence, in-kernel gate activations, initial state,
+V-first state blocks, and the optional-output policy."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn, kda
+from util import assert_close, TOL_BF16, TOL_STATE
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def make_inputs(B, T, Hk, Hv, K, V, seed, *, raw_gate=False, gate_scale=0.3, g_dtype=torch.float32, beta_dtype=torch.float32):
+    gen = torch.Generator().manual_seed(seed)
+    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
+    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
+    v = torch.randn(B, Hv, T, V, generator=gen).to(BF)
+    if raw_gate:
+        g = torch.randn(B, Hv, T, K, generator=gen).to(g_dtype)
+    else:
+        g = (F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * gate_scale).to(g_dtype)
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen)).to(beta_dtype)
+    return q, k, v, g, beta
+
+
+def to_layout(x, layout, scalar=False):
+    """head-major [B,H,T,(D)] -> the caller's layout"""
+    if layout == "BNSD":
+        return x.contiguous()
+    if layout == "BSND":
+        return x.transpose(1, 2).contiguous()
+    if layout == "NTD":
+        return x[0].contiguous()
+    return x[0].transpose(0, 1).contiguous()   # TND
+
+
+def from_layout(x, layout):
+    if layout == "BNSD":
+        return x
+    if layout == "BSND":
+        return x.transpose(1, 2)
+    if layout == "NTD":
+        return x[None]
+    return x.transpose(0, 1)[None]
+
+
+CASES = [
+    # B, T, Hk, Hv, K, V, layout, cu, gate kwargs, h0, v_first
+    dict(B=2, T=256, Hk=2, Hv=2, K=128, V=128, layout="BSND"),
+    dict(B=1, T=200, Hk=2, Hv=4, K=128, V=128, layout="BNSD", h0=True),                       # GVA, ragged tail
+    dict(B=1, T=261, Hk=2, Hv=2, K=128, V=128, layout="TND", cu=[0, 1, 16, 33, 33, 96, 160, 261], h0=True),
+    dict(B=1, T=130, Hk=1, Hv=2, K=64, V=64, layout="NTD", cu=[0, 65, 130]),
+    dict(B=1, T=192, Hk=2, Hv=2, K=128, V=256, layout="BSND", v_first=True, h0=True),
+    dict(B=2, T=100, Hk=2, Hv=2, K=64, V=128, layout="BNSD"),
+    dict(B=1, T=160, Hk=2, Hv=2, K=128, V=128, layout="BSND", gate=dict(use_gate_in_kernel=True, bias=True)),
+    dict(B=1, T=160, Hk=2, Hv=2, K=128, V=128, layout="BSND",
+         gate=dict(use_gate_in_kernel=True, safe_gate=True, lower_bound=-5.0, bias=True), g_dtype=BF, beta_dtype=BF),
+    dict(B=1, T=1, Hk=1, Hv=1, K=128, V=128, layout="BSND"),
+    dict(B=1, T=128, Hk=1, Hv=1, K=128, V=128, layout="BSND", gate_scale=3.0),             # strong decay
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items() if k in ("T", "K", "V", "layout")))
+def test_chunk_kda_fwd(dev, case):
+    from fla_hip import ops
+    B, T, Hk, Hv, K, V, layout = (case[x] for x in ("B", "T", "Hk", "Hv", "K", "V", "layout"))
+    cu = case.get("cu")
+    gate = dict(case.get("gate", {}))
+    use_gate = gate.get("use_gate_in_kernel", False)
+    v_first = case.get("v_first", False)
+    q, k, v, g, beta = make_inputs(B, T, Hk, Hv, K, V, seed=T + K + V, raw_gate=use_gate,
+                                   gate_scale=case.get("gate_scale", 0.3), g_dtype=case.get("g_dtype", torch.float32),
+                                   beta_dtype=case.get("beta_dtype", torch.float32))
+    gen = torch.Generator().manual_seed(11)
+    A_log = torch.randn(Hv, generator=gen) * 0.3 - 1.5 if use_gate else None
+    dt_bias = torch.randn(Hv * K, generator=gen) * 0.3 if gate.pop("bias", False) else None
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, Hv, K, V, generator=gen) * 0.1 if case.get("h0") else None
+    scale = K ** -0.5
+
+    # oracle
+    okw = dict(A_log=A_log, dt_bias=dt_bias, use_gate_in_kernel=use_gate, safe_gate=gate.get("safe_gate", False),
+               lower_bound=gate.get("lower_bound", -5.0))
+    nat = kda.kda_gate(g, **okw)
+    gk_ref = kda.kda_gate_cumsum(g, 64, cu_seqlens=cu, **okw)
+    o_naive, f_naive = kda.naive_recurrent_kda(q, k, v, nat, beta, scale, initial_state=h0, output_final_state=True,
+                                               cu_seqlens=cu)
+    ref = kda.chunk_kda_fwd(q, k, v, gk_ref, beta, scale, 64, initial_state=h0, output_final_state=True, cu_seqlens=cu)
+
+    h0_dev = None
+    if h0 is not None:
+        h0_dev = (h0.transpose(-1, -2).contiguous() if v_first else h0).to(dev)
+    out = ops.chunk_kda_fwd(
+        to_layout(q, layout).to(dev), to_layout(k, layout).to(dev), to_layout(v, layout).to(dev),
+        to_layout(g, layout).to(dev), to_layout(beta, layout).to(dev), scale, 64, layout=layout, initial_state=h0_dev,
+        output_final_state=True, cu_seqlens=cu, A_log=None if A_log is None else A_log.to(dev),
+        dt_bias=None if dt_bias is None else dt_bias.to(dev), disable_recompute=True, state_v_first=v_first, **gate)
+    assert len(out) == 12
+    o, final, gk, Aqk, Akk, w, u, qg, kg, v_new, h, init_back = out
+    assert init_back is h0_dev
+    head = (lambda x: x[None]) if layout in ("TND", "NTD") else (lambda x: x)
+
+    assert_close(from_layout(o, layout), o_naive, TOL_BF16, "o vs recurrence")
+    fin = final.transpose(-1, -2) if v_first else final
+    assert final.dtype == torch.float32
+    assert_close(fin, f_naive, 4 * TOL_STATE, "final state vs recurrence")
+    assert_close(fin, ref["final_state"], TOL_BF16, "final state vs chunked")
+
+    assert gk.dtype == torch.float32
+    assert_close(head(gk), gk_ref, 2e-5 if g.dtype == torch.float32 else 1e-4, "gk")
+    assert_close(head(Aqk), ref["Aqk"], TOL_BF16, "Aqk")
+    assert_close(head(Akk), ref["Akk"], TOL_BF16, "Akk")
+    assert_close(head(w), ref["w"], TOL_BF16, "w")
+    assert_close(head(u), ref["u"], TOL_BF16, "u")
+    assert_close(head(qg), ref["qg"], TOL_BF16, "qg")
+    assert_close(head(kg), ref["kg"], TOL_BF16, "kg")
+    assert_close(head(v_new), ref["v_new"], TOL_BF16, "v_new")
+    hh = head(h).transpose(1, 2)                      # [B,NT,Hv,..] -> [B,Hv,NT,..]
+    hh = hh.transpose(-1, -2) if v_first else hh
+    assert_close(hh, ref["h"], TOL_BF16, "h")
+    # structure of the score matrices: upper triangles are exactly zero
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        blk = head(Akk)[b, :, s:e, : e - s].float().cpu()
+        assert float(torch.triu(blk, 1).abs().max()) == 0.0
+        assert float(torch.triu(head(Aqk)[b, :, s:e, : e - s].float().cpu(), 1).abs().max()) == 0.0
+
+
+def test_chunk_kda_fwd_output_policy(dev):
+    """Hidden outputs are None and do not change the visible ones."""
+    from fla_hip import ops
+    q, k, v, g, beta = make_inputs(1, 128, 2, 2, 128, 128, seed=3)
+    args = [to_layout(x, "BSND").to(dev) for x in (q, k, v, g, beta)]
+    full = ops.chunk_kda_fwd(*args, 0.1, 64, output_final_state=True, disable_recompute=True)
+    lean = ops.chunk_kda_fwd(*args, 0.1, 64)
+    assert [x is None for x in lean] == [False, True, False, False, False, True, True, True, True, True, True, True]
+    assert torch.equal(lean[0], full[0]) and torch.equal(lean[3], full[3]) and torch.equal(lean[4], full[4])
+    mid = ops.chunk_kda_fwd(*args, 0.1, 64, return_intermediate_states=True, use_gate_in_kernel=True,
+                            A_log=torch.zeros(2, device=dev))
+    assert mid[2] is None and mid[10] is not None and mid[5] is None
+
+
+def test_chunk_kda_fwd_errors(dev):
+    from fla_hip import ops
+    q, k, v, g, beta = make_inputs(1, 64, 2, 2, 128, 128, seed=3)
+    a = [to_layout(x, "BSND").to(dev) for x in (q, k, v, g, beta)]
+    with pytest.raises(RuntimeError, match="layout must be uppercase"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, layout="bsnd")
+    with pytest.raises(RuntimeError, match="chunk_size must be 64 or 128"):
+        ops.chunk_kda_fwd(*a, 0.1, 32)
+    with pytest.raises(RuntimeError, match="only chunk_size 64"):
+        ops.chunk_kda_fwd(*a, 0.1, 128)
+    with pytest.raises(RuntimeError, match="rank does not match"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, layout="TND")
+    with pytest.raises(RuntimeError, match="A_log must be float32"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, use_gate_in_kernel=True)
+    with pytest.raises(RuntimeError, match="cu_seqlens must be nondecreasing"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, cu_seqlens=[0, 70, 60, 64])
+    with pytest.raises(RuntimeError, match="canonical"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, cu_seqlens=[0, 64], chunk_indices=[0, 1])
+    with pytest.raises(RuntimeError, match="initial_state shape"):
+        ops.chunk_kda_fwd(*a, 0.1, 64, initial_state=torch.zeros(1, 2, 128, 64, device=dev))
+    with pytest.raises(RuntimeError, match="only bfloat16"):
+        ops.chunk_kda_fwd(*[t.half() if t.dtype == BF else t for t in a], 0.1, 64)
