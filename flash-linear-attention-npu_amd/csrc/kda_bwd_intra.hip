@@ -1,0 +1,298 @@
+// chunk_kda_bwd_intra: intra-chunk part of the KDA backward.
+//
+// For every chunk and head, with A = tril(dAqk), B = tril(dAkk) (64x64, fp32) and the chunk-local
+// cumulated gate g (log2 units):
+//     dq_i += sum_{j<=i} A_ij k_j 2^{g_i-g_j}
+//     dl_i  = sum_{j<=i} B_ij k_j 2^{g_i-g_j}
+//     du_j  = sum_{i>=j} (A_ij q_i + B_ij beta_i k_i) 2^{g_i-g_j}
+//     dk_i += beta_i dl_i + du_i ;  db_i += <dl_i, k_i> ;  dg_i += q_i dq'_i + k_i (beta_i dl_i - du_i)
+// Each 16-row tile is evaluated against an anchor gate c inside the tile (row 8, or the last valid
+// row), 2^{g_i-g_j} = 2^{g_i-c} 2^{c-g_j}, so both factors stay finite for non-increasing gates.
+// Golden: torch_custom/fla_npu/test/test_npu_chunk_kda_bwd_intra.py:7-91 (fp32 products, tolerance
+// 2e-4), operand order: _aclnn_ctypes.py:1534-1768.
+//
+// The golden's tolerance rules out bf16 operands, so the products run on the fp32 matrix pipe
+// (v_mfma_f32_16x16x4_f32).  One workgroup per (chunk, head); wave r owns row tile r: its "lower"
+// products contract over (r+1) tiles and its "upper" product over (4-r) tiles, five in total for
+// every wave.  Channels are processed in blocks of at most 128 so the fp32 gate tile fits in LDS.
+#include "gdn_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
+// D[16x16] += A[16x4] B[4x16]: lane l holds A[l%16][l/16], B[l/16][l%16], D[4*(l/16)+e][l%16]
+__device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+struct BwdIntraParams {
+    ChunkGeom geom;              // Hv = heads, K = head size
+    const bf16 *q, *k;
+    const float *gk, *dq, *dk, *dg;
+    float *dq_o, *dk_o, *dg_o;
+    int64_t sb, sh, st;          // strides of (batch, head, token) of the [..,K] tensors
+    View3 beta;
+    const float *db;
+    float *db_o;
+    const float *daqk, *dakk;    // [..,64]
+    int64_t m_sb, m_sh, m_st;
+};
+
+template <int KC>
+__global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pa = 68, pg = KC + 4, pk = KC + 8;
+    float *aqS = reinterpret_cast<float *>(smem);   // [64][pa] tril(dAqk)
+    float *akS = aqS + kChunk * pa;                 // [64][pa] tril(dAkk)
+    float *gS = akS + kChunk * pa;                  // [64][pg]
+    float *bS = gS + kChunk * pg;                   // [64]
+    bf16 *qS = reinterpret_cast<bf16 *>(bS + kChunk);
+    bf16 *kS = qS + kChunk * pk;
+
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x;
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int K = p.geom.K;
+
+    {   // masked score gradients
+        const int64_t mbase = b * p.m_sb + h * p.m_sh + (int64_t)start * p.m_st;
+        for (int idx = tid; idx < kChunk * 16; idx += kThreads) {
+            const int r = idx >> 4, c4 = (idx & 15) << 2;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, k4 = a;
+            if (r < len) {
+                a = *reinterpret_cast<const f32x4 *>(p.daqk + mbase + (int64_t)r * p.m_st + c4);
+                k4 = *reinterpret_cast<const f32x4 *>(p.dakk + mbase + (int64_t)r * p.m_st + c4);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (c4 + e > r) a[e] = k4[e] = 0.f;
+            *reinterpret_cast<f32x4 *>(aqS + r * pa + c4) = a;
+            *reinterpret_cast<f32x4 *>(akS + r * pa + c4) = k4;
+        }
+        if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, h, start + tid) : 0.f;
+    }
+
+    const int r0 = 16 * wave_id();
+    const int row_end = min(r0 + 16, len);
+    const int anchor = min(r0 + 8, row_end - 1);
+    const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
+    f32x4 dbacc = {0.f, 0.f, 0.f, 0.f};
+
+    for (int ch0 = 0; ch0 < K; ch0 += KC) {
+        __syncthreads();
+        for (int idx = tid; idx < kChunk * (KC / 8); idx += kThreads) {
+            const int r = idx / (KC / 8), c8 = (idx % (KC / 8)) * 8;
+            u32x4 qv = {0u, 0u, 0u, 0u}, kv = qv;
+            if (r < len) {
+                qv = *reinterpret_cast<const u32x4 *>(p.q + base + (int64_t)r * p.st + ch0 + c8);
+                kv = *reinterpret_cast<const u32x4 *>(p.k + base + (int64_t)r * p.st + ch0 + c8);
+            }
+            *reinterpret_cast<u32x4 *>(qS + r * pk + c8) = qv;
+            *reinterpret_cast<u32x4 *>(kS + r * pk + c8) = kv;
+        }
+        for (int idx = tid; idx < kChunk * (KC / 4); idx += kThreads) {   // padded rows repeat the last gate row
+            const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
+            const int rr = min(r, len - 1);
+            *reinterpret_cast<f32x4 *>(gS + r * pg + c4) =
+                *reinterpret_cast<const f32x4 *>(p.gk + base + (int64_t)rr * p.st + ch0 + c4);
+        }
+        __syncthreads();
+        if (r0 >= len) continue;   // wave-uniform: this row tile holds no token
+
+        const int nsteps_lo = (row_end + 3) >> 2;   // contraction over tokens j < row_end, four at a time
+        for (int nt = 0; nt < KC / 16; ++nt) {
+            const int ch = 16 * nt + li;
+            const float ca = gS[anchor * pg + ch];
+            f32x4 D1 = {0.f, 0.f, 0.f, 0.f}, D2 = D1, D3 = D1;
+            for (int js = 0; js < nsteps_lo; ++js) {
+                const int j = 4 * js + lg;
+                const float bval = (float)kS[j * pk + ch] * ex2(ca - gS[j * pg + ch]);
+                D1 = mfma_f32(aqS[(r0 + li) * pa + j], bval, D1);
+                D2 = mfma_f32(akS[(r0 + li) * pa + j], bval, D2);
+            }
+            for (int is = r0 >> 2; is < 16; ++is) {
+                const int i = 4 * is + lg;
+                const float fw = ex2(gS[i * pg + ch] - ca);
+                const float kk = (float)kS[i * pk + ch];
+                D3 = mfma_f32(aqS[i * pa + r0 + li], (float)qS[i * pk + ch] * fw, D3);
+                D3 = mfma_f32(akS[i * pa + r0 + li], kk * bS[i] * fw, D3);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = r0 + 4 * lg + e;
+                if (i < len) {
+                    const float gi = gS[i * pg + ch];
+                    const float up = ex2(gi - ca), down = ex2(ca - gi);
+                    const float dqd = D1[e] * up, dl = D2[e] * up, du = D3[e] * down;
+                    const float qi = (float)qS[i * pk + ch], ki = (float)kS[i * pk + ch];
+                    const float bdl = bS[i] * dl;
+                    const int64_t off = base + (int64_t)i * p.st + ch0 + ch;
+                    p.dq_o[off] = p.dq[off] + dqd;
+                    p.dk_o[off] = p.dk[off] + bdl + du;
+                    p.dg_o[off] = p.dg[off] + qi * dqd + ki * (bdl - du);
+                    dbacc[e] += dl * ki;
+                }
+            }
+        }
+    }
+    if (r0 < len) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float s = group_sum<16>(dbacc[e]);
+            const int i = r0 + 4 * lg + e;
+            if (li == 0 && i < len) {
+                const int64_t off = b * p.beta.sb + h * p.beta.sh + (int64_t)(start + i) * p.beta.st;
+                p.db_o[off] = p.db[off] + s;
+            }
+        }
+    }
+}
+
+template <int KC>
+int launch_bwd_intra(const BwdIntraParams &p, hipStream_t stream) {
+    const size_t smem = (size_t)kChunk * (2 * 68 + (KC + 4) + 1) * 4 + (size_t)2 * kChunk * (KC + 8) * 2;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_bwd_intra_kernel<KC>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("kda_bwd_intra", stream, (kda_bwd_intra_kernel<KC>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem,
+               stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
+                   const fla_tensor *daqk, const fla_tensor *dakk, const fla_tensor *dq, const fla_tensor *dk,
+                   const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu, const fla_int_array *ci,
+                   int64_t chunk_size, bool safe_gate, const char *layout, const fla_tensor *dq_o, const fla_tensor *dk_o,
+                   const fla_tensor *db_o, const fla_tensor *dg_o, void *ws, uint64_t ws_size, hipStream_t stream,
+                   uint64_t *query) {
+    const char *op = "chunk_kda_bwd_intra";
+    FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
+    int ib, ih, it;
+    if (!strcmp(layout, "BSND")) { ib = 0; it = 1; ih = 2; }
+    else if (!strcmp(layout, "BNSD")) { ib = 0; ih = 1; it = 2; }
+    else if (!strcmp(layout, "TND")) { ib = -1; it = 0; ih = 1; }
+    else return fail(FLA_ERR_UNSUPPORTED, "%s: supports dense BSND/BNSD or varlen TND.", op);
+    FLA_REQUIRE(safe_gate, FLA_ERR_UNSUPPORTED, "%s: safe_gate=False is reserved but not supported in v1.", op);
+    FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: chunk_size must be 64.", op);
+    const int rank = ib < 0 ? 3 : 4;
+    int rc;
+    if ((rc = check_tensor(q, op, "q", rank, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_tensor(k, op, "k", rank, dt_bit(FLA_BF16)))) return rc;
+    const fla_tensor *f32s[] = {gk, dq, dk, dg, dq_o, dk_o, dg_o};
+    const char *f32n[] = {"gk", "dq", "dk", "dg", "dq_out", "dk_out", "dg_out"};
+    for (int i = 0; i < 7; ++i) {
+        if ((rc = check_tensor(f32s[i], op, f32n[i], rank, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE(same_shape(f32s[i], q), FLA_ERR_SHAPE, "%s: %s must have the same shape as q.", op, f32n[i]);
+        FLA_REQUIRE(is_contiguous(f32s[i]), FLA_ERR_SHAPE, "%s: %s must be contiguous; implicit copies are disabled.", op,
+                    f32n[i]);
+    }
+    FLA_REQUIRE(same_shape(k, q), FLA_ERR_SHAPE, "%s: k must have the same shape as q.", op);
+    FLA_REQUIRE(is_contiguous(q) && is_contiguous(k), FLA_ERR_SHAPE, "%s: q and k must be contiguous.", op);
+    const int64_t B = ib < 0 ? 1 : q->shape[ib], H = q->shape[ih], T = q->shape[it], K = q->shape[rank - 1];
+    FLA_REQUIRE(B > 0 && H > 0 && T > 0, FLA_ERR_SHAPE, "%s: B/H/T must be positive.", op);
+    FLA_REQUIRE(K == 64 || K == 128 || K == 256, FLA_ERR_UNSUPPORTED, "%s: K must be 64, 128 or 256.", op);
+    FLA_REQUIRE(B < 65536 && H < 65536 && T < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents too large.", op);
+    if ((rc = check_tensor(beta, op, "beta", rank - 1, dt_bit(FLA_BF16) | dt_bit(FLA_F32)))) return rc;
+    const fla_tensor *sc[] = {beta, db, db_o};
+    const char *scn[] = {"beta", "db", "db_out"};
+    for (int i = 0; i < 3; ++i) {
+        if (i && (rc = check_tensor(sc[i], op, scn[i], rank - 1, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE((ib < 0 || sc[i]->shape[ib] == B) && sc[i]->shape[ih] == H && sc[i]->shape[it] == T && is_contiguous(sc[i]),
+                    FLA_ERR_SHAPE, "%s: beta/db shape must match the selected layout.", op);
+    }
+    const fla_tensor *mats[] = {daqk, dakk};
+    for (int i = 0; i < 2; ++i) {
+        if ((rc = check_tensor(mats[i], op, i ? "dAkk" : "dAqk", rank, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE((ib < 0 || mats[i]->shape[ib] == B) && mats[i]->shape[ih] == H && mats[i]->shape[it] == T &&
+                        mats[i]->shape[rank - 1] == kChunk && is_contiguous(mats[i]),
+                    FLA_ERR_SHAPE, "%s: dAqk/dAkk shape must match the selected layout.", op);
+    }
+    const fla_tensor *al[] = {q, k, gk, dq, dk, dg, dq_o, dk_o, dg_o, daqk, dakk};
+    for (const fla_tensor *t : al)
+        FLA_REQUIRE(reinterpret_cast<uintptr_t>(t->data) % 16 == 0, FLA_ERR_SHAPE, "%s: tensors must be 16-byte aligned.", op);
+    const bool varlen = cu && cu->data && cu->size;
+    FLA_REQUIRE(!(varlen && !strcmp(layout, "BNSD")), FLA_ERR_UNSUPPORTED, "%s: varlen supports TND or BSND, not BNSD.", op);
+    FLA_REQUIRE(varlen || ib >= 0, FLA_ERR_SHAPE, "%s: TND requires cu_seqlens.", op);
+    FLA_REQUIRE(varlen || !(ci && ci->data && ci->size), FLA_ERR_SHAPE, "%s: chunk_indices requires cu_seqlens.", op);
+
+    ChunkGeom geom{};
+    geom.B = (int)B;
+    geom.T = (int)T;
+    geom.Hk = geom.Hv = (int)H;
+    geom.K = geom.V = (int)K;
+    geom.NT = (int)((T + kChunk - 1) / kChunk);
+    geom.N = (int)B;
+    Varlen vl;
+    if ((rc = build_varlen(vl, op, cu, ci, kChunk, T))) return rc;
+    FLA_REQUIRE(!vl.enabled || B == 1, FLA_ERR_SHAPE, "%s: varlen BSND compatibility requires B=1.", op);
+    if (vl.enabled) {
+        geom.NT = vl.NT;
+        geom.N = vl.N;
+    }
+    if (query) {
+        *query = vl.bytes();
+        return FLA_OK;
+    }
+    FLA_REQUIRE(vl.bytes() == 0 || (ws && ws_size >= vl.bytes()), FLA_ERR_WORKSPACE, "%s: workspace of %zu bytes required.",
+                op, vl.bytes());
+    if ((rc = upload_varlen(vl, ws, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    if (geom.NT == 0) return FLA_OK;
+
+    BwdIntraParams p{};
+    p.geom = geom;
+    p.q = static_cast<const bf16 *>(q->data);
+    p.k = static_cast<const bf16 *>(k->data);
+    p.gk = static_cast<const float *>(gk->data);
+    p.dq = static_cast<const float *>(dq->data);
+    p.dk = static_cast<const float *>(dk->data);
+    p.dg = static_cast<const float *>(dg->data);
+    p.dq_o = static_cast<float *>(dq_o->data);
+    p.dk_o = static_cast<float *>(dk_o->data);
+    p.dg_o = static_cast<float *>(dg_o->data);
+    p.sb = ib < 0 ? 0 : q->stride[ib];
+    p.sh = q->stride[ih];
+    p.st = q->stride[it];
+    p.beta = View3{beta->data, ib < 0 ? 0 : beta->stride[ib], beta->stride[ih], beta->stride[it], beta->dtype == FLA_BF16 ? 1 : 0};
+    p.db = static_cast<const float *>(db->data);
+    p.db_o = static_cast<float *>(db_o->data);
+    p.daqk = static_cast<const float *>(daqk->data);
+    p.dakk = static_cast<const float *>(dakk->data);
+    p.m_sb = ib < 0 ? 0 : daqk->stride[ib];
+    p.m_sh = daqk->stride[ih];
+    p.m_st = daqk->stride[it];
+    return K == 64 ? launch_bwd_intra<64>(p, stream) : launch_bwd_intra<128>(p, stream);
+}
+
+}  // namespace
+}  // namespace fla
+
+extern "C" int fla_chunk_kda_bwd_intra_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
+    const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
+    const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, uint64_t *workspace_size) {
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_intra: workspace_size must not be null.");
+    return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+                               layout, dq_out, dk_out, db_out, dg_out, nullptr, 0, nullptr, workspace_size);
+}
+
+extern "C" int fla_chunk_kda_bwd_intra(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
+    const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
+    const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+                               layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size,
+                               static_cast<hipStream_t>(stream), nullptr);
+}

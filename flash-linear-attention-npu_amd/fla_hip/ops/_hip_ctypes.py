@@ -39,6 +39,7 @@ OP_ARGTYPES = {
     "kda_gate_cumsum": [_T, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool, ctypes.c_double, _T],
     "chunk_kda_fwd": [_T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_char_p, ctypes.c_double, ctypes.c_int64,
                       ctypes.c_bool, ctypes.c_double, ctypes.c_bool, ctypes.c_bool] + [_T] * 11,
+    "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
 }
@@ -590,6 +591,93 @@ def npu_chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", 
         outputs,
     )
     return (*outputs, initial_state)
+
+
+def npu_chunk_kda_bwd_intra(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_seqlens=None, chunk_indices=None,
+                            chunk_size=64, safe_gate=True, layout="BSND"):
+    """Intra-chunk KDA backward (_aclnn_ctypes.py:1534-1768).  Returns new ``(dq, dk, db, dg)`` = the inputs
+    plus the intra-chunk terms; q/k bf16, beta bf16 or fp32, everything else fp32, all contiguous."""
+    import torch
+
+    op = "npu_chunk_kda_bwd_intra"
+    tensors = {"q": q, "k": k, "gk": gk, "beta": beta, "dAqk": dAqk, "dAkk": dAkk, "dq": dq, "dk": dk, "db": db, "dg": dg}
+    layout = str(layout)
+    if layout not in {"BSND", "BNSD", "TND"}:
+        raise RuntimeError(f"{op}: supports dense BSND/BNSD or varlen TND.")
+    if not bool(safe_gate):
+        raise RuntimeError(f"{op}: safe_gate=False is reserved but not supported in v1.")
+    chunk_size = int(chunk_size)
+    if chunk_size != 64:
+        raise RuntimeError(f"{op}: chunk_size must be 64.")
+    for name, tensor in tensors.items():
+        if name == "beta":
+            if tensor.dtype not in {torch.bfloat16, torch.float32}:
+                raise RuntimeError(f"{op}: beta must be torch.bfloat16 or torch.float32.")
+        else:
+            want = torch.bfloat16 if name in ("q", "k") else torch.float32
+            if tensor.dtype != want:
+                raise RuntimeError(f"{op}: {name} must be {want}.")
+        if tensor.device != q.device:
+            raise RuntimeError(f"{op}: {name} must be on the same device as q.")
+        if not tensor.is_contiguous():
+            raise RuntimeError(f"{op}: {name} must be contiguous; implicit copies are disabled.")
+    if chunk_indices is not None and cu_seqlens is None:
+        raise RuntimeError(f"{op}: chunk_indices requires cu_seqlens.")
+    varlen = cu_seqlens is not None
+    if varlen and layout == "BNSD":
+        raise RuntimeError(f"{op}: varlen supports TND or BSND, not BNSD.")
+    if not varlen and layout == "TND":
+        raise RuntimeError(f"{op}: TND requires cu_seqlens.")
+    qs = _shape(q)
+    if len(qs) != (3 if layout == "TND" else 4):
+        raise RuntimeError(f"{op}: q rank does not match layout.")
+    if layout == "TND":
+        (T, H, K), B = qs, 1
+        scalar_shape, matrix_shape = (T, H), (T, H, chunk_size)
+    elif layout == "BSND":
+        B, T, H, K = qs
+        scalar_shape, matrix_shape = (B, T, H), (B, T, H, chunk_size)
+    else:
+        B, H, T, K = qs
+        scalar_shape, matrix_shape = (B, H, T), (B, H, T, chunk_size)
+    if B <= 0 or H <= 0 or T <= 0:
+        raise RuntimeError(f"{op}: B/H/T must be positive.")
+    if K not in {64, 128, 256}:
+        raise RuntimeError(f"{op}: K must be 64, 128 or 256.")
+    if varlen and layout == "BSND" and B != 1:
+        raise RuntimeError(f"{op}: varlen BSND compatibility requires B=1.")
+    for name in ("k", "gk", "dq", "dk", "dg"):
+        if _shape(tensors[name]) != qs:
+            raise RuntimeError(f"{op}: {name} must have the same shape as q.")
+    if _shape(beta) != scalar_shape or _shape(db) != scalar_shape:
+        raise RuntimeError(f"{op}: beta/db shape must match the selected layout.")
+    if _shape(dAqk) != matrix_shape or _shape(dAkk) != matrix_shape:
+        raise RuntimeError(f"{op}: dAqk/dAkk shape must match the selected layout.")
+    cu = indices = None
+    if varlen:
+        cu = _as_int_tuple(cu_seqlens)
+        if len(cu) < 2 or cu[0] != 0 or cu[-1] != T:
+            raise RuntimeError(f"{op}: cu_seqlens must start at 0 and end at T.")
+        if any(a > b for a, b in zip(cu, cu[1:])):
+            raise RuntimeError(f"{op}: cu_seqlens must be nondecreasing.")
+        canonical = _build_chunk_indices(cu, chunk_size)
+        if not canonical:
+            raise RuntimeError(f"{op}: varlen input has no non-empty sequence.")
+        indices = canonical if chunk_indices is None else _as_int_tuple(chunk_indices)
+        if indices != canonical:
+            raise RuntimeError(f"{op}: chunk_indices must use canonical sequence-major order.")
+    outputs = (_empty_like(dq), _empty_like(dk), _empty_like(db), _empty_like(dg))
+    ins = (q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg)
+    return _call_op(
+        "chunk_kda_bwd_intra", OP_ARGTYPES["chunk_kda_bwd_intra"],
+        lambda ctx: [
+            *[ctx.tensor(t, n) for t, n in zip(ins, tensors)],
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_int64(chunk_size), ctypes.c_bool(True),
+            ctypes.c_char_p(layout.encode("utf-8")),
+            *[ctx.tensor(t, n) for t, n in zip(outputs, ("dq_out", "dk_out", "db_out", "dg_out"))],
+        ],
+        outputs,
+    )
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

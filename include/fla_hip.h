@@ -312,6 +312,31 @@ int fla_chunk_kda_fwd(
     const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
     void *workspace, uint64_t workspace_size, void *stream);
 
+/* ------------------------------------------------------------------------
+ * chunk_kda_bwd_intra - replaces aclnnChunkKdaBwdIntra
+ * (_aclnn_ctypes.py:1534-1768; golden test_npu_chunk_kda_bwd_intra.py:7-91).
+ * layout "BSND", "BNSD" (dense) or "TND" (needs cu_seqlens).  q,k bf16 [..,K];
+ * gk (chunk-local cumulated gate, log2 units), dq, dk, dg f32 like q; beta
+ * bf16/f32 and db f32 [..]; dAqk, dAkk f32 [..,64].  All contiguous.
+ * Outputs dq_out, dk_out, dg_out like dq and db_out like db hold the inputs
+ * plus the intra-chunk terms.  K in {64,128,256}; chunk_size 64; safe_gate
+ * must be true.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_kda_bwd_intra_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
+    const fla_tensor *dAqk, const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate, const char *layout,
+    const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_intra(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
+    const fla_tensor *dAqk, const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate, const char *layout,
+    const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -159,3 +159,86 @@ def test_bwd_dhu_errors(dev):
         ops.chunk_gated_delta_rule_bwd_dhu(*a, 0.1, 64, g=torch.zeros(1, 2, 64, device=dev))
     with pytest.raises(RuntimeError, match="chunk_size"):
         ops.chunk_gated_delta_rule_bwd_dhu(*a, 0.1, 32, g=gate.to(dev))
+
+
+# ---------------------------------------------------------------------------------------------
+# chunk_kda_bwd_intra (fp32 products; the reference's own tolerance is 2e-4)
+# ---------------------------------------------------------------------------------------------
+def intra_inputs(B, T, H, K, seed, beta_dtype, cu=None, decay=0.05):
+    gen = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=gen)
+    q = (rn(B, H, T, K) * 0.1).to(BF)
+    k = (rn(B, H, T, K) * 0.1).to(BF)
+    inc = -torch.rand(B, H, T, K, generator=gen) * decay
+    gk = torch.zeros_like(inc)
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        gk[b, :, s:e] = inc[b, :, s:e].cumsum(dim=1)
+    beta = torch.rand(B, H, T, generator=gen).to(beta_dtype)
+    dAqk, dAkk = rn(B, H, T, 64) * 0.1, rn(B, H, T, 64) * 0.1
+    dq, dk, dg = rn(B, H, T, K) * 0.01, rn(B, H, T, K) * 0.01, rn(B, H, T, K) * 0.01
+    db = rn(B, H, T) * 0.01
+    return q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg
+
+
+def _lay(x, layout):   # head-major [B,H,T,..] -> layout
+    if layout == "BNSD":
+        return x.contiguous()
+    if layout == "BSND":
+        return x.transpose(1, 2).contiguous()
+    return x[0].transpose(0, 1).contiguous()
+
+
+def _unlay(x, layout):
+    if layout == "BNSD":
+        return x
+    if layout == "BSND":
+        return x.transpose(1, 2)
+    return x.transpose(0, 1)[None]
+
+
+INTRA_CASES = [(K, H, T, "BNSD", None, BF) for K in (64, 128, 256) for H, T in ((1, 1), (2, 15), (3, 16), (2, 17), (1, 63),
+                                                                               (2, 64), (3, 65), (2, 129))]
+INTRA_CASES += [
+    (128, 2, 65, "BSND", None, BF),
+    (128, 3, 63, "BNSD", None, torch.float32),
+    (128, 3, 129, "TND", [0, 17, 64, 129], BF),
+    (128, 2, 261, "TND", [0, 1, 16, 33, 33, 96, 160, 261], torch.float32),
+    (128, 2, 130, "BSND", [0, 65, 130], BF),
+    (128, 2, 128, "BNSD", None, BF, 2.0),     # strong decay: 2 bits per token and channel
+]
+
+
+@pytest.mark.parametrize("case", INTRA_CASES, ids=lambda c: f"K{c[0]}-H{c[1]}-T{c[2]}-{c[3]}")
+def test_chunk_kda_bwd_intra(dev, case):
+    from fla_hip import ops
+    K, H, T, layout, cu, beta_dtype = case[:6]
+    decay = case[6] if len(case) > 6 else 0.05
+    B = 1 if layout == "TND" or cu is not None else 2
+    x = intra_inputs(B, T, H, K, seed=K + T, beta_dtype=beta_dtype, cu=cu, decay=decay)
+    ref = kda.chunk_kda_bwd_intra(*x, chunk=64, cu_seqlens=cu)                       # fp64
+    got = ops.chunk_kda_bwd_intra(*[_lay(t, layout).to(dev) for t in x], cu_seqlens=cu, chunk_size=64, safe_gate=True,
+                                  layout=layout)
+    for name, a, e in zip(("dq", "dk", "db", "dg"), got, ref):
+        assert a.dtype == torch.float32
+        assert_close(_unlay(a, layout), e.float(), 2e-4, name)
+
+
+def test_chunk_kda_bwd_intra_errors(dev):
+    from fla_hip import ops
+    x = [t.to(dev) for t in intra_inputs(1, 64, 2, 128, seed=1, beta_dtype=BF)]
+    with pytest.raises(RuntimeError, match="safe_gate=False"):
+        ops.chunk_kda_bwd_intra(*x, safe_gate=False, layout="BNSD")
+    with pytest.raises(RuntimeError, match="chunk_size must be 64"):
+        ops.chunk_kda_bwd_intra(*x, chunk_size=128, layout="BNSD")
+    with pytest.raises(RuntimeError, match="TND requires cu_seqlens"):
+        ops.chunk_kda_bwd_intra(*[t[0] for t in x], layout="TND")
+    with pytest.raises(RuntimeError, match="not BNSD"):
+        ops.chunk_kda_bwd_intra(*x, cu_seqlens=[0, 64], layout="BNSD")
+    bad = list(x)
+    bad[4] = bad[4].to(BF)
+    with pytest.raises(RuntimeError, match="dAqk must be"):
+        ops.chunk_kda_bwd_intra(*bad, layout="BNSD")
+    bad = list(x)
+    bad[8] = torch.zeros(1, 2, 63, device=dev)
+    with pytest.raises(RuntimeError, match="beta/db shape"):
+        ops.chunk_kda_bwd_intra(*bad, layout="BNSD")
