@@ -6,7 +6,7 @@ bf16 in / fp32 accumulation and state, B=4, T=8192, H=32, K=V=128, chunk 64, fp3
 state, final state on.  One "step" is one pass of the whole chunk forward over that batch
 with inputs resident in HBM.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode|conv1d]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode|conv1d|kda]
 
 `roofline` describes the dominant kernel of the step: algorithmic FLOPs (or bytes) per launch
 divided by its average duration, measured with HIP events recorded on the launch stream by the
@@ -271,6 +271,102 @@ def bench_conv1d(args, torch, dev):
     }
 
 
+def bench_kda(args, torch, dev):
+    """KDA chunk forward and the two KDA backward kernels at B=2 T=8192 H=32 K=V=128.  The step is the
+    forward (gate activation + cumsum, intra-chunk kernel, state scan); the backward kernels are timed
+    in the same run and reported under `other_kernels_ms`."""
+    import fla_hip
+    from fla_hip import ops
+    from oracle import kda as okda
+
+    lib = fla_hip.load_library()
+    B, T, H, K, V, C = 2, 8192, 32, 128, 128, 64
+    F = torch.nn.functional
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
+    q = F.normalize(rn(B, T, H, K), dim=-1).bfloat16()
+    k = F.normalize(rn(B, T, H, K), dim=-1).bfloat16()
+    v = rn(B, T, H, V).bfloat16()
+    g = F.logsigmoid(rn(B, T, H, K))
+    beta = torch.sigmoid(rn(B, T, H))
+    h0 = rn(B, H, K, V) * 0.01
+    scale = K ** -0.5
+
+    def step():
+        return ops.chunk_kda_fwd(q, k, v, g, beta, scale, C, layout="BSND", initial_state=h0, output_final_state=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+
+    # backward kernels on the forward's own intermediates
+    full = ops.chunk_kda_fwd(q, k, v, g, beta, scale, C, layout="BSND", initial_state=h0, output_final_state=True,
+                             disable_recompute=True)
+    gk, w, qg, kg = full[2], full[5], full[7], full[8]
+    d_o = rn(B, H, T, V).bfloat16()
+    dv = rn(B, H, T, V).bfloat16()
+    dht = rn(B, H, K, V) * 0.01
+    qh, kh = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+    bh = beta.transpose(1, 2).contiguous()
+    dA1, dA2 = rn(B, H, T, C) * 0.1, rn(B, H, T, C) * 0.1
+    z4 = torch.zeros(B, H, T, K, device=dev)
+    z3 = torch.zeros(B, H, T, device=dev)
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+        ops.chunk_gated_delta_rule_bwd_dhu(qg, kg, w, d_o, dv, scale, C, gK=gk, h0=h0, dht=dht, use_exp2=True,
+                                           dh0_per_sequence=True)
+        ops.chunk_kda_bwd_intra(qh, kh, gk, bh, dA1, dA2, z4, z4, z3, z4, layout="BNSD")
+        ops.kda_gate_cumsum(gk, C)
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    kern = {name: ms / n for name, (n, ms) in profile_report(lib).items()}
+    th = B * T * H
+    flops = {"kda_intra": 2 * (2 * C * K + C * K + C * V + C * C) * th,          # kk, qk, w, u, inverse
+             "kda_scan": 2 * (3 * K * V + C * V) * th,                           # w.S, qg.S, kg^T.v_new, Aqk.v_new
+             "bwd_dhu": 2 * (3 * K * V) * th}
+    dominant = max(("kda_intra", "kda_scan"), key=lambda n: kern.get(n, 0.0))
+    ach = flops[dominant] / (kern[dominant] * 1e-3) / 1e12
+    step_tflops = (flops["kda_intra"] + flops["kda_scan"]) / (ms_per_step * 1e-3) / 1e12
+    cpu = None
+    if not args.no_cpu:
+        import torch as _t
+        cores = os.cpu_count() or 1
+        _t.set_num_threads(cores)
+        Ts = min(args.cpu_tokens, 2048)
+        c = lambda x: x[:1, :Ts].transpose(1, 2).contiguous().cpu()
+        cq, ck, cv, cg, cb = c(q), c(k), c(v), c(g), beta[:1, :Ts].transpose(1, 2).contiguous().cpu()
+        t1 = time.perf_counter()
+        reps = 0
+        while reps == 0 or time.perf_counter() - t1 < args.cpu_seconds:
+            cgk = okda.kda_gate_cumsum(cg, C)
+            okda.chunk_kda_fwd(cq, ck, cv, cgk, cb, scale, C, initial_state=h0[:1].cpu(), output_final_state=True)
+            reps += 1
+        cdt = time.perf_counter() - t1
+        cpu = {"value": round(Ts * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x (B=1 T={Ts} H={H} K=V={K}) chunked fp32 torch oracle, {cdt:.1f} s"}
+    assert bool(torch.isfinite(out[0].float()).all()) and bool(torch.isfinite(out[1]).all())
+    return {
+        "metric": "kda_chunk_fwd_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "KDA chunk forward B=2 T=8192 H=32 K=V=128 chunk=64 BSND, fp32 initial+final state"},
+        "step_tflops": round(step_tflops, 2),
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "avg_kernel_ms": round(kern[dominant], 4)},
+        "other_kernels_ms": {n: round(t, 4) for n, t in kern.items()},
+        "cpu_baseline": cpu,
+    }
+
+
 def bench_copy(args, torch, dev):
     """Calibration only (not a product kernel): a plain device-to-device copy of known size, used to
     scale the FETCH_SIZE / WRITE_SIZE counters and as the practical bandwidth ceiling of the box."""
@@ -299,7 +395,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d", "copy"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d", "kda", "copy"])
     ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -316,7 +412,7 @@ def main():
         print("bench.py: no GPU visible.", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d, "copy": bench_copy}[args.workload]
+    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d, "kda": bench_kda, "copy": bench_copy}[args.workload]
     print(json.dumps(fn(args, torch, dev)))
 
 
