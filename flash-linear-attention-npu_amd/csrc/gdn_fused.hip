@@ -622,6 +622,452 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
     }
 }
 
+// =============================================================================================
+// Pipelined form for 64-column slabs: 512 threads, two groups of four waves that share the CU.
+//   prep group  (waves 0-3)  chunk i  : scores (phase A), WY solve (phase B), tile prefetch
+//   state group (waves 4-7)  chunk i-1: v_new, state update, output (phase C), gate tables
+// Each SIMD holds one wave of each group, so the chunk-parallel work of the next chunk runs under
+// the serial state update of the current one.  Two workgroup barriers per chunk:
+//   before `mid`  prep: A(i) -> aS, dS, pS[i&1]        state: C1 + state update of chunk i-1
+//                                                             (reads wS, uS, q/k/tables of i-1)
+//   after  `mid`  prep: B(i) -> wS, uS; tiles of i+1   state: o += P v_new (pS[(i-1)&1]), o tile;
+//                       -> buffer (i+1)&1                       tables of chunk i+1
+// Every buffer written after `mid` was last read before it (and conversely), which is what makes
+// two barriers enough.
+// =============================================================================================
+template <int K> struct PipeSmem {
+    static constexpr int pq = K + 8, pk = KTile<K>::pitch, pv = 64 + 8, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
+                         po = 64 + 8, pd = 24;
+    static constexpr size_t q_bytes = (size_t)kChunk * pq * 2, k_bytes = (size_t)kChunk * pk * 2,
+                            v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (6 * kChunk + 16) * 4;
+    static constexpr size_t buf_bytes = q_bytes + k_bytes + v_bytes + tab_bytes;
+    static constexpr size_t a_off = 2 * buf_bytes;
+    static constexpr size_t w_off = a_off + (size_t)kChunk * pa * 2;
+    static constexpr size_t p_off = w_off + (size_t)kChunk * pw * 2;          // two P tiles
+    static constexpr size_t o_off = p_off + 2 * (size_t)kChunk * pp * 2;
+    static constexpr size_t d_off = o_off + (size_t)kChunk * po * 2;
+    static constexpr size_t u_off = d_off + (size_t)kChunk * pd * 2;          // u as register images, fp32
+    static constexpr size_t bytes = u_off + (size_t)kChunk * 64 * 4;
+};
+template <int K>
+__device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int buf) {
+    typedef PipeSmem<K> L;
+    unsigned char *b = smem + buf * L::buf_bytes;
+    Tiles t;
+    t.q = reinterpret_cast<bf16 *>(b);
+    t.k = reinterpret_cast<bf16 *>(b + L::q_bytes);
+    t.v = reinterpret_cast<bf16 *>(b + L::q_bytes + L::k_bytes);
+    t.G = reinterpret_cast<float *>(b + L::q_bytes + L::k_bytes + L::v_bytes);
+    t.EGS = t.G + kChunk;
+    t.B = t.EGS + kChunk;
+    t.BEG = t.B + kChunk;
+    t.ROWF = t.BEG + kChunk;
+    t.COLF = t.ROWF + kChunk;
+    t.BLKF = t.COLF + kChunk;
+    return t;
+}
+
+template <int K>
+__global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
+    typedef PipeSmem<K> L;
+    constexpr int VS = 64, pq = L::pq, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, po = L::po, pd = L::pd;
+    constexpr int KT = K / 16, KS = K / 32;
+    constexpr int GT = 256;                              // threads of one group
+    constexpr int QCH = kChunk * (K / 8) / GT, VCH = kChunk * (VS / 8) / GT;
+    constexpr int QROWS = GT / (K / 8), VROWS = GT / (VS / 8);
+    constexpr int NTW = K / 64, NT = NTW + 1;
+    extern __shared__ __align__(16) unsigned char smem[];
+    bf16 *aS = reinterpret_cast<bf16 *>(smem + L::a_off);
+    bf16 *wS = reinterpret_cast<bf16 *>(smem + L::w_off);
+    bf16 *pS0 = reinterpret_cast<bf16 *>(smem + L::p_off);
+    bf16 *oS = reinterpret_cast<bf16 *>(smem + L::o_off);
+    bf16 *dS = reinterpret_cast<bf16 *>(smem + L::d_off);
+    float *uS = reinterpret_cast<float *>(smem + L::u_off);
+
+    const int lin = blockIdx.x;
+    int slab, hv, n;
+    if (p.remap) {
+        const int pair = (lin >> 4) * 8 + (lin & 7);
+        slab = (lin >> 3) & 1;
+        hv = pair % p.geom.Hv;
+        n = pair / p.geom.Hv;
+    } else {
+        slab = lin % p.slabs;
+        hv = (lin / p.slabs) % p.geom.Hv;
+        n = lin / (p.slabs * p.geom.Hv);
+    }
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int wave = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+
+    if (wave < 4) {
+        // ================================ prep group ==============================================
+        const int wv = wave, tid = threadIdx.x;
+        const int rq = tid / (K / 8), cq = (tid % (K / 8)) * 8;
+        const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
+        const char *qbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
+        const char *kbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
+        const char *vbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
+        unsigned qoff[QCH], koff[QCH], voff[VCH];
+#pragma unroll
+        for (int m = 0; m < QCH; ++m) {
+            qoff[m] = (unsigned)(((rq + m * QROWS) * p.q.st + cq) * 2);
+            koff[m] = (unsigned)(((rq + m * QROWS) * p.k.st + cq) * 2);
+        }
+#pragma unroll
+        for (int m = 0; m < VCH; ++m) voff[m] = (unsigned)(((rv + m * VROWS) * p.v.st + cv) * 2);
+        u32x4 pre_q[QCH], pre_k[QCH], pre_v[VCH];
+        // Rows past the end of the sequence must read as zero.  Buffer loads do that without a branch or
+        // an exec mask: the resource of a chunk covers exactly its valid rows, anything beyond returns 0.
+        auto prefetch = [&](int c) {
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            const __amdgpu_buffer_rsrc_t rq_ = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char *>(qbase + (int64_t)c * kChunk * p.q.st * 2), 0, (int)((len - 1) * p.q.st * 2 + K * 2), 0x00020000);
+            const __amdgpu_buffer_rsrc_t rk_ = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char *>(kbase + (int64_t)c * kChunk * p.k.st * 2), 0, (int)((len - 1) * p.k.st * 2 + K * 2), 0x00020000);
+            const __amdgpu_buffer_rsrc_t rv_ = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char *>(vbase + (int64_t)c * kChunk * p.v.st * 2), 0, (int)((len - 1) * p.v.st * 2 + VS * 2), 0x00020000);
+#pragma unroll
+            for (int m = 0; m < QCH; ++m) {
+                pre_q[m] = __builtin_amdgcn_raw_buffer_load_b128(rq_, (int)qoff[m], 0, 0);
+                pre_k[m] = __builtin_amdgcn_raw_buffer_load_b128(rk_, (int)koff[m], 0, 0);
+            }
+#pragma unroll
+            for (int m = 0; m < VCH; ++m) pre_v[m] = __builtin_amdgcn_raw_buffer_load_b128(rv_, (int)voff[m], 0, 0);
+        };
+        auto commit = [&](const Tiles &t) {
+#pragma unroll
+            for (int m = 0; m < QCH; ++m) {
+                *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = pre_q[m];
+                *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = pre_k[m];
+            }
+#pragma unroll
+            for (int m = 0; m < VCH; ++m) *reinterpret_cast<u32x4 *>(t.v + (rv + m * VROWS) * pv + cv) = pre_v[m];
+        };
+        if (nchunks > 0) {
+            prefetch(0);
+            commit(pipe_tiles_at<K>(smem, 0));
+        }
+        __syncthreads();   // start
+#ifdef FLA_FUSED_TIMING
+        long long tacc[16] = {0};
+        long long tlast = clock64();
+#endif
+        for (int i = 0; i <= nchunks; ++i) {
+            const Tiles t = pipe_tiles_at<K>(smem, i & 1);
+            bf16 *pS = pS0 + (i & 1) * kChunk * pp;
+#ifndef FLA_PIPE_SKIP_PREP
+            if (i < nchunks) {
+                if (i + 1 < nchunks) prefetch(i + 1);
+                switch (wv) {
+                    case 0: phase_a<K, 0>(t, aS, pS, dS, p.scale); break;
+                    case 1: phase_a<K, 1>(t, aS, pS, dS, p.scale); break;
+                    case 2: phase_a<K, 2>(t, aS, pS, dS, p.scale); break;
+                    default: phase_a<K, 3>(t, aS, pS, dS, p.scale); break;
+                }
+            }
+#endif
+            FLA_TICK(0)
+            __syncthreads();   // mid
+            FLA_TICK(1)
+#ifndef FLA_PIPE_SKIP_PREP
+            if (i < nchunks) {
+                // tile 0: this wave's u columns; tiles 1..NTW: its w columns
+                f32x4 r[NT][4];
+#pragma unroll
+                for (int bi = 0; bi < 4; ++bi) {
+                    const f32x4 b4 = lds4(t.B + 16 * bi + 4 * lg), be4 = lds4(t.BEG + 16 * bi + 4 * lg);
+                    const bf16x4 vv = frag_tr4(t.v, pv, wv * 16, 16 * bi);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) r[0][bi][e] = (float)vv[e] * b4[e];
+#pragma unroll
+                    for (int m = 0; m < NTW; ++m) {
+                        const bf16x4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * bi);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) r[1 + m][bi][e] = (float)kv[e] * be4[e];
+                    }
+                }
+                {
+                    const bf16x4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
+                                 d3 = frag_kc4(dS, pd, 48, 0);
+                    const bf16x4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
+                    const bf16x8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
+                    bf16x8 x01[NT];
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][0] = diag_mul(d0, r[q][0], q == 0);
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][1] = mfma16x16(a10, cvt4(r[q][0]), r[q][1]);
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][1] = diag_mul(d1, r[q][1], q == 0);
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) {
+                        x01[q] = frag_from_acc(r[q][0], r[q][1]);
+                        r[q][2] = mfma16x32(a2x, x01[q], r[q][2]);
+                        r[q][3] = mfma16x32(a3x, x01[q], r[q][3]);
+                    }
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][2] = diag_mul(d2, r[q][2], q == 0);
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][3] = mfma16x16(a32, cvt4(r[q][2]), r[q][3]);
+#pragma unroll
+                    for (int q = 0; q < NT; ++q) r[q][3] = diag_mul(d3, r[q][3], q == 0);
+                }
+#pragma unroll
+                for (int m = 0; m < NTW; ++m)
+#pragma unroll
+                    for (int bi = 0; bi < 4; ++bi) acc_to_tile(wS, pw, 16 * bi, (wv * NTW + m) * 16, -r[1 + m][bi]);
+#pragma unroll
+                for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<f32x4 *>(uS + ((wv * 4 + bi) * 64 + l) * 4) = r[0][bi];
+                FLA_TICK(2)
+                if (i + 1 < nchunks) commit(pipe_tiles_at<K>(smem, (i + 1) & 1));
+            }
+#endif
+            FLA_TICK(3)
+            __syncthreads();   // end
+            FLA_TICK(4)
+        }
+#ifdef FLA_FUSED_TIMING
+        if (blockIdx.x == 0 && l == 0 && p.g_out)
+            for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
+#endif
+        return;
+    }
+
+    // ================================== state group ===============================================
+    const int wv = wave - 4, tid = threadIdx.x - GT;
+    const int vcol0 = slab * VS + wv * 16;
+    f32x4 hacc[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        f32x4 a = zero4();
+        if (p.h0) {
+            const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li];
+        }
+        hacc[kt] = a;
+    }
+    const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
+    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + slab * VS);
+    unsigned ooff[VCH];
+#pragma unroll
+    for (int m = 0; m < VCH; ++m) ooff[m] = (unsigned)(((rv + m * VROWS) * p.o.st + cv) * 2);
+    auto store_o = [&](int c) {
+        const int len = min(kChunk, eos - (bos + c * kChunk));
+        char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
+#pragma unroll
+        for (int m = 0; m < VCH; ++m)
+            if (rv + m * VROWS < len)
+                *reinterpret_cast<u32x4 *>(ob + ooff[m]) = *reinterpret_cast<const u32x4 *>(oS + (rv + m * VROWS) * po + cv);
+    };
+    const float *gptr = static_cast<const float *>(p.g.p) + b * p.g.sb + hv * p.g.sh;
+    const float *bptr = static_cast<const float *>(p.beta.p) + b * p.beta.sb + hv * p.beta.sh;
+    float pre_g = 0.f, pre_b = 0.f;
+    auto gate_fetch = [&](int c) {   // wave 0 of the group: lane = token
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        const int tok = start + min(l, len - 1);   // clamped: no predicated load, padding is applied in gate_tables
+        pre_g = gptr[(int64_t)tok * p.g.st];
+        pre_b = bptr[(int64_t)tok * p.beta.st];
+    };
+    auto gate_tables = [&](int c, const Tiles &t) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        float G = wave_inclusive_scan(l < len ? pre_g : 0.f);
+        const float g_end = read_lane(G, len - 1);
+        if (l >= len) {
+            G = g_end;
+            pre_b = 0.f;
+        }
+        const float s0 = read_lane(G, 0), s1 = read_lane(G, 16), s2 = read_lane(G, 32), s3 = read_lane(G, 48);
+        const float e0 = read_lane(G, 15), e1 = read_lane(G, 31), e2 = read_lane(G, 47), e3 = read_lane(G, 63);
+        const int blk = l >> 4;
+        const float Gs = blk == 0 ? s0 : (blk == 1 ? s1 : (blk == 2 ? s2 : s3));
+        const float Ge = blk == 0 ? e0 : (blk == 1 ? e1 : (blk == 2 ? e2 : e3));
+        const int bi = (l >> 2) & 3, bj = l & 3;
+        const float gsI = bi == 0 ? s0 : (bi == 1 ? s1 : (bi == 2 ? s2 : s3));
+        const float geJ = bj == 0 ? e0 : (bj == 1 ? e1 : (bj == 2 ? e2 : e3));
+        const float eg = __expf(G);
+        t.G[l] = G;
+        t.EGS[l] = eg * p.scale;
+        t.B[l] = pre_b;
+        t.BEG[l] = pre_b * eg;
+        t.ROWF[l] = __expf(G - Gs);
+        t.COLF[l] = __expf(Ge - G);
+        if (l < 16) t.BLKF[l] = bj < bi ? __expf(gsI - geJ) : 0.f;
+        if (p.g_out != nullptr && slab == 0 && l < len)
+            p.g_out[b * p.go_sb + hv * p.go_sh + (int64_t)(start + l) * p.go_st] = G;
+    };
+    if (wv == 0 && nchunks > 0) {
+        gate_fetch(0);
+        gate_tables(0, pipe_tiles_at<K>(smem, 0));
+    }
+    __syncthreads();   // start
+#ifdef FLA_FUSED_TIMING
+    long long tacc[16] = {0};
+    long long tlast = clock64();
+#endif
+
+    for (int i = 0; i <= nchunks; ++i) {
+        const int c = i - 1;                               // chunk of this group
+        const Tiles t = pipe_tiles_at<K>(smem, c & 1);
+        const bf16 *pS = pS0 + (c & 1) * kChunk * pp;
+        if (wv == 0 && i + 1 < nchunks) gate_fetch(i + 1);
+        f32x4 U[4], oacc[4], eg4[4];
+#ifdef FLA_PIPE_SKIP_STATE
+        if (c >= 1000000) {
+#else
+        if (c >= 0) {
+#endif
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            if (c >= 1) store_o(c - 1);
+            bf16x8 hB[KS];
+#pragma unroll
+            for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                U[rt] = *reinterpret_cast<const f32x4 *>(uS + ((wv * 4 + rt) * 64 + l) * 4);
+                oacc[rt] = zero4();
+            }
+            {
+                bf16x8 wf[2][4], qf[2][4];
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) {
+                    wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
+                    qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
+                }
+#pragma unroll
+                for (int j = 0; j < KS; ++j) {
+                    const int cb = j & 1, nb = cb ^ 1;
+                    if (j + 1 < KS) {
+#pragma unroll
+                        for (int rt = 0; rt < 4; ++rt) {
+                            wf[nb][rt] = frag_kc(wS, pw, rt * 16, 32 * (j + 1));
+                            qf[nb][rt] = frag_kc(t.q, pq, rt * 16, 32 * (j + 1));
+                        }
+                    }
+                    FLA_SCHED_FENCE();
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt) {
+                        U[rt] = mfma16x32(wf[cb][rt], hB[j], U[rt]);
+                        oacc[rt] = mfma16x32(qf[cb][rt], hB[j], oacc[rt]);
+                    }
+                    FLA_SCHED_FENCE();
+                }
+            }
+            FLA_TICK(0)
+            bf16x8 kfa[KT];
+            f32x4 dk4[4];
+            const float g_last = t.G[len - 1];
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                eg4[rt] = lds4(t.EGS + 16 * rt + 4 * lg);
+                dk4[rt] = lds4(t.G + 16 * rt + 4 * lg);
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) kfa[kt] = KTile<K>::tr(t.k, kt * 16, 0);
+            FLA_SCHED_FENCE();
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dk4[rt][e] = __expf(g_last - dk4[rt][e]);
+            // h <- e^{g_last} h + k^T (v_new e^{g_last - g}), the right operand as hi + lo bf16
+            const float dec_all = __expf(g_last);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] *= dec_all;
+            bf16x8 vhi[2], vlo[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const f32x4 a0 = U[2 * j] * dk4[2 * j], a1 = U[2 * j + 1] * dk4[2 * j + 1];
+                const bf16x4 h0 = cvt4(a0), h1 = cvt4(a1);
+                f32x4 r0, r1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    r0[e] = a0[e] - (float)h0[e];
+                    r1[e] = a1[e] - (float)h1[e];
+                }
+                vhi[j] = cat8(h0, h1);
+                vlo[j] = frag_from_acc(r0, r1);
+            }
+            {
+                bf16x8 kfb[KT];
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) kfb[kt] = KTile<K>::tr(t.k, kt * 16, 32);
+                FLA_SCHED_FENCE();
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    hacc[kt] = mfma16x32(kfa[kt], vhi[0], hacc[kt]);
+                    hacc[kt] = mfma16x32(kfa[kt], vlo[0], hacc[kt]);
+                }
+                FLA_SCHED_FENCE();
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    hacc[kt] = mfma16x32(kfb[kt], vhi[1], hacc[kt]);
+                    hacc[kt] = mfma16x32(kfb[kt], vlo[1], hacc[kt]);
+                }
+            }
+        }
+        FLA_TICK(1)
+        __syncthreads();   // mid
+        FLA_TICK(2)
+#ifdef FLA_PIPE_SKIP_STATE
+        if (c >= 1000000) {
+#else
+        if (c >= 0) {
+#endif
+            // o = scale (e^{G_t} q h + P v_new)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16x8 vb = frag_from_acc(U[2 * j], U[2 * j + 1]);
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt)
+                    if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(pS, pp, rt * 16, 32 * j), vb, oacc[rt]);
+            }
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(oS, po, rt * 16, wv * 16, oacc[rt]);
+        }
+        FLA_TICK(3)
+        if (wv == 0 && i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, (i + 1) & 1));
+        FLA_TICK(4)
+        __syncthreads();   // end
+        FLA_TICK(5)
+    }
+#ifdef FLA_FUSED_TIMING
+    if (blockIdx.x == 0 && l == 0 && p.g_out)
+        for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
+#endif
+    if (nchunks > 0) store_o(nchunks - 1);
+    if (p.hT) {
+        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li] = hacc[kt][e];
+    }
+}
+
+template <int K>
+int launch_pipe(FusedParams &p, hipStream_t stream) {
+    typedef PipeSmem<K> L;
+    const int64_t total = (int64_t)p.geom.N * p.geom.Hv * p.slabs;
+    p.remap = (p.slabs == 2 && total % 16 == 0) ? 1 : 0;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gdn_pipe_kernel<K>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::bytes));
+    FLA_LAUNCH("gdn_fused", stream, (gdn_pipe_kernel<K>), dim3((unsigned)total), dim3(512), L::bytes, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
 template <int K, int CT>
 int launch_fused(FusedParams &p, hipStream_t stream) {
     typedef FusedSmem<K, CT> L;
@@ -731,6 +1177,9 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
         if (atoi(env) == 64) wide = false;
     }
     p.slabs = wide ? geom.V / 128 : geom.V / 64;
+    bool pipe = !wide;
+    if (const char *env = getenv("FLA_HIP_GDN_PIPE")) pipe = pipe && atoi(env) != 0;   // tuning override
+    if (pipe) return geom.K == 128 ? launch_pipe<128>(p, stream) : launch_pipe<64>(p, stream);
     if (geom.K == 128) return wide ? launch_fused<128, 2>(p, stream) : launch_fused<128, 1>(p, stream);
     return wide ? launch_fused<64, 2>(p, stream) : launch_fused<64, 1>(p, stream);
 }
