@@ -86,9 +86,31 @@ __device__ __forceinline__ bf16x2 cvt2(float a, float b) {
     const f32x2 v = {a, b};
     return __builtin_convertvector(v, bf16x2);
 }
+// The two packed halves are joined as integers: joined as bf16 vectors the optimiser folds them into
+// one <4 x bf16> conversion, which the backend then splits into four scalar conversions plus permutes.
 __device__ __forceinline__ bf16x4 cvt4(f32x4 v) {
-    const bf16x2 lo = cvt2(v[0], v[1]), hi = cvt2(v[2], v[3]);
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
+    u32x2 t;
+    t[0] = __builtin_bit_cast(unsigned, cvt2(v[0], v[1]));
+    t[1] = __builtin_bit_cast(unsigned, cvt2(v[2], v[3]));
+    return __builtin_bit_cast(bf16x4, t);
+}
+// x = hi + lo with hi = bf16(x) and lo = bf16(x - hi).  The remainder is formed from the packed
+// conversion's bit pattern (a bf16 is the upper half of an fp32), never by extracting vector
+// elements: element extraction makes the optimiser split the packed conversion into four scalar
+// ones plus permutes.
+__device__ __forceinline__ void split_hilo(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
+    const bf16x2 h01 = cvt2(x[0], x[1]), h23 = cvt2(x[2], x[3]);
+    const unsigned u01 = __builtin_bit_cast(unsigned, h01), u23 = __builtin_bit_cast(unsigned, h23);
+    f32x4 rem;
+    rem[0] = x[0] - __builtin_bit_cast(float, u01 << 16);
+    rem[1] = x[1] - __builtin_bit_cast(float, u01 & 0xffff0000u);
+    rem[2] = x[2] - __builtin_bit_cast(float, u23 << 16);
+    rem[3] = x[3] - __builtin_bit_cast(float, u23 & 0xffff0000u);
+    u32x2 t;
+    t[0] = u01;
+    t[1] = u23;
+    hi = __builtin_bit_cast(bf16x4, t);
+    lo = cvt4(rem);
 }
 __device__ __forceinline__ bf16x8 cat8(bf16x4 lo, bf16x4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);

@@ -206,15 +206,10 @@ __device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16
 
 // D^-1 R for one diagonal block; hilo feeds R as hi + lo bf16 pairs.
 __device__ __forceinline__ f32x4 diag_mul(bf16x4 d, f32x4 r, bool hilo) {
-    const bf16x4 hi = cvt4(r);
-    f32x4 acc = mfma16x16(d, hi, zero4());
-    if (hilo) {
-        f32x4 rest;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) rest[e] = r[e] - (float)hi[e];
-        acc = mfma16x16(d, cvt4(rest), acc);
-    }
-    return acc;
+    if (!hilo) return mfma16x16(d, cvt4(r), zero4());
+    bf16x4 hi, lo;
+    split_hilo(r, hi, lo);
+    return mfma16x16(d, lo, mfma16x16(d, hi, zero4()));
 }
 
 template <int K, int CT>
@@ -557,15 +552,11 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 const f32x4 a0 = U[2 * j][ct] * dk4[2 * j], a1 = U[2 * j + 1][ct] * dk4[2 * j + 1];
-                const bf16x4 h0 = cvt4(a0), h1 = cvt4(a1);
-                f32x4 r0, r1;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    r0[e] = a0[e] - (float)h0[e];
-                    r1[e] = a1[e] - (float)h1[e];
-                }
+                bf16x4 h0, h1, l0, l1;
+                split_hilo(a0, h0, l0);
+                split_hilo(a1, h1, l1);
                 vhi[j][ct] = cat8(h0, h1);
-                vlo[j][ct] = frag_from_acc(r0, r1);
+                vlo[j][ct] = cat8(l0, l1);
             }
         {
             bf16x8 kfb[KT];
@@ -987,15 +978,11 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const f32x4 a0 = U[2 * j] * dk4[2 * j], a1 = U[2 * j + 1] * dk4[2 * j + 1];
-                const bf16x4 h0 = cvt4(a0), h1 = cvt4(a1);
-                f32x4 r0, r1;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    r0[e] = a0[e] - (float)h0[e];
-                    r1[e] = a1[e] - (float)h1[e];
-                }
+                bf16x4 h0, h1, l0, l1;
+                split_hilo(a0, h0, l0);
+                split_hilo(a1, h1, l1);
                 vhi[j] = cat8(h0, h1);
-                vlo[j] = frag_from_acc(r0, r1);
+                vlo[j] = cat8(l0, l1);
             }
             {
                 bf16x8 kfb[KT];

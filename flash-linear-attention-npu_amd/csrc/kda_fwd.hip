@@ -54,11 +54,7 @@ struct HiLo {
 };
 __device__ __forceinline__ HiLo split(f32x4 x) {
     HiLo r;
-    r.hi = cvt4(x);
-    f32x4 rem;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) rem[e] = x[e] - (float)r.hi[e];
-    r.lo = cvt4(rem);
+    split_hilo(x, r.hi, r.lo);
     return r;
 }
 // acc += a * b with both operands carried as head + remainder (the lo*lo term is dropped).
