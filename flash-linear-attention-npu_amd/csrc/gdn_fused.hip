@@ -618,37 +618,42 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 //   prep group  (waves 0-3)  chunk i  : scores (phase A), WY solve (phase B), tile prefetch
 //   state group (waves 4-7)  chunk i-1: v_new, state update, output (phase C), gate tables
 // Each SIMD holds one wave of each group, so the chunk-parallel work of the next chunk runs under
-// the serial state update of the current one.  Two workgroup barriers per chunk:
-//   before `mid`  prep: A(i) -> aS, dS, pS[i&1]        state: C1 + state update of chunk i-1
-//                                                             (reads wS, uS, q/k/tables of i-1)
-//   after  `mid`  prep: B(i) -> wS, uS; tiles of i+1   state: o += P v_new (pS[(i-1)&1]), o tile;
-//                       -> buffer (i+1)&1                       tables of chunk i+1
-// Every buffer written after `mid` was last read before it (and conversely), which is what makes
-// two barriers enough.
+// the serial state update of the current one.  Two workgroup barriers per iteration i:
+//   before `mid`  prep : v(i) -> LDS, loads of chunk i+1 issued, A(i) -> aS, dS, pS[i&1]
+//                 state: v_new = u - w h, state update            (reads wS, uS, k and tables of i-1)
+//   after  `mid`  prep : B(i) -> wS, uS; q, k of i+1 -> LDS
+//                 state: o = scale(e^G q h_old + P v_new) -> HBM   (reads q of i-1, pS[(i-1)&1]);
+//                        tables of chunk i+1
+// Every buffer written in one half was last read in the other half or earlier, which is what makes two
+// barriers enough; q therefore needs three buffers, k and the tables two, v one.
 // =============================================================================================
 template <int K> struct PipeSmem {
     static constexpr int pq = K + 8, pk = KTile<K>::pitch, pv = 64 + 8, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
-                         po = 64 + 8, pd = 24;
+                         pd = 24;
     static constexpr size_t q_bytes = (size_t)kChunk * pq * 2, k_bytes = (size_t)kChunk * pk * 2,
                             v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (6 * kChunk + 16) * 4;
-    static constexpr size_t buf_bytes = q_bytes + k_bytes + v_bytes + tab_bytes;
-    static constexpr size_t a_off = 2 * buf_bytes;
+    static constexpr size_t q_off = 0;                                         // three q tiles
+    static constexpr size_t k_off = q_off + 3 * q_bytes;                       // two k tiles
+    static constexpr size_t v_off = k_off + 2 * k_bytes;                       // one v tile
+    static constexpr size_t t_off = v_off + v_bytes;                           // two sets of gate tables
+    static constexpr size_t a_off = t_off + 2 * tab_bytes;
     static constexpr size_t w_off = a_off + (size_t)kChunk * pa * 2;
-    static constexpr size_t p_off = w_off + (size_t)kChunk * pw * 2;          // two P tiles
-    static constexpr size_t o_off = p_off + 2 * (size_t)kChunk * pp * 2;
-    static constexpr size_t d_off = o_off + (size_t)kChunk * po * 2;
-    static constexpr size_t u_off = d_off + (size_t)kChunk * pd * 2;          // u as register images, fp32
+    static constexpr size_t p_off = w_off + (size_t)kChunk * pw * 2;           // two P tiles
+    static constexpr size_t d_off = p_off + 2 * (size_t)kChunk * pp * 2;
+    static constexpr size_t u_off = d_off + (size_t)kChunk * pd * 2;           // u as register images, fp32
     static constexpr size_t bytes = u_off + (size_t)kChunk * 64 * 4;
 };
+// Tiles of chunk c: q cycles through three buffers (it is read until the end of the iteration after
+// the one that prefetches its successor's successor), k and the tables through two, v has one.
 template <int K>
-__device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int buf) {
+__device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
     typedef PipeSmem<K> L;
-    unsigned char *b = smem + buf * L::buf_bytes;
+    const int c3 = (unsigned)(c + 3) % 3u, c2 = c & 1;
     Tiles t;
-    t.q = reinterpret_cast<bf16 *>(b);
-    t.k = reinterpret_cast<bf16 *>(b + L::q_bytes);
-    t.v = reinterpret_cast<bf16 *>(b + L::q_bytes + L::k_bytes);
-    t.G = reinterpret_cast<float *>(b + L::q_bytes + L::k_bytes + L::v_bytes);
+    t.q = reinterpret_cast<bf16 *>(smem + L::q_off + c3 * L::q_bytes);
+    t.k = reinterpret_cast<bf16 *>(smem + L::k_off + c2 * L::k_bytes);
+    t.v = reinterpret_cast<bf16 *>(smem + L::v_off);
+    t.G = reinterpret_cast<float *>(smem + L::t_off + c2 * L::tab_bytes);
     t.EGS = t.G + kChunk;
     t.B = t.EGS + kChunk;
     t.BEG = t.B + kChunk;
@@ -658,10 +663,27 @@ __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int buf) {
     return t;
 }
 
+// One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with
+// `stride` bytes between rows; `base` points at column c0 of row 0).  Lane pairs exchange halves as in
+// acc_to_tile so that every lane writes two whole dwords.
+__device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
+    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
+    const bool odd = li & 1;
+    const unsigned send = odd ? p01 : p23;
+    const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+    const unsigned left = odd ? recv : p01, right = odd ? p23 : recv;
+    const int row = r0 + 4 * lg + (odd ? 2 : 0);
+    char *dst = base + row * stride + (li & ~1) * 2;
+    if (row < len) *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);
+    if (row + 1 < len) *reinterpret_cast<unsigned *>(dst + stride) = __builtin_amdgcn_perm(right, left, 0x07060302u);
+}
+
 template <int K>
 __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     typedef PipeSmem<K> L;
-    constexpr int VS = 64, pq = L::pq, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, po = L::po, pd = L::pd;
+    constexpr int VS = 64, pq = L::pq, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, pd = L::pd;
     constexpr int KT = K / 16, KS = K / 32;
     constexpr int GT = 256;                              // threads of one group
     constexpr int QCH = kChunk * (K / 8) / GT, VCH = kChunk * (VS / 8) / GT;
@@ -671,7 +693,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     bf16 *aS = reinterpret_cast<bf16 *>(smem + L::a_off);
     bf16 *wS = reinterpret_cast<bf16 *>(smem + L::w_off);
     bf16 *pS0 = reinterpret_cast<bf16 *>(smem + L::p_off);
-    bf16 *oS = reinterpret_cast<bf16 *>(smem + L::o_off);
     bf16 *dS = reinterpret_cast<bf16 *>(smem + L::d_off);
     float *uS = reinterpret_cast<float *>(smem + L::u_off);
 
@@ -734,18 +755,17 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int m = 0; m < VCH; ++m) pre_v[m] = __builtin_amdgcn_raw_buffer_load_b128(rv_, (int)voff[m], 0, 0);
         };
-        auto commit = [&](const Tiles &t) {
+        auto commit_qk = [&](const Tiles &t) {
 #pragma unroll
             for (int m = 0; m < QCH; ++m) {
                 *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = pre_q[m];
                 *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = pre_k[m];
             }
-#pragma unroll
-            for (int m = 0; m < VCH; ++m) *reinterpret_cast<u32x4 *>(t.v + (rv + m * VROWS) * pv + cv) = pre_v[m];
         };
+        bf16 *vS = reinterpret_cast<bf16 *>(smem + L::v_off);
         if (nchunks > 0) {
             prefetch(0);
-            commit(pipe_tiles_at<K>(smem, 0));
+            commit_qk(pipe_tiles_at<K>(smem, 0));
         }
         __syncthreads();   // start
 #ifdef FLA_FUSED_TIMING
@@ -753,10 +773,12 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         long long tlast = clock64();
 #endif
         for (int i = 0; i <= nchunks; ++i) {
-            const Tiles t = pipe_tiles_at<K>(smem, i & 1);
+            const Tiles t = pipe_tiles_at<K>(smem, i);
             bf16 *pS = pS0 + (i & 1) * kChunk * pp;
-#ifndef FLA_PIPE_SKIP_PREP
             if (i < nchunks) {
+                // v of this chunk has waited in registers: its single LDS tile was read until the last barrier
+#pragma unroll
+                for (int m = 0; m < VCH; ++m) *reinterpret_cast<u32x4 *>(vS + (rv + m * VROWS) * pv + cv) = pre_v[m];
                 if (i + 1 < nchunks) prefetch(i + 1);
                 switch (wv) {
                     case 0: phase_a<K, 0>(t, aS, pS, dS, p.scale); break;
@@ -765,13 +787,12 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                     default: phase_a<K, 3>(t, aS, pS, dS, p.scale); break;
                 }
             }
-#endif
             FLA_TICK(0)
             __syncthreads();   // mid
             FLA_TICK(1)
-#ifndef FLA_PIPE_SKIP_PREP
             if (i < nchunks) {
-                // tile 0: this wave's u columns; tiles 1..NTW: its w columns
+                // tile 0: this wave's u columns; tiles 1..NTW: its w columns (the table holds -beta e^G, so
+                // the solve yields -w, which is what the state group accumulates)
                 f32x4 r[NT][4];
 #pragma unroll
                 for (int bi = 0; bi < 4; ++bi) {
@@ -814,13 +835,12 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
                 for (int m = 0; m < NTW; ++m)
 #pragma unroll
-                    for (int bi = 0; bi < 4; ++bi) acc_to_tile(wS, pw, 16 * bi, (wv * NTW + m) * 16, -r[1 + m][bi]);
+                    for (int bi = 0; bi < 4; ++bi) acc_to_tile(wS, pw, 16 * bi, (wv * NTW + m) * 16, r[1 + m][bi]);
 #pragma unroll
                 for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<f32x4 *>(uS + ((wv * 4 + bi) * 64 + l) * 4) = r[0][bi];
                 FLA_TICK(2)
-                if (i + 1 < nchunks) commit(pipe_tiles_at<K>(smem, (i + 1) & 1));
+                if (i + 1 < nchunks) commit_qk(pipe_tiles_at<K>(smem, i + 1));
             }
-#endif
             FLA_TICK(3)
             __syncthreads();   // end
             FLA_TICK(4)
@@ -833,7 +853,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     }
 
     // ================================== state group ===============================================
-    const int wv = wave - 4, tid = threadIdx.x - GT;
+    const int wv = wave - 4;
     const int vcol0 = slab * VS + wv * 16;
     f32x4 hacc[KT];
 #pragma unroll
@@ -846,29 +866,22 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         }
         hacc[kt] = a;
     }
-    const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
-    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + slab * VS);
-    unsigned ooff[VCH];
-#pragma unroll
-    for (int m = 0; m < VCH; ++m) ooff[m] = (unsigned)(((rv + m * VROWS) * p.o.st + cv) * 2);
-    auto store_o = [&](int c) {
-        const int len = min(kChunk, eos - (bos + c * kChunk));
-        char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
-#pragma unroll
-        for (int m = 0; m < VCH; ++m)
-            if (rv + m * VROWS < len)
-                *reinterpret_cast<u32x4 *>(ob + ooff[m]) = *reinterpret_cast<const u32x4 *>(oS + (rv + m * VROWS) * po + cv);
-    };
+    // The initial-state loads must be complete before the loop: left pending, the compiler's wait-count
+    // bookkeeping carries them around the loop and turns every first use of the state into a wait for
+    // ALL outstanding memory operations, including the gate loads issued for the next chunk.
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + vcol0);
     const float *gptr = static_cast<const float *>(p.g.p) + b * p.g.sb + hv * p.g.sh;
     const float *bptr = static_cast<const float *>(p.beta.p) + b * p.beta.sb + hv * p.beta.sh;
     float pre_g = 0.f, pre_b = 0.f;
-    auto gate_fetch = [&](int c) {   // wave 0 of the group: lane = token
+    auto gate_fetch = [&](int c) {   // every wave of the group: lane = token
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
         const int tok = start + min(l, len - 1);   // clamped: no predicated load, padding is applied in gate_tables
         pre_g = gptr[(int64_t)tok * p.g.st];
         pre_b = bptr[(int64_t)tok * p.beta.st];
     };
+    // Each wave scans the gates of the chunk itself and writes its share of the tables.
     auto gate_tables = [&](int c, const Tiles &t) {
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
@@ -878,28 +891,36 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             G = g_end;
             pre_b = 0.f;
         }
-        const float s0 = read_lane(G, 0), s1 = read_lane(G, 16), s2 = read_lane(G, 32), s3 = read_lane(G, 48);
-        const float e0 = read_lane(G, 15), e1 = read_lane(G, 31), e2 = read_lane(G, 47), e3 = read_lane(G, 63);
-        const int blk = l >> 4;
-        const float Gs = blk == 0 ? s0 : (blk == 1 ? s1 : (blk == 2 ? s2 : s3));
-        const float Ge = blk == 0 ? e0 : (blk == 1 ? e1 : (blk == 2 ? e2 : e3));
-        const int bi = (l >> 2) & 3, bj = l & 3;
-        const float gsI = bi == 0 ? s0 : (bi == 1 ? s1 : (bi == 2 ? s2 : s3));
-        const float geJ = bj == 0 ? e0 : (bj == 1 ? e1 : (bj == 2 ? e2 : e3));
-        const float eg = __expf(G);
-        t.G[l] = G;
-        t.EGS[l] = eg * p.scale;
-        t.B[l] = pre_b;
-        t.BEG[l] = pre_b * eg;
-        t.ROWF[l] = __expf(G - Gs);
-        t.COLF[l] = __expf(Ge - G);
-        if (l < 16) t.BLKF[l] = bj < bi ? __expf(gsI - geJ) : 0.f;
-        if (p.g_out != nullptr && slab == 0 && l < len)
-            p.g_out[b * p.go_sb + hv * p.go_sh + (int64_t)(start + l) * p.go_st] = G;
+        if (wv == 0) {
+            t.G[l] = G;
+            t.EGS[l] = __expf(G) * p.scale;
+            if (p.g_out != nullptr && slab == 0 && l < len)
+                p.g_out[b * p.go_sb + hv * p.go_sh + (int64_t)(start + l) * p.go_st] = G;
+        } else if (wv == 1) {
+            t.B[l] = pre_b;
+            t.BEG[l] = -pre_b * __expf(G);
+        } else if (wv == 2) {
+            // gate at the first / last token of each 16-token block
+            const float s0 = read_lane(G, 0), s1 = read_lane(G, 16), s2 = read_lane(G, 32), s3 = read_lane(G, 48);
+            const float e0 = read_lane(G, 15), e1 = read_lane(G, 31), e2 = read_lane(G, 47), e3 = read_lane(G, 63);
+            const int blk = l >> 4;
+            const float Gs = blk == 0 ? s0 : (blk == 1 ? s1 : (blk == 2 ? s2 : s3));
+            const float Ge = blk == 0 ? e0 : (blk == 1 ? e1 : (blk == 2 ? e2 : e3));
+            t.ROWF[l] = __expf(G - Gs);
+            t.COLF[l] = __expf(Ge - G);
+        } else {
+            const float s1 = read_lane(G, 16), s2 = read_lane(G, 32), s3 = read_lane(G, 48);
+            const float e0 = read_lane(G, 15), e1 = read_lane(G, 31), e2 = read_lane(G, 47);
+            const int bi = (l >> 2) & 3, bj = l & 3;
+            const float gsI = bi == 1 ? s1 : (bi == 2 ? s2 : s3);
+            const float geJ = bj == 0 ? e0 : (bj == 1 ? e1 : e2);
+            if (l < 16) t.BLKF[l] = bj < bi ? __expf(gsI - geJ) : 0.f;
+        }
     };
-    if (wv == 0 && nchunks > 0) {
+    if (nchunks > 0) {
         gate_fetch(0);
         gate_tables(0, pipe_tiles_at<K>(smem, 0));
+        if (nchunks > 1) gate_fetch(1);
     }
     __syncthreads();   // start
 #ifdef FLA_FUSED_TIMING
@@ -909,48 +930,35 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 
     for (int i = 0; i <= nchunks; ++i) {
         const int c = i - 1;                               // chunk of this group
-        const Tiles t = pipe_tiles_at<K>(smem, c & 1);
+        const Tiles t = pipe_tiles_at<K>(smem, c);
         const bf16 *pS = pS0 + (c & 1) * kChunk * pp;
-        if (wv == 0 && i + 1 < nchunks) gate_fetch(i + 1);
-        f32x4 U[4], oacc[4], eg4[4];
+        const int len = c >= 0 ? min(kChunk, eos - (bos + c * kChunk)) : 0;
+        f32x4 U[4], eg4[4];
+        bf16x8 hB[KS];
 #ifdef FLA_PIPE_SKIP_STATE
         if (c >= 1000000) {
 #else
         if (c >= 0) {
 #endif
-            const int len = min(kChunk, eos - (bos + c * kChunk));
-            if (c >= 1) store_o(c - 1);
-            bf16x8 hB[KS];
+            // state at chunk start as bf16 operand; it also serves q h after the update below
 #pragma unroll
             for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) {
-                U[rt] = *reinterpret_cast<const f32x4 *>(uS + ((wv * 4 + rt) * 64 + l) * 4);
-                oacc[rt] = zero4();
-            }
-            {
-                bf16x8 wf[2][4], qf[2][4];
+            for (int rt = 0; rt < 4; ++rt) U[rt] = *reinterpret_cast<const f32x4 *>(uS + ((wv * 4 + rt) * 64 + l) * 4);
+            {   // v_new = u + (-w) h
+                bf16x8 wf[2][4];
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt) {
-                    wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
-                    qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
-                }
+                for (int rt = 0; rt < 4; ++rt) wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
 #pragma unroll
                 for (int j = 0; j < KS; ++j) {
                     const int cb = j & 1, nb = cb ^ 1;
                     if (j + 1 < KS) {
 #pragma unroll
-                        for (int rt = 0; rt < 4; ++rt) {
-                            wf[nb][rt] = frag_kc(wS, pw, rt * 16, 32 * (j + 1));
-                            qf[nb][rt] = frag_kc(t.q, pq, rt * 16, 32 * (j + 1));
-                        }
+                        for (int rt = 0; rt < 4; ++rt) wf[nb][rt] = frag_kc(wS, pw, rt * 16, 32 * (j + 1));
                     }
                     FLA_SCHED_FENCE();
 #pragma unroll
-                    for (int rt = 0; rt < 4; ++rt) {
-                        U[rt] = mfma16x32(wf[cb][rt], hB[j], U[rt]);
-                        oacc[rt] = mfma16x32(qf[cb][rt], hB[j], oacc[rt]);
-                    }
+                    for (int rt = 0; rt < 4; ++rt) U[rt] = mfma16x32(wf[cb][rt], hB[j], U[rt]);
                     FLA_SCHED_FENCE();
                 }
             }
@@ -1010,7 +1018,27 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #else
         if (c >= 0) {
 #endif
-            // o = scale (e^{G_t} q h + P v_new)
+            // o = scale (e^{G_t} q h + P v_new), h the state at chunk start
+            f32x4 oacc[4];
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) oacc[rt] = zero4();
+            {
+                bf16x8 qf[2][4];
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
+#pragma unroll
+                for (int j = 0; j < KS; ++j) {
+                    const int cb = j & 1, nb = cb ^ 1;
+                    if (j + 1 < KS) {
+#pragma unroll
+                        for (int rt = 0; rt < 4; ++rt) qf[nb][rt] = frag_kc(t.q, pq, rt * 16, 32 * (j + 1));
+                    }
+                    FLA_SCHED_FENCE();
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[cb][rt], hB[j], oacc[rt]);
+                    FLA_SCHED_FENCE();
+                }
+            }
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
 #pragma unroll
@@ -1020,11 +1048,18 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 for (int rt = 0; rt < 4; ++rt)
                     if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(pS, pp, rt * 16, 32 * j), vb, oacc[rt]);
             }
+            // tables of the next chunk, then the gate loads of the one after it, and only then the output
+            // stores: memory operations retire in order, so the loads must not queue behind the stores
+            if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
+            if (i + 2 < nchunks) gate_fetch(i + 2);
+            FLA_TICK(3)
+            char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc_to_tile(oS, po, rt * 16, wv * 16, oacc[rt]);
+            for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
+        } else {
+            if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
+            if (i + 2 < nchunks) gate_fetch(i + 2);
         }
-        FLA_TICK(3)
-        if (wv == 0 && i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, (i + 1) & 1));
         FLA_TICK(4)
         __syncthreads();   // end
         FLA_TICK(5)
@@ -1033,7 +1068,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     if (blockIdx.x == 0 && l == 0 && p.g_out)
         for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
 #endif
-    if (nchunks > 0) store_o(nchunks - 1);
     if (p.hT) {
         float *s = p.hT + n * p.s_sn + hv * p.s_sh;
 #pragma unroll
