@@ -631,7 +631,7 @@ template <int K> struct PipeSmem {
     static constexpr int pq = K + 8, pk = KTile<K>::pitch, pv = 64 + 8, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
                          pd = 24;
     static constexpr size_t q_bytes = (size_t)kChunk * pq * 2, k_bytes = (size_t)kChunk * pk * 2,
-                            v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (6 * kChunk + 16) * 4;
+                            v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (7 * kChunk + 16) * 4;
     static constexpr size_t q_off = 0;                                         // three q tiles
     static constexpr size_t k_off = q_off + 3 * q_bytes;                       // two k tiles
     static constexpr size_t v_off = k_off + 2 * k_bytes;                       // one v tile
@@ -662,6 +662,8 @@ __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
     t.BLKF = t.COLF + kChunk;
     return t;
 }
+// e^{G_last - G_t} per token (decay of v_new towards the chunk end), after the 16 block factors
+__device__ __forceinline__ float *pipe_decay_table(const Tiles &t) { return t.BLKF + 16; }
 
 // One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with
 // `stride` bytes between rows; `base` points at column c0 of row 0).  Lane pairs exchange halves as in
@@ -871,6 +873,9 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     // ALL outstanding memory operations, including the gate loads issued for the next chunk.
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + vcol0);
+    // lane part of an output tile's address: rows 4lg (+2 for odd lanes), column pair of the lane
+    const unsigned o_lane = (unsigned)((4 * lg + ((li & 1) ? 2 : 0)) * p.o.st * 2 + (li & ~1) * 2);
+    const unsigned o_row = (unsigned)(p.o.st * 2);
     const float *gptr = static_cast<const float *>(p.g.p) + b * p.g.sb + hv * p.g.sh;
     const float *bptr = static_cast<const float *>(p.beta.p) + b * p.beta.sb + hv * p.beta.sh;
     float pre_g = 0.f, pre_b = 0.f;
@@ -894,6 +899,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         if (wv == 0) {
             t.G[l] = G;
             t.EGS[l] = __expf(G) * p.scale;
+            pipe_decay_table(t)[l] = l < len ? __expf(g_end - G) : 0.f;
             if (p.g_out != nullptr && slab == 0 && l < len)
                 p.g_out[b * p.go_sb + hv * p.go_sh + (int64_t)(start + l) * p.go_st] = G;
         } else if (wv == 1) {
@@ -969,15 +975,11 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
                 eg4[rt] = lds4(t.EGS + 16 * rt + 4 * lg);
-                dk4[rt] = lds4(t.G + 16 * rt + 4 * lg);
+                dk4[rt] = lds4(pipe_decay_table(t) + 16 * rt + 4 * lg);
             }
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) kfa[kt] = KTile<K>::tr(t.k, kt * 16, 0);
             FLA_SCHED_FENCE();
-#pragma unroll
-            for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dk4[rt][e] = __expf(g_last - dk4[rt][e]);
             // h <- e^{g_last} h + k^T (v_new e^{g_last - g}), the right operand as hi + lo bf16
             const float dec_all = __expf(g_last);
 #pragma unroll
@@ -1010,6 +1012,19 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 }
             }
         }
+        // q of this chunk and its P tile have been in LDS since the previous iteration: the first operands of
+        // the second half are fetched before the barrier, so their latency hides behind the wait
+        bf16x8 qf[2][4], pf[6];
+        if (c >= 0) {
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
+            pf[0] = frag_kc(pS, pp, 0, 0);
+            pf[1] = frag_kc(pS, pp, 16, 0);
+            pf[2] = frag_kc(pS, pp, 32, 0);
+            pf[3] = frag_kc(pS, pp, 32, 32);
+            pf[4] = frag_kc(pS, pp, 48, 0);
+            pf[5] = frag_kc(pS, pp, 48, 32);
+        }
         FLA_TICK(1)
         __syncthreads();   // mid
         FLA_TICK(2)
@@ -1023,9 +1038,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] = zero4();
             {
-                bf16x8 qf[2][4];
-#pragma unroll
-                for (int rt = 0; rt < 4; ++rt) qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
 #pragma unroll
                 for (int j = 0; j < KS; ++j) {
                     const int cb = j & 1, nb = cb ^ 1;
@@ -1041,12 +1053,14 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             }
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const bf16x8 vb = frag_from_acc(U[2 * j], U[2 * j + 1]);
-#pragma unroll
-                for (int rt = 0; rt < 4; ++rt)
-                    if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(pS, pp, rt * 16, 32 * j), vb, oacc[rt]);
+            {
+                const bf16x8 vb0 = frag_from_acc(U[0], U[1]), vb1 = frag_from_acc(U[2], U[3]);
+                oacc[0] = mfma16x32(pf[0], vb0, oacc[0]);
+                oacc[1] = mfma16x32(pf[1], vb0, oacc[1]);
+                oacc[2] = mfma16x32(pf[2], vb0, oacc[2]);
+                oacc[3] = mfma16x32(pf[4], vb0, oacc[3]);
+                oacc[2] = mfma16x32(pf[3], vb1, oacc[2]);
+                oacc[3] = mfma16x32(pf[5], vb1, oacc[3]);
             }
             // tables of the next chunk, then the gate loads of the one after it, and only then the output
             // stores: memory operations retire in order, so the loads must not queue behind the stores
@@ -1055,7 +1069,21 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             FLA_TICK(3)
             char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
+            for (int rt = 0; rt < 4; ++rt) {
+                const f32x4 acc = oacc[rt];
+                const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
+                const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
+                const bool odd = li & 1;
+                const unsigned send = odd ? p01 : p23;
+                const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+                const unsigned left = odd ? recv : p01, right = odd ? p23 : recv;
+                char *tile = ob + (int64_t)rt * 16 * o_row;          // uniform
+                const int row = rt * 16 + 4 * lg + (odd ? 2 : 0);
+                if (len == kChunk || row < len)
+                    *reinterpret_cast<unsigned *>(tile + o_lane) = __builtin_amdgcn_perm(right, left, 0x05040100u);
+                if (len == kChunk || row + 1 < len)
+                    *reinterpret_cast<unsigned *>(tile + (o_lane + o_row)) = __builtin_amdgcn_perm(right, left, 0x07060302u);
+            }
         } else {
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
