@@ -665,23 +665,6 @@ __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
 // e^{G_last - G_t} per token (decay of v_new towards the chunk end), after the 16 block factors
 __device__ __forceinline__ float *pipe_decay_table(const Tiles &t) { return t.BLKF + 16; }
 
-// One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with
-// `stride` bytes between rows; `base` points at column c0 of row 0).  Lane pairs exchange halves as in
-// acc_to_tile so that every lane writes two whole dwords.
-__device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
-    const int l = lane_id(), li = l & 15, lg = l >> 4;
-    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
-    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
-    const bool odd = li & 1;
-    const unsigned send = odd ? p01 : p23;
-    const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
-    const unsigned left = odd ? recv : p01, right = odd ? p23 : recv;
-    const int row = r0 + 4 * lg + (odd ? 2 : 0);
-    char *dst = base + row * stride + (li & ~1) * 2;
-    if (row < len) *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);
-    if (row + 1 < len) *reinterpret_cast<unsigned *>(dst + stride) = __builtin_amdgcn_perm(right, left, 0x07060302u);
-}
-
 template <int K>
 __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     typedef PipeSmem<K> L;

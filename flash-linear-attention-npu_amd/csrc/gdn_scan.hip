@@ -310,19 +310,27 @@ struct DhuParams {
     float scale;
 };
 
-template <int K, int CT, bool GK>
-__global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
+template <int K> struct DhuSmem {
+    static constexpr int pk = K + 8, pt = K + 16, pv = 64 + 16;
+    static constexpr size_t k_off = 0;                                    // k (contraction along channels)
+    static constexpr size_t q_off = k_off + (size_t)kChunk * pk * 2;      // q (read transposed)
+    static constexpr size_t w_off = q_off + (size_t)kChunk * pt * 2;      // w (read transposed)
+    static constexpr size_t o_off = w_off + (size_t)kChunk * pt * 2;      // d_o slab
+    static constexpr size_t v_off = o_off + (size_t)kChunk * pv * 2;      // dv slab
+    static constexpr size_t g_off = v_off + (size_t)kChunk * pv * 2;      // [max(K,64)] gate row, [64] factors
+    static constexpr size_t buf_bytes = g_off + (size_t)((K > kChunk ? K : kChunk) + kChunk) * 4;
+    static constexpr size_t bytes = 2 * buf_bytes;
+};
+
+// 512 threads: waves 0-3 compute chunk c (walking backwards) from LDS buffer c&1 while waves 4-7 copy
+// the tiles of chunk c-1 into the other buffer; one barrier per chunk.  dv2 leaves from registers.
+template <int K, bool GK>
+__global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int VS = 64 * CT;
-    constexpr int pk = K + 8, pt = K + 16, pv = VS + 16;
+    typedef DhuSmem<K> L;
+    constexpr int VS = 64, CT = 1;
+    constexpr int pk = L::pk, pt = L::pt, pv = L::pv;
     constexpr int KT = K / 16, KS = K / 32;
-    bf16 *kS = reinterpret_cast<bf16 *>(smem);
-    bf16 *qS = kS + kChunk * pk;
-    bf16 *wS = qS + kChunk * pt;
-    bf16 *oS = wS + kChunk * pt;     // d_o slab
-    bf16 *vS = oS + kChunk * pv;     // dv slab in, dv2 slab out
-    float *gS = reinterpret_cast<float *>(vS + kChunk * pv);   // [64] gate / [K] last-row channel gate
-    float *fS = gS + (GK ? K : kChunk);                        // [64] factor scale * e^{g_t}
 
     const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
@@ -335,10 +343,60 @@ __global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
         chunk0 = p.geom.choff[n];
     }
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const bf16 *og = static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
+    const bf16 *vg = static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
+
+    if (wave_id() >= 4) {
+        // ------------------------------- loader waves -------------------------------------------
+        const int tid = threadIdx.x - kThreads;
+        auto load = [&](int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            TileCopy<kThreads, kChunk, K> tk, tq, tw;
+            TileCopy<kThreads, kChunk, VS> to, tv;
+            tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
+            tq.fetch(qg + (int64_t)start * p.q.st, p.q.st, len, tid);
+            tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
+            to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+            tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            float *gS = reinterpret_cast<float *>(buf + L::g_off);
+            float *fS = gS + (K > kChunk ? K : kChunk);
+            float gv = 0.f;
+            if (GK) {
+                if (tid < K) gv = p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + tid];
+            } else if (tid < kChunk) {
+                gv = tid < len ? load_scalar(p.g, b, hv, start + tid) : 0.f;
+            }
+            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pk, len, tid);
+            tq.commit(reinterpret_cast<bf16 *>(buf + L::q_off), pt, len, tid);
+            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pt, len, tid);
+            to.commit(reinterpret_cast<bf16 *>(buf + L::o_off), pv, len, tid);
+            tv.commit(reinterpret_cast<bf16 *>(buf + L::v_off), pv, len, tid);
+            if (GK) {
+                if (tid < K) gS[tid] = exp2f(gv);
+                if (tid < kChunk) fS[tid] = p.scale;
+            } else if (tid < kChunk) {
+                gS[tid] = gv;
+                fS[tid] = tid < len ? p.scale * __expf(gv) : 0.f;
+            }
+        };
+        if (nchunks > 0) load(nchunks - 1);
+        __syncthreads();
+        for (int c = nchunks - 1; c >= 0; --c) {
+            if (c > 0) load(c - 1);
+            __syncthreads();
+        }
+        return;
+    }
+
+    // --------------------------------- compute waves ---------------------------------------------
     const int wv = wave_id();
     const int l = lane_id(), li = l & 15, lg = l >> 4;
-    const int vcol0 = slab * VS + wv * 16 * CT;
-
+    const int vcol0 = slab * VS + wv * 16;
     f32x4 dacc[KT][CT];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -352,34 +410,21 @@ __global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
             }
             dacc[kt][ct] = a;
         }
-
-    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
-    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
-    const bf16 *og = static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
-    const bf16 *vg = static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
-    bf16 *v2g = static_cast<bf16 *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + slab * VS;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // terminal gradient loaded before the loop (vmcnt(0))
+    char *v2g = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + vcol0);
+    __syncthreads();
 
     for (int c = nchunks - 1; c >= 0; --c) {
+        const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
+        const bf16 *qS = reinterpret_cast<const bf16 *>(buf + L::q_off);
+        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
+        const bf16 *oS = reinterpret_cast<const bf16 *>(buf + L::o_off);
+        const bf16 *vS = reinterpret_cast<const bf16 *>(buf + L::v_off);
+        const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
+        const float *fS = gS + (K > kChunk ? K : kChunk);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
-        __syncthreads();
-        load_tile<kThreads>(kS, pk, kg + (int64_t)start * p.k.st, p.k.st, kChunk, K, len);
-        load_tile<kThreads>(qS, pt, qg + (int64_t)start * p.q.st, p.q.st, kChunk, K, len);
-        load_tile<kThreads>(wS, pt, wg + (int64_t)start * p.w.st, p.w.st, kChunk, K, len);
-        load_tile<kThreads>(oS, pv, og + (int64_t)start * p.d_o.st, p.d_o.st, kChunk, VS, len);
-        load_tile<kThreads>(vS, pv, vg + (int64_t)start * p.dv.st, p.dv.st, kChunk, VS, len);
-        if (GK) {
-            if (threadIdx.x < K)
-                gS[threadIdx.x] = exp2f(p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + threadIdx.x]);
-            if (threadIdx.x < kChunk) fS[threadIdx.x] = p.scale;
-        } else if (threadIdx.x < kChunk) {
-            const int t = threadIdx.x;
-            const float gt = t < len ? load_scalar(p.g, b, hv, start + t) : 0.f;
-            gS[t] = gt;
-            fS[t] = t < len ? p.scale * __expf(gt) : 0.f;
-        }
-        __syncthreads();
 
         bf16x8 hB[KS][CT];
 #pragma unroll
@@ -424,10 +469,13 @@ __global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
                     dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + (float)old[e] : 0.f;
                 }
             }
+        {
+            char *dst = v2g + (int64_t)start * p.dv2.st * 2;
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
+            for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc_to_tile(vS, pv, rt * 16, (wv * CT + ct) * 16, dv2[rt][ct]);
+                for (int ct = 0; ct < CT; ++ct) acc_to_global(dst + ct * 32, (int64_t)p.dv2.st * 2, rt * 16, len, dv2[rt][ct]);
+        }
 
         // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
 #pragma unroll
@@ -471,7 +519,6 @@ __global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
             }
         }
         __syncthreads();
-        store_tile<kThreads>(v2g + (int64_t)start * p.dv2.st, p.dv2.st, vS, pv, VS, len);
     }
 
     // gradient of the initial state
@@ -488,14 +535,12 @@ __global__ void __launch_bounds__(kThreads) bwd_dhu_kernel(const DhuParams p) {
             }
 }
 
-template <int K, int CT, bool GK>
+template <int K, bool GK>
 int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
-    constexpr int VS = 64 * CT;
-    const size_t smem = ((size_t)kChunk * (K + 8) + 2 * (size_t)kChunk * (K + 16) + 2 * (size_t)kChunk * (VS + 16)) * 2 +
-                        ((GK ? K : kChunk) + kChunk) * 4;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, CT, GK>),
+    const size_t smem = DhuSmem<K>::bytes;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, CT, GK>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -608,8 +653,8 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     }
     p.scale = (float)scale;
     const int slabs = geom.V / 64;
-    if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, 1, true>(p, slabs, stream) : launch_bwd_dhu<128, 1, false>(p, slabs, stream);
-    return has_gk ? launch_bwd_dhu<64, 1, true>(p, slabs, stream) : launch_bwd_dhu<64, 1, false>(p, slabs, stream);
+    if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, true>(p, slabs, stream) : launch_bwd_dhu<128, false>(p, slabs, stream);
+    return has_gk ? launch_bwd_dhu<64, true>(p, slabs, stream) : launch_bwd_dhu<64, false>(p, slabs, stream);
 }
 
 }  // namespace

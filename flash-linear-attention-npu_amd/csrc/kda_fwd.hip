@@ -370,18 +370,27 @@ struct KdaScanParams {
     float scale;
 };
 
+template <int K> struct ScanSmem {
+    static constexpr int pw = K + 8, pt = K + 16, pu = 64 + 16, pb = 72;
+    static constexpr size_t w_off = 0;                                    // w
+    static constexpr size_t q_off = w_off + (size_t)kChunk * pw * 2;      // qg
+    static constexpr size_t k_off = q_off + (size_t)kChunk * pw * 2;      // kg (read transposed)
+    static constexpr size_t u_off = k_off + (size_t)kChunk * pt * 2;      // u slab
+    static constexpr size_t a_off = u_off + (size_t)kChunk * pu * 2;      // Aqk
+    static constexpr size_t d_off = a_off + (size_t)kChunk * pb * 2;      // [K] decay of the chunk
+    static constexpr size_t buf_bytes = d_off + (size_t)K * 4;
+    static constexpr size_t bytes = 2 * buf_bytes;
+};
+
+// 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
+// c+1 from memory into the other buffer; one barrier per chunk.  Outputs leave from registers.
 template <int K>
-__global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams p) {
+__global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
+    typedef ScanSmem<K> L;
     constexpr int VS = 64;
-    constexpr int pw = K + 8, pt = K + 16, pu = VS + 16, pb = 72, po = VS + 8;
+    constexpr int pw = L::pw, pt = L::pt, pu = L::pu, pb = L::pb;
     constexpr int KT = K / 16, KS = K / 32;
-    bf16 *wS = reinterpret_cast<bf16 *>(smem);   // w, later the o staging
-    bf16 *qS = wS + kChunk * pw;                 // qg
-    bf16 *kS = qS + kChunk * pw;                 // kg (read transposed)
-    bf16 *uS = kS + kChunk * pt;                 // u slab, later v_new
-    bf16 *aS = uS + kChunk * pu;                 // Aqk
-    float *dS = reinterpret_cast<float *>(aS + kChunk * pb);   // [K] decay of the chunk
 
     const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
     const int V = p.geom.V;
@@ -393,10 +402,46 @@ __global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams 
         chunk0 = p.geom.choff[n];
     }
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int64_t head_row = ((int64_t)b * p.geom.Hv + hv) * p.geom.T;
+
+    if (wave_id() >= 4) {
+        // ------------------------------- loader waves -------------------------------------------
+        const int tid = threadIdx.x - kThreads;
+        auto load = [&](int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            const int64_t row = head_row + start;
+            TileCopy<kThreads, kChunk, K> tw, tq, tk;
+            TileCopy<kThreads, kChunk, VS> tu;
+            TileCopy<kThreads, kChunk, kChunk> ta;
+            tw.fetch(p.w + row * K, K, len, tid);
+            tq.fetch(p.qg + row * K, K, len, tid);
+            tk.fetch(p.kg + row * K, K, len, tid);
+            tu.fetch(p.u + row * V + slab * VS, V, len, tid);
+            ta.fetch(p.aqk + row * kChunk, kChunk, len, tid);
+            float dec = 0.f;
+            if (tid < K) dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c) * p.geom.Hv + hv) * K + tid];
+            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pw, len, tid);
+            tq.commit(reinterpret_cast<bf16 *>(buf + L::q_off), pw, len, tid);
+            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pt, len, tid);
+            tu.commit(reinterpret_cast<bf16 *>(buf + L::u_off), pu, len, tid);
+            ta.commit(reinterpret_cast<bf16 *>(buf + L::a_off), pb, len, tid);
+            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = dec;
+        };
+        if (nchunks > 0) load(0);
+        __syncthreads();
+        for (int c = 0; c < nchunks; ++c) {
+            if (c + 1 < nchunks) load(c + 1);
+            __syncthreads();
+        }
+        return;
+    }
+
+    // --------------------------------- compute waves ---------------------------------------------
     const int wv = wave_id();
     const int l = lane_id(), li = l & 15, lg = l >> 4;
     const int vcol0 = slab * VS + wv * 16;
-
     f32x4 hacc[KT];
     auto state_off = [&](int kk, int v) -> int64_t { return p.v_first ? (int64_t)v * K + kk : (int64_t)kk * V + v; };
 #pragma unroll
@@ -409,22 +454,21 @@ __global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams 
         }
         hacc[kt] = a;
     }
-
-    const int64_t head_row = ((int64_t)b * p.geom.Hv + hv) * p.geom.T;
-    bf16 *og = static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + slab * VS;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
+    char *og = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
+    __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
+        const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
+        const bf16 *qS = reinterpret_cast<const bf16 *>(buf + L::q_off);
+        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
+        const bf16 *uS = reinterpret_cast<const bf16 *>(buf + L::u_off);
+        const bf16 *aS = reinterpret_cast<const bf16 *>(buf + L::a_off);
+        const float *dS = reinterpret_cast<const float *>(buf + L::d_off);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
         const int64_t row = head_row + start;
-        __syncthreads();
-        load_tile<kThreads>(wS, pw, p.w + row * K, K, kChunk, K, len);
-        load_tile<kThreads>(qS, pw, p.qg + row * K, K, kChunk, K, len);
-        load_tile<kThreads>(kS, pt, p.kg + row * K, K, kChunk, K, len);
-        load_tile<kThreads>(uS, pu, p.u + row * V + slab * VS, V, kChunk, VS, len);
-        load_tile<kThreads>(aS, pb, p.aqk + row * kChunk, kChunk, kChunk, kChunk, len);
-        if (threadIdx.x < K) dS[threadIdx.x] = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c) * p.geom.Hv + hv) * K + threadIdx.x];
-        __syncthreads();
 
         bf16x8 hB[KS];
 #pragma unroll
@@ -458,8 +502,9 @@ __global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams 
             }
         }
         if (p.v_new) {
+            char *vg = reinterpret_cast<char *>(p.v_new + row * V + vcol0);
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
+            for (int rt = 0; rt < 4; ++rt) acc_to_global(vg, (int64_t)V * 2, rt * 16, len, vn[rt]);
         }
         // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same bf16 v_new operand serves both)
         bf16x8 vB[2];
@@ -476,12 +521,10 @@ __global__ void __launch_bounds__(kThreads) kda_scan_kernel(const KdaScanParams 
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 32 * j), vB[j], hacc[kt]);
-        __syncthreads();   // w tile consumed by every wave, v_new tile complete
+        char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) acc_to_tile(wS, po, rt * 16, wv * 16, oacc[rt]);
-        if (p.v_new) store_tile<kThreads>(p.v_new + row * V + slab * VS, V, uS, pu, VS, len);
+        for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
         __syncthreads();
-        store_tile<kThreads>(og + (int64_t)start * p.o.st, p.o.st, wS, po, VS, len);
     }
 
     if (p.hT) {
@@ -558,11 +601,10 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
 
 template <int K>
 int launch_scan(const KdaScanParams &p, hipStream_t stream) {
-    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (K + 16) + 80 + 72)) * 2 + K * 4;
+    const size_t smem = ScanSmem<K>::bytes;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(kThreads), smem,
-               stream, p);
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }

@@ -75,16 +75,55 @@ __device__ __forceinline__ int acc_col() { return lane_id() & 15; }
 // ---- cooperative global <-> LDS tile copies (all threads of the block) -----------
 // Copies rows [0, valid) x cols [0, ncols) of a row-major global matrix (row stride
 // `gstride` elements, 16-byte aligned rows) into `tile`; rows [valid, nrows) are zeroed.
+// A tile copy is split into fetch (global -> registers) and commit (registers -> LDS) so that a caller
+// can issue the loads of all its tiles before the first commit waits for any of them.  Rows past
+// `valid` re-read the last valid row and are zeroed by a select: a predicated load would be waited for
+// inside its own branch, one memory round trip per piece.  `tid` is the thread's index among the
+// THREADS threads that copy; NROWS x NCOLS must be a multiple of 8 * THREADS.
+template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
+    static constexpr int CPR = NCOLS / 8;                    // 16-byte pieces per row
+    static constexpr int N = NROWS * CPR / THREADS;          // pieces per thread
+    static_assert(NROWS * CPR % THREADS == 0, "tile does not divide among the copying threads");
+    u32x4 r[N];
+    __device__ __forceinline__ void fetch(const bf16 *gsrc, int64_t gstride, int valid, int tid) {
+        const int last = valid > 0 ? valid - 1 : 0;
+#pragma unroll
+        for (int m = 0; m < N; ++m) {
+            const int idx = m * THREADS + tid;
+            const int row = idx / CPR, c = (idx % CPR) << 3;
+            r[m] = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)(row < valid ? row : last) * gstride + c);
+        }
+    }
+    __device__ __forceinline__ void commit(bf16 *tile, int pitch, int valid, int tid) const {
+#pragma unroll
+        for (int m = 0; m < N; ++m) {
+            const int idx = m * THREADS + tid;
+            const int row = idx / CPR, c = (idx % CPR) << 3;
+            *reinterpret_cast<u32x4 *>(tile + row * pitch + c) = row < valid ? r[m] : u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+};
+template <int THREADS>
+__device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsrc, int64_t gstride, int nrows,
+                                          int ncols, int valid, int tid) {
+    const int cpr = ncols >> 3;  // 16-byte chunks per row
+    const int total = nrows * cpr;
+    const int last = valid > 0 ? valid - 1 : 0;
+#pragma unroll
+    for (int idx0 = 0; idx0 < total; idx0 += THREADS) {
+        const int idx = idx0 + tid;
+        if (idx < total) {
+            const int r = idx / cpr, c = (idx % cpr) << 3;
+            u32x4 v = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)(r < valid ? r : last) * gstride + c);
+            if (r >= valid) v = u32x4{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4 *>(tile + r * pitch + c) = v;
+        }
+    }
+}
 template <int THREADS>
 __device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsrc, int64_t gstride, int nrows,
                                           int ncols, int valid) {
-    const int cpr = ncols >> 3;  // 16-byte chunks per row
-    for (int idx = threadIdx.x; idx < nrows * cpr; idx += THREADS) {
-        const int r = idx / cpr, c = (idx % cpr) << 3;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (r < valid) v = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)r * gstride + c);
-        *reinterpret_cast<u32x4 *>(tile + r * pitch + c) = v;
-    }
+    load_tile<THREADS>(tile, pitch, gsrc, gstride, nrows, ncols, valid, (int)threadIdx.x);
 }
 template <int THREADS>
 __device__ __forceinline__ void store_tile(bf16 *gdst, int64_t gstride, const bf16 *tile, int pitch, int ncols,
@@ -112,6 +151,23 @@ __device__ __forceinline__ void acc_to_tile(bf16 *tile, int pitch, int r0, int c
     bf16 *dst = tile + (r0 + 4 * lg + (odd ? 2 : 0)) * pitch + c0 + (li & ~1);
     *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);          // low halves
     *reinterpret_cast<unsigned *>(dst + pitch) = __builtin_amdgcn_perm(right, left, 0x07060302u);  // high halves
+}
+
+// One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with
+// `stride` bytes between rows; `base` points at column c0 of row 0).  Lane pairs exchange halves as in
+// acc_to_tile so that every lane writes two whole dwords.
+__device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
+    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
+    const bool odd = li & 1;
+    const unsigned send = odd ? p01 : p23;
+    const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+    const unsigned left = odd ? recv : p01, right = odd ? p23 : recv;
+    const int row = r0 + 4 * lg + (odd ? 2 : 0);
+    char *dst = base + row * stride + (li & ~1) * 2;
+    if (row < len) *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);
+    if (row + 1 < len) *reinterpret_cast<unsigned *>(dst + stride) = __builtin_amdgcn_perm(right, left, 0x07060302u);
 }
 
 // ---- the k tile -------------------------------------------------------------------------------
