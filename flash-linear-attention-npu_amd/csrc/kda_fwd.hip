@@ -269,61 +269,70 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
     const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
     const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
     const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
-    load_tile<kThreads>(qS, pq, qg, p.q.st, kChunk, K, len);
-    load_tile<kThreads>(kS, pk, kg, p.k.st, kChunk, K, len);
-    for (int idx = tid; idx < kChunk * (V / 8); idx += kThreads) {   // v * beta
-        const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
-        bf16x8 out;
-        if (r < len) {
-            const bf16x8 v8 = *reinterpret_cast<const bf16x8 *>(vg + (int64_t)r * p.v.st + c8);
-            const float br = load_scalar(p.beta, b, hv, start + r);
+    // gate loads first (thread = (token segment, channel)); branch-free with a clamped token index so that
+    // they are all in flight together with the tile loads below
+    const int64_t row_base = ((int64_t)b * p.geom.Hv + hv) * p.geom.T + start;   // head-major row of token 0
+    constexpr int TS = kChunk / SEG;
+    const int ch = tid % K, sg = tid / K;
+    float eig = 0.f, bias = 0.f;
+    if (p.use_gate) {
+        eig = __expf(p.a_log[hv]);
+        if (p.dt_bias) bias = p.dt_bias[(int64_t)hv * K + ch];
+    }
+    float raw[TS];
+    {
+        const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
+        if (p.g_bf16) {
+#pragma unroll
+            for (int j = 0; j < TS; ++j)
+                raw[j] = (float)static_cast<const bf16 *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
+        } else {
+#pragma unroll
+            for (int j = 0; j < TS; ++j)
+                raw[j] = static_cast<const float *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
+        }
+    }
+    {   // all loads of the chunk are issued before the first LDS write waits for one of them
+        TileCopy<kThreads, kChunk, K> tq, tk;
+        TileCopy<kThreads, kChunk, V> tv;
+        tq.fetch(qg, p.q.st, len, tid);
+        tk.fetch(kg, p.k.st, len, tid);
+        tv.fetch(vg, p.v.st, len, tid);
+        float br[TileCopy<kThreads, kChunk, V>::N];
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) {
+            const int r = (m * kThreads + tid) / (V / 8);
+            br[m] = load_scalar(p.beta, b, hv, start + min(r, len - 1));
+        }
+        tq.commit(qS, pq, len, tid);
+        tk.commit(kS, pk, len, tid);
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) {   // v * beta
+            const int idx = m * kThreads + tid;
+            const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
+            const bf16x8 v8 = __builtin_bit_cast(bf16x8, tv.r[m]);
+            const float bb = r < len ? br[m] : 0.f;
             f32x4 lo, hi;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                lo[e] = (float)v8[e] * br;
-                hi[e] = (float)v8[4 + e] * br;
+                lo[e] = (float)v8[e] * bb;
+                hi[e] = (float)v8[4 + e] * bb;
             }
-            out = frag_from_acc(lo, hi);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) out[e] = (bf16)0.f;
+            *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
         }
-        *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = out;
     }
     if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
 
-    // gate activation and prefix sum: thread = (token segment, channel)
-    const int64_t row_base = ((int64_t)b * p.geom.Hv + hv) * p.geom.T + start;   // head-major row of token 0
     {
-        constexpr int TS = kChunk / SEG;
-        const int ch = tid % K, sg = tid / K;
-        const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
-        float eig = 0.f, bias = 0.f;
-        if (p.use_gate) {
-            eig = __expf(p.a_log[hv]);
-            if (p.dt_bias) bias = p.dt_bias[(int64_t)hv * K + ch];
-        }
         float acc = 0.f;
-        for (int t0 = 0; t0 < TS; t0 += 8) {
-            float raw[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int t = sg * TS + t0 + j;
-                raw[j] = 0.f;
-                if (t < len) {
-                    const int64_t off = gbase + (int64_t)t * p.g_st;
-                    raw[j] = p.g_bf16 ? (float)static_cast<const bf16 *>(p.g)[off] : static_cast<const float *>(p.g)[off];
-                }
+        for (int j = 0; j < TS; ++j) {
+            const int t = sg * TS + j;
+            if (t < len) {
+                const float a = p.use_gate ? kda_activate(raw[j], bias, eig, p.safe_gate, p.lower_bound) : raw[j];
+                acc += a * kRcpLn2;
             }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int t = sg * TS + t0 + j;
-                if (t < len) {
-                    const float a = p.use_gate ? kda_activate(raw[j], bias, eig, p.safe_gate, p.lower_bound) : raw[j];
-                    acc += a * kRcpLn2;
-                }
-                gS[t * pg + ch] = acc;
-            }
+            gS[t * pg + ch] = acc;
         }
         tS[sg * K + ch] = acc;
         __syncthreads();
