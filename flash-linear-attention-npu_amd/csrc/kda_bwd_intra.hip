@@ -14,7 +14,7 @@
 // The golden's tolerance rules out bf16 operands, so the products run on the fp32 matrix pipe
 // (v_mfma_f32_16x16x4_f32).  One workgroup per (chunk, head); wave r owns row tile r: its "lower"
 // products contract over (r+1) tiles and its "upper" product over (4-r) tiles, five in total for
-// every wave.  Channels are processed in blocks of at most 128 so the fp32 gate tile fits in LDS.
+// every wave.  Channels are processed in blocks of 64 so that two workgroups fit in a CU's LDS.
 #include "gdn_common.h"
 #include "mfma_tiles.h"
 
@@ -60,22 +60,28 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
     const int l = lane_id(), li = l & 15, lg = l >> 4;
     const int K = p.geom.K;
 
-    {   // masked score gradients
+    {   // masked score gradients: branch-free loads (clamped row), all issued before the first LDS write
         const int64_t mbase = b * p.m_sb + h * p.m_sh + (int64_t)start * p.m_st;
-        for (int idx = tid; idx < kChunk * 16; idx += kThreads) {
+        f32x4 a[4], k4[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int idx = m * kThreads + tid;
+            const int r = min(idx >> 4, len - 1), c4 = (idx & 15) << 2;
+            a[m] = *reinterpret_cast<const f32x4 *>(p.daqk + mbase + (int64_t)r * p.m_st + c4);
+            k4[m] = *reinterpret_cast<const f32x4 *>(p.dakk + mbase + (int64_t)r * p.m_st + c4);
+        }
+        const float bt = tid < kChunk ? load_scalar(p.beta, b, h, start + min(tid, len - 1)) : 0.f;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const int idx = m * kThreads + tid;
             const int r = idx >> 4, c4 = (idx & 15) << 2;
-            f32x4 a = {0.f, 0.f, 0.f, 0.f}, k4 = a;
-            if (r < len) {
-                a = *reinterpret_cast<const f32x4 *>(p.daqk + mbase + (int64_t)r * p.m_st + c4);
-                k4 = *reinterpret_cast<const f32x4 *>(p.dakk + mbase + (int64_t)r * p.m_st + c4);
-            }
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (c4 + e > r) a[e] = k4[e] = 0.f;
-            *reinterpret_cast<f32x4 *>(aqS + r * pa + c4) = a;
-            *reinterpret_cast<f32x4 *>(akS + r * pa + c4) = k4;
+                if (c4 + e > r || r >= len) a[m][e] = k4[m][e] = 0.f;
+            *reinterpret_cast<f32x4 *>(aqS + r * pa + c4) = a[m];
+            *reinterpret_cast<f32x4 *>(akS + r * pa + c4) = k4[m];
         }
-        if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, h, start + tid) : 0.f;
+        if (tid < kChunk) bS[tid] = tid < len ? bt : 0.f;
     }
 
     const int r0 = 16 * wave_id();
@@ -86,21 +92,25 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
 
     for (int ch0 = 0; ch0 < K; ch0 += KC) {
         __syncthreads();
-        for (int idx = tid; idx < kChunk * (KC / 8); idx += kThreads) {
-            const int r = idx / (KC / 8), c8 = (idx % (KC / 8)) * 8;
-            u32x4 qv = {0u, 0u, 0u, 0u}, kv = qv;
-            if (r < len) {
-                qv = *reinterpret_cast<const u32x4 *>(p.q + base + (int64_t)r * p.st + ch0 + c8);
-                kv = *reinterpret_cast<const u32x4 *>(p.k + base + (int64_t)r * p.st + ch0 + c8);
+        {
+            TileCopy<kThreads, kChunk, KC> tq, tk;
+            tq.fetch(p.q + base + ch0, p.st, len, tid);
+            tk.fetch(p.k + base + ch0, p.st, len, tid);
+            constexpr int GN = kChunk * (KC / 4) / kThreads;
+            f32x4 gv[GN];
+#pragma unroll
+            for (int m = 0; m < GN; ++m) {   // padded rows repeat the last gate row
+                const int idx = m * kThreads + tid;
+                const int r = min(idx / (KC / 4), len - 1), c4 = (idx % (KC / 4)) * 4;
+                gv[m] = *reinterpret_cast<const f32x4 *>(p.gk + base + (int64_t)r * p.st + ch0 + c4);
             }
-            *reinterpret_cast<u32x4 *>(qS + r * pk + c8) = qv;
-            *reinterpret_cast<u32x4 *>(kS + r * pk + c8) = kv;
-        }
-        for (int idx = tid; idx < kChunk * (KC / 4); idx += kThreads) {   // padded rows repeat the last gate row
-            const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
-            const int rr = min(r, len - 1);
-            *reinterpret_cast<f32x4 *>(gS + r * pg + c4) =
-                *reinterpret_cast<const f32x4 *>(p.gk + base + (int64_t)rr * p.st + ch0 + c4);
+            tq.commit(qS, pk, len, tid);
+            tk.commit(kS, pk, len, tid);
+#pragma unroll
+            for (int m = 0; m < GN; ++m) {
+                const int idx = m * kThreads + tid;
+                *reinterpret_cast<f32x4 *>(gS + (idx / (KC / 4)) * pg + (idx % (KC / 4)) * 4) = gv[m];
+            }
         }
         __syncthreads();
         if (r0 >= len) continue;   // wave-uniform: this row tile holds no token
@@ -109,6 +119,15 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
         for (int nt = 0; nt < KC / 16; ++nt) {
             const int ch = 16 * nt + li;
             const float ca = gS[anchor * pg + ch];
+            // incoming gradients of this tile: requested now (clamped rows, no branch), consumed after the products
+            float pdq[4], pdk[4], pdg[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t off = base + (int64_t)min(r0 + 4 * lg + e, len - 1) * p.st + ch0 + ch;
+                pdq[e] = p.dq[off];
+                pdk[e] = p.dk[off];
+                pdg[e] = p.dg[off];
+            }
             f32x4 D1 = {0.f, 0.f, 0.f, 0.f}, D2 = D1, D3 = D1;
             for (int js = 0; js < nsteps_lo; ++js) {
                 const int j = 4 * js + lg;
@@ -133,9 +152,9 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
                     const float qi = (float)qS[i * pk + ch], ki = (float)kS[i * pk + ch];
                     const float bdl = bS[i] * dl;
                     const int64_t off = base + (int64_t)i * p.st + ch0 + ch;
-                    p.dq_o[off] = p.dq[off] + dqd;
-                    p.dk_o[off] = p.dk[off] + bdl + du;
-                    p.dg_o[off] = p.dg[off] + qi * dqd + ki * (bdl - du);
+                    p.dq_o[off] = pdq[e] + dqd;
+                    p.dk_o[off] = pdk[e] + bdl + du;
+                    p.dg_o[off] = pdg[e] + qi * dqd + ki * (bdl - du);
                     dbacc[e] += dl * ki;
                 }
             }
@@ -269,7 +288,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.m_sb = ib < 0 ? 0 : daqk->stride[ib];
     p.m_sh = daqk->stride[ih];
     p.m_st = daqk->stride[it];
-    return K == 64 ? launch_bwd_intra<64>(p, stream) : launch_bwd_intra<128>(p, stream);
+    return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }
 
 }  // namespace
