@@ -247,11 +247,23 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
     const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
     const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
     const bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
-    load_tile<kThreads>(qS, pq, qg, p.q.st, kChunk, K, len);
-    load_tile<kThreads>(kS, pq, kg, p.k.st, kChunk, K, len);
-    load_tile<kThreads>(vS, pv, vg, p.v.st, kChunk, V, len);
-    load_tile<kThreads>(hS, pv, hg, V, K, V, K);
-    if (threadIdx.x < kChunk) gS[threadIdx.x] = threadIdx.x < len ? load_scalar(p.g, b, hv, start + threadIdx.x) : 0.f;
+    {   // every load of the chunk is in flight before the first LDS write waits
+        const int tid = threadIdx.x;
+        TileCopy<kThreads, kChunk, K> tq, tk;
+        TileCopy<kThreads, kChunk, V> tv;
+        TileCopy<kThreads, K, V> th;
+        tq.fetch(qg, p.q.st, len, tid);
+        tk.fetch(kg, p.k.st, len, tid);
+        tv.fetch(vg, p.v.st, len, tid);
+        th.fetch(hg, V, K, tid);
+        float gv = 0.f;
+        if (tid < kChunk) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+        tq.commit(qS, pq, len, tid);
+        tk.commit(kS, pq, len, tid);
+        tv.commit(vS, pv, len, tid);
+        th.commit(hS, pv, K, tid);
+        if (tid < kChunk) gS[tid] = tid < len ? gv : 0.f;
+    }
     __syncthreads();
 
     const int w = wave_id();

@@ -32,16 +32,25 @@ struct ScanParams {
     int v_first;         // state blocks are [V][K] instead of [K][V]
 };
 
+template <int K, int CT> struct FwdHSmem {
+    static constexpr int VS = 64 * CT;
+    static constexpr int pw = K + 8, pk = K + 16, pu = VS + 16;
+    static constexpr size_t w_off = 0;
+    static constexpr size_t k_off = w_off + (size_t)kChunk * pw * 2;
+    static constexpr size_t u_off = k_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t g_off = u_off + (size_t)kChunk * pu * 2;
+    static constexpr size_t buf_bytes = g_off + (size_t)kChunk * 4;
+    static constexpr size_t bytes = 2 * buf_bytes;
+};
+
+// 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
+// c+1 into the other buffer; one barrier per chunk.  h, v_new and the final state leave from registers.
 template <int K, int CT>
-__global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
+__global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int VS = 64 * CT;           // V columns of this workgroup
-    constexpr int pw = K + 8, pk = K + 16, pu = VS + 16;
+    typedef FwdHSmem<K, CT> L;
+    constexpr int VS = L::VS, pw = L::pw, pk = L::pk, pu = L::pu;
     constexpr int KT = K / 16, KS = K / 32;
-    bf16 *wS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = wS + kChunk * pw;
-    bf16 *uS = kS + kChunk * pk;
-    float *gS = reinterpret_cast<float *>(uS + kChunk * pu);
 
     const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
@@ -54,6 +63,39 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
         chunk0 = p.geom.choff[n];
     }
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const bf16 *ug = static_cast<const bf16 *>(p.u.p) + b * p.u.sb + hv * p.u.sh + slab * VS;
+
+    if (wave_id() >= 4) {
+        // ------------------------------- loader waves -------------------------------------------
+        const int tid = threadIdx.x - kThreads;
+        auto load = [&](int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            TileCopy<kThreads, kChunk, K> tw, tk;
+            TileCopy<kThreads, kChunk, VS> tu;
+            tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
+            tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
+            tu.fetch(ug + (int64_t)start * p.u.st, p.u.st, len, tid);
+            float gv = 0.f;
+            if (tid < kChunk) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pw, len, tid);
+            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pk, len, tid);
+            tu.commit(reinterpret_cast<bf16 *>(buf + L::u_off), pu, len, tid);
+            if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
+        };
+        if (nchunks > 0) load(0);
+        __syncthreads();
+        for (int c = 0; c < nchunks; ++c) {
+            if (c + 1 < nchunks) load(c + 1);
+            __syncthreads();
+        }
+        return;
+    }
+
+    // --------------------------------- compute waves ---------------------------------------------
     const int wv = wave_id();
     const int l = lane_id(), li = l & 15, lg = l >> 4;
     const int vcol0 = slab * VS + wv * 16 * CT;  // first V column of this wave
@@ -73,21 +115,18 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
             }
             hacc[kt][ct] = a;
         }
-
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
-    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
-    const bf16 *ug = static_cast<const bf16 *>(p.u.p) + b * p.u.sb + hv * p.u.sh + slab * VS;
-    bf16 *vng = static_cast<bf16 *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + slab * VS;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
+    char *vng = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + vcol0);
+    __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
+        const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
+        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
+        const bf16 *uS = reinterpret_cast<const bf16 *>(buf + L::u_off);
+        const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
-        __syncthreads();  // previous chunk's tiles fully consumed
-        load_tile<kThreads>(wS, pw, wg + (int64_t)start * p.w.st, p.w.st, kChunk, K, len);
-        load_tile<kThreads>(kS, pk, kg + (int64_t)start * p.k.st, p.k.st, kChunk, K, len);
-        load_tile<kThreads>(uS, pu, ug + (int64_t)start * p.u.st, p.u.st, kChunk, VS, len);
-        if (threadIdx.x < kChunk) gS[threadIdx.x] = threadIdx.x < len ? load_scalar(p.g, b, hv, start + threadIdx.x) : 0.f;
-        __syncthreads();
 
         // state at chunk start as a bf16 operand (and as the emitted h)
         bf16x8 hB[KS][CT];
@@ -97,13 +136,22 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
             for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
         if (p.h) {
             bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+            if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+                for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
+                    for (int ct = 0; ct < CT; ++ct) {
+                        const bf16x8 f = hB[kt >> 1][ct];
+                        const bf16x4 q4 = (kt & 1) ? bf16x4{f[4], f[5], f[6], f[7]} : bf16x4{f[0], f[1], f[2], f[3]};
+                        *reinterpret_cast<bf16x4 *>(hg + (int64_t)(vcol0 + 16 * ct + li) * K + 16 * kt + 4 * lg) = q4;
+                    }
+            } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        hg[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)] = hB[kt >> 1][ct][(kt & 1) * 4 + e];
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct)
+                        acc_to_global(reinterpret_cast<char *>(hg + vcol0 + 16 * ct), (int64_t)V * 2, 16 * kt, K, hacc[kt][ct]);
+            }
         }
 
         // v_new = u - w h   (rows = tokens, columns = this wave's V columns)
@@ -129,11 +177,13 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) vn[rt][ct][e] = (float)uu[e] - vn[rt][ct][e];
             }
-        // emit v_new through this wave's own columns of the u tile
+        {
+            char *dst = vng + (int64_t)start * p.v_new.st * 2;
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt)
+            for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc_to_tile(uS, pu, rt * 16, (wv * CT + ct) * 16, vn[rt][ct]);
+                for (int ct = 0; ct < CT; ++ct) acc_to_global(dst + ct * 32, (int64_t)p.v_new.st * 2, rt * 16, len, vn[rt][ct]);
+        }
 
         // h <- e^{g_last} h + k^T (v_new e^{g_last - g}); padded rows carry zeros
         const float dec_all = __expf(g_last);
@@ -163,8 +213,7 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] = mfma16x32(afrag, vB[j][ct], hacc[kt][ct]);
             }
-        __syncthreads();  // v_new tile complete
-        store_tile<kThreads>(vng + (int64_t)start * p.v_new.st, p.v_new.st, uS, pu, VS, len);
+        __syncthreads();
     }
 
     if (p.hT) {
@@ -180,11 +229,10 @@ __global__ void __launch_bounds__(kThreads) fwd_h_kernel(const ScanParams p) {
 
 template <int K, int CT>
 int launch_fwd_h(const ScanParams &p, int slabs, hipStream_t stream) {
-    constexpr int VS = 64 * CT;
-    const size_t smem = ((size_t)kChunk * (K + 8) + (size_t)kChunk * (K + 16) + (size_t)kChunk * (VS + 16)) * 2 + kChunk * 4;
+    const size_t smem = FwdHSmem<K, CT>::bytes;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_h_kernel<K, CT>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("fwd_h", stream, (fwd_h_kernel<K, CT>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("fwd_h", stream, (fwd_h_kernel<K, CT>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
