@@ -40,11 +40,28 @@ __device__ __forceinline__ unsigned pack_bf16(float lo, float hi) {
 
 // ---- wave-level reductions (xor butterflies through ds_bpermute-free DPP where the
 // compiler can, __shfl_xor otherwise) ---------------------------------------
+// Sum over aligned groups of WIDTH lanes, result in every lane of the group.  Up to 16 lanes the
+// butterfly runs on data-parallel-primitive adds (quad swaps, then the two mirrors, which pair every
+// lane with one of the other half), 32 lanes add one LDS-crossbar swizzle (lane ^ 16); wider or odd
+// widths fall back to generic shuffles.
+#define FLA_DPP_XADD(v, ctrl) \
+    ((v) + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), 0xf, 0xf, true)))
 template <int WIDTH> __device__ __forceinline__ float group_sum(float v) {
+    if constexpr (WIDTH == 2 || WIDTH == 4 || WIDTH == 8 || WIDTH == 16 || WIDTH == 32) {
+        v = FLA_DPP_XADD(v, 0xB1);                          // quad_perm [1,0,3,2]
+        if constexpr (WIDTH >= 4) v = FLA_DPP_XADD(v, 0x4E);   // quad_perm [2,3,0,1]
+        if constexpr (WIDTH >= 8) v = FLA_DPP_XADD(v, 0x141);  // row_half_mirror
+        if constexpr (WIDTH >= 16) v = FLA_DPP_XADD(v, 0x140); // row_mirror
+        if constexpr (WIDTH == 32)
+            v += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));  // lane ^ 16
+        return v;
+    } else {
 #pragma unroll
-    for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+        for (int off = WIDTH / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+        return v;
+    }
 }
+#undef FLA_DPP_XADD
 
 // Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves: four
 // shifts inside each row of 16 lanes (sources outside the row read 0), then lane 15 of rows 0 / 2

@@ -3,10 +3,12 @@
 // streamed once in and once out per (sequence, head); all arithmetic is fp32
 // vector work with wave-level reductions, no MFMA.
 //
-// One 256-thread workgroup owns one (sequence, value head).  A state row (fixed
-// v, Dk contiguous floats) is spread over Dk/4 adjacent lanes, 4 floats each, so
-// every wave load/store instruction touches whole 512-byte (Dk=128) row
-// segments.  The tile stays in registers across the tokens of a sequence.
+// One 256-thread workgroup owns one (sequence, value head).  A state row (fixed v, Dk contiguous
+// floats) is spread over the 16 lanes of one DPP row, Dk/16 floats each in 16-byte pieces 64 columns
+// apart, so that every wave load/store instruction touches 256-byte row segments and the two
+// reductions per token (S k and S q) are four data-parallel-primitive adds each, with no LDS traffic.
+// The tile stays in registers across the tokens of a sequence; q/k/v of the next eight tokens are
+// loaded while the current eight are processed.
 // Semantics: recurrent_gated_delta_rule/README.md:6-33, tests/pta/golden.py:14-99,
 // kernel op_kernel/recurrent_gated_delta_rule.h:364-403.
 #include "common.h"
@@ -53,18 +55,28 @@ template <> struct StateIO<bf16> {
     static __device__ __forceinline__ void store(bf16 *p, f32x4 v) { *reinterpret_cast<bf16x4 *>(p) = cvt4(v); }
 };
 
-template <typename ST, int DK, int DV>
+template <typename ST, int DK, int DV, int LPR>
 __global__ void __launch_bounds__(kThreads) recurrent_gdn_kernel(const RecParams p) {
-    constexpr int LPR = DK / 4;               // lanes per state row
+    // LPR lanes per state row: 16 (one DPP row, reductions without LDS traffic) for multi-token sequences,
+    // Dk/4 (one 16-byte piece per lane, whole 512-byte rows per load instruction) for single-token decode
+    constexpr int SEGW = 4 * LPR;             // columns between the 16-byte pieces of a lane
+    constexpr int NSEG = DK / SEGW;           // pieces of a row per lane
     constexpr int RPW = kWave / LPR;          // rows per wave pass
     constexpr int RPP = RPW * (kThreads / kWave);  // rows per block pass
     constexpr int NP = DV / RPP;              // passes = rows per thread
-    static_assert(DV % RPP == 0, "tile does not divide");
+    static_assert(DV % RPP == 0 && DK % SEGW == 0 && NSEG >= 1, "tile does not divide");
+    constexpr int EQ = kTokBatch * DK / kThreads, EV = kTokBatch * DV / kThreads;   // staged elements per thread
+    static_assert(EQ >= 1 && EV >= 1 && DK % EQ == 0 && DV % EV == 0, "staging does not divide");
+    typedef bf16 vq_t __attribute__((ext_vector_type(EQ)));
+    typedef bf16 vv_t __attribute__((ext_vector_type(EV)));
+    typedef float fq_t __attribute__((ext_vector_type(EQ)));
 
-    __shared__ float s_k[kTokBatch][DK], s_q[kTokBatch][DK], s_gk[kTokBatch][DK];
-    __shared__ float s_v[kTokBatch][DV], s_o[kTokBatch][DV];
-    __shared__ float s_decay[kTokBatch], s_beta[kTokBatch];
-    __shared__ int s_slot[kTokBatch + 1];
+    // token batches are double-buffered: while batch b is consumed from one half, the loads of batch b+1
+    // are in flight and land in the other half
+    __shared__ __align__(16) float s_k[2][kTokBatch][DK], s_q[2][kTokBatch][DK], s_gk[2][kTokBatch][DK];
+    __shared__ __align__(16) float s_v[2][kTokBatch][DV], s_o[kTokBatch][DV];
+    __shared__ float s_decay[2][kTokBatch], s_beta[2][kTokBatch];
+    __shared__ int s_slot[2][kTokBatch + 1];
     __shared__ int s_red[kThreads / kWave];
 
     const int n = blockIdx.x / p.Nv;          // sequence
@@ -95,58 +107,98 @@ __global__ void __launch_bounds__(kThreads) recurrent_gdn_kernel(const RecParams
     if (src_slot < 0 || src_slot >= p.n_blocks) return;
 
     ST *state = static_cast<ST *>(p.state);
-    f32x4 S[NP];
+    f32x4 S[NP][NSEG];
     {
         const ST *sp = state + src_slot * p.s_sb + h * p.s_sh + col;
 #pragma unroll
-        for (int i = 0; i < NP; ++i) S[i] = StateIO<ST>::load(sp + (int64_t)(i * RPP + row0) * p.s_sv);
+        for (int i = 0; i < NP; ++i)
+#pragma unroll
+            for (int sg = 0; sg < NSEG; ++sg) S[i][sg] = StateIO<ST>::load(sp + (int64_t)(i * RPP + row0) * p.s_sv + SEGW * sg);
     }
 
-    for (int tb = 0; tb < len; tb += kTokBatch) {
+    // ---- staging: thread -> (token jq, columns cq..) of q/k/gk and (token jv, columns cv..) of v ----------
+    const int jq = tid * EQ / DK, cq = tid * EQ % DK;
+    const int jv = tid * EV / DV, cv = tid * EV % DV;
+    vq_t pre_q, pre_k;
+    vv_t pre_v;
+    fq_t pre_gk;
+    float pre_g = 0.f, pre_b = 0.f;
+    int pre_slot = -1;
+    auto fetch = [&](int tb) {   // branch-free: tokens past the batch re-read its last token
         const int nb = min(kTokBatch, len - tb);
-        __syncthreads();  // previous batch fully consumed
-        // ---- stage q, k, v, gates of up to kTokBatch tokens -------------------------
-        for (int idx = tid; idx < nb * DK; idx += kThreads) {
-            const int j = idx / DK, c = idx % DK;
-            const int64_t t = tok0 + tb + j;
-            s_k[j][c] = (float)p.k[t * p.k_st + hk * p.k_sh + c];
-            s_q[j][c] = (float)p.q[t * p.q_st + hk * p.q_sh + c] * p.scale;
-            if (p.gk) s_gk[j][c] = __expf(p.gk[t * p.gk_st + h * p.gk_sh + c]);
+        const int64_t tq = tok0 + tb + min(jq, nb - 1), tv = tok0 + tb + min(jv, nb - 1);
+        pre_q = *reinterpret_cast<const vq_t *>(p.q + tq * p.q_st + hk * p.q_sh + cq);
+        pre_k = *reinterpret_cast<const vq_t *>(p.k + tq * p.k_st + hk * p.k_sh + cq);
+        pre_v = *reinterpret_cast<const vv_t *>(p.v + tv * p.v_st + h * p.v_sh + cv);
+        if (p.gk) pre_gk = *reinterpret_cast<const fq_t *>(p.gk + tq * p.gk_st + h * p.gk_sh + cq);
+        if (tid <= kTokBatch) {
+            // entry nb is the look-ahead slot of the token after the batch (or -1 at the end of the sequence)
+            const int64_t t = tok0 + tb + min(tid, tb + nb < len ? nb : nb - 1);
+            pre_slot = p.slot_idx[t];
+            if (tid == nb && tb + nb >= len) pre_slot = -1;
+            const int64_t tg = tok0 + tb + min(tid, nb - 1);
+            if (p.g) pre_g = p.g[tg * p.g_st + h * p.g_sh];
+            pre_b = (float)p.beta[tg * p.b_st + h * p.b_sh];
         }
-        for (int idx = tid; idx < nb * DV; idx += kThreads) {
-            const int j = idx / DV, c = idx % DV;
-            const int64_t t = tok0 + tb + j;
-            s_v[j][c] = (float)p.v[t * p.v_st + h * p.v_sh + c];
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int e = 0; e < EQ; ++e) {
+            s_k[buf][jq][cq + e] = (float)pre_k[e];
+            s_q[buf][jq][cq + e] = (float)pre_q[e] * p.scale;
+            if (p.gk) s_gk[buf][jq][cq + e] = __expf(pre_gk[e]);
         }
-        if (tid < nb) {
-            const int64_t t = tok0 + tb + tid;
-            s_decay[tid] = p.g ? __expf(p.g[t * p.g_st + h * p.g_sh]) : 1.f;
-            s_beta[tid] = (float)p.beta[t * p.b_st + h * p.b_sh];
-            s_slot[tid] = p.slot_idx[t];
+#pragma unroll
+        for (int e = 0; e < EV; ++e) s_v[buf][jv][cv + e] = (float)pre_v[e];
+        if (tid <= kTokBatch) {
+            s_slot[buf][tid] = pre_slot;
+            if (tid < kTokBatch) {
+                s_decay[buf][tid] = p.g ? __expf(pre_g) : 1.f;
+                s_beta[buf][tid] = pre_b;
+            }
         }
-        if (tid == nb) s_slot[nb] = (tb + nb < len) ? p.slot_idx[tok0 + tb + nb] : -1;
-        __syncthreads();
+    };
+    fetch(0);
+    commit(0);
+    __syncthreads();
 
+    for (int tb = 0, buf = 0; tb < len; tb += kTokBatch, buf ^= 1) {
+        const int nb = min(kTokBatch, len - tb);
+        if (tb + kTokBatch < len) fetch(tb + kTokBatch);
         for (int j = 0; j < nb; ++j) {
-            const f32x4 kv = *reinterpret_cast<const f32x4 *>(&s_k[j][col]);
-            const f32x4 qv = *reinterpret_cast<const f32x4 *>(&s_q[j][col]);
-            f32x4 dec = {s_decay[j], s_decay[j], s_decay[j], s_decay[j]};
-            if (p.gk) dec *= *reinterpret_cast<const f32x4 *>(&s_gk[j][col]);
-            const float beta = s_beta[j];
+            f32x4 kv[NSEG], qv[NSEG], dec[NSEG];
+#pragma unroll
+            for (int sg = 0; sg < NSEG; ++sg) {
+                kv[sg] = *reinterpret_cast<const f32x4 *>(&s_k[buf][j][col + SEGW * sg]);
+                qv[sg] = *reinterpret_cast<const f32x4 *>(&s_q[buf][j][col + SEGW * sg]);
+                dec[sg] = f32x4{s_decay[buf][j], s_decay[buf][j], s_decay[buf][j], s_decay[buf][j]};
+                if (p.gk) dec[sg] *= *reinterpret_cast<const f32x4 *>(&s_gk[buf][j][col + SEGW * sg]);
+            }
+            const float beta = s_beta[buf][j];
             float sk[NP];
 #pragma unroll
             for (int i = 0; i < NP; ++i) {
-                S[i] *= dec;
-                sk[i] = S[i][0] * kv[0] + S[i][1] * kv[1] + S[i][2] * kv[2] + S[i][3] * kv[3];
+                float a = 0.f;
+#pragma unroll
+                for (int sg = 0; sg < NSEG; ++sg) {
+                    S[i][sg] *= dec[sg];
+                    a += S[i][sg][0] * kv[sg][0] + S[i][sg][1] * kv[sg][1] + S[i][sg][2] * kv[sg][2] + S[i][sg][3] * kv[sg][3];
+                }
+                sk[i] = a;
             }
 #pragma unroll
             for (int i = 0; i < NP; ++i) sk[i] = group_sum<LPR>(sk[i]);
             float so[NP];
 #pragma unroll
             for (int i = 0; i < NP; ++i) {
-                const float delta = beta * (s_v[j][i * RPP + row0] - sk[i]);
-                S[i] += delta * kv;
-                so[i] = S[i][0] * qv[0] + S[i][1] * qv[1] + S[i][2] * qv[2] + S[i][3] * qv[3];
+                const float delta = beta * (s_v[buf][j][i * RPP + row0] - sk[i]);
+                float a = 0.f;
+#pragma unroll
+                for (int sg = 0; sg < NSEG; ++sg) {
+                    S[i][sg] += delta * kv[sg];
+                    a += S[i][sg][0] * qv[sg][0] + S[i][sg][1] * qv[sg][1] + S[i][sg][2] * qv[sg][2] + S[i][sg][3] * qv[sg][3];
+                }
+                so[i] = a;
             }
 #pragma unroll
             for (int i = 0; i < NP; ++i) so[i] = group_sum<LPR>(so[i]);
@@ -156,19 +208,25 @@ __global__ void __launch_bounds__(kThreads) recurrent_gdn_kernel(const RecParams
             }
             // the state is visible after every token; a write is redundant only when the
             // next token of this sequence targets the same slot
-            const int slot = s_slot[j];
-            if (slot != s_slot[j + 1] && slot >= 0 && slot < p.n_blocks) {
+            const int slot = s_slot[buf][j];
+            if (slot != s_slot[buf][j + 1] && slot >= 0 && slot < p.n_blocks) {
                 ST *dp = state + slot * p.s_sb + h * p.s_sh + col;
 #pragma unroll
-                for (int i = 0; i < NP; ++i) StateIO<ST>::store(dp + (int64_t)(i * RPP + row0) * p.s_sv, S[i]);
+                for (int i = 0; i < NP; ++i)
+#pragma unroll
+                    for (int sg = 0; sg < NSEG; ++sg)
+                        StateIO<ST>::store(dp + (int64_t)(i * RPP + row0) * p.s_sv + SEGW * sg, S[i][sg]);
             }
         }
-        __syncthreads();
-        for (int idx = tid; idx < nb * DV; idx += kThreads) {
-            const int j = idx / DV, c = idx % DV;
-            const int64_t t = tok0 + tb + j;
-            p.out[t * p.o_st + h * p.o_sh + c] = (bf16)s_o[j][c];
+        __syncthreads();   // s_o complete, this half fully consumed
+        if (jv < nb) {
+            vv_t ov;
+#pragma unroll
+            for (int e = 0; e < EV; ++e) ov[e] = (bf16)s_o[jv][cv + e];
+            *reinterpret_cast<vv_t *>(p.out + (int64_t)(tok0 + tb + jv) * p.o_st + h * p.o_sh + cv) = ov;
         }
+        if (tb + kTokBatch < len) commit(buf ^ 1);
+        __syncthreads();   // next half staged, s_o free again
     }
 }
 
@@ -232,6 +290,18 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
     }
     if (T == 0 || B == 0) return FLA_OK;
 
+    // the per-batch staging reads q, k, v, gk and writes out in 16-byte pieces at most
+    {
+        const fla_tensor *vec[] = {query, key, value, out};
+        for (const fla_tensor *t : vec)
+            FLA_REQUIRE(t->stride[2] == 1 && t->stride[0] % 8 == 0 && t->stride[1] % 8 == 0 &&
+                            reinterpret_cast<uintptr_t>(t->data) % 16 == 0,
+                        FLA_ERR_SHAPE, "%s: query/key/value/out rows must be contiguous and 16-byte aligned.", op);
+        if (has_gk)
+            FLA_REQUIRE(gk->stride[2] == 1 && gk->stride[0] % 4 == 0 && gk->stride[1] % 4 == 0 &&
+                            reinterpret_cast<uintptr_t>(gk->data) % 16 == 0,
+                        FLA_ERR_SHAPE, "%s: gk rows must be contiguous and 16-byte aligned.", op);
+    }
     RecParams p{};
     p.q = static_cast<const bf16 *>(query->data);
     p.k = static_cast<const bf16 *>(key->data);
@@ -257,9 +327,17 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
 
     const dim3 grid((unsigned)(B * Nv)), block(kThreads);
     const bool f32s = state->dtype == FLA_F32;
-#define FLA_LAUNCH_REC(DK, DV)                                                                       \
-    if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<float, DK, DV>), grid, block, 0, stream, p);   \
-    else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<bf16, DK, DV>), grid, block, 0, stream, p)
+    // single-token decode is a pure stream of the state: widest rows per load; longer sequences are bound by
+    // the per-token reductions: 16-lane rows
+    const bool one_token = T <= B;
+#define FLA_LAUNCH_REC(DK, DV)                                                                                       \
+    if (one_token) {                                                                                                 \
+        if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<float, DK, DV, DK / 4>), grid, block, 0, stream, p); \
+        else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<bf16, DK, DV, DK / 4>), grid, block, 0, stream, p);       \
+    } else {                                                                                                         \
+        if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<float, DK, DV, 16>), grid, block, 0, stream, p);     \
+        else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<bf16, DK, DV, 16>), grid, block, 0, stream, p);           \
+    }
     if (Dk == 128 && Dv == 128) { FLA_LAUNCH_REC(128, 128); }
     else if (Dk == 64 && Dv == 64) { FLA_LAUNCH_REC(64, 64); }
     else if (Dk == 128 && Dv == 256) { FLA_LAUNCH_REC(128, 256); }
