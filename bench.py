@@ -202,6 +202,27 @@ def bench_decode(args, torch, dev):
         cdt = time.perf_counter() - t1
         cpu = {"value": round(ns * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
                "sample": f"{reps} x ({ns} sequences x 1 token, H=32 K=V=128) fp32 torch oracle, {cdt:.1f} s"}
+    # the same kernel as a variable-length prefill: 64 sequences, lengths uniform in [128, 4096]
+    gl = torch.Generator().manual_seed(0)
+    plens = torch.randint(128, 4097, (64,), generator=gl)
+    PT = int(plens.sum())
+    pq = F.normalize(torch.randn(PT, H, D, device=dev, generator=g), dim=-1).bfloat16()
+    pk = F.normalize(torch.randn(PT, H, D, device=dev, generator=g), dim=-1).bfloat16()
+    pv = torch.randn(PT, H, D, device=dev, generator=g).bfloat16()
+    pbeta = torch.sigmoid(torch.randn(PT, H, device=dev, generator=g)).bfloat16()
+    pgate = F.logsigmoid(torch.randn(PT, H, device=dev, generator=g))
+    pstate = torch.randn(64, H, D, D, device=dev, generator=g) * 0.01
+    pseq = torch.cat([torch.zeros(1, dtype=torch.int32), plens.to(torch.int32)]).to(dev)
+    pidx = torch.repeat_interleave(torch.arange(64, dtype=torch.int32), plens).to(dev)
+    prefill = lambda: ops.recurrent_gated_delta_rule(pq, pk, pv, pstate, beta=pbeta, scale=D ** -0.5,
+                                                     actual_seq_lengths=pseq, ssm_state_indices=pidx, g=pgate)
+    prefill()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(5):
+        prefill()
+    torch.cuda.synchronize()
+    pdt = (time.perf_counter() - t2) / 5
     return {
         "metric": "gdn_decode_tokens_per_s", "value": round(N * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
@@ -210,6 +231,8 @@ def bench_decode(args, torch, dev):
         "roofline": {"bound": "hbm", "kernel": "recurrent_gdn", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
                      "avg_kernel_ms": round(ms / n, 4)},
+        "varlen_prefill": {"sequences": 64, "tokens": PT, "ms": round(pdt * 1e3, 3),
+                           "tokens_per_s": round(PT / pdt, 1)},
         "cpu_baseline": cpu,
     }
 
