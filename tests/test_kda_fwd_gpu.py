@@ -167,3 +167,46 @@ def test_chunk_kda_fwd_errors(dev):
         ops.chunk_kda_fwd(*a, 0.1, 64, initial_state=torch.zeros(1, 2, 128, 64, device=dev))
     with pytest.raises(RuntimeError, match="only bfloat16"):
         ops.chunk_kda_fwd(*[t.half() if t.dtype == BF else t for t in a], 0.1, 64)
+
+
+def test_chunk_kda_fwd_state_handoff_and_determinism(dev):
+    """A sequence processed in one call equals the same sequence cut at a chunk boundary with the final
+    state handed over as initial state (bit for bit), and repeated calls are deterministic; the long
+    case is also held against the fp32 recurrence."""
+    from fla_hip import ops
+    B, T, H, K, V = 1, 1024, 4, 128, 128
+    q, k, v, g, beta = make_inputs(B, T, H, H, K, V, seed=21)
+    scale = K ** -0.5
+    x = [to_layout(t, "BSND").to(dev) for t in (q, k, v, g, beta)]
+    o, final = ops.chunk_kda_fwd(*x, scale, 64, output_final_state=True)[:2]
+    o_again, final_again = ops.chunk_kda_fwd(*x, scale, 64, output_final_state=True)[:2]
+    assert torch.equal(o, o_again) and torch.equal(final, final_again)
+    half = T // 2
+    a = [t[:, :half].contiguous() for t in x]
+    b = [t[:, half:].contiguous() for t in x]
+    o1, f1 = ops.chunk_kda_fwd(*a, scale, 64, output_final_state=True)[:2]
+    o2, f2 = ops.chunk_kda_fwd(*b, scale, 64, initial_state=f1, output_final_state=True)[:2]
+    assert torch.equal(torch.cat([o1, o2], dim=1), o) and torch.equal(f2, final)
+    nat = kda.kda_gate(g)
+    o_naive, f_naive = kda.naive_recurrent_kda(q, k, v, nat, beta, scale, output_final_state=True)
+    assert_close(from_layout(o, "BSND"), o_naive, TOL_BF16, "o vs recurrence, T=1024")
+    assert_close(final, f_naive, 4 * TOL_STATE, "final state vs recurrence, T=1024")
+
+
+def test_chunk_kda_fwd_packed_equals_separate(dev):
+    """A packed variable-length batch gives, sequence by sequence, exactly what separate calls give."""
+    from fla_hip import ops
+    cu = [0, 100, 100, 361, 425]
+    T, H, K, V = cu[-1], 2, 128, 128
+    q, k, v, g, beta = make_inputs(1, T, H, H, K, V, seed=5)
+    x = [to_layout(t, "TND").to(dev) for t in (q, k, v, g, beta)]
+    gen = torch.Generator().manual_seed(2)
+    h0 = (torch.randn(len(cu) - 1, H, K, V, generator=gen) * 0.1).to(dev)
+    o, final = ops.chunk_kda_fwd(*x, 0.1, 64, layout="TND", initial_state=h0, output_final_state=True, cu_seqlens=cu)[:2]
+    for n, (s, e) in enumerate(zip(cu, cu[1:])):
+        if s == e:
+            assert torch.equal(final[n], h0[n])          # an empty sequence hands its state through
+            continue
+        part = [t[s:e].contiguous() for t in x]
+        o_n, f_n = ops.chunk_kda_fwd(*part, 0.1, 64, layout="TND", initial_state=h0[n:n + 1], output_final_state=True)[:2]
+        assert torch.equal(o[s:e], o_n) and torch.equal(final[n], f_n[0])
