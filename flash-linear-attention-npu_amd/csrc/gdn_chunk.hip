@@ -82,12 +82,20 @@ __global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
     chunk_span(p.geom, b, c, seq, start, len);
     const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
     const int lane = threadIdx.x;
-    for (int idx = lane; idx < kChunk * 8; idx += 64) {
-        const int r = idx >> 3, c8 = (idx & 7) << 3;
-        bf16x8 v;
-        if (r < len) v = *reinterpret_cast<const bf16x8 *>(p.x + base + (int64_t)r * p.st + c8);
+    {   // branch-free loads (clamped row), all eight in flight before the first LDS write
+        bf16x8 v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) A[r][c8 + e] = (r < len && c8 + e < r) ? (float)v[e] : 0.f;
+        for (int m = 0; m < 8; ++m) {
+            const int idx = m * 64 + lane;
+            v[m] = *reinterpret_cast<const bf16x8 *>(p.x + base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3));
+        }
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const int idx = m * 64 + lane;
+            const int r = idx >> 3, c8 = (idx & 7) << 3;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) A[r][c8 + e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
+        }
     }
     __syncthreads();
 
@@ -124,7 +132,7 @@ struct WuParams {
     View3 g, beta;
 };
 
-__global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
+__global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int K = p.geom.K, V = p.geom.V;
     const int pa = kChunk + 8, pk = K + 16, pv = V + 16;
@@ -183,6 +191,100 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
             for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
         }
         *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = o;
+    }
+    __syncthreads();
+
+    // Each wave owns a quarter of the output columns of w and of u and overwrites
+    // exactly those columns of the staged operand once its products are done.
+    const int w = wave_id();
+    auto product = [&](bf16 *tile, int pitch, int ncols) {
+        const int per_wave = ncols / 64;  // 16-column tiles per wave
+        for (int m = 0; m < per_wave; ++m) {
+            const int c0 = (w * per_wave + m) * 16;
+            f32x4 acc[4];
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const bf16x8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);
+            }
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(tile, pitch, rt * 16, c0, acc[rt]);
+        }
+    };
+    product(kS, pk, K);
+    product(vS, pv, V);
+    __syncthreads();
+    bf16 *wg = static_cast<bf16 *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
+    bf16 *ug = static_cast<bf16 *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
+    store_tile<kThreads>(wg, p.w.st, kS, pk, K, len);
+    store_tile<kThreads>(ug, p.u.st, vS, pv, V, len);
+}
+
+// Compile-time head sizes: every load of the chunk (A, k, v tiles, gates) is issued before the first
+// LDS write waits for one of them.
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pa = kChunk + 8, pk = K + 16, pv = V + 16;
+    bf16 *aS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = aS + kChunk * pa;
+    bf16 *vS = kS + kChunk * pk;
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x;
+    const bf16 *ag = static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
+    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    {
+        TileCopy<kThreads, kChunk, kChunk> ta;
+        TileCopy<kThreads, kChunk, K> tk;
+        TileCopy<kThreads, kChunk, V> tv;
+        ta.fetch(ag, p.A.st, len, tid);
+        tk.fetch(kg, p.k.st, len, tid);
+        tv.fetch(vg, p.v.st, len, tid);
+        // per-row scale factors of the pieces this thread holds
+        float sk[TileCopy<kThreads, kChunk, K>::N], sv[TileCopy<kThreads, kChunk, V>::N];
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) {
+            const int r = min((m * kThreads + tid) / (K / 8), len - 1);
+            sk[m] = load_scalar(p.beta, b, hv, start + r) * __expf(load_scalar(p.g, b, hv, start + r));
+        }
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m)
+            sv[m] = load_scalar(p.beta, b, hv, start + min((m * kThreads + tid) / (V / 8), len - 1));
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, kChunk>::N; ++m) {   // columns past the tail are not part of the block
+            const int idx = m * kThreads + tid;
+            const int r = idx >> 3, c8 = (idx & 7) << 3;
+            bf16x8 a = __builtin_bit_cast(bf16x8, ta.r[m]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (!(r < len && c8 + e < len)) a[e] = (bf16)0.f;
+            *reinterpret_cast<bf16x8 *>(aS + r * pa + c8) = a;
+        }
+        auto scaled = [&](bf16 *dst, int pitch, int cpr, int m, u32x4 raw, float sc) {
+            const int idx = m * kThreads + tid;
+            const int r = idx / cpr, c8 = (idx % cpr) << 3;
+            const bf16x8 a = __builtin_bit_cast(bf16x8, raw);
+            const float f = r < len ? sc : 0.f;
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)a[e] * f;
+                hi[e] = (float)a[4 + e] * f;
+            }
+            *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
+        };
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) scaled(kS, pk, K / 8, m, tk.r[m], sk[m]);
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) scaled(vS, pv, V / 8, m, tv.r[m], sv[m]);
     }
     __syncthreads();
 
@@ -448,9 +550,19 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     WuParams p{geom, view4(k), view4(v), view4(A), view4(w), view4(u), view3(g), view3(beta)};
     const size_t smem = (size_t)kChunk * ((kChunk + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(wu_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)smem));
-    FLA_LAUNCH("wu", stream, wu_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+#define FLA_LAUNCH_WU(KERNEL)                                                                                      \
+    do {                                                                                                           \
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                          (int)smem));                                                             \
+        FLA_LAUNCH("wu", stream, KERNEL, grid, dim3(kThreads), smem, stream, p);                                    \
+    } while (0)
+    if (geom.K == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128>));
+    else if (geom.K == 128 && geom.V == 256) FLA_LAUNCH_WU((wu_kernel<128, 256>));
+    else if (geom.K == 64 && geom.V == 64) FLA_LAUNCH_WU((wu_kernel<64, 64>));
+    else if (geom.K == 64 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<64, 128>));
+    else FLA_LAUNCH_WU(wu_kernel_generic);
+#undef FLA_LAUNCH_WU
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
