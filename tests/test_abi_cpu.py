@@ -205,3 +205,111 @@ def test_cpu_tensors_are_rejected():
     x = torch.zeros(1, 4, 16, dtype=torch.bfloat16)
     with pytest.raises(TypeError, match="ROCm GPU tensor"):
         ops.causal_conv1d(x, torch.zeros(4, 16, dtype=torch.bfloat16))
+
+
+# ---------------------------------------------------------------------------------------------
+# KDA-side wrappers
+# ---------------------------------------------------------------------------------------------
+class FakeFloatTensor(FakeTensor):
+    device = "cuda:0"
+
+    def is_contiguous(self):
+        return True
+
+
+def test_kda_fwd_wrapper_operands_shapes_and_output_policy():
+    """Operand order of fla_chunk_kda_fwd (= aclnnChunkKdaFwd, _aclnn_ctypes.py:1230-1262) and the
+    12-value visibility mask (_kda_policy.py:16-39)."""
+    from fla_hip.ops import _hip_ctypes as H
+    B, T, Hk, HV, K, V = 2, 130, 2, 4, 128, 256
+    q = FakeTensor((B, T, Hk, K))
+    v = FakeTensor((B, T, HV, V))
+    g = FakeTensor((B, T, HV, K), torch.float32)
+    beta = FakeTensor((B, T, HV), torch.float32)
+    cap, out = capture_call(H.npu_chunk_kda_fwd, q, q, v, g, beta, 0.1, 64, output_final_state=True,
+                            disable_recompute=True, state_v_first=True)
+    assert cap["name"] == "chunk_kda_fwd"
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == [
+        "q", "k", "v", "g", "beta", "A_log", "dt_bias", "initial_state", "attn_out", "final_state", "gk", "Aqk", "Akk",
+        "w", "u", "qg", "kg", "v_new", "h"]
+    assert cap["args"][10].value == b"BSND" and cap["args"][12].value == 64 and cap["args"][16].value is True
+    o, final, gk, aqk, akk, w, u, qg, kg, v_new, h, init = out
+    assert o.shape == (B, T, HV, V) and final.shape == (B, HV, V, K) and final.dtype == torch.float32
+    assert gk.shape == (B, HV, T, K) and gk.dtype == torch.float32
+    assert aqk.shape == akk.shape == (B, HV, T, 64)
+    assert w.shape == qg.shape == kg.shape == (B, HV, T, K) and u.shape == v_new.shape == (B, HV, T, V)
+    assert h.shape == (B, 3, HV, V, K) and init is None
+    # rank-3 layouts, varlen chunk count, hidden outputs
+    cu = [0, 1, 66, 130]
+    q3, v3 = FakeTensor((Hk, T, K)), FakeTensor((HV, T, V))
+    g3, b3 = FakeTensor((HV, T, K), torch.float32), FakeTensor((HV, T), torch.float32)
+    cap, out = capture_call(H.npu_chunk_kda_fwd, q3, q3, v3, g3, b3, 0.1, layout="NTD", cu_seqlens=cu,
+                            return_intermediate_states=True)
+    assert out[0].shape == (HV, T, V) and out[10].shape == (4, HV, K, V) and out[1] is None and out[5] is None
+    assert H.kda_fwd_optional_output_mask(output_final_state=False, use_gate_in_kernel=True, disable_recompute=False,
+                                          return_intermediate_states=False) == (
+        True, False, False, True, True, False, False, False, False, False, False, True)
+
+
+@pytest.mark.parametrize("kwargs,match", [
+    (dict(layout="bsnd"), "layout must be uppercase"),
+    (dict(chunk_size=32), "chunk_size must be 64 or 128"),
+    (dict(layout="TND"), "rank does not match layout"),
+    (dict(use_gate_in_kernel=True), "A_log must be float32"),
+    (dict(cu_seqlens=[0, 70, 60, 130]), "cu_seqlens must be nondecreasing"),
+    (dict(cu_seqlens=[0, 130], chunk_indices=[0, 1, 0, 0, 0, 2]), "canonical sequence-major order"),
+    (dict(initial_state=FakeTensor((1, 2, 64, 128), torch.float32)), "initial_state shape/dtype"),
+])
+def test_kda_fwd_wrapper_rejects_bad_calls_before_launch(kwargs, match):
+    from fla_hip.ops import _hip_ctypes as H
+    q = FakeTensor((1, 130, 2, 128))
+    g = FakeTensor((1, 130, 2, 128), torch.float32)
+    beta = FakeTensor((1, 130, 2), torch.float32)
+    kw = dict(chunk_size=64)
+    kw.update(kwargs)
+    with pytest.raises(RuntimeError, match=match):
+        capture_call(H.npu_chunk_kda_fwd, q, q, q, g, beta, 0.1, **kw)
+
+
+def test_kda_gate_and_bwd_wrappers_operands():
+    from fla_hip.ops import _hip_ctypes as H
+    g = FakeTensor((1, 2, 130, 128), torch.float32)
+    cap, out = capture_call(H.npu_kda_gate_cumsum, g, 64, A_log=FakeTensor((2,), torch.float32), use_gate_in_kernel=True,
+                            safe_gate=True)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["g", "A_log", "dt_bias", "gk"]
+    assert cap["args"][7].value == -5.0 and out.dtype == torch.float32       # lower_bound default (_aclnn_ctypes.py:1292)
+
+    q = FakeTensor((1, 2, 130, 128))
+    dv = FakeTensor((1, 4, 130, 64))
+    gK = FakeTensor((1, 4, 130, 128), torch.float32)
+    cap, (dh, dh0, dv2) = capture_call(H.npu_chunk_gated_delta_rule_bwd_dhu, q, q, FakeTensor((1, 4, 130, 128)), dv, dv,
+                                       0.1, 64, gK=gK, h0=FakeTensor((1, 4, 128, 64), torch.float32), use_exp2=None)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["q", "k", "w", "d_o", "dv", "g", "gK", "h0", "dht", "dh", "dh0", "dv2"]
+    assert cap["args"][13].value is True                                     # use_exp2=None resolves to "gK given"
+    assert dh.shape == dh0.shape == (1, 4, 3, 128, 64) and dv2.shape == dv.shape
+    with pytest.raises(ValueError, match="Exactly one of g and gK"):
+        capture_call(H.npu_chunk_gated_delta_rule_bwd_dhu, q, q, q, dv, dv, 0.1, 64)
+    with pytest.raises(ValueError, match="use_exp2 must be true"):
+        capture_call(H.npu_chunk_gated_delta_rule_bwd_dhu, q, q, q, dv, dv, 0.1, 64, gK=gK, use_exp2=False)
+
+    T, Hh, K = 65, 3, 128
+    f32 = torch.float32
+    mk = lambda shape, dt=f32: FakeFloatTensor(shape, dt)
+    qk = mk((1, Hh, T, K), torch.bfloat16)
+    args = (qk, qk, mk((1, Hh, T, K)), mk((1, Hh, T), torch.bfloat16), mk((1, Hh, T, 64)), mk((1, Hh, T, 64)),
+            mk((1, Hh, T, K)), mk((1, Hh, T, K)), mk((1, Hh, T)), mk((1, Hh, T, K)))
+    cap, outs = capture_call(H.npu_chunk_kda_bwd_intra, *args, layout="BNSD")
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == [
+        "q", "k", "gk", "beta", "dAqk", "dAkk", "dq", "dk", "db", "dg", "dq_out", "dk_out", "db_out", "dg_out"]
+    assert cap["args"][13].value is True and cap["args"][14].value == b"BNSD"
+    assert [o.shape for o in outs] == [(1, Hh, T, K), (1, Hh, T, K), (1, Hh, T), (1, Hh, T, K)]
+    with pytest.raises(RuntimeError, match="safe_gate=False is reserved"):
+        capture_call(H.npu_chunk_kda_bwd_intra, *args, layout="BNSD", safe_gate=False)
+    with pytest.raises(RuntimeError, match="TND requires cu_seqlens"):
+        capture_call(H.npu_chunk_kda_bwd_intra, *[mk(t.shape[1:], t.dtype) for t in args], layout="TND")
+    with pytest.raises(RuntimeError, match="varlen supports TND or BSND"):
+        capture_call(H.npu_chunk_kda_bwd_intra, *args, layout="BNSD", cu_seqlens=[0, T])
