@@ -32,6 +32,20 @@ for _p in (str(ROOT), str(ROOT / "flash-linear-attention-npu_amd")):
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (scaled by the factors a plain copy of known size gives: x2.00 and x1.00).  The summaries with the exact
+# commands are the files named here; bench.py cannot collect hardware counters itself.
+MEASURED_TRAFFIC = {
+    "gdn_fused": (881e6 + 311e6, "profiles/gdn_pipe_kernel_B4_T8192_H32_K128_V128.md"),
+    "recurrent_gdn": (544e6 + 539e6, "profiles/recurrent_gdn_kernel_decode_256x32x128x128.md"),
+    "conv1d_fwd": (160e6 + 134e6, "profiles/conv1d_dense_kernel_B4_T4096_D4096_W4_silu.md"),
+}
+
+
+def measured_traffic(kernel):
+    v = MEASURED_TRAFFIC.get(kernel)
+    return (int(v[0]), v[1]) if v else (None, None)
+
 # Dense-tile FLOP count per token-head of the chunk forward (C=64, K=V=128):
 #   kkt, w, q.k^T = 3*C*K ; u, P.v_new = 2*C*V ; w.h, k^T.v_new, q.h = 3*K*V ; unit-lower inverse C^2/3
 def gdn_flops_per_token_head(C=64, K=128, V=128):
@@ -107,8 +121,10 @@ def bench_gdn(args, torch, dev):
     roofline = None
     if dominant in flops_of:
         ach = flops_of[dominant] / (kern[dominant] * 1e-3) / 1e12
+        traffic, src = measured_traffic(dominant)
         roofline = {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                    "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                    "traffic_source": src,
                     "avg_kernel_ms": round(kern[dominant], 4),
                     "all_kernels_ms": {n: round(t, 4) for n, t in kern.items()}}
     step_tflops = gdn_flops_per_token_head(C, K, V) * th / (ms_per_step * 1e-3) / 1e12
@@ -229,7 +245,8 @@ def bench_decode(args, torch, dev):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "GDN recurrent decode 256 sequences x 1 token, H=32 K=V=128, fp32 state in place"},
         "roofline": {"bound": "hbm", "kernel": "recurrent_gdn", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": measured_traffic("recurrent_gdn")[0],
+                     "traffic_source": measured_traffic("recurrent_gdn")[1],
                      "avg_kernel_ms": round(ms / n, 4)},
         "varlen_prefill": {"sequences": 64, "tokens": PT, "ms": round(pdt * 1e3, 3),
                            "tokens_per_s": round(PT / pdt, 1)},
@@ -288,7 +305,8 @@ def bench_conv1d(args, torch, dev):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "causal_conv1d fwd + SiLU B=4 T=4096 D=4096 width=4 + bias, zero left pad"},
         "roofline": {"bound": "hbm", "kernel": "conv1d_fwd", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": measured_traffic("conv1d_fwd")[0],
+                     "traffic_source": measured_traffic("conv1d_fwd")[1],
                      "avg_kernel_ms": round(ms / n, 4)},
         "cpu_baseline": cpu,
     }
