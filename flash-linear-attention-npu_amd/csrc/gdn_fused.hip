@@ -935,24 +935,21 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) U[rt] = *reinterpret_cast<const f32x4 *>(uS + ((wv * 4 + rt) * 64 + l) * 4);
             {   // v_new = u + (-w) h
-                bf16x8 wf[2][4];
+                // every operand read is in flight before the first product: their latency is paid once
+                bf16x8 wf[KS][4];
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt) wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
+                for (int j = 0; j < KS; ++j)
 #pragma unroll
-                for (int j = 0; j < KS; ++j) {
-                    const int cb = j & 1, nb = cb ^ 1;
-                    if (j + 1 < KS) {
+                    for (int rt = 0; rt < 4; ++rt) wf[j][rt] = frag_kc(wS, pw, rt * 16, 32 * j);
+                FLA_SCHED_FENCE();
 #pragma unroll
-                        for (int rt = 0; rt < 4; ++rt) wf[nb][rt] = frag_kc(wS, pw, rt * 16, 32 * (j + 1));
-                    }
-                    FLA_SCHED_FENCE();
+                for (int j = 0; j < KS; ++j)
 #pragma unroll
-                    for (int rt = 0; rt < 4; ++rt) U[rt] = mfma16x32(wf[cb][rt], hB[j], U[rt]);
-                    FLA_SCHED_FENCE();
-                }
+                    for (int rt = 0; rt < 4; ++rt) U[rt] = mfma16x32(wf[j][rt], hB[j], U[rt]);
+                FLA_SCHED_FENCE();
             }
             FLA_TICK(0)
-            bf16x8 kfa[KT];
+            bf16x8 kfa[KT], kfb[KT];
             f32x4 dk4[4];
             const float g_last = t.G[len - 1];
 #pragma unroll
@@ -961,7 +958,9 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 dk4[rt] = lds4(pipe_decay_table(t) + 16 * rt + 4 * lg);
             }
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) kfa[kt] = KTile<K>::tr(t.k, kt * 16, 0);
+            for (int kt = 0; kt < KT; ++kt) {
+                kfa[kt] = KTile<K>::tr(t.k, kt * 16, 0);
+            }
             FLA_SCHED_FENCE();
             // h <- e^{g_last} h + k^T (v_new e^{g_last - g}), the right operand as hi + lo bf16
             const float dec_all = __expf(g_last);
@@ -978,7 +977,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 vlo[j] = cat8(l0, l1);
             }
             {
-                bf16x8 kfb[KT];
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) kfb[kt] = KTile<K>::tr(t.k, kt * 16, 32);
                 FLA_SCHED_FENCE();

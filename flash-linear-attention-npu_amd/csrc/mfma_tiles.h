@@ -35,16 +35,13 @@ __device__ __forceinline__ bf16x4 lds_tr4(const bf16 *p) {
 
 // Operand with rows r0..r0+15 and contraction c0..c0+31 along the contiguous
 // dimension of `tile` (pitch in elements).
-// The second element offset is made opaque to the optimiser: fused into one two-address LDS read
-// (ds_read2_b64) the pair costs four times the LDS cycles of two single 8-byte reads on gfx950.
-__device__ __forceinline__ int opaque(int x) {
-    asm("" : "+v"(x));
-    return x;
-}
+// The two 8-byte halves stay separate LDS reads: fused into one two-address read (ds_read2_b64) the pair
+// costs four times the LDS cycles on gfx950, which is why this library is built with the load/store
+// merging pass of the backend switched off.
 __device__ __forceinline__ bf16x8 frag_kc(const bf16 *tile, int pitch, int r0, int c0) {
     const int l = lane_id(), i = l & 15, g = l >> 4;
     const int off = (r0 + i) * pitch + c0 + 4 * g;
-    return cat8(*reinterpret_cast<const bf16x4 *>(tile + off), *reinterpret_cast<const bf16x4 *>(tile + opaque(off + 16)));
+    return cat8(*reinterpret_cast<const bf16x4 *>(tile + off), *reinterpret_cast<const bf16x4 *>(tile + off + 16));
 }
 // 16-wide contraction variant for v_mfma_f32_16x16x16_bf16.
 __device__ __forceinline__ bf16x4 frag_kc4(const bf16 *tile, int pitch, int r0, int c0) {
@@ -188,7 +185,7 @@ template <int K> struct KTile {
     static __device__ __forceinline__ bf16x8 kc(const bf16 *t, int r0, int c0) {
         const int l = lane_id(), i = l & 15, g = l >> 4;
         return cat8(*reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 4 * g)),
-                    *reinterpret_cast<const bf16x4 *>(t + opaque(off(r0 + i, c0 + 16 + 4 * g))));
+                    *reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 16 + 4 * g)));
     }
     static __device__ __forceinline__ bf16x4 tr4(const bf16 *t, int r0, int c0) {
         const int l = lane_id(), i = l & 15, g = l >> 4;
