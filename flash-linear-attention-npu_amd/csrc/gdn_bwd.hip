@@ -1,0 +1,776 @@
+// Chunk-parallel stages of the gated-delta-rule BACKWARD, bf16 MFMA with fp32 accumulation, one
+// workgroup of four waves per chunk; wave w owns token rows 16w..16w+15 of every output:
+//   chunk_bwd_dv_local        dv = triu(k q^T e^{G_j-G_i}) scale . do
+//   chunk_bwd_dqkwg           dq, dk, dw and the gradient of the cumsummed gate from h, dh, v_new, do, dv
+//   prepare_wy_repr_bwd_da    gradient of the strictly-lower chunk matrix (stored transposed)
+//   prepare_wy_repr_bwd_full  dk, dv, dbeta, dg of w = A (k beta e^G), u = A (v beta)
+// Stage math: torch_custom/fla_npu/test/golden.py:18-172 (dv_local),
+// tests/atk/chunk_bwd_dqkwg/scripts/chunk_bwd_dqkwg_cpu.py:67-409 (dqkwg),
+// torch_custom/fla_npu/test/test_npu_prepare_wy_repr_bwd_da.py:170-282 (bwd_da),
+// torch_custom/fla_npu/test/test_npu_prepare_wy_repr_bwd_full.py:46-486 (bwd_full).
+// Operators with key-head outputs (dq, dk) loop over the value heads that share a key head inside one
+// workgroup, so grouped value heads need neither atomics nor a second pass.
+#include "gdn_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+// Stages `len` gate values of a chunk (clamped: rows past the tail repeat the last one) into LDS.
+__device__ __forceinline__ void stage_scalars(float *dst, const View3 &v, int b, int h, int start, int len) {
+    if (threadIdx.x < kChunk) dst[threadIdx.x] = load_scalar(v, b, h, start + min((int)threadIdx.x, len - 1));
+}
+
+// =============================================================================
+// chunk_bwd_dv_local
+// =============================================================================
+struct DvLocalParams {
+    ChunkGeom geom;
+    View4 q, k, d_o, dv;
+    View3 g;
+    float scale;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pk = K + 8, pv = V + 16, pa = kChunk + 8;
+    bf16 *qS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = qS + kChunk * pk;
+    bf16 *oS = kS + kChunk * pk;
+    bf16 *aS = oS + kChunk * pv;
+    float *gS = reinterpret_cast<float *>(aS + kChunk * pa);
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {
+        TileCopy<kThreads, kChunk, K> tq, tk;
+        TileCopy<kThreads, kChunk, V> to;
+        tq.fetch(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        to.fetch(static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        stage_scalars(gS, p.g, b, hv, start, len);
+        tq.commit(qS, pk, len, tid);
+        tk.commit(kS, pk, len, tid);
+        to.commit(oS, pv, len, tid);
+    }
+    __syncthreads();
+    // A[i][j] = <k_i, q_j> e^{G_j - G_i} scale for j >= i: row tile w, column tiles w..3
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct >= w) {
+#pragma unroll
+            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(kS, pk, 16 * w, 32 * j), frag_kc(qS, pk, 16 * ct, 32 * j), acc);
+            const int col = 16 * ct + li;
+            const float gc = gS[col];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                const float f = __expf(fminf(gc - gS[row], 0.f)) * p.scale;
+                acc[e] = (col >= row && col < len) ? acc[e] * f : 0.f;
+            }
+        }
+        acc_to_tile(aS, pa, 16 * w, 16 * ct, acc);
+    }
+    __syncthreads();
+    char *dvg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                         (int64_t)start * p.dv.st);
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) {
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (32 * j + 31 >= 16 * w) acc = mfma16x32(frag_kc(aS, pa, 16 * w, 32 * j), frag_tr(oS, pv, 16 * ct, 32 * j), acc);
+        acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+    }
+}
+
+// =============================================================================
+// chunk_bwd_dqkwg
+// =============================================================================
+struct DqkwgParams {
+    ChunkGeom geom;
+    View4 q, k, v, d_o, dv, dq, dk, dw;
+    View3 g;
+    const bf16 *h, *dh;
+    int64_t h_sb, h_sh, h_sc, dh_sb, dh_sh, dh_sc;
+    float *dg;
+    int64_t dg_sb, dg_sh, dg_st;
+    float scale;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
+    constexpr int KT = K / 16;
+    bf16 *qS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = qS + kChunk * pk;
+    bf16 *vS = kS + kChunk * pk;
+    bf16 *oS = vS + kChunk * pv;       // do
+    bf16 *dvS = oS + kChunk * pv;
+    bf16 *hS = dvS + kChunk * pv;      // h, then dh
+    bf16 *sS = hS + K * pv;            // ds
+    float *gS = reinterpret_cast<float *>(sS + kChunk * ps);
+    float *red = gS + kChunk;          // 8 partial sums
+
+    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int rep = p.geom.Hv / p.geom.Hk;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {
+        TileCopy<kThreads, kChunk, K> tq, tk;
+        tq.fetch(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        tq.commit(qS, pk, len, tid);
+        tk.commit(kS, pk, len, tid);
+    }
+    f32x4 dq_acc[KT], dk_acc[KT];
+#pragma unroll
+    for (int ct = 0; ct < KT; ++ct) dq_acc[ct] = dk_acc[ct] = zero4();
+
+    for (int r = 0; r < rep; ++r) {
+        const int hv = hk * rep + r;
+        if (r > 0) __syncthreads();      // the previous head's tiles are no longer read
+        TileCopy<kThreads, K, V> tdh;
+        float hd = 0.f;                  // this thread's share of sum(h . dh)
+        {
+            TileCopy<kThreads, kChunk, V> tv, to, tdv;
+            TileCopy<kThreads, K, V> th;
+            tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+            to.fetch(static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+            tdv.fetch(static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
+            tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
+            stage_scalars(gS, p.g, b, hv, start, len);
+            tv.commit(vS, pv, len, tid);
+            to.commit(oS, pv, len, tid);
+            tdv.commit(dvS, pv, len, tid);
+            th.commit(hS, pv, K, tid);
+#pragma unroll
+            for (int m = 0; m < TileCopy<kThreads, K, V>::N; ++m) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, th.r[m]), d = __builtin_bit_cast(bf16x8, tdh.r[m]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) hd += (float)a[e] * (float)d[e];
+            }
+        }
+        __syncthreads();
+        // ---- products with the state at chunk start: dq (state part), dw; and the ds tile -------------
+        f32x4 dqs[KT];
+        char *dwg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
+                                             (int64_t)start * p.dw.st);
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct) {
+            f32x4 a = zero4(), d = zero4();
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) {
+                const bf16x8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
+                a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
+                d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
+            }
+            dqs[ct] = a;
+            acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -d);
+        }
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            f32x4 acc = zero4();
+            if (ct <= w) {
+#pragma unroll
+                for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+                const int col = 16 * ct + li;
+                const float gc = gS[col];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = 16 * w + 4 * lg + e;
+                    const float f = __expf(fminf(gS[row] - gc, 0.f)) * p.scale;
+                    acc[e] = (col <= row && row < len) ? acc[e] * f : 0.f;
+                }
+            }
+            acc_to_tile(sS, ps, 16 * w, 16 * ct, acc);
+        }
+        __syncthreads();                 // every wave is done with h; ds is complete
+        tdh.commit(hS, pv, K, tid);
+        __syncthreads();
+        // ---- products with the state gradient, gate factors, intra-chunk parts -------------------------
+        const float g_last = gS[len - 1];
+        float grow[4], eq[4], ek[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            grow[e] = gS[16 * w + 4 * lg + e];
+            eq[e] = __expf(grow[e]) * p.scale;
+            ek[e] = __expf(g_last - grow[e]);
+        }
+        float dg_row[4] = {0.f, 0.f, 0.f, 0.f}, kdk_state = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct) {
+            f32x4 dks = zero4();
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) dks = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dks);
+            f32x4 dq = dqs[ct], dk;
+            float kv[4], qv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                kv[e] = (float)kS[row * pk + 16 * ct + li];
+                qv[e] = (float)qS[row * pk + 16 * ct + li];
+                dq[e] *= eq[e];
+                dk[e] = dks[e] * ek[e];
+                kdk_state += row < len ? dk[e] * kv[e] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (32 * j <= 16 * w + 15) dq = mfma16x32(frag_kc(sS, ps, 16 * w, 32 * j), frag_tr(kS, pk, 16 * ct, 32 * j), dq);
+                if (32 * j + 31 >= 16 * w) dk = mfma16x32(frag_tr(sS, ps, 16 * w, 32 * j), frag_tr(qS, pk, 16 * ct, 32 * j), dk);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dg_row[e] += dq[e] * qv[e] - dk[e] * kv[e];
+            dq_acc[ct] += dq;
+            dk_acc[ct] += dk;
+        }
+        // block sums for the gradient that lands on the last token of the chunk
+        float s1 = hd, s2 = kdk_state;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            s1 += __shfl_xor(s1, off, kWave);
+            s2 += __shfl_xor(s2, off, kWave);
+        }
+        if (l == 0) {
+            red[w] = s1;
+            red[4 + w] = s2;
+        }
+        __syncthreads();
+        const float dg_last = (red[0] + red[1] + red[2] + red[3]) * __expf(g_last) + red[4] + red[5] + red[6] + red[7];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float v = group_sum<16>(dg_row[e]);
+            const int row = 16 * w + 4 * lg + e;
+            if (li == 0 && row < len)
+                p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st] = v + (row == len - 1 ? dg_last : 0.f);
+        }
+    }
+    char *dqg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
+    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+#pragma unroll
+    for (int ct = 0; ct < KT; ++ct) {
+        acc_to_global(dqg + 32 * ct, p.dq.st * 2, 16 * w, len, dq_acc[ct]);
+        acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
+    }
+}
+
+// =============================================================================
+// prepare_wy_repr_bwd_da
+// =============================================================================
+struct WyBwdParams {
+    ChunkGeom geom;
+    View4 k, v, A, dA, dw, du, dk, dv;
+    View3 g, beta;
+    float *dbeta, *dg;
+    int64_t db_sb, db_sh, db_st, dg_sb, dg_sh, dg_st;
+};
+
+// Commits a fetched tile with every row scaled by f[row] (rows past `len` become zero).
+template <int NCOLS>
+__device__ __forceinline__ void commit_scaled(const TileCopy<kThreads, kChunk, NCOLS> &t, bf16 *dst, int pitch, int len,
+                                              const float *f, int tid) {
+#pragma unroll
+    for (int m = 0; m < TileCopy<kThreads, kChunk, NCOLS>::N; ++m) {
+        const int idx = m * kThreads + tid;
+        const int r = idx / (NCOLS / 8), c8 = (idx % (NCOLS / 8)) << 3;
+        const bf16x8 a = __builtin_bit_cast(bf16x8, t.r[m]);
+        const float s = r < len ? f[r] : 0.f;
+        f32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo[e] = (float)a[e] * s;
+            hi[e] = (float)a[4 + e] * s;
+        }
+        *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
+    }
+}
+// Commits a 64 x 64 chunk matrix, zeroing rows and columns past the tail; with `colf` every column j is
+// also scaled by colf[j].
+__device__ __forceinline__ void commit_square(const TileCopy<kThreads, kChunk, kChunk> &t, bf16 *dst, int pitch, int len,
+                                              const float *colf, int tid) {
+#pragma unroll
+    for (int m = 0; m < TileCopy<kThreads, kChunk, kChunk>::N; ++m) {
+        const int idx = m * kThreads + tid;
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        bf16x8 a = __builtin_bit_cast(bf16x8, t.r[m]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const bool in = r < len && c8 + e < len;
+            a[e] = in ? (colf ? (bf16)((float)a[e] * colf[c8 + e]) : a[e]) : (bf16)0.f;
+        }
+        *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = a;
+    }
+}
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pk = K + 8, pv = V + 8, pa = kChunk + 8;
+    bf16 *dwS = reinterpret_cast<bf16 *>(smem);
+    bf16 *kS = dwS + kChunk * pk;
+    bf16 *duS = kS + kChunk * pk;
+    bf16 *vS = duS + kChunk * pv;
+    bf16 *aS = vS + kChunk * pv;
+    bf16 *m4S = aS + kChunk * pa;
+    bf16 *m5S = m4S + kChunk * pa;
+    float *gS = reinterpret_cast<float *>(m5S + kChunk * pa);
+    float *bS = gS + kChunk;
+    float *fS = bS + kChunk;           // beta e^G
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {
+        TileCopy<kThreads, kChunk, K> tdw, tk;
+        TileCopy<kThreads, kChunk, V> tdu, tv;
+        TileCopy<kThreads, kChunk, kChunk> ta;
+        tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        tdu.fetch(static_cast<const bf16 *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
+        tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+        ta.fetch(static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
+        if (tid < kChunk) {
+            const int t = start + min(tid, len - 1);
+            const float gg = load_scalar(p.g, b, hv, t), bb = load_scalar(p.beta, b, hv, t);
+            gS[tid] = gg;
+            bS[tid] = bb;
+            fS[tid] = bb * __expf(gg);
+        }
+        __syncthreads();
+        tdw.commit(dwS, pk, len, tid);
+        tdu.commit(duS, pv, len, tid);
+        commit_scaled<K>(tk, kS, pk, len, fS, tid);
+        commit_scaled<V>(tv, vS, pv, len, bS, tid);
+        commit_square(ta, aS, pa, len, nullptr, tid);
+    }
+    __syncthreads();
+    // M4 = strict_lower(dw (k beta e^G)^T + du (v beta)^T), row tile w
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct <= w) {
+#pragma unroll
+            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pk, 16 * w, 32 * j), frag_kc(kS, pk, 16 * ct, 32 * j), acc);
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(duS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+            const int col = 16 * ct + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                acc[e] = (col < row && row < len) ? acc[e] : 0.f;
+            }
+        }
+        acc_to_tile(m4S, pa, 16 * w, 16 * ct, acc);
+    }
+    __syncthreads();
+    // M5 = M4 A^T
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_kc(m4S, pa, 16 * w, 32 * j), frag_kc(aS, pa, 16 * ct, 32 * j), acc);
+        acc_to_tile(m5S, pa, 16 * w, 16 * ct, acc);
+    }
+    __syncthreads();
+    // (A^T M5)^T = M5^T A, gated, negated and masked; rows of this product are the stored rows
+    char *dag = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dA.p)) + b * p.dA.sb + hv * p.dA.sh +
+                                         (int64_t)start * p.dA.st);
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct >= w) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_tr(m5S, pa, 16 * w, 32 * j), frag_tr(aS, pa, 16 * ct, 32 * j), acc);
+            const int col = 16 * ct + li;     // i of the untransposed matrix
+            const float gc = gS[col];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;   // j of the untransposed matrix
+                acc[e] = (col > row && col < len) ? -acc[e] * __expf(fminf(gc - gS[row], 0.f)) : 0.f;
+            }
+        }
+        acc_to_global(dag + 32 * ct, p.dA.st * 2, 16 * w, len, acc);
+    }
+}
+
+// =============================================================================
+// prepare_wy_repr_bwd_full
+// =============================================================================
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pk = K + 16, pv = V + 16, pa = kChunk + 8;
+    constexpr int KT = K / 16, VT = V / 16;
+    bf16 *kS = reinterpret_cast<bf16 *>(smem);
+    bf16 *dwS = kS + kChunk * pk;
+    bf16 *duS = dwS + kChunk * pk;
+    bf16 *vS = duS + kChunk * pv;
+    bf16 *aS = vS + kChunk * pv;
+    bf16 *dS = aS + kChunk * pa;        // dA as stored
+    bf16 *dbS = dS + kChunk * pa;       // dA with column j scaled by beta_j
+    float *gS = reinterpret_cast<float *>(dbS + kChunk * pa);
+    float *bS = gS + kChunk;
+
+    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int rep = p.geom.Hv / p.geom.Hk;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {
+        TileCopy<kThreads, kChunk, K> tk;
+        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        tk.commit(kS, pk, len, tid);
+    }
+    f32x4 dk_acc[KT];
+#pragma unroll
+    for (int ct = 0; ct < KT; ++ct) dk_acc[ct] = zero4();
+
+    for (int r = 0; r < rep; ++r) {
+        const int hv = hk * rep + r;
+        if (r > 0) __syncthreads();
+        {
+            TileCopy<kThreads, kChunk, K> tdw;
+            TileCopy<kThreads, kChunk, V> tdu, tv;
+            TileCopy<kThreads, kChunk, kChunk> ta, td;
+            tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+            tdu.fetch(static_cast<const bf16 *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
+            tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+            ta.fetch(static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
+            td.fetch(static_cast<const bf16 *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
+            if (tid < kChunk) {
+                const int t = start + min(tid, len - 1);
+                gS[tid] = load_scalar(p.g, b, hv, t);
+                bS[tid] = load_scalar(p.beta, b, hv, t);
+            }
+            __syncthreads();
+            tdw.commit(dwS, pk, len, tid);
+            tdu.commit(duS, pv, len, tid);
+            tv.commit(vS, pv, len, tid);
+            commit_square(ta, aS, pa, len, nullptr, tid);
+            commit_square(td, dS, pa, len, nullptr, tid);
+            commit_square(td, dbS, pa, len, bS, tid);
+        }
+        __syncthreads();
+        float br[4], er[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            br[e] = bS[16 * w + 4 * lg + e];
+            er[e] = __expf(gS[16 * w + 4 * lg + e]);
+        }
+        float db_row[4] = {0.f, 0.f, 0.f, 0.f}, dg_row[4] = {0.f, 0.f, 0.f, 0.f};
+        const bf16x8 at0 = frag_tr(aS, pa, 16 * w, 0), at1 = frag_tr(aS, pa, 16 * w, 32);
+        char *dvg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                             (int64_t)start * p.dv.st);
+#pragma unroll
+        for (int ct = 0; ct < VT; ++ct) {      // A^T du
+            f32x4 acc = mfma16x32(at0, frag_tr(duS, pv, 16 * ct, 0), zero4());
+            acc = mfma16x32(at1, frag_tr(duS, pv, 16 * ct, 32), acc);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pv + 16 * ct + li];
+                acc[e] *= br[e];
+            }
+            acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+        }
+        const bf16x8 dt0 = frag_tr(dS, pa, 16 * w, 0), dt1 = frag_tr(dS, pa, 16 * w, 32);
+        const bf16x8 db0 = frag_kc(dbS, pa, 16 * w, 0), db1 = frag_kc(dbS, pa, 16 * w, 32);
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct) {
+            const bf16x8 k0 = frag_tr(kS, pk, 16 * ct, 0), k1 = frag_tr(kS, pk, 16 * ct, 32);
+            f32x4 p1 = mfma16x32(at0, frag_tr(dwS, pk, 16 * ct, 0), zero4());      // A^T dw
+            p1 = mfma16x32(at1, frag_tr(dwS, pk, 16 * ct, 32), p1);
+            f32x4 p2 = mfma16x32(dt0, k0, zero4());                                 // dA^T k
+            p2 = mfma16x32(dt1, k1, p2);
+            f32x4 q3 = mfma16x32(db0, k0, zero4());                                 // dA (k beta)
+            q3 = mfma16x32(db1, k1, q3);
+            f32x4 dk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float kv = (float)kS[(16 * w + 4 * lg + e) * pk + 16 * ct + li];
+                const float p1g = p1[e] * er[e];
+                dk[e] = q3[e] + (p2[e] + p1g) * br[e];
+                db_row[e] += (p2[e] + p1g) * kv;
+                dg_row[e] += (p1g * br[e] + br[e] * p2[e] - q3[e]) * kv;
+            }
+            dk_acc[ct] += dk;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float sb = group_sum<16>(db_row[e]), sg = group_sum<16>(dg_row[e]);
+            const int row = 16 * w + 4 * lg + e;
+            if (li == 0 && row < len) {
+                p.dbeta[b * p.db_sb + hv * p.db_sh + (int64_t)(start + row) * p.db_st] = sb;
+                p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st] = sg;
+            }
+        }
+    }
+    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+#pragma unroll
+    for (int ct = 0; ct < KT; ++ct) acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+#define FLA_BWD_DISPATCH(KERNEL, NAME, GRID, SMEM_EXPR, P)                                                              \
+    do {                                                                                                               \
+        const size_t smem__ = (SMEM_EXPR);                                                                             \
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                          (int)smem__));                                                               \
+        FLA_LAUNCH(NAME, stream, KERNEL, GRID, dim3(kThreads), smem__, stream, P);                                      \
+        FLA_HIP_CHECK(hipGetLastError());                                                                              \
+        return FLA_OK;                                                                                                 \
+    } while (0)
+
+int check_f32_bht(const char *op, const char *name, const fla_tensor *t, const ChunkGeom &g) {
+    int rc = check_tensor(t, op, name, 3, dt_bit(FLA_F32));
+    if (rc) return rc;
+    FLA_REQUIRE(t->shape[0] == g.B && t->shape[1] == g.Hv && t->shape[2] == g.T, FLA_ERR_SHAPE,
+                "%s: %s must be [%d,%d,%d].", op, name, g.B, g.Hv, g.T);
+    return FLA_OK;
+}
+
+int check_state5(const char *op, const char *name, const fla_tensor *h, const ChunkGeom &geom) {
+    int rc = check_tensor(h, op, name, 5, dt_bit(FLA_BF16));
+    if (rc) return rc;
+    FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
+                    h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 8 == 0 &&
+                    h->stride[1] % 8 == 0 && h->stride[0] % 8 == 0,
+                FLA_ERR_SHAPE, "%s: %s must be [B,Hv,NT=%d,K,V] with contiguous K x V blocks.", op, name, geom.NT);
+    return FLA_OK;
+}
+
+int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g,
+                  const fla_tensor *g_gamma, const fla_tensor *A, const fla_int_array *cu, const fla_int_array *ci,
+                  double scale, int64_t chunk_size, const fla_tensor *out, void *ws, uint64_t ws_size, hipStream_t stream,
+                  uint64_t *query) {
+    const char *op = "chunk_bwd_dv_local";
+    FLA_REQUIRE(g_gamma == nullptr || g_gamma->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: g_gamma is not supported.", op);
+    (void)A;   // accepted and unused, as in the reference kernel
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, d_o, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "out", out, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    DvLocalParams p{geom, view4(q), view4(k), view4(d_o), view4(out), view3(g), (float)scale};
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const int K = geom.K, V = geom.V;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (V + 16) + kChunk + 8)) * 2 + kChunk * 4;
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dv_local_kernel<128, 128>), "bwd_dv_local", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dv_local_kernel<64, 64>), "bwd_dv_local", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dv_local_kernel<64, 128>), "bwd_dv_local", grid, smem, p);
+    if (K == 128 && V == 256) FLA_BWD_DISPATCH((dv_local_kernel<128, 256>), "bwd_dv_local", grid, smem, p);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
+}
+
+int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+               const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
+               const fla_int_array *ci, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
+               bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
+               const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_bwd_dqkwg";
+    FLA_REQUIRE(g_gamma == nullptr || g_gamma->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: g_gamma is not supported.", op);
+    FLA_REQUIRE(!use_exp2, FLA_ERR_UNSUPPORTED, "%s: use_exp2 is not supported with a scalar gate.", op);
+    FLA_REQUIRE(!transpose_state_layout, FLA_ERR_UNSUPPORTED, "%s: transpose_state_layout is not supported.", op);
+    (void)w;   // the reference accepts w and does not read it
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dox", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dq", dq, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "dw", dw, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_f32_bht(op, "dg", dg, geom))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
+    if ((rc = check_state5(op, "h", h, geom))) return rc;
+    if ((rc = check_state5(op, "dh", dh, geom))) return rc;
+    if (query) return FLA_OK;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    DqkwgParams p{geom, view4(q), view4(k), view4(v), view4(d_o), view4(dv), view4(dq), view4(dk), view4(dw), view3(g),
+                  static_cast<const bf16 *>(h->data), static_cast<const bf16 *>(dh->data),
+                  h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
+                  static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
+    const dim3 grid(geom.NT, geom.Hk, geom.B);
+    const int K = geom.K, V = geom.V;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (V + 8) + kChunk + 8) + (size_t)K * (V + 8)) * 2 + (kChunk + 8) * 4;
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128>), "bwd_dqkwg", grid, smem, p);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
+}
+
+int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+                  const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, int64_t chunk_size, ChunkGeom &geom) {
+    int rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dw", dw, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "du", du, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    FLA_REQUIRE(g != nullptr && g->data != nullptr && beta != nullptr && beta->data != nullptr, FLA_ERR_NULL,
+                "%s: g and beta must be provided.", op);
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    return FLA_OK;
+}
+
+int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+                   const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu,
+                   const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dA, void *ws, uint64_t ws_size,
+                   hipStream_t stream, uint64_t *query) {
+    const char *op = "prepare_wy_repr_bwd_da";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
+    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, dt_bit(FLA_BF16)))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), View4{}, View4{}, view3(g),
+                  view3(beta), nullptr, nullptr, 0, 0, 0, 0, 0, 0};
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const int K = geom.K, V = geom.V;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8) + 3 * (kChunk + 8))) * 2 + 3 * kChunk * 4;
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da_kernel<128, 128>), "wy_bwd_da", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_da_kernel<64, 64>), "wy_bwd_da", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da_kernel<64, 128>), "wy_bwd_da", grid, smem, p);
+    if (K == 128 && V == 256) FLA_BWD_DISPATCH((wy_bwd_da_kernel<128, 256>), "wy_bwd_da", grid, smem, p);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
+}
+
+int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+                     const fla_tensor *dA, const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g,
+                     const fla_int_array *cu, const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk,
+                     const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size,
+                     hipStream_t stream, uint64_t *query) {
+    const char *op = "prepare_wy_repr_bwd_full";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
+    const int bf = dt_bit(FLA_BF16);
+    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if ((rc = check_f32_bht(op, "dbeta", dbeta, geom))) return rc;
+    if ((rc = check_f32_bht(op, "dg", dg, geom))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), view4(dk), view4(dv), view3(g),
+                  view3(beta), static_cast<float *>(dbeta->data), static_cast<float *>(dg->data),
+                  dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
+    const dim3 grid(geom.NT, geom.Hk, geom.B);
+    const int K = geom.K, V = geom.V;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 2 * (V + 16) + 3 * (kChunk + 8))) * 2 + 2 * kChunk * 4;
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128>), "wy_bwd_full", grid, smem, p);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
+}
+
+}  // namespace
+}  // namespace fla
+
+#define FLA_NULL_WS(op) \
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, op ": workspace_size must not be null.")
+
+extern "C" int fla_chunk_bwd_dv_local_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
+    const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_NULL_WS("chunk_bwd_dv_local");
+    return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0,
+                              nullptr, workspace_size);
+}
+extern "C" int fla_chunk_bwd_dv_local(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
+    const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace,
+                              workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_chunk_bwd_dqkwg_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
+    bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
+    const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_NULL_WS("chunk_bwd_dqkwg");
+    return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
+                           transpose_state_layout, dq, dk, dw, dg, nullptr, 0, nullptr, workspace_size);
+}
+extern "C" int fla_chunk_bwd_dqkwg(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
+    bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
+    const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
+                           transpose_state_layout, dq, dk, dw, dg, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_prepare_wy_repr_bwd_da_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dA, uint64_t *workspace_size) {
+    FLA_NULL_WS("prepare_wy_repr_bwd_da");
+    return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, nullptr, 0, nullptr,
+                               workspace_size);
+}
+extern "C" int fla_prepare_wy_repr_bwd_da(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dA, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace,
+                               workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}
+
+extern "C" int fla_prepare_wy_repr_bwd_full_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_NULL_WS("prepare_wy_repr_bwd_full");
+    return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 nullptr, 0, nullptr, workspace_size);
+}
+extern "C" int fla_prepare_wy_repr_bwd_full(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}

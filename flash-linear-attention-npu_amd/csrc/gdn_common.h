@@ -62,5 +62,9 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
 int check_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, int64_t D,
                int dtype_mask);
 int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T);
+// Validates cu_seqlens / chunk_indices, reports the workspace (query != null) or uploads the chunk table
+// into `workspace` and completes `geom` with the device pointers.
+int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query);
 
 }  // namespace fla

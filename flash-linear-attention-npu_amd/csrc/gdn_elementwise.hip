@@ -59,6 +59,28 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
     return FLA_OK;
 }
 
+int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query) {
+    int rc = build_varlen(vl, op, cu, ci, kChunk, geom.T);
+    if (rc) return rc;
+    FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
+    if (vl.enabled) {
+        geom.NT = vl.NT;
+        geom.N = vl.N;
+    }
+    if (query) {
+        *query = vl.bytes();
+        return FLA_OK;
+    }
+    FLA_REQUIRE(vl.bytes() == 0 || (workspace && workspace_size >= vl.bytes()), FLA_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes required.", op, vl.bytes());
+    if ((rc = upload_varlen(vl, workspace, stream))) return rc;
+    geom.cu = vl.d_cu;
+    geom.choff = vl.d_choff;
+    geom.tab = vl.d_tab;
+    return FLA_OK;
+}
+
 namespace {
 
 template <typename T> __device__ __forceinline__ float ld(const void *p, int64_t i) {

@@ -42,6 +42,11 @@ OP_ARGTYPES = {
     "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
+    "chunk_bwd_dv_local": [_T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
+    "chunk_bwd_dqkwg": [_T] * 8 + [_IA, _IA, _T, _T, ctypes.c_float, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool]
+                       + [_T] * 4,
+    "prepare_wy_repr_bwd_da": [_T] * 7 + [_IA, _IA, ctypes.c_int64, _T],
+    "prepare_wy_repr_bwd_full": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
 }
 
 
@@ -678,6 +683,99 @@ def npu_chunk_kda_bwd_intra(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_se
         ],
         outputs,
     )
+
+
+def _f32_like(t):
+    import torch
+
+    return _empty(_shape(t), t, dtype=torch.float32)
+
+
+def _as_dtype(out, like):
+    return out if out.dtype == like.dtype else out.to(like.dtype)
+
+
+def npu_chunk_bwd_dv_local(q, k, d_o, g, scale, chunk_size, *, g_gamma=None, A=None, cu_seqlens=None,
+                           chunk_indices=None):
+    """_aclnn_ctypes.py:397-427.  q, k [B,Hk,T,K]; d_o [B,Hv,T,V]; g [B,Hv,T] chunk-cumsummed."""
+    if g_gamma is not None:
+        raise NotImplementedError("npu_chunk_bwd_dv_local: g_gamma is not supported.")
+    out = _empty_like(d_o)
+    return _call_op(
+        "chunk_bwd_dv_local", OP_ARGTYPES["chunk_bwd_dv_local"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(d_o, "d_o"), ctx.tensor(g, "g"),
+            ctx.tensor(g_gamma, "g_gamma"), ctx.tensor(A, "A"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def npu_prepare_wy_repr_bwd_da(k, v, beta, A, dw, du, g, *, chunk_size, cu_seqlens=None, chunk_indices=None):
+    """_aclnn_ctypes.py:430-460.  Returns dA [B,Hv,T,C], stored transposed as the reference does."""
+    out = _empty_like(A)
+    return _call_op(
+        "prepare_wy_repr_bwd_da", OP_ARGTYPES["prepare_wy_repr_bwd_da"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"),
+            ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_int64(int(chunk_size)), ctx.tensor(out, "dA"),
+        ],
+        out,
+    )
+
+
+def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):
+    """_aclnn_ctypes.py:242-279.  Returns (dk, dv, dbeta, dg); dbeta and dg are computed in fp32 and
+    returned in the dtype of beta and g."""
+    dk = _empty_like(k)
+    dv = _empty_like(v)
+    dbeta = _f32_like(beta)
+    dg = _f32_like(g)
+    outputs = (dk, dv, dbeta, dg)
+    dk, dv, dbeta, dg = _call_op(
+        "prepare_wy_repr_bwd_full", OP_ARGTYPES["prepare_wy_repr_bwd_full"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"), ctx.tensor(dA, "dA"),
+            ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(dbeta, "dbeta"), ctx.tensor(dg, "dg"),
+        ],
+        outputs,
+    )
+    return dk, dv, _as_dtype(dbeta, beta), _as_dtype(dg, g)
+
+
+def npu_chunk_bwd_dqkwg(q, k, v, g, h, dox, dh, dv, chunk_size, *, cu_seqlens=None, chunk_indices=None, w=None,
+                        g_gamma=None, scale=None, use_exp2=None, transpose_state_layout=None):
+    """_aclnn_ctypes.py:463-510.  Returns (dq, dk [B,Hk,T,K], dw [B,Hv,T,K], dg [B,Hv,T]); ``v`` is v_new."""
+    if g_gamma is not None:
+        raise NotImplementedError("npu_chunk_bwd_dqkwg: g_gamma is not supported.")
+    q_shape = _shape(q)
+    value_num_heads = int(v.shape[1])
+    dq = _empty_like(q)
+    dk = _empty_like(k)
+    dw = _empty((q_shape[0], value_num_heads, q_shape[2], q_shape[3]), q)
+    dg = _f32_like(g)
+    outputs = (dq, dk, dw, dg)
+    dq, dk, dw, dg = _call_op(
+        "chunk_bwd_dqkwg", OP_ARGTYPES["chunk_bwd_dqkwg"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"), ctx.tensor(h, "h"),
+            ctx.tensor(dox, "dox"), ctx.tensor(dh, "dh"), ctx.tensor(dv, "dv"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctx.tensor(w, "w"), ctx.tensor(g_gamma, "g_gamma"),
+            ctypes.c_float(_optional_float(scale, 1.0)), ctypes.c_int64(int(chunk_size)),
+            ctypes.c_bool(_optional_bool(use_exp2, False)), ctypes.c_bool(_optional_bool(transpose_state_layout, False)),
+            ctx.tensor(dq, "dq"), ctx.tensor(dk, "dk"), ctx.tensor(dw, "dw"), ctx.tensor(dg, "dg"),
+        ],
+        outputs,
+    )
+    return dq, dk, dw, _as_dtype(dg, g)
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

@@ -7,8 +7,9 @@ Two routes produce the same results:
 * ``fused=False``: the reference's own composition of the six operators
   (cumsum -> kkt -> solve_tri -> recompute_w_u -> fwd_h -> fwd_o), which also returns the
   inverted chunk matrix ``A``.
-Forward only: inputs that require grad are rejected (the GDN backward operators are outside
-this library).
+The backward (``flash_chunk_gated_delta_rule_bwd``, examples/flash_gated_delta_rule.py:884-1008) is the
+reference's composition of the backward operators; ``flash_gated_delta_rule`` records it for autograd
+(``ChunkGatedDeltaRuleFunction``, examples/flash_gated_delta_rule.py:1026-1123) when an input requires grad.
 """
 from __future__ import annotations
 
@@ -55,6 +56,64 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
         (final if output_final_state else None)
 
 
+def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, do, dht, cu_seqlens=None,
+                                     chunk_size: int = 64):
+    """q,k,v [B,H,T,D] bf16; ``g`` the chunk-cumsummed gate and beta [B,T,H] (as the forward returned /
+    received them); ``A`` [B,H,T,C] the inverted chunk matrices or None (recomputed); do [B,T,H,V];
+    dht [N,H,K,V] fp32 or None.  Returns (dq, dk, dv [B,H,T,D], dbeta, dg [B,T,H] fp32, dh0 [N,H,K,V] fp32 or
+    None); dg is the gradient of the RAW gate.  Unlike the reference, the initial state and the final-state
+    gradient take part (the reference passes neither to its reverse scan and returns dh0 = None)."""
+    import torch
+
+    cu = _cu_list(cu_seqlens)
+    kw = dict(cu_seqlens=cu)
+    gh = g.transpose(1, 2).contiguous().float()
+    bh = beta.transpose(1, 2).contiguous().float()
+    if A is None:
+        A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
+        A = _ops.solve_tri(A.to(k.dtype), layout="bnsd", **kw)
+    w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
+    doh = do.transpose(1, 2).contiguous()
+    h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,
+                                                    output_final_state=False, chunk_size=chunk_size, **kw)
+    dv = _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
+    dh, dh0, dv = _ops.chunk_gated_delta_rule_bwd_dhu(q, k, w, doh, dv, scale, chunk_size, g=gh, h0=initial_state,
+                                                      dht=dht, dh0_per_sequence=True, **kw)
+    dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
+    dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
+    dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
+    dk = (dk.float() + dk2.float()).to(dk.dtype)
+    dg = _ops.chunk_local_cumsum(dg + dg2, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
+    return dq, dk, dv, db.transpose(1, 2).contiguous(), dg.transpose(1, 2).contiguous(), dh0
+
+
+def _autograd_function():
+    """Built on first use so that importing this module does not import torch."""
+    import torch
+
+    class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused):
+            gc, o, A, final = flash_chunk_gated_delta_rule_fwd(
+                q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused)
+            ctx.save_for_backward(q, k, v, gc, beta, A, initial_state)
+            ctx.scale, ctx.cu, ctx.chunk_size = scale, cu, chunk_size
+            ctx.dtypes = (g.dtype, beta.dtype)
+            return o, final
+
+        @staticmethod
+        def backward(ctx, do, dht):
+            q, k, v, gc, beta, A, initial_state = ctx.saved_tensors
+            dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
+                q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(), dht, ctx.cu, ctx.chunk_size)
+            return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None
+
+    return ChunkGatedDeltaRuleFunction
+
+
+_FUNCTION = None
+
+
 def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, initial_state=None,
                            output_final_state: bool = False, use_qk_l2norm_in_kernel: bool = False,
                            cu_seqlens=None, cu_seqlens_list=None, chunk_indices=None, chunk_indices_list=None,
@@ -91,8 +150,6 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
         raise ValueError(f"chunk_size must be a power of 2, got {chunk_size}.")
     if use_qk_l2norm_in_kernel:
         raise NotImplementedError("use_qk_l2norm_in_kernel is not implemented; pass normalised q and k.")
-    if any(isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta)) and torch.is_grad_enabled():
-        raise NotImplementedError("flash_gated_delta_rule: forward only; the GDN backward is not implemented.")
     cu = _cu_list(cu_seqlens if cu_seqlens is not None else cu_seqlens_list)
     if cu is not None:
         if q.shape[0] != 1:
@@ -105,6 +162,13 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
                 f"got initial_state.shape[0]={initial_state.shape[0]} and sequences={len(cu) - 1}.")
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    _, o, _, final = flash_chunk_gated_delta_rule_fwd(
-        q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused)
-    return o, final
+    needs_grad = torch.is_grad_enabled() and any(
+        isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta, initial_state))
+    if not needs_grad:
+        _, o, _, final = flash_chunk_gated_delta_rule_fwd(
+            q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused)
+        return o, final
+    global _FUNCTION
+    if _FUNCTION is None:
+        _FUNCTION = _autograd_function()
+    return _FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused)

@@ -337,6 +337,67 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
+/* ------------------------------------------------------------------------
+ * Gated-delta-rule backward chain (examples/flash_gated_delta_rule.py:884-1008).
+ * All activations head-first: q, k, dq, dk [B,Hk,T,K]; v, d_o, dv, du [B,Hv,T,V];
+ * w, dw [B,Hv,T,K] bf16; g (chunk-cumsummed) and beta [B,Hv,T] f32 or bf16;
+ * A, dA [B,Hv,T,C] bf16; h, dh [B,Hv,NT,K,V] bf16.  Hv may be a multiple of Hk:
+ * dq and dk are then summed over the value heads of a key head.
+ * ------------------------------------------------------------------------ */
+
+/* chunk_bwd_dv_local - replaces aclnnChunkBwdDvLocal (_aclnn_ctypes.py:397-427):
+ * out = triu(k q^T e^{G_j - G_i}) * scale . d_o per chunk.  g_gamma must be NULL; A is
+ * accepted and not read (as in the reference). */
+int fla_chunk_bwd_dv_local_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
+    const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *out, uint64_t *workspace_size);
+int fla_chunk_bwd_dv_local(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
+    const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream);
+
+/* chunk_bwd_dqkwg - replaces aclnnChunkBwdDqkwg (_aclnn_ctypes.py:463-510).  v is v_new of the
+ * forward scan, h the state at each chunk start, dh / dv the outputs of bwd_dhu; dg [B,Hv,T] f32 is the
+ * gradient of the cumsummed gate.  w and g_gamma must be NULL or are ignored as in the reference;
+ * use_exp2 and transpose_state_layout must be false. */
+int fla_chunk_bwd_dqkwg_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
+    bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
+    const fla_tensor *dg, uint64_t *workspace_size);
+int fla_chunk_bwd_dqkwg(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
+    bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
+    const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+
+/* prepare_wy_repr_bwd_da - replaces aclnnPrepareWyReprBwdDa (_aclnn_ctypes.py:430-460): gradient of
+ * the strictly-lower chunk matrix, stored TRANSPOSED (upper triangular) as the reference does. */
+int fla_prepare_wy_repr_bwd_da_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dA, uint64_t *workspace_size);
+int fla_prepare_wy_repr_bwd_da(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dA, void *workspace, uint64_t workspace_size, void *stream);
+
+/* prepare_wy_repr_bwd_full - replaces aclnnPrepareWyReprBwdFull (_aclnn_ctypes.py:242-279):
+ * dk [B,Hk,T,K], dv [B,Hv,T,V] bf16; dbeta, dg [B,Hv,T] f32; dA as written by bwd_da. */
+int fla_prepare_wy_repr_bwd_full_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size);
+int fla_prepare_wy_repr_bwd_full(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -85,7 +85,7 @@ def chunk_local_cumsum(g, chunk: int, *, cu_seqlens=None, reverse=False, scale=1
     ``g`` may have trailing feature dims ([B,H,T] or [B,H,T,K]); the scan runs
     over dim 2.  fp32 accumulation, then cast.
     """
-    gf = g.float()
+    gf = g if g.dtype == torch.float64 else g.float()   # fp64 only for truth runs
     out = torch.empty_like(gf)
     B, T = g.shape[0], g.shape[2]
     for b, _, _, s, e in chunk_spans(B, T, chunk, cu_seqlens):
@@ -119,7 +119,7 @@ def chunk_scaled_dot_kkt(k, g, beta, chunk: int = 64, *, cu_seqlens=None,
         dec = torch.exp(torch.clamp(gc[:, :, None] - gc[:, None, :], -50.0, 50.0))
         a = kk * dec * bf[b, :, s:e, None]
         A[b, :, s:e, :L] = torch.tril(a, -1)
-    return A.float()
+    return A if compute_dtype == torch.float64 else A.float()
 
 
 # ----------------------------------------------------------------------------

@@ -1,0 +1,183 @@
+"""Parity of the GDN backward operators (through the C ABI) against the CPU oracle, operator by operator
+on the same bf16 inputs, and of their composition against autograd through the per-token recurrence.
+Cases follow the reference's sweeps: dense, grouped value heads, ragged tails, packed variable-length
+batches with an empty sequence (test_npu_chunk_bwd_dv_local.py, test_npu_chunk_bwd_dqkwg.py,
+test_npu_prepare_wy_repr_bwd_da.py, test_npu_prepare_wy_repr_bwd_full.py)."""
+import pytest
+import torch
+
+from oracle import gdn, gdn_bwd
+from oracle.kda import chunk_gated_delta_rule_bwd_dhu as dhu_oracle
+from util import assert_close, err_stats, TOL_BF16
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+F = torch.nn.functional
+
+CASES = [
+    # B, T, Hv, Hk, K, V, cu_seqlens
+    (2, 128, 2, 2, 128, 128, None),
+    (1, 200, 4, 2, 128, 128, None),                     # grouped value heads + ragged tail
+    (1, 1, 1, 1, 128, 128, None),
+    (1, 65, 2, 2, 64, 64, None),
+    (1, 130, 2, 1, 64, 128, None),
+    (1, 261, 2, 1, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261]),   # lengths 1,15,17,0,63,64,101
+]
+
+
+def make(B, T, Hv, Hk, K, V, cu, seed):
+    """Forward quantities of one problem, every tensor rounded to the dtype the operators exchange."""
+    gen = torch.Generator().manual_seed(seed)
+    rn = lambda *s: torch.randn(*s, generator=gen)
+    q = F.normalize(rn(B, Hk, T, K), dim=-1).to(BF)
+    k = F.normalize(rn(B, Hk, T, K), dim=-1).to(BF)
+    v = rn(B, Hv, T, V).to(BF)
+    beta = torch.sigmoid(rn(B, Hv, T))
+    g = F.logsigmoid(rn(B, Hv, T))
+    N = B if cu is None else len(cu) - 1
+    h0 = rn(N, Hv, K, V) * 0.1
+    do = rn(B, Hv, T, V).to(BF)
+    dht = rn(N, Hv, K, V) * 0.1
+    G = gdn.chunk_local_cumsum(g, 64, cu_seqlens=cu)
+    A0 = gdn.chunk_scaled_dot_kkt(k, G, beta, 64, cu_seqlens=cu)
+    A = gdn.solve_tri(A0, cu_seqlens=cu, output_dtype=BF)
+    w, u = gdn.recompute_w_u_fwd(k, v, beta, A, 64, g=G, cu_seqlens=cu, output_dtype=BF)
+    h, v_new, _ = gdn.chunk_gated_delta_rule_fwd_h(k, w, u, G, initial_state=h0, chunk=64, cu_seqlens=cu, output_dtype=BF)
+    return dict(q=q, k=k, v=v, beta=beta, g=g, G=G, A=A, w=w, u=u, h=h, v_new=v_new, h0=h0, do=do, dht=dht)
+
+
+def to_dev(d, dev):
+    return {n: t.to(dev) for n, t in d.items()}
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_backward_operators_against_oracle(dev, case):
+    from fla_hip import ops
+    B, T, Hv, Hk, K, V, cu = case
+    scale = K ** -0.5
+    d = make(B, T, Hv, Hk, K, V, cu, seed=T + K)
+    x = to_dev(d, dev)
+    kw = dict(cu_seqlens=cu)
+
+    # chunk_bwd_dv_local
+    dv_l = ops.chunk_bwd_dv_local(x["q"], x["k"], x["do"], x["G"], scale, 64, **kw)
+    dv_l_ref = gdn_bwd.chunk_bwd_dv_local(d["q"], d["k"], d["do"], d["G"], scale, 64, output_dtype=torch.float32, **kw)
+    assert dv_l.dtype == BF and dv_l.shape == d["do"].shape
+    assert_close(dv_l, dv_l_ref, TOL_BF16, "dv_local")
+
+    # the reverse scan feeds the remaining operators (oracle values, rounded as exchanged)
+    dh_ref, dh0_ref, dv2_ref = dhu_oracle(d["q"], d["k"], d["w"], d["do"], dv_l_ref.to(BF), scale, 64, g=d["G"],
+                                          dht=d["dht"], **kw)
+    dh, dv2 = dh_ref.to(BF), dv2_ref.to(BF)
+
+    # chunk_bwd_dqkwg
+    dq, dk, dw, dg = ops.chunk_bwd_dqkwg(x["q"], x["k"], x["v_new"], x["G"], x["h"], x["do"], dh.to(dev), dv2.to(dev), 64,
+                                         scale=scale, **kw)
+    dq_r, dk_r, dw_r, dg_r = gdn_bwd.chunk_bwd_dqkwg(d["q"], d["k"], d["v_new"], d["G"], d["h"], d["do"], dh, dv2, scale, 64,
+                                                     output_dtype=torch.float32, **kw)
+    assert dq.shape == d["q"].shape and dk.shape == d["k"].shape and dw.shape == d["w"].shape and dg.shape == d["G"].shape
+    assert dg.dtype == torch.float32
+    assert_close(dq, dq_r, TOL_BF16, "dq")
+    assert_close(dk, dk_r, TOL_BF16, "dk")
+    assert_close(dw, dw_r, TOL_BF16, "dw")
+    # dg sums hundreds of bf16-rounded products of both signs: bound the error against the gradient's scale
+    st = err_stats(dg, dg_r)
+    assert st["rel_max"] <= TOL_BF16, f"dg: {st}"
+
+    # prepare_wy_repr_bwd_da: transposed (upper-triangular) storage, zero tail columns
+    dwb = dw_r.to(BF)
+    dA = ops.prepare_wy_repr_bwd_da(x["k"], x["v"], x["beta"], x["A"], dwb.to(dev), dv2.to(dev), x["G"], chunk_size=64, **kw)
+    dA_ref = gdn_bwd.prepare_wy_repr_bwd_da(d["k"], d["v"], d["beta"], d["A"], dwb, dv2, d["G"], 64,
+                                            output_dtype=torch.float32, **kw)
+    st = err_stats(dA, dA_ref)
+    assert st["rel_max"] <= TOL_BF16, f"dA: {st}"
+    a = dA.float().cpu()
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        blk = a[b, :, s:e]
+        assert float(torch.tril(blk[:, :, : e - s], 0).abs().max()) == 0.0
+        if e - s < 64:
+            assert float(blk[:, :, e - s:].abs().max()) == 0.0
+
+    # prepare_wy_repr_bwd_full
+    dAb = dA_ref.to(BF)
+    dk2, dv3, db, dg2 = ops.prepare_wy_repr_bwd_full(x["k"], x["v"], x["beta"], x["A"], dAb.to(dev), dwb.to(dev),
+                                                     dv2.to(dev), x["G"], 64, **kw)
+    dk2_r, dv3_r, db_r, dg2_r = gdn_bwd.prepare_wy_repr_bwd_full(d["k"], d["v"], d["beta"], d["A"], dAb, dwb, dv2, d["G"], 64,
+                                                                 output_dtype=torch.float32, **kw)
+    assert db.dtype == torch.float32 and dg2.dtype == torch.float32
+    assert_close(dv3, dv3_r, TOL_BF16, "dv")
+    for name, got, ref in (("dk2", dk2, dk2_r), ("dbeta", db, db_r), ("dg2", dg2, dg2_r)):
+        st = err_stats(got, ref)
+        assert st["rel_max"] <= TOL_BF16, f"{name}: {st}"
+
+
+@pytest.mark.parametrize("case", [CASES[1], CASES[5]])
+def test_backward_pipeline_against_recurrence_autograd(dev, case):
+    """The composed GPU backward against autograd (fp64) through the per-token recurrence on the same bf16
+    inputs: every gradient within 2e-2 of its own scale."""
+    from fla_hip import pipeline
+    B, T, Hv, Hk, K, V, cu = case
+    scale = K ** -0.5
+    d = make(B, T, Hv, Hk, K, V, cu, seed=77)
+    dd = torch.float64
+    leaf = {n: d[n].to(dd).requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
+    o, final = gdn.naive_recurrent_gated_delta_rule(leaf["q"], leaf["k"], leaf["v"], leaf["g"], leaf["beta"], scale,
+                                                    initial_state=leaf["h0"], output_final_state=True, cu_seqlens=cu,
+                                                    compute_dtype=dd)
+    ((o * d["do"].to(dd)).sum() + (final * d["dht"].to(dd)).sum()).backward()
+    x = to_dev(d, dev)
+    # pipeline layouts: g, beta [B,T,H]; do [B,T,H,V]
+    got = pipeline.flash_chunk_gated_delta_rule_bwd(
+        x["q"], x["k"], x["v"], x["G"].transpose(1, 2).contiguous(), x["beta"].transpose(1, 2).contiguous(), None, scale,
+        x["h0"], x["do"].transpose(1, 2).contiguous(), x["dht"], cu_seqlens=cu)
+    dq, dk, dv, db, dg, dh0 = got
+    want = dict(dq=leaf["q"].grad, dk=leaf["k"].grad, dv=leaf["v"].grad, db=leaf["beta"].grad.transpose(1, 2),
+                dg=leaf["g"].grad.transpose(1, 2), dh0=leaf["h0"].grad)
+    for name, t in (("dq", dq), ("dk", dk), ("dv", dv), ("db", db), ("dg", dg), ("dh0", dh0)):
+        st = err_stats(t, want[name])
+        assert st["rel_max"] <= TOL_BF16, f"{name}: {st}"
+
+
+def test_backward_linearity_at_full_head_size(dev):
+    """Size-independent property at the benchmark's head shape (T shortened): the backward is linear in
+    (do, dht), so gradients of a sum of two cotangents equal the sum of gradients up to bf16 rounding."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 1, 1024, 4, 128, 128
+    d = make(B, T, H, H, K, V, None, seed=3)
+    x = to_dev(d, dev)
+    gen = torch.Generator().manual_seed(9)
+    do2 = torch.randn(B, T, H, V, generator=gen).to(BF).to(dev)
+    do1 = x["do"].transpose(1, 2).contiguous()
+    args = (x["q"], x["k"], x["v"], x["G"].transpose(1, 2).contiguous(), x["beta"].transpose(1, 2).contiguous(), None,
+            K ** -0.5, x["h0"])
+    r1 = pipeline.flash_chunk_gated_delta_rule_bwd(*args, do1, x["dht"])
+    r2 = pipeline.flash_chunk_gated_delta_rule_bwd(*args, do2, None)
+    r12 = pipeline.flash_chunk_gated_delta_rule_bwd(*args, (do1.float() + do2.float()).to(BF), x["dht"])
+    for name, a, b2, c in zip(("dq", "dk", "dv", "db", "dg", "dh0"), r1, r2, r12):
+        st = err_stats(c, a.float() + b2.float())
+        assert st["rel_max"] <= TOL_BF16, f"{name}: {st}"
+
+
+def test_autograd_through_flash_gated_delta_rule(dev):
+    """loss.backward() through the pipeline entry (fused forward, composed backward) against fp64 autograd
+    through the recurrence."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 1, 150, 2, 128, 128
+    d = make(B, T, H, H, K, V, None, seed=11)
+    dd = torch.float64
+    leaf = {n: d[n].to(dd).requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
+    o, final = gdn.naive_recurrent_gated_delta_rule(leaf["q"], leaf["k"], leaf["v"], leaf["g"], leaf["beta"], K ** -0.5,
+                                                    initial_state=leaf["h0"], output_final_state=True, compute_dtype=dd)
+    ((o * d["do"].to(dd)).sum() + (final * d["dht"].to(dd)).sum()).backward()
+    x = to_dev(d, dev)
+    q, k, v = (x[n].clone().requires_grad_(True) for n in ("q", "k", "v"))
+    g = x["g"].transpose(1, 2).contiguous().requires_grad_(True)
+    beta = x["beta"].transpose(1, 2).contiguous().requires_grad_(True)
+    h0 = x["h0"].clone().requires_grad_(True)
+    o_g, fin_g = pipeline.flash_gated_delta_rule(q, k, v, g, beta, None, h0, True)
+    ((o_g.float() * x["do"].transpose(1, 2).float()).sum() + (fin_g * x["dht"]).sum()).backward()
+    want = dict(q=leaf["q"].grad, k=leaf["k"].grad, v=leaf["v"].grad, g=leaf["g"].grad.transpose(1, 2),
+                beta=leaf["beta"].grad.transpose(1, 2), h0=leaf["h0"].grad)
+    for name, t in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("h0", h0)):
+        st = err_stats(t.grad, want[name])
+        assert st["rel_max"] <= TOL_BF16, f"d{name}: {st}"
