@@ -6,7 +6,7 @@ bf16 in / fp32 accumulation and state, B=4, T=8192, H=32, K=V=128, chunk 64, fp3
 state, final state on.  One "step" is one pass of the whole chunk forward over that batch
 with inputs resident in HBM.  Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|decode|conv1d|kda]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gdn_chunk|gdn_bwd|decode|conv1d|kda]
 
 `roofline` describes the dominant kernel of the step: algorithmic FLOPs (or bytes) per launch
 divided by its average duration, measured with HIP events recorded on the launch stream by the
@@ -408,6 +408,96 @@ def bench_kda(args, torch, dev):
     }
 
 
+def bench_gdn_bwd(args, torch, dev):
+    """GDN chunk backward at the headline shape: the reference's composition of the backward operators
+    (recompute of A, w, u, h; dv_local; reverse scan; dqkwg; WY backward; reverse cumsum), one step = one
+    pass producing dq, dk, dv, dbeta, dg and dh0.  `roofline` describes the kernel that takes the most time."""
+    import fla_hip
+    from fla_hip import pipeline
+    from oracle import gdn as ogdn, gdn_bwd as obwd
+
+    lib = fla_hip.load_library()
+    B, T, H, K, V, C = 4, 8192, 32, 128, 128, 64
+    F = torch.nn.functional
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
+    q = F.normalize(rn(B, H, T, K), dim=-1).bfloat16()
+    k = F.normalize(rn(B, H, T, K), dim=-1).bfloat16()
+    v = rn(B, H, T, V).bfloat16()
+    beta = torch.sigmoid(rn(B, T, H))
+    gate = F.logsigmoid(rn(B, T, H))
+    h0 = rn(B, H, K, V) * 0.01
+    do = rn(B, T, H, V).bfloat16()
+    dht = rn(B, H, K, V) * 0.01
+    scale = K ** -0.5
+    G = fla_hip.ops.chunk_local_cumsum(gate.transpose(1, 2).contiguous(), C, head_first=True,
+                                       output_dtype=torch.float32).transpose(1, 2).contiguous()
+
+    def step():
+        return pipeline.flash_chunk_gated_delta_rule_bwd(q, k, v, G, beta, None, scale, h0, do, dht, chunk_size=C)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_enable(1)
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    kern = {name: ms / n for name, (n, ms) in profile_report(lib).items()}
+    th = B * T * H
+    flops_of = {  # dense-tile FLOPs per launch
+        "bwd_dv_local": 2 * (C * K + C * V) * th,
+        "bwd_dqkwg": 2 * (3 * K * V + C * V + 2 * C * K) * th,
+        "wy_bwd_da": 2 * (C * K + C * V + 2 * C * C) * th,
+        "wy_bwd_full": 2 * (3 * C * K + C * V) * th,
+        "bwd_dhu": 2 * (3 * K * V) * th,
+        "kkt": 2 * C * K * th, "solve_tri": 2 * (C * C // 3) * th, "wu": 2 * (C * K + C * V) * th,
+        "fwd_h": 2 * (2 * K * V) * th,
+    }
+    timed = {n: t for n, t in kern.items() if n in flops_of}
+    dominant = max(timed, key=timed.get)
+    ach = flops_of[dominant] / (kern[dominant] * 1e-3) / 1e12
+    step_flops = sum(flops_of[n] for n in timed)
+    cpu = None
+    if not args.no_cpu:
+        import torch as _t
+        cores = os.cpu_count() or 1
+        _t.set_num_threads(cores)
+        Ts = min(args.cpu_tokens, 2048)
+        d = ogdn.make_gdn_inputs(1, Ts, H, K, V, dtype=_t.bfloat16, seed=0, init_std=0.01, head_first_gates=True)
+        cdo = _t.randn(1, H, Ts, V).bfloat16()
+        t1 = time.perf_counter()
+        reps = 0
+        while reps == 0 or time.perf_counter() - t1 < args.cpu_seconds:
+            obwd.chunk_gated_delta_rule_bwd(d["q"], d["k"], d["v"], d["g"], d["beta"], scale, cdo,
+                                            initial_state=d["initial_state"], chunk=C)
+            reps += 1
+        cdt = time.perf_counter() - t1
+        cpu = {"value": round(Ts * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
+               "sample": f"{reps} x (B=1 T={Ts} H={H} K=V={K}) composed fp32 torch oracle backward, {cdt:.1f} s"}
+    assert all(bool(torch.isfinite(t.float()).all()) for t in out)
+    return {
+        "metric": "gdn_chunk_bwd_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "GDN chunk backward B=4 T=8192 H=32 K=V=128 chunk=64, initial state and final-state gradient"},
+        "step_tflops": round(step_flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "avg_kernel_ms": round(kern[dominant], 4),
+                     "all_kernels_ms": {n: round(t, 4) for n, t in kern.items()}},
+        "cpu_baseline": cpu,
+    }
+
+
 def bench_copy(args, torch, dev):
     """Calibration only (not a product kernel): a plain device-to-device copy of known size, used to
     scale the FETCH_SIZE / WRITE_SIZE counters and as the practical bandwidth ceiling of the box."""
@@ -436,7 +526,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "decode", "conv1d", "kda", "copy"])
+    ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "gdn_bwd", "decode", "conv1d", "kda", "copy"])
     ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -453,7 +543,7 @@ def main():
         print("bench.py: no GPU visible.", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
-    fn = {"gdn_chunk": bench_gdn, "decode": bench_decode, "conv1d": bench_conv1d, "kda": bench_kda, "copy": bench_copy}[args.workload]
+    fn = {"gdn_chunk": bench_gdn, "gdn_bwd": bench_gdn_bwd, "decode": bench_decode, "conv1d": bench_conv1d, "kda": bench_kda, "copy": bench_copy}[args.workload]
     print(json.dumps(fn(args, torch, dev)))
 
 

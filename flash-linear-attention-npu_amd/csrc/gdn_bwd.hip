@@ -107,7 +107,7 @@ struct DqkwgParams {
     float scale;
 };
 
-template <int K, int V>
+template <int K, int V, bool GVA>
 __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     float *red = gS + kChunk;          // 8 partial sums
 
     const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
-    const int rep = p.geom.Hv / p.geom.Hk;
+    const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
@@ -323,9 +323,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
     bf16 *duS = kS + kChunk * pk;
     bf16 *vS = duS + kChunk * pv;
     bf16 *aS = vS + kChunk * pv;
-    bf16 *m4S = aS + kChunk * pa;
-    bf16 *m5S = m4S + kChunk * pa;
-    float *gS = reinterpret_cast<float *>(m5S + kChunk * pa);
+    // the two intermediate 64 x 64 matrices reuse the dw and du tiles, which are dead by then: the kernel
+    // stays under half of a compute unit's LDS, so two workgroups overlap their load and compute phases
+    bf16 *m4S = dwS;
+    bf16 *m5S = duS;
+    float *gS = reinterpret_cast<float *>(aS + kChunk * pa);
     float *bS = gS + kChunk;
     float *fS = bS + kChunk;           // beta e^G
 
@@ -359,6 +361,7 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
     }
     __syncthreads();
     // M4 = strict_lower(dw (k beta e^G)^T + du (v beta)^T), row tile w
+    f32x4 m4[4];
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct) {
         f32x4 acc = zero4();
@@ -374,8 +377,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
                 acc[e] = (col < row && row < len) ? acc[e] : 0.f;
             }
         }
-        acc_to_tile(m4S, pa, 16 * w, 16 * ct, acc);
+        m4[ct] = acc;
     }
+    __syncthreads();   // every wave has read its dw / du rows: their tiles may be overwritten
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) acc_to_tile(m4S, pa, 16 * w, 16 * ct, m4[ct]);
     __syncthreads();
     // M5 = M4 A^T
 #pragma unroll
@@ -410,43 +416,44 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
 // =============================================================================
 // prepare_wy_repr_bwd_full
 // =============================================================================
-template <int K, int V>
-__global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams p) {
+// GVA: several value heads share the key head, dk is accumulated over them in registers; otherwise every
+// dk tile goes straight to memory and the column loop needs no accumulator array.
+template <int K, int V, bool GVA>
+__global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(const WyBwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int pk = K + 16, pv = V + 16, pa = kChunk + 8;
+    // du and dw share one tile (du is dead once A^T du is formed) and v, which is only read element-wise,
+    // is unpadded: the kernel stays under half of a compute unit's LDS and two workgroups share one
+    constexpr int KV = K > V ? K : V;
+    constexpr int pk = K + 16, px = KV + 16, pvv = V, pa = kChunk + 8;
     constexpr int KT = K / 16, VT = V / 16;
     bf16 *kS = reinterpret_cast<bf16 *>(smem);
-    bf16 *dwS = kS + kChunk * pk;
-    bf16 *duS = dwS + kChunk * pk;
-    bf16 *vS = duS + kChunk * pv;
-    bf16 *aS = vS + kChunk * pv;
+    bf16 *xS = kS + kChunk * pk;        // du, then dw
+    bf16 *vS = xS + kChunk * px;
+    bf16 *aS = vS + kChunk * pvv;
     bf16 *dS = aS + kChunk * pa;        // dA as stored
     bf16 *dbS = dS + kChunk * pa;       // dA with column j scaled by beta_j
     float *gS = reinterpret_cast<float *>(dbS + kChunk * pa);
     float *bS = gS + kChunk;
 
     const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
-    const int rep = p.geom.Hv / p.geom.Hk;
+    const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
-    {
-        TileCopy<kThreads, kChunk, K> tk;
-        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-        tk.commit(kS, pk, len, tid);
-    }
-    f32x4 dk_acc[KT];
+    TileCopy<kThreads, kChunk, K> tk;
+    tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+    f32x4 dk_acc[GVA ? KT : 1];
 #pragma unroll
-    for (int ct = 0; ct < KT; ++ct) dk_acc[ct] = zero4();
+    for (int ct = 0; ct < (GVA ? KT : 1); ++ct) dk_acc[ct] = zero4();
+    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
         if (r > 0) __syncthreads();
+        TileCopy<kThreads, kChunk, K> tdw;
         {
-            TileCopy<kThreads, kChunk, K> tdw;
             TileCopy<kThreads, kChunk, V> tdu, tv;
             TileCopy<kThreads, kChunk, kChunk> ta, td;
-            tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
             tdu.fetch(static_cast<const bf16 *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
             tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
             ta.fetch(static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
@@ -456,14 +463,16 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams
                 gS[tid] = load_scalar(p.g, b, hv, t);
                 bS[tid] = load_scalar(p.beta, b, hv, t);
             }
+            if (r == 0) tk.commit(kS, pk, len, tid);
             __syncthreads();
-            tdw.commit(dwS, pk, len, tid);
-            tdu.commit(duS, pv, len, tid);
-            tv.commit(vS, pv, len, tid);
+            tdu.commit(xS, px, len, tid);
+            tv.commit(vS, pvv, len, tid);
             commit_square(ta, aS, pa, len, nullptr, tid);
             commit_square(td, dS, pa, len, nullptr, tid);
             commit_square(td, dbS, pa, len, bS, tid);
         }
+        // dw is fetched only now, once the registers of the first batch are free; it lands during A^T du
+        tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
         __syncthreads();
         float br[4], er[4];
 #pragma unroll
@@ -477,22 +486,26 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams
                                              (int64_t)start * p.dv.st);
 #pragma unroll
         for (int ct = 0; ct < VT; ++ct) {      // A^T du
-            f32x4 acc = mfma16x32(at0, frag_tr(duS, pv, 16 * ct, 0), zero4());
-            acc = mfma16x32(at1, frag_tr(duS, pv, 16 * ct, 32), acc);
+            f32x4 acc = mfma16x32(at0, frag_tr(xS, px, 16 * ct, 0), zero4());
+            acc = mfma16x32(at1, frag_tr(xS, px, 16 * ct, 32), acc);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pv + 16 * ct + li];
+                db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pvv + 16 * ct + li];
                 acc[e] *= br[e];
             }
             acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        __syncthreads();                 // du has been consumed by every wave
+        tdw.commit(xS, px, len, tid);
+        __syncthreads();
         const bf16x8 dt0 = frag_tr(dS, pa, 16 * w, 0), dt1 = frag_tr(dS, pa, 16 * w, 32);
         const bf16x8 db0 = frag_kc(dbS, pa, 16 * w, 0), db1 = frag_kc(dbS, pa, 16 * w, 32);
 #pragma unroll
         for (int ct = 0; ct < KT; ++ct) {
             const bf16x8 k0 = frag_tr(kS, pk, 16 * ct, 0), k1 = frag_tr(kS, pk, 16 * ct, 32);
-            f32x4 p1 = mfma16x32(at0, frag_tr(dwS, pk, 16 * ct, 0), zero4());      // A^T dw
-            p1 = mfma16x32(at1, frag_tr(dwS, pk, 16 * ct, 32), p1);
+            f32x4 p1 = mfma16x32(at0, frag_tr(xS, px, 16 * ct, 0), zero4());        // A^T dw
+            p1 = mfma16x32(at1, frag_tr(xS, px, 16 * ct, 32), p1);
             f32x4 p2 = mfma16x32(dt0, k0, zero4());                                 // dA^T k
             p2 = mfma16x32(dt1, k1, p2);
             f32x4 q3 = mfma16x32(db0, k0, zero4());                                 // dA (k beta)
@@ -506,7 +519,9 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams
                 db_row[e] += (p2[e] + p1g) * kv;
                 dg_row[e] += (p1g * br[e] + br[e] * p2[e] - q3[e]) * kv;
             }
-            dk_acc[ct] += dk;
+            if constexpr (GVA) dk_acc[ct] += dk;
+            else acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk);
+            __builtin_amdgcn_sched_barrier(0);   // keeps the operand reads of later column tiles from piling up in registers
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -518,9 +533,10 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_full_kernel(const WyBwdParams
             }
         }
     }
-    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+    if constexpr (GVA) {
 #pragma unroll
-    for (int ct = 0; ct < KT; ++ct) acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
+        for (int ct = 0; ct < KT; ++ct) acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
+    }
 }
 
 // ---- host side ------------------------------------------------------------------------------------
@@ -621,9 +637,13 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
     const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (V + 8) + kChunk + 8) + (size_t)K * (V + 8)) * 2 + (kChunk + 8) * 4;
-    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128>), "bwd_dqkwg", grid, smem, p);
+    const bool gva = geom.Hv != geom.Hk;
+    if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, false>), "bwd_dqkwg", grid, smem, p);
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, true>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, false>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, true>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, false>), "bwd_dqkwg", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, true>), "bwd_dqkwg", grid, smem, p);
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
 }
 
@@ -660,7 +680,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
                   view3(beta), nullptr, nullptr, 0, 0, 0, 0, 0, 0};
     const dim3 grid(geom.NT, geom.Hv, geom.B);
     const int K = geom.K, V = geom.V;
-    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8) + 3 * (kChunk + 8))) * 2 + 3 * kChunk * 4;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8) + (kChunk + 8))) * 2 + 3 * kChunk * 4;
     if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da_kernel<128, 128>), "wy_bwd_da", grid, smem, p);
     if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_da_kernel<64, 64>), "wy_bwd_da", grid, smem, p);
     if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da_kernel<64, 128>), "wy_bwd_da", grid, smem, p);
@@ -691,10 +711,14 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
-    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 2 * (V + 16) + 3 * (kChunk + 8))) * 2 + 2 * kChunk * 4;
-    if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128>), "wy_bwd_full", grid, smem, p);
+    const size_t smem = ((size_t)kChunk * ((K + 16) + ((K > V ? K : V) + 16) + V + 3 * (kChunk + 8))) * 2 + 2 * kChunk * 4;
+    const bool gva = geom.Hv != geom.Hk;
+    if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128, false>), "wy_bwd_full", grid, smem, p);
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128, true>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64, false>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64, true>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, false>), "wy_bwd_full", grid, smem, p);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, true>), "wy_bwd_full", grid, smem, p);
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
 }
 

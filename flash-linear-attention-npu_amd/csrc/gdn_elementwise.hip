@@ -17,6 +17,8 @@ int check_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B,
     FLA_REQUIRE(t->stride[0] % 8 == 0 && t->stride[1] % 8 == 0 && t->stride[2] % 8 == 0 &&
                     reinterpret_cast<uintptr_t>(t->data) % 16 == 0,
                 FLA_ERR_SHAPE, "%s: rows of %s must be 16-byte aligned.", op, name);
+    FLA_REQUIRE(t->stride[2] >= 0 && t->stride[2] < (1 << 24), FLA_ERR_SHAPE,
+                "%s: token stride of %s must be below 2^24 elements.", op, name);
     return FLA_OK;
 }
 

@@ -288,6 +288,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.m_sb = ib < 0 ? 0 : daqk->stride[ib];
     p.m_sh = daqk->stride[ih];
     p.m_st = daqk->stride[it];
+    FLA_REQUIRE(p.st >= 0 && p.st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride must be below 2^24 elements.", op);
     return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }
 

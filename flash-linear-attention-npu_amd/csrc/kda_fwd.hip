@@ -578,6 +578,7 @@ int layout_view(const char *op, const char *name, const fla_tensor *t, const Lay
     const int64_t al = 16 / (int64_t)dtype_size(t->dtype);
     FLA_REQUIRE(sb % al == 0 && sh % al == 0 && st % al == 0 && reinterpret_cast<uintptr_t>(t->data) % 16 == 0, FLA_ERR_SHAPE,
                 "%s: rows of %s must be 16-byte aligned.", op, name);
+    FLA_REQUIRE(st >= 0 && st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride of %s must be below 2^24 elements.", op, name);
     return FLA_OK;
 }
 

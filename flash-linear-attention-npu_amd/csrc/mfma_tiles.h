@@ -88,7 +88,10 @@ template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
         for (int m = 0; m < N; ++m) {
             const int idx = m * THREADS + tid;
             const int row = idx / CPR, c = (idx % CPR) << 3;
-            r[m] = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)(row < valid ? row : last) * gstride + c);
+            // 32-bit element offset from the (uniform) tile base: a tile spans 64 rows of a stride the host
+            // checks to be below 2^24 elements, and the load keeps its base in scalar registers
+            const unsigned off = (unsigned)((row < valid ? row : last) * (int)gstride + c);
+            r[m] = *reinterpret_cast<const u32x4 *>(gsrc + off);
         }
     }
     __device__ __forceinline__ void commit(bf16 *tile, int pitch, int valid, int tid) const {
@@ -111,7 +114,7 @@ __device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsr
         const int idx = idx0 + tid;
         if (idx < total) {
             const int r = idx / cpr, c = (idx % cpr) << 3;
-            u32x4 v = *reinterpret_cast<const u32x4 *>(gsrc + (int64_t)(r < valid ? r : last) * gstride + c);
+            u32x4 v = *reinterpret_cast<const u32x4 *>(gsrc + (unsigned)((r < valid ? r : last) * (int)gstride + c));
             if (r >= valid) v = u32x4{0u, 0u, 0u, 0u};
             *reinterpret_cast<u32x4 *>(tile + r * pitch + c) = v;
         }

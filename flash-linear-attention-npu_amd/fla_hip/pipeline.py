@@ -67,13 +67,14 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
 
     cu = _cu_list(cu_seqlens)
     kw = dict(cu_seqlens=cu)
-    gh = g.transpose(1, 2).contiguous().float()
-    bh = beta.transpose(1, 2).contiguous().float()
+    # head-first VIEWS: every kernel takes the outer strides of its operands, nothing is copied
+    gh = g.float().transpose(1, 2)
+    bh = beta.float().transpose(1, 2)
     if A is None:
         A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
         A = _ops.solve_tri(A.to(k.dtype), layout="bnsd", **kw)
     w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
-    doh = do.transpose(1, 2).contiguous()
+    doh = do.transpose(1, 2) if do.stride(-1) == 1 else do.transpose(1, 2).contiguous()
     h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,
                                                     output_final_state=False, chunk_size=chunk_size, **kw)
     dv = _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
@@ -82,9 +83,9 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
     dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
     dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
-    dk = (dk.float() + dk2.float()).to(dk.dtype)
+    dk.add_(dk2)
     dg = _ops.chunk_local_cumsum(dg + dg2, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
-    return dq, dk, dv, db.transpose(1, 2).contiguous(), dg.transpose(1, 2).contiguous(), dh0
+    return dq, dk, dv, db.transpose(1, 2), dg.transpose(1, 2), dh0
 
 
 def _autograd_function():
