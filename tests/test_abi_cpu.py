@@ -313,3 +313,51 @@ def test_kda_gate_and_bwd_wrappers_operands():
         capture_call(H.npu_chunk_kda_bwd_intra, *[mk(t.shape[1:], t.dtype) for t in args], layout="TND")
     with pytest.raises(RuntimeError, match="varlen supports TND or BSND"):
         capture_call(H.npu_chunk_kda_bwd_intra, *args, layout="BNSD", cu_seqlens=[0, T])
+
+
+def test_gdn_backward_wrappers_operands_and_outputs():
+    """Operand order equals the aclnn prototypes (_aclnn_ctypes.py:242-279, 397-510); dq / dk take the key-head
+    shape, dw the value-head count, and the fp32 side outputs come back in the dtype of beta / g."""
+    from fla_hip.ops import _hip_ctypes as H
+    B, Hk, Hv, T, K, V = 1, 2, 4, 130, 128, 64
+    f32 = torch.float32
+    q = FakeFloatTensor((B, Hk, T, K), torch.bfloat16)
+    v = FakeFloatTensor((B, Hv, T, V), torch.bfloat16)
+    w = FakeFloatTensor((B, Hv, T, K), torch.bfloat16)
+    g = FakeFloatTensor((B, Hv, T), f32)
+    A = FakeFloatTensor((B, Hv, T, 64), torch.bfloat16)
+    h = FakeFloatTensor((B, Hv, 3, K, V), torch.bfloat16)
+
+    cap, out = capture_call(H.npu_chunk_bwd_dv_local, q, q, v, g, 0.1, 64, A=A)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["q", "k", "d_o", "g", "g_gamma", "A", "out"]
+    assert out.shape == v.shape and cap["args"][8].value == pytest.approx(0.1) and cap["args"][9].value == 64
+    with pytest.raises(NotImplementedError, match="g_gamma"):
+        capture_call(H.npu_chunk_bwd_dv_local, q, q, v, g, 0.1, 64, g_gamma=g)
+
+    cap, (dq, dk, dw, dg) = capture_call(H.npu_chunk_bwd_dqkwg, q, q, v, g, h, v, h, v, 64, scale=0.25)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == [
+        "q", "k", "v", "g", "h", "dox", "dh", "dv", "w", "g_gamma", "dq", "dk", "dw", "dg"]
+    assert dq.shape == dk.shape == q.shape and dw.shape == (B, Hv, T, K) and dg.shape == g.shape and dg.dtype == f32
+    assert cap["args"][12].value == 0.25 and cap["args"][14].value is False and cap["args"][15].value is False
+    cap, _ = capture_call(H.npu_chunk_bwd_dqkwg, q, q, v, g, h, v, h, v, 64)
+    assert cap["args"][12].value == 1.0                                      # scale=None -> 1.0 (_aclnn_ctypes.py:501)
+
+    cap, dA = capture_call(H.npu_prepare_wy_repr_bwd_da, q, v, g, A, w, v, g, chunk_size=64)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["k", "v", "beta", "A", "dw", "du", "g", "dA"]
+    assert dA.shape == A.shape and dA.dtype == A.dtype
+
+    cap, (dk2, dv2, db, dg2) = capture_call(H.npu_prepare_wy_repr_bwd_full, q, v, g, A, A, w, v, g, 64)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == [
+        "k", "v", "beta", "A", "dA", "dw", "du", "g", "dk", "dv", "dbeta", "dg"]
+    assert dk2.shape == q.shape and dv2.shape == v.shape and db.shape == g.shape and dg2.shape == g.shape
+    assert db.dtype == f32 and dg2.dtype == f32
+
+
+def test_backward_ops_are_exported_under_both_names():
+    from fla_hip import ops
+    for name in ("chunk_bwd_dv_local", "chunk_bwd_dqkwg", "prepare_wy_repr_bwd_da", "prepare_wy_repr_bwd_full"):
+        assert getattr(ops, name) is getattr(ops, "npu_" + name)
