@@ -279,12 +279,242 @@ __global__ void conv1d_state_kernel(const ConvParams p) {
     }
 }
 
+// State-update mode (run_mode = 1), one thread per (sequence, 8 channels): the W-1 history rows come from
+// conv_states[slot] (rows offset .. offset+W-2; offset = accepted-1 under speculative decoding, else 0), the
+// S new tokens are convolved in order, and the state is rewritten: the plain form keeps the last W-1 rows of
+// [history | x] in rows 0..W-2; the speculative form (width 4) keeps old rows offset+1..offset+W-2 in rows
+// 0..W-3 and appends all S new tokens, so that the next call can pick its history by its own accepted count.
+// Semantics: op_kernel/causal_conv1d.h:753-860,955-1025; goldens test_npu_causal_conv1d.py:56-151.
+struct ConvUpdateParams {
+    const void *x;
+    const void *weight;
+    const void *bias;
+    void *conv_states;
+    void *out;
+    const int32_t *qsl;    // [N+1] or null
+    const int32_t *cache;  // [N] or null
+    const int32_t *nat;    // [N] or null (speculative decoding)
+    int64_t x_sb, x_ss, o_sb, o_ss, w_sr, cs_sn, cs_sp;
+    int S, D, W, N, state_len, activation, pad_slot;
+};
+
+template <typename T>
+__global__ void conv1d_update_kernel(const ConvUpdateParams p) {
+    typedef typename Vec8<T>::type V8;
+    const int d0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const int n = blockIdx.y;
+    if (d0 >= p.D) return;
+    const int slot = p.cache ? p.cache[n] : n;
+    if (slot == p.pad_slot) return;
+    int64_t xoff, ooff;
+    int len = p.S;
+    if (p.qsl) {
+        const int bos = p.qsl[n];
+        len = p.qsl[n + 1] - bos;
+        xoff = (int64_t)bos * p.x_ss;
+        ooff = (int64_t)bos * p.o_ss;
+    } else {
+        xoff = n * p.x_sb;
+        ooff = n * p.o_sb;
+    }
+    if (len <= 0) return;
+    const int W = p.W, keep = W - 2;
+    const bool spec = p.nat != nullptr && W == 4;
+    int offset = 0;
+    if (spec) offset = min(max(p.nat[n] - 1, 0), p.state_len - (W - 1));
+    T *cs = static_cast<T *>(p.conv_states) + slot * p.cs_sn + d0;
+    const T *xb = static_cast<const T *>(p.x) + xoff + d0;
+    T *ob = static_cast<T *>(p.out) + ooff + d0;
+    float win[kMaxW - 1][8], wt[kMaxW][8], bias[8];
+#pragma unroll
+    for (int i = 0; i < kMaxW - 1; ++i)
+        if (i < W - 1) load8_cached(cs + (int64_t)(offset + i) * p.cs_sp, win[i]);
+#pragma unroll
+    for (int r = 0; r < kMaxW; ++r)
+        if (r < W) load8_cached(static_cast<const T *>(p.weight) + r * p.w_sr + d0, wt[r]);
+    if (p.bias) load8_cached(static_cast<const T *>(p.bias) + d0, bias);
+    else
+        for (int i = 0; i < 8; ++i) bias[i] = 0.f;
+    const bool spec_write = spec && keep + len <= p.state_len;
+    if (spec_write) {   // rows offset+1 .. offset+keep of the old state move to the front
+#pragma unroll
+        for (int i = 0; i < kMaxW - 2; ++i)
+            if (i < keep) {
+                V8 v;
+                for (int c = 0; c < 8; ++c) v[c] = (T)win[i + 1][c];
+                *reinterpret_cast<V8 *>(cs + (int64_t)i * p.cs_sp) = v;
+            }
+    }
+    for (int t = 0; t < len; ++t) {
+        const V8 raw = *reinterpret_cast<const V8 *>(xb + (int64_t)t * p.x_ss);
+        float cur[8], acc[8];
+        for (int c = 0; c < 8; ++c) cur[c] = (float)raw[c];
+        for (int c = 0; c < 8; ++c) acc[c] = bias[c] + wt[W - 1][c] * cur[c];
+#pragma unroll
+        for (int i = 0; i < kMaxW - 1; ++i)
+            if (i < W - 1)
+                for (int c = 0; c < 8; ++c) acc[c] += wt[i][c] * win[i][c];
+        if (p.activation)
+            for (int c = 0; c < 8; ++c) acc[c] = acc[c] / (1.f + __expf(-acc[c]));
+        V8 o;
+        for (int c = 0; c < 8; ++c) o[c] = (T)acc[c];
+        *reinterpret_cast<V8 *>(ob + (int64_t)t * p.o_ss) = o;
+        if (spec_write) *reinterpret_cast<V8 *>(cs + (int64_t)(keep + t) * p.cs_sp) = raw;
+#pragma unroll
+        for (int i = 0; i < kMaxW - 2; ++i)
+            if (i < W - 2)
+                for (int c = 0; c < 8; ++c) win[i][c] = win[i + 1][c];
+        for (int c = 0; c < 8; ++c) win[W - 2][c] = cur[c];
+    }
+    if (!spec_write) {
+#pragma unroll
+        for (int i = 0; i < kMaxW - 1; ++i)
+            if (i < W - 1) {
+                V8 v;
+                for (int c = 0; c < 8; ++c) v[c] = (T)win[i][c];
+                *reinterpret_cast<V8 *>(cs + (int64_t)i * p.cs_sp) = v;
+            }
+    }
+}
+
 int copy_int_array(std::vector<int32_t> &dst, const fla_int_array *a) {
     dst.clear();
     if (a == nullptr || a->data == nullptr) return 0;
     dst.resize(a->size);
     for (uint64_t i = 0; i < a->size; ++i) dst[i] = (int32_t)a->data[i];
     return (int)a->size;
+}
+
+// run_mode = 1: x [B,S,D], [B,D] (one token per sequence) or packed [T,D] with query_start_loc.
+int conv_update_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias, const fla_tensor *conv_states,
+                     const fla_int_array *query_start_loc, const fla_int_array *cache_indices,
+                     const fla_int_array *initial_state_mode, const fla_int_array *num_accepted_tokens,
+                     int64_t activation_mode, int64_t pad_slot_id, int64_t head_num, const fla_tensor *out, void *workspace,
+                     uint64_t workspace_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "causal_conv1d";
+    int rc;
+    FLA_REQUIRE(initial_state_mode == nullptr || initial_state_mode->data == nullptr, FLA_ERR_UNSUPPORTED,
+                "%s: initial_state_mode is only supported in run_mode=0.", op);
+    FLA_REQUIRE(head_num == 0, FLA_ERR_UNSUPPORTED, "%s: run_mode=1 does not support a head-split output (head_num must be 0).", op);
+    FLA_REQUIRE(activation_mode == 0 || activation_mode == 1, FLA_ERR_SHAPE, "%s: activation_mode must be 0 or 1.", op);
+    FLA_REQUIRE(x->ndim == 2 || x->ndim == 3, FLA_ERR_SHAPE, "%s: x must be [B,S,D], [B,D] or packed [T,D].", op);
+    const int64_t D = x->shape[x->ndim - 1];
+    const int64_t W = weight->shape[0];
+    FLA_REQUIRE(W >= 2 && W <= kMaxW, FLA_ERR_SHAPE, "%s: width must be 2, 3 or 4, got %lld.", op, (long long)W);
+    FLA_REQUIRE(weight->shape[1] == D, FLA_ERR_SHAPE, "%s: weight must be [W,D].", op);
+    FLA_REQUIRE(D % 16 == 0, FLA_ERR_SHAPE, "%s: D must be a multiple of 16, got %lld.", op, (long long)D);
+    FLA_REQUIRE(inner_unit(x) && inner_unit(weight) && inner_unit(out) && same_shape(out, x), FLA_ERR_SHAPE,
+                "%s: out must have the shape of x; innermost strides must be 1.", op);
+    if (bias && bias->data) {
+        if ((rc = check_tensor(bias, op, "bias", 1, dt_bit(x->dtype)))) return rc;
+        FLA_REQUIRE(bias->shape[0] == D && inner_unit(bias), FLA_ERR_SHAPE, "%s: bias must be a contiguous [D].", op);
+    }
+    FLA_REQUIRE(conv_states && conv_states->data, FLA_ERR_NULL, "%s: run_mode=1 needs conv_states.", op);
+    if ((rc = check_tensor(conv_states, op, "conv_states", 3, dt_bit(x->dtype)))) return rc;
+    const int64_t state_len = conv_states->shape[1];
+    FLA_REQUIRE(state_len >= W - 1 && conv_states->shape[2] == D && inner_unit(conv_states), FLA_ERR_SHAPE,
+                "%s: conv_states must be [N, >=W-1, D] with unit channel stride.", op);
+
+    const auto aligned = [](const fla_tensor *t) {
+        for (int i = 0; i + 1 < t->ndim; ++i)
+            if (t->stride[i] % 8 != 0) return false;
+        return reinterpret_cast<uintptr_t>(t->data) % 16 == 0;
+    };
+    FLA_REQUIRE(aligned(x) && aligned(out) && aligned(weight) && aligned(conv_states), FLA_ERR_SHAPE,
+                "%s: rows of x, out, weight and conv_states must be 16-byte aligned.", op);
+    std::vector<int32_t> qsl, cache, nat;
+    const bool has_qsl = query_start_loc && query_start_loc->data;
+    int64_t N, S;
+    bool packed = false;
+    if (x->ndim == 3) {
+        N = x->shape[0];
+        S = x->shape[1];
+        FLA_REQUIRE(!has_qsl || (int64_t)query_start_loc->size == N + 1, FLA_ERR_METADATA,
+                    "%s: query_start_loc.size must equal batch + 1.", op);
+    } else if (has_qsl && (int64_t)query_start_loc->size - 1 != x->shape[0]) {
+        packed = true;                     // 2-D varlen decode: segments of a packed token axis
+        N = (int64_t)query_start_loc->size - 1;
+        S = 0;
+    } else {
+        N = x->shape[0];                   // 2-D decode: one token per sequence
+        S = 1;
+    }
+    if (packed) {
+        copy_int_array(qsl, query_start_loc);
+        FLA_REQUIRE(N >= 1 && qsl[0] == 0 && qsl[N] == x->shape[0], FLA_ERR_METADATA, "%s: query_start_loc must span [0, T].", op);
+        for (int i = 0; i < N; ++i)
+            FLA_REQUIRE(qsl[i] <= qsl[i + 1], FLA_ERR_METADATA, "%s: query_start_loc must be non-decreasing.", op);
+    }
+    if (copy_int_array(cache, cache_indices))
+        FLA_REQUIRE((int64_t)cache.size() == N, FLA_ERR_METADATA, "%s: cache_indices must have one entry per sequence.", op);
+    for (int64_t i = 0; i < N; ++i) {
+        const int64_t slot = cache.empty() ? i : cache[i];
+        FLA_REQUIRE(slot == pad_slot_id || (slot >= 0 && slot < conv_states->shape[0]), FLA_ERR_METADATA,
+                    "%s: cache index %lld out of range.", op, (long long)slot);
+    }
+    if (copy_int_array(nat, num_accepted_tokens)) {
+        FLA_REQUIRE(W == 4, FLA_ERR_UNSUPPORTED, "%s: num_accepted_tokens is only supported for width 4.", op);
+        FLA_REQUIRE((int64_t)nat.size() == N, FLA_ERR_METADATA, "%s: num_accepted_tokens must have one entry per sequence.", op);
+        if (x->ndim == 3)
+            FLA_REQUIRE(state_len >= (W - 1) + (S - 1), FLA_ERR_SHAPE,
+                        "%s: speculative decoding needs state_len >= (W-1) + (S-1) = %lld, got %lld.", op,
+                        (long long)((W - 1) + (S - 1)), (long long)state_len);
+        for (int64_t i = 0; i < N; ++i) {
+            const int64_t limit = packed ? qsl[i + 1] - qsl[i] : S;
+            FLA_REQUIRE(nat[i] >= 0 && nat[i] <= limit, FLA_ERR_METADATA,
+                        "%s: num_accepted_tokens[%lld]=%d must lie in [0, %lld].", op, (long long)i, nat[i], (long long)limit);
+        }
+    }
+    const size_t meta_ints = qsl.size() + cache.size() + nat.size();
+    const uint64_t need = ((meta_ints * 4 + 255) / 256) * 256;
+    if (query) {
+        *query = need;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(need == 0 || (workspace != nullptr && workspace_size >= need), FLA_ERR_WORKSPACE,
+                "%s: workspace of %llu bytes required.", op, (unsigned long long)need);
+    if (N == 0 || x->shape[0] == 0) return FLA_OK;
+    ConvUpdateParams p{};
+    p.x = x->data;
+    p.weight = weight->data;
+    p.bias = (bias && bias->data) ? bias->data : nullptr;
+    p.conv_states = conv_states->data;
+    p.out = out->data;
+    if (meta_ints) {
+        std::vector<int32_t> meta;
+        meta.insert(meta.end(), qsl.begin(), qsl.end());
+        meta.insert(meta.end(), cache.begin(), cache.end());
+        meta.insert(meta.end(), nat.begin(), nat.end());
+        if ((rc = stage_to_device(workspace, meta.data(), meta.size() * 4, stream))) return rc;
+        const int32_t *base = static_cast<const int32_t *>(workspace);
+        p.qsl = qsl.empty() ? nullptr : base;
+        p.cache = cache.empty() ? nullptr : base + qsl.size();
+        p.nat = nat.empty() ? nullptr : base + qsl.size() + cache.size();
+    }
+    if (x->ndim == 3) {
+        p.x_sb = x->stride[0];
+        p.x_ss = x->stride[1];
+        p.o_sb = out->stride[0];
+        p.o_ss = out->stride[1];
+    } else {   // rows of a 2-D x are sequences (S = 1) or packed tokens
+        p.x_sb = p.x_ss = x->stride[0];
+        p.o_sb = p.o_ss = out->stride[0];
+    }
+    p.w_sr = weight->stride[0];
+    p.cs_sn = conv_states->stride[0];
+    p.cs_sp = conv_states->stride[1];
+    p.S = (int)S;
+    p.D = (int)D;
+    p.W = (int)W;
+    p.N = (int)N;
+    p.state_len = (int)state_len;
+    p.activation = (int)activation_mode;
+    p.pad_slot = (int)pad_slot_id;
+    const dim3 block(64), grid((unsigned)((D / 8 + 63) / 64), (unsigned)N);
+    if (x->dtype == FLA_BF16) FLA_LAUNCH("conv1d_update", stream, conv1d_update_kernel<bf16>, grid, block, 0, stream, p);
+    else FLA_LAUNCH("conv1d_update", stream, conv1d_update_kernel<f16>, grid, block, 0, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
 }
 
 int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias, const fla_tensor *conv_states,
@@ -298,8 +528,12 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
     if ((rc = check_tensor(x, op, "x", -1, half_mask))) return rc;
     if ((rc = check_tensor(weight, op, "weight", 2, dt_bit(x->dtype)))) return rc;
     if ((rc = check_tensor(out, op, "out", -1, dt_bit(x->dtype)))) return rc;
-    FLA_REQUIRE(run_mode == 0, FLA_ERR_UNSUPPORTED, "%s: only run_mode=0 (prefill) is implemented, got %lld.", op,
+    FLA_REQUIRE(run_mode == 0 || run_mode == 1, FLA_ERR_SHAPE, "%s: run_mode must be 0 (prefill) or 1 (update), got %lld.", op,
                 (long long)run_mode);
+    if (run_mode == 1)
+        return conv_update_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
+                                num_accepted_tokens, activation_mode, pad_slot_id, head_num, out, workspace, workspace_size,
+                                stream, query);
     FLA_REQUIRE(num_accepted_tokens == nullptr || num_accepted_tokens->data == nullptr, FLA_ERR_UNSUPPORTED,
                 "%s: num_accepted_tokens is only meaningful for run_mode=1.", op);
     FLA_REQUIRE(activation_mode == 0 || activation_mode == 1, FLA_ERR_SHAPE, "%s: activation_mode must be 0 or 1.", op);

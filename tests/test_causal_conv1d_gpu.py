@@ -139,3 +139,124 @@ def test_errors(dev):
     cs.requires_grad_(True)
     with pytest.raises(RuntimeError, match="mutates conv_states"):
         ops.causal_conv1d(x, w[:4], None, cs)
+
+
+# ---------------------------------------------------------------------------------------------
+# state-update mode (run_mode=1): the reference's update / speculative-decode cases
+# (test_npu_causal_conv1d.py:386-520) and random sweeps against the oracle
+# ---------------------------------------------------------------------------------------------
+def run_update(dev, x, w, b, cs, **kw):
+    from fla_hip import ops
+
+    y_ref, cs_ref = oc.causal_conv1d_update(x, w, b, cs, **kw)
+    cs_d = cs.to(dev)
+    y = ops.causal_conv1d(x.to(dev), w.to(dev), None if b is None else b.to(dev), cs_d, run_mode=1, **kw)
+    return y, y_ref, cs_d, cs_ref
+
+
+def test_kat_update_one_token(dev):
+    x = make_tensor((2, 16), start=1.0)
+    w, b = make_tensor((4, 16), start=101.0), make_tensor((16,), start=201.0)
+    cs = make_tensor((2, 3, 16), start=301.0)
+    y, y_ref, cs_d, cs_ref = run_update(dev, x, w, b, cs, cache_indices=[0, 1], activation_mode=1)
+    assert torch.allclose(y.float().cpu(), y_ref.float(), rtol=5e-2, atol=5e-2)      # the reference's tolerance (:186-187)
+    assert torch.equal(cs_d.cpu(), cs_ref)
+
+
+def test_kat_speculative_decode(dev):
+    x = make_tensor((2, 4, 16), start=1.0)
+    w, b = make_tensor((4, 16), start=101.0), make_tensor((16,), start=201.0)
+    cs = make_tensor((2, 6, 16), start=301.0)
+    y, y_ref, cs_d, cs_ref = run_update(dev, x, w, b, cs, cache_indices=[0, 1], num_accepted_tokens=[2, 4])
+    assert torch.allclose(y.float().cpu(), y_ref.float(), rtol=5e-2, atol=5e-2)
+    assert torch.equal(cs_d.cpu(), cs_ref)
+
+
+def test_kat_update_width3_and_padded_batch(dev):
+    x = make_tensor((3, 3, 16), start=1.0)
+    w = make_tensor((3, 16), start=101.0)
+    cs = make_tensor((3, 2, 16), start=301.0)
+    y, y_ref, cs_d, cs_ref = run_update(dev, x, w, None, cs, cache_indices=[0, 1, 2])
+    assert torch.allclose(y.float().cpu(), y_ref.float(), rtol=5e-2, atol=5e-2)
+    assert torch.equal(cs_d.cpu(), cs_ref)
+    # batch gather with padded rows: valid rows match, padded rows and untouched slots stay as they were
+    x = make_tensor((5, 3, 16), start=1.0)
+    w, b = make_tensor((4, 16), start=101.0), make_tensor((16,), start=201.0)
+    cs = make_tensor((7, 3, 16), start=301.0)
+    from fla_hip import ops
+    cs_d = cs.to(dev)
+    y = torch.full((5, 3, 16), 7.0, dtype=x.dtype, device=dev)
+    y_ref, cs_ref = oc.causal_conv1d_update(x, w, b, cs, cache_indices=[1, 3, 5, -1, -1], activation_mode=1)
+    y = ops.causal_conv1d(x.to(dev), w.to(dev), b.to(dev), cs_d, cache_indices=[1, 3, 5, -1, -1], activation_mode=1, run_mode=1)
+    assert torch.allclose(y[:3].float().cpu(), y_ref[:3].float(), rtol=5e-2, atol=5e-2)
+    assert torch.equal(cs_d.cpu(), cs_ref)
+
+
+@pytest.mark.parametrize("W", [2, 3, 4])
+@pytest.mark.parametrize("S", [1, 2, 5])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_random_update(dev, W, S, dtype):
+    gen = torch.Generator().manual_seed(100 * W + S)
+    B, D, slots = 9, 192, 12
+    x = torch.randn(B, S, D, generator=gen).to(dtype)
+    w = (torch.randn(W, D, generator=gen) * 0.3).to(dtype)
+    b = (torch.randn(D, generator=gen) * 0.1).to(dtype)
+    cs = torch.randn(slots, W - 1 + 2, D, generator=gen).to(dtype)          # longer than needed: only rows 0..W-2 take part
+    cache = torch.randperm(slots, generator=gen)[:B].tolist()
+    cache[4] = -1
+    y, y_ref, cs_d, cs_ref = run_update(dev, x, w, b, cs, cache_indices=cache, activation_mode=1)
+    keep = [i for i in range(B) if cache[i] != -1]
+    assert_close(y[keep], y_ref[keep], TOL_BF16, "y")
+    assert torch.equal(cs_d.cpu(), cs_ref)
+    if S == 1:      # the 2-D one-token form gives the same rows
+        y2, _, cs2, _ = run_update(dev, x[:, 0], w, b, cs, cache_indices=cache, activation_mode=1)
+        assert torch.equal(y2[keep].cpu(), y[keep][:, 0].cpu()) and torch.equal(cs2.cpu(), cs_d.cpu())
+
+
+def test_speculative_decode_loop_and_packed_update(dev):
+    """A draft/accept loop on the GPU tracks the oracle step by step (outputs and the whole state pool), and the
+    packed 2-D varlen form equals the per-sequence results."""
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(5)
+    W, D, S, B = 4, 256, 4, 3
+    w = (torch.randn(W, D, generator=gen) * 0.3).bfloat16()
+    cs = torch.zeros(5, (W - 1) + (S - 1), D).bfloat16()
+    cs_d = cs.to(dev)
+    cache = [3, 0, 4]
+    nat = [1, 1, 1]
+    for step in range(5):
+        x = torch.randn(B, S, D, generator=gen).bfloat16()
+        y_ref, cs = oc.causal_conv1d_update(x, w, None, cs, cache_indices=cache, num_accepted_tokens=nat)
+        y = ops.causal_conv1d(x.to(dev), w.to(dev), None, cs_d, cache_indices=cache, num_accepted_tokens=nat, run_mode=1)
+        assert_close(y, y_ref, TOL_BF16, f"step {step}")
+        assert torch.equal(cs_d.cpu(), cs)
+        nat = [int(v) for v in torch.randint(1, S + 1, (B,), generator=gen)]
+    # packed tokens with query_start_loc (segments of different length, one of them padded out)
+    qsl = [0, 3, 4, 9]
+    x = torch.randn(9, D, generator=gen).bfloat16()
+    cs0 = torch.randn(4, 3, D, generator=gen).bfloat16()
+    y_ref, cs_ref = oc.causal_conv1d_update(x, w, None, cs0, query_start_loc=qsl, cache_indices=[2, -1, 0])
+    cs_d = cs0.to(dev)
+    y = ops.causal_conv1d(x.to(dev), w.to(dev), None, cs_d, query_start_loc=qsl, cache_indices=[2, -1, 0], run_mode=1)
+    rows = [0, 1, 2, 4, 5, 6, 7, 8]
+    assert_close(y[rows], y_ref[rows], TOL_BF16, "packed")
+    assert torch.equal(cs_d.cpu(), cs_ref)
+
+
+def test_update_mode_errors(dev):
+    from fla_hip import ops
+    x = torch.zeros(2, 4, 16, dtype=torch.bfloat16, device=dev)
+    w4, w3 = torch.zeros(4, 16, dtype=torch.bfloat16, device=dev), torch.zeros(3, 16, dtype=torch.bfloat16, device=dev)
+    cs = torch.zeros(2, 6, 16, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="needs conv_states"):
+        ops.causal_conv1d(x, w4, run_mode=1)
+    with pytest.raises(RuntimeError, match="only supported for width 4"):
+        ops.causal_conv1d(x, w3, None, cs, num_accepted_tokens=[1, 1], run_mode=1)
+    with pytest.raises(RuntimeError, match="state_len >="):
+        ops.causal_conv1d(x, w4, None, cs[:, :4], num_accepted_tokens=[1, 1], run_mode=1)
+    with pytest.raises(RuntimeError, match=r"must lie in \[0, 4\]"):
+        ops.causal_conv1d(x, w4, None, cs, num_accepted_tokens=[1, 5], run_mode=1)
+    with pytest.raises(RuntimeError, match="initial_state_mode is only supported in run_mode=0"):
+        ops.causal_conv1d(x, w4, None, cs, initial_state_mode=[1, 1], run_mode=1)
+    with pytest.raises(RuntimeError, match="head_num must be 0"):
+        ops.causal_conv1d(x, w4, None, cs, run_mode=1, head_num=2)

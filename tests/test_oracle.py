@@ -412,3 +412,107 @@ def test_gdn_backward_composition_against_recurrence_autograd(cu):
     for name, got, want in (("dq", dq, q.grad), ("dk", dk, k.grad), ("dv", dv, v.grad), ("dbeta", db, beta.grad),
                             ("dg", dg, g.grad), ("dh0", dh0, h0.grad)):
         assert torch.allclose(got, want, atol=1e-8), f"{name}: {(got - want).abs().max().item():.3e}"
+
+
+# ----------------------------------------------------------------------------
+# causal_conv1d: state-update / speculative-decode mode and backward
+# ----------------------------------------------------------------------------
+def test_conv1d_update_in_pieces_equals_one_prefill():
+    """Feeding a sequence piece by piece through the update mode reproduces F.conv1d over the whole sequence,
+    for every width, through shuffled cache slots, and leaves the last W-1 inputs in the state."""
+    gen = torch.Generator().manual_seed(31)
+    for W in (2, 3, 4):
+        B, T, D = 3, 11, 16
+        x = torch.randn(B, T, D, generator=gen)
+        w = torch.randn(W, D, generator=gen)
+        b = torch.randn(D, generator=gen)
+        full = F.conv1d(x.permute(0, 2, 1), w.t().unsqueeze(1), b, padding=W - 1, groups=D)[..., :T].permute(0, 2, 1)
+        cache = [4, 0, 2]
+        cs = torch.zeros(6, W - 1, D)
+        outs = []
+        for s, e in ((0, 1), (1, 4), (4, 5), (5, 11)):
+            piece = x[:, s] if e - s == 1 and s == 0 else x[:, s:e]      # also the 2-D one-token form
+            y, cs = oc.causal_conv1d_update(piece, w, b, cs, cache_indices=cache)
+            outs.append(y.unsqueeze(1) if y.dim() == 2 else y)
+        assert torch.allclose(torch.cat(outs, 1), full, atol=1e-5)
+        for n, slot in enumerate(cache):
+            assert torch.equal(cs[slot], x[n, T - (W - 1):])
+        assert float(cs[[1, 3, 5]].abs().max()) == 0.0                  # untouched slots
+
+
+def test_conv1d_update_padding_and_activation():
+    gen = torch.Generator().manual_seed(32)
+    x = torch.randn(3, 2, 16, generator=gen)
+    w, cs = torch.randn(4, 16, generator=gen), torch.randn(5, 3, 16, generator=gen)
+    y, new = oc.causal_conv1d_update(x, w, None, cs, cache_indices=[3, -1, 0], activation_mode=1)
+    ref = F.silu(F.conv1d(torch.cat([cs[[3, 0]], x[[0, 2]]], 1).permute(0, 2, 1), w.t().unsqueeze(1), None, groups=16)).permute(0, 2, 1)
+    assert torch.allclose(y[[0, 2]], ref, atol=1e-5) and float(y[1].abs().max()) == 0.0
+    assert torch.equal(new[[1, 2, 4]], cs[[1, 2, 4]])
+
+
+def test_conv1d_speculative_decode_tracks_the_accepted_prefix():
+    """A speculative-decoding loop: every step proposes S tokens of which only a prefix is accepted; the next step
+    passes that count.  The outputs at accepted positions must equal a plain causal convolution of the accepted
+    stream (F.conv1d), whatever was drafted beyond it."""
+    gen = torch.Generator().manual_seed(33)
+    W, D, S = 4, 16, 4
+    w, b = torch.randn(W, D, generator=gen), torch.randn(D, generator=gen)
+    truth = torch.randn(1, 40, D, generator=gen)
+    full = F.conv1d(truth.permute(0, 2, 1), w.t().unsqueeze(1), b, padding=W - 1, groups=D)[..., :40].permute(0, 2, 1)
+    cs = torch.zeros(2, (W - 1) + (S - 1), D)
+    pos, accepted_prev = 0, None
+    for accepted in (2, 4, 1, 3, 4, 2):
+        draft = truth[:, pos:pos + S].clone()
+        draft[:, accepted:] = torch.randn(1, S - accepted, D, generator=gen)      # rejected tail
+        kw = {} if accepted_prev is None else dict(num_accepted_tokens=[accepted_prev])
+        if accepted_prev is None:
+            # first step: history is the zero state at rows 0..2, i.e. one accepted token of an empty draft
+            kw = dict(num_accepted_tokens=[1])
+        y, cs = oc.causal_conv1d_update(draft, w, b, cs, cache_indices=[1], **kw)
+        assert torch.allclose(y[:, :accepted], full[:, pos:pos + accepted], atol=1e-5)
+        pos += accepted
+        accepted_prev = accepted
+
+
+def test_conv1d_bwd_against_autograd():
+    """dx, dw, db, dh0 equal autograd through F.conv1d over [state rows 1..W-1 | x], with SiLU, a final-state
+    gradient and packed sequences (including one shorter than the kernel)."""
+    gen = torch.Generator().manual_seed(34)
+    dd = torch.float64
+    for W in (2, 3, 4):
+        D = 16
+        qsl = [0, 2, 9, 10, 21]
+        T = qsl[-1]
+        N = len(qsl) - 1
+        x = torch.randn(T, D, generator=gen, dtype=dd).requires_grad_(True)
+        w = torch.randn(W, D, generator=gen, dtype=dd).requires_grad_(True)
+        bias = torch.randn(D, generator=gen, dtype=dd).requires_grad_(True)
+        h0 = torch.randn(N, W, D, generator=gen, dtype=dd).requires_grad_(True)
+        dy = torch.randn(T, D, generator=gen, dtype=dd)
+        dht = torch.randn(N, W, D, generator=gen, dtype=dd)
+        loss, ys = 0.0, []
+        for n, (s, e) in enumerate(zip(qsl, qsl[1:])):
+            xp = torch.cat([h0[n, 1:], x[s:e]], 0)
+            pre = F.conv1d(xp.t().unsqueeze(0), w.t().unsqueeze(1), bias, groups=D)[0].t()
+            ys.append(pre.detach())
+            loss = loss + (F.silu(pre) * dy[s:e]).sum()
+            if e - s >= W - 1:          # final state = last W-1 inputs (the golden's short-sequence rule differs)
+                loss = loss + (x[e - (W - 1):e] * dht[n, 1:]).sum()
+        loss.backward()
+        long_enough = torch.tensor([e - s >= W - 1 for s, e in zip(qsl, qsl[1:])])
+        dht_used = dht * long_enough[:, None, None]
+        dx, dw, db, dh0 = oc.causal_conv1d_bwd(x.detach().float(), torch.cat(ys).float(), w.detach().float(), dy.float(),
+                                               h0.detach().float(), dht_used.float(), query_start_loc=qsl, activation=1)
+        assert torch.allclose(dx.double(), x.grad, atol=1e-4)
+        assert torch.allclose(dw.double(), w.grad, atol=1e-4)
+        assert torch.allclose(db.double(), bias.grad, atol=1e-4)
+        assert torch.allclose(dh0.double(), h0.grad, atol=1e-4)
+        assert float(dh0[:, 0].abs().max()) == 0.0
+    # dense layout, no activation, no states: the plain transposed convolution
+    x = torch.randn(2, 7, 16, generator=gen, dtype=dd).requires_grad_(True)
+    w = torch.randn(4, 16, generator=gen, dtype=dd).requires_grad_(True)
+    dy = torch.randn(2, 7, 16, generator=gen, dtype=dd)
+    (F.conv1d(x.permute(0, 2, 1), w.t().unsqueeze(1), None, padding=3, groups=16)[..., :7].permute(0, 2, 1) * dy).sum().backward()
+    dx, dw, db, dh0 = oc.causal_conv1d_bwd(x.detach().float(), None, w.detach().float(), dy.float())
+    assert torch.allclose(dx.double(), x.grad, atol=1e-4) and torch.allclose(dw.double(), w.grad, atol=1e-4)
+    assert torch.allclose(db.double(), dy.sum((0, 1)), atol=1e-4) and float(dh0.abs().max()) == 0.0
