@@ -98,23 +98,56 @@ for _name in _REFERENCE_OPS:
     globals()[_strip_npu_prefix(_name)] = _op
 
 
+def _has_tensor_requiring_grad(*tensors) -> bool:
+    import torch
+
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 def causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=None, cache_indices=None,
                   initial_state_mode=None, num_accepted_tokens=None, activation_mode=0, pad_slot_id=-1,
                   run_mode=0, head_num=0):
-    """Causal conv1d prefill (ops/ascendc/__init__.py:299-392).  ``conv_states`` is
-    mutable state and must not require gradients.  The backward operator is outside
-    this library, so inputs that require grad are rejected instead of silently
-    detached."""
+    """Causal conv1d with automatic backward binding for prefill mode (ops/ascendc/__init__.py:299-392).
+
+    ``conv_states`` is mutable state in every mode and must not require gradients.  The update / speculative
+    modes stay on the raw operator; a dense prefill without activation binds gradients for ``x``, ``weight`` and
+    ``bias`` through ``causal_conv1d_bwd``.  Any other call with inputs that require grad is rejected rather than
+    silently detached."""
     import torch
 
-    for t in (x, weight, bias):
-        if isinstance(t, torch.Tensor) and t.requires_grad and torch.is_grad_enabled():
-            raise NotImplementedError("fla_hip.ops.causal_conv1d: backward is not implemented; pass detached inputs.")
-    return globals()["npu_causal_conv1d"](
-        x=x, weight=weight, bias=bias, conv_states=conv_states, query_start_loc=query_start_loc,
-        cache_indices=cache_indices, initial_state_mode=initial_state_mode,
-        num_accepted_tokens=num_accepted_tokens, activation_mode=activation_mode, pad_slot_id=pad_slot_id,
-        run_mode=run_mode, head_num=head_num)
+    direct = globals()["npu_causal_conv1d"]
+    kwargs = dict(query_start_loc=query_start_loc, cache_indices=cache_indices, initial_state_mode=initial_state_mode,
+                  num_accepted_tokens=num_accepted_tokens, activation_mode=activation_mode, pad_slot_id=pad_slot_id,
+                  run_mode=run_mode, head_num=head_num)
+    if not _has_tensor_requiring_grad(x, weight, bias):
+        return direct(x=x, weight=weight, bias=bias, conv_states=conv_states, **kwargs)
+    can_bind_backward = (run_mode == 0 and activation_mode == 0 and query_start_loc is None and cache_indices is None
+                         and initial_state_mode is None and num_accepted_tokens is None)
+    if not can_bind_backward:
+        raise NotImplementedError(
+            "fla_hip.ops.causal_conv1d: gradients are bound only for a dense prefill without activation "
+            "(run_mode=0, activation_mode=0, no query_start_loc / cache_indices / initial_state_mode); pass detached inputs.")
+    bwd = globals()["npu_causal_conv1d_bwd"]
+
+    class Function(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x_, weight_, bias_, conv_states_):
+            y = direct(x=x_, weight=weight_, bias=bias_, conv_states=conv_states_, **kwargs)
+            ctx.has_bias = bias_ is not None
+            ctx.save_for_backward(x_, weight_)
+            return y
+
+        @staticmethod
+        def backward(ctx, grad):
+            x_, weight_ = ctx.saved_tensors
+            layout = "BSH"
+            if head_num > 0:           # the forward returned [B, head_num, S, D/head_num]
+                layout = "BNSD"
+            dx, dw, db, _ = bwd(x_, None, weight_, grad.contiguous(), None, None, query_start_loc=None, activation=0,
+                                input_layout=layout)
+            return dx, dw, (db if ctx.has_bias else None), None
+
+    return Function.apply(x, weight, bias, conv_states)
 
 
 __all__ = [

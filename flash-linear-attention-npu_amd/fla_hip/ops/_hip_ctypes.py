@@ -42,6 +42,7 @@ OP_ARGTYPES = {
     "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
+    "causal_conv1d_bwd": [_T, _T, _T, _T, _T, _T, _IA, ctypes.c_int64, ctypes.c_char_p, _T, _T, _T, _T],
     "chunk_bwd_dv_local": [_T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
     "chunk_bwd_dqkwg": [_T] * 8 + [_IA, _IA, _T, _T, ctypes.c_float, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool]
                        + [_T] * 4,
@@ -776,6 +777,35 @@ def npu_chunk_bwd_dqkwg(q, k, v, g, h, dox, dh, dv, chunk_size, *, cu_seqlens=No
         outputs,
     )
     return dq, dk, dw, _as_dtype(dg, g)
+
+
+def npu_causal_conv1d_bwd(x, y, weight, dy, initial_state=None, dht=None, *, query_start_loc=None, activation=0,
+                          input_layout="BSND"):
+    """_aclnn_ctypes.py:988-1037.  Returns (dx, dw, db, dh0); ``y`` is the pre-activation output."""
+    input_layout = str(input_layout)
+    width, dim = int(weight.shape[0]), int(weight.shape[1])
+    if input_layout in {"NTD", "TND"}:
+        if query_start_loc is None:
+            raise RuntimeError(f"query_start_loc is required for {input_layout} input.")
+        batch = len(query_start_loc) - 1
+    else:
+        batch = int(x.shape[0])
+    dx = _empty(_shape(x), x)
+    dw = _empty((width, dim), weight)
+    db = _empty((dim,), weight)
+    dh0 = _empty((batch, width, dim), x)
+    outputs = (dx, dw, db, dh0)
+    return _call_op(
+        "causal_conv1d_bwd", OP_ARGTYPES["causal_conv1d_bwd"],
+        lambda ctx: [
+            ctx.tensor(x, "x"), ctx.tensor(y, "y"), ctx.tensor(weight, "weight"), ctx.tensor(dy, "dy"),
+            ctx.tensor(initial_state, "initial_state"), ctx.tensor(dht, "dht"),
+            ctx.int_array(_as_int_tuple(query_start_loc)), ctypes.c_int64(int(activation)),
+            ctypes.c_char_p(input_layout.encode("utf-8")),
+            ctx.tensor(dx, "dx"), ctx.tensor(dw, "dw"), ctx.tensor(db, "db"), ctx.tensor(dh0, "dh0"),
+        ],
+        outputs,
+    )
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

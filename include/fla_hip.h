@@ -338,6 +338,24 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * causal_conv1d_bwd - replaces aclnnCausalConv1dBwd (_aclnn_ctypes.py:988-1037;
+ * causal_conv1d_bwd/README.md:54-118).  x, dx: logical [B,T,D] or packed [T,D];
+ * y (pre-activation, needed when activation is 1 or 2) and dy in input_layout
+ * "BSND"/"BSH" [B,T,D], "BNSD" [B,N,T,D/N], "TND" [T,D], "NTD" [N,T,D/N] (the packed
+ * layouts need query_start_loc).  initial_state, dht, dh0: [N,W,D], rows 1..W-1 hold
+ * the last W-1 inputs.  dw [W,D], db [D] and dh0 are optional outputs.  bf16 or f16.
+ * ------------------------------------------------------------------------ */
+int fla_causal_conv1d_bwd_get_workspace_size(
+    const fla_tensor *x, const fla_tensor *y, const fla_tensor *weight, const fla_tensor *dy, const fla_tensor *initial_state,
+    const fla_tensor *dht, const fla_int_array *query_start_loc, int64_t activation, const char *input_layout,
+    const fla_tensor *dx, const fla_tensor *dw, const fla_tensor *db, const fla_tensor *dh0, uint64_t *workspace_size);
+int fla_causal_conv1d_bwd(
+    const fla_tensor *x, const fla_tensor *y, const fla_tensor *weight, const fla_tensor *dy, const fla_tensor *initial_state,
+    const fla_tensor *dht, const fla_int_array *query_start_loc, int64_t activation, const char *input_layout,
+    const fla_tensor *dx, const fla_tensor *dw, const fla_tensor *db, const fla_tensor *dh0, void *workspace,
+    uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
  * Gated-delta-rule backward chain (examples/flash_gated_delta_rule.py:884-1008).
  * All activations head-first: q, k, dq, dk [B,Hk,T,K]; v, d_o, dv, du [B,Hv,T,V];
  * w, dw [B,Hv,T,K] bf16; g (chunk-cumsummed) and beta [B,Hv,T] f32 or bf16;

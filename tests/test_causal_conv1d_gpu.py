@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import conv1d as oc
-from util import assert_close, TOL_BF16
+from util import assert_close, err_stats, TOL_BF16
 
 pytestmark = pytest.mark.gpu
 
@@ -260,3 +260,119 @@ def test_update_mode_errors(dev):
         ops.causal_conv1d(x, w4, None, cs, initial_state_mode=[1, 1], run_mode=1)
     with pytest.raises(RuntimeError, match="head_num must be 0"):
         ops.causal_conv1d(x, w4, None, cs, run_mode=1, head_num=2)
+
+
+# ---------------------------------------------------------------------------------------------
+# backward (test_npu_causal_conv1d_bwd.py: fixed BSH with every activation, BNSD, packed TND / NTD)
+# ---------------------------------------------------------------------------------------------
+def bwd_tensor(shape, *, dtype=torch.bfloat16, offset=0):       # the reference's deterministic inputs (:23-29)
+    numel = 1
+    for d in shape:
+        numel *= d
+    values = torch.arange(offset, offset + numel, dtype=torch.float32)
+    return ((values.remainder(37) - 18.0) / 64.0).reshape(shape).to(dtype)
+
+
+def preactivation(x, w, h0, qsl=None):
+    """fp32 forward pre-activation in the logical layout (the forward oracle with the state's rows 1..W-1)."""
+    W = w.shape[0]
+    cs = None if h0 is None else h0[:, 1:].contiguous()
+    N = (len(qsl) - 1) if qsl is not None else x.shape[0]
+    y, _ = oc.causal_conv1d(x.float(), w.float(), None, cs if cs is None else cs.float(), query_start_loc=qsl,
+                            initial_state_mode=None if cs is None else [1] * N)
+    return y
+
+
+def check_bwd(dev, x, w, dy, h0, dht, *, qsl=None, activation=0, layout="BSND", heads=1, tol=TOL_BF16):
+    from fla_hip import ops
+    y = preactivation(x, w, h0, qsl).to(x.dtype) if activation else None
+    ref = oc.causal_conv1d_bwd(x, y, w, dy, h0, dht, query_start_loc=qsl, activation=activation)
+
+    def phys(t):        # logical -> physical layout of y / dy
+        if t is None or layout in ("BSND", "BSH", "TND"):
+            return t
+        if layout == "BNSD":
+            B, T, D = t.shape
+            return t.reshape(B, T, heads, D // heads).permute(0, 2, 1, 3).contiguous()
+        T, D = t.shape
+        return t.reshape(T, heads, D // heads).permute(1, 0, 2).contiguous()
+
+    d = lambda t: None if t is None else t.to(dev)
+    got = ops.causal_conv1d_bwd(d(x), d(phys(y)), d(w), d(phys(dy)), d(h0), d(dht), query_start_loc=qsl, activation=activation,
+                                input_layout=layout)
+    for name, a, e in zip(("dx", "dw", "db", "dh0"), got, ref):
+        assert a.shape == e.shape and a.dtype == e.dtype, name
+        st = err_stats(a, e)
+        assert st["rel_max"] <= tol, f"{name} ({layout}, act={activation}): {st}"
+    return got
+
+
+@pytest.mark.parametrize("activation", [0, 1, 2])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_bwd_kat_fixed_bsh(dev, activation, dtype):
+    B, T, D, W = 2, 9, 32, 4
+    x, w = bwd_tensor((B, T, D), dtype=dtype, offset=3), bwd_tensor((W, D), dtype=dtype, offset=11)
+    dy = bwd_tensor((B, T, D), dtype=dtype, offset=23)
+    h0, dht = bwd_tensor((B, W, D), dtype=dtype, offset=31), bwd_tensor((B, W, D), dtype=dtype, offset=41)
+    got = check_bwd(dev, x, w, dy, h0, dht, activation=activation, layout="BSH")
+    assert float(got[3][:, 0].abs().max()) == 0.0
+
+
+def test_bwd_bnsd_and_packed_layouts(dev):
+    gen = torch.Generator().manual_seed(17)
+    B, T, D, H = 2, 70, 64, 2
+    for W in (2, 3, 4):
+        x = torch.randn(B, T, D, generator=gen).bfloat16()
+        w = (torch.randn(W, D, generator=gen) * 0.3).bfloat16()
+        dy = torch.randn(B, T, D, generator=gen).bfloat16()
+        h0, dht = torch.randn(B, W, D, generator=gen).bfloat16(), torch.randn(B, W, D, generator=gen).bfloat16()
+        check_bwd(dev, x, w, dy, h0, dht, activation=1, layout="BNSD", heads=H)
+        check_bwd(dev, x, w, dy, None, None, activation=0, layout="BSND")
+        qsl = [0, 1, 3, 3, 40, 41, 140]            # lengths 1, 2, 0, 37, 1, 99: shorter than the kernel, empty, across tiles
+        xp, dyp = x.reshape(B * T, D), dy.reshape(B * T, D)
+        N = len(qsl) - 1
+        h0p, dhtp = torch.randn(N, W, D, generator=gen).bfloat16(), torch.randn(N, W, D, generator=gen).bfloat16()
+        check_bwd(dev, xp, w, dyp, h0p, dhtp, qsl=qsl, activation=1, layout="TND")
+        check_bwd(dev, xp, w, dyp, h0p, None, qsl=qsl, activation=2, layout="NTD", heads=H)
+
+
+def test_bwd_benchmark_shape_and_autograd_binding(dev):
+    """BASELINE config 2 shape: the reductions over 16384 tokens stay within tolerance, and loss.backward()
+    through ops.causal_conv1d reaches the same gradients."""
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(2)
+    B, T, D, W = 4, 4096, 4096, 4
+    x = torch.randn(B, T, D, generator=gen).bfloat16()
+    w = (torch.randn(W, D, generator=gen) * 0.1).bfloat16()
+    b = (torch.randn(D, generator=gen) * 0.01).bfloat16()
+    dy = torch.randn(B, T, D, generator=gen).bfloat16()
+    xd, wd, bd = (t.to(dev).requires_grad_(True) for t in (x, w, b))
+    y = ops.causal_conv1d(xd, wd, bd)
+    (y.float() * dy.to(dev).float()).sum().backward()
+    # fp32 reference on the GPU with torch ops (the CPU oracle's token loop is too slow at this size)
+    xf, wf, dyf = x.to(dev).float(), w.to(dev).float(), dy.to(dev).float()
+    dx_ref = torch.zeros_like(xf)
+    dw_ref = torch.zeros(W, D, device=dev)
+    for j in range(W):
+        tap = W - 1 - j
+        dx_ref[:, :T - j] += dyf[:, j:] * wf[tap]
+        dw_ref[tap] = (dyf[:, j:] * xf[:, :T - j]).sum((0, 1))
+    assert err_stats(xd.grad, dx_ref)["rel_max"] <= TOL_BF16
+    assert err_stats(wd.grad, dw_ref)["rel_max"] <= TOL_BF16
+    assert err_stats(bd.grad, dyf.sum((0, 1)))["rel_max"] <= TOL_BF16
+    with pytest.raises(NotImplementedError, match="gradients are bound only"):
+        ops.causal_conv1d(xd, wd, bd, activation_mode=1)
+
+
+def test_bwd_errors(dev):
+    from fla_hip import ops
+    x = torch.zeros(2, 8, 32, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(4, 32, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="y is required"):
+        ops.causal_conv1d_bwd(x, None, w, x, activation=1)
+    with pytest.raises(RuntimeError, match="query_start_loc is required"):
+        ops.causal_conv1d_bwd(x[0], None, w, x[0], input_layout="TND")
+    with pytest.raises(RuntimeError, match="input_layout must be"):
+        ops.causal_conv1d_bwd(x, None, w, x, input_layout="SBH")
+    with pytest.raises(RuntimeError, match=r"must be \[N=2, W, D\]"):
+        ops.causal_conv1d_bwd(x, None, w, x, torch.zeros(2, 3, 32, dtype=torch.bfloat16, device=dev))
