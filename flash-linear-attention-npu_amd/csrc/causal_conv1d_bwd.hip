@@ -182,18 +182,38 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
     *reinterpret_cast<f32x4 *>(part + (int64_t)W * p.D + 4) = f32x4{db[4], db[5], db[6], db[7]};
 }
 
-// dw[r][d] (r < W) and db[d] (r == W): the tiles' partial sums added in tile order.
+// dw[r][d] (r < W) and db[d] (r == W) from the tiles' partial sums.  A block covers 64 channels; its four
+// slices each add every fourth tile (four independent chains per thread keep loads in flight) and the slices
+// are then added in slice order, so the summation order is fixed.
 template <typename T>
-__global__ void conv1d_bwd_reduce_kernel(const float *partial, int tiles, int W, int D, T *dw, int64_t dw_sr, T *db) {
-    const int d = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void __launch_bounds__(256) conv1d_bwd_reduce_kernel(const float *partial, int tiles, int W, int D, T *dw,
+                                                                int64_t dw_sr, T *db) {
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int d = blockIdx.x * 64 + lane;
     const int r = blockIdx.y;
-    if (d >= D) return;
-    float s = 0.f;
-    for (int t = 0; t < tiles; ++t) s += partial[((int64_t)t * (W + 1) + r) * D + d];
-    if (r < W) {
-        if (dw) dw[r * dw_sr + d] = (T)s;
-    } else if (db) {
-        db[d] = (T)s;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (d < D) {
+        const float *src = partial + (int64_t)r * D + d;
+        const int64_t step = (int64_t)(W + 1) * D;
+        int t = slice;
+        for (; t + 12 < tiles; t += 16) {
+            s0 += src[t * step];
+            s1 += src[(t + 4) * step];
+            s2 += src[(t + 8) * step];
+            s3 += src[(t + 12) * step];
+        }
+        for (; t < tiles; t += 4) s0 += src[t * step];
+    }
+    part[slice][lane] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (slice == 0 && d < D) {
+        const float s = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+        if (r < W) {
+            if (dw) dw[r * dw_sr + d] = (T)s;
+        } else if (db) {
+            db[d] = (T)s;
+        }
     }
 }
 
@@ -376,7 +396,7 @@ int conv_bwd_impl(const fla_tensor *x, const fla_tensor *y, const fla_tensor *we
 #undef FLA_LAUNCH_BWD
     FLA_HIP_CHECK(hipGetLastError());
     if (present(dw) || present(db)) {
-        const dim3 rgrid((unsigned)((D + 255) / 256), (unsigned)(W + 1));
+        const dim3 rgrid((unsigned)((D + 63) / 64), (unsigned)(W + 1));
         if (is_bf16)
             FLA_LAUNCH("conv1d_bwd_reduce", stream, conv1d_bwd_reduce_kernel<bf16>, rgrid, dim3(256), 0, stream, p.partial, (int)tiles,
                        (int)W, (int)D, present(dw) ? static_cast<bf16 *>(dw->data) : nullptr, present(dw) ? dw->stride[0] : 0,
