@@ -338,6 +338,32 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * recurrent_kda - replaces aclnnRecurrentKda (kda/recurrent_kda/docs/api.md:56-88;
+ * _aclnn_ctypes.py:1298-1503).  layout "BSND": q,k [B,T,H,K], v,out [B,T,HV,V],
+ * g [B,T,HV,K], beta [B,T,HV]; "TND": the same without B.  q,k,v,out bf16; g, beta
+ * f32/bf16/f16.  initial_state: pool [capacity,HV,V,K] (state_v_first) or
+ * [capacity,HV,K,V], f32 or bf16, slot and head axes may be strided.  cu_seqlens
+ * [seq_num+1], ssm_state_indices (packed [>=T] or [seq_num,max_step]) and
+ * num_accepted_tokens [seq_num] are DEVICE tensors, int32 or int64; their values are
+ * read by the kernel only.  A_log [HV], dt_bias [HV*K] f32 with use_gate_in_kernel.
+ * final_state: the pool the states are written to when inplace_final_state is false.
+ * ------------------------------------------------------------------------ */
+int fla_recurrent_kda_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
+    const fla_tensor *initial_state, const fla_tensor *cu_seqlens, const fla_tensor *ssm_state_indices, const fla_tensor *A_log,
+    const fla_tensor *dt_bias, const fla_tensor *num_accepted_tokens, const char *layout, double scale, bool output_final_state,
+    bool inplace_final_state, bool use_qk_l2norm_in_kernel, bool use_gate_in_kernel, bool use_beta_sigmoid_in_kernel,
+    bool allow_neg_eigval, bool safe_gate, double lower_bound, bool state_v_first, const fla_tensor *attn_out,
+    const fla_tensor *final_state, uint64_t *workspace_size);
+int fla_recurrent_kda(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
+    const fla_tensor *initial_state, const fla_tensor *cu_seqlens, const fla_tensor *ssm_state_indices, const fla_tensor *A_log,
+    const fla_tensor *dt_bias, const fla_tensor *num_accepted_tokens, const char *layout, double scale, bool output_final_state,
+    bool inplace_final_state, bool use_qk_l2norm_in_kernel, bool use_gate_in_kernel, bool use_beta_sigmoid_in_kernel,
+    bool allow_neg_eigval, bool safe_gate, double lower_bound, bool state_v_first, const fla_tensor *attn_out,
+    const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
  * causal_conv1d_bwd - replaces aclnnCausalConv1dBwd (_aclnn_ctypes.py:988-1037;
  * causal_conv1d_bwd/README.md:54-118).  x, dx: logical [B,T,D] or packed [T,D];
  * y (pre-activation, needed when activation is 1 or 2) and dy in input_layout

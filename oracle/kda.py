@@ -211,3 +211,65 @@ def chunk_kda_bwd_intra(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, chunk: in
         db_o[b, :, s:e] += (dl * kc).sum(-1)
         dg_o[b, :, s:e] += qc * dq_delta + kc * (bdl - du)
     return dq_o, dk_o, db_o, dg_o
+
+
+def recurrent_kda(q, k, v, g, beta, initial_state, *, cu_seqlens=None, ssm_state_indices=None, A_log=None, dt_bias=None,
+                  num_accepted_tokens=None, layout="BSND", scale=None, use_qk_l2norm_in_kernel=False,
+                  use_gate_in_kernel=False, use_beta_sigmoid_in_kernel=False, allow_neg_eigval=False, safe_gate=False,
+                  lower_bound=-5.0, state_v_first=False, compute_dtype=torch.float32):
+    """Decode / speculative-decode KDA over a state pool (kda/recurrent_kda/docs/design.md:47-78,155-166 and
+    op_kernel/recurrent_kda.h:270-366,836-870).  Token-major operands: BSND ``q,k [B,T,H,K]``, ``v [B,T,HV,V]``,
+    ``g [B,T,HV,K]``, ``beta [B,T,HV]`` (TND: without B).  ``initial_state`` is the pool ``[capacity,HV,V,K]``
+    (``state_v_first``) or ``[capacity,HV,K,V]``.  Sequence i covers tokens cu[i]..cu[i+1]; it starts from the pool
+    slot of its token ``accepted_i - 1`` (token 0 without ``num_accepted_tokens``; slot i without indices) and
+    after every token the state is stored in that token's slot.  Returns (out, pool after the call)."""
+    tnd = layout == "TND"
+    flat = lambda t: t if tnd else t.reshape(-1, *t.shape[2:])
+    qf, kf, vf, gf, bf = (flat(t).to(compute_dtype) for t in (q, k, v, g, beta))
+    T, H, K = qf.shape
+    HV, V = vf.shape[1], vf.shape[2]
+    rep = HV // H
+    if scale is None:
+        scale = K ** -0.5
+    if use_qk_l2norm_in_kernel:
+        nq, nk = qf.norm(dim=-1, keepdim=True), kf.norm(dim=-1, keepdim=True)
+        qf = torch.where(nq > 0, qf / nq, qf)
+        kf = torch.where(nk > 0, kf / nk, kf)
+    if use_gate_in_kernel:
+        eig = torch.exp(A_log.to(compute_dtype)).view(1, HV, 1)
+        raw = gf if dt_bias is None else gf + dt_bias.to(compute_dtype).reshape(1, HV, K)
+        if safe_gate:
+            gf = float(lower_bound) * torch.sigmoid(eig * raw)
+        else:
+            gf = -eig * torch.nn.functional.softplus(raw)
+    if use_beta_sigmoid_in_kernel:
+        bf = torch.sigmoid(bf)
+        if allow_neg_eigval:
+            bf = 2.0 * bf
+    if cu_seqlens is None:
+        S_len = T if tnd else q.shape[1]
+        cu = list(range(0, T + 1, S_len))
+    else:
+        cu = [int(x) for x in cu_seqlens]
+    pool = initial_state.clone()
+    out = torch.zeros(T, HV, V, dtype=compute_dtype)
+    idx = None if ssm_state_indices is None else ssm_state_indices
+    for n, (s, e) in enumerate(zip(cu, cu[1:])):
+        if e <= s:
+            continue
+        def slot_of(t):
+            if idx is None:
+                return n
+            return int(idx[n, t - s]) if idx.dim() == 2 else int(idx[t])
+        src = s if num_accepted_tokens is None else s + int(num_accepted_tokens[n]) - 1
+        st = initial_state[slot_of(src)].to(compute_dtype)
+        S = st.clone() if state_v_first else st.transpose(-1, -2).clone()          # [HV, V, K]
+        for t in range(s, e):
+            S = S * torch.exp(gf[t])[:, None, :]
+            kt = kf[t].repeat_interleave(rep, dim=0)                               # [HV, K]
+            delta = bf[t][:, None] * (vf[t] - torch.einsum("hvk,hk->hv", S, kt))
+            S = S + delta[:, :, None] * kt[:, None, :]
+            out[t] = torch.einsum("hvk,hk->hv", S, qf[t].repeat_interleave(rep, dim=0) * scale)
+            pool[slot_of(t)] = (S if state_v_first else S.transpose(-1, -2)).to(pool.dtype)
+    out = out.to(v.dtype)
+    return (out if tnd else out.reshape(v.shape)), pool

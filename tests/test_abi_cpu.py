@@ -361,3 +361,69 @@ def test_backward_ops_are_exported_under_both_names():
     from fla_hip import ops
     for name in ("chunk_bwd_dv_local", "chunk_bwd_dqkwg", "prepare_wy_repr_bwd_da", "prepare_wy_repr_bwd_full"):
         assert getattr(ops, name) is getattr(ops, "npu_" + name)
+
+
+def test_conv1d_bwd_and_recurrent_kda_wrappers_operands():
+    """Operand order of fla_causal_conv1d_bwd (= aclnnCausalConv1dBwd, _aclnn_ctypes.py:988-1037) and of
+    fla_recurrent_kda (= aclnnRecurrentKda, :1468-1493); pre-launch checks of the recurrent wrapper."""
+    from fla_hip.ops import _hip_ctypes as H
+    x = FakeFloatTensor((2, 9, 32), torch.bfloat16)
+    w = FakeFloatTensor((4, 32), torch.bfloat16)
+    cap, (dx, dw, db, dh0) = capture_call(H.npu_causal_conv1d_bwd, x, None, w, x, input_layout="BSH")
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == ["x", "y", "weight", "dy", "initial_state", "dht", "dx", "dw", "db", "dh0"]
+    assert cap["args"][7].value == 0 and cap["args"][8].value == b"BSH"
+    assert dx.shape == x.shape and dw.shape == w.shape and db.shape == (32,) and dh0.shape == (2, 4, 32)
+    cap, (_, _, _, dh0) = capture_call(H.npu_causal_conv1d_bwd, FakeFloatTensor((18, 32)), None, w, FakeFloatTensor((2, 18, 16)),
+                                       query_start_loc=[0, 5, 9, 18], input_layout="NTD")
+    assert dh0.shape == (3, 4, 32)
+    with pytest.raises(RuntimeError, match="query_start_loc is required for TND"):
+        capture_call(H.npu_causal_conv1d_bwd, FakeFloatTensor((18, 32)), None, w, FakeFloatTensor((18, 32)), input_layout="TND")
+
+
+class FakeDevTensor(FakeFloatTensor):
+    def __init__(self, shape, dtype=torch.bfloat16, device="cuda:0"):
+        super().__init__(shape, dtype)
+        self.device = device
+
+    def numel(self):
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+
+def test_recurrent_kda_wrapper_checks_and_operands():
+    from fla_hip.ops import _hip_ctypes as H
+    B, T, Hh, HV, K, V = 2, 2, 2, 4, 128, 128
+    q = FakeDevTensor((B, T, Hh, K))
+    v = FakeDevTensor((B, T, HV, V))
+    g = FakeDevTensor((B, T, HV, K), torch.float32)
+    beta = FakeDevTensor((B, T, HV), torch.float32)
+    state = FakeDevTensor((B, HV, V, K), torch.float32)
+    A_log = FakeDevTensor((HV,), torch.float32)
+    cap, (out, final) = capture_call(H.npu_recurrent_kda, q, q, v, g, beta, state, A_log=A_log, use_gate_in_kernel=True,
+                                     output_final_state=True, state_v_first=True)
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"]] == ["q", "k", "v", "g", "beta", "initial_state", "cu_seqlens", "ssm_state_indices", "A_log",
+                                         "dt_bias", "num_accepted_tokens", "attn_out", "final_state"]
+    assert cap["args"][11].value == b"BSND" and cap["args"][12].value == pytest.approx(K ** -0.5)
+    assert cap["args"][13].value is True and cap["args"][14].value is True            # output_final_state, inplace default
+    assert cap["args"][20].value == -5.0 and cap["args"][21].value is True            # lower_bound default, state_v_first
+    assert out.shape == v.shape and final is state
+    _, (_, final) = capture_call(H.npu_recurrent_kda, q, q, v, g, beta, state, state_v_first=True)
+    assert final is None                                                               # output_final_state defaults to False
+    for kwargs, match in (
+        (dict(layout="BNSD"), "layout must be BSND or TND"),
+        (dict(layout="TND"), "layout/rank mismatch"),
+        (dict(state_v_first=True, safe_gate=True), "require use_gate_in_kernel=True"),
+        (dict(state_v_first=True, use_gate_in_kernel=True), r"A_log must be FP32 \[HV\]"),
+        (dict(state_v_first=True, use_gate_in_kernel=True, A_log=A_log, safe_gate=True, lower_bound=-6.0), r"lower_bound must be in \[-5,0\)"),
+        (dict(state_v_first=True, num_accepted_tokens=FakeDevTensor((B,), torch.int32)), "requires ssm_state_indices"),
+    ):
+        with pytest.raises(RuntimeError, match=match):
+            capture_call(H.npu_recurrent_kda, q, q, v, g, beta, state, **kwargs)
+    with pytest.raises(RuntimeError, match="inplace_final_state=True requires initial_state"):
+        capture_call(H.npu_recurrent_kda, q, q, v, g, beta, None)
+    with pytest.raises(RuntimeError, match="HV must be divisible by H"):
+        capture_call(H.npu_recurrent_kda, FakeDevTensor((B, T, 3, K)), FakeDevTensor((B, T, 3, K)), v, g, beta, state, state_v_first=True)

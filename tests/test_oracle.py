@@ -516,3 +516,94 @@ def test_conv1d_bwd_against_autograd():
     dx, dw, db, dh0 = oc.causal_conv1d_bwd(x.detach().float(), None, w.detach().float(), dy.float())
     assert torch.allclose(dx.double(), x.grad, atol=1e-4) and torch.allclose(dw.double(), w.grad, atol=1e-4)
     assert torch.allclose(db.double(), dy.sum((0, 1)), atol=1e-4) and float(dh0.abs().max()) == 0.0
+
+
+# ----------------------------------------------------------------------------
+# recurrent_kda (decode / speculative decode over a state pool)
+# ----------------------------------------------------------------------------
+def test_recurrent_kda_equals_naive_recurrence_and_gate_operator():
+    """Plain case: equals the per-token recurrence already pinned above (head-major, K-first state); the in-kernel
+    options equal applying the (separately pinned) gate activation, F.normalize and sigmoid outside."""
+    gen = torch.Generator().manual_seed(41)
+    B, T, H, HV, K, V = 2, 5, 1, 2, 8, 6
+    q, k = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen)
+    v = torch.randn(B, T, HV, V, generator=gen)
+    g = -torch.rand(B, T, HV, K, generator=gen) * 0.3
+    beta = torch.rand(B, T, HV, generator=gen)
+    h0 = torch.randn(B, HV, K, V, generator=gen) * 0.5
+    out, pool = kda.recurrent_kda(q, k, v, g, beta, h0, scale=0.7)
+    hm = lambda t: t.transpose(1, 2)
+    o_ref, f_ref = kda.naive_recurrent_kda(hm(q), hm(k), hm(v), hm(g), hm(beta), 0.7, initial_state=h0, output_final_state=True)
+    assert torch.allclose(out, hm(o_ref), atol=1e-5) and torch.allclose(pool, f_ref, atol=1e-5)
+    # V-first pool: the transposed state
+    out2, pool2 = kda.recurrent_kda(q, k, v, g, beta, h0.transpose(-1, -2).contiguous(), scale=0.7, state_v_first=True)
+    assert torch.allclose(out2, out, atol=1e-6) and torch.allclose(pool2.transpose(-1, -2), pool, atol=1e-6)
+    # in-kernel options
+    raw = torch.randn(B, T, HV, K, generator=gen)
+    A_log, dt = torch.randn(HV, generator=gen) * 0.3, torch.randn(HV * K, generator=gen) * 0.1
+    braw = torch.randn(B, T, HV, generator=gen)
+    for safe in (False, True):
+        gate = kda.kda_gate(hm(raw), A_log=A_log, dt_bias=dt.view(HV, K), use_gate_in_kernel=True, safe_gate=safe, lower_bound=-3.0)
+        want, wpool = kda.recurrent_kda(F.normalize(q, dim=-1), F.normalize(k, dim=-1), v, hm(gate), 2 * torch.sigmoid(braw), h0, scale=0.7)
+        got, gpool = kda.recurrent_kda(q, k, v, raw, braw, h0, scale=0.7, A_log=A_log, dt_bias=dt, use_qk_l2norm_in_kernel=True,
+                                       use_gate_in_kernel=True, use_beta_sigmoid_in_kernel=True, allow_neg_eigval=True,
+                                       safe_gate=safe, lower_bound=-3.0)
+        assert torch.allclose(got, want, atol=1e-5) and torch.allclose(gpool, wpool, atol=1e-5)
+
+
+def test_recurrent_kda_slots_and_speculative_decoding():
+    """Packed per-token slots: every token's state lands in its slot and one call equals token-by-token calls.
+    Speculative rows [seq, step]: a draft / accept loop reproduces the plain recurrence on the accepted stream."""
+    gen = torch.Generator().manual_seed(42)
+    H, K, V, cap = 2, 8, 6, 9
+    cu = [0, 3, 3, 4, 8]
+    T = cu[-1]
+    q, k, v = (torch.randn(T, H, d, generator=gen) for d in (K, K, V))
+    g = -torch.rand(T, H, K, generator=gen) * 0.3
+    beta = torch.rand(T, H, generator=gen)
+    pool0 = torch.randn(cap, H, V, K, generator=gen) * 0.5
+    slots = torch.tensor([4, 4, 7, 1, 0, 2, 2, 5])
+    out, pool = kda.recurrent_kda(q, k, v, g, beta, pool0, cu_seqlens=cu, ssm_state_indices=slots, layout="TND", state_v_first=True)
+    # token-by-token: each step is its own one-token sequence that starts from the slot the previous token wrote
+    p = pool0.clone()
+    for n, (s, e) in enumerate(zip(cu, cu[1:])):
+        prev = None
+        for t in range(s, e):
+            if prev is not None and int(slots[t]) != prev:
+                p[int(slots[t])] = p[prev]            # the running state moves on to the next slot
+            o1, p = kda.recurrent_kda(q[t:t + 1], k[t:t + 1], v[t:t + 1], g[t:t + 1], beta[t:t + 1], p, cu_seqlens=[0, 1],
+                                      ssm_state_indices=slots[t:t + 1], layout="TND", state_v_first=True)
+            assert torch.allclose(o1[0], out[t], atol=1e-5)
+            prev = int(slots[t])
+    assert torch.allclose(p[[4, 7, 1, 0, 2, 5]], pool[[4, 7, 1, 0, 2, 5]], atol=1e-5)
+    assert torch.equal(pool[[3, 6, 8]], pool0[[3, 6, 8]])            # untouched slots
+    # speculative decoding: two sequences, 3 draft steps each, slot rows fixed across calls
+    S = 3
+    rows = torch.tensor([[0, 1, 2], [3, 4, 5]])
+    truth_len = 12
+    tq, tk, tv = (torch.randn(2, truth_len, H, d, generator=gen) for d in (K, K, V))
+    tg, tb = -torch.rand(2, truth_len, H, K, generator=gen) * 0.3, torch.rand(2, truth_len, H, generator=gen)
+    ref, _ = kda.recurrent_kda(tq, tk, tv, tg, tb, torch.zeros(2, H, V, K), state_v_first=True)
+    pool = torch.zeros(6, H, V, K)
+    pos = [0, 0]
+    accepted = None
+    for step_accept in ([2, 3], [1, 1], [3, 2]):
+        def draft(src, n):
+            d = src[n, pos[n]:pos[n] + S].clone()
+            d[step_accept[n]:] = torch.randn_like(d[step_accept[n]:])      # rejected tail: garbage
+            return d
+        dq, dk, dv, dg, db = (torch.stack([draft(t, 0), draft(t, 1)]) for t in (tq, tk, tv, tg, tb))
+        db = db.abs().clamp(max=1.0)
+        dg = -dg.abs()
+        for n in range(2):      # accepted prefix carries the true values
+            a = step_accept[n]
+            dg[n, :a], db[n, :a] = tg[n, pos[n]:pos[n] + a], tb[n, pos[n]:pos[n] + a]
+        kw = {} if accepted is None else dict(num_accepted_tokens=torch.tensor(accepted))
+        if accepted is None:
+            kw = dict(num_accepted_tokens=torch.tensor([1, 1]))       # slot of step 0 holds the (zero) start state
+        o, pool = kda.recurrent_kda(dq, dk, dv, dg, db, pool, ssm_state_indices=rows, state_v_first=True, **kw)
+        for n in range(2):
+            a = step_accept[n]
+            assert torch.allclose(o[n, :a], ref[n, pos[n]:pos[n] + a], atol=1e-5)
+            pos[n] += a
+        accepted = step_accept
