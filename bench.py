@@ -239,6 +239,23 @@ def bench_decode(args, torch, dev):
         prefill()
     torch.cuda.synchronize()
     pdt = (time.perf_counter() - t2) / 5
+    # the KDA twin of the decode step (per-channel gate, same state tile), V-first fp32 pool in place
+    kg = F.logsigmoid(torch.randn(N, 1, H, D, device=dev, generator=g)) * 0.3
+    kcu = torch.arange(N + 1, dtype=torch.int32, device=dev)
+    kq, kk, kv, kb = q.view(N, 1, H, D), k.view(N, 1, H, D), v.view(N, 1, H, D), beta.view(N, 1, H).float()
+    kda_step = lambda: ops.recurrent_kda(kq, kk, kv, kg, kb, state, cu_seqlens=kcu, state_v_first=True)
+    for _ in range(5):
+        kda_step()
+    lib.fla_profile_enable(1)
+    for _ in range(50):
+        kda_step()
+    torch.cuda.synchronize()
+    lib.fla_profile_enable(0)
+    kn, kms = profile_report(lib)["recurrent_kda"]
+    kda_bytes = 2 * N * H * D * D * 4 + 4 * N * H * D * 2 + N * H * D * 4 + N * H * 4
+    kda_decode = {"kernel": "recurrent_kda", "avg_kernel_ms": round(kms / kn, 4),
+                  "achieved_GBps": round(kda_bytes / (kms / kn * 1e-3) / 1e9, 1),
+                  "frac_of_hbm_peak": round(kda_bytes / (kms / kn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     return {
         "metric": "gdn_decode_tokens_per_s", "value": round(N * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
@@ -250,6 +267,7 @@ def bench_decode(args, torch, dev):
                      "avg_kernel_ms": round(ms / n, 4)},
         "varlen_prefill": {"sequences": 64, "tokens": PT, "ms": round(pdt * 1e3, 3),
                            "tokens_per_s": round(PT / pdt, 1)},
+        "kda_decode": kda_decode,
         "cpu_baseline": cpu,
     }
 
@@ -299,7 +317,30 @@ def bench_conv1d(args, torch, dev):
         cdt = time.perf_counter() - t1
         cpu = {"value": round(B * T * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
                "sample": f"{reps} x (B=4 T=4096 D=4096 W=4) fp32 torch oracle, {cdt:.1f} s"}
+    # backward of the same shape (no activation / SiLU) and the decode-time state update, timed by the same hooks
+    dy = torch.randn(B, T, D, device=dev, generator=g).bfloat16()
+    ypre = torch.randn(B, T, D, device=dev, generator=g).bfloat16()
+    ux = torch.randn(256, D, device=dev, generator=g).bfloat16()
+    ucs = torch.randn(256, W - 1, D, device=dev, generator=g).bfloat16()
+    other = {}
+    for name, fn, nbytes in (
+        ("bwd", lambda: ops.causal_conv1d_bwd(x, None, w, dy), 3 * B * T * D * 2),
+        ("bwd_silu", lambda: ops.causal_conv1d_bwd(x, ypre, w, dy, activation=1), 4 * B * T * D * 2),
+        ("update_256x1", lambda: ops.causal_conv1d(ux, w, b, ucs, activation_mode=1, run_mode=1), 256 * D * 2 * (2 + 2 * (W - 1))),
+    ):
+        for _ in range(3):
+            fn()
+        lib.fla_profile_enable(1)
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        lib.fla_profile_enable(0)
+        kern = {k_: ms_ / n_ for k_, (n_, ms_) in profile_report(lib).items()}
+        total = sum(kern.values())
+        other[name] = {"kernels_ms": {k_: round(v_, 4) for k_, v_ in kern.items()}, "total_ms": round(total, 4),
+                       "algorithmic_GBps": round(nbytes / (total * 1e-3) / 1e9, 1)}
     return {
+        "other_modes": other,
         "metric": "causal_conv1d_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(dt * 1e3 / args.steps, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",

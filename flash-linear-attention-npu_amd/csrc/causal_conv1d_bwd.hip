@@ -125,6 +125,71 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
         }
     };
     seed(t0, n, bos, eos);
+    if (!p.varlen) {
+        // dense rows: eight tokens per batch, all their loads (look-ahead gradient rows, input rows) issued
+        // before the first use; rows past the end are read from a clamped address and zeroed by a select
+        typedef typename Vec8<T>::type V8;
+        for (int tb = t0; tb < t_end; tb += 8) {
+            V8 rdy[8], ry[8], rx[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int u = min(tb + j + W - 1, p.T - 1), t = min(tb + j, p.T - 1);
+                rdy[j] = *reinterpret_cast<const V8 *>(dyb + (int64_t)u * p.g_st);
+                if (yb) ry[j] = *reinterpret_cast<const V8 *>(yb + (int64_t)u * p.g_st);
+                rx[j] = *reinterpret_cast<const V8 *>(xb + (int64_t)t * p.x_st);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = tb + j;
+                if (t >= t_end) break;
+                const bool live = t + W - 1 < p.T;
+                float cur[8], dx[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    float g = (float)rdy[j][c];
+                    if (yb) {
+                        const float yy = (float)ry[j][c];
+                        const float sg = 1.f / (1.f + __expf(-yy));
+                        g *= sg * (1.f + yy * (1.f - sg));
+                    }
+                    gwin[W - 1][c] = live ? g : 0.f;
+                    cur[c] = (float)rx[j][c];
+                }
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int i = 0; i < W; ++i) a = fmaf(gwin[i][c], w[W - 1 - i][c], a);
+                    dx[c] = a;
+                    const float g = gwin[0][c];
+                    db[c] += g;
+                    dw[W - 1][c] = fmaf(g, cur[c], dw[W - 1][c]);
+#pragma unroll
+                    for (int j2 = 0; j2 < W - 1; ++j2) dw[W - 2 - j2][c] = fmaf(g, xwin[j2][c], dw[W - 2 - j2][c]);
+                }
+                if (p.dht) {
+                    const int tail = max(0, p.T - (W - 1));
+                    if (t >= tail) {
+                        float e[8];
+                        ld8(static_cast<const T *>(p.dht) + n * p.d_sn + (int64_t)(1 + t - tail) * p.d_sp + d0, e);
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) dx[c] += e[c];
+                    }
+                }
+                st8(dxb + (int64_t)t * p.dx_st, dx);
+#pragma unroll
+                for (int i = 0; i + 1 < W; ++i)
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) gwin[i][c] = gwin[i + 1][c];
+#pragma unroll
+                for (int j2 = W - 2; j2 > 0; --j2)
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) xwin[j2][c] = xwin[j2 - 1][c];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) xwin[0][c] = cur[c];
+            }
+        }
+    } else
     for (int t = t0; t < t_end; ++t) {
         if (p.varlen && t >= eos) {   // entered the next non-empty sequence
             do {
