@@ -13,7 +13,7 @@ import functools
 import inspect
 from typing import Callable
 
-from ._hip_ctypes import HIP_CTYPES_OPS, gdn_chunk_fwd
+from ._hip_ctypes import HIP_CTYPES_OPS, gdn_chunk_fwd, l2norm_bwd, l2norm_fwd
 
 _REFERENCE_OPS = (
     "npu_fast_gelu_custom",
@@ -153,6 +153,8 @@ def causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=Non
 __all__ = [
     "MUTATED_ARGUMENTS",
     "gdn_chunk_fwd",
+    "l2norm_bwd",
+    "l2norm_fwd",
     *sorted(set(_REFERENCE_OPS)),
     *sorted({_strip_npu_prefix(n) for n in _REFERENCE_OPS}),
 ]

@@ -42,6 +42,8 @@ OP_ARGTYPES = {
     "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
+    "l2norm_fwd": [_T, ctypes.c_double, _T, _T],
+    "l2norm_bwd": [_T, _T, _T, ctypes.c_double, _T],
     "recurrent_kda": [_T] * 11 + [ctypes.c_char_p, ctypes.c_double] + [ctypes.c_bool] * 7 + [ctypes.c_double, ctypes.c_bool, _T, _T],
     "causal_conv1d_bwd": [_T, _T, _T, _T, _T, _T, _IA, ctypes.c_int64, ctypes.c_char_p, _T, _T, _T, _T],
     "chunk_bwd_dv_local": [_T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
@@ -946,6 +948,29 @@ def npu_recurrent_kda(q, k, v, g, beta, initial_state=None, *, cu_seqlens=None, 
         (out, initial_state_work, final_state_work),
     )
     return out, (final_state_work if output_final else None)
+
+
+def l2norm_fwd(x, eps: float = 1e-6, output_dtype=None):
+    """fla/ops/triton/triton_core/l2norm.py:131-178: returns (y, rstd) with rstd fp32 of shape x.shape[:-1]."""
+    import torch
+
+    if output_dtype is not None and output_dtype != x.dtype:
+        raise NotImplementedError("l2norm_fwd: output_dtype must equal the input dtype.")
+    y = _empty_like(x)
+    rstd = _empty(_shape(x)[:-1], x, dtype=torch.float32)
+    _call_op("l2norm_fwd", OP_ARGTYPES["l2norm_fwd"],
+             lambda ctx: [ctx.tensor(x, "x"), ctypes.c_double(float(eps)), ctx.tensor(y, "y"), ctx.tensor(rstd, "rstd")],
+             (y, rstd))
+    return y, rstd
+
+
+def l2norm_bwd(y, rstd, dy, eps: float = 1e-6):
+    """fla/ops/triton/triton_core/l2norm.py:181-224: dx from the normalised output, its rstd and dy."""
+    dx = _empty_like(y)
+    return _call_op("l2norm_bwd", OP_ARGTYPES["l2norm_bwd"],
+                    lambda ctx: [ctx.tensor(y, "y"), ctx.tensor(rstd.contiguous(), "rstd"), ctx.tensor(dy, "dy"),
+                                 ctypes.c_double(float(eps)), ctx.tensor(dx, "dx")],
+                    dx)
 
 
 HIP_CTYPES_OPS = {name: value for name, value in globals().items() if name.startswith("npu_") and callable(value)}

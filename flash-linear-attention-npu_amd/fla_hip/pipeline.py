@@ -94,20 +94,27 @@ def _autograd_function():
 
     class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         @staticmethod
-        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused):
+        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm):
+            q_rstd = k_rstd = None
+            if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049
+                q, q_rstd = _raw.l2norm_fwd(q)
+                k, k_rstd = _raw.l2norm_fwd(k)
             gc, o, A, final = flash_chunk_gated_delta_rule_fwd(
                 q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused)
-            ctx.save_for_backward(q, k, v, gc, beta, A, initial_state)
+            ctx.save_for_backward(q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd)
             ctx.scale, ctx.cu, ctx.chunk_size = scale, cu, chunk_size
             ctx.dtypes = (g.dtype, beta.dtype)
             return o, final
 
         @staticmethod
         def backward(ctx, do, dht):
-            q, k, v, gc, beta, A, initial_state = ctx.saved_tensors
+            q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd = ctx.saved_tensors
             dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
                 q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(), dht, ctx.cu, ctx.chunk_size)
-            return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None
+            if q_rstd is not None:      # :1104-1106
+                dq = _raw.l2norm_bwd(q, q_rstd, dq)
+                dk = _raw.l2norm_bwd(k, k_rstd, dk)
+            return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None, None
 
     return ChunkGatedDeltaRuleFunction
 
@@ -149,8 +156,6 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
         warnings.warn("head_first is kept only for API compatibility. q/k/v are always [B, H, T, D].", stacklevel=2)
     if chunk_size != 2 ** (chunk_size.bit_length() - 1):
         raise ValueError(f"chunk_size must be a power of 2, got {chunk_size}.")
-    if use_qk_l2norm_in_kernel:
-        raise NotImplementedError("use_qk_l2norm_in_kernel is not implemented; pass normalised q and k.")
     cu = _cu_list(cu_seqlens if cu_seqlens is not None else cu_seqlens_list)
     if cu is not None:
         if q.shape[0] != 1:
@@ -166,10 +171,14 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta, initial_state))
     if not needs_grad:
+        if use_qk_l2norm_in_kernel:
+            q, _ = _raw.l2norm_fwd(q)
+            k, _ = _raw.l2norm_fwd(k)
         _, o, _, final = flash_chunk_gated_delta_rule_fwd(
             q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused)
         return o, final
     global _FUNCTION
     if _FUNCTION is None:
         _FUNCTION = _autograd_function()
-    return _FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused)
+    return _FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused,
+                           bool(use_qk_l2norm_in_kernel))

@@ -338,6 +338,22 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * l2norm_fwd / l2norm_bwd - the q/k normalisation of the chunk pipelines, which the reference
+ * runs as Triton kernels (fla/ops/triton/triton_core/l2norm.py:131-224; called from
+ * examples/flash_gated_delta_rule.py:1047-1049,1104-1106).  Rank 2..4 bf16/f16 tensors with
+ * arbitrary outer strides, last extent 64, 128 or 256; rstd fp32, contiguous, one per row.
+ *   fwd: y = x rstd, rstd = 1/sqrt(sum x^2 + eps) (rstd may be NULL);  bwd: dx = (dy - sum(dy y) y) rstd.
+ * ------------------------------------------------------------------------ */
+int fla_l2norm_fwd_get_workspace_size(const fla_tensor *x, double eps, const fla_tensor *y, const fla_tensor *rstd,
+                                      uint64_t *workspace_size);
+int fla_l2norm_fwd(const fla_tensor *x, double eps, const fla_tensor *y, const fla_tensor *rstd, void *workspace,
+                   uint64_t workspace_size, void *stream);
+int fla_l2norm_bwd_get_workspace_size(const fla_tensor *y, const fla_tensor *rstd, const fla_tensor *dy, double eps,
+                                      const fla_tensor *dx, uint64_t *workspace_size);
+int fla_l2norm_bwd(const fla_tensor *y, const fla_tensor *rstd, const fla_tensor *dy, double eps, const fla_tensor *dx,
+                   void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
  * recurrent_kda - replaces aclnnRecurrentKda (kda/recurrent_kda/docs/api.md:56-88;
  * _aclnn_ctypes.py:1298-1503).  layout "BSND": q,k [B,T,H,K], v,out [B,T,HV,V],
  * g [B,T,HV,K], beta [B,T,HV]; "TND": the same without B.  q,k,v,out bf16; g, beta

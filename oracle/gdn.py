@@ -332,3 +332,23 @@ def make_gdn_inputs(B, T, H, K, V, *, dtype=torch.float32, seed=0, Hk=None, init
     if head_first_gates:
         g, beta = g.transpose(1, 2).contiguous(), beta.transpose(1, 2).contiguous()
     return dict(q=q, k=k, v=v, g=g, beta=beta, initial_state=h0)
+
+
+# ----------------------------------------------------------------------------
+# q/k normalisation of the pipeline entry (fla/ops/triton/triton_core/l2norm.py:16-30,93-128)
+# ----------------------------------------------------------------------------
+def l2norm_fwd(x, eps: float = 1e-6, compute_dtype=torch.float32):
+    """y = x * rstd with rstd = 1 / sqrt(sum x^2 + eps) over the last dimension; returns (y, rstd)."""
+    xf = x.to(compute_dtype)
+    ss = torch.zeros(xf.shape[:-1], dtype=compute_dtype)
+    for i in range(xf.shape[-1]):                     # explicit accumulation: not torch.norm
+        ss = ss + xf[..., i] * xf[..., i]
+    rstd = 1.0 / torch.sqrt(ss + eps)
+    return (xf * rstd[..., None]).to(x.dtype), rstd
+
+
+def l2norm_bwd(y, rstd, dy, compute_dtype=torch.float32):
+    """dx = (dy - sum(dy * y) * y) * rstd, y the normalised output."""
+    yf, df = y.to(compute_dtype), dy.to(compute_dtype)
+    dot = (df * yf).sum(-1, keepdim=True)
+    return ((df - dot * yf) * rstd.to(compute_dtype)[..., None]).to(dy.dtype)

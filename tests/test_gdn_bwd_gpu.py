@@ -181,3 +181,54 @@ def test_autograd_through_flash_gated_delta_rule(dev):
     for name, t in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("h0", h0)):
         st = err_stats(t.grad, want[name])
         assert st["rel_max"] <= TOL_BF16, f"d{name}: {st}"
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_l2norm_kernels_against_oracle(dev, D):
+    """Forward and backward of the q/k normalisation on contiguous and on transposed (strided) views."""
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(D)
+    x = torch.randn(2, 37, 3, D, generator=gen).to(BF)
+    dy = torch.randn(2, 37, 3, D, generator=gen).to(BF)
+    for view in (lambda t: t, lambda t: t.transpose(1, 2)):
+        xv, dv_ = view(x), view(dy)
+        y_ref, r_ref = gdn.l2norm_fwd(xv)
+        y, rstd = ops.l2norm_fwd(view(x.to(dev)))
+        assert y.shape == xv.shape and rstd.shape == xv.shape[:-1] and rstd.dtype == torch.float32
+        assert_close(y, y_ref, 1e-2, "y")
+        assert_close(rstd, r_ref, 1e-5, "rstd")
+        dx = ops.l2norm_bwd(y, rstd, view(dy.to(dev)))
+        dx_ref = gdn.l2norm_bwd(y.cpu(), rstd.cpu(), dv_)
+        assert_close(dx, dx_ref, 1e-2, "dx")
+    h = x.to(torch.float16)
+    y, rstd = ops.l2norm_fwd(h.to(dev))
+    assert_close(y, gdn.l2norm_fwd(h)[0], 2e-3, "y f16")
+
+
+def test_pipeline_with_in_kernel_l2norm(dev):
+    """use_qk_l2norm_in_kernel=True: forward equals the recurrence on normalised q, k; gradients reach the
+    UN-normalised q and k (fp64 autograd through F.normalize and the recurrence)."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 1, 150, 2, 128, 128
+    d = make(B, T, H, H, K, V, None, seed=21)
+    gen = torch.Generator().manual_seed(22)
+    qraw = (torch.randn(B, H, T, K, generator=gen) * 1.7).to(BF)
+    kraw = (torch.randn(B, H, T, K, generator=gen) * 0.6).to(BF)
+    dd = torch.float64
+    leaf = {n: t.to(dd).requires_grad_(True) for n, t in (("q", qraw), ("k", kraw), ("v", d["v"]), ("g", d["g"]), ("beta", d["beta"]))}
+    o, _ = gdn.naive_recurrent_gated_delta_rule(F.normalize(leaf["q"], dim=-1), F.normalize(leaf["k"], dim=-1), leaf["v"], leaf["g"],
+                                                leaf["beta"], K ** -0.5, compute_dtype=dd)
+    (o * d["do"].to(dd)).sum().backward()
+    x = to_dev(d, dev)
+    g = x["g"].transpose(1, 2).contiguous()
+    beta = x["beta"].transpose(1, 2).contiguous()
+    # inference path
+    o_inf, _ = pipeline.flash_gated_delta_rule(qraw.to(dev), kraw.to(dev), x["v"], g, beta, use_qk_l2norm_in_kernel=True)
+    assert_close(o_inf.transpose(1, 2), o.detach(), TOL_BF16, "o")
+    # training path
+    q, k, v = (t.to(dev).clone().requires_grad_(True) for t in (qraw, kraw, d["v"]))
+    o_g, _ = pipeline.flash_gated_delta_rule(q, k, v, g, beta, use_qk_l2norm_in_kernel=True)
+    (o_g.float() * x["do"].transpose(1, 2).float()).sum().backward()
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        st = err_stats(t.grad, leaf[name].grad)
+        assert st["rel_max"] <= TOL_BF16, f"d{name}: {st}"

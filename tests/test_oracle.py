@@ -607,3 +607,23 @@ def test_recurrent_kda_slots_and_speculative_decoding():
             assert torch.allclose(o[n, :a], ref[n, pos[n]:pos[n] + a], atol=1e-5)
             pos[n] += a
         accepted = step_accept
+
+
+def test_l2norm_against_F_normalize_and_autograd():
+    gen = torch.Generator().manual_seed(51)
+    x = torch.randn(3, 5, 16, generator=gen, dtype=torch.float64).requires_grad_(True)
+    dy = torch.randn(3, 5, 16, generator=gen, dtype=torch.float64)
+    y, rstd = gdn.l2norm_fwd(x.detach(), eps=0.0, compute_dtype=torch.float64)
+    assert torch.allclose(y, F.normalize(x.detach(), dim=-1), atol=1e-12)          # eps = 0: the unit vector
+    assert torch.allclose(rstd, 1.0 / x.detach().norm(dim=-1), atol=1e-12)
+    eps = 1e-2                                                                    # a visible eps: the Triton kernel's formula
+    ref = x * torch.rsqrt((x * x).sum(-1, keepdim=True) + eps)
+    (ref * dy).sum().backward()
+    y, rstd = gdn.l2norm_fwd(x.detach(), eps=eps, compute_dtype=torch.float64)
+    assert torch.allclose(y, ref.detach(), atol=1e-12)
+    # the backward formula drops the eps term of the exact derivative (as the reference kernel does): exact for eps -> 0
+    x2 = torch.randn(4, 8, generator=gen, dtype=torch.float64).requires_grad_(True)
+    d2 = torch.randn(4, 8, generator=gen, dtype=torch.float64)
+    (F.normalize(x2, dim=-1) * d2).sum().backward()
+    y2, r2 = gdn.l2norm_fwd(x2.detach(), eps=0.0, compute_dtype=torch.float64)
+    assert torch.allclose(gdn.l2norm_bwd(y2, r2, d2, compute_dtype=torch.float64), x2.grad, atol=1e-10)
