@@ -88,7 +88,8 @@ def bench_gdn(args, torch, dev):
     fused = args.route == "fused"
 
     def step():
-        return pipeline.flash_gated_delta_rule(q, k, v, gate, beta, None, h0, True, chunk_size=C, fused=fused)
+        return pipeline.flash_gated_delta_rule(q, k, v, gate, beta, None, h0, True, chunk_size=C, fused=fused,
+                                               use_qk_l2norm_in_kernel=args.l2norm)
 
     for _ in range(args.warmup):
         step()
@@ -155,7 +156,7 @@ def bench_gdn(args, torch, dev):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "GDN chunk forward B=4 T=8192 H=32 K=V=128 chunk=64, fp32 initial+final state",
-                   "route": args.route},
+                   "route": args.route, "use_qk_l2norm_in_kernel": bool(args.l2norm)},
         "step_tflops": round(step_tflops, 2), "step_frac_of_bf16_peak": round(step_tflops / PEAK_BF16_TFLOPS, 4),
         "roofline": roofline, "cpu_baseline": cpu,
     }
@@ -567,6 +568,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--l2norm", action="store_true", help="gdn_chunk: normalise q and k rows inside the kernel")
     ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "gdn_bwd", "decode", "conv1d", "kda", "copy"])
     ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")

@@ -62,6 +62,7 @@ struct FusedParams {
     float scale;
     int slabs;
     int remap;          // 1: co-locate the slabs of one head on one XCD
+    int l2norm;         // 1: q and k rows are L2-normalised (rstd = 1/sqrt(sum x^2 + 1e-6)) while they are staged
 };
 
 template <int K, int CT> struct FusedSmem {
@@ -740,11 +741,26 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int m = 0; m < VCH; ++m) pre_v[m] = __builtin_amdgcn_raw_buffer_load_b128(rv_, (int)voff[m], 0, 0);
         };
+        // A row is held by K/8 adjacent lanes, so its sum of squares is one DPP reduction; the normalised row is
+        // rounded to bf16 exactly where the separate normalisation kernel would have rounded it.
+        auto unit_row = [&](u32x4 raw) -> u32x4 {
+            const bf16x8 a = __builtin_bit_cast(bf16x8, raw);
+            f32x4 lo, hi;
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)a[e];
+                hi[e] = (float)a[4 + e];
+                ss += lo[e] * lo[e] + hi[e] * hi[e];
+            }
+            const float rstd = __builtin_amdgcn_rsqf(group_sum<K / 8>(ss) + 1e-6f);
+            return __builtin_bit_cast(u32x4, frag_from_acc(lo * rstd, hi * rstd));
+        };
         auto commit_qk = [&](const Tiles &t) {
 #pragma unroll
             for (int m = 0; m < QCH; ++m) {
-                *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = pre_q[m];
-                *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = pre_k[m];
+                *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = p.l2norm ? unit_row(pre_q[m]) : pre_q[m];
+                *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = p.l2norm ? unit_row(pre_k[m]) : pre_k[m];
             }
         };
         bf16 *vS = reinterpret_cast<bf16 *>(smem + L::v_off);
@@ -1112,7 +1128,7 @@ int launch_fused(FusedParams &p, hipStream_t stream) {
 
 int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
                double scale, const fla_tensor *initial_state, bool output_final_state, const fla_int_array *cu,
-               int64_t chunk_size, const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
+               int64_t chunk_size, bool use_qk_l2norm, const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
                void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "gdn_chunk_fwd";
     ChunkGeom geom;
@@ -1196,6 +1212,7 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
         FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1],
                     FLA_ERR_SHAPE, "%s: initial_state and final_state must share strides.", op);
     p.scale = (float)scale;
+    p.l2norm = use_qk_l2norm ? 1 : 0;
 
     // 128-column slabs (two 16-column tiles per wave) halve the per-FLOP LDS traffic and do the
     // score / w work once per head; 64-column slabs double the number of workgroups.  Use the
@@ -1206,9 +1223,10 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
         if (atoi(env) == 128 && geom.V % 128 == 0) wide = true;
         if (atoi(env) == 64) wide = false;
     }
+    if (use_qk_l2norm) wide = false;   // the in-kernel normalisation lives in the pipelined kernel's tile commit
     p.slabs = wide ? geom.V / 128 : geom.V / 64;
     bool pipe = !wide;
-    if (const char *env = getenv("FLA_HIP_GDN_PIPE")) pipe = pipe && atoi(env) != 0;   // tuning override
+    if (const char *env = getenv("FLA_HIP_GDN_PIPE")) pipe = pipe && (atoi(env) != 0 || use_qk_l2norm);   // tuning override
     if (pipe) return geom.K == 128 ? launch_pipe<128>(p, stream) : launch_pipe<64>(p, stream);
     if (geom.K == 128) return wide ? launch_fused<128, 2>(p, stream) : launch_fused<128, 1>(p, stream);
     return wide ? launch_fused<64, 2>(p, stream) : launch_fused<64, 1>(p, stream);
@@ -1221,18 +1239,21 @@ extern "C" int fla_gdn_chunk_fwd_get_workspace_size(const fla_tensor *q, const f
                                                     const fla_tensor *g, const fla_tensor *beta, double scale,
                                                     const fla_tensor *initial_state, bool output_final_state,
                                                     const fla_int_array *cu_seqlens, int64_t chunk_size,
-                                                    const fla_tensor *o, const fla_tensor *g_cumsum,
-                                                    const fla_tensor *final_state, uint64_t *workspace_size) {
+                                                    bool use_qk_l2norm_in_kernel, const fla_tensor *o,
+                                                    const fla_tensor *g_cumsum, const fla_tensor *final_state,
+                                                    uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd: workspace_size must not be null.");
-    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, o,
+    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
+                           use_qk_l2norm_in_kernel, o,
                            g_cumsum, final_state, nullptr, 0, nullptr, workspace_size);
 }
 
 extern "C" int fla_gdn_chunk_fwd(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
                                  const fla_tensor *beta, double scale, const fla_tensor *initial_state,
                                  bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
-                                 const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
-                                 void *workspace, uint64_t workspace_size, void *stream) {
-    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, o,
+                                 bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
+                                 const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
+    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
+                           use_qk_l2norm_in_kernel, o,
                            g_cumsum, final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }

@@ -32,7 +32,8 @@ OP_ARGTYPES = {
     "chunk_gated_delta_rule_fwd_h": [_T, _T, _T, _T, _T, _T, ctypes.c_bool, ctypes.c_int64, _IA, _IA,
                                      ctypes.c_bool, _T, _T, _T],
     "chunk_fwd_o": [_T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
-    "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, _T, _T, _T],
+    "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, ctypes.c_bool,
+                      _T, _T, _T],
     "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
@@ -383,9 +384,11 @@ def npu_solve_tri(x, *, cu_seqlens=None, chunk_indices=None, layout="bsnd"):
     )
 
 
-def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size):
+def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
+                  use_qk_l2norm_in_kernel=False):
     """Whole chunk forward in one library call (replaces the composition at
     examples/flash_gated_delta_rule.py:796-881).  q,k,v [B,H,T,D]; g,beta [B,T,H] f32.
+    use_qk_l2norm_in_kernel normalises q and k rows inside the kernel (flash_gated_delta_rule.py:1047-1049).
     Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], final_state or None)."""
     import torch
 
@@ -402,6 +405,7 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
             ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"),
             ctx.tensor(beta, "beta"), ctypes.c_double(float(scale)), ctx.tensor(initial_state, "initial_state"),
             ctypes.c_bool(bool(output_final_state)), ctx.int_array(cu), ctypes.c_int64(int(chunk_size)),
+            ctypes.c_bool(bool(use_qk_l2norm_in_kernel)),
             ctx.tensor(o, "o"), ctx.tensor(g_out, "g_cumsum"), ctx.tensor(final, "final_state"),
         ],
         (o, g_out, final),

@@ -31,16 +31,22 @@ def _cu_list(cu_seqlens):
 
 
 def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
-                                     cu_seqlens=None, chunk_size: int = 64, *, fused: bool = True):
+                                     cu_seqlens=None, chunk_size: int = 64, *, fused: bool = True,
+                                     use_qk_l2norm_in_kernel: bool = False):
     """q,k,v [B,H,T,D] bf16; g,beta [B,T,H].  Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], A, final_state);
-    ``A`` ([B,H,T,C] bf16, the inverted chunk matrices) is None on the fused route."""
+    ``A`` ([B,H,T,C] bf16, the inverted chunk matrices) is None on the fused route.  With
+    ``use_qk_l2norm_in_kernel`` the fused route normalises q and k rows while it stages them; the composed
+    route runs the two normalisation passes first (examples/flash_gated_delta_rule.py:1047-1049)."""
     import torch
 
     cu = _cu_list(cu_seqlens)
     if fused:
         gc, o, final = _raw.gdn_chunk_fwd(q, k, v, g.float(), beta.float(), scale, initial_state,
-                                          output_final_state, cu, chunk_size)
+                                          output_final_state, cu, chunk_size, use_qk_l2norm_in_kernel)
         return gc, o, None, final
+    if use_qk_l2norm_in_kernel:
+        q, _ = _raw.l2norm_fwd(q)
+        k, _ = _raw.l2norm_fwd(k)
     # reference composition (examples/flash_gated_delta_rule.py:811-881)
     gh = _ops.chunk_local_cumsum(g.transpose(1, 2).contiguous(), chunk_size, cu_seqlens=cu,
                                  head_first=True, output_dtype=torch.float32)
@@ -171,11 +177,9 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta, initial_state))
     if not needs_grad:
-        if use_qk_l2norm_in_kernel:
-            q, _ = _raw.l2norm_fwd(q)
-            k, _ = _raw.l2norm_fwd(k)
         _, o, _, final = flash_chunk_gated_delta_rule_fwd(
-            q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused)
+            q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused,
+            use_qk_l2norm_in_kernel=use_qk_l2norm_in_kernel)
         return o, final
     global _FUNCTION
     if _FUNCTION is None:

@@ -180,19 +180,22 @@ int fla_chunk_fwd_o(
  * pipeline passes them; initial_state [N,Hv,K,V] f32 or NULL.
  * Outputs: o [B,T,Hv,V] bf16, g_cumsum [B,T,Hv] f32 (may be NULL),
  * final_state [N,Hv,K,V] f32 (NULL unless output_final_state).
+ * use_qk_l2norm_in_kernel: q and k rows are scaled by 1/sqrt(sum x^2 + 1e-6)
+ * while they are staged, as fla's l2norm_fwd does ahead of the chunk forward
+ * (examples/flash_gated_delta_rule.py:1086-1089).
  * ------------------------------------------------------------------------ */
 int fla_gdn_chunk_fwd_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, double scale, const fla_tensor *initial_state,
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
-    const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
-    uint64_t *workspace_size);
+    bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
+    const fla_tensor *final_state, uint64_t *workspace_size);
 int fla_gdn_chunk_fwd(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, double scale, const fla_tensor *initial_state,
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
-    const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
-    void *workspace, uint64_t workspace_size, void *stream);
+    bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
+    const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
  * recurrent_gated_delta_rule - replaces aclnnRecurrentGatedDeltaRule
