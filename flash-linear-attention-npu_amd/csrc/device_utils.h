@@ -12,7 +12,18 @@ typedef _Float16 f16;
 typedef bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
 typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+// Element type of the matrix operands of a translation unit: bf16, or f16 when the file is built with
+// -DFLA_ELEM_F16 (the matrix-core kernels are compiled once per element type).
+#ifdef FLA_ELEM_F16
+typedef f16 elem;
+#else
+typedef bf16 elem;
+#endif
+typedef elem elemx2 __attribute__((ext_vector_type(2)));
+typedef elem elemx4 __attribute__((ext_vector_type(4)));
+typedef elem elemx8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -90,33 +101,46 @@ __device__ __forceinline__ float read_lane(float v, int lane) {  // lane must be
 __device__ __forceinline__ f32x4 mfma16x32(bf16x8 a, bf16x8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
+__device__ __forceinline__ f32x4 mfma16x32(f16x8 a, f16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
 // v_mfma_f32_16x16x16_bf16: A lane l holds A[l%16][4*(l/16)+e], B lane l holds
-// B[4*(l/16)+e][l%16], e = 0..3; D as above.  A D tile rounded to bf16 is
+// B[4*(l/16)+e][l%16], e = 0..3; D as above.  A D tile rounded to the element type is
 // therefore directly the B operand (rows = contraction) of a following MFMA.
 __device__ __forceinline__ f32x4 mfma16x16(bf16x4 a, bf16x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c,
                                                      0, 0, 0);
 }
-
-// fp32 -> bf16 (round to nearest even), two values per v_cvt_pk_bf16_f32
-__device__ __forceinline__ bf16x2 cvt2(float a, float b) {
-    const f32x2 v = {a, b};
-    return __builtin_convertvector(v, bf16x2);
+__device__ __forceinline__ f32x4 mfma16x16(f16x4 a, f16x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
 }
-// The two packed halves are joined as integers: joined as bf16 vectors the optimiser folds them into
-// one <4 x bf16> conversion, which the backend then splits into four scalar conversions plus permutes.
-__device__ __forceinline__ bf16x4 cvt4(f32x4 v) {
+
+// fp32 -> element type (round to nearest even), two values per packed conversion
+__device__ __forceinline__ elemx2 cvt2(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_convertvector(v, elemx2);
+}
+// The two packed halves are joined as integers: joined as element vectors the optimiser folds them into
+// one four-wide conversion, which the backend then splits into four scalar conversions plus permutes.
+__device__ __forceinline__ elemx4 cvt4(f32x4 v) {
     u32x2 t;
     t[0] = __builtin_bit_cast(unsigned, cvt2(v[0], v[1]));
     t[1] = __builtin_bit_cast(unsigned, cvt2(v[2], v[3]));
-    return __builtin_bit_cast(bf16x4, t);
+    return __builtin_bit_cast(elemx4, t);
 }
-// x = hi + lo with hi = bf16(x) and lo = bf16(x - hi).  The remainder is formed from the packed
-// conversion's bit pattern (a bf16 is the upper half of an fp32), never by extracting vector
-// elements: element extraction makes the optimiser split the packed conversion into four scalar
-// ones plus permutes.
-__device__ __forceinline__ void split_hilo(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
-    const bf16x2 h01 = cvt2(x[0], x[1]), h23 = cvt2(x[2], x[3]);
+// x = hi + lo with hi = elem(x) and lo = elem(x - hi).
+__device__ __forceinline__ void split_hilo(f32x4 x, elemx4 &hi, elemx4 &lo) {
+#ifdef FLA_ELEM_F16
+    hi = cvt4(x);
+    f32x4 rem;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) rem[e] = x[e] - (float)hi[e];
+    lo = cvt4(rem);
+#else
+    // The remainder is formed from the packed conversion's bit pattern (a bf16 is the upper half of an
+    // fp32), never by extracting vector elements: element extraction makes the optimiser split the packed
+    // conversion into four scalar ones plus permutes.
+    const elemx2 h01 = cvt2(x[0], x[1]), h23 = cvt2(x[2], x[3]);
     const unsigned u01 = __builtin_bit_cast(unsigned, h01), u23 = __builtin_bit_cast(unsigned, h23);
     f32x4 rem;
     rem[0] = x[0] - __builtin_bit_cast(float, u01 << 16);
@@ -126,10 +150,11 @@ __device__ __forceinline__ void split_hilo(f32x4 x, bf16x4 &hi, bf16x4 &lo) {
     u32x2 t;
     t[0] = u01;
     t[1] = u23;
-    hi = __builtin_bit_cast(bf16x4, t);
+    hi = __builtin_bit_cast(elemx4, t);
     lo = cvt4(rem);
+#endif
 }
-__device__ __forceinline__ bf16x8 cat8(bf16x4 lo, bf16x4 hi) {
+__device__ __forceinline__ elemx8 cat8(elemx4 lo, elemx4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 

@@ -39,10 +39,10 @@ template <int K, int V>
 __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 8, pv = V + 16, pa = kChunk + 8;
-    bf16 *qS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = qS + kChunk * pk;
-    bf16 *oS = kS + kChunk * pk;
-    bf16 *aS = oS + kChunk * pv;
+    elem *qS = reinterpret_cast<elem *>(smem);
+    elem *kS = qS + kChunk * pk;
+    elem *oS = kS + kChunk * pk;
+    elem *aS = oS + kChunk * pv;
     float *gS = reinterpret_cast<float *>(aS + kChunk * pa);
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
@@ -53,9 +53,9 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
     {
         TileCopy<kThreads, kChunk, K> tq, tk;
         TileCopy<kThreads, kChunk, V> to;
-        tq.fetch(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
-        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-        to.fetch(static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+        tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
         stage_scalars(gS, p.g, b, hv, start, len);
         tq.commit(qS, pk, len, tid);
         tk.commit(kS, pk, len, tid);
@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
         acc_to_tile(aS, pa, 16 * w, 16 * ct, acc);
     }
     __syncthreads();
-    char *dvg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+    char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
                                          (int64_t)start * p.dv.st);
 #pragma unroll
     for (int ct = 0; ct < V / 16; ++ct) {
@@ -100,7 +100,7 @@ struct DqkwgParams {
     ChunkGeom geom;
     View4 q, k, v, d_o, dv, dq, dk, dw;
     View3 g;
-    const bf16 *h, *dh;
+    const elem *h, *dh;
     int64_t h_sb, h_sh, h_sc, dh_sb, dh_sh, dh_sc;
     float *dg;
     int64_t dg_sb, dg_sh, dg_st;
@@ -112,13 +112,13 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
     constexpr int KT = K / 16;
-    bf16 *qS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = qS + kChunk * pk;
-    bf16 *vS = kS + kChunk * pk;
-    bf16 *oS = vS + kChunk * pv;       // do
-    bf16 *dvS = oS + kChunk * pv;
-    bf16 *hS = dvS + kChunk * pv;      // h, then dh
-    bf16 *sS = hS + K * pv;            // ds
+    elem *qS = reinterpret_cast<elem *>(smem);
+    elem *kS = qS + kChunk * pk;
+    elem *vS = kS + kChunk * pk;
+    elem *oS = vS + kChunk * pv;       // do
+    elem *dvS = oS + kChunk * pv;
+    elem *hS = dvS + kChunk * pv;      // h, then dh
+    elem *sS = hS + K * pv;            // ds
     float *gS = reinterpret_cast<float *>(sS + kChunk * ps);
     float *red = gS + kChunk;          // 8 partial sums
 
@@ -129,8 +129,8 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
     {
         TileCopy<kThreads, kChunk, K> tq, tk;
-        tq.fetch(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
-        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+        tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
         tq.commit(qS, pk, len, tid);
         tk.commit(kS, pk, len, tid);
     }
@@ -146,9 +146,9 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
         {
             TileCopy<kThreads, kChunk, V> tv, to, tdv;
             TileCopy<kThreads, K, V> th;
-            tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
-            to.fetch(static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
-            tdv.fetch(static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+            to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+            tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
             th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
             tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
             stage_scalars(gS, p.g, b, hv, start, len);
@@ -158,7 +158,7 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
             th.commit(hS, pv, K, tid);
 #pragma unroll
             for (int m = 0; m < TileCopy<kThreads, K, V>::N; ++m) {
-                const bf16x8 a = __builtin_bit_cast(bf16x8, th.r[m]), d = __builtin_bit_cast(bf16x8, tdh.r[m]);
+                const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) hd += (float)a[e] * (float)d[e];
             }
@@ -166,14 +166,14 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
         __syncthreads();
         // ---- products with the state at chunk start: dq (state part), dw; and the ds tile -------------
         f32x4 dqs[KT];
-        char *dwg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
+        char *dwg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
                                              (int64_t)start * p.dw.st);
 #pragma unroll
         for (int ct = 0; ct < KT; ++ct) {
             f32x4 a = zero4(), d = zero4();
 #pragma unroll
             for (int j = 0; j < V / 32; ++j) {
-                const bf16x8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
+                const elemx8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
                 a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
                 d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
             }
@@ -257,8 +257,8 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
                 p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st] = v + (row == len - 1 ? dg_last : 0.f);
         }
     }
-    char *dqg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
-    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+    char *dqg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
+    char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
 #pragma unroll
     for (int ct = 0; ct < KT; ++ct) {
         acc_to_global(dqg + 32 * ct, p.dq.st * 2, 16 * w, len, dq_acc[ct]);
@@ -279,13 +279,13 @@ struct WyBwdParams {
 
 // Commits a fetched tile with every row scaled by f[row] (rows past `len` become zero).
 template <int NCOLS>
-__device__ __forceinline__ void commit_scaled(const TileCopy<kThreads, kChunk, NCOLS> &t, bf16 *dst, int pitch, int len,
+__device__ __forceinline__ void commit_scaled(const TileCopy<kThreads, kChunk, NCOLS> &t, elem *dst, int pitch, int len,
                                               const float *f, int tid) {
 #pragma unroll
     for (int m = 0; m < TileCopy<kThreads, kChunk, NCOLS>::N; ++m) {
         const int idx = m * kThreads + tid;
         const int r = idx / (NCOLS / 8), c8 = (idx % (NCOLS / 8)) << 3;
-        const bf16x8 a = __builtin_bit_cast(bf16x8, t.r[m]);
+        const elemx8 a = __builtin_bit_cast(elemx8, t.r[m]);
         const float s = r < len ? f[r] : 0.f;
         f32x4 lo, hi;
 #pragma unroll
@@ -293,24 +293,24 @@ __device__ __forceinline__ void commit_scaled(const TileCopy<kThreads, kChunk, N
             lo[e] = (float)a[e] * s;
             hi[e] = (float)a[4 + e] * s;
         }
-        *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
+        *reinterpret_cast<elemx8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
     }
 }
 // Commits a 64 x 64 chunk matrix, zeroing rows and columns past the tail; with `colf` every column j is
 // also scaled by colf[j].
-__device__ __forceinline__ void commit_square(const TileCopy<kThreads, kChunk, kChunk> &t, bf16 *dst, int pitch, int len,
+__device__ __forceinline__ void commit_square(const TileCopy<kThreads, kChunk, kChunk> &t, elem *dst, int pitch, int len,
                                               const float *colf, int tid) {
 #pragma unroll
     for (int m = 0; m < TileCopy<kThreads, kChunk, kChunk>::N; ++m) {
         const int idx = m * kThreads + tid;
         const int r = idx >> 3, c8 = (idx & 7) << 3;
-        bf16x8 a = __builtin_bit_cast(bf16x8, t.r[m]);
+        elemx8 a = __builtin_bit_cast(elemx8, t.r[m]);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const bool in = r < len && c8 + e < len;
-            a[e] = in ? (colf ? (bf16)((float)a[e] * colf[c8 + e]) : a[e]) : (bf16)0.f;
+            a[e] = in ? (colf ? (elem)((float)a[e] * colf[c8 + e]) : a[e]) : (elem)0.f;
         }
-        *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = a;
+        *reinterpret_cast<elemx8 *>(dst + r * pitch + c8) = a;
     }
 }
 
@@ -318,15 +318,15 @@ template <int K, int V>
 __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 8, pv = V + 8, pa = kChunk + 8;
-    bf16 *dwS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = dwS + kChunk * pk;
-    bf16 *duS = kS + kChunk * pk;
-    bf16 *vS = duS + kChunk * pv;
-    bf16 *aS = vS + kChunk * pv;
+    elem *dwS = reinterpret_cast<elem *>(smem);
+    elem *kS = dwS + kChunk * pk;
+    elem *duS = kS + kChunk * pk;
+    elem *vS = duS + kChunk * pv;
+    elem *aS = vS + kChunk * pv;
     // the two intermediate 64 x 64 matrices reuse the dw and du tiles, which are dead by then: the kernel
     // stays under half of a compute unit's LDS, so two workgroups overlap their load and compute phases
-    bf16 *m4S = dwS;
-    bf16 *m5S = duS;
+    elem *m4S = dwS;
+    elem *m5S = duS;
     float *gS = reinterpret_cast<float *>(aS + kChunk * pa);
     float *bS = gS + kChunk;
     float *fS = bS + kChunk;           // beta e^G
@@ -340,11 +340,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
         TileCopy<kThreads, kChunk, K> tdw, tk;
         TileCopy<kThreads, kChunk, V> tdu, tv;
         TileCopy<kThreads, kChunk, kChunk> ta;
-        tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
-        tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-        tdu.fetch(static_cast<const bf16 *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
-        tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
-        ta.fetch(static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
+        tdw.fetch(static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+        tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+        tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
+        tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+        ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
         if (tid < kChunk) {
             const int t = start + min(tid, len - 1);
             const float gg = load_scalar(p.g, b, hv, t), bb = load_scalar(p.beta, b, hv, t);
@@ -393,7 +393,7 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
     }
     __syncthreads();
     // (A^T M5)^T = M5^T A, gated, negated and masked; rows of this product are the stored rows
-    char *dag = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dA.p)) + b * p.dA.sb + hv * p.dA.sh +
+    char *dag = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dA.p)) + b * p.dA.sb + hv * p.dA.sh +
                                          (int64_t)start * p.dA.st);
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct) {
@@ -426,12 +426,12 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     constexpr int KV = K > V ? K : V;
     constexpr int pk = K + 16, px = KV + 16, pvv = V, pa = kChunk + 8;
     constexpr int KT = K / 16, VT = V / 16;
-    bf16 *kS = reinterpret_cast<bf16 *>(smem);
-    bf16 *xS = kS + kChunk * pk;        // du, then dw
-    bf16 *vS = xS + kChunk * px;
-    bf16 *aS = vS + kChunk * pvv;
-    bf16 *dS = aS + kChunk * pa;        // dA as stored
-    bf16 *dbS = dS + kChunk * pa;       // dA with column j scaled by beta_j
+    elem *kS = reinterpret_cast<elem *>(smem);
+    elem *xS = kS + kChunk * pk;        // du, then dw
+    elem *vS = xS + kChunk * px;
+    elem *aS = vS + kChunk * pvv;
+    elem *dS = aS + kChunk * pa;        // dA as stored
+    elem *dbS = dS + kChunk * pa;       // dA with column j scaled by beta_j
     float *gS = reinterpret_cast<float *>(dbS + kChunk * pa);
     float *bS = gS + kChunk;
 
@@ -441,11 +441,11 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
     TileCopy<kThreads, kChunk, K> tk;
-    tk.fetch(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+    tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
     f32x4 dk_acc[GVA ? KT : 1];
 #pragma unroll
     for (int ct = 0; ct < (GVA ? KT : 1); ++ct) dk_acc[ct] = zero4();
-    char *dkg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+    char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
@@ -454,10 +454,10 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
         {
             TileCopy<kThreads, kChunk, V> tdu, tv;
             TileCopy<kThreads, kChunk, kChunk> ta, td;
-            tdu.fetch(static_cast<const bf16 *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
-            tv.fetch(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
-            ta.fetch(static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
-            td.fetch(static_cast<const bf16 *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
+            tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
+            tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+            ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
+            td.fetch(static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
             if (tid < kChunk) {
                 const int t = start + min(tid, len - 1);
                 gS[tid] = load_scalar(p.g, b, hv, t);
@@ -472,7 +472,7 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             commit_square(td, dbS, pa, len, bS, tid);
         }
         // dw is fetched only now, once the registers of the first batch are free; it lands during A^T du
-        tdw.fetch(static_cast<const bf16 *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+        tdw.fetch(static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
         __syncthreads();
         float br[4], er[4];
 #pragma unroll
@@ -481,8 +481,8 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             er[e] = __expf(gS[16 * w + 4 * lg + e]);
         }
         float db_row[4] = {0.f, 0.f, 0.f, 0.f}, dg_row[4] = {0.f, 0.f, 0.f, 0.f};
-        const bf16x8 at0 = frag_tr(aS, pa, 16 * w, 0), at1 = frag_tr(aS, pa, 16 * w, 32);
-        char *dvg = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+        const elemx8 at0 = frag_tr(aS, pa, 16 * w, 0), at1 = frag_tr(aS, pa, 16 * w, 32);
+        char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
                                              (int64_t)start * p.dv.st);
 #pragma unroll
         for (int ct = 0; ct < VT; ++ct) {      // A^T du
@@ -499,11 +499,11 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
         __syncthreads();                 // du has been consumed by every wave
         tdw.commit(xS, px, len, tid);
         __syncthreads();
-        const bf16x8 dt0 = frag_tr(dS, pa, 16 * w, 0), dt1 = frag_tr(dS, pa, 16 * w, 32);
-        const bf16x8 db0 = frag_kc(dbS, pa, 16 * w, 0), db1 = frag_kc(dbS, pa, 16 * w, 32);
+        const elemx8 dt0 = frag_tr(dS, pa, 16 * w, 0), dt1 = frag_tr(dS, pa, 16 * w, 32);
+        const elemx8 db0 = frag_kc(dbS, pa, 16 * w, 0), db1 = frag_kc(dbS, pa, 16 * w, 32);
 #pragma unroll
         for (int ct = 0; ct < KT; ++ct) {
-            const bf16x8 k0 = frag_tr(kS, pk, 16 * ct, 0), k1 = frag_tr(kS, pk, 16 * ct, 32);
+            const elemx8 k0 = frag_tr(kS, pk, 16 * ct, 0), k1 = frag_tr(kS, pk, 16 * ct, 32);
             f32x4 p1 = mfma16x32(at0, frag_tr(xS, px, 16 * ct, 0), zero4());        // A^T dw
             p1 = mfma16x32(at1, frag_tr(xS, px, 16 * ct, 32), p1);
             f32x4 p2 = mfma16x32(dt0, k0, zero4());                                 // dA^T k
@@ -559,7 +559,7 @@ int check_f32_bht(const char *op, const char *name, const fla_tensor *t, const C
 }
 
 int check_state5(const char *op, const char *name, const fla_tensor *h, const ChunkGeom &geom) {
-    int rc = check_tensor(h, op, name, 5, dt_bit(FLA_BF16));
+    int rc = check_tensor(h, op, name, 5, dt_bit(kElemDtype));
     if (rc) return rc;
     FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
                     h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 8 == 0 &&
@@ -577,14 +577,14 @@ int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_
     (void)A;   // accepted and unused, as in the reference kernel
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, d_o, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, d_o, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "out", out, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
@@ -611,8 +611,8 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     (void)w;   // the reference accepts w and does not read it
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
@@ -622,7 +622,7 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "dw", dw, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if ((rc = check_f32_bht(op, "dg", dg, geom))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
@@ -631,7 +631,7 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (query) return FLA_OK;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     DqkwgParams p{geom, view4(q), view4(k), view4(v), view4(d_o), view4(dv), view4(dq), view4(dk), view4(dw), view3(g),
-                  static_cast<const bf16 *>(h->data), static_cast<const bf16 *>(dh->data),
+                  static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                   h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                   static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
     const dim3 grid(geom.NT, geom.Hk, geom.B);
@@ -650,8 +650,8 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
 int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
                   const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, int64_t chunk_size, ChunkGeom &geom) {
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
@@ -659,8 +659,8 @@ int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, cons
     if ((rc = check_bhtd(op, "du", du, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr && beta != nullptr && beta->data != nullptr, FLA_ERR_NULL,
                 "%s: g and beta must be provided.", op);
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
-    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     return FLA_OK;
 }
 
@@ -672,7 +672,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
     ChunkGeom geom;
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
-    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, dt_bit(kElemDtype)))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
@@ -697,7 +697,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     ChunkGeom geom;
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
     if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
@@ -722,79 +722,144 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
 }
 
+// da + full in one call: dA (bf16, transposed like the stand-alone operator writes it) lives in the caller's workspace
+// behind the shared variable-length metadata.
+int wy_bwd_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
+                const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu,
+                const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+                const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream,
+                uint64_t *query) {
+    const char *op = "prepare_wy_repr_bwd";
+    if (!A) return fail(FLA_ERR_NULL, "%s: A must not be null.", op);
+    fla_tensor dA = *A;     // same shape; contiguous [B,Hv,T,C] bf16
+    dA.data = nullptr;
+    int64_t st = 1;
+    for (int d = dA.ndim - 1; d >= 0; --d) {
+        dA.stride[d] = st;
+        st *= dA.shape[d];
+    }
+    uint64_t meta_da = 0, meta_full = 0;
+    int rc;
+    dA.data = const_cast<void *>(A->data);  // a non-null stand-in for the size queries
+    if ((rc = wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu, ci, chunk_size, &dA, nullptr, 0, nullptr, &meta_da))) return rc;
+    if ((rc = wy_bwd_full_impl(k, v, beta, A, &dA, dw, du, g, cu, ci, chunk_size, dk, dv, dbeta, dg, nullptr, 0, nullptr,
+                               &meta_full)))
+        return rc;
+    const uint64_t meta = ((meta_da > meta_full ? meta_da : meta_full) + 255) & ~(uint64_t)255;
+    const uint64_t need = meta + (uint64_t)st * 2;
+    if (query) {
+        *query = need;
+        return FLA_OK;
+    }
+    if (st == 0) return FLA_OK;
+    if (!ws || ws_size < need) return fail(FLA_ERR_WORKSPACE, "%s: workspace of %llu bytes needed, %llu given.", op,
+                                           (unsigned long long)need, (unsigned long long)ws_size);
+    dA.data = static_cast<char *>(ws) + meta;
+    if ((rc = wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu, ci, chunk_size, &dA, ws, meta, stream, nullptr))) return rc;
+    return wy_bwd_full_impl(k, v, beta, A, &dA, dw, du, g, cu, ci, chunk_size, dk, dv, dbeta, dg, ws, meta, stream, nullptr);
+}
+
 }  // namespace
 }  // namespace fla
 
 #define FLA_NULL_WS(op) \
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, op ": workspace_size must not be null.")
 
-extern "C" int fla_chunk_bwd_dv_local_get_workspace_size(
+FLA_ENTRY(fla_chunk_bwd_dv_local_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
     const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
     int64_t chunk_size, const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dv_local_get_workspace_size, q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_bwd_dv_local");
     return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0,
                               nullptr, workspace_size);
 }
-extern "C" int fla_chunk_bwd_dv_local(
+FLA_ENTRY(fla_chunk_bwd_dv_local)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
     const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
     int64_t chunk_size, const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dv_local, q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size, stream);
     return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace,
                               workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_chunk_bwd_dqkwg_get_workspace_size(
+FLA_ENTRY(fla_chunk_bwd_dqkwg_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
     const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
     bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
     const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg_get_workspace_size, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2, transpose_state_layout, dq, dk, dw, dg, workspace_size);
     FLA_NULL_WS("chunk_bwd_dqkwg");
     return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
                            transpose_state_layout, dq, dk, dw, dg, nullptr, 0, nullptr, workspace_size);
 }
-extern "C" int fla_chunk_bwd_dqkwg(
+FLA_ENTRY(fla_chunk_bwd_dqkwg)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
     const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
     bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
     const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2, transpose_state_layout, dq, dk, dw, dg, workspace, workspace_size, stream);
     return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
                            transpose_state_layout, dq, dk, dw, dg, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_prepare_wy_repr_bwd_da_get_workspace_size(
+FLA_ENTRY(fla_prepare_wy_repr_bwd_da_get_workspace_size)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
     const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
     int64_t chunk_size, const fla_tensor *dA, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_da_get_workspace_size, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd_da");
     return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, nullptr, 0, nullptr,
                                workspace_size);
 }
-extern "C" int fla_prepare_wy_repr_bwd_da(
+FLA_ENTRY(fla_prepare_wy_repr_bwd_da)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
     const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
     int64_t chunk_size, const fla_tensor *dA, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_da, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace, workspace_size, stream);
     return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace,
                                workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_prepare_wy_repr_bwd_full_get_workspace_size(
+FLA_ENTRY(fla_prepare_wy_repr_bwd_full_get_workspace_size)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
     const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_get_workspace_size, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd_full");
     return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
                                  nullptr, 0, nullptr, workspace_size);
 }
-extern "C" int fla_prepare_wy_repr_bwd_full(
+FLA_ENTRY(fla_prepare_wy_repr_bwd_full)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
     const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
     return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
                                  workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}
+
+FLA_ENTRY(fla_prepare_wy_repr_bwd_get_workspace_size)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg,
+    uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_get_workspace_size, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
+    FLA_NULL_WS("prepare_wy_repr_bwd");
+    return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, nullptr, 0,
+                            nullptr, workspace_size);
+}
+FLA_ENTRY(fla_prepare_wy_repr_bwd)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg,
+    void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
+    return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace,
+                            workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }

@@ -29,7 +29,7 @@ struct KktParams {
 __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int K = p.geom.K, pitch = K + 8;
-    bf16 *kS = reinterpret_cast<bf16 *>(smem);
+    elem *kS = reinterpret_cast<elem *>(smem);
     float *gS = reinterpret_cast<float *>(kS + kChunk * pitch);
     float *bS = gS + kChunk;
 
@@ -37,7 +37,7 @@ __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
     load_tile<kThreads>(kS, pitch, kg, p.k.st, kChunk, K, len);
     if (threadIdx.x < kChunk) {
         const int t = threadIdx.x;
@@ -70,8 +70,8 @@ __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
 // =============================================================================
 struct SolveParams {
     ChunkGeom geom;  // Hv = heads of x
-    const bf16 *x;
-    bf16 *out;
+    const elem *x;
+    elem *out;
     int64_t sb, sh, st;  // strides of (batch, head, token) in x and out
 };
 
@@ -83,11 +83,11 @@ __global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
     const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
     const int lane = threadIdx.x;
     {   // branch-free loads (clamped row), all eight in flight before the first LDS write
-        bf16x8 v[8];
+        elemx8 v[8];
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
             const int idx = m * 64 + lane;
-            v[m] = *reinterpret_cast<const bf16x8 *>(p.x + base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3));
+            v[m] = *reinterpret_cast<const elemx8 *>(p.x + base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3));
         }
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
@@ -113,9 +113,9 @@ __global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
         x[i] = acc;
     }
     __syncthreads();
-    bf16 *O = reinterpret_cast<bf16 *>(&A[0][0]);  // [64][72] bf16 staging, fits in the fp32 tile
+    elem *O = reinterpret_cast<elem *>(&A[0][0]);  // [64][72] bf16 staging, fits in the fp32 tile
 #pragma unroll
-    for (int i = 0; i < kChunk; ++i) O[i * 72 + lane] = (bf16)x[i];
+    for (int i = 0; i < kChunk; ++i) O[i * 72 + lane] = (elem)x[i];
     __syncthreads();
     for (int idx = lane; idx < len * 8; idx += 64) {
         const int r = idx >> 3, c8 = (idx & 7) << 3;
@@ -136,9 +136,9 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
     extern __shared__ __align__(16) unsigned char smem[];
     const int K = p.geom.K, V = p.geom.V;
     const int pa = kChunk + 8, pk = K + 16, pv = V + 16;
-    bf16 *aS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = aS + kChunk * pa;
-    bf16 *vS = kS + kChunk * pk;
+    elem *aS = reinterpret_cast<elem *>(smem);
+    elem *kS = aS + kChunk * pa;
+    elem *vS = kS + kChunk * pk;
     float *gS = reinterpret_cast<float *>(vS + kChunk * pv);
     float *bS = gS + kChunk;
 
@@ -151,53 +151,53 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
         gS[t] = t < len ? __expf(load_scalar(p.g, b, hv, start + t)) : 0.f;
         bS[t] = t < len ? load_scalar(p.beta, b, hv, start + t) : 0.f;
     }
-    const bf16 *ag = static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
+    const elem *ag = static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
     for (int idx = threadIdx.x; idx < kChunk * 8; idx += kThreads) {
         const int r = idx >> 3, c8 = (idx & 7) << 3;
-        bf16x8 a;
-        if (r < len) a = *reinterpret_cast<const bf16x8 *>(ag + (int64_t)r * p.A.st + c8);
+        elemx8 a;
+        if (r < len) a = *reinterpret_cast<const elemx8 *>(ag + (int64_t)r * p.A.st + c8);
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-            if (!(r < len && c8 + e < len)) a[e] = (bf16)0.f;  // columns past the tail are not part of the block
-        *reinterpret_cast<bf16x8 *>(aS + r * pa + c8) = a;
+            if (!(r < len && c8 + e < len)) a[e] = (elem)0.f;  // columns past the tail are not part of the block
+        *reinterpret_cast<elemx8 *>(aS + r * pa + c8) = a;
     }
     __syncthreads();  // gS, bS visible
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
     for (int idx = threadIdx.x; idx < kChunk * (K >> 3); idx += kThreads) {
         const int r = idx / (K >> 3), c8 = (idx % (K >> 3)) << 3;
-        bf16x8 o;
+        elemx8 o;
         if (r < len) {
-            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(kg + (int64_t)r * p.k.st + c8);
+            const elemx8 a = *reinterpret_cast<const elemx8 *>(kg + (int64_t)r * p.k.st + c8);
             const float s = bS[r] * gS[r];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)a[e] * s);
+            for (int e = 0; e < 8; ++e) o[e] = (elem)((float)a[e] * s);
         } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
+            for (int e = 0; e < 8; ++e) o[e] = (elem)0.f;
         }
-        *reinterpret_cast<bf16x8 *>(kS + r * pk + c8) = o;
+        *reinterpret_cast<elemx8 *>(kS + r * pk + c8) = o;
     }
     for (int idx = threadIdx.x; idx < kChunk * (V >> 3); idx += kThreads) {
         const int r = idx / (V >> 3), c8 = (idx % (V >> 3)) << 3;
-        bf16x8 o;
+        elemx8 o;
         if (r < len) {
-            const bf16x8 a = *reinterpret_cast<const bf16x8 *>(vg + (int64_t)r * p.v.st + c8);
+            const elemx8 a = *reinterpret_cast<const elemx8 *>(vg + (int64_t)r * p.v.st + c8);
             const float s = bS[r];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)a[e] * s);
+            for (int e = 0; e < 8; ++e) o[e] = (elem)((float)a[e] * s);
         } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16)0.f;
+            for (int e = 0; e < 8; ++e) o[e] = (elem)0.f;
         }
-        *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = o;
+        *reinterpret_cast<elemx8 *>(vS + r * pv + c8) = o;
     }
     __syncthreads();
 
     // Each wave owns a quarter of the output columns of w and of u and overwrites
     // exactly those columns of the staged operand once its products are done.
     const int w = wave_id();
-    auto product = [&](bf16 *tile, int pitch, int ncols) {
+    auto product = [&](elem *tile, int pitch, int ncols) {
         const int per_wave = ncols / 64;  // 16-column tiles per wave
         for (int m = 0; m < per_wave; ++m) {
             const int c0 = (w * per_wave + m) * 16;
@@ -206,7 +206,7 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
             for (int rt = 0; rt < 4; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16x8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
+                const elemx8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
 #pragma unroll
                 for (int rt = 0; rt < 4; ++rt) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);
             }
@@ -217,8 +217,8 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
     product(kS, pk, K);
     product(vS, pv, V);
     __syncthreads();
-    bf16 *wg = static_cast<bf16 *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
-    bf16 *ug = static_cast<bf16 *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
+    elem *wg = static_cast<elem *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
+    elem *ug = static_cast<elem *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
     store_tile<kThreads>(wg, p.w.st, kS, pk, K, len);
     store_tile<kThreads>(ug, p.u.st, vS, pv, V, len);
 }
@@ -229,18 +229,18 @@ template <int K, int V>
 __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pa = kChunk + 8, pk = K + 16, pv = V + 16;
-    bf16 *aS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = aS + kChunk * pa;
-    bf16 *vS = kS + kChunk * pk;
+    elem *aS = reinterpret_cast<elem *>(smem);
+    elem *kS = aS + kChunk * pa;
+    elem *vS = kS + kChunk * pk;
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x;
-    const bf16 *ag = static_cast<const bf16 *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const elem *ag = static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
     {
         TileCopy<kThreads, kChunk, kChunk> ta;
         TileCopy<kThreads, kChunk, K> tk;
@@ -262,16 +262,16 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
         for (int m = 0; m < TileCopy<kThreads, kChunk, kChunk>::N; ++m) {   // columns past the tail are not part of the block
             const int idx = m * kThreads + tid;
             const int r = idx >> 3, c8 = (idx & 7) << 3;
-            bf16x8 a = __builtin_bit_cast(bf16x8, ta.r[m]);
+            elemx8 a = __builtin_bit_cast(elemx8, ta.r[m]);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
-                if (!(r < len && c8 + e < len)) a[e] = (bf16)0.f;
-            *reinterpret_cast<bf16x8 *>(aS + r * pa + c8) = a;
+                if (!(r < len && c8 + e < len)) a[e] = (elem)0.f;
+            *reinterpret_cast<elemx8 *>(aS + r * pa + c8) = a;
         }
-        auto scaled = [&](bf16 *dst, int pitch, int cpr, int m, u32x4 raw, float sc) {
+        auto scaled = [&](elem *dst, int pitch, int cpr, int m, u32x4 raw, float sc) {
             const int idx = m * kThreads + tid;
             const int r = idx / cpr, c8 = (idx % cpr) << 3;
-            const bf16x8 a = __builtin_bit_cast(bf16x8, raw);
+            const elemx8 a = __builtin_bit_cast(elemx8, raw);
             const float f = r < len ? sc : 0.f;
             f32x4 lo, hi;
 #pragma unroll
@@ -279,7 +279,7 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
                 lo[e] = (float)a[e] * f;
                 hi[e] = (float)a[4 + e] * f;
             }
-            *reinterpret_cast<bf16x8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
+            *reinterpret_cast<elemx8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
         };
 #pragma unroll
         for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) scaled(kS, pk, K / 8, m, tk.r[m], sk[m]);
@@ -291,7 +291,7 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     // Each wave owns a quarter of the output columns of w and of u and overwrites
     // exactly those columns of the staged operand once its products are done.
     const int w = wave_id();
-    auto product = [&](bf16 *tile, int pitch, int ncols) {
+    auto product = [&](elem *tile, int pitch, int ncols) {
         const int per_wave = ncols / 64;  // 16-column tiles per wave
         for (int m = 0; m < per_wave; ++m) {
             const int c0 = (w * per_wave + m) * 16;
@@ -300,7 +300,7 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
             for (int rt = 0; rt < 4; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const bf16x8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
+                const elemx8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
 #pragma unroll
                 for (int rt = 0; rt < 4; ++rt) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);
             }
@@ -311,8 +311,8 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     product(kS, pk, K);
     product(vS, pv, V);
     __syncthreads();
-    bf16 *wg = static_cast<bf16 *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
-    bf16 *ug = static_cast<bf16 *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
+    elem *wg = static_cast<elem *>(const_cast<void *>(p.w.p)) + b * p.w.sb + hv * p.w.sh + (int64_t)start * p.w.st;
+    elem *ug = static_cast<elem *>(const_cast<void *>(p.u.p)) + b * p.u.sb + hv * p.u.sh + (int64_t)start * p.u.st;
     store_tile<kThreads>(wg, p.w.st, kS, pk, K, len);
     store_tile<kThreads>(ug, p.u.st, vS, pv, V, len);
 }
@@ -323,7 +323,7 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
 struct FwdOParams {
     ChunkGeom geom;
     View4 q, k, v, o;
-    const bf16 *h;
+    const elem *h;
     int64_t h_sb, h_sh, h_sc;  // h [B,Hv,NT,K,V]: batch, head, chunk strides (K,V contiguous)
     View3 g;
     float scale;
@@ -334,21 +334,21 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pq = K + 8, pv = V + 16, pp = kChunk + 8;
     constexpr int CT = V / 64;  // 16-column tiles per wave
-    bf16 *qS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = qS + kChunk * pq;
-    bf16 *vS = kS + kChunk * pq;
-    bf16 *hS = vS + kChunk * pv;
-    bf16 *pS = hS + K * pv;
+    elem *qS = reinterpret_cast<elem *>(smem);
+    elem *kS = qS + kChunk * pq;
+    elem *vS = kS + kChunk * pq;
+    elem *hS = vS + kChunk * pv;
+    elem *pS = hS + K * pv;
     float *gS = reinterpret_cast<float *>(pS + kChunk * pp);
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
-    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
-    const bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
+    const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
     {   // every load of the chunk is in flight before the first LDS write waits
         const int tid = threadIdx.x;
         TileCopy<kThreads, kChunk, K> tq, tk;
@@ -385,7 +385,7 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
                 acc[e] = (s <= t) ? acc[e] * __expf(fminf(gt - gS[s], 0.f)) : 0.f;
             }
         }
-        *reinterpret_cast<bf16x4 *>(pS + t * pp + J * 16 + 4 * (lane_id() >> 4)) = cvt4(acc);
+        *reinterpret_cast<elemx4 *>(pS + t * pp + J * 16 + 4 * (lane_id() >> 4)) = cvt4(acc);
     }
 
     // inter-chunk term e^{G_t} (q h) for this wave's V columns
@@ -396,12 +396,12 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
         for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < K / 32; ++j) {
-        bf16x8 bfrag[CT];
+        elemx8 bfrag[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(hS, pv, (w * CT + ct) * 16, 32 * j);
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
-            const bf16x8 afrag = frag_kc(qS, pq, rt * 16, 32 * j);
+            const elemx8 afrag = frag_kc(qS, pq, rt * 16, 32 * j);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
         }
@@ -418,12 +418,12 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
 
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        bf16x8 bfrag[CT];
+        elemx8 bfrag[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(vS, pv, (w * CT + ct) * 16, 32 * j);
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
-            const bf16x8 afrag = frag_kc(pS, pp, rt * 16, 32 * j);
+            const elemx8 afrag = frag_kc(pS, pp, rt * 16, 32 * j);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
         }
@@ -434,7 +434,7 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc_to_tile(vS, pv, rt * 16, (w * CT + ct) * 16, acc[rt][ct] * p.scale);
     __syncthreads();
-    bf16 *og = static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)start * p.o.st;
+    elem *og = static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)start * p.o.st;
     store_tile<kThreads>(og, p.o.st, vS, pv, V, len);
 }
 
@@ -445,10 +445,10 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
     const char *op = "chunk_scaled_dot_kkt";
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom))) return rc;
-    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, dt_bit(FLA_BF16)))) return rc;
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
-    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if ((rc = check_tensor(out, op, "out", 4, dt_bit(FLA_F32)))) return rc;
     FLA_REQUIRE(out->shape[0] == geom.B && out->shape[1] == geom.Hv && out->shape[2] == geom.T && out->shape[3] == kChunk &&
                     inner_unit(out) && out->stride[2] % 4 == 0 && out->stride[1] % 4 == 0 && out->stride[0] % 4 == 0,
@@ -470,8 +470,8 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
                const fla_tensor *out, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "solve_tri";
     int rc;
-    if ((rc = check_tensor(x, op, "x", -1, dt_bit(FLA_BF16)))) return rc;
-    if ((rc = check_tensor(out, op, "out", -1, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_tensor(x, op, "x", -1, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_tensor(out, op, "out", -1, dt_bit(kElemDtype)))) return rc;
     FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
     FLA_REQUIRE(same_shape(x, out), FLA_ERR_SHAPE, "%s: out must have the shape of x.", op);
     FLA_REQUIRE(is_contiguous(x) && is_contiguous(out), FLA_ERR_SHAPE, "%s: x and out must be contiguous.", op);
@@ -497,7 +497,7 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0 || geom.Hv == 0) return FLA_OK;
-    SolveParams p{geom, static_cast<const bf16 *>(x->data), static_cast<bf16 *>(out->data), ib < 0 ? 0 : x->stride[ib],
+    SolveParams p{geom, static_cast<const elem *>(x->data), static_cast<elem *>(out->data), ib < 0 ? 0 : x->stride[ib],
                   x->stride[ih], x->stride[it]};
     FLA_LAUNCH("solve_tri", stream, solve_tri_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(64), 0, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
@@ -511,16 +511,16 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     FLA_REQUIRE(gk == nullptr || gk->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: gk must be None.", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(geom.K % 64 == 0 && geom.V % 64 == 0 && geom.K <= 256 && geom.V <= 256, FLA_ERR_UNSUPPORTED,
                 "%s: K and V must be multiples of 64 up to 256, got K=%d V=%d.", op, geom.K, geom.V);
     Varlen vl;
@@ -561,14 +561,14 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const char *op = "chunk_fwd_o";
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "out", out, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
     if ((rc = check_tensor(h, op, "h", 5, bf))) return rc;
@@ -578,7 +578,7 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                 FLA_ERR_SHAPE, "%s: h must be [B,Hv,NT=%d,K,V] with contiguous K x V blocks.", op, geom.NT);
     if (query) return FLA_OK;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
-    FwdOParams p{geom, view4(q), view4(k), view4(v), view4(out), static_cast<const bf16 *>(h->data),
+    FwdOParams p{geom, view4(q), view4(k), view4(v), view4(out), static_cast<const elem *>(h->data),
                  h->stride[0], h->stride[1], h->stride[2], view3(g), (float)scale};
     if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128>(p, stream);
     if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256>(p, stream);
@@ -593,66 +593,74 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
 #define FLA_NULL_WS(op) \
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, op ": workspace_size must not be null.")
 
-extern "C" int fla_chunk_scaled_dot_kkt_get_workspace_size(const fla_tensor *k, const fla_tensor *g,
+FLA_ENTRY(fla_chunk_scaled_dot_kkt_get_workspace_size)(const fla_tensor *k, const fla_tensor *g,
                                                            const fla_tensor *beta, const fla_int_array *cu_seqlens,
                                                            const fla_int_array *chunk_indices, int64_t chunk_size,
                                                            const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_get_workspace_size, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_scaled_dot_kkt");
     return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size);
 }
-extern "C" int fla_chunk_scaled_dot_kkt(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+FLA_ENTRY(fla_chunk_scaled_dot_kkt)(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
                                         const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                         int64_t chunk_size, const fla_tensor *out, void *workspace,
                                         uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size, stream);
     return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
                          static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_solve_tri_get_workspace_size(const fla_tensor *x, const fla_int_array *cu_seqlens,
+FLA_ENTRY(fla_solve_tri_get_workspace_size)(const fla_tensor *x, const fla_int_array *cu_seqlens,
                                                 const fla_int_array *chunk_indices, const char *layout,
                                                 const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(x, fla_solve_tri_get_workspace_size, x, cu_seqlens, chunk_indices, layout, out, workspace_size);
     FLA_NULL_WS("solve_tri");
     return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, nullptr, 0, nullptr, workspace_size);
 }
-extern "C" int fla_solve_tri(const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+FLA_ENTRY(fla_solve_tri)(const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                              const char *layout, const fla_tensor *out, void *workspace, uint64_t workspace_size,
                              void *stream) {
+    FLA_ROUTE_F16(x, fla_solve_tri, x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size, stream);
     return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_recompute_w_u_fwd_get_workspace_size(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
+FLA_ENTRY(fla_recompute_w_u_fwd_get_workspace_size)(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
                                                         const fla_tensor *A, const fla_tensor *g, const fla_tensor *gk,
                                                         const fla_int_array *cu_seqlens,
                                                         const fla_int_array *chunk_indices, int64_t chunk_size,
                                                         const fla_tensor *w, const fla_tensor *u,
                                                         uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_recompute_w_u_fwd_get_workspace_size, k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace_size);
     FLA_NULL_WS("recompute_w_u_fwd");
     return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, nullptr, 0, nullptr,
                         workspace_size);
 }
-extern "C" int fla_recompute_w_u_fwd(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
+FLA_ENTRY(fla_recompute_w_u_fwd)(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
                                      const fla_tensor *A, const fla_tensor *g, const fla_tensor *gk,
                                      const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                      int64_t chunk_size, const fla_tensor *w, const fla_tensor *u, void *workspace,
                                      uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_recompute_w_u_fwd, k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size, stream);
     return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size,
                         static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_chunk_fwd_o_get_workspace_size(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
+FLA_ENTRY(fla_chunk_fwd_o_get_workspace_size)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
                                                   const fla_tensor *h, const fla_tensor *g,
                                                   const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                                   double scale, int64_t chunk_size, const fla_tensor *out,
                                                   uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_fwd_o_get_workspace_size, q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_fwd_o");
     return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0, nullptr,
                            workspace_size);
 }
-extern "C" int fla_chunk_fwd_o(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
+FLA_ENTRY(fla_chunk_fwd_o)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
                                const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                double scale, int64_t chunk_size, const fla_tensor *out, void *workspace,
                                uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_fwd_o, q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size, stream);
     return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
 }

@@ -22,8 +22,8 @@ int check_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B,
     return FLA_OK;
 }
 
-int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T) {
-    int rc = check_tensor(t, op, name, 3, dt_bit(FLA_F32) | dt_bit(FLA_BF16));
+int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, int elem_dtype) {
+    int rc = check_tensor(t, op, name, 3, dt_bit(FLA_F32) | dt_bit(elem_dtype));
     if (rc) return rc;
     FLA_REQUIRE(t->shape[0] == B && t->shape[1] == H && t->shape[2] == T, FLA_ERR_SHAPE,
                 "%s: %s must be [%lld,%lld,%lld].", op, name, (long long)B, (long long)H, (long long)T);
@@ -31,10 +31,10 @@ int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, 
 }
 
 int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, const fla_tensor *g_like,
-                 int64_t chunk_size, ChunkGeom &geom) {
+                 int64_t chunk_size, ChunkGeom &geom, int elem_dtype) {
     FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: chunk_size must be %d, got %lld.", op, kChunk,
                 (long long)chunk_size);
-    int rc = check_tensor(k, op, "k", 4, dt_bit(FLA_BF16));
+    int rc = check_tensor(k, op, "k", 4, dt_bit(elem_dtype));
     if (rc) return rc;
     geom = ChunkGeom{};
     geom.B = (int)k->shape[0];
@@ -46,11 +46,11 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
     FLA_REQUIRE(k->shape[0] < (1 << 16) && k->shape[2] < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents too large.",
                 op);
     if (v_like) {
-        if ((rc = check_tensor(v_like, op, "v", 4, dt_bit(FLA_BF16)))) return rc;
+        if ((rc = check_tensor(v_like, op, "v", 4, dt_bit(elem_dtype)))) return rc;
         geom.Hv = (int)v_like->shape[1];
         geom.V = (int)v_like->shape[3];
     } else if (g_like) {
-        if ((rc = check_tensor(g_like, op, "g", 3, dt_bit(FLA_F32) | dt_bit(FLA_BF16)))) return rc;
+        if ((rc = check_tensor(g_like, op, "g", 3, dt_bit(FLA_F32) | dt_bit(elem_dtype)))) return rc;
         geom.Hv = (int)g_like->shape[1];
     }
     FLA_REQUIRE(geom.Hk > 0 && geom.Hv % geom.Hk == 0, FLA_ERR_SHAPE, "%s: Hv (%d) must be a multiple of Hk (%d).", op,

@@ -83,7 +83,7 @@ template <int K, int CT> struct FusedSmem {
 };
 
 struct Tiles {      // one LDS buffer of chunk inputs
-    bf16 *q, *k, *v;
+    elem *q, *k, *v;
     // per token: cumulated gate G, scale e^G, beta, beta e^G, and the factors of
     //   e^{G_t - G_s} = ROWF[t] * BLKF[blk(t)][blk(s)] * COLF[s]   for blk(s) < blk(t)
     // with ROWF[t] = e^{G_t - G(first token of blk(t))}, COLF[s] = e^{G(last token of blk(s)) - G_s};
@@ -95,9 +95,9 @@ __device__ __forceinline__ Tiles tiles_at(unsigned char *smem, int buf) {
     typedef FusedSmem<K, CT> L;
     unsigned char *b = smem + buf * L::buf_bytes;
     Tiles t;
-    t.q = reinterpret_cast<bf16 *>(b);
-    t.k = reinterpret_cast<bf16 *>(b + L::q_bytes);
-    t.v = reinterpret_cast<bf16 *>(b + L::q_bytes + L::k_bytes);
+    t.q = reinterpret_cast<elem *>(b);
+    t.k = reinterpret_cast<elem *>(b + L::q_bytes);
+    t.v = reinterpret_cast<elem *>(b + L::q_bytes + L::k_bytes);
     t.G = reinterpret_cast<float *>(b + L::q_bytes + L::k_bytes + L::v_bytes);
     t.EGS = t.G + kChunk;
     t.B = t.EGS + kChunk;
@@ -115,7 +115,7 @@ __device__ __forceinline__ f32x4 lds4(const float *p) { return *reinterpret_cast
 // Phase A for wave W: row block I1 = W of the score matrix, row block I2 = 3 - W of P.
 // ---------------------------------------------------------------------------------------------
 template <int K, int W>
-__device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16 *dS, float scale) {
+__device__ __forceinline__ void phase_a(const Tiles &t, elem *aS, elem *pS, elem *dS, float scale) {
     constexpr int I1 = W, I2 = 3 - W, JM = I1 > I2 ? I1 : I2, KS = K / 32;
     constexpr int pq = K + 8, pa = kChunk + 8, pp = kChunk + 8, pd = 24;
     const int l = lane_id(), li = l & 15, lg = l >> 4;
@@ -125,7 +125,7 @@ __device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16
     for (int J = 0; J <= I1; ++J) kacc[J] = zero4();
 #pragma unroll
     for (int J = 0; J <= I2; ++J) pacc[J] = zero4();
-    bf16x8 kf[2][JM + 1], qf[2];
+    elemx8 kf[2][JM + 1], qf[2];
 #pragma unroll
     for (int J = 0; J <= JM; ++J) kf[0][J] = KTile<K>::kc(t.k, 16 * J, 0);
     qf[0] = frag_kc(t.q, pq, 16 * I2, 0);
@@ -157,7 +157,7 @@ __device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16
         f32x4 a;
 #pragma unroll
         for (int e = 0; e < 4; ++e) a[e] = coef * cf[e] * kacc[J][e];
-        *reinterpret_cast<bf16x4 *>(aS + t1 * pa + 16 * J + 4 * lg) = cvt4(a);
+        *reinterpret_cast<elemx4 *>(aS + t1 * pa + 16 * J + 4 * lg) = cvt4(a);
     }
 #pragma unroll
     for (int J = 0; J < 4; ++J) {  // scale * P[t][s] = scale q_t.k_s e^{min(G_t-G_s,0)} for s <= t
@@ -173,7 +173,7 @@ __device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16
             for (int e = 0; e < 4; ++e)
                 a[e] = 4 * lg + e <= li ? scale * __expf(fminf(gt2 - gs[e], 0.f)) * pacc[I2][e] : 0.f;
         }
-        *reinterpret_cast<bf16x4 *>(pS + t2 * pp + 16 * J + 4 * lg) = cvt4(a);
+        *reinterpret_cast<elemx4 *>(pS + t2 * pp + 16 * J + 4 * lg) = cvt4(a);
     }
 
     // diagonal block A (16x16, strictly lower): both operand views from the symmetric raw tile
@@ -190,25 +190,25 @@ __device__ __forceinline__ void phase_a(const Tiles &t, bf16 *aS, bf16 *pS, bf16
     // An accumulator tile of M is the right operand of M and the left operand of M^T, so the
     // chains S_k = A^(2^k) and T_k = S_k^T are advanced together and
     //   Y <- Y + T_k Y   accumulates   Y = ((I-A)(I+A^2)(I+A^4)(I+A^8))^T = ((I+A)^-1)^T.
-    const bf16x4 A1 = cvt4(a1), A2 = cvt4(a2);
+    const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
     const f32x4 S1 = mfma16x16(A1, A2, zero4());
     const f32x4 T1 = mfma16x16(A2, A1, zero4());
-    const bf16x4 S1b = cvt4(S1), T1b = cvt4(T1);
+    const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
     Y = mfma16x16(S1b, cvt4(Y), Y);
     const f32x4 S2 = mfma16x16(T1b, S1b, zero4());
     const f32x4 T2 = mfma16x16(S1b, T1b, zero4());
-    const bf16x4 S2b = cvt4(S2);
+    const elemx4 S2b = cvt4(S2);
     Y = mfma16x16(S2b, cvt4(Y), Y);
     const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());
     Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
     // lane holds Dinv^T[4lg+e][li] = Dinv[li][4lg+e]: the left-operand layout, 8 contiguous bytes
-    *reinterpret_cast<bf16x4 *>(dS + (16 * I1 + li) * pd + 4 * lg) = cvt4(Y);
+    *reinterpret_cast<elemx4 *>(dS + (16 * I1 + li) * pd + 4 * lg) = cvt4(Y);
 }
 
 // D^-1 R for one diagonal block; hilo feeds R as hi + lo bf16 pairs.
-__device__ __forceinline__ f32x4 diag_mul(bf16x4 d, f32x4 r, bool hilo) {
+__device__ __forceinline__ f32x4 diag_mul(elemx4 d, f32x4 r, bool hilo) {
     if (!hilo) return mfma16x16(d, cvt4(r), zero4());
-    bf16x4 hi, lo;
+    elemx4 hi, lo;
     split_hilo(r, hi, lo);
     return mfma16x16(d, lo, mfma16x16(d, hi, zero4()));
 }
@@ -225,11 +225,11 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
     constexpr int QROWS = kThreads / (K / 8), VROWS = kThreads / (VS / 8);
     constexpr int NTW = K / 64, NT = NTW + CT;          // w tiles per wave, all solved tiles per wave
     extern __shared__ __align__(16) unsigned char smem[];
-    bf16 *aS = reinterpret_cast<bf16 *>(smem + L::a_off);
-    bf16 *wS = reinterpret_cast<bf16 *>(smem + L::w_off);
-    bf16 *pS = reinterpret_cast<bf16 *>(smem + L::p_off);
-    bf16 *oS = reinterpret_cast<bf16 *>(smem + L::o_off);
-    bf16 *dS = reinterpret_cast<bf16 *>(smem + L::d_off);
+    elem *aS = reinterpret_cast<elem *>(smem + L::a_off);
+    elem *wS = reinterpret_cast<elem *>(smem + L::w_off);
+    elem *pS = reinterpret_cast<elem *>(smem + L::p_off);
+    elem *oS = reinterpret_cast<elem *>(smem + L::o_off);
+    elem *dS = reinterpret_cast<elem *>(smem + L::d_off);
 
     // ---- which (sequence, head, slab) ---------------------------------------------------
     const int lin = blockIdx.x;
@@ -278,10 +278,10 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
     // (row r of the chunk, 8 columns from cq / cv) computed once ------------------------------------
     const int rq = tid / (K / 8), cq = (tid % (K / 8)) * 8;
     const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
-    const char *qbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
-    const char *kbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
-    const char *vbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
-    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + slab * VS);
+    const char *qbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
+    const char *kbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
+    const char *vbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
+    char *obase = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + slab * VS);
     unsigned qoff[QCH], koff[QCH], voff[VCH], ooff[VCH];
 #pragma unroll
     for (int m = 0; m < QCH; ++m) {
@@ -413,24 +413,24 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
             const f32x4 b4 = lds4(t.B + 16 * i + 4 * lg), be4 = lds4(t.BEG + 16 * i + 4 * lg);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const bf16x4 vv = frag_tr4(t.v, pv, (vtile0 + ct) * 16, 16 * i);
+                const elemx4 vv = frag_tr4(t.v, pv, (vtile0 + ct) * 16, 16 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) r[ct][i][e] = (float)vv[e] * b4[e];
             }
 #pragma unroll
             for (int m = 0; m < NTW; ++m) {
-                const bf16x4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * i);
+                const elemx4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) r[CT + m][i][e] = (float)kv[e] * be4[e];
             }
         }
         {
-            const bf16x4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
+            const elemx4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
                          d3 = frag_kc4(dS, pd, 48, 0);
-            const bf16x4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
-            const bf16x8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
+            const elemx4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
+            const elemx8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
             FLA_SCHED_FENCE();
-            bf16x8 x01[NT];
+            elemx8 x01[NT];
 #pragma unroll
             for (int q = 0; q < NT; ++q) r[q][0] = diag_mul(d0, r[q][0], q < CT);
 #pragma unroll
@@ -461,7 +461,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         FLA_TICK(3)
 
         // =========================== C: scan + output ====================================
-        bf16x8 hB[KS][CT];
+        elemx8 hB[KS][CT];
 #pragma unroll
         for (int j = 0; j < KS; ++j)
 #pragma unroll
@@ -477,7 +477,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
                 oacc[rt][ct] = zero4();
             }
         {
-            bf16x8 wf[2][4], qf[2][4];
+            elemx8 wf[2][4], qf[2][4];
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
                 wf[0][rt] = frag_kc(wS, pw, rt * 16, 0);
@@ -506,7 +506,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         }
         FLA_TICK(8)
         // operands of the next two products, issued before the element-wise work below
-        bf16x8 pf[2][4], kfa[KT];
+        elemx8 pf[2][4], kfa[KT];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -532,7 +532,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         // o = scale (e^{G_t} q h + P v_new)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            bf16x8 vb[CT];
+            elemx8 vb[CT];
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) vb[ct] = frag_from_acc(U[2 * j][ct], U[2 * j + 1][ct]);
 #pragma unroll
@@ -547,20 +547,20 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= dec_all;
-        bf16x8 vhi[2][CT], vlo[2][CT];
+        elemx8 vhi[2][CT], vlo[2][CT];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 const f32x4 a0 = U[2 * j][ct] * dk4[2 * j], a1 = U[2 * j + 1][ct] * dk4[2 * j + 1];
-                bf16x4 h0, h1, l0, l1;
+                elemx4 h0, h1, l0, l1;
                 split_hilo(a0, h0, l0);
                 split_hilo(a1, h1, l1);
                 vhi[j][ct] = cat8(h0, h1);
                 vlo[j][ct] = cat8(l0, l1);
             }
         {
-            bf16x8 kfb[KT];
+            elemx8 kfb[KT];
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) kfb[kt] = KTile<K>::tr(t.k, kt * 16, 32);
             FLA_SCHED_FENCE();
@@ -651,9 +651,9 @@ __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
     typedef PipeSmem<K> L;
     const int c3 = (unsigned)(c + 3) % 3u, c2 = c & 1;
     Tiles t;
-    t.q = reinterpret_cast<bf16 *>(smem + L::q_off + c3 * L::q_bytes);
-    t.k = reinterpret_cast<bf16 *>(smem + L::k_off + c2 * L::k_bytes);
-    t.v = reinterpret_cast<bf16 *>(smem + L::v_off);
+    t.q = reinterpret_cast<elem *>(smem + L::q_off + c3 * L::q_bytes);
+    t.k = reinterpret_cast<elem *>(smem + L::k_off + c2 * L::k_bytes);
+    t.v = reinterpret_cast<elem *>(smem + L::v_off);
     t.G = reinterpret_cast<float *>(smem + L::t_off + c2 * L::tab_bytes);
     t.EGS = t.G + kChunk;
     t.B = t.EGS + kChunk;
@@ -676,10 +676,10 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     constexpr int QROWS = GT / (K / 8), VROWS = GT / (VS / 8);
     constexpr int NTW = K / 64, NT = NTW + 1;
     extern __shared__ __align__(16) unsigned char smem[];
-    bf16 *aS = reinterpret_cast<bf16 *>(smem + L::a_off);
-    bf16 *wS = reinterpret_cast<bf16 *>(smem + L::w_off);
-    bf16 *pS0 = reinterpret_cast<bf16 *>(smem + L::p_off);
-    bf16 *dS = reinterpret_cast<bf16 *>(smem + L::d_off);
+    elem *aS = reinterpret_cast<elem *>(smem + L::a_off);
+    elem *wS = reinterpret_cast<elem *>(smem + L::w_off);
+    elem *pS0 = reinterpret_cast<elem *>(smem + L::p_off);
+    elem *dS = reinterpret_cast<elem *>(smem + L::d_off);
     float *uS = reinterpret_cast<float *>(smem + L::u_off);
 
     const int lin = blockIdx.x;
@@ -711,9 +711,9 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         const int wv = wave, tid = threadIdx.x;
         const int rq = tid / (K / 8), cq = (tid % (K / 8)) * 8;
         const int rv = tid / (VS / 8), cv = (tid % (VS / 8)) * 8;
-        const char *qbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
-        const char *kbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
-        const char *vbase = reinterpret_cast<const char *>(static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
+        const char *qbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)bos * p.q.st);
+        const char *kbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)bos * p.k.st);
+        const char *vbase = reinterpret_cast<const char *>(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)bos * p.v.st + slab * VS);
         unsigned qoff[QCH], koff[QCH], voff[VCH];
 #pragma unroll
         for (int m = 0; m < QCH; ++m) {
@@ -744,7 +744,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         // A row is held by K/8 adjacent lanes, so its sum of squares is one DPP reduction; the normalised row is
         // rounded to bf16 exactly where the separate normalisation kernel would have rounded it.
         auto unit_row = [&](u32x4 raw) -> u32x4 {
-            const bf16x8 a = __builtin_bit_cast(bf16x8, raw);
+            const elemx8 a = __builtin_bit_cast(elemx8, raw);
             f32x4 lo, hi;
             float ss = 0.f;
 #pragma unroll
@@ -763,7 +763,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = p.l2norm ? unit_row(pre_k[m]) : pre_k[m];
             }
         };
-        bf16 *vS = reinterpret_cast<bf16 *>(smem + L::v_off);
+        elem *vS = reinterpret_cast<elem *>(smem + L::v_off);
         if (nchunks > 0) {
             prefetch(0);
             commit_qk(pipe_tiles_at<K>(smem, 0));
@@ -775,7 +775,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #endif
         for (int i = 0; i <= nchunks; ++i) {
             const Tiles t = pipe_tiles_at<K>(smem, i);
-            bf16 *pS = pS0 + (i & 1) * kChunk * pp;
+            elem *pS = pS0 + (i & 1) * kChunk * pp;
             if (i < nchunks) {
                 // v of this chunk has waited in registers: its single LDS tile was read until the last barrier
 #pragma unroll
@@ -798,22 +798,22 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
                 for (int bi = 0; bi < 4; ++bi) {
                     const f32x4 b4 = lds4(t.B + 16 * bi + 4 * lg), be4 = lds4(t.BEG + 16 * bi + 4 * lg);
-                    const bf16x4 vv = frag_tr4(t.v, pv, wv * 16, 16 * bi);
+                    const elemx4 vv = frag_tr4(t.v, pv, wv * 16, 16 * bi);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) r[0][bi][e] = (float)vv[e] * b4[e];
 #pragma unroll
                     for (int m = 0; m < NTW; ++m) {
-                        const bf16x4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * bi);
+                        const elemx4 kv = KTile<K>::tr4(t.k, (wv * NTW + m) * 16, 16 * bi);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) r[1 + m][bi][e] = (float)kv[e] * be4[e];
                     }
                 }
                 {
-                    const bf16x4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
+                    const elemx4 d0 = frag_kc4(dS, pd, 0, 0), d1 = frag_kc4(dS, pd, 16, 0), d2 = frag_kc4(dS, pd, 32, 0),
                                  d3 = frag_kc4(dS, pd, 48, 0);
-                    const bf16x4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
-                    const bf16x8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
-                    bf16x8 x01[NT];
+                    const elemx4 a10 = frag_kc4(aS, pa, 16, 0), a32 = frag_kc4(aS, pa, 48, 32);
+                    const elemx8 a2x = frag_kc(aS, pa, 32, 0), a3x = frag_kc(aS, pa, 48, 0);
+                    elemx8 x01[NT];
 #pragma unroll
                     for (int q = 0; q < NT; ++q) r[q][0] = diag_mul(d0, r[q][0], q == 0);
 #pragma unroll
@@ -871,7 +871,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     // bookkeeping carries them around the loop and turns every first use of the state into a wait for
     // ALL outstanding memory operations, including the gate loads issued for the next chunk.
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    char *obase = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + vcol0);
+    char *obase = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + vcol0);
     // lane part of an output tile's address: rows 4lg (+2 for odd lanes), column pair of the lane
     const unsigned o_lane = (unsigned)((4 * lg + ((li & 1) ? 2 : 0)) * p.o.st * 2 + (li & ~1) * 2);
     const unsigned o_row = (unsigned)(p.o.st * 2);
@@ -936,10 +936,10 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     for (int i = 0; i <= nchunks; ++i) {
         const int c = i - 1;                               // chunk of this group
         const Tiles t = pipe_tiles_at<K>(smem, c);
-        const bf16 *pS = pS0 + (c & 1) * kChunk * pp;
+        const elem *pS = pS0 + (c & 1) * kChunk * pp;
         const int len = c >= 0 ? min(kChunk, eos - (bos + c * kChunk)) : 0;
         f32x4 U[4], eg4[4];
-        bf16x8 hB[KS];
+        elemx8 hB[KS];
 #ifdef FLA_PIPE_SKIP_STATE
         if (c >= 1000000) {
 #else
@@ -952,7 +952,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             for (int rt = 0; rt < 4; ++rt) U[rt] = *reinterpret_cast<const f32x4 *>(uS + ((wv * 4 + rt) * 64 + l) * 4);
             {   // v_new = u + (-w) h
                 // every operand read is in flight before the first product: their latency is paid once
-                bf16x8 wf[KS][4];
+                elemx8 wf[KS][4];
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
 #pragma unroll
@@ -965,7 +965,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 FLA_SCHED_FENCE();
             }
             FLA_TICK(0)
-            bf16x8 kfa[KT], kfb[KT];
+            elemx8 kfa[KT], kfb[KT];
             f32x4 dk4[4];
             const float g_last = t.G[len - 1];
 #pragma unroll
@@ -982,11 +982,11 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             const float dec_all = __expf(g_last);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) hacc[kt] *= dec_all;
-            bf16x8 vhi[2], vlo[2];
+            elemx8 vhi[2], vlo[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const f32x4 a0 = U[2 * j] * dk4[2 * j], a1 = U[2 * j + 1] * dk4[2 * j + 1];
-                bf16x4 h0, h1, l0, l1;
+                elemx4 h0, h1, l0, l1;
                 split_hilo(a0, h0, l0);
                 split_hilo(a1, h1, l1);
                 vhi[j] = cat8(h0, h1);
@@ -1011,7 +1011,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         }
         // q of this chunk and its P tile have been in LDS since the previous iteration: the first operands of
         // the second half are fetched before the barrier, so their latency hides behind the wait
-        bf16x8 qf[2][4], pf[6];
+        elemx8 qf[2][4], pf[6];
         if (c >= 0) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
@@ -1051,7 +1051,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
             {
-                const bf16x8 vb0 = frag_from_acc(U[0], U[1]), vb1 = frag_from_acc(U[2], U[3]);
+                const elemx8 vb0 = frag_from_acc(U[0], U[1]), vb1 = frag_from_acc(U[2], U[3]);
                 oacc[0] = mfma16x32(pf[0], vb0, oacc[0]);
                 oacc[1] = mfma16x32(pf[1], vb0, oacc[1]);
                 oacc[2] = mfma16x32(pf[2], vb0, oacc[2]);
@@ -1133,8 +1133,8 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const char *op = "gdn_chunk_fwd";
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
@@ -1193,8 +1193,8 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     p.k = view4(k);
     p.v = view4(v);
     p.o = View4{o->data, o->stride[0], o->stride[2], o->stride[1]};  // [B,T,Hv,V] seen as [B,Hv,T,V]
-    p.g = View3{g->data, g->stride[0], g->stride[2], g->stride[1], g->dtype == FLA_BF16 ? 1 : 0};
-    p.beta = View3{beta->data, beta->stride[0], beta->stride[2], beta->stride[1], beta->dtype == FLA_BF16 ? 1 : 0};
+    p.g = View3{g->data, g->stride[0], g->stride[2], g->stride[1], g->dtype == FLA_F32 ? 0 : 1};
+    p.beta = View3{beta->data, beta->stride[0], beta->stride[2], beta->stride[1], beta->dtype == FLA_F32 ? 0 : 1};
     if (has_gout) {
         p.g_out = static_cast<float *>(g_cumsum->data);
         p.go_sb = g_cumsum->stride[0];
@@ -1235,24 +1235,26 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
 }  // namespace
 }  // namespace fla
 
-extern "C" int fla_gdn_chunk_fwd_get_workspace_size(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
+FLA_ENTRY(fla_gdn_chunk_fwd_get_workspace_size)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
                                                     const fla_tensor *g, const fla_tensor *beta, double scale,
                                                     const fla_tensor *initial_state, bool output_final_state,
                                                     const fla_int_array *cu_seqlens, int64_t chunk_size,
                                                     bool use_qk_l2norm_in_kernel, const fla_tensor *o,
                                                     const fla_tensor *g_cumsum, const fla_tensor *final_state,
                                                     uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd: workspace_size must not be null.");
     return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
                            g_cumsum, final_state, nullptr, 0, nullptr, workspace_size);
 }
 
-extern "C" int fla_gdn_chunk_fwd(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
                                  const fla_tensor *beta, double scale, const fla_tensor *initial_state,
                                  bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
                                  bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
                                  const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace, workspace_size, stream);
     return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
                            g_cumsum, final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);

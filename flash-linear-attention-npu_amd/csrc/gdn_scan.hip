@@ -26,7 +26,7 @@ struct ScanParams {
     View3 g;
     const float *h0;     // [N,Hv,K,V] or [N,Hv,V,K] fp32, or null
     float *hT;           // final state, same layout, or null
-    bf16 *h;             // [B,Hv,NT,K,V] (or V,K) bf16, or null
+    elem *h;             // [B,Hv,NT,K,V] (or V,K) bf16, or null
     int64_t h_sb, h_sh, h_sc;
     int64_t s_sn, s_sh;  // strides of h0 / hT over (sequence, head)
     int v_first;         // state blocks are [V][K] instead of [K][V]
@@ -63,9 +63,9 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         chunk0 = p.geom.choff[n];
     }
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
-    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
-    const bf16 *ug = static_cast<const bf16 *>(p.u.p) + b * p.u.sb + hv * p.u.sh + slab * VS;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const elem *wg = static_cast<const elem *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const elem *ug = static_cast<const elem *>(p.u.p) + b * p.u.sb + hv * p.u.sh + slab * VS;
 
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
@@ -81,9 +81,9 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             tu.fetch(ug + (int64_t)start * p.u.st, p.u.st, len, tid);
             float gv = 0.f;
             if (tid < kChunk) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
-            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pw, len, tid);
-            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pk, len, tid);
-            tu.commit(reinterpret_cast<bf16 *>(buf + L::u_off), pu, len, tid);
+            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
+            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
+            tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
             if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
         };
         if (nchunks > 0) load(0);
@@ -116,34 +116,34 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             hacc[kt][ct] = a;
         }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
-    char *vng = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + vcol0);
+    char *vng = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + vcol0);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
-        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
-        const bf16 *uS = reinterpret_cast<const bf16 *>(buf + L::u_off);
+        const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
+        const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
+        const elem *uS = reinterpret_cast<const elem *>(buf + L::u_off);
         const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
 
         // state at chunk start as a bf16 operand (and as the emitted h)
-        bf16x8 hB[KS][CT];
+        elemx8 hB[KS][CT];
 #pragma unroll
         for (int j = 0; j < KS; ++j)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
         if (p.h) {
-            bf16 *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
             if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
-                        const bf16x8 f = hB[kt >> 1][ct];
-                        const bf16x4 q4 = (kt & 1) ? bf16x4{f[4], f[5], f[6], f[7]} : bf16x4{f[0], f[1], f[2], f[3]};
-                        *reinterpret_cast<bf16x4 *>(hg + (int64_t)(vcol0 + 16 * ct + li) * K + 16 * kt + 4 * lg) = q4;
+                        const elemx8 f = hB[kt >> 1][ct];
+                        const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
+                        *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + 16 * ct + li) * K + 16 * kt + 4 * lg) = q4;
                     }
             } else {
 #pragma unroll
@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         for (int j = 0; j < KS; ++j)
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
-                const bf16x8 afrag = frag_kc(wS, pw, rt * 16, 32 * j);
+                const elemx8 afrag = frag_kc(wS, pw, rt * 16, 32 * j);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) vn[rt][ct] = mfma16x32(afrag, hB[j][ct], vn[rt][ct]);
             }
@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const bf16x4 uu = frag_tr4(uS, pu, (wv * CT + ct) * 16, rt * 16);  // u[16rt+4g+e][col]
+                const elemx4 uu = frag_tr4(uS, pu, (wv * CT + ct) * 16, rt * 16);  // u[16rt+4g+e][col]
 #pragma unroll
                 for (int e = 0; e < 4; ++e) vn[rt][ct][e] = (float)uu[e] - vn[rt][ct][e];
             }
@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
 
         // h <- e^{g_last} h + k^T (v_new e^{g_last - g}); padded rows carry zeros
         const float dec_all = __expf(g_last);
-        bf16x8 vB[2][CT];
+        elemx8 vB[2][CT];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -196,8 +196,8 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int t0 = 32 * j + 4 * lg + e, t1 = t0 + 16;
-                    lo[e] = t0 < len ? (float)(bf16)lo[e] * __expf(g_last - gS[t0]) : 0.f;
-                    hi[e] = t1 < len ? (float)(bf16)hi[e] * __expf(g_last - gS[t1]) : 0.f;
+                    lo[e] = t0 < len ? (float)(elem)lo[e] * __expf(g_last - gS[t0]) : 0.f;
+                    hi[e] = t1 < len ? (float)(elem)hi[e] * __expf(g_last - gS[t1]) : 0.f;
                 }
                 vB[j][ct] = frag_from_acc(lo, hi);
             }
@@ -209,7 +209,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
-                const bf16x8 afrag = frag_tr(kS, pk, kt * 16, 32 * j);  // k^T: rows kk, contraction over tokens
+                const elemx8 afrag = frag_tr(kS, pk, kt * 16, 32 * j);  // k^T: rows kk, contraction over tokens
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] = mfma16x32(afrag, vB[j][ct], hacc[kt][ct]);
             }
@@ -246,13 +246,13 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: either g or gk must be provided.", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     Varlen vl;
     if ((rc = build_varlen(vl, op, cu, ci, kChunk, geom.T))) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
@@ -312,7 +312,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
         p.s_sn = sref->stride[0];
         p.s_sh = sref->stride[1];
     }
-    p.h = has_h ? static_cast<bf16 *>(h->data) : nullptr;
+    p.h = has_h ? static_cast<elem *>(h->data) : nullptr;
     if (has_h) {
         p.h_sb = h->stride[0];
         p.h_sh = h->stride[1];
@@ -350,11 +350,11 @@ struct DhuParams {
     int64_t gk_sb, gk_sh, gk_st;
     const float *dht;    // [N,Hv,K,V] fp32 or null
     int64_t t_sn, t_sh;
-    bf16 *dh;            // [B,Hv,NT,K,V]
+    elem *dh;            // [B,Hv,NT,K,V]
     int64_t h_sb, h_sh, h_sc;
     float *dh0_f32;      // [N,Hv,K,V] fp32 or null
     int64_t z_sn, z_sh;
-    bf16 *dh0_ref;       // [B,Hv,NT,K,V] bf16 (value stored at each sequence's first chunk) or null
+    elem *dh0_ref;       // [B,Hv,NT,K,V] bf16 (value stored at each sequence's first chunk) or null
     float scale;
 };
 
@@ -391,11 +391,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         chunk0 = p.geom.choff[n];
     }
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
-    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
-    const bf16 *wg = static_cast<const bf16 *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
-    const bf16 *og = static_cast<const bf16 *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
-    const bf16 *vg = static_cast<const bf16 *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
+    const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const elem *wg = static_cast<const elem *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const elem *og = static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
+    const elem *vg = static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
 
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
@@ -419,11 +419,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             } else if (tid < kChunk) {
                 gv = tid < len ? load_scalar(p.g, b, hv, start + tid) : 0.f;
             }
-            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pk, len, tid);
-            tq.commit(reinterpret_cast<bf16 *>(buf + L::q_off), pt, len, tid);
-            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pt, len, tid);
-            to.commit(reinterpret_cast<bf16 *>(buf + L::o_off), pv, len, tid);
-            tv.commit(reinterpret_cast<bf16 *>(buf + L::v_off), pv, len, tid);
+            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
+            tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pt, len, tid);
+            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pt, len, tid);
+            to.commit(reinterpret_cast<elem *>(buf + L::o_off), pv, len, tid);
+            tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
             if (GK) {
                 if (tid < K) gS[tid] = exp2f(gv);
                 if (tid < kChunk) fS[tid] = p.scale;
@@ -459,28 +459,28 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             dacc[kt][ct] = a;
         }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // terminal gradient loaded before the loop (vmcnt(0))
-    char *v2g = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + vcol0);
+    char *v2g = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + vcol0);
     __syncthreads();
 
     for (int c = nchunks - 1; c >= 0; --c) {
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
-        const bf16 *qS = reinterpret_cast<const bf16 *>(buf + L::q_off);
-        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
-        const bf16 *oS = reinterpret_cast<const bf16 *>(buf + L::o_off);
-        const bf16 *vS = reinterpret_cast<const bf16 *>(buf + L::v_off);
+        const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
+        const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
+        const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
+        const elem *oS = reinterpret_cast<const elem *>(buf + L::o_off);
+        const elem *vS = reinterpret_cast<const elem *>(buf + L::v_off);
         const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
         const float *fS = gS + (K > kChunk ? K : kChunk);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
 
-        bf16x8 hB[KS][CT];
+        elemx8 hB[KS][CT];
 #pragma unroll
         for (int j = 0; j < KS; ++j)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
         {   // dh of this chunk = the incoming gradient
-            bf16 *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+            elem *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -500,7 +500,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         for (int j = 0; j < KS; ++j)
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) {
-                const bf16x8 afrag = frag_kc(kS, pk, rt * 16, 32 * j);
+                const elemx8 afrag = frag_kc(kS, pk, rt * 16, 32 * j);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = mfma16x32(afrag, hB[j][ct], dv2[rt][ct]);
             }
@@ -509,7 +509,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const bf16x4 old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
+                const elemx4 old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int t = rt * 16 + 4 * lg + e;
@@ -540,12 +540,12 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            bf16x8 ob[CT], nb[CT];
+            elemx8 ob[CT], nb[CT];
             const f32x4 f0 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 4 * lg),
                         f1 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 16 + 4 * lg);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const bf16x8 raw = frag_tr(oS, pv, (wv * CT + ct) * 16, 32 * j);   // do[t][col], t = 32j + c(g,e)
+                const elemx8 raw = frag_tr(oS, pv, (wv * CT + ct) * 16, 32 * j);   // do[t][col], t = 32j + c(g,e)
                 f32x4 lo, hi;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -557,8 +557,8 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             }
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
-                const bf16x8 qf = frag_tr(qS, pt, kt * 16, 32 * j);
-                const bf16x8 wf = frag_tr(wS, pt, kt * 16, 32 * j);
+                const elemx8 qf = frag_tr(qS, pt, kt * 16, 32 * j);
+                const elemx8 wf = frag_tr(wS, pt, kt * 16, 32 * j);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     dacc[kt][ct] = mfma16x32(qf, ob[ct], dacc[kt][ct]);
@@ -579,7 +579,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 const int64_t off = (int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li;
                 if (p.dh0_f32) p.dh0_f32[n * p.z_sn + hv * p.z_sh + off] = dacc[kt][ct][e];
                 if (p.dh0_ref && nchunks > 0)
-                    p.dh0_ref[b * p.h_sb + hv * p.h_sh + (int64_t)chunk0 * p.h_sc + off] = (bf16)dacc[kt][ct][e];
+                    p.dh0_ref[b * p.h_sb + hv * p.h_sh + (int64_t)chunk0 * p.h_sc + off] = (elem)dacc[kt][ct][e];
             }
 }
 
@@ -606,15 +606,15 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     FLA_REQUIRE(!has_g || !use_exp2, FLA_ERR_UNSUPPORTED, "%s: the scalar gate g is a natural-log gate (use_exp2=false).", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom))) return rc;
-    const int bf = dt_bit(FLA_BF16);
+    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "dv2", dv2, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T))) return rc;
+    if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if (has_gk) {
         if ((rc = check_tensor(gK, op, "gK", 4, dt_bit(FLA_F32)))) return rc;
         FLA_REQUIRE(gK->shape[0] == geom.B && gK->shape[1] == geom.Hv && gK->shape[2] == geom.T && gK->shape[3] == geom.K &&
@@ -689,11 +689,11 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
         p.t_sn = dht->stride[0];
         p.t_sh = dht->stride[1];
     }
-    p.dh = static_cast<bf16 *>(dh->data);
+    p.dh = static_cast<elem *>(dh->data);
     p.h_sb = dh->stride[0];
     p.h_sh = dh->stride[1];
     p.h_sc = dh->stride[2];
-    if (has_dh0 && dh0_is_ref) p.dh0_ref = static_cast<bf16 *>(dh0->data);
+    if (has_dh0 && dh0_is_ref) p.dh0_ref = static_cast<elem *>(dh0->data);
     if (has_dh0 && !dh0_is_ref) {
         p.dh0_f32 = static_cast<float *>(dh0->data);
         p.z_sn = dh0->stride[0];
@@ -708,42 +708,46 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
 }  // namespace
 }  // namespace fla
 
-extern "C" int fla_chunk_gated_delta_rule_fwd_h_get_workspace_size(
+FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h_get_workspace_size)(
     const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g, const fla_tensor *gk,
     const fla_tensor *initial_state, bool output_final_state, int64_t chunk_size, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
     const fla_tensor *final_state, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_chunk_gated_delta_rule_fwd_h_get_workspace_size, k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices, state_v_first, h, v_new, final_state, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_fwd_h: workspace_size must not be null.");
     return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
                            state_v_first, h, v_new, final_state, nullptr, 0, nullptr, workspace_size);
 }
 
-extern "C" int fla_chunk_gated_delta_rule_fwd_h(
+FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h)(
     const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, const fla_tensor *g, const fla_tensor *gk,
     const fla_tensor *initial_state, bool output_final_state, int64_t chunk_size, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
     const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_chunk_gated_delta_rule_fwd_h, k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices, state_v_first, h, v_new, final_state, workspace, workspace_size, stream);
     return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
                            state_v_first, h, v_new, final_state, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
 }
 
-extern "C" int fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size(
+FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
     const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
     const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale, int64_t chunk_size, bool use_exp2,
     const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size, q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0, dv2, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_bwd_dhu: workspace_size must not be null.");
     return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
                              dv2, nullptr, 0, nullptr, workspace_size);
 }
 
-extern "C" int fla_chunk_gated_delta_rule_bwd_dhu(
+FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
     const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
     const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale, int64_t chunk_size, bool use_exp2,
     const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, void *workspace, uint64_t workspace_size,
     void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_gated_delta_rule_bwd_dhu, q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0, dv2, workspace, workspace_size, stream);
     return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
                              dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
 }

@@ -27,10 +27,10 @@ __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 // ds_read_b64_tr_b16: within each group of 16 lanes, lane s supplies the address
 // of 4 consecutive 16-bit elements; lane i receives element (i % 4) of lanes
 // i/4, i/4 + 4, i/4 + 8, i/4 + 12.
-__device__ __forceinline__ bf16x4 lds_tr4(const bf16 *p) {
+__device__ __forceinline__ elemx4 lds_tr4(const elem *p) {
     typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
     s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)p);
-    return __builtin_bit_cast(bf16x4, r);
+    return __builtin_bit_cast(elemx4, r);
 }
 
 // Operand with rows r0..r0+15 and contraction c0..c0+31 along the contiguous
@@ -38,32 +38,32 @@ __device__ __forceinline__ bf16x4 lds_tr4(const bf16 *p) {
 // The two 8-byte halves stay separate LDS reads: fused into one two-address read (ds_read2_b64) the pair
 // costs four times the LDS cycles on gfx950, which is why this library is built with the load/store
 // merging pass of the backend switched off.
-__device__ __forceinline__ bf16x8 frag_kc(const bf16 *tile, int pitch, int r0, int c0) {
+__device__ __forceinline__ elemx8 frag_kc(const elem *tile, int pitch, int r0, int c0) {
     const int l = lane_id(), i = l & 15, g = l >> 4;
     const int off = (r0 + i) * pitch + c0 + 4 * g;
-    return cat8(*reinterpret_cast<const bf16x4 *>(tile + off), *reinterpret_cast<const bf16x4 *>(tile + off + 16));
+    return cat8(*reinterpret_cast<const elemx4 *>(tile + off), *reinterpret_cast<const elemx4 *>(tile + off + 16));
 }
 // 16-wide contraction variant for v_mfma_f32_16x16x16_bf16.
-__device__ __forceinline__ bf16x4 frag_kc4(const bf16 *tile, int pitch, int r0, int c0) {
+__device__ __forceinline__ elemx4 frag_kc4(const elem *tile, int pitch, int r0, int c0) {
     const int l = lane_id(), i = l & 15, g = l >> 4;
-    return *reinterpret_cast<const bf16x4 *>(tile + (r0 + i) * pitch + c0 + 4 * g);
+    return *reinterpret_cast<const elemx4 *>(tile + (r0 + i) * pitch + c0 + 4 * g);
 }
 
 // Operand with index r0..r0+15 along the contiguous dimension and contraction
 // c0..c0+31 along the rows of `tile`:  slot (g,e) = tile[c0 + c(g,e)][r0 + i].
-__device__ __forceinline__ bf16x8 frag_tr(const bf16 *tile, int pitch, int r0, int c0) {
+__device__ __forceinline__ elemx8 frag_tr(const elem *tile, int pitch, int r0, int c0) {
     const int l = lane_id(), i = l & 15, g = l >> 4;
-    const bf16 *p = tile + (c0 + 4 * g + (i >> 2)) * pitch + r0 + 4 * (i & 3);
+    const elem *p = tile + (c0 + 4 * g + (i >> 2)) * pitch + r0 + 4 * (i & 3);
     return cat8(lds_tr4(p), lds_tr4(p + 16 * pitch));
 }
-__device__ __forceinline__ bf16x4 frag_tr4(const bf16 *tile, int pitch, int r0, int c0) {
+__device__ __forceinline__ elemx4 frag_tr4(const elem *tile, int pitch, int r0, int c0) {
     const int l = lane_id(), i = l & 15, g = l >> 4;
     return lds_tr4(tile + (c0 + 4 * g + (i >> 2)) * pitch + r0 + 4 * (i & 3));
 }
 
 // Two accumulator tiles (rows 0..15 and 16..31 of a 32-row block) as an operand
 // whose contraction runs over those rows.
-__device__ __forceinline__ bf16x8 frag_from_acc(f32x4 lo, f32x4 hi) { return cat8(cvt4(lo), cvt4(hi)); }
+__device__ __forceinline__ elemx8 frag_from_acc(f32x4 lo, f32x4 hi) { return cat8(cvt4(lo), cvt4(hi)); }
 
 // Accumulator tile element e of lane l sits at row 4*(l/16)+e, column l%16.
 __device__ __forceinline__ int acc_row(int e) { return 4 * (lane_id() >> 4) + e; }
@@ -82,7 +82,7 @@ template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
     static constexpr int N = NROWS * CPR / THREADS;          // pieces per thread
     static_assert(NROWS * CPR % THREADS == 0, "tile does not divide among the copying threads");
     u32x4 r[N];
-    __device__ __forceinline__ void fetch(const bf16 *gsrc, int64_t gstride, int valid, int tid) {
+    __device__ __forceinline__ void fetch(const elem *gsrc, int64_t gstride, int valid, int tid) {
         const int last = valid > 0 ? valid - 1 : 0;
 #pragma unroll
         for (int m = 0; m < N; ++m) {
@@ -94,7 +94,7 @@ template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
             r[m] = *reinterpret_cast<const u32x4 *>(gsrc + off);
         }
     }
-    __device__ __forceinline__ void commit(bf16 *tile, int pitch, int valid, int tid) const {
+    __device__ __forceinline__ void commit(elem *tile, int pitch, int valid, int tid) const {
 #pragma unroll
         for (int m = 0; m < N; ++m) {
             const int idx = m * THREADS + tid;
@@ -104,7 +104,7 @@ template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
     }
 };
 template <int THREADS>
-__device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsrc, int64_t gstride, int nrows,
+__device__ __forceinline__ void load_tile(elem *tile, int pitch, const elem *gsrc, int64_t gstride, int nrows,
                                           int ncols, int valid, int tid) {
     const int cpr = ncols >> 3;  // 16-byte chunks per row
     const int total = nrows * cpr;
@@ -121,12 +121,12 @@ __device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsr
     }
 }
 template <int THREADS>
-__device__ __forceinline__ void load_tile(bf16 *tile, int pitch, const bf16 *gsrc, int64_t gstride, int nrows,
+__device__ __forceinline__ void load_tile(elem *tile, int pitch, const elem *gsrc, int64_t gstride, int nrows,
                                           int ncols, int valid) {
     load_tile<THREADS>(tile, pitch, gsrc, gstride, nrows, ncols, valid, (int)threadIdx.x);
 }
 template <int THREADS>
-__device__ __forceinline__ void store_tile(bf16 *gdst, int64_t gstride, const bf16 *tile, int pitch, int ncols,
+__device__ __forceinline__ void store_tile(elem *gdst, int64_t gstride, const elem *tile, int pitch, int ncols,
                                            int valid) {
     const int cpr = ncols >> 3;
     for (int idx = threadIdx.x; idx < valid * cpr; idx += THREADS) {
@@ -139,7 +139,7 @@ __device__ __forceinline__ void store_tile(bf16 *gdst, int64_t gstride, const bf
 // Neighbouring lanes hold neighbouring columns; they swap half of their values so that every
 // lane writes two whole dwords (even lanes rows e = 0,1; odd lanes rows e = 2,3 of the column
 // pair) instead of four 16-bit pieces, which also keeps the write free of bank conflicts.
-__device__ __forceinline__ void acc_to_tile(bf16 *tile, int pitch, int r0, int c0, f32x4 acc) {
+__device__ __forceinline__ void acc_to_tile(elem *tile, int pitch, int r0, int c0, f32x4 acc) {
     const int l = lane_id(), li = l & 15, lg = l >> 4;
     const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
     const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
@@ -148,7 +148,7 @@ __device__ __forceinline__ void acc_to_tile(bf16 *tile, int pitch, int r0, int c
     const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
     const unsigned left = odd ? recv : p01;    // column li & ~1
     const unsigned right = odd ? p23 : recv;   // column li | 1
-    bf16 *dst = tile + (r0 + 4 * lg + (odd ? 2 : 0)) * pitch + c0 + (li & ~1);
+    elem *dst = tile + (r0 + 4 * lg + (odd ? 2 : 0)) * pitch + c0 + (li & ~1);
     *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);          // low halves
     *reinterpret_cast<unsigned *>(dst + pitch) = __builtin_amdgcn_perm(right, left, 0x07060302u);  // high halves
 }
@@ -185,16 +185,16 @@ template <int K> struct KTile {
         if (K == 128) return r * 128 + ((((col >> 3) ^ f(r)) << 3) | (col & 7));
         return r * pitch + col;
     }
-    static __device__ __forceinline__ bf16x8 kc(const bf16 *t, int r0, int c0) {
+    static __device__ __forceinline__ elemx8 kc(const elem *t, int r0, int c0) {
         const int l = lane_id(), i = l & 15, g = l >> 4;
-        return cat8(*reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 4 * g)),
-                    *reinterpret_cast<const bf16x4 *>(t + off(r0 + i, c0 + 16 + 4 * g)));
+        return cat8(*reinterpret_cast<const elemx4 *>(t + off(r0 + i, c0 + 4 * g)),
+                    *reinterpret_cast<const elemx4 *>(t + off(r0 + i, c0 + 16 + 4 * g)));
     }
-    static __device__ __forceinline__ bf16x4 tr4(const bf16 *t, int r0, int c0) {
+    static __device__ __forceinline__ elemx4 tr4(const elem *t, int r0, int c0) {
         const int l = lane_id(), i = l & 15, g = l >> 4;
         return lds_tr4(t + off(c0 + 4 * g + (i >> 2), r0 + 4 * (i & 3)));
     }
-    static __device__ __forceinline__ bf16x8 tr(const bf16 *t, int r0, int c0) {
+    static __device__ __forceinline__ elemx8 tr(const elem *t, int r0, int c0) {
         const int l = lane_id(), i = l & 15, g = l >> 4;
         return cat8(lds_tr4(t + off(c0 + 4 * g + (i >> 2), r0 + 4 * (i & 3))),
                     lds_tr4(t + off(c0 + 16 + 4 * g + (i >> 2), r0 + 4 * (i & 3))));

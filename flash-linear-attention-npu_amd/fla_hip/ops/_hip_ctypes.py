@@ -52,6 +52,7 @@ OP_ARGTYPES = {
                        + [_T] * 4,
     "prepare_wy_repr_bwd_da": [_T] * 7 + [_IA, _IA, ctypes.c_int64, _T],
     "prepare_wy_repr_bwd_full": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
+    "prepare_wy_repr_bwd": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
 }
 
 
@@ -748,6 +749,28 @@ def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu
         "prepare_wy_repr_bwd_full", OP_ARGTYPES["prepare_wy_repr_bwd_full"],
         lambda ctx: [
             ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"), ctx.tensor(dA, "dA"),
+            ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(dbeta, "dbeta"), ctx.tensor(dg, "dg"),
+        ],
+        outputs,
+    )
+    return dk, dv, _as_dtype(dbeta, beta), _as_dtype(dg, g)
+
+
+def npu_prepare_wy_repr_bwd(k, v, beta, A, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):
+    """_aclnn_ctypes.py:284-321: bwd_da and bwd_full in one library call (dA stays in the workspace).
+    Returns (dk, dv, dbeta, dg) like npu_prepare_wy_repr_bwd_full."""
+    dk = _empty_like(k)
+    dv = _empty_like(v)
+    dbeta = _f32_like(beta)
+    dg = _f32_like(g)
+    outputs = (dk, dv, dbeta, dg)
+    dk, dv, dbeta, dg = _call_op(
+        "prepare_wy_repr_bwd", OP_ARGTYPES["prepare_wy_repr_bwd"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"),
             ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
             ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
             ctypes.c_int64(int(chunk_size)),

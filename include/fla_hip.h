@@ -448,6 +448,19 @@ int fla_prepare_wy_repr_bwd_da(
     const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
     int64_t chunk_size, const fla_tensor *dA, void *workspace, uint64_t workspace_size, void *stream);
 
+/* prepare_wy_repr_bwd - replaces aclnnPrepareWyReprBwd (_aclnn_ctypes.py:284-321): bwd_da followed by
+ * bwd_full in one call; the intermediate dA (bf16, [B,Hv,T,C]) lives in the workspace. */
+int fla_prepare_wy_repr_bwd_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg,
+    uint64_t *workspace_size);
+int fla_prepare_wy_repr_bwd(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+    const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg,
+    void *workspace, uint64_t workspace_size, void *stream);
+
 /* prepare_wy_repr_bwd_full - replaces aclnnPrepareWyReprBwdFull (_aclnn_ctypes.py:242-279):
  * dk [B,Hk,T,K], dv [B,Hv,T,V] bf16; dbeta, dg [B,Hv,T] f32; dA as written by bwd_da. */
 int fla_prepare_wy_repr_bwd_full_get_workspace_size(

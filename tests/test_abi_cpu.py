@@ -356,10 +356,17 @@ def test_gdn_backward_wrappers_operands_and_outputs():
     assert dk2.shape == q.shape and dv2.shape == v.shape and db.shape == g.shape and dg2.shape == g.shape
     assert db.dtype == f32 and dg2.dtype == f32
 
+    cap, (dk2, dv2, db, dg2) = capture_call(H.npu_prepare_wy_repr_bwd, q, v, g, A, w, v, g, 64)    # :284-321
+    assert_args_match_argtypes(cap)
+    assert [n for n in cap["names"] if n != "int_array"] == [
+        "k", "v", "beta", "A", "dw", "du", "g", "dk", "dv", "dbeta", "dg"]
+    assert dk2.shape == q.shape and dv2.shape == v.shape and db.shape == g.shape and dg2.dtype == f32
+
 
 def test_backward_ops_are_exported_under_both_names():
     from fla_hip import ops
-    for name in ("chunk_bwd_dv_local", "chunk_bwd_dqkwg", "prepare_wy_repr_bwd_da", "prepare_wy_repr_bwd_full"):
+    for name in ("chunk_bwd_dv_local", "chunk_bwd_dqkwg", "prepare_wy_repr_bwd_da", "prepare_wy_repr_bwd_full",
+                 "prepare_wy_repr_bwd"):
         assert getattr(ops, name) is getattr(ops, "npu_" + name)
 
 

@@ -25,24 +25,24 @@ CASES = [
 ]
 
 
-def make(B, T, Hv, Hk, K, V, cu, seed):
+def make(B, T, Hv, Hk, K, V, cu, seed, dtype=BF):
     """Forward quantities of one problem, every tensor rounded to the dtype the operators exchange."""
     gen = torch.Generator().manual_seed(seed)
     rn = lambda *s: torch.randn(*s, generator=gen)
-    q = F.normalize(rn(B, Hk, T, K), dim=-1).to(BF)
-    k = F.normalize(rn(B, Hk, T, K), dim=-1).to(BF)
-    v = rn(B, Hv, T, V).to(BF)
+    q = F.normalize(rn(B, Hk, T, K), dim=-1).to(dtype)
+    k = F.normalize(rn(B, Hk, T, K), dim=-1).to(dtype)
+    v = rn(B, Hv, T, V).to(dtype)
     beta = torch.sigmoid(rn(B, Hv, T))
     g = F.logsigmoid(rn(B, Hv, T))
     N = B if cu is None else len(cu) - 1
     h0 = rn(N, Hv, K, V) * 0.1
-    do = rn(B, Hv, T, V).to(BF)
+    do = rn(B, Hv, T, V).to(dtype)
     dht = rn(N, Hv, K, V) * 0.1
     G = gdn.chunk_local_cumsum(g, 64, cu_seqlens=cu)
     A0 = gdn.chunk_scaled_dot_kkt(k, G, beta, 64, cu_seqlens=cu)
-    A = gdn.solve_tri(A0, cu_seqlens=cu, output_dtype=BF)
-    w, u = gdn.recompute_w_u_fwd(k, v, beta, A, 64, g=G, cu_seqlens=cu, output_dtype=BF)
-    h, v_new, _ = gdn.chunk_gated_delta_rule_fwd_h(k, w, u, G, initial_state=h0, chunk=64, cu_seqlens=cu, output_dtype=BF)
+    A = gdn.solve_tri(A0, cu_seqlens=cu, output_dtype=dtype)
+    w, u = gdn.recompute_w_u_fwd(k, v, beta, A, 64, g=G, cu_seqlens=cu, output_dtype=dtype)
+    h, v_new, _ = gdn.chunk_gated_delta_rule_fwd_h(k, w, u, G, initial_state=h0, chunk=64, cu_seqlens=cu, output_dtype=dtype)
     return dict(q=q, k=k, v=v, beta=beta, g=g, G=G, A=A, w=w, u=u, h=h, v_new=v_new, h0=h0, do=do, dht=dht)
 
 
@@ -50,12 +50,15 @@ def to_dev(d, dev):
     return {n: t.to(dev) for n, t in d.items()}
 
 
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", CASES)
-def test_backward_operators_against_oracle(dev, case):
+def test_backward_operators_against_oracle(dev, case, dtype):
     from fla_hip import ops
     B, T, Hv, Hk, K, V, cu = case
     scale = K ** -0.5
-    d = make(B, T, Hv, Hk, K, V, cu, seed=T + K)
+    d = make(B, T, Hv, Hk, K, V, cu, seed=T + K, dtype=dtype)
+    BF = dtype                   # the dtype the operators exchange
+    TOL_BF16 = 2e-2 if dtype == torch.bfloat16 else 5e-3
     x = to_dev(d, dev)
     kw = dict(cu_seqlens=cu)
 
@@ -110,15 +113,22 @@ def test_backward_operators_against_oracle(dev, case):
         st = err_stats(got, ref)
         assert st["rel_max"] <= TOL_BF16, f"{name}: {st}"
 
+    # prepare_wy_repr_bwd: one call == bwd_da followed by bwd_full, bit for bit
+    one = ops.prepare_wy_repr_bwd(x["k"], x["v"], x["beta"], x["A"], dwb.to(dev), dv2.to(dev), x["G"], 64, **kw)
+    two = ops.prepare_wy_repr_bwd_full(x["k"], x["v"], x["beta"], x["A"], dA, dwb.to(dev), dv2.to(dev), x["G"], 64, **kw)
+    for name, a_, b_ in zip(("dk", "dv", "dbeta", "dg"), one, two):
+        assert torch.equal(a_, b_), name
 
+
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", [CASES[1], CASES[5]])
-def test_backward_pipeline_against_recurrence_autograd(dev, case):
+def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
     """The composed GPU backward against autograd (fp64) through the per-token recurrence on the same bf16
     inputs: every gradient within 2e-2 of its own scale."""
     from fla_hip import pipeline
     B, T, Hv, Hk, K, V, cu = case
     scale = K ** -0.5
-    d = make(B, T, Hv, Hk, K, V, cu, seed=77)
+    d = make(B, T, Hv, Hk, K, V, cu, seed=77, dtype=dtype)
     dd = torch.float64
     leaf = {n: d[n].to(dd).requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
     o, final = gdn.naive_recurrent_gated_delta_rule(leaf["q"], leaf["k"], leaf["v"], leaf["g"], leaf["beta"], scale,
