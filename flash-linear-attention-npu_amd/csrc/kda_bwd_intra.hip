@@ -31,7 +31,7 @@ __device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) {
 
 struct BwdIntraParams {
     ChunkGeom geom;              // Hv = heads, K = head size
-    const bf16 *q, *k;
+    const elem *q, *k;
     const float *gk, *dq, *dk, *dg;
     float *dq_o, *dk_o, *dg_o;
     int64_t sb, sh, st;          // strides of (batch, head, token) of the [..,K] tensors
@@ -50,8 +50,8 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
     float *akS = aqS + kChunk * pa;                 // [64][pa] tril(dAkk)
     float *gS = akS + kChunk * pa;                  // [64][pg]
     float *bS = gS + kChunk * pg;                   // [64]
-    bf16 *qS = reinterpret_cast<bf16 *>(bS + kChunk);
-    bf16 *kS = qS + kChunk * pk;
+    elem *qS = reinterpret_cast<elem *>(bS + kChunk);
+    elem *kS = qS + kChunk * pk;
 
     const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     int seq, start, len;
@@ -201,8 +201,8 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: chunk_size must be 64.", op);
     const int rank = ib < 0 ? 3 : 4;
     int rc;
-    if ((rc = check_tensor(q, op, "q", rank, dt_bit(FLA_BF16)))) return rc;
-    if ((rc = check_tensor(k, op, "k", rank, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_tensor(q, op, "q", rank, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_tensor(k, op, "k", rank, dt_bit(kElemDtype)))) return rc;
     const fla_tensor *f32s[] = {gk, dq, dk, dg, dq_o, dk_o, dg_o};
     const char *f32n[] = {"gk", "dq", "dk", "dg", "dq_out", "dk_out", "dg_out"};
     for (int i = 0; i < 7; ++i) {
@@ -217,7 +217,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     FLA_REQUIRE(B > 0 && H > 0 && T > 0, FLA_ERR_SHAPE, "%s: B/H/T must be positive.", op);
     FLA_REQUIRE(K == 64 || K == 128 || K == 256, FLA_ERR_UNSUPPORTED, "%s: K must be 64, 128 or 256.", op);
     FLA_REQUIRE(B < 65536 && H < 65536 && T < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents too large.", op);
-    if ((rc = check_tensor(beta, op, "beta", rank - 1, dt_bit(FLA_BF16) | dt_bit(FLA_F32)))) return rc;
+    if ((rc = check_tensor(beta, op, "beta", rank - 1, dt_bit(kElemDtype) | dt_bit(FLA_F32)))) return rc;
     const fla_tensor *sc[] = {beta, db, db_o};
     const char *scn[] = {"beta", "db", "db_out"};
     for (int i = 0; i < 3; ++i) {
@@ -268,8 +268,8 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
 
     BwdIntraParams p{};
     p.geom = geom;
-    p.q = static_cast<const bf16 *>(q->data);
-    p.k = static_cast<const bf16 *>(k->data);
+    p.q = static_cast<const elem *>(q->data);
+    p.k = static_cast<const elem *>(k->data);
     p.gk = static_cast<const float *>(gk->data);
     p.dq = static_cast<const float *>(dq->data);
     p.dk = static_cast<const float *>(dk->data);
@@ -280,7 +280,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.sb = ib < 0 ? 0 : q->stride[ib];
     p.sh = q->stride[ih];
     p.st = q->stride[it];
-    p.beta = View3{beta->data, ib < 0 ? 0 : beta->stride[ib], beta->stride[ih], beta->stride[it], beta->dtype == FLA_BF16 ? 1 : 0};
+    p.beta = View3{beta->data, ib < 0 ? 0 : beta->stride[ib], beta->stride[ih], beta->stride[it], beta->dtype == FLA_F32 ? 0 : 1};
     p.db = static_cast<const float *>(db->data);
     p.db_o = static_cast<float *>(db_o->data);
     p.daqk = static_cast<const float *>(daqk->data);
@@ -295,23 +295,25 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
 }  // namespace
 }  // namespace fla
 
-extern "C" int fla_chunk_kda_bwd_intra_get_workspace_size(
+FLA_ENTRY(fla_chunk_kda_bwd_intra_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
     const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
     const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
     const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
     const fla_tensor *dg_out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra_get_workspace_size, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_intra: workspace_size must not be null.");
     return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
                                layout, dq_out, dk_out, db_out, dg_out, nullptr, 0, nullptr, workspace_size);
 }
 
-extern "C" int fla_chunk_kda_bwd_intra(
+FLA_ENTRY(fla_chunk_kda_bwd_intra)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
     const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
     const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
     const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size, stream);
     return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
                                layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size,
                                static_cast<hipStream_t>(stream), nullptr);

@@ -35,7 +35,7 @@ struct KdaIntraParams {
     ChunkGeom geom;
     View4 q, k, v;       // bf16, strides of (batch, head, token) in the caller's layout
     const void *g;       // raw gate, f32 or bf16, same layout family
-    int g_bf16;
+    int g_elem;
     int64_t g_sb, g_sh, g_st;
     View3 beta;
     const float *a_log, *dt_bias;
@@ -43,14 +43,14 @@ struct KdaIntraParams {
     float lower_bound;
     float scale;
     float *gk;                // [B,Hv,T,K] or null
-    bf16 *aqk, *akk;          // [B,Hv,T,64]
-    bf16 *w, *u, *qg, *kg;    // [B,Hv,T,K] / [B,Hv,T,V]
+    elem *aqk, *akk;          // [B,Hv,T,64]
+    elem *w, *u, *qg, *kg;    // [B,Hv,T,K] / [B,Hv,T,V]
     float *dec;               // [B,NT,Hv,K]: 2^{g_last} of every chunk
 };
 
 // A operand of a 16x16x16 product from four fp32 values, split into a bf16 head and remainder.
 struct HiLo {
-    bf16x4 hi, lo;
+    elemx4 hi, lo;
 };
 __device__ __forceinline__ HiLo split(f32x4 x) {
     HiLo r;
@@ -69,10 +69,10 @@ __device__ __forceinline__ f32x4 mm3(f32x4 a, f32x4 b, f32x4 acc) {
 // rows row0..row0+15 of `tile` times 2^{+-(g_row - g_anchor)} as an MFMA operand (contraction
 // slots 32j .. 32j+31 along the channels)
 template <bool LEFT>
-__device__ __forceinline__ bf16x8 scaled_frag(const bf16 *tile, int pitch, const float *gS, int pg, int row0, int arow,
+__device__ __forceinline__ elemx8 scaled_frag(const elem *tile, int pitch, const float *gS, int pg, int row0, int arow,
                                               int j) {
     const int l = lane_id(), li = l & 15, lg = l >> 4;
-    const bf16x8 raw = frag_kc(tile, pitch, row0, 32 * j);
+    const elemx8 raw = frag_kc(tile, pitch, row0, 32 * j);
     const float *gr = gS + (row0 + li) * pg + 32 * j + 4 * lg;
     const float *ga = gS + arow * pg + 32 * j + 4 * lg;
     const f32x4 g0 = lds4(gr), g1 = lds4(gr + 16), s0 = lds4(ga), s1 = lds4(ga + 16);
@@ -94,7 +94,7 @@ template <int K, int V> struct IntraSmem {
 
 // Everything a wave does after the gate scan.  W = wave index (static so tile loops unroll).
 template <int K, int V, int W>
-__device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf16 *kS, bf16 *vS, bf16 *akS, bf16 *aqS,
+__device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
                                            int64_t dec_base) {
     using S = IntraSmem<K, V>;
@@ -110,17 +110,17 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
     for (int c = 0; c <= R2; ++c) qacc[c] = zero4();
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
-        const bf16x8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
+        const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
 #pragma unroll
         for (int c = 0; c <= R1; ++c) {
-            const bf16x8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+            const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
             kacc[c] = mfma16x32(lk, rk, kacc[c]);
             if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
         }
-        const bf16x8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+        const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
 #pragma unroll
         for (int c = 0; c <= R2; ++c) {
-            const bf16x8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+            const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
             qacc[c] = mfma16x32(lq, rk, qacc[c]);
         }
     }
@@ -152,24 +152,24 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
         Y[e] = (r == li ? 1.f : 0.f) - a1[e];   // (I - A^T)[r][li]
     }
     {
-        const bf16x4 A1 = cvt4(a1), A2 = cvt4(a2);
+        const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
         const f32x4 S1 = mfma16x16(A1, A2, zero4());   // A^2
         const f32x4 T1 = mfma16x16(A2, A1, zero4());   // (A^2)^T
-        const bf16x4 S1b = cvt4(S1), T1b = cvt4(T1);
+        const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
         Y = mfma16x16(S1b, cvt4(Y), Y);
         const f32x4 S2 = mfma16x16(T1b, S1b, zero4());  // A^4
         const f32x4 T2 = mfma16x16(S1b, T1b, zero4());  // (A^4)^T
-        const bf16x4 S2b = cvt4(S2);
+        const elemx4 S2b = cvt4(S2);
         Y = mfma16x16(S2b, cvt4(Y), Y);
         const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());  // A^8
         Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
     }
     // lane holds Dinv[li][4lg+e]
     *reinterpret_cast<f32x4 *>(aS + (16 * R1 + li) * pa + 16 * R1 + 4 * lg) = Y;
-    *reinterpret_cast<bf16x4 *>(akS + (16 * R1 + li) * pb + 16 * R1 + 4 * lg) = cvt4(Y);
+    *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * R1 + 4 * lg) = cvt4(Y);
 #pragma unroll
     for (int c = R1 + 1; c < 4; ++c)
-        *reinterpret_cast<bf16x4 *>(akS + (16 * R1 + li) * pb + 16 * c + 4 * lg) = bf16x4{(bf16)0.f, (bf16)0.f, (bf16)0.f, (bf16)0.f};
+        *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * c + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
     __syncthreads();
 
     // ---- off-diagonal blocks of the inverse, column block W: X_rc = -Dinv_r sum_m A_rm X_mc --------
@@ -191,10 +191,10 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
     // ---- gated operands: qg, kg to memory; k beta 2^g over the q tile ----------------------------------
     for (int idx = threadIdx.x; idx < kChunk * (K / 8); idx += kThreads) {
         const int r = idx / (K / 8), c8 = (idx % (K / 8)) * 8;
-        const bf16x8 q8 = *reinterpret_cast<const bf16x8 *>(qS + r * pq + c8);
-        const bf16x8 k8 = *reinterpret_cast<const bf16x8 *>(kS + r * pk + c8);
+        const elemx8 q8 = *reinterpret_cast<const elemx8 *>(qS + r * pq + c8);
+        const elemx8 k8 = *reinterpret_cast<const elemx8 *>(kS + r * pk + c8);
         const float br = bS[r];
-        bf16x8 qg8, kg8, kb8;
+        elemx8 qg8, kg8, kb8;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + 63 * pg + c8 + 4 * h);
@@ -206,7 +206,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
                 b[e] = kk * ex2(gl[e] - gg[e]);
                 c[e] = kk * br * eg;
             }
-            const bf16x4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
+            const elemx4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 qg8[4 * h + e] = a4[e];
@@ -215,10 +215,10 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
             }
         }
         if (r < len) {
-            *reinterpret_cast<bf16x8 *>(p.qg + (row_base + r) * K + c8) = qg8;
-            *reinterpret_cast<bf16x8 *>(p.kg + (row_base + r) * K + c8) = kg8;
+            *reinterpret_cast<elemx8 *>(p.qg + (row_base + r) * K + c8) = qg8;
+            *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
         }
-        *reinterpret_cast<bf16x8 *>(qS + r * pq + c8) = kb8;
+        *reinterpret_cast<elemx8 *>(qS + r * pq + c8) = kb8;
     }
     if (threadIdx.x < K) p.dec[dec_base + threadIdx.x] = ex2(gS[63 * pg + threadIdx.x]);
     __syncthreads();
@@ -231,7 +231,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, bf16 *qS, bf
     for (int ct = 0; ct < V / 16; ++ct) uacc[ct] = zero4();
 #pragma unroll
     for (int j = 0; j < (W < 2 ? 1 : 2); ++j) {   // Akk is lower triangular
-        const bf16x8 a = frag_kc(akS, pb, 16 * W, 32 * j);
+        const elemx8 a = frag_kc(akS, pb, 16 * W, 32 * j);
 #pragma unroll
         for (int ct = 0; ct < K / 16; ++ct) wacc[ct] = mfma16x32(a, frag_tr(qS, pq, 16 * ct, 32 * j), wacc[ct]);
 #pragma unroll
@@ -250,11 +250,11 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb, SEG = S::SEG;
-    bf16 *qS = reinterpret_cast<bf16 *>(smem);
-    bf16 *kS = qS + kChunk * pq;
-    bf16 *vS = kS + kChunk * pk;
-    bf16 *akS = vS + kChunk * pv;
-    bf16 *aqS = akS + kChunk * pb;
+    elem *qS = reinterpret_cast<elem *>(smem);
+    elem *kS = qS + kChunk * pq;
+    elem *vS = kS + kChunk * pk;
+    elem *akS = vS + kChunk * pv;
+    elem *aqS = akS + kChunk * pb;
     float *gS = reinterpret_cast<float *>(aqS + kChunk * pb);
     float *aS = gS + kChunk * pg;
     float *bS = aS + kChunk * pa;
@@ -266,9 +266,9 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x;
 
-    const bf16 *qg = static_cast<const bf16 *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
-    const bf16 *kg = static_cast<const bf16 *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    const bf16 *vg = static_cast<const bf16 *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
     // gate loads first (thread = (token segment, channel)); branch-free with a clamped token index so that
     // they are all in flight together with the tile loads below
     const int64_t row_base = ((int64_t)b * p.geom.Hv + hv) * p.geom.T + start;   // head-major row of token 0
@@ -282,10 +282,10 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
     float raw[TS];
     {
         const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
-        if (p.g_bf16) {
+        if (p.g_elem) {
 #pragma unroll
             for (int j = 0; j < TS; ++j)
-                raw[j] = (float)static_cast<const bf16 *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
+                raw[j] = (float)static_cast<const elem *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
         } else {
 #pragma unroll
             for (int j = 0; j < TS; ++j)
@@ -310,7 +310,7 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
         for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) {   // v * beta
             const int idx = m * kThreads + tid;
             const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
-            const bf16x8 v8 = __builtin_bit_cast(bf16x8, tv.r[m]);
+            const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
             const float bb = r < len ? br[m] : 0.f;
             f32x4 lo, hi;
 #pragma unroll
@@ -318,7 +318,7 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
                 lo[e] = (float)v8[e] * bb;
                 hi[e] = (float)v8[4 + e] * bb;
             }
-            *reinterpret_cast<bf16x8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
+            *reinterpret_cast<elemx8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
         }
     }
     if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
@@ -366,13 +366,13 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
 // =============================================================================================
 struct KdaScanParams {
     ChunkGeom geom;
-    const bf16 *w, *u, *qg, *kg, *aqk;   // head-major [B,Hv,T,*]
+    const elem *w, *u, *qg, *kg, *aqk;   // head-major [B,Hv,T,*]
     const float *dec;                    // [B,NT,Hv,K]
     View4 o;                             // attention output in the caller's layout
-    bf16 *v_new;                         // [B,Hv,T,V] or null
+    elem *v_new;                         // [B,Hv,T,V] or null
     const float *h0;
     float *hT;
-    bf16 *h;
+    elem *h;
     int64_t h_sb, h_sc, h_sh;            // strides of h over (batch, chunk, head)
     int64_t s_sn, s_sh;                  // strides of h0 / hT over (sequence, head)
     int v_first;
@@ -431,11 +431,11 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             ta.fetch(p.aqk + row * kChunk, kChunk, len, tid);
             float dec = 0.f;
             if (tid < K) dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c) * p.geom.Hv + hv) * K + tid];
-            tw.commit(reinterpret_cast<bf16 *>(buf + L::w_off), pw, len, tid);
-            tq.commit(reinterpret_cast<bf16 *>(buf + L::q_off), pw, len, tid);
-            tk.commit(reinterpret_cast<bf16 *>(buf + L::k_off), pt, len, tid);
-            tu.commit(reinterpret_cast<bf16 *>(buf + L::u_off), pu, len, tid);
-            ta.commit(reinterpret_cast<bf16 *>(buf + L::a_off), pb, len, tid);
+            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
+            tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pw, len, tid);
+            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pt, len, tid);
+            tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
+            ta.commit(reinterpret_cast<elem *>(buf + L::a_off), pb, len, tid);
             if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = dec;
         };
         if (nchunks > 0) load(0);
@@ -464,26 +464,26 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         hacc[kt] = a;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
-    char *og = reinterpret_cast<char *>(static_cast<bf16 *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
+    char *og = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-        const bf16 *wS = reinterpret_cast<const bf16 *>(buf + L::w_off);
-        const bf16 *qS = reinterpret_cast<const bf16 *>(buf + L::q_off);
-        const bf16 *kS = reinterpret_cast<const bf16 *>(buf + L::k_off);
-        const bf16 *uS = reinterpret_cast<const bf16 *>(buf + L::u_off);
-        const bf16 *aS = reinterpret_cast<const bf16 *>(buf + L::a_off);
+        const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
+        const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
+        const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
+        const elem *uS = reinterpret_cast<const elem *>(buf + L::u_off);
+        const elem *aS = reinterpret_cast<const elem *>(buf + L::a_off);
         const float *dS = reinterpret_cast<const float *>(buf + L::d_off);
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
         const int64_t row = head_row + start;
 
-        bf16x8 hB[KS];
+        elemx8 hB[KS];
 #pragma unroll
         for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
         if (p.h) {
-            bf16 *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c) * p.h_sc + hv * p.h_sh;
+            elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c) * p.h_sc + hv * p.h_sh;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -503,7 +503,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
-            const bf16x4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
+            const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 vn[rt][e] = (float)uu[e] - vn[rt][e];
@@ -516,7 +516,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             for (int rt = 0; rt < 4; ++rt) acc_to_global(vg, (int64_t)V * 2, rt * 16, len, vn[rt]);
         }
         // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same bf16 v_new operand serves both)
-        bf16x8 vB[2];
+        elemx8 vB[2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
 #pragma unroll
@@ -633,9 +633,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     if ((rc = parse_layout(op, layout, L))) return rc;
     FLA_REQUIRE(chunk_size == 64 || chunk_size == 128, FLA_ERR_SHAPE, "%s: chunk_size must be 64 or 128.", op);
     FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: only chunk_size 64 is implemented.", op);
-    if ((rc = check_tensor(q, op, "q", L.rank3() ? 3 : 4, dt_bit(FLA_BF16) | dt_bit(FLA_F16)))) return rc;
-    FLA_REQUIRE(q->dtype == FLA_BF16, FLA_ERR_UNSUPPORTED, "%s: only bfloat16 q/k/v are implemented.", op);
-    if ((rc = check_tensor(v, op, "v", L.rank3() ? 3 : 4, dt_bit(FLA_BF16)))) return rc;
+    if ((rc = check_tensor(q, op, "q", L.rank3() ? 3 : 4, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_tensor(v, op, "v", L.rank3() ? 3 : 4, dt_bit(kElemDtype)))) return rc;
     const int last = q->ndim - 1;
     ChunkGeom geom{};
     geom.B = L.rank3() ? 1 : (int)q->shape[L.ib];
@@ -651,7 +650,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
                 FLA_ERR_UNSUPPORTED, "%s: implemented head sizes are K in {64,128} with V in {K, 2K}, got K=%d V=%d.", op,
                 geom.K, geom.V);
     const int64_t B = geom.B, T = geom.T, Hk = geom.Hk, Hv = geom.Hv, K = geom.K, V = geom.V;
-    const int bf = dt_bit(FLA_BF16), f32 = dt_bit(FLA_F32);
+    const int bf = dt_bit(kElemDtype), f32 = dt_bit(FLA_F32);
     KdaIntraParams ip{};
     if ((rc = layout_view(op, "q", q, L, B, Hk, T, K, bf, ip.q.sb, ip.q.sh, ip.q.st))) return rc;
     if ((rc = layout_view(op, "k", k, L, B, Hk, T, K, bf, ip.k.sb, ip.k.sh, ip.k.st))) return rc;
@@ -665,7 +664,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
                         g->shape[g->ndim - 1] == K && inner_unit(g),
                     FLA_ERR_SHAPE, "%s: v/g/beta shapes do not match the selected layout.", op);
         ip.g = g->data;
-        ip.g_bf16 = g->dtype == FLA_BF16;
+        ip.g_elem = g->dtype != FLA_F32;
         ip.g_sb = L.rank3() ? 0 : g->stride[L.ib];
         ip.g_sh = g->stride[L.ih];
         ip.g_st = g->stride[L.it];
@@ -675,7 +674,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
         FLA_REQUIRE((L.rank3() || beta->shape[L.ib] == B) && beta->shape[L.ih] == Hv && beta->shape[L.it] == T, FLA_ERR_SHAPE,
                     "%s: v/g/beta shapes do not match the selected layout.", op);
         ip.beta = View3{beta->data, L.rank3() ? 0 : beta->stride[L.ib], beta->stride[L.ih], beta->stride[L.it],
-                        beta->dtype == FLA_BF16 ? 1 : 0};
+                        beta->dtype == FLA_F32 ? 0 : 1};
     }
     if (use_gate) {
         FLA_REQUIRE(present(a_log) && a_log->ndim == 1 && a_log->shape[0] == Hv && a_log->dtype == FLA_F32 &&
@@ -699,14 +698,14 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     KdaScanParams sp{};
     if ((rc = layout_view(op, "attn_out", attn_out, L, B, Hv, T, V, bf, sp.o.sb, sp.o.sh, sp.o.st))) return rc;
     sp.o.p = attn_out->data;
-    if ((rc = head_major(op, "Aqk", aqk, L.rank3(), B, Hv, T, kChunk, FLA_BF16))) return rc;
-    if ((rc = head_major(op, "Akk", akk, L.rank3(), B, Hv, T, kChunk, FLA_BF16))) return rc;
+    if ((rc = head_major(op, "Aqk", aqk, L.rank3(), B, Hv, T, kChunk, kElemDtype))) return rc;
+    if ((rc = head_major(op, "Akk", akk, L.rank3(), B, Hv, T, kChunk, kElemDtype))) return rc;
     if (present(gk) && (rc = head_major(op, "gk", gk, L.rank3(), B, Hv, T, K, FLA_F32))) return rc;
-    if (present(w) && (rc = head_major(op, "w", w, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
-    if (present(u) && (rc = head_major(op, "u", u, L.rank3(), B, Hv, T, V, FLA_BF16))) return rc;
-    if (present(qg) && (rc = head_major(op, "qg", qg, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
-    if (present(kg) && (rc = head_major(op, "kg", kg, L.rank3(), B, Hv, T, K, FLA_BF16))) return rc;
-    if (present(v_new) && (rc = head_major(op, "v_new", v_new, L.rank3(), B, Hv, T, V, FLA_BF16))) return rc;
+    if (present(w) && (rc = head_major(op, "w", w, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
+    if (present(u) && (rc = head_major(op, "u", u, L.rank3(), B, Hv, T, V, kElemDtype))) return rc;
+    if (present(qg) && (rc = head_major(op, "qg", qg, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
+    if (present(kg) && (rc = head_major(op, "kg", kg, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
+    if (present(v_new) && (rc = head_major(op, "v_new", v_new, L.rank3(), B, Hv, T, V, kElemDtype))) return rc;
     const int64_t d2 = state_v_first ? V : K, d3 = state_v_first ? K : V;
     auto check_state = [&](const fla_tensor *s, const char *name) -> int {
         int r = check_tensor(s, op, name, 4, f32);
@@ -724,7 +723,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
         FLA_REQUIRE((L.rank3() || h->shape[0] == B) && h->shape[o] == NT && h->shape[o + 1] == Hv && h->shape[o + 2] == d2 &&
                         h->shape[o + 3] == d3 && h->stride[o + 3] == 1 && h->stride[o + 2] == d3,
                     FLA_ERR_SHAPE, "%s: h must be [..,NT=%lld,HV,%lld,%lld].", op, (long long)NT, (long long)d2, (long long)d3);
-        sp.h = static_cast<bf16 *>(h->data);
+        sp.h = static_cast<elem *>(h->data);
         sp.h_sb = L.rank3() ? 0 : h->stride[0];
         sp.h_sc = h->stride[o];
         sp.h_sh = h->stride[o + 1];
@@ -761,12 +760,12 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     ip.lower_bound = (float)lower_bound;
     ip.scale = (float)scale;
     ip.gk = present(gk) ? static_cast<float *>(gk->data) : nullptr;
-    ip.aqk = static_cast<bf16 *>(aqk->data);
-    ip.akk = static_cast<bf16 *>(akk->data);
-    ip.w = present(w) ? static_cast<bf16 *>(w->data) : reinterpret_cast<bf16 *>(wsb + w_off);
-    ip.u = present(u) ? static_cast<bf16 *>(u->data) : reinterpret_cast<bf16 *>(wsb + u_off);
-    ip.qg = present(qg) ? static_cast<bf16 *>(qg->data) : reinterpret_cast<bf16 *>(wsb + qg_off);
-    ip.kg = present(kg) ? static_cast<bf16 *>(kg->data) : reinterpret_cast<bf16 *>(wsb + kg_off);
+    ip.aqk = static_cast<elem *>(aqk->data);
+    ip.akk = static_cast<elem *>(akk->data);
+    ip.w = present(w) ? static_cast<elem *>(w->data) : reinterpret_cast<elem *>(wsb + w_off);
+    ip.u = present(u) ? static_cast<elem *>(u->data) : reinterpret_cast<elem *>(wsb + u_off);
+    ip.qg = present(qg) ? static_cast<elem *>(qg->data) : reinterpret_cast<elem *>(wsb + qg_off);
+    ip.kg = present(kg) ? static_cast<elem *>(kg->data) : reinterpret_cast<elem *>(wsb + kg_off);
     ip.dec = reinterpret_cast<float *>(wsb + dec_off);
     if (K == 128 && V == 128) rc = launch_intra<128, 128>(ip, stream);
     else if (K == 128 && V == 256) rc = launch_intra<128, 256>(ip, stream);
@@ -781,7 +780,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     sp.kg = ip.kg;
     sp.aqk = ip.aqk;
     sp.dec = ip.dec;
-    sp.v_new = present(v_new) ? static_cast<bf16 *>(v_new->data) : nullptr;
+    sp.v_new = present(v_new) ? static_cast<elem *>(v_new->data) : nullptr;
     if (present(initial_state)) {
         sp.h0 = static_cast<const float *>(initial_state->data);
         sp.s_sn = initial_state->stride[0];
@@ -803,7 +802,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
 }  // namespace
 }  // namespace fla
 
-extern "C" int fla_chunk_kda_fwd_get_workspace_size(
+FLA_ENTRY(fla_chunk_kda_fwd_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
     const fla_tensor *A_log, const fla_tensor *dt_bias, const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size, bool safe_gate,
@@ -811,13 +810,14 @@ extern "C" int fla_chunk_kda_fwd_get_workspace_size(
     const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w,
     const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
     uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_fwd_get_workspace_size, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale, chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_fwd: workspace_size must not be null.");
     return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
                              chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
                              Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, workspace_size);
 }
 
-extern "C" int fla_chunk_kda_fwd(
+FLA_ENTRY(fla_chunk_kda_fwd)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
     const fla_tensor *A_log, const fla_tensor *dt_bias, const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size, bool safe_gate,
@@ -825,6 +825,7 @@ extern "C" int fla_chunk_kda_fwd(
     const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w,
     const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
     void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_fwd, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale, chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, workspace, workspace_size, stream);
     return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
                              chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
                              Aqk, Akk, w, u, qg, kg, v_new, h, workspace, workspace_size, static_cast<hipStream_t>(stream),

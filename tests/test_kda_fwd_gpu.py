@@ -16,11 +16,12 @@ pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
 
 
-def make_inputs(B, T, Hk, Hv, K, V, seed, *, raw_gate=False, gate_scale=0.3, g_dtype=torch.float32, beta_dtype=torch.float32):
+def make_inputs(B, T, Hk, Hv, K, V, seed, *, raw_gate=False, gate_scale=0.3, g_dtype=torch.float32, beta_dtype=torch.float32,
+                dtype=BF):
     gen = torch.Generator().manual_seed(seed)
-    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
-    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
-    v = torch.randn(B, Hv, T, V, generator=gen).to(BF)
+    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(dtype)
+    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(dtype)
+    v = torch.randn(B, Hv, T, V, generator=gen).to(dtype)
     if raw_gate:
         g = torch.randn(B, Hv, T, K, generator=gen).to(g_dtype)
     else:
@@ -63,6 +64,9 @@ CASES = [
          gate=dict(use_gate_in_kernel=True, safe_gate=True, lower_bound=-5.0, bias=True), g_dtype=BF, beta_dtype=BF),
     dict(B=1, T=1, Hk=1, Hv=1, K=128, V=128, layout="BSND"),
     dict(B=1, T=128, Hk=1, Hv=1, K=128, V=128, layout="BSND", gate_scale=3.0),             # strong decay
+    # float16 q/k/v and outputs (gates mild enough for the anchored factors to stay inside float16's range)
+    dict(B=2, T=200, Hk=2, Hv=4, K=128, V=128, layout="BSND", h0=True, dtype=torch.float16),
+    dict(B=1, T=130, Hk=1, Hv=2, K=64, V=64, layout="NTD", cu=[0, 65, 130], dtype=torch.float16),
 ]
 
 
@@ -76,7 +80,8 @@ def test_chunk_kda_fwd(dev, case):
     v_first = case.get("v_first", False)
     q, k, v, g, beta = make_inputs(B, T, Hk, Hv, K, V, seed=T + K + V, raw_gate=use_gate,
                                    gate_scale=case.get("gate_scale", 0.3), g_dtype=case.get("g_dtype", torch.float32),
-                                   beta_dtype=case.get("beta_dtype", torch.float32))
+                                   beta_dtype=case.get("beta_dtype", torch.float32), dtype=case.get("dtype", BF))
+    assert q.dtype == case.get("dtype", BF)
     gen = torch.Generator().manual_seed(11)
     A_log = torch.randn(Hv, generator=gen) * 0.3 - 1.5 if use_gate else None
     dt_bias = torch.randn(Hv * K, generator=gen) * 0.3 if gate.pop("bias", False) else None
@@ -104,6 +109,7 @@ def test_chunk_kda_fwd(dev, case):
     assert len(out) == 12
     o, final, gk, Aqk, Akk, w, u, qg, kg, v_new, h, init_back = out
     assert init_back is h0_dev
+    assert all(t.dtype == q.dtype for t in (o, Aqk, Akk, w, u, qg, kg, v_new, h))
     head = (lambda x: x[None]) if layout in ("TND", "NTD") else (lambda x: x)
 
     assert_close(from_layout(o, layout), o_naive, TOL_BF16, "o vs recurrence")
@@ -165,8 +171,8 @@ def test_chunk_kda_fwd_errors(dev):
         ops.chunk_kda_fwd(*a, 0.1, 64, cu_seqlens=[0, 64], chunk_indices=[0, 1])
     with pytest.raises(RuntimeError, match="initial_state shape"):
         ops.chunk_kda_fwd(*a, 0.1, 64, initial_state=torch.zeros(1, 2, 128, 64, device=dev))
-    with pytest.raises(RuntimeError, match="only bfloat16"):
-        ops.chunk_kda_fwd(*[t.half() if t.dtype == BF else t for t in a], 0.1, 64)
+    with pytest.raises(RuntimeError, match="same float16 or bfloat16 dtype"):
+        ops.chunk_kda_fwd(a[0].half(), *a[1:], 0.1, 64)
 
 
 def test_chunk_kda_fwd_state_handoff_and_determinism(dev):
