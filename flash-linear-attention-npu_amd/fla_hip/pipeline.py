@@ -174,6 +174,12 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
                 f"got initial_state.shape[0]={initial_state.shape[0]} and sequences={len(cu) - 1}.")
     if scale is None:
         scale = k.shape[-1] ** -0.5
+    # (o, final_state) do not depend on the chunk size: it only tiles the same recurrence.  The kernels tile
+    # by 64 tokens, so any other power of two is served by the fused route on 64-token chunks.
+    if chunk_size != 64:
+        if not fused:
+            raise NotImplementedError("the six-operator route is built for chunk_size=64 only; use fused=True.")
+        chunk_size = 64
     needs_grad = torch.is_grad_enabled() and any(
         isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta, initial_state))
     if not needs_grad:

@@ -78,6 +78,23 @@ def test_in_kernel_l2norm_equals_separate_pass(dev, case):
     assert_close(final, f_ref, 2 * TOL_STATE, "final_state")
 
 
+@pytest.mark.parametrize("chunk_size", [16, 128, 256])
+def test_other_chunk_sizes_give_the_same_result(dev, chunk_size):
+    """chunk_size only tiles the recurrence: the entry accepts any power of two and returns the result of the
+    reference's chunked algorithm at that size (oracle run at that chunk size) within the usual tolerance."""
+    from fla_hip import pipeline
+    d = gdn.make_gdn_inputs(1, 300, 2, 128, 128, dtype=BF, seed=5, init_std=0.01)
+    x = {k: v.to(dev) for k, v in d.items()}
+    o, final = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, x["initial_state"], True,
+                                               chunk_size=chunk_size)
+    o_ref, f_ref = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], None, d["initial_state"], True,
+                                              chunk_size=chunk_size, naive=False)
+    assert_close(o, o_ref, TOL_BF16, "o")
+    assert_close(final, f_ref, TOL_STATE, "final_state")
+    with pytest.raises(ValueError, match="power of 2"):
+        pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], chunk_size=96)
+
+
 def test_no_initial_state_and_default_scale(dev):
     from fla_hip import pipeline
     d = gdn.make_gdn_inputs(2, 128, 2, 128, 128, dtype=BF, seed=3)
