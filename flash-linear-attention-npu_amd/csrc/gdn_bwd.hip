@@ -107,11 +107,14 @@ struct DqkwgParams {
     float scale;
 };
 
-template <int K, int V, bool GVA>
+// V is the width of the value slab held in LDS; VSLABS slabs cover the value dimension (1: V itself, 2: V = 256 as
+// two passes of 128 columns, every product over the value dimension accumulated across the passes).
+template <int K, int V, bool GVA, int VSLABS = 1>
 __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
     constexpr int KT = K / 16;
+    constexpr int VF = V * VSLABS;     // full value dimension = row stride of h and dh
     elem *qS = reinterpret_cast<elem *>(smem);
     elem *kS = qS + kChunk * pk;
     elem *vS = kS + kChunk * pk;
@@ -141,65 +144,96 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
         if (r > 0) __syncthreads();      // the previous head's tiles are no longer read
-        TileCopy<kThreads, K, V> tdh;
         float hd = 0.f;                  // this thread's share of sum(h . dh)
-        {
-            TileCopy<kThreads, kChunk, V> tv, to, tdv;
-            TileCopy<kThreads, K, V> th;
-            tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
-            to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
-            tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
-            th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
-            tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
-            stage_scalars(gS, p.g, b, hv, start, len);
-            tv.commit(vS, pv, len, tid);
-            to.commit(oS, pv, len, tid);
-            tdv.commit(dvS, pv, len, tid);
-            th.commit(hS, pv, K, tid);
+        f32x4 dqs[KT], dsacc[4];
+        f32x4 dwacc[VSLABS > 1 ? KT : 1], dksacc[VSLABS > 1 ? KT : 1];   // only carried across slabs
 #pragma unroll
-            for (int m = 0; m < TileCopy<kThreads, K, V>::N; ++m) {
-                const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
+        for (int ct = 0; ct < KT; ++ct) dqs[ct] = zero4();
 #pragma unroll
-                for (int e = 0; e < 8; ++e) hd += (float)a[e] * (float)d[e];
-            }
+        for (int ct = 0; ct < 4; ++ct) dsacc[ct] = zero4();
+        if constexpr (VSLABS > 1) {
+#pragma unroll
+            for (int ct = 0; ct < KT; ++ct) dwacc[ct] = dksacc[ct] = zero4();
         }
-        __syncthreads();
-        // ---- products with the state at chunk start: dq (state part), dw; and the ds tile -------------
-        f32x4 dqs[KT];
         char *dwg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
                                              (int64_t)start * p.dw.st);
 #pragma unroll
-        for (int ct = 0; ct < KT; ++ct) {
-            f32x4 a = zero4(), d = zero4();
+        for (int vs = 0; vs < VSLABS; ++vs) {
+            if (vs > 0) __syncthreads();     // the previous slab's tiles are no longer read
+            TileCopy<kThreads, K, V> tdh;
+            {
+                TileCopy<kThreads, kChunk, V> tv, to, tdv;
+                TileCopy<kThreads, K, V> th;
+                tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st + vs * V, p.v.st, len, tid);
+                to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st + vs * V, p.d_o.st, len, tid);
+                tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st + vs * V, p.dv.st, len, tid);
+                th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc + vs * V, VF, K, tid);
+                tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc + vs * V, VF, K, tid);
+                if (vs == 0) stage_scalars(gS, p.g, b, hv, start, len);
+                tv.commit(vS, pv, len, tid);
+                to.commit(oS, pv, len, tid);
+                tdv.commit(dvS, pv, len, tid);
+                th.commit(hS, pv, K, tid);
 #pragma unroll
-            for (int j = 0; j < V / 32; ++j) {
-                const elemx8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
-                a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
-                d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
-            }
-            dqs[ct] = a;
-            acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -d);
-        }
+                for (int m = 0; m < TileCopy<kThreads, K, V>::N; ++m) {
+                    const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-            f32x4 acc = zero4();
-            if (ct <= w) {
-#pragma unroll
-                for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
-                const int col = 16 * ct + li;
-                const float gc = gS[col];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int row = 16 * w + 4 * lg + e;
-                    const float f = __expf(fminf(gS[row] - gc, 0.f)) * p.scale;
-                    acc[e] = (col <= row && row < len) ? acc[e] * f : 0.f;
+                    for (int e = 0; e < 8; ++e) hd += (float)a[e] * (float)d[e];
                 }
             }
-            acc_to_tile(sS, ps, 16 * w, 16 * ct, acc);
+            __syncthreads();
+            // ---- products with the state at chunk start: dq (state part), dw; and the ds tile ---------
+#pragma unroll
+            for (int ct = 0; ct < KT; ++ct) {
+                f32x4 a = dqs[ct], d = VSLABS > 1 ? dwacc[ct] : zero4();
+#pragma unroll
+                for (int j = 0; j < V / 32; ++j) {
+                    const elemx8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
+                    a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
+                    d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
+                }
+                dqs[ct] = a;
+                if constexpr (VSLABS > 1) dwacc[ct] = d;
+                else acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -d);
+            }
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                if (ct <= w) {
+#pragma unroll
+                    for (int j = 0; j < V / 32; ++j)
+                        dsacc[ct] = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), dsacc[ct]);
+                }
+                if (vs == VSLABS - 1) {      // complete: gate factors, causal mask, to LDS
+                    f32x4 acc = zero4();
+                    if (ct <= w) {
+                        acc = dsacc[ct];
+                        const int col = 16 * ct + li;
+                        const float gc = gS[col];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int row = 16 * w + 4 * lg + e;
+                            const float f = __expf(fminf(gS[row] - gc, 0.f)) * p.scale;
+                            acc[e] = (col <= row && row < len) ? acc[e] * f : 0.f;
+                        }
+                    }
+                    acc_to_tile(sS, ps, 16 * w, 16 * ct, acc);
+                }
+            }
+            __syncthreads();                 // every wave is done with h; ds is complete after the last slab
+            tdh.commit(hS, pv, K, tid);
+            __syncthreads();
+            if constexpr (VSLABS > 1) {      // dk (state part) of this slab; the single-slab form folds it into the loop below
+#pragma unroll
+                for (int ct = 0; ct < KT; ++ct)
+#pragma unroll
+                    for (int j = 0; j < V / 32; ++j)
+                        dksacc[ct] = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dksacc[ct]);
+            }
         }
-        __syncthreads();                 // every wave is done with h; ds is complete
-        tdh.commit(hS, pv, K, tid);
-        __syncthreads();
+        if constexpr (VSLABS > 1) {
+#pragma unroll
+            for (int ct = 0; ct < KT; ++ct) acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -dwacc[ct]);
+        }
         // ---- products with the state gradient, gate factors, intra-chunk parts -------------------------
         const float g_last = gS[len - 1];
         float grow[4], eq[4], ek[4];
@@ -213,8 +247,12 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
 #pragma unroll
         for (int ct = 0; ct < KT; ++ct) {
             f32x4 dks = zero4();
+            if constexpr (VSLABS > 1) {
+                dks = dksacc[ct];
+            } else {
 #pragma unroll
-            for (int j = 0; j < V / 32; ++j) dks = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dks);
+                for (int j = 0; j < V / 32; ++j) dks = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dks);
+            }
             f32x4 dq = dqs[ct], dk;
             float kv[4], qv[4];
 #pragma unroll
@@ -636,15 +674,17 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                   static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
-    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (V + 8) + kChunk + 8) + (size_t)K * (V + 8)) * 2 + (kChunk + 8) * 4;
+    const int VS = V == 256 ? 128 : V;   // value columns held in LDS at a time
+    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 + (kChunk + 8) * 4;
     const bool gva = geom.Hv != geom.Hk;
+    if (K == 128 && V == 256) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, true, 2>), "bwd_dqkwg", grid, smem, p);
     if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, false>), "bwd_dqkwg", grid, smem, p);
     if (K == 128 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, true>), "bwd_dqkwg", grid, smem, p);
     if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, false>), "bwd_dqkwg", grid, smem, p);
     if (K == 64 && V == 64) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, true>), "bwd_dqkwg", grid, smem, p);
     if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, false>), "bwd_dqkwg", grid, smem, p);
     if (K == 64 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, true>), "bwd_dqkwg", grid, smem, p);
-    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 
 int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
@@ -719,7 +759,8 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64, true>), "wy_bwd_full", grid, smem, p);
     if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, false>), "wy_bwd_full", grid, smem, p);
     if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, true>), "wy_bwd_full", grid, smem, p);
-    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128).", op, K, V);
+    if (K == 128 && V == 256) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 256, true>), "wy_bwd_full", grid, smem, p);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 
 // da + full in one call: dA (bf16, transposed like the stand-alone operator writes it) lives in the caller's workspace

@@ -22,6 +22,8 @@ CASES = [
     (1, 65, 2, 2, 64, 64, None),
     (1, 130, 2, 1, 64, 128, None),
     (1, 261, 2, 1, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261]),   # lengths 1,15,17,0,63,64,101
+    (1, 150, 2, 1, 128, 256, None),                     # V = 256: two value slabs in chunk_bwd_dqkwg
+    (1, 200, 2, 2, 128, 256, [0, 70, 200]),
 ]
 
 
@@ -121,7 +123,7 @@ def test_backward_operators_against_oracle(dev, case, dtype):
 
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("case", [CASES[1], CASES[5]])
+@pytest.mark.parametrize("case", [CASES[1], CASES[5], CASES[6]])
 def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
     """The composed GPU backward against autograd (fp64) through the per-token recurrence on the same bf16
     inputs: every gradient within 2e-2 of its own scale."""
