@@ -24,8 +24,9 @@ struct ScanParams {
     ChunkGeom geom;
     View4 k, w, u, v_new;
     View3 g;
-    const float *h0;     // [N,Hv,K,V] or [N,Hv,V,K] fp32, or null
-    float *hT;           // final state, same layout, or null
+    const void *h0;      // [N,Hv,K,V] or [N,Hv,V,K], fp32 or the element type, or null
+    void *hT;            // final state, same layout and type, or null
+    int state_elem;      // 1: h0 / hT hold the element type (the carry itself stays fp32)
     elem *h;             // [B,Hv,NT,K,V] (or V,K) bf16, or null
     int64_t h_sb, h_sh, h_sc;
     int64_t s_sn, s_sh;  // strides of h0 / hT over (sequence, head)
@@ -109,9 +110,12 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         for (int ct = 0; ct < CT; ++ct) {
             f32x4 a = {0.f, 0.f, 0.f, 0.f};
             if (p.h0) {
-                const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+                const int64_t base = n * p.s_sn + hv * p.s_sh;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) a[e] = s[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)];
+                for (int e = 0; e < 4; ++e) {
+                    const int64_t off = base + state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li);
+                    a[e] = p.state_elem ? (float)static_cast<const elem *>(p.h0)[off] : static_cast<const float *>(p.h0)[off];
+                }
             }
             hacc[kt][ct] = a;
         }
@@ -217,13 +221,17 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     }
 
     if (p.hT) {
-        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+        const int64_t base = n * p.s_sn + hv * p.s_sh;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) s[state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li)] = hacc[kt][ct][e];
+                for (int e = 0; e < 4; ++e) {
+                    const int64_t off = base + state_off(16 * kt + 4 * lg + e, vcol0 + 16 * ct + li);
+                    if (p.state_elem) static_cast<elem *>(p.hT)[off] = (elem)hacc[kt][ct][e];
+                    else static_cast<float *>(p.hT)[off] = hacc[kt][ct][e];
+                }
     }
 }
 
@@ -262,7 +270,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     }
     const int64_t d2 = state_v_first ? geom.V : geom.K, d3 = state_v_first ? geom.K : geom.V;
     auto check_state = [&](const fla_tensor *s, const char *name) -> int {
-        int r = check_tensor(s, op, name, 4, dt_bit(FLA_F32));
+        int r = check_tensor(s, op, name, 4, dt_bit(FLA_F32) | bf);
         if (r) return r;
         FLA_REQUIRE(s->shape[0] == geom.N && s->shape[1] == geom.Hv && s->shape[2] == d2 && s->shape[3] == d3 &&
                         s->stride[3] == 1 && s->stride[2] == d3,
@@ -274,8 +282,9 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     if (has_h0 && (rc = check_state(initial_state, "initial_state"))) return rc;
     if (output_final_state && (rc = check_state(final_state, "final_state"))) return rc;
     if (has_h0 && output_final_state)
-        FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1],
-                    FLA_ERR_SHAPE, "%s: initial_state and final_state must share strides.", op);
+        FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1] &&
+                        initial_state->dtype == final_state->dtype,
+                    FLA_ERR_SHAPE, "%s: initial_state and final_state must share strides and dtype.", op);
     const bool has_h = h && h->data;
     if (has_h) {
         if ((rc = check_tensor(h, op, "h", 5, bf))) return rc;
@@ -305,9 +314,10 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     p.u = view4(u);
     p.v_new = view4(v_new);
     p.g = view3(g);
-    p.h0 = has_h0 ? static_cast<const float *>(initial_state->data) : nullptr;
-    p.hT = output_final_state ? static_cast<float *>(final_state->data) : nullptr;
+    p.h0 = has_h0 ? initial_state->data : nullptr;
+    p.hT = output_final_state ? final_state->data : nullptr;
     const fla_tensor *sref = has_h0 ? initial_state : (output_final_state ? final_state : nullptr);
+    p.state_elem = sref != nullptr && sref->dtype != FLA_F32;
     if (sref) {
         p.s_sn = sref->stride[0];
         p.s_sh = sref->stride[1];

@@ -41,8 +41,15 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
 
     cu = _cu_list(cu_seqlens)
     if fused:
-        gc, o, final = _raw.gdn_chunk_fwd(q, k, v, g.float(), beta.float(), scale, initial_state,
+        # the fused kernel carries and exchanges the state in fp32; a 16-bit state is widened here and the final
+        # state returned in the caller's dtype (chunk_gated_delta_rule_fwd_h/README.md:85-91 allows both)
+        h0 = initial_state
+        if h0 is not None and h0.dtype != torch.float32:
+            h0 = h0.float()
+        gc, o, final = _raw.gdn_chunk_fwd(q, k, v, g.float(), beta.float(), scale, h0,
                                           output_final_state, cu, chunk_size, use_qk_l2norm_in_kernel)
+        if final is not None and initial_state is not None and final.dtype != initial_state.dtype:
+            final = final.to(initial_state.dtype)
         return gc, o, None, final
     if use_qk_l2norm_in_kernel:
         q, _ = _raw.l2norm_fwd(q)

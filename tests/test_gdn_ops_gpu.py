@@ -164,6 +164,37 @@ def test_state_v_first_and_no_final(dev):
     assert f_c is None and torch.equal(vn_a, vn_c)
 
 
+@pytest.mark.parametrize("dtype", [BF, F16], ids=["bf16", "f16"])
+def test_fwd_h_sixteen_bit_state(dev, dtype):
+    """initial_state / final_state in the dtype of the matrices (chunk_gated_delta_rule_fwd_h/README.md:85-91):
+    same recurrence, the carry stays fp32 inside the kernel, the final state is rounded once on the way out."""
+    from fla_hip import ops, pipeline
+    B, T, H, K, V = 1, 200, 2, 128, 128
+    d = inputs(B, T, H, K, V, seed=9, dtype=dtype)
+    x = dev_kw(d, dev)
+    gen = torch.Generator().manual_seed(4)
+    h0 = (torch.randn(B, H, K, V, generator=gen) * 0.1).to(dtype)
+    G_ref = gdn.chunk_local_cumsum(d["g"], 64)
+    A = gdn.solve_tri(gdn.chunk_scaled_dot_kkt(d["k"], G_ref, d["beta"], 64), output_dtype=dtype)
+    w, u = gdn.recompute_w_u_fwd(d["k"], d["v"], d["beta"], A, 64, g=G_ref, output_dtype=dtype)
+    h, v_new, final = ops.chunk_gated_delta_rule_fwd_h(x["k"], w.to(dev), u.to(dev), g=G_ref.to(dev), initial_state=h0.to(dev),
+                                                       output_final_state=True, chunk_size=64)
+    h_ref, vn_ref, f_ref = gdn.chunk_gated_delta_rule_fwd_h(d["k"], w, u, G_ref, initial_state=h0.float(),
+                                                            output_final_state=True, chunk=64, output_dtype=torch.float32)
+    assert final.dtype == dtype and h.dtype == dtype
+    assert_close(final, f_ref, TOL_OF[dtype], "final_state")
+    assert_close(v_new, vn_ref, TOL_OF[dtype], "v_new")
+    assert_close(h, h_ref, TOL_OF[dtype], "h")
+    # pipeline entry: fp32 carry inside, caller's dtype outside
+    o, fin = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"].transpose(1, 2).contiguous(),
+                                             x["beta"].transpose(1, 2).contiguous(), None, h0.to(dev), True)
+    o_ref, fin_ref = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"].transpose(1, 2), d["beta"].transpose(1, 2),
+                                                None, h0.float(), True)
+    assert fin.dtype == dtype
+    assert_close(o, o_ref, TOL_OF[dtype], "o")
+    assert_close(fin, fin_ref, TOL_OF[dtype], "final_state (pipeline)")
+
+
 def test_rejects_bad_metadata(dev):
     from fla_hip import ops
     d = inputs(1, 128, 1, 128, 128)
