@@ -75,35 +75,50 @@ struct SolveParams {
     int64_t sb, sh, st;  // strides of (batch, head, token) in x and out
 };
 
-__global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
-    __shared__ __align__(16) float A[kChunk][kChunk];
+// BT x BT blocks, BT in {16, 32, 64, 128}; one thread per column of the inverse (at least one full wave).
+template <int BT>
+__global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const SolveParams p) {
+    constexpr int NTH = BT < 64 ? 64 : BT;       // threads
+    constexpr int CPR = BT / 8;                  // 16-byte pieces per row
+    constexpr int PO = BT + 8;                   // pitch of the 16-bit output staging
+    constexpr int NP = (BT * CPR + NTH - 1) / NTH;
+    __shared__ __align__(16) float A[BT][BT];
     const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    int seq, start, len;
-    chunk_span(p.geom, b, c, seq, start, len);
+    int start, len;
+    if (p.geom.cu == nullptr) {
+        start = c * BT;
+        len = min(BT, p.geom.T - start);
+    } else {
+        const int seq = p.geom.tab[2 * c];
+        start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * BT;
+        len = min(BT, p.geom.cu[seq + 1] - start);
+    }
     const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
     const int lane = threadIdx.x;
-    {   // branch-free loads (clamped row), all eight in flight before the first LDS write
-        elemx8 v[8];
+    {   // branch-free loads (clamped row), all in flight before the first LDS write
+        elemx8 v[NP];
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            const int idx = m * 64 + lane;
-            v[m] = *reinterpret_cast<const elemx8 *>(p.x + base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3));
+        for (int m = 0; m < NP; ++m) {
+            const int idx = min(m * NTH + lane, BT * CPR - 1);
+            v[m] = *reinterpret_cast<const elemx8 *>(p.x + base + (int64_t)min(idx / CPR, len - 1) * p.st + ((idx % CPR) << 3));
         }
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
-            const int idx = m * 64 + lane;
-            const int r = idx >> 3, c8 = (idx & 7) << 3;
+        for (int m = 0; m < NP; ++m) {
+            const int idx = m * NTH + lane;
+            if (idx < BT * CPR) {
+                const int r = idx / CPR, c8 = (idx % CPR) << 3;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) A[r][c8 + e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
+                for (int e = 0; e < 8; ++e) A[r][c8 + e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
+            }
         }
     }
     __syncthreads();
 
-    float x[kChunk];
+    float x[BT];
 #pragma unroll
-    for (int i = 0; i < kChunk; ++i) x[i] = 0.f;
+    for (int i = 0; i < BT; ++i) x[i] = 0.f;
 #pragma unroll
-    for (int i = 0; i < kChunk; ++i) {
+    for (int i = 0; i < BT; ++i) {
         float acc = (i == lane) ? 1.f : 0.f;
 #pragma unroll
         for (int s4 = 0; s4 < (i + 3) / 4; ++s4) {
@@ -113,13 +128,15 @@ __global__ void __launch_bounds__(64) solve_tri_kernel(const SolveParams p) {
         x[i] = acc;
     }
     __syncthreads();
-    elem *O = reinterpret_cast<elem *>(&A[0][0]);  // [64][72] bf16 staging, fits in the fp32 tile
+    elem *O = reinterpret_cast<elem *>(&A[0][0]);  // [BT][BT + 8] 16-bit staging, fits in the fp32 tile
+    if (lane < BT) {
 #pragma unroll
-    for (int i = 0; i < kChunk; ++i) O[i * 72 + lane] = (elem)x[i];
+        for (int i = 0; i < BT; ++i) O[i * PO + lane] = (elem)x[i];
+    }
     __syncthreads();
-    for (int idx = lane; idx < len * 8; idx += 64) {
-        const int r = idx >> 3, c8 = (idx & 7) << 3;
-        *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(O + r * 72 + c8);
+    for (int idx = lane; idx < len * CPR; idx += NTH) {
+        const int r = idx / CPR, c8 = (idx % CPR) << 3;
+        *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(O + r * PO + c8);
     }
 }
 
@@ -484,22 +501,29 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
     else if (!strcmp(lay, "ntd")) { ib = -1; ih = 0; it = 1; }
     else return fail(FLA_ERR_UNSUPPORTED, "%s: unknown layout '%s' (bsnd, bnsd, tnd, ntd).", op, layout);
     FLA_REQUIRE(x->ndim == (ib < 0 ? 3 : 4), FLA_ERR_SHAPE, "%s: rank does not match layout '%s'.", op, layout);
-    FLA_REQUIRE(x->shape[x->ndim - 1] == kChunk, FLA_ERR_UNSUPPORTED, "%s: block size must be %d, got %lld.", op, kChunk,
-                (long long)x->shape[x->ndim - 1]);
+    const int BT = (int)x->shape[x->ndim - 1];
+    FLA_REQUIRE(BT == 16 || BT == 32 || BT == 64 || BT == 128, FLA_ERR_UNSUPPORTED,
+                "%s: block size (last dimension) must be 16, 32, 64 or 128, got %lld.", op, (long long)x->shape[x->ndim - 1]);
     ChunkGeom geom{};
     geom.B = ib < 0 ? 1 : (int)x->shape[ib];
     geom.Hv = geom.Hk = (int)x->shape[ih];
     geom.T = (int)x->shape[it];
     FLA_REQUIRE(x->shape[it] < ((int64_t)1 << 31) && x->shape[ih] < 65536 && geom.B < 65536, FLA_ERR_SHAPE,
                 "%s: extents too large.", op);
-    geom.NT = (geom.T + kChunk - 1) / kChunk;
+    geom.NT = (geom.T + BT - 1) / BT;
     geom.N = geom.B;
     Varlen vl;
-    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query, BT)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0 || geom.Hv == 0) return FLA_OK;
     SolveParams p{geom, static_cast<const elem *>(x->data), static_cast<elem *>(out->data), ib < 0 ? 0 : x->stride[ib],
                   x->stride[ih], x->stride[it]};
-    FLA_LAUNCH("solve_tri", stream, solve_tri_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(64), 0, stream, p);
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    switch (BT) {
+        case 16: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<16>, grid, dim3(64), 0, stream, p); break;
+        case 32: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<32>, grid, dim3(64), 0, stream, p); break;
+        case 64: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<64>, grid, dim3(64), 0, stream, p); break;
+        default: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<128>, grid, dim3(128), 0, stream, p); break;
+    }
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }

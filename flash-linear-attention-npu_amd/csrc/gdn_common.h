@@ -86,6 +86,6 @@ int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, 
 // Validates cu_seqlens / chunk_indices, reports the workspace (query != null) or uploads the chunk table
 // into `workspace` and completes `geom` with the device pointers.
 int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
-                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query);
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query, int chunk = kChunk);
 
 }  // namespace fla

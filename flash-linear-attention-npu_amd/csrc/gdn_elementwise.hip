@@ -62,8 +62,8 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
 }
 
 int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
-                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query) {
-    int rc = build_varlen(vl, op, cu, ci, kChunk, geom.T);
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query, int chunk) {
+    int rc = build_varlen(vl, op, cu, ci, chunk, geom.T);
     if (rc) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
     if (vl.enabled) {

@@ -143,6 +143,35 @@ def test_solve_tri_layouts_and_inverse(dev):
     assert_close(out.transpose(0, 1), ref[0], TOL_BF16, "tnd")
 
 
+@pytest.mark.parametrize("BT", [16, 32, 128])
+@pytest.mark.parametrize("dtype", [BF, F16], ids=["bf16", "f16"])
+def test_solve_tri_other_block_sizes(dev, BT, dtype):
+    """The block size is the last dimension (16 / 32 / 64 / 128, solve_tri.cpp:47-62): numpy inverse per block,
+    ragged tail blocks, a packed batch with an empty sequence, and the reference's residual bound."""
+    import numpy as np
+    from fla_hip import ops
+    gen = torch.Generator().manual_seed(BT)
+    H = 2
+    for T, cu in ((3 * BT + 5, None), (4 * BT + 3, [0, BT - 1, BT - 1, 2 * BT + 1, 4 * BT + 3])):
+        A = torch.tril(torch.randn(1, H, T, BT, generator=gen) * (2.0 / BT ** 0.5), -1)
+        spans = list(gdn.chunk_spans(1, T, BT, cu))
+        Ab = torch.zeros_like(A)
+        for b, n, ci, s, e in spans:            # strictly lower inside each block
+            Ab[b, :, s:e, : e - s] = torch.tril(A[b, :, s:e, : e - s], -1)
+        Ab = Ab.to(dtype)
+        out = ops.solve_tri(Ab.to(dev), cu_seqlens=cu, layout="bnsd").float().cpu()
+        for b, n, ci, s, e in spans:
+            L = e - s
+            M = np.eye(L) + Ab[b, :, s:e, :L].float().numpy()
+            ref = torch.from_numpy(np.linalg.inv(M)).float()
+            assert_close(out[b, :, s:e, :L], ref, TOL_OF[dtype], f"block {s}:{e}")
+            res = torch.from_numpy(M).float() @ out[b, :, s:e, :L] - torch.eye(L)
+            assert float(res.abs().max()) < (2e-2 if dtype == BF else 2e-3) * max(1.0, float(ref.abs().max()))
+            assert float(out[b, :, s:e, L:].abs().max() if L < BT else 0.0) == 0.0
+    with pytest.raises(RuntimeError):
+        ops.solve_tri(torch.zeros(1, 2, 48, 24, dtype=dtype, device=dev), layout="bnsd")
+
+
 def test_state_v_first_and_no_final(dev):
     from fla_hip import ops
     d = inputs(1, 130, 2, 128, 128, seed=4)
