@@ -26,6 +26,7 @@ namespace fla {
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kIntraThreads = 512;   // kda_intra_kernel: two waves per SIMD share one set of LDS tiles
 
 __device__ __forceinline__ f32x4 lds4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
 __device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
@@ -87,13 +88,16 @@ __device__ __forceinline__ elemx8 scaled_frag(const elem *tile, int pitch, const
 
 template <int K, int V> struct IntraSmem {
     static constexpr int pq = K + 16, pk = K + 8, pg = K + 4, pv = V + 16, pa = 68, pb = 72;
-    static constexpr int SEG = 256 / K;  // token segments of the gate scan
+    static constexpr int SEG = kIntraThreads / K;  // token segments of the gate scan
     static constexpr size_t bytes =
         (size_t)kChunk * (pq + pk + pv + 2 * pb) * 2 + (size_t)kChunk * (pg + pa + 1) * 4 + (size_t)SEG * K * 4;
 };
 
-// Everything a wave does after the gate scan.  W = wave index (static so tile loops unroll).
-template <int K, int V, int W>
+// Everything a wave does after the gate scan.  Eight waves: wave W of role 0 owns row tile W of k k^T (with the
+// diagonal block inverse and the off-diagonal solve of column block W) and later row tile W of w; wave W of role 1
+// owns row tile 3 - W of q k^T and later row tile W of u.  The two waves of a SIMD (W and 4 + W) together carry five
+// score tile products, as every other SIMD does.  W and ROLE are static so that the tile loops unroll.
+template <int K, int V, int W, int ROLE>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
                                            int64_t dec_base) {
@@ -102,78 +106,88 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     constexpr int KS = K / 32, R1 = W, R2 = 3 - W;
     const int l = lane_id(), li = l & 15, lg = l >> 4;
 
-    // ---- scores: k k^T row tile R1 (and its transposed diagonal tile), q k^T row tile R2 ------------
+    // ---- scores: k k^T row tile R1 (and its transposed diagonal tile) | q k^T row tile R2 ------------------
     f32x4 kacc[R1 + 1], kaccT = zero4(), qacc[R2 + 1];
 #pragma unroll
     for (int c = 0; c <= R1; ++c) kacc[c] = zero4();
 #pragma unroll
     for (int c = 0; c <= R2; ++c) qacc[c] = zero4();
+    f32x4 brow = zero4();
+    float bcol = 0.f;
+    if constexpr (ROLE == 0) {
 #pragma unroll
-    for (int j = 0; j < KS; ++j) {
-        const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
+        for (int j = 0; j < KS; ++j) {
+            const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
 #pragma unroll
-        for (int c = 0; c <= R1; ++c) {
-            const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
-            kacc[c] = mfma16x32(lk, rk, kacc[c]);
-            if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+            for (int c = 0; c <= R1; ++c) {
+                const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+                kacc[c] = mfma16x32(lk, rk, kacc[c]);
+                if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+            }
         }
-        const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+        // lane holds (row 16R + 4lg + e, column 16c + li) of each tile
+        brow = lds4(bS + 16 * R1 + 4 * lg);
+        bcol = bS[16 * R1 + li];
 #pragma unroll
-        for (int c = 0; c <= R2; ++c) {
-            const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
-            qacc[c] = mfma16x32(lq, rk, qacc[c]);
+        for (int c = 0; c < R1; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) aS[(16 * R1 + 4 * lg + e) * pa + 16 * c + li] = brow[e] * kacc[c][e];
+    } else {
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+#pragma unroll
+            for (int c = 0; c <= R2; ++c) {
+                const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+                qacc[c] = mfma16x32(lq, rk, qacc[c]);
+            }
         }
-    }
-    // lane holds (row 16R + 4lg + e, column 16c + li) of each tile
-    const f32x4 brow = lds4(bS + 16 * R1 + 4 * lg);
-    const float bcol = bS[16 * R1 + li];
 #pragma unroll
-    for (int c = 0; c < R1; ++c)
+        for (int c = 0; c < 4; ++c) {
+            f32x4 a = zero4();
+            if (c <= R2) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) aS[(16 * R1 + 4 * lg + e) * pa + 16 * c + li] = brow[e] * kacc[c][e];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        f32x4 a = zero4();
-        if (c <= R2) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) a[e] = (c < R2 || li <= 4 * lg + e) ? p.scale * qacc[c <= R2 ? c : 0][e] : 0.f;
+                for (int e = 0; e < 4; ++e) a[e] = (c < R2 || li <= 4 * lg + e) ? p.scale * qacc[c <= R2 ? c : 0][e] : 0.f;
+            }
+            acc_to_tile(aqS, pb, 16 * R2, 16 * c, a);
         }
-        acc_to_tile(aqS, pb, 16 * R2, 16 * c, a);
     }
 
-    // ---- inverse of the diagonal block: (I + A)^-1 = (I - A)(I + A^2)(I + A^4)(I + A^8) ------------
-    // a2 = A[4lg+e][li] (right operand of A, left operand of A^T); a1 = A[li][4lg+e] (the converse).
-    f32x4 a1, a2, Y;
+    if constexpr (ROLE == 0) {
+        // ---- inverse of the diagonal block: (I + A)^-1 = (I - A)(I + A^2)(I + A^4)(I + A^8) ------------
+        // a2 = A[4lg+e][li] (right operand of A, left operand of A^T); a1 = A[li][4lg+e] (the converse).
+        f32x4 a1, a2, Y;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const int r = 4 * lg + e;
-        a2[e] = li < r ? brow[e] * kacc[R1][e] : 0.f;
-        a1[e] = r < li ? bcol * kaccT[e] : 0.f;
-        Y[e] = (r == li ? 1.f : 0.f) - a1[e];   // (I - A^T)[r][li]
-    }
-    {
-        const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
-        const f32x4 S1 = mfma16x16(A1, A2, zero4());   // A^2
-        const f32x4 T1 = mfma16x16(A2, A1, zero4());   // (A^2)^T
-        const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
-        Y = mfma16x16(S1b, cvt4(Y), Y);
-        const f32x4 S2 = mfma16x16(T1b, S1b, zero4());  // A^4
-        const f32x4 T2 = mfma16x16(S1b, T1b, zero4());  // (A^4)^T
-        const elemx4 S2b = cvt4(S2);
-        Y = mfma16x16(S2b, cvt4(Y), Y);
-        const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());  // A^8
-        Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
-    }
-    // lane holds Dinv[li][4lg+e]
-    *reinterpret_cast<f32x4 *>(aS + (16 * R1 + li) * pa + 16 * R1 + 4 * lg) = Y;
-    *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * R1 + 4 * lg) = cvt4(Y);
+        for (int e = 0; e < 4; ++e) {
+            const int r = 4 * lg + e;
+            a2[e] = li < r ? brow[e] * kacc[R1][e] : 0.f;
+            a1[e] = r < li ? bcol * kaccT[e] : 0.f;
+            Y[e] = (r == li ? 1.f : 0.f) - a1[e];   // (I - A^T)[r][li]
+        }
+        {
+            const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
+            const f32x4 S1 = mfma16x16(A1, A2, zero4());   // A^2
+            const f32x4 T1 = mfma16x16(A2, A1, zero4());   // (A^2)^T
+            const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
+            Y = mfma16x16(S1b, cvt4(Y), Y);
+            const f32x4 S2 = mfma16x16(T1b, S1b, zero4());  // A^4
+            const f32x4 T2 = mfma16x16(S1b, T1b, zero4());  // (A^4)^T
+            const elemx4 S2b = cvt4(S2);
+            Y = mfma16x16(S2b, cvt4(Y), Y);
+            const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero4());  // A^8
+            Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
+        }
+        // lane holds Dinv[li][4lg+e]
+        *reinterpret_cast<f32x4 *>(aS + (16 * R1 + li) * pa + 16 * R1 + 4 * lg) = Y;
+        *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * R1 + 4 * lg) = cvt4(Y);
 #pragma unroll
-    for (int c = R1 + 1; c < 4; ++c)
-        *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * c + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
+        for (int c = R1 + 1; c < 4; ++c)
+            *reinterpret_cast<elemx4 *>(akS + (16 * R1 + li) * pb + 16 * c + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
+    }
     __syncthreads();
 
     // ---- off-diagonal blocks of the inverse, column block W: X_rc = -Dinv_r sum_m A_rm X_mc --------
-    if constexpr (W < 3) {
+    if constexpr (ROLE == 0 && W < 3) {
         constexpr int C = W;
         f32x4 X[4];
 #pragma unroll
@@ -189,7 +203,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         }
     }
     // ---- gated operands: qg, kg to memory; k beta 2^g over the q tile ----------------------------------
-    for (int idx = threadIdx.x; idx < kChunk * (K / 8); idx += kThreads) {
+    for (int idx = threadIdx.x; idx < kChunk * (K / 8); idx += kIntraThreads) {
         const int r = idx / (K / 8), c8 = (idx % (K / 8)) * 8;
         const elemx8 q8 = *reinterpret_cast<const elemx8 *>(qS + r * pq + c8);
         const elemx8 k8 = *reinterpret_cast<const elemx8 *>(kS + r * pk + c8);
@@ -223,30 +237,29 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     if (threadIdx.x < K) p.dec[dec_base + threadIdx.x] = ex2(gS[63 * pg + threadIdx.x]);
     __syncthreads();
 
-    // ---- w = Akk (k beta 2^g), u = Akk (v beta): row tile W ------------------------------------------------
-    f32x4 wacc[K / 16], uacc[V / 16];
+    // ---- w = Akk (k beta 2^g) (role 0), u = Akk (v beta) (role 1): row tile W -----------------------------------
+    constexpr int NCT = ROLE == 0 ? K / 16 : V / 16;
+    f32x4 oacc[NCT];
 #pragma unroll
-    for (int ct = 0; ct < K / 16; ++ct) wacc[ct] = zero4();
-#pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) uacc[ct] = zero4();
+    for (int ct = 0; ct < NCT; ++ct) oacc[ct] = zero4();
 #pragma unroll
     for (int j = 0; j < (W < 2 ? 1 : 2); ++j) {   // Akk is lower triangular
         const elemx8 a = frag_kc(akS, pb, 16 * W, 32 * j);
 #pragma unroll
-        for (int ct = 0; ct < K / 16; ++ct) wacc[ct] = mfma16x32(a, frag_tr(qS, pq, 16 * ct, 32 * j), wacc[ct]);
-#pragma unroll
-        for (int ct = 0; ct < V / 16; ++ct) uacc[ct] = mfma16x32(a, frag_tr(vS, pv, 16 * ct, 32 * j), uacc[ct]);
+        for (int ct = 0; ct < NCT; ++ct)
+            oacc[ct] = mfma16x32(a, ROLE == 0 ? frag_tr(qS, pq, 16 * ct, 32 * j) : frag_tr(vS, pv, 16 * ct, 32 * j), oacc[ct]);
     }
     __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
 #pragma unroll
-    for (int ct = 0; ct < K / 16; ++ct) acc_to_tile(qS, pq, 16 * W, 16 * ct, wacc[ct]);
-#pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) acc_to_tile(vS, pv, 16 * W, 16 * ct, uacc[ct]);
+    for (int ct = 0; ct < NCT; ++ct) {
+        if constexpr (ROLE == 0) acc_to_tile(qS, pq, 16 * W, 16 * ct, oacc[ct]);
+        else acc_to_tile(vS, pv, 16 * W, 16 * ct, oacc[ct]);
+    }
     __syncthreads();
 }
 
 template <int K, int V>
-__global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParams p) {
+__global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntraParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb, SEG = S::SEG;
@@ -293,22 +306,22 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
         }
     }
     {   // all loads of the chunk are issued before the first LDS write waits for one of them
-        TileCopy<kThreads, kChunk, K> tq, tk;
-        TileCopy<kThreads, kChunk, V> tv;
+        TileCopy<kIntraThreads, kChunk, K> tq, tk;
+        TileCopy<kIntraThreads, kChunk, V> tv;
         tq.fetch(qg, p.q.st, len, tid);
         tk.fetch(kg, p.k.st, len, tid);
         tv.fetch(vg, p.v.st, len, tid);
-        float br[TileCopy<kThreads, kChunk, V>::N];
+        float br[TileCopy<kIntraThreads, kChunk, V>::N];
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) {
-            const int r = (m * kThreads + tid) / (V / 8);
+        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {
+            const int r = (m * kIntraThreads + tid) / (V / 8);
             br[m] = load_scalar(p.beta, b, hv, start + min(r, len - 1));
         }
         tq.commit(qS, pq, len, tid);
         tk.commit(kS, pk, len, tid);
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) {   // v * beta
-            const int idx = m * kThreads + tid;
+        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {   // v * beta
+            const int idx = m * kIntraThreads + tid;
             const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
             const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
             const float bb = r < len ? br[m] : 0.f;
@@ -349,16 +362,20 @@ __global__ void __launch_bounds__(kThreads) kda_intra_kernel(const KdaIntraParam
 
     const int64_t dec_base = (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 1: intra_wave<K, V, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 2: intra_wave<K, V, 2>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        default: intra_wave<K, V, 3>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 0: intra_wave<K, V, 0, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 1: intra_wave<K, V, 1, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 2: intra_wave<K, V, 2, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 3: intra_wave<K, V, 3, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 4: intra_wave<K, V, 0, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 5: intra_wave<K, V, 1, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 6: intra_wave<K, V, 2, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        default: intra_wave<K, V, 3, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
     }
 
-    store_tile<kThreads>(p.w + row_base * K, K, qS, pq, K, len);
-    store_tile<kThreads>(p.u + row_base * V, V, vS, pv, V, len);
-    store_tile<kThreads>(p.aqk + row_base * kChunk, kChunk, aqS, pb, kChunk, len);
-    store_tile<kThreads>(p.akk + row_base * kChunk, kChunk, akS, pb, kChunk, len);
+    store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
+    store_tile<kIntraThreads>(p.u + row_base * V, V, vS, pv, V, len);
+    store_tile<kIntraThreads>(p.aqk + row_base * kChunk, kChunk, aqS, pb, kChunk, len);
+    store_tile<kIntraThreads>(p.akk + row_base * kChunk, kChunk, akS, pb, kChunk, len);
 }
 
 // =============================================================================================
@@ -603,7 +620,7 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
     const size_t smem = IntraSmem<K, V>::bytes;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem,
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kIntraThreads), smem,
                stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
