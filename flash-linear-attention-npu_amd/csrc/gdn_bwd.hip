@@ -96,6 +96,7 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
 // =============================================================================
 // chunk_bwd_dqkwg
 // =============================================================================
+constexpr int kDqkwgThreads = 512;   // two waves per SIMD over one set of LDS tiles
 struct DqkwgParams {
     ChunkGeom geom;
     View4 q, k, v, d_o, dv, dq, dk, dw;
@@ -110,10 +111,10 @@ struct DqkwgParams {
 // V is the width of the value slab held in LDS; VSLABS slabs cover the value dimension (1: V itself, 2: V = 256 as
 // two passes of 128 columns, every product over the value dimension accumulated across the passes).
 template <int K, int V, bool GVA, int VSLABS = 1>
-__global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
+__global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
-    constexpr int KT = K / 16;
+    constexpr int KT = K / 16, KTH = KT / 2;   // column tiles of q/k: all, and per wave
     constexpr int VF = V * VSLABS;     // full value dimension = row stride of h and dh
     elem *qS = reinterpret_cast<elem *>(smem);
     elem *kS = qS + kChunk * pk;
@@ -123,47 +124,49 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
     elem *hS = dvS + kChunk * pv;      // h, then dh
     elem *sS = hS + K * pv;            // ds
     float *gS = reinterpret_cast<float *>(sS + kChunk * ps);
-    float *red = gS + kChunk;          // 8 partial sums
+    float *red = gS + kChunk;          // 16 partial sums
+    float *dgp = red + 16;             // [2][kChunk] row sums of the two column halves
 
     const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
     const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
-    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    // eight waves: wave (w, half) owns token rows 16w.. and column tiles half*KTH .. half*KTH+KTH-1 of q/k;
+    // waves w and 4 + w share a SIMD
+    const int tid = threadIdx.x, w = wave_id() & 3, half = wave_id() >> 2, l = lane_id(), li = l & 15, lg = l >> 4;
     {
-        TileCopy<kThreads, kChunk, K> tq, tk;
+        TileCopy<kDqkwgThreads, kChunk, K> tq, tk;
         tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
         tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
         tq.commit(qS, pk, len, tid);
         tk.commit(kS, pk, len, tid);
     }
-    f32x4 dq_acc[KT], dk_acc[KT];
+    f32x4 dq_acc[KTH], dk_acc[KTH];
 #pragma unroll
-    for (int ct = 0; ct < KT; ++ct) dq_acc[ct] = dk_acc[ct] = zero4();
+    for (int ct = 0; ct < KTH; ++ct) dq_acc[ct] = dk_acc[ct] = zero4();
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
         if (r > 0) __syncthreads();      // the previous head's tiles are no longer read
         float hd = 0.f;                  // this thread's share of sum(h . dh)
-        f32x4 dqs[KT], dsacc[4];
-        f32x4 dwacc[VSLABS > 1 ? KT : 1], dksacc[VSLABS > 1 ? KT : 1];   // only carried across slabs
+        f32x4 dqs[KTH], dsacc[2];
+        f32x4 dwacc[VSLABS > 1 ? KTH : 1], dksacc[VSLABS > 1 ? KTH : 1];   // only carried across slabs
 #pragma unroll
-        for (int ct = 0; ct < KT; ++ct) dqs[ct] = zero4();
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct) dsacc[ct] = zero4();
+        for (int ct = 0; ct < KTH; ++ct) dqs[ct] = zero4();
+        dsacc[0] = dsacc[1] = zero4();
         if constexpr (VSLABS > 1) {
 #pragma unroll
-            for (int ct = 0; ct < KT; ++ct) dwacc[ct] = dksacc[ct] = zero4();
+            for (int ct = 0; ct < KTH; ++ct) dwacc[ct] = dksacc[ct] = zero4();
         }
         char *dwg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
                                              (int64_t)start * p.dw.st);
 #pragma unroll
         for (int vs = 0; vs < VSLABS; ++vs) {
             if (vs > 0) __syncthreads();     // the previous slab's tiles are no longer read
-            TileCopy<kThreads, K, V> tdh;
+            TileCopy<kDqkwgThreads, K, V> tdh;
             {
-                TileCopy<kThreads, kChunk, V> tv, to, tdv;
-                TileCopy<kThreads, K, V> th;
+                TileCopy<kDqkwgThreads, kChunk, V> tv, to, tdv;
+                TileCopy<kDqkwgThreads, K, V> th;
                 tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st + vs * V, p.v.st, len, tid);
                 to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st + vs * V, p.d_o.st, len, tid);
                 tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st + vs * V, p.dv.st, len, tid);
@@ -175,7 +178,7 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
                 tdv.commit(dvS, pv, len, tid);
                 th.commit(hS, pv, K, tid);
 #pragma unroll
-                for (int m = 0; m < TileCopy<kThreads, K, V>::N; ++m) {
+                for (int m = 0; m < TileCopy<kDqkwgThreads, K, V>::N; ++m) {
                     const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) hd += (float)a[e] * (float)d[e];
@@ -184,29 +187,31 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
             __syncthreads();
             // ---- products with the state at chunk start: dq (state part), dw; and the ds tile ---------
 #pragma unroll
-            for (int ct = 0; ct < KT; ++ct) {
+            for (int ct = 0; ct < KTH; ++ct) {
+                const int cg = half * KTH + ct;
                 f32x4 a = dqs[ct], d = VSLABS > 1 ? dwacc[ct] : zero4();
 #pragma unroll
                 for (int j = 0; j < V / 32; ++j) {
-                    const elemx8 hf = frag_kc(hS, pv, 16 * ct, 32 * j);
+                    const elemx8 hf = frag_kc(hS, pv, 16 * cg, 32 * j);
                     a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
                     d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
                 }
                 dqs[ct] = a;
                 if constexpr (VSLABS > 1) dwacc[ct] = d;
-                else acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -d);
+                else acc_to_global(dwg + 32 * cg, p.dw.st * 2, 16 * w, len, -d);
             }
 #pragma unroll
-            for (int ct = 0; ct < 4; ++ct) {
+            for (int cc = 0; cc < 2; ++cc) {     // ds column tiles half and half + 2 of row tile w
+                const int ct = half + 2 * cc;
                 if (ct <= w) {
 #pragma unroll
                     for (int j = 0; j < V / 32; ++j)
-                        dsacc[ct] = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), dsacc[ct]);
+                        dsacc[cc] = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), dsacc[cc]);
                 }
                 if (vs == VSLABS - 1) {      // complete: gate factors, causal mask, to LDS
                     f32x4 acc = zero4();
                     if (ct <= w) {
-                        acc = dsacc[ct];
+                        acc = dsacc[cc];
                         const int col = 16 * ct + li;
                         const float gc = gS[col];
 #pragma unroll
@@ -224,15 +229,15 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
             __syncthreads();
             if constexpr (VSLABS > 1) {      // dk (state part) of this slab; the single-slab form folds it into the loop below
 #pragma unroll
-                for (int ct = 0; ct < KT; ++ct)
+                for (int ct = 0; ct < KTH; ++ct)
 #pragma unroll
                     for (int j = 0; j < V / 32; ++j)
-                        dksacc[ct] = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dksacc[ct]);
+                        dksacc[ct] = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * (half * KTH + ct), 32 * j), dksacc[ct]);
             }
         }
         if constexpr (VSLABS > 1) {
 #pragma unroll
-            for (int ct = 0; ct < KT; ++ct) acc_to_global(dwg + 32 * ct, p.dw.st * 2, 16 * w, len, -dwacc[ct]);
+            for (int ct = 0; ct < KTH; ++ct) acc_to_global(dwg + 32 * (half * KTH + ct), p.dw.st * 2, 16 * w, len, -dwacc[ct]);
         }
         // ---- products with the state gradient, gate factors, intra-chunk parts -------------------------
         const float g_last = gS[len - 1];
@@ -245,29 +250,30 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
         }
         float dg_row[4] = {0.f, 0.f, 0.f, 0.f}, kdk_state = 0.f;
 #pragma unroll
-        for (int ct = 0; ct < KT; ++ct) {
+        for (int ct = 0; ct < KTH; ++ct) {
+            const int cg = half * KTH + ct;
             f32x4 dks = zero4();
             if constexpr (VSLABS > 1) {
                 dks = dksacc[ct];
             } else {
 #pragma unroll
-                for (int j = 0; j < V / 32; ++j) dks = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * ct, 32 * j), dks);
+                for (int j = 0; j < V / 32; ++j) dks = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * cg, 32 * j), dks);
             }
             f32x4 dq = dqs[ct], dk;
             float kv[4], qv[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int row = 16 * w + 4 * lg + e;
-                kv[e] = (float)kS[row * pk + 16 * ct + li];
-                qv[e] = (float)qS[row * pk + 16 * ct + li];
+                kv[e] = (float)kS[row * pk + 16 * cg + li];
+                qv[e] = (float)qS[row * pk + 16 * cg + li];
                 dq[e] *= eq[e];
                 dk[e] = dks[e] * ek[e];
                 kdk_state += row < len ? dk[e] * kv[e] : 0.f;
             }
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                if (32 * j <= 16 * w + 15) dq = mfma16x32(frag_kc(sS, ps, 16 * w, 32 * j), frag_tr(kS, pk, 16 * ct, 32 * j), dq);
-                if (32 * j + 31 >= 16 * w) dk = mfma16x32(frag_tr(sS, ps, 16 * w, 32 * j), frag_tr(qS, pk, 16 * ct, 32 * j), dk);
+                if (32 * j <= 16 * w + 15) dq = mfma16x32(frag_kc(sS, ps, 16 * w, 32 * j), frag_tr(kS, pk, 16 * cg, 32 * j), dq);
+                if (32 * j + 31 >= 16 * w) dk = mfma16x32(frag_tr(sS, ps, 16 * w, 32 * j), frag_tr(qS, pk, 16 * cg, 32 * j), dk);
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) dg_row[e] += dq[e] * qv[e] - dk[e] * kv[e];
@@ -282,25 +288,33 @@ __global__ void __launch_bounds__(kThreads) dqkwg_kernel(const DqkwgParams p) {
             s2 += __shfl_xor(s2, off, kWave);
         }
         if (l == 0) {
-            red[w] = s1;
-            red[4 + w] = s2;
+            red[wave_id()] = s1;
+            red[8 + wave_id()] = s2;
         }
-        __syncthreads();
-        const float dg_last = (red[0] + red[1] + red[2] + red[3]) * __expf(g_last) + red[4] + red[5] + red[6] + red[7];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float v = group_sum<16>(dg_row[e]);
-            const int row = 16 * w + 4 * lg + e;
-            if (li == 0 && row < len)
-                p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st] = v + (row == len - 1 ? dg_last : 0.f);
+            if (li == 0) dgp[half * kChunk + 16 * w + 4 * lg + e] = v;
+        }
+        __syncthreads();
+        if (tid < kChunk && tid < len) {
+            float hs = 0.f, ks = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                hs += red[i];
+                ks += red[8 + i];
+            }
+            const float dg_last = hs * __expf(g_last) + ks;
+            p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + tid) * p.dg_st] =
+                dgp[tid] + dgp[kChunk + tid] + (tid == len - 1 ? dg_last : 0.f);
         }
     }
     char *dqg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
     char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
 #pragma unroll
-    for (int ct = 0; ct < KT; ++ct) {
-        acc_to_global(dqg + 32 * ct, p.dq.st * 2, 16 * w, len, dq_acc[ct]);
-        acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
+    for (int ct = 0; ct < KTH; ++ct) {
+        acc_to_global(dqg + 32 * (half * KTH + ct), p.dq.st * 2, 16 * w, len, dq_acc[ct]);
+        acc_to_global(dkg + 32 * (half * KTH + ct), p.dk.st * 2, 16 * w, len, dk_acc[ct]);
     }
 }
 
@@ -578,15 +592,16 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
 }
 
 // ---- host side ------------------------------------------------------------------------------------
-#define FLA_BWD_DISPATCH(KERNEL, NAME, GRID, SMEM_EXPR, P)                                                              \
+#define FLA_BWD_DISPATCH_T(KERNEL, NAME, GRID, SMEM_EXPR, P, THREADS)                                                   \
     do {                                                                                                               \
         const size_t smem__ = (SMEM_EXPR);                                                                             \
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, \
                                           (int)smem__));                                                               \
-        FLA_LAUNCH(NAME, stream, KERNEL, GRID, dim3(kThreads), smem__, stream, P);                                      \
+        FLA_LAUNCH(NAME, stream, KERNEL, GRID, dim3(THREADS), smem__, stream, P);                                       \
         FLA_HIP_CHECK(hipGetLastError());                                                                              \
         return FLA_OK;                                                                                                 \
     } while (0)
+#define FLA_BWD_DISPATCH(KERNEL, NAME, GRID, SMEM_EXPR, P) FLA_BWD_DISPATCH_T(KERNEL, NAME, GRID, SMEM_EXPR, P, kThreads)
 
 int check_f32_bht(const char *op, const char *name, const fla_tensor *t, const ChunkGeom &g) {
     int rc = check_tensor(t, op, name, 3, dt_bit(FLA_F32));
@@ -675,15 +690,15 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
     const int VS = V == 256 ? 128 : V;   // value columns held in LDS at a time
-    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 + (kChunk + 8) * 4;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 + (kChunk + 16 + 2 * kChunk) * 4;
     const bool gva = geom.Hv != geom.Hk;
-    if (K == 128 && V == 256) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, true, 2>), "bwd_dqkwg", grid, smem, p);
-    if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, false>), "bwd_dqkwg", grid, smem, p);
-    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<128, 128, true>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, false>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dqkwg_kernel<64, 64, true>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, false>), "bwd_dqkwg", grid, smem, p);
-    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dqkwg_kernel<64, 128, true>), "bwd_dqkwg", grid, smem, p);
+    if (K == 128 && V == 256) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, false>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 128 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 64, false>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 64) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 64, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 128, false>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 128, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 

@@ -129,10 +129,9 @@ __global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const Solv
     }
     __syncthreads();
     elem *O = reinterpret_cast<elem *>(&A[0][0]);  // [BT][BT + 8] 16-bit staging, fits in the fp32 tile
-    if (lane < BT) {
+    const int ocol = lane < BT ? lane : BT;   // surplus lanes (BT < 64) land in the pad column, branch-free
 #pragma unroll
-        for (int i = 0; i < BT; ++i) O[i * PO + lane] = (elem)x[i];
-    }
+    for (int i = 0; i < BT; ++i) O[i * PO + ocol] = (elem)x[i];
     __syncthreads();
     for (int idx = lane; idx < len * CPR; idx += NTH) {
         const int r = idx / CPR, c8 = (idx % CPR) << 3;
