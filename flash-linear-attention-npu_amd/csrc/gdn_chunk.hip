@@ -70,13 +70,13 @@ __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
 // =============================================================================
 struct SolveParams {
     ChunkGeom geom;  // Hv = heads of x
-    const elem *x;
+    const void *x;   // element type, or fp32 (rounded to the element type on load: the cast the caller would do)
     elem *out;
     int64_t sb, sh, st;  // strides of (batch, head, token) in x and out
 };
 
 // BT x BT blocks, BT in {16, 32, 64, 128}; one thread per column of the inverse (at least one full wave).
-template <int BT>
+template <int BT, bool F32IN>
 __global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const SolveParams p) {
     constexpr int NTH = BT < 64 ? 64 : BT;       // threads
     constexpr int CPR = BT / 8;                  // 16-byte pieces per row
@@ -100,7 +100,13 @@ __global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const Solv
 #pragma unroll
         for (int m = 0; m < NP; ++m) {
             const int idx = min(m * NTH + lane, BT * CPR - 1);
-            v[m] = *reinterpret_cast<const elemx8 *>(p.x + base + (int64_t)min(idx / CPR, len - 1) * p.st + ((idx % CPR) << 3));
+            const int64_t off = base + (int64_t)min(idx / CPR, len - 1) * p.st + ((idx % CPR) << 3);
+            if constexpr (F32IN) {
+                const float *src = static_cast<const float *>(p.x) + off;
+                v[m] = frag_from_acc(*reinterpret_cast<const f32x4 *>(src), *reinterpret_cast<const f32x4 *>(src + 4));
+            } else {
+                v[m] = *reinterpret_cast<const elemx8 *>(static_cast<const elem *>(p.x) + off);
+            }
         }
 #pragma unroll
         for (int m = 0; m < NP; ++m) {
@@ -486,7 +492,7 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
                const fla_tensor *out, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "solve_tri";
     int rc;
-    if ((rc = check_tensor(x, op, "x", -1, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_tensor(x, op, "x", -1, dt_bit(kElemDtype) | dt_bit(FLA_F32)))) return rc;
     if ((rc = check_tensor(out, op, "out", -1, dt_bit(kElemDtype)))) return rc;
     FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
     FLA_REQUIRE(same_shape(x, out), FLA_ERR_SHAPE, "%s: out must have the shape of x.", op);
@@ -514,15 +520,18 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query, BT)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0 || geom.Hv == 0) return FLA_OK;
-    SolveParams p{geom, static_cast<const elem *>(x->data), static_cast<elem *>(out->data), ib < 0 ? 0 : x->stride[ib],
-                  x->stride[ih], x->stride[it]};
+    SolveParams p{geom, x->data, static_cast<elem *>(out->data), ib < 0 ? 0 : x->stride[ib], x->stride[ih], x->stride[it]};
     const dim3 grid(geom.NT, geom.Hv, geom.B);
+#define FLA_LAUNCH_SOLVE(BTV, NTHV)                                                                          \
+    if (x->dtype == FLA_F32) FLA_LAUNCH("solve_tri", stream, (solve_tri_kernel<BTV, true>), grid, dim3(NTHV), 0, stream, p); \
+    else FLA_LAUNCH("solve_tri", stream, (solve_tri_kernel<BTV, false>), grid, dim3(NTHV), 0, stream, p)
     switch (BT) {
-        case 16: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<16>, grid, dim3(64), 0, stream, p); break;
-        case 32: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<32>, grid, dim3(64), 0, stream, p); break;
-        case 64: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<64>, grid, dim3(64), 0, stream, p); break;
-        default: FLA_LAUNCH("solve_tri", stream, solve_tri_kernel<128>, grid, dim3(128), 0, stream, p); break;
+        case 16: FLA_LAUNCH_SOLVE(16, 64); break;
+        case 32: FLA_LAUNCH_SOLVE(32, 64); break;
+        case 64: FLA_LAUNCH_SOLVE(64, 64); break;
+        default: FLA_LAUNCH_SOLVE(128, 128); break;
     }
+#undef FLA_LAUNCH_SOLVE
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -636,14 +645,14 @@ FLA_ENTRY(fla_chunk_scaled_dot_kkt)(const fla_tensor *k, const fla_tensor *g, co
 FLA_ENTRY(fla_solve_tri_get_workspace_size)(const fla_tensor *x, const fla_int_array *cu_seqlens,
                                                 const fla_int_array *chunk_indices, const char *layout,
                                                 const fla_tensor *out, uint64_t *workspace_size) {
-    FLA_ROUTE_F16(x, fla_solve_tri_get_workspace_size, x, cu_seqlens, chunk_indices, layout, out, workspace_size);
+    FLA_ROUTE_F16(out, fla_solve_tri_get_workspace_size, x, cu_seqlens, chunk_indices, layout, out, workspace_size);
     FLA_NULL_WS("solve_tri");
     return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, nullptr, 0, nullptr, workspace_size);
 }
 FLA_ENTRY(fla_solve_tri)(const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                              const char *layout, const fla_tensor *out, void *workspace, uint64_t workspace_size,
                              void *stream) {
-    FLA_ROUTE_F16(x, fla_solve_tri, x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size, stream);
+    FLA_ROUTE_F16(out, fla_solve_tri, x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size, stream);
     return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr);
 }

@@ -370,10 +370,11 @@ def npu_causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc
     )
 
 
-def npu_solve_tri(x, *, cu_seqlens=None, chunk_indices=None, layout="bsnd"):
-    """_aclnn_ctypes.py:1786-1800."""
+def npu_solve_tri(x, *, cu_seqlens=None, chunk_indices=None, layout="bsnd", output_dtype=None):
+    """_aclnn_ctypes.py:1786-1800.  Beyond the reference: ``x`` may be float32 with ``output_dtype`` bf16/fp16; the
+    kernel then rounds x to that dtype as it loads it (the cast the caller would otherwise run as its own pass)."""
     x_contig = x.contiguous()
-    out = _empty_like(x_contig)
+    out = _empty_like(x_contig) if output_dtype is None else _empty(_shape(x_contig), x_contig, dtype=output_dtype)
     layout_arg = ctypes.c_char_p(str(layout).encode("utf-8"))
     return _call_op(
         "solve_tri", OP_ARGTYPES["solve_tri"],

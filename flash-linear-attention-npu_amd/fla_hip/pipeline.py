@@ -59,7 +59,7 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
                                  head_first=True, output_dtype=torch.float32)
     bh = beta.transpose(1, 2).contiguous().float()
     A = _ops.chunk_scaled_dot_kkt(k, gh, bh, cu_seqlens=cu, chunk_size=chunk_size)
-    A = _ops.solve_tri(A.to(k.dtype), cu_seqlens=cu, layout="bnsd")
+    A = _ops.solve_tri(A, cu_seqlens=cu, layout="bnsd", output_dtype=k.dtype)   # rounds A to k.dtype on load
     w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, cu_seqlens=cu)
     h, v_new, final = _ops.chunk_gated_delta_rule_fwd_h(
         k, w, u, g=gh, initial_state=initial_state, output_final_state=output_final_state,
@@ -85,7 +85,7 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     bh = beta.float().transpose(1, 2)
     if A is None:
         A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
-        A = _ops.solve_tri(A.to(k.dtype), layout="bnsd", **kw)
+        A = _ops.solve_tri(A, layout="bnsd", output_dtype=k.dtype, **kw)   # rounds A to k.dtype on load
     w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
     doh = do.transpose(1, 2) if do.stride(-1) == 1 else do.transpose(1, 2).contiguous()
     h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,

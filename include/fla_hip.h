@@ -109,7 +109,9 @@ int fla_chunk_scaled_dot_kkt(
 /* ------------------------------------------------------------------------
  * solve_tri - replaces aclnnSolveTri (_aclnn_ctypes.py:1786-1800):
  * out = (I + x)^-1 per C x C chunk block, x strictly lower triangular.
- * layout "bnsd": x [B,H,T,C]; "bsnd": x [B,T,H,C]; bf16 in and out.
+ * layout "bnsd": x [B,H,T,C]; "bsnd": x [B,T,H,C]; "tnd" / "ntd" without the batch
+ * dimension; C (the last dimension) in {16, 32, 64, 128}; bf16 or fp16 in and out,
+ * or f32 in (rounded to the dtype of out while it is loaded).
  * ------------------------------------------------------------------------ */
 int fla_solve_tri_get_workspace_size(
     const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,

@@ -141,6 +141,12 @@ def test_solve_tri_layouts_and_inverse(dev):
     assert_close(out, ref[0], TOL_BF16, "ntd")
     out = ops.solve_tri(A[0].transpose(0, 1).contiguous().to(dev), layout="tnd")
     assert_close(out.transpose(0, 1), ref[0], TOL_BF16, "tnd")
+    # fp32 input rounded on load == the caller's own cast followed by the 16-bit call, bit for bit
+    Af = torch.tril(torch.randn(B, H, T // 64, 64, 64, generator=gen) * 0.2, -1).reshape(B, H, T, 64)
+    for dt in (BF, F16):
+        a = ops.solve_tri(Af.to(dev), layout="bnsd", output_dtype=dt)
+        b2 = ops.solve_tri(Af.to(dt).to(dev), layout="bnsd")
+        assert a.dtype == dt and torch.equal(a, b2)
 
 
 @pytest.mark.parametrize("BT", [16, 32, 128])
