@@ -41,11 +41,18 @@ template <int K, int CT> struct FwdHSmem {
     static constexpr size_t u_off = k_off + (size_t)kChunk * pk * 2;
     static constexpr size_t g_off = u_off + (size_t)kChunk * pu * 2;
     static constexpr size_t buf_bytes = g_off + (size_t)kChunk * 4;
-    static constexpr size_t bytes = 2 * buf_bytes;
+    static constexpr bool kStage = CT == 1;                              // wider slabs leave no LDS for the staging
+    static constexpr int ps = VS + 8;                                    // pitch of the h staging tiles
+    static constexpr size_t stage_off = 2 * buf_bytes;                   // two [K][ps] tiles of the emitted h
+    static constexpr size_t stage_bytes = kStage ? (size_t)K * ps * 2 : 0;
+    static constexpr size_t bytes = stage_off + 2 * stage_bytes;
 };
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
-// c+1 into the other buffer; one barrier per chunk.  h, v_new and the final state leave from registers.
+// c+1 into the other buffer; one barrier per chunk.  v_new and the final state leave from registers; the
+// per-chunk state h goes through an LDS tile and is written out by the loader waves one chunk later, as whole
+// 128-byte rows (written from the accumulator layout it would leave as 32-byte pieces of eight different rows
+// per store, which cost 0.19 ms of a 0.48 ms launch at B=4, T=8192, H=32).
 template <int K, int CT>
 __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -87,12 +94,25 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
             if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
         };
+        const bool stage_h = L::kStage && p.h != nullptr && !p.v_first;
+        auto store_h = [&](int c) {   // staged state of chunk c -> h[.., chunk0 + c, :, slab columns]
+            const elem *st = reinterpret_cast<const elem *>(smem + L::stage_off + (c & 1) * L::stage_bytes);
+            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc + slab * VS;
+#pragma unroll
+            for (int m = 0; m < K * (VS / 8) / kThreads; ++m) {
+                const int idx = m * kThreads + tid;
+                const int r = idx / (VS / 8), c8 = (idx % (VS / 8)) << 3;
+                *reinterpret_cast<u32x4 *>(hg + (int64_t)r * V + c8) = *reinterpret_cast<const u32x4 *>(st + r * L::ps + c8);
+            }
+        };
         if (nchunks > 0) load(0);
         __syncthreads();
         for (int c = 0; c < nchunks; ++c) {
+            if (stage_h && c > 0) store_h(c - 1);
             if (c + 1 < nchunks) load(c + 1);
             __syncthreads();
         }
+        if (stage_h && nchunks > 0) store_h(nchunks - 1);
         return;
     }
 
@@ -149,6 +169,12 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                         const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
                         *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + 16 * ct + li) * K + 16 * kt + 4 * lg) = q4;
                     }
+            } else if constexpr (L::kStage) {   // to the staging tile of this chunk; the loader waves write it out during the next one
+                elem *st = reinterpret_cast<elem *>(smem + L::stage_off + (c & 1) * L::stage_bytes);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) acc_to_tile(st, L::ps, 16 * kt, (wv * CT + ct) * 16, hacc[kt][ct]);
             } else {
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt)
