@@ -620,21 +620,22 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 //   state group (waves 4-7)  chunk i-1: v_new, state update, output (phase C), gate tables
 // Each SIMD holds one wave of each group, so the chunk-parallel work of the next chunk runs under
 // the serial state update of the current one.  Two workgroup barriers per iteration i:
-//   before `mid`  prep : v(i) -> LDS, loads of chunk i+1 issued, A(i) -> aS, dS, pS[i&1]
-//                 state: v_new = u - w h, state update            (reads wS, uS, k and tables of i-1)
+//   before `mid`  prep : o(i-2) LDS -> HBM, v(i) -> LDS, loads of chunk i+1 issued, A(i) -> aS, dS, pS[i&1]
+//                 state: v_new = u - w h, state update, q h_old   (reads wS, uS, q, k and tables of i-1)
 //   after  `mid`  prep : B(i) -> wS, uS; q, k of i+1 -> LDS
-//                 state: o = scale(e^G q h_old + P v_new) -> HBM   (reads q of i-1, pS[(i-1)&1]);
-//                        tables of chunk i+1
+//                 state: o = scale e^G (q h_old) + P v_new -> oS  (reads pS[(i-1)&1]); tables of chunk i+1
 // Every buffer written in one half was last read in the other half or earlier, which is what makes two
-// barriers enough; q therefore needs three buffers, k and the tables two, v one.
+// barriers enough: q, k, the tables and P have two buffers, v, -w, u and o one.  The output leaves through an
+// LDS tile because a state wave owns 16 columns: stored from its registers, o went out as 32-byte pieces of
+// eight rows per instruction, which cost 14 % of the launch; the prep group writes whole 128-byte rows.
 // =============================================================================================
 template <int K> struct PipeSmem {
     static constexpr int pq = K + 8, pk = KTile<K>::pitch, pv = 64 + 8, pa = kChunk + 8, pw = K + 8, pp = kChunk + 8,
                          pd = 24;
     static constexpr size_t q_bytes = (size_t)kChunk * pq * 2, k_bytes = (size_t)kChunk * pk * 2,
                             v_bytes = (size_t)kChunk * pv * 2, tab_bytes = (7 * kChunk + 16) * 4;
-    static constexpr size_t q_off = 0;                                         // three q tiles
-    static constexpr size_t k_off = q_off + 3 * q_bytes;                       // two k tiles
+    static constexpr size_t q_off = 0;                                         // two q tiles
+    static constexpr size_t k_off = q_off + 2 * q_bytes;                       // two k tiles
     static constexpr size_t v_off = k_off + 2 * k_bytes;                       // one v tile
     static constexpr size_t t_off = v_off + v_bytes;                           // two sets of gate tables
     static constexpr size_t a_off = t_off + 2 * tab_bytes;
@@ -642,16 +643,17 @@ template <int K> struct PipeSmem {
     static constexpr size_t p_off = w_off + (size_t)kChunk * pw * 2;           // two P tiles
     static constexpr size_t d_off = p_off + 2 * (size_t)kChunk * pp * 2;
     static constexpr size_t u_off = d_off + (size_t)kChunk * pd * 2;           // u as register images, fp32
-    static constexpr size_t bytes = u_off + (size_t)kChunk * 64 * 4;
+    static constexpr int po = 64 + 8;                                          // pitch of the output staging tile
+    static constexpr size_t o_off = u_off + (size_t)kChunk * 64 * 4;           // o of one chunk, [kChunk][po]
+    static constexpr size_t bytes = o_off + (size_t)kChunk * po * 2;
 };
-// Tiles of chunk c: q cycles through three buffers (it is read until the end of the iteration after
-// the one that prefetches its successor's successor), k and the tables through two, v has one.
+// Tiles of chunk c: q, k and the tables cycle through two buffers, v has one.
 template <int K>
 __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
     typedef PipeSmem<K> L;
-    const int c3 = (unsigned)(c + 3) % 3u, c2 = c & 1;
+    const int c2 = c & 1;
     Tiles t;
-    t.q = reinterpret_cast<elem *>(smem + L::q_off + c3 * L::q_bytes);
+    t.q = reinterpret_cast<elem *>(smem + L::q_off + c2 * L::q_bytes);
     t.k = reinterpret_cast<elem *>(smem + L::k_off + c2 * L::k_bytes);
     t.v = reinterpret_cast<elem *>(smem + L::v_off);
     t.G = reinterpret_cast<float *>(smem + L::t_off + c2 * L::tab_bytes);
@@ -681,6 +683,8 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     elem *pS0 = reinterpret_cast<elem *>(smem + L::p_off);
     elem *dS = reinterpret_cast<elem *>(smem + L::d_off);
     float *uS = reinterpret_cast<float *>(smem + L::u_off);
+    elem *oS = reinterpret_cast<elem *>(smem + L::o_off);
+    constexpr int po = L::po;
 
     const int lin = blockIdx.x;
     int slab, hv, n;
@@ -764,6 +768,20 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             }
         };
         elem *vS = reinterpret_cast<elem *>(smem + L::v_off);
+        // The state group leaves o of a chunk in oS during the second half of an iteration; this group writes
+        // it out in the first half of the next one, 16 bytes per lane, eight lanes per 128-byte row.
+        char *og = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh +
+                                            (int64_t)bos * p.o.st + slab * VS);
+        auto store_o = [&](int c) {
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            char *dst = og + (int64_t)c * kChunk * p.o.st * 2;
+#pragma unroll
+            for (int m = 0; m < VCH; ++m) {
+                const int row = rv + m * VROWS;
+                if (row < len)
+                    *reinterpret_cast<u32x4 *>(dst + ((int64_t)row * p.o.st + cv) * 2) = *reinterpret_cast<const u32x4 *>(oS + row * po + cv);
+            }
+        };
         if (nchunks > 0) {
             prefetch(0);
             commit_qk(pipe_tiles_at<K>(smem, 0));
@@ -776,6 +794,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         for (int i = 0; i <= nchunks; ++i) {
             const Tiles t = pipe_tiles_at<K>(smem, i);
             elem *pS = pS0 + (i & 1) * kChunk * pp;
+            if (i >= 2) store_o(i - 2);
             if (i < nchunks) {
                 // v of this chunk has waited in registers: its single LDS tile was read until the last barrier
 #pragma unroll
@@ -846,6 +865,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             __syncthreads();   // end
             FLA_TICK(4)
         }
+        if (nchunks > 0) store_o(nchunks - 1);
 #ifdef FLA_FUSED_TIMING
         if (blockIdx.x == 0 && l == 0 && p.g_out)
             for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
@@ -1009,12 +1029,25 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 }
             }
         }
-        // q of this chunk and its P tile have been in LDS since the previous iteration: the first operands of
-        // the second half are fetched before the barrier, so their latency hides behind the wait
-        elemx8 qf[2][4], pf[6];
+        // q h with the state at chunk start, here rather than after the barrier: q of this chunk is then read in
+        // this half only, which is what lets q live in two buffers.  The P operands of the second half are
+        // fetched before the barrier too, so their latency hides behind the wait.
+        f32x4 oacc[4];
+        elemx8 pf[6];
         if (c >= 0) {
+            elemx8 qf[KS][4];
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) qf[0][rt] = frag_kc(t.q, pq, rt * 16, 0);
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) qf[j][rt] = frag_kc(t.q, pq, rt * 16, 32 * j);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) oacc[rt] = zero4();
+            FLA_SCHED_FENCE();
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[j][rt], hB[j], oacc[rt]);
+            FLA_SCHED_FENCE();
             pf[0] = frag_kc(pS, pp, 0, 0);
             pf[1] = frag_kc(pS, pp, 16, 0);
             pf[2] = frag_kc(pS, pp, 32, 0);
@@ -1031,23 +1064,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         if (c >= 0) {
 #endif
             // o = scale (e^{G_t} q h + P v_new), h the state at chunk start
-            f32x4 oacc[4];
-#pragma unroll
-            for (int rt = 0; rt < 4; ++rt) oacc[rt] = zero4();
-            {
-#pragma unroll
-                for (int j = 0; j < KS; ++j) {
-                    const int cb = j & 1, nb = cb ^ 1;
-                    if (j + 1 < KS) {
-#pragma unroll
-                        for (int rt = 0; rt < 4; ++rt) qf[nb][rt] = frag_kc(t.q, pq, rt * 16, 32 * (j + 1));
-                    }
-                    FLA_SCHED_FENCE();
-#pragma unroll
-                    for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[cb][rt], hB[j], oacc[rt]);
-                    FLA_SCHED_FENCE();
-                }
-            }
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
             {
@@ -1059,28 +1075,13 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 oacc[2] = mfma16x32(pf[3], vb1, oacc[2]);
                 oacc[3] = mfma16x32(pf[5], vb1, oacc[3]);
             }
-            // tables of the next chunk, then the gate loads of the one after it, and only then the output
-            // stores: memory operations retire in order, so the loads must not queue behind the stores
+            // tables of the next chunk, then the gate loads of the one after it
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
             FLA_TICK(3)
-            char *ob = obase + (int64_t)c * kChunk * p.o.st * 2;
+            // this wave's 16 columns of o into the staging tile; the prep group writes whole rows to memory
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) {
-                const f32x4 acc = oacc[rt];
-                const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
-                const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
-                const bool odd = li & 1;
-                const unsigned send = odd ? p01 : p23;
-                const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
-                const unsigned left = odd ? recv : p01, right = odd ? p23 : recv;
-                char *tile = ob + (int64_t)rt * 16 * o_row;          // uniform
-                const int row = rt * 16 + 4 * lg + (odd ? 2 : 0);
-                if (len == kChunk || row < len)
-                    *reinterpret_cast<unsigned *>(tile + o_lane) = __builtin_amdgcn_perm(right, left, 0x05040100u);
-                if (len == kChunk || row + 1 < len)
-                    *reinterpret_cast<unsigned *>(tile + (o_lane + o_row)) = __builtin_amdgcn_perm(right, left, 0x07060302u);
-            }
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(oS, po, 16 * rt, 16 * wv, oacc[rt]);
         } else {
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
