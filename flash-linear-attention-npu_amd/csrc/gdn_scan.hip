@@ -520,10 +520,8 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        hg[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li] = hB[kt >> 1][ct][(kt & 1) * 4 + e];
+                for (int ct = 0; ct < CT; ++ct)   // lane pairs swap halves: two dword stores per tile instead of four 2-byte ones
+                    acc_to_global(reinterpret_cast<char *>(hg + vcol0 + 16 * ct), (int64_t)V * 2, 16 * kt, K, dacc[kt][ct]);
         }
 
         // dv2 = dv + (k . dh) * e^{g_last - g}
