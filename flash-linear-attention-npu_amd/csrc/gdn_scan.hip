@@ -45,7 +45,9 @@ template <int K, int CT> struct FwdHSmem {
     static constexpr int ps = VS + 8;                                    // pitch of the h staging tiles
     static constexpr size_t stage_off = 2 * buf_bytes;                   // two [K][ps] tiles of the emitted h
     static constexpr size_t stage_bytes = kStage ? (size_t)K * ps * 2 : 0;
-    static constexpr size_t bytes = stage_off + 2 * stage_bytes;
+    static constexpr size_t vstage_off = stage_off + 2 * stage_bytes;    // two [kChunk][ps] tiles of v_new
+    static constexpr size_t vstage_bytes = kStage ? (size_t)kChunk * ps * 2 : 0;
+    static constexpr size_t bytes = vstage_off + 2 * vstage_bytes;
 };
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
@@ -105,13 +107,29 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                 *reinterpret_cast<u32x4 *>(hg + (int64_t)r * V + c8) = *reinterpret_cast<const u32x4 *>(st + r * L::ps + c8);
             }
         };
+        elem *vnew_g = static_cast<elem *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + slab * VS;
+        auto store_v = [&](int c) {   // staged v_new of chunk c -> memory, rows of the valid tokens only
+            const elem *st = reinterpret_cast<const elem *>(smem + L::vstage_off + (c & 1) * L::vstage_bytes);
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+#pragma unroll
+            for (int m = 0; m < kChunk * (VS / 8) / kThreads; ++m) {
+                const int idx = m * kThreads + tid;
+                const int r = idx / (VS / 8), c8 = (idx % (VS / 8)) << 3;
+                if (r < len)
+                    *reinterpret_cast<u32x4 *>(vnew_g + (int64_t)(start + r) * p.v_new.st + c8) =
+                        *reinterpret_cast<const u32x4 *>(st + r * L::ps + c8);
+            }
+        };
         if (nchunks > 0) load(0);
         __syncthreads();
         for (int c = 0; c < nchunks; ++c) {
+            if (L::kStage && c > 0) store_v(c - 1);
             if (stage_h && c > 0) store_h(c - 1);
             if (c + 1 < nchunks) load(c + 1);
             __syncthreads();
         }
+        if (L::kStage && nchunks > 0) store_v(nchunks - 1);
         if (stage_h && nchunks > 0) store_h(nchunks - 1);
         return;
     }
@@ -207,7 +225,13 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) vn[rt][ct][e] = (float)uu[e] - vn[rt][ct][e];
             }
-        {
+        if constexpr (L::kStage) {   // through LDS: the loader waves write whole rows during the next chunk
+            elem *st = reinterpret_cast<elem *>(smem + L::vstage_off + (c & 1) * L::vstage_bytes);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) acc_to_tile(st, L::ps, rt * 16, (wv * CT + ct) * 16, vn[rt][ct]);
+        } else {
             char *dst = vng + (int64_t)start * p.v_new.st * 2;
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt)
