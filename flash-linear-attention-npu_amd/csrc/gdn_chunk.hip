@@ -351,11 +351,14 @@ struct FwdOParams {
     float scale;
 };
 
+// Eight waves when the value dimension gives each of them a 16-column tile (V >= 128): the tiles of one chunk
+// take 97 KB of LDS, so a compute unit holds one workgroup and needs the waves of that one to hide latency.
 template <int K, int V>
-__global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
+__global__ void __launch_bounds__(V >= 128 ? 512 : 256) fwd_o_kernel(const FwdOParams p) {
+    constexpr int NTH = V >= 128 ? 512 : 256, NW = NTH / 64;
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pq = K + 8, pv = V + 16, pp = kChunk + 8;
-    constexpr int CT = V / 64;  // 16-column tiles per wave
+    constexpr int CT = V / (16 * NW);  // 16-column tiles per wave
     elem *qS = reinterpret_cast<elem *>(smem);
     elem *kS = qS + kChunk * pq;
     elem *vS = kS + kChunk * pq;
@@ -373,9 +376,9 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
     const elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
     {   // every load of the chunk is in flight before the first LDS write waits
         const int tid = threadIdx.x;
-        TileCopy<kThreads, kChunk, K> tq, tk;
-        TileCopy<kThreads, kChunk, V> tv;
-        TileCopy<kThreads, K, V> th;
+        TileCopy<NTH, kChunk, K> tq, tk;
+        TileCopy<NTH, kChunk, V> tv;
+        TileCopy<NTH, K, V> th;
         tq.fetch(qg, p.q.st, len, tid);
         tk.fetch(kg, p.k.st, len, tid);
         tv.fetch(vg, p.v.st, len, tid);
@@ -393,8 +396,8 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
     const int w = wave_id();
     // masked, decayed scores P[t][s] (computed as the transposed tile so that a lane
     // holds four consecutive s of one row t)
-    for (int m = 0; m < 4; ++m) {
-        const int id = w + 4 * m, I = id >> 2, J = id & 3;  // t block, s block
+    for (int m = 0; m < 16 / NW; ++m) {
+        const int id = w + NW * m, I = id >> 2, J = id & 3;  // t block, s block
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         const int t = I * 16 + acc_col();
         if (J <= I) {
@@ -457,7 +460,7 @@ __global__ void __launch_bounds__(kThreads) fwd_o_kernel(const FwdOParams p) {
         for (int ct = 0; ct < CT; ++ct) acc_to_tile(vS, pv, rt * 16, (w * CT + ct) * 16, acc[rt][ct] * p.scale);
     __syncthreads();
     elem *og = static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)start * p.o.st;
-    store_tile<kThreads>(og, p.o.st, vS, pv, V, len);
+    store_tile<NTH>(og, p.o.st, vS, pv, V, len);
 }
 
 // ---- host side ------------------------------------------------------------------
@@ -582,7 +585,8 @@ int launch_fwd_o(const FwdOParams &p, hipStream_t stream) {
     const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + kChunk * 4;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem, stream, p);
+    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(V >= 128 ? 512 : 256), smem,
+               stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
