@@ -169,3 +169,59 @@ def test_benchmark_shape(dev):
     o_again, f_again = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None,
                                                        x["initial_state"], True)
     assert torch.equal(o_again, o) and torch.equal(f_again, final)
+
+
+def _rel_stats(x, truth):
+    x, truth = x.double().cpu(), truth.double()
+    err = (x - truth).abs()
+    denom = truth.abs().clamp_min(1e-3 * float(truth.abs().max()))
+    re = err / denom
+    return dict(max_re=float(re.max()), avg_re=float(re.mean()),
+                rmse=float(err.pow(2).mean().sqrt()))
+
+
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
+def test_dual_benchmark_against_fp64_truth(dev, dtype):
+    """The reference's acceptance standard (tests/atk/*/atk_*.json "standard" blocks): the device result and a CPU
+    control that rounds where the reference kernels round are both held against an fp64 truth; the device passes
+    when its max / mean relative error and its RMSE stay within 10x / 3x / 3x of the control's."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 2, 512, 4, 128, 128
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=dtype, seed=101, init_std=0.05)
+    dd = torch.float64
+    truth_o, truth_f = gdn.flash_gated_delta_rule(d["q"].to(dd), d["k"].to(dd), d["v"].to(dd), d["g"].to(dd), d["beta"].to(dd),
+                                                  None, d["initial_state"].to(dd), True, naive=True, compute_dtype=dd)
+    ctrl_o, ctrl_f = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], None, d["initial_state"], True,
+                                                naive=False, lowp=dtype)
+    ctrl_o = ctrl_o.to(dtype)                          # the control's output leaves in the element type too
+    x = {k: v.to(dev) for k, v in d.items()}
+    for fused in (True, False):
+        o, f = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, x["initial_state"], True,
+                                               fused=fused)
+        for name, dut, ctrl, truth in (("o", o, ctrl_o, truth_o), ("final_state", f, ctrl_f, truth_f)):
+            a, c = _rel_stats(dut, truth), _rel_stats(ctrl, truth)
+            assert a["max_re"] <= 10 * c["max_re"] + 1e-6, (fused, name, a, c)
+            assert a["avg_re"] <= 3 * c["avg_re"] + 1e-7, (fused, name, a, c)
+            assert a["rmse"] <= 3 * c["rmse"] + 1e-9, (fused, name, a, c)
+
+
+def test_long_context_packed(dev):
+    """T = 65536 in one packed row (the reference example's default length, examples/flash_gated_delta_rule.py:1863):
+    a 40,000-token sequence between two shorter ones.  Chunked fp32 oracle on the whole row; the long sequence alone
+    (dense call) must reproduce its slice of the packed result bit for bit."""
+    from fla_hip import pipeline
+    T, H, K, V = 65536, 2, 128, 128
+    cu = [0, 12345, 52345, 65536]
+    d = gdn.make_gdn_inputs(1, T, H, K, V, dtype=BF, seed=7)
+    h0 = torch.randn(3, H, K, V, generator=torch.Generator().manual_seed(8)) * 0.01
+    x = {k: (None if v is None else v.to(dev)) for k, v in d.items()}
+    o, f = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, h0.to(dev), True, cu_seqlens=cu)
+    o_ref, f_ref = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], None, h0, True, cu_seqlens=cu,
+                                              naive=False)
+    st = assert_close(o, o_ref, TOL_BF16, "o")
+    assert st["rel_max"] < 3e-2, st
+    assert_close(f, f_ref, TOL_STATE, "final_state")
+    s, e = cu[1], cu[2]
+    o1, f1 = pipeline.flash_gated_delta_rule(x["q"][:, :, s:e], x["k"][:, :, s:e], x["v"][:, :, s:e], x["g"][:, s:e],
+                                             x["beta"][:, s:e], None, h0[1:2].to(dev), True)
+    assert torch.equal(o1, o[:, s:e]) and torch.equal(f1, f[1:2])
