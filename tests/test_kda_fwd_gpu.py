@@ -216,3 +216,32 @@ def test_chunk_kda_fwd_packed_equals_separate(dev):
         part = [t[s:e].contiguous() for t in x]
         o_n, f_n = ops.chunk_kda_fwd(*part, 0.1, 64, layout="TND", initial_state=h0[n:n + 1], output_final_state=True)[:2]
         assert torch.equal(o[s:e], o_n) and torch.equal(final[n], f_n[0])
+
+
+def test_chunk_kda_fwd_dual_benchmark(dev):
+    """The reference's acceptance standard for chunk_kda_fwd (tests/atk/chunk_kda_fwd/atk_chunk_kda_fwd.json): device
+    and a CPU control that rounds to bf16 where the kernels round, both against the fp64 recurrence; the device's
+    max / mean relative error and RMSE must stay within 5x / 1.5x / 1.5x of the control's."""
+    from fla_hip import ops
+    B, T, H, K, V = 2, 512, 4, 128, 128
+    q, k, v, g, beta = make_inputs(B, T, H, H, K, V, seed=77)
+    scale = K ** -0.5
+    gen = torch.Generator().manual_seed(5)
+    h0 = torch.randn(B, H, K, V, generator=gen) * 0.05
+    dd = torch.float64
+    t_o, t_f = kda.naive_recurrent_kda(q.to(dd), k.to(dd), v.to(dd), g.to(dd), beta.to(dd), scale, initial_state=h0.to(dd),
+                                       output_final_state=True, compute_dtype=dd)
+    gk = kda.kda_gate_cumsum(g, 64)
+    ctrl = kda.chunk_kda_fwd(q, k, v, gk, beta, scale, 64, initial_state=h0, output_final_state=True, lowp=BF)
+    out = ops.chunk_kda_fwd(*[to_layout(x, "BSND").to(dev) for x in (q, k, v, g, beta)], scale, 64, initial_state=h0.to(dev),
+                            output_final_state=True)
+
+    def stats(x, truth):
+        x, truth = x.double().cpu(), truth.double()
+        err = (x - truth).abs()
+        re = err / truth.abs().clamp_min(1e-3 * float(truth.abs().max()))
+        return float(re.max()), float(re.mean()), float(err.pow(2).mean().sqrt())
+
+    for name, dut, c, truth in (("o", from_layout(out[0], "BSND"), ctrl["o"].to(BF), t_o), ("final_state", out[1], ctrl["final_state"], t_f)):
+        a, cc = stats(dut, truth), stats(c, truth)
+        assert a[0] <= 5 * cc[0] + 1e-6 and a[1] <= 1.5 * cc[1] + 1e-7 and a[2] <= 1.5 * cc[2] + 1e-9, (name, a, cc)
