@@ -337,7 +337,7 @@ def test_bwd_bnsd_and_packed_layouts(dev):
 
 
 def test_bwd_benchmark_shape_and_autograd_binding(dev):
-    """BASELINE config 2 shape: the reductions over 16384 tokens stay within tolerance, and loss.backward()
+    """The conv1d benchmark shape: the reductions over 16384 tokens stay within tolerance, and loss.backward()
     through ops.causal_conv1d reaches the same gradients."""
     from fla_hip import ops
     gen = torch.Generator().manual_seed(2)

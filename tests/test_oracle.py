@@ -14,7 +14,7 @@ F = torch.nn.functional
 
 # --------------------------------------------------------------------------- GDN
 def test_cfg1_chunked_equals_naive_fp32():
-    """BASELINE config 1: fp32, B=1 T=256 H=2 K=V=64, chunk 64, zero initial state, seed 0."""
+    """Self-check configuration of the benchmark set: fp32, B=1 T=256 H=2 K=V=64, chunk 64, zero initial state, seed 0."""
     d = gdn.make_gdn_inputs(1, 256, 2, 64, 64, seed=0)
     o_n, f_n = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True, naive=True)
     o_c, f_c = gdn.flash_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], output_final_state=True, naive=False)
