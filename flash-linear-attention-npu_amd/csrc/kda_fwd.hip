@@ -501,23 +501,50 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
         if (p.h) {
             elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c) * p.h_sc + hv * p.h_sh;
+            if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+                for (int kt = 0; kt < KT; ++kt) {
+                    const elemx8 f = hB[kt >> 1];
+                    const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
+                    *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + li) * K + 16 * kt + 4 * lg) = q4;
+                }
+            } else {           // [K][V] blocks: lane pairs swap halves, two dword stores per tile
 #pragma unroll
-                for (int e = 0; e < 4; ++e) hg[state_off(16 * kt + 4 * lg + e, vcol0 + li)] = hB[kt >> 1][(kt & 1) * 4 + e];
+                for (int kt = 0; kt < KT; ++kt)
+                    acc_to_global(reinterpret_cast<char *>(hg + vcol0), (int64_t)V * 2, 16 * kt, K, hacc[kt]);
+            }
         }
 
-        // v_new = u - w S ;  o = scale qg S
+        // v_new = u - w S ;  o = scale qg S.  Every operand read is in flight before the first product, so the LDS
+        // latency is paid once per chunk instead of once per contraction step.
         f32x4 vn[4], oacc[4];
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) vn[rt] = oacc[rt] = zero4();
+        {
+            elemx8 wf[KS][4];
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
+            for (int j = 0; j < KS; ++j)
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) {
-                vn[rt] = mfma16x32(frag_kc(wS, pw, rt * 16, 32 * j), hB[j], vn[rt]);
-                oacc[rt] = mfma16x32(frag_kc(qS, pw, rt * 16, 32 * j), hB[j], oacc[rt]);
-            }
+                for (int rt = 0; rt < 4; ++rt) wf[j][rt] = frag_kc(wS, pw, rt * 16, 32 * j);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) vn[rt] = mfma16x32(wf[j][rt], hB[j], vn[rt]);
+        }
+        {
+            elemx8 qf[KS][4];
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) qf[j][rt] = frag_kc(qS, pw, rt * 16, 32 * j);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[j][rt], hB[j], oacc[rt]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
             const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
@@ -541,12 +568,25 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(aS, pb, rt * 16, 32 * j), vB[j], oacc[rt]);
+        {
+            f32x4 dk[KT];
+            elemx8 kf[KT];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) hacc[kt] *= lds4(dS + 16 * kt + 4 * lg);
+            for (int kt = 0; kt < KT; ++kt) kf[kt] = frag_tr(kS, pt, kt * 16, 0);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+            for (int kt = 0; kt < KT; ++kt) dk[kt] = lds4(dS + 16 * kt + 4 * lg);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 32 * j), vB[j], hacc[kt]);
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] *= dk[kt];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(kf[kt], vB[0], hacc[kt]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) kf[kt] = frag_tr(kS, pt, kt * 16, 32);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(kf[kt], vB[1], hacc[kt]);
+        }
         char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
