@@ -26,42 +26,45 @@ struct KktParams {
     int64_t o_sb, o_sh, o_st;
 };
 
+// C = tokens per chunk (64 or 128): the k rows of one chunk sit in LDS, wave w owns the 16-row blocks w, w + 4, ...
+template <int C>
 __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int K = p.geom.K, pitch = K + 8;
     elem *kS = reinterpret_cast<elem *>(smem);
-    float *gS = reinterpret_cast<float *>(kS + kChunk * pitch);
-    float *bS = gS + kChunk;
+    float *gS = reinterpret_cast<float *>(kS + C * pitch);
+    float *bS = gS + C;
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    load_tile<kThreads>(kS, pitch, kg, p.k.st, kChunk, K, len);
-    if (threadIdx.x < kChunk) {
+    load_tile<kThreads>(kS, pitch, kg, p.k.st, C, K, len);
+    if (threadIdx.x < C) {
         const int t = threadIdx.x;
         gS[t] = t < len ? load_scalar(p.g, b, hv, start + t) : 0.f;
         bS[t] = t < len ? load_scalar(p.beta, b, hv, start + t) : 0.f;
     }
     __syncthreads();
 
-    const int I = wave_id();  // t block owned by this wave
-    const int t = I * 16 + acc_col();
-    float *orow = p.out + b * p.o_sb + hv * p.o_sh + (int64_t)(start + t) * p.o_st;
-    const float gt = gS[t], bt = bS[t];
-    for (int J = 0; J < 4; ++J) {  // s block
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        if (J <= I) {
-            for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pitch, J * 16, kk), frag_kc(kS, pitch, I * 16, kk), acc);
+    for (int I = wave_id(); I < C / 16; I += kThreads / 64) {  // t block
+        const int t = I * 16 + acc_col();
+        float *orow = p.out + b * p.o_sb + hv * p.o_sh + (int64_t)(start + t) * p.o_st;
+        const float gt = gS[t], bt = bS[t];
+        for (int J = 0; J < C / 16; ++J) {  // s block
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            if (J <= I) {
+                for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pitch, J * 16, kk), frag_kc(kS, pitch, I * 16, kk), acc);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int s = J * 16 + acc_row(e);
-                const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
-                acc[e] = (s < t && t < len) ? bt * __expf(d) * acc[e] : 0.f;
+                for (int e = 0; e < 4; ++e) {
+                    const int s = J * 16 + acc_row(e);
+                    const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
+                    acc[e] = (s < t && t < len) ? bt * __expf(d) * acc[e] : 0.f;
+                }
             }
+            if (t < len) *reinterpret_cast<f32x4 *>(orow + J * 16 + 4 * (lane_id() >> 4)) = acc;
         }
-        if (t < len) *reinterpret_cast<f32x4 *>(orow + J * 16 + 4 * (lane_id() >> 4)) = acc;
     }
 }
 
@@ -247,13 +250,13 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
 
 // Compile-time head sizes: every load of the chunk (A, k, v tiles, gates) is issued before the first
 // LDS write waits for one of them.
-template <int K, int V>
+template <int K, int V, int C = kChunk>
 __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int pa = kChunk + 8, pk = K + 16, pv = V + 16;
+    constexpr int pa = C + 8, pk = K + 16, pv = V + 16;   // C = tokens per chunk (64 or 128)
     elem *aS = reinterpret_cast<elem *>(smem);
-    elem *kS = aS + kChunk * pa;
-    elem *vS = kS + kChunk * pk;
+    elem *kS = aS + C * pa;
+    elem *vS = kS + C * pk;
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
@@ -264,26 +267,26 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
     const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
     {
-        TileCopy<kThreads, kChunk, kChunk> ta;
-        TileCopy<kThreads, kChunk, K> tk;
-        TileCopy<kThreads, kChunk, V> tv;
+        TileCopy<kThreads, C, C> ta;
+        TileCopy<kThreads, C, K> tk;
+        TileCopy<kThreads, C, V> tv;
         ta.fetch(ag, p.A.st, len, tid);
         tk.fetch(kg, p.k.st, len, tid);
         tv.fetch(vg, p.v.st, len, tid);
         // per-row scale factors of the pieces this thread holds
-        float sk[TileCopy<kThreads, kChunk, K>::N], sv[TileCopy<kThreads, kChunk, V>::N];
+        float sk[TileCopy<kThreads, C, K>::N], sv[TileCopy<kThreads, C, V>::N];
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) {
+        for (int m = 0; m < TileCopy<kThreads, C, K>::N; ++m) {
             const int r = min((m * kThreads + tid) / (K / 8), len - 1);
             sk[m] = load_scalar(p.beta, b, hv, start + r) * __expf(load_scalar(p.g, b, hv, start + r));
         }
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m)
+        for (int m = 0; m < TileCopy<kThreads, C, V>::N; ++m)
             sv[m] = load_scalar(p.beta, b, hv, start + min((m * kThreads + tid) / (V / 8), len - 1));
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, kChunk>::N; ++m) {   // columns past the tail are not part of the block
+        for (int m = 0; m < TileCopy<kThreads, C, C>::N; ++m) {   // columns past the tail are not part of the block
             const int idx = m * kThreads + tid;
-            const int r = idx >> 3, c8 = (idx & 7) << 3;
+            const int r = idx / (C / 8), c8 = (idx % (C / 8)) << 3;
             elemx8 a = __builtin_bit_cast(elemx8, ta.r[m]);
 #pragma unroll
             for (int e = 0; e < 8; ++e)
@@ -304,9 +307,9 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
             *reinterpret_cast<elemx8 *>(dst + r * pitch + c8) = frag_from_acc(lo, hi);
         };
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) scaled(kS, pk, K / 8, m, tk.r[m], sk[m]);
+        for (int m = 0; m < TileCopy<kThreads, C, K>::N; ++m) scaled(kS, pk, K / 8, m, tk.r[m], sk[m]);
 #pragma unroll
-        for (int m = 0; m < TileCopy<kThreads, kChunk, V>::N; ++m) scaled(vS, pv, V / 8, m, tv.r[m], sv[m]);
+        for (int m = 0; m < TileCopy<kThreads, C, V>::N; ++m) scaled(vS, pv, V / 8, m, tv.r[m], sv[m]);
     }
     __syncthreads();
 
@@ -317,17 +320,18 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
         const int per_wave = ncols / 64;  // 16-column tiles per wave
         for (int m = 0; m < per_wave; ++m) {
             const int c0 = (w * per_wave + m) * 16;
-            f32x4 acc[4];
+            f32x4 acc[C / 16];
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int rt = 0; rt < C / 16; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < C / 32; ++j) {
                 const elemx8 bfrag = frag_tr(tile, pitch, c0, 32 * j);
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);
+                for (int rt = 0; rt < C / 16; ++rt)
+                    if (32 * j <= 16 * rt + 15) acc[rt] = mfma16x32(frag_kc(aS, pa, rt * 16, 32 * j), bfrag, acc[rt]);   // A is lower triangular
             }
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc_to_tile(tile, pitch, rt * 16, c0, acc[rt]);
+            for (int rt = 0; rt < C / 16; ++rt) acc_to_tile(tile, pitch, rt * 16, c0, acc[rt]);
         }
     };
     product(kS, pk, K);
@@ -353,7 +357,9 @@ struct FwdOParams {
 
 // Eight waves when the value dimension gives each of them a 16-column tile (V >= 128): the tiles of one chunk
 // take 97 KB of LDS, so a compute unit holds one workgroup and needs the waves of that one to hide latency.
-template <int K, int V>
+// SUB = 64-token row tiles per chunk (2 for 128-token chunks): a workgroup owns one row tile; the second tile of a
+// chunk also contracts over the k / v_new rows of the first (whole block, no causal mask), one block at a time.
+template <int K, int V, int SUB = 1>
 __global__ void __launch_bounds__(V >= 128 ? 512 : 256) fwd_o_kernel(const FwdOParams p) {
     constexpr int NTH = V >= 128 ? 512 : 256, NW = NTH / 64;
     extern __shared__ __align__(16) unsigned char smem[];
@@ -364,93 +370,116 @@ __global__ void __launch_bounds__(V >= 128 ? 512 : 256) fwd_o_kernel(const FwdOP
     elem *vS = kS + kChunk * pq;
     elem *hS = vS + kChunk * pv;
     elem *pS = hS + K * pv;
-    float *gS = reinterpret_cast<float *>(pS + kChunk * pp);
+    float *gS = reinterpret_cast<float *>(pS + kChunk * pp);   // gates of the row tile
+    float *gC = gS + kChunk;                                   // gates of the current column block
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int c = blockIdx.x / SUB, r = blockIdx.x % SUB, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
-    int seq, start, len;
-    chunk_span(p.geom, b, c, seq, start, len);
+    int seq, cstart, clen;
+    chunk_span(p.geom, b, c, seq, cstart, clen);
+    const int start = cstart + r * kChunk;          // first token of this row tile
+    const int len = min(kChunk, clen - r * kChunk);
+    if (len <= 0) return;
     const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
-    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    const elem *kbase = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const elem *vbase = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh;
     const elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc;
-    {   // every load of the chunk is in flight before the first LDS write waits
-        const int tid = threadIdx.x;
-        TileCopy<NTH, kChunk, K> tq, tk;
-        TileCopy<NTH, kChunk, V> tv;
-        TileCopy<NTH, K, V> th;
-        tq.fetch(qg, p.q.st, len, tid);
-        tk.fetch(kg, p.k.st, len, tid);
-        tv.fetch(vg, p.v.st, len, tid);
-        th.fetch(hg, V, K, tid);
-        float gv = 0.f;
-        if (tid < kChunk) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
-        tq.commit(qS, pq, len, tid);
-        tk.commit(kS, pq, len, tid);
-        tv.commit(vS, pv, len, tid);
-        th.commit(hS, pv, K, tid);
-        if (tid < kChunk) gS[tid] = tid < len ? gv : 0.f;
-    }
-    __syncthreads();
-
+    const int tid = threadIdx.x;
     const int w = wave_id();
-    // masked, decayed scores P[t][s] (computed as the transposed tile so that a lane
-    // holds four consecutive s of one row t)
-    for (int m = 0; m < 16 / NW; ++m) {
-        const int id = w + NW * m, I = id >> 2, J = id & 3;  // t block, s block
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        const int t = I * 16 + acc_col();
-        if (J <= I) {
-#pragma unroll
-            for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pq, J * 16, kk), frag_kc(qS, pq, I * 16, kk), acc);
-            const float gt = gS[t];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int s = J * 16 + acc_row(e);
-                acc[e] = (s <= t) ? acc[e] * __expf(fminf(gt - gS[s], 0.f)) : 0.f;
-            }
-        }
-        *reinterpret_cast<elemx4 *>(pS + t * pp + J * 16 + 4 * (lane_id() >> 4)) = cvt4(acc);
-    }
 
-    // inter-chunk term e^{G_t} (q h) for this wave's V columns
     f32x4 acc[4][CT];
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < K / 32; ++j) {
-        elemx8 bfrag[CT];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(hS, pv, (w * CT + ct) * 16, 32 * j);
-#pragma unroll
-        for (int rt = 0; rt < 4; ++rt) {
-            const elemx8 afrag = frag_kc(qS, pq, rt * 16, 32 * j);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+    for (int jb = 0; jb <= (SUB > 1 ? r : 0); ++jb) {
+        const int bstart = cstart + jb * kChunk;                    // first token of the column block
+        const int blen = jb == r ? len : kChunk;                    // earlier blocks of the chunk are complete
+        if (jb > 0) __syncthreads();                                // the previous block's tiles are no longer read
+        {   // every load of the pass is in flight before the first LDS write waits
+            TileCopy<NTH, kChunk, K> tq, tk;
+            TileCopy<NTH, kChunk, V> tv;
+            TileCopy<NTH, K, V> th;
+            if (jb == 0) {
+                tq.fetch(qg, p.q.st, len, tid);
+                th.fetch(hg, V, K, tid);
+            }
+            tk.fetch(kbase + (int64_t)bstart * p.k.st, p.k.st, blen, tid);
+            tv.fetch(vbase + (int64_t)bstart * p.v.st, p.v.st, blen, tid);
+            float gv = 0.f, gc = 0.f;
+            if (tid < kChunk) {
+                if (jb == 0) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+                gc = load_scalar(p.g, b, hv, bstart + min(tid, blen - 1));
+            }
+            if (jb == 0) {
+                tq.commit(qS, pq, len, tid);
+                th.commit(hS, pv, K, tid);
+            }
+            tk.commit(kS, pq, blen, tid);
+            tv.commit(vS, pv, blen, tid);
+            if (tid < kChunk) {
+                if (jb == 0) gS[tid] = tid < len ? gv : 0.f;
+                gC[tid] = tid < blen ? gc : 0.f;
+            }
         }
-    }
+        __syncthreads();
+
+        // decayed (and, on the diagonal block, causally masked) scores P[t][s], computed as the transposed tile so
+        // that a lane holds four consecutive s of one row t
+        const bool diag = jb == r;
+        for (int m = 0; m < 16 / NW; ++m) {
+            const int id = w + NW * m, I = id >> 2, J = id & 3;  // t block, s block
+            f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+            const int t = I * 16 + acc_col();
+            if (!diag || J <= I) {
 #pragma unroll
-    for (int rt = 0; rt < 4; ++rt)
+                for (int kk = 0; kk < K; kk += 32) sc = mfma16x32(frag_kc(kS, pq, J * 16, kk), frag_kc(qS, pq, I * 16, kk), sc);
+                const float gt = gS[t];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float eg = __expf(gS[rt * 16 + acc_row(e)]);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc[rt][ct][e] *= eg;
+                for (int e = 0; e < 4; ++e) {
+                    const int s2 = J * 16 + acc_row(e);
+                    sc[e] = (!diag || s2 <= t) ? sc[e] * __expf(fminf(gt - gC[s2], 0.f)) : 0.f;
+                }
+            }
+            *reinterpret_cast<elemx4 *>(pS + t * pp + J * 16 + 4 * (lane_id() >> 4)) = cvt4(sc);
         }
-    __syncthreads();  // P complete
+
+        if (jb == 0) {   // inter-chunk term e^{G_t} (q h) for this wave's V columns
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < K / 32; ++j) {
+                elemx8 bfrag[CT];
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(hS, pv, (w * CT + ct) * 16, 32 * j);
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) {
+                    const elemx8 afrag = frag_kc(qS, pq, rt * 16, 32 * j);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float eg = __expf(gS[rt * 16 + acc_row(e)]);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) acc[rt][ct][e] *= eg;
+                }
+        }
+        __syncthreads();  // P complete
 
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        elemx8 bfrag[CT];
+        for (int j = 0; j < 2; ++j) {
+            elemx8 bfrag[CT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(vS, pv, (w * CT + ct) * 16, 32 * j);
+            for (int ct = 0; ct < CT; ++ct) bfrag[ct] = frag_tr(vS, pv, (w * CT + ct) * 16, 32 * j);
 #pragma unroll
-        for (int rt = 0; rt < 4; ++rt) {
-            const elemx8 afrag = frag_kc(pS, pp, rt * 16, 32 * j);
+            for (int rt = 0; rt < 4; ++rt) {
+                const elemx8 afrag = frag_kc(pS, pp, rt * 16, 32 * j);
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+                for (int ct = 0; ct < CT; ++ct) acc[rt][ct] = mfma16x32(afrag, bfrag[ct], acc[rt][ct]);
+            }
         }
     }
     // this wave's columns of the v tile are no longer needed: stage o there
@@ -470,14 +499,14 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
     const char *op = "chunk_scaled_dot_kkt";
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom, kElemDtype, 128))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, dt_bit(kElemDtype)))) return rc;
     if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if ((rc = check_tensor(out, op, "out", 4, dt_bit(FLA_F32)))) return rc;
-    FLA_REQUIRE(out->shape[0] == geom.B && out->shape[1] == geom.Hv && out->shape[2] == geom.T && out->shape[3] == kChunk &&
+    FLA_REQUIRE(out->shape[0] == geom.B && out->shape[1] == geom.Hv && out->shape[2] == geom.T && out->shape[3] == geom.C &&
                     inner_unit(out) && out->stride[2] % 4 == 0 && out->stride[1] % 4 == 0 && out->stride[0] % 4 == 0,
-                FLA_ERR_SHAPE, "%s: out must be a 16-byte aligned [B,Hv,T,%d].", op, kChunk);
+                FLA_ERR_SHAPE, "%s: out must be a 16-byte aligned [B,Hv,T,%d].", op, geom.C);
     FLA_REQUIRE(geom.K % 32 == 0 && geom.K >= 32 && geom.K <= 256, FLA_ERR_UNSUPPORTED,
                 "%s: K must be a multiple of 32 in [32,256], got %d.", op, geom.K);
     Varlen vl;
@@ -485,8 +514,14 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     KktParams p{geom, view4(k), view3(g), view3(beta), static_cast<float *>(out->data), out->stride[0], out->stride[1],
                 out->stride[2]};
-    const size_t smem = (size_t)kChunk * (geom.K + 8) * 2 + 2 * kChunk * 4;
-    FLA_LAUNCH("kkt", stream, kkt_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    const size_t smem = (size_t)geom.C * (geom.K + 8) * 2 + 2 * geom.C * 4;
+    if (geom.C == 128) {
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kkt_kernel<128>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)smem));
+        FLA_LAUNCH("kkt", stream, kkt_kernel<128>, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    } else {
+        FLA_LAUNCH("kkt", stream, kkt_kernel<64>, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+    }
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -546,15 +581,17 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     FLA_REQUIRE(gk == nullptr || gk->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: gk must be None.", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
+    FLA_REQUIRE(geom.C == kChunk || (geom.K == 128 && (geom.V == 128 || geom.V == 256)), FLA_ERR_UNSUPPORTED,
+                "%s: chunk_size 128 is built for K=128 with V=128 or 256.", op);
     if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(geom.K % 64 == 0 && geom.V % 64 == 0 && geom.K <= 256 && geom.V <= 256, FLA_ERR_UNSUPPORTED,
                 "%s: K and V must be multiples of 64 up to 256, got K=%d V=%d.", op, geom.K, geom.V);
@@ -562,7 +599,7 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     WuParams p{geom, view4(k), view4(v), view4(A), view4(w), view4(u), view3(g), view3(beta)};
-    const size_t smem = (size_t)kChunk * ((kChunk + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
+    const size_t smem = (size_t)geom.C * ((geom.C + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
     const dim3 grid(geom.NT, geom.Hv, geom.B);
 #define FLA_LAUNCH_WU(KERNEL)                                                                                      \
     do {                                                                                                           \
@@ -570,7 +607,9 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
                                           (int)smem));                                                             \
         FLA_LAUNCH("wu", stream, KERNEL, grid, dim3(kThreads), smem, stream, p);                                    \
     } while (0)
-    if (geom.K == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128>));
+    if (geom.C == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128, 128>));
+    else if (geom.C == 128) FLA_LAUNCH_WU((wu_kernel<128, 256, 128>));
+    else if (geom.K == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128>));
     else if (geom.K == 128 && geom.V == 256) FLA_LAUNCH_WU((wu_kernel<128, 256>));
     else if (geom.K == 64 && geom.V == 64) FLA_LAUNCH_WU((wu_kernel<64, 64>));
     else if (geom.K == 64 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<64, 128>));
@@ -580,13 +619,13 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     return FLA_OK;
 }
 
-template <int K, int V>
+template <int K, int V, int SUB = 1>
 int launch_fwd_o(const FwdOParams &p, hipStream_t stream) {
-    const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + kChunk * 4;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V>),
+    const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + 2 * kChunk * 4;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V, SUB>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(V >= 128 ? 512 : 256), smem,
-               stream, p);
+    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V, SUB>), dim3(p.geom.NT * SUB, p.geom.Hv, p.geom.B), dim3(V >= 128 ? 512 : 256),
+               smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -597,7 +636,7 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const char *op = "chunk_fwd_o";
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
@@ -616,6 +655,11 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     FwdOParams p{geom, view4(q), view4(k), view4(v), view4(out), static_cast<const elem *>(h->data),
                  h->stride[0], h->stride[1], h->stride[2], view3(g), (float)scale};
+    if (geom.C == 128) {
+        if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128, 2>(p, stream);
+        if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256, 2>(p, stream);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: chunk_size 128 is built for K=128 with V=128 or 256.", op);
+    }
     if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128>(p, stream);
     if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256>(p, stream);
     if (geom.K == 64 && geom.V == 64) return launch_fwd_o<64, 64>(p, stream);

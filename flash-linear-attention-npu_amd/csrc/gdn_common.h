@@ -23,6 +23,7 @@ struct ChunkGeom {
     const int32_t *cu;   // [N+1] or null (dense)
     const int32_t *choff;  // [N+1] first chunk of each sequence
     const int32_t *tab;  // [NT][2] (sequence, chunk within sequence)
+    int C = kChunk;      // tokens per chunk (128 where an operator supports it)
 };
 
 // Head-first activations [B, H, T, D] with arbitrary outer strides and unit inner stride.
@@ -60,12 +61,12 @@ __device__ __forceinline__ float load_scalar(const View3 &v, int b, int h, int t
 __device__ __forceinline__ void chunk_span(const ChunkGeom &g, int b, int c, int &seq, int &start, int &len) {
     if (g.cu == nullptr) {
         seq = b;
-        start = c * kChunk;
-        len = min(kChunk, g.T - start);
+        start = c * g.C;
+        len = min(g.C, g.T - start);
     } else {
         seq = g.tab[2 * c];
-        start = g.cu[seq] + g.tab[2 * c + 1] * kChunk;
-        len = min(kChunk, g.cu[seq + 1] - start);
+        start = g.cu[seq] + g.tab[2 * c + 1] * g.C;
+        len = min(g.C, g.cu[seq + 1] - start);
     }
 }
 
@@ -77,8 +78,9 @@ inline View3 view3(const fla_tensor *t) {
 // Common validation of the [B,H,T,D] / [B,H,T] operand family; fills geometry
 // (without varlen pointers).  `v` may be null when the op has no V-sized operand.
 // `elem_dtype` is the dtype code the matrices must have (per-token scalars: that or f32).
+// `max_chunk` = 128 for the operators that are also built for 128-token chunks.
 int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, const fla_tensor *g_like,
-                 int64_t chunk_size, ChunkGeom &geom, int elem_dtype = FLA_BF16);
+                 int64_t chunk_size, ChunkGeom &geom, int elem_dtype = FLA_BF16, int max_chunk = kChunk);
 int check_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, int64_t D,
                int dtype_mask);
 int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T,
@@ -86,6 +88,6 @@ int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, 
 // Validates cu_seqlens / chunk_indices, reports the workspace (query != null) or uploads the chunk table
 // into `workspace` and completes `geom` with the device pointers.
 int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
-                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query, int chunk = kChunk);
+                  void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query, int chunk = 0);
 
 }  // namespace fla

@@ -31,9 +31,13 @@ int check_bht(const char *op, const char *name, const fla_tensor *t, int64_t B, 
 }
 
 int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, const fla_tensor *g_like,
-                 int64_t chunk_size, ChunkGeom &geom, int elem_dtype) {
-    FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: chunk_size must be %d, got %lld.", op, kChunk,
-                (long long)chunk_size);
+                 int64_t chunk_size, ChunkGeom &geom, int elem_dtype, int max_chunk) {
+    if (max_chunk >= 128)
+        FLA_REQUIRE(chunk_size == kChunk || chunk_size == 128, FLA_ERR_UNSUPPORTED,
+                    "%s: chunk_size must be %d or 128, got %lld.", op, kChunk, (long long)chunk_size);
+    else
+        FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: chunk_size must be %d, got %lld.", op, kChunk,
+                    (long long)chunk_size);
     int rc = check_tensor(k, op, "k", 4, dt_bit(elem_dtype));
     if (rc) return rc;
     geom = ChunkGeom{};
@@ -56,14 +60,16 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
     FLA_REQUIRE(geom.Hk > 0 && geom.Hv % geom.Hk == 0, FLA_ERR_SHAPE, "%s: Hv (%d) must be a multiple of Hk (%d).", op,
                 geom.Hv, geom.Hk);
     FLA_REQUIRE(geom.Hv < 65536, FLA_ERR_SHAPE, "%s: too many heads.", op);
-    geom.NT = (geom.T + kChunk - 1) / kChunk;
+    geom.C = (int)chunk_size;
+    geom.NT = (geom.T + geom.C - 1) / geom.C;
     geom.N = geom.B;
     return FLA_OK;
 }
 
 int finish_varlen(const char *op, Varlen &vl, ChunkGeom &geom, const fla_int_array *cu, const fla_int_array *ci,
                   void *workspace, uint64_t workspace_size, hipStream_t stream, uint64_t *query, int chunk) {
-    int rc = build_varlen(vl, op, cu, ci, chunk, geom.T);
+    if (chunk > 0) geom.C = chunk;   // operators without gdn_geometry pass their block size here
+    int rc = build_varlen(vl, op, cu, ci, geom.C, geom.T);
     if (rc) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
     if (vl.enabled) {

@@ -27,6 +27,7 @@ struct ScanParams {
     const void *h0;      // [N,Hv,K,V] or [N,Hv,V,K], fp32 or the element type, or null
     void *hT;            // final state, same layout and type, or null
     int state_elem;      // 1: h0 / hT hold the element type (the carry itself stays fp32)
+    int sub;             // 64-token steps per chunk: 1, or 2 for 128-token chunks (g is cumulated over the whole chunk)
     elem *h;             // [B,Hv,NT,K,V] (or V,K) bf16, or null
     int64_t h_sb, h_sh, h_sc;
     int64_t s_sn, s_sh;  // strides of h0 / hT over (sequence, head)
@@ -97,9 +98,11 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
         };
         const bool stage_h = L::kStage && p.h != nullptr && !p.v_first;
-        auto store_h = [&](int c) {   // staged state of chunk c -> h[.., chunk0 + c, :, slab columns]
-            const elem *st = reinterpret_cast<const elem *>(smem + L::stage_off + (c & 1) * L::stage_bytes);
-            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc + slab * VS;
+        auto store_h = [&](int c) {   // staged state at the start of step c (a chunk start) -> h[.., chunk, :, slab columns]
+            if (c % p.sub != 0) return;
+            const int cc = c / p.sub;
+            const elem *st = reinterpret_cast<const elem *>(smem + L::stage_off + (cc & 1) * L::stage_bytes);
+            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + cc) * p.h_sc + slab * VS;
 #pragma unroll
             for (int m = 0; m < K * (VS / 8) / kThreads; ++m) {
                 const int idx = m * kThreads + tid;
@@ -159,6 +162,8 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
     char *vng = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.v_new.p)) + b * p.v_new.sb + hv * p.v_new.sh + vcol0);
+    elemx8 hB[KS][CT];
+    float gbase = 0.f;
     __syncthreads();
 
     for (int c = 0; c < nchunks; ++c) {
@@ -170,14 +175,21 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
 
-        // state at chunk start as a bf16 operand (and as the emitted h)
-        elemx8 hB[KS][CT];
+        // state at chunk start as a bf16 operand (and as the emitted h).  With 128-token chunks a chunk takes two
+        // 64-token steps: the second one still subtracts w times the state at the CHUNK start (w carries the gate
+        // cumulated from there), while the state itself advances step by step with the gate re-based on the
+        // previous step's last token.
+        const bool chunk_start = (c % p.sub) == 0;
+        if (chunk_start) {
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
+            for (int j = 0; j < KS; ++j)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
-        if (p.h) {
-            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+                for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(hacc[2 * j][ct], hacc[2 * j + 1][ct]);
+            gbase = 0.f;
+        }
+        if (p.h && chunk_start) {
+            const int cc = c / p.sub;
+            elem *hg = p.h + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + cc) * p.h_sc;
             if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt)
@@ -188,7 +200,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                         *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + 16 * ct + li) * K + 16 * kt + 4 * lg) = q4;
                     }
             } else if constexpr (L::kStage) {   // to the staging tile of this chunk; the loader waves write it out during the next one
-                elem *st = reinterpret_cast<elem *>(smem + L::stage_off + (c & 1) * L::stage_bytes);
+                elem *st = reinterpret_cast<elem *>(smem + L::stage_off + (cc & 1) * L::stage_bytes);
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -240,7 +252,8 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
         }
 
         // h <- e^{g_last} h + k^T (v_new e^{g_last - g}); padded rows carry zeros
-        const float dec_all = __expf(g_last);
+        const float dec_all = __expf(g_last - gbase);
+        gbase = g_last;
         elemx8 vB[2][CT];
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -304,7 +317,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: either g or gk must be provided.", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
@@ -312,7 +325,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     if ((rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     Varlen vl;
-    if ((rc = build_varlen(vl, op, cu, ci, kChunk, geom.T))) return rc;
+    if ((rc = build_varlen(vl, op, cu, ci, geom.C, geom.T))) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
     if (vl.enabled) {
         geom.NT = vl.NT;
@@ -368,6 +381,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     p.hT = output_final_state ? final_state->data : nullptr;
     const fla_tensor *sref = has_h0 ? initial_state : (output_final_state ? final_state : nullptr);
     p.state_elem = sref != nullptr && sref->dtype != FLA_F32;
+    p.sub = geom.C / kChunk;
     if (sref) {
         p.s_sn = sref->stride[0];
         p.s_sh = sref->stride[1];

@@ -101,6 +101,13 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     return dq, dk, dv, db.transpose(1, 2), dg.transpose(1, 2), dh0
 
 
+def needs_grad_hint(*tensors) -> bool:
+    """True when autograd will record the call (the backward operators are built for 64-token chunks)."""
+    import torch
+
+    return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 def _autograd_function():
     """Built on first use so that importing this module does not import torch."""
     import torch
@@ -181,14 +188,14 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
                 f"got initial_state.shape[0]={initial_state.shape[0]} and sequences={len(cu) - 1}.")
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    # (o, final_state) do not depend on the chunk size: it only tiles the same recurrence.  The kernels tile
-    # by 64 tokens, so any other power of two is served by the fused route on 64-token chunks.
-    if chunk_size != 64:
+    # (o, final_state) do not depend on the chunk size: it only tiles the same recurrence.  The fused kernel and
+    # the backward operators tile by 64 tokens (the forward operators also by 128), so any other request is served
+    # on 64-token chunks.
+    if chunk_size != 64 and (fused or needs_grad_hint(q, k, v, g, beta, initial_state) or chunk_size != 128):
         if not fused:
-            raise NotImplementedError("the six-operator route is built for chunk_size=64 only; use fused=True.")
+            raise NotImplementedError("the six-operator route is built for chunk_size 64 and 128 (forward); use fused=True.")
         chunk_size = 64
-    needs_grad = torch.is_grad_enabled() and any(
-        isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v, g, beta, initial_state))
+    needs_grad = needs_grad_hint(q, k, v, g, beta, initial_state)
     if not needs_grad:
         _, o, _, final = flash_chunk_gated_delta_rule_fwd(
             q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused=fused,

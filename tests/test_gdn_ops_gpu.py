@@ -108,6 +108,69 @@ def test_stagewise_against_oracle(dev, case, dtype):
     assert_close(final, final_nv, TOL_STATE * 4, "final vs naive")   # unfused path rounds A, w, u to bf16
 
 
+CASES_128 = [
+    (2, 256, 2, 2, 128, 128, None),
+    (1, 200, 4, 2, 128, 128, None),                     # GVA; last chunk holds 72 tokens (a full and a ragged row tile)
+    (1, 130, 2, 2, 128, 256, None),                     # V = 256; last chunk holds 2 tokens
+    (1, 389, 2, 1, 128, 128, [0, 1, 65, 193, 193, 389]),  # lengths 1, 64, 128, 0, 196
+]
+
+
+@pytest.mark.parametrize("dtype", [BF, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", CASES_128)
+def test_stagewise_chunk_128(dev, case, dtype):
+    """The forward operators at chunk_size = 128 (chunk_gated_delta_rule_fwd_h/README.md:85-91, chunk_fwd_o/README.md:100):
+    each stage against the oracle at that chunk size, and the composition against the per-token recurrence."""
+    from fla_hip import ops
+    C = 128
+    B, T, H, Hk, K, V, cu = case
+    TOL = TOL_OF[dtype]
+    d = inputs(B, T, H, K, V, Hk=Hk, seed=T + 1, dtype=dtype)
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, H, K, V, generator=torch.Generator().manual_seed(5)) * 0.01
+    x = dev_kw(d, dev)
+    G = ops.chunk_local_cumsum(x["g"], C, cu_seqlens=cu)
+    G_ref = gdn.chunk_local_cumsum(d["g"], C, cu_seqlens=cu)
+    assert_close(G, G_ref, 1e-5, "cumsum")
+    A0 = ops.chunk_scaled_dot_kkt(x["k"], G, x["beta"], cu_seqlens=cu, chunk_size=C)
+    A0_ref = gdn.chunk_scaled_dot_kkt(d["k"], G_ref, d["beta"], C, cu_seqlens=cu)
+    assert A0.shape == (B, H, T, C)
+    assert_close(A0, A0_ref, 1e-4, "kkt")
+    a0 = A0.cpu()
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, C, cu):
+        blk = a0[b, :, s:e]
+        assert float(torch.triu(blk[:, :, : e - s], 0).abs().max()) == 0.0
+        assert float(blk[:, :, e - s:].abs().max() if e - s < C else 0.0) == 0.0
+    Ainv = ops.solve_tri(A0, cu_seqlens=cu, layout="bnsd", output_dtype=dtype)
+    Ainv_ref = gdn.solve_tri(A0.to(dtype).cpu().float(), cu_seqlens=cu, output_dtype=torch.float32)
+    assert_close(Ainv, Ainv_ref, TOL, "solve_tri")
+    w, u = ops.recompute_w_u_fwd(x["k"], x["v"], x["beta"], Ainv, C, g=G, cu_seqlens=cu)
+    w_ref, u_ref = gdn.recompute_w_u_fwd(d["k"], d["v"], d["beta"], Ainv.cpu(), C, g=G_ref, cu_seqlens=cu,
+                                         output_dtype=torch.float32)
+    assert_close(w, w_ref, TOL, "w")
+    assert_close(u, u_ref, TOL, "u")
+    h, v_new, final = ops.chunk_gated_delta_rule_fwd_h(x["k"], w, u, g=G, initial_state=h0.to(dev),
+                                                       output_final_state=True, chunk_size=C, cu_seqlens=cu)
+    h_ref, vn_ref, final_ref = gdn.chunk_gated_delta_rule_fwd_h(
+        d["k"], w.cpu(), u.cpu(), G_ref, initial_state=h0, output_final_state=True, chunk=C, cu_seqlens=cu,
+        output_dtype=torch.float32)
+    assert h.shape == h_ref.shape
+    assert_close(v_new, vn_ref, TOL, "v_new")
+    assert_close(h, h_ref, TOL, "h")
+    # w of a 128-token chunk is larger than that of a 64-token one, and with it the effect of feeding w h with the
+    # 16-bit state (the reference's rounding point, which the fp32 oracle does not have)
+    assert_close(final, final_ref, 4 * TOL_STATE, "final_state")
+    scale = K ** -0.5
+    o = ops.chunk_fwd_o(x["q"], x["k"], v_new, h, scale, g=G, cu_seqlens=cu, chunk_size=C)
+    o_ref = gdn.chunk_fwd_o(d["q"], d["k"], v_new.cpu(), h.cpu(), scale, g=G_ref, chunk=C, cu_seqlens=cu,
+                            output_dtype=torch.float32)
+    assert_close(o, o_ref, TOL, "o")
+    o_nv, final_nv = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], scale,
+                                                          initial_state=h0, output_final_state=True, cu_seqlens=cu)
+    assert_close(o, o_nv, TOL_BF16, "o vs naive")
+    assert_close(final, final_nv, TOL_STATE * 8, "final vs naive")
+
+
 def test_cumsum_variants(dev):
     from fla_hip import ops
     gen = torch.Generator().manual_seed(3)

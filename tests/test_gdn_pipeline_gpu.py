@@ -93,6 +93,11 @@ def test_other_chunk_sizes_give_the_same_result(dev, chunk_size):
     assert_close(final, f_ref, TOL_STATE, "final_state")
     with pytest.raises(ValueError, match="power of 2"):
         pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], chunk_size=96)
+    if chunk_size == 128:      # the six-operator route runs 128-token chunks natively
+        o2, f2 = pipeline.flash_gated_delta_rule(x["q"], x["k"], x["v"], x["g"], x["beta"], None, x["initial_state"], True,
+                                                 chunk_size=128, fused=False)
+        assert_close(o2, o_ref, TOL_BF16, "o (operators, 128)")
+        assert_close(f2, f_ref, 8 * TOL_STATE, "final_state (operators, 128)")
 
 
 def test_no_initial_state_and_default_scale(dev):
