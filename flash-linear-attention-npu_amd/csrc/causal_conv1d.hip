@@ -161,7 +161,7 @@ __global__ void __launch_bounds__(kThreads) conv1d_fwd_kernel(const ConvParams p
 #pragma unroll
                 for (int r = 0; r < W - 1; ++r) a = fmaf(w[r][i], win[r][i], a);
                 a = fmaf(w[W - 1][i], cur[j][i], a);
-                if (p.activation == 1) a = a * __frcp_rn(1.f + __expf(-a));  // SiLU; 1-ulp reciprocal is ample for a 16-bit result
+                if (p.activation == 1) a = a * __builtin_amdgcn_rcpf(1.f + __expf(-a));  // SiLU; the 1-ulp hardware reciprocal is ample for a 16-bit result
                 acc[i] = a;
             }
 #pragma unroll
@@ -184,8 +184,12 @@ __global__ void __launch_bounds__(kThreads) conv1d_dense_kernel(const ConvParams
     typedef typename Vec8<T>::type V8;
     const int d0 = (blockIdx.y * kThreads + threadIdx.x) * 8;
     if (d0 >= p.D) return;
-    const int b = blockIdx.x / p.tiles_per_seq;
-    const int t0 = (blockIdx.x % p.tiles_per_seq) * TOK;
+    // Workgroup ids go round the eight XCDs; give each XCD a contiguous run of row tiles so that
+    // the W-1 halo rows a tile re-reads were fetched into the same L2 by its predecessor.
+    int tile = blockIdx.x;
+    if ((gridDim.x & 7) == 0) tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const int b = tile / p.tiles_per_seq;
+    const int t0 = (tile % p.tiles_per_seq) * TOK;
     const int nvalid = min(TOK, p.S - t0);
     const T *xp = static_cast<const T *>(p.x) + b * p.x_sb + (int64_t)t0 * p.x_ss + d0;
     const int hd = d0 / p.head_dim, dd = d0 % p.head_dim;
@@ -226,7 +230,7 @@ __global__ void __launch_bounds__(kThreads) conv1d_dense_kernel(const ConvParams
 #pragma unroll
                 for (int r = 0; r < W - 1; ++r) a = fmaf(w[r][i], win[r][i], a);
                 a = fmaf(w[W - 1][i], cur[i], a);
-                if (ACT) a = a * __frcp_rn(1.f + __expf(-a));  // SiLU; a 1-ulp reciprocal is ample for a 16-bit result
+                if (ACT) a = a * __builtin_amdgcn_rcpf(1.f + __expf(-a));  // SiLU; the 1-ulp hardware reciprocal is ample for a 16-bit result
                 o[i] = (T)a;
             }
 #pragma unroll
@@ -355,7 +359,7 @@ __global__ void conv1d_update_kernel(const ConvUpdateParams p) {
             if (i < W - 1)
                 for (int c = 0; c < 8; ++c) acc[c] += wt[i][c] * win[i][c];
         if (p.activation)
-            for (int c = 0; c < 8; ++c) acc[c] = acc[c] / (1.f + __expf(-acc[c]));
+            for (int c = 0; c < 8; ++c) acc[c] = acc[c] * __builtin_amdgcn_rcpf(1.f + __expf(-acc[c]));
         V8 o;
         for (int c = 0; c < 8; ++c) o[c] = (T)acc[c];
         *reinterpret_cast<V8 *>(ob + (int64_t)t * p.o_ss) = o;
@@ -675,8 +679,8 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
     const dim3 grid((unsigned)(p.tiles_per_seq * (packed ? 1 : B)), (unsigned)((D / 8 + kThreads - 1) / kThreads));
     const bool dense_fast = !packed && cache.empty() && init.empty();
     if (dense_fast) {
-        // 16-row tiles keep ~4k workgroups in flight for the benchmark shape; the 3-row halo is an L2 hit
-        const int ft = (B * ((S + 31) / 32) * (int64_t)grid.y >= (int64_t)16 * num_cus()) ? 32 : 16;
+        // 32-row tiles while they still give every CU eight workgroups, 16-row tiles below that
+        const int ft = (B * ((S + 31) / 32) * (int64_t)grid.y >= (int64_t)8 * num_cus()) ? 32 : 16;
         p.tok = ft;
         p.tiles_per_seq = (int)((S + ft - 1) / ft);
         const dim3 fgrid((unsigned)(p.tiles_per_seq * B), grid.y);

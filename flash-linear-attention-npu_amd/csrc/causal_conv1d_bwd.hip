@@ -8,8 +8,9 @@
 // Semantics: causal_conv1d_bwd/README.md:24-52 and the golden test_npu_causal_conv1d_bwd.py:59-127,145-182.
 //
 // Bandwidth-bound.  One thread owns 8 adjacent channels and walks a tile of tokens with two register
-// windows (the next W gradients, the last W inputs); its partial dw / db go to a workspace row per tile and a
-// second kernel sums the tiles in a fixed order, so the reductions are deterministic.  x and dx are always in
+// windows (the next W gradients, the last W inputs).  The four waves of a workgroup take four consecutive tiles
+// of the same channels and add their partial dw / db through LDS; one workspace row per workgroup is left for a
+// second kernel, which sums the rows in a fixed order, so the reductions are deterministic.  x and dx are always in
 // the logical layout; y and dy may be head-split (BNSD / NTD), which only changes their row addressing.
 #include "common.h"
 #include "device_utils.h"
@@ -17,21 +18,23 @@
 namespace fla {
 namespace {
 
-constexpr int kThreads = 128;
+constexpr int kTileWaves = 4;              // waves of a workgroup = consecutive token tiles of the same channels
+constexpr int kThreads = 64 * kTileWaves;
 constexpr int kMaxW = 4;
 constexpr int kTok = 32;   // tokens per tile
+constexpr int kBatch = 4;  // dense path: token rows loaded ahead of their use (8 would spill at W = 4)
 
 struct ConvBwdParams {
     const void *x, *y, *weight, *dy, *h0, *dht;
     void *dx, *dh0;
-    float *partial;               // [tiles][W+1][D]
+    float *partial;               // [tile groups][W+1][D]
     const int32_t *qsl;           // [N+1] or null
     int64_t x_sb, x_st;           // x and dx share the logical layout
     int64_t dx_sb, dx_st;
     int64_t g_sb, g_sh, g_st;     // y and dy: batch, head, token strides
     int64_t w_sr, s_sn, s_sp;     // weight rows; states: sequence, position
     int64_t d_sn, d_sp, o_sn, o_sp;   // dht and dh0 strides
-    int B, T, D, W, N, head_dim, tiles_per_seq, activation, varlen;
+    int B, T, D, W, N, head_dim, tiles_per_seq, tiles, activation, varlen;
 };
 
 template <typename T> __device__ __forceinline__ void ld8(const T *p, float (&f)[8]) {
@@ -68,27 +71,36 @@ __device__ __forceinline__ void load_g(const T *dyp, const T *yp, int activation
         ld8(yp, yy);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float s = 1.f / (1.f + __expf(-yy[i]));
+            const float s = __builtin_amdgcn_rcpf(1.f + __expf(-yy[i]));
             g[i] *= s * (1.f + yy[i] * (1.f - s));
         }
     }
 }
 
 template <typename T, int W>
-__global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParams p) {
-    const int d0 = (blockIdx.y * kThreads + threadIdx.x) * 8;
-    if (d0 >= p.D) return;
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) conv1d_bwd_kernel(const ConvBwdParams p) {
+    // lane -> 8 channels, wave -> token tile; the waves' dw / db sums are added through LDS so that one row of
+    // partial sums leaves the workgroup instead of one per tile
+    __shared__ float red[kTileWaves][64][(kMaxW + 1) * 8 + 1];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int d0 = (blockIdx.y * 64 + lane) * 8;
+    const int tile = blockIdx.x * kTileWaves + wv;
+    float dw[W][8], db[8];
+#pragma unroll
+    for (int r = 0; r < W; ++r) zero8(dw[r]);
+    zero8(db);
+    if (d0 < p.D && tile < p.tiles) {
     int b, t0, t_end, n, bos, eos;
     if (p.varlen) {
         b = 0;
-        t0 = blockIdx.x * kTok;
+        t0 = tile * kTok;
         t_end = min(t0 + kTok, p.T);
         n = find_seq(p.qsl, p.N, t0);
         bos = p.qsl[n];
         eos = p.qsl[n + 1];
     } else {
-        b = blockIdx.x / p.tiles_per_seq;
-        t0 = (blockIdx.x % p.tiles_per_seq) * kTok;
+        b = tile / p.tiles_per_seq;
+        t0 = (tile % p.tiles_per_seq) * kTok;
         t_end = min(t0 + kTok, p.T);
         n = b;
         bos = 0;
@@ -103,11 +115,6 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
     float w[W][8];
 #pragma unroll
     for (int r = 0; r < W; ++r) ld8(static_cast<const T *>(p.weight) + r * p.w_sr + d0, w[r]);
-    float dw[W][8], db[8];
-#pragma unroll
-    for (int r = 0; r < W; ++r) zero8(dw[r]);
-    zero8(db);
-
     float gwin[W][8];       // gwin[i] = g_{t+i} (zero past the end of the sequence)
     float xwin[W - 1][8];   // xwin[j] = xpad_{t-1-j}
     auto seed = [&](int t, int seq, int seq_bos, int seq_eos) {
@@ -126,20 +133,20 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
     };
     seed(t0, n, bos, eos);
     if (!p.varlen) {
-        // dense rows: eight tokens per batch, all their loads (look-ahead gradient rows, input rows) issued
+        // dense rows: kBatch tokens per batch, all their loads (look-ahead gradient rows, input rows) issued
         // before the first use; rows past the end are read from a clamped address and zeroed by a select
         typedef typename Vec8<T>::type V8;
-        for (int tb = t0; tb < t_end; tb += 8) {
-            V8 rdy[8], ry[8], rx[8];
+        for (int tb = t0; tb < t_end; tb += kBatch) {
+            V8 rdy[kBatch], ry[kBatch], rx[kBatch];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < kBatch; ++j) {
                 const int u = min(tb + j + W - 1, p.T - 1), t = min(tb + j, p.T - 1);
                 rdy[j] = *reinterpret_cast<const V8 *>(dyb + (int64_t)u * p.g_st);
                 if (yb) ry[j] = *reinterpret_cast<const V8 *>(yb + (int64_t)u * p.g_st);
                 rx[j] = *reinterpret_cast<const V8 *>(xb + (int64_t)t * p.x_st);
             }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < kBatch; ++j) {
                 const int t = tb + j;
                 if (t >= t_end) break;
                 const bool live = t + W - 1 < p.T;
@@ -149,7 +156,7 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
                     float g = (float)rdy[j][c];
                     if (yb) {
                         const float yy = (float)ry[j][c];
-                        const float sg = 1.f / (1.f + __expf(-yy));
+                        const float sg = __builtin_amdgcn_rcpf(1.f + __expf(-yy));
                         g *= sg * (1.f + yy * (1.f - sg));
                     }
                     gwin[W - 1][c] = live ? g : 0.f;
@@ -237,14 +244,30 @@ __global__ void __launch_bounds__(kThreads) conv1d_bwd_kernel(const ConvBwdParam
 #pragma unroll
         for (int c = 0; c < 8; ++c) xwin[0][c] = cur[c];
     }
-    float *part = p.partial + (int64_t)blockIdx.x * (W + 1) * p.D + d0;
-#pragma unroll
-    for (int r = 0; r < W; ++r) {
-        *reinterpret_cast<f32x4 *>(part + (int64_t)r * p.D) = f32x4{dw[r][0], dw[r][1], dw[r][2], dw[r][3]};
-        *reinterpret_cast<f32x4 *>(part + (int64_t)r * p.D + 4) = f32x4{dw[r][4], dw[r][5], dw[r][6], dw[r][7]};
     }
-    *reinterpret_cast<f32x4 *>(part + (int64_t)W * p.D) = f32x4{db[0], db[1], db[2], db[3]};
-    *reinterpret_cast<f32x4 *>(part + (int64_t)W * p.D + 4) = f32x4{db[4], db[5], db[6], db[7]};
+#pragma unroll
+    for (int r = 0; r < W; ++r)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) red[wv][lane][r * 8 + c] = dw[r][c];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) red[wv][lane][W * 8 + c] = db[c];
+    __syncthreads();
+    // (W+1) rows of 512 channels, four channels per thread and step; the waves are added in wave order
+    float *part = p.partial + (int64_t)blockIdx.x * (W + 1) * p.D + (int64_t)blockIdx.y * 512;
+    for (int idx = threadIdx.x; idx < (W + 1) * 128; idx += kThreads) {
+        const int r = idx >> 7, ch = (idx & 127) * 4;
+        if (blockIdx.y * 512 + ch >= p.D) continue;
+        const float *src = &red[0][ch >> 3][r * 8 + (ch & 7)];
+        f32x4 s;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float a = src[k];
+#pragma unroll
+            for (int ww = 1; ww < kTileWaves; ++ww) a += src[ww * 64 * ((kMaxW + 1) * 8 + 1) + k];
+            s[k] = a;
+        }
+        *reinterpret_cast<f32x4 *>(part + (int64_t)r * p.D + ch) = s;
+    }
 }
 
 // dw[r][d] (r < W) and db[d] (r == W) from the tiles' partial sums.  A block covers 64 channels; its four
@@ -407,7 +430,8 @@ int conv_bwd_impl(const fla_tensor *x, const fla_tensor *y, const fla_tensor *we
     const int64_t tiles_per_seq = (T + kTok - 1) / kTok;
     const int64_t tiles = packed ? tiles_per_seq : tiles_per_seq * B;
     const uint64_t meta = ((qsl.size() * 4 + 255) / 256) * 256;
-    const uint64_t need = meta + (uint64_t)tiles * (W + 1) * D * 4;
+    const int64_t groups = (tiles + kTileWaves - 1) / kTileWaves;
+    const uint64_t need = meta + (uint64_t)groups * (W + 1) * D * 4;
     if (query) {
         *query = need;
         return FLA_OK;
@@ -446,10 +470,11 @@ int conv_bwd_impl(const fla_tensor *x, const fla_tensor *y, const fla_tensor *we
     p.N = (int)N;
     p.head_dim = (int)head_dim;
     p.tiles_per_seq = (int)tiles_per_seq;
+    p.tiles = (int)tiles;
     p.activation = (int)activation;
     p.varlen = packed ? 1 : 0;
     const bool is_bf16 = x->dtype == FLA_BF16;
-    const dim3 grid((unsigned)tiles, (unsigned)((D / 8 + kThreads - 1) / kThreads));
+    const dim3 grid((unsigned)groups, (unsigned)((D / 8 + 63) / 64));
 #define FLA_LAUNCH_BWD(WW)                                                                                         \
     if (is_bf16) FLA_LAUNCH("conv1d_bwd", stream, (conv1d_bwd_kernel<bf16, WW>), grid, dim3(kThreads), 0, stream, p); \
     else FLA_LAUNCH("conv1d_bwd", stream, (conv1d_bwd_kernel<f16, WW>), grid, dim3(kThreads), 0, stream, p)
@@ -463,11 +488,11 @@ int conv_bwd_impl(const fla_tensor *x, const fla_tensor *y, const fla_tensor *we
     if (present(dw) || present(db)) {
         const dim3 rgrid((unsigned)((D + 63) / 64), (unsigned)(W + 1));
         if (is_bf16)
-            FLA_LAUNCH("conv1d_bwd_reduce", stream, conv1d_bwd_reduce_kernel<bf16>, rgrid, dim3(256), 0, stream, p.partial, (int)tiles,
+            FLA_LAUNCH("conv1d_bwd_reduce", stream, conv1d_bwd_reduce_kernel<bf16>, rgrid, dim3(256), 0, stream, p.partial, (int)groups,
                        (int)W, (int)D, present(dw) ? static_cast<bf16 *>(dw->data) : nullptr, present(dw) ? dw->stride[0] : 0,
                        present(db) ? static_cast<bf16 *>(db->data) : nullptr);
         else
-            FLA_LAUNCH("conv1d_bwd_reduce", stream, conv1d_bwd_reduce_kernel<f16>, rgrid, dim3(256), 0, stream, p.partial, (int)tiles,
+            FLA_LAUNCH("conv1d_bwd_reduce", stream, conv1d_bwd_reduce_kernel<f16>, rgrid, dim3(256), 0, stream, p.partial, (int)groups,
                        (int)W, (int)D, present(dw) ? static_cast<f16 *>(dw->data) : nullptr, present(dw) ? dw->stride[0] : 0,
                        present(db) ? static_cast<f16 *>(db->data) : nullptr);
         FLA_HIP_CHECK(hipGetLastError());
