@@ -11,7 +11,7 @@ constexpr float kRcpLn2 = 1.4426950408889634f;
 
 __device__ __forceinline__ float kda_activate(float x, float bias, float eig, int safe, float lower_bound) {
     const float raw = x + bias;
-    if (safe) return lower_bound / (1.f + __expf(-eig * raw));
+    if (safe) return lower_bound * __builtin_amdgcn_rcpf(1.f + __expf(-eig * raw));  // 1-ulp reciprocal
     const float sp = fmaxf(raw, 0.f) + __logf(1.f + __expf(-fabsf(raw)));
     return -eig * sp;
 }
