@@ -363,7 +363,7 @@ def bench_kda(args, torch, dev):
     from oracle import kda as okda
 
     lib = fla_hip.load_library()
-    B, T, H, K, V, C = 2, 8192, 32, 128, 128, 64
+    B, T, H, K, V, C = 2, 8192, 32, 128, 128, args.kda_chunk
     F = torch.nn.functional
     gen = torch.Generator(device=dev).manual_seed(0)
     rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
@@ -404,6 +404,8 @@ def bench_kda(args, torch, dev):
     lib.fla_profile_enable(1)
     for _ in range(args.steps):
         step()
+        if C != 64:   # the backward kernels work on 64-token chunks only
+            continue
         ops.chunk_gated_delta_rule_bwd_dhu(qg, kg, w, d_o, dv, scale, C, gK=gk, h0=h0, dht=dht, use_exp2=True,
                                            dh0_per_sequence=True)
         ops.chunk_kda_bwd_intra(qh, kh, gk, bh, dA1, dA2, z4, z4, z3, z4, layout="BNSD")
@@ -415,6 +417,8 @@ def bench_kda(args, torch, dev):
     flops = {"kda_intra": 2 * (2 * C * K + C * K + C * V + C * C) * th,          # kk, qk, w, u, inverse
              "kda_scan": 2 * (3 * K * V + C * V) * th,                           # w.S, qg.S, kg^T.v_new, Aqk.v_new
              "bwd_dhu": 2 * (3 * K * V) * th}
+    if C == 128:   # dense-tile count of the 64-token kernels that run: diagonal blocks in kda_intra, the rest in kda_cross
+        flops["kda_intra"] = 2 * (3 * 64 * K + 64 * V + 64 * 64) * th
     dominant = max(("kda_intra", "kda_scan"), key=lambda n: kern.get(n, 0.0))
     ach = flops[dominant] / (kern[dominant] * 1e-3) / 1e12
     step_tflops = (flops["kda_intra"] + flops["kda_scan"]) / (ms_per_step * 1e-3) / 1e12
@@ -440,7 +444,7 @@ def bench_kda(args, torch, dev):
         "metric": "kda_chunk_fwd_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "KDA chunk forward B=2 T=8192 H=32 K=V=128 chunk=64 BSND, fp32 initial+final state"},
+        "config": {"workload": f"KDA chunk forward B=2 T=8192 H=32 K=V=128 chunk={C} BSND, fp32 initial+final state"},
         "step_tflops": round(step_tflops, 2),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
@@ -569,6 +573,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--l2norm", action="store_true", help="gdn_chunk: normalise q and k rows inside the kernel")
+    ap.add_argument("--kda-chunk", type=int, default=64, choices=[64, 128], help="kda: tokens per chunk")
     ap.add_argument("--workload", default="gdn_chunk", choices=["gdn_chunk", "gdn_bwd", "decode", "conv1d", "kda", "copy"])
     ap.add_argument("--route", default="fused", choices=["fused", "ops"],
                     help="gdn_chunk: one fused library call, or the six per-stage operators")

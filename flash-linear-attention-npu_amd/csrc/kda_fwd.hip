@@ -1,7 +1,7 @@
 // chunk_kda_fwd: chunked forward of the per-channel gated delta rule (KDA).
 //
-// Two kernels:
-//   kda_intra_kernel  one workgroup per (chunk, value head): gate activation + chunk-local prefix
+// Two kernels (a third, kda_cross_kernel, couples the two 64-token halves of a 128-token chunk):
+//   kda_intra_kernel  one workgroup per (64 tokens, value head): gate activation + chunk-local prefix
 //                     sum (log2 units), the decayed scores Aqk = scale * tril(q k^T . 2^{g_i-g_j})
 //                     and A0 = beta * stril(k k^T . 2^{g_i-g_j}), the explicit inverse
 //                     Akk = (I + A0)^-1, and the WY factors  w = Akk (k beta 2^g),  u = Akk (v beta),
@@ -44,9 +44,14 @@ struct KdaIntraParams {
     float lower_bound;
     float scale;
     float *gk;                // [B,Hv,T,K] or null
-    elem *aqk, *akk;          // [B,Hv,T,64]
+    elem *aqk, *akk;          // [B,Hv,T,C], C = tokens per chunk
     elem *w, *u, *qg, *kg;    // [B,Hv,T,K] / [B,Hv,T,V]
     float *dec;               // [B,NT,Hv,K]: 2^{g_last} of every chunk
+    // 128-token chunks: a workgroup still owns 64 tokens (one half of a chunk); the operands of the block that
+    // couples the halves go to x1 (first half: k 2^{G1 - g}; second half: q 2^{g - G1}) and x2 (second half:
+    // beta k 2^{g - G1}), G1 = gate at the end of the first half.  Both [B,Hv,T,K].
+    int c128;
+    elem *x1, *x2;
 };
 
 // A operand of a 16x16x16 product from four fp32 values, split into a bf16 head and remainder.
@@ -90,7 +95,9 @@ template <int K, int V> struct IntraSmem {
     static constexpr int pq = K + 16, pk = K + 8, pg = K + 4, pv = V + 16, pa = 68, pb = 72;
     static constexpr int SEG = kIntraThreads / K;  // token segments of the gate scan
     static constexpr size_t bytes =
-        (size_t)kChunk * (pq + pk + pv + 2 * pb) * 2 + (size_t)kChunk * (pg + pa + 1) * 4 + (size_t)SEG * K * 4;
+        (size_t)kChunk * (pq + pk + pv + 2 * pb) * 2 + (size_t)((kChunk + 2) * pg + kChunk * (pa + 1)) * 4 +
+        (size_t)2 * SEG * K * 4;
+    // gate rows kChunk and kChunk + 1: the gate at the end of the chunk and the anchor of the coupling block
 };
 
 // Everything a wave does after the gate scan.  Eight waves: wave W of role 0 owns row tile W of k k^T (with the
@@ -100,7 +107,7 @@ template <int K, int V> struct IntraSmem {
 template <int K, int V, int W, int ROLE>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
-                                           int64_t dec_base) {
+                                           int64_t dec_base, int half) {
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb;
     constexpr int KS = K / 32, R1 = W, R2 = 3 - W;
@@ -211,7 +218,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         elemx8 qg8, kg8, kb8;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + 63 * pg + c8 + 4 * h);
+            const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + kChunk * pg + c8 + 4 * h);
             f32x4 a, b, c;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -232,9 +239,27 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             *reinterpret_cast<elemx8 *>(p.qg + (row_base + r) * K + c8) = qg8;
             *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
         }
+        if (p.c128) {   // operands of the block that couples the two halves, both factors <= 1
+            f32x4 x1lo, x1hi, x2lo, x2hi;
+            const f32x4 g0 = lds4(gS + r * pg + c8), g1 = lds4(gS + r * pg + c8 + 4);
+            const f32x4 a0 = lds4(gS + (kChunk + 1) * pg + c8), a1 = lds4(gS + (kChunk + 1) * pg + c8 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float d0 = half ? ex2(g0[e] - a0[e]) : ex2(a0[e] - g0[e]);
+                const float d1 = half ? ex2(g1[e] - a1[e]) : ex2(a1[e] - g1[e]);
+                x1lo[e] = (float)(half ? q8[e] : k8[e]) * d0;
+                x1hi[e] = (float)(half ? q8[4 + e] : k8[4 + e]) * d1;
+                x2lo[e] = (float)k8[e] * br * d0;
+                x2hi[e] = (float)k8[4 + e] * br * d1;
+            }
+            if (r < len) {
+                *reinterpret_cast<elemx8 *>(p.x1 + (row_base + r) * K + c8) = frag_from_acc(x1lo, x1hi);
+                if (half) *reinterpret_cast<elemx8 *>(p.x2 + (row_base + r) * K + c8) = frag_from_acc(x2lo, x2hi);
+            }
+        }
         *reinterpret_cast<elemx8 *>(qS + r * pq + c8) = kb8;
     }
-    if (threadIdx.x < K) p.dec[dec_base + threadIdx.x] = ex2(gS[63 * pg + threadIdx.x]);
+    if (threadIdx.x < K && dec_base >= 0) p.dec[dec_base + threadIdx.x] = ex2(gS[kChunk * pg + threadIdx.x]);
     __syncthreads();
 
     // ---- w = Akk (k beta 2^g) (role 0), u = Akk (v beta) (role 1): row tile W -----------------------------------
@@ -269,14 +294,24 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     elem *akS = vS + kChunk * pv;
     elem *aqS = akS + kChunk * pb;
     float *gS = reinterpret_cast<float *>(aqS + kChunk * pb);
-    float *aS = gS + kChunk * pg;
+    float *aS = gS + (kChunk + 2) * pg;
     float *bS = aS + kChunk * pa;
     float *tS = bS + kChunk;
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int half = p.c128 ? (blockIdx.x & 1) : 0;
+    const int c = p.c128 ? blockIdx.x >> 1 : blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
+    int ostart = start, olen = 0;   // the other half of a 128-token chunk: its gates enter this half's sums
+    if (p.c128) {
+        const int whole = len;
+        olen = min(kChunk, max(0, whole - kChunk * (1 - half)));
+        if (olen > 0) ostart = start + kChunk * (1 - half);
+        start += kChunk * half;
+        len = min(kChunk, whole - kChunk * half);
+        if (len <= 0) return;
+    }
     const int tid = threadIdx.x;
 
     const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
@@ -292,17 +327,27 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
         eig = __expf(p.a_log[hv]);
         if (p.dt_bias) bias = p.dt_bias[(int64_t)hv * K + ch];
     }
-    float raw[TS];
+    float raw[TS], oraw[TS];
     {
         const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
+        const int64_t obase = b * p.g_sb + hv * p.g_sh + (int64_t)ostart * p.g_st + ch;
+        const int olast = max(olen, 1) - 1;
         if (p.g_elem) {
 #pragma unroll
             for (int j = 0; j < TS; ++j)
                 raw[j] = (float)static_cast<const elem *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
+            if (p.c128)
+#pragma unroll
+                for (int j = 0; j < TS; ++j)
+                    oraw[j] = (float)static_cast<const elem *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
         } else {
 #pragma unroll
             for (int j = 0; j < TS; ++j)
                 raw[j] = static_cast<const float *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
+            if (p.c128)
+#pragma unroll
+                for (int j = 0; j < TS; ++j)
+                    oraw[j] = static_cast<const float *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
         }
     }
     {   // all loads of the chunk are issued before the first LDS write waits for one of them
@@ -348,9 +393,27 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
             gS[t * pg + ch] = acc;
         }
         tS[sg * K + ch] = acc;
+        float oacc = 0.f;
+        if (p.c128) {
+#pragma unroll
+            for (int j = 0; j < TS; ++j)
+                if (sg * TS + j < olen)
+                    oacc += (p.use_gate ? kda_activate(oraw[j], bias, eig, p.safe_gate, p.lower_bound) : oraw[j]) * kRcpLn2;
+        }
+        tS[(SEG + sg) * K + ch] = oacc;
         __syncthreads();
-        float off = 0.f;
-        for (int s = 0; s < sg; ++s) off += tS[s * K + ch];
+        float off = 0.f, own = 0.f, other = 0.f;
+        for (int s = 0; s < SEG; ++s) {
+            const float v = tS[s * K + ch];
+            if (s < sg) off += v;
+            own += v;
+            other += tS[(SEG + s) * K + ch];
+        }
+        if (half) off += other;   // gates of the second half continue those of the first
+        if (sg == 0) {
+            gS[kChunk * pg + ch] = own + other;                 // gate at the end of the chunk
+            gS[(kChunk + 1) * pg + ch] = half ? other : own;    // gate at the end of the first half
+        }
         for (int j = 0; j < TS; ++j) {
             const int t = sg * TS + j;
             const float v = gS[t * pg + ch] + off;
@@ -360,22 +423,185 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     }
     __syncthreads();
 
-    const int64_t dec_base = (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
+    const int64_t dec_base = half ? -1 : (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 1: intra_wave<K, V, 1, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 2: intra_wave<K, V, 2, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 3: intra_wave<K, V, 3, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 4: intra_wave<K, V, 0, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 5: intra_wave<K, V, 1, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        case 6: intra_wave<K, V, 2, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
-        default: intra_wave<K, V, 3, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base); break;
+        case 0: intra_wave<K, V, 0, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 1: intra_wave<K, V, 1, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 2: intra_wave<K, V, 2, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 3: intra_wave<K, V, 3, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 4: intra_wave<K, V, 0, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 5: intra_wave<K, V, 1, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 6: intra_wave<K, V, 2, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        default: intra_wave<K, V, 3, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
     }
 
     store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
     store_tile<kIntraThreads>(p.u + row_base * V, V, vS, pv, V, len);
-    store_tile<kIntraThreads>(p.aqk + row_base * kChunk, kChunk, aqS, pb, kChunk, len);
-    store_tile<kIntraThreads>(p.akk + row_base * kChunk, kChunk, akS, pb, kChunk, len);
+    const int C = p.geom.C;
+    store_tile<kIntraThreads>(p.aqk + row_base * C + kChunk * half, C, aqS, pb, kChunk, len);
+    store_tile<kIntraThreads>(p.akk + row_base * C + kChunk * half, C, akS, pb, kChunk, len);
+    if (p.c128 && half == 0) {   // nothing of the second half is visible to the first
+        const elemx8 z = {};
+        for (int idx = tid; idx < len * (kChunk / 8); idx += kIntraThreads) {
+            const int64_t at = (row_base + idx / (kChunk / 8)) * C + kChunk + (idx % (kChunk / 8)) * 8;
+            *reinterpret_cast<elemx8 *>(p.aqk + at) = z;
+            *reinterpret_cast<elemx8 *>(p.akk + at) = z;
+        }
+    }
+}
+
+
+// =============================================================================================
+// 128-token chunks: the block that couples the two 64-token halves
+// =============================================================================================
+// With A0 = [[A11, 0], [M21, A22]] the inverse is [[I11, 0], [-I22 M21 I11, I22]] (I11, I22 the inverses the
+// intra kernel has written).  One workgroup per chunk with a second half:
+//     Aqk21 = scale (q2 2^{g2-G1}) (k1 2^{G1-g1})^T          M21 = (beta2 k2 2^{g2-G1}) (k1 2^{G1-g1})^T
+//     P = I22 M21 ;  Akk21 = -P I11 ;  w2 -= P w1 ;  u2 -= P u1
+// (I21 (k beta 2^g)_1 = -P I11 (k beta 2^g)_1 = -P w1, likewise for u).  M21 and P pass between the products
+// as a 16-bit head plus remainder.  Wave r owns rows 16r.. of the second half.
+struct KdaCrossParams {
+    ChunkGeom geom;
+    const elem *x1, *x2;
+    elem *w, *u, *aqk, *akk;
+    float scale;
+};
+
+template <int K, int V> struct CrossSmem {
+    static constexpr int pk = K + 8, pr = K + 16, pv = V + 16, pb = 72;
+    static constexpr size_t qa_off = 0;
+    static constexpr size_t kb_off = qa_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t kc_off = kb_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t w_off = kc_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t u_off = w_off + (size_t)kChunk * pr * 2;
+    static constexpr size_t a11_off = u_off + (size_t)kChunk * pv * 2;
+    static constexpr size_t a22_off = a11_off + (size_t)kChunk * pb * 2;
+    static constexpr size_t mhi_off = a22_off + (size_t)kChunk * pb * 2;
+    static constexpr size_t mlo_off = mhi_off + (size_t)kChunk * pb * 2;
+    static constexpr size_t bytes = mlo_off + (size_t)kChunk * pb * 2;
+};
+
+__device__ __forceinline__ void split8(f32x4 a, f32x4 b, elemx8 &hi, elemx8 &lo) {
+    elemx4 ah, al, bh, bl;
+    split_hilo(a, ah, al);
+    split_hilo(b, bh, bl);
+    hi = cat8(ah, bh);
+    lo = cat8(al, bl);
+}
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef CrossSmem<K, V> L;
+    constexpr int pk = L::pk, pr = L::pr, pv = L::pv, pb = L::pb, KS = K / 32, C = 2 * kChunk;
+    elem *qaS = reinterpret_cast<elem *>(smem + L::qa_off), *kbS = reinterpret_cast<elem *>(smem + L::kb_off);
+    elem *kcS = reinterpret_cast<elem *>(smem + L::kc_off), *wS = reinterpret_cast<elem *>(smem + L::w_off);
+    elem *uS = reinterpret_cast<elem *>(smem + L::u_off), *a11S = reinterpret_cast<elem *>(smem + L::a11_off);
+    elem *a22S = reinterpret_cast<elem *>(smem + L::a22_off), *mhiS = reinterpret_cast<elem *>(smem + L::mhi_off);
+    elem *mloS = reinterpret_cast<elem *>(smem + L::mlo_off);
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int len2 = len - kChunk;
+    if (len2 <= 0) return;
+    const int tid = threadIdx.x;
+    const int64_t row1 = ((int64_t)b * p.geom.Hv + hv) * p.geom.T + start, row2 = row1 + kChunk;
+    {
+        TileCopy<kThreads, kChunk, K> tq, tb, tc, tw;
+        TileCopy<kThreads, kChunk, V> tu;
+        TileCopy<kThreads, kChunk, kChunk> t1, t2;
+        tq.fetch(p.x1 + row2 * K, K, len2, tid);
+        tb.fetch(p.x2 + row2 * K, K, len2, tid);
+        tc.fetch(p.x1 + row1 * K, K, kChunk, tid);
+        tw.fetch(p.w + row1 * K, K, kChunk, tid);
+        tu.fetch(p.u + row1 * V, V, kChunk, tid);
+        t1.fetch(p.akk + row1 * C, C, kChunk, tid);
+        t2.fetch(p.akk + row2 * C + kChunk, C, len2, tid);
+        tq.commit(qaS, pk, len2, tid);
+        tb.commit(kbS, pk, len2, tid);
+        tc.commit(kcS, pk, kChunk, tid);
+        tw.commit(wS, pr, kChunk, tid);
+        tu.commit(uS, pv, kChunk, tid);
+        t1.commit(a11S, pb, kChunk, tid);
+        t2.commit(a22S, pb, len2, tid);
+    }
+    __syncthreads();
+
+    const int r = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {   // scores of the wave's rows against the first half
+        f32x4 sq[4], sk[4];
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) sq[jt] = sk[jt] = zero4();
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            const elemx8 lq = frag_kc(qaS, pk, 16 * r, 32 * j), lk = frag_kc(kbS, pk, 16 * r, 32 * j);
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                const elemx8 rk = frag_kc(kcS, pk, 16 * jt, 32 * j);
+                sq[jt] = mfma16x32(lq, rk, sq[jt]);
+                sk[jt] = mfma16x32(lk, rk, sk[jt]);
+            }
+        }
+        char *ag = reinterpret_cast<char *>(p.aqk + row2 * C);
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) {
+            acc_to_global(ag + 32 * jt, (int64_t)C * 2, 16 * r, len2, sq[jt] * p.scale);
+            elemx4 hi, lo;
+            split_hilo(sk[jt], hi, lo);
+            acc_to_tile(mhiS, pb, 16 * r, 16 * jt, f32x4{(float)hi[0], (float)hi[1], (float)hi[2], (float)hi[3]});
+            acc_to_tile(mloS, pb, 16 * r, 16 * jt, f32x4{(float)lo[0], (float)lo[1], (float)lo[2], (float)lo[3]});
+        }
+    }
+    __syncthreads();
+
+    // P^T tiles (rows = first-half token j, columns = the wave's rows) as operands with contraction j
+    elemx8 phi[2], plo[2];
+    {
+        f32x4 pt[4];
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) pt[jt] = zero4();
+        for (int ii = 0; ii <= (r >> 1); ++ii) {   // I22 is lower triangular
+            const elemx8 a22 = frag_kc(a22S, pb, 16 * r, 32 * ii);
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt) {
+                pt[jt] = mfma16x32(frag_tr(mhiS, pb, 16 * jt, 32 * ii), a22, pt[jt]);
+                pt[jt] = mfma16x32(frag_tr(mloS, pb, 16 * jt, 32 * ii), a22, pt[jt]);
+            }
+        }
+        split8(pt[0], pt[1], phi[0], plo[0]);
+        split8(pt[2], pt[3], phi[1], plo[1]);
+    }
+    // (P R)^T tiles: rows = column of R, columns = the wave's rows; the lane's four values are adjacent in memory
+    const bool live = 16 * r + li < len2;
+    const int64_t orow = row2 + 16 * r + li;
+    auto product = [&](const elem *R, int pitch, int ct) {
+        f32x4 z = zero4();
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const elemx8 a = frag_tr(R, pitch, 16 * ct, 32 * jj);
+            z = mfma16x32(a, phi[jj], z);
+            z = mfma16x32(a, plo[jj], z);
+        }
+        return z;
+    };
+    auto minus = [&](elem *dst, f32x4 z) {   // *dst -= z
+        if (!live) return;
+        const elemx4 old = *reinterpret_cast<const elemx4 *>(dst);
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (float)old[e] - z[e];
+        *reinterpret_cast<elemx4 *>(dst) = cvt4(v);
+    };
+#pragma unroll
+    for (int ct = 0; ct < K / 16; ++ct) minus(p.w + orow * K + 16 * ct + 4 * lg, product(wS, pr, ct));
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) minus(p.u + orow * V + 16 * ct + 4 * lg, product(uS, pv, ct));
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        const f32x4 z = product(a11S, pb, ct);
+        if (live) *reinterpret_cast<elemx4 *>(p.akk + orow * C + 16 * ct + 4 * lg) = cvt4(-z);
+    }
 }
 
 // =============================================================================================
@@ -410,7 +636,11 @@ template <int K> struct ScanSmem {
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
 // c+1 from memory into the other buffer; one barrier per chunk.  Outputs leave from registers.
-template <int K>
+// SUB = 2: 128-token chunks walked as two 64-token steps.  Both steps see the state of the chunk's first token in
+// w S and qg S (the operand copy of the state is refreshed on even steps only), the second step adds the
+// coupling block Aqk21 times the first step's v_new, and the decay of the chunk is applied once, on the first step
+// (kg already carries 2^{g_last - g} up to the end of the whole chunk).
+template <int K, int SUB>
 __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     typedef ScanSmem<K> L;
@@ -445,9 +675,9 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             tq.fetch(p.qg + row * K, K, len, tid);
             tk.fetch(p.kg + row * K, K, len, tid);
             tu.fetch(p.u + row * V + slab * VS, V, len, tid);
-            ta.fetch(p.aqk + row * kChunk, kChunk, len, tid);
+            ta.fetch(p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, len, tid);   // diagonal block
             float dec = 0.f;
-            if (tid < K) dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c) * p.geom.Hv + hv) * K + tid];
+            if (tid < K) dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c / SUB) * p.geom.Hv + hv) * K + tid];
             tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
             tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pw, len, tid);
             tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pt, len, tid);
@@ -484,6 +714,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     char *og = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
     __syncthreads();
 
+    elemx8 hB[KS], vprev[2] = {};
     for (int c = 0; c < nchunks; ++c) {
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
         const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
@@ -495,12 +726,14 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
         const int64_t row = head_row + start;
+        const bool first = SUB == 1 || (c % SUB) == 0;   // first step of a chunk
 
-        elemx8 hB[KS];
+        if (first) {
 #pragma unroll
-        for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
-        if (p.h) {
-            elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c) * p.h_sc + hv * p.h_sh;
+            for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+        }
+        if (p.h && first) {
+            elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c / SUB) * p.h_sc + hv * p.h_sh;
             if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
                 for (int kt = 0; kt < KT; ++kt) {
@@ -531,6 +764,19 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             for (int j = 0; j < KS; ++j)
 #pragma unroll
                 for (int rt = 0; rt < 4; ++rt) vn[rt] = mfma16x32(wf[j][rt], hB[j], vn[rt]);
+        }
+        // second step of a 128-token chunk: rows of the coupling block Aqk21 straight from memory (rows past the
+        // end re-read the last valid row; their outputs are never stored)
+        elemx8 a21[4][2];
+        if (SUB == 2 && !first) {
+            const elem *ag = p.aqk + row * (kChunk * SUB) + 4 * lg;
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                const elem *ar = ag + (int64_t)min(rt * 16 + li, len - 1) * (kChunk * SUB);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    a21[rt][j] = cat8(*reinterpret_cast<const elemx4 *>(ar + 32 * j), *reinterpret_cast<const elemx4 *>(ar + 32 * j + 16));
+            }
         }
         {
             elemx8 qf[KS][4];
@@ -568,6 +814,16 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(aS, pb, rt * 16, 32 * j), vB[j], oacc[rt]);
+        if (SUB == 2) {
+            if (!first) {
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) oacc[rt] = mfma16x32(a21[rt][j], vprev[j], oacc[rt]);
+            }
+            vprev[0] = vB[0];
+            vprev[1] = vB[1];
+        }
         {
             f32x4 dk[KT];
             elemx8 kf[KT];
@@ -577,7 +833,8 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             for (int kt = 0; kt < KT; ++kt) dk[kt] = lds4(dS + 16 * kt + 4 * lg);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) hacc[kt] *= dk[kt];
+            for (int kt = 0; kt < KT; ++kt)
+                if (first) hacc[kt] *= dk[kt];
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(kf[kt], vB[0], hacc[kt]);
             __builtin_amdgcn_sched_barrier(0);
@@ -660,18 +917,28 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
     const size_t smem = IntraSmem<K, V>::bytes;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kIntraThreads), smem,
-               stream, p);
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT * (p.c128 ? 2 : 1), p.geom.Hv, p.geom.B),
+               dim3(kIntraThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
+    if (p.c128) {
+        KdaCrossParams cp{p.geom, p.x1, p.x2, p.w, p.u, p.aqk, p.akk, p.scale};
+        const size_t csmem = CrossSmem<K, V>::bytes;
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_cross_kernel<K, V>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)csmem));
+        FLA_LAUNCH("kda_cross", stream, (kda_cross_kernel<K, V>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), csmem,
+                   stream, cp);
+        FLA_HIP_CHECK(hipGetLastError());
+    }
     return FLA_OK;
 }
 
-template <int K>
+template <int K, int SUB>
 int launch_scan(const KdaScanParams &p, hipStream_t stream) {
     const size_t smem = ScanSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K, SUB>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K, SUB>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem, stream,
+               p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -689,11 +956,12 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     int rc;
     if ((rc = parse_layout(op, layout, L))) return rc;
     FLA_REQUIRE(chunk_size == 64 || chunk_size == 128, FLA_ERR_SHAPE, "%s: chunk_size must be 64 or 128.", op);
-    FLA_REQUIRE(chunk_size == kChunk, FLA_ERR_UNSUPPORTED, "%s: only chunk_size 64 is implemented.", op);
+    const int C = (int)chunk_size;
     if ((rc = check_tensor(q, op, "q", L.rank3() ? 3 : 4, dt_bit(kElemDtype)))) return rc;
     if ((rc = check_tensor(v, op, "v", L.rank3() ? 3 : 4, dt_bit(kElemDtype)))) return rc;
     const int last = q->ndim - 1;
     ChunkGeom geom{};
+    geom.C = C;
     geom.B = L.rank3() ? 1 : (int)q->shape[L.ib];
     geom.T = (int)q->shape[L.it];
     geom.Hk = (int)q->shape[L.ih];
@@ -744,10 +1012,10 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
                     "%s: lower_bound must be in [-5, 0) for safe gate.", op);
     }
     Varlen vl;
-    if ((rc = build_varlen(vl, op, cu, ci, kChunk, T))) return rc;
+    if ((rc = build_varlen(vl, op, cu, ci, C, T))) return rc;
     FLA_REQUIRE(!vl.enabled || B == 1, FLA_ERR_SHAPE, "%s: rank4 varlen input requires B=1.", op);
     FLA_REQUIRE(!vl.enabled || vl.N <= 1024, FLA_ERR_SHAPE, "%s: varlen input supports at most 1024 sequences.", op);
-    geom.NT = vl.enabled ? vl.NT : (int)((T + kChunk - 1) / kChunk);
+    geom.NT = vl.enabled ? vl.NT : (int)((T + C - 1) / C);
     geom.N = vl.enabled ? vl.N : (int)B;
     const int64_t NT = geom.NT, N = geom.N;
 
@@ -755,8 +1023,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     KdaScanParams sp{};
     if ((rc = layout_view(op, "attn_out", attn_out, L, B, Hv, T, V, bf, sp.o.sb, sp.o.sh, sp.o.st))) return rc;
     sp.o.p = attn_out->data;
-    if ((rc = head_major(op, "Aqk", aqk, L.rank3(), B, Hv, T, kChunk, kElemDtype))) return rc;
-    if ((rc = head_major(op, "Akk", akk, L.rank3(), B, Hv, T, kChunk, kElemDtype))) return rc;
+    if ((rc = head_major(op, "Aqk", aqk, L.rank3(), B, Hv, T, C, kElemDtype))) return rc;
+    if ((rc = head_major(op, "Akk", akk, L.rank3(), B, Hv, T, C, kElemDtype))) return rc;
     if (present(gk) && (rc = head_major(op, "gk", gk, L.rank3(), B, Hv, T, K, FLA_F32))) return rc;
     if (present(w) && (rc = head_major(op, "w", w, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
     if (present(u) && (rc = head_major(op, "u", u, L.rank3(), B, Hv, T, V, kElemDtype))) return rc;
@@ -791,7 +1059,13 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     size_t off = vl.bytes();
     const size_t dec_off = off;
     off += align256((size_t)B * NT * Hv * K * 4);
-    size_t w_off = 0, u_off = 0, qg_off = 0, kg_off = 0;
+    size_t w_off = 0, u_off = 0, qg_off = 0, kg_off = 0, x1_off = 0, x2_off = 0;
+    if (C == 128) {
+        x1_off = off;
+        off += align256(rows * K * 2);
+        x2_off = off;
+        off += align256(rows * K * 2);
+    }
     if (!present(w)) { w_off = off; off += align256(rows * K * 2); }
     if (!present(u)) { u_off = off; off += align256(rows * V * 2); }
     if (!present(qg)) { qg_off = off; off += align256(rows * K * 2); }
@@ -824,6 +1098,9 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     ip.qg = present(qg) ? static_cast<elem *>(qg->data) : reinterpret_cast<elem *>(wsb + qg_off);
     ip.kg = present(kg) ? static_cast<elem *>(kg->data) : reinterpret_cast<elem *>(wsb + kg_off);
     ip.dec = reinterpret_cast<float *>(wsb + dec_off);
+    ip.c128 = C == 128;
+    ip.x1 = reinterpret_cast<elem *>(wsb + x1_off);
+    ip.x2 = reinterpret_cast<elem *>(wsb + x2_off);
     if (K == 128 && V == 128) rc = launch_intra<128, 128>(ip, stream);
     else if (K == 128 && V == 256) rc = launch_intra<128, 256>(ip, stream);
     else if (K == 64 && V == 64) rc = launch_intra<64, 64>(ip, stream);
@@ -853,7 +1130,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     sp.v_first = state_v_first;
     sp.scale = (float)scale;
     if (N == 0) return FLA_OK;
-    return K == 128 ? launch_scan<128>(sp, stream) : launch_scan<64>(sp, stream);
+    if (C == 128) return K == 128 ? launch_scan<128, 2>(sp, stream) : launch_scan<64, 2>(sp, stream);
+    return K == 128 ? launch_scan<128, 1>(sp, stream) : launch_scan<64, 1>(sp, stream);
 }
 
 }  // namespace
