@@ -73,7 +73,6 @@ def profile_report(lib):
 def bench_gdn(args, torch, dev):
     import fla_hip
     from fla_hip import pipeline
-    from oracle import gdn as ogdn
 
     lib = fla_hip.load_library()
     B, T, H, K, V, C = 4, 8192, 32, 128, 128, 64
@@ -133,6 +132,7 @@ def bench_gdn(args, torch, dev):
     # CPU baseline: the oracle's chunked fp32 path on the host cores, bounded sample
     cpu = None
     if not args.no_cpu:
+        from oracle import gdn as ogdn   # the CPU oracle is only ever the baseline being timed
         import torch as _t
         cores = os.cpu_count() or 1
         _t.set_num_threads(cores)
@@ -165,7 +165,6 @@ def bench_gdn(args, torch, dev):
 def bench_decode(args, torch, dev):
     import fla_hip
     from fla_hip import ops
-    from oracle import decode as odec
 
     lib = fla_hip.load_library()
     N, H, D = 256, 32, 128
@@ -204,6 +203,7 @@ def bench_decode(args, torch, dev):
     ach = bytes_per_launch / (ms / n * 1e-3) / 1e9
     cpu = None
     if not args.no_cpu:
+        from oracle import decode as odec   # the CPU oracle is only ever the baseline being timed
         cores = os.cpu_count() or 1
         torch.set_num_threads(cores)
         ns = N
@@ -276,7 +276,6 @@ def bench_decode(args, torch, dev):
 def bench_conv1d(args, torch, dev):
     import fla_hip
     from fla_hip import ops
-    from oracle import conv1d as oconv
 
     lib = fla_hip.load_library()
     B, T, D, W = 4, 4096, 4096, 4
@@ -307,6 +306,7 @@ def bench_conv1d(args, torch, dev):
     ach = bytes_per_launch / (ms / n * 1e-3) / 1e9
     cpu = None
     if not args.no_cpu:
+        from oracle import conv1d as oconv   # the CPU oracle is only ever the baseline being timed
         cores = os.cpu_count() or 1
         torch.set_num_threads(cores)
         xs, ws, bs = x.cpu(), w.cpu(), b.cpu()
@@ -360,7 +360,6 @@ def bench_kda(args, torch, dev):
     in the same run and reported under `other_kernels_ms`."""
     import fla_hip
     from fla_hip import ops
-    from oracle import kda as okda
 
     lib = fla_hip.load_library()
     B, T, H, K, V, C = 2, 8192, 32, 128, 128, args.kda_chunk
@@ -424,6 +423,7 @@ def bench_kda(args, torch, dev):
     step_tflops = (flops["kda_intra"] + flops["kda_scan"]) / (ms_per_step * 1e-3) / 1e12
     cpu = None
     if not args.no_cpu:
+        from oracle import kda as okda   # the CPU oracle is only ever the baseline being timed
         import torch as _t
         cores = os.cpu_count() or 1
         _t.set_num_threads(cores)
@@ -460,7 +460,6 @@ def bench_gdn_bwd(args, torch, dev):
     pass producing dq, dk, dv, dbeta, dg and dh0.  `roofline` describes the kernel that takes the most time."""
     import fla_hip
     from fla_hip import pipeline
-    from oracle import gdn as ogdn, gdn_bwd as obwd
 
     lib = fla_hip.load_library()
     B, T, H, K, V, C = 4, 8192, 32, 128, 128, 64
@@ -514,6 +513,7 @@ def bench_gdn_bwd(args, torch, dev):
     step_flops = sum(flops_of[n] for n in timed)
     cpu = None
     if not args.no_cpu:
+        from oracle import gdn as ogdn, gdn_bwd as obwd   # the CPU oracle is only ever the baseline being timed
         import torch as _t
         cores = os.cpu_count() or 1
         _t.set_num_threads(cores)
