@@ -148,6 +148,123 @@ __global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const Solv
     }
 }
 
+// 64 x 64 blocks on the matrix cores: four waves, wave R inverts diagonal block R and then fills column block R
+// of the inverse.  (I + A)^-1 of a strictly lower 16 x 16 block is the finite product (I - A)(I + A^2)(I + A^4)
+// (I + A^8); the blocks below the diagonal follow by block substitution, X_rc = -D_r sum_m A_rm X_mc, with both
+// operands of those products carried as a 16-bit head plus remainder.
+__device__ __forceinline__ f32x4 solve_lds4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
+__device__ __forceinline__ f32x4 solve_mm3(f32x4 a, f32x4 b, f32x4 acc) {   // acc += a b without the lo * lo term
+    elemx4 ah, al, bh, bl;
+    split_hilo(a, ah, al);
+    split_hilo(b, bh, bl);
+    acc = mfma16x16(ah, bh, acc);
+    acc = mfma16x16(al, bh, acc);
+    acc = mfma16x16(ah, bl, acc);
+    return acc;
+}
+
+template <bool F32IN>
+__global__ void __launch_bounds__(256) solve_tri64_kernel(const SolveParams p) {
+    constexpr int BT = 64, pa = 68, pb = 72, NTH = 256;
+    __shared__ __align__(16) float aS[BT * pa];
+    __shared__ __align__(16) elem oS[BT * pb];
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int start, len;
+    if (p.geom.cu == nullptr) {
+        start = c * BT;
+        len = min(BT, p.geom.T - start);
+    } else {
+        const int seq = p.geom.tab[2 * c];
+        start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * BT;
+        len = min(BT, p.geom.cu[seq + 1] - start);
+    }
+    const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
+    const int tid = threadIdx.x;
+    {   // two 8-element pieces per thread, rows past the end re-read the last valid row and are zeroed
+        elemx8 v[2];
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int idx = m * NTH + tid;
+            const int64_t off = base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3);
+            if constexpr (F32IN) {
+                const float *src = static_cast<const float *>(p.x) + off;
+                v[m] = frag_from_acc(*reinterpret_cast<const f32x4 *>(src), *reinterpret_cast<const f32x4 *>(src + 4));
+            } else {
+                v[m] = *reinterpret_cast<const elemx8 *>(static_cast<const elem *>(p.x) + off);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int idx = m * NTH + tid;
+            const int r = idx >> 3, c8 = (idx & 7) << 3;
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
+                hi[e] = (r < len && c8 + 4 + e < r) ? (float)v[m][4 + e] : 0.f;
+            }
+            *reinterpret_cast<f32x4 *>(aS + r * pa + c8) = lo;
+            *reinterpret_cast<f32x4 *>(aS + r * pa + c8 + 4) = hi;
+        }
+    }
+    __syncthreads();
+
+    const int R = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    {   // diagonal block: a2 = A[4lg+e][li] and a1 = A[li][4lg+e] (both orientations feed the squarings)
+        f32x4 a1, a2, Y;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int r = 4 * lg + e;
+            a2[e] = aS[(16 * R + r) * pa + 16 * R + li];
+            a1[e] = aS[(16 * R + li) * pa + 16 * R + r];
+            Y[e] = (r == li ? 1.f : 0.f) - a1[e];
+        }
+        const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
+        const f32x4 S1 = mfma16x16(A1, A2, zero);   // A^2
+        const f32x4 T1 = mfma16x16(A2, A1, zero);   // (A^2)^T
+        const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
+        Y = mfma16x16(S1b, cvt4(Y), Y);
+        const f32x4 S2 = mfma16x16(T1b, S1b, zero);  // A^4
+        const f32x4 T2 = mfma16x16(S1b, T1b, zero);  // (A^4)^T
+        const elemx4 S2b = cvt4(S2);
+        Y = mfma16x16(S2b, cvt4(Y), Y);
+        const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero);  // A^8
+        Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
+        __syncthreads();   // every wave has read its block of A before the inverses replace the diagonal blocks
+        // lane holds D[li][4lg+e]
+        *reinterpret_cast<f32x4 *>(aS + (16 * R + li) * pa + 16 * R + 4 * lg) = Y;
+        *reinterpret_cast<elemx4 *>(oS + (16 * R + li) * pb + 16 * R + 4 * lg) = cvt4(Y);
+#pragma unroll
+        for (int cb = R + 1; cb < 4; ++cb)
+            *reinterpret_cast<elemx4 *>(oS + (16 * R + li) * pb + 16 * cb + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
+    }
+    __syncthreads();
+    {   // column block R of the inverse, top to bottom: X[k] = block (R + k, R)
+        f32x4 X[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) X[0][e] = aS[(16 * R + 4 * lg + e) * pa + 16 * R + li];
+#pragma unroll
+        for (int k = 1; k < 4; ++k) {
+            if (R + k < 4) {
+                const int r = R + k;
+                f32x4 sum = zero;
+#pragma unroll
+                for (int j = 0; j < k; ++j)
+                    sum = solve_mm3(solve_lds4(aS + (16 * r + li) * pa + 16 * (R + j) + 4 * lg), X[j], sum);
+                const f32x4 dinv = solve_lds4(aS + (16 * r + li) * pa + 16 * r + 4 * lg);
+                X[k] = solve_mm3(-dinv, sum, zero);
+                acc_to_tile(oS, pb, 16 * r, 16 * R, X[k]);
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < len * 8; idx += NTH) {
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(oS + r * pb + c8);
+    }
+}
+
 // =============================================================================
 // recompute_w_u_fwd
 // =============================================================================
@@ -566,7 +683,10 @@ int solve_impl(const fla_tensor *x, const fla_int_array *cu, const fla_int_array
     switch (BT) {
         case 16: FLA_LAUNCH_SOLVE(16, 64); break;
         case 32: FLA_LAUNCH_SOLVE(32, 64); break;
-        case 64: FLA_LAUNCH_SOLVE(64, 64); break;
+        case 64:
+            if (x->dtype == FLA_F32) FLA_LAUNCH("solve_tri", stream, (solve_tri64_kernel<true>), grid, dim3(256), 0, stream, p);
+            else FLA_LAUNCH("solve_tri", stream, (solve_tri64_kernel<false>), grid, dim3(256), 0, stream, p);
+            break;
         default: FLA_LAUNCH_SOLVE(128, 128); break;
     }
 #undef FLA_LAUNCH_SOLVE
