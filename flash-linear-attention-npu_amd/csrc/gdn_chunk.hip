@@ -163,52 +163,10 @@ __device__ __forceinline__ f32x4 solve_mm3(f32x4 a, f32x4 b, f32x4 acc) {   // a
     return acc;
 }
 
-template <bool F32IN>
-__global__ void __launch_bounds__(256) solve_tri64_kernel(const SolveParams p) {
-    constexpr int BT = 64, pa = 68, pb = 72, NTH = 256;
-    __shared__ __align__(16) float aS[BT * pa];
-    __shared__ __align__(16) elem oS[BT * pb];
-    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    int start, len;
-    if (p.geom.cu == nullptr) {
-        start = c * BT;
-        len = min(BT, p.geom.T - start);
-    } else {
-        const int seq = p.geom.tab[2 * c];
-        start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * BT;
-        len = min(BT, p.geom.cu[seq + 1] - start);
-    }
-    const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
-    const int tid = threadIdx.x;
-    {   // two 8-element pieces per thread, rows past the end re-read the last valid row and are zeroed
-        elemx8 v[2];
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            const int idx = m * NTH + tid;
-            const int64_t off = base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3);
-            if constexpr (F32IN) {
-                const float *src = static_cast<const float *>(p.x) + off;
-                v[m] = frag_from_acc(*reinterpret_cast<const f32x4 *>(src), *reinterpret_cast<const f32x4 *>(src + 4));
-            } else {
-                v[m] = *reinterpret_cast<const elemx8 *>(static_cast<const elem *>(p.x) + off);
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            const int idx = m * NTH + tid;
-            const int r = idx >> 3, c8 = (idx & 7) << 3;
-            f32x4 lo, hi;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                lo[e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
-                hi[e] = (r < len && c8 + 4 + e < r) ? (float)v[m][4 + e] : 0.f;
-            }
-            *reinterpret_cast<f32x4 *>(aS + r * pa + c8) = lo;
-            *reinterpret_cast<f32x4 *>(aS + r * pa + c8 + 4) = hi;
-        }
-    }
-    __syncthreads();
-
+// (I + A)^-1 of the strictly lower 64 x 64 matrix in aS (fp32, pitch 68), written to oS (pitch 72) in the element
+// type; called by all four waves of a 256-thread workgroup after a barrier that completes aS, ends with one.
+__device__ __forceinline__ void invert64(float *aS, elem *oS) {
+    constexpr int pa = 68, pb = 72;
     const int R = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     {   // diagonal block: a2 = A[4lg+e][li] and a1 = A[li][4lg+e] (both orientations feed the squarings)
@@ -259,9 +217,114 @@ __global__ void __launch_bounds__(256) solve_tri64_kernel(const SolveParams p) {
         }
     }
     __syncthreads();
+}
+
+template <bool F32IN>
+__global__ void __launch_bounds__(256) solve_tri64_kernel(const SolveParams p) {
+    constexpr int BT = 64, pa = 68, pb = 72, NTH = 256;
+    __shared__ __align__(16) float aS[BT * pa];
+    __shared__ __align__(16) elem oS[BT * pb];
+    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int start, len;
+    if (p.geom.cu == nullptr) {
+        start = c * BT;
+        len = min(BT, p.geom.T - start);
+    } else {
+        const int seq = p.geom.tab[2 * c];
+        start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * BT;
+        len = min(BT, p.geom.cu[seq + 1] - start);
+    }
+    const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
+    const int tid = threadIdx.x;
+    {   // two 8-element pieces per thread, rows past the end re-read the last valid row and are zeroed
+        elemx8 v[2];
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int idx = m * NTH + tid;
+            const int64_t off = base + (int64_t)min(idx >> 3, len - 1) * p.st + ((idx & 7) << 3);
+            if constexpr (F32IN) {
+                const float *src = static_cast<const float *>(p.x) + off;
+                v[m] = frag_from_acc(*reinterpret_cast<const f32x4 *>(src), *reinterpret_cast<const f32x4 *>(src + 4));
+            } else {
+                v[m] = *reinterpret_cast<const elemx8 *>(static_cast<const elem *>(p.x) + off);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const int idx = m * NTH + tid;
+            const int r = idx >> 3, c8 = (idx & 7) << 3;
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (r < len && c8 + e < r) ? (float)v[m][e] : 0.f;
+                hi[e] = (r < len && c8 + 4 + e < r) ? (float)v[m][4 + e] : 0.f;
+            }
+            *reinterpret_cast<f32x4 *>(aS + r * pa + c8) = lo;
+            *reinterpret_cast<f32x4 *>(aS + r * pa + c8 + 4) = hi;
+        }
+    }
+    __syncthreads();
+
+    invert64(aS, oS);
     for (int idx = tid; idx < len * 8; idx += NTH) {
         const int r = idx >> 3, c8 = (idx & 7) << 3;
         *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(oS + r * pb + c8);
+    }
+}
+
+// chunk_scaled_dot_kkt followed by the inversion, without the round trip of the fp32 matrix through memory: the
+// scores are rounded to the element type as solve_tri rounds its input, so the result equals the two operators'.
+__global__ void __launch_bounds__(kThreads) kkt_inverse_kernel(const KktParams p, elem *inv) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int C = kChunk, pa = 68, pb = 72;
+    const int K = p.geom.K, pitch = K + 8;
+    // the score tile and the result take the place of the k rows once every wave holds its scores in registers
+    float *gS = reinterpret_cast<float *>(smem);
+    float *bS = gS + C;
+    elem *kS = reinterpret_cast<elem *>(bS + C);
+    float *aS = reinterpret_cast<float *>(kS);
+    elem *oS = reinterpret_cast<elem *>(aS + C * pa);
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    load_tile<kThreads>(kS, pitch, kg, p.k.st, C, K, len);
+    if (threadIdx.x < C) {
+        const int t = threadIdx.x;
+        gS[t] = t < len ? load_scalar(p.g, b, hv, start + t) : 0.f;
+        bS[t] = t < len ? load_scalar(p.beta, b, hv, start + t) : 0.f;
+    }
+    __syncthreads();
+    {
+        const int I = wave_id(), t = I * 16 + acc_col();
+        const float gt = gS[t], bt = bS[t];
+        f32x4 acc[C / 16];
+#pragma unroll
+        for (int J = 0; J < C / 16; ++J) {
+            acc[J] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (J <= I) {
+                for (int kk = 0; kk < K; kk += 32)
+                    acc[J] = mfma16x32(frag_kc(kS, pitch, J * 16, kk), frag_kc(kS, pitch, I * 16, kk), acc[J]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int s = J * 16 + acc_row(e);
+                    const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
+                    acc[J][e] = (s < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[J][e]) : 0.f;
+                }
+            }
+        }
+        __syncthreads();   // the k rows have been read by every wave
+#pragma unroll
+        for (int J = 0; J < C / 16; ++J) *reinterpret_cast<f32x4 *>(aS + t * pa + J * 16 + 4 * (lane_id() >> 4)) = acc[J];
+    }
+    __syncthreads();
+    invert64(aS, oS);
+    elem *og = inv + ((int64_t)(b * p.geom.Hv + hv) * p.geom.T + start) * C;
+    for (int idx = threadIdx.x; idx < len * 8; idx += kThreads) {
+        const int r = idx >> 3, c8 = (idx & 7) << 3;
+        *reinterpret_cast<u32x4 *>(og + (int64_t)r * C + c8) = *reinterpret_cast<const u32x4 *>(oS + r * pb + c8);
     }
 }
 
@@ -612,15 +675,17 @@ __global__ void __launch_bounds__(V >= 128 ? 512 : 256) fwd_o_kernel(const FwdOP
 // ---- host side ------------------------------------------------------------------
 int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, const fla_int_array *cu,
              const fla_int_array *ci, int64_t chunk_size, const fla_tensor *out, void *ws, uint64_t ws_size,
-             hipStream_t stream, uint64_t *query) {
-    const char *op = "chunk_scaled_dot_kkt";
+             hipStream_t stream, uint64_t *query, bool inverse = false) {
+    const char *op = inverse ? "chunk_scaled_dot_kkt_inverse" : "chunk_scaled_dot_kkt";
     ChunkGeom geom;
     int rc;
     if ((rc = gdn_geometry(op, k, nullptr, g, chunk_size, geom, kElemDtype, 128))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, dt_bit(kElemDtype)))) return rc;
     if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
-    if ((rc = check_tensor(out, op, "out", 4, dt_bit(FLA_F32)))) return rc;
+    if ((rc = check_tensor(out, op, "out", 4, dt_bit(inverse ? kElemDtype : FLA_F32)))) return rc;
+    FLA_REQUIRE(!inverse || (geom.C == kChunk && is_contiguous(out)), FLA_ERR_UNSUPPORTED,
+                "%s: built for 64-token chunks and a contiguous result.", op);
     FLA_REQUIRE(out->shape[0] == geom.B && out->shape[1] == geom.Hv && out->shape[2] == geom.T && out->shape[3] == geom.C &&
                     inner_unit(out) && out->stride[2] % 4 == 0 && out->stride[1] % 4 == 0 && out->stride[0] % 4 == 0,
                 FLA_ERR_SHAPE, "%s: out must be a 16-byte aligned [B,Hv,T,%d].", op, geom.C);
@@ -629,10 +694,17 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
-    KktParams p{geom, view4(k), view3(g), view3(beta), static_cast<float *>(out->data), out->stride[0], out->stride[1],
-                out->stride[2]};
+    KktParams p{geom, view4(k), view3(g), view3(beta), inverse ? nullptr : static_cast<float *>(out->data), out->stride[0],
+                out->stride[1], out->stride[2]};
     const size_t smem = (size_t)geom.C * (geom.K + 8) * 2 + 2 * geom.C * 4;
-    if (geom.C == 128) {
+    if (inverse) {
+        const size_t tiles = (size_t)kChunk * 68 * 4 + (size_t)kChunk * 72 * 2, rows = (size_t)kChunk * (geom.K + 8) * 2;
+        const size_t ismem = (tiles > rows ? tiles : rows) + 2 * kChunk * 4;
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kkt_inverse_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)ismem));
+        FLA_LAUNCH("kkt_inverse", stream, kkt_inverse_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), ismem, stream, p,
+                   static_cast<elem *>(out->data));
+    } else if (geom.C == 128) {
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kkt_kernel<128>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)smem));
         FLA_LAUNCH("kkt", stream, kkt_kernel<128>, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
@@ -808,6 +880,22 @@ FLA_ENTRY(fla_chunk_scaled_dot_kkt)(const fla_tensor *k, const fla_tensor *g, co
     FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size, stream);
     return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
                          static_cast<hipStream_t>(stream), nullptr);
+}
+FLA_ENTRY(fla_chunk_scaled_dot_kkt_inverse_get_workspace_size)(const fla_tensor *k, const fla_tensor *g,
+                                                                   const fla_tensor *beta, const fla_int_array *cu_seqlens,
+                                                                   const fla_int_array *chunk_indices, int64_t chunk_size,
+                                                                   const fla_tensor *out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_inverse_get_workspace_size, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace_size);
+    FLA_NULL_WS("chunk_scaled_dot_kkt_inverse");
+    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size, true);
+}
+FLA_ENTRY(fla_chunk_scaled_dot_kkt_inverse)(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+                                                const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+                                                int64_t chunk_size, const fla_tensor *out, void *workspace,
+                                                uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_inverse, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size, stream);
+    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr, true);
 }
 
 FLA_ENTRY(fla_solve_tri_get_workspace_size)(const fla_tensor *x, const fla_int_array *cu_seqlens,

@@ -32,6 +32,7 @@ _REFERENCE_OPS = (
     "npu_recurrent_gated_delta_rule",
     "npu_chunk_local_cumsum",
     "npu_chunk_scaled_dot_kkt",
+    "npu_chunk_scaled_dot_kkt_inverse",
     "npu_solve_tri",
     "npu_chunk_kda_fwd",
     "npu_chunk_kda_bwd_intra",

@@ -27,6 +27,7 @@ OP_ARGTYPES = {
     "chunk_local_cumsum": [_T, _IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_double, ctypes.c_bool,
                            ctypes.c_char_p, _T],
     "chunk_scaled_dot_kkt": [_T, _T, _T, _IA, _IA, ctypes.c_int64, _T],
+    "chunk_scaled_dot_kkt_inverse": [_T, _T, _T, _IA, _IA, ctypes.c_int64, _T],
     "solve_tri": [_T, _IA, _IA, ctypes.c_char_p, _T],
     "recompute_w_u_fwd": [_T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_int64, _T, _T],
     "chunk_gated_delta_rule_fwd_h": [_T, _T, _T, _T, _T, _T, ctypes.c_bool, ctypes.c_int64, _IA, _IA,
@@ -330,6 +331,24 @@ def npu_chunk_scaled_dot_kkt(k, g, beta, *, cu_seqlens=None, chunk_indices=None,
     out = _empty((B, Hv, T, int(chunk_size)), k_contig, dtype=torch.float32)
     return _call_op(
         "chunk_scaled_dot_kkt", OP_ARGTYPES["chunk_scaled_dot_kkt"],
+        lambda ctx: [
+            ctx.tensor(k_contig, "k"), ctx.tensor(g_contig, "g"), ctx.tensor(beta_contig, "beta"),
+            ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+
+
+def npu_chunk_scaled_dot_kkt_inverse(k, g, beta, *, cu_seqlens=None, chunk_indices=None, chunk_size=64):
+    """``solve_tri(chunk_scaled_dot_kkt(k, g, beta), output_dtype=k.dtype)`` in one launch (no reference counterpart;
+    the backward's recompute calls it).  Returns (I + A)^-1 as [B,Hv,T,64] in k's dtype; 64-token chunks only."""
+    k_contig, g_contig, beta_contig = k.contiguous(), g.contiguous(), beta.contiguous()
+    B, _, T, _ = _shape(k_contig)
+    _, Hv, _ = _shape(g_contig)
+    out = _empty((B, Hv, T, int(chunk_size)), k_contig)
+    return _call_op(
+        "chunk_scaled_dot_kkt_inverse", OP_ARGTYPES["chunk_scaled_dot_kkt_inverse"],
         lambda ctx: [
             ctx.tensor(k_contig, "k"), ctx.tensor(g_contig, "g"), ctx.tensor(beta_contig, "beta"),
             ctx.int_array(cu_seqlens), ctx.int_array(chunk_indices), ctypes.c_int64(int(chunk_size)),

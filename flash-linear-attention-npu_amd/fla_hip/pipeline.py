@@ -83,7 +83,9 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     # head-first VIEWS: every kernel takes the outer strides of its operands, nothing is copied
     gh = g.float().transpose(1, 2)
     bh = beta.float().transpose(1, 2)
-    if A is None:
+    if A is None and chunk_size == 64:
+        A = _ops.chunk_scaled_dot_kkt_inverse(k, gh, bh, chunk_size=chunk_size, **kw)   # the two operators below, fused
+    elif A is None:
         A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
         A = _ops.solve_tri(A, layout="bnsd", output_dtype=k.dtype, **kw)   # rounds A to k.dtype on load
     w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)

@@ -107,6 +107,21 @@ int fla_chunk_scaled_dot_kkt(
     const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * chunk_scaled_dot_kkt_inverse - no counterpart in the reference: the two operators above and below in one
+ * launch, for callers that only want the inverse (the backward's recompute).  Same operands as
+ * chunk_scaled_dot_kkt; out = (I + A)^-1 [B,Hv,T,64] in the element type of k, contiguous; 64-token chunks.
+ * The result equals solve_tri(chunk_scaled_dot_kkt(...)) bit for bit.
+ * ------------------------------------------------------------------------ */
+int fla_chunk_scaled_dot_kkt_inverse_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size,
+    const fla_tensor *out, uint64_t *workspace_size);
+int fla_chunk_scaled_dot_kkt_inverse(
+    const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size,
+    const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
  * solve_tri - replaces aclnnSolveTri (_aclnn_ctypes.py:1786-1800):
  * out = (I + x)^-1 per C x C chunk block, x strictly lower triangular.
  * layout "bnsd": x [B,H,T,C]; "bsnd": x [B,T,H,C]; "tnd" / "ntd" without the batch

@@ -304,3 +304,31 @@ def test_rejects_bad_metadata(dev):
         ops.chunk_scaled_dot_kkt(x["k"], G, x["beta"], chunk_size=32)
     with pytest.raises(RuntimeError, match="either g or gk"):
         ops.chunk_gated_delta_rule_fwd_h(x["k"], x["k"], x["v"])
+
+
+@pytest.mark.parametrize("dtype", [BF, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("shape", [dict(B=2, T=256, Hk=2, Hv=2, K=128), dict(B=1, T=200, Hk=2, Hv=4, K=64),
+                                   dict(B=1, T=261, Hk=1, Hv=2, K=128, cu=[0, 1, 16, 33, 33, 96, 160, 261])],
+                         ids=["dense", "gva-ragged", "packed"])
+def test_kkt_inverse_equals_the_two_operators(dev, shape, dtype):
+    """chunk_scaled_dot_kkt_inverse is chunk_scaled_dot_kkt followed by solve_tri in one launch: same rounding
+    points, same inversion code, so the results are compared for equality (and against the oracle's inverse)."""
+    from fla_hip import ops
+    B, T, Hk, Hv, K = (shape[x] for x in ("B", "T", "Hk", "Hv", "K"))
+    cu = shape.get("cu")
+    gen = torch.Generator().manual_seed(T + K)
+    k = torch.nn.functional.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(dtype)
+    g = gdn.chunk_local_cumsum(torch.nn.functional.logsigmoid(torch.randn(B, Hv, T, generator=gen)), 64, cu_seqlens=cu)
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    kd, gd, bd = k.to(dev), g.to(dev), beta.to(dev)
+    A0 = ops.chunk_scaled_dot_kkt(kd, gd, bd, cu_seqlens=cu, chunk_size=64)
+    two = ops.solve_tri(A0, cu_seqlens=cu, layout="bnsd", output_dtype=dtype)
+    one = ops.chunk_scaled_dot_kkt_inverse(kd, gd, bd, cu_seqlens=cu, chunk_size=64)
+    assert one.dtype == dtype and one.shape == two.shape
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        assert torch.equal(one[b, :, s:e, : e - s], two[b, :, s:e, : e - s]), f"chunk {ci}"
+    ref = gdn.solve_tri(gdn.chunk_scaled_dot_kkt(k, g, beta, 64, cu_seqlens=cu), cu_seqlens=cu)
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        assert_close(one[b, :, s:e, : e - s], ref[b, :, s:e, : e - s], TOL_BF16, f"inverse, chunk {ci}")
+    with pytest.raises(RuntimeError, match="64-token chunks"):
+        ops.chunk_scaled_dot_kkt_inverse(kd, gd, bd, chunk_size=128)
