@@ -434,3 +434,15 @@ def test_recurrent_kda_wrapper_checks_and_operands():
         capture_call(H.npu_recurrent_kda, q, q, v, g, beta, None)
     with pytest.raises(RuntimeError, match="HV must be divisible by H"):
         capture_call(H.npu_recurrent_kda, FakeDevTensor((B, T, 3, K)), FakeDevTensor((B, T, 3, K)), v, g, beta, state, state_v_first=True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build runs on one GPU: bench.py --gpus N > 1 exits with a message instead of timing anything."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
