@@ -96,11 +96,17 @@ def _total_chunks(B: int, T: int, chunk_size: int, cu: Optional[tuple]) -> int:
 
 # ---------------------------------------------------------------------------------------------
 def npu_chunk_fwd_o(q, k, v, h, scale, *, g=None, g_gamma=None, cu_seqlens=None, chunk_indices=None,
-                    chunk_size=None, transpose_state_layout=False):
-    """_aclnn_ctypes.py:517-549.  ``g_gamma`` and ``transpose_state_layout`` are ignored there too."""
+                    chunk_size=None, transpose_state_layout=False, out_token_major=False):
+    """_aclnn_ctypes.py:517-549.  ``g_gamma`` and ``transpose_state_layout`` are ignored there too.
+    ``out_token_major`` (not in the reference): the [B,H,T,V] result is a view of [B,T,H,V] storage, so that the
+    caller's ``o.transpose(1, 2)`` is contiguous without a copy (the kernel takes the strides of its output)."""
     del g_gamma, transpose_state_layout
     chunk_size = _optional_int(chunk_size, 64)
-    out = _empty_like(v)
+    if out_token_major:
+        B, H, T, V = _shape(v)
+        out = _empty((B, T, H, V), v).transpose(1, 2)
+    else:
+        out = _empty_like(v)
     return _call_op(
         "chunk_fwd_o", OP_ARGTYPES["chunk_fwd_o"],
         lambda ctx: [

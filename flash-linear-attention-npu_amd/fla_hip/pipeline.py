@@ -64,7 +64,7 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
     h, v_new, final = _ops.chunk_gated_delta_rule_fwd_h(
         k, w, u, g=gh, initial_state=initial_state, output_final_state=output_final_state,
         chunk_size=chunk_size, cu_seqlens=cu)
-    o = _ops.chunk_fwd_o(q, k, v_new, h, scale, g=gh, cu_seqlens=cu, chunk_size=chunk_size)
+    o = _ops.chunk_fwd_o(q, k, v_new, h, scale, g=gh, cu_seqlens=cu, chunk_size=chunk_size, out_token_major=True)
     return gh.transpose(1, 2).contiguous(), o.transpose(1, 2).contiguous(), A, \
         (final if output_final_state else None)
 
