@@ -262,3 +262,36 @@ def test_chunk_kda_fwd_dual_benchmark(dev):
     for name, dut, c, truth in (("o", from_layout(out[0], "BSND"), ctrl["o"].to(BF), t_o), ("final_state", out[1], ctrl["final_state"], t_f)):
         a, cc = stats(dut, truth), stats(c, truth)
         assert a[0] <= 5 * cc[0] + 1e-6 and a[1] <= 1.5 * cc[1] + 1e-7 and a[2] <= 1.5 * cc[2] + 1e-9, (name, a, cc)
+
+
+def test_chunk_kda_fwd_bench_shape_properties(dev):
+    """B=2 T=8192 H=32 K=V=128, too large for the CPU oracle: the result must not depend on the chunk size (64 against
+    128 tokens), a sequence cut at a chunk boundary with the state handed over must equal the uncut run, and the
+    oracle's per-token recurrence is checked on one (batch row, head) slice."""
+    from fla_hip import ops
+    B, T, H, K, V = 2, 8192, 32, 128, 128
+    gen = torch.Generator(device=dev).manual_seed(3)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
+    q = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1).to(BF)
+    k = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1).to(BF)
+    v = rn(B, T, H, V).to(BF)
+    g = torch.nn.functional.logsigmoid(rn(B, T, H, K)) * 0.3
+    beta = torch.sigmoid(rn(B, T, H))
+    h0 = rn(B, H, K, V) * 0.05
+    scale = K ** -0.5
+    o64, f64 = ops.chunk_kda_fwd(q, k, v, g, beta, scale, 64, initial_state=h0, output_final_state=True)[:2]
+    o128, f128 = ops.chunk_kda_fwd(q, k, v, g, beta, scale, 128, initial_state=h0, output_final_state=True)[:2]
+    assert_close(o128, o64, TOL_BF16, "o: 128- against 64-token chunks")
+    assert_close(f128, f64, 8 * TOL_STATE, "final state: 128- against 64-token chunks")
+    cut = 4096 + 128
+    a = [x[:, :cut].contiguous() for x in (q, k, v, g, beta)]
+    b = [x[:, cut:].contiguous() for x in (q, k, v, g, beta)]
+    o1, f1 = ops.chunk_kda_fwd(*a, scale, 128, initial_state=h0, output_final_state=True)[:2]
+    o2, f2 = ops.chunk_kda_fwd(*b, scale, 128, initial_state=f1, output_final_state=True)[:2]
+    assert torch.equal(torch.cat([o1, o2], dim=1), o128) and torch.equal(f2, f128)
+    # one slice against the per-token recurrence on the CPU
+    bi, hi, Ts = 1, 17, 1024
+    sl = lambda x: x[bi:bi + 1, :Ts, hi:hi + 1].transpose(1, 2).float().cpu()
+    o_ref, _ = kda.naive_recurrent_kda(sl(q), sl(k), sl(v), sl(g), beta[bi:bi + 1, :Ts, hi:hi + 1].transpose(1, 2).cpu(), scale,
+                                       initial_state=h0[bi:bi + 1, hi:hi + 1].cpu(), output_final_state=True)
+    assert_close(o128[bi:bi + 1, :Ts, hi:hi + 1].transpose(1, 2), o_ref, TOL_BF16, "o slice vs recurrence")
