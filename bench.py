@@ -506,6 +506,15 @@ def bench_gdn_bwd(args, torch, dev):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
+    # the same step when the forward kept its inverted chunk matrices (the six-operator forward does, as the
+    # reference's forward does; the fused forward keeps none, which is the case timed above)
+    A_saved = fla_hip.ops.chunk_scaled_dot_kkt_inverse(k, G.transpose(1, 2), beta.transpose(1, 2), chunk_size=C)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        pipeline.flash_chunk_gated_delta_rule_bwd(q, k, v, G, beta, A_saved, scale, h0, do, dht, chunk_size=C)
+    torch.cuda.synchronize()
+    ms_saved_A = (time.perf_counter() - t0) * 1e3 / args.steps
     lib.fla_profile_enable.argtypes = [ctypes.c_int]
     lib.fla_profile_enable(1)
     for _ in range(args.steps):
@@ -550,7 +559,9 @@ def bench_gdn_bwd(args, torch, dev):
         "metric": "gdn_chunk_bwd_tokens_per_s", "value": round(B * T * args.steps / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "GDN chunk backward B=4 T=8192 H=32 K=V=128 chunk=64, initial state and final-state gradient"},
+        "config": {"workload": "GDN chunk backward B=4 T=8192 H=32 K=V=128 chunk=64, initial state and final-state gradient, "
+                               "A recomputed from k, g, beta"},
+        "ms_per_step_with_saved_A": round(ms_saved_A, 4),
         "step_tflops": round(step_flops / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
