@@ -13,7 +13,7 @@ import functools
 import inspect
 from typing import Callable
 
-from ._hip_ctypes import HIP_CTYPES_OPS, gdn_chunk_fwd, l2norm_bwd, l2norm_fwd
+from ._hip_ctypes import HIP_CTYPES_OPS, chunk_kda_fwd_noalloc, gdn_chunk_fwd, l2norm_bwd, l2norm_fwd
 
 _REFERENCE_OPS = (
     "npu_fast_gelu_custom",
@@ -153,6 +153,7 @@ def causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=Non
 
 __all__ = [
     "MUTATED_ARGUMENTS",
+    "chunk_kda_fwd_noalloc",
     "gdn_chunk_fwd",
     "l2norm_bwd",
     "l2norm_fwd",

@@ -529,6 +529,27 @@ def npu_chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", 
     """KDA chunk forward (_aclnn_ctypes.py:1066-1265).  Returns the 12-tuple
     ``(o, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, initial_state)``; entries the output policy
     hides are ``None``."""
+    return _chunk_kda_fwd(False, q, k, v, g, beta, scale, chunk_size, layout, initial_state, output_final_state,
+                          cu_seqlens, chunk_indices, safe_gate, lower_bound, use_gate_in_kernel, A_log, dt_bias,
+                          disable_recompute, return_intermediate_states, state_v_first)
+
+
+def chunk_kda_fwd_noalloc(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", initial_state=None,
+                          output_final_state=False, safe_gate=False, lower_bound=None, use_gate_in_kernel=False,
+                          A_log=None, dt_bias=None, disable_recompute=False, return_intermediate_states=False,
+                          state_v_first=False):
+    """``npu_chunk_kda_fwd`` through ``fla_chunk_kda_fwd_noalloc``: the library call allocates nothing and takes
+    no workspace (its scratch is a fixed array of 32 MiB per GPU; dense batches only).  This wrapper still
+    allocates the OUTPUT tensors with torch, as every wrapper here does; a caller that must not allocate at all
+    binds the C entry point with preallocated outputs.  Calls that overlap on one GPU race on the scratch array."""
+    return _chunk_kda_fwd(True, q, k, v, g, beta, scale, chunk_size, layout, initial_state, output_final_state,
+                          None, None, safe_gate, lower_bound, use_gate_in_kernel, A_log, dt_bias,
+                          disable_recompute, return_intermediate_states, state_v_first)
+
+
+def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial_state, output_final_state, cu_seqlens,
+                   chunk_indices, safe_gate, lower_bound, use_gate_in_kernel, A_log, dt_bias, disable_recompute,
+                   return_intermediate_states, state_v_first):
     import torch
 
     op = "npu_chunk_kda_fwd"
@@ -618,8 +639,8 @@ def npu_chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", 
     h = _empty((*lead, NT, HV, *block), q) if mask[10] else None
     outputs = (attn_out, final_state, gk, aqk, akk, w, u, qg, kg, v_new, h)
     names = ("attn_out", "final_state", "gk", "Aqk", "Akk", "w", "u", "qg", "kg", "v_new", "h")
-    _call_op(
-        "chunk_kda_fwd", OP_ARGTYPES["chunk_kda_fwd"],
+    (_runtime.call_op_noalloc if noalloc else _call_op)(
+        "chunk_kda_fwd_noalloc" if noalloc else "chunk_kda_fwd", OP_ARGTYPES["chunk_kda_fwd"],
         lambda ctx: [
             ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"), ctx.tensor(beta, "beta"),
             ctx.tensor(A_log, "A_log"), ctx.tensor(dt_bias, "dt_bias"), ctx.tensor(initial_state, "initial_state"),

@@ -199,3 +199,29 @@ def call_op(name: str, argtypes: Sequence, build_args: Callable[[CallContext], l
             raise RuntimeError(f"fla_{name} failed with status={status}: {last_error()}")
         del workspace  # stream-ordered reuse by the caching allocator keeps this safe
     return outputs
+
+
+def call_op_noalloc(name: str, argtypes: Sequence, build_args: Callable[[CallContext], list], outputs):
+    """One-phase call of ``fla_<name>(<operands>, stream)``: an entry point that brings its own scratch memory.
+    Nothing is allocated here or inside the library; the caller has allocated ``outputs``."""
+    import torch
+
+    anchor = _first_tensor(outputs)
+    if anchor is None:
+        raise RuntimeError(f"fla_{name}: no output tensor to take the device from.")
+    ensure_gpu_tensor(anchor, "output")
+    device = anchor.device
+    launch = _BOUND.get(name)
+    if launch is None:
+        launch = getattr(_library(), f"fla_{name}")
+        launch.argtypes = [*argtypes, ctypes.c_void_p]
+        launch.restype = ctypes.c_int
+        _BOUND[name] = launch
+    with torch.cuda.device(device):
+        ctx = CallContext(device)
+        args = build_args(ctx)
+        stream = ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+        status = launch(*args, stream)
+        if status != FLA_OK:
+            raise RuntimeError(f"fla_{name} failed with status={status}: {last_error()}")
+    return outputs

@@ -333,6 +333,30 @@ int fla_chunk_kda_fwd(
     void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * chunk_kda_fwd_noalloc - no counterpart in the reference.  For callers that cannot allocate
+ * device memory around a call (code under HIP stream capture, serving loops and harnesses that
+ * forbid hipMalloc): fla_chunk_kda_fwd with the same operands and results, minus the workspace
+ * pair.  The per-chunk decay rows and whichever of w, u, qg, kg the caller passes as NULL live
+ * in a fixed array of FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES in device memory, one per GPU,
+ * held until the process ends.  A call whose scratch need exceeds the array returns
+ * FLA_ERR_WORKSPACE (with w, u, qg, kg supplied the need is B*NT*HV*K*4 bytes); cu_seqlens and
+ * chunk_indices must be NULL (FLA_ERR_UNSUPPORTED otherwise).  The call performs no hipMalloc /
+ * hipFree / hipHostMalloc.  All calls on one GPU share the array: calls that may overlap in time
+ * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ * ------------------------------------------------------------------------ */
+#define FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fla_chunk_kda_fwd_noalloc(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const char *layout, double scale, int64_t chunk_size,
+    bool safe_gate, double lower_bound, bool use_gate_in_kernel, bool state_v_first,
+    const fla_tensor *attn_out, const fla_tensor *final_state, const fla_tensor *gk,
+    const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w, const fla_tensor *u,
+    const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
+    void *stream);
+
+/* ------------------------------------------------------------------------
  * chunk_kda_bwd_intra - replaces aclnnChunkKdaBwdIntra
  * (_aclnn_ctypes.py:1534-1768; golden test_npu_chunk_kda_bwd_intra.py:7-91).
  * layout "BSND", "BNSD" (dense) or "TND" (needs cu_seqlens).  q,k bf16 [..,K];
