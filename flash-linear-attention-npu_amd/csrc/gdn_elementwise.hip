@@ -106,6 +106,7 @@ struct CumsumParams {
     int feat;      // trailing feature extent (1 for [B,H,T])
     int reverse;
     float scale;
+    int64_t i_sb, i_sh, i_st, o_sb, o_sh, o_st;   // (batch, head, token) strides of g and out, in elements
 };
 
 // [B,H,T]: one wave per (chunk, head, batch row); lanes scan 64 tokens at a time.
@@ -121,15 +122,16 @@ __global__ void __launch_bounds__(64) cumsum_tokens_kernel(const CumsumParams p)
         start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * p.chunk;
         len = min(p.chunk, p.geom.cu[seq + 1] - start);
     }
-    const int64_t base = ((int64_t)b * p.geom.Hv + h) * p.geom.T + start;
+    const int64_t ibase = b * p.i_sb + h * p.i_sh + (int64_t)start * p.i_st;
+    const int64_t obase = b * p.o_sb + h * p.o_sh + (int64_t)start * p.o_st;
     const int lane = threadIdx.x;
     float carry = 0.f;
     for (int off = 0; off < len; off += kWave) {
         const int j = off + lane;
         const int t = p.reverse ? len - 1 - j : j;
-        float v = j < len ? ld<TI>(p.g, base + t) : 0.f;
+        float v = j < len ? ld<TI>(p.g, ibase + (int64_t)t * p.i_st) : 0.f;
         v = wave_inclusive_scan(v) + carry;
-        if (j < len) st<TO>(p.out, base + t, v * p.scale);
+        if (j < len) st<TO>(p.out, obase + (int64_t)t * p.o_st, v * p.scale);
         carry = __shfl(v, kWave - 1, kWave);
     }
 }
@@ -147,13 +149,14 @@ __global__ void cumsum_features_kernel(const CumsumParams p) {
         start = p.geom.cu[seq] + p.geom.tab[2 * c + 1] * p.chunk;
         len = min(p.chunk, p.geom.cu[seq + 1] - start);
     }
-    const int64_t base = (((int64_t)b * p.geom.Hv + h) * p.geom.T + start) * p.feat;
+    const int64_t ibase = b * p.i_sb + h * p.i_sh + (int64_t)start * p.i_st;
+    const int64_t obase = b * p.o_sb + h * p.o_sh + (int64_t)start * p.o_st;
     for (int f = threadIdx.x; f < p.feat; f += blockDim.x) {
         float acc = 0.f;
         for (int j = 0; j < len; ++j) {
             const int t = p.reverse ? len - 1 - j : j;
-            acc += ld<TI>(p.g, base + (int64_t)t * p.feat + f);
-            st<TO>(p.out, base + (int64_t)t * p.feat + f, acc * p.scale);
+            acc += ld<TI>(p.g, ibase + (int64_t)t * p.i_st + f);
+            st<TO>(p.out, obase + (int64_t)t * p.o_st + f, acc * p.scale);
         }
     }
 }
@@ -180,7 +183,10 @@ int cumsum_impl(const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_
     FLA_REQUIRE(head_first, FLA_ERR_UNSUPPORTED, "%s: head_first must be true ([B,H,T] layout).", op);
     FLA_REQUIRE(g->ndim == 3 || g->ndim == 4, FLA_ERR_SHAPE, "%s: g must be [B,H,T] or [B,H,T,K].", op);
     FLA_REQUIRE(same_shape(g, out), FLA_ERR_SHAPE, "%s: out must have the shape of g.", op);
-    FLA_REQUIRE(is_contiguous(g) && is_contiguous(out), FLA_ERR_SHAPE, "%s: g and out must be contiguous.", op);
+    // [B,H,T] and [B,H,T,K] are index orders: any strides are taken (a [B,T,H,..] tensor is passed as its transposed
+    // view); only the feature dimension of a rank-4 operand must be dense
+    FLA_REQUIRE(g->ndim == 3 || (inner_unit(g) && inner_unit(out)), FLA_ERR_SHAPE,
+                "%s: the innermost stride of a rank-4 g / out must be 1.", op);
     FLA_REQUIRE(chunk_size > 0 && (chunk_size & (chunk_size - 1)) == 0, FLA_ERR_SHAPE,
                 "%s: chunk_size must be a power of 2, got %lld.", op, (long long)chunk_size);
     if (output_dtype != nullptr) {
@@ -223,6 +229,8 @@ int cumsum_impl(const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_
     p.feat = (int)F;
     p.reverse = reverse ? 1 : 0;
     p.scale = (float)scale;
+    p.i_sb = g->stride[0]; p.i_sh = g->stride[1]; p.i_st = g->stride[2];
+    p.o_sb = out->stride[0]; p.o_sh = out->stride[1]; p.o_st = out->stride[2];
     if (p.geom.NT == 0 || B == 0 || H == 0) return FLA_OK;
 
 #define FLA_CS(TI, TO) launch_cumsum<TI, TO>(p, stream)

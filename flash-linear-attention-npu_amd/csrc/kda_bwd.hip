@@ -1,0 +1,624 @@
+// Chunk-parallel stages of the KDA (per-channel gated delta rule) BACKWARD around the reverse scan
+// (chunk_gated_delta_rule_bwd_dhu with gK) and chunk_kda_bwd_intra:
+//   chunk_kda_bwd_dav     dAqk = scale tril(do v_new^T),  dv = Aqk^T do
+//   chunk_kda_bwd_dqkwg   dq, dk, dw and the gate gradient of the state-dependent parts of a chunk step
+//   chunk_kda_bwd_wy      backward of  w = Akk (k beta 2^g),  u = Akk (v beta),  Akk = (I + M)^-1
+// The reference has no kernels for these stages: its deployment leaves them to a third-party Triton package
+// (torch_custom/fla_npu/fla_npu/adapters/triton_ascend_kda.py:1-8); the forward they differentiate is
+// tests/atk/chunk_kda_fwd/executor_chunk_kda_fwd.py:459-484.  g is the chunk-local cumulated gate in log2
+// units; "dg" is the gradient with respect to ln 2 * g, the convention of chunk_kda_bwd_intra
+// (torch_custom/fla_npu/test/test_npu_chunk_kda_bwd_intra.py:7-91), so the stages add into one tensor.
+// One workgroup per (chunk, value head); bf16 MFMA with fp32 accumulation; wave w owns token rows 16w..16w+15.
+// dq, dk, dg are fp32 and per VALUE head (the gate is per value head); grouped heads are summed by the caller.
+#include "gdn_common.h"
+#include "mfma_tiles.h"
+
+namespace fla {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ f32x4 zero4() { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// fp32 [B,H,T,D] through strides, unit innermost stride
+struct ViewF {
+    float *p;
+    int64_t sb, sh, st;
+};
+inline ViewF viewf(const fla_tensor *t) { return ViewF{static_cast<float *>(t->data), t->stride[0], t->stride[1], t->stride[2]}; }
+
+// =============================================================================
+// chunk_kda_bwd_dav
+// =============================================================================
+struct DavParams {
+    ChunkGeom geom;
+    View4 v_new, d_o, aqk, dv;
+    ViewF daqk;
+    float scale;
+};
+
+template <int V>
+__global__ void __launch_bounds__(kThreads) kda_bwd_dav_kernel(const DavParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int po = V + 16, pv = V + 8, pa = kChunk + 16;
+    elem *oS = reinterpret_cast<elem *>(smem);      // do: rows contracted over V (dAqk) and over tokens (dv)
+    elem *vS = oS + kChunk * po;                    // v_new
+    elem *aS = vS + kChunk * pv;                    // Aqk
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    {
+        TileCopy<kThreads, kChunk, V> to, tv;
+        TileCopy<kThreads, kChunk, kChunk> ta;
+        to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        tv.fetch(static_cast<const elem *>(p.v_new.p) + b * p.v_new.sb + hv * p.v_new.sh + (int64_t)start * p.v_new.st, p.v_new.st, len, tid);
+        ta.fetch(static_cast<const elem *>(p.aqk.p) + b * p.aqk.sb + hv * p.aqk.sh + (int64_t)start * p.aqk.st, p.aqk.st, len, tid);
+        to.commit(oS, po, len, tid);
+        tv.commit(vS, pv, len, tid);
+        ta.commit(aS, pa, len, tid);
+    }
+    __syncthreads();
+    // dAqk[i][j] = scale <do_i, v_new_j> for j <= i: row tile w, column tiles 0..w
+    float *dag = p.daqk.p + b * p.daqk.sb + hv * p.daqk.sh + (int64_t)start * p.daqk.st;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct <= w) {
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(oS, po, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+        }
+        const int col = 16 * ct + li;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            if (row < len) dag[(int64_t)row * p.daqk.st + col] = (ct <= w && col <= row) ? acc[e] * p.scale : 0.f;
+        }
+    }
+    // dv_j = sum_{i >= j} Aqk[i][j] do_i
+    char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                         (int64_t)start * p.dv.st);
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) {
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (32 * j + 31 >= 16 * w) acc = mfma16x32(frag_tr(aS, pa, 16 * w, 32 * j), frag_tr(oS, po, 16 * ct, 32 * j), acc);
+        acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+    }
+}
+
+// =============================================================================
+// chunk_kda_bwd_dqkwg
+// =============================================================================
+constexpr int kDqkwgThreads = 512;   // two waves per SIMD over one set of LDS tiles
+struct KdaDqkwgParams {
+    ChunkGeom geom;
+    View4 q, k, v, d_o, dv, dw;
+    const float *gk;
+    int64_t g_sb, g_sh, g_st;
+    const elem *h, *dh;
+    int64_t h_sb, h_sh, h_sc, dh_sb, dh_sh, dh_sc;
+    ViewF dq, dk, dg;
+    float scale;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaDqkwgParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pv = V + 8;
+    constexpr int KT = K / 16, KTH = KT / 2;   // column tiles of the K-sized outputs: all, and per wave
+    constexpr int CPR = V / 8;                 // 16-byte pieces per state row
+    elem *vS = reinterpret_cast<elem *>(smem);  // v_new
+    elem *oS = vS + kChunk * pv;                // do
+    elem *dvS = oS + kChunk * pv;               // total dv_new
+    elem *hS = dvS + kChunk * pv;               // h, then dh
+    float *hdS = reinterpret_cast<float *>(hS + K * pv);   // [K]    sum_v h . dh per state row
+    float *colS = hdS + K;                                  // [4][K] per row tile: sum_j k_j dk_j
+    float *exS = colS + 4 * K;                              // [K]    what lands on the chunk's last token
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    // eight waves: wave (w, half) owns token rows 16w.. and column tiles half*KTH .. half*KTH+KTH-1
+    const int tid = threadIdx.x, w = wave_id() & 3, half = wave_id() >> 2, l = lane_id(), li = l & 15, lg = l >> 4;
+
+    // element-wise operands in the accumulator layout, requested first and consumed in the epilogue
+    // (rows past the tail repeat the last valid row)
+    float qv[KTH][4], kv[KTH][4], gv[KTH][4], glast[KTH];
+    {
+        const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
+        const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+        const float *gg = p.gk + b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st;
+#pragma unroll
+        for (int ct = 0; ct < KTH; ++ct) {
+            const int col = 16 * (half * KTH + ct) + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = min(16 * w + 4 * lg + e, len - 1);
+                qv[ct][e] = (float)qg[(int64_t)row * p.q.st + col];
+                kv[ct][e] = (float)kg[(int64_t)row * p.k.st + col];
+                gv[ct][e] = gg[(int64_t)row * p.g_st + col];
+            }
+            glast[ct] = gg[(int64_t)(len - 1) * p.g_st + col];
+        }
+    }
+    TileCopy<kDqkwgThreads, K, V> tdh;
+    {
+        TileCopy<kDqkwgThreads, kChunk, V> tv, to, tdv;
+        TileCopy<kDqkwgThreads, K, V> th;
+        tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+        to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+        th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
+        tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
+        tv.commit(vS, pv, len, tid);
+        to.commit(oS, pv, len, tid);
+        tdv.commit(dvS, pv, len, tid);
+        th.commit(hS, pv, K, tid);
+        // sum_v h[k][v] dh[k][v]: the CPR threads that hold the pieces of one state row add their shares
+#pragma unroll
+        for (int m = 0; m < TileCopy<kDqkwgThreads, K, V>::N; ++m) {
+            const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)d[e];
+            s = group_sum<CPR>(s);
+            const int idx = m * kDqkwgThreads + tid;
+            if (idx % CPR == 0) hdS[idx / CPR] = s;
+        }
+    }
+    __syncthreads();
+    // ---- products with the state at chunk start: dq (do h^T) and dw (-dv h^T) ---------------------
+    f32x4 dqa[KTH], dka[KTH];
+    char *dwg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
+                                         (int64_t)start * p.dw.st);
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int cg = half * KTH + ct;
+        f32x4 a = zero4(), d = zero4();
+#pragma unroll
+        for (int j = 0; j < V / 32; ++j) {
+            const elemx8 hf = frag_kc(hS, pv, 16 * cg, 32 * j);
+            a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
+            d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
+        }
+        dqa[ct] = a;
+        acc_to_global(dwg + 32 * cg, p.dw.st * 2, 16 * w, len, -d);
+    }
+    __syncthreads();                 // every wave is done with h
+    tdh.commit(hS, pv, K, tid);
+    __syncthreads();
+    // ---- product with the state gradient: dk (v_new dh^T); gate factors; column sums of k . dk -----
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int cg = half * KTH + ct;
+        f32x4 d = zero4();
+#pragma unroll
+        for (int j = 0; j < V / 32; ++j) d = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * cg, 32 * j), d);
+        float colsum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            dqa[ct][e] *= p.scale * ex2(gv[ct][e]);
+            d[e] *= ex2(glast[ct] - gv[ct][e]);
+            colsum += row < len ? kv[ct][e] * d[e] : 0.f;
+        }
+        dka[ct] = d;
+        colsum += __shfl_xor(colsum, 16, kWave);
+        colsum += __shfl_xor(colsum, 32, kWave);
+        if (lg == 0) colS[w * K + 16 * cg + li] = colsum;
+    }
+    __syncthreads();
+    if (tid < K) {
+        const float gl = p.gk[b * p.g_sb + hv * p.g_sh + (int64_t)(start + len - 1) * p.g_st + tid];
+        exS[tid] = colS[tid] + colS[K + tid] + colS[2 * K + tid] + colS[3 * K + tid] + ex2(gl) * hdS[tid];
+    }
+    __syncthreads();
+    float *dqg = p.dq.p + b * p.dq.sb + hv * p.dq.sh + (int64_t)start * p.dq.st;
+    float *dkg = p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st;
+    float *dgg = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int col = 16 * (half * KTH + ct) + li;
+        const float extra = exS[col];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            if (row < len) {
+                dqg[(int64_t)row * p.dq.st + col] = dqa[ct][e];
+                dkg[(int64_t)row * p.dk.st + col] = dka[ct][e];
+                dgg[(int64_t)row * p.dg.st + col] =
+                    qv[ct][e] * dqa[ct][e] - kv[ct][e] * dka[ct][e] + (row == len - 1 ? extra : 0.f);
+            }
+        }
+    }
+}
+
+// =============================================================================
+// chunk_kda_bwd_wy
+// =============================================================================
+struct KdaWyParams {
+    ChunkGeom geom;
+    View4 k, v, akk, dw, du, dv;
+    View3 beta;
+    const float *gk;
+    int64_t g_sb, g_sh, g_st;
+    ViewF dk, dg, dakk;         // dk and dg are added to
+    float *db;
+    int64_t db_sb, db_sh, db_st;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads, 2) kda_bwd_wy_kernel(const KdaWyParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pw = K + 16, pu = V + 16, pk = K + 8, pv = V + 8, pa = kChunk + 8;
+    constexpr int KT = K / 16, VT = V / 16;
+    elem *dwS = reinterpret_cast<elem *>(smem);   // contracted over K (dA) and over tokens (Akk^T dw)
+    elem *duS = dwS + kChunk * pw;
+    elem *kgS = duS + kChunk * pu;                // k 2^g
+    elem *vS = kgS + kChunk * pk;
+    elem *aS = vS + kChunk * pv;                  // Akk
+    float *bS = reinterpret_cast<float *>(aS + kChunk * pa);
+    // the two 64 x 64 intermediates of the chain through the inverse reuse the dw and du tiles once those are dead
+    elem *m4S = dwS;
+    elem *m5S = duS;
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const float *gg = p.gk + b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st;
+    {
+        TileCopy<kThreads, kChunk, K> tdw, tk;
+        TileCopy<kThreads, kChunk, V> tdu, tv;
+        TileCopy<kThreads, kChunk, kChunk> ta;
+        tdw.fetch(static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+        tk.fetch(kg, p.k.st, len, tid);
+        tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
+        tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+        ta.fetch(static_cast<const elem *>(p.akk.p) + b * p.akk.sb + hv * p.akk.sh + (int64_t)start * p.akk.st, p.akk.st, len, tid);
+        // gate pieces that match the k pieces of this thread
+        constexpr int NK = TileCopy<kThreads, kChunk, K>::N;
+        f32x4 g0[NK], g1[NK];
+#pragma unroll
+        for (int m = 0; m < NK; ++m) {
+            const int idx = m * kThreads + tid;
+            const int r = min(idx / (K / 8), len - 1), c8 = (idx % (K / 8)) << 3;
+            g0[m] = *reinterpret_cast<const f32x4 *>(gg + (int64_t)r * p.g_st + c8);
+            g1[m] = *reinterpret_cast<const f32x4 *>(gg + (int64_t)r * p.g_st + c8 + 4);
+        }
+        if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
+        tdw.commit(dwS, pw, len, tid);
+        tdu.commit(duS, pu, len, tid);
+        tv.commit(vS, pv, len, tid);
+        ta.commit(aS, pa, len, tid);
+#pragma unroll
+        for (int m = 0; m < NK; ++m) {
+            const int idx = m * kThreads + tid;
+            const int r = idx / (K / 8), c8 = (idx % (K / 8)) << 3;
+            const elemx8 a = __builtin_bit_cast(elemx8, tk.r[m]);
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = r < len ? (float)a[e] * ex2(g0[m][e]) : 0.f;
+                hi[e] = r < len ? (float)a[4 + e] * ex2(g1[m][e]) : 0.f;
+            }
+            *reinterpret_cast<elemx8 *>(kgS + r * pk + c8) = frag_from_acc(lo, hi);
+        }
+    }
+    __syncthreads();
+    // ---- dA = strict_lower((dw (k 2^g)^T + du v^T) beta_col), row tile w --------------------------
+    f32x4 m4[4];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct <= w) {
+#pragma unroll
+            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pw, 16 * w, 32 * j), frag_kc(kgS, pk, 16 * ct, 32 * j), acc);
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(duS, pu, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+            const int col = 16 * ct + li;
+            const float bc = bS[col];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                acc[e] = (col < row && row < len) ? acc[e] * bc : 0.f;
+            }
+        }
+        m4[ct] = acc;
+    }
+    // ---- x = Akk^T dw, y = Akk^T du and everything element-wise in them ----------------------------
+    float br[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) br[e] = bS[16 * w + 4 * lg + e];
+    float db_row[4] = {0.f, 0.f, 0.f, 0.f};
+    const elemx8 at0 = frag_tr(aS, pa, 16 * w, 0), at1 = frag_tr(aS, pa, 16 * w, 32);
+    char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                         (int64_t)start * p.dv.st);
+#pragma unroll
+    for (int ct = 0; ct < VT; ++ct) {
+        f32x4 acc = mfma16x32(at0, frag_tr(duS, pu, 16 * ct, 0), zero4());
+        acc = mfma16x32(at1, frag_tr(duS, pu, 16 * ct, 32), acc);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pv + 16 * ct + li];
+            acc[e] *= br[e];
+        }
+        acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+    }
+    float *dkg = p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st;
+    float *dgg = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+#pragma unroll
+    for (int ct = 0; ct < KT; ++ct) {
+        const int col = 16 * ct + li;
+        // this tile's k, gate and incoming dk / dg: requested before the products, consumed after them
+        float kv[4], gv[4], pdk[4], pdg[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = min(16 * w + 4 * lg + e, len - 1);
+            kv[e] = (float)kg[(int64_t)row * p.k.st + col];
+            gv[e] = gg[(int64_t)row * p.g_st + col];
+            pdk[e] = dkg[(int64_t)row * p.dk.st + col];
+            pdg[e] = dgg[(int64_t)row * p.dg.st + col];
+        }
+        f32x4 x = mfma16x32(at0, frag_tr(dwS, pw, 16 * ct, 0), zero4());
+        x = mfma16x32(at1, frag_tr(dwS, pw, 16 * ct, 32), x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            const float xe = x[e] * ex2(gv[e]);      // x 2^g
+            const float dk = xe * br[e];
+            db_row[e] += xe * kv[e];
+            if (row < len) {
+                dkg[(int64_t)row * p.dk.st + col] = pdk[e] + dk;
+                dgg[(int64_t)row * p.dg.st + col] = pdg[e] + dk * kv[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float s = group_sum<16>(db_row[e]);
+        const int row = 16 * w + 4 * lg + e;
+        if (li == 0 && row < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + row) * p.db_st] = s;
+    }
+    __syncthreads();   // every wave has read its dw / du rows and columns: their tiles may be overwritten
+    // ---- dM = -strict_lower(Akk^T dA Akk^T) ----------------------------------------------------
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) acc_to_tile(m4S, pa, 16 * w, 16 * ct, m4[ct]);
+    __syncthreads();
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {   // M5 = dA Akk^T
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_kc(m4S, pa, 16 * w, 32 * j), frag_kc(aS, pa, 16 * ct, 32 * j), acc);
+        acc_to_tile(m5S, pa, 16 * w, 16 * ct, acc);
+    }
+    __syncthreads();
+    float *dag = p.dakk.p + b * p.dakk.sb + hv * p.dakk.sh + (int64_t)start * p.dakk.st;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 acc = zero4();
+        if (ct <= w) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (32 * j + 31 >= 16 * w) acc = mfma16x32(frag_tr(aS, pa, 16 * w, 32 * j), frag_tr(m5S, pa, 16 * ct, 32 * j), acc);
+        }
+        const int col = 16 * ct + li;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            if (row < len) dag[(int64_t)row * p.dakk.st + col] = (ct <= w && col < row) ? -acc[e] : 0.f;
+        }
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+#define FLA_KDA_BWD_LAUNCH(KERNEL, NAME, GRID, SMEM_EXPR, P, THREADS)                                                     \
+    do {                                                                                                               \
+        const size_t smem__ = (SMEM_EXPR);                                                                             \
+        FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                          (int)smem__));                                                               \
+        FLA_LAUNCH(NAME, stream, KERNEL, GRID, dim3(THREADS), smem__, stream, P);                                       \
+        FLA_HIP_CHECK(hipGetLastError());                                                                              \
+        return FLA_OK;                                                                                                 \
+    } while (0)
+
+// fp32 [B,H,T,D] with unit innermost stride and 16-byte aligned rows
+int check_f32_bhtd(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, int64_t D) {
+    int rc = check_tensor(t, op, name, 4, dt_bit(FLA_F32));
+    if (rc) return rc;
+    FLA_REQUIRE(t->shape[0] == B && t->shape[1] == H && t->shape[2] == T && t->shape[3] == D, FLA_ERR_SHAPE,
+                "%s: %s must be [%lld,%lld,%lld,%lld].", op, name, (long long)B, (long long)H, (long long)T, (long long)D);
+    FLA_REQUIRE(inner_unit(t) && t->stride[0] % 4 == 0 && t->stride[1] % 4 == 0 && t->stride[2] % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(t->data) % 16 == 0,
+                FLA_ERR_SHAPE, "%s: %s needs a unit innermost stride and 16-byte aligned rows.", op, name);
+    FLA_REQUIRE(t->stride[2] >= 0, FLA_ERR_SHAPE, "%s: %s has a negative token stride.", op, name);
+    return FLA_OK;
+}
+
+int check_state_blocks(const char *op, const char *name, const fla_tensor *h, const ChunkGeom &geom) {
+    int rc = check_tensor(h, op, name, 5, dt_bit(kElemDtype));
+    if (rc) return rc;
+    FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
+                    h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 8 == 0 &&
+                    h->stride[1] % 8 == 0 && h->stride[0] % 8 == 0 && reinterpret_cast<uintptr_t>(h->data) % 16 == 0,
+                FLA_ERR_SHAPE, "%s: %s must be [B,Hv,NT=%d,K,V] (any outer strides) with contiguous K x V blocks.", op, name,
+                geom.NT);
+    return FLA_OK;
+}
+
+int dav_impl(const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *aqk, const fla_int_array *cu,
+             const fla_int_array *ci, double scale, int64_t chunk_size, const fla_tensor *daqk, const fla_tensor *dv, void *ws,
+             uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_kda_bwd_dav";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, v_new, nullptr, nullptr, chunk_size, geom, kElemDtype))) return rc;   // Hk=Hv, K=V here
+    const int bf = dt_bit(kElemDtype);
+    const int64_t B = geom.B, H = geom.Hv, T = geom.T, V = geom.V;
+    if ((rc = check_bhtd(op, "v_new", v_new, B, H, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, B, H, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "Aqk", aqk, B, H, T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, B, H, T, V, bf))) return rc;
+    if ((rc = check_f32_bhtd(op, "dAqk", daqk, B, H, T, kChunk))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    DavParams p{geom, view4(v_new), view4(d_o), view4(aqk), view4(dv), viewf(daqk), (float)scale};
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const size_t smem = ((size_t)kChunk * ((V + 16) + (V + 8) + (kChunk + 16))) * 2;
+    if (V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dav_kernel<128>), "kda_bwd_dav", grid, smem, p, kThreads);
+    if (V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dav_kernel<64>), "kda_bwd_dav", grid, smem, p, kThreads);
+    if (V == 256) FLA_KDA_BWD_LAUNCH((kda_bwd_dav_kernel<256>), "kda_bwd_dav", grid, smem, p, kThreads);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: V=%lld has no kernel; built: 64, 128, 256.", op, (long long)V);
+}
+
+int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+                   const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
+                   const fla_int_array *ci, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+                   const fla_tensor *dw, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_kda_bwd_dqkwg";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v_new, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
+    const int64_t B = geom.B, Hk = geom.Hk, Hv = geom.Hv, T = geom.T, K = geom.K, V = geom.V;
+    if ((rc = check_bhtd(op, "q", q, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v_new", v_new, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dw", dw, B, Hv, T, K, bf))) return rc;
+    if ((rc = check_f32_bhtd(op, "gk", gk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dq", dq, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dk", dk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dg", dg, B, Hv, T, K))) return rc;
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
+    if ((rc = check_state_blocks(op, "h", h, geom))) return rc;
+    if ((rc = check_state_blocks(op, "dh", dh, geom))) return rc;
+    if (query) return FLA_OK;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    KdaDqkwgParams p{geom, view4(q), view4(k), view4(v_new), view4(d_o), view4(dv), view4(dw),
+                     static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
+                     static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
+                     h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
+                     viewf(dq), viewf(dk), viewf(dg), (float)scale};
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4;
+    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<128, 128>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<64, 64>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<64, 128>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(64,128).", op, (long long)K,
+                (long long)V);
+}
+
+int kda_wy_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *akk,
+                const fla_tensor *dw, const fla_tensor *du, const fla_int_array *cu, const fla_int_array *ci, int64_t chunk_size,
+                const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg, const fla_tensor *dakk,
+                void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_kda_bwd_wy";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    const int bf = dt_bit(kElemDtype);
+    const int64_t B = geom.B, Hk = geom.Hk, Hv = geom.Hv, T = geom.T, K = geom.K, V = geom.V;
+    if ((rc = check_bhtd(op, "k", k, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "Akk", akk, B, Hv, T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dw", dw, B, Hv, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "du", du, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, B, Hv, T, V, bf))) return rc;
+    FLA_REQUIRE(beta != nullptr && beta->data != nullptr, FLA_ERR_NULL, "%s: beta must be provided.", op);
+    if ((rc = check_bht(op, "beta", beta, B, Hv, T, kElemDtype))) return rc;
+    if ((rc = check_f32_bhtd(op, "gk", gk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dk", dk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dg", dg, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dAkk", dakk, B, Hv, T, kChunk))) return rc;
+    if ((rc = check_tensor(db, op, "db", 3, dt_bit(FLA_F32)))) return rc;
+    FLA_REQUIRE(db->shape[0] == B && db->shape[1] == Hv && db->shape[2] == T, FLA_ERR_SHAPE, "%s: db must be [%lld,%lld,%lld].",
+                op, (long long)B, (long long)Hv, (long long)T);
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    KdaWyParams p{geom, view4(k), view4(v), view4(akk), view4(dw), view4(du), view4(dv), view3(beta),
+                  static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
+                  viewf(dk), viewf(dg), viewf(dakk), static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2]};
+    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const size_t smem = ((size_t)kChunk * ((K + 16) + (V + 16) + (K + 8) + (V + 8) + (kChunk + 8))) * 2 + kChunk * 4;
+    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_wy_kernel<128, 128>), "kda_bwd_wy", grid, smem, p, kThreads);
+    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_wy_kernel<64, 64>), "kda_bwd_wy", grid, smem, p, kThreads);
+    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_wy_kernel<64, 128>), "kda_bwd_wy", grid, smem, p, kThreads);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(64,128).", op, (long long)K,
+                (long long)V);
+}
+
+}  // namespace
+}  // namespace fla
+
+#define FLA_NULL_WS(op) \
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, op ": workspace_size must not be null.")
+
+FLA_ENTRY(fla_chunk_kda_bwd_dav_get_workspace_size)(
+    const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *Aqk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dAqk, const fla_tensor *dv,
+    uint64_t *workspace_size) {
+    FLA_ROUTE_F16(v_new, fla_chunk_kda_bwd_dav_get_workspace_size, v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace_size);
+    FLA_NULL_WS("chunk_kda_bwd_dav");
+    return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, nullptr, 0, nullptr,
+                         workspace_size);
+}
+FLA_ENTRY(fla_chunk_kda_bwd_dav)(
+    const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *Aqk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dAqk, const fla_tensor *dv,
+    void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(v_new, fla_chunk_kda_bwd_dav, v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace, workspace_size, stream);
+    return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr);
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace_size);
+    FLA_NULL_WS("chunk_kda_bwd_dqkwg");
+    return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
+                               nullptr, 0, nullptr, workspace_size);
+}
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace, workspace_size, stream);
+    return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
+                               workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_wy_get_workspace_size)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *Akk,
+    const fla_tensor *dw, const fla_tensor *du, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
+    const fla_tensor *dAkk, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_chunk_kda_bwd_wy_get_workspace_size, k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace_size);
+    FLA_NULL_WS("chunk_kda_bwd_wy");
+    return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, nullptr, 0,
+                            nullptr, workspace_size);
+}
+FLA_ENTRY(fla_chunk_kda_bwd_wy)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *Akk,
+    const fla_tensor *dw, const fla_tensor *du, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
+    const fla_tensor *dAkk, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_chunk_kda_bwd_wy, k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace, workspace_size, stream);
+    return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace,
+                            workspace_size, static_cast<hipStream_t>(stream), nullptr);
+}

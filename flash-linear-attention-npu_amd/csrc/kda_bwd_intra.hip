@@ -34,10 +34,14 @@ struct BwdIntraParams {
     const elem *q, *k;
     const float *gk, *dq, *dk, *dg;
     float *dq_o, *dk_o, *dg_o;
-    int64_t sb, sh, st;          // strides of (batch, head, token) of the [..,K] tensors
+    int64_t sb, sh, st;          // strides of (batch, head, token) of the six gradient tensors [..,K]
+    int64_t q_sb, q_sh, q_st;    // of q and k, which may have fewer heads (head h reads key head h / rep)
+    int64_t g_sb, g_sh, g_st;    // of gk
+    int rep;
     View3 beta;
     const float *db;
     float *db_o;
+    int64_t db_sb, db_sh, db_st;
     const float *daqk, *dakk;    // [..,64]
     int64_t m_sb, m_sh, m_st;
 };
@@ -88,21 +92,23 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
     const int row_end = min(r0 + 16, len);
     const int anchor = min(r0 + 8, row_end - 1);
     const int64_t base = b * p.sb + h * p.sh + (int64_t)start * p.st;
+    const int64_t qbase = b * p.q_sb + (h / p.rep) * p.q_sh + (int64_t)start * p.q_st;
+    const int64_t gbase = b * p.g_sb + h * p.g_sh + (int64_t)start * p.g_st;
     f32x4 dbacc = {0.f, 0.f, 0.f, 0.f};
 
     for (int ch0 = 0; ch0 < K; ch0 += KC) {
         __syncthreads();
         {
             TileCopy<kThreads, kChunk, KC> tq, tk;
-            tq.fetch(p.q + base + ch0, p.st, len, tid);
-            tk.fetch(p.k + base + ch0, p.st, len, tid);
+            tq.fetch(p.q + qbase + ch0, p.q_st, len, tid);
+            tk.fetch(p.k + qbase + ch0, p.q_st, len, tid);
             constexpr int GN = kChunk * (KC / 4) / kThreads;
             f32x4 gv[GN];
 #pragma unroll
             for (int m = 0; m < GN; ++m) {   // padded rows repeat the last gate row
                 const int idx = m * kThreads + tid;
                 const int r = min(idx / (KC / 4), len - 1), c4 = (idx % (KC / 4)) * 4;
-                gv[m] = *reinterpret_cast<const f32x4 *>(p.gk + base + (int64_t)r * p.st + ch0 + c4);
+                gv[m] = *reinterpret_cast<const f32x4 *>(p.gk + gbase + (int64_t)r * p.g_st + ch0 + c4);
             }
             tq.commit(qS, pk, len, tid);
             tk.commit(kS, pk, len, tid);
@@ -166,7 +172,7 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
             const float s = group_sum<16>(dbacc[e]);
             const int i = r0 + 4 * lg + e;
             if (li == 0 && i < len) {
-                const int64_t off = b * p.beta.sb + h * p.beta.sh + (int64_t)(start + i) * p.beta.st;
+                const int64_t off = b * p.db_sb + h * p.db_sh + (int64_t)(start + i) * p.db_st;
                 p.db_o[off] = p.db[off] + s;
             }
         }
@@ -203,17 +209,35 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     int rc;
     if ((rc = check_tensor(q, op, "q", rank, dt_bit(kElemDtype)))) return rc;
     if ((rc = check_tensor(k, op, "k", rank, dt_bit(kElemDtype)))) return rc;
-    const fla_tensor *f32s[] = {gk, dq, dk, dg, dq_o, dk_o, dg_o};
-    const char *f32n[] = {"gk", "dq", "dk", "dg", "dq_out", "dk_out", "dg_out"};
-    for (int i = 0; i < 7; ++i) {
-        if ((rc = check_tensor(f32s[i], op, f32n[i], rank, dt_bit(FLA_F32)))) return rc;
-        FLA_REQUIRE(same_shape(f32s[i], q), FLA_ERR_SHAPE, "%s: %s must have the same shape as q.", op, f32n[i]);
-        FLA_REQUIRE(is_contiguous(f32s[i]), FLA_ERR_SHAPE, "%s: %s must be contiguous; implicit copies are disabled.", op,
-                    f32n[i]);
+    // The reference demands contiguous tensors of one layout.  Here every [..,K] tensor may be any strided view of that
+    // index order with a unit innermost stride and 16-byte aligned rows; q and k may carry fewer heads than the gate
+    // (grouped value heads: head h of gk and of the gradients reads key head h / (H / Hq)); the six gradient tensors
+    // share one set of strides, and each output may be its own input.
+    const fla_tensor *grads[] = {dq, dk, dg, dq_o, dk_o, dg_o};
+    const char *gradn[] = {"dq", "dk", "dg", "dq_out", "dk_out", "dg_out"};
+    if ((rc = check_tensor(gk, op, "gk", rank, dt_bit(FLA_F32)))) return rc;
+    const int64_t B = ib < 0 ? 1 : gk->shape[ib], H = gk->shape[ih], T = gk->shape[it], K = gk->shape[rank - 1];
+    auto strided_ok = [&](const fla_tensor *t, int64_t heads, int64_t al) {
+        return (ib < 0 || t->shape[ib] == B) && t->shape[ih] == heads && t->shape[it] == T && t->shape[rank - 1] == K &&
+               inner_unit(t) && (ib < 0 || t->stride[ib] % al == 0) && t->stride[ih] % al == 0 && t->stride[it] % al == 0 &&
+               t->stride[it] >= 0 && reinterpret_cast<uintptr_t>(t->data) % 16 == 0;
+    };
+    for (int i = 0; i < 6; ++i) {
+        if ((rc = check_tensor(grads[i], op, gradn[i], rank, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE(strided_ok(grads[i], H, 4), FLA_ERR_SHAPE,
+                    "%s: %s must have the shape of gk, a unit innermost stride and 16-byte aligned rows.", op, gradn[i]);
+        FLA_REQUIRE((ib < 0 || grads[i]->stride[ib] == dq->stride[ib]) && grads[i]->stride[ih] == dq->stride[ih] &&
+                        grads[i]->stride[it] == dq->stride[it],
+                    FLA_ERR_SHAPE, "%s: dq, dk, dg and their outputs must share one set of strides.", op);
     }
-    FLA_REQUIRE(same_shape(k, q), FLA_ERR_SHAPE, "%s: k must have the same shape as q.", op);
-    FLA_REQUIRE(is_contiguous(q) && is_contiguous(k), FLA_ERR_SHAPE, "%s: q and k must be contiguous.", op);
-    const int64_t B = ib < 0 ? 1 : q->shape[ib], H = q->shape[ih], T = q->shape[it], K = q->shape[rank - 1];
+    FLA_REQUIRE(strided_ok(gk, H, 4), FLA_ERR_SHAPE, "%s: gk needs a unit innermost stride and 16-byte aligned rows.", op);
+    const int64_t Hq = q->shape[ih];
+    FLA_REQUIRE(Hq > 0 && H % Hq == 0, FLA_ERR_SHAPE, "%s: heads of gk (%lld) must be a multiple of the heads of q (%lld).", op,
+                (long long)H, (long long)Hq);
+    FLA_REQUIRE(strided_ok(q, Hq, 8) && strided_ok(k, Hq, 8), FLA_ERR_SHAPE,
+                "%s: q and k must be [..,%lld heads,..,K] with a unit innermost stride and 16-byte aligned rows.", op, (long long)Hq);
+    FLA_REQUIRE((ib < 0 || q->stride[ib] == k->stride[ib]) && q->stride[ih] == k->stride[ih] && q->stride[it] == k->stride[it],
+                FLA_ERR_SHAPE, "%s: q and k must share one set of strides.", op);
     FLA_REQUIRE(B > 0 && H > 0 && T > 0, FLA_ERR_SHAPE, "%s: B/H/T must be positive.", op);
     FLA_REQUIRE(K == 64 || K == 128 || K == 256, FLA_ERR_UNSUPPORTED, "%s: K must be 64, 128 or 256.", op);
     FLA_REQUIRE(B < 65536 && H < 65536 && T < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents too large.", op);
@@ -222,21 +246,26 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     const char *scn[] = {"beta", "db", "db_out"};
     for (int i = 0; i < 3; ++i) {
         if (i && (rc = check_tensor(sc[i], op, scn[i], rank - 1, dt_bit(FLA_F32)))) return rc;
-        FLA_REQUIRE((ib < 0 || sc[i]->shape[ib] == B) && sc[i]->shape[ih] == H && sc[i]->shape[it] == T && is_contiguous(sc[i]),
-                    FLA_ERR_SHAPE, "%s: beta/db shape must match the selected layout.", op);
+        FLA_REQUIRE((ib < 0 || sc[i]->shape[ib] == B) && sc[i]->shape[ih] == H && sc[i]->shape[it] == T, FLA_ERR_SHAPE,
+                    "%s: beta/db shape must match the selected layout.", op);
     }
+    FLA_REQUIRE((ib < 0 || db->stride[ib] == db_o->stride[ib]) && db->stride[ih] == db_o->stride[ih] &&
+                    db->stride[it] == db_o->stride[it],
+                FLA_ERR_SHAPE, "%s: db and db_out must share one set of strides.", op);
     const fla_tensor *mats[] = {daqk, dakk};
     for (int i = 0; i < 2; ++i) {
         if ((rc = check_tensor(mats[i], op, i ? "dAkk" : "dAqk", rank, dt_bit(FLA_F32)))) return rc;
         FLA_REQUIRE((ib < 0 || mats[i]->shape[ib] == B) && mats[i]->shape[ih] == H && mats[i]->shape[it] == T &&
-                        mats[i]->shape[rank - 1] == kChunk && is_contiguous(mats[i]),
+                        mats[i]->shape[rank - 1] == kChunk && inner_unit(mats[i]) && mats[i]->stride[it] % 4 == 0 &&
+                        mats[i]->stride[ih] % 4 == 0 && (ib < 0 || mats[i]->stride[ib] % 4 == 0) &&
+                        reinterpret_cast<uintptr_t>(mats[i]->data) % 16 == 0,
                     FLA_ERR_SHAPE, "%s: dAqk/dAkk shape must match the selected layout.", op);
+        FLA_REQUIRE((ib < 0 || mats[i]->stride[ib] == daqk->stride[ib]) && mats[i]->stride[ih] == daqk->stride[ih] &&
+                        mats[i]->stride[it] == daqk->stride[it],
+                    FLA_ERR_SHAPE, "%s: dAqk and dAkk must share one set of strides.", op);
     }
-    const fla_tensor *al[] = {q, k, gk, dq, dk, dg, dq_o, dk_o, dg_o, daqk, dakk};
-    for (const fla_tensor *t : al)
-        FLA_REQUIRE(reinterpret_cast<uintptr_t>(t->data) % 16 == 0, FLA_ERR_SHAPE, "%s: tensors must be 16-byte aligned.", op);
     const bool varlen = cu && cu->data && cu->size;
-    FLA_REQUIRE(!(varlen && !strcmp(layout, "BNSD")), FLA_ERR_UNSUPPORTED, "%s: varlen supports TND or BSND, not BNSD.", op);
+    // (the reference rejects packed BNSD input; with strided views it is the same addressing as BSND with B = 1)
     FLA_REQUIRE(varlen || ib >= 0, FLA_ERR_SHAPE, "%s: TND requires cu_seqlens.", op);
     FLA_REQUIRE(varlen || !(ci && ci->data && ci->size), FLA_ERR_SHAPE, "%s: chunk_indices requires cu_seqlens.", op);
 
@@ -249,7 +278,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     geom.N = (int)B;
     Varlen vl;
     if ((rc = build_varlen(vl, op, cu, ci, kChunk, T))) return rc;
-    FLA_REQUIRE(!vl.enabled || B == 1, FLA_ERR_SHAPE, "%s: varlen BSND compatibility requires B=1.", op);
+    FLA_REQUIRE(!vl.enabled || B == 1, FLA_ERR_SHAPE, "%s: packed rank-4 input requires B=1.", op);
     if (vl.enabled) {
         geom.NT = vl.NT;
         geom.N = vl.N;
@@ -277,18 +306,28 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.dq_o = static_cast<float *>(dq_o->data);
     p.dk_o = static_cast<float *>(dk_o->data);
     p.dg_o = static_cast<float *>(dg_o->data);
-    p.sb = ib < 0 ? 0 : q->stride[ib];
-    p.sh = q->stride[ih];
-    p.st = q->stride[it];
+    p.sb = ib < 0 ? 0 : dq->stride[ib];
+    p.sh = dq->stride[ih];
+    p.st = dq->stride[it];
+    p.q_sb = ib < 0 ? 0 : q->stride[ib];
+    p.q_sh = q->stride[ih];
+    p.q_st = q->stride[it];
+    p.g_sb = ib < 0 ? 0 : gk->stride[ib];
+    p.g_sh = gk->stride[ih];
+    p.g_st = gk->stride[it];
+    p.rep = (int)(H / Hq);
     p.beta = View3{beta->data, ib < 0 ? 0 : beta->stride[ib], beta->stride[ih], beta->stride[it], beta->dtype == FLA_F32 ? 0 : 1};
     p.db = static_cast<const float *>(db->data);
     p.db_o = static_cast<float *>(db_o->data);
+    p.db_sb = ib < 0 ? 0 : db->stride[ib];
+    p.db_sh = db->stride[ih];
+    p.db_st = db->stride[it];
     p.daqk = static_cast<const float *>(daqk->data);
     p.dakk = static_cast<const float *>(dakk->data);
     p.m_sb = ib < 0 ? 0 : daqk->stride[ib];
     p.m_sh = daqk->stride[ih];
     p.m_st = daqk->stride[it];
-    FLA_REQUIRE(p.st >= 0 && p.st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride must be below 2^24 elements.", op);
+    FLA_REQUIRE(p.q_st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride of q and k must be below 2^24 elements.", op);
     return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }
 

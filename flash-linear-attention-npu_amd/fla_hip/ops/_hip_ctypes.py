@@ -54,6 +54,9 @@ OP_ARGTYPES = {
     "prepare_wy_repr_bwd_da": [_T] * 7 + [_IA, _IA, ctypes.c_int64, _T],
     "prepare_wy_repr_bwd_full": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
     "prepare_wy_repr_bwd": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
+    "chunk_kda_bwd_dav": [_T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T, _T],
+    "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 4,
+    "chunk_kda_bwd_wy": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 5,
 }
 
 
@@ -739,6 +742,133 @@ def npu_chunk_kda_bwd_intra(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_se
         ],
         outputs,
     )
+
+
+# ---------------------------------------------------------------------------------------------
+# KDA chunk backward: the stages the reference leaves to a third-party package
+# (torch_custom/fla_npu/fla_npu/adapters/triton_ascend_kda.py:1-8).  Operands are [B,H,T,D] index order; any
+# strided view with a unit innermost stride is taken as is (pass ``x.transpose(1, 2)`` for a [B,T,H,D] tensor).
+# ``out_like`` tensors let a caller choose the memory layout of the fp32 results.
+def _empty_strided_like(shape, like, dtype, device=None):
+    """A tensor of ``shape`` whose memory order follows ``like`` (same permutation of dimensions)."""
+    import torch
+
+    order = sorted(range(len(shape)), key=lambda d: (-like.stride(d), d))
+    perm_shape = [shape[d] for d in order]
+    base = torch.empty(perm_shape, dtype=dtype, device=like.device if device is None else device)
+    inverse = [order.index(d) for d in range(len(shape))]
+    return base.permute(inverse)
+
+
+def chunk_kda_bwd_dav(v_new, d_o, Aqk, scale, chunk_size=64, *, cu_seqlens=None, chunk_indices=None, layout_like=None):
+    """``dAqk = scale * tril(d_o v_new^T)`` (fp32 [B,Hv,T,64]) and ``dv = Aqk^T d_o`` ([B,Hv,T,V], dtype of v_new).
+    ``layout_like`` ([B,Hv,T,*] view): dAqk is laid out in memory like it (default: like ``d_o``)."""
+    import torch
+
+    B, Hv, T, V = _shape(d_o)
+    like = d_o if layout_like is None else layout_like
+    dA = _empty_strided_like((B, Hv, T, int(chunk_size)), like, torch.float32, d_o.device)
+    dv = _empty_strided_like((B, Hv, T, V), v_new, v_new.dtype)
+    cu = _as_int_tuple(cu_seqlens)
+    _call_op(
+        "chunk_kda_bwd_dav", OP_ARGTYPES["chunk_kda_bwd_dav"],
+        lambda ctx: [
+            ctx.tensor(v_new, "v_new"), ctx.tensor(d_o, "d_o"), ctx.tensor(Aqk, "Aqk"), ctx.int_array(cu),
+            ctx.int_array(_as_int_tuple(chunk_indices)), ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(dA, "dAqk"), ctx.tensor(dv, "dv"),
+        ],
+        (dA, dv),
+    )
+    return dA, dv
+
+
+def chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, d_o, dh, dv, scale, chunk_size=64, *, cu_seqlens=None, chunk_indices=None,
+                        layout_like=None):
+    """State-dependent part of the KDA backward: returns ``(dq, dk, dw, dg)``, dq / dk / dg fp32 [B,Hv,T,K] per value
+    head laid out like ``layout_like`` (default: like ``gk``), dw [B,Hv,T,K] in the dtype of q.
+    ``h`` and ``dh`` are [B,Hv,NT,K,V] views (any outer strides)."""
+    import torch
+
+    B, Hv, T, K = _shape(gk)
+    like = gk if layout_like is None else layout_like
+    dq = _empty_strided_like((B, Hv, T, K), like, torch.float32, q.device)
+    dk = _empty_strided_like((B, Hv, T, K), like, torch.float32, q.device)
+    dg = _empty_strided_like((B, Hv, T, K), like, torch.float32, q.device)
+    dw = _empty((B, Hv, T, K), q)
+    cu = _as_int_tuple(cu_seqlens)
+    outs = (dq, dk, dw, dg)
+    _call_op(
+        "chunk_kda_bwd_dqkwg", OP_ARGTYPES["chunk_kda_bwd_dqkwg"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v_new, "v_new"), ctx.tensor(gk, "gk"), ctx.tensor(h, "h"),
+            ctx.tensor(d_o, "d_o"), ctx.tensor(dh, "dh"), ctx.tensor(dv, "dv"), ctx.int_array(cu),
+            ctx.int_array(_as_int_tuple(chunk_indices)), ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
+            *[ctx.tensor(t, n) for t, n in zip(outs, ("dq", "dk", "dw", "dg"))],
+        ],
+        outs,
+    )
+    return outs
+
+
+def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, dk, dg, chunk_size=64, *, cu_seqlens=None, chunk_indices=None):
+    """Backward of ``w = Akk (k beta 2^g)``, ``u = Akk (v beta)``.  ``dk`` and ``dg`` (fp32 [B,Hv,T,K]) are ADDED TO in
+    place; returns ``(dv, db, dAkk)``: dv like v, db fp32 [B,Hv,T], dAkk fp32 [B,Hv,T,64], both laid out like ``dk``."""
+    import torch
+
+    B, Hv, T, V = _shape(du)
+    dv = _empty_strided_like((B, Hv, T, V), v, v.dtype)
+    db = _empty_strided_like((B, Hv, T, 1), dk, torch.float32)[..., 0]
+    dA = _empty_strided_like((B, Hv, T, int(chunk_size)), dk, torch.float32)
+    cu = _as_int_tuple(cu_seqlens)
+    outs = (dv, db, dA)
+    _call_op(
+        "chunk_kda_bwd_wy", OP_ARGTYPES["chunk_kda_bwd_wy"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(gk, "gk"), ctx.tensor(Akk, "Akk"),
+            ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.int_array(cu), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_int64(int(chunk_size)), ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(db, "db"),
+            ctx.tensor(dg, "dg"), ctx.tensor(dA, "dAkk"),
+        ],
+        outs,
+    )
+    return outs
+
+
+def chunk_kda_bwd_intra_inplace(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_seqlens=None, chunk_size=64):
+    """``npu_chunk_kda_bwd_intra`` on [B,H,T,*] index-order views with the results written over ``dq, dk, db, dg``.
+    The library accepts strided views, grouped heads (q, k with fewer heads than gk) and outputs that alias their
+    inputs; the public operator keeps the reference's contiguous, allocate-new contract."""
+    cu = _as_int_tuple(cu_seqlens)
+    indices = None if cu is None else _build_chunk_indices(cu, int(chunk_size))
+    ins = (q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg)
+    names = ("q", "k", "gk", "beta", "dAqk", "dAkk", "dq", "dk", "db", "dg")
+    outs = (dq, dk, db, dg)
+    _call_op(
+        "chunk_kda_bwd_intra", OP_ARGTYPES["chunk_kda_bwd_intra"],
+        lambda ctx: [
+            *[ctx.tensor(t, n) for t, n in zip(ins, names)],
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_int64(int(chunk_size)), ctypes.c_bool(True),
+            ctypes.c_char_p(b"BNSD"),
+            *[ctx.tensor(t, n) for t, n in zip(outs, ("dq_out", "dk_out", "db_out", "dg_out"))],
+        ],
+        outs,
+    )
+    return outs
+
+
+def chunk_local_cumsum_into(g, out, chunk_size, *, cu_seqlens=None, reverse=False, scale=1.0):
+    """``npu_chunk_local_cumsum`` on [B,H,T] / [B,H,T,K] index-order views, written into ``out`` (which may be ``g``)."""
+    name_buf = ctypes.create_string_buffer(str(out.dtype).removeprefix("torch.").encode("utf-8"))
+    _call_op(
+        "chunk_local_cumsum", OP_ARGTYPES["chunk_local_cumsum"],
+        lambda ctx: [
+            ctx.tensor(g, "g"), ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(None),
+            ctypes.c_int64(int(chunk_size)), ctypes.c_bool(bool(reverse)), ctypes.c_double(float(scale)),
+            ctypes.c_bool(True), ctypes.cast(name_buf, ctypes.c_char_p), ctx.tensor(out, "out"),
+        ],
+        out,
+    )
+    return out
 
 
 def _f32_like(t):

@@ -208,3 +208,136 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
         _FUNCTION = _autograd_function()
     return _FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused,
                            bool(use_qk_l2norm_in_kernel))
+
+
+# =============================================================================================
+# KDA (per-channel gated delta rule): chunk forward + backward as one differentiable call
+# =============================================================================================
+# The reference exposes the forward operator and two backward stages (bwd_dhu with gK, chunk_kda_bwd_intra) and
+# leaves the composition to a third-party package it patches (adapters/triton_ascend_kda.py:141-242 hands that
+# package the forward's saved tensors gk, Aqk, Akk, w, u, qg, kg, v_new, h).  Here the whole chain is the library's.
+def _index_order(x, layout, *, scalar=False):
+    """View of a tensor in ``layout`` (BSND / BNSD / TND / NTD) in [B,H,T,(D)] index order; nothing is copied."""
+    if layout == "BSND":
+        return x.transpose(1, 2)
+    if layout == "BNSD":
+        return x
+    if layout == "TND":
+        return x.transpose(0, 1)[None]
+    if layout == "NTD":
+        return x[None]
+    raise ValueError(f"layout must be one of BSND, BNSD, TND, NTD, got {layout!r}.")
+
+
+def _from_index_order(x, layout):
+    if layout == "BSND":
+        return x.transpose(1, 2)
+    if layout == "BNSD":
+        return x
+    if layout == "TND":
+        return x[0].transpose(0, 1)
+    return x[0]
+
+
+def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, dht=None, *, initial_state=None,
+                  layout="BSND", cu_seqlens=None, chunk_size: int = 64):
+    """KDA chunk backward from the tensors the forward keeps (``chunk_kda_fwd(..., disable_recompute=True)``).
+
+    q, k, v, beta, do in ``layout``; gk, Aqk, Akk, w, qg, kg, v_new head-major and h as the forward returned them;
+    dht fp32 [N,Hv,K,V] or None.  Returns ``(dq, dk, dv, dg, dbeta, dh0)``: dq, dk, dv, dbeta in ``layout`` and the
+    dtype of their inputs, dg fp32 in the layout of the gate = gradient of the per-token log decay (natural log),
+    dh0 fp32 [N,Hv,K,V] or None.  Stages: dAqk / dv -> reverse scan (bwd_dhu, gK) -> dq, dk, dw, dg of the
+    state-dependent parts -> backward of the WY factors (dv, dbeta, dAkk) -> chunk_kda_bwd_intra -> reverse
+    chunk-local cumulative sum of dg."""
+    import torch
+
+    if chunk_size != 64:
+        raise NotImplementedError("chunk_kda_bwd: the backward operators are built for chunk_size 64.")
+    cu = _cu_list(cu_seqlens)
+    kw = dict(cu_seqlens=cu)
+    rank3 = layout in ("TND", "NTD")
+    hm = lambda t: _index_order(t, layout)
+    lead = (lambda t: t[None]) if rank3 else (lambda t: t)
+    qh, kh, vh, bh, doh = hm(q), hm(k), hm(v), hm(beta), hm(do)
+    if doh.stride(-1) != 1:
+        doh = hm(do.contiguous())
+    gk4, Aqk4, Akk4, w4, qg4, kg4, vn4 = (lead(t) for t in (gk, Aqk, Akk, w, qg, kg, v_new))
+    h5 = lead(h).transpose(1, 2)                                  # [B,NT,Hv,K,V] -> [B,Hv,NT,K,V] view
+    Hk, Hv = qh.shape[1], vh.shape[1]
+    # fp32 gradients per value head, laid out in memory like the caller's tensors (heads = Hv)
+    layout_like = _index_order(_empty_in_layout(layout, gk4.shape), layout)
+    dAqk, dv0 = _raw.chunk_kda_bwd_dav(vn4, doh, Aqk4, scale, chunk_size, layout_like=layout_like, **kw)
+    dh, dh0, dv2 = _ops.chunk_gated_delta_rule_bwd_dhu(qg4, kg4, w4, doh, dv0, scale, chunk_size, gK=gk4,
+                                                       h0=initial_state, dht=dht, use_exp2=True, dh0_per_sequence=True,
+                                                       **kw)
+    dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
+                                              layout_like=layout_like, **kw)
+    dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
+    _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size)
+    _raw.chunk_local_cumsum_into(dg, dg, chunk_size, cu_seqlens=cu, reverse=True)
+    if Hv != Hk:          # value heads that share a key head add their gradients
+        dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2)
+        dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2)
+    back = lambda t: _from_index_order(t, layout)
+    return (back(dq).to(q.dtype), back(dk).to(k.dtype), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
+
+
+def _empty_in_layout(layout, index_shape):
+    """A storage-less tensor in ``layout`` whose index-order shape is ``index_shape`` ([B,H,T,D]); only its strides are
+    used (as the memory order of the gradients)."""
+    import torch
+
+    B, H, T, D = index_shape
+    shape = {"BSND": (B, T, H, D), "BNSD": (B, H, T, D), "TND": (T, H, D), "NTD": (H, T, D)}[layout]
+    return torch.empty(shape, dtype=torch.float32, device="meta")
+
+
+_KDA_FUNCTION = None
+
+
+def _kda_autograd_function():
+    import torch
+
+    class ChunkKdaFunction(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, layout, chunk_size):
+            out = _ops.chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size, layout=layout, initial_state=initial_state,
+                                     output_final_state=output_final_state, cu_seqlens=cu, disable_recompute=True,
+                                     return_intermediate_states=True)
+            o, final, gk, Aqk, Akk, w, _u, qg, kg, v_new, h, _ = out
+            ctx.save_for_backward(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state)
+            ctx.scale, ctx.cu, ctx.layout, ctx.chunk_size, ctx.g_dtype = scale, cu, layout, chunk_size, g.dtype
+            return o, final
+
+        @staticmethod
+        def backward(ctx, do, dht):
+            q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state = ctx.saved_tensors
+            dq, dk, dv, dg, db, dh0 = chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, ctx.scale, do, dht,
+                                                    initial_state=initial_state, layout=ctx.layout, cu_seqlens=ctx.cu,
+                                                    chunk_size=ctx.chunk_size)
+            return dq, dk, dv, dg.to(ctx.g_dtype), db, None, dh0, None, None, None, None
+
+    return ChunkKdaFunction
+
+
+def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=None, output_final_state: bool = False,
+              cu_seqlens=None, *, layout: str = "BSND", chunk_size: int = 64):
+    """KDA chunk attention, differentiable: ``(o, final_state)`` with q, k [..H,K], v [..HV,V], per-channel log decay
+    g [..HV,K] (natural log, one value per token and channel), beta [..HV] in ``layout``; states fp32 [N,HV,K,V].
+    The forward is ``chunk_kda_fwd``; when an input requires grad the forward keeps its intermediates and
+    ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0."""
+    import torch
+
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    cu = _cu_list(cu_seqlens)
+    if not needs_grad_hint(q, k, v, g, beta, initial_state):
+        out = _ops.chunk_kda_fwd(q, k, v, g, beta, float(scale), chunk_size, layout=layout, initial_state=initial_state,
+                                 output_final_state=output_final_state, cu_seqlens=cu)
+        return out[0], out[1]
+    if chunk_size != 64:
+        raise NotImplementedError("chunk_kda: gradients are built for chunk_size 64.")
+    global _KDA_FUNCTION
+    if _KDA_FUNCTION is None:
+        _KDA_FUNCTION = _kda_autograd_function()
+    return _KDA_FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, layout, chunk_size)

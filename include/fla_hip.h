@@ -382,6 +382,57 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
+ * KDA chunk backward, the stages around chunk_gated_delta_rule_bwd_dhu (gK) and chunk_kda_bwd_intra.
+ * The reference has no operators for them: its deployment keeps them in a third-party Triton package
+ * (torch_custom/fla_npu/fla_npu/adapters/triton_ascend_kda.py:1-8); they differentiate the forward of
+ * tests/atk/chunk_kda_fwd/executor_chunk_kda_fwd.py:459-484.  All activations in [B,H,T,D] index order
+ * through strides (unit innermost stride; a [B,T,H,D] tensor is passed as its transposed view).  gk is
+ * the chunk-local cumulated gate in log2 units, f32 [B,Hv,T,K].  dq, dk, dg are f32 [B,Hv,T,K], one per
+ * VALUE head; "dg" is the gradient with respect to ln2 * gk, as in chunk_kda_bwd_intra.  chunk_size 64.
+ * ------------------------------------------------------------------------ */
+
+/* chunk_kda_bwd_dav: dAqk = scale * tril(d_o v_new^T) (f32 [B,Hv,T,64], zero above the diagonal),
+ * dv = Aqk^T d_o.  v_new, d_o, dv [B,Hv,T,V], Aqk [B,Hv,T,64] in the element type. */
+int fla_chunk_kda_bwd_dav_get_workspace_size(
+    const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *Aqk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dAqk, const fla_tensor *dv,
+    uint64_t *workspace_size);
+int fla_chunk_kda_bwd_dav(
+    const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *Aqk, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dAqk, const fla_tensor *dv,
+    void *workspace, uint64_t workspace_size, void *stream);
+
+/* chunk_kda_bwd_dqkwg: with h the state at each chunk start, dh the gradient of the state at each chunk
+ * end and dv the total gradient of v_new (dh, dv: outputs of bwd_dhu), both [B,Hv,NT,K,V] with any outer strides:
+ *   dq = scale (d_o h^T) 2^g,  dk = (v_new dh^T) 2^{g_last - g},  dw = -dv h^T (element type, [B,Hv,T,K]),
+ *   dg = q dq - k dk, plus on the last token of a chunk  sum_j k_j dk_j + 2^{g_last} rowsum(h . dh). */
+int fla_chunk_kda_bwd_dqkwg_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_dqkwg(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+
+/* chunk_kda_bwd_wy: backward of w = Akk (k beta 2^g), u = Akk (v beta), Akk = (I + M)^-1 given dw, du:
+ *   x = Akk^T dw, y = Akk^T du;  dk += x beta 2^g;  dg += (x beta 2^g) k   (dk, dg are read and added to);
+ *   dv = y beta (element type);  db = <x, k 2^g> + <y, v> (f32 [B,Hv,T], written);
+ *   dAkk = -strict_lower(Akk^T (dw (k beta 2^g)^T + du (v beta)^T) Akk^T)  (f32 [B,Hv,T,64], written). */
+int fla_chunk_kda_bwd_wy_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *Akk,
+    const fla_tensor *dw, const fla_tensor *du, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
+    const fla_tensor *dAkk, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_wy(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *Akk,
+    const fla_tensor *dw, const fla_tensor *du, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
+    int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
+    const fla_tensor *dAkk, void *workspace, uint64_t workspace_size, void *stream);
+
+/* ------------------------------------------------------------------------
  * l2norm_fwd / l2norm_bwd - the q/k normalisation of the chunk pipelines, which the reference
  * runs as Triton kernels (fla/ops/triton/triton_core/l2norm.py:131-224; called from
  * examples/flash_gated_delta_rule.py:1047-1049,1104-1106).  Rank 2..4 bf16/f16 tensors with

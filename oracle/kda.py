@@ -273,3 +273,122 @@ def recurrent_kda(q, k, v, g, beta, initial_state, *, cu_seqlens=None, ssm_state
             pool[slot_of(t)] = (S if state_v_first else S.transpose(-1, -2)).to(pool.dtype)
     out = out.to(v.dtype)
     return (out if tnd else out.reshape(v.shape)), pool
+
+
+# ---------------------------------------------------------------------------------------------
+# KDA chunk backward.  The reference ships only two of its stages (bwd_dhu with gK and chunk_kda_bwd_intra); the
+# rest of the chain lives in a third-party Triton package it patches around
+# (torch_custom/fla_npu/fla_npu/adapters/triton_ascend_kda.py:1-8).  The three stages below are this build's own
+# decomposition of the remaining work; each is the exact derivative of the forward stage it names and is pinned
+# against torch autograd of that stage, the composition against autograd through naive_recurrent_kda
+# (tests/test_oracle.py).  "dg" everywhere is the gradient with respect to the cumulated gate in natural-log
+# units per step (dL/dgk / ln 2): a reverse chunk-local cumulative sum of it is the gradient of the per-token gate.
+# ---------------------------------------------------------------------------------------------
+def chunk_kda_bwd_dav(v_new, do, Aqk, scale, chunk: int = 64, *, cu_seqlens=None, compute_dtype=torch.float32):
+    """Derivative of  o_intra = Aqk v_new,  Aqk = scale * tril(score):
+        dAqk = scale * tril(do v_new^T)   (gradient of the unscaled score, what chunk_kda_bwd_intra consumes)
+        dv   = Aqk^T do                   (first part of the gradient of v_new)."""
+    cd = compute_dtype
+    B, Hv, T, V = do.shape
+    dA = torch.zeros(B, Hv, T, chunk, dtype=cd)
+    dv = torch.zeros(B, Hv, T, V, dtype=cd)
+    for b, _, _, s, e in chunk_spans(B, T, chunk, cu_seqlens):
+        L = e - s
+        doc, vc = do[b, :, s:e].to(cd), v_new[b, :, s:e].to(cd)
+        dA[b, :, s:e, :L] = torch.tril(torch.matmul(doc, vc.transpose(1, 2))) * scale
+        dv[b, :, s:e] = torch.matmul(torch.tril(Aqk[b, :, s:e, :L].to(cd)).transpose(1, 2), doc)
+    return dA, dv
+
+
+def chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, do, dh, dv, scale, chunk: int = 64, *, cu_seqlens=None,
+                        compute_dtype=torch.float32):
+    """Derivative of the parts of a chunk step that see the carried state:
+        o_inter = scale (q 2^g) h ;  v_new = u - w h ;  h' = diag(2^{g_last}) h + (k 2^{g_last - g})^T v_new
+    given do, dh = dL/dh' and dv = total dL/dv_new.  h, dh: [B,Hv,NT,K,V].  Returns per VALUE head
+        dq = scale (do h^T) 2^g ;  dk = (v_new dh^T) 2^{g_last - g} ;  dw = -dv h^T ;
+        dg = q dq - k dk, plus on the chunk's last token  sum_j k_j dk_j + 2^{g_last} rowsum(h . dh)."""
+    cd = compute_dtype
+    B, Hk, T, K = q.shape
+    Hv = do.shape[1]
+    rep = Hv // Hk
+    dq = torch.zeros(B, Hv, T, K, dtype=cd)
+    dk, dw, dg = torch.zeros_like(dq), torch.zeros_like(dq), torch.zeros_like(dq)
+    for b, _, ci, s, e in chunk_spans(B, T, chunk, cu_seqlens):
+        qc = q[b, :, s:e].to(cd).repeat_interleave(rep, dim=0)
+        kc = k[b, :, s:e].to(cd).repeat_interleave(rep, dim=0)
+        gc = gk[b, :, s:e].to(cd)
+        hc, dhc = h[b, :, ci].to(cd), dh[b, :, ci].to(cd)
+        glast = gc[:, -1:]
+        bdq = torch.matmul(do[b, :, s:e].to(cd), hc.transpose(1, 2)) * scale * torch.exp2(gc)
+        bdk = torch.matmul(v_new[b, :, s:e].to(cd), dhc.transpose(1, 2)) * torch.exp2(glast - gc)
+        bdg = qc * bdq - kc * bdk
+        bdg[:, -1] += (kc * bdk).sum(1) + torch.exp2(glast[:, 0]) * (hc * dhc).sum(-1)
+        dq[b, :, s:e], dk[b, :, s:e], dg[b, :, s:e] = bdq, bdk, bdg
+        dw[b, :, s:e] = -torch.matmul(dv[b, :, s:e].to(cd), hc.transpose(1, 2))
+    return dq, dk, dw, dg
+
+
+def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, chunk: int = 64, *, cu_seqlens=None, compute_dtype=torch.float32):
+    """Derivative of  w = Akk (k beta 2^g),  u = Akk (v beta),  Akk = (I + M)^-1  (M strictly lower):
+        dM  = -stril(Akk^T (dw (k beta 2^g)^T + du (v beta)^T) Akk^T)    [B,Hv,T,C]
+        x   = Akk^T dw ;  y = Akk^T du
+        dk  = x beta 2^g ;  dv = y beta ;  dbeta = <x, k 2^g> + <y, v> ;  dg = dk k.
+    Returns (dk, dv, dbeta, dg, dM) per value head."""
+    cd = compute_dtype
+    B, Hk, T, K = k.shape
+    Hv, V = v.shape[1], v.shape[3]
+    rep = Hv // Hk
+    dk = torch.zeros(B, Hv, T, K, dtype=cd)
+    dg = torch.zeros_like(dk)
+    dv = torch.zeros(B, Hv, T, V, dtype=cd)
+    db = torch.zeros(B, Hv, T, dtype=cd)
+    dM = torch.zeros(B, Hv, T, chunk, dtype=cd)
+    for b, _, _, s, e in chunk_spans(B, T, chunk, cu_seqlens):
+        L = e - s
+        kc = k[b, :, s:e].to(cd).repeat_interleave(rep, dim=0)
+        vc, bc, gc = v[b, :, s:e].to(cd), beta[b, :, s:e].to(cd), gk[b, :, s:e].to(cd)
+        A = torch.tril(Akk[b, :, s:e, :L].to(cd))
+        dwc, duc = dw[b, :, s:e].to(cd), du[b, :, s:e].to(cd)
+        eg = torch.exp2(gc)
+        kbg, vb = kc * bc[..., None] * eg, vc * bc[..., None]
+        dA = torch.tril(torch.matmul(dwc, kbg.transpose(1, 2)) + torch.matmul(duc, vb.transpose(1, 2)), -1)
+        At = A.transpose(1, 2)
+        dM[b, :, s:e, :L] = -torch.tril(torch.matmul(torch.matmul(At, dA), At), -1)
+        x, y = torch.matmul(At, dwc), torch.matmul(At, duc)
+        dk[b, :, s:e] = x * bc[..., None] * eg
+        dg[b, :, s:e] = dk[b, :, s:e] * kc
+        dv[b, :, s:e] = y * bc[..., None]
+        db[b, :, s:e] = (x * kc * eg).sum(-1) + (y * vc).sum(-1)
+    return dk, dv, db, dg, dM
+
+
+def chunk_kda_bwd(q, k, v, gate, beta, scale, do, *, chunk: int = 64, initial_state=None, dht=None, cu_seqlens=None,
+                  compute_dtype=torch.float32):
+    """Whole KDA chunk backward from the per-token natural-log gate: forward intermediates recomputed with
+    chunk_kda_fwd, then dav -> bwd_dhu (gK) -> dqkwg -> wy -> bwd_intra -> reverse chunk-local cumsum.
+    Head-major operands; returns (dq, dk [B,Hk,T,K], dv [B,Hv,T,V], dg [B,Hv,T,K], dbeta [B,Hv,T], dh0 [N,Hv,K,V])."""
+    cd = compute_dtype
+    B, Hk, T, K = q.shape
+    Hv = v.shape[1]
+    rep = Hv // Hk
+    gk = torch.empty(B, Hv, T, K, dtype=cd)
+    for b, _, _, s, e in chunk_spans(B, T, chunk, cu_seqlens):
+        gk[b, :, s:e] = torch.cumsum(gate[b, :, s:e].to(cd), dim=1) * RCP_LN2
+    f = chunk_kda_fwd(q, k, v, gk, beta, scale, chunk, initial_state=initial_state, cu_seqlens=cu_seqlens,
+                      compute_dtype=cd)
+    dAqk, dv0 = chunk_kda_bwd_dav(f["v_new"], do, f["Aqk"], scale, chunk, cu_seqlens=cu_seqlens, compute_dtype=cd)
+    dh, dh0, dv2 = chunk_gated_delta_rule_bwd_dhu(f["qg"], f["kg"], f["w"], do, dv0, scale, chunk, gK=gk, dht=dht,
+                                                  cu_seqlens=cu_seqlens, compute_dtype=cd)
+    dq, dk, dw, dg = chunk_kda_bwd_dqkwg(q, k, f["v_new"], gk, f["h"], do, dh, dv2, scale, chunk,
+                                         cu_seqlens=cu_seqlens, compute_dtype=cd)
+    dk2, dv, db, dg2, dM = chunk_kda_bwd_wy(k, v, beta, gk, f["Akk"], dw, dv2, chunk, cu_seqlens=cu_seqlens,
+                                            compute_dtype=cd)
+    qe = q.to(cd).repeat_interleave(rep, dim=1)
+    ke = k.to(cd).repeat_interleave(rep, dim=1)
+    dq, dk, db, dg = chunk_kda_bwd_intra(qe, ke, gk, beta, dAqk, dM, dq, dk + dk2, db, dg + dg2, chunk=chunk,
+                                         cu_seqlens=cu_seqlens, compute_dtype=cd)
+    for b, _, _, s, e in chunk_spans(B, T, chunk, cu_seqlens):
+        dg[b, :, s:e] = torch.flip(torch.cumsum(torch.flip(dg[b, :, s:e], dims=[1]), dim=1), dims=[1])
+    dq = dq.view(B, Hk, rep, T, K).sum(2)
+    dk = dk.view(B, Hk, rep, T, K).sum(2)
+    return dq, dk, dv, dg, db, dh0

@@ -1,0 +1,274 @@
+"""KDA chunk backward on the GPU (through the C ABI): the three chunk-parallel stages against the CPU oracle, and the
+whole composition (dq, dk, dv, dg, dbeta, dh0) against fp64 autograd through the per-token KDA recurrence.
+
+Tolerance: every gradient within 2e-2 of its own scale (max |error| <= 2e-2 * max |reference|) -- the activations and
+intermediates are 16-bit, the reductions fp32.  The stage tests feed the oracle the same 16-bit-rounded operands the
+kernels read, so only the kernels' own arithmetic is measured there."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gdn, kda
+from util import err_stats
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+REL = 2e-2
+
+
+def close(actual, expected, name, rel=REL):
+    st = err_stats(actual, expected)
+    assert torch.isfinite(actual.float()).all(), f"{name}: non-finite"
+    assert st["max_abs"] <= rel * max(st["max_ref"], 1e-6), f"{name}: {st}"
+    return st
+
+
+def amax(t):
+    return float(t.abs().max()) if t.numel() else 0.0
+
+
+def gate_cumsum(raw, cu=None):
+    out = torch.empty_like(raw)
+    for b, _, _, s, e in gdn.chunk_spans(raw.shape[0], raw.shape[2], 64, cu):
+        out[b, :, s:e] = torch.cumsum(raw[b, :, s:e], dim=1) * kda.RCP_LN2
+    return out
+
+
+def rnd(gen, *shape, scale=1.0, dtype=BF):
+    return (torch.randn(*shape, generator=gen) * scale).to(dtype)
+
+
+STAGE_CASES = [
+    # B, T, Hk, Hv, K, V, cu
+    (2, 128, 2, 2, 128, 128, None),
+    (1, 200, 2, 4, 128, 128, None),                                   # grouped value heads, ragged tail
+    (1, 261, 2, 2, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261]),       # packed, with an empty sequence
+    (1, 130, 1, 2, 64, 64, None),
+    (2, 70, 2, 2, 64, 128, None),
+]
+
+
+@pytest.mark.parametrize("case", STAGE_CASES)
+def test_bwd_dav(dev, case):
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, _, Hv, _, V, cu = case
+    gen = torch.Generator().manual_seed(T + V)
+    v_new, do = rnd(gen, B, Hv, T, V), rnd(gen, B, Hv, T, V)
+    Aqk = torch.zeros(B, Hv, T, 64)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        Aqk[b, :, s:e, :e - s] = torch.tril(torch.randn(Hv, e - s, e - s, generator=gen) * 0.3)
+    Aqk = Aqk.to(BF)
+    dA, dv = raw.chunk_kda_bwd_dav(v_new.to(dev), do.to(dev), Aqk.to(dev), 0.7, cu_seqlens=cu)
+    dA_ref, dv_ref = kda.chunk_kda_bwd_dav(v_new, do, Aqk, 0.7, cu_seqlens=cu)
+    assert dA.dtype == torch.float32 and dv.dtype == BF
+    close(dA, dA_ref, "dAqk", 1e-3)          # fp32 out of exact 16-bit products
+    close(dv, dv_ref, "dv")
+    # strictly above the diagonal, and past a ragged tail, the score gradient is exactly zero
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        blk = dA[b, :, s:e].cpu()
+        assert amax(torch.triu(blk[:, :, :e - s], 1)) == 0.0 and amax(blk[:, :, e - s:]) == 0.0
+
+
+@pytest.mark.parametrize("case", STAGE_CASES)
+def test_bwd_dqkwg(dev, case):
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, Hk, Hv, K, V, cu = case
+    gen = torch.Generator().manual_seed(T + K)
+    NT = gdn.total_chunks(B, T, 64, cu)
+    q, k = rnd(gen, B, Hk, T, K, scale=0.3), rnd(gen, B, Hk, T, K, scale=0.3)
+    v_new, do, dv = (rnd(gen, B, Hv, T, V) for _ in range(3))
+    gk = gate_cumsum(F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, cu)
+    h, dh = rnd(gen, B, Hv, NT, K, V, scale=0.5), rnd(gen, B, Hv, NT, K, V, scale=0.5)
+    to = lambda *ts: [t.to(dev) for t in ts]
+    dq, dk, dw, dg = raw.chunk_kda_bwd_dqkwg(*to(q, k, v_new, gk, h, do, dh, dv), 0.7, cu_seqlens=cu)
+    ref = kda.chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, do, dh, dv, 0.7, cu_seqlens=cu)
+    assert dq.dtype == dk.dtype == dg.dtype == torch.float32 and dw.dtype == BF
+    for name, a, e, rel in zip(("dq", "dk", "dw", "dg"), (dq, dk, dw, dg), ref, (1e-3, 1e-3, REL, 2e-3)):
+        close(a, e, name, rel)
+    # the same call with h / dh handed over sequence-major ([B,NT,Hv,K,V], as chunk_kda_fwd returns h) and the fp32
+    # results laid out token-major: views only, identical numbers
+    h_sm, dh_sm = h.transpose(1, 2).contiguous().to(dev), dh.transpose(1, 2).contiguous().to(dev)
+    like = torch.empty(B, T, Hv, K, device="meta").transpose(1, 2)
+    out2 = raw.chunk_kda_bwd_dqkwg(*to(q, k, v_new, gk), h_sm.transpose(1, 2), do.to(dev), dh_sm.transpose(1, 2), dv.to(dev),
+                                   0.7, cu_seqlens=cu, layout_like=like)
+    assert out2[0].transpose(1, 2).is_contiguous()
+    for a, e in zip(out2, (dq, dk, dw, dg)):
+        assert torch.equal(a, e)
+
+
+@pytest.mark.parametrize("case", STAGE_CASES)
+def test_bwd_wy(dev, case):
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, Hk, Hv, K, V, cu = case
+    gen = torch.Generator().manual_seed(T + 2 * K)
+    k, v = rnd(gen, B, Hk, T, K, scale=0.3), rnd(gen, B, Hv, T, V)
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    gk = gate_cumsum(F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, cu)
+    dw, du = rnd(gen, B, Hv, T, K), rnd(gen, B, Hv, T, V)
+    Akk = torch.zeros(B, Hv, T, 64)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        L = e - s
+        M = torch.tril(torch.randn(Hv, L, L, generator=gen) * 0.1, -1)
+        Akk[b, :, s:e, :L] = torch.linalg.inv(torch.eye(L) + M)
+    Akk = Akk.to(BF)
+    dk0, dg0 = torch.randn(B, Hv, T, K, generator=gen), torch.randn(B, Hv, T, K, generator=gen)
+    dk, dg = dk0.to(dev), dg0.to(dev)
+    to = lambda *ts: [t.to(dev) for t in ts]
+    dv, db, dM = raw.chunk_kda_bwd_wy(*to(k, v, beta, gk, Akk, dw, du), dk, dg, cu_seqlens=cu)
+    dk_r, dv_r, db_r, dg_r, dM_r = kda.chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, cu_seqlens=cu)
+    close(dk.cpu() - dk0, dk_r, "dk (added)", 2e-3)
+    close(dg.cpu() - dg0, dg_r, "dg (added)", 2e-3)
+    close(dv, dv_r, "dv")
+    close(db, db_r, "dbeta", 2e-3)
+    close(dM, dM_r, "dAkk")               # the chain through the inverse rounds two 64x64 intermediates to 16 bits
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        blk = dM[b, :, s:e].cpu()
+        assert amax(torch.triu(blk[:, :, :e - s], 0)) == 0.0 and amax(blk[:, :, e - s:]) == 0.0
+
+
+# ---------------------------------------------------------------------------------------------
+# composition
+# ---------------------------------------------------------------------------------------------
+def lay(x, layout):
+    """head-major [B,H,T,..] -> layout"""
+    if layout == "BNSD":
+        return x.contiguous()
+    if layout == "BSND":
+        return x.transpose(1, 2).contiguous()
+    if layout == "NTD":
+        return x[0].contiguous()
+    return x[0].transpose(0, 1).contiguous()
+
+
+def unlay(x, layout):
+    if layout == "BNSD":
+        return x
+    if layout == "BSND":
+        return x.transpose(1, 2)
+    if layout == "NTD":
+        return x[None]
+    return x.transpose(0, 1)[None]
+
+
+def autograd_truth(q, k, v, gate, beta, scale, do, h0, dht, cu):
+    """fp64 autograd through the per-token recurrence on the 16-bit-rounded inputs (head-major)."""
+    dd = torch.float64
+    leaves = [t.to(dd).requires_grad_(True) for t in (q, k, v, gate, beta)]
+    h0d = None if h0 is None else h0.to(dd).requires_grad_(True)
+    o, final = kda.naive_recurrent_kda(*leaves, scale, initial_state=h0d, output_final_state=True, cu_seqlens=cu,
+                                       compute_dtype=dd)
+    loss = (o * do.to(dd)).sum()
+    if dht is not None:
+        loss = loss + (final * dht.to(dd)).sum()
+    loss.backward()
+    return [t.grad for t in leaves] + [None if h0d is None else h0d.grad]
+
+
+COMPOSITION_CASES = [
+    dict(B=2, T=192, Hk=2, Hv=2, K=128, V=128, layout="BSND", h0=True, dht=True),
+    dict(B=1, T=200, Hk=2, Hv=4, K=128, V=128, layout="BNSD", h0=True, dht=True),             # grouped heads, ragged tail
+    dict(B=1, T=261, Hk=2, Hv=2, K=128, V=128, layout="TND", cu=[0, 1, 16, 33, 33, 96, 160, 261], h0=True, dht=True),
+    dict(B=1, T=130, Hk=1, Hv=2, K=64, V=64, layout="NTD", cu=[0, 65, 130]),
+    dict(B=2, T=100, Hk=2, Hv=2, K=64, V=128, layout="BSND", dht=True),
+    dict(B=1, T=128, Hk=1, Hv=1, K=128, V=128, layout="BSND", gate_scale=2.0, h0=True),       # strong decay
+    dict(B=1, T=150, Hk=2, Hv=2, K=128, V=128, layout="BSND", dtype=torch.float16, h0=True, dht=True),
+]
+
+
+@pytest.mark.parametrize("case", COMPOSITION_CASES)
+def test_chunk_kda_backward_against_autograd_through_the_recurrence(dev, case):
+    from fla_hip import pipeline
+    B, T, Hk, Hv, K, V = (case[n] for n in ("B", "T", "Hk", "Hv", "K", "V"))
+    layout, cu, dtype = case["layout"], case.get("cu"), case.get("dtype", BF)
+    gen = torch.Generator().manual_seed(T + Hv)
+    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(dtype)
+    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(dtype)
+    v = torch.randn(B, Hv, T, V, generator=gen).to(dtype)
+    gate = F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * case.get("gate_scale", 0.5)
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    do = torch.randn(B, Hv, T, V, generator=gen).to(dtype)
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, Hv, K, V, generator=gen) * 0.1 if case.get("h0") else None
+    dht = torch.randn(N, Hv, K, V, generator=gen) * 0.1 if case.get("dht") else None
+    scale = K ** -0.5
+
+    ins = [lay(t, layout).to(dev).requires_grad_(True) for t in (q, k, v, gate, beta)]
+    h0_d = None if h0 is None else h0.to(dev).requires_grad_(True)
+    o, final = pipeline.chunk_kda(*ins, scale, h0_d, True, cu, layout=layout)
+    loss = (o.float() * lay(do, layout).to(dev).float()).sum()
+    if dht is not None:
+        loss = loss + (final * dht.to(dev)).sum()
+    loss.backward()
+    want = autograd_truth(q, k, v, gate, beta, scale, do, h0, dht, cu)
+    got = [unlay(t.grad, layout) for t in ins] + [None if h0_d is None else h0_d.grad]
+    assert ins[0].grad.dtype == dtype and ins[3].grad.dtype == torch.float32 and ins[0].grad.shape == ins[0].shape
+    stats = {}
+    for name, a, e in zip(("dq", "dk", "dv", "dg", "dbeta", "dh0"), got, want):
+        if e is None:
+            assert a is None
+            continue
+        stats[name] = close(a, e, name)["rel_max"]
+    print(f"\n[kda bwd {layout} T={T} Hv={Hv} K={K} V={V}] rel_max " + " ".join(f"{n}={s:.1e}" for n, s in stats.items()))
+
+
+def test_chunk_kda_backward_at_the_bench_shape(dev):
+    """B=2 T=8192 H=32 K=V=128 (the KDA configuration of the benchmark): (a) a second run gives the same bits;
+    (b) one (batch, head) slice equals fp64 autograd through the 8192-step recurrence; (c) hand-off: the backward of
+    the second half seeded with dht, followed by the backward of the first half seeded with that call's dh0, equals
+    the backward over the whole sequence."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 2, 8192, 32, 128, 128
+    gen = torch.Generator().manual_seed(0)
+    q = F.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).to(BF)
+    k = F.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).to(BF)
+    v = torch.randn(B, T, H, V, generator=gen).to(BF)
+    gate = F.logsigmoid(torch.randn(B, T, H, K, generator=gen))
+    beta = torch.sigmoid(torch.randn(B, T, H, generator=gen))
+    do = torch.randn(B, T, H, V, generator=gen).to(BF)
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.01
+    h0 = torch.randn(B, H, K, V, generator=gen) * 0.01
+    scale = K ** -0.5
+
+    def run(sl, init, seed_grad):
+        ins = [t[:, sl].to(dev).requires_grad_(True) for t in (q, k, v, gate, beta)]
+        init_d = init.to(dev).requires_grad_(True)
+        o, final = pipeline.chunk_kda(*ins, scale, init_d, True)
+        ((o.float() * do[:, sl].to(dev).float()).sum() + (final * seed_grad.to(dev)).sum()).backward()
+        return [t.grad for t in ins] + [init_d.grad], final.detach()
+
+    whole, _ = run(slice(0, T), h0, dht)
+    again, _ = run(slice(0, T), h0, dht)
+    for a, e in zip(whole, again):
+        assert torch.equal(a, e), "the backward is not deterministic"
+    # (b) slice (batch 1, head 5)
+    b, h = 1, 5
+    hm = lambda t: t[b:b + 1, :, h:h + 1].transpose(1, 2)
+    want = autograd_truth(hm(q), hm(k), hm(v), hm(gate), beta[b:b + 1, :, h:h + 1].transpose(1, 2), scale, hm(do),
+                          h0[b:b + 1, h:h + 1], dht[b:b + 1, h:h + 1], None)
+    names = ("dq", "dk", "dv", "dg", "dbeta", "dh0")
+    stats = {}
+    for name, a, e in zip(names[:4], whole[:4], want[:4]):
+        stats[name] = close(a[b:b + 1, :, h:h + 1].transpose(1, 2), e, name)["rel_max"]
+    stats["dbeta"] = close(whole[4][b:b + 1, :, h:h + 1].transpose(1, 2), want[4], "dbeta")["rel_max"]
+    stats["dh0"] = close(whole[5][b:b + 1, h:h + 1], want[5], "dh0")["rel_max"]
+    print("\n[kda bwd B=2 T=8192 H=32] slice rel_max " + " ".join(f"{n}={s:.1e}" for n, s in stats.items()))
+    # (c) hand-off at the middle
+    half = T // 2
+    _, mid_state = run(slice(0, half), h0, torch.zeros_like(dht))
+    second, _ = run(slice(half, T), mid_state.cpu(), dht)
+    first, _ = run(slice(0, half), h0, second[5].cpu())
+    for i, name in enumerate(names[:5]):
+        joined = torch.cat([first[i], second[i]], dim=1)
+        close(joined, whole[i].float().cpu(), f"hand-off {name}", 5e-3)
+    close(first[5], whole[5].cpu(), "hand-off dh0", 5e-3)
+
+
+def test_chunk_kda_rejections(dev):
+    from fla_hip import pipeline
+    q = torch.zeros(1, 64, 1, 128, dtype=BF, device=dev, requires_grad=True)
+    g = torch.zeros(1, 64, 1, 128, device=dev)
+    beta = torch.ones(1, 64, 1, device=dev)
+    with pytest.raises(NotImplementedError, match="chunk_size 64"):
+        pipeline.chunk_kda(q, q, q, g, beta, chunk_size=128)

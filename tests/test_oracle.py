@@ -276,6 +276,119 @@ def test_bwd_intra_against_autograd_and_anchored_evaluation():
     assert torch.allclose(dg, gk.grad / math.log(2.0), atol=1e-9)   # dg is the gradient w.r.t. ln2 * gk
 
 
+def _cumsum_log2(raw, C, cu=None):
+    out = torch.empty_like(raw)
+    for b, _, _, s, e in gdn.chunk_spans(raw.shape[0], raw.shape[2], C, cu):
+        out[b, :, s:e] = torch.cumsum(raw[b, :, s:e], dim=1) / math.log(2.0)
+    return out
+
+
+@pytest.mark.parametrize("cu", [None, [0, 70, 70, 150]])
+def test_kda_bwd_dav_against_autograd(cu):
+    """dAqk and dv are the gradients of o_intra = (scale tril(S)) v_new with respect to S and v_new."""
+    gen = torch.Generator().manual_seed(21)
+    B, H, T, V, C, dd = 1, 2, 150, 6, 64, torch.float64
+    S = torch.randn(B, H, T, C, generator=gen, dtype=dd).requires_grad_(True)
+    vn = torch.randn(B, H, T, V, generator=gen, dtype=dd).requires_grad_(True)
+    do = torch.randn(B, H, T, V, generator=gen, dtype=dd)
+    loss, Aqk = 0.0, torch.zeros(B, H, T, C, dtype=dd)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, C, cu):
+        L = e - s
+        A = torch.tril(S[b, :, s:e, :L]) * 0.7
+        Aqk[b, :, s:e, :L] = A.detach()
+        loss = loss + ((A @ vn[b, :, s:e]) * do[b, :, s:e]).sum()
+    loss.backward()
+    dA, dv = kda.chunk_kda_bwd_dav(vn.detach(), do, Aqk, 0.7, C, cu_seqlens=cu, compute_dtype=dd)
+    assert torch.allclose(dA, S.grad, atol=1e-10) and torch.allclose(dv, vn.grad, atol=1e-10)
+
+
+@pytest.mark.parametrize("cu,rep", [(None, 1), ([0, 70, 70, 150], 2)])
+def test_kda_bwd_dqkwg_against_autograd(cu, rep):
+    """dq, dk, dw, dg are the gradients of one chunk step's state-dependent parts with h, dh, dv given."""
+    gen = torch.Generator().manual_seed(22)
+    B, Hk, T, K, V, C, dd = 1, 2, 150, 8, 6, 64, torch.float64
+    Hv = Hk * rep
+    NT = gdn.total_chunks(B, T, C, cu)
+    q = torch.randn(B, Hk, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    k = torch.randn(B, Hk, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    w = torch.randn(B, Hv, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    gk = _cumsum_log2(-torch.rand(B, Hv, T, K, generator=gen, dtype=dd) * 0.2, C, cu).requires_grad_(True)
+    vn, do, dv = (torch.randn(B, Hv, T, V, generator=gen, dtype=dd) for _ in range(3))
+    h, dh = (torch.randn(B, Hv, NT, K, V, generator=gen, dtype=dd) for _ in range(2))
+    loss = 0.0
+    for b, _, ci, s, e in gdn.chunk_spans(B, T, C, cu):
+        qc = q[b, :, s:e].repeat_interleave(rep, dim=0)
+        kc = k[b, :, s:e].repeat_interleave(rep, dim=0)
+        gc = gk[b, :, s:e]
+        o = 0.7 * (qc * torch.exp2(gc)) @ h[b, :, ci]
+        h_next = torch.exp2(gc[:, -1])[..., None] * h[b, :, ci] + (kc * torch.exp2(gc[:, -1:] - gc)).transpose(1, 2) @ vn[b, :, s:e]
+        loss = loss + (o * do[b, :, s:e]).sum() + (h_next * dh[b, :, ci]).sum() - ((w[b, :, s:e] @ h[b, :, ci]) * dv[b, :, s:e]).sum()
+    loss.backward()
+    dq, dk, dw, dg = kda.chunk_kda_bwd_dqkwg(q.detach(), k.detach(), vn, gk.detach(), h, do, dh, dv, 0.7, C, cu_seqlens=cu,
+                                             compute_dtype=dd)
+    fold = lambda x: x.view(B, Hk, rep, T, K).sum(2)
+    assert torch.allclose(fold(dq), q.grad, atol=1e-9) and torch.allclose(fold(dk), k.grad, atol=1e-9)
+    assert torch.allclose(dw, w.grad, atol=1e-9)
+    assert torch.allclose(dg, gk.grad / math.log(2.0), atol=1e-9)
+
+
+@pytest.mark.parametrize("cu,rep", [(None, 1), ([0, 70, 70, 150], 2)])
+def test_kda_bwd_wy_against_autograd(cu, rep):
+    """dk, dv, dbeta, dg, dM are the gradients of w = (I+M)^-1 (k beta 2^g), u = (I+M)^-1 (v beta), M an independent
+    strictly lower matrix."""
+    gen = torch.Generator().manual_seed(23)
+    B, Hk, T, K, V, C, dd = 1, 2, 150, 8, 6, 64, torch.float64
+    Hv = Hk * rep
+    k = torch.randn(B, Hk, T, K, generator=gen, dtype=dd).requires_grad_(True)
+    v = torch.randn(B, Hv, T, V, generator=gen, dtype=dd).requires_grad_(True)
+    beta = torch.rand(B, Hv, T, generator=gen, dtype=dd).requires_grad_(True)
+    gk = _cumsum_log2(-torch.rand(B, Hv, T, K, generator=gen, dtype=dd) * 0.2, C, cu).requires_grad_(True)
+    M = (torch.randn(B, Hv, T, C, generator=gen, dtype=dd) * 0.2).requires_grad_(True)
+    dw = torch.randn(B, Hv, T, K, generator=gen, dtype=dd)
+    du = torch.randn(B, Hv, T, V, generator=gen, dtype=dd)
+    loss, Akk = 0.0, torch.zeros(B, Hv, T, C, dtype=dd)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, C, cu):
+        L = e - s
+        A = torch.linalg.inv(torch.eye(L, dtype=dd) + torch.tril(M[b, :, s:e, :L], -1))
+        Akk[b, :, s:e, :L] = A.detach()
+        kc = k[b, :, s:e].repeat_interleave(rep, dim=0)
+        bc = beta[b, :, s:e, None]
+        loss = loss + ((A @ (kc * bc * torch.exp2(gk[b, :, s:e]))) * dw[b, :, s:e]).sum() + ((A @ (v[b, :, s:e] * bc)) * du[b, :, s:e]).sum()
+    loss.backward()
+    dk, dv, db, dg, dM = kda.chunk_kda_bwd_wy(k.detach(), v.detach(), beta.detach(), gk.detach(), Akk, dw, du, C,
+                                              cu_seqlens=cu, compute_dtype=dd)
+    assert torch.allclose(dk.view(B, Hk, rep, T, K).sum(2), k.grad, atol=1e-9)
+    assert torch.allclose(dv, v.grad, atol=1e-9) and torch.allclose(db, beta.grad, atol=1e-9)
+    assert torch.allclose(dg, gk.grad / math.log(2.0), atol=1e-9)
+    assert torch.allclose(dM, M.grad, atol=1e-9)
+
+
+@pytest.mark.parametrize("cu,rep", [(None, 1), ([0, 70, 70, 150], 2), ([0, 5, 133], 1)])
+def test_kda_bwd_composition_against_autograd_through_the_recurrence(cu, rep):
+    """The whole chunked backward (every gradient, with an initial state and a final-state gradient) equals fp64
+    autograd through the per-token KDA recurrence."""
+    gen = torch.Generator().manual_seed(24)
+    T = cu[-1] if cu else 150
+    B, Hk, K, V, dd = 1, 2, 8, 6, torch.float64
+    Hv = Hk * rep
+    N = len(cu) - 1 if cu else B
+    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen, dtype=dd), dim=-1).requires_grad_(True)
+    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen, dtype=dd), dim=-1).requires_grad_(True)
+    v = torch.randn(B, Hv, T, V, generator=gen, dtype=dd).requires_grad_(True)
+    gate = (F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen, dtype=dd)) * 0.5).requires_grad_(True)
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen, dtype=dd)).requires_grad_(True)
+    h0 = (torch.randn(N, Hv, K, V, generator=gen, dtype=dd) * 0.3).requires_grad_(True)
+    do = torch.randn(B, Hv, T, V, generator=gen, dtype=dd)
+    dht = torch.randn(N, Hv, K, V, generator=gen, dtype=dd)
+    o, final = kda.naive_recurrent_kda(q, k, v, gate, beta, 0.7, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                                       compute_dtype=dd)
+    ((o * do).sum() + (final * dht).sum()).backward()
+    got = kda.chunk_kda_bwd(q.detach(), k.detach(), v.detach(), gate.detach(), beta.detach(), 0.7, do, initial_state=h0.detach(),
+                            dht=dht, cu_seqlens=cu, compute_dtype=dd)
+    for name, a, e in zip(("dq", "dk", "dv", "dg", "dbeta", "dh0"), got, (q.grad, k.grad, v.grad, gate.grad, beta.grad, h0.grad)):
+        assert torch.allclose(a, e, atol=1e-8), f"{name}: {float((a - e).abs().max())}"
+
+
 # ----------------------------------------------------------------------------
 # GDN backward chain: every operator against autograd of the stage it differentiates (fp64)
 # ----------------------------------------------------------------------------
