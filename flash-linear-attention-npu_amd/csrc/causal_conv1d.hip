@@ -13,10 +13,7 @@
 namespace fla {
 namespace {
 
-#ifndef FLA_CONV_THREADS
-#define FLA_CONV_THREADS 128
-#endif
-constexpr int kThreads = FLA_CONV_THREADS;
+constexpr int kThreads = 128;
 constexpr int kMaxW = 4;
 
 struct ConvParams {
@@ -42,11 +39,7 @@ struct ConvParams {
 };
 
 template <typename T> __device__ __forceinline__ void load8(const T *p, float (&f)[8]) {
-#ifdef FLA_CONV_NT_LOAD
-    typename Vec8<T>::type v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec8<T>::type *>(p));
-#else
     typename Vec8<T>::type v = *reinterpret_cast<const typename Vec8<T>::type *>(p);
-#endif
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
 }
@@ -59,11 +52,7 @@ template <typename T> __device__ __forceinline__ void store8(T *p, const float (
     typename Vec8<T>::type v;
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (T)f[i];
-#ifdef FLA_CONV_NT_STORE
-    __builtin_nontemporal_store(v, reinterpret_cast<typename Vec8<T>::type *>(p));
-#else
     *reinterpret_cast<typename Vec8<T>::type *>(p) = v;
-#endif
 }
 
 __device__ __forceinline__ int find_seq(const int32_t *qsl, int N, int t) {
@@ -381,6 +370,13 @@ __global__ void conv1d_update_kernel(const ConvUpdateParams p) {
     }
 }
 
+// The kernels move 16-byte pieces: every row must start on a 16-byte boundary.
+bool aligned(const fla_tensor *t) {
+    for (int i = 0; i + 1 < t->ndim; ++i)
+        if (t->stride[i] % 8 != 0) return false;
+    return reinterpret_cast<uintptr_t>(t->data) % 16 == 0;
+}
+
 int copy_int_array(std::vector<int32_t> &dst, const fla_int_array *a) {
     dst.clear();
     if (a == nullptr || a->data == nullptr) return 0;
@@ -419,11 +415,6 @@ int conv_update_impl(const fla_tensor *x, const fla_tensor *weight, const fla_te
     FLA_REQUIRE(state_len >= W - 1 && conv_states->shape[2] == D && inner_unit(conv_states), FLA_ERR_SHAPE,
                 "%s: conv_states must be [N, >=W-1, D] with unit channel stride.", op);
 
-    const auto aligned = [](const fla_tensor *t) {
-        for (int i = 0; i + 1 < t->ndim; ++i)
-            if (t->stride[i] % 8 != 0) return false;
-        return reinterpret_cast<uintptr_t>(t->data) % 16 == 0;
-    };
     FLA_REQUIRE(aligned(x) && aligned(out) && aligned(weight) && aligned(conv_states), FLA_ERR_SHAPE,
                 "%s: rows of x, out, weight and conv_states must be 16-byte aligned.", op);
     std::vector<int32_t> qsl, cache, nat;
@@ -435,6 +426,11 @@ int conv_update_impl(const fla_tensor *x, const fla_tensor *weight, const fla_te
         S = x->shape[1];
         FLA_REQUIRE(!has_qsl || (int64_t)query_start_loc->size == N + 1, FLA_ERR_METADATA,
                     "%s: query_start_loc.size must equal batch + 1.", op);
+        if (has_qsl)   // a [B,S,D] batch has S tokens per sequence: any other segmentation would be silently ignored
+            for (int64_t i = 0; i <= N; ++i)
+                FLA_REQUIRE(query_start_loc->data[i] == i * S, FLA_ERR_METADATA,
+                            "%s: with a rank-3 x, query_start_loc must be [0, S, 2S, ...]; pack the tokens as [T,D] for "
+                            "ragged sequences.", op);
     } else if (has_qsl && (int64_t)query_start_loc->size - 1 != x->shape[0]) {
         packed = true;                     // 2-D varlen decode: segments of a packed token axis
         N = (int64_t)query_start_loc->size - 1;
@@ -553,9 +549,12 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
     FLA_REQUIRE(inner_unit(x) && inner_unit(weight) && inner_unit(out), FLA_ERR_SHAPE,
                 "%s: innermost stride of x, weight and out must be 1.", op);
     FLA_REQUIRE(B * S < ((int64_t)1 << 31) && D < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents exceed int32.", op);
+    FLA_REQUIRE(aligned(x) && aligned(out) && aligned(weight), FLA_ERR_SHAPE,
+                "%s: rows of x, out and weight must be 16-byte aligned.", op);
     if (bias && bias->data) {
         if ((rc = check_tensor(bias, op, "bias", 1, dt_bit(x->dtype)))) return rc;
-        FLA_REQUIRE(bias->shape[0] == D && inner_unit(bias), FLA_ERR_SHAPE, "%s: bias must be a contiguous [D].", op);
+        FLA_REQUIRE(bias->shape[0] == D && inner_unit(bias) && aligned(bias), FLA_ERR_SHAPE,
+                    "%s: bias must be a contiguous, 16-byte aligned [D].", op);
     }
     FLA_REQUIRE(head_num >= 0, FLA_ERR_SHAPE, "%s: head_num must be >= 0.", op);
     int64_t head_dim = D;
@@ -589,6 +588,7 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
         if ((rc = check_tensor(conv_states, op, "conv_states", 3, dt_bit(x->dtype)))) return rc;
         FLA_REQUIRE(conv_states->shape[1] >= W - 1 && conv_states->shape[2] == D && inner_unit(conv_states),
                     FLA_ERR_SHAPE, "%s: conv_states must be [N, >=W-1, D] with unit channel stride.", op);
+        FLA_REQUIRE(aligned(conv_states), FLA_ERR_SHAPE, "%s: rows of conv_states must be 16-byte aligned.", op);
         for (int i = 0; i < N; ++i) {
             const int64_t slot = cache.empty() ? i : cache[i];
             FLA_REQUIRE(slot == pad_slot_id || (slot >= 0 && slot < conv_states->shape[0]), FLA_ERR_METADATA,
@@ -663,10 +663,6 @@ int conv_impl(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *b
     {
         const int64_t col_blocks = (D / 8 + kThreads - 1) / kThreads;
         while (tok > 8 && ((B * S + tok - 1) / tok) * col_blocks < (int64_t)24 * num_cus()) tok >>= 1;
-        if (const char *env = getenv("FLA_HIP_CONV_TOK")) {
-            const int v = atoi(env);
-            if (v == 8 || v == 16 || v == 32 || v == 64) tok = v;
-        }
     }
     p.tok = tok;
     p.tiles_per_seq = (int)((S + tok - 1) / tok);
@@ -739,9 +735,9 @@ extern "C" int fla_causal_conv1d_get_workspace_size(
     const fla_int_array *num_accepted_tokens, int64_t activation_mode, int64_t pad_slot_id, int64_t run_mode,
     int64_t head_num, const fla_tensor *out, uint64_t *workspace_size) {
     if (workspace_size == nullptr) return fla::fail(FLA_ERR_NULL, "causal_conv1d: workspace_size must not be null.");
-    return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
+    return fla::guarded([&] { return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
                           num_accepted_tokens, activation_mode, pad_slot_id, run_mode, head_num, out, nullptr, 0,
-                          nullptr, workspace_size);
+                          nullptr, workspace_size); });
 }
 
 extern "C" int fla_causal_conv1d(const fla_tensor *x, const fla_tensor *weight, const fla_tensor *bias,
@@ -750,7 +746,7 @@ extern "C" int fla_causal_conv1d(const fla_tensor *x, const fla_tensor *weight, 
                                  const fla_int_array *num_accepted_tokens, int64_t activation_mode,
                                  int64_t pad_slot_id, int64_t run_mode, int64_t head_num, const fla_tensor *out,
                                  void *workspace, uint64_t workspace_size, void *stream) {
-    return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
+    return fla::guarded([&] { return fla::conv_impl(x, weight, bias, conv_states, query_start_loc, cache_indices, initial_state_mode,
                           num_accepted_tokens, activation_mode, pad_slot_id, run_mode, head_num, out, workspace,
-                          workspace_size, static_cast<hipStream_t>(stream), nullptr);
+                          workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

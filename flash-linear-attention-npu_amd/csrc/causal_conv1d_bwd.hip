@@ -514,14 +514,14 @@ extern "C" int fla_causal_conv1d_bwd_get_workspace_size(
     const fla_tensor *dht, const fla_int_array *query_start_loc, int64_t activation, const char *input_layout,
     const fla_tensor *dx, const fla_tensor *dw, const fla_tensor *db, const fla_tensor *dh0, uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "causal_conv1d_bwd: workspace_size must not be null.");
-    return fla::conv_bwd_impl(x, y, weight, dy, initial_state, dht, query_start_loc, activation, input_layout, dx, dw, db, dh0,
-                              nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::conv_bwd_impl(x, y, weight, dy, initial_state, dht, query_start_loc, activation, input_layout, dx, dw, db, dh0,
+                              nullptr, 0, nullptr, workspace_size); });
 }
 extern "C" int fla_causal_conv1d_bwd(
     const fla_tensor *x, const fla_tensor *y, const fla_tensor *weight, const fla_tensor *dy, const fla_tensor *initial_state,
     const fla_tensor *dht, const fla_int_array *query_start_loc, int64_t activation, const char *input_layout,
     const fla_tensor *dx, const fla_tensor *dw, const fla_tensor *db, const fla_tensor *dh0, void *workspace,
     uint64_t workspace_size, void *stream) {
-    return fla::conv_bwd_impl(x, y, weight, dy, initial_state, dht, query_start_loc, activation, input_layout, dx, dw, db, dh0,
-                              workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::conv_bwd_impl(x, y, weight, dy, initial_state, dht, query_start_loc, activation, input_layout, dx, dw, db, dh0,
+                              workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

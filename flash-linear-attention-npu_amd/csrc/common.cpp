@@ -123,6 +123,14 @@ Ring g_rings[16];
 
 int stage_to_device(void *dst, const void *src, size_t bytes, hipStream_t stream) {
     if (bytes == 0) return FLA_OK;
+    // A captured copy would be replayed from a pinned slot that later calls recycle, i.e. with other calls' metadata,
+    // never validated for the replayed launch; and the slot's event would belong to the capture.  Calls that carry host
+    // integer arrays therefore stay out of graphs.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+        return fail(FLA_ERR_UNSUPPORTED,
+                    "host integer arrays (cu_seqlens, chunk_indices, query_start_loc, cache_indices, ...) cannot be uploaded "
+                    "while the stream is being captured; keep this call out of the graph.");
     int dev = 0;
     FLA_HIP_CHECK(hipGetDevice(&dev));
     if (dev < 0 || dev >= 16) return fail(FLA_ERR_UNSUPPORTED, "device index %d out of range.", dev);
@@ -131,8 +139,8 @@ int stage_to_device(void *dst, const void *src, size_t bytes, hipStream_t stream
     Slot &s = ring.slots[ring.next];
     ring.next = (ring.next + 1) % 16;
     if (s.busy) {
+        s.busy = false;   // cleared first: a failed wait must not wedge the slot for every later call
         FLA_HIP_CHECK(hipEventSynchronize(s.ev));
-        s.busy = false;
     }
     if (s.cap < bytes) {
         if (s.host) FLA_HIP_CHECK(hipHostFree(s.host));
@@ -175,13 +183,25 @@ bool g_prof_on = false;
 }  // namespace
 
 bool profile_enabled() { return g_prof_on; }
+int profile_report_impl(char *buf, uint64_t cap);
 
-void profile_begin(const char *name, hipStream_t stream) {
+bool profile_begin(const char *name, hipStream_t stream) {
     ProfRec r{name, nullptr, nullptr};
-    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) return;
+    if (hipEventCreate(&r.start) != hipSuccess) return false;
+    if (hipEventCreate(&r.stop) != hipSuccess) {
+        (void)hipEventDestroy(r.start);
+        return false;
+    }
     (void)hipEventRecord(r.start, stream);
-    std::lock_guard<std::mutex> lock(g_prof_mu);
-    g_prof.push_back(r);
+    try {
+        std::lock_guard<std::mutex> lock(g_prof_mu);
+        g_prof.push_back(r);
+    } catch (...) {   // no room for the record: this launch goes untimed
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+        return false;
+    }
+    return true;
 }
 
 void profile_end(hipStream_t stream) {
@@ -196,6 +216,12 @@ extern "C" void fla_profile_enable(int on) { fla::g_prof_on = on != 0; }
 // Waits for every recorded launch, writes one "name count total_ms" line per kernel
 // name into buf (NUL-terminated, truncated to cap) and clears the records.
 extern "C" int fla_profile_report(char *buf, uint64_t cap) {
+    const int names = fla::guarded([&] { return fla::profile_report_impl(buf, cap); });
+    return names;
+}
+
+namespace fla {
+int profile_report_impl(char *buf, uint64_t cap) {
     std::lock_guard<std::mutex> lock(fla::g_prof_mu);
     struct Agg { const char *name; int n; double ms; };
     std::vector<Agg> agg;
@@ -221,6 +247,7 @@ extern "C" int fla_profile_report(char *buf, uint64_t cap) {
     }
     return (int)agg.size();
 }
+}  // namespace fla
 
 extern "C" const char *fla_last_error(void) { return fla::last_error_buffer(); }
 extern "C" int fla_abi_version(void) { return 1; }

@@ -8,6 +8,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <exception>
+#include <new>
 #include <vector>
 
 #include "../../include/fla_hip.h"
@@ -29,6 +31,20 @@ int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)))
         if (err__ != hipSuccess)                                                      \
             return ::fla::fail(FLA_ERR_LAUNCH, "%s failed: %s", #expr, hipGetErrorString(err__)); \
     } while (0)
+
+// Every extern "C" entry point runs its body through this: host-side bookkeeping uses std::vector and a mutex, and
+// nothing they throw may cross the C boundary.
+template <typename F> inline int guarded(F &&body) noexcept {
+    try {
+        return body();
+    } catch (const std::bad_alloc &) {
+        return fail(FLA_ERR_HOST, "host memory allocation failed inside the call.");
+    } catch (const std::exception &e) {
+        return fail(FLA_ERR_HOST, "host-side failure inside the call: %s", e.what());
+    } catch (...) {
+        return fail(FLA_ERR_HOST, "unknown host-side failure inside the call.");
+    }
+}
 
 // ---- tensor descriptor helpers --------------------------------------------
 inline size_t dtype_size(int dt) {
@@ -98,13 +114,13 @@ int num_cus();
 // its launch with two HIP events on the launch stream; fla_profile_report()
 // synchronises them and returns "name count total_ms" lines.
 bool profile_enabled();
-void profile_begin(const char *name, hipStream_t stream);
+bool profile_begin(const char *name, hipStream_t stream);   // false: nothing was recorded
 void profile_end(hipStream_t stream);
 struct ProfileScope {
     hipStream_t s;
     bool on;
     ProfileScope(const char *name, hipStream_t stream) : s(stream), on(profile_enabled()) {
-        if (on) profile_begin(name, s);
+        if (on) on = profile_begin(name, s);
     }
     ~ProfileScope() {
         if (on) profile_end(s);

@@ -827,16 +827,16 @@ FLA_ENTRY(fla_chunk_bwd_dv_local_get_workspace_size)(
     int64_t chunk_size, const fla_tensor *out, uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_bwd_dv_local_get_workspace_size, q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_bwd_dv_local");
-    return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0,
-                              nullptr, workspace_size);
+    return fla::guarded([&] { return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0,
+                              nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_bwd_dv_local)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g, const fla_tensor *g_gamma,
     const fla_tensor *A, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
     int64_t chunk_size, const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_bwd_dv_local, q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size, stream);
-    return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace,
-                              workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::dv_local_impl(q, k, d_o, g, g_gamma, A, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace,
+                              workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_bwd_dqkwg_get_workspace_size)(
@@ -847,8 +847,8 @@ FLA_ENTRY(fla_chunk_bwd_dqkwg_get_workspace_size)(
     const fla_tensor *dg, uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg_get_workspace_size, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2, transpose_state_layout, dq, dk, dw, dg, workspace_size);
     FLA_NULL_WS("chunk_bwd_dqkwg");
-    return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
-                           transpose_state_layout, dq, dk, dw, dg, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
+                           transpose_state_layout, dq, dk, dw, dg, nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_bwd_dqkwg)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
@@ -857,9 +857,9 @@ FLA_ENTRY(fla_chunk_bwd_dqkwg)(
     bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
     const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2, transpose_state_layout, dq, dk, dw, dg, workspace, workspace_size, stream);
-    return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
+    return fla::guarded([&] { return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, w, g_gamma, scale, chunk_size, use_exp2,
                            transpose_state_layout, dq, dk, dw, dg, workspace, workspace_size,
-                           static_cast<hipStream_t>(stream), nullptr);
+                           static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_prepare_wy_repr_bwd_da_get_workspace_size)(
@@ -868,16 +868,16 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_da_get_workspace_size)(
     int64_t chunk_size, const fla_tensor *dA, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_da_get_workspace_size, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd_da");
-    return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, nullptr, 0, nullptr,
-                               workspace_size);
+    return fla::guarded([&] { return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, nullptr, 0, nullptr,
+                               workspace_size); });
 }
 FLA_ENTRY(fla_prepare_wy_repr_bwd_da)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
     const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
     int64_t chunk_size, const fla_tensor *dA, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_da, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace, workspace_size, stream);
-    return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace,
-                               workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::wy_bwd_da_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dA, workspace,
+                               workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_prepare_wy_repr_bwd_full_get_workspace_size)(
@@ -887,8 +887,8 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_full_get_workspace_size)(
     const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_get_workspace_size, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd_full");
-    return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
-                                 nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_prepare_wy_repr_bwd_full)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
@@ -896,8 +896,8 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_full)(
     const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
     const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
-    return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
-                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_prepare_wy_repr_bwd_get_workspace_size)(
@@ -907,8 +907,8 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_get_workspace_size)(
     uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_get_workspace_size, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd");
-    return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, nullptr, 0,
-                            nullptr, workspace_size);
+    return fla::guarded([&] { return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, nullptr, 0,
+                            nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_prepare_wy_repr_bwd)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
@@ -916,6 +916,6 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd)(
     int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg,
     void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd, k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
-    return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace,
-                            workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::wy_bwd_impl(k, v, beta, A, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace,
+                            workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

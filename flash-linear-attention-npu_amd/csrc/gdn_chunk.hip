@@ -855,8 +855,9 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128>(p, stream);
     if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256>(p, stream);
     if (geom.K == 64 && geom.V == 64) return launch_fwd_o<64, 64>(p, stream);
-    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(128,256),(64,64).", op, geom.K,
-                geom.V);
+    if (geom.K == 64 && geom.V == 128) return launch_fwd_o<64, 128>(p, stream);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(128,256),(64,64),(64,128).", op,
+                geom.K, geom.V);
 }
 
 }  // namespace
@@ -871,15 +872,15 @@ FLA_ENTRY(fla_chunk_scaled_dot_kkt_get_workspace_size)(const fla_tensor *k, cons
                                                            const fla_tensor *out, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_get_workspace_size, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_scaled_dot_kkt");
-    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_scaled_dot_kkt)(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
                                         const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                         int64_t chunk_size, const fla_tensor *out, void *workspace,
                                         uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size, stream);
-    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
-                         static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr); });
 }
 FLA_ENTRY(fla_chunk_scaled_dot_kkt_inverse_get_workspace_size)(const fla_tensor *k, const fla_tensor *g,
                                                                    const fla_tensor *beta, const fla_int_array *cu_seqlens,
@@ -887,15 +888,15 @@ FLA_ENTRY(fla_chunk_scaled_dot_kkt_inverse_get_workspace_size)(const fla_tensor 
                                                                    const fla_tensor *out, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_inverse_get_workspace_size, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_scaled_dot_kkt_inverse");
-    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size, true);
+    return fla::guarded([&] { return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, nullptr, 0, nullptr, workspace_size, true); });
 }
 FLA_ENTRY(fla_chunk_scaled_dot_kkt_inverse)(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta,
                                                 const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                                 int64_t chunk_size, const fla_tensor *out, void *workspace,
                                                 uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_chunk_scaled_dot_kkt_inverse, k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size, stream);
-    return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
-                         static_cast<hipStream_t>(stream), nullptr, true);
+    return fla::guarded([&] { return fla::kkt_impl(k, g, beta, cu_seqlens, chunk_indices, chunk_size, out, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr, true); });
 }
 
 FLA_ENTRY(fla_solve_tri_get_workspace_size)(const fla_tensor *x, const fla_int_array *cu_seqlens,
@@ -903,14 +904,14 @@ FLA_ENTRY(fla_solve_tri_get_workspace_size)(const fla_tensor *x, const fla_int_a
                                                 const fla_tensor *out, uint64_t *workspace_size) {
     FLA_ROUTE_F16(out, fla_solve_tri_get_workspace_size, x, cu_seqlens, chunk_indices, layout, out, workspace_size);
     FLA_NULL_WS("solve_tri");
-    return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_solve_tri)(const fla_tensor *x, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                              const char *layout, const fla_tensor *out, void *workspace, uint64_t workspace_size,
                              void *stream) {
     FLA_ROUTE_F16(out, fla_solve_tri, x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size, stream);
-    return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size,
-                           static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::solve_impl(x, cu_seqlens, chunk_indices, layout, out, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_recompute_w_u_fwd_get_workspace_size)(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
@@ -921,8 +922,8 @@ FLA_ENTRY(fla_recompute_w_u_fwd_get_workspace_size)(const fla_tensor *k, const f
                                                         uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_recompute_w_u_fwd_get_workspace_size, k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace_size);
     FLA_NULL_WS("recompute_w_u_fwd");
-    return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, nullptr, 0, nullptr,
-                        workspace_size);
+    return fla::guarded([&] { return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, nullptr, 0, nullptr,
+                        workspace_size); });
 }
 FLA_ENTRY(fla_recompute_w_u_fwd)(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta,
                                      const fla_tensor *A, const fla_tensor *g, const fla_tensor *gk,
@@ -930,8 +931,8 @@ FLA_ENTRY(fla_recompute_w_u_fwd)(const fla_tensor *k, const fla_tensor *v, const
                                      int64_t chunk_size, const fla_tensor *w, const fla_tensor *u, void *workspace,
                                      uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_recompute_w_u_fwd, k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size, stream);
-    return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size,
-                        static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::wu_impl(k, v, beta, A, g, gk, cu_seqlens, chunk_indices, chunk_size, w, u, workspace, workspace_size,
+                        static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_fwd_o_get_workspace_size)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
@@ -941,14 +942,14 @@ FLA_ENTRY(fla_chunk_fwd_o_get_workspace_size)(const fla_tensor *q, const fla_ten
                                                   uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_fwd_o_get_workspace_size, q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace_size);
     FLA_NULL_WS("chunk_fwd_o");
-    return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0, nullptr,
-                           workspace_size);
+    return fla::guarded([&] { return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, nullptr, 0, nullptr,
+                           workspace_size); });
 }
 FLA_ENTRY(fla_chunk_fwd_o)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *h,
                                const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
                                double scale, int64_t chunk_size, const fla_tensor *out, void *workspace,
                                uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_fwd_o, q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size, stream);
-    return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size,
-                           static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::fwd_o_impl(q, k, v, h, g, cu_seqlens, chunk_indices, scale, chunk_size, out, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr); });
 }

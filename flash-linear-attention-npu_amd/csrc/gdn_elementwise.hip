@@ -260,14 +260,14 @@ extern "C" int fla_chunk_local_cumsum_get_workspace_size(const fla_tensor *g, co
                                                          const char *output_dtype, const fla_tensor *out,
                                                          uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_local_cumsum: workspace_size must not be null.");
-    return fla::cumsum_impl(g, cu_seqlens, chunk_indices_out, chunk_size, reverse, scale, head_first, output_dtype, out,
-                            nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::cumsum_impl(g, cu_seqlens, chunk_indices_out, chunk_size, reverse, scale, head_first, output_dtype, out,
+                            nullptr, 0, nullptr, workspace_size); });
 }
 
 extern "C" int fla_chunk_local_cumsum(const fla_tensor *g, const fla_int_array *cu_seqlens,
                                       const fla_int_array *chunk_indices_out, int64_t chunk_size, bool reverse,
                                       double scale, bool head_first, const char *output_dtype, const fla_tensor *out,
                                       void *workspace, uint64_t workspace_size, void *stream) {
-    return fla::cumsum_impl(g, cu_seqlens, chunk_indices_out, chunk_size, reverse, scale, head_first, output_dtype, out,
-                            workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::cumsum_impl(g, cu_seqlens, chunk_indices_out, chunk_size, reverse, scale, head_first, output_dtype, out,
+                            workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

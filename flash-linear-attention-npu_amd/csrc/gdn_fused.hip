@@ -33,22 +33,7 @@ namespace {
 
 constexpr int kThreads = 256;
 
-#ifdef FLA_NO_FENCE
-#define FLA_SCHED_FENCE()
-#else
 #define FLA_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#endif
-
-#ifdef FLA_FUSED_TIMING
-#define FLA_TICK(i)                      \
-    {                                    \
-        long long now_ = clock64();      \
-        tacc[i] += now_ - tlast;         \
-        tlast = now_;                    \
-    }
-#else
-#define FLA_TICK(i)
-#endif
 
 struct FusedParams {
     ChunkGeom geom;
@@ -380,20 +365,12 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         commit(0, tiles_at<K, CT>(smem, 0));
     }
     __syncthreads();
-#ifdef FLA_FUSED_TIMING
-    long long tacc[16] = {0};
-#endif
 
     for (int c = 0; c < nchunks; ++c) {
         const int len = min(kChunk, eos - (bos + c * kChunk));
         const Tiles t = tiles_at<K, CT>(smem, DB ? (c & 1) : 0);
-#ifdef FLA_FUSED_TIMING
-        long long tlast = clock64();
-#endif
         if (DB && c > 0) store_o(c - 1);
         if (c + 1 < nchunks) prefetch(c + 1);
-        FLA_TICK(0)
-
         // =========================== A: scores ===========================================
         switch (wv) {
             case 0: phase_a<K, 0>(t, aS, pS, dS, p.scale); break;
@@ -401,10 +378,7 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
             case 2: phase_a<K, 2>(t, aS, pS, dS, p.scale); break;
             default: phase_a<K, 3>(t, aS, pS, dS, p.scale); break;
         }
-        FLA_TICK(1)
         __syncthreads();  // #1: aS, dS, pS complete
-        FLA_TICK(2)
-
         // =========================== B: WY solve =========================================
         // tiles 0..CT-1: this wave's u columns; tiles CT..NT-1: its w columns
         f32x4 r[NT][4];
@@ -454,12 +428,8 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
         for (int m = 0; m < NTW; ++m)
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc_to_tile(wS, pw, 16 * i, (wv * NTW + m) * 16, -r[CT + m][i]);
-        FLA_TICK(6)
         if (DB && c + 1 < nchunks) commit(c + 1, tiles_at<K, CT>(smem, (c + 1) & 1));
-        FLA_TICK(7)
         __syncthreads();  // #2: wS complete (and, double-buffered, the next chunk's tiles)
-        FLA_TICK(3)
-
         // =========================== C: scan + output ====================================
         elemx8 hB[KS][CT];
 #pragma unroll
@@ -504,7 +474,6 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
                 FLA_SCHED_FENCE();
             }
         }
-        FLA_TICK(8)
         // operands of the next two products, issued before the element-wise work below
         elemx8 pf[2][4], kfa[KT];
 #pragma unroll
@@ -528,7 +497,6 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] *= eg4[rt];  // scale e^{G_t} (q h)
         }
-        FLA_TICK(9)
         // o = scale (e^{G_t} q h + P v_new)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -540,7 +508,6 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) oacc[rt][ct] = mfma16x32(pf[j][rt], vb[ct], oacc[rt][ct]);
         }
-        FLA_TICK(10)
         // h <- e^{g_last} h + k^T (v_new e^{g_last - g}), the right operand as hi + lo bf16
         const float dec_all = __expf(g_last);
 #pragma unroll
@@ -580,27 +547,18 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
                     hacc[kt][ct] = mfma16x32(kfb[kt], vlo[1][ct], hacc[kt][ct]);
                 }
         }
-        FLA_TICK(11)
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc_to_tile(oS, po, rt * 16, (vtile0 + ct) * 16, oacc[rt][ct]);
-        FLA_TICK(12)
         __syncthreads();  // #3: every read of this chunk's tiles is done, oS complete
-        FLA_TICK(4)
-
         if (!DB) {
             store_o(c);
             if (c + 1 < nchunks) commit(c + 1, tiles_at<K, CT>(smem, 0));
             __syncthreads();  // #4
         }
-        FLA_TICK(5)
     }
     if (DB && nchunks > 0) store_o(nchunks - 1);
-#ifdef FLA_FUSED_TIMING
-    if (blockIdx.x == 0 && l == 0 && p.g_out)
-        for (int i = 0; i < 16; ++i) p.g_out[wv * 16 + i] = (float)tacc[i] / (float)nchunks;
-#endif
 
     if (p.hT) {
         float *s = p.hT + n * p.s_sn + hv * p.s_sh;
@@ -787,10 +745,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             commit_qk(pipe_tiles_at<K>(smem, 0));
         }
         __syncthreads();   // start
-#ifdef FLA_FUSED_TIMING
-        long long tacc[16] = {0};
-        long long tlast = clock64();
-#endif
         for (int i = 0; i <= nchunks; ++i) {
             const Tiles t = pipe_tiles_at<K>(smem, i);
             elem *pS = pS0 + (i & 1) * kChunk * pp;
@@ -807,9 +761,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                     default: phase_a<K, 3>(t, aS, pS, dS, p.scale); break;
                 }
             }
-            FLA_TICK(0)
             __syncthreads();   // mid
-            FLA_TICK(1)
             if (i < nchunks) {
                 // tile 0: this wave's u columns; tiles 1..NTW: its w columns (the table holds -beta e^G, so
                 // the solve yields -w, which is what the state group accumulates)
@@ -858,18 +810,11 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                     for (int bi = 0; bi < 4; ++bi) acc_to_tile(wS, pw, 16 * bi, (wv * NTW + m) * 16, r[1 + m][bi]);
 #pragma unroll
                 for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<f32x4 *>(uS + ((wv * 4 + bi) * 64 + l) * 4) = r[0][bi];
-                FLA_TICK(2)
                 if (i + 1 < nchunks) commit_qk(pipe_tiles_at<K>(smem, i + 1));
             }
-            FLA_TICK(3)
             __syncthreads();   // end
-            FLA_TICK(4)
         }
         if (nchunks > 0) store_o(nchunks - 1);
-#ifdef FLA_FUSED_TIMING
-        if (blockIdx.x == 0 && l == 0 && p.g_out)
-            for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
-#endif
         return;
     }
 
@@ -948,10 +893,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         if (nchunks > 1) gate_fetch(1);
     }
     __syncthreads();   // start
-#ifdef FLA_FUSED_TIMING
-    long long tacc[16] = {0};
-    long long tlast = clock64();
-#endif
 
     for (int i = 0; i <= nchunks; ++i) {
         const int c = i - 1;                               // chunk of this group
@@ -960,11 +901,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         const int len = c >= 0 ? min(kChunk, eos - (bos + c * kChunk)) : 0;
         f32x4 U[4], eg4[4];
         elemx8 hB[KS];
-#ifdef FLA_PIPE_SKIP_STATE
-        if (c >= 1000000) {
-#else
         if (c >= 0) {
-#endif
             // state at chunk start as bf16 operand; it also serves q h after the update below
 #pragma unroll
             for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
@@ -984,7 +921,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                     for (int rt = 0; rt < 4; ++rt) U[rt] = mfma16x32(wf[j][rt], hB[j], U[rt]);
                 FLA_SCHED_FENCE();
             }
-            FLA_TICK(0)
             elemx8 kfa[KT], kfb[KT];
             f32x4 dk4[4];
             const float g_last = t.G[len - 1];
@@ -1055,14 +991,8 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             pf[4] = frag_kc(pS, pp, 48, 0);
             pf[5] = frag_kc(pS, pp, 48, 32);
         }
-        FLA_TICK(1)
         __syncthreads();   // mid
-        FLA_TICK(2)
-#ifdef FLA_PIPE_SKIP_STATE
-        if (c >= 1000000) {
-#else
         if (c >= 0) {
-#endif
             // o = scale (e^{G_t} q h + P v_new), h the state at chunk start
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) oacc[rt] *= eg4[rt];
@@ -1078,7 +1008,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             // tables of the next chunk, then the gate loads of the one after it
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
-            FLA_TICK(3)
             // this wave's 16 columns of o into the staging tile; the prep group writes whole rows to memory
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) acc_to_tile(oS, po, 16 * rt, 16 * wv, oacc[rt]);
@@ -1086,14 +1015,8 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
         }
-        FLA_TICK(4)
         __syncthreads();   // end
-        FLA_TICK(5)
     }
-#ifdef FLA_FUSED_TIMING
-    if (blockIdx.x == 0 && l == 0 && p.g_out)
-        for (int i = 0; i < 16; ++i) p.g_out[wave * 16 + i] = (float)tacc[i] / (float)nchunks;
-#endif
     if (p.hT) {
         float *s = p.hT + n * p.s_sn + hv * p.s_sh;
 #pragma unroll
@@ -1215,22 +1138,14 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     p.scale = (float)scale;
     p.l2norm = use_qk_l2norm ? 1 : 0;
 
-    // 128-column slabs (two 16-column tiles per wave) halve the per-FLOP LDS traffic and do the
-    // score / w work once per head; 64-column slabs double the number of workgroups.  Use the
-    // wide form once it alone fills the GPU.
+    // 128-column slabs (two 16-column tiles per wave) halve the per-FLOP LDS traffic and do the score / w work once
+    // per head; 64-column slabs double the number of workgroups and run as the two-group pipelined kernel.  The wide
+    // form is used once it alone fills the GPU; the in-kernel normalisation lives in the pipelined kernel's tile commit.
     const int64_t chains = (int64_t)geom.N * geom.Hv;
-    bool wide = geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
-    if (const char *env = getenv("FLA_HIP_GDN_SLAB")) {  // tuning override: 64 or 128 columns per workgroup
-        if (atoi(env) == 128 && geom.V % 128 == 0) wide = true;
-        if (atoi(env) == 64) wide = false;
-    }
-    if (use_qk_l2norm) wide = false;   // the in-kernel normalisation lives in the pipelined kernel's tile commit
+    const bool wide = !use_qk_l2norm && geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
     p.slabs = wide ? geom.V / 128 : geom.V / 64;
-    bool pipe = !wide;
-    if (const char *env = getenv("FLA_HIP_GDN_PIPE")) pipe = pipe && (atoi(env) != 0 || use_qk_l2norm);   // tuning override
-    if (pipe) return geom.K == 128 ? launch_pipe<128>(p, stream) : launch_pipe<64>(p, stream);
-    if (geom.K == 128) return wide ? launch_fused<128, 2>(p, stream) : launch_fused<128, 1>(p, stream);
-    return wide ? launch_fused<64, 2>(p, stream) : launch_fused<64, 1>(p, stream);
+    if (!wide) return geom.K == 128 ? launch_pipe<128>(p, stream) : launch_pipe<64>(p, stream);
+    return geom.K == 128 ? launch_fused<128, 2>(p, stream) : launch_fused<64, 2>(p, stream);
 }
 
 }  // namespace
@@ -1245,9 +1160,9 @@ FLA_ENTRY(fla_gdn_chunk_fwd_get_workspace_size)(const fla_tensor *q, const fla_t
                                                     uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd: workspace_size must not be null.");
-    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
+    return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, nullptr, 0, nullptr, workspace_size);
+                           g_cumsum, final_state, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
@@ -1256,7 +1171,7 @@ FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla
                                  bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
                                  const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace, workspace_size, stream);
-    return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
+    return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+                           g_cumsum, final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -23,7 +23,9 @@ constexpr int kThreads = 256;
 struct ScanParams {
     ChunkGeom geom;
     View4 k, w, u, v_new;
-    View3 g;
+    View3 g;             // scalar gate (natural log), or p == null
+    const float *gk;     // per-channel gate [B,Hv,T,K] f32 (log2; k then already carries 2^{gk_last - gk}), or null
+    int64_t gk_sb, gk_sh, gk_st;
     const void *h0;      // [N,Hv,K,V] or [N,Hv,V,K], fp32 or the element type, or null
     void *hT;            // final state, same layout and type, or null
     int state_elem;      // 1: h0 / hT hold the element type (the carry itself stays fp32)
@@ -41,7 +43,8 @@ template <int K, int CT> struct FwdHSmem {
     static constexpr size_t k_off = w_off + (size_t)kChunk * pw * 2;
     static constexpr size_t u_off = k_off + (size_t)kChunk * pk * 2;
     static constexpr size_t g_off = u_off + (size_t)kChunk * pu * 2;
-    static constexpr size_t buf_bytes = g_off + (size_t)kChunk * 4;
+    static constexpr size_t d_off = g_off + (size_t)kChunk * 4;          // [K] per-channel decay 2^{gk_last} of the chunk
+    static constexpr size_t buf_bytes = d_off + (size_t)K * 4;
     static constexpr bool kStage = CT == 1;                              // wider slabs leave no LDS for the staging
     static constexpr int ps = VS + 8;                                    // pitch of the h staging tiles
     static constexpr size_t stage_off = 2 * buf_bytes;                   // two [K][ps] tiles of the emitted h
@@ -90,12 +93,15 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
             tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
             tu.fetch(ug + (int64_t)start * p.u.st, p.u.st, len, tid);
-            float gv = 0.f;
-            if (tid < kChunk) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+            float gv = 0.f, dk = 1.f;
+            if (tid < kChunk && p.g.p) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+            if (p.gk && tid < K)
+                dk = __builtin_amdgcn_exp2f(p.gk[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + tid]);
             tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
             tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
             tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
             if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
+            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = dk;
         };
         const bool stage_h = L::kStage && p.h != nullptr && !p.v_first;
         auto store_h = [&](int c) {   // staged state at the start of step c (a chunk start) -> h[.., chunk, :, slab columns]
@@ -268,10 +274,20 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                 }
                 vB[j][ct] = frag_from_acc(lo, hi);
             }
+        if (p.gk) {   // per-channel decay: row kk of the state by 2^{gk_last[kk]} (times the scalar decay, if any)
+            const float *dS = reinterpret_cast<const float *>(buf + L::d_off);
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
+            for (int kt = 0; kt < KT; ++kt) {
+                const f32x4 d = *reinterpret_cast<const f32x4 *>(dS + 16 * kt + 4 * lg) * dec_all;
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= dec_all;
+                for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= d;
+            }
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] *= dec_all;
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -313,8 +329,8 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
                const fla_int_array *ci, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
                const fla_tensor *final_state, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "chunk_gated_delta_rule_fwd_h";
-    FLA_REQUIRE(gk == nullptr || gk->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: gk is not supported; pass g.", op);
-    FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: either g or gk must be provided.", op);
+    const bool has_g = g != nullptr && g->data != nullptr, has_gk = gk != nullptr && gk->data != nullptr;
+    FLA_REQUIRE(has_g || has_gk, FLA_ERR_NULL, "%s: either g or gk must be provided.", op);
     ChunkGeom geom;
     int rc;
     if ((rc = gdn_geometry(op, k, u, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;
@@ -323,7 +339,14 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
+    if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
+    if (has_gk) {   // key-wise gate, log2 units (README.md:16-30): the state rows decay by 2^{gk_last}, k arrives gated
+        if ((rc = check_tensor(gk, op, "gk", 4, dt_bit(FLA_F32)))) return rc;
+        FLA_REQUIRE(gk->shape[0] == geom.B && gk->shape[1] == geom.Hv && gk->shape[2] == geom.T && gk->shape[3] == geom.K &&
+                        inner_unit(gk),
+                    FLA_ERR_SHAPE, "%s: gk must be float32 [B,Hv,T,K] with a unit innermost stride.", op);
+        FLA_REQUIRE(geom.C == kChunk, FLA_ERR_UNSUPPORTED, "%s: gk is built for chunk_size 64.", op);
+    }
     Varlen vl;
     if ((rc = build_varlen(vl, op, cu, ci, geom.C, geom.T))) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
@@ -376,7 +399,13 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
     p.w = view4(w);
     p.u = view4(u);
     p.v_new = view4(v_new);
-    p.g = view3(g);
+    p.g = has_g ? view3(g) : View3{nullptr, 0, 0, 0, 0};
+    if (has_gk) {
+        p.gk = static_cast<const float *>(gk->data);
+        p.gk_sb = gk->stride[0];
+        p.gk_sh = gk->stride[1];
+        p.gk_st = gk->stride[2];
+    }
     p.h0 = has_h0 ? initial_state->data : nullptr;
     p.hT = output_final_state ? final_state->data : nullptr;
     const fla_tensor *sref = has_h0 ? initial_state : (output_final_state ? final_state : nullptr);
@@ -787,8 +816,8 @@ FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h_get_workspace_size)(
     const fla_tensor *final_state, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_chunk_gated_delta_rule_fwd_h_get_workspace_size, k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices, state_v_first, h, v_new, final_state, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_fwd_h: workspace_size must not be null.");
-    return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
-                           state_v_first, h, v_new, final_state, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
+                           state_v_first, h, v_new, final_state, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h)(
@@ -797,9 +826,9 @@ FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h)(
     const fla_int_array *chunk_indices, bool state_v_first, const fla_tensor *h, const fla_tensor *v_new,
     const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_chunk_gated_delta_rule_fwd_h, k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices, state_v_first, h, v_new, final_state, workspace, workspace_size, stream);
-    return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
+    return fla::guarded([&] { return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
                            state_v_first, h, v_new, final_state, workspace, workspace_size,
-                           static_cast<hipStream_t>(stream), nullptr);
+                           static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size)(
@@ -809,8 +838,8 @@ FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size)(
     const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size, q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0, dv2, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_gated_delta_rule_bwd_dhu: workspace_size must not be null.");
-    return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
-                             dv2, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
+                             dv2, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu)(
@@ -820,6 +849,6 @@ FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu)(
     const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, void *workspace, uint64_t workspace_size,
     void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_gated_delta_rule_bwd_dhu, q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0, dv2, workspace, workspace_size, stream);
-    return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
-                             dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, dv, g, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, use_exp2, dh, dh0,
+                             dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

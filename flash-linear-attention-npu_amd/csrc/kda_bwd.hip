@@ -571,16 +571,16 @@ FLA_ENTRY(fla_chunk_kda_bwd_dav_get_workspace_size)(
     uint64_t *workspace_size) {
     FLA_ROUTE_F16(v_new, fla_chunk_kda_bwd_dav_get_workspace_size, v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace_size);
     FLA_NULL_WS("chunk_kda_bwd_dav");
-    return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, nullptr, 0, nullptr,
-                         workspace_size);
+    return fla::guarded([&] { return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, nullptr, 0, nullptr,
+                         workspace_size); });
 }
 FLA_ENTRY(fla_chunk_kda_bwd_dav)(
     const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *Aqk, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dAqk, const fla_tensor *dv,
     void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(v_new, fla_chunk_kda_bwd_dav, v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace, workspace_size, stream);
-    return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace, workspace_size,
-                         static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::dav_impl(v_new, d_o, Aqk, cu_seqlens, chunk_indices, scale, chunk_size, dAqk, dv, workspace, workspace_size,
+                         static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_get_workspace_size)(
@@ -590,8 +590,8 @@ FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_get_workspace_size)(
     const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace_size);
     FLA_NULL_WS("chunk_kda_bwd_dqkwg");
-    return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
-                               nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
+                               nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_kda_bwd_dqkwg)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
@@ -599,8 +599,8 @@ FLA_ENTRY(fla_chunk_kda_bwd_dqkwg)(
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
     const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace, workspace_size, stream);
-    return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
-                               workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
+                               workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_kda_bwd_wy_get_workspace_size)(
@@ -610,8 +610,8 @@ FLA_ENTRY(fla_chunk_kda_bwd_wy_get_workspace_size)(
     const fla_tensor *dAkk, uint64_t *workspace_size) {
     FLA_ROUTE_F16(k, fla_chunk_kda_bwd_wy_get_workspace_size, k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace_size);
     FLA_NULL_WS("chunk_kda_bwd_wy");
-    return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, nullptr, 0,
-                            nullptr, workspace_size);
+    return fla::guarded([&] { return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, nullptr, 0,
+                            nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_kda_bwd_wy)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *gk, const fla_tensor *Akk,
@@ -619,6 +619,6 @@ FLA_ENTRY(fla_chunk_kda_bwd_wy)(
     int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
     const fla_tensor *dAkk, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(k, fla_chunk_kda_bwd_wy, k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace, workspace_size, stream);
-    return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace,
-                            workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace,
+                            workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

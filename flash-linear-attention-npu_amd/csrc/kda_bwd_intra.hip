@@ -342,8 +342,8 @@ FLA_ENTRY(fla_chunk_kda_bwd_intra_get_workspace_size)(
     const fla_tensor *dg_out, uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra_get_workspace_size, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_intra: workspace_size must not be null.");
-    return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
-                               layout, dq_out, dk_out, db_out, dg_out, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+                               layout, dq_out, dk_out, db_out, dg_out, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_chunk_kda_bwd_intra)(
@@ -353,7 +353,7 @@ FLA_ENTRY(fla_chunk_kda_bwd_intra)(
     const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size, stream);
-    return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+    return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
                                layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size,
-                               static_cast<hipStream_t>(stream), nullptr);
+                               static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -1148,9 +1148,9 @@ FLA_ENTRY(fla_chunk_kda_fwd_get_workspace_size)(
     uint64_t *workspace_size) {
     FLA_ROUTE_F16(q, fla_chunk_kda_fwd_get_workspace_size, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale, chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_fwd: workspace_size must not be null.");
-    return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
+    return fla::guarded([&] { return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
                              chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
-                             Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, workspace_size);
+                             Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_chunk_kda_fwd)(
@@ -1162,10 +1162,10 @@ FLA_ENTRY(fla_chunk_kda_fwd)(
     const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
     void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_kda_fwd, q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale, chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, workspace, workspace_size, stream);
-    return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
+    return fla::guarded([&] { return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, cu_seqlens, chunk_indices, layout, scale,
                              chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk,
                              Aqk, Akk, w, u, qg, kg, v_new, h, workspace, workspace_size, static_cast<hipStream_t>(stream),
-                             nullptr);
+                             nullptr); });
 }
 
 #ifndef FLA_ELEM_F16
@@ -1237,9 +1237,9 @@ extern "C" int fla_chunk_kda_fwd_noalloc(
                                      chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out,
                                      final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, ptr,
                                      FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES, stream);
-    return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale, chunk_size,
+    return fla::guarded([&] { return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale, chunk_size,
                              safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk,
                              w, u, qg, kg, v_new, h, ptr, FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES,
-                             static_cast<hipStream_t>(stream), nullptr);
+                             static_cast<hipStream_t>(stream), nullptr); });
 }
 #endif  // !FLA_ELEM_F16

@@ -164,14 +164,14 @@ extern "C" int fla_kda_gate_cumsum_get_workspace_size(const fla_tensor *g, const
                                                       bool use_gate_in_kernel, bool safe_gate, double lower_bound,
                                                       const fla_tensor *gk, uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "kda_gate_cumsum: workspace_size must not be null.");
-    return fla::gate_impl(g, A_log, dt_bias, cu_seqlens, chunk_size, use_gate_in_kernel, safe_gate, lower_bound, gk, nullptr, 0,
-                          nullptr, workspace_size);
+    return fla::guarded([&] { return fla::gate_impl(g, A_log, dt_bias, cu_seqlens, chunk_size, use_gate_in_kernel, safe_gate, lower_bound, gk, nullptr, 0,
+                          nullptr, workspace_size); });
 }
 
 extern "C" int fla_kda_gate_cumsum(const fla_tensor *g, const fla_tensor *A_log, const fla_tensor *dt_bias,
                                    const fla_int_array *cu_seqlens, int64_t chunk_size, bool use_gate_in_kernel,
                                    bool safe_gate, double lower_bound, const fla_tensor *gk, void *workspace,
                                    uint64_t workspace_size, void *stream) {
-    return fla::gate_impl(g, A_log, dt_bias, cu_seqlens, chunk_size, use_gate_in_kernel, safe_gate, lower_bound, gk, workspace,
-                          workspace_size, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::gate_impl(g, A_log, dt_bias, cu_seqlens, chunk_size, use_gate_in_kernel, safe_gate, lower_bound, gk, workspace,
+                          workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -141,22 +141,22 @@ int l2_impl(const char *op, const fla_tensor *x, const fla_tensor *dy, const fla
 extern "C" int fla_l2norm_fwd_get_workspace_size(const fla_tensor *x, double eps, const fla_tensor *y, const fla_tensor *rstd,
                                                  uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "l2norm_fwd: workspace_size must not be null.");
-    return fla::l2_impl<false>("l2norm_fwd", x, nullptr, rstd, eps, y, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::l2_impl<false>("l2norm_fwd", x, nullptr, rstd, eps, y, nullptr, workspace_size); });
 }
 extern "C" int fla_l2norm_fwd(const fla_tensor *x, double eps, const fla_tensor *y, const fla_tensor *rstd, void *workspace,
                               uint64_t workspace_size, void *stream) {
     (void)workspace;
     (void)workspace_size;
-    return fla::l2_impl<false>("l2norm_fwd", x, nullptr, rstd, eps, y, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::l2_impl<false>("l2norm_fwd", x, nullptr, rstd, eps, y, static_cast<hipStream_t>(stream), nullptr); });
 }
 extern "C" int fla_l2norm_bwd_get_workspace_size(const fla_tensor *y, const fla_tensor *rstd, const fla_tensor *dy, double eps,
                                                  const fla_tensor *dx, uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "l2norm_bwd: workspace_size must not be null.");
-    return fla::l2_impl<true>("l2norm_bwd", y, dy, rstd, eps, dx, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::l2_impl<true>("l2norm_bwd", y, dy, rstd, eps, dx, nullptr, workspace_size); });
 }
 extern "C" int fla_l2norm_bwd(const fla_tensor *y, const fla_tensor *rstd, const fla_tensor *dy, double eps, const fla_tensor *dx,
                               void *workspace, uint64_t workspace_size, void *stream) {
     (void)workspace;
     (void)workspace_size;
-    return fla::l2_impl<true>("l2norm_bwd", y, dy, rstd, eps, dx, static_cast<hipStream_t>(stream), nullptr);
+    return fla::guarded([&] { return fla::l2_impl<true>("l2norm_bwd", y, dy, rstd, eps, dx, static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -357,8 +357,8 @@ extern "C" int fla_recurrent_gated_delta_rule_get_workspace_size(
     const fla_tensor *out, uint64_t *workspace_size) {
     if (workspace_size == nullptr)
         return fla::fail(FLA_ERR_NULL, "recurrent_gated_delta_rule: workspace_size must not be null.");
-    return fla::rec_impl(query, key, value, beta, state, actual_seq_lengths, ssm_state_indices, g, gk,
-                         num_accepted_tokens, scale, out, nullptr, 0, nullptr, workspace_size);
+    return fla::guarded([&] { return fla::rec_impl(query, key, value, beta, state, actual_seq_lengths, ssm_state_indices, g, gk,
+                         num_accepted_tokens, scale, out, nullptr, 0, nullptr, workspace_size); });
 }
 
 extern "C" int fla_recurrent_gated_delta_rule(
@@ -366,7 +366,7 @@ extern "C" int fla_recurrent_gated_delta_rule(
     const fla_tensor *state, const fla_tensor *actual_seq_lengths, const fla_tensor *ssm_state_indices,
     const fla_tensor *g, const fla_tensor *gk, const fla_tensor *num_accepted_tokens, float scale,
     const fla_tensor *out, void *workspace, uint64_t workspace_size, void *stream) {
-    return fla::rec_impl(query, key, value, beta, state, actual_seq_lengths, ssm_state_indices, g, gk,
+    return fla::guarded([&] { return fla::rec_impl(query, key, value, beta, state, actual_seq_lengths, ssm_state_indices, g, gk,
                          num_accepted_tokens, scale, out, workspace, workspace_size, static_cast<hipStream_t>(stream),
-                         nullptr);
+                         nullptr); });
 }

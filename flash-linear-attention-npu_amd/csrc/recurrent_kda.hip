@@ -441,10 +441,10 @@ extern "C" int fla_recurrent_kda_get_workspace_size(
     bool allow_neg_eigval, bool safe_gate, double lower_bound, bool state_v_first, const fla_tensor *attn_out,
     const fla_tensor *final_state, uint64_t *workspace_size) {
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "recurrent_kda: workspace_size must not be null.");
-    return fla::rkda_impl(q, k, v, g, beta, initial_state, cu_seqlens, ssm_state_indices, A_log, dt_bias, num_accepted_tokens, layout,
+    return fla::guarded([&] { return fla::rkda_impl(q, k, v, g, beta, initial_state, cu_seqlens, ssm_state_indices, A_log, dt_bias, num_accepted_tokens, layout,
                           scale, output_final_state, inplace_final_state, use_qk_l2norm_in_kernel, use_gate_in_kernel,
                           use_beta_sigmoid_in_kernel, allow_neg_eigval, safe_gate, lower_bound, state_v_first, attn_out,
-                          final_state, nullptr, 0, nullptr, workspace_size);
+                          final_state, nullptr, 0, nullptr, workspace_size); });
 }
 extern "C" int fla_recurrent_kda(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
@@ -453,8 +453,8 @@ extern "C" int fla_recurrent_kda(
     bool inplace_final_state, bool use_qk_l2norm_in_kernel, bool use_gate_in_kernel, bool use_beta_sigmoid_in_kernel,
     bool allow_neg_eigval, bool safe_gate, double lower_bound, bool state_v_first, const fla_tensor *attn_out,
     const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
-    return fla::rkda_impl(q, k, v, g, beta, initial_state, cu_seqlens, ssm_state_indices, A_log, dt_bias, num_accepted_tokens, layout,
+    return fla::guarded([&] { return fla::rkda_impl(q, k, v, g, beta, initial_state, cu_seqlens, ssm_state_indices, A_log, dt_bias, num_accepted_tokens, layout,
                           scale, output_final_state, inplace_final_state, use_qk_l2norm_in_kernel, use_gate_in_kernel,
                           use_beta_sigmoid_in_kernel, allow_neg_eigval, safe_gate, lower_bound, state_v_first, attn_out,
-                          final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr);
+                          final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

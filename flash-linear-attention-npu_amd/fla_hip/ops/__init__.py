@@ -40,11 +40,18 @@ _REFERENCE_OPS = (
     "npu_recurrent_kda",
 )
 
+# Operators that write into one of their arguments through the library (invisible to autograd), and, where the write
+# depends on a flag, the test that says whether this call writes (ops/ascendc/__init__.py:61-71).
 MUTATED_ARGUMENTS = {
     "causal_conv1d": ("conv_states",),
     "npu_causal_conv1d": ("conv_states",),
+    "npu_recurrent_kda": ("initial_state",),
     "recurrent_gated_delta_rule": ("state",),
     "npu_recurrent_gated_delta_rule": ("state",),
+}
+
+MUTATION_PREDICATES = {
+    "npu_recurrent_kda": lambda arguments: bool(arguments["inplace_final_state"]),
 }
 
 
@@ -53,32 +60,36 @@ def _strip_npu_prefix(name: str) -> str:
 
 
 def _wrap_mutable_op(name: str, op: Callable) -> Callable:
-    mutated_names = MUTATED_ARGUMENTS.get(name, ())
-    if not mutated_names:
+    """Guard for an operator that overwrites arguments in place (contract of ops/ascendc/__init__.py:146-185):
+    a tensor about to be overwritten must not require grad, and after the launch its autograd version counter is
+    bumped so that graphs which saved it notice.  ``MUTATION_PREDICATES`` can switch the guard off per call."""
+    declared = MUTATED_ARGUMENTS.get(name, ())
+    if not declared:
         return op
-    signature = inspect.signature(op)
+    parameters = inspect.signature(op)
+    writes_this_call = MUTATION_PREDICATES.get(name)
 
     @functools.wraps(op)
-    def wrapper(*args, **kwargs):
+    def guarded(*args, **kwargs):
         import torch
 
-        bound = signature.bind(*args, **kwargs)
-        bound.apply_defaults()
-        mutated = [bound.arguments[n] for n in mutated_names]
-        requiring_grad = [n for n in mutated_names if getattr(bound.arguments[n], "requires_grad", False)]
-        if requiring_grad:
-            names = ", ".join(requiring_grad)
+        call = parameters.bind(*args, **kwargs)
+        call.apply_defaults()
+        written = declared if writes_this_call is None or writes_this_call(call.arguments) else ()
+        targets = {arg: call.arguments[arg] for arg in written}
+        blocked = [arg for arg, value in targets.items() if getattr(value, "requires_grad", False)]
+        if blocked:
             raise RuntimeError(
-                f"{name} mutates {names} in place through ctypes. Mutable state tensors "
+                f"{name} mutates {', '.join(blocked)} in place through ctypes. Mutable state tensors "
                 "must not require gradients; use a functional state API for training."
             )
         result = op(*args, **kwargs)
-        mutated = [t for t in mutated if isinstance(t, torch.Tensor)]
-        if mutated:
-            torch.autograd.graph.increment_version(mutated)
+        touched = [value for value in targets.values() if isinstance(value, torch.Tensor)]
+        if touched:
+            torch.autograd.graph.increment_version(touched)
         return result
 
-    return wrapper
+    return guarded
 
 
 def _missing_op(name: str) -> Callable:
@@ -153,6 +164,7 @@ def causal_conv1d(x, weight, bias=None, conv_states=None, *, query_start_loc=Non
 
 __all__ = [
     "MUTATED_ARGUMENTS",
+    "MUTATION_PREDICATES",
     "chunk_kda_fwd_noalloc",
     "gdn_chunk_fwd",
     "l2norm_bwd",

@@ -55,7 +55,8 @@ typedef enum fla_status {
     FLA_ERR_UNSUPPORTED = 4, /* valid request this build has no kernel for      */
     FLA_ERR_WORKSPACE = 5,   /* workspace missing or smaller than required      */
     FLA_ERR_LAUNCH = 6,      /* the HIP runtime refused the launch              */
-    FLA_ERR_METADATA = 7     /* cu_seqlens / chunk_indices are inconsistent     */
+    FLA_ERR_METADATA = 7,    /* cu_seqlens / chunk_indices are inconsistent     */
+    FLA_ERR_HOST = 8         /* host-side failure (allocation, lock) in the call */
 } fla_status;
 
 /* Replaces the opaque aclTensor built by aclCreateTensor(shape, ndim, dtype,
@@ -78,6 +79,15 @@ typedef struct fla_int_array {
 const char *fla_last_error(void);
 /* ABI version of this header; bumped on any signature change. */
 int fla_abi_version(void);
+
+/* Per-kernel timing, no counterpart in the reference (it profiles from outside with msopprof,
+ * fla/ops/ascendc/kda/KDA_FORWARD_VALIDATION_REPORT.md:77-84).  After fla_profile_enable(1) every kernel
+ * launch is bracketed by two HIP events on its launch stream.  fla_profile_report waits for them, writes
+ * one "name count total_ms" line per kernel name into buf (NUL-terminated, truncated to cap bytes),
+ * clears the records and returns the number of kernel names.  Process-wide; not for use under stream
+ * capture. */
+void fla_profile_enable(int on);
+int fla_profile_report(char *buf, uint64_t cap);
 
 /* ------------------------------------------------------------------------
  * chunk_local_cumsum - replaces aclnnChunkLocalCumsum
@@ -155,8 +165,9 @@ int fla_recompute_w_u_fwd(
 /* ------------------------------------------------------------------------
  * chunk_gated_delta_rule_fwd_h - replaces aclnnChunkGatedDeltaRuleFwdH
  * (_aclnn_ctypes.py:552-615).  k [B,Hk,T,K], w [B,Hv,T,K], u [B,Hv,T,V] bf16;
- * g [B,Hv,T] f32 (chunk-cumsummed); gk must be NULL; initial_state
- * [N,Hv,K,V] f32 or NULL.  Outputs h [B,Hv,NT,K,V] bf16 (state at chunk
+ * g [B,Hv,T] f32 (chunk-cumsummed, natural log) and / or gk [B,Hv,T,K] f32
+ * (chunk-cumsummed per-channel gate, log2 units; k then already carries
+ * 2^{gk_last - gk}; chunk_size 64); initial_state [N,Hv,K,V] f32 or NULL.  Outputs h [B,Hv,NT,K,V] bf16 (state at chunk
  * start), v_new [B,Hv,T,V] bf16, final_state [N,Hv,K,V] f32 (NULL unless
  * output_final_state).
  * ------------------------------------------------------------------------ */

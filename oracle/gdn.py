@@ -174,11 +174,15 @@ def recompute_w_u_fwd(k, v, beta, A, chunk: int, *, g, cu_seqlens=None,
 # ----------------------------------------------------------------------------
 # stage 5: sequential state scan
 # ----------------------------------------------------------------------------
-def chunk_gated_delta_rule_fwd_h(k, w, u, g, *, initial_state=None, output_final_state=False,
+def chunk_gated_delta_rule_fwd_h(k, w, u, g=None, *, gk=None, initial_state=None, output_final_state=False,
                                  chunk: int = 64, cu_seqlens=None,
                                  compute_dtype=torch.float32, lowp=None, output_dtype=None):
     """Returns (h [B,Hv,NT,K,V] = state at each chunk start, v_new [B,Hv,T,V],
-    final_state [N,Hv,K,V] fp32 or None)."""
+    final_state [N,Hv,K,V] fp32 or None).  ``g`` [B,Hv,T]: scalar gate (natural log); ``gk`` [B,Hv,T,K]:
+    key-wise gate in log2 units, whose decay 2^{gk_last} multiplies the state rows while k arrives already gated
+    (chunk_gated_delta_rule_fwd_h/README.md:16-30)."""
+    if g is None:
+        g = torch.zeros(u.shape[:3], dtype=compute_dtype)
     B, Hk, T, K = k.shape
     Hv, V = u.shape[1], u.shape[3]
     rep = Hv // Hk
@@ -200,7 +204,10 @@ def chunk_gated_delta_rule_fwd_h(k, w, u, g, *, initial_state=None, output_final
         v_new[b, :, s:e] = vn
         glast = gc[:, -1]
         vdec = _round(_round(vn, lowp) * torch.exp(glast[:, None] - gc)[..., None], lowp)
-        state[n] = S * torch.exp(glast)[:, None, None] + torch.matmul(kc.transpose(-1, -2), vdec)
+        decay = torch.exp(glast)[:, None, None]
+        if gk is not None:
+            decay = decay * torch.exp2(gk[b, :, e - 1].to(compute_dtype))[:, :, None]
+        state[n] = S * decay + torch.matmul(kc.transpose(-1, -2), vdec)
     od = output_dtype if output_dtype is not None else k.dtype
     return h.to(od), v_new.to(od), (state.float() if output_final_state else None)
 

@@ -169,6 +169,34 @@ def test_public_namespace_and_mutation_contract():
                                        ssm_state_indices=None, g=torch.zeros(1))
 
 
+def test_recurrent_kda_mutation_follows_the_inplace_flag():
+    """`npu_recurrent_kda` overwrites its state pool only with inplace_final_state (MUTATION_PREDICATES,
+    ops/ascendc/__init__.py:61-71): then a pool that requires grad is rejected and the version counter of the pool
+    is bumped after the call; with the flag off neither happens."""
+    from fla_hip import ops
+    from fla_hip.ops import _hip_ctypes as H
+    assert ops.MUTATED_ARGUMENTS["npu_recurrent_kda"] == ("initial_state",)
+    assert ops.MUTATION_PREDICATES["npu_recurrent_kda"]({"inplace_final_state": True}) is True
+    assert ops.MUTATION_PREDICATES["npu_recurrent_kda"]({"inplace_final_state": 0}) is False
+    calls = []
+    guarded = ops._wrap_mutable_op("npu_recurrent_kda", lambda q, k, v, g, beta, initial_state=None, *,
+                                   inplace_final_state=True, **kw: calls.append(inplace_final_state) or "out")
+    pool = torch.zeros(2, 1, 4, 4, requires_grad=True)
+    with pytest.raises(RuntimeError, match="npu_recurrent_kda mutates initial_state in place"):
+        guarded(None, None, None, None, None, pool)
+    assert not calls                                                    # rejected before the operator ran
+    assert guarded(None, None, None, None, None, pool, inplace_final_state=False) == "out"
+    plain = torch.zeros(2, 1, 4, 4)
+    before = plain._version
+    guarded(None, None, None, None, None, plain, inplace_final_state=False)
+    assert plain._version == before                                     # not written: no bump
+    guarded(None, None, None, None, None, plain)
+    assert plain._version == before + 1
+    assert calls == [False, False, True]
+    # the exported operator is the guarded one
+    assert ops.npu_recurrent_kda is ops.recurrent_kda and ops.npu_recurrent_kda is not H.npu_recurrent_kda
+
+
 def test_recurrent_wrapper_requires_a_gate_before_any_launch():
     from fla_hip.ops import _hip_ctypes as H
     with mock.patch.object(H, "_call_op") as call:

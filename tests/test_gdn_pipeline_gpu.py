@@ -51,6 +51,38 @@ def test_against_naive_recurrence(dev, case, fused, dtype):
     assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
 
 
+# Batches large enough that the host picks the kernels with 128-column value slabs: the fused forward once
+# sequences x heads x (V / 128) reaches the number of compute units (256), the stand-alone state scan at twice that.
+WIDE_CASES = [
+    (8, 200, 32, 32, 128, 128, None),                    # fused: 256 chains
+    (4, 130, 32, 32, 128, 256, None),                    # fused: 128 chains x 2 slabs, V = 256
+    (16, 130, 32, 16, 128, 128, None),                   # fused and the six-operator scan (512 chains), grouped heads
+    (1, 8 * 70, 32, 32, 128, 128, [70 * i for i in range(9)]),   # packed: 8 sequences x 32 heads, initial states
+    (1, 600, 32, 32, 64, 128, [0, 1, 65, 130, 130, 258, 300, 450, 600]),   # K = 64, ragged packed sequences
+]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("case", WIDE_CASES)
+def test_large_batches_on_the_wide_slab_kernels(dev, case, fused):
+    B, T, H, Hk, K, V, cu = case
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=BF, seed=T + H, Hk=Hk)
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, H, K, V, generator=torch.Generator().manual_seed(2)) * 0.01
+    o, final, o_ref, f_ref = run_both(dev, d, cu=cu, h0=h0, fused=fused)
+    st = assert_close(o, o_ref, TOL_BF16, "o")
+    assert st["rel_max"] < 2e-2, st
+    assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
+
+
+def test_six_operator_route_with_k64_v128(dev):
+    d = gdn.make_gdn_inputs(1, 130, 2, 64, 128, dtype=BF, seed=7, Hk=2)
+    h0 = torch.randn(1, 2, 64, 128, generator=torch.Generator().manual_seed(2)) * 0.01
+    o, final, o_ref, f_ref = run_both(dev, d, h0=h0, fused=False)
+    assert_close(o, o_ref, TOL_BF16, "o")
+    assert_close(final, f_ref, 4 * TOL_STATE, "final_state")
+
+
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", CASES)
 def test_in_kernel_l2norm_equals_separate_pass(dev, case, dtype):

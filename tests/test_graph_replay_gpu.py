@@ -123,3 +123,26 @@ def test_conv1d_update_and_dense_prefill_replay(dev):
         torch.cuda.synchronize()
         assert torch.equal(y, y_eager) and torch.equal(static_states, eager_states), f"replay {trial}: conv1d update"
         assert torch.equal(o, o_eager) and torch.equal(hT, hT_eager), f"replay {trial}: chunk forward"
+
+
+def test_calls_with_host_integer_arrays_refuse_stream_capture(dev):
+    """A packed batch hands cu_seqlens over as a host array that the library uploads through a recycled pinned slot: a
+    captured upload would replay other calls' metadata, so the call is refused while the stream is capturing (nothing is
+    launched), and the same call works eagerly before and after."""
+    from fla_hip import pipeline
+    from oracle import gdn
+    d = gdn.make_gdn_inputs(1, 130, 2, 128, 128, dtype=BF, seed=3)
+    cu = [0, 65, 130]
+    args = [d[n].to(dev) for n in ("q", "k", "v", "g", "beta")]
+    call = lambda: pipeline.flash_gated_delta_rule(*args, None, None, True, cu_seqlens=cu)
+    o_before, f_before = call()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be uploaded while the stream is being captured"):
+        with torch.cuda.graph(graph):
+            call()
+    torch.cuda.synchronize()
+    for _ in range(20):            # more calls than the staging ring has slots
+        o_after, f_after = call()
+    torch.cuda.synchronize()
+    assert torch.equal(o_before, o_after) and torch.equal(f_before, f_after)

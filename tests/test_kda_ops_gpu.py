@@ -162,6 +162,44 @@ def test_bwd_dhu_errors(dev):
 
 
 # ---------------------------------------------------------------------------------------------
+# chunk_gated_delta_rule_fwd_h with the key-wise gate gk (README.md:16-30 of the operator): the KDA state scan
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("case", [(2, 200, 2, 2, 128, 128, None, False), (1, 261, 2, 4, 128, 128, [0, 1, 16, 33, 33, 96, 160, 261], False),
+                                  (1, 130, 1, 2, 64, 64, None, True), (1, 96, 1, 1, 128, 256, None, False)])
+def test_fwd_h_with_key_wise_gate(dev, case):
+    from fla_hip import ops
+    B, T, Hk, Hv, K, V, cu, v_first = case
+    gen = torch.Generator().manual_seed(T + K)
+    N = B if cu is None else len(cu) - 1
+    kgt = (torch.randn(B, Hv, T, K, generator=gen) * 0.1).to(BF)           # k with its gate applied, per value head
+    w = (torch.randn(B, Hv, T, K, generator=gen) * 0.1).to(BF)
+    u = torch.randn(B, Hv, T, V, generator=gen).to(BF)
+    gk = kda.kda_gate_cumsum(torch.nn.functional.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, 64, cu_seqlens=cu)
+    h0 = torch.randn(N, Hv, K, V, generator=gen) * 0.1
+    h_ref, vn_ref, f_ref = gdn.chunk_gated_delta_rule_fwd_h(kgt, w, u, gk=gk, initial_state=h0, output_final_state=True,
+                                                            cu_seqlens=cu, lowp=BF, output_dtype=torch.float32)
+    h0_d = (h0.transpose(-1, -2).contiguous() if v_first else h0).to(dev)
+    h, v_new, final = ops.chunk_gated_delta_rule_fwd_h(kgt.to(dev), w.to(dev), u.to(dev), gk=gk.to(dev), initial_state=h0_d,
+                                                       output_final_state=True, cu_seqlens=cu, state_v_first=v_first)
+    if v_first:
+        h, final = h.transpose(-1, -2), final.transpose(-1, -2)
+    assert_close(v_new, vn_ref, TOL_BF16, "v_new")
+    assert_close(h, h_ref, TOL_BF16, "h")
+    assert_close(final, f_ref, 4e-3, "final_state")
+    # both gates together: the scalar one multiplies the same rows
+    g = gdn.chunk_local_cumsum(torch.nn.functional.logsigmoid(torch.randn(B, Hv, T, generator=gen)) * 0.2, 64, cu_seqlens=cu)
+    if not v_first:
+        ref2 = gdn.chunk_gated_delta_rule_fwd_h(kgt, w, u, g, gk=gk, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                                                lowp=BF, output_dtype=torch.float32)
+        got2 = ops.chunk_gated_delta_rule_fwd_h(kgt.to(dev), w.to(dev), u.to(dev), g.to(dev), gk=gk.to(dev), initial_state=h0_d,
+                                                output_final_state=True, cu_seqlens=cu)
+        assert_close(got2[1], ref2[1], TOL_BF16, "v_new (g and gk)")
+        assert_close(got2[2], ref2[2], 4e-3, "final_state (g and gk)")
+    with pytest.raises(RuntimeError, match="chunk_size 64"):
+        ops.chunk_gated_delta_rule_fwd_h(kgt.to(dev), w.to(dev), u.to(dev), gk=gk.to(dev), chunk_size=128)
+
+
+# ---------------------------------------------------------------------------------------------
 # chunk_kda_bwd_intra (fp32 products; the reference's own tolerance is 2e-4)
 # ---------------------------------------------------------------------------------------------
 def intra_inputs(B, T, H, K, seed, beta_dtype, cu=None, decay=0.05):

@@ -190,6 +190,22 @@ def test_kda_chunked_equals_naive(cu):
     assert float((out["final_state"] - f_n.float()).abs().max()) < 1e-5
 
 
+@pytest.mark.parametrize("cu", [None, [0, 5, 70, 150]])
+def test_fwd_h_with_key_wise_gate_is_the_kda_state_scan(cu):
+    """chunk_gated_delta_rule_fwd_h(kg, w, u, gk=gk) walks the same states as the KDA chunk forward (itself pinned
+    against the per-token recurrence above): h, v_new and the final state agree."""
+    q, k, v, gate, beta = kda_inputs(1, 150, 2, 16, 24, seed=3, gate_scale=0.3)
+    h0 = torch.randn(1 if cu is None else 3, 2, 16, 24, generator=torch.Generator().manual_seed(4))
+    gk = kda.kda_gate_cumsum(gate, 64, cu_seqlens=cu)
+    ref = kda.chunk_kda_fwd(q, k, v, gk, beta, 0.3, 64, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                            compute_dtype=torch.float64)
+    h, v_new, final = gdn.chunk_gated_delta_rule_fwd_h(ref["kg"], ref["w"], ref["u"], gk=gk, initial_state=h0,
+                                                       output_final_state=True, cu_seqlens=cu, compute_dtype=torch.float64,
+                                                       output_dtype=torch.float64)
+    assert torch.allclose(h, ref["h"], atol=1e-10) and torch.allclose(v_new, ref["v_new"], atol=1e-10)
+    assert torch.allclose(final, ref["final_state"], atol=1e-6)
+
+
 def test_kda_reduces_to_gdn_for_channel_constant_gate():
     d = gdn.make_gdn_inputs(1, 100, 2, 16, 16, seed=5, head_first_gates=True)
     gate = d["g"][..., None].expand(-1, -1, -1, 16).contiguous()
