@@ -126,32 +126,28 @@ def npu_chunk_gated_delta_rule_fwd_h(k, w, u, g=None, *, gk=None, initial_state=
     """_aclnn_ctypes.py:552-615."""
     import torch
 
-    if g is None and gk is None:
-        raise RuntimeError("npu_chunk_gated_delta_rule_fwd_h: either g or gk must be provided.")
-    output_final_state = _optional_bool(output_final_state, False)
-    state_v_first = _optional_bool(state_v_first, False)
+    op = "npu_chunk_gated_delta_rule_fwd_h"
+    if (g, gk) == (None, None):
+        raise RuntimeError(f"{op}: either g or gk must be provided.")
+    want_final = _optional_bool(output_final_state, False)
+    v_first = _optional_bool(state_v_first, False)
     chunk_size = _optional_int(chunk_size, 64)
-    B, _, T, K = _shape(k)
-    _, HV, _, V = _shape(u)
-    cu = _as_int_tuple(cu_seqlens)
-    indices = _as_int_tuple(chunk_indices)
-    if indices is None and cu is not None:
+    (B, _, T, K), (_, HV, _, V) = _shape(k), _shape(u)
+    cu, indices = _as_int_tuple(cu_seqlens), _as_int_tuple(chunk_indices)
+    if cu is not None and indices is None:
         indices = _build_chunk_indices(cu, chunk_size)
     NT = _total_chunks(B, T, chunk_size, cu)
-    N = len(cu) - 1 if cu is not None else B
-    state_tail = (V, K) if state_v_first else (K, V)
-    if initial_state is not None and _shape(initial_state) != (N, HV, *state_tail):
-        raise RuntimeError("npu_chunk_gated_delta_rule_fwd_h: initial_state shape does not match state_v_first.")
-    h_out = _empty((B, HV, NT, *state_tail), k)
+    N = B if cu is None else len(cu) - 1
+    block = (V, K) if v_first else (K, V)
+    if initial_state is not None and _shape(initial_state) != (N, HV, *block):
+        raise RuntimeError(f"{op}: initial_state shape does not match state_v_first.")
+    h_out = _empty((B, HV, NT, *block), k)
     v_new_out = _empty_like(u)
-    if output_final_state:
-        if initial_state is not None:
-            final_state_out = _empty((N, HV, *state_tail), initial_state)
-        else:
-            final_state_out = _empty((N, HV, *state_tail), k, dtype=torch.float32)
-    else:
-        final_state_out = None
-    outputs = (h_out, v_new_out, final_state_out if output_final_state else None)
+    final_state_out = None
+    if want_final:   # the carried state keeps the dtype of the state the caller supplied, fp32 otherwise
+        final_state_out = _empty((N, HV, *block), k, dtype=torch.float32 if initial_state is None else initial_state.dtype)
+    output_final_state, state_v_first = want_final, v_first
+    outputs = (h_out, v_new_out, final_state_out)
     return _call_op(
         "chunk_gated_delta_rule_fwd_h", OP_ARGTYPES["chunk_gated_delta_rule_fwd_h"],
         lambda ctx: [
@@ -196,40 +192,33 @@ def npu_recurrent_gated_delta_rule(query, key, value, state, *, beta, scale=1.0,
 
     import torch
 
-    tensors = {
-        "query": query, "key": key, "value": value, "state": state, "beta": beta,
-        "actual_seq_lengths": actual_seq_lengths, "ssm_state_indices": ssm_state_indices,
+    bf, f32, i32 = torch.bfloat16, torch.float32, torch.int32
+    # operand -> (value, required, accepted dtypes, rank); checked in this order: presence and type, device, dtype, rank
+    spec = {
+        "query": (query, True, (bf,), 3), "key": (key, True, (bf,), 3), "value": (value, True, (bf,), 3),
+        "state": (state, True, (bf, f32), 4), "beta": (beta, True, (bf,), 2),
+        "actual_seq_lengths": (actual_seq_lengths, True, (i32,), 1),
+        "ssm_state_indices": (ssm_state_indices, True, (i32,), 1),
+        "g": (g, False, (f32,), 2), "gk": (gk, False, (f32,), 3),
+        "num_accepted_tokens": (num_accepted_tokens, False, (i32,), 1),
     }
-    optional_tensors = {"g": g, "gk": gk, "num_accepted_tokens": num_accepted_tokens}
-    for name, tensor in (*tensors.items(), *optional_tensors.items()):
-        if tensor is None:
-            if name in tensors:
-                raise TypeError(f"{op_name}: {name} must be a torch.Tensor, got None.")
+    for name, (tensor, required, _, _) in spec.items():
+        if tensor is None and not required:
             continue
         if not isinstance(tensor, torch.Tensor):
-            raise TypeError(f"{op_name}: {name} must be a torch.Tensor, got {type(tensor)!r}.")
+            shown = "None" if tensor is None else repr(type(tensor))
+            raise TypeError(f"{op_name}: {name} must be a torch.Tensor, got {shown}.")
         if tensor.device.type != "cuda":
             raise TypeError(f"{op_name}: {name} must be a torch GPU tensor, got device {tensor.device}.")
-
-    dtype_requirements = {
-        "query": (torch.bfloat16,), "key": (torch.bfloat16,), "value": (torch.bfloat16,),
-        "beta": (torch.bfloat16,), "state": (torch.bfloat16, torch.float32),
-        "actual_seq_lengths": (torch.int32,), "ssm_state_indices": (torch.int32,),
-        "g": (torch.float32,), "gk": (torch.float32,), "num_accepted_tokens": (torch.int32,),
-    }
-    for name, supported in dtype_requirements.items():
-        tensor = tensors.get(name, optional_tensors.get(name))
-        if tensor is not None and tensor.dtype not in supported:
-            names = ", ".join(str(d) for d in supported)
-            raise TypeError(f"{op_name}: {name} dtype must be one of ({names}), got {tensor.dtype}.")
-
-    shapes = {n: _shape(t) for n, t in (*tensors.items(), *optional_tensors.items()) if t is not None}
-    expected_ranks = {"query": 3, "key": 3, "value": 3, "beta": 2, "state": 4, "actual_seq_lengths": 1,
-                      "ssm_state_indices": 1, "g": 2, "gk": 3, "num_accepted_tokens": 1}
-    for name, rank in expected_ranks.items():
-        shp = shapes.get(name)
-        if shp is not None and len(shp) != rank:
-            raise RuntimeError(f"{op_name}: {name} must be rank {rank}, got shape {shp}.")
+    present = {name: entry for name, entry in spec.items() if entry[0] is not None}
+    for name, (tensor, _, accepted, _) in present.items():
+        if tensor.dtype not in accepted:
+            listed = ", ".join(str(d) for d in accepted)
+            raise TypeError(f"{op_name}: {name} dtype must be one of ({listed}), got {tensor.dtype}.")
+    shapes = {name: _shape(entry[0]) for name, entry in present.items()}
+    for name, (_, _, _, rank) in present.items():
+        if len(shapes[name]) != rank:
+            raise RuntimeError(f"{op_name}: {name} must be rank {rank}, got shape {shapes[name]}.")
 
     if shapes["query"] != shapes["key"]:
         raise RuntimeError(
@@ -287,28 +276,20 @@ def npu_recurrent_gated_delta_rule(query, key, value, state, *, beta, scale=1.0,
 
 
 def _chunk_local_cumsum_output_dtype(g, output_dtype):
-    """_aclnn_ctypes.py:849-872."""
+    """Name handed to the library and torch dtype of the output; accepted spellings as in _aclnn_ctypes.py:849-872
+    (a torch dtype, its name with or without ``torch.``, the short forms, or same / input / none for g's dtype)."""
     import torch
 
+    names = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+    aliases = {"float": "float32", "half": "float16", "bf16": "bfloat16"}
     if output_dtype is None:
         return "float32", torch.float32
-    if isinstance(output_dtype, torch.dtype):
-        if output_dtype in (torch.float, torch.float32):
-            return "float32", torch.float32
-        if output_dtype in (torch.float16, torch.half):
-            return "float16", torch.float16
-        if output_dtype == torch.bfloat16:
-            return "bfloat16", torch.bfloat16
-        raise TypeError(f"Unsupported chunk_local_cumsum output_dtype: {output_dtype}.")
-    normalized = str(output_dtype).removeprefix("torch.").lower()
-    if normalized in {"float", "float32"}:
-        return "float32", torch.float32
-    if normalized in {"half", "float16"}:
-        return "float16", torch.float16
-    if normalized in {"bf16", "bfloat16"}:
-        return "bfloat16", torch.bfloat16
-    if normalized in {"same", "input", "none"}:
-        return normalized, g.dtype
+    key = str(output_dtype).removeprefix("torch.").lower()
+    key = aliases.get(key, key)
+    if key in names:
+        return key, names[key]
+    if key in ("same", "input", "none") and not isinstance(output_dtype, torch.dtype):
+        return key, g.dtype
     raise TypeError(f"Unsupported chunk_local_cumsum output_dtype: {output_dtype}.")
 
 
@@ -473,20 +454,20 @@ def npu_chunk_gated_delta_rule_bwd_dhu(q, k, w, d_o, dv, scale, chunk_size, *, g
     import torch
 
     B, _, T, K = _shape(q)
-    Hv, V = _shape(dv)[1], _shape(dv)[3]
-    if (g is None) == (gK is None):
+    _, Hv, _, V = _shape(dv)
+    gates = {"g": (g, (B, Hv, T)), "gK": (gK, (B, Hv, T, K))}
+    given = [name for name, (t, _) in gates.items() if t is not None]
+    if len(given) != 1:
         raise ValueError("Exactly one of g and gK must be provided.")
-    if gK is not None and not _optional_bool(use_exp2, True):
+    if given == ["gK"] and not _optional_bool(use_exp2, True):
         raise ValueError("use_exp2 must be true when gK is provided.")
-    if any(t.dtype != q.dtype for t in (k, w, d_o, dv)):
+    if {t.dtype for t in (k, w, d_o, dv)} != {q.dtype}:
         raise ValueError("q, k, w, d_o and dv must have the same dtype.")
-    gate = g if g is not None else gK
+    gate, gate_shape = gates[given[0]]
     if gate.dtype not in (q.dtype, torch.float32):
         raise ValueError("g or gK must be float32 or have the same dtype as q and k.")
-    if g is not None and _shape(g) != (B, Hv, T):
-        raise ValueError(f"g must have shape {(B, Hv, T)}, got {_shape(g)}.")
-    if gK is not None and _shape(gK) != (B, Hv, T, K):
-        raise ValueError(f"gK must have shape {(B, Hv, T, K)}, got {_shape(gK)}.")
+    if _shape(gate) != gate_shape:
+        raise ValueError(f"{given[0]} must have shape {gate_shape}, got {_shape(gate)}.")
     chunk_size = int(chunk_size)
     cu = _as_int_tuple(cu_seqlens)
     indices = _as_int_tuple(chunk_indices)
@@ -1023,114 +1004,89 @@ def npu_recurrent_kda(q, k, v, g, beta, initial_state=None, *, cu_seqlens=None, 
     """_aclnn_ctypes.py:1298-1503: same checks, defaults and error texts.  Returns (out, final_state or None)."""
     import torch
 
+    def need(ok, text):
+        if not ok:
+            raise RuntimeError("npu_recurrent_kda: " + text)
+
+    def on_q_device(t, name):
+        need(t.device == q.device, f"{name} must be on the same device as q.")
+
     layout = str(layout)
-    if layout not in ("BSND", "TND"):
-        raise RuntimeError("npu_recurrent_kda: layout must be BSND or TND.")
+    need(layout in ("BSND", "TND"), "layout must be BSND or TND.")
     is_tnd = layout == "TND"
-    q_shape, k_shape, v_shape = _shape(q), _shape(k), _shape(v)
-    g_shape, beta_shape = _shape(g), _shape(beta)
     rank = 3 if is_tnd else 4
-    if (len(q_shape) != rank or len(k_shape) != rank or len(v_shape) != rank or len(g_shape) != rank
-            or len(beta_shape) != rank - 1):
-        raise RuntimeError(
-            "npu_recurrent_kda: layout/rank mismatch. TND expects q/k [T,H,K], v [T,HV,V], "
-            "g [T,HV,K], beta [T,HV]; BSND expects q/k [B,T,H,K], v [B,T,HV,V], "
-            "g [B,T,HV,K], beta [B,T,HV].")
-    if q_shape != k_shape:
-        raise RuntimeError("npu_recurrent_kda: q and k must have identical shape.")
-    if q.dtype != torch.bfloat16 or k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16:
-        raise RuntimeError("npu_recurrent_kda: q/k/v currently support bfloat16 only.")
-    if any(t.device != q.device for t in (k, v, g, beta)):
-        raise RuntimeError("npu_recurrent_kda: q/k/v/g/beta must be on the same device.")
+    shapes = [_shape(t) for t in (q, k, v, g, beta)]
+    q_shape, k_shape, v_shape, g_shape, beta_shape = shapes
+    need([len(x) for x in shapes] == [rank] * 4 + [rank - 1],
+         "layout/rank mismatch. TND expects q/k [T,H,K], v [T,HV,V], g [T,HV,K], beta [T,HV]; "
+         "BSND expects q/k [B,T,H,K], v [B,T,HV,V], g [B,T,HV,K], beta [B,T,HV].")
+    need(q_shape == k_shape, "q and k must have identical shape.")
+    need({q.dtype, k.dtype, v.dtype} == {torch.bfloat16}, "q/k/v currently support bfloat16 only.")
+    need(all(t.device == q.device for t in (k, v, g, beta)), "q/k/v/g/beta must be on the same device.")
     floats = (torch.float16, torch.bfloat16, torch.float32)
-    if g.dtype not in floats:
-        raise RuntimeError("npu_recurrent_kda: g must use FP16, BF16 or FP32.")
-    if beta.dtype not in floats:
-        raise RuntimeError("npu_recurrent_kda: beta must use FP16, BF16 or FP32.")
-    if is_tnd:
-        total_tokens, heads, key_dim = q_shape
-        batch, dense_seq_len = 1, total_tokens
-        value_heads, value_dim = v_shape[1], v_shape[2]
-        ok = (v_shape[0] == total_tokens and g_shape == (total_tokens, value_heads, key_dim)
-              and beta_shape == (total_tokens, value_heads))
-    else:
-        batch, dense_seq_len, heads, key_dim = q_shape
-        total_tokens = batch * dense_seq_len
-        value_heads, value_dim = v_shape[2], v_shape[3]
-        ok = (v_shape[:2] == (batch, dense_seq_len) and g_shape == (batch, dense_seq_len, value_heads, key_dim)
-              and beta_shape == (batch, dense_seq_len, value_heads))
-    if not ok:
-        raise RuntimeError("npu_recurrent_kda: v/g/beta shape mismatch.")
-    if min(total_tokens, dense_seq_len, heads, value_heads, key_dim, value_dim) <= 0:
-        raise RuntimeError("npu_recurrent_kda: all shape dimensions must be positive.")
-    if value_heads % heads != 0:
-        raise RuntimeError("npu_recurrent_kda: HV must be divisible by H.")
-    if (key_dim, value_dim) not in ((128, 128), (128, 256)):
-        raise RuntimeError("npu_recurrent_kda: K/V currently support only K=128,V=128 or K=128,V=256.")
+    need(g.dtype in floats, "g must use FP16, BF16 or FP32.")
+    need(beta.dtype in floats, "beta must use FP16, BF16 or FP32.")
+    # token axes first, then (heads, width): the same test serves both layouts
+    lead = q_shape[:-2]
+    heads, key_dim = q_shape[-2:]
+    value_heads, value_dim = v_shape[-2:]
+    batch, dense_seq_len = (1, lead[0]) if is_tnd else lead
+    total_tokens = batch * dense_seq_len
+    need(v_shape[:-2] == lead and g_shape == (*lead, value_heads, key_dim) and beta_shape == (*lead, value_heads),
+         "v/g/beta shape mismatch.")
+    need(min(total_tokens, dense_seq_len, heads, value_heads, key_dim, value_dim) > 0, "all shape dimensions must be positive.")
+    need(value_heads % heads == 0, "HV must be divisible by H.")
+    need((key_dim, value_dim) in ((128, 128), (128, 256)), "K/V currently support only K=128,V=128 or K=128,V=256.")
     ints = (torch.int32, torch.int64)
-    if cu_seqlens is None:
-        seq_num = batch if not is_tnd else 1
-    else:
-        if not isinstance(cu_seqlens, torch.Tensor) or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 2 \
-                or cu_seqlens.dtype not in ints:
-            raise RuntimeError("npu_recurrent_kda: cu_seqlens must be a 1D INT32 or INT64 tensor.")
-        if cu_seqlens.device != q.device:
-            raise RuntimeError("npu_recurrent_kda: cu_seqlens must be on the same device as q.")
+    seq_num = 1 if is_tnd else batch
+    if cu_seqlens is not None:
+        need(isinstance(cu_seqlens, torch.Tensor) and cu_seqlens.dim() == 1 and cu_seqlens.numel() >= 2
+             and cu_seqlens.dtype in ints, "cu_seqlens must be a 1D INT32 or INT64 tensor.")
+        on_q_device(cu_seqlens, "cu_seqlens")
         seq_num = int(cu_seqlens.shape[0]) - 1
     state_v_first = _optional_bool(state_v_first, False)
-    expected_tail = (value_heads, value_dim, key_dim) if state_v_first else (value_heads, key_dim, value_dim)
+    block = (value_dim, key_dim) if state_v_first else (key_dim, value_dim)
+    expected_tail = (value_heads, *block)
     inplace = _optional_bool(inplace_final_state, True)
     if initial_state is None:
-        if inplace:
-            raise RuntimeError("npu_recurrent_kda: inplace_final_state=True requires initial_state.")
+        need(not inplace, "inplace_final_state=True requires initial_state.")
         state_shape = (seq_num, *expected_tail)
         initial_state_work = torch.zeros(state_shape, device=q.device, dtype=torch.float32)
     else:
-        if initial_state.dtype not in (torch.float32, torch.bfloat16):
-            raise RuntimeError("npu_recurrent_kda: initial_state must use FP32 or BF16.")
-        if initial_state.device != q.device:
-            raise RuntimeError("npu_recurrent_kda: initial_state must be on the same device as q.")
+        need(initial_state.dtype in (torch.float32, torch.bfloat16), "initial_state must use FP32 or BF16.")
+        on_q_device(initial_state, "initial_state")
         state_shape = _shape(initial_state)
-        if len(state_shape) != 4 or state_shape[0] <= 0 or state_shape[1:] != expected_tail:
-            layout_desc = "[state_capacity,HV,V,K]" if state_v_first else "[state_capacity,HV,K,V]"
-            raise RuntimeError(f"npu_recurrent_kda: initial_state must be {layout_desc}.")
+        need(len(state_shape) == 4 and state_shape[0] > 0 and state_shape[1:] == expected_tail,
+             "initial_state must be [state_capacity,HV,%s]." % ("V,K" if state_v_first else "K,V"))
         initial_state_work = initial_state
-    if ssm_state_indices is not None:
-        packed_1d = ssm_state_indices.dim() == 1 and int(ssm_state_indices.shape[0]) >= total_tokens
-        speculative_2d = (ssm_state_indices.dim() == 2 and int(ssm_state_indices.shape[0]) == seq_num
-                          and int(ssm_state_indices.shape[1]) > 0)
-        if ssm_state_indices.dtype not in ints or not (packed_1d or speculative_2d):
-            raise RuntimeError(
-                "npu_recurrent_kda: ssm_state_indices must be INT32/INT64 packed [T] "
-                "or speculative [seq_num,max_step].")
-        if ssm_state_indices.device != q.device:
-            raise RuntimeError("npu_recurrent_kda: ssm_state_indices must be on the same device as q.")
-    elif state_shape[0] != seq_num:
-        raise RuntimeError("npu_recurrent_kda: without ssm_state_indices, state_capacity must equal seq_num.")
+    if ssm_state_indices is None:
+        need(state_shape[0] == seq_num, "without ssm_state_indices, state_capacity must equal seq_num.")
+    else:
+        idx_shape = _shape(ssm_state_indices)
+        per_token = len(idx_shape) == 1 and idx_shape[0] >= total_tokens
+        per_step = len(idx_shape) == 2 and idx_shape[0] == seq_num and idx_shape[1] > 0
+        need(ssm_state_indices.dtype in ints and (per_token or per_step),
+             "ssm_state_indices must be INT32/INT64 packed [T] or speculative [seq_num,max_step].")
+        on_q_device(ssm_state_indices, "ssm_state_indices")
     if num_accepted_tokens is not None:
-        if ssm_state_indices is None:
-            raise RuntimeError("npu_recurrent_kda: num_accepted_tokens requires ssm_state_indices.")
-        if num_accepted_tokens.dtype not in ints or _shape(num_accepted_tokens) != (seq_num,):
-            raise RuntimeError("npu_recurrent_kda: num_accepted_tokens must be INT32/INT64 [seq_num].")
-        if num_accepted_tokens.device != q.device:
-            raise RuntimeError("npu_recurrent_kda: num_accepted_tokens must be on the same device as q.")
+        need(ssm_state_indices is not None, "num_accepted_tokens requires ssm_state_indices.")
+        need(num_accepted_tokens.dtype in ints and _shape(num_accepted_tokens) == (seq_num,),
+             "num_accepted_tokens must be INT32/INT64 [seq_num].")
+        on_q_device(num_accepted_tokens, "num_accepted_tokens")
     use_gate = _optional_bool(use_gate_in_kernel, False)
     safe = _optional_bool(safe_gate, False)
     lower = _optional_float(lower_bound, -5.0)
-    if use_gate:
-        if A_log is None or A_log.dtype != torch.float32 or _shape(A_log) != (value_heads,):
-            raise RuntimeError("npu_recurrent_kda: A_log must be FP32 [HV] when use_gate_in_kernel=True.")
-        if A_log.device != q.device:
-            raise RuntimeError("npu_recurrent_kda: A_log must be on the same device as q.")
-        if safe and not -5.0 <= lower < 0.0:
-            raise RuntimeError("npu_recurrent_kda: lower_bound must be in [-5,0) when safe_gate=True.")
+    if not use_gate:
+        need(not safe and A_log is None and dt_bias is None, "A_log, dt_bias and safe_gate require use_gate_in_kernel=True.")
+    else:
+        need(A_log is not None and A_log.dtype == torch.float32 and _shape(A_log) == (value_heads,),
+             "A_log must be FP32 [HV] when use_gate_in_kernel=True.")
+        on_q_device(A_log, "A_log")
+        need(not safe or -5.0 <= lower < 0.0, "lower_bound must be in [-5,0) when safe_gate=True.")
         if dt_bias is not None:
-            if dt_bias.dtype != torch.float32 or _shape(dt_bias) not in ((value_heads * key_dim,), (value_heads, key_dim)):
-                raise RuntimeError("npu_recurrent_kda: dt_bias must be FP32 [HV*K] or [HV,K].")
-            if dt_bias.device != q.device:
-                raise RuntimeError("npu_recurrent_kda: dt_bias must be on the same device as q.")
-    elif safe or A_log is not None or dt_bias is not None:
-        raise RuntimeError("npu_recurrent_kda: A_log, dt_bias and safe_gate require use_gate_in_kernel=True.")
+            need(dt_bias.dtype == torch.float32 and _shape(dt_bias) in ((value_heads * key_dim,), (value_heads, key_dim)),
+                 "dt_bias must be FP32 [HV*K] or [HV,K].")
+            on_q_device(dt_bias, "dt_bias")
     out = _empty_like(v)
     final_state_work = initial_state_work if inplace else _empty(state_shape, initial_state_work)
     output_final = _optional_bool(output_final_state, False)

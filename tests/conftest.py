@@ -26,3 +26,20 @@ def dev():
 
     fla_hip.load_library()  # fail loudly if the HIP library is missing
     return torch.device("cuda:0")
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a GPU run: the measured error of every assert_close, largest share of its tolerance first."""
+    import json
+
+    import util
+
+    if not util.RECORDS:
+        return
+    out = ROOT / "gpurun_out"
+    try:
+        out.mkdir(exist_ok=True)
+        rows = sorted(util.RECORDS, key=lambda r: -(r["max_abs"] / (r["tol"] * (1.0 + r["max_ref"]))))
+        (out / "parity_errors.json").write_text(json.dumps(rows, indent=0))
+    except OSError:
+        pass

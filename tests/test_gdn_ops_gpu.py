@@ -104,7 +104,7 @@ def test_stagewise_against_oracle(dev, case, dtype):
     o_nv, final_nv = gdn.naive_recurrent_gated_delta_rule(d["q"], d["k"], d["v"], d["g"], d["beta"], scale,
                                                           initial_state=h0, output_final_state=True, cu_seqlens=cu)
     st = assert_close(o, o_nv, TOL, "o vs naive")
-    assert st["rel_max"] < 5e-2, st
+    assert st["rel_max"] < 2e-2, st
     assert_close(final, final_nv, TOL_STATE * 4, "final vs naive")   # unfused path rounds A, w, u to bf16
 
 

@@ -129,6 +129,53 @@ def test_decode_benchmark_shape_properties(dev):
         assert_close(st[t:t + 1], s_ref, TOL_STATE, "state")
 
 
+def test_varlen_prefill_benchmark_shape(dev):
+    """The variable-length prefill of the decode benchmark at full size: 64 sequences with lengths uniform in
+    [128, 4096] (about 135 K tokens), 32 heads, K=V=128, one state slot per sequence.  (a) Every sequence run on its own
+    gives the bits of the packed run (a sequence never sees its neighbours); (b) the shortest, the longest and a
+    middle sequence equal the fp32 per-token recurrence.  Far beyond the reference operator's 8-token limit, so the
+    recurrence is the only oracle."""
+    from fla_hip import ops
+    H, D, NSEQ = 32, 128, 64
+    lens = torch.randint(128, 4097, (NSEQ,), generator=torch.Generator().manual_seed(0))
+    T = int(lens.sum())
+    cu = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).tolist()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
+    q = F.normalize(rn(T, H, D), dim=-1).bfloat16()
+    k = F.normalize(rn(T, H, D), dim=-1).bfloat16()
+    v = rn(T, H, D).bfloat16()
+    beta = torch.sigmoid(rn(T, H)).bfloat16()
+    gate = F.logsigmoid(rn(T, H))
+    state0 = rn(NSEQ, H, D, D) * 0.01
+    seq = torch.cat([torch.zeros(1, dtype=torch.int32), lens.to(torch.int32)]).to(dev)
+    idx = torch.repeat_interleave(torch.arange(NSEQ, dtype=torch.int32), lens).to(dev)
+    state = state0.clone()
+    o = ops.recurrent_gated_delta_rule(q, k, v, state, beta=beta, scale=D ** -0.5, actual_seq_lengths=seq,
+                                       ssm_state_indices=idx, g=gate)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(state).all())
+    one = torch.tensor([0, 0], dtype=torch.int32)
+    for n in range(NSEQ):
+        s, e = cu[n], cu[n + 1]
+        st = state0[n:n + 1].clone()
+        one[1] = e - s
+        o_n = ops.recurrent_gated_delta_rule(q[s:e], k[s:e], v[s:e], st, beta=beta[s:e], scale=D ** -0.5,
+                                             actual_seq_lengths=one.to(dev),
+                                             ssm_state_indices=torch.zeros(e - s, dtype=torch.int32, device=dev), g=gate[s:e])
+        assert torch.equal(o_n, o[s:e]) and torch.equal(st[0], state[n]), f"sequence {n} differs from the packed run"
+    order = torch.argsort(lens).tolist()
+    for n in (order[0], order[NSEQ // 2], order[-1]):
+        s, e = cu[n], cu[n + 1]
+        c = lambda t: t[s:e].cpu()
+        o_ref, s_ref = od.recurrent_gated_delta_rule(
+            c(q), c(k), c(v), state0[n:n + 1].cpu(), beta=c(beta), scale=D ** -0.5,
+            actual_seq_lengths=torch.tensor([0, e - s], dtype=torch.int32),
+            ssm_state_indices=torch.zeros(e - s, dtype=torch.int32), g=c(gate))
+        assert_close(o[s:e], o_ref, TOL_BF16, f"out of sequence {n} ({e - s} tokens)")
+        assert_close(state[n:n + 1], s_ref, TOL_STATE, f"state of sequence {n}")
+
+
 def test_wrapper_errors(dev):
     from fla_hip import ops
     with pytest.raises(RuntimeError, match=r"^npu_recurrent_gated_delta_rule: either g or gk must be provided\.$"):
