@@ -570,6 +570,30 @@ def bench_gdn_bwd(args, torch, dev):
         pipeline.flash_chunk_gated_delta_rule_bwd(q, k, v, G, beta, A_saved, scale, h0, do, dht, chunk_size=C)
     torch.cuda.synchronize()
     ms_saved_A = (time.perf_counter() - t0) * 1e3 / args.steps
+    # training as the autograd entry runs it: the fused forward also writes h, v_new and w, the backward recomputes
+    # only the inverted chunk matrices
+    def fwd_train():
+        return pipeline.flash_chunk_gated_delta_rule_fwd(q, k, v, gate, beta, scale, h0, True, None, C,
+                                                         save_for_backward=True)
+
+    def train_step():
+        gc, _, _, _, saved = fwd_train()
+        return pipeline.flash_chunk_gated_delta_rule_bwd(q, k, v, gc, beta, None, scale, h0, do, dht, chunk_size=C,
+                                                         saved=saved)
+
+    def timed(fn):
+        for _ in range(max(2, args.warmup // 4)):
+            fn()
+        torch.cuda.synchronize()
+        t_ = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t_) * 1e3 / args.steps
+
+    ms_train = timed(train_step)
+    ms_fwd_train = timed(fwd_train)
+    ms_fwd_plain = timed(lambda: pipeline.flash_chunk_gated_delta_rule_fwd(q, k, v, gate, beta, scale, h0, True, None, C))
     lib.fla_profile_enable.argtypes = [ctypes.c_int]
     lib.fla_profile_enable(1)
     for _ in range(args.steps):
@@ -617,6 +641,9 @@ def bench_gdn_bwd(args, torch, dev):
         "config": {"workload": "GDN chunk backward B=4 T=8192 H=32 K=V=128 chunk=64, initial state and final-state gradient, "
                                "A recomputed from k, g, beta"},
         "ms_per_step_with_saved_A": round(ms_saved_A, 4),
+        "training": {"fwd_bwd_ms": round(ms_train, 4), "fwd_saving_h_vnew_w_ms": round(ms_fwd_train, 4),
+                     "bwd_with_saved_ms": round(ms_train - ms_fwd_train, 4), "fwd_inference_ms": round(ms_fwd_plain, 4),
+                     "fwd_inference_plus_bwd_recompute_ms": round(ms_fwd_plain + ms_per_step, 4)},
         "step_tflops": round(step_flops / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,

@@ -470,7 +470,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
 // =============================================================================
 // GVA: several value heads share the key head, dk is accumulated over them in registers; otherwise every
 // dk tile goes straight to memory and the column loop needs no accumulator array.
-template <int K, int V, bool GVA>
+// ACC: dk and dg are added to what the caller's tensors hold.  The dk tiles then wait in registers like the GVA sums and
+// leave through an fp32 LDS tile (the k and dw tiles, dead by then), so that memory is read and written in whole
+// 16-byte row pieces: adding tile by tile from the accumulator layout, four bytes per lane, cost more than the separate
+// elementwise pass it replaces.
+template <int K, int V, bool GVA, bool ACC = false>
 __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(const WyBwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     // du and dw share one tile (du is dead once A^T du is formed) and v, which is only read element-wise,
@@ -494,10 +498,13 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
     TileCopy<kThreads, kChunk, K> tk;
     tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-    f32x4 dk_acc[GVA ? KT : 1];
+    constexpr bool HOLD = GVA || ACC;   // dk tiles stay in registers until the head loop ends
+    f32x4 dk_acc[HOLD ? KT : 1];
 #pragma unroll
-    for (int ct = 0; ct < (GVA ? KT : 1); ++ct) dk_acc[ct] = zero4();
+    for (int ct = 0; ct < (HOLD ? KT : 1); ++ct) dk_acc[ct] = zero4();
     char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
+    TileCopy<kThreads, kChunk, K> tdk;
+    if constexpr (ACC) tdk.fetch(reinterpret_cast<const elem *>(dkg), p.dk.st, len, tid);
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
@@ -571,7 +578,7 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
                 db_row[e] += (p2[e] + p1g) * kv;
                 dg_row[e] += (p1g * br[e] + br[e] * p2[e] - q3[e]) * kv;
             }
-            if constexpr (GVA) dk_acc[ct] += dk;
+            if constexpr (HOLD) dk_acc[ct] += dk;
             else acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk);
             __builtin_amdgcn_sched_barrier(0);   // keeps the operand reads of later column tiles from piling up in registers
         }
@@ -581,11 +588,36 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             const int row = 16 * w + 4 * lg + e;
             if (li == 0 && row < len) {
                 p.dbeta[b * p.db_sb + hv * p.db_sh + (int64_t)(start + row) * p.db_st] = sb;
-                p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st] = sg;
+                float *dgp = p.dg + b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + row) * p.dg_st;
+                *dgp = ACC ? *dgp + sg : sg;
             }
         }
     }
-    if constexpr (GVA) {
+    if constexpr (ACC) {
+        constexpr int pf = K + 4;
+        static_assert((size_t)kChunk * pf * 4 <= (size_t)kChunk * (pk + px) * 2, "the fp32 dk tile must fit the k and dw tiles");
+        float *fS = reinterpret_cast<float *>(smem);
+        __syncthreads();   // the last reads of k and dw are done
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) fS[(16 * w + 4 * lg + e) * pf + 16 * ct + li] = dk_acc[ct][e];
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < TileCopy<kThreads, kChunk, K>::N; ++m) {
+            const int idx = m * kThreads + tid;
+            const int r = idx / (K / 8), c8 = (idx % (K / 8)) << 3;
+            const elemx8 in = __builtin_bit_cast(elemx8, tdk.r[m]);
+            const f32x4 lo = *reinterpret_cast<const f32x4 *>(fS + r * pf + c8), hi = *reinterpret_cast<const f32x4 *>(fS + r * pf + c8 + 4);
+            f32x4 a, c;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                a[e] = lo[e] + (float)in[e];
+                c[e] = hi[e] + (float)in[4 + e];
+            }
+            if (r < len) *reinterpret_cast<elemx8 *>(dkg + ((int64_t)r * p.dk.st + c8) * 2) = frag_from_acc(a, c);
+        }
+    } else if constexpr (GVA) {
 #pragma unroll
         for (int ct = 0; ct < KT; ++ct) acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, len, dk_acc[ct]);
     }
@@ -747,8 +779,8 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
                      const fla_tensor *dA, const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g,
                      const fla_int_array *cu, const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk,
                      const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size,
-                     hipStream_t stream, uint64_t *query) {
-    const char *op = "prepare_wy_repr_bwd_full";
+                     hipStream_t stream, uint64_t *query, bool accumulate = false) {
+    const char *op = accumulate ? "prepare_wy_repr_bwd_full_accumulate" : "prepare_wy_repr_bwd_full";
     ChunkGeom geom;
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
@@ -768,13 +800,19 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     const int K = geom.K, V = geom.V;
     const size_t smem = ((size_t)kChunk * ((K + 16) + ((K > V ? K : V) + 16) + V + 3 * (kChunk + 8))) * 2 + 2 * kChunk * 4;
     const bool gva = geom.Hv != geom.Hk;
-    if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128, false>), "wy_bwd_full", grid, smem, p);
-    if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 128, true>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 64 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64, false>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 64, true>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 128 && !gva) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, false>), "wy_bwd_full", grid, smem, p);
-    if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full_kernel<64, 128, true>), "wy_bwd_full", grid, smem, p);
-    if (K == 128 && V == 256) FLA_BWD_DISPATCH((wy_bwd_full_kernel<128, 256, true>), "wy_bwd_full", grid, smem, p);
+#define FLA_WY_FULL(KK, VV, G)                                                                                      \
+    do {                                                                                                            \
+        if (accumulate) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true>), "wy_bwd_full", grid, smem, p);      \
+        FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, false>), "wy_bwd_full", grid, smem, p);                     \
+    } while (0)
+    if (K == 128 && V == 128 && !gva) FLA_WY_FULL(128, 128, false);
+    if (K == 128 && V == 128) FLA_WY_FULL(128, 128, true);
+    if (K == 64 && V == 64 && !gva) FLA_WY_FULL(64, 64, false);
+    if (K == 64 && V == 64) FLA_WY_FULL(64, 64, true);
+    if (K == 64 && V == 128 && !gva) FLA_WY_FULL(64, 128, false);
+    if (K == 64 && V == 128) FLA_WY_FULL(64, 128, true);
+    if (K == 128 && V == 256) FLA_WY_FULL(128, 256, true);
+#undef FLA_WY_FULL
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 
@@ -898,6 +936,26 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_full)(
     FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
                                  workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
+    FLA_NULL_WS("prepare_wy_repr_bwd_full_accumulate");
+    return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 nullptr, 0, nullptr, workspace_size, true); });
+}
+FLA_ENTRY(fla_prepare_wy_repr_bwd_full_accumulate)(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
+    return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
+                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, true); });
 }
 
 FLA_ENTRY(fla_prepare_wy_repr_bwd_get_workspace_size)(

@@ -48,6 +48,10 @@ struct FusedParams {
     int slabs;
     int remap;          // 1: co-locate the slabs of one head on one XCD
     int l2norm;         // 1: q and k rows are L2-normalised (rstd = 1/sqrt(sum x^2 + 1e-6)) while they are staged
+    // what a backward pass needs from the forward, each or null (pipelined kernel only):
+    elem *h_out;        // state at the start of every chunk [B,Hv,NT,K,V]
+    int64_t h_sb, h_sh, h_sc;
+    View4 vn_out, w_out;   // v_new [B,Hv,T,V], w [B,Hv,T,K]
 };
 
 template <int K, int CT> struct FusedSmem {
@@ -626,7 +630,8 @@ __device__ __forceinline__ Tiles pipe_tiles_at(unsigned char *smem, int c) {
 // e^{G_last - G_t} per token (decay of v_new towards the chunk end), after the 16 block factors
 __device__ __forceinline__ float *pipe_decay_table(const Tiles &t) { return t.BLKF + 16; }
 
-template <int K>
+// TRAIN: the state group also writes h, v_new and w (the operands the backward operators would otherwise recompute).
+template <int K, bool TRAIN>
 __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     typedef PipeSmem<K> L;
     constexpr int VS = 64, pq = L::pq, pv = L::pv, pa = L::pa, pw = L::pw, pp = L::pp, pd = L::pd;
@@ -836,10 +841,6 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     // bookkeeping carries them around the loop and turns every first use of the state into a wait for
     // ALL outstanding memory operations, including the gate loads issued for the next chunk.
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
-    char *obase = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + (int64_t)bos * p.o.st + vcol0);
-    // lane part of an output tile's address: rows 4lg (+2 for odd lanes), column pair of the lane
-    const unsigned o_lane = (unsigned)((4 * lg + ((li & 1) ? 2 : 0)) * p.o.st * 2 + (li & ~1) * 2);
-    const unsigned o_row = (unsigned)(p.o.st * 2);
     const float *gptr = static_cast<const float *>(p.g.p) + b * p.g.sb + hv * p.g.sh;
     const float *bptr = static_cast<const float *>(p.beta.p) + b * p.beta.sb + hv * p.beta.sh;
     float pre_g = 0.f, pre_b = 0.f;
@@ -920,6 +921,21 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
                     for (int rt = 0; rt < 4; ++rt) U[rt] = mfma16x32(wf[j][rt], hB[j], U[rt]);
                 FLA_SCHED_FENCE();
+            }
+            if constexpr (TRAIN) {
+                if (p.w_out.p != nullptr && slab == 0) {   // the tile holds -w: whole rows out, sign bits flipped
+                    const int gt = threadIdx.x - GT, rw = gt / (K / 8), cw = (gt % (K / 8)) * 8;
+                    char *wg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.w_out.p)) + b * p.w_out.sb +
+                                                        hv * p.w_out.sh + (int64_t)(bos + c * kChunk) * p.w_out.st);
+#pragma unroll
+                    for (int m = 0; m < QCH; ++m) {
+                        const int row = rw + m * QROWS;
+                        u32x4 x = *reinterpret_cast<const u32x4 *>(wS + row * pw + cw);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[e] ^= 0x80008000u;
+                        if (row < len) *reinterpret_cast<u32x4 *>(wg + ((int64_t)row * p.w_out.st + cw) * 2) = x;
+                    }
+                }
             }
             elemx8 kfa[KT], kfb[KT];
             f32x4 dk4[4];
@@ -1011,6 +1027,25 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
             // this wave's 16 columns of o into the staging tile; the prep group writes whole rows to memory
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) acc_to_tile(oS, po, 16 * rt, 16 * wv, oacc[rt]);
+            if constexpr (TRAIN) {
+                // this half leaves the state group waiting for the prep group: the stores ride in that slack
+                if (p.h_out != nullptr) {   // the state the chunk started from, rounded as the products above used it
+                    const int chunk = (p.geom.choff != nullptr ? p.geom.choff[n] : 0) + c;
+                    char *hg = reinterpret_cast<char *>(p.h_out + b * p.h_sb + hv * p.h_sh + (int64_t)chunk * p.h_sc + vcol0);
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) {
+                        const u32x4 d = __builtin_bit_cast(u32x4, hB[j]);
+                        packed_to_global(hg, (int64_t)V * 2, 32 * j, K, d[0], d[1]);
+                        packed_to_global(hg, (int64_t)V * 2, 32 * j + 16, K, d[2], d[3]);
+                    }
+                }
+                if (p.vn_out.p != nullptr) {
+                    char *vg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.vn_out.p)) + b * p.vn_out.sb +
+                                                        hv * p.vn_out.sh + (int64_t)(bos + c * kChunk) * p.vn_out.st + vcol0);
+#pragma unroll
+                    for (int rt = 0; rt < 4; ++rt) acc_to_global(vg, p.vn_out.st * 2, 16 * rt, len, U[rt]);
+                }
+            }
         } else {
             if (i + 1 < nchunks) gate_tables(i + 1, pipe_tiles_at<K>(smem, i + 1));
             if (i + 2 < nchunks) gate_fetch(i + 2);
@@ -1026,14 +1061,15 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
     }
 }
 
-template <int K>
+template <int K, bool TRAIN>
 int launch_pipe(FusedParams &p, hipStream_t stream) {
     typedef PipeSmem<K> L;
     const int64_t total = (int64_t)p.geom.N * p.geom.Hv * p.slabs;
     p.remap = (p.slabs == 2 && total % 16 == 0) ? 1 : 0;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gdn_pipe_kernel<K>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gdn_pipe_kernel<K, TRAIN>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::bytes));
-    FLA_LAUNCH("gdn_fused", stream, (gdn_pipe_kernel<K>), dim3((unsigned)total), dim3(512), L::bytes, stream, p);
+    FLA_LAUNCH(TRAIN ? "gdn_fused_train" : "gdn_fused", stream, (gdn_pipe_kernel<K, TRAIN>), dim3((unsigned)total), dim3(512),
+               L::bytes, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -1053,6 +1089,7 @@ int launch_fused(FusedParams &p, hipStream_t stream) {
 int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
                double scale, const fla_tensor *initial_state, bool output_final_state, const fla_int_array *cu,
                int64_t chunk_size, bool use_qk_l2norm, const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
+               const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w,
                void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "gdn_chunk_fwd";
     ChunkGeom geom;
@@ -1099,6 +1136,17 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (output_final_state && (rc = check_state(final_state, "final_state"))) return rc;
     FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
     FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
+    // operands of the backward pass, each optional
+    const bool has_h = h && h->data, has_vn = v_new && v_new->data, has_w = w && w->data;
+    if (has_h) {
+        if ((rc = check_tensor(h, op, "h", 5, bf))) return rc;
+        FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
+                        h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 2 == 0 &&
+                        h->stride[1] % 2 == 0 && h->stride[0] % 2 == 0 && reinterpret_cast<uintptr_t>(h->data) % 4 == 0,
+                    FLA_ERR_SHAPE, "%s: h must be [B,Hv,NT=%d,K,V] with contiguous K x V blocks.", op, geom.NT);
+    }
+    if (has_vn && (rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if (has_w && (rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if (query) {
         *query = vl.bytes();
         return FLA_OK;
@@ -1142,9 +1190,19 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     // per head; 64-column slabs double the number of workgroups and run as the two-group pipelined kernel.  The wide
     // form is used once it alone fills the GPU; the in-kernel normalisation lives in the pipelined kernel's tile commit.
     const int64_t chains = (int64_t)geom.N * geom.Hv;
-    const bool wide = !use_qk_l2norm && geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
+    const bool train = has_h || has_vn || has_w;
+    if (has_h) {
+        p.h_out = static_cast<elem *>(h->data);
+        p.h_sb = h->stride[0];
+        p.h_sh = h->stride[1];
+        p.h_sc = h->stride[2];
+    }
+    if (has_vn) p.vn_out = view4(v_new);
+    if (has_w) p.w_out = view4(w);
+    const bool wide = !train && !use_qk_l2norm && geom.V % 128 == 0 && chains * (geom.V / 128) >= (int64_t)num_cus();
     p.slabs = wide ? geom.V / 128 : geom.V / 64;
-    if (!wide) return geom.K == 128 ? launch_pipe<128>(p, stream) : launch_pipe<64>(p, stream);
+    if (train) return geom.K == 128 ? launch_pipe<128, true>(p, stream) : launch_pipe<64, true>(p, stream);
+    if (!wide) return geom.K == 128 ? launch_pipe<128, false>(p, stream) : launch_pipe<64, false>(p, stream);
     return geom.K == 128 ? launch_fused<128, 2>(p, stream) : launch_fused<64, 2>(p, stream);
 }
 
@@ -1157,21 +1215,23 @@ FLA_ENTRY(fla_gdn_chunk_fwd_get_workspace_size)(const fla_tensor *q, const fla_t
                                                     const fla_int_array *cu_seqlens, int64_t chunk_size,
                                                     bool use_qk_l2norm_in_kernel, const fla_tensor *o,
                                                     const fla_tensor *g_cumsum, const fla_tensor *final_state,
+                                                    const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w,
                                                     uint64_t *workspace_size) {
-    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace_size);
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd: workspace_size must not be null.");
     return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, nullptr, 0, nullptr, workspace_size); });
+                           g_cumsum, final_state, h, v_new, w, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
                                  const fla_tensor *beta, double scale, const fla_tensor *initial_state,
                                  bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
                                  bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
-                                 const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream) {
-    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, workspace, workspace_size, stream);
+                                 const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
+                                 const fla_tensor *w, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+                           g_cumsum, final_state, h, v_new, w, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -155,11 +155,10 @@ __device__ __forceinline__ void acc_to_tile(elem *tile, int pitch, int r0, int c
 
 // One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with
 // `stride` bytes between rows; `base` points at column c0 of row 0).  Lane pairs exchange halves as in
-// acc_to_tile so that every lane writes two whole dwords.
-__device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
+// acc_to_tile so that every lane writes two whole dwords.  packed_to_global takes the tile already rounded:
+// p01 = rows 4lg, 4lg + 1 and p23 = rows 4lg + 2, 4lg + 3 of the lane's column, two elements per dword.
+__device__ __forceinline__ void packed_to_global(char *base, int64_t stride, int r0, int len, unsigned p01, unsigned p23) {
     const int l = lane_id(), li = l & 15, lg = l >> 4;
-    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
-    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
     const bool odd = li & 1;
     const unsigned send = odd ? p01 : p23;
     const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
@@ -168,6 +167,10 @@ __device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0
     char *dst = base + row * stride + (li & ~1) * 2;
     if (row < len) *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);
     if (row + 1 < len) *reinterpret_cast<unsigned *>(dst + stride) = __builtin_amdgcn_perm(right, left, 0x07060302u);
+}
+__device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
+    packed_to_global(base, stride, r0, len, __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1])),
+                     __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3])));
 }
 
 // ---- the k tile -------------------------------------------------------------------------------

@@ -34,7 +34,7 @@ OP_ARGTYPES = {
                                      ctypes.c_bool, _T, _T, _T],
     "chunk_fwd_o": [_T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
     "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, ctypes.c_bool,
-                      _T, _T, _T],
+                      _T, _T, _T, _T, _T, _T],
     "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
@@ -53,6 +53,7 @@ OP_ARGTYPES = {
                        + [_T] * 4,
     "prepare_wy_repr_bwd_da": [_T] * 7 + [_IA, _IA, ctypes.c_int64, _T],
     "prepare_wy_repr_bwd_full": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
+    "prepare_wy_repr_bwd_full_accumulate": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
     "prepare_wy_repr_bwd": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
     "chunk_kda_bwd_dav": [_T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T, _T],
     "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 4,
@@ -396,11 +397,13 @@ def npu_solve_tri(x, *, cu_seqlens=None, chunk_indices=None, layout="bsnd", outp
 
 
 def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
-                  use_qk_l2norm_in_kernel=False):
+                  use_qk_l2norm_in_kernel=False, *, save_for_backward=False):
     """Whole chunk forward in one library call (replaces the composition at
     examples/flash_gated_delta_rule.py:796-881).  q,k,v [B,H,T,D]; g,beta [B,T,H] f32.
     use_qk_l2norm_in_kernel normalises q and k rows inside the kernel (flash_gated_delta_rule.py:1047-1049).
-    Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], final_state or None)."""
+    Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], final_state or None); with ``save_for_backward`` also
+    (h [B,HV,NT,K,V], v_new [B,HV,T,V], w [B,HV,T,K]), the operands the reference's backward recomputes
+    (flash_gated_delta_rule.py:913-951)."""
     import torch
 
     B, _, T, K = _shape(k)
@@ -410,6 +413,13 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
     o = _empty((B, T, HV, V), v)
     g_out = _empty((B, T, HV), v, dtype=torch.float32)
     final = _empty((N, HV, K, V), v, dtype=torch.float32) if output_final_state else None
+    h = v_new = w = None
+    if save_for_backward:
+        C = 64
+        NT = -(-T // C) if cu is None else sum(-(-(cu[i + 1] - cu[i]) // C) for i in range(N))
+        h = _empty((B, HV, NT, K, V), v)
+        v_new = _empty((B, HV, T, V), v)
+        w = _empty((B, HV, T, K), v)
     _call_op(
         "gdn_chunk_fwd", OP_ARGTYPES["gdn_chunk_fwd"],
         lambda ctx: [
@@ -418,9 +428,12 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
             ctypes.c_bool(bool(output_final_state)), ctx.int_array(cu), ctypes.c_int64(int(chunk_size)),
             ctypes.c_bool(bool(use_qk_l2norm_in_kernel)),
             ctx.tensor(o, "o"), ctx.tensor(g_out, "g_cumsum"), ctx.tensor(final, "final_state"),
+            ctx.tensor(h, "h"), ctx.tensor(v_new, "v_new"), ctx.tensor(w, "w"),
         ],
         (o, g_out, final),
     )
+    if save_for_backward:
+        return g_out, o, final, h, v_new, w
     return g_out, o, final
 
 
@@ -915,6 +928,27 @@ def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu
         outputs,
     )
     return dk, dv, _as_dtype(dbeta, beta), _as_dtype(dg, g)
+
+
+def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, chunk_size, *, cu_seqlens=None,
+                                        chunk_indices=None):
+    """npu_prepare_wy_repr_bwd_full with its key and gate gradients ADDED to ``dk`` ([B,Hk,T,K], dtype of k) and
+    ``dg`` ([B,Hv,T] f32) in place: the reference's composition adds them with a separate pass
+    (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32)."""
+    dv = _empty_like(v)
+    dbeta = _f32_like(beta)
+    dv, dbeta = _call_op(
+        "prepare_wy_repr_bwd_full_accumulate", OP_ARGTYPES["prepare_wy_repr_bwd_full_accumulate"],
+        lambda ctx: [
+            ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"), ctx.tensor(dA, "dA"),
+            ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(dbeta, "dbeta"), ctx.tensor(dg, "dg"),
+        ],
+        (dv, dbeta),
+    )
+    return dv, dbeta
 
 
 def npu_prepare_wy_repr_bwd(k, v, beta, A, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):

@@ -32,11 +32,13 @@ def _cu_list(cu_seqlens):
 
 def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
                                      cu_seqlens=None, chunk_size: int = 64, *, fused: bool = True,
-                                     use_qk_l2norm_in_kernel: bool = False):
+                                     use_qk_l2norm_in_kernel: bool = False, save_for_backward: bool = False):
     """q,k,v [B,H,T,D] bf16; g,beta [B,T,H].  Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], A, final_state);
     ``A`` ([B,H,T,C] bf16, the inverted chunk matrices) is None on the fused route.  With
     ``use_qk_l2norm_in_kernel`` the fused route normalises q and k rows while it stages them; the composed
-    route runs the two normalisation passes first (examples/flash_gated_delta_rule.py:1047-1049)."""
+    route runs the two normalisation passes first (examples/flash_gated_delta_rule.py:1047-1049).
+    ``save_for_backward`` appends a dict with h, v_new and w, which the backward then does not recompute
+    (64-token chunks only)."""
     import torch
 
     cu = _cu_list(cu_seqlens)
@@ -46,10 +48,13 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
         h0 = initial_state
         if h0 is not None and h0.dtype != torch.float32:
             h0 = h0.float()
-        gc, o, final = _raw.gdn_chunk_fwd(q, k, v, g.float(), beta.float(), scale, h0,
-                                          output_final_state, cu, chunk_size, use_qk_l2norm_in_kernel)
+        res = _raw.gdn_chunk_fwd(q, k, v, g.float(), beta.float(), scale, h0, output_final_state, cu, chunk_size,
+                                 use_qk_l2norm_in_kernel, save_for_backward=save_for_backward)
+        gc, o, final = res[:3]
         if final is not None and initial_state is not None and final.dtype != initial_state.dtype:
             final = final.to(initial_state.dtype)
+        if save_for_backward:
+            return gc, o, None, final, dict(zip(("h", "v_new", "w"), res[3:]))
         return gc, o, None, final
     if use_qk_l2norm_in_kernel:
         q, _ = _raw.l2norm_fwd(q)
@@ -65,17 +70,21 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
         k, w, u, g=gh, initial_state=initial_state, output_final_state=output_final_state,
         chunk_size=chunk_size, cu_seqlens=cu)
     o = _ops.chunk_fwd_o(q, k, v_new, h, scale, g=gh, cu_seqlens=cu, chunk_size=chunk_size, out_token_major=True)
-    return gh.transpose(1, 2).contiguous(), o.transpose(1, 2).contiguous(), A, \
-        (final if output_final_state else None)
+    out = (gh.transpose(1, 2).contiguous(), o.transpose(1, 2).contiguous(), A, (final if output_final_state else None))
+    if save_for_backward:
+        return out + (dict(h=h, v_new=v_new, w=w),)
+    return out
 
 
 def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, do, dht, cu_seqlens=None,
-                                     chunk_size: int = 64):
+                                     chunk_size: int = 64, *, saved=None):
     """q,k,v [B,H,T,D] bf16; ``g`` the chunk-cumsummed gate and beta [B,T,H] (as the forward returned /
     received them); ``A`` [B,H,T,C] the inverted chunk matrices or None (recomputed); do [B,T,H,V];
     dht [N,H,K,V] fp32 or None.  Returns (dq, dk, dv [B,H,T,D], dbeta, dg [B,T,H] fp32, dh0 [N,H,K,V] fp32 or
     None); dg is the gradient of the RAW gate.  Unlike the reference, the initial state and the final-state
-    gradient take part (the reference passes neither to its reverse scan and returns dh0 = None)."""
+    gradient take part (the reference passes neither to its reverse scan and returns dh0 = None).
+    ``saved``: the dict of h, v_new and w the forward wrote with ``save_for_backward``; without it they are
+    recomputed as the reference does (examples/flash_gated_delta_rule.py:913-951)."""
     import torch
 
     cu = _cu_list(cu_seqlens)
@@ -88,18 +97,22 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     elif A is None:
         A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
         A = _ops.solve_tri(A, layout="bnsd", output_dtype=k.dtype, **kw)   # rounds A to k.dtype on load
-    w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
     doh = do.transpose(1, 2) if do.stride(-1) == 1 else do.transpose(1, 2).contiguous()
-    h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,
-                                                    output_final_state=False, chunk_size=chunk_size, **kw)
+    if saved is not None:
+        h, v_new, w = saved["h"], saved["v_new"], saved["w"]
+    else:
+        w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
+        h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,
+                                                        output_final_state=False, chunk_size=chunk_size, **kw)
     dv = _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
     dh, dh0, dv = _ops.chunk_gated_delta_rule_bwd_dhu(q, k, w, doh, dv, scale, chunk_size, g=gh, h0=initial_state,
                                                       dht=dht, dh0_per_sequence=True, **kw)
     dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
     dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
-    dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
-    dk.add_(dk2)
-    dg = _ops.chunk_local_cumsum(dg + dg2, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
+    # the second part of dk and dg is added where it is produced (the reference adds with separate passes,
+    # examples/flash_gated_delta_rule.py:994-1012)
+    dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size, **kw)
+    dg = _ops.chunk_local_cumsum(dg, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
     return dq, dk, dv, db.transpose(1, 2), dg.transpose(1, 2), dh0
 
 
@@ -121,18 +134,20 @@ def _autograd_function():
             if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049
                 q, q_rstd = _raw.l2norm_fwd(q)
                 k, k_rstd = _raw.l2norm_fwd(k)
-            gc, o, A, final = flash_chunk_gated_delta_rule_fwd(
-                q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused)
-            ctx.save_for_backward(q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd)
+            gc, o, A, final, saved = flash_chunk_gated_delta_rule_fwd(
+                q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused,
+                save_for_backward=True)
+            ctx.save_for_backward(q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd, saved["h"], saved["v_new"], saved["w"])
             ctx.scale, ctx.cu, ctx.chunk_size = scale, cu, chunk_size
             ctx.dtypes = (g.dtype, beta.dtype)
             return o, final
 
         @staticmethod
         def backward(ctx, do, dht):
-            q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd = ctx.saved_tensors
+            q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd, h, v_new, w = ctx.saved_tensors
             dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
-                q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(), dht, ctx.cu, ctx.chunk_size)
+                q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(), dht, ctx.cu, ctx.chunk_size,
+                saved=dict(h=h, v_new=v_new, w=w))
             if q_rstd is not None:      # :1104-1106
                 dq = _raw.l2norm_bwd(q, q_rstd, dq)
                 dk = _raw.l2norm_bwd(k, k_rstd, dk)

@@ -211,19 +211,25 @@ int fla_chunk_fwd_o(
  * use_qk_l2norm_in_kernel: q and k rows are scaled by 1/sqrt(sum x^2 + 1e-6)
  * while they are staged, as fla's l2norm_fwd does ahead of the chunk forward
  * (examples/flash_gated_delta_rule.py:1086-1089).
+ * h [B,Hv,NT,K,V] (state at the start of every chunk), v_new [B,Hv,T,V] and
+ * w [B,Hv,T,K], all bf16 and each NULL or given: what the reference's backward
+ * recomputes with recompute_w_u_fwd and chunk_gated_delta_rule_fwd_h
+ * (examples/flash_gated_delta_rule.py:913-951), written by the forward instead.
  * ------------------------------------------------------------------------ */
 int fla_gdn_chunk_fwd_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, double scale, const fla_tensor *initial_state,
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
     bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
-    const fla_tensor *final_state, uint64_t *workspace_size);
+    const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *w, uint64_t *workspace_size);
 int fla_gdn_chunk_fwd(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, double scale, const fla_tensor *initial_state,
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
     bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
-    const fla_tensor *final_state, void *workspace, uint64_t workspace_size, void *stream);
+    const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
+    const fla_tensor *w, void *workspace, uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
  * recurrent_gated_delta_rule - replaces aclnnRecurrentGatedDeltaRule
@@ -572,6 +578,21 @@ int fla_prepare_wy_repr_bwd_full_get_workspace_size(
     const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
     const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size);
 int fla_prepare_wy_repr_bwd_full(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+
+/* prepare_wy_repr_bwd_full_accumulate - no counterpart in the reference, whose composition adds the two
+ * key gradients with a separate elementwise pass (examples/flash_gated_delta_rule.py:994-1010, dk.add_(dk2)).
+ * Same operands as prepare_wy_repr_bwd_full; dk and dg are read, the operator's results added in fp32, and
+ * written back in place (dk rounded once).  dv and dbeta are written as usual. */
+int fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size(
+    const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+    const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size);
+int fla_prepare_wy_repr_bwd_full_accumulate(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,

@@ -121,6 +121,18 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     for name, a_, b_ in zip(("dk", "dv", "dbeta", "dg"), one, two):
         assert torch.equal(a_, b_), name
 
+    # the accumulating form adds the same dk and dg (taken in fp32) to what the caller's tensors hold
+    from fla_hip.ops import _hip_ctypes as raw
+    torch.manual_seed(5)
+    dk_acc = (torch.randn_like(two[0].float()) * two[0].float().abs().mean()).to(dtype)
+    dg_acc = torch.randn_like(two[3]) * two[3].abs().mean()
+    dk0, dg0 = dk_acc.clone(), dg_acc.clone()
+    dv_a, db_a = raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], x["A"], dA, dwb.to(dev), dv2.to(dev),
+                                                         x["G"], dk_acc, dg_acc, 64, **kw)
+    assert torch.equal(dv_a, two[1]) and torch.equal(db_a, two[2])
+    assert_close(dk_acc, dk0.float() + dk2_r.to(dev), TOL_BF16, "dk accumulated")
+    assert_close(dg_acc, dg0 + two[3], 1e-6, "dg accumulated")
+
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", [CASES[1], CASES[5], CASES[6]])

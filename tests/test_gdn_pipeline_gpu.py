@@ -51,6 +51,36 @@ def test_against_naive_recurrence(dev, case, fused, dtype):
     assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
 
 
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", CASES)
+def test_forward_writes_the_operands_of_the_backward(dev, case, dtype):
+    """save_for_backward: h (state at every chunk start), v_new and w as the stage-by-stage fp32 restatement computes
+    them (recompute_w_u_fwd/README.md:12-32, chunk_gated_delta_rule_fwd_h/README.md:16-30), while o, the final state
+    and the cumulated gate stay bit-identical to the call without them."""
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, H, Hk, K, V, cu = case
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=dtype, seed=T + 2 * H, Hk=Hk)
+    N = B if cu is None else len(cu) - 1
+    h0 = torch.randn(N, H, K, V, generator=torch.Generator().manual_seed(4)) * 0.01
+    x = {n: d[n].to(dev) for n in ("q", "k", "v", "g", "beta")}
+    scale = K ** -0.5
+    plain = raw.gdn_chunk_fwd(x["q"], x["k"], x["v"], x["g"], x["beta"], scale, h0.to(dev), True, cu, 64)
+    gc, o, final, h, v_new, w = raw.gdn_chunk_fwd(x["q"], x["k"], x["v"], x["g"], x["beta"], scale, h0.to(dev), True,
+                                                  cu, 64, save_for_backward=True)
+    for name, a, b in zip(("g_cumsum", "o", "final_state"), (gc, o, final), plain):
+        assert torch.equal(a, b), name
+    _, _, mid = gdn.chunk_gated_delta_rule_fwd(d["q"], d["k"], d["v"], d["g"].transpose(1, 2), d["beta"].transpose(1, 2),
+                                               scale, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                                               return_intermediates=True)
+    NT = gdn.total_chunks(B, T, 64, cu)
+    assert h.shape == (B, H, NT, K, V) and v_new.shape == (B, H, T, V) and w.shape == (B, H, T, K)
+    assert h.dtype == dtype and v_new.dtype == dtype and w.dtype == dtype
+    tol = TOL_BF16 if dtype == BF else TOL_BF16 / 4
+    assert_close(w, mid["w"], tol, "w")
+    assert_close(v_new, mid["v_new"], tol, "v_new")
+    assert_close(h, mid["h"], tol, "h")
+
+
 # Batches large enough that the host picks the kernels with 128-column value slabs: the fused forward once
 # sequences x heads x (V / 128) reaches the number of compute units (256), the stand-alone state scan at twice that.
 WIDE_CASES = [
