@@ -230,6 +230,103 @@ __global__ void __launch_bounds__(kThreads) recurrent_gdn_kernel(const RecParams
     }
 }
 
+// Any head size up to 512 x 512 with Dk a multiple of 4: the rows of the state are independent recurrences
+// (row v needs only S[v,:], k_t, q_t, v_t[v]), so the workgroup takes 16 rows at a time through all tokens of the
+// sequence, a row spread over one 16-lane DPP row in 16-byte pieces 64 columns apart, as in the sized kernel.
+// The state still moves once in and out per slot change; q, k and the gates are re-read for every 16 rows.
+template <typename ST>
+__global__ void __launch_bounds__(kThreads) recurrent_gdn_anysize_kernel(const RecParams p, int Dk, int Dv) {
+    constexpr int MAXSEG = 8;                 // 512 columns
+    __shared__ int s_red[kThreads / kWave];
+    const int n = blockIdx.x / p.Nv, h = blockIdx.x % p.Nv;
+    const int hk = h / (p.Nv / p.Nk);
+    const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+    const int col = (lane % 16) * 4, rw = wave * 4 + lane / 16;
+
+    int part = 0;
+    for (int j = tid; j <= n; j += kThreads) part += p.seq_lens[j];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+    if (lane == 0) s_red[wave] = part;
+    __syncthreads();
+    int tok0 = 0;
+#pragma unroll
+    for (int w = 0; w < kThreads / kWave; ++w) tok0 += s_red[w];
+    const int len = p.seq_lens[n + 1];
+    if (len <= 0 || tok0 + len > p.T) return;
+    int src_tok = tok0;
+    if (p.accepted) src_tok = tok0 + p.accepted[n] - 1;
+    if (src_tok < 0 || src_tok >= p.T) return;
+    const int src_slot = p.slot_idx[src_tok];
+    if (src_slot < 0 || src_slot >= p.n_blocks) return;
+
+    ST *state = static_cast<ST *>(p.state);
+    const int nseg = (Dk + 63) / 64;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int r0 = 0; r0 < Dv; r0 += 16) {
+        const int row = r0 + rw;
+        const bool row_ok = row < Dv;
+        f32x4 S[MAXSEG];
+#pragma unroll
+        for (int sg = 0; sg < MAXSEG; ++sg) {
+            const int c = col + 64 * sg;
+            S[sg] = zero;
+            if (sg < nseg && row_ok && c < Dk) S[sg] = StateIO<ST>::load(state + src_slot * p.s_sb + h * p.s_sh + (int64_t)row * p.s_sv + c);
+        }
+        for (int j = 0; j < len; ++j) {
+            const int64_t tok = tok0 + j;
+            const float decay = p.g ? __expf(p.g[tok * p.g_st + h * p.g_sh]) : 1.f;
+            const float beta = (float)p.beta[tok * p.b_st + h * p.b_sh];
+            const float vt = row_ok ? (float)p.v[tok * p.v_st + h * p.v_sh + row] : 0.f;
+            f32x4 kv[MAXSEG], qv[MAXSEG];
+            float sk = 0.f;
+#pragma unroll
+            for (int sg = 0; sg < MAXSEG; ++sg) {
+                const int c = col + 64 * sg;
+                kv[sg] = zero;
+                qv[sg] = zero;
+                if (sg < nseg && c < Dk) {
+                    const bf16x4 k4 = *reinterpret_cast<const bf16x4 *>(p.k + tok * p.k_st + hk * p.k_sh + c);
+                    const bf16x4 q4 = *reinterpret_cast<const bf16x4 *>(p.q + tok * p.q_st + hk * p.q_sh + c);
+                    f32x4 dec = {decay, decay, decay, decay};
+                    if (p.gk) {
+                        const f32x4 g4 = *reinterpret_cast<const f32x4 *>(p.gk + tok * p.gk_st + h * p.gk_sh + c);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) dec[e] *= __expf(g4[e]);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        kv[sg][e] = (float)k4[e];
+                        qv[sg][e] = (float)q4[e] * p.scale;
+                    }
+                    S[sg] *= dec;
+                    sk += S[sg][0] * kv[sg][0] + S[sg][1] * kv[sg][1] + S[sg][2] * kv[sg][2] + S[sg][3] * kv[sg][3];
+                }
+            }
+            const float delta = beta * (vt - group_sum<16>(sk));
+            float so = 0.f;
+#pragma unroll
+            for (int sg = 0; sg < MAXSEG; ++sg) {
+                if (sg < nseg) {
+                    S[sg] += delta * kv[sg];
+                    so += S[sg][0] * qv[sg][0] + S[sg][1] * qv[sg][1] + S[sg][2] * qv[sg][2] + S[sg][3] * qv[sg][3];
+                }
+            }
+            so = group_sum<16>(so);
+            if (lane % 16 == 0 && row_ok) p.out[tok * p.o_st + h * p.o_sh + row] = (bf16)so;
+            const int slot = p.slot_idx[tok];
+            const int next = j + 1 < len ? p.slot_idx[tok + 1] : -1;
+            if (slot != next && slot >= 0 && slot < p.n_blocks && row_ok) {
+#pragma unroll
+                for (int sg = 0; sg < MAXSEG; ++sg) {
+                    const int c = col + 64 * sg;
+                    if (sg < nseg && c < Dk) StateIO<ST>::store(state + slot * p.s_sb + h * p.s_sh + (int64_t)row * p.s_sv + c, S[sg]);
+                }
+            }
+        }
+    }
+}
+
 int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *value, const fla_tensor *beta,
              const fla_tensor *state, const fla_tensor *actual_seq_lengths, const fla_tensor *ssm_state_indices,
              const fla_tensor *g, const fla_tensor *gk, const fla_tensor *num_accepted_tokens, float scale,
@@ -279,10 +376,13 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
     FLA_REQUIRE(is_contiguous(actual_seq_lengths) && is_contiguous(ssm_state_indices) &&
                     (!has_acc || is_contiguous(num_accepted_tokens)),
                 FLA_ERR_SHAPE, "%s: index tensors must be contiguous.", op);
-    const bool ok_dims = (Dk == 128 && Dv == 128) || (Dk == 64 && Dv == 64) || (Dk == 128 && Dv == 256) ||
-                         (Dk == 64 && Dv == 128);
-    FLA_REQUIRE(ok_dims, FLA_ERR_UNSUPPORTED, "%s: (Dk,Dv)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(128,256),(64,128).",
+    // four head sizes have a kernel that keeps the whole state tile in registers; every other one up to the
+    // reference's 512 x 512 (torch_custom/fla_npu/fla_npu/ops/ascendc/_aclnn_ctypes.py:813-817) takes the row-block kernel
+    const bool sized = (Dk == 128 && Dv == 128) || (Dk == 64 && Dv == 64) || (Dk == 128 && Dv == 256) ||
+                       (Dk == 64 && Dv == 128);
+    FLA_REQUIRE(Dk >= 1 && Dv >= 1 && Dk <= 512 && Dv <= 512, FLA_ERR_SHAPE, "%s: Dk and Dv must be <= 512, got Dk=%lld, Dv=%lld.",
                 op, (long long)Dk, (long long)Dv);
+    FLA_REQUIRE(sized || Dk % 4 == 0, FLA_ERR_UNSUPPORTED, "%s: Dk must be a multiple of 4, got %lld.", op, (long long)Dk);
     FLA_REQUIRE(B * Nv < ((int64_t)1 << 31) && T < ((int64_t)1 << 31), FLA_ERR_SHAPE, "%s: extents exceed int32.", op);
     if (query_ws) {
         *query_ws = 0;
@@ -290,8 +390,16 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
     }
     if (T == 0 || B == 0) return FLA_OK;
 
-    // the per-batch staging reads q, k, v, gk and writes out in 16-byte pieces at most
-    {
+    if (!sized) {   // 8-byte pieces of q and k, 16-byte pieces of gk, scalar v and out
+        const fla_tensor *vec[] = {query, key};
+        for (const fla_tensor *t : vec)
+            FLA_REQUIRE(t->stride[0] % 4 == 0 && t->stride[1] % 4 == 0 && reinterpret_cast<uintptr_t>(t->data) % 8 == 0,
+                        FLA_ERR_SHAPE, "%s: query/key rows must be 8-byte aligned.", op);
+        if (has_gk)
+            FLA_REQUIRE(gk->stride[0] % 4 == 0 && gk->stride[1] % 4 == 0 && reinterpret_cast<uintptr_t>(gk->data) % 16 == 0,
+                        FLA_ERR_SHAPE, "%s: gk rows must be 16-byte aligned.", op);
+    } else {
+        // the per-batch staging reads q, k, v, gk and writes out in 16-byte pieces at most
         const fla_tensor *vec[] = {query, key, value, out};
         for (const fla_tensor *t : vec)
             FLA_REQUIRE(t->stride[2] == 1 && t->stride[0] % 8 == 0 && t->stride[1] % 8 == 0 &&
@@ -338,7 +446,10 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
         if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<float, DK, DV, 16>), grid, block, 0, stream, p);     \
         else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_kernel<bf16, DK, DV, 16>), grid, block, 0, stream, p);           \
     }
-    if (Dk == 128 && Dv == 128) { FLA_LAUNCH_REC(128, 128); }
+    if (!sized) {
+        if (f32s) FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_anysize_kernel<float>), grid, block, 0, stream, p, (int)Dk, (int)Dv);
+        else FLA_LAUNCH("recurrent_gdn", stream, (recurrent_gdn_anysize_kernel<bf16>), grid, block, 0, stream, p, (int)Dk, (int)Dv);
+    } else if (Dk == 128 && Dv == 128) { FLA_LAUNCH_REC(128, 128); }
     else if (Dk == 64 && Dv == 64) { FLA_LAUNCH_REC(64, 64); }
     else if (Dk == 128 && Dv == 256) { FLA_LAUNCH_REC(128, 256); }
     else { FLA_LAUNCH_REC(64, 128); }

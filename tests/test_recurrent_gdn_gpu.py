@@ -52,6 +52,23 @@ def test_single_token_decode(dev, dims):
     assert_close(st, s_ref, TOL_STATE, "state")
 
 
+@pytest.mark.parametrize("dims", [(16, 16), (48, 80), (96, 32), (192, 160), (256, 256), (512, 512), (320, 24), (128, 64), (100, 36)])
+def test_other_head_sizes(dev, dims):
+    """Head sizes without a register-resident kernel (the reference admits any Dk, Dv <= 512,
+    _aclnn_ctypes.py:813-817): multi-token sequences with slot changes, accepted-token source slots, both gates,
+    fp32 and bf16 pools."""
+    Dk, Dv = dims
+    d = make_inputs([3, 1, 6, 2], 2, 4, Dk, Dv, seed=Dk + Dv, blocks=30, gk=True)
+    acc = torch.tensor([2, 1, 4, 1], dtype=torch.int32)
+    o, o_ref, st, s_ref = run(dev, d, accepted=acc)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref, TOL_STATE, "state")
+    d = make_inputs([1] * 5, 2, 2, Dk, Dv, seed=Dk, state_dtype=torch.bfloat16)
+    o, o_ref, st, s_ref = run(dev, d)
+    assert_close(o, o_ref, TOL_BF16, "out")
+    assert_close(st, s_ref.bfloat16(), TOL_BF16, "state")
+
+
 def test_multi_token_and_skip_prefix(dev):
     d = make_inputs([3, 8, 1, 0, 5], 2, 2, 128, 128, seed=2, skip=2, blocks=40)
     o, o_ref, st, s_ref = run(dev, d)
