@@ -618,6 +618,33 @@ def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial
     if initial_state is not None and (_shape(initial_state) != state_shape or initial_state.dtype != torch.float32):
         raise RuntimeError(f"{op}: initial_state shape/dtype does not match state_v_first.")
 
+    # The kernels are built for K in {64, 128} with V in {K, 2K}.  Every other admitted head size with K <= 128 runs on
+    # the next built size with zero channels appended: a zero q/k channel adds nothing to any product and a zero v
+    # column yields zero u, v_new, o and state columns, so the leading K x V part of every result is unchanged.
+    Kp = 64 if K <= 64 and V <= 128 else 128
+    Vp = Kp if V <= Kp else 2 * Kp
+    if K > 128:
+        raise NotImplementedError(f"{op}: K={K} has no kernel; built: K <= 128 (V <= 256).")
+    if (Kp, Vp) != (K, V):
+        if noalloc:
+            raise NotImplementedError(f"{op}: (K,V)=({K},{V}) needs padded copies; the no-allocation entry takes "
+                                      "K in {64,128} with V in {K,2K} only.")
+        F = torch.nn.functional
+        padk = lambda t: F.pad(t, (0, Kp - K))
+        padv = lambda t: F.pad(t, (0, Vp - V))
+        state_pad = (0, Kp - K, 0, Vp - V) if state_v_first else (0, Vp - V, 0, Kp - K)
+        bias = None if dt_bias is None else padk(dt_bias.view(HV, K)).reshape(-1)
+        h0 = None if initial_state is None else F.pad(initial_state, state_pad)
+        res = _chunk_kda_fwd(noalloc, padk(q), padk(k), padv(v), padk(g), beta, scale, chunk_size, layout, h0,
+                             output_final_state, cu_seqlens, chunk_indices, safe_gate, lower_bound, use_gate_in_kernel, A_log,
+                             bias, disable_recompute, return_intermediate_states, state_v_first)
+        attn_out, final_state, gk, aqk, akk, w, u, qg, kg, v_new, h = res[:11]
+        cut = lambda t, n: None if t is None else t[..., :n].contiguous()
+        cut2 = lambda t: None if t is None else \
+            (t[..., :V, :K] if state_v_first else t[..., :K, :V]).contiguous()
+        return (cut(attn_out, V), cut2(final_state), cut(gk, K), aqk, akk, cut(w, K), cut(u, V), cut(qg, K), cut(kg, K),
+                cut(v_new, V), cut2(h), initial_state)
+
     lead = () if rank3 else (B,)
     block = (V, K) if state_v_first else (K, V)
     mask = kda_fwd_optional_output_mask(output_final_state=output_final_state, use_gate_in_kernel=use_gate_in_kernel,

@@ -87,6 +87,18 @@ CASES += [
 ]
 
 
+# head sizes between the built ones (the reference admits multiples of 16 up to 256, _aclnn_ctypes.py:1141): served by
+# zero channels appended in the wrapper
+CASES += [
+    dict(B=1, T=150, Hk=2, Hv=2, K=96, V=80, layout="BSND", h0=True),
+    dict(B=1, T=130, Hk=1, Hv=2, K=16, V=16, layout="TND", cu=[0, 65, 130], h0=True),
+    dict(B=1, T=100, Hk=2, Hv=2, K=48, V=160, layout="BNSD", v_first=True, h0=True),
+    dict(B=1, T=192, Hk=1, Hv=2, K=112, V=256, layout="BSND", chunk=128,
+         gate=dict(use_gate_in_kernel=True, bias=True, safe_gate=True, lower_bound=-5.0)),
+    dict(B=1, T=70, Hk=1, Hv=1, K=128, V=64, layout="NTD"),
+]
+
+
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items() if k in ("T", "K", "V", "layout", "chunk")))
 def test_chunk_kda_fwd(dev, case):
     from fla_hip import ops
