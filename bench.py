@@ -277,6 +277,25 @@ def bench_decode(args, torch, dev):
         prefill()
     torch.cuda.synchronize()
     pdt = (time.perf_counter() - t2) / 5
+    # the same prefill through the chunked forward, which is what a prefill belongs to: token-major q/k/v are strided
+    # views, the V-first pool rows are transposed into the chunk kernel's [N,H,K,V] state and back (inside the timing)
+    from fla_hip import pipeline
+    pcu = [0] + torch.cumsum(plens, 0).tolist()
+    hm = lambda t: t.transpose(0, 1)[None]
+
+    def prefill_chunked():
+        h0 = pstate.transpose(-1, -2).contiguous()
+        o, fin = pipeline.flash_gated_delta_rule(hm(pq), hm(pk), hm(pv), pgate[None], pbeta[None].float(), D ** -0.5, h0, True,
+                                                 cu_seqlens=pcu)
+        return o, fin.transpose(-1, -2).contiguous()
+
+    prefill_chunked()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(5):
+        prefill_chunked()
+    torch.cuda.synchronize()
+    cdt2 = (time.perf_counter() - t2) / 5
     # the KDA twin of the decode step (per-channel gate, same state tile), V-first fp32 pool in place
     kg = F.logsigmoid(torch.randn(N, 1, H, D, device=dev, generator=g)) * 0.3
     kcu = torch.arange(N + 1, dtype=torch.int32, device=dev)
@@ -307,7 +326,8 @@ def bench_decode(args, torch, dev):
                      "traffic_source": measured_traffic("recurrent_gdn")[1],
                      "avg_kernel_ms": round(ms / n, 4)},
         "varlen_prefill": {"sequences": 64, "tokens": PT, "ms": round(pdt * 1e3, 3),
-                           "tokens_per_s": round(PT / pdt, 1)},
+                           "tokens_per_s": round(PT / pdt, 1),
+                           "through_chunk_forward": {"ms": round(cdt2 * 1e3, 3), "tokens_per_s": round(PT / cdt2, 1)}},
         "kda_decode": kda_decode,
         "cpu_baseline": cpu,
     }

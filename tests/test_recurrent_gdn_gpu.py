@@ -191,6 +191,14 @@ def test_varlen_prefill_benchmark_shape(dev):
             ssm_state_indices=torch.zeros(e - s, dtype=torch.int32), g=c(gate))
         assert_close(o[s:e], o_ref, TOL_BF16, f"out of sequence {n} ({e - s} tokens)")
         assert_close(state[n:n + 1], s_ref, TOL_STATE, f"state of sequence {n}")
+    # (c) the chunked forward on the same packed tokens (strided head-major views, the pool rows transposed into its
+    # [N,H,K,V] state) agrees with the token-by-token kernel on every sequence
+    from fla_hip import pipeline
+    hm = lambda t: t.transpose(0, 1)[None]
+    o_c, fin = pipeline.flash_gated_delta_rule(hm(q), hm(k), hm(v), gate[None], beta[None].float(), D ** -0.5,
+                                               state0.transpose(-1, -2).contiguous(), True, cu_seqlens=cu)
+    assert_close(o_c[0], o.float(), TOL_BF16, "chunked forward vs recurrent kernel, out")
+    assert_close(fin.transpose(-1, -2), state, 2 * TOL_STATE, "chunked forward vs recurrent kernel, state")
 
 
 def test_wrapper_errors(dev):
