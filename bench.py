@@ -476,6 +476,12 @@ def bench_kda(args, torch, dev):
     ach = flops[dominant] / (kern[dominant] * 1e-3) / 1e12
     fwd_flops = flops["kda_intra"] + flops["kda_scan"]
     step_tflops = fwd_flops / (ms_per_step * 1e-3) / 1e12
+    # The same step against the memory roofline, which is the nearer of the two for this operator: at 8 TB/s the bytes
+    # below take 7 times longer than the FLOPs above at the bf16 peak.  Inputs q, k, v, raw gate, beta; results o, gk,
+    # Aqk, Akk; and w, u, qg, kg once out of the intra-chunk kernel and once into the state scan, with Aqk read again.
+    io_bytes = th * (2 * K * 2 + V * 2 + K * 4 + 4) + th * (V * 2 + K * 4 + 2 * C * 2)
+    hop_bytes = 2 * th * (3 * K * 2 + V * 2) + th * C * 2
+    step_gbps = (io_bytes + hop_bytes) / (ms_per_step * 1e-3) / 1e9
 
     fwd_bwd = None
     if C == 64:   # the backward operators work on 64-token chunks
@@ -534,8 +540,10 @@ def bench_kda(args, torch, dev):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "preheat_ms": heated, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"KDA chunk forward B=2 T=8192 H=32 K=V=128 chunk={C} BSND, fp32 initial+final state"},
-        "algorithmic": {"flops_per_step": fwd_flops},
+        "algorithmic": {"flops_per_step": fwd_flops, "bytes_per_step_results_and_inputs": io_bytes,
+                        "bytes_per_step_between_the_two_kernels": hop_bytes},
         "step_tflops": round(step_tflops, 2), "step_frac_of_bf16_peak": round(step_tflops / PEAK_BF16_TFLOPS, 4),
+        "step_GBps": round(step_gbps, 1), "step_frac_of_hbm_peak": round(step_gbps / PEAK_HBM_GBS, 4),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "avg_kernel_ms": round(kern[dominant], 4)},
@@ -736,7 +744,7 @@ def main():
         for name, sub in (("decode", bench_decode), ("conv1d", bench_conv1d), ("kda", bench_kda)):
             r = sub(brief, torch, dev)
             keep = ("metric", "value", "unit", "steps", "ms_per_step", "dtype", "config", "algorithmic", "step_tflops",
-                    "roofline", "cpu_baseline", "fwd_bwd", "varlen_prefill", "eager_ms_per_step")
+                    "step_GBps", "step_frac_of_hbm_peak", "roofline", "cpu_baseline", "fwd_bwd", "varlen_prefill", "eager_ms_per_step")
             secondary[name] = {k_: r[k_] for k_ in keep if k_ in r}
             secondary[name]["ms"] = r["ms_per_step"]
             secondary[name]["frac"] = r["roofline"]["frac"]
