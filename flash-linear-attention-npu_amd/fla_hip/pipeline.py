@@ -335,23 +335,53 @@ def _kda_autograd_function():
     return ChunkKdaFunction
 
 
+def _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound):
+    """The in-kernel gate of chunk_kda_fwd (fla/ops/ascendc/kda/chunk_kda_fwd/docs/api.md:103-113) as differentiable
+    tensor operations: -exp(A_log) * softplus(g + dt_bias), or lower_bound * sigmoid(exp(A_log) * (g + dt_bias)) with
+    ``safe_gate``; A_log [HV] and dt_bias [HV*K] broadcast along the head axis of ``layout``."""
+    import torch
+
+    HV, K = A_log.shape[0], g.shape[-1]
+    head_axis = {"BSND": 2, "BNSD": 1, "TND": 1, "NTD": 0}[layout]
+    shape = [1] * g.dim()
+    shape[head_axis] = HV
+    eig = torch.exp(A_log.float()).view(shape)
+    raw = g.float()
+    if dt_bias is not None:
+        shape[-1] = K
+        raw = raw + dt_bias.float().view(HV, K).view(shape)
+    if safe_gate:
+        return float(lower_bound) * torch.sigmoid(eig * raw)
+    return -eig * torch.nn.functional.softplus(raw)
+
+
 def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=None, output_final_state: bool = False,
-              cu_seqlens=None, *, layout: str = "BSND", chunk_size: int = 64):
+              cu_seqlens=None, *, layout: str = "BSND", chunk_size: int = 64, use_gate_in_kernel: bool = False,
+              A_log=None, dt_bias=None, safe_gate: bool = False, lower_bound: Optional[float] = None):
     """KDA chunk attention, differentiable: ``(o, final_state)`` with q, k [..H,K], v [..HV,V], per-channel log decay
     g [..HV,K] (natural log, one value per token and channel), beta [..HV] in ``layout``; states fp32 [N,HV,K,V].
     The forward is ``chunk_kda_fwd``; when an input requires grad the forward keeps its intermediates and
-    ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0."""
+    ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0.  With ``use_gate_in_kernel`` g is the raw gate input: without
+    gradients the forward kernel activates it; with gradients the activation runs as tensor operations ahead of the
+    kernels, so that autograd also reaches ``A_log`` and ``dt_bias``."""
     import torch
 
     if scale is None:
         scale = q.shape[-1] ** -0.5
     cu = _cu_list(cu_seqlens)
-    if not needs_grad_hint(q, k, v, g, beta, initial_state):
+    lower_bound = -5.0 if lower_bound is None else float(lower_bound)
+    if not needs_grad_hint(q, k, v, g, beta, initial_state, A_log, dt_bias):
         out = _ops.chunk_kda_fwd(q, k, v, g, beta, float(scale), chunk_size, layout=layout, initial_state=initial_state,
-                                 output_final_state=output_final_state, cu_seqlens=cu)
+                                 output_final_state=output_final_state, cu_seqlens=cu,
+                                 use_gate_in_kernel=use_gate_in_kernel, A_log=A_log, dt_bias=dt_bias, safe_gate=safe_gate,
+                                 lower_bound=lower_bound)
         return out[0], out[1]
     if chunk_size != 64:
         raise NotImplementedError("chunk_kda: gradients are built for chunk_size 64.")
+    if use_gate_in_kernel:
+        if A_log is None:
+            raise RuntimeError("chunk_kda: A_log must be float32 [HV] when use_gate_in_kernel=True.")
+        g = _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound)
     global _KDA_FUNCTION
     if _KDA_FUNCTION is None:
         _KDA_FUNCTION = _kda_autograd_function()
