@@ -385,4 +385,20 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     global _KDA_FUNCTION
     if _KDA_FUNCTION is None:
         _KDA_FUNCTION = _kda_autograd_function()
+    # The backward kernels are built for (K, V) in {(64,64), (64,128), (128,128)}.  Other admitted head sizes up to
+    # 128 x 128 run on the next built one with zero channels appended (a zero q/k channel adds nothing to any product, a
+    # zero v column yields zero columns of o and of the state); the padding is itself differentiable, so autograd
+    # returns the gradients of the unpadded tensors.
+    K, V = q.shape[-1], v.shape[-1]
+    Kp = 64 if K <= 64 and V <= 128 else 128
+    Vp = Kp if V <= Kp else 2 * Kp
+    if K > 128 or (Kp, Vp) == (128, 256):
+        raise NotImplementedError(f"chunk_kda: gradients are built for K <= 128 with V <= 128 (K <= 64: V <= 128), got K={K} V={V}.")
+    if (Kp, Vp) != (K, V):
+        F = torch.nn.functional
+        h0 = None if initial_state is None else F.pad(initial_state, (0, Vp - V, 0, Kp - K))
+        o, final = _KDA_FUNCTION.apply(F.pad(q, (0, Kp - K)), F.pad(k, (0, Kp - K)), F.pad(v, (0, Vp - V)),
+                                       F.pad(g, (0, Kp - K)), beta, float(scale), h0, output_final_state, cu, layout,
+                                       chunk_size)
+        return o[..., :V], (None if final is None else final[..., :K, :V])
     return _KDA_FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, layout, chunk_size)

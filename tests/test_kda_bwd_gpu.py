@@ -174,6 +174,9 @@ COMPOSITION_CASES = [
     dict(B=2, T=100, Hk=2, Hv=2, K=64, V=128, layout="BSND", dht=True),
     dict(B=1, T=128, Hk=1, Hv=1, K=128, V=128, layout="BSND", gate_scale=2.0, h0=True),       # strong decay
     dict(B=1, T=150, Hk=2, Hv=2, K=128, V=128, layout="BSND", dtype=torch.float16, h0=True, dht=True),
+    # head sizes between the built ones: zero channels appended around the kernels
+    dict(B=1, T=100, Hk=1, Hv=2, K=96, V=80, layout="BSND", h0=True, dht=True),
+    dict(B=1, T=130, Hk=1, Hv=1, K=32, V=112, layout="TND", cu=[0, 65, 130], h0=True, dht=True),
 ]
 
 
