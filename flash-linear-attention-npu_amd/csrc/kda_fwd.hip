@@ -105,7 +105,7 @@ template <int K, int V> struct IntraSmem {
 // diagonal block inverse and the off-diagonal solve of column block W) and later row tile W of w; wave W of role 1
 // owns row tile 3 - W of q k^T and later row tile W of u.  The two waves of a SIMD (W and 4 + W) together carry five
 // score tile products, as every other SIMD does.  W and ROLE are static so that the tile loops unroll.
-template <int K, int V, int W, int ROLE>
+template <int K, int V, int W, int ROLE, bool C128>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
                                            int64_t dec_base, int half) {
@@ -240,7 +240,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             *reinterpret_cast<elemx8 *>(p.qg + (row_base + r) * K + c8) = qg8;
             *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
         }
-        if (p.c128) {   // operands of the block that couples the two halves, both factors <= 1
+        if constexpr (C128) {   // operands of the block that couples the two halves, both factors <= 1
             f32x4 x1lo, x1hi, x2lo, x2hi;
             const f32x4 g0 = lds4(gS + r * pg + c8), g1 = lds4(gS + r * pg + c8 + 4);
             const f32x4 a0 = lds4(gS + (kChunk + 1) * pg + c8), a1 = lds4(gS + (kChunk + 1) * pg + c8 + 4);
@@ -284,7 +284,9 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     __syncthreads();
 }
 
-template <int K, int V>
+// C128: the workgroup owns one half of a 128-token chunk (a template flag, so that the 64-token form carries none of
+// the second gate stream, the coupling operands or the zero fill).
+template <int K, int V, bool C128>
 __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntraParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
@@ -299,13 +301,13 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     float *bS = aS + kChunk * pa;
     float *tS = bS + kChunk;
 
-    const int half = p.c128 ? (blockIdx.x & 1) : 0;
-    const int c = p.c128 ? blockIdx.x >> 1 : blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int half = C128 ? (blockIdx.x & 1) : 0;
+    const int c = C128 ? blockIdx.x >> 1 : blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     int ostart = start, olen = 0;   // the other half of a 128-token chunk: its gates enter this half's sums
-    if (p.c128) {
+    if constexpr (C128) {
         const int whole = len;
         olen = min(kChunk, max(0, whole - kChunk * (1 - half)));
         if (olen > 0) ostart = start + kChunk * (1 - half);
@@ -337,7 +339,7 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
 #pragma unroll
             for (int j = 0; j < TS; ++j)
                 raw[j] = (float)static_cast<const elem *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
-            if (p.c128)
+            if constexpr (C128)
 #pragma unroll
                 for (int j = 0; j < TS; ++j)
                     oraw[j] = (float)static_cast<const elem *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
@@ -345,7 +347,7 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
 #pragma unroll
             for (int j = 0; j < TS; ++j)
                 raw[j] = static_cast<const float *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
-            if (p.c128)
+            if constexpr (C128)
 #pragma unroll
                 for (int j = 0; j < TS; ++j)
                     oraw[j] = static_cast<const float *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
@@ -395,7 +397,7 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
         }
         tS[sg * K + ch] = acc;
         float oacc = 0.f;
-        if (p.c128) {
+        if constexpr (C128) {
 #pragma unroll
             for (int j = 0; j < TS; ++j)
                 if (sg * TS + j < olen)
@@ -426,14 +428,14 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
 
     const int64_t dec_base = half ? -1 : (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 1: intra_wave<K, V, 1, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 2: intra_wave<K, V, 2, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 3: intra_wave<K, V, 3, 0>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 4: intra_wave<K, V, 0, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 5: intra_wave<K, V, 1, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 6: intra_wave<K, V, 2, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        default: intra_wave<K, V, 3, 1>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
     }
 
     store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
@@ -441,7 +443,7 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     const int C = p.geom.C;
     store_tile<kIntraThreads>(p.aqk + row_base * C + kChunk * half, C, aqS, pb, kChunk, len);
     store_tile<kIntraThreads>(p.akk + row_base * C + kChunk * half, C, akS, pb, kChunk, len);
-    if (p.c128 && half == 0) {   // nothing of the second half is visible to the first
+    if (C128 && half == 0) {   // nothing of the second half is visible to the first
         const elemx8 z = {};
         for (int idx = tid; idx < len * (kChunk / 8); idx += kIntraThreads) {
             const int64_t at = (row_base + idx / (kChunk / 8)) * C + kChunk + (idx % (kChunk / 8)) * 8;
@@ -913,14 +915,21 @@ int head_major(const char *op, const char *name, const fla_tensor *t, bool rank3
 inline bool present(const fla_tensor *t) { return t != nullptr && t->data != nullptr; }
 inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
-template <int K, int V>
-int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
+template <int K, int V, bool C128>
+int launch_intra_kernel(const KdaIntraParams &p, hipStream_t stream) {
     const size_t smem = IntraSmem<K, V>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V, C128>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V>), dim3(p.geom.NT * (p.c128 ? 2 : 1), p.geom.Hv, p.geom.B),
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V, C128>), dim3(p.geom.NT * (C128 ? 2 : 1), p.geom.Hv, p.geom.B),
                dim3(kIntraThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
+template <int K, int V>
+int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
+    const int rc = p.c128 ? launch_intra_kernel<K, V, true>(p, stream) : launch_intra_kernel<K, V, false>(p, stream);
+    if (rc) return rc;
     if (p.c128) {
         KdaCrossParams cp{p.geom, p.x1, p.x2, p.w, p.u, p.aqk, p.akk, p.scale};
         const size_t csmem = CrossSmem<K, V>::bytes;
