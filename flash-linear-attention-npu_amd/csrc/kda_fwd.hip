@@ -332,26 +332,28 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     }
     float raw[TS], oraw[TS];
     {
-        const int64_t gbase = b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st + ch;
-        const int64_t obase = b * p.g_sb + hv * p.g_sh + (int64_t)ostart * p.g_st + ch;
+        // one buffer resource per gate stream (the workgroup's first token of the head), 32-bit offsets per lane:
+        // a clamped row index, one multiply and one add per load instead of 64-bit address arithmetic
+        const int esz = p.g_elem ? 2 : 4, gst = (int)p.g_st;
+        const char *gwg = static_cast<const char *>(p.g) + (b * p.g_sb + hv * p.g_sh) * esz;
+        const __amdgpu_buffer_rsrc_t rg = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(gwg + (int64_t)start * p.g_st * esz), 0, 0x7fffffff, 0x00020000);
+        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char *>(gwg + (int64_t)ostart * p.g_st * esz), 0, 0x7fffffff, 0x00020000);
         const int olast = max(olen, 1) - 1;
-        if (p.g_elem) {
+        auto gate_at = [&](const __amdgpu_buffer_rsrc_t &r, int row) -> float {
+            const int off = (row * gst + ch) * esz;
+            if (p.g_elem) {
+                const unsigned short h = __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+                return (float)__builtin_bit_cast(elem, h);
+            }
+            return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+        };
 #pragma unroll
-            for (int j = 0; j < TS; ++j)
-                raw[j] = (float)static_cast<const elem *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
-            if constexpr (C128)
+        for (int j = 0; j < TS; ++j) raw[j] = gate_at(rg, min(sg * TS + j, len - 1));
+        if constexpr (C128)
 #pragma unroll
-                for (int j = 0; j < TS; ++j)
-                    oraw[j] = (float)static_cast<const elem *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
-        } else {
-#pragma unroll
-            for (int j = 0; j < TS; ++j)
-                raw[j] = static_cast<const float *>(p.g)[gbase + (int64_t)min(sg * TS + j, len - 1) * p.g_st];
-            if constexpr (C128)
-#pragma unroll
-                for (int j = 0; j < TS; ++j)
-                    oraw[j] = static_cast<const float *>(p.g)[obase + (int64_t)min(sg * TS + j, olast) * p.g_st];
-        }
+            for (int j = 0; j < TS; ++j) oraw[j] = gate_at(ro, min(sg * TS + j, olast));
     }
     {   // all loads of the chunk are issued before the first LDS write waits for one of them
         TileCopy<kIntraThreads, kChunk, K> tq, tk;
@@ -417,11 +419,13 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
             gS[kChunk * pg + ch] = own + other;                 // gate at the end of the chunk
             gS[(kChunk + 1) * pg + ch] = half ? other : own;    // gate at the end of the first half
         }
+        float *gkp = p.gk ? p.gk + row_base * K + ch : nullptr;
+#pragma unroll
         for (int j = 0; j < TS; ++j) {
             const int t = sg * TS + j;
             const float v = gS[t * pg + ch] + off;
             gS[t * pg + ch] = v;
-            if (p.gk && t < len) p.gk[(row_base + t) * K + ch] = v;
+            if (gkp != nullptr && t < len) gkp[t * K] = v;
         }
     }
     __syncthreads();
@@ -1003,6 +1007,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
         ip.g_sb = L.rank3() ? 0 : g->stride[L.ib];
         ip.g_sh = g->stride[L.ih];
         ip.g_st = g->stride[L.it];
+        FLA_REQUIRE(ip.g_st >= 0 && ip.g_st < ((int64_t)1 << 23), FLA_ERR_SHAPE, "%s: token stride of g too large.", op);
     }
     {
         if ((rc = check_tensor(beta, op, "beta", L.rank3() ? 2 : 3, bf | f32))) return rc;
