@@ -459,6 +459,7 @@ struct DhuParams {
     int64_t z_sn, z_sh;
     elem *dh0_ref;       // [B,Hv,NT,K,V] bf16 (value stored at each sequence's first chunk) or null
     float scale;
+    int sub;             // 64-token steps per chunk: 1, or 2 for 128-token chunks (scalar gate only)
 };
 
 template <int K> struct DhuSmem {
@@ -565,7 +566,14 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     char *v2g = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + vcol0);
     __syncthreads();
 
+    // With 128-token chunks a chunk takes two 64-token steps, the later tokens first.  Every token of the chunk sees the
+    // gradient that ENTERS the chunk (k . dh uses one 16-bit copy, refreshed and stored at the chunk's last step only) and
+    // the gate of the chunk's last token; the decay of the carried gradient is applied once, at that step, and the two
+    // steps' q^T do and w^T dv2 terms add up.
+    elemx8 hB[KS][CT];
+    float g_end = 0.f;
     for (int c = nchunks - 1; c >= 0; --c) {
+        const bool chunk_end = (c % p.sub) == p.sub - 1 || c == nchunks - 1;
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
         const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
         const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
@@ -577,13 +585,12 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         const int start = bos + c * kChunk;
         const int len = min(kChunk, eos - start);
 
-        elemx8 hB[KS][CT];
+        if (chunk_end) {   // dh of this chunk = the incoming gradient
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
+            for (int j = 0; j < KS; ++j)
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
-        {   // dh of this chunk = the incoming gradient
-            elem *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc;
+                for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
+            elem *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c / p.sub) * p.h_sc;
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -605,7 +612,8 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = mfma16x32(afrag, hB[j][ct], dv2[rt][ct]);
             }
-        const float g_last = GK ? 0.f : gS[len - 1];
+        if (chunk_end) g_end = GK ? 0.f : gS[len - 1];
+        const float g_last = g_end;
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
@@ -627,17 +635,19 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         }
 
         // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
+        if (chunk_end) {
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-            f32x4 dec;
-            if (GK) {
-                dec = *reinterpret_cast<const f32x4 *>(gS + 16 * kt + 4 * lg);
-            } else {
-                const float d = __expf(g_last);
-                dec = f32x4{d, d, d, d};
+            for (int kt = 0; kt < KT; ++kt) {
+                f32x4 dec;
+                if (GK) {
+                    dec = *reinterpret_cast<const f32x4 *>(gS + 16 * kt + 4 * lg);
+                } else {
+                    const float d = __expf(g_last);
+                    dec = f32x4{d, d, d, d};
+                }
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) dacc[kt][ct] *= dec;
             }
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) dacc[kt][ct] *= dec;
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -707,7 +717,8 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     FLA_REQUIRE(!has_g || !use_exp2, FLA_ERR_UNSUPPORTED, "%s: the scalar gate g is a natural-log gate (use_exp2=false).", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
+    FLA_REQUIRE(geom.C == kChunk || !has_gk, FLA_ERR_UNSUPPORTED, "%s: gK is built for chunk_size 64.", op);
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
@@ -723,7 +734,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
                     FLA_ERR_SHAPE, "%s: gK must be fp32 [B,Hv,T,K].", op);
     }
     Varlen vl;
-    if ((rc = build_varlen(vl, op, cu, ci, kChunk, geom.T))) return rc;
+    if ((rc = build_varlen(vl, op, cu, ci, geom.C, geom.T))) return rc;
     FLA_REQUIRE(!vl.enabled || geom.B == 1, FLA_ERR_SHAPE, "%s: batch must be 1 with cu_seqlens.", op);
     if (vl.enabled) {
         geom.NT = vl.NT;
@@ -801,6 +812,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
         p.z_sh = dh0->stride[1];
     }
     p.scale = (float)scale;
+    p.sub = geom.C / kChunk;
     const int slabs = geom.V / 64;
     if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, true>(p, slabs, stream) : launch_bwd_dhu<128, false>(p, slabs, stream);
     return has_gk ? launch_bwd_dhu<64, true>(p, slabs, stream) : launch_bwd_dhu<64, false>(p, slabs, stream);

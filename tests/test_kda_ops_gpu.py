@@ -86,24 +86,33 @@ DHU_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", DHU_CASES)
+# 128-token chunks (chunk_gated_delta_rule_bwd_dhu/README.md:101-104) with the scalar gate: full chunks, a last chunk with
+# only its first half, packed sequences of every remainder
+DHU_CASES_128 = [c for c in DHU_CASES if not c[7]] + [
+    (1, 421, 2, 2, 128, 128, [0, 1, 66, 66, 194, 300, 421], False, True),
+    (1, 192, 1, 2, 128, 128, None, False, True),
+]
+
+
+@pytest.mark.parametrize("case", [(c, 64) for c in DHU_CASES] + [(c, 128) for c in DHU_CASES_128],
+                         ids=lambda cc: f"T{cc[0][1]}-K{cc[0][4]}-V{cc[0][5]}-{'gK' if cc[0][7] else 'g'}-C{cc[1]}")
 def test_bwd_dhu(dev, case):
     from fla_hip import ops
-    B, T, Hk, Hv, K, V, cu, per_channel, with_dht = case
+    (B, T, Hk, Hv, K, V, cu, per_channel, with_dht), C = case
     q, k, w, d_o, dv, gate = dhu_inputs(B, T, Hk, Hv, K, V, seed=T + V, per_channel=per_channel)
     scale = K ** -0.5
     # chunk-local cumulated gates, as the callers provide them
     if per_channel:
-        gcum = kda.kda_gate_cumsum(gate, 64, cu_seqlens=cu)        # log2 units
+        gcum = kda.kda_gate_cumsum(gate, C, cu_seqlens=cu)        # log2 units
         # q and k carry their gates in this variant (they stay O(1): 2^{gk} <= 1, 2^{gk_last - gk} <= 1)
         qg = (q.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(gcum)).to(BF)
         last = torch.zeros_like(gcum)
-        for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        for b, n, ci, s, e in gdn.chunk_spans(B, T, C, cu):
             last[b, :, s:e] = gcum[b, :, e - 1:e]
         kg = (k.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(last - gcum)).to(BF)
         q_in, k_in = qg, kg
     else:
-        gcum = gdn.chunk_local_cumsum(gate, 64, cu_seqlens=cu)
+        gcum = gdn.chunk_local_cumsum(gate, C, cu_seqlens=cu)
         q_in, k_in = q, k
     N = B if cu is None else len(cu) - 1
     gen = torch.Generator().manual_seed(3)
@@ -112,11 +121,11 @@ def test_bwd_dhu(dev, case):
 
     kw = dict(gK=gcum.to(dev), use_exp2=True) if per_channel else dict(g=gcum.to(dev))
     args = [t.to(dev) for t in (q_in, k_in, w, d_o, dv)]
-    dh, dh0, dv2 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, h0=h0.to(dev),
+    dh, dh0, dv2 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, C, h0=h0.to(dev),
                                                       dht=None if dht is None else dht.to(dev), cu_seqlens=cu,
                                                       dh0_per_sequence=True, **kw)
     okw = dict(gK=gcum) if per_channel else dict(g=gcum)
-    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(q_in, k_in, w, d_o, dv, scale, 64, dht=dht,
+    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(q_in, k_in, w, d_o, dv, scale, C, dht=dht,
                                                                   cu_seqlens=cu, **okw)
     assert dh.dtype == BF and dv2.dtype == BF and dh0.dtype == torch.float32
     assert_close(dv2, dv2_ref, TOL_BF16, "dv2")
@@ -124,18 +133,18 @@ def test_bwd_dhu(dev, case):
     assert_close(dh0, dh0_ref, TOL_BF16, "dh0")
 
     # reference-form dh0: bf16 buffer of dh's shape, written at the first chunk of each sequence
-    dh_b, dh0_b, dv2_b = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, h0=h0.to(dev),
+    dh_b, dh0_b, dv2_b = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, C, h0=h0.to(dev),
                                                             dht=None if dht is None else dht.to(dev), cu_seqlens=cu,
                                                             **kw)
     assert torch.equal(dh_b, dh) and torch.equal(dv2_b, dv2)
     assert dh0_b.shape == dh.shape and dh0_b.dtype == BF
     first = {}
-    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, C, cu):
         first.setdefault(n, (b, ci))
     for n, (b, ci) in first.items():
         assert torch.equal(dh0_b[b, :, ci].float(), dh0[n].to(BF).float())
     # without h0 no dh0 is produced
-    out3 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, 64, cu_seqlens=cu, **kw)
+    out3 = ops.chunk_gated_delta_rule_bwd_dhu(*args, scale, C, cu_seqlens=cu, **kw)
     assert out3[1] is None
 
 
