@@ -35,7 +35,10 @@ struct DvLocalParams {
     float scale;
 };
 
-template <int K, int V>
+// C128: 128-token chunks, one workgroup per 64-row half.  The first half also receives the block that couples it to the
+// second half (every column of it lies after every row, so it carries no mask); the gate is cumulated over the whole
+// chunk, so the factors e^{G_j - G_i} need no re-basing.
+template <int K, int V, bool C128>
 __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 8, pv = V + 16, pa = kChunk + 8;
@@ -43,54 +46,72 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
     elem *kS = qS + kChunk * pk;
     elem *oS = kS + kChunk * pk;
     elem *aS = oS + kChunk * pv;
-    float *gS = reinterpret_cast<float *>(aS + kChunk * pa);
+    float *gS = reinterpret_cast<float *>(aS + kChunk * pa);   // gates of the rows
+    float *cS = gS + kChunk;                                   // gates of the columns of the current tile
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int c = C128 ? blockIdx.x >> 1 : blockIdx.x, half = C128 ? blockIdx.x & 1 : 0;
+    const int hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
-    int seq, start, len;
-    chunk_span(p.geom, b, c, seq, start, len);
+    int seq, cstart, clen;
+    chunk_span(p.geom, b, c, seq, cstart, clen);
+    const int start = cstart + kChunk * half, len = min(kChunk, clen - kChunk * half);
+    if (len <= 0) return;
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
     {
-        TileCopy<kThreads, kChunk, K> tq, tk;
-        TileCopy<kThreads, kChunk, V> to;
-        tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+        TileCopy<kThreads, kChunk, K> tk;
         tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-        to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
         stage_scalars(gS, p.g, b, hv, start, len);
-        tq.commit(qS, pk, len, tid);
         tk.commit(kS, pk, len, tid);
-        to.commit(oS, pv, len, tid);
     }
-    __syncthreads();
-    // A[i][j] = <k_i, q_j> e^{G_j - G_i} scale for j >= i: row tile w, column tiles w..3
+    f32x4 dacc[V / 16];
 #pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
-        f32x4 acc = zero4();
-        if (ct >= w) {
-#pragma unroll
-            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(kS, pk, 16 * w, 32 * j), frag_kc(qS, pk, 16 * ct, 32 * j), acc);
-            const int col = 16 * ct + li;
-            const float gc = gS[col];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int row = 16 * w + 4 * lg + e;
-                const float f = __expf(fminf(gc - gS[row], 0.f)) * p.scale;
-                acc[e] = (col >= row && col < len) ? acc[e] * f : 0.f;
-            }
+    for (int ct = 0; ct < V / 16; ++ct) dacc[ct] = zero4();
+    for (int t = half; t < (C128 ? 2 : 1); ++t) {
+        const int tstart = cstart + kChunk * t, tlen = min(kChunk, clen - kChunk * t);
+        if (tlen <= 0) break;
+        const bool diag = t == half;
+        if (!diag) __syncthreads();   // the products of the diagonal tile are done with qS, oS, aS
+        {
+            TileCopy<kThreads, kChunk, K> tq;
+            TileCopy<kThreads, kChunk, V> to;
+            tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)tstart * p.q.st, p.q.st, tlen, tid);
+            to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)tstart * p.d_o.st, p.d_o.st, tlen, tid);
+            stage_scalars(cS, p.g, b, hv, tstart, tlen);
+            tq.commit(qS, pk, tlen, tid);
+            to.commit(oS, pv, tlen, tid);
         }
-        acc_to_tile(aS, pa, 16 * w, 16 * ct, acc);
+        __syncthreads();
+        // A[i][j] = <k_i, q_j> e^{G_j - G_i} scale for j >= i: row tile w, column tiles w..3 (all four off the diagonal)
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            f32x4 acc = zero4();
+            if (!diag || ct >= w) {
+#pragma unroll
+                for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(kS, pk, 16 * w, 32 * j), frag_kc(qS, pk, 16 * ct, 32 * j), acc);
+                const int col = 16 * ct + li;
+                const float gc = cS[col];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = 16 * w + 4 * lg + e;
+                    const float f = __expf(fminf(gc - gS[row], 0.f)) * p.scale;
+                    acc[e] = ((!diag || col >= row) && col < tlen) ? acc[e] * f : 0.f;
+                }
+            }
+            acc_to_tile(aS, pa, 16 * w, 16 * ct, acc);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ct = 0; ct < V / 16; ++ct) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (!diag || 32 * j + 31 >= 16 * w)
+                    dacc[ct] = mfma16x32(frag_kc(aS, pa, 16 * w, 32 * j), frag_tr(oS, pv, 16 * ct, 32 * j), dacc[ct]);
+        }
     }
-    __syncthreads();
     char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
                                          (int64_t)start * p.dv.st);
 #pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) {
-        f32x4 acc = zero4();
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            if (32 * j + 31 >= 16 * w) acc = mfma16x32(frag_kc(aS, pa, 16 * w, 32 * j), frag_tr(oS, pv, 16 * ct, 32 * j), acc);
-        acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
-    }
+    for (int ct = 0; ct < V / 16; ++ct) acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, dacc[ct]);
 }
 
 // =============================================================================
@@ -662,7 +683,7 @@ int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_
     (void)A;   // accepted and unused, as in the reference kernel
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, d_o, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, d_o, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // chunk_bwd_dv_local/README.md:114
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
@@ -674,13 +695,20 @@ int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     DvLocalParams p{geom, view4(q), view4(k), view4(d_o), view4(out), view3(g), (float)scale};
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const bool c128 = geom.C == 128;
+    const dim3 grid(geom.NT * (c128 ? 2 : 1), geom.Hv, geom.B);
     const int K = geom.K, V = geom.V;
-    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (V + 16) + kChunk + 8)) * 2 + kChunk * 4;
-    if (K == 128 && V == 128) FLA_BWD_DISPATCH((dv_local_kernel<128, 128>), "bwd_dv_local", grid, smem, p);
-    if (K == 64 && V == 64) FLA_BWD_DISPATCH((dv_local_kernel<64, 64>), "bwd_dv_local", grid, smem, p);
-    if (K == 64 && V == 128) FLA_BWD_DISPATCH((dv_local_kernel<64, 128>), "bwd_dv_local", grid, smem, p);
-    if (K == 128 && V == 256) FLA_BWD_DISPATCH((dv_local_kernel<128, 256>), "bwd_dv_local", grid, smem, p);
+    const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (V + 16) + kChunk + 8)) * 2 + 2 * kChunk * 4;
+#define FLA_DV_LOCAL(KK, VV)                                                                                \
+    do {                                                                                                    \
+        if (c128) FLA_BWD_DISPATCH((dv_local_kernel<KK, VV, true>), "bwd_dv_local", grid, smem, p);         \
+        FLA_BWD_DISPATCH((dv_local_kernel<KK, VV, false>), "bwd_dv_local", grid, smem, p);                  \
+    } while (0)
+    if (K == 128 && V == 128) FLA_DV_LOCAL(128, 128);
+    if (K == 64 && V == 64) FLA_DV_LOCAL(64, 64);
+    if (K == 64 && V == 128) FLA_DV_LOCAL(64, 128);
+    if (K == 128 && V == 256) FLA_DV_LOCAL(128, 256);
+#undef FLA_DV_LOCAL
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 

@@ -134,6 +134,32 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     assert_close(dg_acc, dg0 + two[3], 1e-6, "dg accumulated")
 
 
+CASES_128 = [
+    # B, T, Hv, Hk, K, V, cu_seqlens: full chunks, a last chunk with only its first half, every remainder when packed
+    (2, 256, 2, 2, 128, 128, None),
+    (1, 200, 4, 2, 128, 128, None),
+    (1, 192, 2, 1, 64, 128, None),
+    (1, 421, 2, 1, 128, 128, [0, 1, 66, 66, 194, 300, 421]),
+    (1, 330, 2, 2, 128, 256, None),
+    (1, 130, 2, 2, 64, 64, None),
+]
+
+
+@pytest.mark.parametrize("case", CASES_128)
+def test_dv_local_with_128_token_chunks(dev, case):
+    """chunk_bwd_dv_local on 128-token chunks (chunk_bwd_dv_local/README.md:114): the gate is cumulated over the whole
+    chunk and a row of the first half also sees the queries of the second."""
+    from fla_hip import ops
+    B, T, Hv, Hk, K, V, cu = case
+    d = make(B, T, Hv, Hk, K, V, cu, seed=T + V)
+    G = gdn.chunk_local_cumsum(d["g"], 128, cu_seqlens=cu)
+    scale = K ** -0.5
+    got = ops.chunk_bwd_dv_local(d["q"].to(dev), d["k"].to(dev), d["do"].to(dev), G.to(dev), scale, 128, cu_seqlens=cu)
+    ref = gdn_bwd.chunk_bwd_dv_local(d["q"], d["k"], d["do"], G, scale, 128, output_dtype=torch.float32, cu_seqlens=cu)
+    assert got.dtype == BF and got.shape == d["do"].shape
+    assert_close(got, ref, TOL_BF16, "dv_local, 128-token chunks")
+
+
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", [CASES[1], CASES[5], CASES[6]])
 def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
