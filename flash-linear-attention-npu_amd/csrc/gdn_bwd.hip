@@ -118,6 +118,7 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
 // chunk_bwd_dqkwg
 // =============================================================================
 constexpr int kDqkwgThreads = 512;   // two waves per SIMD over one set of LDS tiles
+constexpr int kMaxRep = 64;          // value heads per key head that the 128-token-chunk form can carry sums for
 struct DqkwgParams {
     ChunkGeom geom;
     View4 q, k, v, d_o, dv, dq, dk, dw;
@@ -131,8 +132,13 @@ struct DqkwgParams {
 
 // V is the width of the value slab held in LDS; VSLABS slabs cover the value dimension (1: V itself, 2: V = 256 as
 // two passes of 128 columns, every product over the value dimension accumulated across the passes).
-template <int K, int V, bool GVA, int VSLABS = 1>
+// CH = 2: 128-token chunks.  The workgroup takes the two 64-token halves of its chunk one after the other: both read
+// the chunk's one h / dh block and the gate cumulated over the whole chunk; a row of the second half also gets
+// ds_21 k_1 in dq, a row of the first half ds_21^T q_2 in dk (ds_21 = do_2 v_1^T e^{G_i - G_j} scale, unmasked), and
+// the sum that lands on the chunk's last token collects sum_t k_t . dk_state_t over both halves.
+template <int K, int V, bool GVA, int VSLABS = 1, int CH = 1>
 __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams p) {
+    static_assert(CH == 1 || VSLABS == 1, "128-token chunks are built for one value slab");
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
     constexpr int KT = K / 16, KTH = KT / 2;   // column tiles of q/k: all, and per wave
@@ -147,11 +153,19 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
     float *gS = reinterpret_cast<float *>(sS + kChunk * ps);
     float *red = gS + kChunk;          // 16 partial sums
     float *dgp = red + 16;             // [2][kChunk] row sums of the two column halves
+    float *goS = dgp + 2 * kChunk;     // gates of the other half (CH = 2)
+    float *ksS = goS + kChunk;         // [kMaxRep] sum_t k_t . dk_state_t of the first half, per value head (CH = 2)
 
     const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
     const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
-    int seq, start, len;
-    chunk_span(p.geom, b, c, seq, start, len);
+    int seq, cstart, clen;
+    chunk_span(p.geom, b, c, seq, cstart, clen);
+    for (int hh = 0; hh < CH; ++hh) {
+    const int start = cstart + kChunk * hh, len = min(kChunk, clen - kChunk * hh);
+    if (len <= 0) break;
+    const int ostart = cstart + kChunk * (1 - hh), olen = CH > 1 ? min(kChunk, clen - kChunk * (1 - hh)) : 0;
+    const bool last_half = kChunk * (hh + 1) >= clen;   // the chunk's last token is one of this half's rows
+    if (hh > 0) __syncthreads();
     // eight waves: wave (w, half) owns token rows 16w.. and column tiles half*KTH .. half*KTH+KTH-1 of q/k;
     // waves w and 4 + w share a SIMD
     const int tid = threadIdx.x, w = wave_id() & 3, half = wave_id() >> 2, l = lane_id(), li = l & 15, lg = l >> 4;
@@ -261,7 +275,7 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
             for (int ct = 0; ct < KTH; ++ct) acc_to_global(dwg + 32 * (half * KTH + ct), p.dw.st * 2, 16 * w, len, -dwacc[ct]);
         }
         // ---- products with the state gradient, gate factors, intra-chunk parts -------------------------
-        const float g_last = gS[len - 1];
+        const float g_last = CH > 1 ? load_scalar(p.g, b, hv, cstart + clen - 1) : gS[len - 1];
         float grow[4], eq[4], ek[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -301,6 +315,59 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
             dq_acc[ct] += dq;
             dk_acc[ct] += dk;
         }
+        if constexpr (CH > 1) {
+            if (olen > 0) {   // the block that couples the halves
+                __syncthreads();   // dv, dh and ds are no longer read: their tiles take the other half's operands
+                elem *xS = dvS;    // other half: v (hh = 1) or do (hh = 0)
+                elem *yS = hS;     // other half: k (hh = 1) or q (hh = 0); the state tile is K x pv elements
+                constexpr int py = K * pv >= kChunk * pk ? pk : K + 8;
+                static_assert(K * pv >= kChunk * py, "the other half's k/q tile must fit the state tile");
+                {
+                    TileCopy<kDqkwgThreads, kChunk, V> tx;
+                    TileCopy<kDqkwgThreads, kChunk, K> ty;
+                    const View4 &xv = hh ? p.v : p.d_o, &yv = hh ? p.k : p.q;
+                    tx.fetch(static_cast<const elem *>(xv.p) + b * xv.sb + hv * xv.sh + (int64_t)ostart * xv.st, xv.st, olen, tid);
+                    ty.fetch(static_cast<const elem *>(yv.p) + b * yv.sb + hk * yv.sh + (int64_t)ostart * yv.st, yv.st, olen, tid);
+                    stage_scalars(goS, p.g, b, hv, ostart, olen);
+                    tx.commit(xS, pv, olen, tid);
+                    ty.commit(yS, py, olen, tid);
+                }
+                __syncthreads();
+                const elem *rowS = hh ? oS : vS;   // own do (second half) or own v (first half)
+#pragma unroll
+                for (int cc = 0; cc < 2; ++cc) {
+                    const int ct = half + 2 * cc;
+                    f32x4 acc = zero4();
+#pragma unroll
+                    for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(rowS, pv, 16 * w, 32 * j), frag_kc(xS, pv, 16 * ct, 32 * j), acc);
+                    const int col = 16 * ct + li;
+                    const float go = goS[col];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = 16 * w + 4 * lg + e;
+                        const float d = hh ? gS[row] - go : go - gS[row];   // later token minus earlier token
+                        acc[e] = (row < len && col < olen) ? acc[e] * __expf(fminf(d, 0.f)) * p.scale : 0.f;
+                    }
+                    acc_to_tile(sS, ps, 16 * w, 16 * ct, acc);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int ct = 0; ct < KTH; ++ct) {
+                    const int cg = half * KTH + ct;
+                    f32x4 d = zero4();
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) d = mfma16x32(frag_kc(sS, ps, 16 * w, 32 * j), frag_tr(yS, py, 16 * cg, 32 * j), d);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = 16 * w + 4 * lg + e;
+                        const float own = (float)(hh ? qS : kS)[row * pk + 16 * cg + li];
+                        dg_row[e] += hh ? d[e] * own : -d[e] * own;
+                    }
+                    if (hh) dq_acc[ct] += d;
+                    else dk_acc[ct] += d;
+                }
+            }
+        }
         // block sums for the gradient that lands on the last token of the chunk
         float s1 = hd, s2 = kdk_state;
 #pragma unroll
@@ -325,9 +392,11 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
                 hs += red[i];
                 ks += red[8 + i];
             }
+            if (CH > 1 && hh > 0) ks += ksS[r];
             const float dg_last = hs * __expf(g_last) + ks;
             p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + tid) * p.dg_st] =
-                dgp[tid] + dgp[kChunk + tid] + (tid == len - 1 ? dg_last : 0.f);
+                dgp[tid] + dgp[kChunk + tid] + (last_half && tid == len - 1 ? dg_last : 0.f);
+            if (CH > 1 && hh == 0 && tid == 0) ksS[r] = ks;
         }
     }
     char *dqg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
@@ -337,6 +406,7 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
         acc_to_global(dqg + 32 * (half * KTH + ct), p.dq.st * 2, 16 * w, len, dq_acc[ct]);
         acc_to_global(dkg + 32 * (half * KTH + ct), p.dk.st * 2, 16 * w, len, dk_acc[ct]);
     }
+    }   // halves of the chunk
 }
 
 // =============================================================================
@@ -724,7 +794,7 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     (void)w;   // the reference accepts w and does not read it
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // chunk_bwd_dqkwg/README.md:117
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
@@ -750,8 +820,17 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
     const int VS = V == 256 ? 128 : V;   // value columns held in LDS at a time
-    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 + (kChunk + 16 + 2 * kChunk) * 4;
+    const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 +
+                        (kChunk + 16 + 2 * kChunk + kChunk + kMaxRep) * 4;
     const bool gva = geom.Hv != geom.Hk;
+    if (geom.C == 128) {   // one workgroup per chunk, its two halves in turn
+        FLA_REQUIRE(geom.Hv / geom.Hk <= kMaxRep, FLA_ERR_UNSUPPORTED, "%s: at most %d value heads per key head with chunk_size 128.", op, kMaxRep);
+        if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, false, 1, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 128 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true, 1, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 64 && V == 64) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 64, true, 1, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 64 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 128, true, 1, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel for chunk_size 128; built: (128,128),(64,64),(64,128).", op, K, V);
+    }
     if (K == 128 && V == 256) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
     if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, false>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
     if (K == 128 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);

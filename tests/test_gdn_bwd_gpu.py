@@ -27,7 +27,7 @@ CASES = [
 ]
 
 
-def make(B, T, Hv, Hk, K, V, cu, seed, dtype=BF):
+def make(B, T, Hv, Hk, K, V, cu, seed, dtype=BF, C=64):
     """Forward quantities of one problem, every tensor rounded to the dtype the operators exchange."""
     gen = torch.Generator().manual_seed(seed)
     rn = lambda *s: torch.randn(*s, generator=gen)
@@ -40,11 +40,11 @@ def make(B, T, Hv, Hk, K, V, cu, seed, dtype=BF):
     h0 = rn(N, Hv, K, V) * 0.1
     do = rn(B, Hv, T, V).to(dtype)
     dht = rn(N, Hv, K, V) * 0.1
-    G = gdn.chunk_local_cumsum(g, 64, cu_seqlens=cu)
-    A0 = gdn.chunk_scaled_dot_kkt(k, G, beta, 64, cu_seqlens=cu)
+    G = gdn.chunk_local_cumsum(g, C, cu_seqlens=cu)
+    A0 = gdn.chunk_scaled_dot_kkt(k, G, beta, C, cu_seqlens=cu)
     A = gdn.solve_tri(A0, cu_seqlens=cu, output_dtype=dtype)
-    w, u = gdn.recompute_w_u_fwd(k, v, beta, A, 64, g=G, cu_seqlens=cu, output_dtype=dtype)
-    h, v_new, _ = gdn.chunk_gated_delta_rule_fwd_h(k, w, u, G, initial_state=h0, chunk=64, cu_seqlens=cu, output_dtype=dtype)
+    w, u = gdn.recompute_w_u_fwd(k, v, beta, A, C, g=G, cu_seqlens=cu, output_dtype=dtype)
+    h, v_new, _ = gdn.chunk_gated_delta_rule_fwd_h(k, w, u, G, initial_state=h0, chunk=C, cu_seqlens=cu, output_dtype=dtype)
     return dict(q=q, k=k, v=v, beta=beta, g=g, G=G, A=A, w=w, u=u, h=h, v_new=v_new, h0=h0, do=do, dht=dht)
 
 
@@ -158,6 +158,32 @@ def test_dv_local_with_128_token_chunks(dev, case):
     ref = gdn_bwd.chunk_bwd_dv_local(d["q"], d["k"], d["do"], G, scale, 128, output_dtype=torch.float32, cu_seqlens=cu)
     assert got.dtype == BF and got.shape == d["do"].shape
     assert_close(got, ref, TOL_BF16, "dv_local, 128-token chunks")
+
+
+@pytest.mark.parametrize("case", [c for c in CASES_128 if c[5] <= 128])
+def test_backward_operators_with_128_token_chunks(dev, case):
+    """The operators that follow dv_local, each on 128-token operands (A [T,128], one h / dh block per 128 tokens, the
+    gate cumulated over the chunk) against the oracle on the same 16-bit inputs
+    (chunk_gated_delta_rule_bwd_dhu/README.md:101-104, chunk_bwd_dqkwg/README.md:117)."""
+    from fla_hip import ops
+    B, T, Hv, Hk, K, V, cu = case
+    C, scale = 128, K ** -0.5
+    d = make(B, T, Hv, Hk, K, V, cu, seed=T + K, C=C)
+    x = to_dev(d, dev)
+    kw = dict(cu_seqlens=cu)
+    dv_l = gdn_bwd.chunk_bwd_dv_local(d["q"], d["k"], d["do"], d["G"], scale, C, output_dtype=torch.float32, **kw).to(BF)
+    dh_ref, _, dv2_ref = dhu_oracle(d["q"], d["k"], d["w"], d["do"], dv_l, scale, C, g=d["G"], dht=d["dht"], **kw)
+    dh, dv2 = dh_ref.to(BF), dv2_ref.to(BF)
+
+    dq, dk, dw, dg = ops.chunk_bwd_dqkwg(x["q"], x["k"], x["v_new"], x["G"], x["h"], x["do"], dh.to(dev), dv2.to(dev), C,
+                                         scale=scale, **kw)
+    dq_r, dk_r, dw_r, dg_r = gdn_bwd.chunk_bwd_dqkwg(d["q"], d["k"], d["v_new"], d["G"], d["h"], d["do"], dh, dv2, scale, C,
+                                                     output_dtype=torch.float32, **kw)
+    assert_close(dq, dq_r, TOL_BF16, "dq, 128-token chunks")
+    assert_close(dk, dk_r, TOL_BF16, "dk, 128-token chunks")
+    assert_close(dw, dw_r, TOL_BF16, "dw, 128-token chunks")
+    st = err_stats(dg, dg_r)
+    assert st["rel_max"] <= TOL_BF16, f"dg: {st}"
 
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
