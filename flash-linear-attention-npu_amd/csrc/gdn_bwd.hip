@@ -57,25 +57,34 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
     const int start = cstart + kChunk * half, len = min(kChunk, clen - kChunk * half);
     if (len <= 0) return;
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
-    {
-        TileCopy<kThreads, kChunk, K> tk;
+    const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
+    const elem *og = static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh;
+    {   // the rows' k and gates together with the diagonal tile's q and do: one round trip to memory
+        TileCopy<kThreads, kChunk, K> tk, tq;
+        TileCopy<kThreads, kChunk, V> to;
         tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
-        stage_scalars(gS, p.g, b, hv, start, len);
+        tq.fetch(qg + (int64_t)start * p.q.st, p.q.st, len, tid);
+        to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        if (tid < kChunk) gS[tid] = cS[tid] = load_scalar(p.g, b, hv, start + min(tid, len - 1));
         tk.commit(kS, pk, len, tid);
+        tq.commit(qS, pk, len, tid);
+        to.commit(oS, pv, len, tid);
     }
-    f32x4 dacc[V / 16];
+    char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                         (int64_t)start * p.dv.st);
+    f32x4 dacc[C128 ? V / 16 : 1];
 #pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) dacc[ct] = zero4();
+    for (int ct = 0; ct < (C128 ? V / 16 : 1); ++ct) dacc[ct] = zero4();
     for (int t = half; t < (C128 ? 2 : 1); ++t) {
         const int tstart = cstart + kChunk * t, tlen = min(kChunk, clen - kChunk * t);
         if (tlen <= 0) break;
         const bool diag = t == half;
-        if (!diag) __syncthreads();   // the products of the diagonal tile are done with qS, oS, aS
-        {
+        if (!diag) {
+            __syncthreads();   // the products of the diagonal tile are done with qS, oS, aS
             TileCopy<kThreads, kChunk, K> tq;
             TileCopy<kThreads, kChunk, V> to;
-            tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)tstart * p.q.st, p.q.st, tlen, tid);
-            to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)tstart * p.d_o.st, p.d_o.st, tlen, tid);
+            tq.fetch(qg + (int64_t)tstart * p.q.st, p.q.st, tlen, tid);
+            to.fetch(og + (int64_t)tstart * p.d_o.st, p.d_o.st, tlen, tid);
             stage_scalars(cS, p.g, b, hv, tstart, tlen);
             tq.commit(qS, pk, tlen, tid);
             to.commit(oS, pv, tlen, tid);
@@ -102,16 +111,19 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
         __syncthreads();
 #pragma unroll
         for (int ct = 0; ct < V / 16; ++ct) {
+            f32x4 acc = C128 ? dacc[ct] : zero4();
 #pragma unroll
             for (int j = 0; j < 2; ++j)
                 if (!diag || 32 * j + 31 >= 16 * w)
-                    dacc[ct] = mfma16x32(frag_kc(aS, pa, 16 * w, 32 * j), frag_tr(oS, pv, 16 * ct, 32 * j), dacc[ct]);
+                    acc = mfma16x32(frag_kc(aS, pa, 16 * w, 32 * j), frag_tr(oS, pv, 16 * ct, 32 * j), acc);
+            if constexpr (C128) dacc[ct] = acc;
+            else acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);   // one tile: each store leaves under the next product
         }
     }
-    char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
-                                         (int64_t)start * p.dv.st);
+    if constexpr (C128) {
 #pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, dacc[ct]);
+        for (int ct = 0; ct < V / 16; ++ct) acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, dacc[ct]);
+    }
 }
 
 // =============================================================================
@@ -714,6 +726,264 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     }
 }
 
+// =============================================================================
+// 128-token chunks in the two WY backward operators (prepare_wy_repr_bwd_full/README.md:74,101).  A and dA are
+// 128 x 128 per chunk.  One workgroup per chunk; the products are the ones of the 64-token kernels with the
+// contraction over 128 tokens, the operand tiles staged in 64-row pieces so that everything fits one CU's LDS.
+// =============================================================================
+// rows [0, valid) of a row-major source into an LDS tile of `nrows` rows, the rest zero; with `scale` every row r is
+// multiplied by scale[r]; with `colf` every column c by colf[c]; columns >= `vcols` are zeroed.
+template <int NCOLS>
+__device__ __forceinline__ void stage_rows(elem *tile, int pitch, const elem *src, int64_t stride, int nrows, int valid,
+                                           const float *scale, const float *colf = nullptr, int vcols = NCOLS) {
+    constexpr int CPR = NCOLS / 8;
+    for (int idx = threadIdx.x; idx < nrows * CPR; idx += kThreads) {
+        const int r = idx / CPR, c8 = (idx % CPR) << 3;
+        elemx8 a = {};
+        if (r < valid) {
+            a = *reinterpret_cast<const elemx8 *>(src + (int64_t)r * stride + c8);
+            if (scale != nullptr || colf != nullptr || vcols < NCOLS) {
+                const float sr = scale ? scale[r] : 1.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = c8 + e < vcols ? sr * (colf ? colf[c8 + e] : 1.f) : 0.f;
+                    a[e] = (elem)((float)a[e] * f);
+                }
+            }
+        }
+        *reinterpret_cast<elemx8 *>(tile + r * pitch + c8) = a;
+    }
+}
+
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) wy_bwd_da128_kernel(const WyBwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int C = 128, pk = K + 8, pv = V + 8, pa = C + 8;
+    elem *dwS = reinterpret_cast<elem *>(smem);      // 64 rows each: dw, k beta e^G, du, v beta of the block at hand
+    elem *kS = dwS + kChunk * pk;
+    elem *duS = kS + kChunk * pk;
+    elem *vS = duS + kChunk * pv;
+    elem *m4S = vS + kChunk * pv;                    // [128][pa]
+    elem *aS = m4S + C * pa;                         // [128][pa]
+    elem *m5S = dwS;                                 // [128][pa] over the operand tiles, dead by then
+    static_assert((size_t)kChunk * (2 * pk + 2 * pv) >= (size_t)C * pa, "M5 must fit the operand tiles");
+    float *gS = reinterpret_cast<float *>(aS + C * pa);
+    float *bS = gS + C;
+    float *fS = bS + C;                              // beta e^G
+
+    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    if (tid < C) {
+        const int t = start + min(tid, len - 1);
+        const float gg = load_scalar(p.g, b, hv, t), bb = load_scalar(p.beta, b, hv, t);
+        gS[tid] = gg;
+        bS[tid] = bb;
+        fS[tid] = bb * __expf(gg);
+    }
+    stage_rows<C>(aS, pa, static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, C, len,
+                  nullptr, nullptr, len);
+    __syncthreads();
+    const elem *dwg = static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st;
+    const elem *dug = static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
+    const elem *vg = static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st;
+    // M4 = strict_lower(dw (k beta e^G)^T + du (v beta)^T) in 64 x 64 blocks (0,0), (1,0), (1,1); block (0,1) is zero
+    for (int blk = 0; blk < 3; ++blk) {
+        const int rh = blk > 0, ch = blk > 1;
+        if (blk > 0) __syncthreads();   // the previous block's products are done with the tiles that change
+        if (blk != 2) {
+            const int rv = max(0, min(kChunk, len - kChunk * rh));
+            stage_rows<K>(dwS, pk, dwg + (int64_t)kChunk * rh * p.dw.st, p.dw.st, kChunk, rv, nullptr);
+            stage_rows<V>(duS, pv, dug + (int64_t)kChunk * rh * p.du.st, p.du.st, kChunk, rv, nullptr);
+        }
+        if (blk != 1) {
+            const int cv = max(0, min(kChunk, len - kChunk * ch));
+            stage_rows<K>(kS, pk, kg + (int64_t)kChunk * ch * p.k.st, p.k.st, kChunk, cv, fS + kChunk * ch);
+            stage_rows<V>(vS, pv, vg + (int64_t)kChunk * ch * p.v.st, p.v.st, kChunk, cv, bS + kChunk * ch);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            f32x4 acc = zero4();
+            if (rh != ch || ct <= w) {
+#pragma unroll
+                for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pk, 16 * w, 32 * j), frag_kc(kS, pk, 16 * ct, 32 * j), acc);
+#pragma unroll
+                for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(duS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+                const int col = kChunk * ch + 16 * ct + li;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = kChunk * rh + 16 * w + 4 * lg + e;
+                    acc[e] = (col < row && row < len) ? acc[e] : 0.f;
+                }
+            }
+            acc_to_tile(m4S, pa, kChunk * rh + 16 * w, kChunk * ch + 16 * ct, acc);
+            if (blk == 0) acc_to_tile(m4S, pa, 16 * w, kChunk + 16 * ct, zero4());
+        }
+    }
+    __syncthreads();
+    // M5 = M4 A^T: wave w owns row tiles w and w + 4
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+        const int rt = w + 4 * rr;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+            f32x4 acc = zero4();
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc = mfma16x32(frag_kc(m4S, pa, 16 * rt, 32 * j), frag_kc(aS, pa, 16 * ct, 32 * j), acc);
+            acc_to_tile(m5S, pa, 16 * rt, 16 * ct, acc);
+        }
+    }
+    __syncthreads();
+    // (A^T M5)^T = M5^T A, gated, negated and masked; rows of this product are the stored rows
+    char *dag = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dA.p)) + b * p.dA.sb + hv * p.dA.sh +
+                                         (int64_t)start * p.dA.st);
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+        const int rt = w + 4 * rr;
+#pragma unroll
+        for (int ct = 0; ct < 8; ++ct) {
+            f32x4 acc = zero4();
+            if (ct >= rt) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc = mfma16x32(frag_tr(m5S, pa, 16 * rt, 32 * j), frag_tr(aS, pa, 16 * ct, 32 * j), acc);
+                const int col = 16 * ct + li;
+                const float gc = gS[col];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int row = 16 * rt + 4 * lg + e;
+                    acc[e] = (col > row && col < len) ? -acc[e] * __expf(fminf(gc - gS[row], 0.f)) : 0.f;
+                }
+            }
+            acc_to_global(dag + 32 * ct, p.dA.st * 2, 16 * rt, len, acc);
+        }
+    }
+}
+
+// prepare_wy_repr_bwd_full on 128-token chunks: one workgroup per chunk and key head.  The 64 output rows of a half
+// are produced in one pass: A^T and dA^T need the 64-column slab of A and dA that belongs to those rows (all 128 token
+// rows of it), dA (k beta) the 64-row slab of dA; k of the whole chunk stays in LDS, du and dw take turns in one tile.
+template <int K, int V>
+__global__ void __launch_bounds__(kThreads) wy_bwd_full128_kernel(const WyBwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int C = 128, KV = K > V ? K : V;
+    constexpr int pk = K + 16, px = KV + 16, pc = kChunk + 8, pa = C + 8, pvv = V;
+    constexpr int KT = K / 16, VT = V / 16;
+    elem *kS = reinterpret_cast<elem *>(smem);   // [128][pk]
+    elem *xS = kS + C * pk;                      // [128][px] du, then dw
+    elem *aS = xS + C * px;                      // [128][pc] columns of A for this half's rows
+    elem *dS = aS + C * pc;                      // [128][pc] the same columns of dA as stored
+    elem *dbS = dS + C * pc;                     // [64][pa] this half's rows of dA, column j scaled by beta_j
+    elem *vS = dbS + kChunk * pa;                // [64][V]
+    float *gS = reinterpret_cast<float *>(vS + kChunk * pvv);
+    float *bS = gS + C;
+
+    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int rep = p.geom.Hv / p.geom.Hk;
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
+    stage_rows<K>(kS, pk, static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, C, len, nullptr);
+
+    for (int hh = 0; hh < 2; ++hh) {
+        const int rlen = min(kChunk, len - kChunk * hh);   // rows of this half
+        if (rlen <= 0) break;
+        const int rstart = start + kChunk * hh, vcols = rlen;
+        f32x4 dk_acc[KT];
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct) dk_acc[ct] = zero4();
+        for (int r = 0; r < rep; ++r) {
+            const int hv = hk * rep + r;
+            __syncthreads();   // the previous pass is done with every tile
+            if (tid < C) {
+                const int t = start + min(tid, len - 1);
+                gS[tid] = load_scalar(p.g, b, hv, t);
+                bS[tid] = load_scalar(p.beta, b, hv, t);
+            }
+            __syncthreads();
+            const elem *Ag = static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st;
+            const elem *dAg = static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st;
+            stage_rows<kChunk>(aS, pc, Ag + kChunk * hh, p.A.st, C, len, nullptr, nullptr, vcols);
+            stage_rows<kChunk>(dS, pc, dAg + kChunk * hh, p.dA.st, C, len, nullptr, nullptr, vcols);
+            stage_rows<C>(dbS, pa, dAg + (int64_t)kChunk * hh * p.dA.st, p.dA.st, kChunk, rlen, nullptr, bS, len);
+            stage_rows<V>(vS, pvv, static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)rstart * p.v.st, p.v.st,
+                          kChunk, rlen, nullptr);
+            stage_rows<V>(xS, px, static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st,
+                          C, len, nullptr);
+            __syncthreads();
+            float br[4], er[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                br[e] = bS[kChunk * hh + 16 * w + 4 * lg + e];
+                er[e] = __expf(gS[kChunk * hh + 16 * w + 4 * lg + e]);
+            }
+            float db_row[4] = {0.f, 0.f, 0.f, 0.f}, dg_row[4] = {0.f, 0.f, 0.f, 0.f};
+            elemx8 at[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) at[j] = frag_tr(aS, pc, 16 * w, 32 * j);
+            char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                                 (int64_t)rstart * p.dv.st);
+#pragma unroll
+            for (int ct = 0; ct < VT; ++ct) {      // A^T du
+                f32x4 acc = zero4();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc = mfma16x32(at[j], frag_tr(xS, px, 16 * ct, 32 * j), acc);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pvv + 16 * ct + li];
+                    acc[e] *= br[e];
+                }
+                acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, rlen, acc);
+            }
+            __syncthreads();                 // du has been consumed by every wave
+            stage_rows<K>(xS, px, static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st,
+                          C, len, nullptr);
+            __syncthreads();
+            elemx8 dt[4], db[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                dt[j] = frag_tr(dS, pc, 16 * w, 32 * j);
+                db[j] = frag_kc(dbS, pa, 16 * w, 32 * j);
+            }
+#pragma unroll
+            for (int ct = 0; ct < KT; ++ct) {
+                f32x4 p1 = zero4(), p2 = zero4(), q3 = zero4();
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const elemx8 kf = frag_tr(kS, pk, 16 * ct, 32 * j);
+                    p1 = mfma16x32(at[j], frag_tr(xS, px, 16 * ct, 32 * j), p1);   // A^T dw
+                    p2 = mfma16x32(dt[j], kf, p2);                                  // dA^T k
+                    q3 = mfma16x32(db[j], kf, q3);                                  // dA (k beta)
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float kv = (float)kS[(kChunk * hh + 16 * w + 4 * lg + e) * pk + 16 * ct + li];
+                    const float p1g = p1[e] * er[e];
+                    dk_acc[ct][e] += q3[e] + (p2[e] + p1g) * br[e];
+                    db_row[e] += (p2[e] + p1g) * kv;
+                    dg_row[e] += (p1g * br[e] + br[e] * p2[e] - q3[e]) * kv;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float sb = group_sum<16>(db_row[e]), sg = group_sum<16>(dg_row[e]);
+                const int row = 16 * w + 4 * lg + e;
+                if (li == 0 && row < rlen) {
+                    p.dbeta[b * p.db_sb + hv * p.db_sh + (int64_t)(rstart + row) * p.db_st] = sb;
+                    p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(rstart + row) * p.dg_st] = sg;
+                }
+            }
+        }
+        char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh +
+                                             (int64_t)rstart * p.dk.st);
+#pragma unroll
+        for (int ct = 0; ct < KT; ++ct) acc_to_global(dkg + 32 * ct, p.dk.st * 2, 16 * w, rlen, dk_acc[ct]);
+    }
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 #define FLA_BWD_DISPATCH_T(KERNEL, NAME, GRID, SMEM_EXPR, P, THREADS)                                                   \
     do {                                                                                                               \
@@ -844,11 +1114,11 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
 int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A,
                   const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, int64_t chunk_size, ChunkGeom &geom) {
     int rc;
-    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // prepare_wy_repr_bwd_full/README.md:74
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
     if ((rc = check_bhtd(op, "dw", dw, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "du", du, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr && beta != nullptr && beta->data != nullptr, FLA_ERR_NULL,
@@ -866,7 +1136,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
     ChunkGeom geom;
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
-    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, dt_bit(kElemDtype)))) return rc;
+    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, dt_bit(kElemDtype)))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
@@ -874,6 +1144,13 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
                   view3(beta), nullptr, nullptr, 0, 0, 0, 0, 0, 0};
     const dim3 grid(geom.NT, geom.Hv, geom.B);
     const int K = geom.K, V = geom.V;
+    if (geom.C == 128) {
+        const size_t smem128 = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8)) + (size_t)2 * 128 * (128 + 8)) * 2 + 3 * 128 * 4;
+        if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da128_kernel<128, 128>), "wy_bwd_da", grid, smem128, p);
+        if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_da128_kernel<64, 64>), "wy_bwd_da", grid, smem128, p);
+        if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da128_kernel<64, 128>), "wy_bwd_da", grid, smem128, p);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel for chunk_size 128; built: (128,128),(64,64),(64,128).", op, K, V);
+    }
     const size_t smem = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8) + (kChunk + 8))) * 2 + 3 * kChunk * 4;
     if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_da_kernel<128, 128>), "wy_bwd_da", grid, smem, p);
     if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_da_kernel<64, 64>), "wy_bwd_da", grid, smem, p);
@@ -892,7 +1169,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
     const int bf = dt_bit(kElemDtype);
-    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
     if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_f32_bht(op, "dbeta", dbeta, geom))) return rc;
@@ -905,6 +1182,15 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
     const dim3 grid(geom.NT, geom.Hk, geom.B);
     const int K = geom.K, V = geom.V;
+    if (geom.C == 128) {
+        FLA_REQUIRE(!accumulate, FLA_ERR_UNSUPPORTED, "%s: the accumulating form is built for chunk_size 64.", op);
+        const int KV = K > V ? K : V;
+        const size_t smem128 = ((size_t)128 * ((K + 16) + (KV + 16) + 2 * (kChunk + 8)) + (size_t)kChunk * (128 + 8 + V)) * 2 + 2 * 128 * 4;
+        if (K == 128 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full128_kernel<128, 128>), "wy_bwd_full", grid, smem128, p);
+        if (K == 64 && V == 64) FLA_BWD_DISPATCH((wy_bwd_full128_kernel<64, 64>), "wy_bwd_full", grid, smem128, p);
+        if (K == 64 && V == 128) FLA_BWD_DISPATCH((wy_bwd_full128_kernel<64, 128>), "wy_bwd_full", grid, smem128, p);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel for chunk_size 128; built: (128,128),(64,64),(64,128).", op, K, V);
+    }
     const size_t smem = ((size_t)kChunk * ((K + 16) + ((K > V ? K : V) + 16) + V + 3 * (kChunk + 8))) * 2 + 2 * kChunk * 4;
     const bool gva = geom.Hv != geom.Hk;
 #define FLA_WY_FULL(KK, VV, G)                                                                                      \

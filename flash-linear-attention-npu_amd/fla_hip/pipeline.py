@@ -111,13 +111,18 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
     # the second part of dk and dg is added where it is produced (the reference adds with separate passes,
     # examples/flash_gated_delta_rule.py:994-1012)
-    dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size, **kw)
+    if chunk_size == 64:
+        dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size, **kw)
+    else:   # 128-token chunks: the plain operator and the reference's two additions
+        dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
+        dk.add_(dk2)
+        dg.add_(dg2)
     dg = _ops.chunk_local_cumsum(dg, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
     return dq, dk, dv, db.transpose(1, 2), dg.transpose(1, 2), dh0
 
 
 def needs_grad_hint(*tensors) -> bool:
-    """True when autograd will record the call (the backward operators are built for 64-token chunks)."""
+    """True when autograd will record the call."""
     import torch
 
     return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
@@ -205,12 +210,12 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
                 f"got initial_state.shape[0]={initial_state.shape[0]} and sequences={len(cu) - 1}.")
     if scale is None:
         scale = k.shape[-1] ** -0.5
-    # (o, final_state) do not depend on the chunk size: it only tiles the same recurrence.  The fused kernel and
-    # the backward operators tile by 64 tokens (the forward operators also by 128), so any other request is served
-    # on 64-token chunks.
-    if chunk_size != 64 and (fused or needs_grad_hint(q, k, v, g, beta, initial_state) or chunk_size != 128):
+    # (o, final_state) do not depend on the chunk size: it only tiles the same recurrence.  The fused kernel tiles by
+    # 64 tokens, so it serves every request on 64-token chunks; the operators, forward and backward, are built for 64
+    # and 128.
+    if chunk_size != 64 and (fused or chunk_size != 128):
         if not fused:
-            raise NotImplementedError("the six-operator route is built for chunk_size 64 and 128 (forward); use fused=True.")
+            raise NotImplementedError("the six-operator route is built for chunk_size 64 and 128; use fused=True.")
         chunk_size = 64
     needs_grad = needs_grad_hint(q, k, v, g, beta, initial_state)
     if not needs_grad:

@@ -185,16 +185,45 @@ def test_backward_operators_with_128_token_chunks(dev, case):
     st = err_stats(dg, dg_r)
     assert st["rel_max"] <= TOL_BF16, f"dg: {st}"
 
+    # prepare_wy_repr_bwd_da / _full / both in one call, A and dA 128 wide
+    dwb = dw_r.to(BF)
+    dA = ops.prepare_wy_repr_bwd_da(x["k"], x["v"], x["beta"], x["A"], dwb.to(dev), dv2.to(dev), x["G"], chunk_size=C, **kw)
+    dA_ref = gdn_bwd.prepare_wy_repr_bwd_da(d["k"], d["v"], d["beta"], d["A"], dwb, dv2, d["G"], C,
+                                            output_dtype=torch.float32, **kw)
+    assert dA.shape == d["A"].shape and dA.shape[-1] == C
+    st = err_stats(dA, dA_ref)
+    assert st["rel_max"] <= TOL_BF16, f"dA: {st}"
+    a = dA.float().cpu()
+    for b, n, ci, s0, e0 in gdn.chunk_spans(B, T, C, cu):
+        blk = a[b, :, s0:e0]
+        assert float(torch.tril(blk[:, :, : e0 - s0], 0).abs().max()) == 0.0
+        if e0 - s0 < C:
+            assert float(blk[:, :, e0 - s0:].abs().max()) == 0.0
+    dAb = dA_ref.to(BF)
+    dk2, dv3, db, dg2 = ops.prepare_wy_repr_bwd_full(x["k"], x["v"], x["beta"], x["A"], dAb.to(dev), dwb.to(dev),
+                                                     dv2.to(dev), x["G"], C, **kw)
+    dk2_r, dv3_r, db_r, dg2_r = gdn_bwd.prepare_wy_repr_bwd_full(d["k"], d["v"], d["beta"], d["A"], dAb, dwb, dv2, d["G"], C,
+                                                                 output_dtype=torch.float32, **kw)
+    assert_close(dv3, dv3_r, TOL_BF16, "dv, 128-token chunks")
+    for name, got, ref in (("dk2", dk2, dk2_r), ("dbeta", db, db_r), ("dg2", dg2, dg2_r)):
+        st = err_stats(got, ref)
+        assert st["rel_max"] <= TOL_BF16, f"{name}: {st}"
+    one = ops.prepare_wy_repr_bwd(x["k"], x["v"], x["beta"], x["A"], dwb.to(dev), dv2.to(dev), x["G"], C, **kw)
+    two = ops.prepare_wy_repr_bwd_full(x["k"], x["v"], x["beta"], x["A"], dA, dwb.to(dev), dv2.to(dev), x["G"], C, **kw)
+    for name, a_, b_ in zip(("dk", "dv", "dbeta", "dg"), one, two):
+        assert torch.equal(a_, b_), name
+
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("case", [CASES[1], CASES[5], CASES[6]])
+@pytest.mark.parametrize("case", [(CASES[1], 64), (CASES[5], 64), (CASES[6], 64), (CASES_128[1], 128), (CASES_128[3], 128)],
+                         ids=lambda cc: f"T{cc[0][1]}-V{cc[0][5]}-C{cc[1]}")
 def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
     """The composed GPU backward against autograd (fp64) through the per-token recurrence on the same bf16
-    inputs: every gradient within 2e-2 of its own scale."""
+    inputs: every gradient within 2e-2 of its own scale; on 64- and on 128-token chunks."""
     from fla_hip import pipeline
-    B, T, Hv, Hk, K, V, cu = case
+    (B, T, Hv, Hk, K, V, cu), C = case
     scale = K ** -0.5
-    d = make(B, T, Hv, Hk, K, V, cu, seed=77, dtype=dtype)
+    d = make(B, T, Hv, Hk, K, V, cu, seed=77, dtype=dtype, C=C)
     dd = torch.float64
     leaf = {n: d[n].to(dd).requires_grad_(True) for n in ("q", "k", "v", "g", "beta", "h0")}
     o, final = gdn.naive_recurrent_gated_delta_rule(leaf["q"], leaf["k"], leaf["v"], leaf["g"], leaf["beta"], scale,
@@ -205,7 +234,7 @@ def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
     # pipeline layouts: g, beta [B,T,H]; do [B,T,H,V]
     got = pipeline.flash_chunk_gated_delta_rule_bwd(
         x["q"], x["k"], x["v"], x["G"].transpose(1, 2).contiguous(), x["beta"].transpose(1, 2).contiguous(), None, scale,
-        x["h0"], x["do"].transpose(1, 2).contiguous(), x["dht"], cu_seqlens=cu)
+        x["h0"], x["do"].transpose(1, 2).contiguous(), x["dht"], cu_seqlens=cu, chunk_size=C)
     dq, dk, dv, db, dg, dh0 = got
     want = dict(dq=leaf["q"].grad, dk=leaf["k"].grad, dv=leaf["v"].grad, db=leaf["beta"].grad.transpose(1, 2),
                 dg=leaf["g"].grad.transpose(1, 2), dh0=leaf["h0"].grad)
@@ -250,13 +279,17 @@ def test_autograd_through_flash_gated_delta_rule(dev):
     g = x["g"].transpose(1, 2).contiguous().requires_grad_(True)
     beta = x["beta"].transpose(1, 2).contiguous().requires_grad_(True)
     h0 = x["h0"].clone().requires_grad_(True)
-    o_g, fin_g = pipeline.flash_gated_delta_rule(q, k, v, g, beta, None, h0, True)
-    ((o_g.float() * x["do"].transpose(1, 2).float()).sum() + (fin_g * x["dht"]).sum()).backward()
     want = dict(q=leaf["q"].grad, k=leaf["k"].grad, v=leaf["v"].grad, g=leaf["g"].grad.transpose(1, 2),
                 beta=leaf["beta"].grad.transpose(1, 2), h0=leaf["h0"].grad)
-    for name, t in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("h0", h0)):
-        st = err_stats(t.grad, want[name])
-        assert st["rel_max"] <= TOL_BF16, f"d{name}: {st}"
+    # fused forward + backward on 64-token chunks; the six operators forward and backward on 64- and 128-token chunks
+    for kwargs in (dict(), dict(fused=False), dict(fused=False, chunk_size=128)):
+        for t in (q, k, v, g, beta, h0):
+            t.grad = None
+        o_g, fin_g = pipeline.flash_gated_delta_rule(q, k, v, g, beta, None, h0, True, **kwargs)
+        ((o_g.float() * x["do"].transpose(1, 2).float()).sum() + (fin_g * x["dht"]).sum()).backward()
+        for name, t in (("q", q), ("k", k), ("v", v), ("g", g), ("beta", beta), ("h0", h0)):
+            st = err_stats(t.grad, want[name])
+            assert st["rel_max"] <= TOL_BF16, f"d{name} with {kwargs}: {st}"
 
 
 @pytest.mark.parametrize("D", [64, 128, 256])
