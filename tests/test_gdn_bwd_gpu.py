@@ -142,6 +142,9 @@ CASES_128 = [
     (1, 421, 2, 1, 128, 128, [0, 1, 66, 66, 194, 300, 421]),
     (1, 330, 2, 2, 128, 256, None),
     (1, 130, 2, 2, 64, 64, None),
+    (1, 1, 1, 1, 128, 128, None),
+    (1, 65, 2, 2, 128, 128, None),
+    (2, 129, 2, 1, 128, 128, None),
 ]
 
 
