@@ -118,6 +118,17 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
     float *hdS = reinterpret_cast<float *>(hS + K * pv);   // [K]    sum_v h . dh per state row
     float *colS = hdS + K;                                  // [4][K] per row tile: sum_j k_j dk_j
     float *exS = colS + 4 * K;                              // [K]    what lands on the chunk's last token
+    // q, k and the gate of the chunk as whole rows (the epilogue reads them element by element in the accumulator
+    // layout; fetched that way from memory they came as 32- and 64-byte pieces)
+    constexpr int pq = K + 8, pg = K + 4;
+    elem *qS = reinterpret_cast<elem *>(exS + K);
+    elem *kS = qS + kChunk * pq;
+    float *gS = reinterpret_cast<float *>(kS + kChunk * pq);
+    // the three fp32 results leave through tiles laid over everything above once the products are done
+    float *outS = reinterpret_cast<float *>(smem);
+    static_assert((size_t)3 * kChunk * pg * 4 <= ((size_t)3 * kChunk * pv + (size_t)K * pv) * 2 + (size_t)6 * K * 4 +
+                                                     (size_t)2 * kChunk * pq * 2 + (size_t)kChunk * pg * 4,
+                  "the result tiles must fit the operand tiles");
 
     const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
@@ -126,26 +137,18 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
     // eight waves: wave (w, half) owns token rows 16w.. and column tiles half*KTH .. half*KTH+KTH-1
     const int tid = threadIdx.x, w = wave_id() & 3, half = wave_id() >> 2, l = lane_id(), li = l & 15, lg = l >> 4;
 
-    // element-wise operands in the accumulator layout, requested first and consumed in the epilogue
-    // (rows past the tail repeat the last valid row)
-    float qv[KTH][4], kv[KTH][4], gv[KTH][4], glast[KTH];
-    {
-        const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st;
-        const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st;
-        const float *gg = p.gk + b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st;
+    const float *gg = p.gk + b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st;
+    constexpr int GN = kChunk * (K / 4) / kDqkwgThreads;   // 16-byte pieces of the gate tile per thread
+    f32x4 gpre[GN];
 #pragma unroll
-        for (int ct = 0; ct < KTH; ++ct) {
-            const int col = 16 * (half * KTH + ct) + li;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int row = min(16 * w + 4 * lg + e, len - 1);
-                qv[ct][e] = (float)qg[(int64_t)row * p.q.st + col];
-                kv[ct][e] = (float)kg[(int64_t)row * p.k.st + col];
-                gv[ct][e] = gg[(int64_t)row * p.g_st + col];
-            }
-            glast[ct] = gg[(int64_t)(len - 1) * p.g_st + col];
-        }
+    for (int m = 0; m < GN; ++m) {
+        const int idx = m * kDqkwgThreads + tid;
+        const int r = min(idx / (K / 4), len - 1), c4 = (idx % (K / 4)) * 4;   // rows past the tail repeat the last valid row
+        gpre[m] = *reinterpret_cast<const f32x4 *>(gg + (int64_t)r * p.g_st + c4);
     }
+    TileCopy<kDqkwgThreads, kChunk, K> tq, tk;
+    tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+    tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
     TileCopy<kDqkwgThreads, K, V> tdh;
     {
         TileCopy<kDqkwgThreads, kChunk, V> tv, to, tdv;
@@ -155,6 +158,13 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
         tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st, p.dv.st, len, tid);
         th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
         tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
+#pragma unroll
+        for (int m = 0; m < GN; ++m) {
+            const int idx = m * kDqkwgThreads + tid;
+            *reinterpret_cast<f32x4 *>(gS + (idx / (K / 4)) * pg + (idx % (K / 4)) * 4) = gpre[m];
+        }
+        tq.commit(qS, pq, len, tid);
+        tk.commit(kS, pq, len, tid);
         tv.commit(vS, pv, len, tid);
         to.commit(oS, pv, len, tid);
         tdv.commit(dvS, pv, len, tid);
@@ -193,49 +203,61 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
     tdh.commit(hS, pv, K, tid);
     __syncthreads();
     // ---- product with the state gradient: dk (v_new dh^T); gate factors; column sums of k . dk -----
+    float qv[KTH][4], kv[KTH][4];
 #pragma unroll
     for (int ct = 0; ct < KTH; ++ct) {
-        const int cg = half * KTH + ct;
+        const int cg = half * KTH + ct, col = 16 * cg + li;
         f32x4 d = zero4();
 #pragma unroll
         for (int j = 0; j < V / 32; ++j) d = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * cg, 32 * j), d);
+        const float gl = gS[(len - 1) * pg + col];
         float colsum = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = 16 * w + 4 * lg + e;
-            dqa[ct][e] *= p.scale * ex2(gv[ct][e]);
-            d[e] *= ex2(glast[ct] - gv[ct][e]);
+            const float gv = gS[row * pg + col];
+            qv[ct][e] = (float)qS[row * pq + col];
+            kv[ct][e] = (float)kS[row * pq + col];
+            dqa[ct][e] *= p.scale * ex2(gv);
+            d[e] *= ex2(gl - gv);
             colsum += row < len ? kv[ct][e] * d[e] : 0.f;
         }
         dka[ct] = d;
         colsum += __shfl_xor(colsum, 16, kWave);
         colsum += __shfl_xor(colsum, 32, kWave);
-        if (lg == 0) colS[w * K + 16 * cg + li] = colsum;
+        if (lg == 0) colS[w * K + col] = colsum;
     }
     __syncthreads();
-    if (tid < K) {
-        const float gl = p.gk[b * p.g_sb + hv * p.g_sh + (int64_t)(start + len - 1) * p.g_st + tid];
-        exS[tid] = colS[tid] + colS[K + tid] + colS[2 * K + tid] + colS[3 * K + tid] + ex2(gl) * hdS[tid];
-    }
+    if (tid < K) exS[tid] = colS[tid] + colS[K + tid] + colS[2 * K + tid] + colS[3 * K + tid] + ex2(gS[(len - 1) * pg + tid]) * hdS[tid];
     __syncthreads();
-    float *dqg = p.dq.p + b * p.dq.sb + hv * p.dq.sh + (int64_t)start * p.dq.st;
-    float *dkg = p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st;
-    float *dgg = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+    float extra[KTH];
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) extra[ct] = exS[16 * (half * KTH + ct) + li];
+    __syncthreads();   // every operand tile is dead: the results take their place
 #pragma unroll
     for (int ct = 0; ct < KTH; ++ct) {
         const int col = 16 * (half * KTH + ct) + li;
-        const float extra = exS[col];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = 16 * w + 4 * lg + e;
-            if (row < len) {
-                dqg[(int64_t)row * p.dq.st + col] = dqa[ct][e];
-                dkg[(int64_t)row * p.dk.st + col] = dka[ct][e];
-                dgg[(int64_t)row * p.dg.st + col] =
-                    qv[ct][e] * dqa[ct][e] - kv[ct][e] * dka[ct][e] + (row == len - 1 ? extra : 0.f);
-            }
+            outS[row * pg + col] = dqa[ct][e];
+            outS[(kChunk + row) * pg + col] = dka[ct][e];
+            outS[(2 * kChunk + row) * pg + col] = qv[ct][e] * dqa[ct][e] - kv[ct][e] * dka[ct][e] + (row == len - 1 ? extra[ct] : 0.f);
         }
     }
+    __syncthreads();
+    float *dst[3] = {p.dq.p + b * p.dq.sb + hv * p.dq.sh + (int64_t)start * p.dq.st,
+                     p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st,
+                     p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st};
+    const int64_t dst_st[3] = {p.dq.st, p.dk.st, p.dg.st};
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int m = 0; m < GN; ++m) {
+            const int idx = m * kDqkwgThreads + tid;
+            const int r = idx / (K / 4), c4 = (idx % (K / 4)) * 4;
+            if (r < len) *reinterpret_cast<f32x4 *>(dst[t] + (int64_t)r * dst_st[t] + c4) = *reinterpret_cast<const f32x4 *>(outS + (t * kChunk + r) * pg + c4);
+        }
 }
 
 // =============================================================================
@@ -511,7 +533,8 @@ int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v
                      h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                      viewf(dq), viewf(dk), viewf(dg), (float)scale};
     const dim3 grid(geom.NT, geom.Hv, geom.B);
-    const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4;
+    const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
+                        (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
     if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<128, 128>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
     if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<64, 64>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
     if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<64, 128>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
