@@ -374,40 +374,59 @@ __global__ void __launch_bounds__(kThreads, 2) kda_bwd_wy_kernel(const KdaWyPara
         }
         acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
     }
-    float *dkg = p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st;
-    float *dgg = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+    // ---- x = Akk^T dw goes to an fp32 tile over the du, k 2^g and v tiles (dead by now); everything element-wise in
+    // it (dk += x 2^g beta, dg += that k, dbeta += <x 2^g, k>) then runs over whole rows, 16 bytes per lane: read and
+    // written from the accumulator layout the fp32 dk and dg moved as 64-byte pieces
+    constexpr int px = K + 4;
+    float *xS = reinterpret_cast<float *>(duS);
+    static_assert((size_t)kChunk * px * 4 + kChunk * 4 <= (size_t)kChunk * (pu + pk + pv) * 2, "x must fit the dead tiles");
+    float *dbS = xS + kChunk * px;   // [64] the <y, v> part of dbeta
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float s_ = group_sum<16>(db_row[e]);
+        if (li == 0) dbS[16 * w + 4 * lg + e] = s_;
+    }
 #pragma unroll
     for (int ct = 0; ct < KT; ++ct) {
-        const int col = 16 * ct + li;
-        // this tile's k, gate and incoming dk / dg: requested before the products, consumed after them
-        float kv[4], gv[4], pdk[4], pdg[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int row = min(16 * w + 4 * lg + e, len - 1);
-            kv[e] = (float)kg[(int64_t)row * p.k.st + col];
-            gv[e] = gg[(int64_t)row * p.g_st + col];
-            pdk[e] = dkg[(int64_t)row * p.dk.st + col];
-            pdg[e] = dgg[(int64_t)row * p.dg.st + col];
-        }
         f32x4 x = mfma16x32(at0, frag_tr(dwS, pw, 16 * ct, 0), zero4());
         x = mfma16x32(at1, frag_tr(dwS, pw, 16 * ct, 32), x);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int row = 16 * w + 4 * lg + e;
-            const float xe = x[e] * ex2(gv[e]);      // x 2^g
-            const float dk = xe * br[e];
-            db_row[e] += xe * kv[e];
-            if (row < len) {
-                dkg[(int64_t)row * p.dk.st + col] = pdk[e] + dk;
-                dgg[(int64_t)row * p.dg.st + col] = pdg[e] + dk * kv[e];
+        for (int e = 0; e < 4; ++e) xS[(16 * w + 4 * lg + e) * px + 16 * ct + li] = x[e];
+    }
+    __syncthreads();
+    {
+        float *dkg = p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st;
+        float *dgg = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+        constexpr int PPR = K / 4;                        // 16-byte pieces per row: one row = PPR consecutive lanes
+        constexpr int NP = kChunk * PPR / kThreads;
+        static_assert(PPR <= kWave && kWave % PPR == 0, "a row's pieces must sit in one wave");
+#pragma unroll
+        for (int m = 0; m < NP; ++m) {
+            const int idx = m * kThreads + tid;
+            const int r = idx / PPR, c4 = (idx % PPR) * 4, rr = min(r, len - 1);
+            const f32x4 x = *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
+            const f32x4 g4 = *reinterpret_cast<const f32x4 *>(gg + (int64_t)rr * p.g_st + c4);
+            const elemx4 k4 = *reinterpret_cast<const elemx4 *>(kg + (int64_t)rr * p.k.st + c4);
+            f32x4 dk4 = *reinterpret_cast<const f32x4 *>(dkg + (int64_t)rr * p.dk.st + c4);
+            f32x4 dg4 = *reinterpret_cast<const f32x4 *>(dgg + (int64_t)rr * p.dg.st + c4);
+            const float beta = bS[r];
+            float dbp = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float xe = x[e] * ex2(g4[e]), kk = (float)k4[e];
+                const float dk = xe * beta;
+                dbp += xe * kk;
+                dk4[e] += dk;
+                dg4[e] += dk * kk;
+            }
+            dbp = group_sum<PPR>(dbp);
+            if (r < len) {
+                *reinterpret_cast<f32x4 *>(dkg + (int64_t)r * p.dk.st + c4) = dk4;
+                *reinterpret_cast<f32x4 *>(dgg + (int64_t)r * p.dg.st + c4) = dg4;
+                if (idx % PPR == 0) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + r) * p.db_st] = dbp + dbS[r];
             }
         }
-    }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const float s = group_sum<16>(db_row[e]);
-        const int row = 16 * w + 4 * lg + e;
-        if (li == 0 && row < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + row) * p.db_st] = s;
     }
     __syncthreads();   // every wave has read its dw / du rows and columns: their tiles may be overwritten
     // ---- dM = -strict_lower(Akk^T dA Akk^T) ----------------------------------------------------
