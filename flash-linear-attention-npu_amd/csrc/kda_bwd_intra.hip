@@ -98,6 +98,7 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
 
     for (int ch0 = 0; ch0 < K; ch0 += KC) {
         __syncthreads();
+        f32x4 old[3][kChunk * (KC / 4) / kThreads];
         {
             TileCopy<kThreads, kChunk, KC> tq, tk;
             tq.fetch(p.q + qbase + ch0, p.q_st, len, tid);
@@ -110,6 +111,14 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
                 const int r = min(idx / (KC / 4), len - 1), c4 = (idx % (KC / 4)) * 4;
                 gv[m] = *reinterpret_cast<const f32x4 *>(p.gk + gbase + (int64_t)r * p.g_st + ch0 + c4);
             }
+#pragma unroll
+            for (int t = 0; t < 3; ++t)
+#pragma unroll
+                for (int m = 0; m < GN; ++m) {   // the incoming gradients of the block, consumed after the products
+                    const int idx = m * kThreads + tid;
+                    const int r = min(idx / (KC / 4), len - 1), c4 = (idx % (KC / 4)) * 4;
+                    old[t][m] = *reinterpret_cast<const f32x4 *>((t == 0 ? p.dq : t == 1 ? p.dk : p.dg) + base + (int64_t)r * p.st + ch0 + c4);
+                }
             tq.commit(qS, pk, len, tid);
             tk.commit(kS, pk, len, tid);
 #pragma unroll
@@ -119,49 +128,71 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
             }
         }
         __syncthreads();
-        if (r0 >= len) continue;   // wave-uniform: this row tile holds no token
-
+        // what this wave adds to dq, dk, dg of its 16 rows x KC channels, kept in registers until the products of the
+        // channel block are done; a row tile without a token (wave-uniform) adds nothing
+        f32x4 inc[KC / 16][3];
+#pragma unroll
+        for (int nt = 0; nt < KC / 16; ++nt) inc[nt][0] = inc[nt][1] = inc[nt][2] = f32x4{0.f, 0.f, 0.f, 0.f};
         const int nsteps_lo = (row_end + 3) >> 2;   // contraction over tokens j < row_end, four at a time
-        for (int nt = 0; nt < KC / 16; ++nt) {
-            const int ch = 16 * nt + li;
-            const float ca = gS[anchor * pg + ch];
-            // incoming gradients of this tile: requested now (clamped rows, no branch), consumed after the products
-            float pdq[4], pdk[4], pdg[4];
+        if (r0 < len) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int64_t off = base + (int64_t)min(r0 + 4 * lg + e, len - 1) * p.st + ch0 + ch;
-                pdq[e] = p.dq[off];
-                pdk[e] = p.dk[off];
-                pdg[e] = p.dg[off];
-            }
-            f32x4 D1 = {0.f, 0.f, 0.f, 0.f}, D2 = D1, D3 = D1;
-            for (int js = 0; js < nsteps_lo; ++js) {
-                const int j = 4 * js + lg;
-                const float bval = (float)kS[j * pk + ch] * ex2(ca - gS[j * pg + ch]);
-                D1 = mfma_f32(aqS[(r0 + li) * pa + j], bval, D1);
-                D2 = mfma_f32(akS[(r0 + li) * pa + j], bval, D2);
-            }
-            for (int is = r0 >> 2; is < 16; ++is) {
-                const int i = 4 * is + lg;
-                const float fw = ex2(gS[i * pg + ch] - ca);
-                const float kk = (float)kS[i * pk + ch];
-                D3 = mfma_f32(aqS[i * pa + r0 + li], (float)qS[i * pk + ch] * fw, D3);
-                D3 = mfma_f32(akS[i * pa + r0 + li], kk * bS[i] * fw, D3);
-            }
+            for (int nt = 0; nt < KC / 16; ++nt) {
+                const int ch = 16 * nt + li;
+                const float ca = gS[anchor * pg + ch];
+                f32x4 D1 = {0.f, 0.f, 0.f, 0.f}, D2 = D1, D3 = D1;
+                for (int js = 0; js < nsteps_lo; ++js) {
+                    const int j = 4 * js + lg;
+                    const float bval = (float)kS[j * pk + ch] * ex2(ca - gS[j * pg + ch]);
+                    D1 = mfma_f32(aqS[(r0 + li) * pa + j], bval, D1);
+                    D2 = mfma_f32(akS[(r0 + li) * pa + j], bval, D2);
+                }
+                for (int is = r0 >> 2; is < 16; ++is) {
+                    const int i = 4 * is + lg;
+                    const float fw = ex2(gS[i * pg + ch] - ca);
+                    const float kk = (float)kS[i * pk + ch];
+                    D3 = mfma_f32(aqS[i * pa + r0 + li], (float)qS[i * pk + ch] * fw, D3);
+                    D3 = mfma_f32(akS[i * pa + r0 + li], kk * bS[i] * fw, D3);
+                }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int i = r0 + 4 * lg + e;
-                if (i < len) {
-                    const float gi = gS[i * pg + ch];
-                    const float up = ex2(gi - ca), down = ex2(ca - gi);
-                    const float dqd = D1[e] * up, dl = D2[e] * up, du = D3[e] * down;
-                    const float qi = (float)qS[i * pk + ch], ki = (float)kS[i * pk + ch];
-                    const float bdl = bS[i] * dl;
-                    const int64_t off = base + (int64_t)i * p.st + ch0 + ch;
-                    p.dq_o[off] = pdq[e] + dqd;
-                    p.dk_o[off] = pdk[e] + bdl + du;
-                    p.dg_o[off] = pdg[e] + qi * dqd + ki * (bdl - du);
-                    dbacc[e] += dl * ki;
+                for (int e = 0; e < 4; ++e) {
+                    const int i = r0 + 4 * lg + e;
+                    if (i < len) {
+                        const float gi = gS[i * pg + ch];
+                        const float up = ex2(gi - ca), down = ex2(ca - gi);
+                        const float dqd = D1[e] * up, dl = D2[e] * up, du = D3[e] * down;
+                        const float qi = (float)qS[i * pk + ch], ki = (float)kS[i * pk + ch];
+                        const float bdl = bS[i] * dl;
+                        inc[nt][0][e] = dqd;
+                        inc[nt][1][e] = bdl + du;
+                        inc[nt][2][e] = qi * dqd + ki * (bdl - du);
+                        dbacc[e] += dl * ki;
+                    }
+                }
+            }
+        }
+        // The increments leave through an fp32 tile laid over the q and k tiles (dead once every wave is past its
+        // products), one gradient at a time, and are added to memory over whole rows, 16 bytes per lane: from the
+        // accumulator layout the fp32 gradients moved in and out as 64-byte pieces.
+        float *xS = reinterpret_cast<float *>(qS);
+        constexpr int px = KC + 4;
+        static_assert((size_t)kChunk * px * 4 <= (size_t)2 * kChunk * pk * 2, "the staging tile must fit the q and k tiles");
+        float *gout[3] = {p.dq_o, p.dk_o, p.dg_o};
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            __syncthreads();
+#pragma unroll
+            for (int nt = 0; nt < KC / 16; ++nt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) xS[(r0 + 4 * lg + e) * px + 16 * nt + li] = inc[nt][t][e];
+            __syncthreads();
+            constexpr int PN = kChunk * (KC / 4) / kThreads;
+#pragma unroll
+            for (int m = 0; m < PN; ++m) {
+                const int idx = m * kThreads + tid;
+                const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
+                if (r < len) {
+                    const int64_t off = base + (int64_t)r * p.st + ch0 + c4;
+                    *reinterpret_cast<f32x4 *>(gout[t] + off) = old[t][m] + *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
                 }
             }
         }
