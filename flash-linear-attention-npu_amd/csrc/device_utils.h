@@ -154,6 +154,28 @@ __device__ __forceinline__ void split_hilo(f32x4 x, elemx4 &hi, elemx4 &lo) {
     lo = cvt4(rem);
 #endif
 }
+// Persistent scans launch a (slabs, heads, sequences) grid: the `slabs` workgroups of one (sequence, head) chain read
+// the same key-side operands.  Workgroups are handed to the eight XCDs in turn (linear id % 8), each XCD with an L2 of
+// its own, so ids L, L + 8, ... go to one chain and its second and later reads of those operands hit that L2.
+__device__ __forceinline__ void chain_of_block(int &slab, int &head, int &seq) {
+    const int slabs = gridDim.x, heads = gridDim.y, total = slabs * heads * gridDim.z;
+    const int lin = blockIdx.x + slabs * (blockIdx.y + heads * blockIdx.z);
+    int chain;
+    if (slabs > 1 && total % (8 * slabs) == 0) {
+        chain = (lin / (8 * slabs)) * 8 + (lin & 7);
+        slab = (lin >> 3) % slabs;
+    } else {
+        chain = lin / slabs;
+        slab = lin % slabs;
+    }
+    head = chain % heads;
+    seq = chain / heads;
+}
+
+// Workgroup barrier that orders LDS traffic only: the wave waits for its own LDS operations, not for its global loads
+// and stores, which stay in flight across the barrier.  For data handed over through LDS while prefetches are pending.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 __device__ __forceinline__ elemx8 cat8(elemx4 lo, elemx4 hi) {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }

@@ -475,7 +475,9 @@ template <int K> struct DhuSmem {
 };
 
 // 512 threads: waves 0-3 compute chunk c (walking backwards) from LDS buffer c&1 while waves 4-7 copy
-// the tiles of chunk c-1 into the other buffer; one barrier per chunk.  dv2 leaves from registers.
+// the tiles of chunk c-1 into the other buffer and have those of chunk c-2 in flight.  Both results leave through LDS
+// as whole 128-byte rows, stored by the copying waves one step later: dv2 replaces the wave's own columns of the dv
+// tile, dh goes over the k tile once every wave is past its k . dh products (the barrier in the middle of a step).
 template <int K, bool GK>
 __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -483,8 +485,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     constexpr int VS = 64, CT = 1;
     constexpr int pk = L::pk, pt = L::pt, pv = L::pv;
     constexpr int KT = K / 16, KS = K / 32;
+    constexpr int ph = VS + 4;   // pitch of dh [K][VS] laid over the k tile: rows are 8-byte aligned
+    static_assert(K * ph <= kChunk * pk, "dh must fit the k tile");
 
-    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    int slab, hv, n;
+    chain_of_block(slab, hv, n);
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     const int V = p.geom.V;
     int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
@@ -504,43 +509,113 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
         const int tid = threadIdx.x - kThreads;
-        auto load = [&](int c) {
-            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-            const int start = bos + c * kChunk;
-            const int len = min(kChunk, eos - start);
+        // Two register sets: while chunk c is computed, the tiles of chunk c - 1 are committed to LDS and those of
+        // chunk c - 2 are on their way.  Before the first chunk the loads re-read it (never committed), so that the same
+        // number of operations lies between a load and the commit that waits for it in every step.
+        struct Tiles {
             TileCopy<kThreads, kChunk, K> tk, tq, tw;
             TileCopy<kThreads, kChunk, VS> to, tv;
-            tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
-            tq.fetch(qg + (int64_t)start * p.q.st, p.q.st, len, tid);
-            tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
-            to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
-            tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            float gv;
+        };
+        Tiles t0, t1;
+        auto fetch = [&](Tiles &t, int c) {
+            c = max(c, 0);
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            t.tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
+            t.tq.fetch(qg + (int64_t)start * p.q.st, p.q.st, len, tid);
+            t.tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
+            t.to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+            t.tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            if (GK) t.gv = p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + min(tid, K - 1)];
+            else t.gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+        };
+        auto commit = [&](const Tiles &t, int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int len = min(kChunk, eos - (bos + c * kChunk));
             float *gS = reinterpret_cast<float *>(buf + L::g_off);
             float *fS = gS + (K > kChunk ? K : kChunk);
-            float gv = 0.f;
+            t.tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
+            t.tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pt, len, tid);
+            t.tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pt, len, tid);
+            t.to.commit(reinterpret_cast<elem *>(buf + L::o_off), pv, len, tid);
+            t.tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
             if (GK) {
-                if (tid < K) gv = p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + tid];
-            } else if (tid < kChunk) {
-                gv = tid < len ? load_scalar(p.g, b, hv, start + tid) : 0.f;
-            }
-            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
-            tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pt, len, tid);
-            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pt, len, tid);
-            to.commit(reinterpret_cast<elem *>(buf + L::o_off), pv, len, tid);
-            tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
-            if (GK) {
-                if (tid < K) gS[tid] = exp2f(gv);
+                if (tid < K) gS[tid] = exp2f(t.gv);
                 if (tid < kChunk) fS[tid] = p.scale;
             } else if (tid < kChunk) {
-                gS[tid] = gv;
-                fS[tid] = tid < len ? p.scale * __expf(gv) : 0.f;
+                gS[tid] = tid < len ? t.gv : 0.f;
+                fS[tid] = tid < len ? p.scale * __expf(t.gv) : 0.f;
             }
         };
-        if (nchunks > 0) load(nchunks - 1);
-        __syncthreads();
-        for (int c = nchunks - 1; c >= 0; --c) {
-            if (c > 0) load(c - 1);
-            __syncthreads();
+        // results of the step before (chunk c): read from LDS ahead of the barrier, stored behind the commit
+        constexpr int NV = TileCopy<kThreads, kChunk, VS>::N, NH = K * (VS / 8) / kThreads;
+        u32x4 vr[NV];
+        u32x2 hr[NH][2];
+        auto chunk_end = [&](int c) { return (c % p.sub) == p.sub - 1 || c == nchunks - 1; };
+        auto read_out = [&](int c) {
+            const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const elem *vS = reinterpret_cast<const elem *>(buf + L::v_off);
+            const elem *hS = reinterpret_cast<const elem *>(buf + L::k_off);
+#pragma unroll
+            for (int m = 0; m < NV; ++m) {
+                const int idx = m * kThreads + tid;
+                vr[m] = *reinterpret_cast<const u32x4 *>(vS + (idx / (VS / 8)) * pv + (idx % (VS / 8)) * 8);
+            }
+            if (chunk_end(c)) {
+#pragma unroll
+                for (int m = 0; m < NH; ++m) {
+                    const int idx = m * kThreads + tid;
+                    const elem *src = hS + (idx / (VS / 8)) * ph + (idx % (VS / 8)) * 8;
+                    hr[m][0] = *reinterpret_cast<const u32x2 *>(src);
+                    hr[m][1] = *reinterpret_cast<const u32x2 *>(src + 4);
+                }
+            }
+        };
+        auto store_out = [&](int c) {
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            elem *v2 = static_cast<elem *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + (int64_t)start * p.dv2.st + slab * VS;
+#pragma unroll
+            for (int m = 0; m < NV; ++m) {
+                const int idx = m * kThreads + tid;
+                const int r = idx / (VS / 8), c8 = (idx % (VS / 8)) * 8;
+                if (r < len) *reinterpret_cast<u32x4 *>(v2 + (int64_t)r * p.dv2.st + c8) = vr[m];
+            }
+            if (chunk_end(c)) {
+                elem *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c / p.sub) * p.h_sc + slab * VS;
+#pragma unroll
+                for (int m = 0; m < NH; ++m) {
+                    const int idx = m * kThreads + tid;
+                    *reinterpret_cast<u32x4 *>(hg + (int64_t)(idx / (VS / 8)) * V + (idx % (VS / 8)) * 8) =
+                        u32x4{hr[m][0][0], hr[m][0][1], hr[m][1][0], hr[m][1][1]};
+                }
+            }
+        };
+        // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
+        auto step = [&](Tiles &ahead, const Tiles &next, int c) {
+            if (c + 1 < nchunks) read_out(c + 1);
+            lds_barrier();   // results of chunk c + 1 are in registers; the compute waves are past the k tile of chunk c
+            fetch(ahead, c - 2);
+            if (c > 0) commit(next, c - 1);
+            // the stores go last: a commit waits for everything issued before the loads it needs, and by the next
+            // commit these stores are a whole step old
+            if (c + 1 < nchunks) store_out(c + 1);
+            lds_barrier();   // the loads of chunk c - 2 stay in flight
+        };
+        if (nchunks > 0) {
+            fetch(t0, nchunks - 1);
+            commit(t0, nchunks - 1);
+            fetch(t1, nchunks - 2);
+        }
+        lds_barrier();
+        for (int c = nchunks - 1; c >= 0; c -= 2) {
+            step(t0, t1, c);
+            if (c > 0) step(t1, t0, c - 1);
+        }
+        if (nchunks > 0) {
+            read_out(0);
+            store_out(0);
         }
         return;
     }
@@ -563,7 +638,6 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             dacc[kt][ct] = a;
         }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // terminal gradient loaded before the loop (vmcnt(0))
-    char *v2g = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh + vcol0);
     __syncthreads();
 
     // With 128-token chunks a chunk takes two 64-token steps, the later tokens first.  Every token of the chunk sees the
@@ -575,11 +649,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     for (int c = nchunks - 1; c >= 0; --c) {
         const bool chunk_end = (c % p.sub) == p.sub - 1 || c == nchunks - 1;
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-        const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
+        elem *kS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::k_off));
         const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
         const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
         const elem *oS = reinterpret_cast<const elem *>(buf + L::o_off);
-        const elem *vS = reinterpret_cast<const elem *>(buf + L::v_off);
+        elem *vS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::v_off));
         const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
         const float *fS = gS + (K > kChunk ? K : kChunk);
         const int start = bos + c * kChunk;
@@ -590,12 +664,6 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             for (int j = 0; j < KS; ++j)
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
-            elem *hg = p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c / p.sub) * p.h_sc;
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct)   // lane pairs swap halves: two dword stores per tile instead of four 2-byte ones
-                    acc_to_global(reinterpret_cast<char *>(hg + vcol0 + 16 * ct), (int64_t)V * 2, 16 * kt, K, dacc[kt][ct]);
         }
 
         // dv2 = dv + (k . dh) * e^{g_last - g}
@@ -614,6 +682,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             }
         if (chunk_end) g_end = GK ? 0.f : gS[len - 1];
         const float g_last = g_end;
+        lds_barrier();   // every wave is past the k tile, which now takes dh on its way to memory
+        if (chunk_end) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) acc_to_tile(kS, ph, 16 * kt, wv * 16, dacc[kt][0]);
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
@@ -626,13 +699,8 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                     dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + (float)old[e] : 0.f;
                 }
             }
-        {
-            char *dst = v2g + (int64_t)start * p.dv2.st * 2;
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt)
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) acc_to_global(dst + ct * 32, (int64_t)p.dv2.st * 2, rt * 16, len, dv2[rt][ct]);
-        }
+        for (int rt = 0; rt < 4; ++rt) acc_to_tile(vS, pv, rt * 16, wv * 16, dv2[rt][0]);   // over the wave's own columns of dv
 
         // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
         if (chunk_end) {
@@ -677,7 +745,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
     }
 
     // gradient of the initial state

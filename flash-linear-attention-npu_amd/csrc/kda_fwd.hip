@@ -630,7 +630,7 @@ struct KdaScanParams {
 };
 
 template <int K> struct ScanSmem {
-    static constexpr int pw = K + 8, pt = K + 16, pu = 64 + 16, pb = 72;
+    static constexpr int pw = K + 8, pt = K + 16, pu = 64 + 8, pb = 72, ph = 64 + 8;
     static constexpr size_t w_off = 0;                                    // w
     static constexpr size_t q_off = w_off + (size_t)kChunk * pw * 2;      // qg
     static constexpr size_t k_off = q_off + (size_t)kChunk * pw * 2;      // kg (read transposed)
@@ -638,11 +638,16 @@ template <int K> struct ScanSmem {
     static constexpr size_t a_off = u_off + (size_t)kChunk * pu * 2;      // Aqk
     static constexpr size_t d_off = a_off + (size_t)kChunk * pb * 2;      // [K] decay of the chunk
     static constexpr size_t buf_bytes = d_off + (size_t)K * 4;
-    static constexpr size_t bytes = 2 * buf_bytes;
+    static constexpr size_t h_off = 2 * buf_bytes;                        // [K][ph]: the state on its way to memory
+    static constexpr size_t bytes = h_off + (size_t)K * ph * 2;
 };
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
-// c+1 from memory into the other buffer; one barrier per chunk.  Outputs leave from registers.
+// c+1 from memory into the other buffer; one barrier per chunk.  o leaves from registers.  The optional outputs
+// for a backward pass leave through LDS as whole 128-byte rows, stored by the copying waves: v_new replaces the
+// wave's own columns of the u tile and is written out one step later, before the tile is loaded again; h (default
+// [K][V] blocks) goes through a tile of its own, written at the end of the step before and guarded by a second
+// barrier per step.
 // SUB = 2: 128-token chunks walked as two 64-token steps.  Both steps see the state of the chunk's first token in
 // w S and qg S (the operand copy of the state is refreshed on even steps only), the second step adds the
 // coupling block Aqk21 times the first step's v_new, and the decay of the chunk is applied once, on the first step
@@ -652,10 +657,11 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     typedef ScanSmem<K> L;
     constexpr int VS = 64;
-    constexpr int pw = L::pw, pt = L::pt, pu = L::pu, pb = L::pb;
+    constexpr int pw = L::pw, pt = L::pt, pu = L::pu, pb = L::pb, ph = L::ph;
     constexpr int KT = K / 16, KS = K / 32;
 
-    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    int slab, hv, n;
+    chain_of_block(slab, hv, n);
     const int V = p.geom.V;
     int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
     if (p.geom.cu != nullptr) {
@@ -667,36 +673,110 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     const int nchunks = (eos - bos + kChunk - 1) / kChunk;
     const int64_t head_row = ((int64_t)b * p.geom.Hv + hv) * p.geom.T;
 
+    elem *hS = reinterpret_cast<elem *>(smem + L::h_off);
+    const bool stage_h = p.h != nullptr && !p.v_first;   // uniform: both groups run the second barrier or neither
+
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
         const int tid = threadIdx.x - kThreads;
-        auto load = [&](int c) {
-            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-            const int start = bos + c * kChunk;
-            const int len = min(kChunk, eos - start);
-            const int64_t row = head_row + start;
+        // The tiles of two steps are in flight at once: while step c is computed, those of step c + 1 are committed to
+        // LDS and those of step c + 2 are on their way into the other register set, so that a load has two steps
+        // to arrive.  Past the last step the loads re-read the last one (never committed), which keeps the number of
+        // operations between a load and the commit that waits for it the same in every step.
+        struct Tiles {
             TileCopy<kThreads, kChunk, K> tw, tq, tk;
             TileCopy<kThreads, kChunk, VS> tu;
             TileCopy<kThreads, kChunk, kChunk> ta;
-            tw.fetch(p.w + row * K, K, len, tid);
-            tq.fetch(p.qg + row * K, K, len, tid);
-            tk.fetch(p.kg + row * K, K, len, tid);
-            tu.fetch(p.u + row * V + slab * VS, V, len, tid);
-            ta.fetch(p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, len, tid);   // diagonal block
-            float dec = 0.f;
-            if (tid < K) dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c / SUB) * p.geom.Hv + hv) * K + tid];
-            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
-            tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pw, len, tid);
-            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pt, len, tid);
-            tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
-            ta.commit(reinterpret_cast<elem *>(buf + L::a_off), pb, len, tid);
-            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = dec;
+            float dec;
         };
-        if (nchunks > 0) load(0);
-        __syncthreads();
-        for (int c = 0; c < nchunks; ++c) {
-            if (c + 1 < nchunks) load(c + 1);
-            __syncthreads();
+        Tiles t0, t1;
+        auto fetch = [&](Tiles &t, int c) {
+            c = min(c, nchunks - 1);
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            const int64_t row = head_row + start;
+            t.tw.fetch(p.w + row * K, K, len, tid);
+            t.tq.fetch(p.qg + row * K, K, len, tid);
+            t.tk.fetch(p.kg + row * K, K, len, tid);
+            t.tu.fetch(p.u + row * V + slab * VS, V, len, tid);
+            t.ta.fetch(p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, len, tid);   // diagonal block
+            t.dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c / SUB) * p.geom.Hv + hv) * K + min(tid, K - 1)];
+        };
+        auto commit = [&](const Tiles &t, int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            t.tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
+            t.tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pw, len, tid);
+            t.tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pt, len, tid);
+            t.tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
+            t.ta.commit(reinterpret_cast<elem *>(buf + L::a_off), pb, len, tid);
+            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = t.dec;
+        };
+        // v_new of step c sits in the u tile of buffer c & 1; a thread writes out exactly the pieces it later commits.
+        // Both outputs are read from LDS before the barrier and stored after it, behind the loads of the next step.
+        constexpr int NV = TileCopy<kThreads, kChunk, VS>::N, NH = K * (VS / 8) / kThreads;
+        u32x4 vr[NV], hr[NH];
+        auto read_vn = [&](int c) {
+            const elem *uS = reinterpret_cast<const elem *>(smem + (c & 1) * L::buf_bytes + L::u_off);
+#pragma unroll
+            for (int m = 0; m < NV; ++m) {
+                const int idx = m * kThreads + tid;
+                vr[m] = *reinterpret_cast<const u32x4 *>(uS + (idx / (VS / 8)) * pu + (idx % (VS / 8)) * 8);
+            }
+        };
+        auto store_vn = [&](int c) {
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            elem *vg = p.v_new + (head_row + start) * V + slab * VS;
+#pragma unroll
+            for (int m = 0; m < NV; ++m) {
+                const int idx = m * kThreads + tid;
+                const int r = idx / (VS / 8), c8 = (idx % (VS / 8)) * 8;
+                if (r < len) *reinterpret_cast<u32x4 *>(vg + (int64_t)r * V + c8) = vr[m];
+            }
+        };
+        auto read_h = [&]() {
+#pragma unroll
+            for (int m = 0; m < NH; ++m) {
+                const int idx = m * kThreads + tid;
+                hr[m] = *reinterpret_cast<const u32x4 *>(hS + (idx / (VS / 8)) * ph + (idx % (VS / 8)) * 8);
+            }
+        };
+        auto store_h = [&](int c) {   // the state at the start of step c, the first of its chunk
+            elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c / SUB) * p.h_sc + hv * p.h_sh + slab * VS;
+#pragma unroll
+            for (int m = 0; m < NH; ++m) {
+                const int idx = m * kThreads + tid;
+                *reinterpret_cast<u32x4 *>(hg + (int64_t)(idx / (VS / 8)) * V + (idx % (VS / 8)) * 8) = hr[m];
+            }
+        };
+        // one step: `ahead` takes the tiles of step c + 2, `next` holds those of step c + 1
+        auto step = [&](Tiles &ahead, const Tiles &next, int c) {
+            const bool with_h = stage_h && (c % SUB) == 0, with_vn = p.v_new && c > 0;
+            if (with_h) read_h();
+            if (with_vn) read_vn(c - 1);
+            if (stage_h) lds_barrier();   // the state tile has been read
+            fetch(ahead, c + 2);
+            if (c + 1 < nchunks) commit(next, c + 1);
+            // the stores go last: the commit waits for everything issued before the loads it needs, and by the next
+            // commit these stores are a whole step old
+            if (with_h) store_h(c);
+            if (with_vn) store_vn(c - 1);
+            lds_barrier();                // the loads of step c + 2 stay in flight
+        };
+        if (nchunks > 0) {
+            fetch(t0, 0);
+            commit(t0, 0);
+            fetch(t1, 1);
+        }
+        lds_barrier();
+        for (int c = 0; c < nchunks; c += 2) {
+            step(t0, t1, c);
+            if (c + 1 < nchunks) step(t1, t0, c + 1);
+        }
+        if (p.v_new && nchunks > 0) {
+            read_vn(nchunks - 1);
+            store_vn(nchunks - 1);
         }
         return;
     }
@@ -719,6 +799,11 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);   // initial state loaded before the loop (vmcnt(0))
     char *og = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
+    auto state_to_tile = [&]() {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) acc_to_tile(hS, ph, 16 * kt, wv * 16, hacc[kt]);
+    };
+    if (stage_h && nchunks > 0) state_to_tile();
     __syncthreads();
 
     elemx8 hB[KS], vprev[2] = {};
@@ -727,7 +812,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
         const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
         const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
-        const elem *uS = reinterpret_cast<const elem *>(buf + L::u_off);
+        elem *uS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::u_off));
         const elem *aS = reinterpret_cast<const elem *>(buf + L::a_off);
         const float *dS = reinterpret_cast<const float *>(buf + L::d_off);
         const int start = bos + c * kChunk;
@@ -739,19 +824,13 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
             for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
         }
-        if (p.h && first) {
+        if (p.h && p.v_first && first) {   // [V][K] blocks: the lane's four K rows are contiguous
             elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c / SUB) * p.h_sc + hv * p.h_sh;
-            if (p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
 #pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-                    const elemx8 f = hB[kt >> 1];
-                    const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
-                    *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + li) * K + 16 * kt + 4 * lg) = q4;
-                }
-            } else {           // [K][V] blocks: lane pairs swap halves, two dword stores per tile
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt)
-                    acc_to_global(reinterpret_cast<char *>(hg + vcol0), (int64_t)V * 2, 16 * kt, K, hacc[kt]);
+            for (int kt = 0; kt < KT; ++kt) {
+                const elemx8 f = hB[kt >> 1];
+                const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
+                *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + li) * K + 16 * kt + 4 * lg) = q4;
             }
         }
 
@@ -798,6 +877,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
                 for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[j][rt], hB[j], oacc[rt]);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (stage_h) lds_barrier();   // the copying waves have read the state tile of this step
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
             const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
@@ -807,10 +887,9 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
                 oacc[rt][e] *= p.scale;
             }
         }
-        if (p.v_new) {
-            char *vg = reinterpret_cast<char *>(p.v_new + row * V + vcol0);
+        if (p.v_new) {   // over the wave's own columns of u, which no other wave reads
 #pragma unroll
-            for (int rt = 0; rt < 4; ++rt) acc_to_global(vg, (int64_t)V * 2, rt * 16, len, vn[rt]);
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
         }
         // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same bf16 v_new operand serves both)
         elemx8 vB[2];
@@ -854,7 +933,8 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
-        __syncthreads();
+        if (stage_h && c + 1 < nchunks && (SUB == 1 || ((c + 1) % SUB) == 0)) state_to_tile();
+        lds_barrier();   // nothing waits for the stores of o
     }
 
     if (p.hT) {
