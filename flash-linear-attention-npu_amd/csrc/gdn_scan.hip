@@ -55,7 +55,8 @@ template <int K, int CT> struct FwdHSmem {
 };
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
-// c+1 into the other buffer; one barrier per chunk.  v_new and the final state leave from registers; the
+// c+1 into the other buffer and have those of chunk c+2 in flight; one barrier per chunk, which waits for LDS
+// traffic only.  v_new and the final state leave from registers; the
 // per-chunk state h goes through an LDS tile and is written out by the loader waves one chunk later, as whole
 // 128-byte rows (written from the accumulator layout it would leave as 32-byte pieces of eight different rows
 // per store, which cost 0.19 ms of a 0.48 ms launch at B=4, T=8192, H=32).
@@ -66,7 +67,8 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     constexpr int VS = L::VS, pw = L::pw, pk = L::pk, pu = L::pu;
     constexpr int KT = K / 16, KS = K / 32;
 
-    const int slab = blockIdx.x, hv = blockIdx.y, n = blockIdx.z;
+    int slab, hv, n;
+    chain_of_block(slab, hv, n);
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     const int V = p.geom.V;
     int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
@@ -84,24 +86,36 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
         const int tid = threadIdx.x - kThreads;
-        auto load = [&](int c) {
-            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
-            const int start = bos + c * kChunk;
-            const int len = min(kChunk, eos - start);
+        // Two register sets: while step c is computed, the tiles of step c + 1 are committed to LDS and those of step
+        // c + 2 are on their way.  Past the last step the loads re-read the last one (never committed), so that the same
+        // number of operations lies between a load and the commit that waits for it in every step.
+        struct Tiles {
             TileCopy<kThreads, kChunk, K> tw, tk;
             TileCopy<kThreads, kChunk, VS> tu;
-            tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
-            tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
-            tu.fetch(ug + (int64_t)start * p.u.st, p.u.st, len, tid);
-            float gv = 0.f, dk = 1.f;
-            if (tid < kChunk && p.g.p) gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
-            if (p.gk && tid < K)
-                dk = __builtin_amdgcn_exp2f(p.gk[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + tid]);
-            tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
-            tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
-            tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
-            if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? gv : 0.f;
-            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = dk;
+            float gv, dk;
+        };
+        Tiles t0, t1;
+        auto fetch = [&](Tiles &t, int c) {
+            c = min(c, nchunks - 1);
+            const int start = bos + c * kChunk;
+            const int len = min(kChunk, eos - start);
+            t.tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
+            t.tk.fetch(kg + (int64_t)start * p.k.st, p.k.st, len, tid);
+            t.tu.fetch(ug + (int64_t)start * p.u.st, p.u.st, len, tid);
+            t.gv = 0.f;
+            t.dk = 1.f;
+            if (p.g.p) t.gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
+            if (p.gk)
+                t.dk = __builtin_amdgcn_exp2f(p.gk[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + min(tid, K - 1)]);
+        };
+        auto commit = [&](const Tiles &t, int c) {
+            unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            t.tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pw, len, tid);
+            t.tk.commit(reinterpret_cast<elem *>(buf + L::k_off), pk, len, tid);
+            t.tu.commit(reinterpret_cast<elem *>(buf + L::u_off), pu, len, tid);
+            if (tid < kChunk) reinterpret_cast<float *>(buf + L::g_off)[tid] = tid < len ? t.gv : 0.f;
+            if (tid < K) reinterpret_cast<float *>(buf + L::d_off)[tid] = t.dk;
         };
         const bool stage_h = L::kStage && p.h != nullptr && !p.v_first;
         auto store_h = [&](int c) {   // staged state at the start of step c (a chunk start) -> h[.., chunk, :, slab columns]
@@ -130,13 +144,24 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                         *reinterpret_cast<const u32x4 *>(st + r * L::ps + c8);
             }
         };
-        if (nchunks > 0) load(0);
-        __syncthreads();
-        for (int c = 0; c < nchunks; ++c) {
+        // one step: `ahead` takes the tiles of step c + 2, `next` holds those of step c + 1.  The stores go last: a
+        // commit waits for everything issued before the loads it needs, and by the next commit they are a step old.
+        auto step = [&](Tiles &ahead, const Tiles &next, int c) {
+            fetch(ahead, c + 2);
+            if (c + 1 < nchunks) commit(next, c + 1);
             if (L::kStage && c > 0) store_v(c - 1);
             if (stage_h && c > 0) store_h(c - 1);
-            if (c + 1 < nchunks) load(c + 1);
-            __syncthreads();
+            lds_barrier();   // the loads of step c + 2 stay in flight
+        };
+        if (nchunks > 0) {
+            fetch(t0, 0);
+            commit(t0, 0);
+            fetch(t1, 1);
+        }
+        lds_barrier();
+        for (int c = 0; c < nchunks; c += 2) {
+            step(t0, t1, c);
+            if (c + 1 < nchunks) step(t1, t0, c + 1);
         }
         if (L::kStage && nchunks > 0) store_v(nchunks - 1);
         if (stage_h && nchunks > 0) store_h(nchunks - 1);
@@ -296,7 +321,7 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) hacc[kt][ct] = mfma16x32(afrag, vB[j][ct], hacc[kt][ct]);
             }
-        __syncthreads();
+        lds_barrier();   // nothing waits for stores to memory
     }
 
     if (p.hT) {
