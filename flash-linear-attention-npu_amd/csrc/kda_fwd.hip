@@ -646,8 +646,8 @@ template <int K> struct ScanSmem {
 // c+1 from memory into the other buffer; one barrier per chunk.  o leaves from registers.  The optional outputs
 // for a backward pass leave through LDS as whole 128-byte rows, stored by the copying waves: v_new replaces the
 // wave's own columns of the u tile and is written out one step later, before the tile is loaded again; h (default
-// [K][V] blocks) goes through a tile of its own, written at the end of the step before and guarded by a second
-// barrier per step.
+// [K][V] blocks) goes through a tile of its own, written behind a second barrier in the middle of the step (the
+// state changes only at the step's end) and written out one step later as well.
 // SUB = 2: 128-token chunks walked as two 64-token steps.  Both steps see the state of the chunk's first token in
 // w S and qg S (the operand copy of the state is refreshed on even steps only), the second step adds the
 // coupling block Aqk21 times the first step's v_new, and the decay of the chunk is applied once, on the first step
@@ -752,15 +752,15 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         };
         // one step: `ahead` takes the tiles of step c + 2, `next` holds those of step c + 1
         auto step = [&](Tiles &ahead, const Tiles &next, int c) {
-            const bool with_h = stage_h && (c % SUB) == 0, with_vn = p.v_new && c > 0;
+            const bool with_h = stage_h && c > 0 && ((c - 1) % SUB) == 0, with_vn = p.v_new && c > 0;
             if (with_h) read_h();
             if (with_vn) read_vn(c - 1);
-            if (stage_h) lds_barrier();   // the state tile has been read
+            if (stage_h) lds_barrier();   // the state tile of the step before has been read
             fetch(ahead, c + 2);
             if (c + 1 < nchunks) commit(next, c + 1);
             // the stores go last: the commit waits for everything issued before the loads it needs, and by the next
             // commit these stores are a whole step old
-            if (with_h) store_h(c);
+            if (with_h) store_h(c - 1);
             if (with_vn) store_vn(c - 1);
             lds_barrier();                // the loads of step c + 2 stay in flight
         };
@@ -777,6 +777,10 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         if (p.v_new && nchunks > 0) {
             read_vn(nchunks - 1);
             store_vn(nchunks - 1);
+        }
+        if (stage_h && nchunks > 0 && ((nchunks - 1) % SUB) == 0) {
+            read_h();
+            store_h(nchunks - 1);
         }
         return;
     }
@@ -803,7 +807,6 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) acc_to_tile(hS, ph, 16 * kt, wv * 16, hacc[kt]);
     };
-    if (stage_h && nchunks > 0) state_to_tile();
     __syncthreads();
 
     elemx8 hB[KS], vprev[2] = {};
@@ -877,7 +880,10 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
                 for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[j][rt], hB[j], oacc[rt]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (stage_h) lds_barrier();   // the copying waves have read the state tile of this step
+        if (stage_h) {   // the copying waves have read the state tile of the step before; the state is still that of
+            lds_barrier();   // this step's start
+            if (first) state_to_tile();
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
             const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
@@ -933,7 +939,6 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
-        if (stage_h && c + 1 < nchunks && (SUB == 1 || ((c + 1) % SUB) == 0)) state_to_tile();
         lds_barrier();   // nothing waits for the stores of o
     }
 
