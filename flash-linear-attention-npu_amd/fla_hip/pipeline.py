@@ -151,7 +151,8 @@ def _autograd_function():
         def backward(ctx, do, dht):
             q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd, h, v_new, w = ctx.saved_tensors
             dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
-                q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(), dht, ctx.cu, ctx.chunk_size,
+                q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(),
+                None if dht is None else dht.contiguous(), ctx.cu, ctx.chunk_size,
                 saved=dict(h=h, v_new=v_new, w=w))
             if q_rstd is not None:      # :1104-1106
                 dq = _raw.l2norm_bwd(q, q_rstd, dq)
@@ -332,6 +333,7 @@ def _kda_autograd_function():
         @staticmethod
         def backward(ctx, do, dht):
             q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state = ctx.saved_tensors
+            dht = None if dht is None else dht.contiguous()   # a view when the caller sliced or joined the final state
             dq, dk, dv, dg, db, dh0 = chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, ctx.scale, do, dht,
                                                     initial_state=initial_state, layout=ctx.layout, cu_seqlens=ctx.cu,
                                                     chunk_size=ctx.chunk_size)
@@ -368,7 +370,8 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     The forward is ``chunk_kda_fwd``; when an input requires grad the forward keeps its intermediates and
     ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0.  With ``use_gate_in_kernel`` g is the raw gate input: without
     gradients the forward kernel activates it; with gradients the activation runs as tensor operations ahead of the
-    kernels, so that autograd also reaches ``A_log`` and ``dt_bias``."""
+    kernels, so that autograd also reaches ``A_log`` and ``dt_bias``.  Gradients cover every admitted head size with
+    K <= 128 (V up to 256 as two passes over 128 value columns) and run on 64-token tiles whatever ``chunk_size``."""
     import torch
 
     if scale is None:
@@ -381,12 +384,29 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
                                  use_gate_in_kernel=use_gate_in_kernel, A_log=A_log, dt_bias=dt_bias, safe_gate=safe_gate,
                                  lower_bound=lower_bound)
         return out[0], out[1]
-    if chunk_size != 64:
-        raise NotImplementedError("chunk_kda: gradients are built for chunk_size 64.")
+    if chunk_size not in (64, 128):
+        raise RuntimeError("chunk_kda: chunk_size must be 64 or 128.")
+    # The chunk size tiles the same function.  The gradient kernels are built for 64-token tiles, as the reference's own
+    # backward kernel is (npu_chunk_kda_bwd_intra, _aclnn_ctypes.py:1582-1584), so a differentiated call runs on them.
+    chunk_size = 64
     if use_gate_in_kernel:
         if A_log is None:
             raise RuntimeError("chunk_kda: A_log must be float32 [HV] when use_gate_in_kernel=True.")
         g = _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound)
+    K, V = q.shape[-1], v.shape[-1]
+    if K > 128:
+        raise NotImplementedError(f"chunk_kda: gradients are built for K <= 128, got K={K}.")
+    if V > 128:
+        # Value columns never mix: o[.., c] and the state column c depend on v[.., c] only.  Two passes over 128 columns
+        # each share q, k, g and beta, whose gradients autograd adds up.
+        parts = []
+        for lo in (0, 128):
+            h0 = None if initial_state is None else initial_state[..., lo:lo + 128].contiguous()
+            parts.append(chunk_kda(q, k, v[..., lo:lo + 128], g, beta, scale, h0, output_final_state, cu_seqlens,
+                                   layout=layout, chunk_size=chunk_size))
+        o = torch.cat([parts[0][0], parts[1][0]], dim=-1)
+        final = None if parts[0][1] is None else torch.cat([parts[0][1], parts[1][1]], dim=-1)
+        return o, final
     global _KDA_FUNCTION
     if _KDA_FUNCTION is None:
         _KDA_FUNCTION = _kda_autograd_function()
@@ -394,11 +414,8 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     # 128 x 128 run on the next built one with zero channels appended (a zero q/k channel adds nothing to any product, a
     # zero v column yields zero columns of o and of the state); the padding is itself differentiable, so autograd
     # returns the gradients of the unpadded tensors.
-    K, V = q.shape[-1], v.shape[-1]
-    Kp = 64 if K <= 64 and V <= 128 else 128
-    Vp = Kp if V <= Kp else 2 * Kp
-    if K > 128 or (Kp, Vp) == (128, 256):
-        raise NotImplementedError(f"chunk_kda: gradients are built for K <= 128 with V <= 128 (K <= 64: V <= 128), got K={K} V={V}.")
+    Kp = 64 if K <= 64 else 128
+    Vp = Kp if V <= Kp else 128
     if (Kp, Vp) != (K, V):
         F = torch.nn.functional
         h0 = None if initial_state is None else F.pad(initial_state, (0, Vp - V, 0, Kp - K))

@@ -177,6 +177,11 @@ COMPOSITION_CASES = [
     # head sizes between the built ones: zero channels appended around the kernels
     dict(B=1, T=100, Hk=1, Hv=2, K=96, V=80, layout="BSND", h0=True, dht=True),
     dict(B=1, T=130, Hk=1, Hv=1, K=32, V=112, layout="TND", cu=[0, 65, 130], h0=True, dht=True),
+    # more than 128 value columns: two passes that share q, k, g and beta
+    dict(B=1, T=140, Hk=1, Hv=2, K=128, V=256, layout="BSND", h0=True, dht=True),
+    dict(B=1, T=100, Hk=1, Hv=1, K=48, V=192, layout="BNSD", h0=True, dht=True),
+    # a 128-token chunk size asks for the same function
+    dict(B=1, T=200, Hk=1, Hv=2, K=128, V=128, layout="BSND", h0=True, dht=True, chunk=128),
 ]
 
 
@@ -199,7 +204,7 @@ def test_chunk_kda_backward_against_autograd_through_the_recurrence(dev, case):
 
     ins = [lay(t, layout).to(dev).requires_grad_(True) for t in (q, k, v, gate, beta)]
     h0_d = None if h0 is None else h0.to(dev).requires_grad_(True)
-    o, final = pipeline.chunk_kda(*ins, scale, h0_d, True, cu, layout=layout)
+    o, final = pipeline.chunk_kda(*ins, scale, h0_d, True, cu, layout=layout, chunk_size=case.get("chunk", 64))
     loss = (o.float() * lay(do, layout).to(dev).float()).sum()
     if dht is not None:
         loss = loss + (final * dht.to(dev)).sum()
@@ -314,5 +319,8 @@ def test_chunk_kda_rejections(dev):
     q = torch.zeros(1, 64, 1, 128, dtype=BF, device=dev, requires_grad=True)
     g = torch.zeros(1, 64, 1, 128, device=dev)
     beta = torch.ones(1, 64, 1, device=dev)
-    with pytest.raises(NotImplementedError, match="chunk_size 64"):
-        pipeline.chunk_kda(q, q, q, g, beta, chunk_size=128)
+    with pytest.raises(RuntimeError, match="chunk_size must be 64 or 128"):
+        pipeline.chunk_kda(q, q, q, g, beta, chunk_size=32)
+    q = torch.zeros(1, 64, 1, 144, dtype=BF, device=dev, requires_grad=True)
+    with pytest.raises(NotImplementedError, match="K <= 128"):
+        pipeline.chunk_kda(q, q, q, torch.zeros(1, 64, 1, 144, device=dev), beta)
