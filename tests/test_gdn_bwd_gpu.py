@@ -163,7 +163,7 @@ def test_dv_local_with_128_token_chunks(dev, case):
     assert_close(got, ref, TOL_BF16, "dv_local, 128-token chunks")
 
 
-@pytest.mark.parametrize("case", [c for c in CASES_128 if c[5] <= 128])
+@pytest.mark.parametrize("case", CASES_128)
 def test_backward_operators_with_128_token_chunks(dev, case):
     """The operators that follow dv_local, each on 128-token operands (A [T,128], one h / dh block per 128 tokens, the
     gate cumulated over the chunk) against the oracle on the same 16-bit inputs
@@ -218,7 +218,8 @@ def test_backward_operators_with_128_token_chunks(dev, case):
 
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("case", [(CASES[1], 64), (CASES[5], 64), (CASES[6], 64), (CASES_128[1], 128), (CASES_128[3], 128)],
+@pytest.mark.parametrize("case", [(CASES[1], 64), (CASES[5], 64), (CASES[6], 64), (CASES_128[1], 128), (CASES_128[3], 128),
+                                  (CASES_128[4], 128)],
                          ids=lambda cc: f"T{cc[0][1]}-V{cc[0][5]}-C{cc[1]}")
 def test_backward_pipeline_against_recurrence_autograd(dev, case, dtype):
     """The composed GPU backward against autograd (fp64) through the per-token recurrence on the same bf16
