@@ -44,6 +44,7 @@ struct BwdIntraParams {
     int64_t db_sb, db_sh, db_st;
     const float *daqk, *dakk;    // [..,64]
     int64_t m_sb, m_sh, m_st;
+    int cumsum_dg;               // 1: dg leaves as its reverse running sum over the tokens of the chunk
 };
 
 template <int KC>
@@ -186,6 +187,48 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
                 for (int e = 0; e < 4; ++e) xS[(r0 + 4 * lg + e) * px + 16 * nt + li] = inc[nt][t][e];
             __syncthreads();
             constexpr int PN = kChunk * (KC / 4) / kThreads;
+            if (t == 2 && p.cumsum_dg) {
+                // The gate gradient is complete with this kernel's part, and a workgroup holds a whole chunk of it: the
+                // reverse running sum over the chunk's tokens (what follows in the composition) is taken here, column by
+                // column in the tile, instead of by a pass of its own over memory.
+#pragma unroll
+                for (int m = 0; m < PN; ++m) {
+                    const int idx = m * kThreads + tid;
+                    const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
+                    f32x4 v = old[t][m] + *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
+                    if (r >= len) v = f32x4{0.f, 0.f, 0.f, 0.f};
+                    *reinterpret_cast<f32x4 *>(xS + r * px + c4) = v;
+                }
+                __syncthreads();
+                constexpr int SEGS = kThreads / KC, RS = kChunk / SEGS;   // a thread sums RS rows of one column
+                const int col = tid % KC, seg = tid / KC;
+                float *tot = gS;                                          // the gates of this block are no longer read
+                float run = 0.f;
+#pragma unroll
+                for (int j = RS - 1; j >= 0; --j) {
+                    float *x = xS + (seg * RS + j) * px + col;
+                    run += *x;
+                    *x = run;
+                }
+                tot[seg * KC + col] = run;
+                __syncthreads();
+                float later = 0.f;
+#pragma unroll
+                for (int s2 = 1; s2 < SEGS; ++s2)
+                    if (seg + s2 < SEGS) later += tot[(seg + s2) * KC + col];
+#pragma unroll
+                for (int j = 0; j < RS; ++j) xS[(seg * RS + j) * px + col] += later;
+                __syncthreads();
+#pragma unroll
+                for (int m = 0; m < PN; ++m) {
+                    const int idx = m * kThreads + tid;
+                    const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
+                    if (r < len)
+                        *reinterpret_cast<f32x4 *>(gout[t] + base + (int64_t)r * p.st + ch0 + c4) =
+                            *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
+                }
+                continue;
+            }
 #pragma unroll
             for (int m = 0; m < PN; ++m) {
                 const int idx = m * kThreads + tid;
@@ -225,9 +268,9 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
                    const fla_tensor *daqk, const fla_tensor *dakk, const fla_tensor *dq, const fla_tensor *dk,
                    const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu, const fla_int_array *ci,
                    int64_t chunk_size, bool safe_gate, const char *layout, const fla_tensor *dq_o, const fla_tensor *dk_o,
-                   const fla_tensor *db_o, const fla_tensor *dg_o, void *ws, uint64_t ws_size, hipStream_t stream,
-                   uint64_t *query) {
-    const char *op = "chunk_kda_bwd_intra";
+                   const fla_tensor *db_o, const fla_tensor *dg_o, bool cumsum_dg, void *ws, uint64_t ws_size,
+                   hipStream_t stream, uint64_t *query) {
+    const char *op = cumsum_dg ? "chunk_kda_bwd_intra_cumsum" : "chunk_kda_bwd_intra";
     FLA_REQUIRE(layout != nullptr, FLA_ERR_NULL, "%s: layout must not be null.", op);
     int ib, ih, it;
     if (!strcmp(layout, "BSND")) { ib = 0; it = 1; ih = 2; }
@@ -359,6 +402,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.m_sh = daqk->stride[ih];
     p.m_st = daqk->stride[it];
     FLA_REQUIRE(p.q_st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride of q and k must be below 2^24 elements.", op);
+    p.cumsum_dg = cumsum_dg ? 1 : 0;
     return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }
 
@@ -374,7 +418,7 @@ FLA_ENTRY(fla_chunk_kda_bwd_intra_get_workspace_size)(
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra_get_workspace_size, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_intra: workspace_size must not be null.");
     return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
-                               layout, dq_out, dk_out, db_out, dg_out, nullptr, 0, nullptr, workspace_size); });
+                               layout, dq_out, dk_out, db_out, dg_out, false, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_chunk_kda_bwd_intra)(
@@ -385,6 +429,30 @@ FLA_ENTRY(fla_chunk_kda_bwd_intra)(
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream) {
     FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
-                               layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size,
+                               layout, dq_out, dk_out, db_out, dg_out, false, workspace, workspace_size,
+                               static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_intra_cumsum_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
+    const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
+    const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra_cumsum_get_workspace_size, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace_size);
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_intra_cumsum: workspace_size must not be null.");
+    return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+                               layout, dq_out, dk_out, db_out, dg_out, true, nullptr, 0, nullptr, workspace_size); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_intra_cumsum)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta, const fla_tensor *dAqk,
+    const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *db, const fla_tensor *dg,
+    const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate,
+    const char *layout, const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_intra_cumsum, q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate, layout, dq_out, dk_out, db_out, dg_out, workspace, workspace_size, stream);
+    return fla::guarded([&] { return fla::bwd_intra_impl(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, cu_seqlens, chunk_indices, chunk_size, safe_gate,
+                               layout, dq_out, dk_out, db_out, dg_out, true, workspace, workspace_size,
                                static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -42,6 +42,7 @@ OP_ARGTYPES = {
     "chunk_kda_fwd": [_T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_char_p, ctypes.c_double, ctypes.c_int64,
                       ctypes.c_bool, ctypes.c_double, ctypes.c_bool, ctypes.c_bool] + [_T] * 11,
     "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
+    "chunk_kda_bwd_intra_cumsum": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
                                        ctypes.c_bool, _T, _T, _T],
     "l2norm_fwd": [_T, ctypes.c_double, _T, _T],
@@ -855,17 +856,20 @@ def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, dk, dg, chunk_size=64, *, cu_s
     return outs
 
 
-def chunk_kda_bwd_intra_inplace(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_seqlens=None, chunk_size=64):
+def chunk_kda_bwd_intra_inplace(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_seqlens=None, chunk_size=64,
+                                cumsum_dg=False):
     """``npu_chunk_kda_bwd_intra`` on [B,H,T,*] index-order views with the results written over ``dq, dk, db, dg``.
     The library accepts strided views, grouped heads (q, k with fewer heads than gk) and outputs that alias their
-    inputs; the public operator keeps the reference's contiguous, allocate-new contract."""
+    inputs; the public operator keeps the reference's contiguous, allocate-new contract.  ``cumsum_dg``: dg leaves as
+    its reverse chunk-local running sum, the pass that follows this operator in the KDA backward."""
     cu = _as_int_tuple(cu_seqlens)
     indices = None if cu is None else _build_chunk_indices(cu, int(chunk_size))
     ins = (q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg)
     names = ("q", "k", "gk", "beta", "dAqk", "dAkk", "dq", "dk", "db", "dg")
     outs = (dq, dk, db, dg)
+    name = "chunk_kda_bwd_intra_cumsum" if cumsum_dg else "chunk_kda_bwd_intra"
     _call_op(
-        "chunk_kda_bwd_intra", OP_ARGTYPES["chunk_kda_bwd_intra"],
+        name, OP_ARGTYPES[name],
         lambda ctx: [
             *[ctx.tensor(t, n) for t, n in zip(ins, names)],
             ctx.int_array(cu), ctx.int_array(indices), ctypes.c_int64(int(chunk_size)), ctypes.c_bool(True),

@@ -294,8 +294,9 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
                                               layout_like=layout_like, **kw)
     dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
-    _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size)
-    _raw.chunk_local_cumsum_into(dg, dg, chunk_size, cu_seqlens=cu, reverse=True)
+    # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
+    _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size,
+                                     cumsum_dg=True)
     if Hv != Hk:          # value heads that share a key head add their gradients
         dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2)
         dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2)

@@ -398,6 +398,25 @@ int fla_chunk_kda_bwd_intra(
     const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
     const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
 
+/* chunk_kda_bwd_intra followed by the reverse chunk-local running sum of dg_out.  No counterpart in the reference, whose
+ * composition (and this build's, fla_hip.pipeline.chunk_kda_bwd) runs chunk_local_cumsum(reverse) over the gate gradient
+ * right after this operator: here the workgroup that holds a chunk of dg takes the sum before it stores it.  Same
+ * operands and rules as fla_chunk_kda_bwd_intra. */
+int fla_chunk_kda_bwd_intra_cumsum_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
+    const fla_tensor *dAqk, const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate, const char *layout,
+    const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_intra_cumsum(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
+    const fla_tensor *dAqk, const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk,
+    const fla_tensor *db, const fla_tensor *dg, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, int64_t chunk_size, bool safe_gate, const char *layout,
+    const fla_tensor *dq_out, const fla_tensor *dk_out, const fla_tensor *db_out,
+    const fla_tensor *dg_out, void *workspace, uint64_t workspace_size, void *stream);
+
 /* ------------------------------------------------------------------------
  * KDA chunk backward, the stages around chunk_gated_delta_rule_bwd_dhu (gK) and chunk_kda_bwd_intra.
  * The reference has no operators for them: its deployment keeps them in a third-party Triton package

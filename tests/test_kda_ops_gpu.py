@@ -270,6 +270,32 @@ def test_chunk_kda_bwd_intra(dev, case):
         assert_close(_unlay(a, layout), e.float(), 2e-4, name)
 
 
+@pytest.mark.parametrize("case", [(64, 2, 130, None), (128, 3, 200, None), (128, 2, 261, [0, 1, 16, 33, 33, 96, 160, 261]),
+                                  (256, 1, 65, None)], ids=lambda c: f"K{c[0]}-H{c[1]}-T{c[2]}")
+def test_chunk_kda_bwd_intra_with_the_reverse_running_sum(dev, case):
+    """The library-only form that also takes the reverse chunk-local running sum of dg (the pass that follows the
+    operator in the KDA backward): dq, dk, db equal the operator's bit for bit, dg equals the fp64 reference of the
+    operator summed backwards over each chunk."""
+    from fla_hip.ops import _hip_ctypes as raw
+    K, H, T, cu = case
+    x = intra_inputs(1, T, H, K, seed=K + T, beta_dtype=BF, cu=cu)
+    ref = kda.chunk_kda_bwd_intra(*x, chunk=64, cu_seqlens=cu)
+    dg_ref = ref[3].double().clone()
+    for b, n, ci, s, e in gdn.chunk_spans(1, T, 64, cu):
+        dg_ref[b, :, s:e] = torch.flip(torch.cumsum(torch.flip(dg_ref[b, :, s:e], dims=[1]), dim=1), dims=[1])
+    xd = [t.to(dev) for t in x]
+    plain = [t.clone() for t in xd]
+    raw.chunk_kda_bwd_intra_inplace(*plain, cu_seqlens=cu)
+    fused = [t.clone() for t in xd]
+    raw.chunk_kda_bwd_intra_inplace(*fused, cu_seqlens=cu, cumsum_dg=True)
+    for i in (6, 7, 8):
+        assert torch.equal(plain[i], fused[i])
+    assert_close(fused[9], dg_ref.float(), 2e-4, "dg, reverse running sum")
+    again = [t.clone() for t in xd]
+    raw.chunk_kda_bwd_intra_inplace(*again, cu_seqlens=cu, cumsum_dg=True)
+    assert torch.equal(again[9], fused[9])
+
+
 def test_chunk_kda_bwd_intra_errors(dev):
     from fla_hip import ops
     x = [t.to(dev) for t in intra_inputs(1, 64, 2, 128, seed=1, beta_dtype=BF)]
