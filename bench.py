@@ -64,16 +64,30 @@ def gdn_kernel_flops_per_token_head(C=64, K=128, V=128):
 
 
 def preheat(step, torch, ms):
-    """Untimed: repeats ``step`` for about ``ms`` milliseconds of GPU work so that the timed region that follows
-    sees the sustained device clock (a few tens of launches do not ramp it).  Returns the milliseconds spent."""
+    """Untimed: repeats ``step`` for at least ``ms`` milliseconds of GPU work so that the timed region that follows
+    sees the sustained device clock (a few tens of launches do not ramp it, and after seconds of host-only work -- a
+    CPU baseline -- the device needs longer than after a short pause).  It goes on until two consecutive batches take
+    the same time to within 3 %, for at most six times ``ms``.  Returns the milliseconds spent."""
     if ms <= 0:
         return 0.0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    while (time.perf_counter() - t0) * 1e3 < ms:
-        for _ in range(8):
+    n, prev = 8, None
+    while True:
+        tb = time.perf_counter()
+        for _ in range(n):
             step()
         torch.cuda.synchronize()
+        now = time.perf_counter()
+        cur, spent = (now - tb) / n, (now - t0) * 1e3
+        if (now - tb) * 1e3 < 3.0:      # batches long enough for the host clock to compare them
+            n *= 2
+            continue
+        if spent >= ms and prev is not None and abs(cur - prev) <= 0.03 * prev:
+            break
+        if spent >= 6 * ms:
+            break
+        prev = cur
     return round((time.perf_counter() - t0) * 1e3, 1)
 
 
@@ -745,7 +759,7 @@ def main():
         brief.steps, brief.warmup, brief.preheat_ms = 100, 10, min(args.preheat_ms, 100.0)
         brief.cpu_seconds, brief.cpu_tokens = min(args.cpu_seconds, 2.0), 512
         secondary = {}
-        for name, sub in (("decode", bench_decode), ("conv1d", bench_conv1d), ("kda", bench_kda)):
+        for name, sub in (("kda", bench_kda), ("decode", bench_decode), ("conv1d", bench_conv1d)):
             r = sub(brief, torch, dev)
             keep = ("metric", "value", "unit", "steps", "ms_per_step", "dtype", "config", "algorithmic", "step_tflops",
                     "step_GBps", "step_frac_of_hbm_peak", "roofline", "cpu_baseline", "fwd_bwd", "varlen_prefill", "eager_ms_per_step")
