@@ -56,10 +56,10 @@ template <int K, int CT> struct FwdHSmem {
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
 // c+1 into the other buffer and have those of chunk c+2 in flight; one barrier per chunk, which waits for LDS
-// traffic only.  v_new and the final state leave from registers; the
-// per-chunk state h goes through an LDS tile and is written out by the loader waves one chunk later, as whole
-// 128-byte rows (written from the accumulator layout it would leave as 32-byte pieces of eight different rows
-// per store, which cost 0.19 ms of a 0.48 ms launch at B=4, T=8192, H=32).
+// traffic only.  The final state leaves from registers; v_new and the per-chunk state h go through LDS tiles and are
+// written out by the loader waves one chunk later, as whole 128-byte rows (written from the accumulator layout they
+// would leave as 32-byte pieces of eight different rows per store, which cost 0.19 ms of a 0.48 ms launch at B=4,
+// T=8192, H=32; the 128-column slab form has no LDS left for the tiles and stores from registers).
 template <int K, int CT>
 __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];

@@ -643,7 +643,8 @@ template <int K> struct ScanSmem {
 };
 
 // 512 threads: waves 0-3 compute chunk c from LDS buffer c&1 while waves 4-7 copy the tiles of chunk
-// c+1 from memory into the other buffer; one barrier per chunk.  o leaves from registers.  The optional outputs
+// c+1 from memory into the other buffer and have those of chunk c+2 in flight; the barriers wait for LDS traffic
+// only, so that loads and stores stay in flight across them.  o leaves from registers.  The optional outputs
 // for a backward pass leave through LDS as whole 128-byte rows, stored by the copying waves: v_new replaces the
 // wave's own columns of the u tile and is written out one step later, before the tile is loaded again; h (default
 // [K][V] blocks) goes through a tile of its own, written behind a second barrier in the middle of the step (the
