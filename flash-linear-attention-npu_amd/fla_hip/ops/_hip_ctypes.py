@@ -18,6 +18,19 @@ from ._runtime import INT_ARRAY_P, TENSOR_P
 _call_op = _runtime.call_op
 _empty = _runtime.empty
 _empty_like = _runtime.empty_like
+
+
+def _empty_ordered_like(like, *, dtype=None, shape=None):
+    """An uninitialised tensor of ``shape`` (default: that of ``like``) whose dimensions sit in memory in the order of
+    ``like``'s.  For a contiguous ``like`` this is a contiguous tensor, as the reference's operators return; for a
+    token-major view [B,H,T,D] (what a caller holds after ``x.transpose(1, 2)``) the result is such a view too, so that
+    a gradient flows back through the transpose without a copy.  The kernels take outer strides either way."""
+    import torch
+
+    shape = tuple(like.shape) if shape is None else tuple(int(d) for d in shape)
+    order = sorted(range(len(shape)), key=lambda d: (-like.stride(d), d))
+    base = torch.empty([shape[d] for d in order], dtype=dtype or like.dtype, device=like.device)
+    return base.permute([order.index(d) for d in range(len(shape))])
 _shape = _runtime.shape
 
 _T, _IA = TENSOR_P, INT_ARRAY_P
@@ -335,7 +348,7 @@ def npu_chunk_scaled_dot_kkt(k, g, beta, *, cu_seqlens=None, chunk_indices=None,
 def npu_chunk_scaled_dot_kkt_inverse(k, g, beta, *, cu_seqlens=None, chunk_indices=None, chunk_size=64):
     """``solve_tri(chunk_scaled_dot_kkt(k, g, beta), output_dtype=k.dtype)`` in one launch (no reference counterpart;
     the backward's recompute calls it).  Returns (I + A)^-1 as [B,Hv,T,64] in k's dtype; 64-token chunks only."""
-    k_contig, g_contig, beta_contig = k.contiguous(), g.contiguous(), beta.contiguous()
+    k_contig, g_contig, beta_contig = k, g, beta   # the library takes the outer strides of all three: no copies
     B, _, T, _ = _shape(k_contig)
     _, Hv, _ = _shape(g_contig)
     out = _empty((B, Hv, T, int(chunk_size)), k_contig)
@@ -923,7 +936,7 @@ def npu_chunk_bwd_dv_local(q, k, d_o, g, scale, chunk_size, *, g_gamma=None, A=N
     """_aclnn_ctypes.py:397-427.  q, k [B,Hk,T,K]; d_o [B,Hv,T,V]; g [B,Hv,T] chunk-cumsummed."""
     if g_gamma is not None:
         raise NotImplementedError("npu_chunk_bwd_dv_local: g_gamma is not supported.")
-    out = _empty_like(d_o)
+    out = _empty_ordered_like(d_o)
     return _call_op(
         "chunk_bwd_dv_local", OP_ARGTYPES["chunk_bwd_dv_local"],
         lambda ctx: [
@@ -970,8 +983,8 @@ def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu
         _, dv2, db2, _ = npu_prepare_wy_repr_bwd_full(k, v[..., 128:], beta.float(), A, torch.zeros_like(dA),
                                                       torch.zeros_like(dw), du[..., 128:], g.float(), chunk_size, **kw)
         return dk, torch.cat([dv1, dv2], dim=-1), _as_dtype(db1 + db2, beta), _as_dtype(dg, g)
-    dk = _empty_like(k)
-    dv = _empty_like(v)
+    dk = _empty_ordered_like(k)
+    dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dg = _f32_like(g)
     outputs = (dk, dv, dbeta, dg)
@@ -994,7 +1007,7 @@ def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, ch
     """npu_prepare_wy_repr_bwd_full with its key and gate gradients ADDED to ``dk`` ([B,Hk,T,K], dtype of k) and
     ``dg`` ([B,Hv,T] f32) in place: the reference's composition adds them with a separate pass
     (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32)."""
-    dv = _empty_like(v)
+    dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dv, dbeta = _call_op(
         "prepare_wy_repr_bwd_full_accumulate", OP_ARGTYPES["prepare_wy_repr_bwd_full_accumulate"],
@@ -1017,8 +1030,8 @@ def npu_prepare_wy_repr_bwd(k, v, beta, A, dw, du, g, chunk_size, *, cu_seqlens=
         kw = dict(cu_seqlens=cu_seqlens, chunk_indices=chunk_indices)
         dA = npu_prepare_wy_repr_bwd_da(k, v, beta, A, dw, du, g, chunk_size=chunk_size, **kw)
         return npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, **kw)
-    dk = _empty_like(k)
-    dv = _empty_like(v)
+    dk = _empty_ordered_like(k)
+    dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dg = _f32_like(g)
     outputs = (dk, dv, dbeta, dg)
@@ -1049,8 +1062,8 @@ def npu_chunk_bwd_dqkwg(q, k, v, g, h, dox, dh, dv, chunk_size, *, cu_seqlens=No
         return _add_as(dq1, dq2, q), _add_as(dk1, dk2, k), _add_as(dw1, dw2, q), _as_dtype(dg1 + dg2, g)
     q_shape = _shape(q)
     value_num_heads = int(v.shape[1])
-    dq = _empty_like(q)
-    dk = _empty_like(k)
+    dq = _empty_ordered_like(q)
+    dk = _empty_ordered_like(k)
     dw = _empty((q_shape[0], value_num_heads, q_shape[2], q_shape[3]), q)
     dg = _f32_like(g)
     outputs = (dq, dk, dw, dg)

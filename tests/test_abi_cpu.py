@@ -84,8 +84,12 @@ def capture_call(fn, *args, **kwargs):
         captured.update(name=name, argtypes=list(argtypes), args=build_args(ctx), names=ctx.names)
         return outputs
 
+    def fake_empty_ordered_like(like, *, dtype=None, shape=None):
+        return FakeTensor(like.shape if shape is None else shape, dtype or like.dtype)
+
     with mock.patch.object(H, "_empty", side_effect=fake_empty), \
             mock.patch.object(H, "_empty_like", side_effect=fake_empty_like), \
+            mock.patch.object(H, "_empty_ordered_like", side_effect=fake_empty_ordered_like), \
             mock.patch.object(H, "_call_op", side_effect=fake_call), \
             mock.patch.object(H, "_shape", side_effect=lambda t: tuple(t.shape)):
         out = fn(*args, **kwargs)
@@ -474,3 +478,19 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_outputs_follow_the_memory_order_of_their_inputs():
+    """dq, dk, dv of the GDN backward operators are allocated in the memory order of q, k, v: contiguous for the
+    reference's contiguous [B,H,T,D] operands, a token-major view for ``x.transpose(1, 2)`` of a [B,T,H,D] tensor, so
+    that the gradient passes back through the transpose without a copy."""
+    from fla_hip.ops import _hip_ctypes as H
+    x = torch.empty(2, 3, 5, 8)
+    y = H._empty_ordered_like(x)
+    assert y.shape == x.shape and y.is_contiguous()
+    xt = torch.empty(2, 5, 3, 8).transpose(1, 2)            # [B,H,T,D] view of token-major memory
+    yt = H._empty_ordered_like(xt, dtype=torch.float32)
+    assert yt.shape == xt.shape and yt.stride() == xt.stride() and yt.dtype == torch.float32
+    assert yt.transpose(1, 2).is_contiguous()
+    z = H._empty_ordered_like(xt, shape=(2, 3, 5, 16))
+    assert z.shape == (2, 3, 5, 16) and z.transpose(1, 2).is_contiguous()

@@ -296,6 +296,30 @@ def test_autograd_through_flash_gated_delta_rule(dev):
             assert st["rel_max"] <= TOL_BF16, f"d{name} with {kwargs}: {st}"
 
 
+def test_autograd_with_token_major_operands(dev):
+    """q, k, v as [B,H,T,D] views of token-major [B,T,H,D] tensors (what a model holds after its projections): the same
+    gradients as for head-major operands, returned in the memory order of the inputs (no layout copy on the way back)."""
+    from fla_hip import pipeline
+    B, T, H, K, V = 2, 200, 2, 128, 128
+    d = make(B, T, H, H, K, V, None, seed=5)
+    x = to_dev(d, dev)
+    g = x["g"].transpose(1, 2).contiguous()
+    beta = x["beta"].transpose(1, 2).contiguous()
+    grads = []
+    for token_major in (False, True):
+        leaves = []
+        for n in ("q", "k", "v"):
+            t = x[n].transpose(1, 2).contiguous().transpose(1, 2) if token_major else x[n].clone()
+            leaves.append(t.detach().requires_grad_(True))
+        o, _ = pipeline.flash_gated_delta_rule(*leaves, g, beta, None, None, True)
+        (o.float() * x["do"].transpose(1, 2).float()).sum().backward()
+        for t in leaves:
+            assert t.grad.stride() == t.stride()
+        grads.append([t.grad for t in leaves])
+    for a, b_ in zip(*grads):
+        assert torch.equal(a, b_)
+
+
 @pytest.mark.parametrize("D", [64, 128, 256])
 def test_l2norm_kernels_against_oracle(dev, D):
     """Forward and backward of the q/k normalisation on contiguous and on transposed (strided) views."""
