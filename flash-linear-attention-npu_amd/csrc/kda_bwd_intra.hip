@@ -45,6 +45,7 @@ struct BwdIntraParams {
     const float *daqk, *dakk;    // [..,64]
     int64_t m_sb, m_sh, m_st;
     int cumsum_dg;               // 1: dg leaves as its reverse running sum over the tokens of the chunk
+    int out16;                   // 1: dq_o and dk_o point at 16-bit elements (same strides in elements)
 };
 
 template <int KC>
@@ -235,7 +236,9 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
                 const int r = idx / (KC / 4), c4 = (idx % (KC / 4)) * 4;
                 if (r < len) {
                     const int64_t off = base + (int64_t)r * p.st + ch0 + c4;
-                    *reinterpret_cast<f32x4 *>(gout[t] + off) = old[t][m] + *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
+                    const f32x4 sum = old[t][m] + *reinterpret_cast<const f32x4 *>(xS + r * px + c4);
+                    if (t < 2 && p.out16) *reinterpret_cast<elemx4 *>(reinterpret_cast<elem *>(gout[t]) + off) = cvt4(sum);
+                    else *reinterpret_cast<f32x4 *>(gout[t] + off) = sum;
                 }
             }
         }
@@ -296,9 +299,13 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
                inner_unit(t) && (ib < 0 || t->stride[ib] % al == 0) && t->stride[ih] % al == 0 && t->stride[it] % al == 0 &&
                t->stride[it] >= 0 && reinterpret_cast<uintptr_t>(t->data) % 16 == 0;
     };
+    // The library-only form that also sums dg may hand dq_out and dk_out over in the element type of q: they are final
+    // with this stage, and the conversion that follows in a training step would read and write them once more.
+    const bool out16 = cumsum_dg && dq_o != nullptr && dk_o != nullptr && dq_o->dtype == kElemDtype && dk_o->dtype == kElemDtype;
     for (int i = 0; i < 6; ++i) {
-        if ((rc = check_tensor(grads[i], op, gradn[i], rank, dt_bit(FLA_F32)))) return rc;
-        FLA_REQUIRE(strided_ok(grads[i], H, 4), FLA_ERR_SHAPE,
+        const bool narrow = out16 && (i == 3 || i == 4);
+        if ((rc = check_tensor(grads[i], op, gradn[i], rank, dt_bit(narrow ? kElemDtype : FLA_F32)))) return rc;
+        FLA_REQUIRE(strided_ok(grads[i], H, narrow ? 8 : 4), FLA_ERR_SHAPE,
                     "%s: %s must have the shape of gk, a unit innermost stride and 16-byte aligned rows.", op, gradn[i]);
         FLA_REQUIRE((ib < 0 || grads[i]->stride[ib] == dq->stride[ib]) && grads[i]->stride[ih] == dq->stride[ih] &&
                         grads[i]->stride[it] == dq->stride[it],
@@ -403,6 +410,7 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.m_st = daqk->stride[it];
     FLA_REQUIRE(p.q_st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride of q and k must be below 2^24 elements.", op);
     p.cumsum_dg = cumsum_dg ? 1 : 0;
+    p.out16 = out16 ? 1 : 0;
     return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }
 

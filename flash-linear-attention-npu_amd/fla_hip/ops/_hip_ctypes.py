@@ -870,16 +870,17 @@ def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, dk, dg, chunk_size=64, *, cu_s
 
 
 def chunk_kda_bwd_intra_inplace(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, cu_seqlens=None, chunk_size=64,
-                                cumsum_dg=False):
+                                cumsum_dg=False, dq_out=None, dk_out=None):
     """``npu_chunk_kda_bwd_intra`` on [B,H,T,*] index-order views with the results written over ``dq, dk, db, dg``.
     The library accepts strided views, grouped heads (q, k with fewer heads than gk) and outputs that alias their
     inputs; the public operator keeps the reference's contiguous, allocate-new contract.  ``cumsum_dg``: dg leaves as
-    its reverse chunk-local running sum, the pass that follows this operator in the KDA backward."""
+    its reverse chunk-local running sum, the pass that follows this operator in the KDA backward; with it, ``dq_out`` /
+    ``dk_out`` may be tensors of q's dtype (same memory order as dq, dk) that take the final dq, dk instead."""
     cu = _as_int_tuple(cu_seqlens)
     indices = None if cu is None else _build_chunk_indices(cu, int(chunk_size))
     ins = (q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg)
     names = ("q", "k", "gk", "beta", "dAqk", "dAkk", "dq", "dk", "db", "dg")
-    outs = (dq, dk, db, dg)
+    outs = (dq if dq_out is None else dq_out, dk if dk_out is None else dk_out, db, dg)
     name = "chunk_kda_bwd_intra_cumsum" if cumsum_dg else "chunk_kda_bwd_intra"
     _call_op(
         name, OP_ARGTYPES[name],

@@ -295,13 +295,19 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
                                               layout_like=layout_like, **kw)
     dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
     # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
-    _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size,
-                                     cumsum_dg=True)
-    if Hv != Hk:          # value heads that share a key head add their gradients
-        dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2)
-        dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2)
     back = lambda t: _from_index_order(t, layout)
-    return (back(dq).to(q.dtype), back(dk).to(k.dtype), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
+    if Hv == Hk:          # dq, dk are final with the last stage: it writes them in the dtype of q and k
+        dq16 = _raw._empty_strided_like(dq.shape, dq, q.dtype)
+        dk16 = _raw._empty_strided_like(dk.shape, dk, k.dtype)
+        _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size,
+                                         cumsum_dg=True, dq_out=dq16, dk_out=dk16)
+        dq, dk = dq16, dk16
+    else:                 # value heads that share a key head add their gradients
+        _raw.chunk_kda_bwd_intra_inplace(qh, kh, gk4, bh, dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, chunk_size=chunk_size,
+                                         cumsum_dg=True)
+        dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2).to(q.dtype)
+        dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2).to(k.dtype)
+    return (back(dq), back(dk), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
 
 
 def _empty_in_layout(layout, index_shape):

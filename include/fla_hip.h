@@ -401,7 +401,9 @@ int fla_chunk_kda_bwd_intra(
 /* chunk_kda_bwd_intra followed by the reverse chunk-local running sum of dg_out.  No counterpart in the reference, whose
  * composition (and this build's, fla_hip.pipeline.chunk_kda_bwd) runs chunk_local_cumsum(reverse) over the gate gradient
  * right after this operator: here the workgroup that holds a chunk of dg takes the sum before it stores it.  Same
- * operands and rules as fla_chunk_kda_bwd_intra. */
+ * operands and rules as fla_chunk_kda_bwd_intra, except that dq_out and dk_out (both or neither) may be tensors of q's
+ * element type with the strides of dq: dq and dk are final with this stage, and a training step would otherwise
+ * convert them in a pass of its own. */
 int fla_chunk_kda_bwd_intra_cumsum_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *gk, const fla_tensor *beta,
     const fla_tensor *dAqk, const fla_tensor *dAkk, const fla_tensor *dq, const fla_tensor *dk,

@@ -294,6 +294,12 @@ def test_chunk_kda_bwd_intra_with_the_reverse_running_sum(dev, case):
     again = [t.clone() for t in xd]
     raw.chunk_kda_bwd_intra_inplace(*again, cu_seqlens=cu, cumsum_dg=True)
     assert torch.equal(again[9], fused[9])
+    # dq and dk handed over in the 16-bit type of q: the fp32 results rounded once
+    narrow = [t.clone() for t in xd]
+    dq16, dk16 = torch.empty_like(narrow[6], dtype=BF), torch.empty_like(narrow[7], dtype=BF)
+    raw.chunk_kda_bwd_intra_inplace(*narrow, cu_seqlens=cu, cumsum_dg=True, dq_out=dq16, dk_out=dk16)
+    assert torch.equal(dq16, fused[6].to(BF)) and torch.equal(dk16, fused[7].to(BF))
+    assert torch.equal(narrow[9], fused[9]) and torch.equal(narrow[8], fused[8])
 
 
 def test_chunk_kda_bwd_intra_errors(dev):
