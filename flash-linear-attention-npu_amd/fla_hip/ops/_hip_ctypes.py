@@ -20,7 +20,7 @@ _empty = _runtime.empty
 _empty_like = _runtime.empty_like
 
 
-def _empty_ordered_like(like, *, dtype=None, shape=None):
+def _empty_ordered_like(like, *, dtype=None, shape=None, device=None):
     """An uninitialised tensor of ``shape`` (default: that of ``like``) whose dimensions sit in memory in the order of
     ``like``'s.  For a contiguous ``like`` this is a contiguous tensor, as the reference's operators return; for a
     token-major view [B,H,T,D] (what a caller holds after ``x.transpose(1, 2)``) the result is such a view too, so that
@@ -29,8 +29,10 @@ def _empty_ordered_like(like, *, dtype=None, shape=None):
 
     shape = tuple(like.shape) if shape is None else tuple(int(d) for d in shape)
     order = sorted(range(len(shape)), key=lambda d: (-like.stride(d), d))
-    base = torch.empty([shape[d] for d in order], dtype=dtype or like.dtype, device=like.device)
+    base = torch.empty([shape[d] for d in order], dtype=dtype or like.dtype, device=like.device if device is None else device)
     return base.permute([order.index(d) for d in range(len(shape))])
+
+
 _shape = _runtime.shape
 
 _T, _IA = TENSOR_P, INT_ARRAY_P
@@ -1241,9 +1243,10 @@ def l2norm_fwd(x, eps: float = 1e-6, output_dtype=None):
     return y, rstd
 
 
-def l2norm_bwd(y, rstd, dy, eps: float = 1e-6):
-    """fla/ops/triton/triton_core/l2norm.py:181-224: dx from the normalised output, its rstd and dy."""
-    dx = _empty_like(y)
+def l2norm_bwd(y, rstd, dy, eps: float = 1e-6, *, like=None):
+    """fla/ops/triton/triton_core/l2norm.py:181-224: dx from the normalised output, its rstd and dy.  ``like``: a tensor
+    (it may be storage-less) whose memory order dx takes, e.g. the input the forward normalised; default: contiguous."""
+    dx = _empty_like(y) if like is None else _empty_ordered_like(like, dtype=y.dtype, shape=tuple(y.shape), device=y.device)
     return _call_op("l2norm_bwd", OP_ARGTYPES["l2norm_bwd"],
                     lambda ctx: [ctx.tensor(y, "y"), ctx.tensor(rstd.contiguous(), "rstd"), ctx.tensor(dy, "dy"),
                                  ctypes.c_double(float(eps)), ctx.tensor(dx, "dx")],

@@ -136,6 +136,8 @@ def _autograd_function():
         @staticmethod
         def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm):
             q_rstd = k_rstd = None
+            # the memory order of the caller's q and k: their gradients go back in it, whatever the kernels worked on
+            ctx.qk_like = tuple(torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device="meta") for t in (q, k))
             if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049
                 q, q_rstd = _raw.l2norm_fwd(q)
                 k, k_rstd = _raw.l2norm_fwd(k)
@@ -155,8 +157,8 @@ def _autograd_function():
                 None if dht is None else dht.contiguous(), ctx.cu, ctx.chunk_size,
                 saved=dict(h=h, v_new=v_new, w=w))
             if q_rstd is not None:      # :1104-1106
-                dq = _raw.l2norm_bwd(q, q_rstd, dq)
-                dk = _raw.l2norm_bwd(k, k_rstd, dk)
+                dq = _raw.l2norm_bwd(q, q_rstd, dq, like=ctx.qk_like[0])
+                dk = _raw.l2norm_bwd(k, k_rstd, dk, like=ctx.qk_like[1])
             return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None, None
 
     return ChunkGatedDeltaRuleFunction

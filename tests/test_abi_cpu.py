@@ -84,7 +84,7 @@ def capture_call(fn, *args, **kwargs):
         captured.update(name=name, argtypes=list(argtypes), args=build_args(ctx), names=ctx.names)
         return outputs
 
-    def fake_empty_ordered_like(like, *, dtype=None, shape=None):
+    def fake_empty_ordered_like(like, *, dtype=None, shape=None, device=None):
         return FakeTensor(like.shape if shape is None else shape, dtype or like.dtype)
 
     with mock.patch.object(H, "_empty", side_effect=fake_empty), \

@@ -305,19 +305,20 @@ def test_autograd_with_token_major_operands(dev):
     x = to_dev(d, dev)
     g = x["g"].transpose(1, 2).contiguous()
     beta = x["beta"].transpose(1, 2).contiguous()
-    grads = []
-    for token_major in (False, True):
-        leaves = []
-        for n in ("q", "k", "v"):
-            t = x[n].transpose(1, 2).contiguous().transpose(1, 2) if token_major else x[n].clone()
-            leaves.append(t.detach().requires_grad_(True))
-        o, _ = pipeline.flash_gated_delta_rule(*leaves, g, beta, None, None, True)
-        (o.float() * x["do"].transpose(1, 2).float()).sum().backward()
-        for t in leaves:
-            assert t.grad.stride() == t.stride()
-        grads.append([t.grad for t in leaves])
-    for a, b_ in zip(*grads):
-        assert torch.equal(a, b_)
+    for l2norm in (False, True):
+        grads = []
+        for token_major in (False, True):
+            leaves = []
+            for n in ("q", "k", "v"):
+                t = x[n].transpose(1, 2).contiguous().transpose(1, 2) if token_major else x[n].clone()
+                leaves.append(t.detach().requires_grad_(True))
+            o, _ = pipeline.flash_gated_delta_rule(*leaves, g, beta, None, None, True, use_qk_l2norm_in_kernel=l2norm)
+            (o.float() * x["do"].transpose(1, 2).float()).sum().backward()
+            for t in leaves:
+                assert t.grad.stride() == t.stride()
+            grads.append([t.grad for t in leaves])
+        for a, b_ in zip(*grads):
+            assert torch.equal(a, b_)
 
 
 @pytest.mark.parametrize("D", [64, 128, 256])
