@@ -56,6 +56,7 @@ OP_ARGTYPES = {
     "kda_gate_cumsum": [_T, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool, ctypes.c_double, _T],
     "chunk_kda_fwd": [_T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_char_p, ctypes.c_double, ctypes.c_int64,
                       ctypes.c_bool, ctypes.c_double, ctypes.c_bool, ctypes.c_bool] + [_T] * 11,
+    "kda_gate_bwd": [_T, _T, _T, _T, ctypes.c_char_p, ctypes.c_bool, ctypes.c_double, _T, _T, _T],
     "chunk_kda_bwd_intra": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_kda_bwd_intra_cumsum": [_T] * 10 + [_IA, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_char_p] + [_T] * 4,
     "chunk_gated_delta_rule_bwd_dhu": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64,
@@ -895,6 +896,32 @@ def chunk_kda_bwd_intra_inplace(q, k, gk, beta, dAqk, dAkk, dq, dk, db, dg, *, c
         outs,
     )
     return outs
+
+
+def kda_gate_bwd(g, dgate, A_log, dt_bias=None, *, layout="BSND", safe_gate=False, lower_bound=-5.0):
+    """Gradient of the in-kernel KDA gate activation (fla/ops/ascendc/kda/chunk_kda_fwd/docs/api.md:103-113):
+    ``(dg_raw, dA_log, ddt_bias)`` from the raw gate ``g`` and the gradient ``dgate`` (f32, shape of g) of the activated
+    gate; dg_raw has the dtype and memory order of g, dA_log is f32 [HV], ddt_bias f32 [HV*K] or None."""
+    import torch
+
+    head_axis = {"BSND": 2, "BNSD": 1, "TND": 1, "NTD": 0}[layout]
+    token_axis = {"BSND": 1, "BNSD": 2, "TND": 0, "NTD": 1}[layout]
+    HV, K, T = int(g.shape[head_axis]), int(g.shape[-1]), int(g.shape[token_axis])
+    B = int(g.shape[0]) if g.dim() == 4 else 1
+    parts = B * ((T + 255) // 256)
+    dg_raw = _empty_ordered_like(g)
+    da_part = _empty((parts, HV), g, dtype=torch.float32)
+    db_part = None if dt_bias is None else _empty((parts, HV, K), g, dtype=torch.float32)
+    _call_op(
+        "kda_gate_bwd", OP_ARGTYPES["kda_gate_bwd"],
+        lambda ctx: [
+            ctx.tensor(g, "g"), ctx.tensor(dgate, "dgate"), ctx.tensor(A_log, "A_log"), ctx.tensor(dt_bias, "dt_bias"),
+            ctypes.c_char_p(layout.encode("utf-8")), ctypes.c_bool(bool(safe_gate)), ctypes.c_double(float(lower_bound)),
+            ctx.tensor(dg_raw, "dg_raw"), ctx.tensor(db_part, "ddt_bias_partial"), ctx.tensor(da_part, "dA_log_partial"),
+        ],
+        (dg_raw, da_part),
+    )
+    return dg_raw, da_part.sum(0), (None if db_part is None else db_part.sum(0).reshape(HV * K))
 
 
 def chunk_local_cumsum_into(g, out, chunk_size, *, cu_seqlens=None, reverse=False, scale=1.0):

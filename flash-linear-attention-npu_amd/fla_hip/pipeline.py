@@ -329,24 +329,36 @@ def _kda_autograd_function():
     import torch
 
     class ChunkKdaFunction(torch.autograd.Function):
+        # ``gate``: None (g is the log decay itself) or (A_log, dt_bias, safe_gate, lower_bound): g is the raw gate, the
+        # forward kernel activates it, and the backward ends with the gradient of that activation (kda_gate_bwd).
         @staticmethod
-        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, layout, chunk_size):
+        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, layout, chunk_size, A_log=None,
+                    dt_bias=None, safe_gate=False, lower_bound=-5.0):
+            in_kernel = A_log is not None
             out = _ops.chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size, layout=layout, initial_state=initial_state,
                                      output_final_state=output_final_state, cu_seqlens=cu, disable_recompute=True,
-                                     return_intermediate_states=True)
+                                     return_intermediate_states=True, use_gate_in_kernel=in_kernel, A_log=A_log,
+                                     dt_bias=dt_bias, safe_gate=safe_gate, lower_bound=lower_bound)
             o, final, gk, Aqk, Akk, w, _u, qg, kg, v_new, h, _ = out
-            ctx.save_for_backward(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state)
+            ctx.save_for_backward(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state,
+                                  *((g, A_log, dt_bias) if in_kernel else ()))
             ctx.scale, ctx.cu, ctx.layout, ctx.chunk_size, ctx.g_dtype = scale, cu, layout, chunk_size, g.dtype
+            ctx.gate = (safe_gate, lower_bound) if in_kernel else None
             return o, final
 
         @staticmethod
         def backward(ctx, do, dht):
-            q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state = ctx.saved_tensors
+            q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state = ctx.saved_tensors[:13]
             dht = None if dht is None else dht.contiguous()   # a view when the caller sliced or joined the final state
             dq, dk, dv, dg, db, dh0 = chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, ctx.scale, do, dht,
                                                     initial_state=initial_state, layout=ctx.layout, cu_seqlens=ctx.cu,
                                                     chunk_size=ctx.chunk_size)
-            return dq, dk, dv, dg.to(ctx.g_dtype), db, None, dh0, None, None, None, None
+            if ctx.gate is None:
+                return dq, dk, dv, dg.to(ctx.g_dtype), db, None, dh0, None, None, None, None, None, None, None, None
+            g, A_log, dt_bias = ctx.saved_tensors[13:]
+            dg_raw, dA, dbias = _raw.kda_gate_bwd(g, dg, A_log, dt_bias, layout=ctx.layout, safe_gate=ctx.gate[0],
+                                                  lower_bound=ctx.gate[1])
+            return dq, dk, dv, dg_raw, db, None, dh0, None, None, None, None, dA, dbias, None, None
 
     return ChunkKdaFunction
 
@@ -377,9 +389,10 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     """KDA chunk attention, differentiable: ``(o, final_state)`` with q, k [..H,K], v [..HV,V], per-channel log decay
     g [..HV,K] (natural log, one value per token and channel), beta [..HV] in ``layout``; states fp32 [N,HV,K,V].
     The forward is ``chunk_kda_fwd``; when an input requires grad the forward keeps its intermediates and
-    ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0.  With ``use_gate_in_kernel`` g is the raw gate input: without
-    gradients the forward kernel activates it; with gradients the activation runs as tensor operations ahead of the
-    kernels, so that autograd also reaches ``A_log`` and ``dt_bias``.  Gradients cover every admitted head size with
+    ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0.  With ``use_gate_in_kernel`` g is the raw gate input and the
+    forward kernel activates it; with gradients ``kda_gate_bwd`` ends the backward, so that autograd also reaches
+    ``A_log`` and ``dt_bias`` (for a head size served by padding or by two value passes the activation runs as tensor
+    operations ahead of the kernels instead).  Gradients cover every admitted head size with
     K <= 128 (V up to 256 as two passes over 128 value columns) and run on 64-token tiles whatever ``chunk_size``."""
     import torch
 
@@ -398,11 +411,17 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     # The chunk size tiles the same function.  The gradient kernels are built for 64-token tiles, as the reference's own
     # backward kernel is (npu_chunk_kda_bwd_intra, _aclnn_ctypes.py:1582-1584), so a differentiated call runs on them.
     chunk_size = 64
+    K, V = q.shape[-1], v.shape[-1]
+    gate_args = ()
     if use_gate_in_kernel:
         if A_log is None:
             raise RuntimeError("chunk_kda: A_log must be float32 [HV] when use_gate_in_kernel=True.")
-        g = _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound)
-    K, V = q.shape[-1], v.shape[-1]
+        if (K, V) in ((64, 64), (64, 128), (128, 128)) and A_log.dtype == torch.float32 and \
+                (dt_bias is None or dt_bias.dtype == torch.float32):
+            # a built head size: the forward kernel activates the gate, kda_gate_bwd differentiates the activation
+            gate_args = (A_log, dt_bias, bool(safe_gate), lower_bound)
+        else:   # the activation as tensor operations ahead of the padding and the split below
+            g = _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound)
     if K > 128:
         raise NotImplementedError(f"chunk_kda: gradients are built for K <= 128, got K={K}.")
     if V > 128:
@@ -432,4 +451,5 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
                                        F.pad(g, (0, Kp - K)), beta, float(scale), h0, output_final_state, cu, layout,
                                        chunk_size)
         return o[..., :V], (None if final is None else final[..., :K, :V])
-    return _KDA_FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, layout, chunk_size)
+    return _KDA_FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, layout, chunk_size,
+                               *gate_args)

@@ -290,6 +290,24 @@ int fla_kda_gate_cumsum(
     bool safe_gate, double lower_bound, const fla_tensor *gk, void *workspace,
     uint64_t workspace_size, void *stream);
 
+/* kda_gate_bwd - gradient of the gate activation that chunk_kda_fwd / kda_gate_cumsum apply with use_gate_in_kernel.
+ * No counterpart among the reference's kernels (its KDA backward is a third-party Triton package,
+ * adapters/triton_ascend_kda.py:141-242); fla_hip.pipeline.chunk_kda uses it so that a training step with the gate in
+ * the kernel needs no tensor-operation copy of the activation.  g: the raw gate, f32 or bf16, in `layout`
+ * ("BSND", "BNSD", "TND", "NTD"; any outer strides); dgate: f32, gradient of the activated gate, same shape;
+ * A_log f32 [Hv]; dt_bias f32 [Hv*K] or NULL.  Outputs: dg_raw (dtype and shape of g); partial sums over tiles of 256
+ * tokens, contiguous f32: ddt_bias_partial [B*ceil(T/256), Hv, K] (NULL without dt_bias) and dA_log_partial
+ * [B*ceil(T/256), Hv] - the caller adds them over the first dimension.  K in {32, 64, 128, 256}. */
+int fla_kda_gate_bwd_get_workspace_size(
+    const fla_tensor *g, const fla_tensor *dgate, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const char *layout, bool safe_gate, double lower_bound, const fla_tensor *dg_raw,
+    const fla_tensor *ddt_bias_partial, const fla_tensor *dA_log_partial, uint64_t *workspace_size);
+int fla_kda_gate_bwd(
+    const fla_tensor *g, const fla_tensor *dgate, const fla_tensor *A_log, const fla_tensor *dt_bias,
+    const char *layout, bool safe_gate, double lower_bound, const fla_tensor *dg_raw,
+    const fla_tensor *ddt_bias_partial, const fla_tensor *dA_log_partial, void *workspace,
+    uint64_t workspace_size, void *stream);
+
 /* ------------------------------------------------------------------------
  * chunk_gated_delta_rule_bwd_dhu - replaces aclnnChunkGatedDeltaRuleBwdDhu
  * (_aclnn_ctypes.py:324-394; chunk_gated_delta_rule_bwd_dhu/README.md:6-13).

@@ -274,13 +274,16 @@ def test_chunk_kda_backward_at_the_bench_shape(dev):
 
 
 @pytest.mark.parametrize("safe", [False, True])
-@pytest.mark.parametrize("layout", ["BSND", "NTD"])
-def test_chunk_kda_gradients_through_the_gate_activation(dev, safe, layout):
+@pytest.mark.parametrize("layout,K,V,with_bias", [("BSND", 128, 128, True), ("NTD", 128, 128, True), ("BNSD", 64, 128, False),
+                                                  ("BSND", 96, 80, True)],
+                         ids=["BSND", "NTD", "BNSD-64x128-nobias", "BSND-96x80-padded"])
+def test_chunk_kda_gradients_through_the_gate_activation(dev, safe, layout, K, V, with_bias):
     """use_gate_in_kernel with gradients: the raw gate, A_log and dt_bias against fp64 autograd through the activation
     (chunk_kda_fwd/docs/api.md:103-113) and the per-token recurrence; without gradients the forward kernel's own
-    activation gives the same o and final state."""
+    activation gives the same o and final state.  Built head sizes activate in the forward kernel and end the backward
+    with kda_gate_bwd; a padded one runs the activation as tensor operations."""
     from fla_hip import pipeline
-    B, T, Hk, Hv, K, V = 1, 150, 1, 2, 128, 128
+    B, T, Hk, Hv = 1, 150, 1, 2
     gen = torch.Generator().manual_seed(7 + safe)
     q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
     k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
@@ -289,27 +292,31 @@ def test_chunk_kda_gradients_through_the_gate_activation(dev, safe, layout):
     beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
     do = torch.randn(B, Hv, T, V, generator=gen).to(BF)
     A_log = torch.randn(Hv, generator=gen) * 0.3 - 1.5
-    dt_bias = torch.randn(Hv * K, generator=gen) * 0.3
+    dt_bias = torch.randn(Hv * K, generator=gen) * 0.3 if with_bias else None
     scale, lb = K ** -0.5, -4.0
     kw = dict(use_gate_in_kernel=True, safe_gate=safe, lower_bound=lb)
 
     ins = [lay(t, layout).to(dev).requires_grad_(True) for t in (q, k, v, raw, beta)]
-    A_d, b_d = A_log.to(dev).requires_grad_(True), dt_bias.to(dev).requires_grad_(True)
+    A_d = A_log.to(dev).requires_grad_(True)
+    b_d = None if dt_bias is None else dt_bias.to(dev).requires_grad_(True)
     o, final = pipeline.chunk_kda(*ins, scale, None, True, layout=layout, A_log=A_d, dt_bias=b_d, **kw)
     (o.float() * lay(do, layout).to(dev).float()).sum().backward()
     with torch.no_grad():
         o2, final2 = pipeline.chunk_kda(*[t.detach() for t in ins], scale, None, True, layout=layout, A_log=A_d.detach(),
-                                        dt_bias=b_d.detach(), **kw)
+                                        dt_bias=None if b_d is None else b_d.detach(), **kw)
     close(o2, o.detach().float(), "o: kernel activation vs tensor-operation activation", rel=1e-2)
     close(final2, final.detach(), "final state: kernel activation vs tensor-operation activation", rel=1e-2)
 
     dd = torch.float64
-    leaves = [t.to(dd).requires_grad_(True) for t in (q, k, v, raw, beta, A_log, dt_bias)]
-    gate = kda.kda_gate(leaves[3], A_log=leaves[5], dt_bias=leaves[6], use_gate_in_kernel=True, safe_gate=safe, lower_bound=lb)
+    leaves = [t.to(dd).requires_grad_(True) for t in (q, k, v, raw, beta, A_log)]
+    if with_bias:
+        leaves.append(dt_bias.to(dd).requires_grad_(True))
+    gate = kda.kda_gate(leaves[3], A_log=leaves[5], dt_bias=leaves[6] if with_bias else None, use_gate_in_kernel=True,
+                        safe_gate=safe, lower_bound=lb)
     o_ref, _ = kda.naive_recurrent_kda(leaves[0], leaves[1], leaves[2], gate, leaves[4], scale, output_final_state=True,
                                        compute_dtype=dd)
     (o_ref * do.to(dd)).sum().backward()
-    got = [unlay(t.grad, layout) for t in ins] + [A_d.grad, b_d.grad]
+    got = [unlay(t.grad, layout) for t in ins] + [A_d.grad] + ([b_d.grad] if with_bias else [])
     for name, a, e in zip(("dq", "dk", "dv", "dg_raw", "dbeta", "dA_log", "ddt_bias"), got, [t.grad for t in leaves]):
         close(a, e, name)
 
