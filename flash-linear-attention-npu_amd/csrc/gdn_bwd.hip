@@ -49,8 +49,9 @@ __global__ void __launch_bounds__(kThreads) dv_local_kernel(const DvLocalParams 
     float *gS = reinterpret_cast<float *>(aS + kChunk * pa);   // gates of the rows
     float *cS = gS + kChunk;                                   // gates of the columns of the current tile
 
-    const int c = C128 ? blockIdx.x >> 1 : blockIdx.x, half = C128 ? blockIdx.x & 1 : 0;
-    const int hv = blockIdx.y, b = blockIdx.z;
+    int cx, hv;
+    block_chunk_head(p.geom, cx, hv);
+    const int c = C128 ? cx >> 1 : cx, half = C128 ? cx & 1 : 0, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, cstart, clen;
     chunk_span(p.geom, b, c, seq, cstart, clen);
@@ -168,7 +169,9 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
     float *goS = dgp + 2 * kChunk;     // gates of the other half (CH = 2)
     float *ksS = goS + kChunk;         // [kMaxRep] sum_t k_t . dk_state_t of the first half, per value head (CH = 2)
 
-    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    int c, hk;
+    block_chunk_head(p.geom, c, hk);
+    const int b = blockIdx.z;
     const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
     int seq, cstart, clen;
     chunk_span(p.geom, b, c, seq, cstart, clen);
@@ -486,7 +489,9 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
     float *bS = gS + kChunk;
     float *fS = bS + kChunk;           // beta e^G
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -594,7 +599,9 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     float *gS = reinterpret_cast<float *>(dbS + kChunk * pa);
     float *bS = gS + kChunk;
 
-    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    int c, hk;
+    block_chunk_head(p.geom, c, hk);
+    const int b = blockIdx.z;
     const int rep = GVA ? p.geom.Hv / p.geom.Hk : 1;   // without grouping the head loop is a single pass
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -771,7 +778,9 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da128_kernel(const WyBwdParam
     float *bS = gS + C;
     float *fS = bS + C;                              // beta e^G
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -881,7 +890,9 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_full128_kernel(const WyBwdPar
     float *gS = reinterpret_cast<float *>(vS + kChunk * pvv);
     float *bS = gS + C;
 
-    const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    int c, hk;
+    block_chunk_head(p.geom, c, hk);
+    const int b = blockIdx.z;
     const int rep = p.geom.Hv / p.geom.Hk;
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -1036,7 +1047,7 @@ int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     DvLocalParams p{geom, view4(q), view4(k), view4(d_o), view4(out), view3(g), (float)scale};
     const bool c128 = geom.C == 128;
-    const dim3 grid(geom.NT * (c128 ? 2 : 1), geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT * (c128 ? 2 : 1), geom.Hv);
     const int K = geom.K, V = geom.V;
     const size_t smem = ((size_t)kChunk * (2 * (K + 8) + (V + 16) + kChunk + 8)) * 2 + 2 * kChunk * 4;
 #define FLA_DV_LOCAL(KK, VV)                                                                                \
@@ -1087,7 +1098,8 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                   static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                   h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                   static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
-    const dim3 grid(geom.NT, geom.Hk, geom.B);
+    // token-major operands (the row of a token holds all heads): neighbouring workgroups take the heads of one chunk
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hk);
     const int K = geom.K, V = geom.V;
     const int VS = V == 256 ? 128 : V;   // value columns held in LDS at a time
     const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 +
@@ -1142,7 +1154,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), View4{}, View4{}, view3(g),
                   view3(beta), nullptr, nullptr, 0, 0, 0, 0, 0, 0};
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
     const int K = geom.K, V = geom.V;
     if (geom.C == 128) {
         const size_t smem128 = ((size_t)kChunk * (2 * (K + 8) + 2 * (V + 8)) + (size_t)2 * 128 * (128 + 8)) * 2 + 3 * 128 * 4;
@@ -1180,7 +1192,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), view4(dk), view4(dv), view3(g),
                   view3(beta), static_cast<float *>(dbeta->data), static_cast<float *>(dg->data),
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
-    const dim3 grid(geom.NT, geom.Hk, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hk);
     const int K = geom.K, V = geom.V;
     if (geom.C == 128) {
         FLA_REQUIRE(!accumulate, FLA_ERR_UNSUPPORTED, "%s: the accumulating form is built for chunk_size 64.", op);

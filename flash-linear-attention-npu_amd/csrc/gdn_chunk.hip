@@ -35,7 +35,9 @@ __global__ void __launch_bounds__(kThreads) kkt_kernel(const KktParams p) {
     float *gS = reinterpret_cast<float *>(kS + C * pitch);
     float *bS = gS + C;
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -285,7 +287,9 @@ __global__ void __launch_bounds__(kThreads) kkt_inverse_kernel(const KktParams p
     float *aS = reinterpret_cast<float *>(kS);
     elem *oS = reinterpret_cast<elem *>(aS + C * pa);
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -347,7 +351,9 @@ __global__ void __launch_bounds__(kThreads) wu_kernel_generic(const WuParams p) 
     float *gS = reinterpret_cast<float *>(vS + kChunk * pv);
     float *bS = gS + kChunk;
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -438,7 +444,9 @@ __global__ void __launch_bounds__(kThreads) wu_kernel(const WuParams p) {
     elem *kS = aS + C * pa;
     elem *vS = kS + C * pk;
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -553,7 +561,9 @@ __global__ void __launch_bounds__(V >= 128 ? 512 : 256) fwd_o_kernel(const FwdOP
     float *gS = reinterpret_cast<float *>(pS + kChunk * pp);   // gates of the row tile
     float *gC = gS + kChunk;                                   // gates of the current column block
 
-    const int c = blockIdx.x / SUB, r = blockIdx.x % SUB, hv = blockIdx.y, b = blockIdx.z;
+    int cx, hv;
+    block_chunk_head(p.geom, cx, hv);
+    const int c = cx / SUB, r = cx % SUB, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, cstart, clen;
     chunk_span(p.geom, b, c, seq, cstart, clen);
@@ -702,14 +712,14 @@ int kkt_impl(const fla_tensor *k, const fla_tensor *g, const fla_tensor *beta, c
         const size_t ismem = (tiles > rows ? tiles : rows) + 2 * kChunk * 4;
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kkt_inverse_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)ismem));
-        FLA_LAUNCH("kkt_inverse", stream, kkt_inverse_kernel, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), ismem, stream, p,
+        FLA_LAUNCH("kkt_inverse", stream, kkt_inverse_kernel, chunk_head_grid(geom, geom.NT, geom.Hv), dim3(kThreads), ismem, stream, p,
                    static_cast<elem *>(out->data));
     } else if (geom.C == 128) {
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kkt_kernel<128>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                           (int)smem));
-        FLA_LAUNCH("kkt", stream, kkt_kernel<128>, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+        FLA_LAUNCH("kkt", stream, kkt_kernel<128>, chunk_head_grid(geom, geom.NT, geom.Hv), dim3(kThreads), smem, stream, p);
     } else {
-        FLA_LAUNCH("kkt", stream, kkt_kernel<64>, dim3(geom.NT, geom.Hv, geom.B), dim3(kThreads), smem, stream, p);
+        FLA_LAUNCH("kkt", stream, kkt_kernel<64>, chunk_head_grid(geom, geom.NT, geom.Hv), dim3(kThreads), smem, stream, p);
     }
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
@@ -792,7 +802,7 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     WuParams p{geom, view4(k), view4(v), view4(A), view4(w), view4(u), view3(g), view3(beta)};
     const size_t smem = (size_t)geom.C * ((geom.C + 8) + (geom.K + 16) + (geom.V + 16)) * 2 + 2 * kChunk * 4;
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
 #define FLA_LAUNCH_WU(KERNEL)                                                                                      \
     do {                                                                                                           \
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -816,7 +826,7 @@ int launch_fwd_o(const FwdOParams &p, hipStream_t stream) {
     const size_t smem = ((size_t)2 * kChunk * (K + 8) + (size_t)(kChunk + K) * (V + 16) + kChunk * (kChunk + 8)) * 2 + 2 * kChunk * 4;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(fwd_o_kernel<K, V, SUB>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V, SUB>), dim3(p.geom.NT * SUB, p.geom.Hv, p.geom.B), dim3(V >= 128 ? 512 : 256),
+    FLA_LAUNCH("fwd_o", stream, (fwd_o_kernel<K, V, SUB>), chunk_head_grid(p.geom, p.geom.NT * SUB, p.geom.Hv), dim3(V >= 128 ? 512 : 256),
                smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;

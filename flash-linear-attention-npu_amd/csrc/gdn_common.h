@@ -24,7 +24,19 @@ struct ChunkGeom {
     const int32_t *choff;  // [N+1] first chunk of each sequence
     const int32_t *tab;  // [NT][2] (sequence, chunk within sequence)
     int C = kChunk;      // tokens per chunk (128 where an operator supports it)
+    int head_fast = 0;   // chunk-parallel launches: 1 = grid (heads, chunks, batch), neighbouring workgroups take the heads
+                         // of one chunk (token-major operands: those rows are neighbours in memory); 0 = (chunks, heads, batch)
 };
+
+// Chunk-parallel launches: the (x, head) pair of this workgroup, x = chunk index (times whatever the kernel packs into
+// it).  The grid is (x, heads, batch), or (heads, x, batch) when geom.head_fast is set.
+__device__ __forceinline__ void block_chunk_head(const ChunkGeom &g, int &x, int &head) {
+    x = g.head_fast ? blockIdx.y : blockIdx.x;
+    head = g.head_fast ? blockIdx.x : blockIdx.y;
+}
+inline dim3 chunk_head_grid(const ChunkGeom &g, int x, int heads) {
+    return g.head_fast ? dim3(heads, x, g.B) : dim3(x, heads, g.B);
+}
 
 // Head-first activations [B, H, T, D] with arbitrary outer strides and unit inner stride.
 struct View4 {

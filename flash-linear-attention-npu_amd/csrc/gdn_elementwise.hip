@@ -63,6 +63,10 @@ int gdn_geometry(const char *op, const fla_tensor *k, const fla_tensor *v_like, 
     geom.C = (int)chunk_size;
     geom.NT = (geom.T + geom.C - 1) / geom.C;
     geom.N = geom.B;
+    // token-major k (a token's row holds every head): chunk-parallel launches put the heads of a chunk next to each other.
+    // The chunk index then sits in a grid dimension limited to 65535, hence the bound on T (varlen adds a chunk per sequence
+    // at most, a kernel may pack two steps into the index).
+    geom.head_fast = geom.Hk > 1 && k->stride[2] > k->stride[1] && geom.T <= (1 << 20) ? 1 : 0;
     return FLA_OK;
 }
 

@@ -46,7 +46,9 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_dav_kernel(const DavParams p
     elem *vS = oS + kChunk * po;                    // v_new
     elem *aS = vS + kChunk * pv;                    // Aqk
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x, w = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
@@ -130,7 +132,9 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
                                                      (size_t)2 * kChunk * pq * 2 + (size_t)kChunk * pg * 4,
                   "the result tiles must fit the operand tiles");
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -289,7 +293,9 @@ __global__ void __launch_bounds__(kThreads, 2) kda_bwd_wy_kernel(const KdaWyPara
     elem *m4S = dwS;
     elem *m5S = duS;
 
-    const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -501,6 +507,8 @@ int dav_impl(const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *a
     ChunkGeom geom;
     int rc;
     if ((rc = gdn_geometry(op, v_new, nullptr, nullptr, chunk_size, geom, kElemDtype))) return rc;   // Hk=Hv, K=V here
+    // v_new and Aqk are head-major whatever the caller's layout; d_o and dAqk follow it and carry more bytes
+    geom.head_fast = d_o != nullptr && d_o->ndim == 4 && geom.Hv > 1 && d_o->stride[2] > d_o->stride[1] && geom.T <= (1 << 20) ? 1 : 0;
     const int bf = dt_bit(kElemDtype);
     const int64_t B = geom.B, H = geom.Hv, T = geom.T, V = geom.V;
     if ((rc = check_bhtd(op, "v_new", v_new, B, H, T, V, bf))) return rc;
@@ -512,7 +520,7 @@ int dav_impl(const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *a
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
     DavParams p{geom, view4(v_new), view4(d_o), view4(aqk), view4(dv), viewf(daqk), (float)scale};
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
     const size_t smem = ((size_t)kChunk * ((V + 16) + (V + 8) + (kChunk + 16))) * 2;
     if (V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dav_kernel<128>), "kda_bwd_dav", grid, smem, p, kThreads);
     if (V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dav_kernel<64>), "kda_bwd_dav", grid, smem, p, kThreads);
@@ -551,7 +559,7 @@ int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v
                      static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                      h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                      viewf(dq), viewf(dk), viewf(dg), (float)scale};
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
     const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
                         (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
     if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_kernel<128, 128>), "kda_bwd_dqkwg", grid, smem, p, kDqkwgThreads);
@@ -592,7 +600,7 @@ int kda_wy_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta
     KdaWyParams p{geom, view4(k), view4(v), view4(akk), view4(dw), view4(du), view4(dv), view3(beta),
                   static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
                   viewf(dk), viewf(dg), viewf(dakk), static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2]};
-    const dim3 grid(geom.NT, geom.Hv, geom.B);
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
     const size_t smem = ((size_t)kChunk * ((K + 16) + (V + 16) + (K + 8) + (V + 8) + (kChunk + 8))) * 2 + kChunk * 4;
     if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_wy_kernel<128, 128>), "kda_bwd_wy", grid, smem, p, kThreads);
     if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_wy_kernel<64, 64>), "kda_bwd_wy", grid, smem, p, kThreads);

@@ -59,7 +59,9 @@ __global__ void __launch_bounds__(kThreads) kda_bwd_intra_kernel(const BwdIntraP
     elem *qS = reinterpret_cast<elem *>(bS + kChunk);
     elem *kS = qS + kChunk * pk;
 
-    const int c = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    int c, h;
+    block_chunk_head(p.geom, c, h);
+    const int b = blockIdx.z;
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
     const int tid = threadIdx.x;
@@ -261,7 +263,7 @@ int launch_bwd_intra(const BwdIntraParams &p, hipStream_t stream) {
     const size_t smem = (size_t)kChunk * (2 * 68 + (KC + 4) + 1) * 4 + (size_t)2 * kChunk * (KC + 8) * 2;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_bwd_intra_kernel<KC>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_bwd_intra", stream, (kda_bwd_intra_kernel<KC>), dim3(p.geom.NT, p.geom.Hv, p.geom.B), dim3(kThreads), smem,
+    FLA_LAUNCH("kda_bwd_intra", stream, (kda_bwd_intra_kernel<KC>), chunk_head_grid(p.geom, p.geom.NT, p.geom.Hv), dim3(kThreads), smem,
                stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
@@ -410,6 +412,8 @@ int bwd_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *g
     p.m_st = daqk->stride[it];
     FLA_REQUIRE(p.q_st < (1 << 24), FLA_ERR_SHAPE, "%s: token stride of q and k must be below 2^24 elements.", op);
     p.cumsum_dg = cumsum_dg ? 1 : 0;
+    // gradients laid out token-major (a token's row holds every head): neighbouring workgroups take the heads of one chunk
+    p.geom.head_fast = H > 1 && p.st > p.sh && p.geom.NT <= 65535 ? 1 : 0;
     p.out16 = out16 ? 1 : 0;
     return launch_bwd_intra<64>(p, stream);   // 64-channel blocks: two workgroups fit on a CU
 }

@@ -301,8 +301,9 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     float *bS = aS + kChunk * pa;
     float *tS = bS + kChunk;
 
-    const int half = C128 ? (blockIdx.x & 1) : 0;
-    const int c = C128 ? blockIdx.x >> 1 : blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+    int cx, hv;
+    block_chunk_head(p.geom, cx, hv);
+    const int half = C128 ? (cx & 1) : 0, c = C128 ? cx >> 1 : cx, b = blockIdx.z;
     const int hk = hv / (p.geom.Hv / p.geom.Hk);
     int seq, start, len;
     chunk_span(p.geom, b, c, seq, start, len);
@@ -1010,7 +1011,7 @@ int launch_intra_kernel(const KdaIntraParams &p, hipStream_t stream) {
     const size_t smem = IntraSmem<K, V>::bytes;
     FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V, C128>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V, C128>), dim3(p.geom.NT * (C128 ? 2 : 1), p.geom.Hv, p.geom.B),
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V, C128>), chunk_head_grid(p.geom, p.geom.NT * (C128 ? 2 : 1), p.geom.Hv),
                dim3(kIntraThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
@@ -1185,6 +1186,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     unsigned char *wsb = static_cast<unsigned char *>(ws);
 
     ip.geom = geom;
+    // token-major q, k, v, g (a token's row holds every head): neighbouring workgroups take the heads of one chunk
+    ip.geom.head_fast = geom.Hv > 1 && ip.q.st > ip.q.sh && (int64_t)geom.NT * 2 <= 65535 ? 1 : 0;
     ip.a_log = use_gate ? static_cast<const float *>(a_log->data) : nullptr;
     ip.dt_bias = use_gate && present(dt_bias) ? static_cast<const float *>(dt_bias->data) : nullptr;
     ip.use_gate = use_gate;
