@@ -141,6 +141,9 @@ struct DqkwgParams {
     float *dg;
     int64_t dg_sb, dg_sh, dg_st;
     float scale;
+    // q was l2-normalised by the caller: rstd [B,Hk,T] of that pass, and dq leaves as the gradient of the raw q
+    const float *q_rstd = nullptr;
+    int64_t r_sb = 0, r_sh = 0;
 };
 
 // V is the width of the value slab held in LDS; VSLABS slabs cover the value dimension (1: V itself, 2: V = 256 as
@@ -149,7 +152,9 @@ struct DqkwgParams {
 // the chunk's one h / dh block and the gate cumulated over the whole chunk; a row of the second half also gets
 // ds_21 k_1 in dq, a row of the first half ds_21^T q_2 in dk (ds_21 = do_2 v_1^T e^{G_i - G_j} scale, unmasked), and
 // the sum that lands on the chunk's last token collects sum_t k_t . dk_state_t over both halves.
-template <int K, int V, bool GVA, int VSLABS = 1, int CH = 1>
+// QNORM: q is an l2-normalised tensor and dq leaves as the gradient of the raw one (p.q_rstd); an instance of its own,
+// so that the plain operator carries none of it.
+template <int K, int V, bool GVA, int VSLABS = 1, int CH = 1, bool QNORM = false>
 __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams p) {
     static_assert(CH == 1 || VSLABS == 1, "128-token chunks are built for one value slab");
     extern __shared__ __align__(16) unsigned char smem[];
@@ -194,6 +199,13 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
     f32x4 dq_acc[KTH], dk_acc[KTH];
 #pragma unroll
     for (int ct = 0; ct < KTH; ++ct) dq_acc[ct] = dk_acc[ct] = zero4();
+    static_assert(!QNORM || CH == 1, "the de-normalising form is built for 64-token chunks");
+    float qdot[4] = {0.f, 0.f, 0.f, 0.f};   // QNORM: <q, dq> of this lane's four rows, over every value head
+    float q_rs[4] = {1.f, 1.f, 1.f, 1.f};   // QNORM: rstd of those rows, fetched ahead of everything else
+    if constexpr (QNORM) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q_rs[e] = p.q_rstd[b * p.r_sb + hk * p.r_sh + start + min(16 * w + 4 * lg + e, len - 1)];
+    }
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
@@ -298,7 +310,7 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
             eq[e] = __expf(grow[e]) * p.scale;
             ek[e] = __expf(g_last - grow[e]);
         }
-        float dg_row[4] = {0.f, 0.f, 0.f, 0.f}, kdk_state = 0.f;
+        float dg_row[4] = {0.f, 0.f, 0.f, 0.f}, qdq[4] = {0.f, 0.f, 0.f, 0.f}, kdk_state = 0.f;
 #pragma unroll
         for (int ct = 0; ct < KTH; ++ct) {
             const int cg = half * KTH + ct;
@@ -326,7 +338,10 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
                 if (32 * j + 31 >= 16 * w) dk = mfma16x32(frag_tr(sS, ps, 16 * w, 32 * j), frag_tr(qS, pk, 16 * cg, 32 * j), dk);
             }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) dg_row[e] += dq[e] * qv[e] - dk[e] * kv[e];
+            for (int e = 0; e < 4; ++e) {
+                dg_row[e] += dq[e] * qv[e] - dk[e] * kv[e];
+                if constexpr (QNORM) qdq[e] += dq[e] * qv[e];
+            }
             dq_acc[ct] += dq;
             dk_acc[ct] += dk;
         }
@@ -398,8 +413,16 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
         for (int e = 0; e < 4; ++e) {
             const float v = group_sum<16>(dg_row[e]);
             if (li == 0) dgp[half * kChunk + 16 * w + 4 * lg + e] = v;
+            if constexpr (QNORM) {   // the two column halves of <q, dq> meet in the arrays the 128-token form uses
+                const float u = group_sum<16>(qdq[e]);
+                if (li == 0) goS[half * kChunk + 16 * w + 4 * lg + e] = u;
+            }
         }
         __syncthreads();
+        if constexpr (QNORM) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) qdot[e] += goS[16 * w + 4 * lg + e] + goS[kChunk + 16 * w + 4 * lg + e];
+        }
         if (tid < kChunk && tid < len) {
             float hs = 0.f, ks = 0.f;
 #pragma unroll
@@ -412,6 +435,17 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
             p.dg[b * p.dg_sb + hv * p.dg_sh + (int64_t)(start + tid) * p.dg_st] =
                 dgp[tid] + dgp[kChunk + tid] + (last_half && tid == len - 1 ? dg_last : 0.f);
             if (CH > 1 && hh == 0 && tid == 0) ksS[r] = ks;
+        }
+    }
+    if constexpr (QNORM) {
+        // q is the l2-normalised tile y = x rstd: the gradient of x is (dq - y <y, dq>) rstd per row; <y, dq> was summed
+        // with the gate gradient's row sums above
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+#pragma unroll
+            for (int ct = 0; ct < KTH; ++ct)
+                dq_acc[ct][e] = (dq_acc[ct][e] - (float)qS[row * pk + 16 * (half * KTH + ct) + li] * qdot[e]) * q_rs[e];
         }
     }
     char *dqg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dq.p)) + b * p.dq.sb + hk * p.dq.sh + (int64_t)start * p.dq.st);
@@ -433,6 +467,9 @@ struct WyBwdParams {
     View3 g, beta;
     float *dbeta, *dg;
     int64_t db_sb, db_sh, db_st, dg_sb, dg_sh, dg_st;
+    // accumulating form only: k was l2-normalised by the caller, rstd [B,Hk,T]; dk leaves as the gradient of the raw k
+    const float *k_rstd = nullptr;
+    int64_t r_sb = 0, r_sh = 0;
 };
 
 // Commits a fetched tile with every row scaled by f[row] (rows past `len` become zero).
@@ -724,6 +761,19 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             for (int e = 0; e < 4; ++e) {
                 a[e] = lo[e] + (float)in[e];
                 c[e] = hi[e] + (float)in[4 + e];
+            }
+            if (p.k_rstd != nullptr) {   // k is the l2-normalised y = x rstd: dk of x is (dk - y <y, dk>) rstd per row
+                const elemx8 y = __builtin_bit_cast(elemx8, tk.r[m]);   // the piece of k this thread fetched: same row, same columns
+                float dot = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dot += a[e] * (float)y[e] + c[e] * (float)y[4 + e];
+                dot = group_sum<K / 8>(dot);                            // the K / 8 lanes that hold the row
+                const float rs = p.k_rstd[b * p.r_sb + hk * p.r_sh + start + min(r, len - 1)];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a[e] = (a[e] - (float)y[e] * dot) * rs;
+                    c[e] = (c[e] - (float)y[4 + e] * dot) * rs;
+                }
             }
             if (r < len) *reinterpret_cast<elemx8 *>(dkg + ((int64_t)r * p.dk.st + c8) * 2) = frag_from_acc(a, c);
         }
@@ -1063,12 +1113,24 @@ int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
 }
 
+// rstd of an l2norm_fwd over [B,H,T,K]: contiguous fp32 [B,H,T]; null / no data = absent
+int check_rstd(const char *op, const char *name, const fla_tensor *t, int64_t B, int64_t H, int64_t T, bool &present) {
+    present = t != nullptr && t->data != nullptr;
+    if (!present) return FLA_OK;
+    int rc = check_tensor(t, op, name, 3, dt_bit(FLA_F32));
+    if (rc) return rc;
+    FLA_REQUIRE(t->shape[0] == B && t->shape[1] == H && t->shape[2] == T && is_contiguous(t), FLA_ERR_SHAPE,
+                "%s: %s must be contiguous fp32 [%lld,%lld,%lld].", op, name, (long long)B, (long long)H, (long long)T);
+    return FLA_OK;
+}
+
 int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
                const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
                const fla_int_array *ci, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
                bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
-               const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
-    const char *op = "chunk_bwd_dqkwg";
+               const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query,
+               const fla_tensor *q_rstd = nullptr) {
+    const char *op = q_rstd ? "chunk_bwd_dqkwg_l2norm" : "chunk_bwd_dqkwg";
     FLA_REQUIRE(g_gamma == nullptr || g_gamma->data == nullptr, FLA_ERR_UNSUPPORTED, "%s: g_gamma is not supported.", op);
     FLA_REQUIRE(!use_exp2, FLA_ERR_UNSUPPORTED, "%s: use_exp2 is not supported with a scalar gate.", op);
     FLA_REQUIRE(!transpose_state_layout, FLA_ERR_UNSUPPORTED, "%s: transpose_state_layout is not supported.", op);
@@ -1098,6 +1160,13 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                   static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                   h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                   static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
+    bool has_rstd;
+    if ((rc = check_rstd(op, "q_rstd", q_rstd, geom.B, geom.Hk, geom.T, has_rstd))) return rc;
+    if (has_rstd) {
+        p.q_rstd = static_cast<const float *>(q_rstd->data);
+        p.r_sb = q_rstd->stride[0];
+        p.r_sh = q_rstd->stride[1];
+    }
     // token-major operands (the row of a token holds all heads): neighbouring workgroups take the heads of one chunk
     const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hk);
     const int K = geom.K, V = geom.V;
@@ -1105,6 +1174,15 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     const size_t smem = ((size_t)kChunk * (2 * (K + 16) + 3 * (VS + 8) + kChunk + 8) + (size_t)K * (VS + 8)) * 2 +
                         (kChunk + 16 + 2 * kChunk + kChunk + kMaxRep) * 4;
     const bool gva = geom.Hv != geom.Hk;
+    if (has_rstd) {   // dq de-normalised in the kernel: 64-token chunks
+        FLA_REQUIRE(geom.C == kChunk, FLA_ERR_UNSUPPORTED, "%s: built for chunk_size 64.", op);
+        if (K == 128 && V == 256) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true, 2, 1, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, false, 1, 1, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 128 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, true, 1, 1, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 64 && V == 64) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 64, true, 1, 1, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        if (K == 64 && V == 128) FLA_BWD_DISPATCH_T((dqkwg_kernel<64, 128, true, 1, 1, true>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
+    }
     if (geom.C == 128) {   // one workgroup per chunk, its two halves in turn
         FLA_REQUIRE(geom.Hv / geom.Hk <= kMaxRep, FLA_ERR_UNSUPPORTED, "%s: at most %d value heads per key head with chunk_size 128.", op, kMaxRep);
         if (K == 128 && V == 128 && !gva) FLA_BWD_DISPATCH_T((dqkwg_kernel<128, 128, false, 1, 2>), "bwd_dqkwg", grid, smem, p, kDqkwgThreads);
@@ -1175,7 +1253,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
                      const fla_tensor *dA, const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g,
                      const fla_int_array *cu, const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk,
                      const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size,
-                     hipStream_t stream, uint64_t *query, bool accumulate = false) {
+                     hipStream_t stream, uint64_t *query, bool accumulate = false, const fla_tensor *k_rstd = nullptr) {
     const char *op = accumulate ? "prepare_wy_repr_bwd_full_accumulate" : "prepare_wy_repr_bwd_full";
     ChunkGeom geom;
     int rc;
@@ -1192,6 +1270,13 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), view4(dk), view4(dv), view3(g),
                   view3(beta), static_cast<float *>(dbeta->data), static_cast<float *>(dg->data),
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
+    bool has_rstd;
+    if ((rc = check_rstd(op, "k_rstd", k_rstd, geom.B, geom.Hk, geom.T, has_rstd))) return rc;
+    if (has_rstd) {
+        p.k_rstd = static_cast<const float *>(k_rstd->data);
+        p.r_sb = k_rstd->stride[0];
+        p.r_sh = k_rstd->stride[1];
+    }
     const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hk);
     const int K = geom.K, V = geom.V;
     if (geom.C == 128) {
@@ -1305,6 +1390,29 @@ FLA_ENTRY(fla_chunk_bwd_dqkwg)(
                            static_cast<hipStream_t>(stream), nullptr); });
 }
 
+FLA_ENTRY(fla_chunk_bwd_dqkwg_l2norm_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *q_rstd, float scale, int64_t chunk_size, const fla_tensor *dq,
+    const fla_tensor *dk, const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg_l2norm_get_workspace_size, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, q_rstd, scale, chunk_size, dq, dk, dw, dg, workspace_size);
+    FLA_NULL_WS("chunk_bwd_dqkwg_l2norm");
+    if (!q_rstd || !q_rstd->data) return fla::fail(FLA_ERR_NULL, "chunk_bwd_dqkwg_l2norm: q_rstd must be provided.");
+    return fla::guarded([&] { return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, nullptr, nullptr, scale, chunk_size, false,
+                           false, dq, dk, dw, dg, nullptr, 0, nullptr, workspace_size, q_rstd); });
+}
+FLA_ENTRY(fla_chunk_bwd_dqkwg_l2norm)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *q_rstd, float scale, int64_t chunk_size, const fla_tensor *dq,
+    const fla_tensor *dk, const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size,
+    void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_bwd_dqkwg_l2norm, q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, q_rstd, scale, chunk_size, dq, dk, dw, dg, workspace, workspace_size, stream);
+    if (!q_rstd || !q_rstd->data) return fla::fail(FLA_ERR_NULL, "chunk_bwd_dqkwg_l2norm: q_rstd must be provided.");
+    return fla::guarded([&] { return fla::dqkwg_impl(q, k, v, g, h, dox, dh, dv, cu_seqlens, chunk_indices, nullptr, nullptr, scale, chunk_size, false,
+                           false, dq, dk, dw, dg, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, q_rstd); });
+}
+
 FLA_ENTRY(fla_prepare_wy_repr_bwd_da_get_workspace_size)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
     const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices,
@@ -1346,21 +1454,22 @@ FLA_ENTRY(fla_prepare_wy_repr_bwd_full)(
 FLA_ENTRY(fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
-    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
-    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
-    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace_size);
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *k_rstd, const fla_tensor *dk,
+    const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, k_rstd, dk, dv, dbeta, dg, workspace_size);
     FLA_NULL_WS("prepare_wy_repr_bwd_full_accumulate");
     return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
-                                 nullptr, 0, nullptr, workspace_size, true); });
+                                 nullptr, 0, nullptr, workspace_size, true, k_rstd); });
 }
 FLA_ENTRY(fla_prepare_wy_repr_bwd_full_accumulate)(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
-    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
-    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
-    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg, workspace, workspace_size, stream);
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *k_rstd, const fla_tensor *dk,
+    const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size,
+    void *stream) {
+    FLA_ROUTE_F16(k, fla_prepare_wy_repr_bwd_full_accumulate, k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, k_rstd, dk, dv, dbeta, dg, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::wy_bwd_full_impl(k, v, beta, A, dA, dw, du, g, cu_seqlens, chunk_indices, chunk_size, dk, dv, dbeta, dg,
-                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, true); });
+                                 workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, true, k_rstd); });
 }
 
 FLA_ENTRY(fla_prepare_wy_repr_bwd_get_workspace_size)(

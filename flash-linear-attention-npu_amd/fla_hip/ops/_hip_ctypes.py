@@ -70,7 +70,8 @@ OP_ARGTYPES = {
                        + [_T] * 4,
     "prepare_wy_repr_bwd_da": [_T] * 7 + [_IA, _IA, ctypes.c_int64, _T],
     "prepare_wy_repr_bwd_full": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
-    "prepare_wy_repr_bwd_full_accumulate": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
+    "prepare_wy_repr_bwd_full_accumulate": [_T] * 8 + [_IA, _IA, ctypes.c_int64] + [_T] * 5,
+    "chunk_bwd_dqkwg_l2norm": [_T] * 8 + [_IA, _IA, _T, ctypes.c_float, ctypes.c_int64] + [_T] * 4,
     "prepare_wy_repr_bwd": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
     "chunk_kda_bwd_dav": [_T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T, _T],
     "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 4,
@@ -1033,10 +1034,11 @@ def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu
 
 
 def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, chunk_size, *, cu_seqlens=None,
-                                        chunk_indices=None):
+                                        chunk_indices=None, k_rstd=None):
     """npu_prepare_wy_repr_bwd_full with its key and gate gradients ADDED to ``dk`` ([B,Hk,T,K], dtype of k) and
     ``dg`` ([B,Hv,T] f32) in place: the reference's composition adds them with a separate pass
-    (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32)."""
+    (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32).  ``k_rstd`` (f32 [B,Hk,T], the second result
+    of ``l2norm_fwd``): k is the normalised tensor and the completed dk leaves as the gradient of the raw k."""
     dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dv, dbeta = _call_op(
@@ -1045,12 +1047,35 @@ def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, ch
             ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"), ctx.tensor(A, "A"), ctx.tensor(dA, "dA"),
             ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.tensor(g, "g"),
             ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
-            ctypes.c_int64(int(chunk_size)),
+            ctypes.c_int64(int(chunk_size)), ctx.tensor(k_rstd, "k_rstd"),
             ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(dbeta, "dbeta"), ctx.tensor(dg, "dg"),
         ],
         (dv, dbeta),
     )
     return dv, dbeta
+
+
+def chunk_bwd_dqkwg_l2norm(q, k, v, g, h, dox, dh, dv, q_rstd, chunk_size, *, scale, cu_seqlens=None, chunk_indices=None):
+    """``npu_chunk_bwd_dqkwg`` for an l2-normalised q: dq comes back as the gradient of the raw q (``q_rstd`` f32
+    [B,Hk,T] from ``l2norm_fwd``), which replaces the ``l2norm_bwd`` pass over dq.  dk is the gradient of the normalised
+    k (it is completed, and de-normalised, by ``prepare_wy_repr_bwd_full_accumulate(..., k_rstd=)``)."""
+    q_shape = _shape(q)
+    dq = _empty_ordered_like(q)
+    dk = _empty_ordered_like(k)
+    dw = _empty((q_shape[0], int(v.shape[1]), q_shape[2], q_shape[3]), q)
+    dg = _f32_like(g)
+    outputs = (dq, dk, dw, dg)
+    return _call_op(
+        "chunk_bwd_dqkwg_l2norm", OP_ARGTYPES["chunk_bwd_dqkwg_l2norm"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"), ctx.tensor(h, "h"),
+            ctx.tensor(dox, "dox"), ctx.tensor(dh, "dh"), ctx.tensor(dv, "dv"),
+            ctx.int_array(_as_int_tuple(cu_seqlens)), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctx.tensor(q_rstd, "q_rstd"), ctypes.c_float(float(scale)), ctypes.c_int64(int(chunk_size)),
+            ctx.tensor(dq, "dq"), ctx.tensor(dk, "dk"), ctx.tensor(dw, "dw"), ctx.tensor(dg, "dg"),
+        ],
+        outputs,
+    )
 
 
 def npu_prepare_wy_repr_bwd(k, v, beta, A, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):
@@ -1262,7 +1287,7 @@ def l2norm_fwd(x, eps: float = 1e-6, output_dtype=None):
 
     if output_dtype is not None and output_dtype != x.dtype:
         raise NotImplementedError("l2norm_fwd: output_dtype must equal the input dtype.")
-    y = _empty_like(x)
+    y = _empty_ordered_like(x)   # in the memory order of x, so that what is computed on y needs no layout copy back
     rstd = _empty(_shape(x)[:-1], x, dtype=torch.float32)
     _call_op("l2norm_fwd", OP_ARGTYPES["l2norm_fwd"],
              lambda ctx: [ctx.tensor(x, "x"), ctypes.c_double(float(eps)), ctx.tensor(y, "y"), ctx.tensor(rstd, "rstd")],
@@ -1272,8 +1297,8 @@ def l2norm_fwd(x, eps: float = 1e-6, output_dtype=None):
 
 def l2norm_bwd(y, rstd, dy, eps: float = 1e-6, *, like=None):
     """fla/ops/triton/triton_core/l2norm.py:181-224: dx from the normalised output, its rstd and dy.  ``like``: a tensor
-    (it may be storage-less) whose memory order dx takes, e.g. the input the forward normalised; default: contiguous."""
-    dx = _empty_like(y) if like is None else _empty_ordered_like(like, dtype=y.dtype, shape=tuple(y.shape), device=y.device)
+    (it may be storage-less) whose memory order dx takes; default: that of y."""
+    dx = _empty_ordered_like(y if like is None else like, dtype=y.dtype, shape=tuple(y.shape), device=y.device)
     return _call_op("l2norm_bwd", OP_ARGTYPES["l2norm_bwd"],
                     lambda ctx: [ctx.tensor(y, "y"), ctx.tensor(rstd.contiguous(), "rstd"), ctx.tensor(dy, "dy"),
                                  ctypes.c_double(float(eps)), ctx.tensor(dx, "dx")],

@@ -77,14 +77,17 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
 
 
 def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, do, dht, cu_seqlens=None,
-                                     chunk_size: int = 64, *, saved=None):
+                                     chunk_size: int = 64, *, saved=None, qk_rstd=None):
     """q,k,v [B,H,T,D] bf16; ``g`` the chunk-cumsummed gate and beta [B,T,H] (as the forward returned /
     received them); ``A`` [B,H,T,C] the inverted chunk matrices or None (recomputed); do [B,T,H,V];
     dht [N,H,K,V] fp32 or None.  Returns (dq, dk, dv [B,H,T,D], dbeta, dg [B,T,H] fp32, dh0 [N,H,K,V] fp32 or
     None); dg is the gradient of the RAW gate.  Unlike the reference, the initial state and the final-state
     gradient take part (the reference passes neither to its reverse scan and returns dh0 = None).
     ``saved``: the dict of h, v_new and w the forward wrote with ``save_for_backward``; without it they are
-    recomputed as the reference does (examples/flash_gated_delta_rule.py:913-951)."""
+    recomputed as the reference does (examples/flash_gated_delta_rule.py:913-951).  ``qk_rstd``: (q_rstd, k_rstd) of
+    ``l2norm_fwd`` when q and k are the normalised tensors; dq and dk then come back as the gradients of the raw q and k
+    (the reference runs ``l2norm_bwd`` over both afterwards, :1104-1106).  With 64-token chunks the two kernels that
+    complete dq and dk do it themselves; otherwise two ``l2norm_bwd`` passes follow."""
     import torch
 
     cu = _cu_list(cu_seqlens)
@@ -107,16 +110,24 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     dv = _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
     dh, dh0, dv = _ops.chunk_gated_delta_rule_bwd_dhu(q, k, w, doh, dv, scale, chunk_size, g=gh, h0=initial_state,
                                                       dht=dht, dh0_per_sequence=True, **kw)
-    dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
+    in_kernel_norm = qk_rstd is not None and chunk_size == 64
+    if in_kernel_norm:
+        dq, dk, dw, dg = _raw.chunk_bwd_dqkwg_l2norm(q, k, v_new, gh, h, doh, dh, dv, qk_rstd[0], chunk_size, scale=scale, **kw)
+    else:
+        dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
     dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
     # the second part of dk and dg is added where it is produced (the reference adds with separate passes,
     # examples/flash_gated_delta_rule.py:994-1012)
     if chunk_size == 64:
-        dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size, **kw)
+        dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size,
+                                                          k_rstd=qk_rstd[1] if in_kernel_norm else None, **kw)
     else:   # 128-token chunks: the plain operator and the reference's two additions
         dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
         dk.add_(dk2)
         dg.add_(dg2)
+    if qk_rstd is not None and not in_kernel_norm:
+        dq = _raw.l2norm_bwd(q, qk_rstd[0], dq)
+        dk = _raw.l2norm_bwd(k, qk_rstd[1], dk)
     dg = _ops.chunk_local_cumsum(dg, chunk_size, reverse=True, head_first=True, output_dtype=torch.float32, **kw)
     return dq, dk, dv, db.transpose(1, 2), dg.transpose(1, 2), dh0
 
@@ -136,9 +147,7 @@ def _autograd_function():
         @staticmethod
         def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm):
             q_rstd = k_rstd = None
-            # the memory order of the caller's q and k: their gradients go back in it, whatever the kernels worked on
-            ctx.qk_like = tuple(torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device="meta") for t in (q, k))
-            if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049
+            if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049; y comes back in the memory order of x
                 q, q_rstd = _raw.l2norm_fwd(q)
                 k, k_rstd = _raw.l2norm_fwd(k)
             gc, o, A, final, saved = flash_chunk_gated_delta_rule_fwd(
@@ -155,10 +164,7 @@ def _autograd_function():
             dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
                 q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(),
                 None if dht is None else dht.contiguous(), ctx.cu, ctx.chunk_size,
-                saved=dict(h=h, v_new=v_new, w=w))
-            if q_rstd is not None:      # :1104-1106
-                dq = _raw.l2norm_bwd(q, q_rstd, dq, like=ctx.qk_like[0])
-                dk = _raw.l2norm_bwd(k, k_rstd, dk, like=ctx.qk_like[1])
+                saved=dict(h=h, v_new=v_new, w=w), qk_rstd=None if q_rstd is None else (q_rstd, k_rstd))
             return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None, None
 
     return ChunkGatedDeltaRuleFunction

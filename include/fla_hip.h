@@ -585,6 +585,23 @@ int fla_chunk_bwd_dqkwg(
     bool use_exp2, bool transpose_state_layout, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dw,
     const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
 
+/* chunk_bwd_dqkwg_l2norm - no counterpart in the reference, whose entry normalises q and k ahead of the forward and runs
+ * l2norm_bwd over dq and dk after the backward (examples/flash_gated_delta_rule.py:1047-1049, 1104-1106).  q is the
+ * normalised tensor; q_rstd (f32 [B,Hk,T], contiguous: the second result of l2norm_fwd) lets the kernel return dq as the
+ * gradient of the un-normalised q, dq <- (dq - q <q, dq>) rstd per row, instead of a pass of its own over dq.  dk is
+ * not final here (prepare_wy_repr_bwd_full_accumulate takes k_rstd for it).  Other operands as chunk_bwd_dqkwg. */
+int fla_chunk_bwd_dqkwg_l2norm_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *q_rstd, float scale, int64_t chunk_size, const fla_tensor *dq,
+    const fla_tensor *dk, const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size);
+int fla_chunk_bwd_dqkwg_l2norm(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+    const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, const fla_tensor *q_rstd, float scale, int64_t chunk_size, const fla_tensor *dq,
+    const fla_tensor *dk, const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size,
+    void *stream);
+
 /* prepare_wy_repr_bwd_da - replaces aclnnPrepareWyReprBwdDa (_aclnn_ctypes.py:430-460): gradient of
  * the strictly-lower chunk matrix, stored TRANSPOSED (upper triangular) as the reference does. */
 int fla_prepare_wy_repr_bwd_da_get_workspace_size(
@@ -625,17 +642,20 @@ int fla_prepare_wy_repr_bwd_full(
 /* prepare_wy_repr_bwd_full_accumulate - no counterpart in the reference, whose composition adds the two
  * key gradients with a separate elementwise pass (examples/flash_gated_delta_rule.py:994-1010, dk.add_(dk2)).
  * Same operands as prepare_wy_repr_bwd_full; dk and dg are read, the operator's results added in fp32, and
- * written back in place (dk rounded once).  dv and dbeta are written as usual. */
+ * written back in place (dk rounded once).  dv and dbeta are written as usual.  k_rstd (f32 [B,Hk,T] contiguous, or
+ * NULL): k is the l2-normalised tensor and the completed dk leaves as the gradient of the un-normalised k,
+ * dk <- (dk - k <k, dk>) rstd per row (what l2norm_bwd would do in a pass of its own). */
 int fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
-    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
-    const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size);
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *k_rstd, const fla_tensor *dk,
+    const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, uint64_t *workspace_size);
 int fla_prepare_wy_repr_bwd_full_accumulate(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,
-    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
-    const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+    const fla_int_array *chunk_indices, int64_t chunk_size, const fla_tensor *k_rstd, const fla_tensor *dk,
+    const fla_tensor *dv, const fla_tensor *dbeta, const fla_tensor *dg, void *workspace, uint64_t workspace_size,
+    void *stream);
 
 #ifdef __cplusplus
 }

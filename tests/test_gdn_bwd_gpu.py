@@ -343,15 +343,19 @@ def test_l2norm_kernels_against_oracle(dev, D):
     assert_close(y, gdn.l2norm_fwd(h)[0], 2e-3, "y f16")
 
 
-def test_pipeline_with_in_kernel_l2norm(dev):
+@pytest.mark.parametrize("Hk,Hv,kwargs", [(2, 2, {}), (1, 2, {}), (2, 2, dict(fused=False, chunk_size=128))],
+                         ids=["64-token chunks", "grouped heads", "128-token chunks"])
+def test_pipeline_with_in_kernel_l2norm(dev, Hk, Hv, kwargs):
     """use_qk_l2norm_in_kernel=True: forward equals the recurrence on normalised q, k; gradients reach the
-    UN-normalised q and k (fp64 autograd through F.normalize and the recurrence)."""
+    UN-normalised q and k (fp64 autograd through F.normalize and the recurrence).  With 64-token chunks the kernels
+    that complete dq and dk de-normalise them (chunk_bwd_dqkwg_l2norm, prepare_wy_repr_bwd_full_accumulate with k_rstd);
+    with 128-token chunks two l2norm_bwd passes do."""
     from fla_hip import pipeline
-    B, T, H, K, V = 1, 150, 2, 128, 128
-    d = make(B, T, H, H, K, V, None, seed=21)
+    B, T, K, V = 1, 150, 128, 128
+    d = make(B, T, Hv, Hk, K, V, None, seed=21)
     gen = torch.Generator().manual_seed(22)
-    qraw = (torch.randn(B, H, T, K, generator=gen) * 1.7).to(BF)
-    kraw = (torch.randn(B, H, T, K, generator=gen) * 0.6).to(BF)
+    qraw = (torch.randn(B, Hk, T, K, generator=gen) * 1.7).to(BF)
+    kraw = (torch.randn(B, Hk, T, K, generator=gen) * 0.6).to(BF)
     dd = torch.float64
     leaf = {n: t.to(dd).requires_grad_(True) for n, t in (("q", qraw), ("k", kraw), ("v", d["v"]), ("g", d["g"]), ("beta", d["beta"]))}
     o, _ = gdn.naive_recurrent_gated_delta_rule(F.normalize(leaf["q"], dim=-1), F.normalize(leaf["k"], dim=-1), leaf["v"], leaf["g"],
@@ -365,7 +369,7 @@ def test_pipeline_with_in_kernel_l2norm(dev):
     assert_close(o_inf.transpose(1, 2), o.detach(), TOL_BF16, "o")
     # training path
     q, k, v = (t.to(dev).clone().requires_grad_(True) for t in (qraw, kraw, d["v"]))
-    o_g, _ = pipeline.flash_gated_delta_rule(q, k, v, g, beta, use_qk_l2norm_in_kernel=True)
+    o_g, _ = pipeline.flash_gated_delta_rule(q, k, v, g, beta, use_qk_l2norm_in_kernel=True, **kwargs)
     (o_g.float() * x["do"].transpose(1, 2).float()).sum().backward()
     for name, t in (("q", q), ("k", k), ("v", v)):
         st = err_stats(t.grad, leaf[name].grad)
