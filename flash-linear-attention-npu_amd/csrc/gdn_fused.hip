@@ -52,6 +52,10 @@ struct FusedParams {
     elem *h_out;        // state at the start of every chunk [B,Hv,NT,K,V]
     int64_t h_sb, h_sh, h_sc;
     View4 vn_out, w_out;   // v_new [B,Hv,T,V], w [B,Hv,T,K]
+    // with l2norm: the normalised q and k [B,Hk,T,K] and their rstd (fp32 [B,Hk,T], contiguous), all four or none
+    View4 qn_out, kn_out;
+    float *q_rstd, *k_rstd;
+    int64_t rs_sb, rs_sh;
 };
 
 template <int K, int CT> struct FusedSmem {
@@ -710,7 +714,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         };
         // A row is held by K/8 adjacent lanes, so its sum of squares is one DPP reduction; the normalised row is
         // rounded to bf16 exactly where the separate normalisation kernel would have rounded it.
-        auto unit_row = [&](u32x4 raw) -> u32x4 {
+        auto unit_row = [&](u32x4 raw, float &rstd) -> u32x4 {
             const elemx8 a = __builtin_bit_cast(elemx8, raw);
             f32x4 lo, hi;
             float ss = 0.f;
@@ -720,14 +724,36 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                 hi[e] = (float)a[4 + e];
                 ss += lo[e] * lo[e] + hi[e] * hi[e];
             }
-            const float rstd = __builtin_amdgcn_rsqf(group_sum<K / 8>(ss) + 1e-6f);
+            rstd = __builtin_amdgcn_rsqf(group_sum<K / 8>(ss) + 1e-6f);
             return __builtin_bit_cast(u32x4, frag_from_acc(lo * rstd, hi * rstd));
         };
-        auto commit_qk = [&](const Tiles &t) {
+        // For a backward pass the normalised rows and their rstd also go to memory, once per key head: from the first slab
+        // of the first value head that shares it.  A row is a run of 16-byte pieces in neighbouring lanes.
+        const bool emit_qk = TRAIN && p.qn_out.p != nullptr && slab == 0 && hv % (p.geom.Hv / p.geom.Hk) == 0;
+        auto commit_qk = [&](const Tiles &t, int c) {
+            const int len = min(kChunk, eos - (bos + c * kChunk));
 #pragma unroll
             for (int m = 0; m < QCH; ++m) {
-                *reinterpret_cast<u32x4 *>(t.q + (rq + m * QROWS) * pq + cq) = p.l2norm ? unit_row(pre_q[m]) : pre_q[m];
-                *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(rq + m * QROWS, cq)) = p.l2norm ? unit_row(pre_k[m]) : pre_k[m];
+                const int row = rq + m * QROWS;
+                u32x4 qv = pre_q[m], kv = pre_k[m];
+                if (p.l2norm) {
+                    float qr, kr;
+                    qv = unit_row(qv, qr);
+                    kv = unit_row(kv, kr);
+                    if constexpr (TRAIN) {
+                        if (emit_qk && row < len) {
+                            const int64_t tok = bos + c * kChunk + row;
+                            *reinterpret_cast<u32x4 *>(static_cast<elem *>(const_cast<void *>(p.qn_out.p)) + b * p.qn_out.sb + hk * p.qn_out.sh + tok * p.qn_out.st + cq) = qv;
+                            *reinterpret_cast<u32x4 *>(static_cast<elem *>(const_cast<void *>(p.kn_out.p)) + b * p.kn_out.sb + hk * p.kn_out.sh + tok * p.kn_out.st + cq) = kv;
+                            if (cq == 0) {
+                                p.q_rstd[b * p.rs_sb + hk * p.rs_sh + tok] = qr;
+                                p.k_rstd[b * p.rs_sb + hk * p.rs_sh + tok] = kr;
+                            }
+                        }
+                    }
+                }
+                *reinterpret_cast<u32x4 *>(t.q + row * pq + cq) = qv;
+                *reinterpret_cast<u32x4 *>(t.k + KTile<K>::off(row, cq)) = kv;
             }
         };
         elem *vS = reinterpret_cast<elem *>(smem + L::v_off);
@@ -747,7 +773,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         };
         if (nchunks > 0) {
             prefetch(0);
-            commit_qk(pipe_tiles_at<K>(smem, 0));
+            commit_qk(pipe_tiles_at<K>(smem, 0), 0);
         }
         __syncthreads();   // start
         for (int i = 0; i <= nchunks; ++i) {
@@ -815,7 +841,7 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
                     for (int bi = 0; bi < 4; ++bi) acc_to_tile(wS, pw, 16 * bi, (wv * NTW + m) * 16, r[1 + m][bi]);
 #pragma unroll
                 for (int bi = 0; bi < 4; ++bi) *reinterpret_cast<f32x4 *>(uS + ((wv * 4 + bi) * 64 + l) * 4) = r[0][bi];
-                if (i + 1 < nchunks) commit_qk(pipe_tiles_at<K>(smem, i + 1));
+                if (i + 1 < nchunks) commit_qk(pipe_tiles_at<K>(smem, i + 1), i + 1);
             }
             __syncthreads();   // end
         }
@@ -1089,7 +1115,8 @@ int launch_fused(FusedParams &p, hipStream_t stream) {
 int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
                double scale, const fla_tensor *initial_state, bool output_final_state, const fla_int_array *cu,
                int64_t chunk_size, bool use_qk_l2norm, const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
-               const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w,
+               const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w, const fla_tensor *qn, const fla_tensor *kn,
+               const fla_tensor *q_rstd, const fla_tensor *k_rstd,
                void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
     const char *op = "gdn_chunk_fwd";
     ChunkGeom geom;
@@ -1147,6 +1174,19 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     }
     if (has_vn && (rc = check_bhtd(op, "v_new", v_new, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if (has_w && (rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
+    const bool has_qn = qn && qn->data;
+    if (has_qn) {
+        FLA_REQUIRE(use_qk_l2norm && kn && kn->data && q_rstd && q_rstd->data && k_rstd && k_rstd->data, FLA_ERR_NULL,
+                    "%s: q_normalised, k_normalised, q_rstd and k_rstd come together, with use_qk_l2norm_in_kernel.", op);
+        if ((rc = check_bhtd(op, "q_normalised", qn, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+        if ((rc = check_bhtd(op, "k_normalised", kn, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
+        const fla_tensor *rs[] = {q_rstd, k_rstd};
+        for (int i = 0; i < 2; ++i) {
+            if ((rc = check_tensor(rs[i], op, i ? "k_rstd" : "q_rstd", 3, dt_bit(FLA_F32)))) return rc;
+            FLA_REQUIRE(rs[i]->shape[0] == geom.B && rs[i]->shape[1] == geom.Hk && rs[i]->shape[2] == geom.T && is_contiguous(rs[i]),
+                        FLA_ERR_SHAPE, "%s: rstd must be contiguous fp32 [B,Hk,T].", op);
+        }
+    }
     if (query) {
         *query = vl.bytes();
         return FLA_OK;
@@ -1190,7 +1230,15 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     // per head; 64-column slabs double the number of workgroups and run as the two-group pipelined kernel.  The wide
     // form is used once it alone fills the GPU; the in-kernel normalisation lives in the pipelined kernel's tile commit.
     const int64_t chains = (int64_t)geom.N * geom.Hv;
-    const bool train = has_h || has_vn || has_w;
+    const bool train = has_h || has_vn || has_w || has_qn;
+    if (has_qn) {
+        p.qn_out = view4(qn);
+        p.kn_out = view4(kn);
+        p.q_rstd = static_cast<float *>(q_rstd->data);
+        p.k_rstd = static_cast<float *>(k_rstd->data);
+        p.rs_sb = q_rstd->stride[0];
+        p.rs_sh = q_rstd->stride[1];
+    }
     if (has_h) {
         p.h_out = static_cast<elem *>(h->data);
         p.h_sb = h->stride[0];
@@ -1216,12 +1264,14 @@ FLA_ENTRY(fla_gdn_chunk_fwd_get_workspace_size)(const fla_tensor *q, const fla_t
                                                     bool use_qk_l2norm_in_kernel, const fla_tensor *o,
                                                     const fla_tensor *g_cumsum, const fla_tensor *final_state,
                                                     const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w,
+                                                    const fla_tensor *q_normalised, const fla_tensor *k_normalised,
+                                                    const fla_tensor *q_rstd, const fla_tensor *k_rstd,
                                                     uint64_t *workspace_size) {
-    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, workspace_size);
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_get_workspace_size, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, q_normalised, k_normalised, q_rstd, k_rstd, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd: workspace_size must not be null.");
     return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
-                           use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, h, v_new, w, nullptr, 0, nullptr, workspace_size); });
+                           use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, q_normalised, k_normalised, q_rstd,
+                           k_rstd, nullptr, 0, nullptr, workspace_size); });
 }
 
 FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
@@ -1229,9 +1279,11 @@ FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla
                                  bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
                                  bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
                                  const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
-                                 const fla_tensor *w, void *workspace, uint64_t workspace_size, void *stream) {
-    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, workspace, workspace_size, stream);
+                                 const fla_tensor *w, const fla_tensor *q_normalised, const fla_tensor *k_normalised,
+                                 const fla_tensor *q_rstd, const fla_tensor *k_rstd, void *workspace,
+                                 uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd, q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, q_normalised, k_normalised, q_rstd, k_rstd, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
-                           use_qk_l2norm_in_kernel, o,
-                           g_cumsum, final_state, h, v_new, w, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+                           use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, q_normalised, k_normalised, q_rstd,
+                           k_rstd, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }

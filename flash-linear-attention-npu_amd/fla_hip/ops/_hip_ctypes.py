@@ -49,7 +49,7 @@ OP_ARGTYPES = {
                                      ctypes.c_bool, _T, _T, _T],
     "chunk_fwd_o": [_T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
     "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, ctypes.c_bool,
-                      _T, _T, _T, _T, _T, _T],
+                      _T, _T, _T, _T, _T, _T, _T, _T, _T, _T],
     "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
@@ -421,7 +421,8 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
     use_qk_l2norm_in_kernel normalises q and k rows inside the kernel (flash_gated_delta_rule.py:1047-1049).
     Returns (g_cumsum [B,T,H] f32, o [B,T,H,V], final_state or None); with ``save_for_backward`` also
     (h [B,HV,NT,K,V], v_new [B,HV,T,V], w [B,HV,T,K]), the operands the reference's backward recomputes
-    (flash_gated_delta_rule.py:913-951)."""
+    (flash_gated_delta_rule.py:913-951), and with both flags further (q_normalised, k_normalised, q_rstd, k_rstd):
+    what ``l2norm_fwd`` hands its backward (flash_gated_delta_rule.py:1086-1089), in the memory order of q and k."""
     import torch
 
     B, _, T, K = _shape(k)
@@ -431,13 +432,17 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
     o = _empty((B, T, HV, V), v)
     g_out = _empty((B, T, HV), v, dtype=torch.float32)
     final = _empty((N, HV, K, V), v, dtype=torch.float32) if output_final_state else None
-    h = v_new = w = None
+    h = v_new = w = qn = kn = q_rstd = k_rstd = None
     if save_for_backward:
         C = 64
         NT = -(-T // C) if cu is None else sum(-(-(cu[i + 1] - cu[i]) // C) for i in range(N))
         h = _empty((B, HV, NT, K, V), v)
         v_new = _empty((B, HV, T, V), v)
         w = _empty((B, HV, T, K), v)
+        if use_qk_l2norm_in_kernel:
+            qn, kn = _empty_ordered_like(q), _empty_ordered_like(k)
+            q_rstd = _empty(_shape(q)[:-1], q, dtype=torch.float32)
+            k_rstd = _empty(_shape(k)[:-1], k, dtype=torch.float32)
     _call_op(
         "gdn_chunk_fwd", OP_ARGTYPES["gdn_chunk_fwd"],
         lambda ctx: [
@@ -447,9 +452,13 @@ def gdn_chunk_fwd(q, k, v, g, beta, scale, initial_state, output_final_state, cu
             ctypes.c_bool(bool(use_qk_l2norm_in_kernel)),
             ctx.tensor(o, "o"), ctx.tensor(g_out, "g_cumsum"), ctx.tensor(final, "final_state"),
             ctx.tensor(h, "h"), ctx.tensor(v_new, "v_new"), ctx.tensor(w, "w"),
+            ctx.tensor(qn, "q_normalised"), ctx.tensor(kn, "k_normalised"),
+            ctx.tensor(q_rstd, "q_rstd"), ctx.tensor(k_rstd, "k_rstd"),
         ],
         (o, g_out, final),
     )
+    if save_for_backward and use_qk_l2norm_in_kernel:
+        return g_out, o, final, h, v_new, w, qn, kn, q_rstd, k_rstd
     if save_for_backward:
         return g_out, o, final, h, v_new, w
     return g_out, o, final

@@ -38,7 +38,8 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
     ``use_qk_l2norm_in_kernel`` the fused route normalises q and k rows while it stages them; the composed
     route runs the two normalisation passes first (examples/flash_gated_delta_rule.py:1047-1049).
     ``save_for_backward`` appends a dict with h, v_new and w, which the backward then does not recompute
-    (64-token chunks only)."""
+    (64-token chunks only); the fused route with ``use_qk_l2norm_in_kernel`` adds the normalised q and k and their
+    q_rstd, k_rstd, written by the same kernel."""
     import torch
 
     cu = _cu_list(cu_seqlens)
@@ -54,7 +55,7 @@ def flash_chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, out
         if final is not None and initial_state is not None and final.dtype != initial_state.dtype:
             final = final.to(initial_state.dtype)
         if save_for_backward:
-            return gc, o, None, final, dict(zip(("h", "v_new", "w"), res[3:]))
+            return gc, o, None, final, dict(zip(("h", "v_new", "w", "q", "k", "q_rstd", "k_rstd"), res[3:]))
         return gc, o, None, final
     if use_qk_l2norm_in_kernel:
         q, _ = _raw.l2norm_fwd(q)
@@ -147,12 +148,17 @@ def _autograd_function():
         @staticmethod
         def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm):
             q_rstd = k_rstd = None
-            if l2norm:      # examples/flash_gated_delta_rule.py:1047-1049; y comes back in the memory order of x
+            # examples/flash_gated_delta_rule.py:1047-1049.  The fused forward normalises the rows itself and writes
+            # them with their rstd; the composed route runs l2norm_fwd (y comes back in the memory order of x).
+            in_kernel = bool(l2norm and fused)
+            if l2norm and not in_kernel:
                 q, q_rstd = _raw.l2norm_fwd(q)
                 k, k_rstd = _raw.l2norm_fwd(k)
             gc, o, A, final, saved = flash_chunk_gated_delta_rule_fwd(
                 q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused,
-                save_for_backward=True)
+                use_qk_l2norm_in_kernel=in_kernel, save_for_backward=True)
+            if in_kernel:
+                q, k, q_rstd, k_rstd = saved["q"], saved["k"], saved["q_rstd"], saved["k_rstd"]
             ctx.save_for_backward(q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd, saved["h"], saved["v_new"], saved["w"])
             ctx.scale, ctx.cu, ctx.chunk_size = scale, cu, chunk_size
             ctx.dtypes = (g.dtype, beta.dtype)

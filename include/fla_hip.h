@@ -215,6 +215,12 @@ int fla_chunk_fwd_o(
  * w [B,Hv,T,K], all bf16 and each NULL or given: what the reference's backward
  * recomputes with recompute_w_u_fwd and chunk_gated_delta_rule_fwd_h
  * (examples/flash_gated_delta_rule.py:913-951), written by the forward instead.
+ * q_normalised [B,Hk,T,K], k_normalised [B,Hk,T,K] (element type of q, any
+ * strides with unit innermost stride) and q_rstd, k_rstd [B,Hk,T] f32
+ * (contiguous): all four given or all NULL, and only with
+ * use_qk_l2norm_in_kernel.  The scaled rows and the factors they were scaled
+ * by, which fla's l2norm_fwd returns to its autograd function
+ * (examples/flash_gated_delta_rule.py:1086-1089) and a backward needs.
  * ------------------------------------------------------------------------ */
 int fla_gdn_chunk_fwd_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
@@ -222,14 +228,17 @@ int fla_gdn_chunk_fwd_get_workspace_size(
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
     bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
     const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
-    const fla_tensor *w, uint64_t *workspace_size);
+    const fla_tensor *w, const fla_tensor *q_normalised, const fla_tensor *k_normalised,
+    const fla_tensor *q_rstd, const fla_tensor *k_rstd, uint64_t *workspace_size);
 int fla_gdn_chunk_fwd(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, double scale, const fla_tensor *initial_state,
     bool output_final_state, const fla_int_array *cu_seqlens, int64_t chunk_size,
     bool use_qk_l2norm_in_kernel, const fla_tensor *o, const fla_tensor *g_cumsum,
     const fla_tensor *final_state, const fla_tensor *h, const fla_tensor *v_new,
-    const fla_tensor *w, void *workspace, uint64_t workspace_size, void *stream);
+    const fla_tensor *w, const fla_tensor *q_normalised, const fla_tensor *k_normalised,
+    const fla_tensor *q_rstd, const fla_tensor *k_rstd, void *workspace,
+    uint64_t workspace_size, void *stream);
 
 /* ------------------------------------------------------------------------
  * recurrent_gated_delta_rule - replaces aclnnRecurrentGatedDeltaRule

@@ -141,6 +141,44 @@ def test_in_kernel_l2norm_equals_separate_pass(dev, case, dtype):
     assert_close(final, f_ref, 2 * TOL_STATE, "final_state")
 
 
+@pytest.mark.parametrize("token_major", [False, True], ids=["head_major", "token_major"])
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", CASES)
+def test_forward_writes_normalised_q_k_and_rstd(dev, case, dtype, token_major):
+    """use_qk_l2norm_in_kernel with save_for_backward: the kernel also writes the normalised q, k and their rstd, what
+    l2norm_fwd hands its backward (examples/flash_gated_delta_rule.py:1086-1089).  Checked against the oracle's
+    l2norm_fwd (fla/ops/triton/triton_core/l2norm.py:131-178): rstd to fp32 rounding of the sum, the rows to one
+    rounding of the element type; they come in the memory order of q and k, and o, the state and the gate are
+    bit-identical to the call that does not ask for them."""
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, H, Hk, K, V, cu = case
+    d = gdn.make_gdn_inputs(B, T, H, K, V, dtype=dtype, seed=T + 5 * H, Hk=Hk)
+    gen = torch.Generator().manual_seed(T + 1)
+    q = (d["q"].float() * (0.3 + 3 * torch.rand(B, Hk, T, 1, generator=gen))).to(dtype)
+    k = (d["k"].float() * (0.3 + 3 * torch.rand(B, Hk, T, 1, generator=gen))).to(dtype)
+    place = (lambda t: t.transpose(1, 2).contiguous().to(dev).transpose(1, 2)) if token_major else (lambda t: t.to(dev))
+    qd, kd = place(q), place(k)
+    v, g, beta = (d[n].to(dev) for n in ("v", "g", "beta"))
+    N = B if cu is None else len(cu) - 1
+    h0 = (torch.randn(N, H, K, V, generator=gen) * 0.01).to(dev)
+    scale = K ** -0.5
+    plain = raw.gdn_chunk_fwd(qd, kd, v, g, beta, scale, h0, True, cu, 64, True)
+    res = raw.gdn_chunk_fwd(qd, kd, v, g, beta, scale, h0, True, cu, 64, True, save_for_backward=True)
+    assert len(res) == 10
+    for name, a, b in zip(("g_cumsum", "o", "final_state"), res[:3], plain):
+        assert torch.equal(a, b), name
+    qn, kn, q_rstd, k_rstd = res[6:]
+    for name, x, y, rstd in (("q", q, qn, q_rstd), ("k", k, kn, k_rstd)):
+        y_ref, r_ref = gdn.l2norm_fwd(x)
+        assert y.shape == x.shape and y.dtype == dtype and y.stride() == (qd if name == "q" else kd).stride(), name
+        assert rstd.shape == x.shape[:-1] and rstd.dtype == torch.float32 and rstd.is_contiguous(), name
+        assert_close(rstd, r_ref, 1e-5, name + "_rstd")
+        assert_close(y, y_ref.float(), 4e-3 if dtype == BF else 5e-4, name + "_normalised")
+    # the backward's operands are those of the normalised problem
+    w_ref = raw.gdn_chunk_fwd(qn, kn, v, g, beta, scale, h0, True, cu, 64, save_for_backward=True)[5]
+    assert_close(res[5], w_ref.float(), 1e-2 if dtype == BF else 2e-3, "w")
+
+
 @pytest.mark.parametrize("chunk_size", [16, 128, 256])
 def test_other_chunk_sizes_give_the_same_result(dev, chunk_size):
     """chunk_size only tiles the recurrence: the entry accepts any power of two and returns the result of the
