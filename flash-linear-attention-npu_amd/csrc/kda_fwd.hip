@@ -93,12 +93,25 @@ __device__ __forceinline__ elemx8 scaled_frag(const elem *tile, int pitch, const
 }
 
 template <int K, int V> struct IntraSmem {
-    static constexpr int pq = K + 16, pk = K + 8, pg = K + 4, pv = V + 16, pa = 68, pb = 72;
+    // WIDE (more than 128 channels): the tiles of the 128-channel form do not fit together.  The gate tile is dead
+    // once the gated operands are formed, so v (times beta) and the Aqk staging tile take its place afterwards, and
+    // the scratch of the gate scan lies over the fp32 score tile, which is first written after the scan.
+    static constexpr bool WIDE = K > 128;
+    static constexpr int pq = WIDE ? K + 8 : K + 16, pk = K + 8, pg = K + 4, pv = V + 16, pa = 68, pb = 72;
     static constexpr int SEG = kIntraThreads / K;  // token segments of the gate scan
-    static constexpr size_t bytes =
-        (size_t)kChunk * (pq + pk + pv + 2 * pb) * 2 + (size_t)((kChunk + 2) * pg + kChunk * (pa + 1)) * 4 +
-        (size_t)2 * SEG * K * 4;
+    static constexpr size_t g_bytes = (size_t)(kChunk + 2) * pg * 4;
     // gate rows kChunk and kChunk + 1: the gate at the end of the chunk and the anchor of the coupling block
+    static constexpr size_t q_off = 0;
+    static constexpr size_t k_off = q_off + (size_t)kChunk * pq * 2;
+    static constexpr size_t ak_off = k_off + (size_t)kChunk * pk * 2 + (WIDE ? 0 : (size_t)kChunk * pv * 2);
+    static constexpr size_t g_off = ak_off + (size_t)kChunk * pb * 2 * (WIDE ? 1 : 2);
+    static constexpr size_t v_off = WIDE ? g_off : k_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t aq_off = WIDE ? g_off + (size_t)kChunk * pv * 2 : ak_off + (size_t)kChunk * pb * 2;
+    static constexpr size_t a_off = g_off + g_bytes;                       // fp32 scores [kChunk][pa], then beta [kChunk]
+    static constexpr size_t t_off = WIDE ? a_off : a_off + (size_t)kChunk * (pa + 1) * 4;   // scan scratch [2 SEG][K]
+    static constexpr size_t bytes = WIDE ? a_off + (size_t)kChunk * (pa + 1) * 4 : t_off + (size_t)2 * SEG * K * 4;
+    static_assert(!WIDE || ((size_t)kChunk * (pv + pb) * 2 <= g_bytes && (size_t)2 * SEG * K <= (size_t)kChunk * pa),
+                  "the tiles that replace the gate tile and the scan scratch must fit where they are put");
 };
 
 // Everything a wave does after the gate scan.  Eight waves: wave W of role 0 owns row tile W of k k^T (with the
@@ -108,11 +121,13 @@ template <int K, int V> struct IntraSmem {
 template <int K, int V, int W, int ROLE, bool C128>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
-                                           int64_t dec_base, int half) {
+                                           int64_t dec_base, int half, const elem *vg) {
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb;
     constexpr int KS = K / 32, R1 = W, R2 = 3 - W;
+    constexpr bool WIDE = S::WIDE;
     const int l = lane_id(), li = l & 15, lg = l >> 4;
+    f32x4 aqv[4];   // WIDE: the wave's Aqk tiles wait in registers until the gate tile has made room for them
 
     // ---- scores: k k^T row tile R1 (and its transposed diagonal tile) | q k^T row tile R2 ------------------
     f32x4 kacc[R1 + 1], kaccT = zero4(), qacc[R2 + 1];
@@ -123,14 +138,27 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     f32x4 brow = zero4();
     float bcol = 0.f;
     if constexpr (ROLE == 0) {
+        if constexpr (WIDE) {   // rolled: with eight steps unrolled the scaled operands of all of them are formed up front
+#pragma unroll 1
+            for (int j = 0; j < KS; ++j) {
+                const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
 #pragma unroll
-        for (int j = 0; j < KS; ++j) {
-            const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
+                for (int c = 0; c <= R1; ++c) {
+                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+                    kacc[c] = mfma16x32(lk, rk, kacc[c]);
+                    if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+                }
+            }
+        } else {
 #pragma unroll
-            for (int c = 0; c <= R1; ++c) {
-                const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
-                kacc[c] = mfma16x32(lk, rk, kacc[c]);
-                if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+            for (int j = 0; j < KS; ++j) {
+                const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
+#pragma unroll
+                for (int c = 0; c <= R1; ++c) {
+                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+                    kacc[c] = mfma16x32(lk, rk, kacc[c]);
+                    if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
+                }
             }
         }
         // lane holds (row 16R + 4lg + e, column 16c + li) of each tile
@@ -141,13 +169,25 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
 #pragma unroll
             for (int e = 0; e < 4; ++e) aS[(16 * R1 + 4 * lg + e) * pa + 16 * c + li] = brow[e] * kacc[c][e];
     } else {
+        if constexpr (WIDE) {
+#pragma unroll 1
+            for (int j = 0; j < KS; ++j) {
+                const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
 #pragma unroll
-        for (int j = 0; j < KS; ++j) {
-            const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+                for (int c = 0; c <= R2; ++c) {
+                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+                    qacc[c] = mfma16x32(lq, rk, qacc[c]);
+                }
+            }
+        } else {
 #pragma unroll
-            for (int c = 0; c <= R2; ++c) {
-                const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
-                qacc[c] = mfma16x32(lq, rk, qacc[c]);
+            for (int j = 0; j < KS; ++j) {
+                const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
+#pragma unroll
+                for (int c = 0; c <= R2; ++c) {
+                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+                    qacc[c] = mfma16x32(lq, rk, qacc[c]);
+                }
             }
         }
 #pragma unroll
@@ -157,7 +197,8 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
 #pragma unroll
                 for (int e = 0; e < 4; ++e) a[e] = (c < R2 || li <= 4 * lg + e) ? p.scale * qacc[c <= R2 ? c : 0][e] : 0.f;
             }
-            acc_to_tile(aqS, pb, 16 * R2, 16 * c, a);
+            if constexpr (WIDE) aqv[c] = a;
+            else acc_to_tile(aqS, pb, 16 * R2, 16 * c, a);
         }
     }
 
@@ -211,6 +252,8 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         }
     }
     // ---- gated operands: qg, kg to memory; k beta 2^g over the q tile ----------------------------------
+    // WIDE: one piece at a time (unrolled, the four pieces of a thread do not fit the registers together)
+#pragma unroll(WIDE ? 1 : 2)
     for (int idx = threadIdx.x; idx < kChunk * (K / 8); idx += kIntraThreads) {
         const int r = idx / (K / 8), c8 = (idx % (K / 8)) * 8;
         const elemx8 q8 = *reinterpret_cast<const elemx8 *>(qS + r * pq + c8);
@@ -261,6 +304,29 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         *reinterpret_cast<elemx8 *>(qS + r * pq + c8) = kb8;
     }
     if (threadIdx.x < K && dec_base >= 0) p.dec[dec_base + threadIdx.x] = ex2(gS[kChunk * pg + threadIdx.x]);
+    if constexpr (WIDE) {
+        __syncthreads();   // last read of the gate tile
+        TileCopy<kIntraThreads, kChunk, V> tv;
+        tv.fetch(vg, p.v.st, len, threadIdx.x);
+#pragma unroll
+        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {   // v * beta
+            const int idx = m * kIntraThreads + threadIdx.x;
+            const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
+            const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
+            const float bb = bS[r];
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)v8[e] * bb;
+                hi[e] = (float)v8[4 + e] * bb;
+            }
+            *reinterpret_cast<elemx8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
+        }
+        if constexpr (ROLE == 1) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc_to_tile(aqS, pb, 16 * R2, 16 * c, aqv[c]);
+        }
+    }
     __syncthreads();
 
     // ---- w = Akk (k beta 2^g) (role 0), u = Akk (v beta) (role 1): row tile W -----------------------------------
@@ -272,8 +338,12 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     for (int j = 0; j < (W < 2 ? 1 : 2); ++j) {   // Akk is lower triangular
         const elemx8 a = frag_kc(akS, pb, 16 * W, 32 * j);
 #pragma unroll
-        for (int ct = 0; ct < NCT; ++ct)
+        for (int ct = 0; ct < NCT; ++ct) {
             oacc[ct] = mfma16x32(a, ROLE == 0 ? frag_tr(qS, pq, 16 * ct, 32 * j) : frag_tr(vS, pv, 16 * ct, 32 * j), oacc[ct]);
+            if constexpr (WIDE) {
+                if (ct % 4 == 3) __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     }
     __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
 #pragma unroll
@@ -291,15 +361,15 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb, SEG = S::SEG;
-    elem *qS = reinterpret_cast<elem *>(smem);
-    elem *kS = qS + kChunk * pq;
-    elem *vS = kS + kChunk * pk;
-    elem *akS = vS + kChunk * pv;
-    elem *aqS = akS + kChunk * pb;
-    float *gS = reinterpret_cast<float *>(aqS + kChunk * pb);
-    float *aS = gS + (kChunk + 2) * pg;
+    elem *qS = reinterpret_cast<elem *>(smem + S::q_off);
+    elem *kS = reinterpret_cast<elem *>(smem + S::k_off);
+    elem *vS = reinterpret_cast<elem *>(smem + S::v_off);
+    elem *akS = reinterpret_cast<elem *>(smem + S::ak_off);
+    elem *aqS = reinterpret_cast<elem *>(smem + S::aq_off);
+    float *gS = reinterpret_cast<float *>(smem + S::g_off);
+    float *aS = reinterpret_cast<float *>(smem + S::a_off);
     float *bS = aS + kChunk * pa;
-    float *tS = bS + kChunk;
+    float *tS = reinterpret_cast<float *>(smem + S::t_off);
 
     int cx, hv;
     block_chunk_head(p.geom, cx, hv);
@@ -358,20 +428,21 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     }
     {   // all loads of the chunk are issued before the first LDS write waits for one of them
         TileCopy<kIntraThreads, kChunk, K> tq, tk;
+        constexpr int NVP = S::WIDE ? 0 : TileCopy<kIntraThreads, kChunk, V>::N;   // WIDE: v is staged later
         TileCopy<kIntraThreads, kChunk, V> tv;
         tq.fetch(qg, p.q.st, len, tid);
         tk.fetch(kg, p.k.st, len, tid);
-        tv.fetch(vg, p.v.st, len, tid);
-        float br[TileCopy<kIntraThreads, kChunk, V>::N];
+        if constexpr (!S::WIDE) tv.fetch(vg, p.v.st, len, tid);
+        float br[NVP + 1];
 #pragma unroll
-        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {
+        for (int m = 0; m < NVP; ++m) {
             const int r = (m * kIntraThreads + tid) / (V / 8);
             br[m] = load_scalar(p.beta, b, hv, start + min(r, len - 1));
         }
         tq.commit(qS, pq, len, tid);
         tk.commit(kS, pk, len, tid);
 #pragma unroll
-        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {   // v * beta
+        for (int m = 0; m < NVP; ++m) {   // v * beta
             const int idx = m * kIntraThreads + tid;
             const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
             const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
@@ -433,14 +504,14 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
 
     const int64_t dec_base = half ? -1 : (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
-        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half); break;
+        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
     }
 
     store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
@@ -476,13 +547,16 @@ struct KdaCrossParams {
 };
 
 template <int K, int V> struct CrossSmem {
-    static constexpr int pk = K + 8, pr = K + 16, pv = V + 16, pb = 72;
+    // WIDE (more than 128 channels): w1 and u1 are staged after the scores, over the two operand tiles of the second half
+    static constexpr bool WIDE = K > 128;
+    static constexpr int pk = K + 8, pr = WIDE ? K + 8 : K + 16, pv = WIDE ? V + 8 : V + 16, pb = 72;
+    static_assert(!WIDE || V <= K, "u1 takes the place of a K-wide tile");
     static constexpr size_t qa_off = 0;
     static constexpr size_t kb_off = qa_off + (size_t)kChunk * pk * 2;
     static constexpr size_t kc_off = kb_off + (size_t)kChunk * pk * 2;
-    static constexpr size_t w_off = kc_off + (size_t)kChunk * pk * 2;
-    static constexpr size_t u_off = w_off + (size_t)kChunk * pr * 2;
-    static constexpr size_t a11_off = u_off + (size_t)kChunk * pv * 2;
+    static constexpr size_t w_off = WIDE ? qa_off : kc_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t u_off = WIDE ? kb_off : w_off + (size_t)kChunk * pr * 2;
+    static constexpr size_t a11_off = WIDE ? kc_off + (size_t)kChunk * pk * 2 : u_off + (size_t)kChunk * pv * 2;
     static constexpr size_t a22_off = a11_off + (size_t)kChunk * pb * 2;
     static constexpr size_t mhi_off = a22_off + (size_t)kChunk * pb * 2;
     static constexpr size_t mlo_off = mhi_off + (size_t)kChunk * pb * 2;
@@ -522,15 +596,19 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
         tq.fetch(p.x1 + row2 * K, K, len2, tid);
         tb.fetch(p.x2 + row2 * K, K, len2, tid);
         tc.fetch(p.x1 + row1 * K, K, kChunk, tid);
-        tw.fetch(p.w + row1 * K, K, kChunk, tid);
-        tu.fetch(p.u + row1 * V, V, kChunk, tid);
+        if constexpr (!L::WIDE) {
+            tw.fetch(p.w + row1 * K, K, kChunk, tid);
+            tu.fetch(p.u + row1 * V, V, kChunk, tid);
+        }
         t1.fetch(p.akk + row1 * C, C, kChunk, tid);
         t2.fetch(p.akk + row2 * C + kChunk, C, len2, tid);
         tq.commit(qaS, pk, len2, tid);
         tb.commit(kbS, pk, len2, tid);
         tc.commit(kcS, pk, kChunk, tid);
-        tw.commit(wS, pr, kChunk, tid);
-        tu.commit(uS, pv, kChunk, tid);
+        if constexpr (!L::WIDE) {
+            tw.commit(wS, pr, kChunk, tid);
+            tu.commit(uS, pv, kChunk, tid);
+        }
         t1.commit(a11S, pb, kChunk, tid);
         t2.commit(a22S, pb, len2, tid);
     }
@@ -562,6 +640,15 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
         }
     }
     __syncthreads();
+    if constexpr (L::WIDE) {   // the score operands are spent: w1 and u1 over the tiles of the second half
+        TileCopy<kThreads, kChunk, K> tw;
+        TileCopy<kThreads, kChunk, V> tu;
+        tw.fetch(p.w + row1 * K, K, kChunk, tid);
+        tu.fetch(p.u + row1 * V, V, kChunk, tid);
+        tw.commit(wS, pr, kChunk, tid);
+        tu.commit(uS, pv, kChunk, tid);
+        __syncthreads();
+    }
 
     // P^T tiles (rows = first-half token j, columns = the wave's rows) as operands with contraction j
     elemx8 phi[2], plo[2];
@@ -953,6 +1040,173 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     }
 }
 
+// More than 128 channels: the tiles of one step fill the LDS, so nothing is double-buffered.  256 threads, all four
+// waves copy the tiles of a step, compute it (same products, operand fragments read as they are used so that the
+// registers hold the 256 x 16 state of the wave and little else), and write the staged outputs.  Three barriers a step.
+template <int K> struct WideScanSmem {
+    static constexpr int pw = K + 8, pt = K + 16, pu = 64 + 8, pb = 72, ph = 64 + 8;
+    static constexpr size_t w_off = 0;
+    static constexpr size_t q_off = w_off + (size_t)kChunk * pw * 2;
+    static constexpr size_t k_off = q_off + (size_t)kChunk * pw * 2;
+    static constexpr size_t u_off = k_off + (size_t)kChunk * pt * 2;
+    static constexpr size_t a_off = u_off + (size_t)kChunk * pu * 2;
+    static constexpr size_t d_off = a_off + (size_t)kChunk * pb * 2;
+    static constexpr size_t h_off = d_off + (size_t)K * 4;
+    static constexpr size_t bytes = h_off + (size_t)K * ph * 2;
+};
+
+template <int K, int SUB>
+__global__ void __launch_bounds__(kThreads) kda_scan_wide_kernel(const KdaScanParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef WideScanSmem<K> L;
+    constexpr int VS = 64;
+    constexpr int pw = L::pw, pt = L::pt, pu = L::pu, pb = L::pb, ph = L::ph;
+    constexpr int KT = K / 16, KS = K / 32;
+    elem *wS = reinterpret_cast<elem *>(smem + L::w_off), *qS = reinterpret_cast<elem *>(smem + L::q_off);
+    elem *kS = reinterpret_cast<elem *>(smem + L::k_off), *uS = reinterpret_cast<elem *>(smem + L::u_off);
+    elem *aS = reinterpret_cast<elem *>(smem + L::a_off), *hS = reinterpret_cast<elem *>(smem + L::h_off);
+    float *dS = reinterpret_cast<float *>(smem + L::d_off);
+
+    int slab, hv, n;
+    chain_of_block(slab, hv, n);
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+        chunk0 = p.geom.choff[n];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const int64_t head_row = ((int64_t)b * p.geom.Hv + hv) * p.geom.T;
+    const bool stage_h = p.h != nullptr && !p.v_first;
+    const int tid = threadIdx.x, wv = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int vcol0 = slab * VS + wv * 16;
+
+    f32x4 hacc[KT];
+    auto state_off = [&](int kk, int v) -> int64_t { return p.v_first ? (int64_t)v * K + kk : (int64_t)kk * V + v; };
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        f32x4 a = zero4();
+        if (p.h0) {
+            const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = s[state_off(16 * kt + 4 * lg + e, vcol0 + li)];
+        }
+        hacc[kt] = a;
+    }
+    char *og = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.o.p)) + b * p.o.sb + hv * p.o.sh + vcol0);
+
+    elemx8 hB[KS], vprev[2] = {};
+    for (int c = 0; c < nchunks; ++c) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        const int64_t row = head_row + start;
+        const bool first = SUB == 1 || (c % SUB) == 0;   // first step of a chunk
+        const int chunk = chunk0 + c / SUB;
+
+        load_tile<kThreads>(wS, pw, p.w + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(qS, pw, p.qg + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(kS, pt, p.kg + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(uS, pu, p.u + row * V + slab * VS, V, kChunk, VS, len);
+        load_tile<kThreads>(aS, pb, p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, kChunk, kChunk, len);
+        for (int i = tid; i < K; i += kThreads) dS[i] = p.dec[(((int64_t)b * p.geom.NT + chunk) * p.geom.Hv + hv) * K + i];
+        __syncthreads();   // tiles of this step in place
+
+        if (first) {
+#pragma unroll
+            for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+            if (p.h && p.v_first) {   // [V][K] blocks: the lane's four K rows are contiguous
+                elem *hg = p.h + b * p.h_sb + (int64_t)chunk * p.h_sc + hv * p.h_sh;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    const elemx8 f = hB[kt >> 1];
+                    const elemx4 q4 = (kt & 1) ? elemx4{f[4], f[5], f[6], f[7]} : elemx4{f[0], f[1], f[2], f[3]};
+                    *reinterpret_cast<elemx4 *>(hg + (int64_t)(vcol0 + li) * K + 16 * kt + 4 * lg) = q4;
+                }
+            }
+            if (stage_h) {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) acc_to_tile(hS, ph, 16 * kt, wv * 16, hacc[kt]);
+            }
+        }
+
+        // v_new = u - w S ;  o = scale qg S
+        f32x4 vn[4], oacc[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) vn[rt] = oacc[rt] = zero4();
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) vn[rt] = mfma16x32(frag_kc(wS, pw, rt * 16, 32 * j), hB[j], vn[rt]);
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(frag_kc(qS, pw, rt * 16, 32 * j), hB[j], oacc[rt]);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vn[rt][e] = (float)uu[e] - vn[rt][e];
+                oacc[rt][e] *= p.scale;
+            }
+        }
+        if (p.v_new) {   // over the wave's own columns of u, which no other wave reads
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
+        }
+        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same 16-bit v_new operand serves both)
+        elemx8 vB[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                if (2 * j <= rt) oacc[rt] = mfma16x32(frag_kc(aS, pb, rt * 16, 32 * j), vB[j], oacc[rt]);
+        if (SUB == 2) {
+            if (!first) {   // second step of a 128-token chunk: the coupling block Aqk21 times the first step's v_new,
+                            // its rows straight from memory (rows past the end re-read the last valid row)
+                const elem *ag = p.aqk + row * (kChunk * SUB) + 4 * lg;
+#pragma unroll
+                for (int rt = 0; rt < 4; ++rt) {
+                    const elem *ar = ag + (int64_t)min(rt * 16 + li, len - 1) * (kChunk * SUB);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        oacc[rt] = mfma16x32(cat8(*reinterpret_cast<const elemx4 *>(ar + 32 * j),
+                                                  *reinterpret_cast<const elemx4 *>(ar + 32 * j + 16)), vprev[j], oacc[rt]);
+                }
+            }
+            vprev[0] = vB[0];
+            vprev[1] = vB[1];
+        }
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) {
+            if (first) hacc[kt] *= lds4(dS + 16 * kt + 4 * lg);
+            hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 0), vB[0], hacc[kt]);
+            hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 32), vB[1], hacc[kt]);
+        }
+        char *ob = og + (int64_t)start * p.o.st * 2;
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) acc_to_global(ob, (int64_t)p.o.st * 2, rt * 16, len, oacc[rt]);
+        __syncthreads();   // every tile has been read; v_new and the state tile are complete
+        if (p.v_new) store_tile<kThreads>(p.v_new + row * V + slab * VS, V, uS, pu, VS, len);
+        if (stage_h && first)
+            store_tile<kThreads>(p.h + b * p.h_sb + (int64_t)chunk * p.h_sc + hv * p.h_sh + slab * VS, V, hS, ph, VS, K);
+        __syncthreads();   // staged outputs read before the next step's tiles replace them
+    }
+
+    if (p.hT) {
+        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[state_off(16 * kt + 4 * lg + e, vcol0 + li)] = hacc[kt][e];
+    }
+}
+
 // =============================================================================================
 // host side
 // =============================================================================================
@@ -1044,6 +1298,17 @@ int launch_scan(const KdaScanParams &p, hipStream_t stream) {
     return FLA_OK;
 }
 
+template <int K, int SUB>
+int launch_scan_wide(const KdaScanParams &p, hipStream_t stream) {
+    const size_t smem = WideScanSmem<K>::bytes;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_wide_kernel<K, SUB>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_wide_kernel<K, SUB>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(kThreads), smem,
+               stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
 int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
                  const fla_tensor *a_log, const fla_tensor *dt_bias, const fla_tensor *initial_state,
                  const fla_int_array *cu, const fla_int_array *ci, const char *layout, double scale, int64_t chunk_size,
@@ -1072,9 +1337,9 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     FLA_REQUIRE(q->shape[L.it] < ((int64_t)1 << 31) && geom.B < 65536, FLA_ERR_SHAPE, "%s: extents too large.", op);
     FLA_REQUIRE(geom.Hk > 0 && geom.Hv >= geom.Hk && geom.Hv % geom.Hk == 0 && geom.Hv <= 128, FLA_ERR_SHAPE,
                 "%s: H/HV must satisfy 0 < H <= HV <= 128 and HV %% H == 0.", op);
-    FLA_REQUIRE((geom.K == 64 || geom.K == 128) && (geom.V == 64 || geom.V == 128 || geom.V == 256) && geom.V >= geom.K,
-                FLA_ERR_UNSUPPORTED, "%s: implemented head sizes are K in {64,128} with V in {K, 2K}, got K=%d V=%d.", op,
-                geom.K, geom.V);
+    FLA_REQUIRE(((geom.K == 64 || geom.K == 128) && (geom.V == geom.K || geom.V == 2 * geom.K)) || (geom.K == 256 && geom.V == 256),
+                FLA_ERR_UNSUPPORTED, "%s: implemented head sizes are K in {64,128} with V in {K, 2K} and K = V = 256, got K=%d V=%d.",
+                op, geom.K, geom.V);
     const int64_t B = geom.B, T = geom.T, Hk = geom.Hk, Hv = geom.Hv, K = geom.K, V = geom.V;
     const int bf = dt_bit(kElemDtype), f32 = dt_bit(FLA_F32);
     KdaIntraParams ip{};
@@ -1205,7 +1470,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     ip.c128 = C == 128;
     ip.x1 = reinterpret_cast<elem *>(wsb + x1_off);
     ip.x2 = reinterpret_cast<elem *>(wsb + x2_off);
-    if (K == 128 && V == 128) rc = launch_intra<128, 128>(ip, stream);
+    if (K == 256) rc = launch_intra<256, 256>(ip, stream);
+    else if (K == 128 && V == 128) rc = launch_intra<128, 128>(ip, stream);
     else if (K == 128 && V == 256) rc = launch_intra<128, 256>(ip, stream);
     else if (K == 64 && V == 64) rc = launch_intra<64, 64>(ip, stream);
     else rc = launch_intra<64, 128>(ip, stream);
@@ -1234,6 +1500,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     sp.v_first = state_v_first;
     sp.scale = (float)scale;
     if (N == 0) return FLA_OK;
+    if (K == 256) return C == 128 ? launch_scan_wide<256, 2>(sp, stream) : launch_scan_wide<256, 1>(sp, stream);
     if (C == 128) return K == 128 ? launch_scan<128, 2>(sp, stream) : launch_scan<64, 2>(sp, stream);
     return K == 128 ? launch_scan<128, 1>(sp, stream) : launch_scan<64, 1>(sp, stream);
 }

@@ -645,17 +645,18 @@ def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial
     if initial_state is not None and (_shape(initial_state) != state_shape or initial_state.dtype != torch.float32):
         raise RuntimeError(f"{op}: initial_state shape/dtype does not match state_v_first.")
 
-    # The kernels are built for K in {64, 128} with V in {K, 2K}.  Every other admitted head size with K <= 128 runs on
-    # the next built size with zero channels appended: a zero q/k channel adds nothing to any product and a zero v
+    # The kernels are built for K in {64, 128} with V in {K, 2K} and for K = V = 256.  Every other admitted head size runs
+    # on the next built size with zero channels appended: a zero q/k channel adds nothing to any product and a zero v
     # column yields zero u, v_new, o and state columns, so the leading K x V part of every result is unchanged.
-    Kp = 64 if K <= 64 and V <= 128 else 128
-    Vp = Kp if V <= Kp else 2 * Kp
     if K > 128:
-        raise NotImplementedError(f"{op}: K={K} has no kernel; built: K <= 128 (V <= 256).")
+        Kp = Vp = 256
+    else:
+        Kp = 64 if K <= 64 and V <= 128 else 128
+        Vp = Kp if V <= Kp else 2 * Kp
     if (Kp, Vp) != (K, V):
         if noalloc:
             raise NotImplementedError(f"{op}: (K,V)=({K},{V}) needs padded copies; the no-allocation entry takes "
-                                      "K in {64,128} with V in {K,2K} only.")
+                                      "K in {64,128} with V in {K,2K} and K = V = 256 only.")
         F = torch.nn.functional
         padk = lambda t: F.pad(t, (0, Kp - K))
         padv = lambda t: F.pad(t, (0, Vp - V))

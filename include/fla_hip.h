@@ -353,7 +353,7 @@ int fla_chunk_gated_delta_rule_bwd_dhu(
  * Aqk, Akk [..HV,T,chunk], w, qg, kg [..HV,T,K], u, v_new [..HV,T,V], and
  * h [B,NT,HV,K,V] (rank-3 layouts: [NT,HV,K,V]).  final_state, gk, w, u, qg,
  * kg, v_new and h may be null.  Implemented: bf16 or f16 q/k/v, chunk_size 64
- * and 128, K in {64,128}, V in {K, 2K}.
+ * and 128, K in {64,128} with V in {K, 2K}, and K = V = 256.
  * ------------------------------------------------------------------------ */
 int fla_chunk_kda_fwd_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,

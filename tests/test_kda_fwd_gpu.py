@@ -99,6 +99,22 @@ CASES += [
 ]
 
 
+# more than 128 channels (up to 256, _aclnn_ctypes.py:1141): kernels for K = V = 256, sizes between on zero channels
+CASES += [
+    dict(B=2, T=200, Hk=2, Hv=4, K=256, V=256, layout="BSND", h0=True),                       # GVA, ragged tail
+    dict(B=1, T=261, Hk=2, Hv=2, K=256, V=256, layout="TND", cu=[0, 1, 16, 33, 33, 96, 160, 261], h0=True),
+    dict(B=1, T=192, Hk=1, Hv=2, K=256, V=256, layout="BNSD", v_first=True, h0=True,
+         gate=dict(use_gate_in_kernel=True, bias=True, safe_gate=True, lower_bound=-5.0), g_dtype=BF, beta_dtype=BF),
+    dict(B=1, T=128, Hk=1, Hv=1, K=256, V=256, layout="BSND", gate_scale=3.0),              # strong decay
+    dict(B=1, T=330, Hk=2, Hv=4, K=256, V=256, layout="BNSD", chunk=128, h0=True),
+    dict(B=1, T=421, Hk=1, Hv=2, K=256, V=256, layout="TND", chunk=128, cu=[0, 1, 66, 66, 194, 300, 421], h0=True,
+         v_first=True),
+    dict(B=1, T=192, Hk=1, Hv=1, K=256, V=256, layout="NTD", chunk=128, gate=dict(use_gate_in_kernel=True, bias=True)),
+    dict(B=1, T=150, Hk=1, Hv=2, K=192, V=96, layout="BSND", h0=True),                       # padded to 256 x 256
+    dict(B=1, T=140, Hk=1, Hv=1, K=144, V=256, layout="BSND", chunk=128, dtype=torch.float16),
+]
+
+
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "-".join(f"{k}{v}" for k, v in c.items() if k in ("T", "K", "V", "layout", "chunk")))
 def test_chunk_kda_fwd(dev, case):
     from fla_hip import ops
