@@ -792,8 +792,8 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
     if ((rc = check_bhtd(op, "u", u, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bht(op, "beta", beta, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr, FLA_ERR_NULL, "%s: g must be provided.", op);
-    FLA_REQUIRE(geom.C == kChunk || (geom.K == 128 && (geom.V == 128 || geom.V == 256)), FLA_ERR_UNSUPPORTED,
-                "%s: chunk_size 128 is built for K=128 with V=128 or 256.", op);
+    FLA_REQUIRE(geom.C == kChunk || ((geom.K == 128 || geom.K == 64) && (geom.V == geom.K || geom.V == 2 * geom.K)),
+                FLA_ERR_UNSUPPORTED, "%s: chunk_size 128 is built for (K,V) in (128,128),(128,256),(64,64),(64,128).", op);
     if ((rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     FLA_REQUIRE(geom.K % 64 == 0 && geom.V % 64 == 0 && geom.K <= 256 && geom.V <= 256, FLA_ERR_UNSUPPORTED,
                 "%s: K and V must be multiples of 64 up to 256, got K=%d V=%d.", op, geom.K, geom.V);
@@ -809,8 +809,10 @@ int wu_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, co
                                           (int)smem));                                                             \
         FLA_LAUNCH("wu", stream, KERNEL, grid, dim3(kThreads), smem, stream, p);                                    \
     } while (0)
-    if (geom.C == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128, 128>));
-    else if (geom.C == 128) FLA_LAUNCH_WU((wu_kernel<128, 256, 128>));
+    if (geom.C == 128 && geom.K == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128, 128>));
+    else if (geom.C == 128 && geom.K == 128) FLA_LAUNCH_WU((wu_kernel<128, 256, 128>));
+    else if (geom.C == 128 && geom.V == 64) FLA_LAUNCH_WU((wu_kernel<64, 64, 128>));
+    else if (geom.C == 128) FLA_LAUNCH_WU((wu_kernel<64, 128, 128>));
     else if (geom.K == 128 && geom.V == 128) FLA_LAUNCH_WU((wu_kernel<128, 128>));
     else if (geom.K == 128 && geom.V == 256) FLA_LAUNCH_WU((wu_kernel<128, 256>));
     else if (geom.K == 64 && geom.V == 64) FLA_LAUNCH_WU((wu_kernel<64, 64>));
@@ -860,7 +862,9 @@ int fwd_o_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (geom.C == 128) {
         if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128, 2>(p, stream);
         if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256, 2>(p, stream);
-        return fail(FLA_ERR_UNSUPPORTED, "%s: chunk_size 128 is built for K=128 with V=128 or 256.", op);
+        if (geom.K == 64 && geom.V == 64) return launch_fwd_o<64, 64, 2>(p, stream);
+        if (geom.K == 64 && geom.V == 128) return launch_fwd_o<64, 128, 2>(p, stream);
+        return fail(FLA_ERR_UNSUPPORTED, "%s: chunk_size 128 is built for (K,V) in (128,128),(128,256),(64,64),(64,128).", op);
     }
     if (geom.K == 128 && geom.V == 128) return launch_fwd_o<128, 128>(p, stream);
     if (geom.K == 128 && geom.V == 256) return launch_fwd_o<128, 256>(p, stream);

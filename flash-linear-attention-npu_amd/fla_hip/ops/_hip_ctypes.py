@@ -964,7 +964,8 @@ def _two_value_passes(v, chunk_size) -> bool:
     """The 128-token forms of chunk_bwd_dqkwg and of the WY backward operators hold 128 value columns.  With 256 they run
     twice, over 128 columns each: every result is either a per-column one (dv) or a sum over the value columns that is
     linear in the column-wise operands, so the two passes add up (the second one sees zeros for the operands that do
-    not belong to the value dimension)."""
+    not belong to the value dimension).  Each pass returns its part in the 16-bit element type, so a sum carries one more
+    rounding than a single pass, at the magnitude of the parts: visible where the two parts nearly cancel."""
     return int(chunk_size) == 128 and int(v.shape[-1]) == 256
 
 
