@@ -639,6 +639,21 @@ def bench_gdn_bwd(args, torch, dev):
 
     ms_train = timed(train_step)
     ms_fwd_train = timed(fwd_train)
+
+    # the same step as a model runs it: token-major q, k, v (one row per token holds every head, as a projection
+    # leaves them) through the autograd entry, without and with the row normalisation of q and k inside the kernels
+    def autograd_step(l2norm):
+        tq, tk, tv = (t.transpose(1, 2).contiguous().transpose(1, 2).detach().requires_grad_(True) for t in (q, k, v))
+        tg, tb = gate.detach().clone().requires_grad_(True), beta.detach().clone().requires_grad_(True)
+
+        def run():
+            o, _ = pipeline.flash_gated_delta_rule(tq, tk, tv, tg, tb, output_final_state=True, use_qk_l2norm_in_kernel=l2norm)
+            o.backward(do)
+            for t in (tq, tk, tv, tg, tb):
+                t.grad = None
+        return timed(run)
+
+    ms_autograd, ms_autograd_l2 = autograd_step(False), autograd_step(True)
     ms_fwd_plain = timed(lambda: pipeline.flash_chunk_gated_delta_rule_fwd(q, k, v, gate, beta, scale, h0, True, None, C))
     lib.fla_profile_enable.argtypes = [ctypes.c_int]
     lib.fla_profile_enable(1)
@@ -689,7 +704,9 @@ def bench_gdn_bwd(args, torch, dev):
         "ms_per_step_with_saved_A": round(ms_saved_A, 4),
         "training": {"fwd_bwd_ms": round(ms_train, 4), "fwd_saving_h_vnew_w_ms": round(ms_fwd_train, 4),
                      "bwd_with_saved_ms": round(ms_train - ms_fwd_train, 4), "fwd_inference_ms": round(ms_fwd_plain, 4),
-                     "fwd_inference_plus_bwd_recompute_ms": round(ms_fwd_plain + ms_per_step, 4)},
+                     "fwd_inference_plus_bwd_recompute_ms": round(ms_fwd_plain + ms_per_step, 4),
+                     "autograd_token_major_ms": round(ms_autograd, 4),
+                     "autograd_token_major_qk_l2norm_ms": round(ms_autograd_l2, 4)},
         "step_tflops": round(step_flops / (ms_per_step * 1e-3) / 1e12, 2),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
