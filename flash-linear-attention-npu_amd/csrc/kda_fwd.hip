@@ -108,11 +108,35 @@ template <int K, int V> struct IntraSmem {
     static constexpr size_t v_off = WIDE ? g_off : k_off + (size_t)kChunk * pk * 2;
     static constexpr size_t aq_off = WIDE ? g_off + (size_t)kChunk * pv * 2 : ak_off + (size_t)kChunk * pb * 2;
     static constexpr size_t a_off = g_off + g_bytes;                       // fp32 scores [kChunk][pa], then beta [kChunk]
-    static constexpr size_t t_off = WIDE ? a_off : a_off + (size_t)kChunk * (pa + 1) * 4;   // scan scratch [2 SEG][K]
-    static constexpr size_t bytes = WIDE ? a_off + (size_t)kChunk * (pa + 1) * 4 : t_off + (size_t)2 * SEG * K * 4;
-    static_assert(!WIDE || ((size_t)kChunk * (pv + pb) * 2 <= g_bytes && (size_t)2 * SEG * K <= (size_t)kChunk * pa),
-                  "the tiles that replace the gate tile and the scan scratch must fit where they are put");
+    static constexpr size_t t_off = a_off;                                 // scan scratch [2 SEG][K], dead before the scores
+    // FACT: the right-hand score operand k_j 2^{s_R - g_j} (s_R = gate at the last row of row tile R) is formed as
+    // (k_j 2^{s_c - g_j}) 2^{s_R - s_c}, c the 16-row tile of j: a tile computed once per chunk and a [6][K] table of the
+    // tile-to-tile factors, instead of eight exponentials per operand fragment in every wave that needs it.
+    static constexpr bool FACT = !WIDE;
+    static constexpr size_t kh_off = a_off + (size_t)kChunk * (pa + 1) * 4;
+    static constexpr size_t f_off = kh_off + (FACT ? (size_t)kChunk * pk * 2 : 0);
+    static constexpr size_t bytes = f_off + (FACT ? (size_t)6 * K * 4 : 0);
+    static_assert((size_t)2 * SEG * K <= (size_t)kChunk * pa, "the scan scratch must fit the score tile it lies over");
+    static_assert(!WIDE || (size_t)kChunk * (pv + pb) * 2 <= g_bytes, "the tiles that replace the gate tile must fit it");
 };
+
+// rows 16c.. of the tile k 2^{s_c - g} times the factor 2^{s_R - s_c} of the row tile R > c it is paired with (none on
+// the diagonal), as an MFMA operand with contraction slots 32j .. 32j+31 along the channels
+template <int K>
+__device__ __forceinline__ elemx8 paired_frag(const elem *khS, int pk, const float *fS, int R, int c, int j) {
+    const elemx8 raw = frag_kc(khS, pk, 16 * c, 32 * j);
+    if (c == R) return raw;
+    const int lg = lane_id() >> 4;
+    const float *f = fS + (R * (R - 1) / 2 + c) * K + 32 * j + 4 * lg;
+    const f32x4 f0 = lds4(f), f1 = lds4(f + 16);
+    f32x4 lo, hi;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        lo[e] = (float)raw[e] * f0[e];
+        hi[e] = (float)raw[4 + e] * f1[e];
+    }
+    return frag_from_acc(lo, hi);
+}
 
 // Everything a wave does after the gate scan.  Eight waves: wave W of role 0 owns row tile W of k k^T (with the
 // diagonal block inverse and the off-diagonal solve of column block W) and later row tile W of w; wave W of role 1
@@ -121,7 +145,7 @@ template <int K, int V> struct IntraSmem {
 template <int K, int V, int W, int ROLE, bool C128>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
-                                           int64_t dec_base, int half, const elem *vg) {
+                                           int64_t dec_base, int half, const elem *vg, const elem *khS, const float *fS) {
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb;
     constexpr int KS = K / 32, R1 = W, R2 = 3 - W;
@@ -155,7 +179,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
                 const elemx8 lk = scaled_frag<true>(kS, pk, gS, pg, 16 * R1, 16 * R1 + 15, j);
 #pragma unroll
                 for (int c = 0; c <= R1; ++c) {
-                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R1 + 15, j);
+                    const elemx8 rk = paired_frag<K>(khS, pk, fS, R1, c, j);
                     kacc[c] = mfma16x32(lk, rk, kacc[c]);
                     if (c == R1) kaccT = mfma16x32(rk, lk, kaccT);
                 }
@@ -185,7 +209,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
                 const elemx8 lq = scaled_frag<true>(qS, pq, gS, pg, 16 * R2, 16 * R2 + 15, j);
 #pragma unroll
                 for (int c = 0; c <= R2; ++c) {
-                    const elemx8 rk = scaled_frag<false>(kS, pk, gS, pg, 16 * c, 16 * R2 + 15, j);
+                    const elemx8 rk = paired_frag<K>(khS, pk, fS, R2, c, j);
                     qacc[c] = mfma16x32(lq, rk, qacc[c]);
                 }
             }
@@ -370,6 +394,8 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     float *aS = reinterpret_cast<float *>(smem + S::a_off);
     float *bS = aS + kChunk * pa;
     float *tS = reinterpret_cast<float *>(smem + S::t_off);
+    elem *khS = reinterpret_cast<elem *>(smem + S::kh_off);
+    float *fS = reinterpret_cast<float *>(smem + S::f_off);
 
     int cx, hv;
     block_chunk_head(p.geom, cx, hv);
@@ -439,6 +465,27 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
             const int r = (m * kIntraThreads + tid) / (V / 8);
             br[m] = load_scalar(p.beta, b, hv, start + min(r, len - 1));
         }
+        {   // segment sums of the gates (they were requested first) while the tiles are still on their way
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < TS; ++j) {
+                const int t = sg * TS + j;
+                if (t < len) {
+                    const float a = p.use_gate ? kda_activate(raw[j], bias, eig, p.safe_gate, p.lower_bound) : raw[j];
+                    acc += a * kRcpLn2;
+                }
+                raw[j] = acc;   // the running sum within the segment stays in the register of its gate
+            }
+            tS[sg * K + ch] = acc;
+            float oacc = 0.f;
+            if constexpr (C128) {
+#pragma unroll
+                for (int j = 0; j < TS; ++j)
+                    if (sg * TS + j < olen)
+                        oacc += (p.use_gate ? kda_activate(oraw[j], bias, eig, p.safe_gate, p.lower_bound) : oraw[j]) * kRcpLn2;
+            }
+            tS[(SEG + sg) * K + ch] = oacc;
+        }
         tq.commit(qS, pq, len, tid);
         tk.commit(kS, pk, len, tid);
 #pragma unroll
@@ -459,31 +506,15 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
     if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
 
     {
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < TS; ++j) {
-            const int t = sg * TS + j;
-            if (t < len) {
-                const float a = p.use_gate ? kda_activate(raw[j], bias, eig, p.safe_gate, p.lower_bound) : raw[j];
-                acc += a * kRcpLn2;
-            }
-            gS[t * pg + ch] = acc;
-        }
-        tS[sg * K + ch] = acc;
-        float oacc = 0.f;
-        if constexpr (C128) {
-#pragma unroll
-            for (int j = 0; j < TS; ++j)
-                if (sg * TS + j < olen)
-                    oacc += (p.use_gate ? kda_activate(oraw[j], bias, eig, p.safe_gate, p.lower_bound) : oraw[j]) * kRcpLn2;
-        }
-        tS[(SEG + sg) * K + ch] = oacc;
         __syncthreads();
         float off = 0.f, own = 0.f, other = 0.f;
+        float upto[SEG];   // gate at the end of every segment, relative to the start of this half
+#pragma unroll
         for (int s = 0; s < SEG; ++s) {
             const float v = tS[s * K + ch];
             if (s < sg) off += v;
             own += v;
+            upto[s] = own;
             other += tS[(SEG + s) * K + ch];
         }
         if (half) off += other;   // gates of the second half continue those of the first
@@ -495,23 +526,46 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
 #pragma unroll
         for (int j = 0; j < TS; ++j) {
             const int t = sg * TS + j;
-            const float v = gS[t * pg + ch] + off;
+            const float v = raw[j] + off;
             gS[t * pg + ch] = v;
             if (gkp != nullptr && t < len) gkp[t * K] = v;
+        }
+        if constexpr (S::FACT) {
+            // k 2^{s_c - g} for this thread's tokens (s_c: the gate at the last row of their 16-row tile) and, from the
+            // first segment's threads, the tile-to-tile factors 2^{s_R - s_c} of the channel
+            constexpr int SPT = 16 / TS;   // segments per 16-row tile
+            static_assert(TS <= 16 && 16 % TS == 0, "a segment must not straddle two row tiles");
+            float anchor = 0.f;
+#pragma unroll
+            for (int s = 0; s < SEG; ++s)
+                if (s == (sg / SPT) * SPT + SPT - 1) anchor = upto[s];
+            anchor += half ? other : 0.f;
+#pragma unroll
+            for (int j = 0; j < TS; ++j) {
+                const int t = sg * TS + j;
+                khS[t * pk + ch] = (elem)((float)kS[t * pk + ch] * ex2(anchor - (raw[j] + off)));
+            }
+            if (sg == 0) {
+#pragma unroll
+                for (int R = 1; R < 4; ++R)
+#pragma unroll
+                    for (int cc = 0; cc < R; ++cc)
+                        fS[(R * (R - 1) / 2 + cc) * K + ch] = ex2(upto[R * SPT + SPT - 1] - upto[cc * SPT + SPT - 1]);
+            }
         }
     }
     __syncthreads();
 
     const int64_t dec_base = half ? -1 : (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
-        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg); break;
+        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
     }
 
     store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
