@@ -116,6 +116,9 @@ template <int K, int V> struct IntraSmem {
     static constexpr size_t kh_off = a_off + (size_t)kChunk * (pa + 1) * 4;
     static constexpr size_t f_off = kh_off + (FACT ? (size_t)kChunk * pk * 2 : 0);
     static constexpr size_t bytes = f_off + (FACT ? (size_t)6 * K * 4 : 0);
+    // w and u leave through LDS as whole rows.  Where the dead k 2^{s_c - g} tile and the dead gate tile can take them
+    // (pitches pk and pv), the products are staged there at once; otherwise over their own operand tiles, behind a barrier.
+    static constexpr bool FREE_STAGE = FACT && (size_t)kChunk * pv * 2 <= g_bytes;
     static_assert((size_t)2 * SEG * K <= (size_t)kChunk * pa, "the scan scratch must fit the score tile it lies over");
     static_assert(!WIDE || (size_t)kChunk * (pv + pb) * 2 <= g_bytes, "the tiles that replace the gate tile must fit it");
 };
@@ -369,11 +372,20 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             }
         }
     }
-    __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
+    if constexpr (S::FREE_STAGE) {   // nobody reads the two dead tiles any more
+        elem *wT = const_cast<elem *>(khS), *uT = reinterpret_cast<elem *>(gS);
 #pragma unroll
-    for (int ct = 0; ct < NCT; ++ct) {
-        if constexpr (ROLE == 0) acc_to_tile(qS, pq, 16 * W, 16 * ct, oacc[ct]);
-        else acc_to_tile(vS, pv, 16 * W, 16 * ct, oacc[ct]);
+        for (int ct = 0; ct < NCT; ++ct) {
+            if constexpr (ROLE == 0) acc_to_tile(wT, pk, 16 * W, 16 * ct, oacc[ct]);
+            else acc_to_tile(uT, pv, 16 * W, 16 * ct, oacc[ct]);
+        }
+    } else {
+        __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) {
+            if constexpr (ROLE == 0) acc_to_tile(qS, pq, 16 * W, 16 * ct, oacc[ct]);
+            else acc_to_tile(vS, pv, 16 * W, 16 * ct, oacc[ct]);
+        }
     }
     __syncthreads();
 }
@@ -568,8 +580,13 @@ __global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntra
         default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
     }
 
-    store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
-    store_tile<kIntraThreads>(p.u + row_base * V, V, vS, pv, V, len);
+    if constexpr (S::FREE_STAGE) {
+        store_tile<kIntraThreads>(p.w + row_base * K, K, khS, pk, K, len);
+        store_tile<kIntraThreads>(p.u + row_base * V, V, reinterpret_cast<const elem *>(gS), pv, V, len);
+    } else {
+        store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
+        store_tile<kIntraThreads>(p.u + row_base * V, V, vS, pv, V, len);
+    }
     const int C = p.geom.C;
     store_tile<kIntraThreads>(p.aqk + row_base * C + kChunk * half, C, aqS, pb, kChunk, len);
     store_tile<kIntraThreads>(p.akk + row_base * C + kChunk * half, C, akS, pb, kChunk, len);
