@@ -157,6 +157,10 @@ __device__ __forceinline__ void split_hilo(f32x4 x, elemx4 &hi, elemx4 &lo) {
 // Persistent scans launch a (slabs, heads, sequences) grid: the `slabs` workgroups of one (sequence, head) chain read
 // the same key-side operands.  Workgroups are handed to the eight XCDs in turn (linear id % 8), each XCD with an L2 of
 // its own, so ids L, L + 8, ... go to one chain and its second and later reads of those operands hit that L2.
+// For kernels whose LDS footprint or launch shape leaves two waves on a SIMD whatever their register count: tells the
+// compiler that keeping registers low buys no occupancy, so that it schedules for latency instead.
+#define FLA_TWO_WAVES_PER_SIMD __attribute__((amdgpu_waves_per_eu(2, 2)))
+
 __device__ __forceinline__ void chain_of_block(int &slab, int &head, int &seq) {
     const int slabs = gridDim.x, heads = gridDim.y, total = slabs * heads * gridDim.z;
     const int lin = blockIdx.x + slabs * (blockIdx.y + heads * blockIdx.z);

@@ -393,7 +393,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
 // C128: the workgroup owns one half of a 128-token chunk (a template flag, so that the 64-token form carries none of
 // the second gate stream, the coupling operands or the zero fill).
 template <int K, int V, bool C128>
-__global__ void __launch_bounds__(kIntraThreads) kda_intra_kernel(const KdaIntraParams p) {
+__global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intra_kernel(const KdaIntraParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
     constexpr int pq = S::pq, pk = S::pk, pg = S::pg, pv = S::pv, pa = S::pa, pb = S::pb, SEG = S::SEG;
