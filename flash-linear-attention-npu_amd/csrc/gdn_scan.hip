@@ -405,7 +405,8 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
                     (long long)d2, (long long)d3);
     }
     FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
-    FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
+    FLA_REQUIRE(geom.K == 128 || geom.K == 64 || (geom.K == 256 && has_gk), FLA_ERR_UNSUPPORTED,
+                "%s: K must be 64 or 128 (256 with gK), got %d.", op, geom.K);
     if (query) {
         *query = vl.bytes();
         return FLA_OK;
@@ -787,6 +788,148 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             }
 }
 
+// More than 128 channels (per-channel gate only): the k, q and w tiles of one step fill the LDS, so nothing is
+// double-buffered.  256 threads: all four waves copy the tiles of a step, then compute it with the 256 x 16 gradient of
+// each wave in registers; dh and dv2 leave straight from the accumulators.  Two barriers a step.
+template <int K> struct WideDhuSmem {
+    static constexpr int pk = K + 8, pt = K + 16, pv = 64 + 16;
+    static constexpr size_t k_off = 0;
+    static constexpr size_t q_off = k_off + (size_t)kChunk * pk * 2;
+    static constexpr size_t w_off = q_off + (size_t)kChunk * pt * 2;
+    static constexpr size_t o_off = w_off + (size_t)kChunk * pt * 2;
+    static constexpr size_t v_off = o_off + (size_t)kChunk * pv * 2;
+    static constexpr size_t g_off = v_off + (size_t)kChunk * pv * 2;
+    static constexpr size_t bytes = g_off + (size_t)K * 4;
+};
+
+template <int K>
+__global__ void __launch_bounds__(kThreads) bwd_dhu_wide_kernel(const DhuParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef WideDhuSmem<K> L;
+    constexpr int VS = 64;
+    constexpr int pk = L::pk, pt = L::pt, pv = L::pv;
+    constexpr int KT = K / 16, KS = K / 32;
+    elem *kS = reinterpret_cast<elem *>(smem + L::k_off), *qS = reinterpret_cast<elem *>(smem + L::q_off);
+    elem *wS = reinterpret_cast<elem *>(smem + L::w_off), *oS = reinterpret_cast<elem *>(smem + L::o_off);
+    elem *vS = reinterpret_cast<elem *>(smem + L::v_off);
+    float *gS = reinterpret_cast<float *>(smem + L::g_off);
+
+    int slab, hv, n;
+    chain_of_block(slab, hv, n);
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    const int V = p.geom.V;
+    int b = n, bos = 0, eos = p.geom.T, chunk0 = 0;
+    if (p.geom.cu != nullptr) {
+        b = 0;
+        bos = p.geom.cu[n];
+        eos = p.geom.cu[n + 1];
+        chunk0 = p.geom.choff[n];
+    }
+    const int nchunks = (eos - bos + kChunk - 1) / kChunk;
+    const elem *qg = static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh;
+    const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
+    const elem *wg = static_cast<const elem *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
+    const elem *og = static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
+    const elem *vg = static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
+    const int tid = threadIdx.x, wv = wave_id();
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const int vcol0 = slab * VS + wv * 16;
+
+    f32x4 dacc[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+        f32x4 a = {0.f, 0.f, 0.f, 0.f};
+        if (p.dht) {
+            const float *s = p.dht + n * p.t_sn + hv * p.t_sh;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li];
+        }
+        dacc[kt] = a;
+    }
+
+    for (int c = nchunks - 1; c >= 0; --c) {
+        const int start = bos + c * kChunk;
+        const int len = min(kChunk, eos - start);
+        load_tile<kThreads>(kS, pk, kg + (int64_t)start * p.k.st, p.k.st, kChunk, K, len);
+        load_tile<kThreads>(qS, pt, qg + (int64_t)start * p.q.st, p.q.st, kChunk, K, len);
+        load_tile<kThreads>(wS, pt, wg + (int64_t)start * p.w.st, p.w.st, kChunk, K, len);
+        load_tile<kThreads>(oS, pv, og + (int64_t)start * p.d_o.st, p.d_o.st, kChunk, VS, len);
+        load_tile<kThreads>(vS, pv, vg + (int64_t)start * p.dv.st, p.dv.st, kChunk, VS, len);
+        for (int i = tid; i < K; i += kThreads)
+            gS[i] = exp2f(p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + i]);
+        __syncthreads();
+
+        // dh of this chunk = the incoming gradient; k . dh uses its 16-bit copy
+        elemx8 hB[KS];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(dacc[2 * j], dacc[2 * j + 1]);
+        {
+            char *hg = reinterpret_cast<char *>(p.dh + b * p.h_sb + hv * p.h_sh + (int64_t)(chunk0 + c) * p.h_sc + vcol0);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) acc_to_global(hg, (int64_t)V * 2, 16 * kt, K, dacc[kt]);
+        }
+        // dv2 = dv + k . dh   (k arrives gated)
+        f32x4 dv2[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) dv2[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) dv2[rt] = mfma16x32(frag_kc(kS, pk, rt * 16, 32 * j), hB[j], dv2[rt]);
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) {
+            const elemx4 old = frag_tr4(vS, pv, wv * 16, rt * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dv2[rt][e] = rt * 16 + 4 * lg + e < len ? dv2[rt][e] + (float)old[e] : 0.f;
+        }
+        {
+            char *v2 = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv2.p)) + b * p.dv2.sb + hv * p.dv2.sh +
+                                                (int64_t)start * p.dv2.st + vcol0);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) acc_to_global(v2, p.dv2.st * 2, 16 * rt, len, dv2[rt]);
+        }
+        // dh <- 2^{gK_last} dh + scale q^T do - w^T dv2   (q arrives gated)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) dacc[kt] *= *reinterpret_cast<const f32x4 *>(gS + 16 * kt + 4 * lg);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const elemx8 raw = frag_tr(oS, pv, wv * 16, 32 * j);
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)raw[e] * p.scale;
+                hi[e] = (float)raw[4 + e] * p.scale;
+            }
+            const elemx8 ob = frag_from_acc(lo, hi), nb = frag_from_acc(-dv2[2 * j], -dv2[2 * j + 1]);
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                dacc[kt] = mfma16x32(frag_tr(qS, pt, kt * 16, 32 * j), ob, dacc[kt]);
+                dacc[kt] = mfma16x32(frag_tr(wS, pt, kt * 16, 32 * j), nb, dacc[kt]);
+            }
+        }
+        __syncthreads();   // every tile has been read before the next step's tiles replace them
+    }
+
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int64_t off = (int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li;
+            if (p.dh0_f32) p.dh0_f32[n * p.z_sn + hv * p.z_sh + off] = dacc[kt][e];
+            if (p.dh0_ref && nchunks > 0) p.dh0_ref[b * p.h_sb + hv * p.h_sh + (int64_t)chunk0 * p.h_sc + off] = (elem)dacc[kt][e];
+        }
+}
+
+template <int K>
+int launch_bwd_dhu_wide(const DhuParams &p, int slabs, hipStream_t stream) {
+    const size_t smem = WideDhuSmem<K>::bytes;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_wide_kernel<K>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_wide_kernel<K>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(kThreads), smem, stream, p);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
 template <int K, bool GK>
 int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
     const size_t smem = DhuSmem<K>::bytes;
@@ -860,7 +1003,8 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
                         dht->stride[3] == 1 && dht->stride[2] == geom.V,
                     FLA_ERR_SHAPE, "%s: dht must be fp32 [N=%d,Hv,K,V].", op, geom.N);
     }
-    FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
+    FLA_REQUIRE(geom.K == 128 || geom.K == 64 || (geom.K == 256 && has_gk), FLA_ERR_UNSUPPORTED,
+                "%s: K must be 64 or 128 (256 with gK), got %d.", op, geom.K);
     FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
     if (query) {
         *query = vl.bytes();
@@ -907,6 +1051,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.scale = (float)scale;
     p.sub = geom.C / kChunk;
     const int slabs = geom.V / 64;
+    if (geom.K == 256) return launch_bwd_dhu_wide<256>(p, slabs, stream);
     if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, true>(p, slabs, stream) : launch_bwd_dhu<128, false>(p, slabs, stream);
     return has_gk ? launch_bwd_dhu<64, true>(p, slabs, stream) : launch_bwd_dhu<64, false>(p, slabs, stream);
 }

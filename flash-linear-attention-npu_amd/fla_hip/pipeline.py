@@ -305,9 +305,13 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     dh, dh0, dv2 = _ops.chunk_gated_delta_rule_bwd_dhu(qg4, kg4, w4, doh, dv0, scale, chunk_size, gK=gk4,
                                                        h0=initial_state, dht=dht, use_exp2=True, dh0_per_sequence=True,
                                                        **kw)
-    dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
-                                              layout_like=layout_like, **kw)
-    dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
+    if qh.shape[-1] > 128:
+        dq, dk, dg, dv, db, dAkk = _kda_bwd_state_stages_by_channel_halves(qh, kh, vh, bh, gk4, Akk4, vn4, h5, doh, dh, dv2, scale,
+                                                                            chunk_size, layout_like, kw)
+    else:
+        dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
+                                                  layout_like=layout_like, **kw)
+        dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
     # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
     back = lambda t: _from_index_order(t, layout)
     if Hv == Hk:          # dq, dk are final with the last stage: it writes them in the dtype of q and k
@@ -322,6 +326,39 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
         dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2).to(q.dtype)
         dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2).to(k.dtype)
     return (back(dq), back(dk), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
+
+
+def _kda_bwd_state_stages_by_channel_halves(qh, kh, vh, bh, gk4, Akk4, vn4, h5, doh, dh, dv2, scale, chunk_size, layout_like, kw):
+    """``chunk_kda_bwd_dqkwg`` and ``chunk_kda_bwd_wy`` for 256 channels on their 128-channel kernels.  Both stages are
+    channel-wise except for sums over the channels that enter linearly: dq, dk, dw, dg of a channel need the state rows
+    h[c,:], dh[c,:] of that channel only; in the WY backward dk and dg are channel-wise, while dAkk and dbeta add a part
+    per channel half to the part of the value columns, which the first pass carries alone (the second one is given
+    du = 0).  Returns (dq, dk, dg, dv, dbeta, dAkk) as the two stages leave them for 128 channels."""
+    import torch
+
+    K = qh.shape[-1]
+    assert K == 256, K
+    parts, dv, db, dAkk = [], None, None, None
+    for lo in (0, 128):
+        sl = slice(lo, lo + 128)
+        q_, k_, g_ = qh[..., sl].contiguous(), kh[..., sl].contiguous(), gk4[..., sl].contiguous()
+        h_, dh_ = h5[..., sl, :].contiguous(), dh[..., sl, :].contiguous()
+        dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(q_, k_, vn4, g_, h_, doh, dh_, dv2, scale, chunk_size,
+                                                  layout_like=None if layout_like is None else layout_like[..., sl], **kw)
+        du = dv2 if lo == 0 else torch.zeros_like(dv2)
+        dv_, db_, dA_ = _raw.chunk_kda_bwd_wy(k_, vh, bh, g_, Akk4, dw, du, dk, dg, chunk_size, **kw)
+        parts.append((dq, dk, dg))
+        if lo == 0:
+            dv, db, dAkk = dv_, db_, dA_
+        else:
+            db, dAkk = db + db_, dAkk + dA_
+    like = parts[0][0] if layout_like is None else layout_like
+
+    def joined(i):
+        out = _raw._empty_strided_like(tuple(parts[0][i].shape[:-1]) + (K,), like, torch.float32, parts[0][i].device)
+        out[..., :128], out[..., 128:] = parts[0][i], parts[1][i]
+        return out
+    return joined(0), joined(1), joined(2), dv, db, dAkk
 
 
 def _empty_in_layout(layout, index_shape):
@@ -404,8 +441,9 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     ``chunk_kda_bwd`` returns dq, dk, dv, dg, dbeta, dh0.  With ``use_gate_in_kernel`` g is the raw gate input and the
     forward kernel activates it; with gradients ``kda_gate_bwd`` ends the backward, so that autograd also reaches
     ``A_log`` and ``dt_bias`` (for a head size served by padding or by two value passes the activation runs as tensor
-    operations ahead of the kernels instead).  Gradients cover every admitted head size with
-    K <= 128 (V up to 256 as two passes over 128 value columns) and run on 64-token tiles whatever ``chunk_size``."""
+    operations ahead of the kernels instead).  Gradients cover every admitted head size (V above 128 as two passes over
+    128 value columns; K above 128 on 256 channels, with the two state-dependent stages run per channel half) and run on
+    64-token tiles whatever ``chunk_size``."""
     import torch
 
     if scale is None:
@@ -424,6 +462,8 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     # backward kernel is (npu_chunk_kda_bwd_intra, _aclnn_ctypes.py:1582-1584), so a differentiated call runs on them.
     chunk_size = 64
     K, V = q.shape[-1], v.shape[-1]
+    if K < 16 or K > 256 or K % 16 or V < 16 or V > 256 or V % 16:      # _aclnn_ctypes.py:1141
+        raise RuntimeError("chunk_kda: K/V must be multiples of 16 with K,V <= 256.")
     gate_args = ()
     if use_gate_in_kernel:
         if A_log is None:
@@ -434,8 +474,6 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
             gate_args = (A_log, dt_bias, bool(safe_gate), lower_bound)
         else:   # the activation as tensor operations ahead of the padding and the split below
             g = _kda_gate_activation(g, A_log, dt_bias, layout, safe_gate, lower_bound)
-    if K > 128:
-        raise NotImplementedError(f"chunk_kda: gradients are built for K <= 128, got K={K}.")
     if V > 128:
         # Value columns never mix: o[.., c] and the state column c depend on v[.., c] only.  Two passes over 128 columns
         # each share q, k, g and beta, whose gradients autograd adds up.
@@ -450,12 +488,12 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     global _KDA_FUNCTION
     if _KDA_FUNCTION is None:
         _KDA_FUNCTION = _kda_autograd_function()
-    # The backward kernels are built for (K, V) in {(64,64), (64,128), (128,128)}.  Other admitted head sizes up to
-    # 128 x 128 run on the next built one with zero channels appended (a zero q/k channel adds nothing to any product, a
+    # The backward kernels are built for (K, V) in {(64,64), (64,128), (128,128)}, and (256,128) is composed from them
+    # (chunk_kda_bwd).  Other admitted head sizes run on the next of these with zero channels appended (a zero q/k channel adds nothing to any product, a
     # zero v column yields zero columns of o and of the state); the padding is itself differentiable, so autograd
     # returns the gradients of the unpadded tensors.
-    Kp = 64 if K <= 64 else 128
-    Vp = Kp if V <= Kp else 128
+    Kp = 64 if K <= 64 else (128 if K <= 128 else 256)
+    Vp = 128 if Kp == 256 else (Kp if V <= Kp else 128)
     if (Kp, Vp) != (K, V):
         F = torch.nn.functional
         h0 = None if initial_state is None else F.pad(initial_state, (0, Vp - V, 0, Kp - K))

@@ -326,7 +326,8 @@ int fla_kda_gate_bwd(
  * h0 is only a presence flag for the caller; dht [N,Hv,K,V] f32 optional.
  * Outputs dh [B,Hv,NT,K,V] bf16, dv2 like dv, dh0 optional: either the
  * reference form (bf16, shape of dh, written at each sequence's first chunk)
- * or f32 [N,Hv,K,V].
+ * or f32 [N,Hv,K,V].  Implemented: K in {64,128} (K = 256 with gK), V a
+ * multiple of 64; chunk_size 64, and 128 with the scalar gate.
  * ------------------------------------------------------------------------ */
 int fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o,

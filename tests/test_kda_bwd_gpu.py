@@ -182,6 +182,10 @@ COMPOSITION_CASES = [
     dict(B=1, T=100, Hk=1, Hv=1, K=48, V=192, layout="BNSD", h0=True, dht=True),
     # a 128-token chunk size asks for the same function
     dict(B=1, T=200, Hk=1, Hv=2, K=128, V=128, layout="BSND", h0=True, dht=True, chunk=128),
+    # more than 128 channels: the wide reverse scan, the state stages by channel halves, chunk_kda_bwd_intra for K = 256
+    dict(B=2, T=150, Hk=1, Hv=2, K=256, V=128, layout="BSND", h0=True, dht=True),
+    dict(B=1, T=261, Hk=2, Hv=2, K=256, V=256, layout="TND", cu=[0, 1, 16, 33, 33, 96, 160, 261], h0=True, dht=True),
+    dict(B=1, T=100, Hk=1, Hv=1, K=192, V=80, layout="BNSD", h0=True),
 ]
 
 
@@ -328,6 +332,6 @@ def test_chunk_kda_rejections(dev):
     beta = torch.ones(1, 64, 1, device=dev)
     with pytest.raises(RuntimeError, match="chunk_size must be 64 or 128"):
         pipeline.chunk_kda(q, q, q, g, beta, chunk_size=32)
-    q = torch.zeros(1, 64, 1, 144, dtype=BF, device=dev, requires_grad=True)
-    with pytest.raises(NotImplementedError, match="K <= 128"):
-        pipeline.chunk_kda(q, q, q, torch.zeros(1, 64, 1, 144, device=dev), beta)
+    q = torch.zeros(1, 64, 1, 272, dtype=BF, device=dev, requires_grad=True)
+    with pytest.raises(RuntimeError, match="K/V must be multiples of 16 with K,V <= 256"):
+        pipeline.chunk_kda(q, q, q, torch.zeros(1, 64, 1, 272, device=dev), beta)

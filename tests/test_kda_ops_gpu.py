@@ -83,6 +83,8 @@ DHU_CASES = [
     (1, 130, 2, 2, 64, 64, None, False, False),
     (1, 130, 1, 2, 64, 128, None, True, True),
     (1, 96, 1, 1, 128, 256, None, False, False),
+    (2, 200, 1, 2, 256, 128, None, True, True),                       # 256 channels: the unpipelined per-channel scan
+    (1, 261, 2, 2, 256, 256, [0, 1, 16, 33, 33, 96, 160, 261], True, True),
 ]
 
 
