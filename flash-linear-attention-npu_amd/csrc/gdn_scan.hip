@@ -498,14 +498,24 @@ template <int K> struct DhuSmem {
     static constexpr size_t g_off = v_off + (size_t)kChunk * pv * 2;      // [max(K,64)] gate row, [64] factors
     static constexpr size_t buf_bytes = g_off + (size_t)((K > kChunk ? K : kChunk) + kChunk) * 4;
     static constexpr size_t bytes = 2 * buf_bytes;
+    // the form that builds dv itself: four strips [16][ptl] behind the two buffers, one per copying wave
+    static constexpr int ptl = kChunk + 8;
+    static constexpr size_t t_off = bytes;
+    static constexpr size_t bytes_dvl = t_off + (size_t)4 * 16 * ptl * 2;
 };
 
 // 512 threads: waves 0-3 compute chunk c (walking backwards) from LDS buffer c&1 while waves 4-7 copy
 // the tiles of chunk c-1 into the other buffer and have those of chunk c-2 in flight.  Both results leave through LDS
 // as whole 128-byte rows, stored by the copying waves one step later: dv2 replaces the wave's own columns of the dv
 // tile, dh goes over the k tile once every wave is past its k . dh products (the barrier in the middle of a step).
-template <int K, bool GK>
+// DVL (scalar gate, 64-token chunks): dv is not an input.  Its intra-chunk part, chunk_bwd_dv_local's result
+//     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i,
+// is formed by the copying waves from the k, q and do tiles they have just staged, into the place of the dv tile, in
+// the first half of the chunk's step (the compute waves read that tile in the second half): the compute waves run the
+// same code as with dv from memory.
+template <int K, bool GK, bool DVL = false>
 __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
+    static_assert(!DVL || !GK, "the in-kernel dv is built for the scalar gate");
     extern __shared__ __align__(16) unsigned char smem[];
     typedef DhuSmem<K> L;
     constexpr int VS = 64, CT = 1;
@@ -530,7 +540,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     const elem *kg = static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh;
     const elem *wg = static_cast<const elem *>(p.w.p) + b * p.w.sb + hv * p.w.sh;
     const elem *og = static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
-    const elem *vg = static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
+    const elem *vg = DVL ? nullptr : static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
 
     if (wave_id() >= 4) {
         // ------------------------------- loader waves -------------------------------------------
@@ -552,7 +562,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             t.tq.fetch(qg + (int64_t)start * p.q.st, p.q.st, len, tid);
             t.tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
             t.to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
-            t.tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            if constexpr (!DVL) t.tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
             if (GK) t.gv = p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + min(tid, K - 1)];
             else t.gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
         };
@@ -565,7 +575,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             t.tq.commit(reinterpret_cast<elem *>(buf + L::q_off), pt, len, tid);
             t.tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pt, len, tid);
             t.to.commit(reinterpret_cast<elem *>(buf + L::o_off), pv, len, tid);
-            t.tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
+            if constexpr (!DVL) t.tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
             if (GK) {
                 if (tid < K) gS[tid] = exp2f(t.gv);
                 if (tid < kChunk) fS[tid] = p.scale;
@@ -618,8 +628,48 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 }
             }
         };
+        // DVL: the dv tile of chunk c from its k, q and do tiles (visible since the last barrier).  Copying wave lw forms
+        // rows 16 lw.. of T[j][i] = scale (k_j . q_i) e^{g_i - g_j} (i >= j), turns them into a left operand through a
+        // strip of LDS of its own (no other wave touches it, so no barrier), and takes T do for those rows.
+        auto build_dv = [&](int c) {
+            const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
+            const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
+            const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
+            const elem *oS = reinterpret_cast<const elem *>(buf + L::o_off);
+            elem *vS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::v_off));
+            const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
+            const int len = min(kChunk, eos - (bos + c * kChunk));
+            const int lw = wave_id() - 4, l = lane_id(), li = l & 15, lg = l >> 4;
+            elem *tS = reinterpret_cast<elem *>(smem + L::t_off) + lw * 16 * L::ptl;
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                f32x4 t = {0.f, 0.f, 0.f, 0.f};
+                if (ct >= lw) {
+#pragma unroll
+                    for (int j = 0; j < KS; ++j) t = mfma16x32(frag_kc(kS, pk, 16 * lw, 32 * j), frag_kc(qS, pt, 16 * ct, 32 * j), t);
+                    const int i = 16 * ct + li;
+                    const float gi = gS[i];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int jrow = 16 * lw + 4 * lg + e;
+                        t[e] = (i >= jrow && i < len) ? t[e] * p.scale * __expf(gi - gS[jrow]) : 0.f;
+                    }
+                }
+                acc_to_tile(tS, L::ptl, 0, 16 * ct, t);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own strip, written and read by itself
+#pragma unroll
+            for (int vt = 0; vt < VS / 16; ++vt) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (32 * j + 31 >= 16 * lw) acc = mfma16x32(frag_kc(tS, L::ptl, 0, 32 * j), frag_tr(oS, pv, 16 * vt, 32 * j), acc);
+                acc_to_tile(vS, pv, 16 * lw, 16 * vt, acc);
+            }
+        };
         // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
         auto step = [&](Tiles &ahead, const Tiles &next, int c) {
+            if constexpr (DVL) build_dv(c);     // into the dv tile, which the compute waves read behind the next barrier
             if (c + 1 < nchunks) read_out(c + 1);
             lds_barrier();   // results of chunk c + 1 are in registers; the compute waves are past the k tile of chunk c
             fetch(ahead, c - 2);
@@ -708,10 +758,54 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             }
         if (chunk_end) g_end = GK ? 0.f : gS[len - 1];
         const float g_last = g_end;
+        // decay of the carried gradient and the q^T do term
+        auto decay_and_q_term = [&]() {
+            if (chunk_end) {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    f32x4 dec;
+                    if (GK) {
+                        dec = *reinterpret_cast<const f32x4 *>(gS + 16 * kt + 4 * lg);
+                    } else {
+                        const float d = __expf(g_last);
+                        dec = f32x4{d, d, d, d};
+                    }
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) dacc[kt][ct] *= dec;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const f32x4 f0 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 4 * lg),
+                            f1 = *reinterpret_cast<const f32x4 *>(fS + 32 * j + 16 + 4 * lg);
+                const elemx8 raw = frag_tr(oS, pv, wv * 16, 32 * j);   // do[t][col], t = 32j + c(g,e)
+                f32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = (float)raw[e] * f0[e];
+                    hi[e] = (float)raw[4 + e] * f1[e];
+                }
+                const elemx8 ob = frag_from_acc(lo, hi);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) dacc[kt][0] = mfma16x32(frag_tr(qS, pt, kt * 16, 32 * j), ob, dacc[kt][0]);
+            }
+        };
+        // DVL: the copying waves form the dv tile in this half of the step, so the part of the update that needs neither
+        // dv nor the place of the k tile moves in front of the barrier; dh then leaves from its 16-bit copy
+        if constexpr (DVL) decay_and_q_term();
         lds_barrier();   // every wave is past the k tile, which now takes dh on its way to memory
         if (chunk_end) {
+            if constexpr (DVL) {
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) acc_to_tile(kS, ph, 16 * kt, wv * 16, dacc[kt][0]);
+                for (int j = 0; j < KS; ++j) {
+                    const u32x4 d = __builtin_bit_cast(u32x4, hB[j][0]);
+                    packed_to_tile(kS, ph, 32 * j, wv * 16, d[0], d[1]);
+                    packed_to_tile(kS, ph, 32 * j + 16, wv * 16, d[2], d[3]);
+                }
+            } else {
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) acc_to_tile(kS, ph, 16 * kt, wv * 16, dacc[kt][0]);
+            }
         }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
@@ -729,6 +823,14 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         for (int rt = 0; rt < 4; ++rt) acc_to_tile(vS, pv, rt * 16, wv * 16, dv2[rt][0]);   // over the wave's own columns of dv
 
         // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
+        if constexpr (DVL) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const elemx8 nb = frag_from_acc(-dv2[2 * j][0], -dv2[2 * j + 1][0]);
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) dacc[kt][0] = mfma16x32(frag_tr(wS, pt, kt * 16, 32 * j), nb, dacc[kt][0]);
+            }
+        } else {
         if (chunk_end) {
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
@@ -770,6 +872,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                     dacc[kt][ct] = mfma16x32(wf, nb[ct], dacc[kt][ct]);
                 }
             }
+        }
         }
         lds_barrier();
     }
@@ -930,12 +1033,12 @@ int launch_bwd_dhu_wide(const DhuParams &p, int slabs, hipStream_t stream) {
     return FLA_OK;
 }
 
-template <int K, bool GK>
+template <int K, bool GK, bool DVL = false>
 int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
-    const size_t smem = DhuSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK>),
+    const size_t smem = DVL ? DhuSmem<K>::bytes_dvl : DhuSmem<K>::bytes;
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK, DVL>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK, DVL>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -953,14 +1056,18 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     FLA_REQUIRE(!has_g || !use_exp2, FLA_ERR_UNSUPPORTED, "%s: the scalar gate g is a natural-log gate (use_exp2=false).", op);
     ChunkGeom geom;
     int rc;
-    if ((rc = gdn_geometry(op, k, dv, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
+    // dv absent: the intra-chunk part of dv (chunk_bwd_dv_local's result) is formed inside the scan
+    const bool has_dv = dv && dv->data;
+    FLA_REQUIRE(has_dv || (has_g && chunk_size == kChunk), FLA_ERR_UNSUPPORTED,
+                "%s: dv may be left out with the scalar gate g and chunk_size 64 only.", op);
+    if ((rc = gdn_geometry(op, k, has_dv ? dv : d_o, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
     FLA_REQUIRE(geom.C == kChunk || !has_gk, FLA_ERR_UNSUPPORTED, "%s: gK is built for chunk_size 64.", op);
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if (has_dv && (rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_bhtd(op, "dv2", dv2, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if (has_gk) {
@@ -1024,7 +1131,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.k = view4(k);
     p.w = view4(w);
     p.d_o = view4(d_o);
-    p.dv = view4(dv);
+    if (has_dv) p.dv = view4(dv);
     p.dv2 = view4(dv2);
     if (has_g) p.g = view3(g);
     if (has_gk) {
@@ -1051,6 +1158,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.scale = (float)scale;
     p.sub = geom.C / kChunk;
     const int slabs = geom.V / 64;
+    if (!has_dv) return geom.K == 128 ? launch_bwd_dhu<128, false, true>(p, slabs, stream) : launch_bwd_dhu<64, false, true>(p, slabs, stream);
     if (geom.K == 256) return launch_bwd_dhu_wide<256>(p, slabs, stream);
     if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, true>(p, slabs, stream) : launch_bwd_dhu<128, false>(p, slabs, stream);
     return has_gk ? launch_bwd_dhu<64, true>(p, slabs, stream) : launch_bwd_dhu<64, false>(p, slabs, stream);

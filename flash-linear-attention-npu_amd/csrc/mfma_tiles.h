@@ -139,10 +139,10 @@ __device__ __forceinline__ void store_tile(elem *gdst, int64_t gstride, const el
 // Neighbouring lanes hold neighbouring columns; they swap half of their values so that every
 // lane writes two whole dwords (even lanes rows e = 0,1; odd lanes rows e = 2,3 of the column
 // pair) instead of four 16-bit pieces, which also keeps the write free of bank conflicts.
-__device__ __forceinline__ void acc_to_tile(elem *tile, int pitch, int r0, int c0, f32x4 acc) {
+// packed_to_tile takes the tile already rounded: p01 = rows 4lg, 4lg + 1 and p23 = rows 4lg + 2, 4lg + 3 of the lane's
+// column, two elements per dword.
+__device__ __forceinline__ void packed_to_tile(elem *tile, int pitch, int r0, int c0, unsigned p01, unsigned p23) {
     const int l = lane_id(), li = l & 15, lg = l >> 4;
-    const unsigned p01 = __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1]));
-    const unsigned p23 = __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3]));
     const bool odd = li & 1;
     const unsigned send = odd ? p01 : p23;
     const unsigned recv = (unsigned)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xf, 0xf, true);  // lane ^ 1
@@ -151,6 +151,10 @@ __device__ __forceinline__ void acc_to_tile(elem *tile, int pitch, int r0, int c
     elem *dst = tile + (r0 + 4 * lg + (odd ? 2 : 0)) * pitch + c0 + (li & ~1);
     *reinterpret_cast<unsigned *>(dst) = __builtin_amdgcn_perm(right, left, 0x05040100u);          // low halves
     *reinterpret_cast<unsigned *>(dst + pitch) = __builtin_amdgcn_perm(right, left, 0x07060302u);  // high halves
+}
+__device__ __forceinline__ void acc_to_tile(elem *tile, int pitch, int r0, int c0, f32x4 acc) {
+    packed_to_tile(tile, pitch, r0, c0, __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1])),
+                   __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3])));
 }
 
 // One accumulator tile, rounded to bf16, straight to global memory (rows r0.. of a row-major matrix with

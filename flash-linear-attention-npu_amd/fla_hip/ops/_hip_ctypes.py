@@ -490,18 +490,20 @@ def npu_chunk_gated_delta_rule_bwd_dhu(q, k, w, d_o, dv, scale, chunk_size, *, g
     ``dh0_per_sequence=True`` (an extension) returns ``dh0`` as fp32 ``[N,Hv,K,V]`` instead of the
     reference's bf16 ``[B,Hv,NT,K,V]`` buffer whose first chunk of each sequence holds the value.
     ``dht`` (fp32 ``[N,Hv,K,V]``) seeds the scan; the reference accepts and ignores it.
+    ``dv=None`` (an extension; scalar gate, 64-token chunks): the scan forms the intra-chunk part of dv itself, what
+    ``chunk_bwd_dv_local`` would have been called for, from the q, k and d_o tiles it holds anyway.
     """
     import torch
 
     B, _, T, K = _shape(q)
-    _, Hv, _, V = _shape(dv)
+    _, Hv, _, V = _shape(d_o)
     gates = {"g": (g, (B, Hv, T)), "gK": (gK, (B, Hv, T, K))}
     given = [name for name, (t, _) in gates.items() if t is not None]
     if len(given) != 1:
         raise ValueError("Exactly one of g and gK must be provided.")
     if given == ["gK"] and not _optional_bool(use_exp2, True):
         raise ValueError("use_exp2 must be true when gK is provided.")
-    if {t.dtype for t in (k, w, d_o, dv)} != {q.dtype}:
+    if {t.dtype for t in (k, w, d_o) + (() if dv is None else (dv,))} != {q.dtype}:
         raise ValueError("q, k, w, d_o and dv must have the same dtype.")
     gate, gate_shape = gates[given[0]]
     if gate.dtype not in (q.dtype, torch.float32):
@@ -522,7 +524,7 @@ def npu_chunk_gated_delta_rule_bwd_dhu(q, k, w, d_o, dv, scale, chunk_size, *, g
         dh0 = _empty((N, Hv, K, V), q, dtype=torch.float32)
     else:
         dh0 = _empty((B, Hv, NT, K, V), q)
-    dv2 = _empty_like(dv)
+    dv2 = _empty_ordered_like(d_o) if dv is None else _empty_like(dv)
     outputs = (dh, dh0, dv2)
     return _call_op(
         "chunk_gated_delta_rule_bwd_dhu", OP_ARGTYPES["chunk_gated_delta_rule_bwd_dhu"],

@@ -108,7 +108,9 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
         w, u = _ops.recompute_w_u_fwd(k, v, bh, A, chunk_size, g=gh, **kw)
         h, v_new, _ = _ops.chunk_gated_delta_rule_fwd_h(k, w, u, g=gh, initial_state=initial_state,
                                                         output_final_state=False, chunk_size=chunk_size, **kw)
-    dv = _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
+    # 64-token chunks: the reverse scan forms the intra-chunk part of dv from the tiles it holds; otherwise
+    # chunk_bwd_dv_local runs first, as in the reference (examples/flash_gated_delta_rule.py:953-966)
+    dv = None if chunk_size == 64 else _ops.chunk_bwd_dv_local(q, k, doh, gh, scale, chunk_size, **kw)
     dh, dh0, dv = _ops.chunk_gated_delta_rule_bwd_dhu(q, k, w, doh, dv, scale, chunk_size, g=gh, h0=initial_state,
                                                       dht=dht, dh0_per_sequence=True, **kw)
     in_kernel_norm = qk_rstd is not None and chunk_size == 64

@@ -328,6 +328,9 @@ int fla_kda_gate_bwd(
  * reference form (bf16, shape of dh, written at each sequence's first chunk)
  * or f32 [N,Hv,K,V].  Implemented: K in {64,128} (K = 256 with gK), V a
  * multiple of 64; chunk_size 64, and 128 with the scalar gate.
+ * Extension: dv may be NULL (scalar gate, chunk_size 64).  The scan then forms
+ * the intra-chunk part of dv itself, the result of chunk_bwd_dv_local on
+ * (q, k, d_o, g, scale), from the tiles it stages anyway.
  * ------------------------------------------------------------------------ */
 int fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o,

@@ -134,6 +134,37 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     assert_close(dg_acc, dg0 + two[3], 1e-6, "dg accumulated")
 
 
+@pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("case", CASES)
+def test_reverse_scan_forms_the_local_dv_itself(dev, case, dtype):
+    """chunk_gated_delta_rule_bwd_dhu without dv (an extension for 64-token chunks and the scalar gate): the scan forms
+    chunk_bwd_dv_local's result from the q, k and d_o tiles it holds.  Against the oracle's two operators on the same
+    inputs (the local part enters in fp32 there, unrounded as in the kernel), and against the two-operator route."""
+    from fla_hip import ops
+    B, T, Hv, Hk, K, V, cu = case
+    scale = K ** -0.5
+    d = make(B, T, Hv, Hk, K, V, cu, seed=T + V, dtype=dtype)
+    tol = 2e-2 if dtype == torch.bfloat16 else 5e-3
+    x = to_dev(d, dev)
+    kw = dict(cu_seqlens=cu)
+    dv_l_ref = gdn_bwd.chunk_bwd_dv_local(d["q"], d["k"], d["do"], d["G"], scale, 64, output_dtype=torch.float32, **kw)
+    dh_ref, dh0_ref, dv2_ref = dhu_oracle(d["q"], d["k"], d["w"], d["do"], dv_l_ref, scale, 64, g=d["G"], dht=d["dht"], **kw)
+    args = (x["q"], x["k"], x["w"], x["do"])
+    okw = dict(g=x["G"], h0=x["h0"], dht=x["dht"], dh0_per_sequence=True, **kw)
+    dh, dh0, dv2 = ops.chunk_gated_delta_rule_bwd_dhu(*args, None, scale, 64, **okw)
+    assert dv2.shape == d["do"].shape and dv2.dtype == dtype and dh.dtype == dtype and dh0.dtype == torch.float32
+    assert_close(dv2, dv2_ref, tol, "dv2")
+    assert_close(dh, dh_ref, tol, "dh")
+    assert_close(dh0, dh0_ref, tol, "dh0")
+    dv_l = ops.chunk_bwd_dv_local(x["q"], x["k"], x["do"], x["G"], scale, 64, **kw)
+    dh_b, dh0_b, dv2_b = ops.chunk_gated_delta_rule_bwd_dhu(*args, dv_l, scale, 64, **okw)
+    assert_close(dv2, dv2_b.float(), tol, "dv2 against the two operators")
+    assert_close(dh0, dh0_b, tol, "dh0 against the two operators")
+    # 128-token chunks and the per-channel gate keep the operator's own signature
+    with pytest.raises(RuntimeError, match="dv may be left out"):
+        ops.chunk_gated_delta_rule_bwd_dhu(*args, None, scale, 128, g=x["G"], **kw)
+
+
 CASES_128 = [
     # B, T, Hv, Hk, K, V, cu_seqlens: full chunks, a last chunk with only its first half, every remainder when packed
     (2, 256, 2, 2, 128, 128, None),
