@@ -508,6 +508,51 @@ template <int K> struct DhuSmem {
 // the tiles of chunk c-1 into the other buffer and have those of chunk c-2 in flight.  Both results leave through LDS
 // as whole 128-byte rows, stored by the copying waves one step later: dv2 replaces the wave's own columns of the dv
 // tile, dh goes over the k tile once every wave is past its k . dh products (the barrier in the middle of a step).
+// Rows 16 LW.. of the intra-chunk dv of one chunk (see bwd_dhu_kernel, DVL), by one wave.
+template <int K, int LW>
+__device__ __forceinline__ void dv_rows(const elem *kS, const elem *qS, const elem *oS, elem *vS, const float *gS, elem *strips,
+                                        int len, float scale) {
+    typedef DhuSmem<K> L;
+    constexpr int pk = L::pk, pt = L::pt, pv = L::pv, ptl = L::ptl, KS = K / 32;
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    elem *tS = strips + LW * 16 * ptl;
+    f32x4 t[4];
+#pragma unroll
+    for (int ct = LW; ct < 4; ++ct) t[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+        const elemx8 a = frag_kc(kS, pk, 16 * LW, 32 * j);
+#pragma unroll
+        for (int ct = LW; ct < 4; ++ct) t[ct] = mfma16x32(a, frag_kc(qS, pt, 16 * ct, 32 * j), t[ct]);
+    }
+    f32x4 gj;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) gj[e] = gS[16 * LW + 4 * lg + e];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+        f32x4 x = {0.f, 0.f, 0.f, 0.f};
+        if (ct >= LW) {
+            const int i = 16 * ct + li;
+            const float gi = gS[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = (i >= 16 * LW + 4 * lg + e && i < len) ? t[ct][e] * scale * __expf(gi - gj[e]) : 0.f;
+        }
+        acc_to_tile(tS, ptl, 0, 16 * ct, x);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own strip, written and read by itself
+    constexpr int J0 = LW / 2;   // contraction steps (32 tokens i each) that hold a non-zero tile of these rows
+    elemx8 tf[2];
+#pragma unroll
+    for (int j = J0; j < 2; ++j) tf[j] = frag_kc(tS, ptl, 0, 32 * j);
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = J0; j < 2; ++j) acc = mfma16x32(tf[j], frag_tr(oS, pv, 16 * vt, 32 * j), acc);
+        acc_to_tile(vS, pv, 16 * LW, 16 * vt, acc);
+    }
+}
+
 // DVL (scalar gate, 64-token chunks): dv is not an input.  Its intra-chunk part, chunk_bwd_dv_local's result
 //     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i,
 // is formed by the copying waves from the k, q and do tiles they have just staged, into the place of the dv tile, in
@@ -639,32 +684,12 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             elem *vS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::v_off));
             const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
             const int len = min(kChunk, eos - (bos + c * kChunk));
-            const int lw = wave_id() - 4, l = lane_id(), li = l & 15, lg = l >> 4;
-            elem *tS = reinterpret_cast<elem *>(smem + L::t_off) + lw * 16 * L::ptl;
-#pragma unroll
-            for (int ct = 0; ct < 4; ++ct) {
-                f32x4 t = {0.f, 0.f, 0.f, 0.f};
-                if (ct >= lw) {
-#pragma unroll
-                    for (int j = 0; j < KS; ++j) t = mfma16x32(frag_kc(kS, pk, 16 * lw, 32 * j), frag_kc(qS, pt, 16 * ct, 32 * j), t);
-                    const int i = 16 * ct + li;
-                    const float gi = gS[i];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int jrow = 16 * lw + 4 * lg + e;
-                        t[e] = (i >= jrow && i < len) ? t[e] * p.scale * __expf(gi - gS[jrow]) : 0.f;
-                    }
-                }
-                acc_to_tile(tS, L::ptl, 0, 16 * ct, t);
-            }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own strip, written and read by itself
-#pragma unroll
-            for (int vt = 0; vt < VS / 16; ++vt) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (32 * j + 31 >= 16 * lw) acc = mfma16x32(frag_kc(tS, L::ptl, 0, 32 * j), frag_tr(oS, pv, 16 * vt, 32 * j), acc);
-                acc_to_tile(vS, pv, 16 * lw, 16 * vt, acc);
+            elem *strips = reinterpret_cast<elem *>(smem + L::t_off);
+            switch (wave_id() - 4) {   // the row tile as a constant: every operand read of the wave is issued at once
+                case 0: dv_rows<K, 0>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                case 1: dv_rows<K, 1>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                case 2: dv_rows<K, 2>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                default: dv_rows<K, 3>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
             }
         };
         // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
