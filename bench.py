@@ -672,6 +672,8 @@ def bench_gdn_bwd(args, torch, dev):
         "kkt": 2 * C * K * th, "solve_tri": 2 * (C * C // 3) * th, "wu": 2 * (C * K + C * V) * th,
         "fwd_h": 2 * (2 * K * V) * th,
     }
+    if "bwd_dv_local" not in kern:   # 64-token chunks: the reverse scan forms the intra-chunk dv itself
+        flops_of["bwd_dhu"] += flops_of.pop("bwd_dv_local")
     timed = {n: t for n, t in kern.items() if n in flops_of}
     dominant = max(timed, key=timed.get)
     ach = flops_of[dominant] / (kern[dominant] * 1e-3) / 1e12
