@@ -674,6 +674,8 @@ def bench_gdn_bwd(args, torch, dev):
     }
     if "bwd_dv_local" not in kern:   # 64-token chunks: the reverse scan forms the intra-chunk dv itself
         flops_of["bwd_dhu"] += flops_of.pop("bwd_dv_local")
+    if "wy_bwd_da" not in kern:      # and the WY backward forms dA itself
+        flops_of["wy_bwd_full"] += flops_of.pop("wy_bwd_da")
     timed = {n: t for n, t in kern.items() if n in flops_of}
     dominant = max(timed, key=timed.get)
     ach = flops_of[dominant] / (kern[dominant] * 1e-3) / 1e12

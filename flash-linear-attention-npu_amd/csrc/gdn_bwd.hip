@@ -619,7 +619,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
 // leave through an fp32 LDS tile (the k and dw tiles, dead by then), so that memory is read and written in whole
 // 16-byte row pieces: adding tile by tile from the accumulator layout, four bytes per lane, cost more than the separate
 // elementwise pass it replaces.
-template <int K, int V, bool GVA, bool ACC = false>
+// DA: dA is not an input.  prepare_wy_repr_bwd_da's result for the chunk is formed in place, from the tiles this kernel
+// stages anyway (du v^T while du is in its tile, dw k^T once dw has taken it; the row scales beta and beta e^G of the
+// second operands become column scales of the products), through the same two 64 x 64 intermediates, which pass through
+// the tiles that then receive dA and its beta-scaled copy.
+template <int K, int V, bool GVA, bool ACC = false, bool DA = false>
 __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(const WyBwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     // du and dw share one tile (du is dead once A^T du is formed) and v, which is only read element-wise,
@@ -663,7 +667,7 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
             tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
             ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
-            td.fetch(static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
+            if constexpr (!DA) td.fetch(static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
             if (tid < kChunk) {
                 const int t = start + min(tid, len - 1);
                 gS[tid] = load_scalar(p.g, b, hv, t);
@@ -674,8 +678,10 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             tdu.commit(xS, px, len, tid);
             tv.commit(vS, pvv, len, tid);
             commit_square(ta, aS, pa, len, nullptr, tid);
-            commit_square(td, dS, pa, len, nullptr, tid);
-            commit_square(td, dbS, pa, len, bS, tid);
+            if constexpr (!DA) {
+                commit_square(td, dS, pa, len, nullptr, tid);
+                commit_square(td, dbS, pa, len, bS, tid);
+            }
         }
         // dw is fetched only now, once the registers of the first batch are free; it lands during A^T du
         tdw.fetch(static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
@@ -702,9 +708,76 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
             __builtin_amdgcn_sched_barrier(0);
         }
+        f32x4 m4[4];                     // DA: row tile w of strict_lower(dw (k beta e^G)^T + du (v beta)^T)
+        if constexpr (DA) {
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                f32x4 acc = zero4();
+                if (ct <= w) {
+#pragma unroll
+                    for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(xS, px, 16 * w, 32 * j), frag_kc(vS, pvv, 16 * ct, 32 * j), acc);
+                }
+                m4[ct] = acc;
+            }
+        }
         __syncthreads();                 // du has been consumed by every wave
         tdw.commit(xS, px, len, tid);
         __syncthreads();
+        if constexpr (DA) {
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                f32x4 acc = zero4();
+                if (ct <= w) {
+#pragma unroll
+                    for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(xS, px, 16 * w, 32 * j), frag_kc(kS, pk, 16 * ct, 32 * j), acc);
+                    const int col = 16 * ct + li;
+                    const float bc = bS[col], fc = bc * __expf(gS[col]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = 16 * w + 4 * lg + e;
+                        acc[e] = (col < row && row < len) ? acc[e] * fc + m4[ct][e] * bc : 0.f;
+                    }
+                }
+                acc_to_tile(dS, pa, 16 * w, 16 * ct, acc);      // M4
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {                     // M5 = M4 A^T
+                f32x4 acc = zero4();
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_kc(dS, pa, 16 * w, 32 * j), frag_kc(aS, pa, 16 * ct, 32 * j), acc);
+                acc_to_tile(dbS, pa, 16 * w, 16 * ct, acc);
+            }
+            __syncthreads();
+            f32x4 da[4];                                         // rows 16 w.. of dA as stored: (A^T M5)^T, gated, negated, masked
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                f32x4 acc = zero4();
+                if (ct >= w) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_tr(dbS, pa, 16 * w, 32 * j), frag_tr(aS, pa, 16 * ct, 32 * j), acc);
+                    const int col = 16 * ct + li;
+                    const float gc = gS[col];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int row = 16 * w + 4 * lg + e;
+                        acc[e] = (col > row && col < len) ? -acc[e] * __expf(fminf(gc - gS[row], 0.f)) : 0.f;
+                    }
+                }
+                da[ct] = acc;
+                acc_to_tile(dS, pa, 16 * w, 16 * ct, acc);      // M4 was last read before the barrier above
+            }
+            __syncthreads();                                     // every wave has read M5
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct) {
+                // the stored value is the rounded one: the copy with column j scaled by beta_j starts from it, as a copy
+                // made from memory would
+                const elemx4 r4 = cvt4(da[ct]);
+                const float bc = bS[16 * ct + li];
+                acc_to_tile(dbS, pa, 16 * w, 16 * ct, f32x4{(float)r4[0] * bc, (float)r4[1] * bc, (float)r4[2] * bc, (float)r4[3] * bc});
+            }
+            __syncthreads();
+        }
         const elemx8 dt0 = frag_tr(dS, pa, 16 * w, 0), dt1 = frag_tr(dS, pa, 16 * w, 32);
         const elemx8 db0 = frag_kc(dbS, pa, 16 * w, 0), db1 = frag_kc(dbS, pa, 16 * w, 32);
 #pragma unroll
@@ -1259,7 +1332,10 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     int rc;
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
     const int bf = dt_bit(kElemDtype);
-    if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
+    // dA absent (the accumulating form on 64-token chunks only): the kernel forms prepare_wy_repr_bwd_da's result itself
+    const bool has_da = dA && dA->data;
+    FLA_REQUIRE(has_da || (accumulate && geom.C == kChunk), FLA_ERR_NULL, "%s: dA must not be null.", op);
+    if (has_da && (rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
     if ((rc = check_bhtd(op, "dk", dk, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if ((rc = check_f32_bht(op, "dbeta", dbeta, geom))) return rc;
@@ -1267,7 +1343,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
-    WyBwdParams p{geom, view4(k), view4(v), view4(A), view4(dA), view4(dw), view4(du), view4(dk), view4(dv), view3(g),
+    WyBwdParams p{geom, view4(k), view4(v), view4(A), has_da ? view4(dA) : View4{nullptr, 0, 0, 0}, view4(dw), view4(du), view4(dk), view4(dv), view3(g),
                   view3(beta), static_cast<float *>(dbeta->data), static_cast<float *>(dg->data),
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
     bool has_rstd;
@@ -1292,6 +1368,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     const bool gva = geom.Hv != geom.Hk;
 #define FLA_WY_FULL(KK, VV, G)                                                                                      \
     do {                                                                                                            \
+        if (accumulate && !has_da) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true, true>), "wy_bwd_full", grid, smem, p); \
         if (accumulate) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true>), "wy_bwd_full", grid, smem, p);      \
         FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, false>), "wy_bwd_full", grid, smem, p);                     \
     } while (0)

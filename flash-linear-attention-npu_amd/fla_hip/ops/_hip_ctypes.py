@@ -1051,7 +1051,9 @@ def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, ch
     """npu_prepare_wy_repr_bwd_full with its key and gate gradients ADDED to ``dk`` ([B,Hk,T,K], dtype of k) and
     ``dg`` ([B,Hv,T] f32) in place: the reference's composition adds them with a separate pass
     (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32).  ``k_rstd`` (f32 [B,Hk,T], the second result
-    of ``l2norm_fwd``): k is the normalised tensor and the completed dk leaves as the gradient of the raw k."""
+    of ``l2norm_fwd``): k is the normalised tensor and the completed dk leaves as the gradient of the raw k.
+    ``dA=None`` (64-token chunks): the kernel forms ``npu_prepare_wy_repr_bwd_da``'s result itself, from the tiles it
+    stages anyway, and dA never goes through memory."""
     dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dv, dbeta = _call_op(

@@ -118,13 +118,14 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
         dq, dk, dw, dg = _raw.chunk_bwd_dqkwg_l2norm(q, k, v_new, gh, h, doh, dh, dv, qk_rstd[0], chunk_size, scale=scale, **kw)
     else:
         dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
-    dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
     # the second part of dk and dg is added where it is produced (the reference adds with separate passes,
-    # examples/flash_gated_delta_rule.py:994-1012)
+    # examples/flash_gated_delta_rule.py:994-1012), and on 64-token chunks dA is formed by the same kernel
+    # (prepare_wy_repr_bwd_da, :985-992, as a pass of its own otherwise)
     if chunk_size == 64:
-        dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, dA, dw, dv, gh, dk, dg, chunk_size,
+        dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, None, dw, dv, gh, dk, dg, chunk_size,
                                                           k_rstd=qk_rstd[1] if in_kernel_norm else None, **kw)
-    else:   # 128-token chunks: the plain operator and the reference's two additions
+    else:   # 128-token chunks: the plain operators and the reference's two additions
+        dA = _ops.prepare_wy_repr_bwd_da(k, v, bh, A, dw, dv, gh, chunk_size=chunk_size, **kw)
         dk2, dv, db, dg2 = _ops.prepare_wy_repr_bwd_full(k, v, bh, A, dA, dw, dv, gh, chunk_size, **kw)
         dk.add_(dk2)
         dg.add_(dg2)

@@ -132,6 +132,15 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     assert torch.equal(dv_a, two[1]) and torch.equal(db_a, two[2])
     assert_close(dk_acc, dk0.float() + dk2_r.to(dev), TOL_BF16, "dk accumulated")
     assert_close(dg_acc, dg0 + two[3], 1e-6, "dg accumulated")
+    # without dA the same kernel forms prepare_wy_repr_bwd_da's result itself (dA never goes through memory)
+    dk_f, dg_f = dk0.clone(), dg0.clone()
+    dv_f, db_f = raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], x["A"], None, dwb.to(dev), dv2.to(dev),
+                                                         x["G"], dk_f, dg_f, 64, **kw)
+    assert torch.equal(dv_f, two[1])
+    assert_close(dk_f, dk0.float() + dk2_r.to(dev), TOL_BF16, "dk accumulated, dA formed in the kernel")
+    for name, got, ref in (("dbeta", db_f, db_r), ("dg2", dg_f - dg0, dg2_r)):
+        st = err_stats(got, ref)
+        assert st["rel_max"] <= TOL_BF16, f"{name}, dA formed in the kernel: {st}"
 
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
