@@ -11,6 +11,7 @@
 // Operators with key-head outputs (dq, dk) loop over the value heads that share a key head inside one
 // workgroup, so grouped value heads need neither atomics nor a second pass.
 #include "gdn_common.h"
+#include "chunk_inverse.h"
 #include "mfma_tiles.h"
 
 namespace fla {
@@ -623,7 +624,11 @@ __global__ void __launch_bounds__(kThreads) wy_bwd_da_kernel(const WyBwdParams p
 // stages anyway (du v^T while du is in its tile, dw k^T once dw has taken it; the row scales beta and beta e^G of the
 // second operands become column scales of the products), through the same two 64 x 64 intermediates, which pass through
 // the tiles that then receive dA and its beta-scaled copy.
-template <int K, int V, bool GVA, bool ACC = false, bool DA = false>
+// AINV: A is not an input either.  The chunk's (I + strict_lower(beta k k^T e^{G_i - G_j}))^-1 is rebuilt from the k
+// tile, g and beta that are staged anyway, with the arithmetic of the fused kkt + inverse kernel (scores rounded to
+// the element type, the same block inversion), so the matrix equals the one that kernel would have stored; the fp32
+// scores pass through the two tiles that later hold dA.
+template <int K, int V, bool GVA, bool ACC = false, bool DA = false, bool AINV = false>
 __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(const WyBwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     // du and dw share one tile (du is dead once A^T du is formed) and v, which is only read element-wise,
@@ -666,7 +671,7 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             TileCopy<kThreads, kChunk, kChunk> ta, td;
             tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
             tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
-            ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
+            if constexpr (!AINV) ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
             if constexpr (!DA) td.fetch(static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
             if (tid < kChunk) {
                 const int t = start + min(tid, len - 1);
@@ -677,7 +682,33 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
             __syncthreads();
             tdu.commit(xS, px, len, tid);
             tv.commit(vS, pvv, len, tid);
-            commit_square(ta, aS, pa, len, nullptr, tid);
+            if constexpr (AINV) {
+                static_assert(DA && pa == 72, "the fp32 score block lies over the two dA tiles; the inverse is written at pitch 72");
+                static_assert(kChunk * 68 * 4 <= 2 * kChunk * pa * 2, "the fp32 score block must fit the two dA tiles");
+                float *sS = reinterpret_cast<float *>(dS);
+                const int t = 16 * w + li;
+                const float gt = gS[t], bt = bS[t];
+#pragma unroll
+                for (int J = 0; J < 4; ++J) {
+                    f32x4 acc = zero4();
+                    if (J <= w) {
+#pragma unroll
+                        for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(kS, pk, 16 * J, 32 * j), frag_kc(kS, pk, 16 * w, 32 * j), acc);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int s0 = 16 * J + 4 * lg + e;
+                            const float d = fminf(fmaxf(gt - gS[s0], -50.f), 50.f);
+                            acc[e] = (s0 < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[e]) : 0.f;
+                        }
+                    }
+                    *reinterpret_cast<f32x4 *>(sS + t * 68 + 16 * J + 4 * lg) = acc;
+                }
+                __syncthreads();
+                invert64(sS, aS);
+                if (tid < kChunk && tid >= len) aS[tid * pa + tid] = (elem)0.f;   // rows past the end hold nothing, as a staged A would
+            } else {
+                commit_square(ta, aS, pa, len, nullptr, tid);
+            }
             if constexpr (!DA) {
                 commit_square(td, dS, pa, len, nullptr, tid);
                 commit_square(td, dbS, pa, len, bS, tid);
@@ -1281,7 +1312,7 @@ int wy_bwd_common(const char *op, const fla_tensor *k, const fla_tensor *v, cons
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "v", v, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
-    if ((rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;
+    if (A != nullptr && (rc = check_bhtd(op, "A", A, geom.B, geom.Hv, geom.T, geom.C, bf))) return rc;   // null: the caller has checked that the kernel can do without
     if ((rc = check_bhtd(op, "dw", dw, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "du", du, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     FLA_REQUIRE(g != nullptr && g->data != nullptr && beta != nullptr && beta->data != nullptr, FLA_ERR_NULL,
@@ -1298,6 +1329,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
     const char *op = "prepare_wy_repr_bwd_da";
     ChunkGeom geom;
     int rc;
+    FLA_REQUIRE(A != nullptr && A->data != nullptr, FLA_ERR_NULL, "%s: A must not be null.", op);
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
     if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, dt_bit(kElemDtype)))) return rc;
     Varlen vl;
@@ -1330,7 +1362,10 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     const char *op = accumulate ? "prepare_wy_repr_bwd_full_accumulate" : "prepare_wy_repr_bwd_full";
     ChunkGeom geom;
     int rc;
-    if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
+    // A absent (only together with dA, below): the kernel rebuilds the chunk's inverse from k, g and beta
+    const bool has_a = A && A->data;
+    FLA_REQUIRE(has_a || !(dA && dA->data), FLA_ERR_NULL, "%s: A must not be null when dA is given.", op);
+    if ((rc = wy_bwd_common(op, k, v, beta, has_a ? A : nullptr, dw, du, g, chunk_size, geom))) return rc;
     const int bf = dt_bit(kElemDtype);
     // dA absent (the accumulating form on 64-token chunks only): the kernel forms prepare_wy_repr_bwd_da's result itself
     const bool has_da = dA && dA->data;
@@ -1343,7 +1378,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query)) || query) return rc;
     if (geom.NT == 0 || geom.B == 0) return FLA_OK;
-    WyBwdParams p{geom, view4(k), view4(v), view4(A), has_da ? view4(dA) : View4{nullptr, 0, 0, 0}, view4(dw), view4(du), view4(dk), view4(dv), view3(g),
+    WyBwdParams p{geom, view4(k), view4(v), has_a ? view4(A) : View4{nullptr, 0, 0, 0}, has_da ? view4(dA) : View4{nullptr, 0, 0, 0}, view4(dw), view4(du), view4(dk), view4(dv), view3(g),
                   view3(beta), static_cast<float *>(dbeta->data), static_cast<float *>(dg->data),
                   dbeta->stride[0], dbeta->stride[1], dbeta->stride[2], dg->stride[0], dg->stride[1], dg->stride[2]};
     bool has_rstd;
@@ -1368,6 +1403,7 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     const bool gva = geom.Hv != geom.Hk;
 #define FLA_WY_FULL(KK, VV, G)                                                                                      \
     do {                                                                                                            \
+        if (accumulate && !has_da && !has_a) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true, true, true>), "wy_bwd_full", grid, smem, p); \
         if (accumulate && !has_da) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true, true>), "wy_bwd_full", grid, smem, p); \
         if (accumulate) FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, true>), "wy_bwd_full", grid, smem, p);      \
         FLA_BWD_DISPATCH((wy_bwd_full_kernel<KK, VV, G, false>), "wy_bwd_full", grid, smem, p);                     \

@@ -8,6 +8,7 @@
 // solve_tri/README.md:7-19, recompute_w_u_fwd/README.md:12-32,
 // chunk_fwd_o/README.md:6-15 (+ qkmask epilogue, op_kernel/.../block_epilogue_gdn_fwdo_qkmask.hpp:210-262).
 #include "gdn_common.h"
+#include "chunk_inverse.h"
 #include "mfma_tiles.h"
 
 namespace fla {
@@ -148,77 +149,6 @@ __global__ void __launch_bounds__(BT < 64 ? 64 : BT) solve_tri_kernel(const Solv
         const int r = idx / CPR, c8 = (idx % CPR) << 3;
         *reinterpret_cast<u32x4 *>(p.out + base + (int64_t)r * p.st + c8) = *reinterpret_cast<const u32x4 *>(O + r * PO + c8);
     }
-}
-
-// 64 x 64 blocks on the matrix cores: four waves, wave R inverts diagonal block R and then fills column block R
-// of the inverse.  (I + A)^-1 of a strictly lower 16 x 16 block is the finite product (I - A)(I + A^2)(I + A^4)
-// (I + A^8); the blocks below the diagonal follow by block substitution, X_rc = -D_r sum_m A_rm X_mc, with both
-// operands of those products carried as a 16-bit head plus remainder.
-__device__ __forceinline__ f32x4 solve_lds4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
-__device__ __forceinline__ f32x4 solve_mm3(f32x4 a, f32x4 b, f32x4 acc) {   // acc += a b without the lo * lo term
-    elemx4 ah, al, bh, bl;
-    split_hilo(a, ah, al);
-    split_hilo(b, bh, bl);
-    acc = mfma16x16(ah, bh, acc);
-    acc = mfma16x16(al, bh, acc);
-    acc = mfma16x16(ah, bl, acc);
-    return acc;
-}
-
-// (I + A)^-1 of the strictly lower 64 x 64 matrix in aS (fp32, pitch 68), written to oS (pitch 72) in the element
-// type; called by all four waves of a 256-thread workgroup after a barrier that completes aS, ends with one.
-__device__ __forceinline__ void invert64(float *aS, elem *oS) {
-    constexpr int pa = 68, pb = 72;
-    const int R = wave_id(), l = lane_id(), li = l & 15, lg = l >> 4;
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    {   // diagonal block: a2 = A[4lg+e][li] and a1 = A[li][4lg+e] (both orientations feed the squarings)
-        f32x4 a1, a2, Y;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int r = 4 * lg + e;
-            a2[e] = aS[(16 * R + r) * pa + 16 * R + li];
-            a1[e] = aS[(16 * R + li) * pa + 16 * R + r];
-            Y[e] = (r == li ? 1.f : 0.f) - a1[e];
-        }
-        const elemx4 A1 = cvt4(a1), A2 = cvt4(a2);
-        const f32x4 S1 = mfma16x16(A1, A2, zero);   // A^2
-        const f32x4 T1 = mfma16x16(A2, A1, zero);   // (A^2)^T
-        const elemx4 S1b = cvt4(S1), T1b = cvt4(T1);
-        Y = mfma16x16(S1b, cvt4(Y), Y);
-        const f32x4 S2 = mfma16x16(T1b, S1b, zero);  // A^4
-        const f32x4 T2 = mfma16x16(S1b, T1b, zero);  // (A^4)^T
-        const elemx4 S2b = cvt4(S2);
-        Y = mfma16x16(S2b, cvt4(Y), Y);
-        const f32x4 S3 = mfma16x16(cvt4(T2), S2b, zero);  // A^8
-        Y = mfma16x16(cvt4(S3), cvt4(Y), Y);
-        __syncthreads();   // every wave has read its block of A before the inverses replace the diagonal blocks
-        // lane holds D[li][4lg+e]
-        *reinterpret_cast<f32x4 *>(aS + (16 * R + li) * pa + 16 * R + 4 * lg) = Y;
-        *reinterpret_cast<elemx4 *>(oS + (16 * R + li) * pb + 16 * R + 4 * lg) = cvt4(Y);
-#pragma unroll
-        for (int cb = R + 1; cb < 4; ++cb)
-            *reinterpret_cast<elemx4 *>(oS + (16 * R + li) * pb + 16 * cb + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
-    }
-    __syncthreads();
-    {   // column block R of the inverse, top to bottom: X[k] = block (R + k, R)
-        f32x4 X[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) X[0][e] = aS[(16 * R + 4 * lg + e) * pa + 16 * R + li];
-#pragma unroll
-        for (int k = 1; k < 4; ++k) {
-            if (R + k < 4) {
-                const int r = R + k;
-                f32x4 sum = zero;
-#pragma unroll
-                for (int j = 0; j < k; ++j)
-                    sum = solve_mm3(solve_lds4(aS + (16 * r + li) * pa + 16 * (R + j) + 4 * lg), X[j], sum);
-                const f32x4 dinv = solve_lds4(aS + (16 * r + li) * pa + 16 * r + 4 * lg);
-                X[k] = solve_mm3(-dinv, sum, zero);
-                acc_to_tile(oS, pb, 16 * r, 16 * R, X[k]);
-            }
-        }
-    }
-    __syncthreads();
 }
 
 template <bool F32IN>

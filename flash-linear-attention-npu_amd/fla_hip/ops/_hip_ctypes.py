@@ -1053,7 +1053,8 @@ def prepare_wy_repr_bwd_full_accumulate(k, v, beta, A, dA, dw, du, g, dk, dg, ch
     (examples/flash_gated_delta_rule.py:994-1010).  Returns (dv, dbeta f32).  ``k_rstd`` (f32 [B,Hk,T], the second result
     of ``l2norm_fwd``): k is the normalised tensor and the completed dk leaves as the gradient of the raw k.
     ``dA=None`` (64-token chunks): the kernel forms ``npu_prepare_wy_repr_bwd_da``'s result itself, from the tiles it
-    stages anyway, and dA never goes through memory."""
+    stages anyway, and dA never goes through memory.  Then ``A`` may be None as well: the kernel rebuilds each chunk's
+    inverse from k, g and beta with the arithmetic of ``chunk_scaled_dot_kkt_inverse``, so neither matrix is read."""
     dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
     dv, dbeta = _call_op(

@@ -96,7 +96,9 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
     # head-first VIEWS: every kernel takes the outer strides of its operands, nothing is copied
     gh = g.float().transpose(1, 2)
     bh = beta.float().transpose(1, 2)
-    if A is None and chunk_size == 64:
+    if A is None and chunk_size == 64 and saved is not None:
+        pass   # nothing but the WY backward needs A then, and that kernel rebuilds it per chunk from k, g and beta
+    elif A is None and chunk_size == 64:
         A = _ops.chunk_scaled_dot_kkt_inverse(k, gh, bh, chunk_size=chunk_size, **kw)   # the two operators below, fused
     elif A is None:
         A = _ops.chunk_scaled_dot_kkt(k, gh, bh, chunk_size=chunk_size, **kw)
@@ -120,7 +122,7 @@ def flash_chunk_gated_delta_rule_bwd(q, k, v, g, beta, A, scale, initial_state, 
         dq, dk, dw, dg = _ops.chunk_bwd_dqkwg(q, k, v_new, gh, h, doh, dh, dv, chunk_size, scale=scale, **kw)
     # the second part of dk and dg is added where it is produced (the reference adds with separate passes,
     # examples/flash_gated_delta_rule.py:994-1012), and on 64-token chunks dA is formed by the same kernel
-    # (prepare_wy_repr_bwd_da, :985-992, as a pass of its own otherwise)
+    # (prepare_wy_repr_bwd_da, :985-992, as a pass of its own otherwise); A = None: see above
     if chunk_size == 64:
         dv, db = _raw.prepare_wy_repr_bwd_full_accumulate(k, v, bh, A, None, dw, dv, gh, dk, dg, chunk_size,
                                                           k_rstd=qk_rstd[1] if in_kernel_norm else None, **kw)

@@ -659,7 +659,9 @@ int fla_prepare_wy_repr_bwd_full(
  * NULL): k is the l2-normalised tensor and the completed dk leaves as the gradient of the un-normalised k,
  * dk <- (dk - k <k, dk>) rstd per row (what l2norm_bwd would do in a pass of its own).
  * dA may be NULL (chunk_size 64): the kernel then forms the result of prepare_wy_repr_bwd_da on the same operands
- * itself, from the tiles it stages anyway, and dA never goes through memory. */
+ * itself, from the tiles it stages anyway, and dA never goes through memory.  With dA NULL, A may be NULL too: each
+ * chunk's (I + strict_lower(beta k k^T e^{g_i - g_j}))^-1 is rebuilt in the kernel from k, g and beta, by the arithmetic
+ * of fla_chunk_scaled_dot_kkt_inverse (bit-identical to the matrix that operator stores). */
 int fla_prepare_wy_repr_bwd_full_accumulate_get_workspace_size(
     const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
     const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu_seqlens,

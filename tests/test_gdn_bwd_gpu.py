@@ -141,6 +141,20 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     for name, got, ref in (("dbeta", db_f, db_r), ("dg2", dg_f - dg0, dg2_r)):
         st = err_stats(got, ref)
         assert st["rel_max"] <= TOL_BF16, f"{name}, dA formed in the kernel: {st}"
+    # without A as well the kernel rebuilds each chunk's inverse as chunk_scaled_dot_kkt_inverse does: bit for bit the
+    # results of a call that is handed that operator's matrix
+    A_dev = ops.chunk_scaled_dot_kkt_inverse(x["k"], x["G"], x["beta"], chunk_size=64, **kw)
+    outs = []
+    for A_in in (A_dev, None):
+        dk_i, dg_i = dk0.clone(), dg0.clone()
+        dv_i, db_i = raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], A_in, None, dwb.to(dev), dv2.to(dev),
+                                                             x["G"], dk_i, dg_i, 64, **kw)
+        outs.append((dk_i, dg_i, dv_i, db_i))
+    for name, a_, b_ in zip(("dk", "dg", "dv", "dbeta"), *outs):
+        assert torch.equal(a_, b_), f"{name}: A rebuilt in the kernel"
+    with pytest.raises(RuntimeError, match="A must not be null"):
+        raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], None, dA, dwb.to(dev), dv2.to(dev), x["G"],
+                                                dk0.clone(), dg0.clone(), 64, **kw)
 
 
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
