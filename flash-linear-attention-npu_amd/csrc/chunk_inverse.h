@@ -21,6 +21,54 @@ __device__ __forceinline__ f32x4 solve_mm3(f32x4 a, f32x4 b, f32x4 acc) {   // a
     return acc;
 }
 
+// Column block R of the inverse below its diagonal block, top to bottom: X[k] = block (R + k, R).
+template <int R>
+__device__ __forceinline__ void invert64_column(const float *aS, elem *oS) {
+    constexpr int pa = 68, pb = 72;
+    const int l = lane_id(), li = l & 15, lg = l >> 4;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 X[4 - R];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) X[0][e] = aS[(16 * R + 4 * lg + e) * pa + 16 * R + li];
+#pragma unroll
+    for (int k = 1; k < 4 - R; ++k) {
+        const int r = R + k;
+        f32x4 sum = zero;
+#pragma unroll
+        for (int j = 0; j < k; ++j)
+            sum = solve_mm3(solve_lds4(aS + (16 * r + li) * pa + 16 * (R + j) + 4 * lg), X[j], sum);
+        const f32x4 dinv = solve_lds4(aS + (16 * r + li) * pa + 16 * r + 4 * lg);
+        X[k] = solve_mm3(-dinv, sum, zero);
+        acc_to_tile(oS, pb, 16 * r, 16 * R, X[k]);
+    }
+}
+
+// Rows 16 W .. 16 W + 15 of strict_lower(beta_t e^{g_t - g_s} <k_t, k_s>), rounded to the element type as solve_tri
+// rounds its input (chunk_scaled_dot_kkt/README.md:8-15): acc[J][e] is entry (t = 16 W + acc_col(), s = 16 J + acc_row(e)).
+// W is the calling wave's index as a compile-time value, so its W + 1 column tiles advance together through the
+// contraction instead of one branch per tile.
+template <int W>
+__device__ __forceinline__ void kkt_score_rows(const elem *kS, int pitch, int K, const float *gS, const float *bS, int len,
+                                               f32x4 (&acc)[4]) {
+    const int t = 16 * W + acc_col();
+    const float gt = gS[t], bt = bS[t];
+#pragma unroll
+    for (int J = 0; J < 4; ++J) acc[J] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int kk = 0; kk < K; kk += 32) {
+        const elemx8 own = frag_kc(kS, pitch, 16 * W, kk);
+#pragma unroll
+        for (int J = 0; J <= W; ++J) acc[J] = mfma16x32(frag_kc(kS, pitch, 16 * J, kk), own, acc[J]);
+    }
+#pragma unroll
+    for (int J = 0; J <= W; ++J)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int s = 16 * J + acc_row(e);
+            const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
+            acc[J][e] = (s < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[J][e]) : 0.f;
+        }
+}
+
 // (I + A)^-1 of the strictly lower 64 x 64 matrix in aS (fp32, pitch 68), written to oS (pitch 72) in the element
 // type; called by all four waves of a 256-thread workgroup after a barrier that completes aS, ends with one.
 __device__ __forceinline__ void invert64(float *aS, elem *oS) {
@@ -56,23 +104,11 @@ __device__ __forceinline__ void invert64(float *aS, elem *oS) {
             *reinterpret_cast<elemx4 *>(oS + (16 * R + li) * pb + 16 * cb + 4 * lg) = elemx4{(elem)0.f, (elem)0.f, (elem)0.f, (elem)0.f};
     }
     __syncthreads();
-    {   // column block R of the inverse, top to bottom: X[k] = block (R + k, R)
-        f32x4 X[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) X[0][e] = aS[(16 * R + 4 * lg + e) * pa + 16 * R + li];
-#pragma unroll
-        for (int k = 1; k < 4; ++k) {
-            if (R + k < 4) {
-                const int r = R + k;
-                f32x4 sum = zero;
-#pragma unroll
-                for (int j = 0; j < k; ++j)
-                    sum = solve_mm3(solve_lds4(aS + (16 * r + li) * pa + 16 * (R + j) + 4 * lg), X[j], sum);
-                const f32x4 dinv = solve_lds4(aS + (16 * r + li) * pa + 16 * r + 4 * lg);
-                X[k] = solve_mm3(-dinv, sum, zero);
-                acc_to_tile(oS, pb, 16 * r, 16 * R, X[k]);
-            }
-        }
+    switch (R) {   // the wave's position as a compile-time value: straight-line code per wave, operands hoisted and split once
+        case 0: invert64_column<0>(aS, oS); break;
+        case 1: invert64_column<1>(aS, oS); break;
+        case 2: invert64_column<2>(aS, oS); break;
+        default: break;   // wave 3 owns the last diagonal block only
     }
     __syncthreads();
 }

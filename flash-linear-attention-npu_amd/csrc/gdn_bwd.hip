@@ -660,7 +660,7 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
     for (int ct = 0; ct < (HOLD ? KT : 1); ++ct) dk_acc[ct] = zero4();
     char *dkg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dk.p)) + b * p.dk.sb + hk * p.dk.sh + (int64_t)start * p.dk.st);
     TileCopy<kThreads, kChunk, K> tdk;
-    if constexpr (ACC) tdk.fetch(reinterpret_cast<const elem *>(dkg), p.dk.st, len, tid);
+    if constexpr (ACC && !AINV) tdk.fetch(reinterpret_cast<const elem *>(dkg), p.dk.st, len, tid);
 
     for (int r = 0; r < rep; ++r) {
         const int hv = hk * rep + r;
@@ -669,43 +669,54 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
         {
             TileCopy<kThreads, kChunk, V> tdu, tv;
             TileCopy<kThreads, kChunk, kChunk> ta, td;
+            // AINV: k, g and beta are asked for before everything else.  Loads return in order, so the scores and the
+            // inversion can start as soon as these three are there and run while du and v are still on their way.
+            float gv = 0.f, bv = 0.f;
+            if constexpr (AINV) {
+                if (tid < kChunk) {
+                    const int t = start + min(tid, len - 1);
+                    gv = load_scalar(p.g, b, hv, t);
+                    bv = load_scalar(p.beta, b, hv, t);
+                }
+            }
             tdu.fetch(static_cast<const elem *>(p.du.p) + b * p.du.sb + hv * p.du.sh + (int64_t)start * p.du.st, p.du.st, len, tid);
             tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
             if constexpr (!AINV) ta.fetch(static_cast<const elem *>(p.A.p) + b * p.A.sb + hv * p.A.sh + (int64_t)start * p.A.st, p.A.st, len, tid);
             if constexpr (!DA) td.fetch(static_cast<const elem *>(p.dA.p) + b * p.dA.sb + hv * p.dA.sh + (int64_t)start * p.dA.st, p.dA.st, len, tid);
             if (tid < kChunk) {
-                const int t = start + min(tid, len - 1);
-                gS[tid] = load_scalar(p.g, b, hv, t);
-                bS[tid] = load_scalar(p.beta, b, hv, t);
+                if constexpr (AINV) {
+                    gS[tid] = gv;
+                    bS[tid] = bv;
+                } else {
+                    const int t = start + min(tid, len - 1);
+                    gS[tid] = load_scalar(p.g, b, hv, t);
+                    bS[tid] = load_scalar(p.beta, b, hv, t);
+                }
             }
             if (r == 0) tk.commit(kS, pk, len, tid);
             __syncthreads();
-            tdu.commit(xS, px, len, tid);
-            tv.commit(vS, pvv, len, tid);
+            if constexpr (!AINV) {
+                tdu.commit(xS, px, len, tid);
+                tv.commit(vS, pvv, len, tid);
+            }
             if constexpr (AINV) {
                 static_assert(DA && pa == 72, "the fp32 score block lies over the two dA tiles; the inverse is written at pitch 72");
                 static_assert(kChunk * 68 * 4 <= 2 * kChunk * pa * 2, "the fp32 score block must fit the two dA tiles");
                 float *sS = reinterpret_cast<float *>(dS);
-                const int t = 16 * w + li;
-                const float gt = gS[t], bt = bS[t];
-#pragma unroll
-                for (int J = 0; J < 4; ++J) {
-                    f32x4 acc = zero4();
-                    if (J <= w) {
-#pragma unroll
-                        for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(kS, pk, 16 * J, 32 * j), frag_kc(kS, pk, 16 * w, 32 * j), acc);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int s0 = 16 * J + 4 * lg + e;
-                            const float d = fminf(fmaxf(gt - gS[s0], -50.f), 50.f);
-                            acc[e] = (s0 < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[e]) : 0.f;
-                        }
-                    }
-                    *reinterpret_cast<f32x4 *>(sS + t * 68 + 16 * J + 4 * lg) = acc;
+                f32x4 sc[4];
+                switch (w) {
+                    case 0: kkt_score_rows<0>(kS, pk, K, gS, bS, len, sc); break;
+                    case 1: kkt_score_rows<1>(kS, pk, K, gS, bS, len, sc); break;
+                    case 2: kkt_score_rows<2>(kS, pk, K, gS, bS, len, sc); break;
+                    default: kkt_score_rows<3>(kS, pk, K, gS, bS, len, sc); break;
                 }
+#pragma unroll
+                for (int J = 0; J < 4; ++J) *reinterpret_cast<f32x4 *>(sS + (16 * w + li) * 68 + 16 * J + 4 * lg) = sc[J];
                 __syncthreads();
                 invert64(sS, aS);
                 if (tid < kChunk && tid >= len) aS[tid * pa + tid] = (elem)0.f;   // rows past the end hold nothing, as a staged A would
+                tdu.commit(xS, px, len, tid);
+                tv.commit(vS, pvv, len, tid);
             } else {
                 commit_square(ta, aS, pa, len, nullptr, tid);
             }
@@ -716,6 +727,9 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
         }
         // dw is fetched only now, once the registers of the first batch are free; it lands during A^T du
         tdw.fetch(static_cast<const elem *>(p.dw.p) + b * p.dw.sb + hv * p.dw.sh + (int64_t)start * p.dw.st, p.dw.st, len, tid);
+        if constexpr (ACC && AINV) {   // not needed before the end: asked for behind everything the products wait for
+            if (r == 0) tdk.fetch(reinterpret_cast<const elem *>(dkg), p.dk.st, len, tid);
+        }
         __syncthreads();
         float br[4], er[4];
 #pragma unroll

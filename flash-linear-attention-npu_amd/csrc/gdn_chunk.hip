@@ -232,22 +232,13 @@ __global__ void __launch_bounds__(kThreads) kkt_inverse_kernel(const KktParams p
     }
     __syncthreads();
     {
-        const int I = wave_id(), t = I * 16 + acc_col();
-        const float gt = gS[t], bt = bS[t];
+        const int t = wave_id() * 16 + acc_col();
         f32x4 acc[C / 16];
-#pragma unroll
-        for (int J = 0; J < C / 16; ++J) {
-            acc[J] = f32x4{0.f, 0.f, 0.f, 0.f};
-            if (J <= I) {
-                for (int kk = 0; kk < K; kk += 32)
-                    acc[J] = mfma16x32(frag_kc(kS, pitch, J * 16, kk), frag_kc(kS, pitch, I * 16, kk), acc[J]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int s = J * 16 + acc_row(e);
-                    const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
-                    acc[J][e] = (s < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[J][e]) : 0.f;
-                }
-            }
+        switch (wave_id()) {
+            case 0: kkt_score_rows<0>(kS, pitch, K, gS, bS, len, acc); break;
+            case 1: kkt_score_rows<1>(kS, pitch, K, gS, bS, len, acc); break;
+            case 2: kkt_score_rows<2>(kS, pitch, K, gS, bS, len, acc); break;
+            default: kkt_score_rows<3>(kS, pitch, K, gS, bS, len, acc); break;
         }
         __syncthreads();   // the k rows have been read by every wave
 #pragma unroll
