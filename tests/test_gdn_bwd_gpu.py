@@ -141,10 +141,11 @@ def test_backward_operators_against_oracle(dev, case, dtype):
     for name, got, ref in (("dbeta", db_f, db_r), ("dg2", dg_f - dg0, dg2_r)):
         st = err_stats(got, ref)
         assert st["rel_max"] <= TOL_BF16, f"{name}, dA formed in the kernel: {st}"
-    # without A as well the kernel rebuilds each chunk's inverse as chunk_scaled_dot_kkt_inverse does: the results are
-    # those of a call that is handed that operator's matrix, up to the last bit of the sums after it (the two forms are
-    # separate instances of the kernel, and the compiler is free to contract their multiply-adds differently); one
-    # element of A off by one step of the 16-bit type would show thousands of times above these bounds
+    # without A as well the kernel rebuilds each chunk's inverse as chunk_scaled_dot_kkt_inverse does.  dv = (A^T du) beta
+    # is one matrix product and one multiply per element, so it pins the rebuilt matrix bit for bit against a call that
+    # is handed that operator's result; the sums behind dk, dg and dbeta may differ in their last fp32 bit (the two forms
+    # are separate instances of the kernel, and the compiler is free to contract their multiply-adds differently), which
+    # now and then rounds a 16-bit result to the other neighbour
     A_dev = ops.chunk_scaled_dot_kkt_inverse(x["k"], x["G"], x["beta"], chunk_size=64, **kw)
     outs = []
     for A_in in (A_dev, None):
@@ -152,11 +153,13 @@ def test_backward_operators_against_oracle(dev, case, dtype):
         dv_i, db_i = raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], A_in, None, dwb.to(dev), dv2.to(dev),
                                                              x["G"], dk_i, dg_i, 64, **kw)
         outs.append((dk_i, dg_i, dv_i, db_i))
+    assert torch.equal(outs[0][2], outs[1][2]), "dv: A rebuilt in the kernel"
     for name, a_, b_ in zip(("dk", "dg", "dv", "dbeta"), *outs):
         st = err_stats(a_, b_)
-        assert st["rel_max"] <= (2e-6 if a_.dtype == torch.float32 else 2.0 ** -7), f"{name}: A rebuilt in the kernel: {st}"
+        # dg and dbeta are differences of sums that nearly cancel: their last-bit differences are larger relative to the result
+        assert st["rel_max"] <= (1e-4 if a_.dtype == torch.float32 else 2.0 ** -7), f"{name}: A rebuilt in the kernel: {st}"
         if a_.dtype != torch.float32:
-            assert float((a_ != b_).float().mean()) <= 1e-3, f"{name}: A rebuilt in the kernel"
+            assert int((a_ != b_).sum()) <= 2 + 1e-2 * a_.numel(), f"{name}: A rebuilt in the kernel"
     with pytest.raises(RuntimeError, match="A must not be null"):
         raw.prepare_wy_repr_bwd_full_accumulate(x["k"], x["v"], x["beta"], None, dA, dwb.to(dev), dv2.to(dev), x["G"],
                                                 dk0.clone(), dg0.clone(), 64, **kw)
