@@ -474,6 +474,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
 struct DhuParams {
     ChunkGeom geom;
     View4 q, k, w, d_o, dv, dv2;
+    View4 aqk;           // per-channel gate without dv: the chunk-diagonal blocks Aqk [B,Hv,T,64], dv = Aqk^T d_o per chunk
     View3 g;             // scalar gate [B,Hv,T] (natural log) or null
     const float *gK;     // per-channel gate [B,Hv,T,K] fp32 (log2) or null
     int64_t gk_sb, gk_sh, gk_st;
@@ -553,14 +554,34 @@ __device__ __forceinline__ void dv_rows(const elem *kS, const elem *qS, const el
     }
 }
 
-// DVL (scalar gate, 64-token chunks): dv is not an input.  Its intra-chunk part, chunk_bwd_dv_local's result
+// The same rows when the chunk's score block is an operand (per-channel gate): dv_j = sum_{i >= j} Aqk[i][j] do_i, the
+// dv of chunk_kda_bwd_dav.  Aqk is zero above its diagonal and in the rows past the chunk's end.
+template <int K, int LW>
+__device__ __forceinline__ void dv_rows_from_scores(const elem *aS, const elem *oS, elem *vS) {
+    typedef DhuSmem<K> L;
+    constexpr int pv = L::pv, ptl = L::ptl;
+    constexpr int J0 = LW / 2;   // contraction steps (32 tokens i each) that hold a non-zero tile of these rows
+    elemx8 tf[2];
+#pragma unroll
+    for (int j = J0; j < 2; ++j) tf[j] = frag_tr(aS, ptl, 16 * LW, 32 * j);
+#pragma unroll
+    for (int vt = 0; vt < 4; ++vt) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = J0; j < 2; ++j) acc = mfma16x32(tf[j], frag_tr(oS, pv, 16 * vt, 32 * j), acc);
+        acc_to_tile(vS, pv, 16 * LW, 16 * vt, acc);
+    }
+}
+
+// DVL (64-token chunks): dv is not an input.  With the per-channel gate it is Aqk^T do per chunk, from the score blocks
+// the forward kept (p.aqk; the copying waves stage the block with the other tiles, where the scalar form keeps its
+// strips).  With the scalar gate:  Its intra-chunk part, chunk_bwd_dv_local's result
 //     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i,
 // is formed by the copying waves from the k, q and do tiles they have just staged, into the place of the dv tile, in
 // the first half of the chunk's step (the compute waves read that tile in the second half): the compute waves run the
 // same code as with dv from memory.
 template <int K, bool GK, bool DVL = false>
 __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
-    static_assert(!DVL || !GK, "the in-kernel dv is built for the scalar gate");
     extern __shared__ __align__(16) unsigned char smem[];
     typedef DhuSmem<K> L;
     constexpr int VS = 64, CT = 1;
@@ -596,9 +617,11 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         struct Tiles {
             TileCopy<kThreads, kChunk, K> tk, tq, tw;
             TileCopy<kThreads, kChunk, VS> to, tv;
+            TileCopy<kThreads, kChunk, kChunk> ta;   // DVL with the per-channel gate only
             float gv;
         };
         Tiles t0, t1;
+        const elem *ag = (DVL && GK) ? static_cast<const elem *>(p.aqk.p) + b * p.aqk.sb + hv * p.aqk.sh : nullptr;
         auto fetch = [&](Tiles &t, int c) {
             c = max(c, 0);
             const int start = bos + c * kChunk;
@@ -608,6 +631,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             t.tw.fetch(wg + (int64_t)start * p.w.st, p.w.st, len, tid);
             t.to.fetch(og + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
             if constexpr (!DVL) t.tv.fetch(vg + (int64_t)start * p.dv.st, p.dv.st, len, tid);
+            if constexpr (DVL && GK) t.ta.fetch(ag + (int64_t)start * p.aqk.st, p.aqk.st, len, tid);
             if (GK) t.gv = p.gK[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + min(tid, K - 1)];
             else t.gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
         };
@@ -621,6 +645,9 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             t.tw.commit(reinterpret_cast<elem *>(buf + L::w_off), pt, len, tid);
             t.to.commit(reinterpret_cast<elem *>(buf + L::o_off), pv, len, tid);
             if constexpr (!DVL) t.tv.commit(reinterpret_cast<elem *>(buf + L::v_off), pv, len, tid);
+            // one score tile serves both buffers: it is written in the second half of a step and read in the first half
+            // of the next one, by the copying waves only
+            if constexpr (DVL && GK) t.ta.commit(reinterpret_cast<elem *>(smem + L::t_off), L::ptl, len, tid);
             if (GK) {
                 if (tid < K) gS[tid] = exp2f(t.gv);
                 if (tid < kChunk) fS[tid] = p.scale;
@@ -685,11 +712,20 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
             const int len = min(kChunk, eos - (bos + c * kChunk));
             elem *strips = reinterpret_cast<elem *>(smem + L::t_off);
-            switch (wave_id() - 4) {   // the row tile as a constant: every operand read of the wave is issued at once
-                case 0: dv_rows<K, 0>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                case 1: dv_rows<K, 1>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                case 2: dv_rows<K, 2>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                default: dv_rows<K, 3>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+            if constexpr (GK) {
+                switch (wave_id() - 4) {
+                    case 0: dv_rows_from_scores<K, 0>(strips, oS, vS); break;
+                    case 1: dv_rows_from_scores<K, 1>(strips, oS, vS); break;
+                    case 2: dv_rows_from_scores<K, 2>(strips, oS, vS); break;
+                    default: dv_rows_from_scores<K, 3>(strips, oS, vS); break;
+                }
+            } else {
+                switch (wave_id() - 4) {   // the row tile as a constant: every operand read of the wave is issued at once
+                    case 0: dv_rows<K, 0>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                    case 1: dv_rows<K, 1>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                    case 2: dv_rows<K, 2>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                    default: dv_rows<K, 3>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                }
             }
         };
         // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
@@ -1072,8 +1108,10 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
                  const fla_tensor *g, const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht,
                  const fla_int_array *cu, const fla_int_array *ci, double scale, int64_t chunk_size, bool use_exp2,
                  const fla_tensor *dh, const fla_tensor *dh0, const fla_tensor *dv2, void *ws, uint64_t ws_size,
-                 hipStream_t stream, uint64_t *query) {
-    const char *op = "chunk_gated_delta_rule_bwd_dhu";
+                 hipStream_t stream, uint64_t *query, const fla_tensor *aqk = nullptr) {
+    // with aqk: the form for the KDA backward, whose dv operand is Aqk^T d_o per chunk and is formed inside the scan
+    const bool has_aqk = aqk && aqk->data;
+    const char *op = has_aqk ? "chunk_kda_bwd_dhu" : "chunk_gated_delta_rule_bwd_dhu";
     (void)h0;  // only its presence matters to the caller (it decides whether dh0 is allocated)
     const bool has_g = g && g->data, has_gk = gK && gK->data;
     FLA_REQUIRE(has_g != has_gk, FLA_ERR_NULL, "%s: exactly one of g and gK must be provided.", op);
@@ -1083,8 +1121,10 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     int rc;
     // dv absent: the intra-chunk part of dv (chunk_bwd_dv_local's result) is formed inside the scan
     const bool has_dv = dv && dv->data;
-    FLA_REQUIRE(has_dv || (has_g && chunk_size == kChunk), FLA_ERR_UNSUPPORTED,
+    FLA_REQUIRE(has_dv || has_aqk || (has_g && chunk_size == kChunk), FLA_ERR_UNSUPPORTED,
                 "%s: dv may be left out with the scalar gate g and chunk_size 64 only.", op);
+    FLA_REQUIRE(!has_aqk || (has_gk && !has_dv && chunk_size == kChunk), FLA_ERR_UNSUPPORTED,
+                "%s: Aqk takes the place of dv with the per-channel gate gK and chunk_size 64 only.", op);
     if ((rc = gdn_geometry(op, k, has_dv ? dv : d_o, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
     FLA_REQUIRE(geom.C == kChunk || !has_gk, FLA_ERR_UNSUPPORTED, "%s: gK is built for chunk_size 64.", op);
     const int bf = dt_bit(kElemDtype);
@@ -1093,6 +1133,8 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     if ((rc = check_bhtd(op, "w", w, geom.B, geom.Hv, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "d_o", d_o, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if (has_dv && (rc = check_bhtd(op, "dv", dv, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
+    if (has_aqk && (rc = check_bhtd(op, "Aqk", aqk, geom.B, geom.Hv, geom.T, kChunk, bf))) return rc;
+    FLA_REQUIRE(!has_aqk || geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
     if ((rc = check_bhtd(op, "dv2", dv2, geom.B, geom.Hv, geom.T, geom.V, bf))) return rc;
     if (has_g && (rc = check_bht(op, "g", g, geom.B, geom.Hv, geom.T, kElemDtype))) return rc;
     if (has_gk) {
@@ -1157,6 +1199,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.w = view4(w);
     p.d_o = view4(d_o);
     if (has_dv) p.dv = view4(dv);
+    if (has_aqk) p.aqk = view4(aqk);
     p.dv2 = view4(dv2);
     if (has_g) p.g = view3(g);
     if (has_gk) {
@@ -1183,6 +1226,7 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.scale = (float)scale;
     p.sub = geom.C / kChunk;
     const int slabs = geom.V / 64;
+    if (has_aqk) return geom.K == 128 ? launch_bwd_dhu<128, true, true>(p, slabs, stream) : launch_bwd_dhu<64, true, true>(p, slabs, stream);
     if (!has_dv) return geom.K == 128 ? launch_bwd_dhu<128, false, true>(p, slabs, stream) : launch_bwd_dhu<64, false, true>(p, slabs, stream);
     if (geom.K == 256) return launch_bwd_dhu_wide<256>(p, slabs, stream);
     if (geom.K == 128) return has_gk ? launch_bwd_dhu<128, true>(p, slabs, stream) : launch_bwd_dhu<128, false>(p, slabs, stream);
@@ -1212,6 +1256,29 @@ FLA_ENTRY(fla_chunk_gated_delta_rule_fwd_h)(
     return fla::guarded([&] { return fla::fwd_h_impl(k, w, u, g, gk, initial_state, output_final_state, chunk_size, cu_seqlens, chunk_indices,
                            state_v_first, h, v_new, final_state, workspace, workspace_size,
                            static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_dhu_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *Aqk,
+    const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
+    const fla_tensor *dv2, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dhu_get_workspace_size, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace_size);
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: workspace_size must not be null.");
+    if (!Aqk || !Aqk->data) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: Aqk must not be null.");
+    return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, nullptr, nullptr, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, true,
+                             dh, dh0, dv2, nullptr, 0, nullptr, workspace_size, Aqk); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_dhu)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *Aqk,
+    const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
+    const fla_tensor *dv2, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dhu, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace, workspace_size, stream);
+    if (!Aqk || !Aqk->data) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: Aqk must not be null.");
+    return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, nullptr, nullptr, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, true,
+                             dh, dh0, dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, Aqk); });
 }
 
 FLA_ENTRY(fla_chunk_gated_delta_rule_bwd_dhu_get_workspace_size)(

@@ -105,6 +105,7 @@ struct KdaDqkwgParams {
     int64_t h_sb, h_sh, h_sc, dh_sb, dh_sh, dh_sc;
     ViewF dq, dk, dg;
     float scale;
+    ViewF daqk;   // optional f32 [B,Hv,T,64]: dAqk = scale tril(d_o v_new^T), the first result of chunk_kda_bwd_dav
 };
 
 template <int K, int V>
@@ -186,6 +187,24 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_kernel(const KdaD
         }
     }
     __syncthreads();
+    if (p.daqk.p != nullptr) {   // dAqk[i][j] = scale <do_i, v_new_j>, j <= i: row tile w, two column tiles per wave
+        float *dag = p.daqk.p + b * p.daqk.sb + hv * p.daqk.sh + (int64_t)start * p.daqk.st;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int ct = 2 * half + cc;
+            f32x4 acc = zero4();
+            if (ct <= w) {
+#pragma unroll
+                for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+            }
+            const int col = 16 * ct + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                if (row < len) dag[(int64_t)row * p.daqk.st + col] = (ct <= w && col <= row) ? acc[e] * p.scale : 0.f;
+            }
+        }
+    }
     // ---- products with the state at chunk start: dq (do h^T) and dw (-dv h^T) ---------------------
     f32x4 dqa[KTH], dka[KTH];
     char *dwg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dw.p)) + b * p.dw.sb + hv * p.dw.sh +
@@ -531,7 +550,8 @@ int dav_impl(const fla_tensor *v_new, const fla_tensor *d_o, const fla_tensor *a
 int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
                    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
                    const fla_int_array *ci, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
-                   const fla_tensor *dw, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+                   const fla_tensor *dw, const fla_tensor *dg, const fla_tensor *daqk, void *ws, uint64_t ws_size, hipStream_t stream,
+                   uint64_t *query) {
     const char *op = "chunk_kda_bwd_dqkwg";
     ChunkGeom geom;
     int rc;
@@ -548,6 +568,8 @@ int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v
     if ((rc = check_f32_bhtd(op, "dq", dq, B, Hv, T, K))) return rc;
     if ((rc = check_f32_bhtd(op, "dk", dk, B, Hv, T, K))) return rc;
     if ((rc = check_f32_bhtd(op, "dg", dg, B, Hv, T, K))) return rc;
+    const bool has_daqk = daqk && daqk->data;
+    if (has_daqk && (rc = check_f32_bhtd(op, "dAqk", daqk, B, Hv, T, kChunk))) return rc;
     Varlen vl;
     if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
     if ((rc = check_state_blocks(op, "h", h, geom))) return rc;
@@ -558,7 +580,7 @@ int kda_dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v
                      static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
                      static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                      h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
-                     viewf(dq), viewf(dk), viewf(dg), (float)scale};
+                     viewf(dq), viewf(dk), viewf(dg), (float)scale, has_daqk ? viewf(daqk) : ViewF{nullptr, 0, 0, 0}};
     const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
     const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
                         (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
@@ -637,20 +659,20 @@ FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_get_workspace_size)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
     const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
-    const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size) {
-    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace_size);
+    const fla_tensor *dw, const fla_tensor *dg, const fla_tensor *dAqk, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, dAqk, workspace_size);
     FLA_NULL_WS("chunk_kda_bwd_dqkwg");
     return fla::guarded([&] { return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
-                               nullptr, 0, nullptr, workspace_size); });
+                               dAqk, nullptr, 0, nullptr, workspace_size); });
 }
 FLA_ENTRY(fla_chunk_kda_bwd_dqkwg)(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
     const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
-    const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream) {
-    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, workspace, workspace_size, stream);
+    const fla_tensor *dw, const fla_tensor *dg, const fla_tensor *dAqk, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg, q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg, dAqk, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::kda_dqkwg_impl(q, k, v_new, gk, h, d_o, dh, dv, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dw, dg,
-                               workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+                               dAqk, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
 }
 
 FLA_ENTRY(fla_chunk_kda_bwd_wy_get_workspace_size)(

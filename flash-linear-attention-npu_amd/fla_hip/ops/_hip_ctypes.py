@@ -74,7 +74,8 @@ OP_ARGTYPES = {
     "chunk_bwd_dqkwg_l2norm": [_T] * 8 + [_IA, _IA, _T, ctypes.c_float, ctypes.c_int64] + [_T] * 4,
     "prepare_wy_repr_bwd": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 4,
     "chunk_kda_bwd_dav": [_T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T, _T],
-    "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 4,
+    "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 5,
+    "chunk_kda_bwd_dhu": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 3,
     "chunk_kda_bwd_wy": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 5,
 }
 
@@ -834,10 +835,11 @@ def chunk_kda_bwd_dav(v_new, d_o, Aqk, scale, chunk_size=64, *, cu_seqlens=None,
 
 
 def chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, d_o, dh, dv, scale, chunk_size=64, *, cu_seqlens=None, chunk_indices=None,
-                        layout_like=None):
+                        layout_like=None, with_dAqk=False):
     """State-dependent part of the KDA backward: returns ``(dq, dk, dw, dg)``, dq / dk / dg fp32 [B,Hv,T,K] per value
     head laid out like ``layout_like`` (default: like ``gk``), dw [B,Hv,T,K] in the dtype of q.
-    ``h`` and ``dh`` are [B,Hv,NT,K,V] views (any outer strides)."""
+    ``h`` and ``dh`` are [B,Hv,NT,K,V] views (any outer strides).  ``with_dAqk=True``: a fifth result, the dAqk of
+    ``chunk_kda_bwd_dav`` (fp32 [B,Hv,T,64] laid out like the others), from the d_o and v_new tiles staged anyway."""
     import torch
 
     B, Hv, T, K = _shape(gk)
@@ -846,19 +848,52 @@ def chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, d_o, dh, dv, scale, chunk_size=64, *
     dk = _empty_strided_like((B, Hv, T, K), like, torch.float32, q.device)
     dg = _empty_strided_like((B, Hv, T, K), like, torch.float32, q.device)
     dw = _empty((B, Hv, T, K), q)
+    dAqk = _empty_strided_like((B, Hv, T, 64), like, torch.float32, q.device) if with_dAqk else None
     cu = _as_int_tuple(cu_seqlens)
-    outs = (dq, dk, dw, dg)
+    outs = (dq, dk, dw, dg) + ((dAqk,) if with_dAqk else ())
     _call_op(
         "chunk_kda_bwd_dqkwg", OP_ARGTYPES["chunk_kda_bwd_dqkwg"],
         lambda ctx: [
             ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v_new, "v_new"), ctx.tensor(gk, "gk"), ctx.tensor(h, "h"),
             ctx.tensor(d_o, "d_o"), ctx.tensor(dh, "dh"), ctx.tensor(dv, "dv"), ctx.int_array(cu),
             ctx.int_array(_as_int_tuple(chunk_indices)), ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
-            *[ctx.tensor(t, n) for t, n in zip(outs, ("dq", "dk", "dw", "dg"))],
+            *[ctx.tensor(t, n) for t, n in zip((dq, dk, dw, dg, dAqk), ("dq", "dk", "dw", "dg", "dAqk"))],
         ],
         outs,
     )
     return outs
+
+
+def chunk_kda_bwd_dhu(qg, kg, w, d_o, Aqk, scale, chunk_size=64, *, gK, h0=None, dht=None, cu_seqlens=None, chunk_indices=None):
+    """``npu_chunk_gated_delta_rule_bwd_dhu`` for the KDA backward (per-channel gate ``gK`` in log2 units, 64-token
+    chunks) with its dv operand formed inside the scan: dv = Aqk^T d_o per chunk, the second result of
+    ``chunk_kda_bwd_dav``, from the forward's score blocks ``Aqk`` [B,Hv,T,64] and the d_o tiles the scan stages anyway.
+    Returns ``(dh, dh0, dv2)`` with dh0 fp32 [N,Hv,K,V] (None without ``h0``).  No counterpart in the reference."""
+    import torch
+
+    B, _, T, K = _shape(qg)
+    _, Hv, _, V = _shape(d_o)
+    chunk_size = int(chunk_size)
+    cu = _as_int_tuple(cu_seqlens)
+    indices = _as_int_tuple(chunk_indices)
+    if indices is None and cu is not None:
+        indices = _build_chunk_indices(cu, chunk_size)
+    NT = _total_chunks(B, T, chunk_size, cu) if indices is None else len(indices) // 2
+    N = len(cu) - 1 if cu is not None else B
+    dh = _empty((B, Hv, NT, K, V), qg)
+    dh0 = None if h0 is None else _empty((N, Hv, K, V), qg, dtype=torch.float32)
+    dv2 = _empty_ordered_like(d_o)
+    outputs = (dh, dh0, dv2)
+    return _call_op(
+        "chunk_kda_bwd_dhu", OP_ARGTYPES["chunk_kda_bwd_dhu"],
+        lambda ctx: [
+            ctx.tensor(qg, "q"), ctx.tensor(kg, "k"), ctx.tensor(w, "w"), ctx.tensor(d_o, "d_o"), ctx.tensor(Aqk, "Aqk"),
+            ctx.tensor(gK, "gK"), ctx.tensor(h0, "h0"), ctx.tensor(dht, "dht"),
+            ctx.int_array(cu), ctx.int_array(indices), ctypes.c_double(float(scale)), ctypes.c_int64(chunk_size),
+            ctx.tensor(dh, "dh"), ctx.tensor(dh0, "dh0"), ctx.tensor(dv2, "dv2"),
+        ],
+        outputs,
+    )
 
 
 def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, dk, dg, chunk_size=64, *, cu_seqlens=None, chunk_indices=None):

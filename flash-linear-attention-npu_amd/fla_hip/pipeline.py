@@ -286,8 +286,8 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     q, k, v, beta, do in ``layout``; gk, Aqk, Akk, w, qg, kg, v_new head-major and h as the forward returned them;
     dht fp32 [N,Hv,K,V] or None.  Returns ``(dq, dk, dv, dg, dbeta, dh0)``: dq, dk, dv, dbeta in ``layout`` and the
     dtype of their inputs, dg fp32 in the layout of the gate = gradient of the per-token log decay (natural log),
-    dh0 fp32 [N,Hv,K,V] or None.  Stages: dAqk / dv -> reverse scan (bwd_dhu, gK) -> dq, dk, dw, dg of the
-    state-dependent parts -> backward of the WY factors (dv, dbeta, dAkk) -> chunk_kda_bwd_intra -> reverse
+    dh0 fp32 [N,Hv,K,V] or None.  Stages: reverse scan (bwd_dhu, gK; it forms dv = Aqk^T do itself) -> dq, dk, dw, dg of
+    the state-dependent parts and dAqk -> backward of the WY factors (dv, dbeta, dAkk) -> chunk_kda_bwd_intra -> reverse
     chunk-local cumulative sum of dg."""
     import torch
 
@@ -306,16 +306,19 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     Hk, Hv = qh.shape[1], vh.shape[1]
     # fp32 gradients per value head, laid out in memory like the caller's tensors (heads = Hv)
     layout_like = _index_order(_empty_in_layout(layout, gk4.shape), layout)
-    dAqk, dv0 = _raw.chunk_kda_bwd_dav(vn4, doh, Aqk4, scale, chunk_size, layout_like=layout_like, **kw)
-    dh, dh0, dv2 = _ops.chunk_gated_delta_rule_bwd_dhu(qg4, kg4, w4, doh, dv0, scale, chunk_size, gK=gk4,
-                                                       h0=initial_state, dht=dht, use_exp2=True, dh0_per_sequence=True,
-                                                       **kw)
     if qh.shape[-1] > 128:
+        dAqk, dv0 = _raw.chunk_kda_bwd_dav(vn4, doh, Aqk4, scale, chunk_size, layout_like=layout_like, **kw)
+        dh, dh0, dv2 = _ops.chunk_gated_delta_rule_bwd_dhu(qg4, kg4, w4, doh, dv0, scale, chunk_size, gK=gk4,
+                                                           h0=initial_state, dht=dht, use_exp2=True, dh0_per_sequence=True,
+                                                           **kw)
         dq, dk, dg, dv, db, dAkk = _kda_bwd_state_stages_by_channel_halves(qh, kh, vh, bh, gk4, Akk4, vn4, h5, doh, dh, dv2, scale,
                                                                             chunk_size, layout_like, kw)
     else:
-        dq, dk, dw, dg = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
-                                                  layout_like=layout_like, **kw)
+        # no pass for chunk_kda_bwd_dav: the reverse scan forms dv = Aqk^T do from the score blocks, the next stage writes
+        # dAqk = scale tril(do v_new^T) from the do and v_new tiles it stages anyway
+        dh, dh0, dv2 = _raw.chunk_kda_bwd_dhu(qg4, kg4, w4, doh, Aqk4, scale, chunk_size, gK=gk4, h0=initial_state, dht=dht, **kw)
+        dq, dk, dw, dg, dAqk = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
+                                                        layout_like=layout_like, with_dAqk=True, **kw)
         dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
     # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
     back = lambda t: _from_index_order(t, layout)

@@ -474,17 +474,36 @@ int fla_chunk_kda_bwd_dav(
 /* chunk_kda_bwd_dqkwg: with h the state at each chunk start, dh the gradient of the state at each chunk
  * end and dv the total gradient of v_new (dh, dv: outputs of bwd_dhu), both [B,Hv,NT,K,V] with any outer strides:
  *   dq = scale (d_o h^T) 2^g,  dk = (v_new dh^T) 2^{g_last - g},  dw = -dv h^T (element type, [B,Hv,T,K]),
- *   dg = q dq - k dk, plus on the last token of a chunk  sum_j k_j dk_j + 2^{g_last} rowsum(h . dh). */
+ *   dg = q dq - k dk, plus on the last token of a chunk  sum_j k_j dk_j + 2^{g_last} rowsum(h . dh).
+ * dAqk (f32 [B,Hv,T,64], or NULL): also written, the first result of chunk_kda_bwd_dav (scale * tril(d_o v_new^T)),
+ * from the d_o and v_new tiles this operator stages anyway. */
 int fla_chunk_kda_bwd_dqkwg_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
     const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
-    const fla_tensor *dw, const fla_tensor *dg, uint64_t *workspace_size);
+    const fla_tensor *dw, const fla_tensor *dg, const fla_tensor *dAqk, uint64_t *workspace_size);
 int fla_chunk_kda_bwd_dqkwg(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
     const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
-    const fla_tensor *dw, const fla_tensor *dg, void *workspace, uint64_t workspace_size, void *stream);
+    const fla_tensor *dw, const fla_tensor *dg, const fla_tensor *dAqk, void *workspace, uint64_t workspace_size,
+    void *stream);
+
+/* chunk_kda_bwd_dhu: chunk_gated_delta_rule_bwd_dhu with the per-channel gate gK (log2 units, use_exp2) whose dv
+ * operand, dv = Aqk^T d_o per chunk (the second result of chunk_kda_bwd_dav), is formed inside the scan from the
+ * forward's score blocks Aqk [B,Hv,T,64] and the d_o tiles it stages anyway, so that dv never goes through memory.
+ * No counterpart in the reference (see the note above); q, k are the gated qg, kg of the forward.  chunk_size 64,
+ * K in {64,128}.  Outputs as chunk_gated_delta_rule_bwd_dhu. */
+int fla_chunk_kda_bwd_dhu_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *Aqk,
+    const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
+    const fla_tensor *dv2, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_dhu(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *Aqk,
+    const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
+    const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
+    const fla_tensor *dv2, void *workspace, uint64_t workspace_size, void *stream);
 
 /* chunk_kda_bwd_wy: backward of w = Akk (k beta 2^g), u = Akk (v beta), Akk = (I + M)^-1 given dw, du:
  *   x = Akk^T dw, y = Akk^T du;  dk += x beta 2^g;  dg += (x beta 2^g) k   (dk, dg are read and added to);

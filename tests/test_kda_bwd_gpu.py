@@ -96,6 +96,15 @@ def test_bwd_dqkwg(dev, case):
     assert out2[0].transpose(1, 2).is_contiguous()
     for a, e in zip(out2, (dq, dk, dw, dg)):
         assert torch.equal(a, e)
+    # with dAqk asked for: chunk_kda_bwd_dav's first result from the do and v_new tiles staged here, the rest unchanged
+    out3 = raw.chunk_kda_bwd_dqkwg(*to(q, k, v_new, gk, h, do, dh, dv), 0.7, cu_seqlens=cu, with_dAqk=True)
+    for a, e in zip(out3[:4], (dq, dk, dw, dg)):
+        assert torch.equal(a, e)
+    dA_ref, _ = kda.chunk_kda_bwd_dav(v_new, do, torch.zeros(B, Hv, T, 64, dtype=BF), 0.7, cu_seqlens=cu)
+    assert out3[4].dtype == torch.float32
+    close(out3[4], dA_ref, "dAqk", 1e-3)
+    dA_dev, _ = raw.chunk_kda_bwd_dav(v_new.to(dev), do.to(dev), torch.zeros(B, Hv, T, 64, dtype=BF, device=dev), 0.7, cu_seqlens=cu)
+    assert torch.equal(out3[4], dA_dev)
 
 
 @pytest.mark.parametrize("case", STAGE_CASES)

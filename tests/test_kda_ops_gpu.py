@@ -150,6 +150,51 @@ def test_bwd_dhu(dev, case):
     assert out3[1] is None
 
 
+@pytest.mark.parametrize("case", [c for c in DHU_CASES if c[7] and c[4] <= 128],
+                         ids=lambda c: f"T{c[1]}-K{c[4]}-V{c[5]}")
+def test_kda_bwd_dhu_forms_dv_from_the_score_blocks(dev, case):
+    """chunk_kda_bwd_dhu (no counterpart in the reference): the per-channel-gate scan with dv = Aqk^T d_o formed
+    inside.  Against the oracle's two operators (chunk_kda_bwd_dav's dv, rounded as it is exchanged, then the scan) and
+    against the two-operator route on the device, whose dv tile holds the same 16-bit values."""
+    from fla_hip import ops
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, Hk, Hv, K, V, cu, _, with_dht = case
+    q, k, w, d_o, _, gate = dhu_inputs(B, T, Hk, Hv, K, V, seed=T + V + 1, per_channel=True)
+    scale = K ** -0.5
+    gcum = kda.kda_gate_cumsum(gate, 64, cu_seqlens=cu)
+    qg = (q.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(gcum)).to(BF)
+    last = torch.zeros_like(gcum)
+    gen = torch.Generator().manual_seed(11)
+    Aqk = torch.zeros(B, Hv, T, 64)
+    for b, n, ci, s, e in gdn.chunk_spans(B, T, 64, cu):
+        last[b, :, s:e] = gcum[b, :, e - 1:e]
+        Aqk[b, :, s:e, :e - s] = torch.tril(torch.randn(Hv, e - s, e - s, generator=gen) * 0.3)
+    Aqk = Aqk.to(BF)
+    kg = (k.float().repeat_interleave(Hv // Hk, 1) * torch.exp2(last - gcum)).to(BF)
+    N = B if cu is None else len(cu) - 1
+    dht = torch.randn(N, Hv, K, V, generator=gen) * 0.1 if with_dht else None
+    h0 = torch.zeros(N, Hv, K, V, device=dev)
+    dht_d = None if dht is None else dht.to(dev)
+    qd, kd, wd, od, ad, gd = (t.to(dev) for t in (qg, kg, w, d_o, Aqk, gcum))
+    dh, dh0, dv2 = raw.chunk_kda_bwd_dhu(qd, kd, wd, od, ad, scale, 64, gK=gd, h0=h0, dht=dht_d, cu_seqlens=cu)
+    assert dh.dtype == BF and dv2.dtype == BF and dh0.dtype == torch.float32 and dv2.shape == d_o.shape
+    _, dv_ref = kda.chunk_kda_bwd_dav(d_o, d_o, Aqk, scale, cu_seqlens=cu)
+    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(qg, kg, w, d_o, dv_ref.to(BF), scale, 64, dht=dht, cu_seqlens=cu,
+                                                                  gK=gcum)
+    assert_close(dv2, dv2_ref, TOL_BF16, "dv2")
+    assert_close(dh, dh_ref, TOL_BF16, "dh")
+    assert_close(dh0, dh0_ref, TOL_BF16, "dh0")
+    _, dv_two = raw.chunk_kda_bwd_dav(od, od, ad, scale, cu_seqlens=cu)
+    two = ops.chunk_gated_delta_rule_bwd_dhu(qd, kd, wd, od, dv_two, scale, 64, gK=gd, use_exp2=True, h0=h0, dht=dht_d,
+                                             cu_seqlens=cu, dh0_per_sequence=True)
+    # the same operands in another order of accumulation: far inside the oracle's bound
+    for name, a_, b_ in zip(("dh", "dh0", "dv2"), (dh, dh0, dv2), two):
+        assert_close(a_, b_, 2.0 ** -7 if a_.dtype != torch.float32 else 1e-4, name + " against the two-operator route")
+    assert raw.chunk_kda_bwd_dhu(qd, kd, wd, od, ad, scale, 64, gK=gd, cu_seqlens=cu)[1] is None
+    with pytest.raises(RuntimeError, match="Aqk"):
+        raw.chunk_kda_bwd_dhu(qd, kd, wd, od, None, scale, 64, gK=gd, cu_seqlens=cu)
+
+
 def test_bwd_dhu_first_chunk_is_terminal_gradient(dev):
     """dh of the last chunk is the terminal gradient itself (zero without dht)."""
     from fla_hip import ops
