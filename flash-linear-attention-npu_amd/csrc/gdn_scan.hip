@@ -851,12 +851,14 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 for (int kt = 0; kt < KT; ++kt) dacc[kt][0] = mfma16x32(frag_tr(qS, pt, kt * 16, 32 * j), ob, dacc[kt][0]);
             }
         };
-        // DVL: the copying waves form the dv tile in this half of the step, so the part of the update that needs neither
-        // dv nor the place of the k tile moves in front of the barrier; dh then leaves from its 16-bit copy
-        if constexpr (DVL) decay_and_q_term();
+        // DVL with the scalar gate: the copying waves spend this half of the step on the dv tile, so the part of the update
+        // that needs neither dv nor the place of the k tile moves in front of the barrier; dh then leaves from its 16-bit
+        // copy.  (From score blocks the dv tile is two products per wave: the order of the plain form is kept.)
+        constexpr bool EARLY = DVL && !GK;
+        if constexpr (EARLY) decay_and_q_term();
         lds_barrier();   // every wave is past the k tile, which now takes dh on its way to memory
         if (chunk_end) {
-            if constexpr (DVL) {
+            if constexpr (EARLY) {
 #pragma unroll
                 for (int j = 0; j < KS; ++j) {
                     const u32x4 d = __builtin_bit_cast(u32x4, hB[j][0]);
@@ -884,7 +886,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         for (int rt = 0; rt < 4; ++rt) acc_to_tile(vS, pv, rt * 16, wv * 16, dv2[rt][0]);   // over the wave's own columns of dv
 
         // dh <- decay * dh + scale (q e^g)^T do - w^T dv2
-        if constexpr (DVL) {
+        if constexpr (EARLY) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const elemx8 nb = frag_from_acc(-dv2[2 * j][0], -dv2[2 * j + 1][0]);
