@@ -499,7 +499,7 @@ template <int K> struct DhuSmem {
     static constexpr size_t g_off = v_off + (size_t)kChunk * pv * 2;      // [max(K,64)] gate row, [64] factors
     static constexpr size_t buf_bytes = g_off + (size_t)((K > kChunk ? K : kChunk) + kChunk) * 4;
     static constexpr size_t bytes = 2 * buf_bytes;
-    // the form that builds dv itself: four strips [16][ptl] behind the two buffers, one per copying wave
+    // the form that builds dv itself: one [64][ptl] tile behind the two buffers (T, or the chunk's score block)
     static constexpr int ptl = kChunk + 8;
     static constexpr size_t t_off = bytes;
     static constexpr size_t bytes_dvl = t_off + (size_t)4 * 16 * ptl * 2;
@@ -509,53 +509,48 @@ template <int K> struct DhuSmem {
 // the tiles of chunk c-1 into the other buffer and have those of chunk c-2 in flight.  Both results leave through LDS
 // as whole 128-byte rows, stored by the copying waves one step later: dv2 replaces the wave's own columns of the dv
 // tile, dh goes over the k tile once every wave is past its k . dh products (the barrier in the middle of a step).
-// Rows 16 LW.. of the intra-chunk dv of one chunk (see bwd_dhu_kernel, DVL), by one wave.
-template <int K, int LW>
-__device__ __forceinline__ void dv_rows(const elem *kS, const elem *qS, const elem *oS, elem *vS, const float *gS, elem *strips,
-                                        int len, float scale) {
+// Tile (R, CT) of T[j][i] = scale (k_j . q_i) e^{g_i - g_j}, i >= j (see bwd_dhu_kernel, DVL), into the chunk's 64 x 64
+// tile tS, rounded to the element type: rows are the tokens j whose dv the tile feeds, columns the tokens i of do.
+template <int K, int R, int CT>
+__device__ __forceinline__ void t_tile(const elem *kS, const elem *qS, const float *gS, elem *tS, int len, float scale) {
     typedef DhuSmem<K> L;
-    constexpr int pk = L::pk, pt = L::pt, pv = L::pv, ptl = L::ptl, KS = K / 32;
+    constexpr int pk = L::pk, pt = L::pt, ptl = L::ptl, KS = K / 32;
     const int l = lane_id(), li = l & 15, lg = l >> 4;
-    elem *tS = strips + LW * 16 * ptl;
-    f32x4 t[4];
+    f32x4 t = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ct = LW; ct < 4; ++ct) t[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < KS; ++j) t = mfma16x32(frag_kc(kS, pk, 16 * R, 32 * j), frag_kc(qS, pt, 16 * CT, 32 * j), t);
+    const int i = 16 * CT + li;
+    const float gi = gS[i];
+    f32x4 x;
 #pragma unroll
-    for (int j = 0; j < KS; ++j) {
-        const elemx8 a = frag_kc(kS, pk, 16 * LW, 32 * j);
-#pragma unroll
-        for (int ct = LW; ct < 4; ++ct) t[ct] = mfma16x32(a, frag_kc(qS, pt, 16 * ct, 32 * j), t[ct]);
+    for (int e = 0; e < 4; ++e) {
+        const int j = 16 * R + 4 * lg + e;
+        // the gates enter as a difference: e^{g_i} and e^{-g_j} on their own leave the fp32 range for strong decays
+        x[e] = ((CT > R || i >= j) && i < len) ? t[e] * scale * __expf(gi - gS[j]) : 0.f;
     }
-    f32x4 gj;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) gj[e] = gS[16 * LW + 4 * lg + e];
-#pragma unroll
-    for (int ct = 0; ct < 4; ++ct) {
-        f32x4 x = {0.f, 0.f, 0.f, 0.f};
-        if (ct >= LW) {
-            const int i = 16 * ct + li;
-            const float gi = gS[i];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] = (i >= 16 * LW + 4 * lg + e && i < len) ? t[ct][e] * scale * __expf(gi - gj[e]) : 0.f;
-        }
-        acc_to_tile(tS, ptl, 0, 16 * ct, x);
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own strip, written and read by itself
-    constexpr int J0 = LW / 2;   // contraction steps (32 tokens i each) that hold a non-zero tile of these rows
-    elemx8 tf[2];
-#pragma unroll
-    for (int j = J0; j < 2; ++j) tf[j] = frag_kc(tS, ptl, 0, 32 * j);
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = J0; j < 2; ++j) acc = mfma16x32(tf[j], frag_tr(oS, pv, 16 * vt, 32 * j), acc);
-        acc_to_tile(vS, pv, 16 * LW, 16 * vt, acc);
+    acc_to_tile(tS, ptl, 16 * R, 16 * CT, x);
+}
+
+// The six tiles above the diagonal, dealt to the four copying waves (2, 2, 1, 1); the four diagonal tiles are taken by
+// the compute waves, one each, which otherwise wait for the copying waves in that half of the step.
+template <int K, int LW>
+__device__ __forceinline__ void t_tiles(const elem *kS, const elem *qS, const float *gS, elem *tS, int len, float scale) {
+    if constexpr (LW == 0) {
+        t_tile<K, 0, 1>(kS, qS, gS, tS, len, scale);
+        t_tile<K, 0, 2>(kS, qS, gS, tS, len, scale);
+    } else if constexpr (LW == 1) {
+        t_tile<K, 0, 3>(kS, qS, gS, tS, len, scale);
+        t_tile<K, 1, 2>(kS, qS, gS, tS, len, scale);
+    } else if constexpr (LW == 2) {
+        t_tile<K, 1, 3>(kS, qS, gS, tS, len, scale);
+    } else {
+        t_tile<K, 2, 3>(kS, qS, gS, tS, len, scale);
     }
 }
 
-// The same rows when the chunk's score block is an operand (per-channel gate): dv_j = sum_{i >= j} Aqk[i][j] do_i, the
-// dv of chunk_kda_bwd_dav.  Aqk is zero above its diagonal and in the rows past the chunk's end.
+// Rows 16 LW.. of the dv operand when the chunk's score block is an operand (per-channel gate):
+// dv_j = sum_{i >= j} Aqk[i][j] do_i, the dv of chunk_kda_bwd_dav, by one wave.  Aqk is zero above its diagonal and in
+// the rows past the chunk's end.
 template <int K, int LW>
 __device__ __forceinline__ void dv_rows_from_scores(const elem *aS, const elem *oS, elem *vS) {
     typedef DhuSmem<K> L;
@@ -574,12 +569,14 @@ __device__ __forceinline__ void dv_rows_from_scores(const elem *aS, const elem *
 }
 
 // DVL (64-token chunks): dv is not an input.  With the per-channel gate it is Aqk^T do per chunk, from the score blocks
-// the forward kept (p.aqk; the copying waves stage the block with the other tiles, where the scalar form keeps its
-// strips).  With the scalar gate:  Its intra-chunk part, chunk_bwd_dv_local's result
-//     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i,
-// is formed by the copying waves from the k, q and do tiles they have just staged, into the place of the dv tile, in
-// the first half of the chunk's step (the compute waves read that tile in the second half): the compute waves run the
-// same code as with dv from memory.
+// the forward kept (p.aqk): the copying waves stage the block with the other tiles and write Aqk^T do where the dv tile
+// would have been loaded, and the compute waves run the code of the plain form.  With the scalar gate it is
+// chunk_bwd_dv_local's result
+//     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i = (T do)_j :
+// in the first half of the chunk's step T is formed from the k and q tiles of the chunk (ten 16 x 16 tiles: the six
+// above the diagonal by the copying waves, the four on it by the compute waves), in the second half every compute wave
+// takes T do for its own 16 columns, which lands in accumulators of the layout of dv2, so the intra-chunk dv is never
+// rounded or stored.
 template <int K, bool GK, bool DVL = false>
 __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -700,9 +697,10 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 }
             }
         };
-        // DVL: the dv tile of chunk c from its k, q and do tiles (visible since the last barrier).  Copying wave lw forms
-        // rows 16 lw.. of T[j][i] = scale (k_j . q_i) e^{g_i - g_j} (i >= j), turns them into a left operand through a
-        // strip of LDS of its own (no other wave touches it, so no barrier), and takes T do for those rows.
+        // DVL, chunk c, from its tiles (visible since the last barrier).  Scalar gate: the tiles above the diagonal of
+        // T[j][i] = scale (k_j . q_i) e^{g_i - g_j}, i >= j, dealt over the copying waves, into one 64 x 64 tile;
+        // the compute waves take T do for their own columns behind the next barrier.  Per-channel gate: wave lw takes
+        // rows 16 lw.. of Aqk^T do from the staged score block and writes them where the dv tile would have been loaded.
         auto build_dv = [&](int c) {
             const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
             const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
@@ -720,19 +718,20 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                     default: dv_rows_from_scores<K, 3>(strips, oS, vS); break;
                 }
             } else {
-                switch (wave_id() - 4) {   // the row tile as a constant: every operand read of the wave is issued at once
-                    case 0: dv_rows<K, 0>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                    case 1: dv_rows<K, 1>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                    case 2: dv_rows<K, 2>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
-                    default: dv_rows<K, 3>(kS, qS, oS, vS, gS, strips, len, p.scale); break;
+                switch (wave_id() - 4) {   // the wave's tiles as constants: every operand read of the wave is issued at once
+                    case 0: t_tiles<K, 0>(kS, qS, gS, strips, len, p.scale); break;
+                    case 1: t_tiles<K, 1>(kS, qS, gS, strips, len, p.scale); break;
+                    case 2: t_tiles<K, 2>(kS, qS, gS, strips, len, p.scale); break;
+                    default: t_tiles<K, 3>(kS, qS, gS, strips, len, p.scale); break;
                 }
             }
         };
         // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
         auto step = [&](Tiles &ahead, const Tiles &next, int c) {
-            if constexpr (DVL) build_dv(c);     // into the dv tile, which the compute waves read behind the next barrier
+            if constexpr (DVL) build_dv(c);     // read by the compute waves behind the next barrier
             if (c + 1 < nchunks) read_out(c + 1);
             lds_barrier();   // results of chunk c + 1 are in registers; the compute waves are past the k tile of chunk c
+            // (issued at the top of the step instead, the loads made both DVL forms a third slower)
             fetch(ahead, c - 2);
             if (c > 0) commit(next, c - 1);
             // the stores go last: a commit waits for everything issued before the loads it needs, and by the next
@@ -740,6 +739,10 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             if (c + 1 < nchunks) store_out(c + 1);
             lds_barrier();   // the loads of chunk c - 2 stay in flight
         };
+        if constexpr (DVL && !GK) {   // the tiles of T below the diagonal are never written: they read as zero
+            u32x4 *z = reinterpret_cast<u32x4 *>(smem + L::t_off);
+            for (int idx = tid; idx < kChunk * L::ptl * 2 / 16; idx += kThreads) z[idx] = u32x4{0u, 0u, 0u, 0u};
+        }
         if (nchunks > 0) {
             fetch(t0, nchunks - 1);
             commit(t0, nchunks - 1);
@@ -855,7 +858,16 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         // that needs neither dv nor the place of the k tile moves in front of the barrier; dh then leaves from its 16-bit
         // copy.  (From score blocks the dv tile is two products per wave: the order of the plain form is kept.)
         constexpr bool EARLY = DVL && !GK;
-        if constexpr (EARLY) decay_and_q_term();
+        if constexpr (EARLY) {
+            elem *tS = reinterpret_cast<elem *>(smem + L::t_off);
+            switch (wv) {   // the wave's diagonal tile of T (see t_tiles)
+                case 0: t_tile<K, 0, 0>(kS, qS, gS, tS, len, p.scale); break;
+                case 1: t_tile<K, 1, 1>(kS, qS, gS, tS, len, p.scale); break;
+                case 2: t_tile<K, 2, 2>(kS, qS, gS, tS, len, p.scale); break;
+                default: t_tile<K, 3, 3>(kS, qS, gS, tS, len, p.scale); break;
+            }
+            decay_and_q_term();
+        }
         lds_barrier();   // every wave is past the k tile, which now takes dh on its way to memory
         if (chunk_end) {
             if constexpr (EARLY) {
@@ -870,16 +882,32 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 for (int kt = 0; kt < KT; ++kt) acc_to_tile(kS, ph, 16 * kt, wv * 16, dacc[kt][0]);
             }
         }
+        // DVL with the scalar gate: the intra-chunk dv of the wave's 16 columns, T do, straight into accumulators of the
+        // layout of dv2 (T complete since the barrier; its tiles (1,0) and (3,2) were zeroed once, (2,0), (2,1), (3,0),
+        // (3,1) are skipped with their contraction step)
+        f32x4 dvl[4];
+        if constexpr (EARLY) {
+            const elem *tS = reinterpret_cast<const elem *>(smem + L::t_off);
+            const elemx8 ob0 = frag_tr(oS, pv, wv * 16, 0), ob1 = frag_tr(oS, pv, wv * 16, 32);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f};
+                if (rt < 2) a = mfma16x32(frag_kc(tS, L::ptl, 16 * rt, 0), ob0, a);
+                dvl[rt] = mfma16x32(frag_kc(tS, L::ptl, 16 * rt, 32), ob1, a);
+            }
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const elemx4 old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
+                elemx4 old = {};
+                if constexpr (!EARLY) old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int t = rt * 16 + 4 * lg + e;
                     const float f = GK ? 1.f : __expf(g_last - gS[t]);
-                    dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + (float)old[e] : 0.f;
+                    const float add = EARLY ? dvl[rt][e] : (float)old[e];
+                    dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + add : 0.f;
                 }
             }
 #pragma unroll
