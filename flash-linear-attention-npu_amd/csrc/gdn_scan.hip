@@ -548,29 +548,9 @@ __device__ __forceinline__ void t_tiles(const elem *kS, const elem *qS, const fl
     }
 }
 
-// Rows 16 LW.. of the dv operand when the chunk's score block is an operand (per-channel gate):
-// dv_j = sum_{i >= j} Aqk[i][j] do_i, the dv of chunk_kda_bwd_dav, by one wave.  Aqk is zero above its diagonal and in
-// the rows past the chunk's end.
-template <int K, int LW>
-__device__ __forceinline__ void dv_rows_from_scores(const elem *aS, const elem *oS, elem *vS) {
-    typedef DhuSmem<K> L;
-    constexpr int pv = L::pv, ptl = L::ptl;
-    constexpr int J0 = LW / 2;   // contraction steps (32 tokens i each) that hold a non-zero tile of these rows
-    elemx8 tf[2];
-#pragma unroll
-    for (int j = J0; j < 2; ++j) tf[j] = frag_tr(aS, ptl, 16 * LW, 32 * j);
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = J0; j < 2; ++j) acc = mfma16x32(tf[j], frag_tr(oS, pv, 16 * vt, 32 * j), acc);
-        acc_to_tile(vS, pv, 16 * LW, 16 * vt, acc);
-    }
-}
-
 // DVL (64-token chunks): dv is not an input.  With the per-channel gate it is Aqk^T do per chunk, from the score blocks
-// the forward kept (p.aqk): the copying waves stage the block with the other tiles and write Aqk^T do where the dv tile
-// would have been loaded, and the compute waves run the code of the plain form.  With the scalar gate it is
+// the forward kept (p.aqk): the copying waves stage the block with the other tiles and every compute wave takes
+// Aqk^T do for its own 16 columns, in the order of the plain form otherwise.  With the scalar gate it is
 // chunk_bwd_dv_local's result
 //     dv_j = sum_{i >= j} scale (q_i . k_j) e^{g_i - g_j} do_i = (T do)_j :
 // in the first half of the chunk's step T is formed from the k and q tiles of the chunk (ten 16 x 16 tiles: the six
@@ -699,36 +679,25 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         };
         // DVL, chunk c, from its tiles (visible since the last barrier).  Scalar gate: the tiles above the diagonal of
         // T[j][i] = scale (k_j . q_i) e^{g_i - g_j}, i >= j, dealt over the copying waves, into one 64 x 64 tile;
-        // the compute waves take T do for their own columns behind the next barrier.  Per-channel gate: wave lw takes
-        // rows 16 lw.. of Aqk^T do from the staged score block and writes them where the dv tile would have been loaded.
+        // the compute waves take T do for their own columns behind the next barrier.  (Per-channel gate: nothing to build,
+        // the staged score block is the operand.)
         auto build_dv = [&](int c) {
             const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
             const elem *kS = reinterpret_cast<const elem *>(buf + L::k_off);
             const elem *qS = reinterpret_cast<const elem *>(buf + L::q_off);
-            const elem *oS = reinterpret_cast<const elem *>(buf + L::o_off);
-            elem *vS = const_cast<elem *>(reinterpret_cast<const elem *>(buf + L::v_off));
             const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
             const int len = min(kChunk, eos - (bos + c * kChunk));
-            elem *strips = reinterpret_cast<elem *>(smem + L::t_off);
-            if constexpr (GK) {
-                switch (wave_id() - 4) {
-                    case 0: dv_rows_from_scores<K, 0>(strips, oS, vS); break;
-                    case 1: dv_rows_from_scores<K, 1>(strips, oS, vS); break;
-                    case 2: dv_rows_from_scores<K, 2>(strips, oS, vS); break;
-                    default: dv_rows_from_scores<K, 3>(strips, oS, vS); break;
-                }
-            } else {
-                switch (wave_id() - 4) {   // the wave's tiles as constants: every operand read of the wave is issued at once
-                    case 0: t_tiles<K, 0>(kS, qS, gS, strips, len, p.scale); break;
-                    case 1: t_tiles<K, 1>(kS, qS, gS, strips, len, p.scale); break;
-                    case 2: t_tiles<K, 2>(kS, qS, gS, strips, len, p.scale); break;
-                    default: t_tiles<K, 3>(kS, qS, gS, strips, len, p.scale); break;
-                }
+            elem *tS = reinterpret_cast<elem *>(smem + L::t_off);
+            switch (wave_id() - 4) {   // the wave's tiles as constants: every operand read of the wave is issued at once
+                case 0: t_tiles<K, 0>(kS, qS, gS, tS, len, p.scale); break;
+                case 1: t_tiles<K, 1>(kS, qS, gS, tS, len, p.scale); break;
+                case 2: t_tiles<K, 2>(kS, qS, gS, tS, len, p.scale); break;
+                default: t_tiles<K, 3>(kS, qS, gS, tS, len, p.scale); break;
             }
         };
         // one step: `ahead` takes the tiles of chunk c - 2, `next` holds those of chunk c - 1
         auto step = [&](Tiles &ahead, const Tiles &next, int c) {
-            if constexpr (DVL) build_dv(c);     // read by the compute waves behind the next barrier
+            if constexpr (DVL && !GK) build_dv(c);     // read by the compute waves behind the next barrier
             if (c + 1 < nchunks) read_out(c + 1);
             lds_barrier();   // results of chunk c + 1 are in registers; the compute waves are past the k tile of chunk c
             // (issued at the top of the step instead, the loads made both DVL forms a third slower)
@@ -858,6 +827,20 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         // that needs neither dv nor the place of the k tile moves in front of the barrier; dh then leaves from its 16-bit
         // copy.  (From score blocks the dv tile is two products per wave: the order of the plain form is kept.)
         constexpr bool EARLY = DVL && !GK;
+        f32x4 dvl[4];   // DVL: the dv operand of the wave's 16 columns, in the layout of dv2
+        if constexpr (DVL && GK) {
+            // per-channel gate: dv_j = sum_{i >= j} Aqk[i][j] do_i (the dv of chunk_kda_bwd_dav) from the score block the
+            // copying waves staged with the chunk's tiles; Aqk is zero above its diagonal and past the chunk's end.  Taken
+            // in this half of the step: the block's place is written again behind the barrier.
+            const elem *aS = reinterpret_cast<const elem *>(smem + L::t_off);
+            const elemx8 ob0 = frag_tr(oS, pv, wv * 16, 0), ob1 = frag_tr(oS, pv, wv * 16, 32);
+#pragma unroll
+            for (int rt = 0; rt < 4; ++rt) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f};
+                if (rt < 2) a = mfma16x32(frag_tr(aS, L::ptl, 16 * rt, 0), ob0, a);
+                dvl[rt] = mfma16x32(frag_tr(aS, L::ptl, 16 * rt, 32), ob1, a);
+            }
+        }
         if constexpr (EARLY) {
             elem *tS = reinterpret_cast<elem *>(smem + L::t_off);
             switch (wv) {   // the wave's diagonal tile of T (see t_tiles)
@@ -885,7 +868,6 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
         // DVL with the scalar gate: the intra-chunk dv of the wave's 16 columns, T do, straight into accumulators of the
         // layout of dv2 (T complete since the barrier; its tiles (1,0) and (3,2) were zeroed once, (2,0), (2,1), (3,0),
         // (3,1) are skipped with their contraction step)
-        f32x4 dvl[4];
         if constexpr (EARLY) {
             const elem *tS = reinterpret_cast<const elem *>(smem + L::t_off);
             const elemx8 ob0 = frag_tr(oS, pv, wv * 16, 0), ob1 = frag_tr(oS, pv, wv * 16, 32);
@@ -901,12 +883,12 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 elemx4 old = {};
-                if constexpr (!EARLY) old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
+                if constexpr (!DVL) old = frag_tr4(vS, pv, (wv * CT + ct) * 16, rt * 16);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int t = rt * 16 + 4 * lg + e;
                     const float f = GK ? 1.f : __expf(g_last - gS[t]);
-                    const float add = EARLY ? dvl[rt][e] : (float)old[e];
+                    const float add = DVL ? dvl[rt][e] : (float)old[e];
                     dv2[rt][ct][e] = t < len ? dv2[rt][ct][e] * f + add : 0.f;
                 }
             }

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import gdn, kda
-from util import assert_close, TOL_BF16, TOL_STATE
+from util import assert_close, err_stats, TOL_BF16, TOL_STATE
 
 pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
@@ -154,8 +154,8 @@ def test_bwd_dhu(dev, case):
                          ids=lambda c: f"T{c[1]}-K{c[4]}-V{c[5]}")
 def test_kda_bwd_dhu_forms_dv_from_the_score_blocks(dev, case):
     """chunk_kda_bwd_dhu (no counterpart in the reference): the per-channel-gate scan with dv = Aqk^T d_o formed
-    inside.  Against the oracle's two operators (chunk_kda_bwd_dav's dv, rounded as it is exchanged, then the scan) and
-    against the two-operator route on the device, whose dv tile holds the same 16-bit values."""
+    inside.  Against the oracle's two operators (chunk_kda_bwd_dav's dv, then the scan) and against the two-operator
+    route on the device."""
     from fla_hip import ops
     from fla_hip.ops import _hip_ctypes as raw
     B, T, Hk, Hv, K, V, cu, _, with_dht = case
@@ -179,7 +179,8 @@ def test_kda_bwd_dhu_forms_dv_from_the_score_blocks(dev, case):
     dh, dh0, dv2 = raw.chunk_kda_bwd_dhu(qd, kd, wd, od, ad, scale, 64, gK=gd, h0=h0, dht=dht_d, cu_seqlens=cu)
     assert dh.dtype == BF and dv2.dtype == BF and dh0.dtype == torch.float32 and dv2.shape == d_o.shape
     _, dv_ref = kda.chunk_kda_bwd_dav(d_o, d_o, Aqk, scale, cu_seqlens=cu)
-    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(qg, kg, w, d_o, dv_ref.to(BF), scale, 64, dht=dht, cu_seqlens=cu,
+    # dv enters the oracle's scan unrounded, as it stays in the kernel's accumulators
+    dh_ref, dh0_ref, dv2_ref = kda.chunk_gated_delta_rule_bwd_dhu(qg, kg, w, d_o, dv_ref, scale, 64, dht=dht, cu_seqlens=cu,
                                                                   gK=gcum)
     assert_close(dv2, dv2_ref, TOL_BF16, "dv2")
     assert_close(dh, dh_ref, TOL_BF16, "dh")
@@ -187,9 +188,11 @@ def test_kda_bwd_dhu_forms_dv_from_the_score_blocks(dev, case):
     _, dv_two = raw.chunk_kda_bwd_dav(od, od, ad, scale, cu_seqlens=cu)
     two = ops.chunk_gated_delta_rule_bwd_dhu(qd, kd, wd, od, dv_two, scale, 64, gK=gd, use_exp2=True, h0=h0, dht=dht_d,
                                              cu_seqlens=cu, dh0_per_sequence=True)
-    # the same operands in another order of accumulation: far inside the oracle's bound
+    # the two-operator route rounds dv to 16 bits on its way through memory, the scan takes it unrounded: a couple of
+    # steps of the 16-bit results apart, inside the oracle's bound
     for name, a_, b_ in zip(("dh", "dh0", "dv2"), (dh, dh0, dv2), two):
-        assert_close(a_, b_, 2.0 ** -7 if a_.dtype != torch.float32 else 1e-4, name + " against the two-operator route")
+        st = err_stats(a_, b_)
+        assert st["rel_max"] <= 1e-2, f"{name} against the two-operator route: {st}"
     assert raw.chunk_kda_bwd_dhu(qd, kd, wd, od, ad, scale, 64, gK=gd, cu_seqlens=cu)[1] is None
     with pytest.raises(RuntimeError, match="Aqk"):
         raw.chunk_kda_bwd_dhu(qd, kd, wd, od, None, scale, 64, gK=gd, cu_seqlens=cu)
