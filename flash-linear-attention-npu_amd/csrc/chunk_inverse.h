@@ -69,6 +69,23 @@ __device__ __forceinline__ void kkt_score_rows(const elem *kS, int pitch, int K,
         }
 }
 
+// One 16 x 16 tile of the same scores, rows 16 I.., columns 16 J.. (J <= I), written to its place in the fp32 block sS
+// (pitch 68), so that the ten tiles can be dealt over the waves by count instead of by row block.
+template <int I, int J>
+__device__ __forceinline__ void kkt_score_tile(const elem *kS, int pitch, int K, const float *gS, const float *bS, int len, float *sS) {
+    const int t = 16 * I + acc_col();
+    const float gt = gS[t], bt = bS[t];
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int kk = 0; kk < K; kk += 32) acc = mfma16x32(frag_kc(kS, pitch, 16 * J, kk), frag_kc(kS, pitch, 16 * I, kk), acc);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int s = 16 * J + acc_row(e);
+        const float d = fminf(fmaxf(gt - gS[s], -50.f), 50.f);
+        acc[e] = (s < t && t < len) ? (float)(elem)(bt * __expf(d) * acc[e]) : 0.f;
+    }
+    *reinterpret_cast<f32x4 *>(sS + t * 68 + 16 * J + 4 * (lane_id() >> 4)) = acc;
+}
+
 // (I + A)^-1 of the strictly lower 64 x 64 matrix in aS (fp32, pitch 68), written to oS (pitch 72) in the element
 // type; called by all four waves of a 256-thread workgroup after a barrier that completes aS, ends with one.
 __device__ __forceinline__ void invert64(float *aS, elem *oS) {

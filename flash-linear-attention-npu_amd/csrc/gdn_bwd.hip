@@ -703,15 +703,30 @@ __global__ void __launch_bounds__(kThreads, GVA ? 1 : 2) wy_bwd_full_kernel(cons
                 static_assert(DA && pa == 72, "the fp32 score block lies over the two dA tiles; the inverse is written at pitch 72");
                 static_assert(kChunk * 68 * 4 <= 2 * kChunk * pa * 2, "the fp32 score block must fit the two dA tiles");
                 float *sS = reinterpret_cast<float *>(dS);
-                f32x4 sc[4];
+                // the ten tiles on and below the diagonal dealt 3, 3, 2, 2 (by row block it would be 1, 2, 3, 4)
                 switch (w) {
-                    case 0: kkt_score_rows<0>(kS, pk, K, gS, bS, len, sc); break;
-                    case 1: kkt_score_rows<1>(kS, pk, K, gS, bS, len, sc); break;
-                    case 2: kkt_score_rows<2>(kS, pk, K, gS, bS, len, sc); break;
-                    default: kkt_score_rows<3>(kS, pk, K, gS, bS, len, sc); break;
+                    case 0:
+                        kkt_score_tile<0, 0>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<3, 0>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<3, 1>(kS, pk, K, gS, bS, len, sS);
+                        break;
+                    case 1:
+                        kkt_score_tile<1, 0>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<1, 1>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<2, 0>(kS, pk, K, gS, bS, len, sS);
+                        break;
+                    case 2:
+                        kkt_score_tile<2, 1>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<2, 2>(kS, pk, K, gS, bS, len, sS);
+                        break;
+                    default:
+                        kkt_score_tile<3, 2>(kS, pk, K, gS, bS, len, sS);
+                        kkt_score_tile<3, 3>(kS, pk, K, gS, bS, len, sS);
+                        break;
                 }
 #pragma unroll
-                for (int J = 0; J < 4; ++J) *reinterpret_cast<f32x4 *>(sS + (16 * w + li) * 68 + 16 * J + 4 * lg) = sc[J];
+                for (int J = 1; J < 4; ++J)   // above the diagonal: zero
+                    if (J > w) *reinterpret_cast<f32x4 *>(sS + (16 * w + li) * 68 + 16 * J + 4 * lg) = zero4();
                 __syncthreads();
                 invert64(sS, aS);
                 if (tid < kChunk && tid >= len) aS[tid * pa + tid] = (elem)0.f;   // rows past the end hold nothing, as a staged A would
