@@ -46,7 +46,11 @@ struct KdaIntraParams {
     float scale;
     float *gk;                // [B,Hv,T,K] or null
     elem *aqk, *akk;          // [B,Hv,T,C], C = tokens per chunk
-    elem *w, *u, *qg, *kg;    // [B,Hv,T,K] / [B,Hv,T,V]
+    elem *w, *qg;             // [B,Hv,T,K]
+    // u [B,Hv,T,V] and kg [B,Hv,T,K] reach the scan as fp16 (u16, kg16: see `fine`); u and kg are the caller's
+    // tensors of the element type, written as well when they are not null (never set when elem is fp16 itself)
+    fine *u16, *kg16;
+    elem *u, *kg;
     float *dec;               // [B,NT,Hv,K]: 2^{g_last} of every chunk
     // 128-token chunks: a workgroup still owns 64 tokens (one half of a chunk); the operands of the block that
     // couples the halves go to x1 (first half: k 2^{G1 - g}; second half: q 2^{g - G1}) and x2 (second half:
@@ -287,6 +291,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         const elemx8 k8 = *reinterpret_cast<const elemx8 *>(kS + r * pk + c8);
         const float br = bS[r];
         elemx8 qg8, kg8, kb8;
+        u32x4 kgf;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + kChunk * pg + c8 + 4 * h);
@@ -299,6 +304,8 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
                 c[e] = kk * br * eg;
             }
             const elemx4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
+            kgf[2 * h] = cvt2_fine(b[0], b[1]);
+            kgf[2 * h + 1] = cvt2_fine(b[2], b[3]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 qg8[4 * h + e] = a4[e];
@@ -308,7 +315,10 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         }
         if (r < len) {
             *reinterpret_cast<elemx8 *>(p.qg + (row_base + r) * K + c8) = qg8;
-            *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
+            *reinterpret_cast<u32x4 *>(p.kg16 + (row_base + r) * K + c8) = kgf;
+            if constexpr (!kFineIsElem) {
+                if (p.kg != nullptr) *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
+            }
         }
         if constexpr (C128) {   // operands of the block that couples the two halves, both factors <= 1
             f32x4 x1lo, x1hi, x2lo, x2hi;
@@ -335,20 +345,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         __syncthreads();   // last read of the gate tile
         TileCopy<kIntraThreads, kChunk, V> tv;
         tv.fetch(vg, p.v.st, len, threadIdx.x);
-#pragma unroll
-        for (int m = 0; m < TileCopy<kIntraThreads, kChunk, V>::N; ++m) {   // v * beta
-            const int idx = m * kIntraThreads + threadIdx.x;
-            const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
-            const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
-            const float bb = bS[r];
-            f32x4 lo, hi;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                lo[e] = (float)v8[e] * bb;
-                hi[e] = (float)v8[4 + e] * bb;
-            }
-            *reinterpret_cast<elemx8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
-        }
+        tv.commit(vS, pv, len, threadIdx.x);
         if constexpr (ROLE == 1) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) acc_to_tile(aqS, pb, 16 * R2, 16 * c, aqv[c]);
@@ -357,13 +354,26 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
     __syncthreads();
 
     // ---- w = Akk (k beta 2^g) (role 0), u = Akk (v beta) (role 1): row tile W -----------------------------------
+    // u is formed as (Akk diag(beta)) v from the v tile as it came from memory: the unit diagonal of Akk carries
+    // beta_i v_i, the leading term of u_i, and its only rounding (beta_i to the element type in the left operand) is
+    // made good below, so that u is accurate to fp32 products of the 16-bit Akk rather than to a rounded v beta.
     constexpr int NCT = ROLE == 0 ? K / 16 : V / 16;
     f32x4 oacc[NCT];
 #pragma unroll
     for (int ct = 0; ct < NCT; ++ct) oacc[ct] = zero4();
 #pragma unroll
     for (int j = 0; j < (W < 2 ? 1 : 2); ++j) {   // Akk is lower triangular
-        const elemx8 a = frag_kc(akS, pb, 16 * W, 32 * j);
+        elemx8 a = frag_kc(akS, pb, 16 * W, 32 * j);
+        if constexpr (ROLE == 1) {
+            const f32x4 b0 = lds4(bS + 32 * j + 4 * lg), b1 = lds4(bS + 32 * j + 16 + 4 * lg);
+            f32x4 lo, hi;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                lo[e] = (float)a[e] * b0[e];
+                hi[e] = (float)a[4 + e] * b1[e];
+            }
+            a = frag_from_acc(lo, hi);
+        }
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
             oacc[ct] = mfma16x32(a, ROLE == 0 ? frag_tr(qS, pq, 16 * ct, 32 * j) : frag_tr(vS, pv, 16 * ct, 32 * j), oacc[ct]);
@@ -372,19 +382,31 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             }
         }
     }
+    if constexpr (ROLE == 1) {   // u_i += (beta_i - rounded beta_i) v_i
+        const f32x4 bw = lds4(bS + 16 * W + 4 * lg);
+        f32x4 db;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) db[e] = bw[e] - (float)(elem)bw[e];
+#pragma unroll
+        for (int ct = 0; ct < NCT; ++ct) {
+            const elemx4 vv = frag_tr4(vS, pv, 16 * ct, 16 * W);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) oacc[ct][e] += db[e] * (float)vv[e];
+        }
+    }
     if constexpr (S::FREE_STAGE) {   // nobody reads the two dead tiles any more
         elem *wT = const_cast<elem *>(khS), *uT = reinterpret_cast<elem *>(gS);
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
             if constexpr (ROLE == 0) acc_to_tile(wT, pk, 16 * W, 16 * ct, oacc[ct]);
-            else acc_to_tile(uT, pv, 16 * W, 16 * ct, oacc[ct]);
+            else acc_to_tile_fine(uT, pv, 16 * W, 16 * ct, oacc[ct]);
         }
     } else {
         __syncthreads();   // every wave has consumed the operand tiles; they become the output staging
 #pragma unroll
         for (int ct = 0; ct < NCT; ++ct) {
             if constexpr (ROLE == 0) acc_to_tile(qS, pq, 16 * W, 16 * ct, oacc[ct]);
-            else acc_to_tile(vS, pv, 16 * W, 16 * ct, oacc[ct]);
+            else acc_to_tile_fine(vS, pv, 16 * W, 16 * ct, oacc[ct]);
         }
     }
     __syncthreads();
@@ -466,17 +488,10 @@ __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intr
     }
     {   // all loads of the chunk are issued before the first LDS write waits for one of them
         TileCopy<kIntraThreads, kChunk, K> tq, tk;
-        constexpr int NVP = S::WIDE ? 0 : TileCopy<kIntraThreads, kChunk, V>::N;   // WIDE: v is staged later
         TileCopy<kIntraThreads, kChunk, V> tv;
         tq.fetch(qg, p.q.st, len, tid);
         tk.fetch(kg, p.k.st, len, tid);
         if constexpr (!S::WIDE) tv.fetch(vg, p.v.st, len, tid);
-        float br[NVP + 1];
-#pragma unroll
-        for (int m = 0; m < NVP; ++m) {
-            const int r = (m * kIntraThreads + tid) / (V / 8);
-            br[m] = load_scalar(p.beta, b, hv, start + min(r, len - 1));
-        }
         {   // segment sums of the gates (they were requested first) while the tiles are still on their way
             float acc = 0.f;
 #pragma unroll
@@ -500,20 +515,7 @@ __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intr
         }
         tq.commit(qS, pq, len, tid);
         tk.commit(kS, pk, len, tid);
-#pragma unroll
-        for (int m = 0; m < NVP; ++m) {   // v * beta
-            const int idx = m * kIntraThreads + tid;
-            const int r = idx / (V / 8), c8 = (idx % (V / 8)) * 8;
-            const elemx8 v8 = __builtin_bit_cast(elemx8, tv.r[m]);
-            const float bb = r < len ? br[m] : 0.f;
-            f32x4 lo, hi;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                lo[e] = (float)v8[e] * bb;
-                hi[e] = (float)v8[4 + e] * bb;
-            }
-            *reinterpret_cast<elemx8 *>(vS + r * pv + c8) = frag_from_acc(lo, hi);
-        }
+        if constexpr (!S::WIDE) tv.commit(vS, pv, len, tid);
     }
     if (tid < kChunk) bS[tid] = tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f;
 
@@ -580,12 +582,13 @@ __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intr
         default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
     }
 
-    if constexpr (S::FREE_STAGE) {
-        store_tile<kIntraThreads>(p.w + row_base * K, K, khS, pk, K, len);
-        store_tile<kIntraThreads>(p.u + row_base * V, V, reinterpret_cast<const elem *>(gS), pv, V, len);
-    } else {
-        store_tile<kIntraThreads>(p.w + row_base * K, K, qS, pq, K, len);
-        store_tile<kIntraThreads>(p.u + row_base * V, V, vS, pv, V, len);
+    {
+        const elem *wT = S::FREE_STAGE ? khS : qS, *uT = S::FREE_STAGE ? reinterpret_cast<const elem *>(gS) : vS;
+        store_tile<kIntraThreads>(p.w + row_base * K, K, wT, S::FREE_STAGE ? pk : pq, K, len);
+        store_tile<kIntraThreads>(reinterpret_cast<elem *>(p.u16) + row_base * V, V, uT, pv, V, len);
+        if constexpr (!kFineIsElem) {
+            if (p.u != nullptr) store_tile_fine_as_elem<kIntraThreads>(p.u + row_base * V, V, uT, pv, V, len);
+        }
     }
     const int C = p.geom.C;
     store_tile<kIntraThreads>(p.aqk + row_base * C + kChunk * half, C, aqS, pb, kChunk, len);
@@ -613,7 +616,9 @@ __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intr
 struct KdaCrossParams {
     ChunkGeom geom;
     const elem *x1, *x2;
-    elem *w, *u, *aqk, *akk;
+    elem *w, *aqk, *akk;
+    fine *u16;   // u as the scan reads it
+    elem *u;     // the caller's u of the element type, or null
     float scale;
 };
 
@@ -669,7 +674,7 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
         tc.fetch(p.x1 + row1 * K, K, kChunk, tid);
         if constexpr (!L::WIDE) {
             tw.fetch(p.w + row1 * K, K, kChunk, tid);
-            tu.fetch(p.u + row1 * V, V, kChunk, tid);
+            tu.fetch(reinterpret_cast<const elem *>(p.u16) + row1 * V, V, kChunk, tid);
         }
         t1.fetch(p.akk + row1 * C, C, kChunk, tid);
         t2.fetch(p.akk + row2 * C + kChunk, C, len2, tid);
@@ -678,6 +683,7 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
         tc.commit(kcS, pk, kChunk, tid);
         if constexpr (!L::WIDE) {
             tw.commit(wS, pr, kChunk, tid);
+            tu.to_elem();
             tu.commit(uS, pv, kChunk, tid);
         }
         t1.commit(a11S, pb, kChunk, tid);
@@ -715,8 +721,9 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
         TileCopy<kThreads, kChunk, K> tw;
         TileCopy<kThreads, kChunk, V> tu;
         tw.fetch(p.w + row1 * K, K, kChunk, tid);
-        tu.fetch(p.u + row1 * V, V, kChunk, tid);
+        tu.fetch(reinterpret_cast<const elem *>(p.u16) + row1 * V, V, kChunk, tid);
         tw.commit(wS, pr, kChunk, tid);
+        tu.to_elem();
         tu.commit(uS, pv, kChunk, tid);
         __syncthreads();
     }
@@ -761,8 +768,19 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
     };
 #pragma unroll
     for (int ct = 0; ct < K / 16; ++ct) minus(p.w + orow * K + 16 * ct + 4 * lg, product(wS, pr, ct));
+    auto minus_u = [&](int64_t at, f32x4 z) {   // u -= z, in the scan's copy and in the caller's
+        if (!live) return;
+        const finex4 old = *reinterpret_cast<const finex4 *>(p.u16 + at);
+        f32x4 v;
 #pragma unroll
-    for (int ct = 0; ct < V / 16; ++ct) minus(p.u + orow * V + 16 * ct + 4 * lg, product(uS, pv, ct));
+        for (int e = 0; e < 4; ++e) v[e] = (float)old[e] - z[e];
+        *reinterpret_cast<finex4 *>(p.u16 + at) = cvt4_fine(v);
+        if constexpr (!kFineIsElem) {
+            if (p.u != nullptr) *reinterpret_cast<elemx4 *>(p.u + at) = cvt4(v);
+        }
+    };
+#pragma unroll
+    for (int ct = 0; ct < V / 16; ++ct) minus_u(orow * V + 16 * ct + 4 * lg, product(uS, pv, ct));
 #pragma unroll
     for (int ct = 0; ct < 4; ++ct) {
         const f32x4 z = product(a11S, pb, ct);
@@ -775,7 +793,8 @@ __global__ void __launch_bounds__(kThreads) kda_cross_kernel(const KdaCrossParam
 // =============================================================================================
 struct KdaScanParams {
     ChunkGeom geom;
-    const elem *w, *u, *qg, *kg, *aqk;   // head-major [B,Hv,T,*]
+    const elem *w, *qg, *aqk;            // head-major [B,Hv,T,*]
+    const fine *u, *kg;                  // fp16 whatever the element type (see `fine`)
     const float *dec;                    // [B,NT,Hv,K]
     View4 o;                             // attention output in the caller's layout
     elem *v_new;                         // [B,Hv,T,V] or null
@@ -857,8 +876,8 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             const int64_t row = head_row + start;
             t.tw.fetch(p.w + row * K, K, len, tid);
             t.tq.fetch(p.qg + row * K, K, len, tid);
-            t.tk.fetch(p.kg + row * K, K, len, tid);
-            t.tu.fetch(p.u + row * V + slab * VS, V, len, tid);
+            t.tk.fetch(reinterpret_cast<const elem *>(p.kg) + row * K, K, len, tid);
+            t.tu.fetch(reinterpret_cast<const elem *>(p.u) + row * V + slab * VS, V, len, tid);
             t.ta.fetch(p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, len, tid);   // diagonal block
             t.dec = p.dec[(((int64_t)b * p.geom.NT + chunk0 + c / SUB) * p.geom.Hv + hv) * K + min(tid, K - 1)];
         };
@@ -1046,7 +1065,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
         }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
-            const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
+            const finex4 uu = as_fine(frag_tr4(uS, pu, wv * 16, rt * 16));
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 vn[rt][e] = (float)uu[e] - vn[rt][e];
@@ -1057,10 +1076,14 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
         }
-        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same bf16 v_new operand serves both)
+        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (v_new as fp16 against the fp16 kg)
         elemx8 vB[2];
+        finex8 vF[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+        for (int j = 0; j < 2; ++j) {
+            vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+            vF[j] = fine_from_acc(vn[2 * j], vn[2 * j + 1]);
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
@@ -1088,13 +1111,13 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
             for (int kt = 0; kt < KT; ++kt)
                 if (first) hacc[kt] *= dk[kt];
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(kf[kt], vB[0], hacc[kt]);
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(as_fine(kf[kt]), vF[0], hacc[kt]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) kf[kt] = frag_tr(kS, pt, kt * 16, 32);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(kf[kt], vB[1], hacc[kt]);
+            for (int kt = 0; kt < KT; ++kt) hacc[kt] = mfma16x32(as_fine(kf[kt]), vF[1], hacc[kt]);
         }
         char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
@@ -1179,8 +1202,8 @@ __global__ void __launch_bounds__(kThreads) kda_scan_wide_kernel(const KdaScanPa
 
         load_tile<kThreads>(wS, pw, p.w + row * K, K, kChunk, K, len);
         load_tile<kThreads>(qS, pw, p.qg + row * K, K, kChunk, K, len);
-        load_tile<kThreads>(kS, pt, p.kg + row * K, K, kChunk, K, len);
-        load_tile<kThreads>(uS, pu, p.u + row * V + slab * VS, V, kChunk, VS, len);
+        load_tile<kThreads>(kS, pt, reinterpret_cast<const elem *>(p.kg) + row * K, K, kChunk, K, len);
+        load_tile<kThreads>(uS, pu, reinterpret_cast<const elem *>(p.u) + row * V + slab * VS, V, kChunk, VS, len);
         load_tile<kThreads>(aS, pb, p.aqk + row * (kChunk * SUB) + kChunk * (c % SUB), kChunk * SUB, kChunk, kChunk, len);
         for (int i = tid; i < K; i += kThreads) dS[i] = p.dec[(((int64_t)b * p.geom.NT + chunk) * p.geom.Hv + hv) * K + i];
         __syncthreads();   // tiles of this step in place
@@ -1217,7 +1240,7 @@ __global__ void __launch_bounds__(kThreads) kda_scan_wide_kernel(const KdaScanPa
             for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(frag_kc(qS, pw, rt * 16, 32 * j), hB[j], oacc[rt]);
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt) {
-            const elemx4 uu = frag_tr4(uS, pu, wv * 16, rt * 16);
+            const finex4 uu = as_fine(frag_tr4(uS, pu, wv * 16, rt * 16));
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 vn[rt][e] = (float)uu[e] - vn[rt][e];
@@ -1228,10 +1251,14 @@ __global__ void __launch_bounds__(kThreads) kda_scan_wide_kernel(const KdaScanPa
 #pragma unroll
             for (int rt = 0; rt < 4; ++rt) acc_to_tile(uS, pu, rt * 16, wv * 16, vn[rt]);
         }
-        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (the same 16-bit v_new operand serves both)
+        // o += Aqk v_new ;  S <- 2^{g_last} S + kg^T v_new   (v_new as fp16 against the fp16 kg)
         elemx8 vB[2];
+        finex8 vF[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+        for (int j = 0; j < 2; ++j) {
+            vB[j] = frag_from_acc(vn[2 * j], vn[2 * j + 1]);
+            vF[j] = fine_from_acc(vn[2 * j], vn[2 * j + 1]);
+        }
 #pragma unroll
         for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
@@ -1256,8 +1283,8 @@ __global__ void __launch_bounds__(kThreads) kda_scan_wide_kernel(const KdaScanPa
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt) {
             if (first) hacc[kt] *= lds4(dS + 16 * kt + 4 * lg);
-            hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 0), vB[0], hacc[kt]);
-            hacc[kt] = mfma16x32(frag_tr(kS, pt, kt * 16, 32), vB[1], hacc[kt]);
+            hacc[kt] = mfma16x32(as_fine(frag_tr(kS, pt, kt * 16, 0)), vF[0], hacc[kt]);
+            hacc[kt] = mfma16x32(as_fine(frag_tr(kS, pt, kt * 16, 32)), vF[1], hacc[kt]);
         }
         char *ob = og + (int64_t)start * p.o.st * 2;
 #pragma unroll
@@ -1347,7 +1374,7 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
     const int rc = p.c128 ? launch_intra_kernel<K, V, true>(p, stream) : launch_intra_kernel<K, V, false>(p, stream);
     if (rc) return rc;
     if (p.c128) {
-        KdaCrossParams cp{p.geom, p.x1, p.x2, p.w, p.u, p.aqk, p.akk, p.scale};
+        KdaCrossParams cp{p.geom, p.x1, p.x2, p.w, p.aqk, p.akk, p.u16, p.u, p.scale};
         const size_t csmem = CrossSmem<K, V>::bytes;
         FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_cross_kernel<K, V>),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)csmem));
@@ -1498,6 +1525,9 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     const size_t dec_off = off;
     off += align256((size_t)B * NT * Hv * K * 4);
     size_t w_off = 0, u_off = 0, qg_off = 0, kg_off = 0, x1_off = 0, x2_off = 0;
+    // u and kg go to the scan as fp16 (`fine`): with fp16 elements the caller's tensors serve, otherwise the workspace
+    // holds the fp16 copies whether or not the caller also takes u and kg
+    const bool fine_u_ws = !kFineIsElem || !present(u), fine_kg_ws = !kFineIsElem || !present(kg);
     if (C == 128) {
         x1_off = off;
         off += align256(rows * K * 2);
@@ -1505,9 +1535,9 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
         off += align256(rows * K * 2);
     }
     if (!present(w)) { w_off = off; off += align256(rows * K * 2); }
-    if (!present(u)) { u_off = off; off += align256(rows * V * 2); }
+    if (fine_u_ws) { u_off = off; off += align256(rows * V * 2); }
     if (!present(qg)) { qg_off = off; off += align256(rows * K * 2); }
-    if (!present(kg)) { kg_off = off; off += align256(rows * K * 2); }
+    if (fine_kg_ws) { kg_off = off; off += align256(rows * K * 2); }
     if (query) {
         *query = off;
         return FLA_OK;
@@ -1534,9 +1564,11 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     ip.aqk = static_cast<elem *>(aqk->data);
     ip.akk = static_cast<elem *>(akk->data);
     ip.w = present(w) ? static_cast<elem *>(w->data) : reinterpret_cast<elem *>(wsb + w_off);
-    ip.u = present(u) ? static_cast<elem *>(u->data) : reinterpret_cast<elem *>(wsb + u_off);
+    ip.u16 = fine_u_ws ? reinterpret_cast<fine *>(wsb + u_off) : static_cast<fine *>(u->data);
+    ip.u = !kFineIsElem && present(u) ? static_cast<elem *>(u->data) : nullptr;
     ip.qg = present(qg) ? static_cast<elem *>(qg->data) : reinterpret_cast<elem *>(wsb + qg_off);
-    ip.kg = present(kg) ? static_cast<elem *>(kg->data) : reinterpret_cast<elem *>(wsb + kg_off);
+    ip.kg16 = fine_kg_ws ? reinterpret_cast<fine *>(wsb + kg_off) : static_cast<fine *>(kg->data);
+    ip.kg = !kFineIsElem && present(kg) ? static_cast<elem *>(kg->data) : nullptr;
     ip.dec = reinterpret_cast<float *>(wsb + dec_off);
     ip.c128 = C == 128;
     ip.x1 = reinterpret_cast<elem *>(wsb + x1_off);
@@ -1550,9 +1582,9 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
 
     sp.geom = geom;
     sp.w = ip.w;
-    sp.u = ip.u;
+    sp.u = ip.u16;
     sp.qg = ip.qg;
-    sp.kg = ip.kg;
+    sp.kg = ip.kg16;
     sp.aqk = ip.aqk;
     sp.dec = ip.dec;
     sp.v_new = present(v_new) ? static_cast<elem *>(v_new->data) : nullptr;
@@ -1669,7 +1701,9 @@ extern "C" int fla_chunk_kda_fwd_noalloc(
     if (need > (uint64_t)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES)
         return fla::fail(FLA_ERR_WORKSPACE,
                          "%s: this call needs %llu bytes of scratch, the fixed array holds %llu; pass w, u, qg and kg "
-                         "(1 KiB per token and head at K=V=128 otherwise) or use fla_chunk_kda_fwd with a workspace.",
+                         "(1 KiB per token and head at K=V=128 otherwise; the fp16 copies of u and kg that the state "
+                         "scan reads stay in the scratch with bf16 elements, 512 B) or use fla_chunk_kda_fwd with a "
+                         "workspace.",
                          op, (unsigned long long)need, (unsigned long long)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES);
     void *ptr = nullptr;
     if ((rc = fla::scratch_address(&ptr))) return rc;

@@ -69,6 +69,49 @@ __device__ __forceinline__ elemx8 frag_from_acc(f32x4 lo, f32x4 hi) { return cat
 __device__ __forceinline__ int acc_row(int e) { return 4 * (lane_id() >> 4) + e; }
 __device__ __forceinline__ int acc_col() { return lane_id() & 15; }
 
+// ---- the hand-off type of the KDA forward ---------------------------------------------------------
+// u = Akk (v beta) and kg = k 2^{g_last - g} pass from the chunk-parallel kernel to the state scan, and v_new enters
+// the state update, as fp16 whatever the element type: with 8 significand bits (bf16) each of the three roundings
+// alone moves the fp32 final state by about 2e-3 of its scale, with 11 bits all three together stay below 4e-4.
+// Values beyond the fp16 range saturate instead of turning into infinities.
+typedef f16 fine;
+typedef f16 finex2 __attribute__((ext_vector_type(2)));
+typedef f16x4 finex4;
+typedef f16x8 finex8;
+#ifdef FLA_ELEM_F16
+constexpr bool kFineIsElem = true;
+#else
+constexpr bool kFineIsElem = false;
+#endif
+__device__ __forceinline__ unsigned cvt2_fine(float a, float b) {
+    const f32x2 v = {__builtin_amdgcn_fmed3f(a, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(b, -65504.f, 65504.f)};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, finex2));
+}
+__device__ __forceinline__ finex4 cvt4_fine(f32x4 v) {
+    u32x2 t;
+    t[0] = cvt2_fine(v[0], v[1]);
+    t[1] = cvt2_fine(v[2], v[3]);
+    return __builtin_bit_cast(finex4, t);
+}
+__device__ __forceinline__ finex8 fine_from_acc(f32x4 lo, f32x4 hi) {
+    return __builtin_shufflevector(cvt4_fine(lo), cvt4_fine(hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// tiles of `fine` values live in LDS behind elem pointers (both are 16 bits wide); these reinterpret what was read
+__device__ __forceinline__ finex8 as_fine(elemx8 x) { return __builtin_bit_cast(finex8, x); }
+__device__ __forceinline__ finex4 as_fine(elemx4 x) { return __builtin_bit_cast(finex4, x); }
+__device__ __forceinline__ elemx8 fine_to_elem(finex8 x) {
+    if constexpr (kFineIsElem) {
+        return __builtin_bit_cast(elemx8, x);
+    } else {
+        f32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo[e] = (float)x[e];
+            hi[e] = (float)x[4 + e];
+        }
+        return frag_from_acc(lo, hi);
+    }
+}
 // ---- cooperative global <-> LDS tile copies (all threads of the block) -----------
 // Copies rows [0, valid) x cols [0, ncols) of a row-major global matrix (row stride
 // `gstride` elements, 16-byte aligned rows) into `tile`; rows [valid, nrows) are zeroed.
@@ -93,6 +136,11 @@ template <int THREADS, int NROWS, int NCOLS> struct TileCopy {
             const unsigned off = (unsigned)((row < valid ? row : last) * (int)gstride + c);
             r[m] = *reinterpret_cast<const u32x4 *>(gsrc + off);
         }
+    }
+    // the pieces were fetched from a tensor of `fine` values and are to be committed as elements
+    __device__ __forceinline__ void to_elem() {
+#pragma unroll
+        for (int m = 0; m < N; ++m) r[m] = __builtin_bit_cast(u32x4, fine_to_elem(__builtin_bit_cast(finex8, r[m])));
     }
     __device__ __forceinline__ void commit(elem *tile, int pitch, int valid, int tid) const {
 #pragma unroll
@@ -175,6 +223,22 @@ __device__ __forceinline__ void packed_to_global(char *base, int64_t stride, int
 __device__ __forceinline__ void acc_to_global(char *base, int64_t stride, int r0, int len, f32x4 acc) {
     packed_to_global(base, stride, r0, len, __builtin_bit_cast(unsigned, cvt2(acc[0], acc[1])),
                      __builtin_bit_cast(unsigned, cvt2(acc[2], acc[3])));
+}
+
+// ---- tiles of `fine` values ------------------------------------------------------------------------
+__device__ __forceinline__ void acc_to_tile_fine(elem *tile, int pitch, int r0, int c0, f32x4 acc) {
+    packed_to_tile(tile, pitch, r0, c0, cvt2_fine(acc[0], acc[1]), cvt2_fine(acc[2], acc[3]));
+}
+// store_tile for a tile of `fine` values that leaves as the element type
+template <int THREADS>
+__device__ __forceinline__ void store_tile_fine_as_elem(elem *gdst, int64_t gstride, const elem *tile, int pitch, int ncols,
+                                                        int valid) {
+    const int cpr = ncols >> 3;
+    for (int idx = threadIdx.x; idx < valid * cpr; idx += THREADS) {
+        const int r = idx / cpr, c = (idx % cpr) << 3;
+        *reinterpret_cast<elemx8 *>(gdst + (int64_t)r * gstride + c) =
+            fine_to_elem(*reinterpret_cast<const finex8 *>(tile + r * pitch + c));
+    }
 }
 
 // ---- the k tile -------------------------------------------------------------------------------

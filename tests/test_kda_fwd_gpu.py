@@ -158,11 +158,12 @@ def test_chunk_kda_fwd(dev, case):
     assert all(t.dtype == q.dtype for t in (o, Aqk, Akk, w, u, qg, kg, v_new, h))
     head = (lambda x: x[None]) if layout in ("TND", "NTD") else (lambda x: x)
 
-    assert_close(from_layout(o, layout), o_naive, TOL_BF16, "o vs recurrence")
+    st = assert_close(from_layout(o, layout), o_naive, TOL_BF16, "o vs recurrence")
+    assert st["rel_max"] < 2e-2, st
     fin = final.transpose(-1, -2) if v_first else final
     assert final.dtype == torch.float32
     # a 128-token chunk works against one 16-bit copy of the state for twice as many tokens
-    assert_close(fin, f_naive, (4 if C == 64 else 8) * TOL_STATE, "final state vs recurrence")
+    assert_close(fin, f_naive, (1 if C == 64 else 2) * TOL_STATE, "final state vs recurrence")
     assert_close(fin, ref["final_state"], TOL_BF16, "final state vs chunked")
 
     assert gk.dtype == torch.float32
@@ -241,7 +242,7 @@ def test_chunk_kda_fwd_state_handoff_and_determinism(dev):
     nat = kda.kda_gate(g)
     o_naive, f_naive = kda.naive_recurrent_kda(q, k, v, nat, beta, scale, output_final_state=True)
     assert_close(from_layout(o, "BSND"), o_naive, TOL_BF16, "o vs recurrence, T=1024")
-    assert_close(final, f_naive, 4 * TOL_STATE, "final state vs recurrence, T=1024")
+    assert_close(final, f_naive, TOL_STATE, "final state vs recurrence, T=1024")
 
 
 def test_chunk_kda_fwd_packed_equals_separate(dev):
@@ -310,7 +311,7 @@ def test_chunk_kda_fwd_bench_shape_properties(dev):
     o64, f64 = ops.chunk_kda_fwd(q, k, v, g, beta, scale, 64, initial_state=h0, output_final_state=True)[:2]
     o128, f128 = ops.chunk_kda_fwd(q, k, v, g, beta, scale, 128, initial_state=h0, output_final_state=True)[:2]
     assert_close(o128, o64, TOL_BF16, "o: 128- against 64-token chunks")
-    assert_close(f128, f64, 8 * TOL_STATE, "final state: 128- against 64-token chunks")
+    assert_close(f128, f64, 2 * TOL_STATE, "final state: 128- against 64-token chunks")
     cut = 4096 + 128
     a = [x[:, :cut].contiguous() for x in (q, k, v, g, beta)]
     b = [x[:, cut:].contiguous() for x in (q, k, v, g, beta)]
@@ -323,3 +324,28 @@ def test_chunk_kda_fwd_bench_shape_properties(dev):
     o_ref, _ = kda.naive_recurrent_kda(sl(q), sl(k), sl(v), sl(g), beta[bi:bi + 1, :Ts, hi:hi + 1].transpose(1, 2).cpu(), scale,
                                        initial_state=h0[bi:bi + 1, hi:hi + 1].cpu(), output_final_state=True)
     assert_close(o128[bi:bi + 1, :Ts, hi:hi + 1].transpose(1, 2), o_ref, TOL_BF16, "o slice vs recurrence")
+
+
+def test_chunk_kda_fwd_bench_shape_unscaled_gate(dev):
+    """B=2 T=8192 H=32 K=V=128 with the gate as the benchmark configuration draws it (logsigmoid of a standard normal,
+    not scaled down): attention output and fp32 final state of one (batch row, head) slice over all 8192 tokens against
+    the per-token recurrence on the CPU, at the acceptance tolerances."""
+    from fla_hip import ops
+    B, T, H, K, V = 2, 8192, 32, 128, 128
+    gen = torch.Generator(device=dev).manual_seed(5)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=gen)
+    q = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1).to(BF)
+    k = torch.nn.functional.normalize(rn(B, T, H, K), dim=-1).to(BF)
+    v = rn(B, T, H, V).to(BF)
+    g = torch.nn.functional.logsigmoid(rn(B, T, H, K))
+    beta = torch.sigmoid(rn(B, T, H))
+    h0 = rn(B, H, K, V) * 0.01
+    scale = K ** -0.5
+    o, final = ops.chunk_kda_fwd(q, k, v, g, beta, scale, 64, initial_state=h0, output_final_state=True)[:2]
+    for bi, hi in ((1, 17), (0, 0)):
+        sl = lambda x: x[bi:bi + 1, :, hi:hi + 1].transpose(1, 2).float().cpu()
+        o_ref, f_ref = kda.naive_recurrent_kda(sl(q), sl(k), sl(v), sl(g), beta[bi:bi + 1, :, hi:hi + 1].transpose(1, 2).cpu(),
+                                               scale, initial_state=h0[bi:bi + 1, hi:hi + 1].cpu(), output_final_state=True)
+        st = assert_close(o[bi:bi + 1, :, hi:hi + 1].transpose(1, 2), o_ref, TOL_BF16, f"o of slice ({bi}, {hi})")
+        assert st["rel_max"] < 2e-2, st
+        assert_close(final[bi:bi + 1, hi:hi + 1], f_ref, TOL_STATE, f"final state of slice ({bi}, {hi})")
