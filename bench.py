@@ -437,6 +437,7 @@ def bench_kda(args, torch, dev):
     in the same run and reported under ``fwd_bwd``, every kernel with its dense-tile FLOP count."""
     import fla_hip
     from fla_hip import ops, pipeline
+    from fla_hip.ops import _hip_ctypes as raw_ops
 
     lib = fla_hip.load_library()
     B, T, H, K, V, C = 2, 8192, 32, 128, 128, args.kda_chunk
@@ -457,8 +458,10 @@ def bench_kda(args, torch, dev):
         return ops.chunk_kda_fwd(q, k, v, g, beta, scale, C, layout="BSND", initial_state=h0, output_final_state=True)
 
     def train_step():
-        f = ops.chunk_kda_fwd(q, k, v, g, beta, scale, C, layout="BSND", initial_state=h0, output_final_state=True,
-                              disable_recompute=True, return_intermediate_states=True)
+        # the forward as the autograd entry (pipeline.chunk_kda) runs it: every intermediate the backward reads, qg and kg
+        # as float16 for the reverse scan, no u
+        f = raw_ops.chunk_kda_fwd_for_backward(q, k, v, g, beta, scale, C, layout="BSND", initial_state=h0,
+                                               output_final_state=True)
         _o, _final, gk, Aqk, Akk, w, _u, qg, kg, v_new, h, _ = f
         return pipeline.chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, d_o, dht,
                                       initial_state=h0, layout="BSND", chunk_size=C)

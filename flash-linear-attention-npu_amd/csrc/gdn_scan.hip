@@ -557,8 +557,12 @@ __device__ __forceinline__ void t_tiles(const elem *kS, const elem *qS, const fl
 // above the diagonal by the copying waves, the four on it by the compute waves), in the second half every compute wave
 // takes T do for its own 16 columns, which lands in accumulators of the layout of dv2, so the intra-chunk dv is never
 // rounded or stored.
-template <int K, bool GK, bool DVL = false>
+// FQ (per-channel gate only): q and k hold `fine` values (chunk_kda_fwd keeps qg and kg so for a training step) and meet
+// fp16 copies of d_o * scale and of the incoming gradient; the two products that carry the leading terms of dh then round
+// their operands to 11 bits instead of 8.
+template <int K, bool GK, bool DVL = false, bool FQ = false>
 __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
+    static_assert(!FQ || (GK && DVL), "fp16 q and k are built for the KDA form");
     extern __shared__ __align__(16) unsigned char smem[];
     typedef DhuSmem<K> L;
     constexpr int VS = 64, CT = 1;
@@ -772,7 +776,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
 #pragma unroll
             for (int j = 0; j < KS; ++j)
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) hB[j][ct] = frag_from_acc(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
+                for (int ct = 0; ct < CT; ++ct) hB[j][ct] = pack_operand<FQ>(dacc[2 * j][ct], dacc[2 * j + 1][ct]);
         }
 
         // dv2 = dv + (k . dh) * e^{g_last - g}
@@ -787,7 +791,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             for (int rt = 0; rt < 4; ++rt) {
                 const elemx8 afrag = frag_kc(kS, pk, rt * 16, 32 * j);
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = mfma16x32(afrag, hB[j][ct], dv2[rt][ct]);
+                for (int ct = 0; ct < CT; ++ct) dv2[rt][ct] = mfma16x32_as<FQ>(afrag, hB[j][ct], dv2[rt][ct]);
             }
         if (chunk_end) g_end = GK ? 0.f : gS[len - 1];
         const float g_last = g_end;
@@ -932,7 +936,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                     lo[e] = (float)raw[e] * f0[e];
                     hi[e] = (float)raw[4 + e] * f1[e];
                 }
-                ob[ct] = frag_from_acc(lo, hi);
+                ob[ct] = pack_operand<FQ>(lo, hi);
                 nb[ct] = frag_from_acc(-dv2[2 * j][ct], -dv2[2 * j + 1][ct]);
             }
 #pragma unroll
@@ -941,7 +945,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
                 const elemx8 wf = frag_tr(wS, pt, kt * 16, 32 * j);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
-                    dacc[kt][ct] = mfma16x32(qf, ob[ct], dacc[kt][ct]);
+                    dacc[kt][ct] = mfma16x32_as<FQ>(qf, ob[ct], dacc[kt][ct]);
                     dacc[kt][ct] = mfma16x32(wf, nb[ct], dacc[kt][ct]);
                 }
             }
@@ -1106,12 +1110,12 @@ int launch_bwd_dhu_wide(const DhuParams &p, int slabs, hipStream_t stream) {
     return FLA_OK;
 }
 
-template <int K, bool GK, bool DVL = false>
+template <int K, bool GK, bool DVL = false, bool FQ = false>
 int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
     const size_t smem = DVL ? DhuSmem<K>::bytes_dvl : DhuSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK, DVL>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK, DVL, FQ>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK, DVL>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK, DVL, FQ>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
@@ -1137,6 +1141,16 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
                 "%s: dv may be left out with the scalar gate g and chunk_size 64 only.", op);
     FLA_REQUIRE(!has_aqk || (has_gk && !has_dv && chunk_size == kChunk), FLA_ERR_UNSUPPORTED,
                 "%s: Aqk takes the place of dv with the per-channel gate gK and chunk_size 64 only.", op);
+    // The KDA form also takes q and k (qg and kg of chunk_kda_fwd) as float16 tensors beside bf16 w, d_o and Aqk.
+    const bool fine_qk = has_aqk && !kFineIsElem && q && k && q->dtype == FLA_F16 && k->dtype == FLA_F16;
+    fla_tensor q_as_elem, k_as_elem;
+    if (fine_qk) {
+        q_as_elem = *q;
+        k_as_elem = *k;
+        q_as_elem.dtype = k_as_elem.dtype = kElemDtype;
+        q = &q_as_elem;
+        k = &k_as_elem;
+    }
     if ((rc = gdn_geometry(op, k, has_dv ? dv : d_o, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
     FLA_REQUIRE(geom.C == kChunk || !has_gk, FLA_ERR_UNSUPPORTED, "%s: gK is built for chunk_size 64.", op);
     const int bf = dt_bit(kElemDtype);
@@ -1238,6 +1252,11 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
     p.scale = (float)scale;
     p.sub = geom.C / kChunk;
     const int slabs = geom.V / 64;
+    if constexpr (!kFineIsElem) {
+        if (fine_qk)
+            return geom.K == 128 ? launch_bwd_dhu<128, true, true, true>(p, slabs, stream)
+                                 : launch_bwd_dhu<64, true, true, true>(p, slabs, stream);
+    }
     if (has_aqk) return geom.K == 128 ? launch_bwd_dhu<128, true, true>(p, slabs, stream) : launch_bwd_dhu<64, true, true>(p, slabs, stream);
     if (!has_dv) return geom.K == 128 ? launch_bwd_dhu<128, false, true>(p, slabs, stream) : launch_bwd_dhu<64, false, true>(p, slabs, stream);
     if (geom.K == 256) return launch_bwd_dhu_wide<256>(p, slabs, stream);
@@ -1275,7 +1294,7 @@ FLA_ENTRY(fla_chunk_kda_bwd_dhu_get_workspace_size)(
     const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
     const fla_tensor *dv2, uint64_t *workspace_size) {
-    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dhu_get_workspace_size, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace_size);
+    FLA_ROUTE_F16(d_o, fla_chunk_kda_bwd_dhu_get_workspace_size, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace_size);
     if (!workspace_size) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: workspace_size must not be null.");
     if (!Aqk || !Aqk->data) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: Aqk must not be null.");
     return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, nullptr, nullptr, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, true,
@@ -1287,7 +1306,7 @@ FLA_ENTRY(fla_chunk_kda_bwd_dhu)(
     const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
     const fla_int_array *chunk_indices, double scale, int64_t chunk_size, const fla_tensor *dh, const fla_tensor *dh0,
     const fla_tensor *dv2, void *workspace, uint64_t workspace_size, void *stream) {
-    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dhu, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace, workspace_size, stream);
+    FLA_ROUTE_F16(d_o, fla_chunk_kda_bwd_dhu, q, k, w, d_o, Aqk, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, dh, dh0, dv2, workspace, workspace_size, stream);
     if (!Aqk || !Aqk->data) return fla::fail(FLA_ERR_NULL, "chunk_kda_bwd_dhu: Aqk must not be null.");
     return fla::guarded([&] { return fla::bwd_dhu_impl(q, k, w, d_o, nullptr, nullptr, gK, h0, dht, cu_seqlens, chunk_indices, scale, chunk_size, true,
                              dh, dh0, dv2, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr, Aqk); });

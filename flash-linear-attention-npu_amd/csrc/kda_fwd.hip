@@ -51,6 +51,7 @@ struct KdaIntraParams {
     // tensors of the element type, written as well when they are not null (never set when elem is fp16 itself)
     fine *u16, *kg16;
     elem *u, *kg;
+    int qg_fine;              // qg is a tensor of `fine` values (the caller keeps it for a reverse scan that reads it so)
     float *dec;               // [B,NT,Hv,K]: 2^{g_last} of every chunk
     // 128-token chunks: a workgroup still owns 64 tokens (one half of a chunk); the operands of the block that
     // couples the halves go to x1 (first half: k 2^{G1 - g}; second half: q 2^{g - G1}) and x2 (second half:
@@ -291,7 +292,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         const elemx8 k8 = *reinterpret_cast<const elemx8 *>(kS + r * pk + c8);
         const float br = bS[r];
         elemx8 qg8, kg8, kb8;
-        u32x4 kgf;
+        u32x4 kgf, qgf;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + kChunk * pg + c8 + 4 * h);
@@ -306,6 +307,8 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             const elemx4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
             kgf[2 * h] = cvt2_fine(b[0], b[1]);
             kgf[2 * h + 1] = cvt2_fine(b[2], b[3]);
+            qgf[2 * h] = cvt2_fine(a[0], a[1]);
+            qgf[2 * h + 1] = cvt2_fine(a[2], a[3]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 qg8[4 * h + e] = a4[e];
@@ -314,7 +317,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             }
         }
         if (r < len) {
-            *reinterpret_cast<elemx8 *>(p.qg + (row_base + r) * K + c8) = qg8;
+            *reinterpret_cast<u32x4 *>(p.qg + (row_base + r) * K + c8) = p.qg_fine ? qgf : __builtin_bit_cast(u32x4, qg8);
             *reinterpret_cast<u32x4 *>(p.kg16 + (row_base + r) * K + c8) = kgf;
             if constexpr (!kFineIsElem) {
                 if (p.kg != nullptr) *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
@@ -805,6 +808,7 @@ struct KdaScanParams {
     int64_t s_sn, s_sh;                  // strides of h0 / hT over (sequence, head)
     int v_first;
     float scale;
+    int qg_fine;                         // qg holds `fine` values
 };
 
 template <int K> struct ScanSmem {
@@ -831,7 +835,9 @@ template <int K> struct ScanSmem {
 // w S and qg S (the operand copy of the state is refreshed on even steps only), the second step adds the
 // coupling block Aqk21 times the first step's v_new, and the decay of the chunk is applied once, on the first step
 // (kg already carries 2^{g_last - g} up to the end of the whole chunk).
-template <int K, int SUB>
+// QF: qg holds `fine` values (the forward of a training step keeps it so for the reverse scan) and meets a `fine` copy
+// of the state.
+template <int K, int SUB, bool QF>
 __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     typedef ScanSmem<K> L;
@@ -988,7 +994,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     };
     __syncthreads();
 
-    elemx8 hB[KS], vprev[2] = {};
+    elemx8 hB[KS], hQ[QF ? KS : 1], vprev[2] = {};
     for (int c = 0; c < nchunks; ++c) {
         const unsigned char *buf = smem + (c & 1) * L::buf_bytes;
         const elem *wS = reinterpret_cast<const elem *>(buf + L::w_off);
@@ -1004,7 +1010,10 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 
         if (first) {
 #pragma unroll
-            for (int j = 0; j < KS; ++j) hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+            for (int j = 0; j < KS; ++j) {
+                hB[j] = frag_from_acc(hacc[2 * j], hacc[2 * j + 1]);
+                if constexpr (QF) hQ[j] = pack_operand<true>(hacc[2 * j], hacc[2 * j + 1]);
+            }
         }
         if (p.h && p.v_first && first) {   // [V][K] blocks: the lane's four K rows are contiguous
             elem *hg = p.h + b * p.h_sb + (int64_t)(chunk0 + c / SUB) * p.h_sc + hv * p.h_sh;
@@ -1056,7 +1065,7 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
 #pragma unroll
             for (int j = 0; j < KS; ++j)
 #pragma unroll
-                for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32(qf[j][rt], hB[j], oacc[rt]);
+                for (int rt = 0; rt < 4; ++rt) oacc[rt] = mfma16x32_as<QF>(qf[j][rt], QF ? hQ[j] : hB[j], oacc[rt]);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (stage_h) {   // the copying waves have read the state tile of the step before; the state is still that of
@@ -1344,8 +1353,8 @@ int layout_view(const char *op, const char *name, const fla_tensor *t, const Lay
 
 // head-major output [B,Hv,T,D] (or [Hv,T,D]); contiguous
 int head_major(const char *op, const char *name, const fla_tensor *t, bool rank3, int64_t B, int64_t H, int64_t T, int64_t D,
-               int dtype) {
-    int rc = check_tensor(t, op, name, rank3 ? 3 : 4, dt_bit(dtype));
+               int dtype, int also = -1) {
+    int rc = check_tensor(t, op, name, rank3 ? 3 : 4, dt_bit(dtype) | (also < 0 ? 0 : dt_bit(also)));
     if (rc) return rc;
     const int o = rank3 ? 0 : 1;
     FLA_REQUIRE((rank3 || t->shape[0] == B) && t->shape[o] == H && t->shape[o + 1] == T && t->shape[o + 2] == D &&
@@ -1385,15 +1394,22 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
     return FLA_OK;
 }
 
-template <int K, int SUB>
-int launch_scan(const KdaScanParams &p, hipStream_t stream) {
+template <int K, int SUB, bool QF>
+int launch_scan_as(const KdaScanParams &p, hipStream_t stream) {
     const size_t smem = ScanSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K, SUB>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K, SUB, QF>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K, SUB>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem, stream,
-               p);
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K, SUB, QF>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem,
+               stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
+}
+template <int K, int SUB>
+int launch_scan(const KdaScanParams &p, hipStream_t stream) {
+    if constexpr (!kFineIsElem) {
+        if (p.qg_fine) return launch_scan_as<K, SUB, true>(p, stream);
+    }
+    return launch_scan_as<K, SUB, false>(p, stream);
 }
 
 template <int K, int SUB>
@@ -1493,8 +1509,12 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     if (present(gk) && (rc = head_major(op, "gk", gk, L.rank3(), B, Hv, T, K, FLA_F32))) return rc;
     if (present(w) && (rc = head_major(op, "w", w, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
     if (present(u) && (rc = head_major(op, "u", u, L.rank3(), B, Hv, T, V, kElemDtype))) return rc;
-    if (present(qg) && (rc = head_major(op, "qg", qg, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
-    if (present(kg) && (rc = head_major(op, "kg", kg, L.rank3(), B, Hv, T, K, kElemDtype))) return rc;
+    // qg and kg may be float16 tensors whatever the element type: the precision in which the scan reads kg anyway, and
+    // in which a reverse scan (chunk_kda_bwd_dhu) wants both
+    if (present(qg) && (rc = head_major(op, "qg", qg, L.rank3(), B, Hv, T, K, kElemDtype, FLA_F16))) return rc;
+    if (present(kg) && (rc = head_major(op, "kg", kg, L.rank3(), B, Hv, T, K, kElemDtype, FLA_F16))) return rc;
+    FLA_REQUIRE(geom.K <= 128 || ((!present(qg) || qg->dtype == kElemDtype) && (!present(kg) || kg->dtype == kElemDtype)),
+                FLA_ERR_UNSUPPORTED, "%s: float16 qg / kg beside other elements are built for K <= 128.", op);
     if (present(v_new) && (rc = head_major(op, "v_new", v_new, L.rank3(), B, Hv, T, V, kElemDtype))) return rc;
     const int64_t d2 = state_v_first ? V : K, d3 = state_v_first ? K : V;
     auto check_state = [&](const fla_tensor *s, const char *name) -> int {
@@ -1527,7 +1547,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     size_t w_off = 0, u_off = 0, qg_off = 0, kg_off = 0, x1_off = 0, x2_off = 0;
     // u and kg go to the scan as fp16 (`fine`): with fp16 elements the caller's tensors serve, otherwise the workspace
     // holds the fp16 copies whether or not the caller also takes u and kg
-    const bool fine_u_ws = !kFineIsElem || !present(u), fine_kg_ws = !kFineIsElem || !present(kg);
+    const bool kg_is_fine = present(kg) && kg->dtype == FLA_F16;   // always so with fp16 elements
+    const bool fine_u_ws = !kFineIsElem || !present(u), fine_kg_ws = !kg_is_fine;
     if (C == 128) {
         x1_off = off;
         off += align256(rows * K * 2);
@@ -1568,7 +1589,8 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     ip.u = !kFineIsElem && present(u) ? static_cast<elem *>(u->data) : nullptr;
     ip.qg = present(qg) ? static_cast<elem *>(qg->data) : reinterpret_cast<elem *>(wsb + qg_off);
     ip.kg16 = fine_kg_ws ? reinterpret_cast<fine *>(wsb + kg_off) : static_cast<fine *>(kg->data);
-    ip.kg = !kFineIsElem && present(kg) ? static_cast<elem *>(kg->data) : nullptr;
+    ip.kg = present(kg) && !kg_is_fine ? static_cast<elem *>(kg->data) : nullptr;
+    ip.qg_fine = !kFineIsElem && present(qg) && qg->dtype == FLA_F16;
     ip.dec = reinterpret_cast<float *>(wsb + dec_off);
     ip.c128 = C == 128;
     ip.x1 = reinterpret_cast<elem *>(wsb + x1_off);
@@ -1602,6 +1624,7 @@ int kda_fwd_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, 
     }
     sp.v_first = state_v_first;
     sp.scale = (float)scale;
+    sp.qg_fine = ip.qg_fine;
     if (N == 0) return FLA_OK;
     if (K == 256) return C == 128 ? launch_scan_wide<256, 2>(sp, stream) : launch_scan_wide<256, 1>(sp, stream);
     if (C == 128) return K == 128 ? launch_scan<128, 2>(sp, stream) : launch_scan<64, 2>(sp, stream);

@@ -112,6 +112,16 @@ __device__ __forceinline__ elemx8 fine_to_elem(finex8 x) {
         return frag_from_acc(lo, hi);
     }
 }
+// Operand pairs that are `fine` values when F is set and elements otherwise, both carried as elemx8 bit patterns.
+template <bool F> __device__ __forceinline__ elemx8 pack_operand(f32x4 lo, f32x4 hi) {
+    if constexpr (F) return __builtin_bit_cast(elemx8, fine_from_acc(lo, hi));
+    else return frag_from_acc(lo, hi);
+}
+template <bool F> __device__ __forceinline__ f32x4 mfma16x32_as(elemx8 a, elemx8 b, f32x4 c) {
+    if constexpr (F) return mfma16x32(as_fine(a), as_fine(b), c);
+    else return mfma16x32(a, b, c);
+}
+
 // ---- cooperative global <-> LDS tile copies (all threads of the block) -----------
 // Copies rows [0, valid) x cols [0, ncols) of a row-major global matrix (row stride
 // `gstride` elements, 16-byte aligned rows) into `tile`; rows [valid, nrows) are zeroed.

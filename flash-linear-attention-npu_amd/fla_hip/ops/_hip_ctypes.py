@@ -574,9 +574,23 @@ def chunk_kda_fwd_noalloc(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSN
                           disable_recompute, return_intermediate_states, state_v_first)
 
 
+def chunk_kda_fwd_for_backward(q, k, v, g, beta, scale, chunk_size=64, *, layout="BSND", initial_state=None,
+                               output_final_state=False, cu_seqlens=None, safe_gate=False, lower_bound=None,
+                               use_gate_in_kernel=False, A_log=None, dt_bias=None):
+    """``npu_chunk_kda_fwd`` keeping every intermediate, as the forward of a training step: the same 12-tuple, except
+    that ``u`` is None (no stage of the backward reads it) and that ``qg`` and ``kg`` are float16 tensors also when q is
+    bfloat16 (head sizes up to 128 channels).  They only
+    serve the reverse scan ``chunk_kda_bwd_dhu``, whose q^T d_o product carries the leading term of the state gradient:
+    rounded to 8 significand bits they move dh0 by 3e-3 of its scale, to 11 bits by 5e-4.  No counterpart in the
+    reference, whose backward is a third-party package."""
+    return _chunk_kda_fwd(False, q, k, v, g, beta, scale, chunk_size, layout, initial_state, output_final_state,
+                          cu_seqlens, None, safe_gate, lower_bound, use_gate_in_kernel, A_log, dt_bias, True, True, False,
+                          fine_qk=True)
+
+
 def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial_state, output_final_state, cu_seqlens,
                    chunk_indices, safe_gate, lower_bound, use_gate_in_kernel, A_log, dt_bias, disable_recompute,
-                   return_intermediate_states, state_v_first):
+                   return_intermediate_states, state_v_first, fine_qk=False):
     import torch
 
     op = "npu_chunk_kda_fwd"
@@ -668,7 +682,7 @@ def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial
         h0 = None if initial_state is None else F.pad(initial_state, state_pad)
         res = _chunk_kda_fwd(noalloc, padk(q), padk(k), padv(v), padk(g), beta, scale, chunk_size, layout, h0,
                              output_final_state, cu_seqlens, chunk_indices, safe_gate, lower_bound, use_gate_in_kernel, A_log,
-                             bias, disable_recompute, return_intermediate_states, state_v_first)
+                             bias, disable_recompute, return_intermediate_states, state_v_first, fine_qk=fine_qk)
         attn_out, final_state, gk, aqk, akk, w, u, qg, kg, v_new, h = res[:11]
         cut = lambda t, n: None if t is None else t[..., :n].contiguous()
         cut2 = lambda t: None if t is None else \
@@ -687,9 +701,10 @@ def _chunk_kda_fwd(noalloc, q, k, v, g, beta, scale, chunk_size, layout, initial
     aqk = _empty((*lead, HV, T, chunk_size), q)
     akk = _empty((*lead, HV, T, chunk_size), q)
     w = _empty((*lead, HV, T, K), q) if mask[5] else None
-    u = _empty((*lead, HV, T, V), q) if mask[6] else None
-    qg = _empty((*lead, HV, T, K), q) if mask[7] else None
-    kg = _empty((*lead, HV, T, K), q) if mask[8] else None
+    u = _empty((*lead, HV, T, V), q) if mask[6] and not fine_qk else None   # no stage of the backward reads u
+    qk_dtype = torch.float16 if fine_qk and K <= 128 else q.dtype
+    qg = _empty((*lead, HV, T, K), q, dtype=qk_dtype) if mask[7] else None
+    kg = _empty((*lead, HV, T, K), q, dtype=qk_dtype) if mask[8] else None
     v_new = _empty((*lead, HV, T, V), q) if mask[9] else None
     h = _empty((*lead, NT, HV, *block), q) if mask[10] else None
     outputs = (attn_out, final_state, gk, aqk, akk, w, u, qg, kg, v_new, h)
@@ -868,6 +883,7 @@ def chunk_kda_bwd_dhu(qg, kg, w, d_o, Aqk, scale, chunk_size=64, *, gK, h0=None,
     """``npu_chunk_gated_delta_rule_bwd_dhu`` for the KDA backward (per-channel gate ``gK`` in log2 units, 64-token
     chunks) with its dv operand formed inside the scan: dv = Aqk^T d_o per chunk, the second result of
     ``chunk_kda_bwd_dav``, from the forward's score blocks ``Aqk`` [B,Hv,T,64] and the d_o tiles the scan stages anyway.
+    ``qg`` and ``kg`` may be float16 tensors beside bfloat16 ``w``, ``d_o`` and ``Aqk`` (``chunk_kda_fwd_for_backward``).
     Returns ``(dh, dh0, dv2)`` with dh0 fp32 [N,Hv,K,V] (None without ``h0``).  No counterpart in the reference."""
     import torch
 
@@ -880,8 +896,8 @@ def chunk_kda_bwd_dhu(qg, kg, w, d_o, Aqk, scale, chunk_size=64, *, gK, h0=None,
         indices = _build_chunk_indices(cu, chunk_size)
     NT = _total_chunks(B, T, chunk_size, cu) if indices is None else len(indices) // 2
     N = len(cu) - 1 if cu is not None else B
-    dh = _empty((B, Hv, NT, K, V), qg)
-    dh0 = None if h0 is None else _empty((N, Hv, K, V), qg, dtype=torch.float32)
+    dh = _empty((B, Hv, NT, K, V), w)
+    dh0 = None if h0 is None else _empty((N, Hv, K, V), w, dtype=torch.float32)
     dv2 = _empty_ordered_like(d_o)
     outputs = (dh, dh0, dv2)
     return _call_op(

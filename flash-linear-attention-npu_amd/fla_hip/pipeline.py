@@ -392,10 +392,10 @@ def _kda_autograd_function():
         def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, layout, chunk_size, A_log=None,
                     dt_bias=None, safe_gate=False, lower_bound=-5.0):
             in_kernel = A_log is not None
-            out = _ops.chunk_kda_fwd(q, k, v, g, beta, scale, chunk_size, layout=layout, initial_state=initial_state,
-                                     output_final_state=output_final_state, cu_seqlens=cu, disable_recompute=True,
-                                     return_intermediate_states=True, use_gate_in_kernel=in_kernel, A_log=A_log,
-                                     dt_bias=dt_bias, safe_gate=safe_gate, lower_bound=lower_bound)
+            out = _raw.chunk_kda_fwd_for_backward(q, k, v, g, beta, scale, chunk_size, layout=layout,
+                                                  initial_state=initial_state, output_final_state=output_final_state,
+                                                  cu_seqlens=cu, use_gate_in_kernel=in_kernel, A_log=A_log, dt_bias=dt_bias,
+                                                  safe_gate=safe_gate, lower_bound=lower_bound)
             o, final, gk, Aqk, Akk, w, _u, qg, kg, v_new, h, _ = out
             ctx.save_for_backward(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, initial_state,
                                   *((g, A_log, dt_bias) if in_kernel else ()))

@@ -18,6 +18,9 @@ BF = torch.bfloat16
 REL = 2e-2
 
 
+DH0_REL = 2e-3
+
+
 def close(actual, expected, name, rel=REL):
     st = err_stats(actual, expected)
     assert torch.isfinite(actual.float()).all(), f"{name}: non-finite"
@@ -230,7 +233,9 @@ def test_chunk_kda_backward_against_autograd_through_the_recurrence(dev, case):
         if e is None:
             assert a is None
             continue
-        stats[name] = close(a, e, name)["rel_max"]
+        # the gradient of the fp32 initial state is held to 2e-3 of its scale on the kernels built for up to 128
+        # channels, whose reverse scan reads qg and kg as float16
+        stats[name] = close(a, e, name, DH0_REL if name == "dh0" and K <= 128 and dtype == BF else REL)["rel_max"]
     print(f"\n[kda bwd {layout} T={T} Hv={Hv} K={K} V={V}] rel_max " + " ".join(f"{n}={s:.1e}" for n, s in stats.items()))
 
 
@@ -273,7 +278,7 @@ def test_chunk_kda_backward_at_the_bench_shape(dev):
     for name, a, e in zip(names[:4], whole[:4], want[:4]):
         stats[name] = close(a[b:b + 1, :, h:h + 1].transpose(1, 2), e, name)["rel_max"]
     stats["dbeta"] = close(whole[4][b:b + 1, :, h:h + 1].transpose(1, 2), want[4], "dbeta")["rel_max"]
-    stats["dh0"] = close(whole[5][b:b + 1, h:h + 1], want[5], "dh0")["rel_max"]
+    stats["dh0"] = close(whole[5][b:b + 1, h:h + 1], want[5], "dh0", DH0_REL)["rel_max"]
     print("\n[kda bwd B=2 T=8192 H=32] slice rel_max " + " ".join(f"{n}={s:.1e}" for n, s in stats.items()))
     # (c) hand-off at the middle
     half = T // 2
