@@ -105,8 +105,10 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
             t.gv = 0.f;
             t.dk = 1.f;
             if (p.g.p) t.gv = load_scalar(p.g, b, hv, start + min(tid, len - 1));
-            if (p.gk)
-                t.dk = __builtin_amdgcn_exp2f(p.gk[b * p.gk_sb + hv * p.gk_sh + (int64_t)(start + len - 1) * p.gk_st + min(tid, K - 1)]);
+            if (p.gk) {   // the decay of the whole chunk, 2^{gk at its last token} (a 128-token chunk: of both steps)
+                const int chunk_end = min(bos + (c / p.sub + 1) * p.sub * kChunk, eos);
+                t.dk = __builtin_amdgcn_exp2f(p.gk[b * p.gk_sb + hv * p.gk_sh + (int64_t)(chunk_end - 1) * p.gk_st + min(tid, K - 1)]);
+            }
         };
         auto commit = [&](const Tiles &t, int c) {
             unsigned char *buf = smem + (c & 1) * L::buf_bytes;
@@ -299,7 +301,8 @@ __global__ void __launch_bounds__(512) fwd_h_kernel(const ScanParams p) {
                 }
                 vB[j][ct] = frag_from_acc(lo, hi);
             }
-        if (p.gk) {   // per-channel decay: row kk of the state by 2^{gk_last[kk]} (times the scalar decay, if any)
+        if (p.gk && chunk_start) {   // per-channel decay: row kk of the state by 2^{gk_last[kk]} (times the scalar decay, if
+            // any), once per chunk: k arrives gated up to the end of the whole chunk, in both steps of a 128-token one
             const float *dS = reinterpret_cast<const float *>(buf + L::d_off);
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
@@ -370,7 +373,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
         FLA_REQUIRE(gk->shape[0] == geom.B && gk->shape[1] == geom.Hv && gk->shape[2] == geom.T && gk->shape[3] == geom.K &&
                         inner_unit(gk),
                     FLA_ERR_SHAPE, "%s: gk must be float32 [B,Hv,T,K] with a unit innermost stride.", op);
-        FLA_REQUIRE(geom.C == kChunk, FLA_ERR_UNSUPPORTED, "%s: gk is built for chunk_size 64.", op);
+        FLA_REQUIRE(geom.C == kChunk || geom.K <= 128, FLA_ERR_UNSUPPORTED, "%s: gk with 128-token chunks is built for K <= 128.", op);
     }
     Varlen vl;
     if ((rc = build_varlen(vl, op, cu, ci, geom.C, geom.T))) return rc;
@@ -405,8 +408,7 @@ int fwd_h_impl(const fla_tensor *k, const fla_tensor *w, const fla_tensor *u, co
                     (long long)d2, (long long)d3);
     }
     FLA_REQUIRE(geom.V % 64 == 0, FLA_ERR_UNSUPPORTED, "%s: V must be a multiple of 64, got %d.", op, geom.V);
-    FLA_REQUIRE(geom.K == 128 || geom.K == 64 || (geom.K == 256 && has_gk), FLA_ERR_UNSUPPORTED,
-                "%s: K must be 64 or 128 (256 with gK), got %d.", op, geom.K);
+    FLA_REQUIRE(geom.K == 128 || geom.K == 64, FLA_ERR_UNSUPPORTED, "%s: K must be 64 or 128, got %d.", op, geom.K);
     if (query) {
         *query = vl.bytes();
         return FLA_OK;
@@ -1152,7 +1154,10 @@ int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, 
         k = &k_as_elem;
     }
     if ((rc = gdn_geometry(op, k, has_dv ? dv : d_o, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // README.md:101-104: 64 or 128
-    FLA_REQUIRE(geom.C == kChunk || !has_gk, FLA_ERR_UNSUPPORTED, "%s: gK is built for chunk_size 64.", op);
+    // gK with 128-token chunks (README.md:104): q and k carry their gates relative to the whole chunk, the decay
+    // 2^{gK at the chunk's last token} is applied once, at the chunk's last step
+    FLA_REQUIRE(geom.C == kChunk || !has_gk || geom.K <= 128, FLA_ERR_UNSUPPORTED,
+                "%s: gK with 128-token chunks is built for K <= 128.", op);
     const int bf = dt_bit(kElemDtype);
     if ((rc = check_bhtd(op, "q", q, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;
     if ((rc = check_bhtd(op, "k", k, geom.B, geom.Hk, geom.T, geom.K, bf))) return rc;

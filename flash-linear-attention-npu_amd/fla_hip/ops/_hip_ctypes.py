@@ -280,6 +280,10 @@ def npu_recurrent_gated_delta_rule(query, key, value, state, *, beta, scale=1.0,
     if not math.isfinite(scale):
         raise ValueError(f"{op_name}: scale must be finite, got {scale}.")
 
+    routed = _recurrent_prefill_on_chunk_kernels(query, key, value, state, beta, scale, actual_seq_lengths,
+                                                 ssm_state_indices, num_accepted_tokens, g, gk)
+    if routed is not None:
+        return routed
     out = _empty_like(value)
     return _call_op(
         "recurrent_gated_delta_rule", OP_ARGTYPES["recurrent_gated_delta_rule"],
@@ -293,6 +297,76 @@ def npu_recurrent_gated_delta_rule(query, key, value, state, *, beta, scale=1.0,
         ],
         out,
     )
+
+
+# A call of recurrent_gated_delta_rule with this many tokens per sequence on average is looked at as a prefill (the
+# reference operator stops at 8 tokens per sequence, recurrent_gated_delta_rule.h:28,168-170); a prefill whose longest
+# sequence has at least PREFILL_MIN_TOKENS tokens runs on the chunk kernels.
+PREFILL_AVERAGE_TOKENS = 32
+PREFILL_MIN_TOKENS = 64
+
+
+def _recurrent_prefill_on_chunk_kernels(query, key, value, state, beta, scale, actual_seq_lengths, ssm_state_indices,
+                                        num_accepted_tokens, g, gk):
+    """Long sequences of ``recurrent_gated_delta_rule`` on the fused chunk forward (``gdn_chunk_fwd``) instead of the
+    token-by-token kernel, whose time is the latency of the longest sequence.  Returns ``out`` with ``state`` updated
+    in place, or None when the call stays on the token-by-token kernel: few tokens per sequence (decode and
+    speculative decoding), a key-wise gate, accepted-token counts, a head size the chunk kernel is not built for,
+    slots that change inside a sequence or are shared between sequences (then the state after EVERY token is part of
+    the contract; here only the state after a sequence's last token is written, to that sequence's slot), or a stream
+    under capture (the sequence lengths are read on the host, one synchronising copy)."""
+    import torch
+
+    total, nk, dk = _shape(query)
+    _, nv, dv = _shape(value)
+    batch = _shape(actual_seq_lengths)[0] - 1
+    if g is None or gk is not None or num_accepted_tokens is not None:
+        return None
+    if total < PREFILL_AVERAGE_TOKENS * batch or dk not in (64, 128) or dv % 64 != 0 or dv > 256:
+        return None
+    if any(t.stride(-1) != 1 for t in (query, key, value)) or state.stride(-1) != 1 or torch.cuda.is_current_stream_capturing():
+        return None
+    # The plan is formed on the device and read with ONE synchronising copy: the sequence lengths and a flag that says
+    # whether every token of a sequence names the slot of its first token, whether the slots are valid and whether no
+    # two sequences share one.  The pool rows are gathered ahead of that copy, so that they are on their way while the host waits.
+    dev, blocks = query.device, _shape(state)[0]
+    lens_d = actual_seq_lengths.to(torch.int64)
+    span = lens_d[1:]
+    ends = lens_d[0] + torch.cumsum(span, 0)
+    starts = ends - span
+    tok = torch.arange(total, device=dev)
+    seq = torch.searchsorted(ends, tok, right=True)                  # sequence of token t; `batch` past the last one
+    inside = (tok >= lens_d[0]) & (seq < batch)
+    slot = ssm_state_indices[starts.clamp(0, total - 1)].to(torch.int64)
+    live = span > 0
+    valid = (slot >= 0) & (slot < blocks)
+    same = ((ssm_state_indices == slot[seq.clamp(max=batch - 1)]) | ~inside).all()
+    uses = torch.zeros(blocks + 1, dtype=torch.int64, device=dev)
+    uses.index_add_(0, torch.where(live & valid, slot, torch.full_like(slot, blocks)), torch.ones_like(slot))
+    ok = same & (valid | ~live).all() & (uses[:blocks] <= 1).all() & (span >= 0).all() & (ends[-1] <= total)
+    slot = slot.clamp(0, blocks - 1)
+    h0 = state.transpose(-1, -2)[slot].float().contiguous()         # V-first pool rows -> [N,H,K,V] fp32
+    plan = torch.cat([lens_d, ok.to(torch.int64)[None]]).tolist()
+    skip, lens, ok = plan[0], plan[1:-1], plan[-1]
+    if not ok or skip < 0 or max(lens) < PREFILL_MIN_TOKENS:
+        return None
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    at = skip + cu[-1]
+    head_major = lambda t: t[skip:at].transpose(0, 1)[None]            # [T,H,D] -> [1,H,T,D] view, nothing copied
+    _, o, final = gdn_chunk_fwd(head_major(query), head_major(key), head_major(value), g[skip:at][None],
+                                beta[skip:at][None].float(), scale, h0, True, cu, 64)
+    if min(lens) > 0:
+        state[slot] = final.transpose(-1, -2).to(state.dtype)
+    else:   # a sequence without tokens names no slot
+        rows = torch.tensor([i for i, n in enumerate(lens) if n > 0], dtype=torch.int64, device=dev)
+        state[slot[rows]] = final[rows].transpose(-1, -2).to(state.dtype)
+    if skip == 0 and at == total:
+        return o[0]
+    out = torch.zeros_like(value)
+    out[skip:at] = o[0]
+    return out
 
 
 def _chunk_local_cumsum_output_dtype(g, output_dtype):

@@ -51,6 +51,20 @@ def test_against_naive_recurrence(dev, case, fused, dtype):
     assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
 
 
+@pytest.mark.parametrize("fused", [True, False], ids=["fused", "operators"])
+def test_cfg1_shape_and_seed_in_bf16(dev, fused):
+    """The self-check configuration of the benchmark set on the GPU: B=1 T=256 H=2 K=V=64, chunk 64, seed 0, zero
+    initial state (the CPU oracle runs it in fp32, tests/test_oracle.py); here the same tensors rounded to bf16 go
+    through both routes of the pipeline entry and are held to the acceptance tolerances against the fp32 per-token
+    recurrence on those bf16 inputs."""
+    d = gdn.make_gdn_inputs(1, 256, 2, 64, 64, dtype=BF, seed=0)
+    o, final, o_ref, f_ref = run_both(dev, d, fused=fused)
+    assert o.shape == (1, 256, 2, 64) and o.dtype == BF and final.shape == (1, 2, 64, 64) and final.dtype == torch.float32
+    st = assert_close(o, o_ref, TOL_BF16, "o")
+    assert st["rel_max"] < 2e-2, st
+    assert_close(final, f_ref, TOL_STATE if fused else 4 * TOL_STATE, "final_state")
+
+
 @pytest.mark.parametrize("dtype", [BF, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("case", CASES)
 def test_forward_writes_the_operands_of_the_backward(dev, case, dtype):

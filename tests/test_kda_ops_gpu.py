@@ -88,11 +88,13 @@ DHU_CASES = [
 ]
 
 
-# 128-token chunks (chunk_gated_delta_rule_bwd_dhu/README.md:101-104) with the scalar gate: full chunks, a last chunk with
-# only its first half, packed sequences of every remainder
-DHU_CASES_128 = [c for c in DHU_CASES if not c[7]] + [
+# 128-token chunks (chunk_gated_delta_rule_bwd_dhu/README.md:101-104) with either gate (the per-channel one on the kernels
+# for up to 128 channels): full chunks, a last chunk with only its first half, packed sequences of every remainder
+DHU_CASES_128 = [c for c in DHU_CASES if not c[7] or c[4] <= 128] + [
     (1, 421, 2, 2, 128, 128, [0, 1, 66, 66, 194, 300, 421], False, True),
     (1, 192, 1, 2, 128, 128, None, False, True),
+    (1, 421, 2, 2, 128, 128, [0, 1, 66, 66, 194, 300, 421], True, True),
+    (1, 192, 1, 2, 128, 128, None, True, False),
 ]
 
 
@@ -254,8 +256,16 @@ def test_fwd_h_with_key_wise_gate(dev, case):
                                                 output_final_state=True, cu_seqlens=cu)
         assert_close(got2[1], ref2[1], TOL_BF16, "v_new (g and gk)")
         assert_close(got2[2], ref2[2], 4e-3, "final_state (g and gk)")
-    with pytest.raises(RuntimeError, match="chunk_size 64"):
-        ops.chunk_gated_delta_rule_fwd_h(kgt.to(dev), w.to(dev), u.to(dev), gk=gk.to(dev), chunk_size=128)
+    # 128-token chunks (README.md:87): the gate cumulated over the whole chunk, its decay applied once per chunk
+    gk128 = kda.kda_gate_cumsum(torch.nn.functional.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, 128, cu_seqlens=cu)
+    ref3 = gdn.chunk_gated_delta_rule_fwd_h(kgt, w, u, gk=gk128, initial_state=h0, output_final_state=True, chunk=128,
+                                            cu_seqlens=cu, lowp=BF, output_dtype=torch.float32)
+    got3 = ops.chunk_gated_delta_rule_fwd_h(kgt.to(dev), w.to(dev), u.to(dev), gk=gk128.to(dev), initial_state=h0_d,
+                                            output_final_state=True, chunk_size=128, cu_seqlens=cu, state_v_first=v_first)
+    h3, f3 = (got3[0].transpose(-1, -2), got3[2].transpose(-1, -2)) if v_first else (got3[0], got3[2])
+    assert_close(got3[1], ref3[1], TOL_BF16, "v_new (gk, 128-token chunks)")
+    assert_close(h3, ref3[0], TOL_BF16, "h (gk, 128-token chunks)")
+    assert_close(f3, ref3[2], 8e-3, "final_state (gk, 128-token chunks)")
 
 
 # ---------------------------------------------------------------------------------------------

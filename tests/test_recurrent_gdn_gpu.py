@@ -10,6 +10,7 @@ from util import assert_close, TOL_BF16, TOL_STATE
 
 pytestmark = pytest.mark.gpu
 F = torch.nn.functional
+BF = torch.bfloat16
 
 
 def make_inputs(lens, Nk, Nv, Dk, Dv, *, seed=0, skip=0, blocks=None, state_dtype=torch.float32, gk=False, g=True):
@@ -127,6 +128,39 @@ def test_strided_state_pool(dev):
     assert float(pool_d[:, 1::2].abs().max()) == 0.0
 
 
+def launches(kernel, call):
+    """Runs ``call`` and checks through the library's own launch records that ``kernel`` ran."""
+    import ctypes
+
+    import fla_hip
+    lib = fla_hip.load_library()
+    lib.fla_profile_enable.argtypes = [ctypes.c_int]
+    lib.fla_profile_report.argtypes = [ctypes.c_char_p, ctypes.c_uint64]
+    lib.fla_profile_enable(1)
+    try:
+        out = call()
+        torch.cuda.synchronize()
+    finally:
+        lib.fla_profile_enable(0)
+    buf = ctypes.create_string_buffer(1 << 14)
+    lib.fla_profile_report(buf, len(buf))
+    names = [line.split()[0] for line in buf.value.decode().splitlines()]
+    assert kernel in names, (kernel, names)
+    return out
+
+
+class token_by_token:
+    """Keeps recurrent_gated_delta_rule on its token-by-token kernel whatever the sequence lengths."""
+
+    def __enter__(self):
+        from fla_hip.ops import _hip_ctypes as raw
+        self.raw, self.saved = raw, raw.PREFILL_MIN_TOKENS
+        raw.PREFILL_MIN_TOKENS = 1 << 62
+
+    def __exit__(self, *exc):
+        self.raw.PREFILL_MIN_TOKENS = self.saved
+
+
 def test_decode_benchmark_shape_properties(dev):
     """256 sequences x 1 token, 32 heads, K=V=128: oracle on a subset of sequences."""
     from fla_hip import ops
@@ -148,9 +182,10 @@ def test_decode_benchmark_shape_properties(dev):
 
 def test_varlen_prefill_benchmark_shape(dev):
     """The variable-length prefill of the decode benchmark at full size: 64 sequences with lengths uniform in
-    [128, 4096] (about 135 K tokens), 32 heads, K=V=128, one state slot per sequence.  (a) Every sequence run on its own
-    gives the bits of the packed run (a sequence never sees its neighbours); (b) the shortest, the longest and a
-    middle sequence equal the fp32 per-token recurrence.  Far beyond the reference operator's 8-token limit, so the
+    [128, 4096] (about 135 K tokens), 32 heads, K=V=128, one state slot per sequence.  The operator runs it on the chunk
+    kernels; the token-by-token kernel is run on the same call beside it.  (a) Every sequence run on its own gives what
+    the packed run gives (a sequence never sees its neighbours); (b) the shortest, the longest and a middle sequence
+    equal the fp32 per-token recurrence on both kernels.  Far beyond the reference operator's 8-token limit, so the
     recurrence is the only oracle."""
     from fla_hip import ops
     H, D, NSEQ = 32, 128, 64
@@ -168,10 +203,17 @@ def test_varlen_prefill_benchmark_shape(dev):
     seq = torch.cat([torch.zeros(1, dtype=torch.int32), lens.to(torch.int32)]).to(dev)
     idx = torch.repeat_interleave(torch.arange(NSEQ, dtype=torch.int32), lens).to(dev)
     state = state0.clone()
-    o = ops.recurrent_gated_delta_rule(q, k, v, state, beta=beta, scale=D ** -0.5, actual_seq_lengths=seq,
-                                       ssm_state_indices=idx, g=gate)
+    o = launches("gdn_fused", lambda: ops.recurrent_gated_delta_rule(
+        q, k, v, state, beta=beta, scale=D ** -0.5, actual_seq_lengths=seq, ssm_state_indices=idx, g=gate))
     torch.cuda.synchronize()
     assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(state).all())
+    # the token-by-token kernel on the same call (what the operator runs for short sequences)
+    state_tok = state0.clone()
+    with token_by_token():
+        o_tok = launches("recurrent_gdn", lambda: ops.recurrent_gated_delta_rule(
+            q, k, v, state_tok, beta=beta, scale=D ** -0.5, actual_seq_lengths=seq, ssm_state_indices=idx, g=gate))
+    assert_close(o, o_tok.float(), TOL_BF16, "chunk kernels vs token-by-token kernel, out")
+    assert_close(state, state_tok, 2 * TOL_STATE, "chunk kernels vs token-by-token kernel, state")
     one = torch.tensor([0, 0], dtype=torch.int32)
     for n in range(NSEQ):
         s, e = cu[n], cu[n + 1]
@@ -180,7 +222,9 @@ def test_varlen_prefill_benchmark_shape(dev):
         o_n = ops.recurrent_gated_delta_rule(q[s:e], k[s:e], v[s:e], st, beta=beta[s:e], scale=D ** -0.5,
                                              actual_seq_lengths=one.to(dev),
                                              ssm_state_indices=torch.zeros(e - s, dtype=torch.int32, device=dev), g=gate[s:e])
-        assert torch.equal(o_n, o[s:e]) and torch.equal(st[0], state[n]), f"sequence {n} differs from the packed run"
+        # (the chunk kernels pick their slab width by the size of the batch: the same products in another order)
+        assert_close(o_n, o[s:e], 1e-2, f"sequence {n} on its own, out")
+        assert_close(st[0], state[n], 1e-5, f"sequence {n} on its own, state")
     order = torch.argsort(lens).tolist()
     for n in (order[0], order[NSEQ // 2], order[-1]):
         s, e = cu[n], cu[n + 1]
@@ -191,14 +235,45 @@ def test_varlen_prefill_benchmark_shape(dev):
             ssm_state_indices=torch.zeros(e - s, dtype=torch.int32), g=c(gate))
         assert_close(o[s:e], o_ref, TOL_BF16, f"out of sequence {n} ({e - s} tokens)")
         assert_close(state[n:n + 1], s_ref, TOL_STATE, f"state of sequence {n}")
-    # (c) the chunked forward on the same packed tokens (strided head-major views, the pool rows transposed into its
-    # [N,H,K,V] state) agrees with the token-by-token kernel on every sequence
-    from fla_hip import pipeline
-    hm = lambda t: t.transpose(0, 1)[None]
-    o_c, fin = pipeline.flash_gated_delta_rule(hm(q), hm(k), hm(v), gate[None], beta[None].float(), D ** -0.5,
-                                               state0.transpose(-1, -2).contiguous(), True, cu_seqlens=cu)
-    assert_close(o_c[0], o.float(), TOL_BF16, "chunked forward vs recurrent kernel, out")
-    assert_close(fin.transpose(-1, -2), state, 2 * TOL_STATE, "chunked forward vs recurrent kernel, state")
+        o_ref_t, s_ref_t = o_tok[s:e], state_tok[n:n + 1]
+        assert_close(o_ref_t, o_ref, TOL_BF16, f"token-by-token kernel, out of sequence {n}")
+        assert_close(s_ref_t, s_ref, TOL_STATE, f"token-by-token kernel, state of sequence {n}")
+
+
+def test_prefill_route_keeps_the_operator_contract(dev):
+    """Which calls leave the token-by-token kernel, and what they write: a skipped prefix, an empty sequence, a bf16
+    pool, slots in arbitrary order and untouched slots of the pool; slots that change inside a sequence, slots shared by
+    two sequences, a key-wise gate and accepted-token counts stay on the token-by-token kernel."""
+    from fla_hip import ops
+    lens = [100, 0, 333, 64]
+    d = make_inputs(lens, 2, 4, 128, 128, seed=5, skip=3, blocks=9)
+    slots = [7, 2, 0, 5]
+    d["idx"] = torch.cat([torch.zeros(3, dtype=torch.int32)] +
+                         [torch.full((n,), s, dtype=torch.int32) for n, s in zip(lens, slots)])
+    to = lambda t: None if t is None else t.to(dev)
+    for pool_dtype, tol in ((torch.float32, TOL_STATE), (BF, TOL_BF16)):
+        pool = d["state"].to(pool_dtype)
+        o_ref, s_ref = od.recurrent_gated_delta_rule(d["q"], d["k"], d["v"], pool.float(), beta=d["beta"], scale=d["scale"],
+                                                     actual_seq_lengths=d["lens"], ssm_state_indices=d["idx"], g=d["g"])
+        st = pool.to(dev)
+        o = launches("gdn_fused", lambda: ops.recurrent_gated_delta_rule(
+            to(d["q"]), to(d["k"]), to(d["v"]), st, beta=to(d["beta"]), scale=d["scale"], actual_seq_lengths=to(d["lens"]),
+            ssm_state_indices=to(d["idx"]), g=to(d["g"])))
+        assert_close(o[3:], o_ref[3:], TOL_BF16, "out")
+        assert_close(st, s_ref.to(pool_dtype), tol, "pool")
+        untouched = [b for b in range(9) if b not in (7, 0, 5)]
+        assert torch.equal(st[untouched].cpu(), pool[untouched]), "slots of no sequence must keep their contents"
+    # not a prefill in the sense of the route
+    changing = d["idx"].clone()
+    changing[50] = 8
+    shared = d["idx"].clone()
+    shared[d["idx"] == 5] = 7
+    for what, idx, extra in (("changing", changing, {}), ("shared", shared, {}),
+                             ("accepted", d["idx"], dict(num_accepted_tokens=torch.tensor([1, 1, 1, 1], dtype=torch.int32)))):
+        st = d["state"].to(dev)
+        launches("recurrent_gdn", lambda: ops.recurrent_gated_delta_rule(
+            to(d["q"]), to(d["k"]), to(d["v"]), st, beta=to(d["beta"]), scale=d["scale"], actual_seq_lengths=to(d["lens"]),
+            ssm_state_indices=to(idx), g=to(d["g"]), **{k_: to(v_) for k_, v_ in extra.items()}))
 
 
 def test_wrapper_errors(dev):
