@@ -139,8 +139,17 @@ int stage_to_device(void *dst, const void *src, size_t bytes, hipStream_t stream
     Slot &s = ring.slots[ring.next];
     ring.next = (ring.next + 1) % 16;
     if (s.busy) {
-        s.busy = false;   // cleared first: a failed wait must not wedge the slot for every later call
-        FLA_HIP_CHECK(hipEventSynchronize(s.ev));
+        s.busy = false;
+        if (hipEventSynchronize(s.ev) != hipSuccess) {
+            // The copy that was reading this slot's buffer may never have completed.  The buffer and the event are
+            // retired (dropped, not freed or reused: a stuck copy may still read the memory) and the slot starts
+            // again with fresh ones on its next use, so that no later call writes into memory a copy still reads.
+            (void)hipGetLastError();
+            s.host = nullptr;
+            s.cap = 0;
+            s.ev = nullptr;
+            return fail(FLA_ERR_LAUNCH, "waiting for an earlier upload of host integer arrays failed.");
+        }
     }
     if (s.cap < bytes) {
         if (s.host) FLA_HIP_CHECK(hipHostFree(s.host));

@@ -1680,12 +1680,20 @@ static __device__ __align__(256) unsigned char scratch[FLA_CHUNK_KDA_FWD_NOALLOC
 std::mutex g_scratch_mu;
 void *g_scratch_ptr[16] = {};   // device address of `scratch` per device, resolved on the first call there
 
-int scratch_address(void **out) {
+// The address is resolved on the first call on a device.  That call must not come while `stream` is being captured
+// (a symbol lookup is no stream operation; inside a capture it is refused here rather than tried): one call outside
+// the capture - fla_chunk_kda_fwd_noalloc itself, or fla_chunk_kda_fwd_noalloc_init - comes first.
+int scratch_address(void **out, hipStream_t stream) {
     int dev = 0;
     FLA_HIP_CHECK(hipGetDevice(&dev));
     FLA_REQUIRE(dev >= 0 && dev < 16, FLA_ERR_UNSUPPORTED, "chunk_kda_fwd_noalloc: device index %d out of range.", dev);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     if (g_scratch_ptr[dev] == nullptr) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (stream != nullptr && hipStreamIsCapturing(stream, &capturing) == hipSuccess)
+            FLA_REQUIRE(capturing == hipStreamCaptureStatusNone, FLA_ERR_UNSUPPORTED,
+                        "chunk_kda_fwd_noalloc: the first call on a device resolves the scratch array's address and must "
+                        "come before stream capture (call fla_chunk_kda_fwd_noalloc_init once).");
         void *ptr = nullptr;
         FLA_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         FLA_REQUIRE(ptr != nullptr, FLA_ERR_LAUNCH, "chunk_kda_fwd_noalloc: the scratch array has no device address.");
@@ -1698,6 +1706,13 @@ int scratch_address(void **out) {
 }  // namespace
 }  // namespace fla
 
+extern "C" int fla_chunk_kda_fwd_noalloc_init(void) {
+    return fla::guarded([&] {
+        void *ptr = nullptr;
+        return fla::scratch_address(&ptr, nullptr);
+    });
+}
+
 extern "C" int fla_chunk_kda_fwd_noalloc(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *beta,
     const fla_tensor *A_log, const fla_tensor *dt_bias, const fla_tensor *initial_state, const fla_int_array *cu_seqlens,
@@ -1706,38 +1721,40 @@ extern "C" int fla_chunk_kda_fwd_noalloc(
     const fla_tensor *final_state, const fla_tensor *gk, const fla_tensor *Aqk, const fla_tensor *Akk, const fla_tensor *w,
     const fla_tensor *u, const fla_tensor *qg, const fla_tensor *kg, const fla_tensor *v_new, const fla_tensor *h,
     void *stream) {
-    const char *op = "chunk_kda_fwd_noalloc";
-    // packed batches upload their chunk table through a pinned staging ring that grows on demand
-    if ((cu_seqlens && cu_seqlens->data && cu_seqlens->size) || (chunk_indices && chunk_indices->data && chunk_indices->size))
-        return fla::fail(FLA_ERR_UNSUPPORTED, "%s: cu_seqlens / chunk_indices are not accepted (their upload allocates "
-                         "pinned staging memory); use fla_chunk_kda_fwd.", op);
-    const bool f16 = q != nullptr && q->dtype == FLA_F16;
-    uint64_t need = 0;
-    int rc = f16 ? fla_chunk_kda_fwd_get_workspace_size_f16(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr,
-                                                           layout, scale, chunk_size, safe_gate, lower_bound,
-                                                           use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk,
-                                                           Akk, w, u, qg, kg, v_new, h, &need)
-                 : fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale,
-                                     chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out,
-                                     final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, &need);
-    if (rc) return rc;
-    if (need > (uint64_t)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES)
-        return fla::fail(FLA_ERR_WORKSPACE,
-                         "%s: this call needs %llu bytes of scratch, the fixed array holds %llu; pass w, u, qg and kg "
-                         "(1 KiB per token and head at K=V=128 otherwise; the fp16 copies of u and kg that the state "
-                         "scan reads stay in the scratch with bf16 elements, 512 B) or use fla_chunk_kda_fwd with a "
-                         "workspace.",
-                         op, (unsigned long long)need, (unsigned long long)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES);
-    void *ptr = nullptr;
-    if ((rc = fla::scratch_address(&ptr))) return rc;
-    if (f16)
-        return fla_chunk_kda_fwd_f16(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale,
-                                     chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out,
-                                     final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, ptr,
-                                     FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES, stream);
-    return fla::guarded([&] { return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale, chunk_size,
-                             safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk,
-                             w, u, qg, kg, v_new, h, ptr, FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES,
-                             static_cast<hipStream_t>(stream), nullptr); });
+    return fla::guarded([&]() -> int {
+        const char *op = "chunk_kda_fwd_noalloc";
+        // packed batches upload their chunk table through a pinned staging ring that grows on demand
+        if ((cu_seqlens && cu_seqlens->data && cu_seqlens->size) || (chunk_indices && chunk_indices->data && chunk_indices->size))
+            return fla::fail(FLA_ERR_UNSUPPORTED, "%s: cu_seqlens / chunk_indices are not accepted (their upload allocates "
+                             "pinned staging memory); use fla_chunk_kda_fwd.", op);
+        const bool f16 = q != nullptr && q->dtype == FLA_F16;
+        uint64_t need = 0;
+        int rc = f16 ? fla_chunk_kda_fwd_get_workspace_size_f16(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr,
+                                                               layout, scale, chunk_size, safe_gate, lower_bound,
+                                                               use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk,
+                                                               Akk, w, u, qg, kg, v_new, h, &need)
+                     : fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale,
+                                         chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out,
+                                         final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, nullptr, 0, nullptr, &need);
+        if (rc) return rc;
+        if (need > (uint64_t)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES)
+            return fla::fail(FLA_ERR_WORKSPACE,
+                             "%s: this call needs %llu bytes of scratch, the fixed array holds %llu; pass w, u, qg and kg "
+                             "(1 KiB per token and head at K=V=128 otherwise; the fp16 copies of u and kg that the state "
+                             "scan reads stay in the scratch with bf16 elements, 512 B) or use fla_chunk_kda_fwd with a "
+                             "workspace.",
+                             op, (unsigned long long)need, (unsigned long long)FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES);
+        void *ptr = nullptr;
+        if ((rc = fla::scratch_address(&ptr, static_cast<hipStream_t>(stream)))) return rc;
+        if (f16)
+            return fla_chunk_kda_fwd_f16(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale,
+                                         chunk_size, safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out,
+                                         final_state, gk, Aqk, Akk, w, u, qg, kg, v_new, h, ptr,
+                                         FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES, stream);
+        return fla::kda_fwd_impl(q, k, v, g, beta, A_log, dt_bias, initial_state, nullptr, nullptr, layout, scale, chunk_size,
+                                 safe_gate, lower_bound, use_gate_in_kernel, state_v_first, attn_out, final_state, gk, Aqk, Akk,
+                                 w, u, qg, kg, v_new, h, ptr, FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES,
+                                 static_cast<hipStream_t>(stream), nullptr);
+    });
 }
 #endif  // !FLA_ELEM_F16

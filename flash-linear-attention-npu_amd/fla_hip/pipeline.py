@@ -151,8 +151,21 @@ def _autograd_function():
 
     class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         @staticmethod
-        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm):
+        def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused, l2norm,
+                    save_intermediates=True):
             q_rstd = k_rstd = None
+            if not save_intermediates:
+                # the reference's memory profile (examples/flash_gated_delta_rule.py:1084): only q, k, v, the cumulated
+                # gate, beta and the state are kept; w, u, h and v_new are recomputed by the backward (:913-951)
+                if l2norm:
+                    q, q_rstd = _raw.l2norm_fwd(q)
+                    k, k_rstd = _raw.l2norm_fwd(k)
+                gc, o, A, final = flash_chunk_gated_delta_rule_fwd(
+                    q, k, v, g, beta, scale, initial_state, output_final_state, cu, chunk_size, fused=fused)
+                ctx.save_for_backward(q, k, v, gc, beta, A, initial_state, q_rstd, k_rstd, None, None, None)
+                ctx.scale, ctx.cu, ctx.chunk_size = scale, cu, chunk_size
+                ctx.dtypes = (g.dtype, beta.dtype)
+                return o, final
             # examples/flash_gated_delta_rule.py:1047-1049.  The fused forward normalises the rows itself and writes
             # them with their rstd; the composed route runs l2norm_fwd (y comes back in the memory order of x).
             in_kernel = bool(l2norm and fused)
@@ -175,8 +188,9 @@ def _autograd_function():
             dq, dk, dv, db, dg, dh0 = flash_chunk_gated_delta_rule_bwd(
                 q, k, v, gc, beta, A, ctx.scale, initial_state, do.contiguous(),
                 None if dht is None else dht.contiguous(), ctx.cu, ctx.chunk_size,
-                saved=dict(h=h, v_new=v_new, w=w), qk_rstd=None if q_rstd is None else (q_rstd, k_rstd))
-            return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None, None
+                saved=None if h is None else dict(h=h, v_new=v_new, w=w),
+                qk_rstd=None if q_rstd is None else (q_rstd, k_rstd))
+            return dq, dk, dv, dg.to(ctx.dtypes[0]), db.to(ctx.dtypes[1]), None, dh0, None, None, None, None, None, None
 
     return ChunkGatedDeltaRuleFunction
 
@@ -187,9 +201,15 @@ _FUNCTION = None
 def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, initial_state=None,
                            output_final_state: bool = False, use_qk_l2norm_in_kernel: bool = False,
                            cu_seqlens=None, cu_seqlens_list=None, chunk_indices=None, chunk_indices_list=None,
-                           chunk_size: int = 64, head_first: bool = False, *, fused: bool = True):
+                           chunk_size: int = 64, head_first: bool = False, *, fused: bool = True,
+                           save_intermediates: bool = True):
     """Same checks, defaults and layouts as the reference entry: q,k [B,H,T,K], v [B,H,T,V],
-    g,beta [B,T,H]; returns (o [B,T,H,V], final_state [N,H,K,V] or None)."""
+    g,beta [B,T,H]; returns (o [B,T,H,V], final_state [N,H,K,V] or None).
+
+    ``save_intermediates`` (only matters when autograd records the call): True keeps h [B,H,NT,K,V], v_new and w of the
+    forward for the backward, which then skips their recomputation (about 0.5 ms of a 2.8 ms training step at
+    B=4, T=8192, H=32, d=128) at the price of roughly twice the activation memory per layer (h alone is 0.5 GB
+    there); False keeps what the reference keeps (q, k, v, g, beta, the state) and recomputes the rest."""
     import torch
 
     del chunk_indices, chunk_indices_list  # derived from cu_seqlens inside the library
@@ -247,7 +267,7 @@ def flash_gated_delta_rule(q, k, v, g, beta, scale: Optional[float] = None, init
     if _FUNCTION is None:
         _FUNCTION = _autograd_function()
     return _FUNCTION.apply(q, k, v, g, beta, float(scale), initial_state, output_final_state, cu, chunk_size, fused,
-                           bool(use_qk_l2norm_in_kernel))
+                           bool(use_qk_l2norm_in_kernel), bool(save_intermediates))
 
 
 # =============================================================================================
@@ -469,15 +489,23 @@ def chunk_kda(q, k, v, g, beta, scale: Optional[float] = None, initial_state=Non
     # The chunk size tiles the same function.  The gradient kernels are built for 64-token tiles, as the reference's own
     # backward kernel is (npu_chunk_kda_bwd_intra, _aclnn_ctypes.py:1582-1584), so a differentiated call runs on them.
     chunk_size = 64
+    if layout not in ("BSND", "BNSD", "TND", "NTD"):
+        raise RuntimeError("chunk_kda: layout must be uppercase and one of BSND, BNSD, TND, NTD.")
     K, V = q.shape[-1], v.shape[-1]
     if K < 16 or K > 256 or K % 16 or V < 16 or V > 256 or V % 16:      # _aclnn_ctypes.py:1141
         raise RuntimeError("chunk_kda: K/V must be multiples of 16 with K,V <= 256.")
     gate_args = ()
     if use_gate_in_kernel:
-        if A_log is None:
+        # the operator's own checks (_aclnn_ctypes.py:1150-1165), ahead of the choice of route: a call is accepted or
+        # rejected alike whether or not it asks for gradients and whatever its head size
+        HV = v.shape[{"BSND": 2, "BNSD": 1, "TND": 1, "NTD": 0}[layout]]
+        if A_log is None or tuple(A_log.shape) != (HV,) or A_log.dtype != torch.float32:
             raise RuntimeError("chunk_kda: A_log must be float32 [HV] when use_gate_in_kernel=True.")
-        if (K, V) in ((64, 64), (64, 128), (128, 128)) and A_log.dtype == torch.float32 and \
-                (dt_bias is None or dt_bias.dtype == torch.float32):
+        if dt_bias is not None and (tuple(dt_bias.shape) != (HV * K,) or dt_bias.dtype != torch.float32):
+            raise RuntimeError("chunk_kda: dt_bias must be float32 [HV*K].")
+        if safe_gate and not (-5.0 <= lower_bound < 0.0):
+            raise RuntimeError("chunk_kda: lower_bound must be in [-5, 0) for safe gate.")
+        if (K, V) in ((64, 64), (64, 128), (128, 128)):
             # a built head size: the forward kernel activates the gate, kda_gate_bwd differentiates the activation
             gate_args = (A_log, dt_bias, bool(safe_gate), lower_bound)
         else:   # the activation as tensor operations ahead of the padding and the split below

@@ -387,12 +387,18 @@ int fla_chunk_kda_fwd(
  * pair.  The per-chunk decay rows and whichever of w, u, qg, kg the caller passes as NULL live
  * in a fixed array of FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES in device memory, one per GPU,
  * held until the process ends.  A call whose scratch need exceeds the array returns
- * FLA_ERR_WORKSPACE (with w, u, qg, kg supplied the need is B*NT*HV*K*4 bytes); cu_seqlens and
- * chunk_indices must be NULL (FLA_ERR_UNSUPPORTED otherwise).  The call performs no hipMalloc /
- * hipFree / hipHostMalloc.  All calls on one GPU share the array: calls that may overlap in time
- * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ * FLA_ERR_WORKSPACE (with w, u, qg, kg supplied the need is B*NT*HV*K*4 bytes, plus, with bf16
+ * elements, the fp16 copies of u and kg that the state scan reads: 2 bytes per element of each);
+ * cu_seqlens and chunk_indices must be NULL (FLA_ERR_UNSUPPORTED otherwise).  The call performs no
+ * hipMalloc / hipFree / hipHostMalloc.  All calls on one GPU share the array: calls that may
+ * overlap in time on one GPU (different streams, different threads) race and must be serialised
+ * by the caller.  The array's device address is resolved by the first call on a device, which
+ * must not be made while `stream` is being captured (FLA_ERR_UNSUPPORTED then):
+ * fla_chunk_kda_fwd_noalloc_init(), called once per device with that device current, resolves it
+ * ahead of time; it launches nothing and allocates nothing.
  * ------------------------------------------------------------------------ */
 #define FLA_CHUNK_KDA_FWD_NOALLOC_SCRATCH_BYTES (32u << 20)
+int fla_chunk_kda_fwd_noalloc_init(void);
 int fla_chunk_kda_fwd_noalloc(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
     const fla_tensor *beta, const fla_tensor *A_log, const fla_tensor *dt_bias,

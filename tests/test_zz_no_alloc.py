@@ -86,3 +86,36 @@ def test_packed_batches_are_rejected(dev):
 
     with pytest.raises(RuntimeError, match="cu_seqlens"):
         _runtime.call_op_noalloc("chunk_kda_fwd_noalloc", raw.OP_ARGTYPES["chunk_kda_fwd"], build, o)
+
+
+def test_capture_and_replay(dev):
+    """The entry point under stream capture, which is what it is for: the scratch address is resolved ahead of the
+    capture (fla_chunk_kda_fwd_noalloc_init), one call is captured and the graph replayed with new contents in the same
+    input buffers, the program's own eager launches and synchronisations in between; every replay must equal the eager
+    result of fla_chunk_kda_fwd on the same inputs bit for bit."""
+    import fla_hip
+    from fla_hip import ops
+
+    assert fla_hip.load_library().fla_chunk_kda_fwd_noalloc_init() == 0
+    B, T, Hk, Hv, K, V = 1, 200, 2, 2, 128, 128
+    static = make(B, T, Hk, Hv, K, V, 11, dev)
+    kw = dict(layout="BSND", output_final_state=True)
+    run = lambda: ops.chunk_kda_fwd_noalloc(*static[:5], K ** -0.5, 64, initial_state=static[5], **kw)[:2]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_static, f_static = run()
+    for trial in range(3):
+        fresh = make(B, T, Hk, Hv, K, V, 20 + trial, dev)
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        want_o, want_f = ops.chunk_kda_fwd(*fresh[:5], K ** -0.5, 64, initial_state=fresh[5], **kw)[:2]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o_static, want_o) and torch.equal(f_static, want_f), f"replay {trial}"
