@@ -150,7 +150,7 @@ __device__ __forceinline__ elemx8 paired_frag(const elem *khS, int pk, const flo
 // diagonal block inverse and the off-diagonal solve of column block W) and later row tile W of w; wave W of role 1
 // owns row tile 3 - W of q k^T and later row tile W of u.  The two waves of a SIMD (W and 4 + W) together carry five
 // score tile products, as every other SIMD does.  W and ROLE are static so that the tile loops unroll.
-template <int K, int V, int W, int ROLE, bool C128>
+template <int K, int V, int W, int ROLE, bool C128, bool QGF>
 __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, elem *kS, elem *vS, elem *akS, elem *aqS,
                                            float *gS, float *aS, const float *bS, int len, int64_t row_base,
                                            int64_t dec_base, int half, const elem *vg, const elem *khS, const float *fS) {
@@ -292,7 +292,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
         const elemx8 k8 = *reinterpret_cast<const elemx8 *>(kS + r * pk + c8);
         const float br = bS[r];
         elemx8 qg8, kg8, kb8;
-        u32x4 kgf, qgf;
+        u32x4 kgf, qgf = {};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const f32x4 gg = lds4(gS + r * pg + c8 + 4 * h), gl = lds4(gS + kChunk * pg + c8 + 4 * h);
@@ -305,10 +305,12 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
                 c[e] = kk * br * eg;
             }
             const elemx4 a4 = cvt4(a), b4 = cvt4(b), c4 = cvt4(c);
-            kgf[2 * h] = cvt2_fine(b[0], b[1]);
-            kgf[2 * h + 1] = cvt2_fine(b[2], b[3]);
-            qgf[2 * h] = cvt2_fine(a[0], a[1]);
-            qgf[2 * h + 1] = cvt2_fine(a[2], a[3]);
+            kgf[2 * h] = cvt2_fine_bounded(b[0], b[1]);
+            kgf[2 * h + 1] = cvt2_fine_bounded(b[2], b[3]);
+            if constexpr (QGF) {
+                qgf[2 * h] = cvt2_fine_bounded(a[0], a[1]);
+                qgf[2 * h + 1] = cvt2_fine_bounded(a[2], a[3]);
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 qg8[4 * h + e] = a4[e];
@@ -317,7 +319,7 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
             }
         }
         if (r < len) {
-            *reinterpret_cast<u32x4 *>(p.qg + (row_base + r) * K + c8) = p.qg_fine ? qgf : __builtin_bit_cast(u32x4, qg8);
+            *reinterpret_cast<u32x4 *>(p.qg + (row_base + r) * K + c8) = QGF ? qgf : __builtin_bit_cast(u32x4, qg8);
             *reinterpret_cast<u32x4 *>(p.kg16 + (row_base + r) * K + c8) = kgf;
             if constexpr (!kFineIsElem) {
                 if (p.kg != nullptr) *reinterpret_cast<elemx8 *>(p.kg + (row_base + r) * K + c8) = kg8;
@@ -416,8 +418,9 @@ __device__ __forceinline__ void intra_wave(const KdaIntraParams &p, elem *qS, el
 }
 
 // C128: the workgroup owns one half of a 128-token chunk (a template flag, so that the 64-token form carries none of
-// the second gate stream, the coupling operands or the zero fill).
-template <int K, int V, bool C128>
+// the second gate stream, the coupling operands or the zero fill).  QGF: qg is written as `fine` values (a template
+// flag as well: as a run-time choice the second conversion cost the kernel 0.04 ms of 0.36 at B=2, T=8192, H=32).
+template <int K, int V, bool C128, bool QGF>
 __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intra_kernel(const KdaIntraParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     using S = IntraSmem<K, V>;
@@ -575,14 +578,14 @@ __global__ void __launch_bounds__(kIntraThreads) FLA_TWO_WAVES_PER_SIMD kda_intr
 
     const int64_t dec_base = half ? -1 : (((int64_t)b * p.geom.NT + c) * p.geom.Hv + hv) * K;
     switch (wave_id()) {
-        case 0: intra_wave<K, V, 0, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 1: intra_wave<K, V, 1, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 2: intra_wave<K, V, 2, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 3: intra_wave<K, V, 3, 0, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 4: intra_wave<K, V, 0, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 5: intra_wave<K, V, 1, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        case 6: intra_wave<K, V, 2, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
-        default: intra_wave<K, V, 3, 1, C128>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 0: intra_wave<K, V, 0, 0, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 1: intra_wave<K, V, 1, 0, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 2: intra_wave<K, V, 2, 0, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 3: intra_wave<K, V, 3, 0, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 4: intra_wave<K, V, 0, 1, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 5: intra_wave<K, V, 1, 1, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        case 6: intra_wave<K, V, 2, 1, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
+        default: intra_wave<K, V, 3, 1, C128, QGF>(p, qS, kS, vS, akS, aqS, gS, aS, bS, len, row_base, dec_base, half, vg, khS, fS); break;
     }
 
     {
@@ -837,11 +840,15 @@ template <int K> struct ScanSmem {
 // (kg already carries 2^{g_last - g} up to the end of the whole chunk).
 // QF: qg holds `fine` values (the forward of a training step keeps it so for the reverse scan) and meets a `fine` copy
 // of the state.
-template <int K, int SUB, bool QF>
-__global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
+// VS: value columns per workgroup, 64 or 32 (VS / 16 compute waves in front of the four copying waves).  Every compute
+// wave reads the whole w, qg and kg tiles for its 16 columns, so a workgroup's step is bound by its LDS traffic; when
+// 64-column slabs leave compute units without a workgroup, 32-column slabs put half of that traffic on twice as many
+// units (the slabs of a head share an XCD, so the tiles still come from memory once).
+template <int K, int SUB, bool QF, int VS>
+__global__ void __launch_bounds__((VS / 16 + 4) * 64) kda_scan_kernel(const KdaScanParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
     typedef ScanSmem<K> L;
-    constexpr int VS = 64;
+    constexpr int CW = VS / 16;   // compute waves
     constexpr int pw = L::pw, pt = L::pt, pu = L::pu, pb = L::pb, ph = L::ph;
     constexpr int KT = K / 16, KS = K / 32;
 
@@ -861,9 +868,9 @@ __global__ void __launch_bounds__(512) kda_scan_kernel(const KdaScanParams p) {
     elem *hS = reinterpret_cast<elem *>(smem + L::h_off);
     const bool stage_h = p.h != nullptr && !p.v_first;   // uniform: both groups run the second barrier or neither
 
-    if (wave_id() >= 4) {
+    if (wave_id() >= CW) {
         // ------------------------------- loader waves -------------------------------------------
-        const int tid = threadIdx.x - kThreads;
+        const int tid = threadIdx.x - CW * 64;
         // The tiles of two steps are in flight at once: while step c is computed, those of step c + 1 are committed to
         // LDS and those of step c + 2 are on their way into the other register set, so that a load has two steps
         // to arrive.  Past the last step the loads re-read the last one (never committed), which keeps the number of
@@ -1367,12 +1374,12 @@ int head_major(const char *op, const char *name, const fla_tensor *t, bool rank3
 inline bool present(const fla_tensor *t) { return t != nullptr && t->data != nullptr; }
 inline size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
-template <int K, int V, bool C128>
+template <int K, int V, bool C128, bool QGF>
 int launch_intra_kernel(const KdaIntraParams &p, hipStream_t stream) {
     const size_t smem = IntraSmem<K, V>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V, C128>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_intra_kernel<K, V, C128, QGF>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V, C128>), chunk_head_grid(p.geom, p.geom.NT * (C128 ? 2 : 1), p.geom.Hv),
+    FLA_LAUNCH("kda_intra", stream, (kda_intra_kernel<K, V, C128, QGF>), chunk_head_grid(p.geom, p.geom.NT * (C128 ? 2 : 1), p.geom.Hv),
                dim3(kIntraThreads), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
@@ -1380,7 +1387,17 @@ int launch_intra_kernel(const KdaIntraParams &p, hipStream_t stream) {
 
 template <int K, int V>
 int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
-    const int rc = p.c128 ? launch_intra_kernel<K, V, true>(p, stream) : launch_intra_kernel<K, V, false>(p, stream);
+    int rc;
+    if (p.qg_fine) {
+        if constexpr (K <= 128 && !kFineIsElem) {
+            FLA_REQUIRE(!p.c128, FLA_ERR_UNSUPPORTED, "chunk_kda_fwd: a float16 qg beside other elements is built for chunk_size 64.");
+            rc = launch_intra_kernel<K, V, false, true>(p, stream);
+        } else {
+            return fail(FLA_ERR_UNSUPPORTED, "chunk_kda_fwd: a float16 qg beside other elements is built for K <= 128.");
+        }
+    } else {
+        rc = p.c128 ? launch_intra_kernel<K, V, true, false>(p, stream) : launch_intra_kernel<K, V, false, false>(p, stream);
+    }
     if (rc) return rc;
     if (p.c128) {
         KdaCrossParams cp{p.geom, p.x1, p.x2, p.w, p.aqk, p.akk, p.u16, p.u, p.scale};
@@ -1394,22 +1411,24 @@ int launch_intra(const KdaIntraParams &p, hipStream_t stream) {
     return FLA_OK;
 }
 
-template <int K, int SUB, bool QF>
+template <int K, int SUB, bool QF, int VS>
 int launch_scan_as(const KdaScanParams &p, hipStream_t stream) {
     const size_t smem = ScanSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K, SUB, QF>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kda_scan_kernel<K, SUB, QF, VS>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K, SUB, QF>), dim3(p.geom.V / 64, p.geom.Hv, p.geom.N), dim3(512), smem,
-               stream, p);
+    FLA_LAUNCH("kda_scan", stream, (kda_scan_kernel<K, SUB, QF, VS>), dim3(p.geom.V / VS, p.geom.Hv, p.geom.N),
+               dim3((VS / 16 + 4) * 64), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
 }
 template <int K, int SUB>
 int launch_scan(const KdaScanParams &p, hipStream_t stream) {
+    // 32-column slabs when 64-column ones leave compute units idle (see kda_scan_kernel)
+    const bool narrow = SUB == 1 && (int64_t)p.geom.N * p.geom.Hv * (p.geom.V / 64) < (int64_t)num_cus();
     if constexpr (!kFineIsElem) {
-        if (p.qg_fine) return launch_scan_as<K, SUB, true>(p, stream);
+        if (p.qg_fine) return narrow ? launch_scan_as<K, SUB, true, 32>(p, stream) : launch_scan_as<K, SUB, true, 64>(p, stream);
     }
-    return launch_scan_as<K, SUB, false>(p, stream);
+    return narrow ? launch_scan_as<K, SUB, false, 32>(p, stream) : launch_scan_as<K, SUB, false, 64>(p, stream);
 }
 
 template <int K, int SUB>

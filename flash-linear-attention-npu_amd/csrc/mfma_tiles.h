@@ -87,6 +87,12 @@ __device__ __forceinline__ unsigned cvt2_fine(float a, float b) {
     const f32x2 v = {__builtin_amdgcn_fmed3f(a, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(b, -65504.f, 65504.f)};
     return __builtin_bit_cast(unsigned, __builtin_convertvector(v, finex2));
 }
+// Without the saturation, for values bounded by an input of the caller: q and k times a decay factor <= 1 (the gated
+// operands qg, kg).  |q|, |k| beyond 65504 would turn into infinities here.
+__device__ __forceinline__ unsigned cvt2_fine_bounded(float a, float b) {
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(v, finex2));
+}
 __device__ __forceinline__ finex4 cvt4_fine(f32x4 v) {
     u32x2 t;
     t[0] = cvt2_fine(v[0], v[1]);
