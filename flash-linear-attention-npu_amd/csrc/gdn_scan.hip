@@ -562,12 +562,16 @@ __device__ __forceinline__ void t_tiles(const elem *kS, const elem *qS, const fl
 // FQ (per-channel gate only): q and k hold `fine` values (chunk_kda_fwd keeps qg and kg so for a training step) and meet
 // fp16 copies of d_o * scale and of the incoming gradient; the two products that carry the leading terms of dh then round
 // their operands to 11 bits instead of 8.
-template <int K, bool GK, bool DVL = false, bool FQ = false>
-__global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
+// VS: value columns per workgroup, 64 or 32 (VS / 16 compute waves in front of the four copying waves; 32 when 64 leave
+// compute units without a workgroup: every compute wave reads the whole k, q and w tiles for its 16 columns, so half the
+// columns are half the LDS traffic of a step).  The form that builds T deals its diagonal tiles to four compute waves.
+template <int K, bool GK, bool DVL = false, bool FQ = false, int VS = 64>
+__global__ void __launch_bounds__((VS / 16 + 4) * 64) bwd_dhu_kernel(const DhuParams p) {
     static_assert(!FQ || (GK && DVL), "fp16 q and k are built for the KDA form");
+    static_assert(VS == 64 || !(DVL && !GK), "the form that builds T itself needs four compute waves");
     extern __shared__ __align__(16) unsigned char smem[];
     typedef DhuSmem<K> L;
-    constexpr int VS = 64, CT = 1;
+    constexpr int CT = 1, CW = VS / 16;
     constexpr int pk = L::pk, pt = L::pt, pv = L::pv;
     constexpr int KT = K / 16, KS = K / 32;
     constexpr int ph = VS + 4;   // pitch of dh [K][VS] laid over the k tile: rows are 8-byte aligned
@@ -591,9 +595,9 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
     const elem *og = static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + slab * VS;
     const elem *vg = DVL ? nullptr : static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + slab * VS;
 
-    if (wave_id() >= 4) {
+    if (wave_id() >= CW) {
         // ------------------------------- loader waves -------------------------------------------
-        const int tid = threadIdx.x - kThreads;
+        const int tid = threadIdx.x - CW * 64;
         // Two register sets: while chunk c is computed, the tiles of chunk c - 1 are committed to LDS and those of
         // chunk c - 2 are on their way.  Before the first chunk the loads re-read it (never committed), so that the same
         // number of operations lies between a load and the commit that waits for it in every step.
@@ -694,7 +698,7 @@ __global__ void __launch_bounds__(512) bwd_dhu_kernel(const DhuParams p) {
             const float *gS = reinterpret_cast<const float *>(buf + L::g_off);
             const int len = min(kChunk, eos - (bos + c * kChunk));
             elem *tS = reinterpret_cast<elem *>(smem + L::t_off);
-            switch (wave_id() - 4) {   // the wave's tiles as constants: every operand read of the wave is issued at once
+            switch (wave_id() - CW) {   // the wave's tiles as constants: every operand read of the wave is issued at once
                 case 0: t_tiles<K, 0>(kS, qS, gS, tS, len, p.scale); break;
                 case 1: t_tiles<K, 1>(kS, qS, gS, tS, len, p.scale); break;
                 case 2: t_tiles<K, 2>(kS, qS, gS, tS, len, p.scale); break;
@@ -1112,14 +1116,24 @@ int launch_bwd_dhu_wide(const DhuParams &p, int slabs, hipStream_t stream) {
     return FLA_OK;
 }
 
-template <int K, bool GK, bool DVL = false, bool FQ = false>
-int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
+template <int K, bool GK, bool DVL, bool FQ, int VS>
+int launch_bwd_dhu_as(const DhuParams &p, hipStream_t stream) {
     const size_t smem = DVL ? DhuSmem<K>::bytes_dvl : DhuSmem<K>::bytes;
-    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK, DVL, FQ>),
+    FLA_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(bwd_dhu_kernel<K, GK, DVL, FQ, VS>),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK, DVL, FQ>), dim3(slabs, p.geom.Hv, p.geom.N), dim3(512), smem, stream, p);
+    FLA_LAUNCH("bwd_dhu", stream, (bwd_dhu_kernel<K, GK, DVL, FQ, VS>), dim3(p.geom.V / VS, p.geom.Hv, p.geom.N),
+               dim3((VS / 16 + 4) * 64), smem, stream, p);
     FLA_HIP_CHECK(hipGetLastError());
     return FLA_OK;
+}
+template <int K, bool GK, bool DVL = false, bool FQ = false>
+int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
+    // per-channel gate (the KDA forms): 32-column slabs when 64-column ones leave compute units idle
+    if constexpr (GK) {
+        if (p.sub == 1 && (int64_t)p.geom.N * p.geom.Hv * slabs < (int64_t)num_cus())
+            return launch_bwd_dhu_as<K, GK, DVL, FQ, 32>(p, stream);
+    }
+    return launch_bwd_dhu_as<K, GK, DVL, FQ, 64>(p, stream);
 }
 
 int bwd_dhu_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *dv,
