@@ -484,6 +484,326 @@ __global__ void __launch_bounds__(kThreads, 2) kda_bwd_wy_kernel(const KdaWyPara
     }
 }
 
+// =============================================================================
+// chunk_kda_bwd_dqkwg_wy: the two stages above for one (chunk, value head) in one workgroup
+// =============================================================================
+// Run one after the other, chunk_kda_bwd_dqkwg writes dk, dg (fp32) and dw, and chunk_kda_bwd_wy reads all three back,
+// adds to dk and dg and writes them again: 4 KB of the 9.5 KB the pair moves per token and head.  Here dw passes through
+// an LDS tile, and the x = Akk^T dw tiles land in the accumulator layout of the state part of dk (same row tile, same
+// column tiles per wave), so dk and dg are completed in registers and written once.  Eight waves: wave (w, half) owns
+// token rows 16w.. and one half of the column tiles of every result.  The tiles of the first stage make room for those of
+// the second as they die: dw over d_o, v over v_new, Akk over dh, the two 64 x 64 intermediates of the chain through the
+// inverse over q and the gate tile; k turns into k 2^g in place.
+struct KdaDqkwgWyParams {
+    ChunkGeom geom;
+    View4 q, k, v_new, d_o, dv2, v, akk, dv;   // dv2: the total gradient of v_new (= du); dv: result, gradient of v
+    View3 beta;
+    const float *gk;
+    int64_t g_sb, g_sh, g_st;
+    const elem *h, *dh;
+    int64_t h_sb, h_sh, h_sc, dh_sb, dh_sh, dh_sc;
+    ViewF dq, dk, dg, daqk, dakk;
+    float *db;
+    int64_t db_sb, db_sh, db_st;
+    float scale;
+};
+
+template <int K, int V>
+__global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const KdaDqkwgWyParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int pv = V + 8, pq = K + 8, pg = K + 4, pa = kChunk + 8;
+    constexpr int KT = K / 16, KTH = KT / 2, VTH = V / 32;   // column tiles per wave of the K- and V-sized results
+    constexpr int CPR = V / 8;
+    static_assert(K <= V, "the dw tile takes the place of the d_o tile");
+    elem *vS = reinterpret_cast<elem *>(smem);  // v_new, then v
+    elem *oS = vS + kChunk * pv;                // d_o, then dw [kChunk][pq]
+    elem *dvS = oS + kChunk * pv;               // dv2 = du
+    elem *hS = dvS + kChunk * pv;               // h, then dh, then Akk [kChunk][pa]
+    float *hdS = reinterpret_cast<float *>(hS + K * pv);
+    float *colS = hdS + K;                      // [4][K]; later beta [kChunk] and the two halves of dbeta [2][kChunk]
+    float *exS = colS + 4 * K;
+    elem *qS = reinterpret_cast<elem *>(exS + K);   // q, then the first intermediate of the chain through the inverse
+    elem *kS = qS + kChunk * pq;                    // k, then k 2^g
+    float *gS = reinterpret_cast<float *>(kS + kChunk * pq);   // gate, then the second intermediate
+    float *outS = reinterpret_cast<float *>(smem);
+    elem *dwS = oS, *aS = hS, *m4S = qS, *m5S = reinterpret_cast<elem *>(gS);
+    float *bS = colS, *dbS = colS + kChunk;
+    static_assert((size_t)kChunk * pa * 2 <= (size_t)K * pv * 2 && (size_t)kChunk * pa * 2 <= (size_t)kChunk * pq * 2 &&
+                      (size_t)kChunk * pa * 2 <= (size_t)kChunk * pg * 4 && 3 * kChunk <= 4 * K,
+                  "the tiles of the second stage must fit the dead tiles of the first");
+    static_assert((size_t)3 * kChunk * pg * 4 <= ((size_t)3 * kChunk * pv + (size_t)K * pv) * 2 + (size_t)6 * K * 4 +
+                                                     (size_t)2 * kChunk * pq * 2 + (size_t)kChunk * pg * 4,
+                  "the result tiles must fit the operand tiles");
+
+    int c, hv;
+    block_chunk_head(p.geom, c, hv);
+    const int b = blockIdx.z;
+    const int hk = hv / (p.geom.Hv / p.geom.Hk);
+    int seq, start, len;
+    chunk_span(p.geom, b, c, seq, start, len);
+    const int tid = threadIdx.x, w = wave_id() & 3, half = wave_id() >> 2, l = lane_id(), li = l & 15, lg = l >> 4;
+
+    // ---------------------------------- first stage: as kda_bwd_dqkwg_kernel -------------------------------------
+    const float *gg = p.gk + b * p.g_sb + hv * p.g_sh + (int64_t)start * p.g_st;
+    constexpr int GN = kChunk * (K / 4) / kDqkwgThreads;
+    f32x4 gpre[GN];
+#pragma unroll
+    for (int m = 0; m < GN; ++m) {
+        const int idx = m * kDqkwgThreads + tid;
+        const int r = min(idx / (K / 4), len - 1), c4 = (idx % (K / 4)) * 4;
+        gpre[m] = *reinterpret_cast<const f32x4 *>(gg + (int64_t)r * p.g_st + c4);
+    }
+    TileCopy<kDqkwgThreads, kChunk, K> tq, tk;
+    tq.fetch(static_cast<const elem *>(p.q.p) + b * p.q.sb + hk * p.q.sh + (int64_t)start * p.q.st, p.q.st, len, tid);
+    tk.fetch(static_cast<const elem *>(p.k.p) + b * p.k.sb + hk * p.k.sh + (int64_t)start * p.k.st, p.k.st, len, tid);
+    TileCopy<kDqkwgThreads, K, V> tdh;
+    {
+        TileCopy<kDqkwgThreads, kChunk, V> tv, to, tdv;
+        TileCopy<kDqkwgThreads, K, V> th;
+        tv.fetch(static_cast<const elem *>(p.v_new.p) + b * p.v_new.sb + hv * p.v_new.sh + (int64_t)start * p.v_new.st, p.v_new.st, len, tid);
+        to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st, p.d_o.st, len, tid);
+        tdv.fetch(static_cast<const elem *>(p.dv2.p) + b * p.dv2.sb + hv * p.dv2.sh + (int64_t)start * p.dv2.st, p.dv2.st, len, tid);
+        th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc, V, K, tid);
+        tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc, V, K, tid);
+#pragma unroll
+        for (int m = 0; m < GN; ++m) {
+            const int idx = m * kDqkwgThreads + tid;
+            *reinterpret_cast<f32x4 *>(gS + (idx / (K / 4)) * pg + (idx % (K / 4)) * 4) = gpre[m];
+        }
+        tq.commit(qS, pq, len, tid);
+        tk.commit(kS, pq, len, tid);
+        tv.commit(vS, pv, len, tid);
+        to.commit(oS, pv, len, tid);
+        tdv.commit(dvS, pv, len, tid);
+        th.commit(hS, pv, K, tid);
+#pragma unroll
+        for (int m = 0; m < TileCopy<kDqkwgThreads, K, V>::N; ++m) {
+            const elemx8 a = __builtin_bit_cast(elemx8, th.r[m]), d = __builtin_bit_cast(elemx8, tdh.r[m]);
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)d[e];
+            s = group_sum<CPR>(s);
+            const int idx = m * kDqkwgThreads + tid;
+            if (idx % CPR == 0) hdS[idx / CPR] = s;
+        }
+    }
+    __syncthreads();
+    {   // dAqk[i][j] = scale <do_i, v_new_j>, j <= i
+        float *dag = p.daqk.p + b * p.daqk.sb + hv * p.daqk.sh + (int64_t)start * p.daqk.st;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int ct = 2 * half + cc;
+            f32x4 acc = zero4();
+            if (ct <= w) {
+#pragma unroll
+                for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+            }
+            const int col = 16 * ct + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                if (row < len) dag[(int64_t)row * p.daqk.st + col] = (ct <= w && col <= row) ? acc[e] * p.scale : 0.f;
+            }
+        }
+    }
+    f32x4 dqa[KTH], dka[KTH], dwa[KTH];
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int cg = half * KTH + ct;
+        f32x4 a = zero4(), d = zero4();
+#pragma unroll
+        for (int j = 0; j < V / 32; ++j) {
+            const elemx8 hf = frag_kc(hS, pv, 16 * cg, 32 * j);
+            a = mfma16x32(frag_kc(oS, pv, 16 * w, 32 * j), hf, a);
+            d = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), hf, d);
+        }
+        dqa[ct] = a;
+        dwa[ct] = -d;
+    }
+    // the operands of the second stage are asked for now and land while the state-gradient product runs
+    TileCopy<kDqkwgThreads, kChunk, V> tvv;
+    TileCopy<kDqkwgThreads, kChunk, kChunk> ta;
+    tvv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st, p.v.st, len, tid);
+    ta.fetch(static_cast<const elem *>(p.akk.p) + b * p.akk.sb + hv * p.akk.sh + (int64_t)start * p.akk.st, p.akk.st, len, tid);
+    const float beta_own = tid < kChunk ? (tid < len ? load_scalar(p.beta, b, hv, start + tid) : 0.f) : 0.f;
+    __syncthreads();                 // every wave is done with h and d_o
+    tdh.commit(hS, pv, K, tid);
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) acc_to_tile(dwS, pq, 16 * w, 16 * (half * KTH + ct), dwa[ct]);   // dw, rounded as it is stored
+    __syncthreads();
+    float qv[KTH][4], kv[KTH][4], eg[KTH][4];
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int cg = half * KTH + ct, col = 16 * cg + li;
+        f32x4 d = zero4();
+#pragma unroll
+        for (int j = 0; j < V / 32; ++j) d = mfma16x32(frag_kc(vS, pv, 16 * w, 32 * j), frag_kc(hS, pv, 16 * cg, 32 * j), d);
+        const float gl = gS[(len - 1) * pg + col];
+        float colsum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            const float gv = gS[row * pg + col];
+            qv[ct][e] = (float)qS[row * pq + col];
+            kv[ct][e] = (float)kS[row * pq + col];
+            eg[ct][e] = ex2(gv);
+            dqa[ct][e] *= p.scale * eg[ct][e];
+            d[e] *= ex2(gl - gv);
+            colsum += row < len ? kv[ct][e] * d[e] : 0.f;
+        }
+        dka[ct] = d;
+        colsum += __shfl_xor(colsum, 16, kWave);
+        colsum += __shfl_xor(colsum, 32, kWave);
+        if (lg == 0) colS[w * K + col] = colsum;
+    }
+    __syncthreads();
+    if (tid < K) exS[tid] = colS[tid] + colS[K + tid] + colS[2 * K + tid] + colS[3 * K + tid] + ex2(gS[(len - 1) * pg + tid]) * hdS[tid];
+    __syncthreads();
+    float extra[KTH];
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) extra[ct] = exS[16 * (half * KTH + ct) + li];
+    // ---------------------------------- second stage: as kda_bwd_wy_kernel ----------------------------------------
+    // v_new, dh, q and the column sums are dead (the barrier above came after their last reads; extra is in registers)
+    tvv.commit(vS, pv, len, tid);
+    ta.commit(aS, pa, len, tid);
+    if (tid < kChunk) bS[tid] = beta_own;   // over the column sums, last read two barriers ago
+#pragma unroll
+    for (int m = 0; m < TileCopy<kDqkwgThreads, kChunk, K>::N; ++m) {   // k -> k 2^g, every thread its own pieces
+        const int idx = m * kDqkwgThreads + tid;
+        const int r = idx / (K / 8), c8 = (idx % (K / 8)) << 3;
+        const elemx8 a = *reinterpret_cast<const elemx8 *>(kS + r * pq + c8);
+        const f32x4 g0 = *reinterpret_cast<const f32x4 *>(gS + r * pg + c8), g1 = *reinterpret_cast<const f32x4 *>(gS + r * pg + c8 + 4);
+        f32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo[e] = r < len ? (float)a[e] * ex2(g0[e]) : 0.f;
+            hi[e] = r < len ? (float)a[4 + e] * ex2(g1[e]) : 0.f;
+        }
+        *reinterpret_cast<elemx8 *>(kS + r * pq + c8) = frag_from_acc(lo, hi);
+    }
+    __syncthreads();
+    // dA = strict_lower((dw (k 2^g)^T + du v^T) beta_col): row tile w, two column tiles per wave
+    f32x4 m4[2];
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+        const int ct = 2 * half + cc;
+        f32x4 acc = zero4();
+        if (ct <= w) {
+#pragma unroll
+            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pq, 16 * w, 32 * j), frag_kc(kS, pq, 16 * ct, 32 * j), acc);
+#pragma unroll
+            for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
+            const int col = 16 * ct + li;
+            const float bc = bS[col];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                acc[e] = (col < row && row < len) ? acc[e] * bc : 0.f;
+            }
+        }
+        m4[cc] = acc;
+    }
+    float br[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) br[e] = bS[16 * w + 4 * lg + e];
+    float db_row[4] = {0.f, 0.f, 0.f, 0.f};
+    const elemx8 at0 = frag_tr(aS, pa, 16 * w, 0), at1 = frag_tr(aS, pa, 16 * w, 32);
+    {   // y = Akk^T du: dv = y beta, dbeta += <y, v>
+        char *dvg = reinterpret_cast<char *>(static_cast<elem *>(const_cast<void *>(p.dv.p)) + b * p.dv.sb + hv * p.dv.sh +
+                                             (int64_t)start * p.dv.st);
+#pragma unroll
+        for (int cc = 0; cc < VTH; ++cc) {
+            const int ct = half * VTH + cc;
+            f32x4 acc = mfma16x32(at0, frag_tr(dvS, pv, 16 * ct, 0), zero4());
+            acc = mfma16x32(at1, frag_tr(dvS, pv, 16 * ct, 32), acc);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                db_row[e] += acc[e] * (float)vS[(16 * w + 4 * lg + e) * pv + 16 * ct + li];
+                acc[e] *= br[e];
+            }
+            acc_to_global(dvg + 32 * ct, p.dv.st * 2, 16 * w, len, acc);
+        }
+    }
+    f32x4 dga[KTH];
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {   // x = Akk^T dw in the layout of the state part of dk: dk += x 2^g beta, dg += that k
+        const int cg = half * KTH + ct;
+        f32x4 x = mfma16x32(at0, frag_tr(dwS, pq, 16 * cg, 0), zero4());
+        x = mfma16x32(at1, frag_tr(dwS, pq, 16 * cg, 32), x);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            const float xe = x[e] * eg[ct][e], add = xe * br[e];
+            db_row[e] += xe * kv[ct][e];
+            dga[ct][e] = qv[ct][e] * dqa[ct][e] - kv[ct][e] * dka[ct][e] + (row == len - 1 ? extra[ct] : 0.f) + add * kv[ct][e];
+            dka[ct][e] += add;
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float s_ = group_sum<16>(db_row[e]);
+        if (li == 0) dbS[half * kChunk + 16 * w + 4 * lg + e] = s_;
+    }
+    // dAkk = -strict_lower(Akk^T dA Akk^T) through two 64 x 64 tiles
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) acc_to_tile(m4S, pa, 16 * w, 16 * (2 * half + cc), m4[cc]);
+    __syncthreads();                 // dA complete; every wave is past the gate tile, which takes the second intermediate
+    if (tid < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + tid) * p.db_st] = dbS[tid] + dbS[kChunk + tid];
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {   // M5 = dA Akk^T
+        const int ct = 2 * half + cc;
+        f32x4 acc = zero4();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc = mfma16x32(frag_kc(m4S, pa, 16 * w, 32 * j), frag_kc(aS, pa, 16 * ct, 32 * j), acc);
+        acc_to_tile(m5S, pa, 16 * w, 16 * ct, acc);
+    }
+    __syncthreads();
+    {
+        float *dag = p.dakk.p + b * p.dakk.sb + hv * p.dakk.sh + (int64_t)start * p.dakk.st;
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int ct = 2 * half + cc;
+            f32x4 acc = zero4();
+            if (ct <= w) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (32 * j + 31 >= 16 * w) acc = mfma16x32(frag_tr(aS, pa, 16 * w, 32 * j), frag_tr(m5S, pa, 16 * ct, 32 * j), acc);
+            }
+            const int col = 16 * ct + li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                if (row < len) dag[(int64_t)row * p.dakk.st + col] = (ct <= w && col < row) ? -acc[e] : 0.f;
+            }
+        }
+    }
+    __syncthreads();   // every operand tile is dead: the results take their place
+#pragma unroll
+    for (int ct = 0; ct < KTH; ++ct) {
+        const int col = 16 * (half * KTH + ct) + li;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 16 * w + 4 * lg + e;
+            outS[row * pg + col] = dqa[ct][e];
+            outS[(kChunk + row) * pg + col] = dka[ct][e];
+            outS[(2 * kChunk + row) * pg + col] = dga[ct][e];
+        }
+    }
+    __syncthreads();
+    float *dst[3] = {p.dq.p + b * p.dq.sb + hv * p.dq.sh + (int64_t)start * p.dq.st,
+                     p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st,
+                     p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st};
+    const int64_t dst_st[3] = {p.dq.st, p.dk.st, p.dg.st};
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int m = 0; m < GN; ++m) {
+            const int idx = m * kDqkwgThreads + tid;
+            const int r = idx / (K / 4), c4 = (idx % (K / 4)) * 4;
+            if (r < len) *reinterpret_cast<f32x4 *>(dst[t] + (int64_t)r * dst_st[t] + c4) = *reinterpret_cast<const f32x4 *>(outS + (t * kChunk + r) * pg + c4);
+        }
+}
+
 // ---- host side ------------------------------------------------------------------------------------
 #define FLA_KDA_BWD_LAUNCH(KERNEL, NAME, GRID, SMEM_EXPR, P, THREADS)                                                     \
     do {                                                                                                               \
@@ -631,6 +951,60 @@ int kda_wy_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta
                 (long long)V);
 }
 
+int kda_dqkwg_wy_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+                      const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v,
+                      const fla_tensor *beta, const fla_tensor *akk, const fla_int_array *cu, const fla_int_array *ci, double scale,
+                      int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *daqk,
+                      const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dakk, void *ws, uint64_t ws_size,
+                      hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_kda_bwd_dqkwg_wy";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v_new, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if (d_o != nullptr && d_o->ndim == 4 && geom.Hv > 1 && geom.T <= (1 << 20)) geom.head_fast = d_o->stride[2] > d_o->stride[1] ? 1 : 0;
+    const int bf = dt_bit(kElemDtype);
+    const int64_t B = geom.B, Hk = geom.Hk, Hv = geom.Hv, T = geom.T, K = geom.K, V = geom.V;
+    if ((rc = check_bhtd(op, "q", q, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v_new", v_new, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv2", dv2, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "Akk", akk, B, Hv, T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, B, Hv, T, V, bf))) return rc;
+    FLA_REQUIRE(beta != nullptr && beta->data != nullptr, FLA_ERR_NULL, "%s: beta must be provided.", op);
+    if ((rc = check_bht(op, "beta", beta, B, Hv, T, kElemDtype))) return rc;
+    if ((rc = check_f32_bhtd(op, "gk", gk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dq", dq, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dk", dk, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dg", dg, B, Hv, T, K))) return rc;
+    if ((rc = check_f32_bhtd(op, "dAqk", daqk, B, Hv, T, kChunk))) return rc;
+    if ((rc = check_f32_bhtd(op, "dAkk", dakk, B, Hv, T, kChunk))) return rc;
+    if ((rc = check_tensor(db, op, "db", 3, dt_bit(FLA_F32)))) return rc;
+    FLA_REQUIRE(db->shape[0] == B && db->shape[1] == Hv && db->shape[2] == T, FLA_ERR_SHAPE, "%s: db must be [%lld,%lld,%lld].",
+                op, (long long)B, (long long)Hv, (long long)T);
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
+    if ((rc = check_state_blocks(op, "h", h, geom))) return rc;
+    if ((rc = check_state_blocks(op, "dh", dh, geom))) return rc;
+    if (query) return FLA_OK;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    KdaDqkwgWyParams p{geom, view4(q), view4(k), view4(v_new), view4(d_o), view4(dv2), view4(v), view4(akk), view4(dv), view3(beta),
+                       static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
+                       static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
+                       h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
+                       viewf(dq), viewf(dk), viewf(dg), viewf(daqk), viewf(dakk),
+                       static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2], (float)scale};
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
+    const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
+                        (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
+    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<128, 128>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 64>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
+    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 128>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(64,128).", op, (long long)K,
+                (long long)V);
+}
+
 }  // namespace
 }  // namespace fla
 
@@ -693,4 +1067,27 @@ FLA_ENTRY(fla_chunk_kda_bwd_wy)(
     FLA_ROUTE_F16(k, fla_chunk_kda_bwd_wy, k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace, workspace_size, stream);
     return fla::guarded([&] { return fla::kda_wy_impl(k, v, beta, gk, Akk, dw, du, cu_seqlens, chunk_indices, chunk_size, dk, dv, db, dg, dAkk, workspace,
                             workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_wy_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dAqk,
+    const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dAkk, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_wy_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dg, dAqk, dv, db, dAkk, workspace_size);
+    FLA_NULL_WS("chunk_kda_bwd_dqkwg_wy");
+    return fla::guarded([&] { return fla::kda_dqkwg_wy_impl(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale,
+                                  chunk_size, dq, dk, dg, dAqk, dv, db, dAkk, nullptr, 0, nullptr, workspace_size); });
+}
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_wy)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dAqk,
+    const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dAkk, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_wy, q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dg, dAqk, dv, db, dAkk, workspace, workspace_size, stream);
+    return fla::guarded([&] { return fla::kda_dqkwg_wy_impl(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale,
+                                  chunk_size, dq, dk, dg, dAqk, dv, db, dAkk, workspace, workspace_size,
+                                  static_cast<hipStream_t>(stream), nullptr); });
 }

@@ -77,6 +77,7 @@ OP_ARGTYPES = {
     "chunk_kda_bwd_dqkwg": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 5,
     "chunk_kda_bwd_dhu": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 3,
     "chunk_kda_bwd_wy": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 5,
+    "chunk_kda_bwd_dqkwg_wy": [_T] * 11 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 7,
 }
 
 
@@ -1004,6 +1005,38 @@ def chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw, du, dk, dg, chunk_size=64, *, cu_s
             ctx.tensor(dw, "dw"), ctx.tensor(du, "du"), ctx.int_array(cu), ctx.int_array(_as_int_tuple(chunk_indices)),
             ctypes.c_int64(int(chunk_size)), ctx.tensor(dk, "dk"), ctx.tensor(dv, "dv"), ctx.tensor(db, "db"),
             ctx.tensor(dg, "dg"), ctx.tensor(dA, "dAkk"),
+        ],
+        outs,
+    )
+    return outs
+
+
+def chunk_kda_bwd_dqkwg_wy(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, scale, chunk_size=64, *, cu_seqlens=None,
+                           chunk_indices=None, layout_like=None):
+    """``chunk_kda_bwd_dqkwg`` (with dAqk) followed by ``chunk_kda_bwd_wy`` in one launch: dw passes through on-chip memory
+    and dk, dg are completed in registers, so neither is written, read back, added to and written again.  Returns
+    ``(dq, dk, dg, dAqk, dv, db, dAkk)``: dq / dk / dg fp32 [B,Hv,T,K], dAqk / dAkk fp32 [B,Hv,T,64] and db fp32
+    [B,Hv,T] laid out like ``layout_like`` (default: like ``gk``), dv like ``v``.  Head sizes (K,V) in (128,128),
+    (64,64), (64,128), 64-token chunks."""
+    import torch
+
+    B, Hv, T, K = _shape(gk)
+    V = _shape(v)[-1]
+    like = gk if layout_like is None else layout_like
+    f32 = lambda d: _empty_strided_like((B, Hv, T, d), like, torch.float32, q.device)
+    dq, dk, dg, dAqk, dAkk = f32(K), f32(K), f32(K), f32(64), f32(64)
+    db = f32(1)[..., 0]
+    dv = _empty_strided_like((B, Hv, T, V), v, v.dtype)
+    cu = _as_int_tuple(cu_seqlens)
+    outs = (dq, dk, dg, dAqk, dv, db, dAkk)
+    _call_op(
+        "chunk_kda_bwd_dqkwg_wy", OP_ARGTYPES["chunk_kda_bwd_dqkwg_wy"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v_new, "v_new"), ctx.tensor(gk, "gk"), ctx.tensor(h, "h"),
+            ctx.tensor(d_o, "d_o"), ctx.tensor(dh, "dh"), ctx.tensor(dv2, "dv2"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"),
+            ctx.tensor(Akk, "Akk"), ctx.int_array(cu), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
+            *[ctx.tensor(t, n) for t, n in zip(outs, ("dq", "dk", "dg", "dAqk", "dv", "db", "dAkk"))],
         ],
         outs,
     )

@@ -337,9 +337,10 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
         # no pass for chunk_kda_bwd_dav: the reverse scan forms dv = Aqk^T do from the score blocks, the next stage writes
         # dAqk = scale tril(do v_new^T) from the do and v_new tiles it stages anyway
         dh, dh0, dv2 = _raw.chunk_kda_bwd_dhu(qg4, kg4, w4, doh, Aqk4, scale, chunk_size, gK=gk4, h0=initial_state, dht=dht, **kw)
-        dq, dk, dw, dg, dAqk = _raw.chunk_kda_bwd_dqkwg(qh, kh, vn4, gk4, h5, doh, dh, dv2, scale, chunk_size,
-                                                        layout_like=layout_like, with_dAqk=True, **kw)
-        dv, db, dAkk = _raw.chunk_kda_bwd_wy(kh, vh, bh, gk4, Akk4, dw, dv2, dk, dg, chunk_size, **kw)
+        # the state-dependent stage and the backward of the WY factors in one launch (chunk_kda_bwd_dqkwg and
+        # chunk_kda_bwd_wy as operators of their own write dk, dg and dw, read them back and write dk, dg again)
+        dq, dk, dg, dAqk, dv, db, dAkk = _raw.chunk_kda_bwd_dqkwg_wy(qh, kh, vn4, gk4, h5, doh, dh, dv2, vh, bh, Akk4, scale,
+                                                                     chunk_size, layout_like=layout_like, **kw)
     # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
     back = lambda t: _from_index_order(t, layout)
     if Hv == Hk:          # dq, dk are final with the last stage: it writes them in the dtype of q and k

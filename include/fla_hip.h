@@ -526,6 +526,26 @@ int fla_chunk_kda_bwd_wy(
     int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dg,
     const fla_tensor *dAkk, void *workspace, uint64_t workspace_size, void *stream);
 
+/* chunk_kda_bwd_dqkwg_wy: chunk_kda_bwd_dqkwg (with dAqk) and chunk_kda_bwd_wy of the same chunks in one launch, for
+ * the composition of the KDA backward: dw = -dv2 h^T passes from the first stage to the second through on-chip memory
+ * and dk, dg leave once, complete (as two operators they are written, read back, added to and written again).  dv2 is
+ * the total gradient of v_new (the dv2 of chunk_kda_bwd_dhu; du of the second stage), v and beta the forward's inputs,
+ * Akk its inverse blocks.  Results: dq, dk, dg f32 [B,Hv,T,K]; dAqk, dAkk f32 [B,Hv,T,64]; dv (element type,
+ * [B,Hv,T,V]); db f32 [B,Hv,T].  (K,V) in (128,128), (64,64), (64,128); chunk_size 64.  No counterpart in the reference. */
+int fla_chunk_kda_bwd_dqkwg_wy_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dAqk,
+    const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dAkk, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_dqkwg_wy(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dAqk,
+    const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dAkk, void *workspace, uint64_t workspace_size,
+    void *stream);
+
 /* ------------------------------------------------------------------------
  * l2norm_fwd / l2norm_bwd - the q/k normalisation of the chunk pipelines, which the reference
  * runs as Triton kernels (fla/ops/triton/triton_core/l2norm.py:131-224; called from

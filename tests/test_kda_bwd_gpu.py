@@ -140,6 +140,54 @@ def test_bwd_wy(dev, case):
         assert amax(torch.triu(blk[:, :, :e - s], 0)) == 0.0 and amax(blk[:, :, e - s:]) == 0.0
 
 
+@pytest.mark.parametrize("case", STAGE_CASES)
+def test_bwd_dqkwg_and_wy_in_one_launch(dev, case):
+    """chunk_kda_bwd_dqkwg_wy against the oracle's two stages run one after the other and against the two operators: dw
+    passes between the stages rounded to 16 bits in all three, so the fused launch and the two operators agree to the
+    last bits of their fp32 sums."""
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, Hk, Hv, K, V, cu = case
+    gen = torch.Generator().manual_seed(T + 3 * K)
+    NT = gdn.total_chunks(B, T, 64, cu)
+    q, k = rnd(gen, B, Hk, T, K, scale=0.3), rnd(gen, B, Hk, T, K, scale=0.3)
+    v_new, do, dv2, v = (rnd(gen, B, Hv, T, V) for _ in range(4))
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    gk = gate_cumsum(F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, cu)
+    h, dh = rnd(gen, B, Hv, NT, K, V, scale=0.5), rnd(gen, B, Hv, NT, K, V, scale=0.5)
+    Akk = torch.zeros(B, Hv, T, 64)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        L = e - s
+        Akk[b, :, s:e, :L] = torch.linalg.inv(torch.eye(L) + torch.tril(torch.randn(Hv, L, L, generator=gen) * 0.1, -1))
+    Akk = Akk.to(BF)
+    to = lambda *ts: [t.to(dev) for t in ts]
+    got = raw.chunk_kda_bwd_dqkwg_wy(*to(q, k, v_new, gk, h, do, dh, dv2, v, beta, Akk), 0.7, cu_seqlens=cu)
+    dq, dk, dg, dAqk, dv, db, dAkk = got
+    assert all(t.dtype == torch.float32 for t in (dq, dk, dg, dAqk, db, dAkk)) and dv.dtype == BF
+    # the oracle: stage one, dw rounded as the operators hand it over, stage two
+    dq_r, dk1_r, dw_r, dg1_r = kda.chunk_kda_bwd_dqkwg(q, k, v_new, gk, h, do, dh, dv2, 0.7, cu_seqlens=cu)
+    dk2_r, dv_r, db_r, dg2_r, dAkk_r = kda.chunk_kda_bwd_wy(k, v, beta, gk, Akk, dw_r.to(BF), dv2, cu_seqlens=cu)
+    dAqk_r, _ = kda.chunk_kda_bwd_dav(v_new, do, torch.zeros(B, Hv, T, 64, dtype=BF), 0.7, cu_seqlens=cu)
+    for name, a, e, rel in (("dq", dq, dq_r, 1e-3), ("dk", dk, dk1_r + dk2_r, 2e-3), ("dg", dg, dg1_r + dg2_r, 3e-3),
+                            ("dAqk", dAqk, dAqk_r, 1e-3), ("dv", dv, dv_r, REL), ("dbeta", db, db_r, 2e-3),
+                            ("dAkk", dAkk, dAkk_r, REL)):
+        close(a, e, name, rel)
+    # the two operators on the same operands
+    dq2, dk2, dw2, dg2, dAqk2 = raw.chunk_kda_bwd_dqkwg(*to(q, k, v_new, gk, h, do, dh, dv2), 0.7, cu_seqlens=cu, with_dAqk=True)
+    dv3, db3, dAkk3 = raw.chunk_kda_bwd_wy(*to(k, v, beta, gk, Akk), dw2, dv2.to(dev), dk2, dg2, cu_seqlens=cu)
+    assert torch.equal(dq, dq2) and torch.equal(dAqk, dAqk2) and torch.equal(dv, dv3) and torch.equal(dAkk, dAkk3)
+    for name, a, e in (("dk", dk, dk2), ("dg", dg, dg2), ("dbeta", db, db3)):
+        close(a, e, name + " against the two operators", 1e-5)
+    # results laid out token-major, h / dh sequence-major: views only, identical numbers
+    h_sm, dh_sm = h.transpose(1, 2).contiguous().to(dev), dh.transpose(1, 2).contiguous().to(dev)
+    like = torch.empty(B, T, Hv, K, device="meta").transpose(1, 2)
+    tm = lambda t: t.to(dev).transpose(1, 2).contiguous().transpose(1, 2)
+    out2 = raw.chunk_kda_bwd_dqkwg_wy(*to(q, k, v_new, gk), h_sm.transpose(1, 2), tm(do), dh_sm.transpose(1, 2), tm(dv2), tm(v),
+                                      *to(beta, Akk), 0.7, cu_seqlens=cu, layout_like=like)
+    assert out2[0].transpose(1, 2).is_contiguous() and out2[4].transpose(1, 2).is_contiguous()
+    for a, e in zip(out2, got):
+        assert torch.equal(a, e)
+
+
 # ---------------------------------------------------------------------------------------------
 # composition
 # ---------------------------------------------------------------------------------------------
