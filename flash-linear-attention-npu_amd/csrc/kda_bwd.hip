@@ -506,12 +506,37 @@ struct KdaDqkwgWyParams {
     float *db;
     int64_t db_sb, db_sh, db_st;
     float scale;
+    int out16;   // with the intra-chunk stage: dq and dk point at 16-bit elements (strides in elements)
 };
 
-template <int K, int V>
+// Bytes of LDS of the kernel below.  The first two stages live in the tiles of the first; the intra-chunk stage keeps q, k
+// and the gate to its end and needs the two masked 64 x 64 score gradients in fp32: with 128 channels they take the places
+// of v and of the state tile, with 64 channels (smaller tiles) they get room of their own behind the others.
+template <int K, int V, bool INTRA>
+constexpr size_t kda_bwd_fused_smem() {
+    const size_t base = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
+                        (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
+    if (!INTRA) return base;
+    const size_t tail = base + 2 * kChunk * 4;   // the two halves of dbeta
+    const size_t pair = (size_t)2 * kChunk * (kChunk + 4) * 4;
+    // the transposed copies of the score gradients take the dw and du tiles where those are large enough
+    return (K == 128 ? tail : tail + (size_t)kChunk * (K + 8) * 2 + pair) + (V == 128 ? 0 : pair);
+}
+
+// D[16x16] += A[16x4] B[4x16] in fp32: lane l holds A[l%16][l/16], B[l/16][l%16], D[4*(l/16)+e][l%16]
+__device__ __forceinline__ f32x4 mfma_f32(float a, float b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+// INTRA: chunk_kda_bwd_intra (with the reverse running sum of dg) follows in the same workgroup.  Its increments of dq, dk,
+// dg have the accumulator layout of the first two stages (wave (w, half): row tile w, one half of the channel tiles), so
+// they are added in registers; dAqk and dAkk stay on chip as fp32 tiles, and dq, dk, dg, dbeta are written once, final.
+template <int K, int V, bool INTRA>
 __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const KdaDqkwgWyParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int pv = V + 8, pq = K + 8, pg = K + 4, pa = kChunk + 8;
+    constexpr int pv = V + 8, pq = K + 8, pg = K + 4, pa = kChunk + 8, pf = kChunk + 4;
+    constexpr bool BIG = K == 128;
+    constexpr size_t kBase = kda_bwd_fused_smem<K, V, false>();
     constexpr int KT = K / 16, KTH = KT / 2, VTH = V / 32;   // column tiles per wave of the K- and V-sized results
     constexpr int CPR = V / 8;
     static_assert(K <= V, "the dw tile takes the place of the d_o tile");
@@ -526,8 +551,21 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
     elem *kS = qS + kChunk * pq;                    // k, then k 2^g
     float *gS = reinterpret_cast<float *>(kS + kChunk * pq);   // gate, then the second intermediate
     float *outS = reinterpret_cast<float *>(smem);
-    elem *dwS = oS, *aS = hS, *m4S = qS, *m5S = reinterpret_cast<elem *>(gS);
-    float *bS = colS, *dbS = colS + kChunk;
+    elem *dwS = oS, *aS = hS;
+    // the intermediates of the chain through the inverse: over q and the gate, or (q, k, gate kept) over dw and du
+    elem *m4S = INTRA ? oS : qS, *m5S = INTRA ? dvS : reinterpret_cast<elem *>(gS);
+    elem *kgS = !INTRA ? kS : BIG ? hS + kChunk * pa : reinterpret_cast<elem *>(smem + kBase + 2 * kChunk * 4);   // k 2^g
+    float *bS = colS, *dbS = INTRA ? reinterpret_cast<float *>(smem + kBase) : colS + kChunk;
+    float *aqS = BIG ? reinterpret_cast<float *>(vS) : reinterpret_cast<float *>(kgS + kChunk * pq);   // tril(dAqk) [kChunk][pf]
+    float *akS = BIG ? reinterpret_cast<float *>(hS) : aqS + kChunk * pf;                              // tril(dAkk)
+    // their transposes, for the product that contracts over the rows
+    float *aqT = V == 128 ? reinterpret_cast<float *>(oS) : reinterpret_cast<float *>(smem + kda_bwd_fused_smem<K, V, true>()) - 2 * kChunk * pf;
+    float *akT = V == 128 ? reinterpret_cast<float *>(dvS) : aqT + kChunk * pf;
+    static_assert(!INTRA || !BIG || ((size_t)kChunk * (pa + pq) * 2 <= (size_t)K * pv * 2 && (size_t)kChunk * pf * 4 <= (size_t)kChunk * pv * 2),
+                  "k 2^g behind Akk in the state tile, a score gradient in the v tile");
+    static_assert((size_t)kChunk * pa * 2 <= (size_t)kChunk * pv * 2, "an intermediate fits the dw and du tiles");
+    static_assert((size_t)3 * kChunk * pg * 4 <= ((size_t)3 * kChunk * pv + (size_t)K * pv) * 2 + (size_t)6 * K * 4 + (size_t)2 * kChunk * pq * 2,
+                  "the result tiles end before the gate tile, which holds the partial sums of the running sum of dg");
     static_assert((size_t)kChunk * pa * 2 <= (size_t)K * pv * 2 && (size_t)kChunk * pa * 2 <= (size_t)kChunk * pq * 2 &&
                       (size_t)kChunk * pa * 2 <= (size_t)kChunk * pg * 4 && 3 * kChunk <= 4 * K,
                   "the tiles of the second stage must fit the dead tiles of the first");
@@ -588,8 +626,9 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
         }
     }
     __syncthreads();
+    f32x4 daq[2];   // INTRA: this wave's two tiles of the masked dAqk, kept until their LDS tile is free
     {   // dAqk[i][j] = scale <do_i, v_new_j>, j <= i
-        float *dag = p.daqk.p + b * p.daqk.sb + hv * p.daqk.sh + (int64_t)start * p.daqk.st;
+        float *dag = INTRA ? nullptr : p.daqk.p + b * p.daqk.sb + hv * p.daqk.sh + (int64_t)start * p.daqk.st;
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
             const int ct = 2 * half + cc;
@@ -602,7 +641,9 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int row = 16 * w + 4 * lg + e;
-                if (row < len) dag[(int64_t)row * p.daqk.st + col] = (ct <= w && col <= row) ? acc[e] * p.scale : 0.f;
+                const float val = (ct <= w && col <= row) ? acc[e] * p.scale : 0.f;
+                if constexpr (INTRA) daq[cc][e] = row < len ? val : 0.f;
+                else if (row < len) dag[(int64_t)row * p.daqk.st + col] = val;
             }
         }
     }
@@ -679,7 +720,7 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
             lo[e] = r < len ? (float)a[e] * ex2(g0[e]) : 0.f;
             hi[e] = r < len ? (float)a[4 + e] * ex2(g1[e]) : 0.f;
         }
-        *reinterpret_cast<elemx8 *>(kS + r * pq + c8) = frag_from_acc(lo, hi);
+        *reinterpret_cast<elemx8 *>(kgS + r * pq + c8) = frag_from_acc(lo, hi);
     }
     __syncthreads();
     // dA = strict_lower((dw (k 2^g)^T + du v^T) beta_col): row tile w, two column tiles per wave
@@ -690,7 +731,7 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
         f32x4 acc = zero4();
         if (ct <= w) {
 #pragma unroll
-            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pq, 16 * w, 32 * j), frag_kc(kS, pq, 16 * ct, 32 * j), acc);
+            for (int j = 0; j < K / 32; ++j) acc = mfma16x32(frag_kc(dwS, pq, 16 * w, 32 * j), frag_kc(kgS, pq, 16 * ct, 32 * j), acc);
 #pragma unroll
             for (int j = 0; j < V / 32; ++j) acc = mfma16x32(frag_kc(dvS, pv, 16 * w, 32 * j), frag_kc(vS, pv, 16 * ct, 32 * j), acc);
             const int col = 16 * ct + li;
@@ -745,10 +786,18 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
         if (li == 0) dbS[half * kChunk + 16 * w + 4 * lg + e] = s_;
     }
     // dAkk = -strict_lower(Akk^T dA Akk^T) through two 64 x 64 tiles
+    if constexpr (INTRA) __syncthreads();   // every wave is done with dw, du, v and k 2^g
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) acc_to_tile(m4S, pa, 16 * w, 16 * (2 * half + cc), m4[cc]);
-    __syncthreads();                 // dA complete; every wave is past the gate tile, which takes the second intermediate
-    if (tid < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + tid) * p.db_st] = dbS[tid] + dbS[kChunk + tid];
+    if constexpr (INTRA) {
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) aqS[(16 * w + 4 * lg + e) * pf + 16 * (2 * half + cc) + li] = daq[cc][e];
+    }
+    __syncthreads();                 // dA complete; every wave is past the tile that takes the second intermediate
+    if constexpr (!INTRA)
+        if (tid < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + tid) * p.db_st] = dbS[tid] + dbS[kChunk + tid];
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {   // M5 = dA Akk^T
         const int ct = 2 * half + cc;
@@ -758,8 +807,20 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
         acc_to_tile(m5S, pa, 16 * w, 16 * ct, acc);
     }
     __syncthreads();
+    // third stage: CPL neighbouring channels per lane; its increments of dq, dk, dg by row e of the lane's four rows
+    constexpr int CPL = KTH;
+    typedef float gvec __attribute__((ext_vector_type(CPL)));
+    typedef elem kvec __attribute__((ext_vector_type(CPL)));
+    gvec incq[4], inck[4], incg[4];
+    if constexpr (INTRA) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int c_ = 0; c_ < CPL; ++c_) incq[e][c_] = inck[e][c_] = incg[e][c_] = 0.f;
+    }
+    f32x4 dak[2];
     {
-        float *dag = p.dakk.p + b * p.dakk.sb + hv * p.dakk.sh + (int64_t)start * p.dakk.st;
+        float *dag = INTRA ? nullptr : p.dakk.p + b * p.dakk.sb + hv * p.dakk.sh + (int64_t)start * p.dakk.st;
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
             const int ct = 2 * half + cc;
@@ -773,7 +834,94 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int row = 16 * w + 4 * lg + e;
-                if (row < len) dag[(int64_t)row * p.dakk.st + col] = (ct <= w && col < row) ? -acc[e] : 0.f;
+                const float val = (ct <= w && col < row) ? -acc[e] : 0.f;
+                if constexpr (INTRA) dak[cc][e] = row < len ? val : 0.f;
+                else if (row < len) dag[(int64_t)row * p.dakk.st + col] = val;
+            }
+        }
+    }
+    if constexpr (INTRA) {
+        // ------------------------- third stage: as kda_bwd_intra_kernel, for this wave's rows ----------------------
+        // Wave (w, half): rows 16w.., one half of the channels; a lane's accumulator columns are CPL neighbouring channels
+        // (cb + c in accumulator c), and step s of a 16-token tile contracts over tokens 4 lg + s, so that every operand
+        // is one wide LDS read: four steps of a score-gradient row, CPL channels of a k, q or gate row.
+        __syncthreads();             // every wave is done with Akk and both intermediates
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+            const int ct = 2 * half + cc;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) akS[(16 * w + 4 * lg + e) * pf + 16 * ct + li] = dak[cc][e];
+            *reinterpret_cast<f32x4 *>(aqT + (16 * ct + li) * pf + 16 * w + 4 * lg) = daq[cc];
+            *reinterpret_cast<f32x4 *>(akT + (16 * ct + li) * pf + 16 * w + 4 * lg) = dak[cc];
+        }
+        __syncthreads();
+        const int r0 = 16 * w, row_end = min(r0 + 16, len), anchor = min(r0 + 8, row_end - 1);
+        const int cb = half * (K / 2) + CPL * li;
+        if (r0 < len) {              // a row tile without a token (wave-uniform) adds nothing
+            const gvec ca = *reinterpret_cast<const gvec *>(gS + anchor * pg + cb);
+            f32x4 D1[CPL], D2[CPL], D3[CPL];
+#pragma unroll
+            for (int c_ = 0; c_ < CPL; ++c_) D1[c_] = D2[c_] = D3[c_] = zero4();
+            // padded rows of the tiles hold k = 0, a score gradient of 0 and the gate of the chunk's last token
+            for (int jt = 0; jt <= w; ++jt) {
+                const f32x4 a1 = *reinterpret_cast<const f32x4 *>(aqS + (r0 + li) * pf + 16 * jt + 4 * lg);
+                const f32x4 a2 = *reinterpret_cast<const f32x4 *>(akS + (r0 + li) * pf + 16 * jt + 4 * lg);
+#pragma unroll
+                for (int s_ = 0; s_ < 4; ++s_) {
+                    const int j = 16 * jt + 4 * lg + s_;
+                    const kvec kk = *reinterpret_cast<const kvec *>(kS + j * pq + cb);
+                    const gvec gg = *reinterpret_cast<const gvec *>(gS + j * pg + cb);
+#pragma unroll
+                    for (int c_ = 0; c_ < CPL; ++c_) {
+                        const float bval = (float)kk[c_] * ex2(ca[c_] - gg[c_]);
+                        D1[c_] = mfma_f32(a1[s_], bval, D1[c_]);
+                        D2[c_] = mfma_f32(a2[s_], bval, D2[c_]);
+                    }
+                }
+            }
+            for (int it = w; it < 4; ++it) {
+                const f32x4 a1 = *reinterpret_cast<const f32x4 *>(aqT + (r0 + li) * pf + 16 * it + 4 * lg);
+                const f32x4 a2 = *reinterpret_cast<const f32x4 *>(akT + (r0 + li) * pf + 16 * it + 4 * lg);
+#pragma unroll
+                for (int s_ = 0; s_ < 4; ++s_) {
+                    const int i = 16 * it + 4 * lg + s_;
+                    const kvec kk = *reinterpret_cast<const kvec *>(kS + i * pq + cb);
+                    const kvec qq = *reinterpret_cast<const kvec *>(qS + i * pq + cb);
+                    const gvec gg = *reinterpret_cast<const gvec *>(gS + i * pg + cb);
+                    const float bi = bS[i];
+#pragma unroll
+                    for (int c_ = 0; c_ < CPL; ++c_) {
+                        const float fw = ex2(gg[c_] - ca[c_]);
+                        D3[c_] = mfma_f32(a1[s_], (float)qq[c_] * fw, D3[c_]);
+                        D3[c_] = mfma_f32(a2[s_], (float)kk[c_] * bi * fw, D3[c_]);
+                    }
+                }
+            }
+            f32x4 dbacc = zero4();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = r0 + 4 * lg + e;
+                if (i < len) {
+                    const kvec kk = *reinterpret_cast<const kvec *>(kS + i * pq + cb);
+                    const kvec qq = *reinterpret_cast<const kvec *>(qS + i * pq + cb);
+                    const gvec gg = *reinterpret_cast<const gvec *>(gS + i * pg + cb);
+#pragma unroll
+                    for (int c_ = 0; c_ < CPL; ++c_) {
+                        const float up = ex2(gg[c_] - ca[c_]), down = ex2(ca[c_] - gg[c_]);
+                        const float dqd = D1[c_][e] * up, dl = D2[c_][e] * up, du = D3[c_][e] * down;
+                        const float qi = (float)qq[c_], ki = (float)kk[c_];
+                        const float bdl = br[e] * dl;
+                        incq[e][c_] = dqd;
+                        inck[e][c_] = bdl + du;
+                        incg[e][c_] = qi * dqd + ki * (bdl - du);
+                        dbacc[e] += dl * ki;
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float s_ = group_sum<16>(dbacc[e]);
+                if (li == 0) dbS[half * kChunk + r0 + 4 * lg + e] += s_;   // the lane that wrote the entry
             }
         }
     }
@@ -786,10 +934,69 @@ __global__ void __launch_bounds__(kDqkwgThreads) kda_bwd_dqkwg_wy_kernel(const K
             const int row = 16 * w + 4 * lg + e;
             outS[row * pg + col] = dqa[ct][e];
             outS[(kChunk + row) * pg + col] = dka[ct][e];
-            outS[(2 * kChunk + row) * pg + col] = dga[ct][e];
+            outS[(2 * kChunk + row) * pg + col] = INTRA && row >= len ? 0.f : dga[ct][e];
         }
     }
     __syncthreads();
+    if constexpr (INTRA) {
+        {   // the increments of the third stage, in its own assignment of channels to lanes
+            const int cb = half * (K / 2) + CPL * li;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = 16 * w + 4 * lg + e;
+                *reinterpret_cast<gvec *>(outS + row * pg + cb) += incq[e];
+                *reinterpret_cast<gvec *>(outS + (kChunk + row) * pg + cb) += inck[e];
+                *reinterpret_cast<gvec *>(outS + (2 * kChunk + row) * pg + cb) += incg[e];
+            }
+        }
+        __syncthreads();
+        if (tid < len) p.db[b * p.db_sb + hv * p.db_sh + (int64_t)(start + tid) * p.db_st] = dbS[tid] + dbS[kChunk + tid];
+        // dg is complete and a workgroup holds a whole chunk of it: the reverse running sum over the chunk's tokens is taken
+        // in the tile, a thread per column and run of rows, the runs joined through their totals
+        constexpr int SEGS = kDqkwgThreads / K, RS = kChunk / SEGS;
+        const int col = tid % K, seg = tid / K;
+        float *x0 = outS + 2 * kChunk * pg, *tot = gS;
+        float run = 0.f;
+#pragma unroll
+        for (int j = RS - 1; j >= 0; --j) {
+            float *x = x0 + (seg * RS + j) * pg + col;
+            run += *x;
+            *x = run;
+        }
+        tot[seg * K + col] = run;
+        __syncthreads();
+        float later = 0.f;
+#pragma unroll
+        for (int s2 = 1; s2 < SEGS; ++s2)
+            if (seg + s2 < SEGS) later += tot[(seg + s2) * K + col];
+#pragma unroll
+        for (int j = 0; j < RS; ++j) x0[(seg * RS + j) * pg + col] += later;
+        __syncthreads();
+        char *d16[2] = {reinterpret_cast<char *>(p.dq.p), reinterpret_cast<char *>(p.dk.p)};
+        const ViewF *vw[2] = {&p.dq, &p.dk};
+        const int64_t esz = p.out16 ? 2 : 4;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int m = 0; m < GN; ++m) {
+                const int idx = m * kDqkwgThreads + tid;
+                const int r = idx / (K / 4), c4 = (idx % (K / 4)) * 4;
+                if (r < len) {
+                    const f32x4 val = *reinterpret_cast<const f32x4 *>(outS + (t * kChunk + r) * pg + c4);
+                    char *at = d16[t] + (b * vw[t]->sb + hv * vw[t]->sh + (int64_t)(start + r) * vw[t]->st + c4) * esz;
+                    if (p.out16) *reinterpret_cast<elemx4 *>(at) = cvt4(val);
+                    else *reinterpret_cast<f32x4 *>(at) = val;
+                }
+            }
+        float *dgd = p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st;
+#pragma unroll
+        for (int m = 0; m < GN; ++m) {
+            const int idx = m * kDqkwgThreads + tid;
+            const int r = idx / (K / 4), c4 = (idx % (K / 4)) * 4;
+            if (r < len) *reinterpret_cast<f32x4 *>(dgd + (int64_t)r * p.dg.st + c4) = *reinterpret_cast<const f32x4 *>(x0 + r * pg + c4);
+        }
+        return;
+    }
     float *dst[3] = {p.dq.p + b * p.dq.sb + hv * p.dq.sh + (int64_t)start * p.dq.st,
                      p.dk.p + b * p.dk.sb + hv * p.dk.sh + (int64_t)start * p.dk.st,
                      p.dg.p + b * p.dg.sb + hv * p.dg.sh + (int64_t)start * p.dg.st};
@@ -994,13 +1201,73 @@ int kda_dqkwg_wy_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor
                        static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                        h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                        viewf(dq), viewf(dk), viewf(dg), viewf(daqk), viewf(dakk),
-                       static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2], (float)scale};
+                       static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2], (float)scale, 0};
     const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
-    const size_t smem = ((size_t)3 * kChunk * (V + 8) + (size_t)K * (V + 8)) * 2 + (size_t)6 * K * 4 +
-                        (size_t)2 * kChunk * (K + 8) * 2 + (size_t)kChunk * (K + 4) * 4;
-    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<128, 128>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
-    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 64>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
-    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 128>), "kda_bwd_dqkwg_wy", grid, smem, p, kDqkwgThreads);
+    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<128, 128, false>), "kda_bwd_dqkwg_wy", grid, (kda_bwd_fused_smem<128, 128, false>()), p, kDqkwgThreads);
+    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 64, false>), "kda_bwd_dqkwg_wy", grid, (kda_bwd_fused_smem<64, 64, false>()), p, kDqkwgThreads);
+    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 128, false>), "kda_bwd_dqkwg_wy", grid, (kda_bwd_fused_smem<64, 128, false>()), p, kDqkwgThreads);
+    return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(64,128).", op, (long long)K,
+                (long long)V);
+}
+
+// chunk_kda_bwd_dqkwg_wy_intra: the three stages after the reverse scan in one launch; dq, dk (fp32, or the element type
+// when no two value heads share a key head), dg (reverse running sum taken), dv and dbeta leave final.
+int kda_dqkwg_wy_intra_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk,
+                            const fla_tensor *h, const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2,
+                            const fla_tensor *v, const fla_tensor *beta, const fla_tensor *akk, const fla_int_array *cu,
+                            const fla_int_array *ci, double scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+                            const fla_tensor *dg, const fla_tensor *dv, const fla_tensor *db, void *ws, uint64_t ws_size,
+                            hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_kda_bwd_dqkwg_wy_intra";
+    ChunkGeom geom;
+    int rc;
+    if ((rc = gdn_geometry(op, k, v_new, nullptr, chunk_size, geom, kElemDtype))) return rc;
+    if (d_o != nullptr && d_o->ndim == 4 && geom.Hv > 1 && geom.T <= (1 << 20)) geom.head_fast = d_o->stride[2] > d_o->stride[1] ? 1 : 0;
+    const int bf = dt_bit(kElemDtype);
+    const int64_t B = geom.B, Hk = geom.Hk, Hv = geom.Hv, T = geom.T, K = geom.K, V = geom.V;
+    if ((rc = check_bhtd(op, "q", q, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "k", k, B, Hk, T, K, bf))) return rc;
+    if ((rc = check_bhtd(op, "v_new", v_new, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "d_o", d_o, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv2", dv2, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "v", v, B, Hv, T, V, bf))) return rc;
+    if ((rc = check_bhtd(op, "Akk", akk, B, Hv, T, kChunk, bf))) return rc;
+    if ((rc = check_bhtd(op, "dv", dv, B, Hv, T, V, bf))) return rc;
+    FLA_REQUIRE(beta != nullptr && beta->data != nullptr, FLA_ERR_NULL, "%s: beta must be provided.", op);
+    if ((rc = check_bht(op, "beta", beta, B, Hv, T, kElemDtype))) return rc;
+    if ((rc = check_f32_bhtd(op, "gk", gk, B, Hv, T, K))) return rc;
+    FLA_REQUIRE(dq != nullptr && dk != nullptr, FLA_ERR_NULL, "%s: dq and dk must be provided.", op);
+    FLA_REQUIRE(dq->dtype == dk->dtype, FLA_ERR_DTYPE, "%s: dq and dk must share one dtype.", op);
+    const bool out16 = dq->dtype == kElemDtype;
+    if (out16) {
+        if ((rc = check_bhtd(op, "dq", dq, B, Hv, T, K, bf))) return rc;
+        if ((rc = check_bhtd(op, "dk", dk, B, Hv, T, K, bf))) return rc;
+    } else {
+        if ((rc = check_f32_bhtd(op, "dq", dq, B, Hv, T, K))) return rc;
+        if ((rc = check_f32_bhtd(op, "dk", dk, B, Hv, T, K))) return rc;
+    }
+    if ((rc = check_f32_bhtd(op, "dg", dg, B, Hv, T, K))) return rc;
+    if ((rc = check_tensor(db, op, "db", 3, dt_bit(FLA_F32)))) return rc;
+    FLA_REQUIRE(db->shape[0] == B && db->shape[1] == Hv && db->shape[2] == T, FLA_ERR_SHAPE, "%s: db must be [%lld,%lld,%lld].",
+                op, (long long)B, (long long)Hv, (long long)T);
+    Varlen vl;
+    if ((rc = finish_varlen(op, vl, geom, cu, ci, ws, ws_size, stream, query))) return rc;
+    if ((rc = check_state_blocks(op, "h", h, geom))) return rc;
+    if ((rc = check_state_blocks(op, "dh", dh, geom))) return rc;
+    if (query) return FLA_OK;
+    if (geom.NT == 0 || geom.B == 0) return FLA_OK;
+    const ViewF none{nullptr, 0, 0, 0};
+    auto any_view = [](const fla_tensor *t) { return ViewF{static_cast<float *>(t->data), t->stride[0], t->stride[1], t->stride[2]}; };
+    KdaDqkwgWyParams p{geom, view4(q), view4(k), view4(v_new), view4(d_o), view4(dv2), view4(v), view4(akk), view4(dv), view3(beta),
+                       static_cast<const float *>(gk->data), gk->stride[0], gk->stride[1], gk->stride[2],
+                       static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
+                       h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
+                       any_view(dq), any_view(dk), viewf(dg), none, none,
+                       static_cast<float *>(db->data), db->stride[0], db->stride[1], db->stride[2], (float)scale, out16 ? 1 : 0};
+    const dim3 grid = chunk_head_grid(geom, geom.NT, geom.Hv);
+    if (K == 128 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<128, 128, true>), "kda_bwd_dqkwg_wy_intra", grid, (kda_bwd_fused_smem<128, 128, true>()), p, kDqkwgThreads);
+    if (K == 64 && V == 64) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 64, true>), "kda_bwd_dqkwg_wy_intra", grid, (kda_bwd_fused_smem<64, 64, true>()), p, kDqkwgThreads);
+    if (K == 64 && V == 128) FLA_KDA_BWD_LAUNCH((kda_bwd_dqkwg_wy_kernel<64, 128, true>), "kda_bwd_dqkwg_wy_intra", grid, (kda_bwd_fused_smem<64, 128, true>()), p, kDqkwgThreads);
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%lld,%lld) has no kernel; built: (128,128),(64,64),(64,128).", op, (long long)K,
                 (long long)V);
 }
@@ -1090,4 +1357,27 @@ FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_wy)(
     return fla::guarded([&] { return fla::kda_dqkwg_wy_impl(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale,
                                   chunk_size, dq, dk, dg, dAqk, dv, db, dAkk, workspace, workspace_size,
                                   static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_wy_intra_get_workspace_size)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dv,
+    const fla_tensor *db, uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_wy_intra_get_workspace_size, q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dg, dv, db, workspace_size);
+    FLA_NULL_WS("chunk_kda_bwd_dqkwg_wy_intra");
+    return fla::guarded([&] { return fla::kda_dqkwg_wy_intra_impl(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale,
+                                        chunk_size, dq, dk, dg, dv, db, nullptr, 0, nullptr, workspace_size); });
+}
+FLA_ENTRY(fla_chunk_kda_bwd_dqkwg_wy_intra)(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dv,
+    const fla_tensor *db, void *workspace, uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_chunk_kda_bwd_dqkwg_wy_intra, q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale, chunk_size, dq, dk, dg, dv, db, workspace, workspace_size, stream);
+    return fla::guarded([&] { return fla::kda_dqkwg_wy_intra_impl(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, cu_seqlens, chunk_indices, scale,
+                                        chunk_size, dq, dk, dg, dv, db, workspace, workspace_size,
+                                        static_cast<hipStream_t>(stream), nullptr); });
 }

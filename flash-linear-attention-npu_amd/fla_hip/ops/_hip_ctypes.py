@@ -78,6 +78,7 @@ OP_ARGTYPES = {
     "chunk_kda_bwd_dhu": [_T] * 8 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 3,
     "chunk_kda_bwd_wy": [_T] * 7 + [_IA, _IA, ctypes.c_int64] + [_T] * 5,
     "chunk_kda_bwd_dqkwg_wy": [_T] * 11 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 7,
+    "chunk_kda_bwd_dqkwg_wy_intra": [_T] * 11 + [_IA, _IA, ctypes.c_double, ctypes.c_int64] + [_T] * 5,
 }
 
 
@@ -1037,6 +1038,40 @@ def chunk_kda_bwd_dqkwg_wy(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, scale
             ctx.tensor(Akk, "Akk"), ctx.int_array(cu), ctx.int_array(_as_int_tuple(chunk_indices)),
             ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
             *[ctx.tensor(t, n) for t, n in zip(outs, ("dq", "dk", "dg", "dAqk", "dv", "db", "dAkk"))],
+        ],
+        outs,
+    )
+    return outs
+
+
+def chunk_kda_bwd_dqkwg_wy_intra(q, k, v_new, gk, h, d_o, dh, dv2, v, beta, Akk, scale, chunk_size=64, *, cu_seqlens=None,
+                                 chunk_indices=None, layout_like=None, grad_dtype=None):
+    """Everything of the KDA chunk backward after the reverse scan in one launch: ``chunk_kda_bwd_dqkwg_wy`` followed by
+    ``chunk_kda_bwd_intra`` with the reverse chunk-local running sum of dg.  dAqk and dAkk never leave the chip and dq,
+    dk, dg, dbeta are written once, final.  Returns ``(dq, dk, dg, dv, db)``: dq / dk [B,Hv,T,K] in ``grad_dtype``
+    (default fp32; q's dtype is meant for Hv == Hk, where no sum over the value heads of a key head follows), dg fp32
+    [B,Hv,T,K] and db fp32 [B,Hv,T] laid out like ``layout_like`` (default: like ``gk``), dv like ``v``."""
+    import torch
+
+    B, Hv, T, K = _shape(gk)
+    V = _shape(v)[-1]
+    like = gk if layout_like is None else layout_like
+    f32 = lambda d: _empty_strided_like((B, Hv, T, d), like, torch.float32, q.device)
+    gdt = torch.float32 if grad_dtype is None else grad_dtype
+    dq, dk = (_empty_strided_like((B, Hv, T, K), like, gdt, q.device) for _ in range(2))
+    dg = f32(K)
+    db = f32(1)[..., 0]
+    dv = _empty_strided_like((B, Hv, T, V), v, v.dtype)
+    cu = _as_int_tuple(cu_seqlens)
+    outs = (dq, dk, dg, dv, db)
+    _call_op(
+        "chunk_kda_bwd_dqkwg_wy_intra", OP_ARGTYPES["chunk_kda_bwd_dqkwg_wy_intra"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v_new, "v_new"), ctx.tensor(gk, "gk"), ctx.tensor(h, "h"),
+            ctx.tensor(d_o, "d_o"), ctx.tensor(dh, "dh"), ctx.tensor(dv2, "dv2"), ctx.tensor(v, "v"), ctx.tensor(beta, "beta"),
+            ctx.tensor(Akk, "Akk"), ctx.int_array(cu), ctx.int_array(_as_int_tuple(chunk_indices)),
+            ctypes.c_double(float(scale)), ctypes.c_int64(int(chunk_size)),
+            *[ctx.tensor(t, n) for t, n in zip(outs, ("dq", "dk", "dg", "dv", "db"))],
         ],
         outs,
     )

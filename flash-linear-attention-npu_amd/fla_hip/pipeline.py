@@ -308,7 +308,7 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     dtype of their inputs, dg fp32 in the layout of the gate = gradient of the per-token log decay (natural log),
     dh0 fp32 [N,Hv,K,V] or None.  Stages: reverse scan (bwd_dhu, gK; it forms dv = Aqk^T do itself) -> dq, dk, dw, dg of
     the state-dependent parts and dAqk -> backward of the WY factors (dv, dbeta, dAkk) -> chunk_kda_bwd_intra -> reverse
-    chunk-local cumulative sum of dg."""
+    chunk-local cumulative sum of dg; up to 128 channels the stages after the scan are one launch."""
     import torch
 
     if chunk_size != 64:
@@ -337,10 +337,17 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
         # no pass for chunk_kda_bwd_dav: the reverse scan forms dv = Aqk^T do from the score blocks, the next stage writes
         # dAqk = scale tril(do v_new^T) from the do and v_new tiles it stages anyway
         dh, dh0, dv2 = _raw.chunk_kda_bwd_dhu(qg4, kg4, w4, doh, Aqk4, scale, chunk_size, gK=gk4, h0=initial_state, dht=dht, **kw)
-        # the state-dependent stage and the backward of the WY factors in one launch (chunk_kda_bwd_dqkwg and
-        # chunk_kda_bwd_wy as operators of their own write dk, dg and dw, read them back and write dk, dg again)
-        dq, dk, dg, dAqk, dv, db, dAkk = _raw.chunk_kda_bwd_dqkwg_wy(qh, kh, vn4, gk4, h5, doh, dh, dv2, vh, bh, Akk4, scale,
-                                                                     chunk_size, layout_like=layout_like, **kw)
+        # everything after the reverse scan in one launch: the state-dependent stage, the backward of the WY factors and the
+        # intra-chunk stage with the reverse running sum of dg (as operators of their own they pass dk, dg, dw, dq and the two
+        # score gradients through memory between them)
+        dq, dk, dg, dv, db = _raw.chunk_kda_bwd_dqkwg_wy_intra(qh, kh, vn4, gk4, h5, doh, dh, dv2, vh, bh, Akk4, scale, chunk_size,
+                                                               layout_like=layout_like, grad_dtype=q.dtype if Hv == Hk else None,
+                                                               **kw)
+        if Hv != Hk:      # value heads that share a key head add their gradients
+            dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2).to(q.dtype)
+            dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2).to(k.dtype)
+        back = lambda t: _from_index_order(t, layout)
+        return (back(dq), back(dk), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
     # the last stage also takes the reverse chunk-local running sum of dg, which is complete with its own part
     back = lambda t: _from_index_order(t, layout)
     if Hv == Hk:          # dq, dk are final with the last stage: it writes them in the dtype of q and k

@@ -546,6 +546,26 @@ int fla_chunk_kda_bwd_dqkwg_wy(
     const fla_tensor *dv, const fla_tensor *db, const fla_tensor *dAkk, void *workspace, uint64_t workspace_size,
     void *stream);
 
+/* chunk_kda_bwd_dqkwg_wy_intra: the same two stages followed by chunk_kda_bwd_intra_cumsum in the same launch, i.e.
+ * everything of the KDA backward after the reverse scan.  dAqk and dAkk stay on chip (the intra-chunk stage reads them
+ * as fp32 tiles, masked as that operator masks them), its increments are added to dq, dk, dg in registers (same fp32
+ * products and order of additions as the separate operators), dg leaves as its reverse chunk-local running sum and
+ * dbeta complete.  dq and dk (one dtype for both): f32 [B,Hv,T,K], or the element type, which is meant for Hv == Hk
+ * where they are final; with grouped value heads the caller adds the fp32 results of the heads of a group.  Other
+ * operands, head sizes and chunk size as chunk_kda_bwd_dqkwg_wy.  No counterpart in the reference. */
+int fla_chunk_kda_bwd_dqkwg_wy_intra_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dv,
+    const fla_tensor *db, uint64_t *workspace_size);
+int fla_chunk_kda_bwd_dqkwg_wy_intra(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v_new, const fla_tensor *gk, const fla_tensor *h,
+    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv2, const fla_tensor *v, const fla_tensor *beta,
+    const fla_tensor *Akk, const fla_int_array *cu_seqlens, const fla_int_array *chunk_indices, double scale,
+    int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk, const fla_tensor *dg, const fla_tensor *dv,
+    const fla_tensor *db, void *workspace, uint64_t workspace_size, void *stream);
+
 /* ------------------------------------------------------------------------
  * l2norm_fwd / l2norm_bwd - the q/k normalisation of the chunk pipelines, which the reference
  * runs as Triton kernels (fla/ops/triton/triton_core/l2norm.py:131-224; called from

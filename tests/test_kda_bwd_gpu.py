@@ -188,6 +188,55 @@ def test_bwd_dqkwg_and_wy_in_one_launch(dev, case):
         assert torch.equal(a, e)
 
 
+@pytest.mark.parametrize("case", STAGE_CASES)
+def test_bwd_after_the_scan_in_one_launch(dev, case):
+    """chunk_kda_bwd_dqkwg_wy_intra against chunk_kda_bwd_dqkwg_wy followed by chunk_kda_bwd_intra with the running sum of
+    dg: the same fp32 products, the score gradients kept on chip instead of passing through memory and the increments added
+    in registers (where a product and the addition may contract to one rounding), so the results agree to the last bits of
+    fp32, and to a rounding of the element type when dq, dk leave in it."""
+    from fla_hip.ops import _hip_ctypes as raw
+    B, T, Hk, Hv, K, V, cu = case
+    gen = torch.Generator().manual_seed(T + 5 * K)
+    NT = gdn.total_chunks(B, T, 64, cu)
+    q, k = rnd(gen, B, Hk, T, K, scale=0.3), rnd(gen, B, Hk, T, K, scale=0.3)
+    v_new, do, dv2, v = (rnd(gen, B, Hv, T, V) for _ in range(4))
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    gk = gate_cumsum(F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.3, cu)
+    h, dh = rnd(gen, B, Hv, NT, K, V, scale=0.5), rnd(gen, B, Hv, NT, K, V, scale=0.5)
+    Akk = torch.zeros(B, Hv, T, 64)
+    for b, _, _, s, e in gdn.chunk_spans(B, T, 64, cu):
+        L = e - s
+        Akk[b, :, s:e, :L] = torch.linalg.inv(torch.eye(L) + torch.tril(torch.randn(Hv, L, L, generator=gen) * 0.1, -1))
+    Akk = Akk.to(BF)
+    ops = [t.to(dev) for t in (q, k, v_new, gk, h, do, dh, dv2, v, beta, Akk)]
+    dq, dk, dg, dAqk, dv, db, dAkk = raw.chunk_kda_bwd_dqkwg_wy(*ops, 0.7, cu_seqlens=cu)
+    dq16, dk16 = torch.empty_like(dq, dtype=BF), torch.empty_like(dk, dtype=BF)
+    dq_f, dk_f, db_f, dg_f = dq.clone(), dk.clone(), db.clone(), dg.clone()
+    raw.chunk_kda_bwd_intra_inplace(ops[0], ops[1], ops[3], ops[9], dAqk, dAkk, dq_f, dk_f, db_f, dg_f, cu_seqlens=cu, cumsum_dg=True)
+    one = raw.chunk_kda_bwd_dqkwg_wy_intra(*ops, 0.7, cu_seqlens=cu)
+    assert [t.dtype for t in one] == [torch.float32] * 3 + [BF, torch.float32]
+    assert torch.equal(one[3], dv)
+    for name, a, e in zip(("dq", "dk", "dg", "dbeta"), (one[0], one[1], one[2], one[4]), (dq_f, dk_f, dg_f, db_f)):
+        close(a, e, name, 2e-6)
+    if Hk == Hv:
+        raw.chunk_kda_bwd_intra_inplace(ops[0], ops[1], ops[3], ops[9], dAqk, dAkk, dq, dk, db, dg, cu_seqlens=cu, cumsum_dg=True,
+                                        dq_out=dq16, dk_out=dk16)
+        low = raw.chunk_kda_bwd_dqkwg_wy_intra(*ops, 0.7, cu_seqlens=cu, grad_dtype=BF)
+        assert low[0].dtype == BF and low[1].dtype == BF
+        assert torch.equal(low[2], one[2]) and torch.equal(low[3], dv) and torch.equal(low[4], one[4])
+        for name, a, e in zip(("dq", "dk"), low, (dq16, dk16)):
+            close(a, e, name + " in the element type", 2.0 ** -8)   # a last-bit difference in fp32 may flip the rounding
+            assert (a != e).float().mean().item() < 1e-2, name
+    # results laid out token-major: views only, identical numbers
+    like = torch.empty(B, T, Hv, K, device="meta").transpose(1, 2)
+    tm = lambda t: t.transpose(1, 2).contiguous().transpose(1, 2)
+    out2 = raw.chunk_kda_bwd_dqkwg_wy_intra(*ops[:5], tm(ops[5]), ops[6], tm(ops[7]), tm(ops[8]), ops[9], ops[10], 0.7, cu_seqlens=cu,
+                                            layout_like=like)
+    assert out2[0].transpose(1, 2).is_contiguous() and out2[2].transpose(1, 2).is_contiguous()
+    for a, e in zip(out2, one):
+        assert torch.equal(a, e)
+
+
 # ---------------------------------------------------------------------------------------------
 # composition
 # ---------------------------------------------------------------------------------------------
