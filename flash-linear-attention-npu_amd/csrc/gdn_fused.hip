@@ -43,7 +43,9 @@ struct FusedParams {
     int64_t go_sb, go_sh, go_st;
     const float *h0;
     float *hT;
-    int64_t s_sn, s_sh;
+    int64_t s_sn, s_sh, s_sk, s_sv;   // strides of (sequence or pool row, head, key channel, value channel)
+    const int32_t *slot;               // per sequence: the pool row that holds its state; null: row n
+    int pool_rows;
     float scale;
     int slabs;
     int remap;          // 1: co-locate the slabs of one head on one XCD
@@ -57,6 +59,13 @@ struct FusedParams {
     float *q_rstd, *k_rstd;
     int64_t rs_sb, rs_sh;
 };
+
+// Row of the state tensors that belongs to sequence n: n itself, or the pool row the caller names for it.  A negative
+// index means no row (the sequence starts from zero and its final state is dropped); one past the pool is clamped
+// into it, so that a wrong index reads and writes a wrong row, never outside the allocation.
+__device__ __forceinline__ int64_t state_row(const FusedParams &p, int n) {
+    return p.slot ? (int64_t)min(p.slot[n], p.pool_rows - 1) : (int64_t)n;
+}
 
 template <int K, int CT> struct FusedSmem {
     static constexpr int VS = 64 * CT;
@@ -259,10 +268,10 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             f32x4 a = zero4();
-            if (p.h0) {
-                const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+            if (p.h0 && state_row(p, n) >= 0) {
+                const float *s = p.h0 + state_row(p, n) * p.s_sn + hv * p.s_sh;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li];
+                for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * p.s_sk + (int64_t)(vcol0 + 16 * ct + li) * p.s_sv];
             }
             hacc[kt][ct] = a;
         }
@@ -568,15 +577,15 @@ __global__ void __launch_bounds__(kThreads) gdn_fused_kernel(const FusedParams p
     }
     if (DB && nchunks > 0) store_o(nchunks - 1);
 
-    if (p.hT) {
-        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+    if (p.hT && state_row(p, n) >= 0) {
+        float *s = p.hT + state_row(p, n) * p.s_sn + hv * p.s_sh;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + 16 * ct + li] = hacc[kt][ct][e];
+                    s[(int64_t)(16 * kt + 4 * lg + e) * p.s_sk + (int64_t)(vcol0 + 16 * ct + li) * p.s_sv] = hacc[kt][ct][e];
     }
 }
 
@@ -856,10 +865,10 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
         f32x4 a = zero4();
-        if (p.h0) {
-            const float *s = p.h0 + n * p.s_sn + hv * p.s_sh;
+        if (p.h0 && state_row(p, n) >= 0) {
+            const float *s = p.h0 + state_row(p, n) * p.s_sn + hv * p.s_sh;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li];
+            for (int e = 0; e < 4; ++e) a[e] = s[(int64_t)(16 * kt + 4 * lg + e) * p.s_sk + (int64_t)(vcol0 + li) * p.s_sv];
         }
         hacc[kt] = a;
     }
@@ -1078,12 +1087,12 @@ __global__ void __launch_bounds__(512) gdn_pipe_kernel(const FusedParams p) {
         }
         __syncthreads();   // end
     }
-    if (p.hT) {
-        float *s = p.hT + n * p.s_sn + hv * p.s_sh;
+    if (p.hT && state_row(p, n) >= 0) {
+        float *s = p.hT + state_row(p, n) * p.s_sn + hv * p.s_sh;
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) s[(int64_t)(16 * kt + 4 * lg + e) * V + vcol0 + li] = hacc[kt][e];
+            for (int e = 0; e < 4; ++e) s[(int64_t)(16 * kt + 4 * lg + e) * p.s_sk + (int64_t)(vcol0 + li) * p.s_sv] = hacc[kt][e];
     }
 }
 
@@ -1117,8 +1126,8 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                int64_t chunk_size, bool use_qk_l2norm, const fla_tensor *o, const fla_tensor *g_cumsum, const fla_tensor *final_state,
                const fla_tensor *h, const fla_tensor *v_new, const fla_tensor *w, const fla_tensor *qn, const fla_tensor *kn,
                const fla_tensor *q_rstd, const fla_tensor *k_rstd,
-               void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
-    const char *op = "gdn_chunk_fwd";
+               void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query, const fla_tensor *state_indices = nullptr) {
+    const char *op = state_indices ? "gdn_chunk_fwd_state_pool" : "gdn_chunk_fwd";
     ChunkGeom geom;
     int rc;
     if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype))) return rc;
@@ -1153,11 +1162,26 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     auto check_state = [&](const fla_tensor *s, const char *name) -> int {
         int r = check_tensor(s, op, name, 4, dt_bit(FLA_F32));
         if (r) return r;
+        if (state_indices) {   // rows of a pool, K x V blocks in either order
+            FLA_REQUIRE(s->shape[0] >= 1 && s->shape[0] <= INT32_MAX && s->shape[1] == geom.Hv && s->shape[2] == geom.K &&
+                            s->shape[3] == geom.V && s->stride[0] >= 0 && s->stride[1] >= 0 &&
+                            ((s->stride[3] == 1 && s->stride[2] == geom.V) || (s->stride[2] == 1 && s->stride[3] == geom.K)),
+                        FLA_ERR_SHAPE, "%s: %s must be [rows,Hv,K,V] fp32 with contiguous K x V or V x K blocks.", op, name);
+            return FLA_OK;
+        }
         FLA_REQUIRE(s->shape[0] == geom.N && s->shape[1] == geom.Hv && s->shape[2] == geom.K && s->shape[3] == geom.V &&
                         s->stride[3] == 1 && s->stride[2] == geom.V,
                     FLA_ERR_SHAPE, "%s: %s must be [N=%d,Hv,K,V] fp32 with contiguous K x V blocks.", op, name, geom.N);
         return FLA_OK;
     };
+    if (state_indices) {
+        if ((rc = check_tensor(state_indices, op, "state_indices", 1, dt_bit(FLA_I32)))) return rc;
+        FLA_REQUIRE(state_indices->shape[0] == geom.N && (geom.N <= 1 || state_indices->stride[0] == 1), FLA_ERR_SHAPE,
+                    "%s: state_indices must be a contiguous int32 [N=%d].", op, geom.N);
+        FLA_REQUIRE(initial_state && initial_state->data && output_final_state && final_state &&
+                        final_state->data == initial_state->data,
+                    FLA_ERR_NULL, "%s: the state pool is both the initial and the final state.", op);
+    }
     const bool has_h0 = initial_state && initial_state->data;
     if (has_h0 && (rc = check_state(initial_state, "initial_state"))) return rc;
     if (output_final_state && (rc = check_state(final_state, "final_state"))) return rc;
@@ -1219,9 +1243,14 @@ int fused_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     if (sref) {
         p.s_sn = sref->stride[0];
         p.s_sh = sref->stride[1];
+        p.s_sk = sref->stride[2];
+        p.s_sv = sref->stride[3];
+        p.pool_rows = (int)sref->shape[0];
     }
+    if (state_indices) p.slot = static_cast<const int32_t *>(state_indices->data);
     if (has_h0 && output_final_state)
-        FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1],
+        FLA_REQUIRE(initial_state->stride[0] == final_state->stride[0] && initial_state->stride[1] == final_state->stride[1] &&
+                        initial_state->stride[2] == final_state->stride[2] && initial_state->stride[3] == final_state->stride[3],
                     FLA_ERR_SHAPE, "%s: initial_state and final_state must share strides.", op);
     p.scale = (float)scale;
     p.l2norm = use_qk_l2norm ? 1 : 0;
@@ -1286,4 +1315,30 @@ FLA_ENTRY(fla_gdn_chunk_fwd)(const fla_tensor *q, const fla_tensor *k, const fla
     return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, initial_state, output_final_state, cu_seqlens, chunk_size,
                            use_qk_l2norm_in_kernel, o, g_cumsum, final_state, h, v_new, w, q_normalised, k_normalised, q_rstd,
                            k_rstd, workspace, workspace_size, static_cast<hipStream_t>(stream), nullptr); });
+}
+
+FLA_ENTRY(fla_gdn_chunk_fwd_state_pool_get_workspace_size)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v,
+                                                           const fla_tensor *g, const fla_tensor *beta, double scale,
+                                                           const fla_tensor *state_pool, const fla_tensor *state_indices,
+                                                           const fla_int_array *cu_seqlens, int64_t chunk_size,
+                                                           bool use_qk_l2norm_in_kernel, const fla_tensor *o,
+                                                           uint64_t *workspace_size) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_state_pool_get_workspace_size, q, k, v, g, beta, scale, state_pool, state_indices, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, workspace_size);
+    if (!workspace_size) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd_state_pool: workspace_size must not be null.");
+    if (!state_indices) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd_state_pool: state_indices must not be null.");
+    return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, state_pool, true, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o,
+                           nullptr, state_pool, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr,
+                           workspace_size, state_indices); });
+}
+
+FLA_ENTRY(fla_gdn_chunk_fwd_state_pool)(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+                                        const fla_tensor *beta, double scale, const fla_tensor *state_pool,
+                                        const fla_tensor *state_indices, const fla_int_array *cu_seqlens, int64_t chunk_size,
+                                        bool use_qk_l2norm_in_kernel, const fla_tensor *o, void *workspace,
+                                        uint64_t workspace_size, void *stream) {
+    FLA_ROUTE_F16(q, fla_gdn_chunk_fwd_state_pool, q, k, v, g, beta, scale, state_pool, state_indices, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o, workspace, workspace_size, stream);
+    if (!state_indices) return fla::fail(FLA_ERR_NULL, "gdn_chunk_fwd_state_pool: state_indices must not be null.");
+    return fla::guarded([&] { return fla::fused_impl(q, k, v, g, beta, scale, state_pool, true, cu_seqlens, chunk_size, use_qk_l2norm_in_kernel, o,
+                           nullptr, state_pool, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, workspace, workspace_size,
+                           static_cast<hipStream_t>(stream), nullptr, state_indices); });
 }

@@ -458,6 +458,86 @@ int rec_impl(const fla_tensor *query, const fla_tensor *key, const fla_tensor *v
     return FLA_OK;
 }
 
+// -------------------------------------------------------------------------------------------------
+// Plan for running the sequences of a call on the chunk kernels: whether every sequence keeps ONE pool row (the
+// row its first token names) that no other sequence uses, which row that is, and the lengths for the host.
+// One workgroup per sequence; every workgroup scans the (short) list of lengths for its own offsets.
+// -------------------------------------------------------------------------------------------------
+constexpr int kPlanMaxSeqs = 8192;
+
+__global__ void __launch_bounds__(kThreads) prefill_plan_kernel(const int32_t *lens, const int32_t *idx, int batch, int64_t total,
+                                                                int pool_rows, int32_t *slots, int32_t *report) {
+    __shared__ int32_t startS[kPlanMaxSeqs + 1];   // token offset of every sequence (capped at total + 1), then the end of the last
+    __shared__ int64_t partS[kThreads];
+    __shared__ int badS;
+    const int tid = threadIdx.x, i = blockIdx.x;
+    const int per = (batch + kThreads - 1) / kThreads;
+    int64_t sum = 0;
+    bool negative = false;
+    for (int j = tid * per; j < min(batch, (tid + 1) * per); ++j) {
+        const int n = lens[1 + j];
+        negative |= n < 0;
+        sum += max(n, 0);
+    }
+    partS[tid] = sum;
+    if (tid == 0) badS = 0;
+    __syncthreads();
+    int64_t off = lens[0];
+    for (int t = 0; t < tid; ++t) off += partS[t];
+    for (int j = tid * per; j < min(batch, (tid + 1) * per); ++j) {
+        startS[j] = (int32_t)min(off, total + 1);
+        off += max(lens[1 + j], 0);
+    }
+    if ((tid + 1) * per >= batch) startS[batch] = (int32_t)min(off, total + 1);   // every such thread holds the same end
+    __syncthreads();
+    const int64_t start = startS[i], end = startS[i + 1];
+    const int len = lens[1 + i];
+    bool bad = negative || lens[0] < 0 || startS[batch] > total;
+    int slot = -1;
+    if (!__syncthreads_or(bad) && len > 0) {
+        slot = idx[start];
+        if (slot < 0 || slot >= pool_rows) bad = true;
+        for (int64_t t = start + tid; t < end; t += kThreads) bad |= idx[t] != slot;          // one row for the whole sequence
+        for (int j = tid; j < batch; j += kThreads)                                            // and for no other one
+            if (j != i && lens[1 + j] > 0 && idx[startS[j]] == slot) bad = true;
+    }
+    if (bad) badS = 1;
+    __syncthreads();
+    if (tid == 0) {
+        slots[i] = badS ? -1 : slot;
+        report[1 + i] = len;
+        report[1 + batch + i] = badS;
+        if (i == 0) report[0] = lens[0];
+    }
+}
+
+int prefill_plan_impl(const fla_tensor *actual_seq_lengths, const fla_tensor *ssm_state_indices, int64_t pool_rows,
+                      const fla_tensor *slots, const fla_tensor *report, hipStream_t stream) {
+    const char *op = "recurrent_gdn_prefill_plan";
+    int rc;
+    const int i32 = dt_bit(FLA_I32);
+    if ((rc = check_tensor(actual_seq_lengths, op, "actual_seq_lengths", 1, i32))) return rc;
+    if ((rc = check_tensor(ssm_state_indices, op, "ssm_state_indices", 1, i32))) return rc;
+    if ((rc = check_tensor(slots, op, "slots", 1, i32))) return rc;
+    if ((rc = check_tensor(report, op, "report", 1, i32))) return rc;
+    const int64_t batch = actual_seq_lengths->shape[0] - 1;
+    FLA_REQUIRE(batch >= 1 && batch <= kPlanMaxSeqs, FLA_ERR_UNSUPPORTED, "%s: between 1 and %d sequences, got %lld.", op,
+                kPlanMaxSeqs, (long long)batch);
+    FLA_REQUIRE(pool_rows >= 1 && pool_rows <= INT32_MAX, FLA_ERR_SHAPE, "%s: pool_rows out of range.", op);
+    FLA_REQUIRE(ssm_state_indices->shape[0] < INT32_MAX, FLA_ERR_SHAPE, "%s: too many tokens.", op);
+    const fla_tensor *flat[] = {actual_seq_lengths, ssm_state_indices, slots, report};
+    for (const fla_tensor *t : flat)
+        FLA_REQUIRE(t->shape[0] <= 1 || t->stride[0] == 1, FLA_ERR_SHAPE, "%s: the index tensors must be contiguous.", op);
+    FLA_REQUIRE(slots->shape[0] == batch && report->shape[0] == 2 * batch + 1, FLA_ERR_SHAPE,
+                "%s: slots must be int32 [B] and report int32 [2B+1].", op);
+    FLA_LAUNCH("recurrent_gdn_prefill_plan", stream, prefill_plan_kernel, dim3((unsigned)batch), dim3(kThreads), 0, stream,
+               static_cast<const int32_t *>(actual_seq_lengths->data), static_cast<const int32_t *>(ssm_state_indices->data),
+               (int)batch, ssm_state_indices->shape[0], (int)pool_rows, static_cast<int32_t *>(slots->data),
+               static_cast<int32_t *>(report->data));
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+
 }  // namespace
 }  // namespace fla
 
@@ -480,4 +560,10 @@ extern "C" int fla_recurrent_gated_delta_rule(
     return fla::guarded([&] { return fla::rec_impl(query, key, value, beta, state, actual_seq_lengths, ssm_state_indices, g, gk,
                          num_accepted_tokens, scale, out, workspace, workspace_size, static_cast<hipStream_t>(stream),
                          nullptr); });
+}
+
+extern "C" int fla_recurrent_gdn_prefill_plan(const fla_tensor *actual_seq_lengths, const fla_tensor *ssm_state_indices,
+                                              int64_t pool_rows, const fla_tensor *slots, const fla_tensor *report, void *stream) {
+    return fla::guarded([&] { return fla::prefill_plan_impl(actual_seq_lengths, ssm_state_indices, pool_rows, slots, report,
+                                                            static_cast<hipStream_t>(stream)); });
 }

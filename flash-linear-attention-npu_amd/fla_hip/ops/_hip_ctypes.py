@@ -50,7 +50,9 @@ OP_ARGTYPES = {
     "chunk_fwd_o": [_T, _T, _T, _T, _T, _IA, _IA, ctypes.c_double, ctypes.c_int64, _T],
     "gdn_chunk_fwd": [_T, _T, _T, _T, _T, ctypes.c_double, _T, ctypes.c_bool, _IA, ctypes.c_int64, ctypes.c_bool,
                       _T, _T, _T, _T, _T, _T, _T, _T, _T, _T],
+    "gdn_chunk_fwd_state_pool": [_T, _T, _T, _T, _T, ctypes.c_double, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, _T],
     "recurrent_gated_delta_rule": [_T, _T, _T, _T, _T, _T, _T, _T, _T, _T, ctypes.c_float, _T],
+    "recurrent_gdn_prefill_plan": [_T, _T, ctypes.c_int64, _T, _T],
     "causal_conv1d": [_T, _T, _T, _T, _IA, _IA, _IA, _IA, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                       ctypes.c_int64, _T],
     "kda_gate_cumsum": [_T, _T, _T, _IA, ctypes.c_int64, ctypes.c_bool, ctypes.c_bool, ctypes.c_double, _T],
@@ -328,47 +330,68 @@ def _recurrent_prefill_on_chunk_kernels(query, key, value, state, beta, scale, a
         return None
     if any(t.stride(-1) != 1 for t in (query, key, value)) or state.stride(-1) != 1 or torch.cuda.is_current_stream_capturing():
         return None
-    # The plan is formed on the device and read with ONE synchronising copy: the sequence lengths and a flag that says
-    # whether every token of a sequence names the slot of its first token, whether the slots are valid and whether no
-    # two sequences share one.  The pool rows are gathered ahead of that copy, so that they are on their way while the host waits.
+    # The plan is formed on the device by one launch and read with ONE synchronising copy: the sequence lengths and, per
+    # sequence, a flag that says whether every token names the pool row of the first token, whether that row is valid
+    # and whether no other sequence names it.
     dev, blocks = query.device, _shape(state)[0]
-    lens_d = actual_seq_lengths.to(torch.int64)
-    span = lens_d[1:]
-    ends = lens_d[0] + torch.cumsum(span, 0)
-    starts = ends - span
-    tok = torch.arange(total, device=dev)
-    seq = torch.searchsorted(ends, tok, right=True)                  # sequence of token t; `batch` past the last one
-    inside = (tok >= lens_d[0]) & (seq < batch)
-    slot = ssm_state_indices[starts.clamp(0, total - 1)].to(torch.int64)
-    live = span > 0
-    valid = (slot >= 0) & (slot < blocks)
-    same = ((ssm_state_indices == slot[seq.clamp(max=batch - 1)]) | ~inside).all()
-    uses = torch.zeros(blocks + 1, dtype=torch.int64, device=dev)
-    uses.index_add_(0, torch.where(live & valid, slot, torch.full_like(slot, blocks)), torch.ones_like(slot))
-    ok = same & (valid | ~live).all() & (uses[:blocks] <= 1).all() & (span >= 0).all() & (ends[-1] <= total)
-    slot = slot.clamp(0, blocks - 1)
-    h0 = state.transpose(-1, -2)[slot].float().contiguous()         # V-first pool rows -> [N,H,K,V] fp32
-    plan = torch.cat([lens_d, ok.to(torch.int64)[None]]).tolist()
-    skip, lens, ok = plan[0], plan[1:-1], plan[-1]
-    if not ok or skip < 0 or max(lens) < PREFILL_MIN_TOKENS:
+    if batch > 8192:
+        return None
+    lens_d = actual_seq_lengths.to(torch.int32).contiguous()
+    idx_d = ssm_state_indices.to(torch.int32).contiguous()
+    slots = torch.empty(batch, dtype=torch.int32, device=dev)
+    report = torch.empty(2 * batch + 1, dtype=torch.int32, device=dev)
+    _runtime.call_op_noalloc(
+        "recurrent_gdn_prefill_plan", OP_ARGTYPES["recurrent_gdn_prefill_plan"],
+        lambda ctx: [ctx.tensor(lens_d, "actual_seq_lengths"), ctx.tensor(idx_d, "ssm_state_indices"),
+                     ctypes.c_int64(int(blocks)), ctx.tensor(slots, "slots"), ctx.tensor(report, "report")],
+        (slots, report),
+    )
+    plan = report.tolist()
+    skip, lens, flags = plan[0], plan[1:1 + batch], plan[1 + batch:]
+    if any(flags) or skip < 0 or max(lens) < PREFILL_MIN_TOKENS:
         return None
     cu = [0]
     for n in lens:
         cu.append(cu[-1] + n)
     at = skip + cu[-1]
     head_major = lambda t: t[skip:at].transpose(0, 1)[None]            # [T,H,D] -> [1,H,T,D] view, nothing copied
-    _, o, final = gdn_chunk_fwd(head_major(query), head_major(key), head_major(value), g[skip:at][None],
-                                beta[skip:at][None].float(), scale, h0, True, cu, 64)
-    if min(lens) > 0:
-        state[slot] = final.transpose(-1, -2).to(state.dtype)
-    else:   # a sequence without tokens names no slot
-        rows = torch.tensor([i for i, n in enumerate(lens) if n > 0], dtype=torch.int64, device=dev)
-        state[slot[rows]] = final[rows].transpose(-1, -2).to(state.dtype)
+    qh, kh, vh = head_major(query), head_major(key), head_major(value)
+    gate, bet = g[skip:at][None], beta[skip:at][None].float()
+    if state.dtype == torch.float32 and state.stride(-2) == dk and state.stride(0) >= 0 and state.stride(1) >= 0:
+        # the chunk forward reads each sequence's pool row before its first token and writes it after its last one
+        o = gdn_chunk_fwd_state_pool(qh, kh, vh, gate, bet, scale, state.transpose(-1, -2), slots, cu, 64)
+    else:
+        rows = slots.to(torch.int64).clamp(min=0)
+        h0 = state.transpose(-1, -2)[rows].float().contiguous()       # V-first pool rows -> [N,H,K,V] fp32
+        _, o, final = gdn_chunk_fwd(qh, kh, vh, gate, bet, scale, h0, True, cu, 64)
+        live = torch.tensor([i for i, n in enumerate(lens) if n > 0], dtype=torch.int64, device=dev)   # an empty sequence names no row
+        state[rows[live]] = final[live].transpose(-1, -2).to(state.dtype)
     if skip == 0 and at == total:
         return o[0]
     out = torch.zeros_like(value)
     out[skip:at] = o[0]
     return out
+
+
+def gdn_chunk_fwd_state_pool(q, k, v, g, beta, scale, state_pool, state_indices, cu_seqlens, chunk_size=64,
+                             use_qk_l2norm_in_kernel=False):
+    """``gdn_chunk_fwd`` whose initial and final states are rows of ``state_pool`` (fp32 [rows,H,K,V] as a view with
+    contiguous K x V or V x K blocks), row ``state_indices[n]`` (int32, on the device) for sequence n: read before the
+    sequence's first token, overwritten after its last one; a negative index means no row.  Returns o [B,T,H,V]."""
+    B, _, T, _ = _shape(k)
+    _, HV, _, V = _shape(v)
+    o = _empty((B, T, HV, V), v)
+    cu = _as_int_tuple(cu_seqlens)
+    _call_op(
+        "gdn_chunk_fwd_state_pool", OP_ARGTYPES["gdn_chunk_fwd_state_pool"],
+        lambda ctx: [
+            ctx.tensor(q, "q"), ctx.tensor(k, "k"), ctx.tensor(v, "v"), ctx.tensor(g, "g"), ctx.tensor(beta, "beta"),
+            ctypes.c_double(float(scale)), ctx.tensor(state_pool, "state_pool"), ctx.tensor(state_indices, "state_indices"),
+            ctx.int_array(cu), ctypes.c_int64(int(chunk_size)), ctypes.c_bool(bool(use_qk_l2norm_in_kernel)), ctx.tensor(o, "o"),
+        ],
+        (o,),
+    )
+    return o
 
 
 def _chunk_local_cumsum_output_dtype(g, output_dtype):

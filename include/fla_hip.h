@@ -262,6 +262,34 @@ int fla_recurrent_gated_delta_rule(
     const fla_tensor *num_accepted_tokens, float scale, const fla_tensor *out,
     void *workspace, uint64_t workspace_size, void *stream);
 
+/* gdn_chunk_fwd_state_pool and recurrent_gdn_prefill_plan: what recurrent_gated_delta_rule needs to run the long
+ * sequences of a call (prefill) on the chunk kernels instead of token by token.  No counterpart in the reference.
+ *
+ * gdn_chunk_fwd_state_pool: gdn_chunk_fwd (operands as there) whose initial and final states are rows of one pool:
+ * state_pool f32 [rows,Hv,K,V] with contiguous K x V or V x K blocks (the recurrent operator's V-first pool is passed
+ * as its transposed view), state_indices i32 [N] on the device names the row of each sequence.  A sequence reads its
+ * row before its first token and overwrites it after its last one; a negative index means no row (zero initial state,
+ * final state dropped), an index past the pool is clamped into it.  Two sequences that name one row race.
+ *
+ * recurrent_gdn_prefill_plan: one launch over actual_seq_lengths i32 [B+1] and ssm_state_indices i32 [T] (device, as
+ * the recurrent operator takes them) that writes slots i32 [B] (the pool row of each sequence's first token, -1 for an
+ * empty or rejected sequence) and report i32 [2B+1] = {offset, length of each sequence, flag of each sequence}; a flag
+ * is 1 when the lengths are inconsistent with T, when a token of the sequence names another row than its first token,
+ * when that row is outside the pool (pool_rows) or when another sequence names it too.  B <= 8192. */
+int fla_gdn_chunk_fwd_state_pool_get_workspace_size(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, double scale, const fla_tensor *state_pool, const fla_tensor *state_indices,
+    const fla_int_array *cu_seqlens, int64_t chunk_size, bool use_qk_l2norm_in_kernel,
+    const fla_tensor *o, uint64_t *workspace_size);
+int fla_gdn_chunk_fwd_state_pool(
+    const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
+    const fla_tensor *beta, double scale, const fla_tensor *state_pool, const fla_tensor *state_indices,
+    const fla_int_array *cu_seqlens, int64_t chunk_size, bool use_qk_l2norm_in_kernel,
+    const fla_tensor *o, void *workspace, uint64_t workspace_size, void *stream);
+int fla_recurrent_gdn_prefill_plan(
+    const fla_tensor *actual_seq_lengths, const fla_tensor *ssm_state_indices, int64_t pool_rows,
+    const fla_tensor *slots, const fla_tensor *report, void *stream);
+
 /* ------------------------------------------------------------------------
  * causal_conv1d - replaces aclnnCausalConv1d (docs/aclnnCausalConv1d.md:31-48;
  * _aclnn_ctypes.py:951-985).  x [B,S,D] or [T,D] bf16/f16; weight [W,D];

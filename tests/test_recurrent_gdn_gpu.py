@@ -4,6 +4,7 @@ Shapes follow fla/ops/ascendc/gdn/recurrent_gdn/recurrent_gated_delta_rule/tests
 (T=2..., K=V=128) plus the decode benchmark layout; tolerance: bf16 out 2e-2, fp32 state 1e-3."""
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import decode as od
 from util import assert_close, TOL_BF16, TOL_STATE
@@ -274,6 +275,61 @@ def test_prefill_route_keeps_the_operator_contract(dev):
         launches("recurrent_gdn", lambda: ops.recurrent_gated_delta_rule(
             to(d["q"]), to(d["k"]), to(d["v"]), st, beta=to(d["beta"]), scale=d["scale"], actual_seq_lengths=to(d["lens"]),
             ssm_state_indices=to(idx), g=to(d["g"]), **{k_: to(v_) for k_, v_ in extra.items()}))
+
+
+def test_prefill_plan_and_pooled_forward(dev):
+    """The two entry points under the prefill route on their own: the plan's slots and flags for good and bad index
+    lists, and the chunk forward on pool rows (K x V blocks here; the route passes V x K ones) against the same forward
+    on gathered rows."""
+    import ctypes
+    from fla_hip.ops import _hip_ctypes as raw, _runtime
+
+    def plan(lens, idx, blocks, skip=0):
+        B = len(lens)
+        lens_d = torch.tensor([skip] + lens, dtype=torch.int32, device=dev)
+        idx_d = torch.tensor(idx, dtype=torch.int32, device=dev)
+        slots = torch.full((B,), 99, dtype=torch.int32, device=dev)
+        report = torch.full((2 * B + 1,), 99, dtype=torch.int32, device=dev)
+        _runtime.call_op_noalloc("recurrent_gdn_prefill_plan", raw.OP_ARGTYPES["recurrent_gdn_prefill_plan"],
+                                 lambda ctx: [ctx.tensor(lens_d), ctx.tensor(idx_d), ctypes.c_int64(blocks), ctx.tensor(slots),
+                                              ctx.tensor(report)], (slots, report))
+        r = report.tolist()
+        assert r[0] == skip and r[1:1 + B] == lens
+        return slots.tolist(), r[1 + B:]
+
+    rows = lambda lens, slots: [s for n, s in zip(lens, slots) for _ in range(n)]
+    lens = [3, 0, 5, 2]
+    assert plan(lens, [4, 4] + rows(lens, [6, 1, 0, 2]), 7, skip=2) == ([6, -1, 0, 2], [0, 0, 0, 0])
+    changing = rows(lens, [6, 1, 0, 2])
+    changing[4] = 3
+    assert plan(lens, changing, 7) == ([6, -1, -1, 2], [0, 0, 1, 0])
+    assert plan(lens, rows(lens, [6, 1, 6, 2]), 7) == ([-1, -1, -1, 2], [1, 0, 1, 0])        # two sequences on one row
+    assert plan(lens, rows(lens, [6, 1, 7, 2]), 7) == ([6, -1, -1, 2], [0, 0, 1, 0])         # a row outside the pool
+    assert plan(lens, rows(lens, [6, 1, -1, 2]), 7) == ([6, -1, -1, 2], [0, 0, 1, 0])
+    assert plan(lens, rows(lens, [6, 1, 0, 2])[:-1], 7)[1] == [1, 1, 1, 1]                   # lengths that overrun the token list
+    assert plan([3, -1, 5, 2], rows(lens, [6, 1, 0, 2]), 7)[1] == [1, 1, 1, 1]
+    big = list(range(300))
+    assert plan([1] * 300, big, 300) == (big, [0] * 300)                                      # more sequences than threads
+
+    gen = torch.Generator().manual_seed(3)
+    H, K, V, seqs = 2, 128, 128, [70, 0, 130]
+    T = sum(seqs)
+    cu = [0, 70, 70, 200]
+    q = F.normalize(torch.randn(1, H, T, K, generator=gen), dim=-1).to(BF).to(dev)
+    k = F.normalize(torch.randn(1, H, T, K, generator=gen), dim=-1).to(BF).to(dev)
+    v = torch.randn(1, H, T, V, generator=gen).to(BF).to(dev)
+    g = F.logsigmoid(torch.randn(1, T, H, generator=gen)).to(dev)
+    beta = torch.sigmoid(torch.randn(1, T, H, generator=gen)).to(dev)
+    pool0 = (torch.randn(5, H, K, V, generator=gen) * 0.1).to(dev)
+    slots = torch.tensor([3, -1, 1], dtype=torch.int32, device=dev)
+    h0 = pool0[[3, 0, 1]].clone()
+    h0[1] = 0
+    _, o_ref, final = raw.gdn_chunk_fwd(q, k, v, g, beta, K ** -0.5, h0, True, cu, 64)
+    for vfirst in (False, True):
+        pool = pool0.transpose(-1, -2).contiguous().transpose(-1, -2) if vfirst else pool0.clone()
+        o = raw.gdn_chunk_fwd_state_pool(q, k, v, g, beta, K ** -0.5, pool, slots, cu, 64)
+        assert torch.equal(o, o_ref)
+        assert torch.equal(pool[[3, 1]], final[[0, 2]]) and torch.equal(pool[[0, 2, 4]], pool0[[0, 2, 4]])
 
 
 def test_wrapper_errors(dev):
