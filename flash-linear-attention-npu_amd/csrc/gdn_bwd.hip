@@ -142,6 +142,7 @@ struct DqkwgParams {
     float *dg;
     int64_t dg_sb, dg_sh, dg_st;
     float scale;
+    int h_row = 0, dh_row = 0;   // row stride of the K x V blocks of h and dh (V, or more for a column slab of wider blocks)
     // q was l2-normalised by the caller: rstd [B,Hk,T] of that pass, and dq leaves as the gradient of the raw q
     const float *q_rstd = nullptr;
     int64_t r_sb = 0, r_sh = 0;
@@ -161,7 +162,6 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int pk = K + 16, pv = V + 8, ps = kChunk + 8;
     constexpr int KT = K / 16, KTH = KT / 2;   // column tiles of q/k: all, and per wave
-    constexpr int VF = V * VSLABS;     // full value dimension = row stride of h and dh
     elem *qS = reinterpret_cast<elem *>(smem);
     elem *kS = qS + kChunk * pk;
     elem *vS = kS + kChunk * pk;
@@ -233,8 +233,8 @@ __global__ void __launch_bounds__(kDqkwgThreads) dqkwg_kernel(const DqkwgParams 
                 tv.fetch(static_cast<const elem *>(p.v.p) + b * p.v.sb + hv * p.v.sh + (int64_t)start * p.v.st + vs * V, p.v.st, len, tid);
                 to.fetch(static_cast<const elem *>(p.d_o.p) + b * p.d_o.sb + hv * p.d_o.sh + (int64_t)start * p.d_o.st + vs * V, p.d_o.st, len, tid);
                 tdv.fetch(static_cast<const elem *>(p.dv.p) + b * p.dv.sb + hv * p.dv.sh + (int64_t)start * p.dv.st + vs * V, p.dv.st, len, tid);
-                th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc + vs * V, VF, K, tid);
-                tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc + vs * V, VF, K, tid);
+                th.fetch(p.h + b * p.h_sb + hv * p.h_sh + (int64_t)c * p.h_sc + vs * V, p.h_row, K, tid);
+                tdh.fetch(p.dh + b * p.dh_sb + hv * p.dh_sh + (int64_t)c * p.dh_sc + vs * V, p.dh_row, K, tid);
                 if (vs == 0) stage_scalars(gS, p.g, b, hv, start, len);
                 tv.commit(vS, pv, len, tid);
                 to.commit(oS, pv, len, tid);
@@ -1202,11 +1202,116 @@ int check_state5(const char *op, const char *name, const fla_tensor *h, const Ch
     int rc = check_tensor(h, op, name, 5, dt_bit(kElemDtype));
     if (rc) return rc;
     FLA_REQUIRE(h->shape[0] == geom.B && h->shape[1] == geom.Hv && h->shape[2] == geom.NT && h->shape[3] == geom.K &&
-                    h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] == geom.V && h->stride[2] % 8 == 0 &&
-                    h->stride[1] % 8 == 0 && h->stride[0] % 8 == 0,
-                FLA_ERR_SHAPE, "%s: %s must be [B,Hv,NT=%d,K,V] with contiguous K x V blocks.", op, name, geom.NT);
+                    h->shape[4] == geom.V && h->stride[4] == 1 && h->stride[3] >= geom.V && h->stride[3] % 8 == 0 &&
+                    h->stride[3] < (1 << 16) && h->stride[2] % 8 == 0 && h->stride[1] % 8 == 0 && h->stride[0] % 8 == 0 &&
+                    reinterpret_cast<uintptr_t>(h->data) % 16 == 0,
+                FLA_ERR_SHAPE, "%s: %s must be [B,Hv,NT=%d,K,V] with K x V blocks of 16-byte aligned rows.", op, name, geom.NT);
     return FLA_OK;
 }
+
+// ---- 128-token chunks with 256 value columns --------------------------------------------------------------------
+// The 128-token kernels of chunk_bwd_dqkwg and of the two WY backward operators hold 128 value columns.  With 256 the
+// launcher runs them twice, over 128 columns each: every result is either a per-column one (dv) or a sum over the value
+// columns that is linear in the column-wise operands, so the second pass (which sees zeros for the operands that do not
+// belong to the value dimension) lands in the workspace and is added to the first.  Each pass rounds its part to the
+// element type, so a sum carries one more rounding than a single pass would, at the magnitude of the parts.
+inline bool two_value_slabs(int64_t chunk_size, const fla_tensor *v) {
+    return chunk_size == 128 && v != nullptr && v->ndim == 4 && v->shape[3] == 256;
+}
+inline size_t dtype_bytes(int dtype) { return dtype == FLA_F32 || dtype == FLA_I32 ? 4 : dtype == FLA_I64 ? 8 : 2; }
+// columns [lo, lo + n) of the innermost dimension, as a view
+inline fla_tensor column_slab(const fla_tensor *t, int64_t lo, int64_t n) {
+    fla_tensor s = *t;
+    s.shape[t->ndim - 1] = n;
+    s.data = static_cast<char *>(t->data) + lo * t->stride[t->ndim - 1] * (int64_t)dtype_bytes(t->dtype);
+    return s;
+}
+// a contiguous tensor shaped like `like` except for its innermost extent and dtype, at `data`
+inline fla_tensor dense_like(const fla_tensor *like, int64_t inner, int dtype, void *data) {
+    fla_tensor s = *like;
+    s.dtype = dtype;
+    s.data = data;
+    if (inner > 0) s.shape[s.ndim - 1] = inner;
+    int64_t st = 1;
+    for (int d = s.ndim - 1; d >= 0; --d) {
+        s.stride[d] = st;
+        st *= s.shape[d];
+    }
+    return s;
+}
+inline uint64_t dense_bytes(const fla_tensor &t) {
+    uint64_t n = dtype_bytes(t.dtype);
+    for (int d = 0; d < t.ndim; ++d) n *= (uint64_t)t.shape[d];
+    return (n + 255) & ~(uint64_t)255;
+}
+
+// out[b,h,t,:] = round(out + part) for a strided [B,H,T,D] element tensor and a contiguous part (D a multiple of 8)
+__global__ void __launch_bounds__(256) add_part_kernel(View4 out, const elem *part, int H, int T, int D, int64_t rows) {
+    const int per = D / 8;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < rows * per; i += (int64_t)gridDim.x * 256) {
+        const int64_t row = i / per;
+        const int c8 = (int)(i % per) * 8;
+        const int t = (int)(row % T), h = (int)((row / T) % H);
+        const int64_t b = row / ((int64_t)T * H);
+        elem *o = static_cast<elem *>(const_cast<void *>(out.p)) + b * out.sb + h * out.sh + (int64_t)t * out.st + c8;
+        const elemx8 a = *reinterpret_cast<const elemx8 *>(o), c = *reinterpret_cast<const elemx8 *>(part + row * D + c8);
+        f32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            lo[e] = (float)a[e] + (float)c[e];
+            hi[e] = (float)a[4 + e] + (float)c[4 + e];
+        }
+        *reinterpret_cast<elemx8 *>(o) = frag_from_acc(lo, hi);
+    }
+}
+// out[b,h,t] += part for a strided fp32 [B,H,T] tensor and a contiguous part
+__global__ void __launch_bounds__(256) add_scalars_kernel(float *out, int64_t sb, int64_t sh, int64_t st, const float *part, int H,
+                                                          int T, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int t = (int)(i % T), h = (int)((i / T) % H);
+        const int64_t b = i / ((int64_t)T * H);
+        out[b * sb + h * sh + (int64_t)t * st] += part[i];
+    }
+}
+__global__ void __launch_bounds__(256) zero_fill_kernel(u32x4 *dst, int64_t n16) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) dst[i] = u32x4{0u, 0u, 0u, 0u};
+}
+int add_part(const fla_tensor *out, const fla_tensor &part, hipStream_t stream) {
+    const int64_t rows = out->shape[0] * out->shape[1] * out->shape[2];
+    if (rows == 0) return FLA_OK;
+    const unsigned blocks = (unsigned)std::min<int64_t>((rows * (out->shape[3] / 8) + 255) / 256, 8192);
+    FLA_LAUNCH("add_part", stream, add_part_kernel, dim3(blocks), dim3(256), 0, stream, view4(out), static_cast<const elem *>(part.data),
+               (int)out->shape[1], (int)out->shape[2], (int)out->shape[3], rows);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+int add_scalars(const fla_tensor *out, const fla_tensor &part, hipStream_t stream) {
+    const int64_t n = out->shape[0] * out->shape[1] * out->shape[2];
+    if (n == 0) return FLA_OK;
+    const unsigned blocks = (unsigned)std::min<int64_t>((n + 255) / 256, 4096);
+    FLA_LAUNCH("add_scalars", stream, add_scalars_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<float *>(out->data), out->stride[0],
+               out->stride[1], out->stride[2], static_cast<const float *>(part.data), (int)out->shape[1], (int)out->shape[2], n);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+int zero_fill(void *dst, uint64_t bytes, hipStream_t stream) {   // bytes: a multiple of 256
+    if (bytes == 0) return FLA_OK;
+    const int64_t n16 = (int64_t)(bytes / 16);
+    const unsigned blocks = (unsigned)std::min<int64_t>((n16 + 255) / 256, 8192);
+    FLA_LAUNCH("zero_fill", stream, zero_fill_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<u32x4 *>(dst), n16);
+    FLA_HIP_CHECK(hipGetLastError());
+    return FLA_OK;
+}
+// hands out 256-byte aligned pieces of the workspace behind the first `used` bytes
+struct Carver {
+    char *base;
+    uint64_t used;
+    void *take(uint64_t bytes) {
+        void *ptr = base ? base + used : reinterpret_cast<void *>(uintptr_t(256));   // size queries get a non-null stand-in
+        used += bytes;
+        return ptr;
+    }
+};
 
 int dv_local_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *d_o, const fla_tensor *g,
                   const fla_tensor *g_gamma, const fla_tensor *A, const fla_int_array *cu, const fla_int_array *ci,
@@ -1257,6 +1362,19 @@ int check_rstd(const char *op, const char *name, const fla_tensor *t, int64_t B,
     return FLA_OK;
 }
 
+int dqkwg_two_slabs(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+                    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
+                    const fla_int_array *ci, float scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+                    const fla_tensor *dw, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query);
+int wy_bwd_da_two_slabs(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+                        const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu, const fla_int_array *ci,
+                        int64_t chunk_size, const fla_tensor *dA, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query);
+int wy_bwd_full_two_slabs(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+                          const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu,
+                          const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+                          const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream,
+                          uint64_t *query);
+
 int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
                const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
                const fla_int_array *ci, const fla_tensor *w, const fla_tensor *g_gamma, float scale, int64_t chunk_size,
@@ -1268,6 +1386,8 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
     FLA_REQUIRE(!use_exp2, FLA_ERR_UNSUPPORTED, "%s: use_exp2 is not supported with a scalar gate.", op);
     FLA_REQUIRE(!transpose_state_layout, FLA_ERR_UNSUPPORTED, "%s: transpose_state_layout is not supported.", op);
     (void)w;   // the reference accepts w and does not read it
+    if (two_value_slabs(chunk_size, v) && !q_rstd)
+        return dqkwg_two_slabs(q, k, v, g, h, d_o, dh, dv, cu, ci, scale, chunk_size, dq, dk, dw, dg, ws, ws_size, stream, query);
     ChunkGeom geom;
     int rc;
     if ((rc = gdn_geometry(op, k, v, nullptr, chunk_size, geom, kElemDtype, 128))) return rc;   // chunk_bwd_dqkwg/README.md:117
@@ -1293,6 +1413,8 @@ int dqkwg_impl(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, co
                   static_cast<const elem *>(h->data), static_cast<const elem *>(dh->data),
                   h->stride[0], h->stride[1], h->stride[2], dh->stride[0], dh->stride[1], dh->stride[2],
                   static_cast<float *>(dg->data), dg->stride[0], dg->stride[1], dg->stride[2], scale};
+    p.h_row = (int)h->stride[3];
+    p.dh_row = (int)dh->stride[3];
     bool has_rstd;
     if ((rc = check_rstd(op, "q_rstd", q_rstd, geom.B, geom.Hk, geom.T, has_rstd))) return rc;
     if (has_rstd) {
@@ -1359,6 +1481,7 @@ int wy_bwd_da_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor *b
     ChunkGeom geom;
     int rc;
     FLA_REQUIRE(A != nullptr && A->data != nullptr, FLA_ERR_NULL, "%s: A must not be null.", op);
+    if (two_value_slabs(chunk_size, v)) return wy_bwd_da_two_slabs(k, v, beta, A, dw, du, g, cu, ci, chunk_size, dA, ws, ws_size, stream, query);
     if ((rc = wy_bwd_common(op, k, v, beta, A, dw, du, g, chunk_size, geom))) return rc;
     if ((rc = check_bhtd(op, "dA", dA, geom.B, geom.Hv, geom.T, geom.C, dt_bit(kElemDtype)))) return rc;
     Varlen vl;
@@ -1394,6 +1517,8 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     // A absent (only together with dA, below): the kernel rebuilds the chunk's inverse from k, g and beta
     const bool has_a = A && A->data;
     FLA_REQUIRE(has_a || !(dA && dA->data), FLA_ERR_NULL, "%s: A must not be null when dA is given.", op);
+    if (two_value_slabs(chunk_size, v) && !accumulate)
+        return wy_bwd_full_two_slabs(k, v, beta, A, dA, dw, du, g, cu, ci, chunk_size, dk, dv, dbeta, dg, ws, ws_size, stream, query);
     if ((rc = wy_bwd_common(op, k, v, beta, has_a ? A : nullptr, dw, du, g, chunk_size, geom))) return rc;
     const int bf = dt_bit(kElemDtype);
     // dA absent (the accumulating form on 64-token chunks only): the kernel forms prepare_wy_repr_bwd_da's result itself
@@ -1446,6 +1571,123 @@ int wy_bwd_full_impl(const fla_tensor *k, const fla_tensor *v, const fla_tensor 
     if (K == 128 && V == 256) FLA_WY_FULL(128, 256, true);
 #undef FLA_WY_FULL
     return fail(FLA_ERR_UNSUPPORTED, "%s: (K,V)=(%d,%d) has no kernel; built: (128,128),(64,64),(64,128),(128,256).", op, K, V);
+}
+
+int dqkwg_two_slabs(const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
+                    const fla_tensor *d_o, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu,
+                    const fla_int_array *ci, float scale, int64_t chunk_size, const fla_tensor *dq, const fla_tensor *dk,
+                    const fla_tensor *dw, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "chunk_bwd_dqkwg";
+    const fla_tensor *need[] = {q, k, v, g, h, d_o, dh, dv, dq, dk, dw, dg};
+    for (const fla_tensor *t : need) FLA_REQUIRE(t != nullptr && t->data != nullptr, FLA_ERR_NULL, "%s: an operand is null.", op);
+    FLA_REQUIRE(d_o->ndim == 4 && dv->ndim == 4 && h->ndim == 5 && dh->ndim == 5 && d_o->shape[3] == 256 && dv->shape[3] == 256 &&
+                    h->shape[4] == 256 && dh->shape[4] == 256 && dq->ndim == 4 && dk->ndim == 4 && dw->ndim == 4 && dg->ndim == 3,
+                FLA_ERR_SHAPE, "%s: dox, dv, h and dh must carry the 256 value columns of v.", op);
+    int rc;
+    fla_tensor vs[2], os[2], dvs[2], hs[2], dhs[2];
+    for (int i = 0; i < 2; ++i) {
+        vs[i] = column_slab(v, 128 * i, 128);
+        os[i] = column_slab(d_o, 128 * i, 128);
+        dvs[i] = column_slab(dv, 128 * i, 128);
+        hs[i] = column_slab(h, 128 * i, 128);
+        dhs[i] = column_slab(dh, 128 * i, 128);
+    }
+    uint64_t meta = 0;
+    if ((rc = dqkwg_impl(q, k, &vs[0], g, &hs[0], &os[0], &dhs[0], &dvs[0], cu, ci, nullptr, nullptr, scale, chunk_size, false, false,
+                         dq, dk, dw, dg, nullptr, 0, nullptr, &meta)))
+        return rc;
+    Carver carve{static_cast<char *>(query ? nullptr : ws), (meta + 255) & ~(uint64_t)255};
+    fla_tensor dq2 = dense_like(dq, 0, dq->dtype, nullptr), dk2 = dense_like(dk, 0, dk->dtype, nullptr),
+               dw2 = dense_like(dw, 0, dw->dtype, nullptr), dg2 = dense_like(dg, 0, FLA_F32, nullptr);
+    dq2.data = carve.take(dense_bytes(dq2));
+    dk2.data = carve.take(dense_bytes(dk2));
+    dw2.data = carve.take(dense_bytes(dw2));
+    dg2.data = carve.take(dense_bytes(dg2));
+    if (query) {
+        *query = carve.used;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(ws && ws_size >= carve.used, FLA_ERR_WORKSPACE, "%s: workspace of %llu bytes required.", op, (unsigned long long)carve.used);
+    if ((rc = dqkwg_impl(q, k, &vs[0], g, &hs[0], &os[0], &dhs[0], &dvs[0], cu, ci, nullptr, nullptr, scale, chunk_size, false, false, dq, dk,
+                         dw, dg, ws, meta, stream, nullptr)))
+        return rc;
+    if ((rc = dqkwg_impl(q, k, &vs[1], g, &hs[1], &os[1], &dhs[1], &dvs[1], cu, ci, nullptr, nullptr, scale, chunk_size, false, false, &dq2,
+                         &dk2, &dw2, &dg2, ws, meta, stream, nullptr)))
+        return rc;
+    if ((rc = add_part(dq, dq2, stream)) || (rc = add_part(dk, dk2, stream)) || (rc = add_part(dw, dw2, stream))) return rc;
+    return add_scalars(dg, dg2, stream);
+}
+
+int wy_bwd_da_two_slabs(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dw,
+                        const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu, const fla_int_array *ci,
+                        int64_t chunk_size, const fla_tensor *dA, void *ws, uint64_t ws_size, hipStream_t stream, uint64_t *query) {
+    const char *op = "prepare_wy_repr_bwd_da";
+    const fla_tensor *need[] = {k, v, beta, A, dw, du, g, dA};
+    for (const fla_tensor *t : need) FLA_REQUIRE(t != nullptr && t->data != nullptr, FLA_ERR_NULL, "%s: an operand is null.", op);
+    FLA_REQUIRE(du->ndim == 4 && du->shape[3] == 256 && dw->ndim == 4 && dA->ndim == 4, FLA_ERR_SHAPE,
+                "%s: du must carry the 256 value columns of v.", op);
+    int rc;
+    fla_tensor vs[2] = {column_slab(v, 0, 128), column_slab(v, 128, 128)}, dus[2] = {column_slab(du, 0, 128), column_slab(du, 128, 128)};
+    uint64_t meta = 0;
+    if ((rc = wy_bwd_da_impl(k, &vs[0], beta, A, dw, &dus[0], g, cu, ci, chunk_size, dA, nullptr, 0, nullptr, &meta))) return rc;
+    Carver carve{static_cast<char *>(query ? nullptr : ws), (meta + 255) & ~(uint64_t)255};
+    fla_tensor zero_dw = dense_like(dw, 0, dw->dtype, nullptr), part = dense_like(dA, 0, dA->dtype, nullptr);
+    const uint64_t zero_bytes = dense_bytes(zero_dw);
+    zero_dw.data = carve.take(zero_bytes);
+    part.data = carve.take(dense_bytes(part));
+    if (query) {
+        *query = carve.used;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(ws && ws_size >= carve.used, FLA_ERR_WORKSPACE, "%s: workspace of %llu bytes required.", op, (unsigned long long)carve.used);
+    if ((rc = zero_fill(zero_dw.data, zero_bytes, stream))) return rc;
+    if ((rc = wy_bwd_da_impl(k, &vs[0], beta, A, dw, &dus[0], g, cu, ci, chunk_size, dA, ws, meta, stream, nullptr))) return rc;
+    if ((rc = wy_bwd_da_impl(k, &vs[1], beta, A, &zero_dw, &dus[1], g, cu, ci, chunk_size, &part, ws, meta, stream, nullptr))) return rc;
+    return add_part(dA, part, stream);
+}
+
+int wy_bwd_full_two_slabs(const fla_tensor *k, const fla_tensor *v, const fla_tensor *beta, const fla_tensor *A, const fla_tensor *dA,
+                          const fla_tensor *dw, const fla_tensor *du, const fla_tensor *g, const fla_int_array *cu,
+                          const fla_int_array *ci, int64_t chunk_size, const fla_tensor *dk, const fla_tensor *dv,
+                          const fla_tensor *dbeta, const fla_tensor *dg, void *ws, uint64_t ws_size, hipStream_t stream,
+                          uint64_t *query) {
+    const char *op = "prepare_wy_repr_bwd_full";
+    const fla_tensor *need[] = {k, v, beta, A, dA, dw, du, g, dk, dv, dbeta, dg};
+    for (const fla_tensor *t : need) FLA_REQUIRE(t != nullptr && t->data != nullptr, FLA_ERR_NULL, "%s: an operand is null.", op);
+    FLA_REQUIRE(du->ndim == 4 && du->shape[3] == 256 && dv->ndim == 4 && dv->shape[3] == 256 && dw->ndim == 4 && dA->ndim == 4 &&
+                    dk->ndim == 4 && dbeta->ndim == 3 && dg->ndim == 3,
+                FLA_ERR_SHAPE, "%s: du and dv must carry the 256 value columns of v.", op);
+    int rc;
+    fla_tensor vs[2], dus[2], dvs[2];
+    for (int i = 0; i < 2; ++i) {
+        vs[i] = column_slab(v, 128 * i, 128);
+        dus[i] = column_slab(du, 128 * i, 128);
+        dvs[i] = column_slab(dv, 128 * i, 128);
+    }
+    uint64_t meta = 0;
+    if ((rc = wy_bwd_full_impl(k, &vs[0], beta, A, dA, dw, &dus[0], g, cu, ci, chunk_size, dk, &dvs[0], dbeta, dg, nullptr, 0, nullptr, &meta)))
+        return rc;
+    Carver carve{static_cast<char *>(query ? nullptr : ws), (meta + 255) & ~(uint64_t)255};
+    // the second pass reads zeros for dA and dw (one zeroed piece serves both) and drops its dk and dg
+    fla_tensor zero_dw = dense_like(dw, 0, dw->dtype, nullptr), zero_da = dense_like(dA, 0, dA->dtype, nullptr);
+    const uint64_t zero_bytes = std::max(dense_bytes(zero_dw), dense_bytes(zero_da));
+    zero_dw.data = zero_da.data = carve.take(zero_bytes);
+    fla_tensor dk2 = dense_like(dk, 0, dk->dtype, nullptr), db2 = dense_like(dbeta, 0, FLA_F32, nullptr), dg2 = dense_like(dg, 0, FLA_F32, nullptr);
+    dk2.data = carve.take(dense_bytes(dk2));
+    db2.data = carve.take(dense_bytes(db2));
+    dg2.data = carve.take(dense_bytes(dg2));
+    if (query) {
+        *query = carve.used;
+        return FLA_OK;
+    }
+    FLA_REQUIRE(ws && ws_size >= carve.used, FLA_ERR_WORKSPACE, "%s: workspace of %llu bytes required.", op, (unsigned long long)carve.used);
+    if ((rc = zero_fill(zero_dw.data, zero_bytes, stream))) return rc;
+    if ((rc = wy_bwd_full_impl(k, &vs[0], beta, A, dA, dw, &dus[0], g, cu, ci, chunk_size, dk, &dvs[0], dbeta, dg, ws, meta, stream, nullptr)))
+        return rc;
+    if ((rc = wy_bwd_full_impl(k, &vs[1], beta, A, &zero_da, &zero_dw, &dus[1], g, cu, ci, chunk_size, &dk2, &dvs[1], &db2, &dg2, ws, meta,
+                               stream, nullptr)))
+        return rc;
+    return add_scalars(dbeta, db2, stream);
 }
 
 // da + full in one call: dA (bf16, transposed like the stand-alone operator writes it) lives in the caller's workspace

@@ -1178,19 +1178,6 @@ def _as_dtype(out, like):
     return out if out.dtype == like.dtype else out.to(like.dtype)
 
 
-def _two_value_passes(v, chunk_size) -> bool:
-    """The 128-token forms of chunk_bwd_dqkwg and of the WY backward operators hold 128 value columns.  With 256 they run
-    twice, over 128 columns each: every result is either a per-column one (dv) or a sum over the value columns that is
-    linear in the column-wise operands, so the two passes add up (the second one sees zeros for the operands that do
-    not belong to the value dimension).  Each pass returns its part in the 16-bit element type, so a sum carries one more
-    rounding than a single pass, at the magnitude of the parts: visible where the two parts nearly cancel."""
-    return int(chunk_size) == 128 and int(v.shape[-1]) == 256
-
-
-def _add_as(a, b, like):
-    return (a.float() + b.float()).to(like.dtype)
-
-
 def npu_chunk_bwd_dv_local(q, k, d_o, g, scale, chunk_size, *, g_gamma=None, A=None, cu_seqlens=None,
                            chunk_indices=None):
     """_aclnn_ctypes.py:397-427.  q, k [B,Hk,T,K]; d_o [B,Hv,T,V]; g [B,Hv,T] chunk-cumsummed."""
@@ -1211,13 +1198,6 @@ def npu_chunk_bwd_dv_local(q, k, d_o, g, scale, chunk_size, *, g_gamma=None, A=N
 
 def npu_prepare_wy_repr_bwd_da(k, v, beta, A, dw, du, g, *, chunk_size, cu_seqlens=None, chunk_indices=None):
     """_aclnn_ctypes.py:430-460.  Returns dA [B,Hv,T,C], stored transposed as the reference does."""
-    if _two_value_passes(v, chunk_size):
-        import torch
-
-        kw = dict(chunk_size=chunk_size, cu_seqlens=cu_seqlens, chunk_indices=chunk_indices)
-        first = npu_prepare_wy_repr_bwd_da(k, v[..., :128], beta, A, dw, du[..., :128], g, **kw)
-        second = npu_prepare_wy_repr_bwd_da(k, v[..., 128:], beta, A, torch.zeros_like(dw), du[..., 128:], g, **kw)
-        return _add_as(first, second, A)
     out = _empty_like(A)
     return _call_op(
         "prepare_wy_repr_bwd_da", OP_ARGTYPES["prepare_wy_repr_bwd_da"],
@@ -1234,15 +1214,6 @@ def npu_prepare_wy_repr_bwd_da(k, v, beta, A, dw, du, g, *, chunk_size, cu_seqle
 def npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):
     """_aclnn_ctypes.py:242-279.  Returns (dk, dv, dbeta, dg); dbeta and dg are computed in fp32 and
     returned in the dtype of beta and g."""
-    if _two_value_passes(v, chunk_size):
-        import torch
-
-        kw = dict(cu_seqlens=cu_seqlens, chunk_indices=chunk_indices)
-        dk, dv1, db1, dg = npu_prepare_wy_repr_bwd_full(k, v[..., :128], beta.float(), A, dA, dw, du[..., :128], g.float(),
-                                                        chunk_size, **kw)
-        _, dv2, db2, _ = npu_prepare_wy_repr_bwd_full(k, v[..., 128:], beta.float(), A, torch.zeros_like(dA),
-                                                      torch.zeros_like(dw), du[..., 128:], g.float(), chunk_size, **kw)
-        return dk, torch.cat([dv1, dv2], dim=-1), _as_dtype(db1 + db2, beta), _as_dtype(dg, g)
     dk = _empty_ordered_like(k)
     dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
@@ -1313,10 +1284,6 @@ def chunk_bwd_dqkwg_l2norm(q, k, v, g, h, dox, dh, dv, q_rstd, chunk_size, *, sc
 def npu_prepare_wy_repr_bwd(k, v, beta, A, dw, du, g, chunk_size, *, cu_seqlens=None, chunk_indices=None):
     """_aclnn_ctypes.py:284-321: bwd_da and bwd_full in one library call (dA stays in the workspace).
     Returns (dk, dv, dbeta, dg) like npu_prepare_wy_repr_bwd_full."""
-    if _two_value_passes(v, chunk_size):
-        kw = dict(cu_seqlens=cu_seqlens, chunk_indices=chunk_indices)
-        dA = npu_prepare_wy_repr_bwd_da(k, v, beta, A, dw, du, g, chunk_size=chunk_size, **kw)
-        return npu_prepare_wy_repr_bwd_full(k, v, beta, A, dA, dw, du, g, chunk_size, **kw)
     dk = _empty_ordered_like(k)
     dv = _empty_ordered_like(v)
     dbeta = _f32_like(beta)
@@ -1341,12 +1308,6 @@ def npu_chunk_bwd_dqkwg(q, k, v, g, h, dox, dh, dv, chunk_size, *, cu_seqlens=No
     """_aclnn_ctypes.py:463-510.  Returns (dq, dk [B,Hk,T,K], dw [B,Hv,T,K], dg [B,Hv,T]); ``v`` is v_new."""
     if g_gamma is not None:
         raise NotImplementedError("npu_chunk_bwd_dqkwg: g_gamma is not supported.")
-    if _two_value_passes(v, chunk_size) and not _optional_bool(transpose_state_layout, False):
-        kw = dict(cu_seqlens=cu_seqlens, chunk_indices=chunk_indices, w=w, scale=scale, use_exp2=use_exp2)
-        parts = [npu_chunk_bwd_dqkwg(q, k, v[..., c], g.float(), h[..., c].contiguous(), dox[..., c], dh[..., c].contiguous(),
-                                     dv[..., c], chunk_size, **kw) for c in (slice(0, 128), slice(128, 256))]
-        (dq1, dk1, dw1, dg1), (dq2, dk2, dw2, dg2) = parts
-        return _add_as(dq1, dq2, q), _add_as(dk1, dk2, k), _add_as(dw1, dw2, q), _as_dtype(dg1 + dg2, g)
     q_shape = _shape(q)
     value_num_heads = int(v.shape[1])
     dq = _empty_ordered_like(q)

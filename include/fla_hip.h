@@ -677,7 +677,11 @@ int fla_chunk_bwd_dv_local(
 /* chunk_bwd_dqkwg - replaces aclnnChunkBwdDqkwg (_aclnn_ctypes.py:463-510).  v is v_new of the
  * forward scan, h the state at each chunk start, dh / dv the outputs of bwd_dhu; dg [B,Hv,T] f32 is the
  * gradient of the cumsummed gate.  w and g_gamma must be NULL or are ignored as in the reference;
- * use_exp2 and transpose_state_layout must be false. */
+ * use_exp2 and transpose_state_layout must be false.  h and dh: K x V blocks whose rows may be wider than V (a column
+ * slab of wider blocks), 16-byte aligned.  chunk_size 128 with V = 256 (also in prepare_wy_repr_bwd_da / _full and
+ * prepare_wy_repr_bwd): the launcher runs the 128-column kernels over the two halves of the value dimension and adds
+ * the second pass, which lands in the workspace (reported by the size query), to the first; each pass rounds its part
+ * to the element type. */
 int fla_chunk_bwd_dqkwg_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g, const fla_tensor *h,
     const fla_tensor *dox, const fla_tensor *dh, const fla_tensor *dv, const fla_int_array *cu_seqlens,
