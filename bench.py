@@ -44,6 +44,7 @@ MEASURED_TRAFFIC = {
     "gdn_fused": (881e6 + 311e6, "profiles/gdn_pipe_kernel_B4_T8192_H32_K128_V128.md"),
     "recurrent_gdn": (544e6 + 539e6, "profiles/recurrent_gdn_kernel_decode_256x32x128x128.md"),
     "conv1d_fwd": (147e6 + 134e6, "profiles/conv1d_dense_kernel_B4_T4096_D4096_W4_silu.md"),
+    "kda_intra": (689e6 + 944e6, "profiles/kda_kernels_B2_T8192_H32_K128_V128.md"),
 }
 
 
@@ -279,7 +280,8 @@ def bench_decode(args, torch, dev):
         cdt = time.perf_counter() - t1
         cpu = {"value": round(ns * reps / cdt, 1), "unit": "tokens/s", "cores": cores, "kind": "port",
                "sample": f"{reps} x ({ns} sequences x 1 token, H=32 K=V=128) fp32 torch oracle, {cdt:.1f} s"}
-    # the same kernel as a variable-length prefill: 64 sequences, lengths uniform in [128, 4096]
+    # the same operator as a variable-length prefill (it routes such a call to the chunk forward): 64 sequences, lengths
+    # uniform in [128, 4096]
     gl = torch.Generator().manual_seed(0)
     plens = torch.randint(128, 4097, (64,), generator=gl)
     PT = int(plens.sum())
@@ -581,7 +583,8 @@ def bench_kda(args, torch, dev):
         "step_GBps": round(step_gbps, 1), "step_frac_of_hbm_peak": round(step_gbps / PEAK_HBM_GBS, 4),
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": round(kbytes[dominant] / (kern[dominant] * 1e-3) / 1e9, 1),
                      "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(kbytes[dominant] / (kern[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "traffic": None,
+                     "frac": round(kbytes[dominant] / (kern[dominant] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                     "traffic": measured_traffic(dominant)[0], "traffic_source": measured_traffic(dominant)[1],
                      "avg_kernel_ms": round(kern[dominant], 4),
                      "against_bf16_peak": {"achieved_tflops": round(ach, 2), "frac": round(ach / PEAK_BF16_TFLOPS, 4)}},
         "other_kernels_ms": {n: round(t, 4) for n, t in kern.items()},
