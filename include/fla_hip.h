@@ -385,7 +385,9 @@ int fla_chunk_gated_delta_rule_bwd_dhu(
  * Aqk, Akk [..HV,T,chunk], w, qg, kg [..HV,T,K], u, v_new [..HV,T,V], and
  * h [B,NT,HV,K,V] (rank-3 layouts: [NT,HV,K,V]).  final_state, gk, w, u, qg,
  * kg, v_new and h may be null.  Implemented: bf16 or f16 q/k/v, chunk_size 64
- * and 128, K in {64,128} with V in {K, 2K}, and K = V = 256.
+ * and 128, K in {64,128} with V in {K, 2K}, and K = V = 256.  With bf16
+ * inputs and K <= 128, qg and kg may also be f16 tensors (11-bit significands
+ * for the reverse scan of a training step, see chunk_kda_bwd_dhu).
  * ------------------------------------------------------------------------ */
 int fla_chunk_kda_fwd_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *v, const fla_tensor *g,
@@ -526,8 +528,9 @@ int fla_chunk_kda_bwd_dqkwg(
 /* chunk_kda_bwd_dhu: chunk_gated_delta_rule_bwd_dhu with the per-channel gate gK (log2 units, use_exp2) whose dv
  * operand, dv = Aqk^T d_o per chunk (the second result of chunk_kda_bwd_dav), is formed inside the scan from the
  * forward's score blocks Aqk [B,Hv,T,64] and the d_o tiles it stages anyway, so that dv never goes through memory.
- * No counterpart in the reference (see the note above); q, k are the gated qg, kg of the forward.  chunk_size 64,
- * K in {64,128}.  Outputs as chunk_gated_delta_rule_bwd_dhu. */
+ * No counterpart in the reference (see the note above); q, k are the gated qg, kg of the forward, in the element type
+ * of w and d_o or both f16 beside bf16 w and d_o (the tensors chunk_kda_fwd writes when asked for f16 qg, kg).
+ * chunk_size 64, K in {64,128}.  Outputs as chunk_gated_delta_rule_bwd_dhu. */
 int fla_chunk_kda_bwd_dhu_get_workspace_size(
     const fla_tensor *q, const fla_tensor *k, const fla_tensor *w, const fla_tensor *d_o, const fla_tensor *Aqk,
     const fla_tensor *gK, const fla_tensor *h0, const fla_tensor *dht, const fla_int_array *cu_seqlens,
