@@ -232,6 +232,90 @@ def test_library_rejects_null_and_bad_descriptors_without_a_gpu(lib):
     assert b"chunk_size must be 64" in lib.fla_last_error()
 
 
+def _descriptor(shape, dtype_code, data=4096, strides=None):
+    """A descriptor over a pointer that is never dereferenced (validation and size queries only)."""
+    from fla_hip.ops._runtime import FlaTensor
+    t = FlaTensor()
+    t.data, t.dtype, t.ndim = data, dtype_code, len(shape)
+    st = 1
+    for i in reversed(range(len(shape))):
+        t.shape[i] = shape[i]
+        t.stride[i] = st if strides is None else strides[i]
+        st *= shape[i]
+    return t
+
+
+def test_value_slab_workspace_and_new_entries_without_a_gpu(lib):
+    """Size queries and validation of the entry points that loop value slabs or serve the prefill route; nothing is
+    launched.  chunk_bwd_dqkwg with 128-token chunks and V = 256 asks for room for the second pass (dq, dk, dw in the
+    element type and dg in fp32, each rounded up to 256 bytes)."""
+    from fla_hip.ops._runtime import TENSOR_P, INT_ARRAY_P
+    from fla_hip.ops import _hip_ctypes as H
+    lib.fla_last_error.restype = ctypes.c_char_p
+    BF, F32, I32 = 2, 0, 3
+    p = ctypes.pointer
+    B, Hh, T, K, V = 1, 2, 256, 128, 256
+    qk = _descriptor((B, Hh, T, K), BF)
+    vv = _descriptor((B, Hh, T, V), BF)
+    g = _descriptor((B, Hh, T), F32)
+    h = _descriptor((B, Hh, 2, K, V), BF)
+    ws = ctypes.c_uint64(0)
+    fn = lib.fla_chunk_bwd_dqkwg_get_workspace_size
+    fn.restype = ctypes.c_int
+    fn.argtypes = [*H.OP_ARGTYPES["chunk_bwd_dqkwg"], ctypes.POINTER(ctypes.c_uint64)]
+    null, nia = TENSOR_P(), INT_ARRAY_P()
+    args = [p(qk), p(qk), p(vv), p(g), p(h), p(vv), p(h), p(vv), nia, nia, null, null, 1.0, 128, False, False,
+            p(qk), p(qk), p(qk), p(g)]
+    assert fn(*args, ctypes.byref(ws)) == 0, lib.fla_last_error()
+    assert ws.value == 3 * B * Hh * T * K * 2 + B * Hh * T * 4
+    args[13] = 64                                     # 64-token chunks: one pass, the kernel walks both slabs itself
+    h64 = _descriptor((B, Hh, 4, K, V), BF)
+    args[4] = args[6] = p(h64)
+    assert fn(*args, ctypes.byref(ws)) == 0 and ws.value == 0
+
+    fn = lib.fla_gdn_chunk_fwd_state_pool_get_workspace_size
+    fn.restype = ctypes.c_int
+    fn.argtypes = [*H.OP_ARGTYPES["gdn_chunk_fwd_state_pool"], ctypes.POINTER(ctypes.c_uint64)]
+    q4 = _descriptor((1, Hh, T, K), BF)
+    gate = _descriptor((1, T, Hh), F32)
+    o = _descriptor((1, T, Hh, K), BF)
+    pool = _descriptor((5, Hh, K, K), F32, strides=(Hh * K * K, K * K, 1, K))      # V-first rows seen as [rows,H,K,V]
+    idx = _descriptor((1,), I32)
+    assert fn(p(q4), p(q4), p(q4), p(gate), p(gate), 0.1, p(pool), null, nia, 64, False, p(o), ctypes.byref(ws)) == 1
+    assert b"state_indices must not be null" in lib.fla_last_error()
+    assert fn(p(q4), p(q4), p(q4), p(gate), p(gate), 0.1, p(pool), p(idx), nia, 64, False, p(o), ctypes.byref(ws)) == 0
+    bad_pool = _descriptor((5, Hh, K, K), F32, strides=(Hh * K * K, K * K, 2 * K, 2))
+    assert fn(p(q4), p(q4), p(q4), p(gate), p(gate), 0.1, p(bad_pool), p(idx), nia, 64, False, p(o), ctypes.byref(ws)) == 3
+    two = _descriptor((2,), I32)                     # one sequence, two indices
+    assert fn(p(q4), p(q4), p(q4), p(gate), p(gate), 0.1, p(pool), p(two), nia, 64, False, p(o), ctypes.byref(ws)) == 3
+
+    plan = lib.fla_recurrent_gdn_prefill_plan
+    plan.restype = ctypes.c_int
+    plan.argtypes = [*H.OP_ARGTYPES["recurrent_gdn_prefill_plan"], ctypes.c_void_p]
+    lens = _descriptor((9000,), I32)
+    assert plan(p(lens), p(idx), 4, p(_descriptor((8999,), I32)), p(_descriptor((17999,), I32)), None) == 4
+    assert b"between 1 and 8192 sequences" in lib.fla_last_error()
+    lens = _descriptor((3,), I32)
+    assert plan(p(lens), p(idx), 4, p(_descriptor((2,), I32)), p(_descriptor((4,), I32)), None) == 3   # report must be [2B+1]
+    assert plan(p(lens), p(idx), 0, p(_descriptor((2,), I32)), p(_descriptor((5,), I32)), None) == 3   # empty pool
+
+    fn = lib.fla_chunk_kda_bwd_dqkwg_wy_intra_get_workspace_size
+    fn.restype = ctypes.c_int
+    fn.argtypes = [*H.OP_ARGTYPES["chunk_kda_bwd_dqkwg_wy_intra"], ctypes.POINTER(ctypes.c_uint64)]
+    T2 = 128
+    x = _descriptor((1, Hh, T2, K), BF)
+    f = _descriptor((1, Hh, T2, K), F32)
+    a = _descriptor((1, Hh, T2, 64), BF)
+    hb = _descriptor((1, Hh, 2, K, K), BF)
+    beta = _descriptor((1, Hh, T2), F32)
+    db = _descriptor((1, Hh, T2), F32)
+    base = [p(x), p(x), p(x), p(f), p(hb), p(x), p(hb), p(x), p(x), p(beta), p(a), nia, nia, 0.1, 64]
+    assert fn(*base, p(f), p(f), p(f), p(x), p(db), ctypes.byref(ws)) == 0, lib.fla_last_error()
+    assert fn(*base, p(x), p(x), p(f), p(x), p(db), ctypes.byref(ws)) == 0          # dq, dk in the element type
+    assert fn(*base, p(x), p(f), p(f), p(x), p(db), ctypes.byref(ws)) == 2          # one of each
+    assert b"dq and dk must share one dtype" in lib.fla_last_error()
+
+
 def test_cpu_tensors_are_rejected():
     from fla_hip import ops
     x = torch.zeros(1, 4, 16, dtype=torch.bfloat16)
