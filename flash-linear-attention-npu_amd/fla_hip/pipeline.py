@@ -301,7 +301,8 @@ def _from_index_order(x, layout):
 
 def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, dht=None, *, initial_state=None,
                   layout="BSND", cu_seqlens=None, chunk_size: int = 64):
-    """KDA chunk backward from the tensors the forward keeps (``chunk_kda_fwd(..., disable_recompute=True)``).
+    """KDA chunk backward from the tensors the forward keeps (``chunk_kda_fwd(..., disable_recompute=True)``), on 64- or
+    128-token chunks (with 128 only q, k, v, beta, gk and the initial state of what is passed are used, see below).
 
     q, k, v, beta, do in ``layout``; gk, Aqk, Akk, w, qg, kg, v_new head-major and h as the forward returned them;
     dht fp32 [N,Hv,K,V] or None.  Returns ``(dq, dk, dv, dg, dbeta, dh0)``: dq, dk, dv, dbeta in ``layout`` and the
@@ -311,9 +312,19 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
     chunk-local cumulative sum of dg; up to 128 channels the stages after the scan are one launch."""
     import torch
 
-    if chunk_size != 64:
-        raise NotImplementedError("chunk_kda_bwd: the backward operators are built for chunk_size 64.")
     cu = _cu_list(cu_seqlens)
+    if chunk_size == 128:
+        # The gradient kernels take 64-token tiles (as the reference's own backward kernel, _aclnn_ctypes.py:1582-1584).
+        # What the forward kept on 128-token chunks (Aqk, Akk, w, qg, kg, v_new, h) tiles the same function differently,
+        # so those intermediates are formed again on 64-token chunks from q, k, v, beta and the per-token gate, which the
+        # cumulated gate determines: g_t = ln2 (gk_t - gk_{t-1}), and g_t = ln2 gk_t on the first token of a 128-token chunk.
+        g_raw = _per_token_gate(gk, 128, cu, layout)
+        f = _raw.chunk_kda_fwd_for_backward(q, k, v, g_raw, beta, float(scale), 64, layout=layout, initial_state=initial_state,
+                                            cu_seqlens=cu)
+        _, _, gk, Aqk, Akk, w, _, qg, kg, v_new, h, _ = f
+        chunk_size = 64
+    if chunk_size != 64:
+        raise NotImplementedError("chunk_kda_bwd: chunk_size must be 64 or 128.")
     kw = dict(cu_seqlens=cu)
     rank3 = layout in ("TND", "NTD")
     hm = lambda t: _index_order(t, layout)
@@ -362,6 +373,23 @@ def chunk_kda_bwd(q, k, v, beta, gk, Aqk, Akk, w, qg, kg, v_new, h, scale, do, d
         dq = dq.unflatten(1, (Hk, Hv // Hk)).sum(2).to(q.dtype)
         dk = dk.unflatten(1, (Hk, Hv // Hk)).sum(2).to(k.dtype)
     return (back(dq), back(dk), back(dv), back(dg), back(db[..., None])[..., 0].to(beta.dtype), dh0)
+
+
+def _per_token_gate(gk, chunk_size, cu, layout):
+    """The per-token log decay (natural log, in ``layout``) behind a chunk-local cumulated gate ``gk`` (head-major
+    [..,Hv,T,K] fp32 in log2 units, cumulated over ``chunk_size``-token chunks that restart with every sequence)."""
+    import math
+
+    import torch
+
+    g4 = gk if gk.dim() == 4 else gk[None]
+    T = g4.shape[2]
+    first = torch.zeros(T, dtype=torch.bool, device=gk.device)
+    for bos, eos in ([(0, T)] if cu is None else zip(cu[:-1], cu[1:])):
+        first[bos:eos:chunk_size] = True
+    prev = torch.cat([torch.zeros_like(g4[:, :, :1]), g4[:, :, :-1]], dim=2)
+    raw = (g4 - torch.where(first[None, None, :, None], torch.zeros_like(prev), prev)) * math.log(2.0)
+    return _from_index_order(raw, layout).contiguous()
 
 
 def _kda_bwd_state_stages_by_channel_halves(qh, kh, vh, bh, gk4, Akk4, vn4, h5, doh, dh, dv2, scale, chunk_size, layout_like, kw):

@@ -436,6 +436,39 @@ def test_chunk_kda_gradients_through_the_gate_activation(dev, safe, layout, K, V
         close(a, e, name)
 
 
+@pytest.mark.parametrize("layout,cu", [("BSND", None), ("TND", [0, 70, 70, 300, 421])])
+def test_chunk_kda_bwd_from_a_forward_on_128_token_chunks(dev, layout, cu):
+    """chunk_kda_bwd fed with what a forward on 128-token chunks kept: the gradients are those of the same function, so
+    they agree with the route through 64-token chunks (the gate is cumulated, differenced and cumulated again on the way)."""
+    from fla_hip import ops, pipeline
+    B, T, Hk, Hv, K, V = (1 if cu else 2), (421 if cu else 330), 2, 4, 128, 128
+    gen = torch.Generator().manual_seed(11)
+    q = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
+    k = F.normalize(torch.randn(B, Hk, T, K, generator=gen), dim=-1).to(BF)
+    v = torch.randn(B, Hv, T, V, generator=gen).to(BF)
+    gate = F.logsigmoid(torch.randn(B, Hv, T, K, generator=gen)) * 0.5
+    beta = torch.sigmoid(torch.randn(B, Hv, T, generator=gen))
+    do = torch.randn(B, Hv, T, V, generator=gen).to(BF)
+    N = B if cu is None else len(cu) - 1
+    h0 = (torch.randn(N, Hv, K, V, generator=gen) * 0.1).to(dev)
+    dht = (torch.randn(N, Hv, K, V, generator=gen) * 0.1).to(dev)
+    ins = [lay(t, layout).to(dev) for t in (q, k, v, gate, beta)]
+    scale = K ** -0.5
+    results = {}
+    for C in (64, 128):
+        f = ops.chunk_kda_fwd(*ins, scale, C, layout=layout, initial_state=h0, output_final_state=True, cu_seqlens=cu,
+                              disable_recompute=True)
+        _, _, gk, Aqk, Akk, w, u, qg, kg, v_new, h, _ = f
+        results[C] = pipeline.chunk_kda_bwd(ins[0], ins[1], ins[2], ins[4], gk, Aqk, Akk, w, qg, kg, v_new, h, scale,
+                                            lay(do, layout).to(dev), dht, initial_state=h0, layout=layout, cu_seqlens=cu,
+                                            chunk_size=C)
+    for name, a, e in zip(("dq", "dk", "dv", "dg", "dbeta", "dh0"), results[128], results[64]):
+        assert a.shape == e.shape and a.dtype == e.dtype
+        # the gate reaches the kernels cumulated, differenced and cumulated again: last-bit changes there flip roundings of
+        # the 16-bit intermediates, so the two routes agree to the level of those roundings, not to fp32
+        close(a, e, name + " (128- against 64-token chunks)", 1e-2)
+
+
 def test_chunk_kda_rejections(dev):
     from fla_hip import pipeline
     q = torch.zeros(1, 64, 1, 128, dtype=BF, device=dev, requires_grad=True)
