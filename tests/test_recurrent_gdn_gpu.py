@@ -330,6 +330,16 @@ def test_prefill_plan_and_pooled_forward(dev):
         o = raw.gdn_chunk_fwd_state_pool(q, k, v, g, beta, K ** -0.5, pool, slots, cu, 64)
         assert torch.equal(o, o_ref)
         assert torch.equal(pool[[3, 1]], final[[0, 2]]) and torch.equal(pool[[0, 2, 4]], pool0[[0, 2, 4]])
+    # 64 channels, 128 value columns, rows normalised inside the kernel
+    K2 = 64
+    q2, k2 = (torch.randn(1, H, T, K2, generator=gen).to(BF).to(dev) for _ in range(2))
+    pool2 = (torch.randn(5, H, K2, V, generator=gen) * 0.1).to(dev)
+    h2 = pool2[[3, 0, 1]].clone()
+    h2[1] = 0
+    _, o_ref, final = raw.gdn_chunk_fwd(q2, k2, v, g, beta, K2 ** -0.5, h2, True, cu, 64, True)
+    pool = pool2.clone()
+    o = raw.gdn_chunk_fwd_state_pool(q2, k2, v, g, beta, K2 ** -0.5, pool, slots, cu, 64, use_qk_l2norm_in_kernel=True)
+    assert torch.equal(o, o_ref) and torch.equal(pool[[3, 1]], final[[0, 2]]) and torch.equal(pool[[0, 2, 4]], pool2[[0, 2, 4]])
 
 
 def test_wrapper_errors(dev):
