@@ -1424,7 +1424,7 @@ int launch_scan_as(const KdaScanParams &p, hipStream_t stream) {
 template <int K, int SUB>
 int launch_scan(const KdaScanParams &p, hipStream_t stream) {
     // 32-column slabs when 64-column ones leave compute units idle (see kda_scan_kernel)
-    const bool narrow = SUB == 1 && (int64_t)p.geom.N * p.geom.Hv * (p.geom.V / 64) < (int64_t)num_cus();
+    const bool narrow = (int64_t)p.geom.N * p.geom.Hv * (p.geom.V / 64) < (int64_t)num_cus();
     if constexpr (!kFineIsElem) {
         if (p.qg_fine) return narrow ? launch_scan_as<K, SUB, true, 32>(p, stream) : launch_scan_as<K, SUB, true, 64>(p, stream);
     }
