@@ -1130,7 +1130,7 @@ template <int K, bool GK, bool DVL = false, bool FQ = false>
 int launch_bwd_dhu(const DhuParams &p, int slabs, hipStream_t stream) {
     // per-channel gate (the KDA forms): 32-column slabs when 64-column ones leave compute units idle
     if constexpr (GK) {
-        if (p.sub == 1 && (int64_t)p.geom.N * p.geom.Hv * slabs < (int64_t)num_cus())
+        if ((int64_t)p.geom.N * p.geom.Hv * slabs < (int64_t)num_cus())
             return launch_bwd_dhu_as<K, GK, DVL, FQ, 32>(p, stream);
     }
     return launch_bwd_dhu_as<K, GK, DVL, FQ, 64>(p, stream);
